@@ -1,0 +1,25 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+
+
+@pytest.fixture(scope="session")
+def golden():
+    import json
+
+    out = {}
+    gdir = os.path.join(ROOT, "tests", "golden")
+    for name in os.listdir(gdir):
+        if name.endswith(".json"):
+            with open(os.path.join(gdir, name)) as f:
+                out[name[:-5]] = json.load(f)
+    return out

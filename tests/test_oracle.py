@@ -1,0 +1,610 @@
+"""Pins the CPU oracle (oracle/) before anything is compared against it.
+
+Each oracle function is checked against (i) the known-answer vectors the
+reference's own tests hold (tests/golden/*.json, transcribed from
+tests/test-rnn.cc, tests/test-nodes.cc, tests/test-tensor.cc,
+tests/python/test.py of the DyNet tree), and (ii) what the mathematics fixes:
+independent fp64 numpy formulas, central differences, invariances and brute
+force on tiny inputs -- chosen so that a dropped term, a wrong sign or a
+transposed operand fails.  No GPU needed.
+"""
+import numpy as np
+import pytest
+from scipy.special import logsumexp as sp_logsumexp
+
+from oracle import cpu_oracle as orc
+
+F32 = np.float32
+
+
+def f32(a):
+    return np.asarray(a, dtype=F32)
+
+
+def sigmoid64(x):
+    return 1.0 / (1.0 + np.exp(-np.asarray(x, np.float64)))
+
+
+def assert_rel(a, b, rel, what=""):
+    a = np.asarray(a, np.float64)
+    b = np.asarray(b, np.float64)
+    err = np.abs(a - b)
+    tol = rel * np.abs(b)
+    assert np.all(err <= tol), "%s: max rel err %g" % (what, np.max(err / np.maximum(np.abs(b), 1e-300)))
+
+
+# ---------------------------------------------------------------------------
+# logistic functor
+# ---------------------------------------------------------------------------
+def test_logistic_packet_matches_exact_sigmoid_absolutely():
+    xs = np.concatenate([np.linspace(-25, 25, 20001), [0.0, -18.0, 18.0, -1e-8, 1e-8]]).astype(F32)
+    y = orc.logistic_packet(xs)
+    assert np.max(np.abs(y.astype(np.float64) - sigmoid64(xs))) < 2e-7
+    assert y.min() >= 0.0 and y.max() <= 1.0
+    # clamp: everything beyond +-18 equals the value at +-18
+    assert np.all(orc.logistic_packet(f32([19, 100, 1e30])) == orc.logistic_packet(f32([18])))
+    assert np.all(orc.logistic_packet(f32([-19, -100, -1e30])) == orc.logistic_packet(f32([-18])))
+
+
+def test_logistic_packet_symmetry_and_midpoint():
+    xs = np.linspace(0, 18, 1801).astype(F32)
+    s = orc.logistic_packet(xs).astype(np.float64) + orc.logistic_packet(-xs).astype(np.float64)
+    assert np.max(np.abs(s - 1.0)) <= 1.2e-7
+    assert orc.logistic_packet(f32([0.0]))[0] == F32(0.5)
+
+
+def test_logistic_packet_is_not_relatively_accurate_in_the_left_tail():
+    # documents WHY the kernel mirrors the polynomial: against the exact form the
+    # packet form is off by far more than 1e-5 relative once sigma(x) is small
+    x = f32([-12.0])
+    rel = abs(float(orc.logistic_packet(x)[0]) - sigmoid64(-12.0)) / sigmoid64(-12.0)
+    assert rel > 1e-4
+
+
+def test_logistic_scalar_is_exact_form():
+    xs = np.linspace(-30, 30, 2001).astype(F32)
+    assert_rel(orc.logistic_scalar(xs), sigmoid64(xs), 3e-7, "logistic_scalar")
+
+
+# ---------------------------------------------------------------------------
+# elementwise
+# ---------------------------------------------------------------------------
+def test_unary_forward_against_fp64(golden):
+    rng = np.random.default_rng(1)
+    x = np.concatenate([rng.standard_normal(4096) * 3, golden["node_values"]["fixture_params"]["param1"], [0.0, -0.0]])
+    x = f32(x)
+    assert_rel(orc.unary_forward(orc.OP_TANH, x), np.tanh(x.astype(np.float64)), 3e-7, "tanh")
+    assert np.array_equal(orc.unary_forward(orc.OP_RECTIFY, x), np.maximum(x, 0))
+    assert np.array_equal(orc.unary_forward(orc.OP_NEGATE, x), -x)
+    assert np.max(np.abs(orc.unary_forward(orc.OP_LOGISTIC, x).astype(np.float64) - sigmoid64(x))) < 2e-7
+    assert_rel(orc.unary_forward(orc.OP_LOGISTIC, x, orc.LOGISTIC_SCALAR), sigmoid64(x), 3e-7, "logistic scalar")
+
+
+@pytest.mark.parametrize("op", [orc.OP_TANH, orc.OP_LOGISTIC, orc.OP_RECTIFY, orc.OP_NEGATE])
+def test_unary_backward_accumulates_the_derivative(op):
+    rng = np.random.default_rng(2)
+    x = f32(rng.standard_normal(513))
+    x[:3] = [0.0, -1.0, 2.0]
+    dy = f32(rng.standard_normal(513))
+    fx = orc.unary_forward(op, x, orc.LOGISTIC_SCALAR)
+    base = f32(rng.standard_normal(513))
+    dx = orc.unary_backward(op, fx, dy, base.copy())
+    x64 = x.astype(np.float64)
+    deriv = {orc.OP_TANH: 1 - np.tanh(x64) ** 2, orc.OP_LOGISTIC: sigmoid64(x64) * (1 - sigmoid64(x64)),
+             orc.OP_RECTIFY: (x64 > 0).astype(np.float64), orc.OP_NEGATE: -np.ones_like(x64)}[op]
+    want = base.astype(np.float64) + deriv * dy
+    assert np.max(np.abs(dx - want)) < 1e-6 * max(1.0, np.max(np.abs(want)))
+    if op == orc.OP_RECTIFY:  # ReLU'(0) = 0 because the mask is cast<bool>(fx)
+        assert dx[0] == base[0]
+
+
+def test_cmult_and_csum_broadcast_forward_backward():
+    rng = np.random.default_rng(3)
+    n, bd = 7, 5
+    a, b1, dy = f32(rng.standard_normal((bd, n))), f32(rng.standard_normal((1, n))), f32(rng.standard_normal((bd, n)))
+    assert np.allclose(orc.cmult_forward(n, bd, 1, a, b1), a * b1, rtol=0, atol=0)
+    assert np.allclose(orc.cmult_forward(n, 1, bd, b1, a), a * b1, rtol=0, atol=0)
+    assert np.allclose(orc.csum_forward(n, bd, 1, a, b1), a + b1, rtol=0, atol=0)
+    # backward to the full-batch argument and to the broadcast argument
+    da = orc.cmult_backward(n, bd, 1, a, b1, dy, 0, np.ones((bd, n), F32))
+    assert np.allclose(da, 1 + dy * b1, rtol=1e-6)
+    db = orc.cmult_backward(n, bd, 1, a, b1, dy, 1, np.ones((1, n), F32))
+    assert np.allclose(db, 1 + (dy.astype(np.float64) * a).sum(0), rtol=1e-5)
+    db = orc.csum_backward(n, bd, 1, dy, 1, np.ones((1, n), F32))
+    assert np.allclose(db, 1 + dy.astype(np.float64).sum(0), rtol=1e-5)
+    da = orc.csum_backward(n, bd, 1, dy, 0, np.ones((bd, n), F32))
+    assert np.allclose(da, 1 + dy)
+
+
+# ---------------------------------------------------------------------------
+# reductions (golden: cadd_broadcast2_neg_val, std_dim_value)
+# ---------------------------------------------------------------------------
+def test_sum_batches_golden_cadd_broadcast2_neg_val(golden):
+    g = golden["node_values"]
+    x1 = f32(g["fixture_params"]["param1"]).reshape(1, 3)
+    x2 = f32(g["fixture_params"]["param4"]).reshape(2, 3)
+    neg = orc.unary_forward(orc.OP_NEGATE, x2)
+    y = orc.csum_forward(3, 1, 2, x1, neg)  # x1 - x2 == x1 + (-x2), dynet/expr.cc:70
+    z = orc.sum_batches_forward(3, 2, y).astype(np.float64).sum()
+    exp = g["cadd_broadcast2_neg_val"]
+    assert abs(z - exp["expected"]) <= exp["rel_tol"] * abs(exp["expected"])
+
+
+def test_sum_batches_backward_broadcasts():
+    dy = f32([1, 2, 3])
+    dx = orc.sum_batches_backward(3, 4, dy, np.full((4, 3), 10, F32))
+    assert np.array_equal(dx, np.tile(dy, (4, 1)) + 10)
+
+
+def test_std_golden_std_dim_value(golden):
+    g = golden["node_values"]
+    # x is Dim({3,3},3): element (i,j,b) at i + 3j + 9b.  std over rows AND batch per
+    # column j == std_elems of the 9 gathered values
+    x = f32(g["fixture_params"]["param_cube1"]).reshape(3, 3, 3)  # [b][j][i]
+    cols = np.ascontiguousarray(np.stack([x[:, j, :].reshape(-1) for j in range(3)]))
+    y = orc.std_elems_forward(9, 3, cols)
+    z = float(orc.mean_elems_forward(3, 1, y)[0])
+    exp = g["std_dim_value"]
+    assert abs(z - exp["expected"]) <= exp["rel_tol"] * exp["expected"]
+    assert np.allclose(y, cols.astype(np.float64).std(axis=1), rtol=1e-6)
+
+
+def test_mean_std_backward_against_fp64_central_differences():
+    rng = np.random.default_rng(4)
+    n, bd = 6, 3
+    x = f32(rng.standard_normal((bd, n)))
+    dy = f32(rng.standard_normal(bd))
+    sd = orc.std_elems_forward(n, bd, x)
+    dx = orc.std_elems_backward(n, bd, x, sd, dy, np.zeros((bd, n), F32))
+    dm = orc.mean_elems_backward(n, bd, dy, np.zeros((bd, n), F32))
+    x64 = x.astype(np.float64)
+    eps = 1e-6
+    for b in range(bd):
+        for j in range(n):
+            xp, xm = x64.copy(), x64.copy()
+            xp[b, j] += eps
+            xm[b, j] -= eps
+            num = (xp.std(1) - xm.std(1)) @ dy / (2 * eps)
+            assert abs(dx[b, j] - num) < 1e-5
+            assert abs(dm[b, j] - dy[b] / n) < 1e-7
+
+
+# ---------------------------------------------------------------------------
+# layer norm
+# ---------------------------------------------------------------------------
+def ln64(x, g, b):
+    x = np.asarray(x, np.float64)
+    mu = x.mean(-1, keepdims=True)
+    sd = x.std(-1, keepdims=True)
+    return g * (x - mu) / (sd + 1e-8) + b
+
+
+def test_layer_norm_forward_golden_properties(golden):
+    g = golden["node_values"]
+    x = f32(g["fixture_params"]["param1"]).reshape(1, 3)
+    y = orc.layer_norm_forward(3, 1, x, np.ones(3, F32), np.zeros(3, F32)).astype(np.float64)
+    exp = g["layer_norm_forward"]
+    assert abs(y.sum() / 3.0) < exp["mean_abs_max"]
+    assert abs(np.sqrt((y ** 2).sum() / 3.0) - exp["rms"]) <= exp["rms_rel_tol"]
+
+
+def test_layer_norm_forward_golden_python_closed_form(golden):
+    exp = golden["node_values"]["layer_norm_python"]
+    v = np.arange(exp["n"]).astype(np.float64)
+    y = orc.layer_norm_forward(exp["n"], 1, f32(v), f32(v), f32(v))
+    want = v / v.std() * (v - v.mean()) + v
+    assert np.allclose(y.reshape(-1), want, rtol=exp["rtol"], atol=exp["atol"])
+
+
+def test_layer_norm_forward_fp64_and_invariances():
+    rng = np.random.default_rng(5)
+    n, bd = 64, 9
+    x = f32(rng.standard_normal((bd, n)) * 2 + 0.3)
+    g = f32(rng.uniform(0.5, 1.5, n))
+    b = f32(rng.standard_normal(n) * 0.1)
+    y = orc.layer_norm_forward(n, bd, x, g, b)
+    assert np.max(np.abs(y - ln64(x, g, b))) < 2e-6
+    y_shift = orc.layer_norm_forward(n, bd, x + F32(4.0), g, b)
+    assert np.max(np.abs(y_shift - y)) < 2e-5  # LN(x + c) == LN(x)
+    y_scale = orc.layer_norm_forward(n, bd, x * F32(8.0), g, b)
+    assert np.max(np.abs(y_scale - y)) < 2e-6  # LN(a x) == LN(x), a > 0 (power of two: exact scaling)
+    # epsilon sits on sigma, not on the variance: a constant row gives exactly b
+    yc = orc.layer_norm_forward(4, 1, np.full((1, 4), 3.0, F32), np.ones(4, F32), f32([1, 2, 3, 4]))
+    assert np.array_equal(yc.reshape(-1), f32([1, 2, 3, 4]))
+
+
+def ln_backward64(x, g, dy):
+    """Analytic LayerNorm gradient (epsilon ignored), independent of the composite."""
+    x, g, dy = (np.asarray(a, np.float64) for a in (x, g, dy))
+    n = x.shape[-1]
+    mu = x.mean(-1, keepdims=True)
+    sd = x.std(-1, keepdims=True)
+    xh = (x - mu) / sd
+    dxh = dy * g
+    dx = (dxh - dxh.mean(-1, keepdims=True) - xh * (dxh * xh).mean(-1, keepdims=True)) / sd
+    return dx, (dy * xh).sum(0), dy.sum(0)
+
+
+def test_layer_norm_backward_matches_analytic_fp64_and_accumulates():
+    rng = np.random.default_rng(6)
+    n, bd = 48, 7
+    x = f32(rng.standard_normal((bd, n)))
+    g = f32(rng.uniform(0.5, 1.5, n))
+    dy = f32(rng.standard_normal((bd, n)))
+    dx0, dg0, db0 = f32(rng.standard_normal((bd, n))), f32(rng.standard_normal(n)), f32(rng.standard_normal(n))
+    dx, dg, db = orc.layer_norm_backward(n, bd, x, g, dy, dx0.copy(), dg0.copy(), db0.copy())
+    wx, wg, wb = ln_backward64(x, g, dy)
+    assert np.max(np.abs(dx - (dx0 + wx))) < 5e-6
+    assert np.max(np.abs(dg - (dg0 + wg))) < 5e-6
+    assert np.max(np.abs(db - (db0 + wb))) < 5e-6
+    # NULL outputs are skipped
+    dx_only, _, _ = orc.layer_norm_backward(n, bd, x, g, dy, dx0.copy(), None, None)
+    assert np.array_equal(dx_only, dx)
+
+
+def test_layer_norm_backward_golden_grad_check_recipe(golden):
+    """tests/test-nodes.cc:2404-2412 with dynet/grad-check.cc's alpha and tolerances."""
+    gp = golden["node_values"]["fixture_params"]
+    rec = golden["node_values"]["grad_check"]
+    x, g, b = f32(gp["param1"]), f32(gp["param2"]), f32(gp["param3"])
+
+    def loss(x, g, b):  # to_scalar(y) = sqrt(sum(y^2)), tests/test-nodes.cc:102-107
+        y = orc.layer_norm_forward(3, 1, f32(x).reshape(1, 3), f32(g), f32(b)).astype(np.float64)
+        return np.sqrt((y ** 2).sum())
+
+    y = orc.layer_norm_forward(3, 1, x.reshape(1, 3), g, b).astype(np.float64)
+    dy = f32(y / np.sqrt((y ** 2).sum()))
+    dx, dg, db = orc.layer_norm_backward(3, 1, x.reshape(1, 3), g, dy, np.zeros((1, 3), F32), np.zeros(3, F32),
+                                         np.zeros(3, F32))
+    a = rec["alpha"]
+    for which, grad in (("x", dx.reshape(-1)), ("g", dg), ("b", db)):
+        for i in range(3):
+            args = {"x": x.copy(), "g": g.copy(), "b": b.copy()}
+            args[which][i] += a
+            right = loss(**args)
+            args[which][i] -= 2 * a
+            left = loss(**args)
+            num = (right - left) / (2 * a)
+            f = abs(num - grad[i])
+            m = max(abs(num), abs(grad[i]))
+            if f > rec["abs_tol"] and m > 0:
+                f /= m
+            assert f <= rec["rel_tol"], (which, i, num, grad[i])
+
+
+# ---------------------------------------------------------------------------
+# GEMM shim
+# ---------------------------------------------------------------------------
+def test_gemm_three_forms_against_fp64():
+    rng = np.random.default_rng(7)
+    M, N, K = 5, 4, 6
+    # column-major [rows x cols] == numpy (cols, rows) C-order
+    l = f32(rng.standard_normal((K, M)))  # M x K
+    r = f32(rng.standard_normal((N, K)))  # K x N
+    y0 = f32(rng.standard_normal((N, M)))
+    y = orc.gemm_nn(M, N, K, l, r, 1.0, y0.copy())
+    want = y0.T.astype(np.float64) + l.T.astype(np.float64) @ r.T.astype(np.float64)
+    assert np.allclose(y.T, want, rtol=1e-5, atol=1e-6)
+    y = orc.gemm_nn(M, N, K, l, r, 0.0, y0.copy())
+    assert np.allclose(y.T, l.T.astype(np.float64) @ r.T, rtol=1e-5, atol=1e-6)
+    lt = f32(rng.standard_normal((M, K)))  # K x M, used transposed
+    y = orc.gemm_tn_acc(M, N, K, lt, r, y0.copy())
+    assert np.allclose(y.T, y0.T + lt.astype(np.float64) @ r.T, rtol=1e-5, atol=1e-6)
+    rt = f32(rng.standard_normal((K, N)))  # N x K, used transposed
+    y = orc.gemm_nt_acc(M, N, K, l, rt, y0.copy())
+    assert np.allclose(y.T, y0.T + l.T.astype(np.float64) @ rt, rtol=1e-5, atol=1e-6)
+
+
+# ---------------------------------------------------------------------------
+# fused LSTM nodes: golden vectors of tests/test-rnn.cc
+# ---------------------------------------------------------------------------
+def test_lstm_h_golden(golden):
+    t = golden["lstm_nodes"]["lstm_node_h_fwd"]
+    h = orc.lstm_h_forward(t["hidden_dim"], t["batch_size"], f32(t["c_t"]), f32(t["gates_t"])).reshape(-1)
+    assert abs(h[0]) < t["small_abs"]
+    assert_rel(h[1:], t["h_t"][1:], golden["lstm_nodes"]["rel_tol"], "lstm_h")
+
+
+def test_lstm_c_golden(golden):
+    t = golden["lstm_nodes"]["lstm_node_c_fwd"]
+    c = orc.lstm_c_forward(t["hidden_dim"], t["batch_size"], f32(t["c_tm1"]), f32(t["gates_t"])).reshape(-1)
+    assert np.all(np.abs(c[:3]) < t["small_abs"])
+    assert_rel(c[3:], t["c_t"][3:], golden["lstm_nodes"]["rel_tol"], "lstm_c")
+
+
+@pytest.mark.parametrize("mode", [orc.LOGISTIC_PACKET, orc.LOGISTIC_SCALAR])
+def test_lstm_gates_golden(golden, mode):
+    t = golden["lstm_nodes"]["lstm_node_gates_fwd"]
+    g = orc.lstm_gates_forward([f32(t["x_t"])], [t["input_dim"]], t["hidden_dim"], t["batch_size"], f32(t["h_tm1"]),
+                               f32(t["Wx"]), f32(t["Wh"]), f32(t["b"]), logistic_mode=mode)
+    assert_rel(g.reshape(-1), t["gates"], golden["lstm_nodes"]["rel_tol"], "lstm_gates")
+
+
+@pytest.mark.parametrize("mode", [orc.LOGISTIC_PACKET, orc.LOGISTIC_SCALAR])
+def test_lstm_gates_dropout_golden(golden, mode):
+    t = golden["lstm_nodes"]["lstm_node_gates_dropout_fwd"]
+    B = t["batch_size"]
+    g = orc.lstm_gates_forward([f32(t["x_t"])], [t["input_dim"]], t["hidden_dim"], B, f32(t["h_tm1"]),
+                               f32(t["Wx"]), f32(t["Wh"]), f32(t["b"]), f32(t["mask_x"]), B, f32(t["mask_h"]), B,
+                               logistic_mode=mode)
+    assert_rel(g.reshape(-1), t["gates"], golden["lstm_nodes"]["rel_tol"], "lstm_gates_dropout")
+
+
+# independent fp64 model of the three nodes ---------------------------------
+def gates64(x, h, Wx, Wh, b, H, mask_x=None, mask_h=None):
+    """x: (B, I), h: (B, H), Wx: (4H, I), Wh: (4H, H); returns (B, 4H)."""
+    x, h = np.asarray(x, np.float64), np.asarray(h, np.float64)
+    if mask_x is not None:
+        x = x * mask_x
+        h = h * mask_h
+    pre = x @ np.asarray(Wx, np.float64).T + h @ np.asarray(Wh, np.float64).T + np.asarray(b, np.float64)
+    pre[:, H:2 * H] += 1.0
+    out = np.empty_like(pre)
+    out[:, :3 * H] = sigmoid64(pre[:, :3 * H])
+    out[:, 3 * H:] = np.tanh(pre[:, 3 * H:])
+    return out
+
+
+def cm(a, rows, cols):
+    """column-major flat buffer of a (rows x cols) matrix -> numpy (rows, cols)."""
+    return np.asarray(a).reshape(cols, rows).T
+
+
+def lstm_case(rng, I, H, B):
+    x = f32(rng.standard_normal((B, I)))
+    h = f32(rng.standard_normal((B, H)))
+    Wx = f32(rng.uniform(-0.4, 0.4, (I, 4 * H)))  # column-major 4H x I
+    Wh = f32(rng.uniform(-0.4, 0.4, (H, 4 * H)))
+    b = f32(rng.standard_normal(4 * H) * 0.1)
+    return x, h, Wx, Wh, b
+
+
+def test_lstm_gates_forward_fp64_and_multi_input_equivalence():
+    rng = np.random.default_rng(8)
+    I, H, B = 4, 5, 3
+    x, h, Wx, Wh, b = lstm_case(rng, I, H, B)
+    got = orc.lstm_gates_forward([x], [I], H, B, h, Wx, Wh, b, logistic_mode=orc.LOGISTIC_SCALAR)
+    want = gates64(x, h, cm(Wx, 4 * H, I), cm(Wh, 4 * H, H), b, H)
+    assert np.max(np.abs(got - want)) < 1e-6
+    # multi-input == single concatenated input (tests/test-rnn.cc:462-497)
+    x1, x3 = np.ascontiguousarray(x[:, :1]), np.ascontiguousarray(x[:, 1:])
+    got2 = orc.lstm_gates_forward([x1, x3], [1, 3], H, B, h, Wx, Wh, b, logistic_mode=orc.LOGISTIC_SCALAR)
+    assert np.array_equal(got, got2)
+    # batch-broadcast masks == masks tiled over the batch
+    mx, mh = f32(rng.integers(0, 2, (1, I)) * 0.9), f32(rng.integers(0, 2, (1, H)) * 0.8)
+    ga = orc.lstm_gates_forward([x], [I], H, B, h, Wx, Wh, b, mx, 1, mh, 1)
+    gb = orc.lstm_gates_forward([x], [I], H, B, h, Wx, Wh, b, np.tile(mx, (B, 1)), B, np.tile(mh, (B, 1)), B)
+    assert np.array_equal(ga, gb)
+    want = gates64(x, h, cm(Wx, 4 * H, I), cm(Wh, 4 * H, H), b, H, mx, mh)
+    assert np.max(np.abs(ga - want)) < 1e-6
+
+
+def test_fused_nodes_equal_unfused_builder_path():
+    """tests/test-rnn.cc:155-184,214-243: three steps of gates/C/H equal the
+    VanillaLSTMBuilder recurrence (dynet/lstm.cc:519-545: affine, pick_range,
+    logistic(+1 on f), tanh, cmult) to 1e-5."""
+    rng = np.random.default_rng(9)
+    I, H, B = 3, 5, 2
+    x, h, Wx, Wh, b = lstm_case(rng, I, H, B)
+    c = f32(rng.standard_normal((B, H)))
+    W64x, W64h = cm(Wx, 4 * H, I).astype(np.float64), cm(Wh, 4 * H, H).astype(np.float64)
+    h64, c64 = h.astype(np.float64), c.astype(np.float64)
+    for _ in range(3):
+        gates = orc.lstm_gates_forward([x], [I], H, B, h, Wx, Wh, b, logistic_mode=orc.LOGISTIC_SCALAR)
+        c = orc.lstm_c_forward(H, B, c, gates)
+        h = orc.lstm_h_forward(H, B, c, gates)
+        tmp = x.astype(np.float64) @ W64x.T + h64 @ W64h.T + b
+        i_t, f_t = sigmoid64(tmp[:, :H]), sigmoid64(tmp[:, H:2 * H] + 1.0)
+        o_t, g_t = sigmoid64(tmp[:, 2 * H:3 * H]), np.tanh(tmp[:, 3 * H:])
+        c64 = f_t * c64 + i_t * g_t
+        h64 = o_t * np.tanh(c64)
+        assert_rel(h, h64, 1e-5, "fused vs unfused h")
+
+
+@pytest.mark.parametrize("dropout,mask_bd_full,multi", [(False, True, False), (True, True, False),
+                                                        (True, False, False), (False, True, True),
+                                                        (True, True, True)])
+def test_lstm_gates_backward_all_args_fp64(dropout, mask_bd_full, multi):
+    """Gradients of every argument against central differences of the
+    independent fp64 model, on the shapes of tests/test-rnn.cc:341-357,
+    402-460,499-529,601-630 (I=5 or 4, H=3 or 5, B=2)."""
+    rng = np.random.default_rng(10)
+    I, H, B = (4, 5, 2) if multi else (5, 3, 2)
+    x, h, Wx, Wh, b = lstm_case(rng, I, H, B)
+    dims = [1, 3] if multi else [I]
+    offs = np.cumsum([0] + dims)
+    xs = [np.ascontiguousarray(x[:, offs[k]:offs[k + 1]]) for k in range(len(dims))]
+    mx = mh = None
+    mbd = 0
+    if dropout:
+        mbd = B if mask_bd_full else 1
+        mx = f32(rng.integers(0, 2, (mbd, I)) * 0.9)
+        mh = f32(rng.integers(0, 2, (mbd, H)) * 0.8)
+    dy = f32(rng.standard_normal((B, 4 * H)))
+    fx = orc.lstm_gates_forward(xs, dims, H, B, h, Wx, Wh, b, mx, mbd, mh, mbd, logistic_mode=orc.LOGISTIC_SCALAR)
+
+    def loss(x_, h_, Wx_, Wh_, b_):
+        return (gates64(x_, h_, cm(Wx_, 4 * H, I), cm(Wh_, 4 * H, H), b_, H, mx, mh) * dy).sum()
+
+    base = [x.astype(np.float64), h.astype(np.float64), Wx.astype(np.float64), Wh.astype(np.float64),
+            b.astype(np.float64)]
+
+    def numgrad(k):
+        g = np.zeros_like(base[k])
+        it = np.nditer(base[k], flags=["multi_index"])
+        eps = 1e-6
+        for _ in it:
+            idx = it.multi_index
+            args = [a.copy() for a in base]
+            args[k][idx] += eps
+            up = loss(*args)
+            args[k][idx] -= 2 * eps
+            g[idx] = (up - loss(*args)) / (2 * eps)
+        return g
+
+    k_in = len(dims)
+    # inputs
+    gx = numgrad(0)
+    for k in range(k_in):
+        acc0 = f32(rng.standard_normal((B, dims[k])))
+        got = orc.lstm_gates_backward(xs, dims, H, B, h, Wx, Wh, fx, dy, k, acc0.copy(), mx, mbd, mh, mbd)
+        assert np.max(np.abs(got - (acc0 + gx[:, offs[k]:offs[k + 1]]))) < 2e-5, "dx%d" % k
+    for j, (arg_i, shape) in enumerate([(k_in, (B, H)), (k_in + 1, (I, 4 * H)), (k_in + 2, (H, 4 * H)),
+                                        (k_in + 3, (4 * H,))]):
+        acc0 = f32(rng.standard_normal(shape))
+        got = orc.lstm_gates_backward(xs, dims, H, B, h, Wx, Wh, fx, dy, arg_i, acc0.copy(), mx, mbd, mh, mbd)
+        assert np.max(np.abs(got - (acc0 + numgrad(j + 1)))) < 2e-5, "arg %d" % arg_i
+
+
+def test_lstm_c_h_backward_fp64():
+    rng = np.random.default_rng(11)
+    H, B = 3, 2
+    c_prev = f32(rng.standard_normal((B, H)))
+    gates = f32(rng.uniform(0.05, 0.95, (B, 4 * H)))
+    dc = f32(rng.standard_normal((B, H)))
+    g64 = gates.astype(np.float64)
+    i_, f_, o_, g_ = (g64[:, k * H:(k + 1) * H] for k in range(4))
+    got = orc.lstm_c_backward(H, B, c_prev, gates, dc, 0, np.ones((B, H), F32))
+    assert np.allclose(got, 1 + dc * f_, rtol=1e-6)
+    got = orc.lstm_c_backward(H, B, c_prev, gates, dc, 1, np.ones((B, 4 * H), F32))
+    want = np.ones((B, 4 * H))
+    want[:, :H] += dc * g_
+    want[:, H:2 * H] += dc * c_prev
+    want[:, 3 * H:] += dc * i_
+    assert np.allclose(got, want, rtol=1e-6)  # the o rows stay untouched
+    c = orc.lstm_c_forward(H, B, c_prev, gates)
+    t = np.tanh(c.astype(np.float64))
+    got = orc.lstm_h_backward(H, B, c, gates, dc, 0, np.ones((B, H), F32))
+    assert np.allclose(got, 1 + dc * o_ * (1 - t * t), rtol=1e-5)
+    got = orc.lstm_h_backward(H, B, c, gates, dc, 1, np.ones((B, 4 * H), F32))
+    want = np.ones((B, 4 * H))
+    want[:, 2 * H:3 * H] += dc * t
+    assert np.allclose(got, want, rtol=1e-5)
+
+
+# ---------------------------------------------------------------------------
+# lookup
+# ---------------------------------------------------------------------------
+def test_lookup_forward_is_a_bit_exact_gather_and_checks_bounds(golden):
+    table = f32(golden["node_values"]["fixture_params"]["param_square1"]).reshape(3, 3)  # lookup1: 3 rows of dim 3
+    ids = [0, 2, 2, 1, 0]
+    out = orc.lookup_forward(ids, 3, 3, table)
+    assert out.tobytes() == table[ids].tobytes()
+    assert np.array_equal(orc.lookup_forward(ids, 3, 3, table, 0.5), table[ids] * F32(0.5))
+    with pytest.raises(ValueError):
+        orc.lookup_forward([0, 3], 3, 3, table)
+
+
+def test_lookup_accumulate_grads_brute_force_with_duplicates():
+    rng = np.random.default_rng(12)
+    V, D, n = 5, 4, 64
+    ids = rng.integers(0, 3, n).astype(np.uint32)  # heavy duplication, rows 3..4 untouched
+    g = f32(rng.standard_normal((n, D)))
+    grads0 = f32(rng.standard_normal((V, D)))
+    got = orc.lookup_accumulate_grads(ids, D, V, g, grads0.copy())
+    want = grads0.copy()
+    for b in range(n):  # sequential fp32, the CPU path's order
+        want[ids[b]] = want[ids[b]] + g[b]
+    assert got.tobytes() == want.tobytes()
+    assert np.array_equal(got[3:], grads0[3:])
+    assert abs(got.astype(np.float64).sum() - grads0.astype(np.float64).sum() - g.astype(np.float64).sum()) < 1e-4
+    with pytest.raises(ValueError):
+        orc.lookup_accumulate_grads([7], D, V, g[:1], grads0.copy())
+
+
+# ---------------------------------------------------------------------------
+# logsumexp / pickneglogsoftmax / argmax
+# ---------------------------------------------------------------------------
+def test_logsumexp_cols_against_scipy_and_shift_invariance():
+    rng = np.random.default_rng(13)
+    rows, bd = 301, 6
+    x = f32(rng.standard_normal((bd, rows)) * 2)
+    m, z = orc.logsumexp_cols(rows, bd, x)
+    assert np.array_equal(m, x.max(1))
+    assert_rel(z, sp_logsumexp(x.astype(np.float64), axis=1), 2e-6, "lse")
+    _, z2 = orc.logsumexp_cols(rows, bd, x + F32(16.0))
+    assert np.max(np.abs(z2 - z - 16.0)) < 1e-5
+    _, zbig = orc.logsumexp_cols(3, 1, f32([[1000.0, 1000.0, -1000.0]]))
+    assert abs(zbig[0] - (1000.0 + np.log(2.0))) < 1e-4  # no overflow
+
+
+def test_pnls_forward_backward_fp64(golden):
+    rng = np.random.default_rng(14)
+    rows, bd = 37, 5
+    x = f32(rng.standard_normal((bd, rows)) * 2)
+    labels = rng.integers(0, rows, bd).astype(np.uint32)
+    fx, aux = orc.pnls_forward(rows, bd, x, labels)
+    ids = aux.view(np.uint32)[2 * bd:]
+    assert np.array_equal(ids, np.arange(bd) * rows + labels)  # picks are index lookups: bit exact
+    lse = sp_logsumexp(x.astype(np.float64), axis=1)
+    want = lse - x[np.arange(bd), labels]
+    assert_rel(fx, want, 1e-5, "pnls fwd")
+    dy = f32(rng.standard_normal(bd))
+    dx0 = f32(rng.standard_normal((bd, rows)))
+    dx = orc.pnls_backward(rows, bd, x, aux, dy, dx0.copy())
+    soft = np.exp(x.astype(np.float64) - lse[:, None])
+    onehot = np.zeros((bd, rows))
+    onehot[np.arange(bd), labels] = 1
+    assert np.max(np.abs(dx - (dx0 + (soft - onehot) * dy[:, None]))) < 2e-6
+    # sum_v (softmax - onehot) == 0 per row
+    assert np.max(np.abs((dx - dx0).astype(np.float64).sum(1))) < 2e-6
+    with pytest.raises(ValueError):
+        orc.pnls_forward(rows, bd, x, np.full(bd, rows, np.uint32))
+    # tests/test-nodes.cc:2088-2094: x1 = param1, idx = 1
+    x1 = f32(golden["node_values"]["fixture_params"]["param1"]).reshape(1, 3)
+    fx1, _ = orc.pnls_forward(3, 1, x1, [1])
+    assert abs(fx1[0] - (sp_logsumexp(x1.astype(np.float64)) - x1[0, 1])) < 1e-6
+
+
+def test_logsumexp_node_forward_backward():
+    rng = np.random.default_rng(15)
+    n, bd = 6, 4
+    a, b, c1 = f32(rng.standard_normal((bd, n))), f32(rng.standard_normal((bd, n))), f32(rng.standard_normal((1, n)))
+    fx = orc.logsumexp_node_forward(n, bd, [a, b, c1], [bd, bd, 1])
+    want = np.log(np.exp(a.astype(np.float64)) + np.exp(b) + np.exp(c1))
+    assert_rel(fx, want, 2e-6, "logsumexp node")
+    dy = f32(rng.standard_normal((bd, n)))
+    da = orc.logsumexp_node_backward(n, bd, [a, b, c1], [bd, bd, 1], fx, dy, 0, np.zeros((bd, n), F32))
+    assert np.max(np.abs(da - np.exp(a - want) * dy)) < 2e-6
+    dc = orc.logsumexp_node_backward(n, bd, [a, b, c1], [bd, bd, 1], fx, dy, 2, np.zeros((1, n), F32))
+    assert np.max(np.abs(dc - (np.exp(c1 - want) * dy).sum(0))) < 2e-6
+    one = orc.logsumexp_node_forward(n, bd, [a], [bd])
+    assert np.array_equal(one, a)
+
+
+def test_argmax_golden(golden):
+    t = golden["node_values"]["argmax"]
+    assert list(orc.argmax_cols(t["rows"], t["bd"], f32(t["x"]))) == t["expected"]
+    assert list(orc.argmax_cols(4, 1, f32([3, 7, 7, 1]))) == [1]  # first maximum on ties
+
+
+# ---------------------------------------------------------------------------
+# scatter/gather helpers, parameter copy, trainer
+# ---------------------------------------------------------------------------
+def test_gpu_ops_helpers_against_numpy():
+    rng = np.random.default_rng(16)
+    src = f32(rng.standard_normal(10))
+    idx = np.array([3, 0, 7], np.uint32)
+    assert np.array_equal(orc.sparse_to_dense_assign(idx, src), src[idx])
+    trg = np.zeros(10, F32)
+    orc.dense_to_sparse_assign(idx, src[:3], trg)
+    assert np.array_equal(trg[idx], src[:3]) and trg.sum() == src[:3].sum()
+    trg = np.ones(10, F32)
+    orc.dense_to_sparse_subtract(np.array([2, 2, 5], np.uint32), f32([1, 2, 3]), trg)
+    assert trg[2] == -2 and trg[5] == -2
+    table = f32(rng.standard_normal((6, 4)))
+    out = orc.sparse_to_dense_block_assign_and_multiply(np.array([5, 5, 1], np.uint32), 4, 2.0, table)
+    assert np.array_equal(out, table[[5, 5, 1]] * 2)
+    acc = np.zeros((6, 4), F32)
+    orc.dense_to_sparse_block_add(np.array([5, 5, 1], np.uint32), 4, out, acc)
+    assert np.allclose(acc[5], out[0] + out[1]) and np.array_equal(acc[1], out[2])
+
+
+def test_scale_copy_sgd_and_norm():
+    rng = np.random.default_rng(17)
+    p, g = f32(rng.standard_normal(33)), f32(rng.standard_normal(33))
+    assert np.array_equal(orc.scale_copy(p, 1.0), p)
+    # p -= g * (lr * gscale / wd), dynet/training.cc:621
+    want = p - g * F32(F32(0.1) * F32(0.5) / F32(1.0))
+    assert np.array_equal(orc.sgd_update(p.copy(), g, 0.1, 0.5, 1.0), want)
+    assert abs(orc.squared_l2norm(g) - (g.astype(np.float64) ** 2).sum()) < 1e-4
