@@ -1,0 +1,189 @@
+// Shared internals of libdynet_hip.so: status/error plumbing, the device and
+// pool objects behind the opaque C handles, and wavefront-level primitives.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstddef>
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "dynet_hip.h"
+
+namespace dyhip {
+
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+// ceil(a / b) for positive integers
+template <class T>
+constexpr T cdiv(T a, T b) {
+  return (a + b - 1) / b;
+}
+
+__host__ __device__ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- allocators (MemAllocator of the reference: align, malloc, free, zero) --
+struct MemAllocator {
+  explicit MemAllocator(size_t align) : align(align) {}
+  virtual ~MemAllocator() {}
+  virtual void* malloc(size_t n) = 0;
+  virtual void free(void* p) = 0;
+  virtual bool zero(void* p, size_t n) = 0;
+  size_t round_up_align(size_t n) const { return align < 2 ? n : ((n + align - 1) / align) * align; }
+  const size_t align;
+};
+
+}  // namespace dyhip
+
+// One growable bump-allocated region set: a list of blocks, allocation only
+// from the newest block, consolidation on free().
+struct dyhip_pool {
+  struct Block {
+    char* mem;
+    size_t capacity;
+    size_t used;
+  };
+  std::string name;
+  std::vector<Block> blocks;
+  size_t cap;             // sum of block capacities
+  size_t expanding_unit;  // growth granularity (1 << 24 in the reference)
+  dyhip::MemAllocator* alloc;
+  bool owns_alloc;
+};
+
+struct dyhip_device {
+  int ordinal;
+  int num_cus;
+  hipStream_t stream;
+  dyhip::MemAllocator* alloc;
+  dyhip_pool* pools[4];
+  float* scalars;  // device: {-1, 1, 0}
+  void* gemm_ws;   // split-K partial tiles (the analogue of a BLAS handle's workspace)
+  size_t gemm_ws_bytes;
+  hipEvent_t ev_start, ev_stop;
+};
+
+#define DYHIP_CHECK_HIP(expr)                                                                   \
+  do {                                                                                          \
+    hipError_t e_ = (expr);                                                                     \
+    if (e_ != hipSuccess)                                                                       \
+      return dyhip::fail(DYHIP_ERR_RUNTIME, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), \
+                         __FILE__, __LINE__);                                                   \
+  } while (0)
+
+#define DYHIP_REQUIRE(cond, ...)                                          \
+  do {                                                                    \
+    if (!(cond)) return dyhip::fail(DYHIP_ERR_INVALID_ARG, __VA_ARGS__);  \
+  } while (0)
+
+#define DYHIP_CHECK_DEV(dev)                                                      \
+  do {                                                                            \
+    if ((dev) == nullptr) return dyhip::fail(DYHIP_ERR_INVALID_ARG, "null device handle"); \
+  } while (0)
+
+#define DYHIP_CHECK_LAUNCH() DYHIP_CHECK_HIP(hipGetLastError())
+
+#define DYHIP_CHECK_STATUS(expr) \
+  do {                           \
+    int s_ = (expr);             \
+    if (s_ != DYHIP_OK) return s_; \
+  } while (0)
+
+#ifdef __HIPCC__
+namespace dyhip {
+
+// ---- wavefront reductions (64 lanes) -----------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+  return v;
+}
+
+// Block-wide sum for blockDim.x = 64 * NW.  Every thread gets the result.
+// `red` is an LDS array of at least NW floats; safe to call repeatedly.
+template <int NW>
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  if (NW == 1) return v;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) red[w] = v;
+  __syncthreads();
+  float t = red[0];
+#pragma unroll
+  for (int i = 1; i < NW; ++i) t += red[i];
+  return t;
+}
+
+template <int NW>
+__device__ __forceinline__ float block_max(float v, float* red) {
+  v = wave_max(v);
+  if (NW == 1) return v;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) red[w] = v;
+  __syncthreads();
+  float t = red[0];
+#pragma unroll
+  for (int i = 1; i < NW; ++i) t = fmaxf(t, red[i]);
+  return t;
+}
+
+// ---- scalar math shared by several kernels -----------------------------------
+
+// scalar_logistic_sigmoid_op::packetOp of the reference (dynet/simd-functors.h:81-125):
+// clamp to [-18,18], rational polynomial in Horner form with one fused
+// multiply-add per pmadd, IEEE division, +0.5, clamp to [0,1].
+__device__ __forceinline__ float logistic_packet(float _x) {
+  const float x = fmaxf(fminf(_x, 18.0f), -18.0f);
+  const float x2 = x * x;
+  float p = fmaf(x2, (float)4.37031012579801e-11, (float)1.15627324459942e-07);
+  p = fmaf(x2, p, (float)6.08574864600143e-05);
+  p = fmaf(x2, p, (float)8.51377133304701e-03);
+  p = fmaf(x2, p, (float)2.48287947061529e-01);
+  p = x * p;
+  float q = fmaf(x2, (float)6.10247389755681e-13, (float)5.76102136993427e-09);
+  q = fmaf(x2, q, (float)6.29106785017040e-06);
+  q = fmaf(x2, q, (float)1.70198817374094e-03);
+  q = fmaf(x2, q, (float)1.16817656904453e-01);
+  q = fmaf(x2, q, (float)9.93151921023180e-01);
+  return fmaxf(fminf(p / q + 0.5f, 1.0f), 0.0f);
+}
+
+// scalar operator() of the same functor (:76-79)
+__device__ __forceinline__ float logistic_scalar(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+__device__ __forceinline__ float logistic(int mode, float x) {
+  return mode == DYHIP_LOGISTIC_SCALAR ? logistic_scalar(x) : logistic_packet(x);
+}
+
+// tanh accurate to ~3e-7 relative over the whole range: odd series for
+// |x| < 0.25 (where 1 - e^{-2|x|} would cancel), (1-t)/(1+t) with
+// t = e^{-2|x|} elsewhere.
+__device__ __forceinline__ float tanh_accurate(float x) {
+  const float ax = fabsf(x);
+  if (ax < 0.25f) {
+    const float x2 = x * x;
+    float p = fmaf(x2, -1382.0f / 155925.0f, 62.0f / 2835.0f);
+    p = fmaf(x2, p, -17.0f / 315.0f);
+    p = fmaf(x2, p, 2.0f / 15.0f);
+    p = fmaf(x2, p, -1.0f / 3.0f);
+    return fmaf(x * x2, p, x);
+  }
+  const float t = __expf(-2.0f * ax);
+  const float r = (1.0f - t) / (1.0f + t);
+  return copysignf(r, x);
+}
+
+}  // namespace dyhip
+#endif  // __HIPCC__

@@ -1,0 +1,288 @@
+// Elementwise launch layer: y = f(inputs) or y += f(inputs) over flat fp32
+// buffers, with optional broadcast of an input over the batch dimension.
+//
+// Replaces the Eigen-on-GPU statements of Tanh / LogisticSigmoid / Rectify /
+// Negate (dynet/nodes-trig.cc:312-326, nodes-activations.cc:31-78,
+// nodes-arith-unary.cc:195-209), CwiseMultiply / CwiseSum without dimension
+// broadcast (dynet/nodes-arith-cwise.cc:50-122,196-273), SumDimension's
+// backward broadcast (dynet/nodes-arith-sum.cc:219-230), TensorTools::constant
+// and accumulate, ParameterNode's scaled copy (dynet/param-nodes.cc:201-215),
+// the SGD rule (dynet/training.cc:619-622), and takes the shape of the unused
+// templated kernels of dynet/gpu-kernels.h:9-52.
+//
+// Layout: a tensor of n elements per batch element and bd batch elements is one
+// flat buffer of n*bd floats.  A block owns one tile of 256 threads x UNROLL
+// 128-bit accesses inside ONE batch element, so a broadcast input (batch 1) is
+// indexed by the in-batch offset without any division per element.  All loads
+// of a thread are issued before the first use to keep 4 x 16 B per lane in
+// flight.  Tensors whose n is not a multiple of 4, or whose base is not
+// 16-byte aligned, take the scalar variant of the same kernel.
+#include "common.h"
+
+namespace dyhip {
+
+constexpr int kEwThreads = 256;
+constexpr int kEwUnroll = 4;
+
+struct EwArgs {
+  const float* in[3];
+  float* out;
+  size_t n;                 // elements per batch element (of the output)
+  unsigned tiles_per_batch; // tiles covering one batch element
+};
+
+// F: struct with  __device__ float operator()(float a, float b, float c, float old) const
+// NIN: number of inputs read; ACC: also read the output (old value).
+// BMASK: bit k set => input k has batch 1 and is indexed by the in-batch offset.
+template <int NIN, bool ACC, int BMASK, class F>
+__global__ __launch_bounds__(kEwThreads) void ew_vec4_kernel(EwArgs a, F f) {
+  const unsigned batch = blockIdx.x / a.tiles_per_batch;
+  const unsigned tile = blockIdx.x - batch * a.tiles_per_batch;
+  const size_t n4 = a.n >> 2;
+  const size_t base4 = size_t(batch) * n4;
+  const size_t j0 = size_t(tile) * (kEwThreads * kEwUnroll) + threadIdx.x;
+  float4 v[3][kEwUnroll];
+  float4 o[kEwUnroll];
+#pragma unroll
+  for (int u = 0; u < kEwUnroll; ++u) {
+    const size_t j = j0 + size_t(u) * kEwThreads;
+    if (j < n4) {
+#pragma unroll
+      for (int k = 0; k < NIN; ++k) {
+        const float4* p = reinterpret_cast<const float4*>(a.in[k]);
+        v[k][u] = p[((BMASK >> k) & 1) ? j : base4 + j];
+      }
+      if (ACC) o[u] = reinterpret_cast<const float4*>(a.out)[base4 + j];
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < kEwUnroll; ++u) {
+    const size_t j = j0 + size_t(u) * kEwThreads;
+    if (j < n4) {
+      const float4 x0 = NIN > 0 ? v[0][u] : make_float4(0, 0, 0, 0);
+      const float4 x1 = NIN > 1 ? v[1][u] : make_float4(0, 0, 0, 0);
+      const float4 x2 = NIN > 2 ? v[2][u] : make_float4(0, 0, 0, 0);
+      const float4 od = ACC ? o[u] : make_float4(0, 0, 0, 0);
+      float4 r;
+      r.x = f(x0.x, x1.x, x2.x, od.x);
+      r.y = f(x0.y, x1.y, x2.y, od.y);
+      r.z = f(x0.z, x1.z, x2.z, od.z);
+      r.w = f(x0.w, x1.w, x2.w, od.w);
+      reinterpret_cast<float4*>(a.out)[base4 + j] = r;
+    }
+  }
+}
+
+template <int NIN, bool ACC, int BMASK, class F>
+__global__ __launch_bounds__(kEwThreads) void ew_scalar_kernel(EwArgs a, F f) {
+  const unsigned batch = blockIdx.x / a.tiles_per_batch;
+  const unsigned tile = blockIdx.x - batch * a.tiles_per_batch;
+  const size_t base = size_t(batch) * a.n;
+  const size_t j0 = size_t(tile) * (kEwThreads * kEwUnroll) + threadIdx.x;
+#pragma unroll
+  for (int u = 0; u < kEwUnroll; ++u) {
+    const size_t j = j0 + size_t(u) * kEwThreads;
+    if (j < a.n) {
+      const float x0 = NIN > 0 ? a.in[0][(BMASK & 1) ? j : base + j] : 0.f;
+      const float x1 = NIN > 1 ? a.in[1][(BMASK & 2) ? j : base + j] : 0.f;
+      const float x2 = NIN > 2 ? a.in[2][(BMASK & 4) ? j : base + j] : 0.f;
+      const float od = ACC ? a.out[base + j] : 0.f;
+      a.out[base + j] = f(x0, x1, x2, od);
+    }
+  }
+}
+
+// Launch over an (n x bd) output.  Inputs whose bit is set in BMASK have batch 1.
+template <int NIN, bool ACC, int BMASK, class F>
+int ew_launch(dyhip_device* dev, size_t n, unsigned bd, const float* in0, const float* in1, const float* in2,
+              float* out, F f) {
+  if (n == 0 || bd == 0) return DYHIP_OK;
+  if (BMASK == 0) {  // nothing is broadcast: one flat buffer
+    n *= bd;
+    bd = 1;
+  }
+  EwArgs a;
+  a.in[0] = in0;
+  a.in[1] = in1;
+  a.in[2] = in2;
+  a.out = out;
+  a.n = n;
+  bool vec = (n % 4 == 0) && aligned16(out);
+  for (int k = 0; k < NIN; ++k) vec = vec && aligned16(a.in[k]);
+  const size_t per_tile = size_t(kEwThreads) * kEwUnroll * (vec ? 4 : 1);
+  const size_t tiles = cdiv(n, per_tile);
+  DYHIP_REQUIRE(tiles * bd < (size_t(1) << 31), "elementwise launch too large: %zu tiles x %u batches", tiles, bd);
+  a.tiles_per_batch = static_cast<unsigned>(tiles);
+  const dim3 grid(static_cast<unsigned>(tiles * bd));
+  if (vec)
+    hipLaunchKernelGGL((ew_vec4_kernel<NIN, ACC, BMASK, F>), grid, dim3(kEwThreads), 0, dev->stream, a, f);
+  else
+    hipLaunchKernelGGL((ew_scalar_kernel<NIN, ACC, BMASK, F>), grid, dim3(kEwThreads), 0, dev->stream, a, f);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+// ---- functors -----------------------------------------------------------------
+struct TanhFwd { __device__ float operator()(float x, float, float, float) const { return tanh_accurate(x); } };
+struct LogisticPacketFwd { __device__ float operator()(float x, float, float, float) const { return logistic_packet(x); } };
+struct LogisticScalarFwd { __device__ float operator()(float x, float, float, float) const { return logistic_scalar(x); } };
+struct RectifyFwd { __device__ float operator()(float x, float, float, float) const { return x > 0.f ? x : 0.f; } };
+struct NegateFwd { __device__ float operator()(float x, float, float, float) const { return -x; } };
+struct IdentityFwd { __device__ float operator()(float x, float, float, float) const { return x; } };
+
+// backward functors: (fx, dEdf, -, old) -> old + g(fx, dEdf); the expression
+// order follows the scalar operators of dynet/simd-functors.h:509-544
+struct TanhBwd { __device__ float operator()(float t, float d, float, float o) const { return o + (1.f - t * t) * d; } };
+struct LogisticBwd { __device__ float operator()(float t, float d, float, float o) const { return o + (1.f - t) * t * d; } };
+struct RectifyBwd { __device__ float operator()(float t, float d, float, float o) const { return o + (t != 0.f ? 1.f : 0.f) * d; } };
+struct NegateBwd { __device__ float operator()(float, float d, float, float o) const { return o - d; } };
+
+struct Mul2 { __device__ float operator()(float a, float b, float, float) const { return a * b; } };
+struct Add2 { __device__ float operator()(float a, float b, float, float) const { return a + b; } };
+struct AccMul2 { __device__ float operator()(float a, float b, float, float o) const { return o + a * b; } };
+struct AccIn0 { __device__ float operator()(float a, float, float, float o) const { return o + a; } };
+struct ConstFill {
+  float c;
+  __device__ float operator()(float, float, float, float) const { return c; }
+};
+struct ScaleCopy {
+  float m;
+  __device__ float operator()(float a, float, float, float) const { return a * m; }
+};
+struct SgdStep {  // p -= g * s
+  float s;
+  __device__ float operator()(float g, float, float, float p) const { return p - g * s; }
+};
+
+// Batch reduction used by the broadcast-argument backward (defined in reduce.hip):
+// out[j] (+)= sum_b in0[b*n+j] * (in1 ? in1[b*n+j] : 1)
+int batch_reduce(dyhip_device* dev, size_t n, unsigned bd, const float* in0, const float* in1, float* out,
+                 bool accumulate, void* ws, size_t ws_bytes);
+
+static int check_bd(unsigned bd0, unsigned bd1) {
+  DYHIP_REQUIRE(bd0 >= 1 && bd1 >= 1 && (bd0 == bd1 || bd0 == 1 || bd1 == 1),
+                "batch size must match or equal 1 (got %u and %u)", bd0, bd1);
+  return DYHIP_OK;
+}
+
+template <class F>
+static int binary_forward(dyhip_device* dev, size_t n, unsigned bd0, unsigned bd1, const float* a, const float* b,
+                          float* y, F f) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_CHECK_STATUS(check_bd(bd0, bd1));
+  DYHIP_REQUIRE(n == 0 || (a && b && y), "null tensor pointer");
+  const unsigned bd = bd0 > bd1 ? bd0 : bd1;
+  if (bd0 == bd1) return ew_launch<2, false, 0>(dev, n, bd, a, b, nullptr, y, f);
+  if (bd0 == 1) return ew_launch<2, false, 1>(dev, n, bd, a, b, nullptr, y, f);
+  return ew_launch<2, false, 2>(dev, n, bd, a, b, nullptr, y, f);
+}
+
+}  // namespace dyhip
+
+using namespace dyhip;
+
+extern "C" {
+
+int dyhip_unary_forward(dyhip_device* dev, int op, int logistic_mode, size_t n, const float* x, float* y) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(n == 0 || (x != nullptr && y != nullptr), "null tensor pointer");
+  switch (op) {
+    case DYHIP_OP_TANH: return ew_launch<1, false, 0>(dev, n, 1, x, nullptr, nullptr, y, TanhFwd());
+    case DYHIP_OP_LOGISTIC:
+      if (logistic_mode == DYHIP_LOGISTIC_SCALAR)
+        return ew_launch<1, false, 0>(dev, n, 1, x, nullptr, nullptr, y, LogisticScalarFwd());
+      DYHIP_REQUIRE(logistic_mode == DYHIP_LOGISTIC_PACKET, "unknown logistic mode %d", logistic_mode);
+      return ew_launch<1, false, 0>(dev, n, 1, x, nullptr, nullptr, y, LogisticPacketFwd());
+    case DYHIP_OP_RECTIFY: return ew_launch<1, false, 0>(dev, n, 1, x, nullptr, nullptr, y, RectifyFwd());
+    case DYHIP_OP_NEGATE: return ew_launch<1, false, 0>(dev, n, 1, x, nullptr, nullptr, y, NegateFwd());
+    case DYHIP_OP_IDENTITY: return ew_launch<1, false, 0>(dev, n, 1, x, nullptr, nullptr, y, IdentityFwd());
+    default: return fail(DYHIP_ERR_INVALID_ARG, "unknown unary operator %d", op);
+  }
+}
+
+int dyhip_unary_backward(dyhip_device* dev, int op, size_t n, const float* fx, const float* dEdf, float* dEdx) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(n == 0 || (fx != nullptr && dEdf != nullptr && dEdx != nullptr), "null tensor pointer");
+  switch (op) {
+    case DYHIP_OP_TANH: return ew_launch<2, true, 0>(dev, n, 1, fx, dEdf, nullptr, dEdx, TanhBwd());
+    case DYHIP_OP_LOGISTIC: return ew_launch<2, true, 0>(dev, n, 1, fx, dEdf, nullptr, dEdx, LogisticBwd());
+    case DYHIP_OP_RECTIFY: return ew_launch<2, true, 0>(dev, n, 1, fx, dEdf, nullptr, dEdx, RectifyBwd());
+    case DYHIP_OP_NEGATE: return ew_launch<2, true, 0>(dev, n, 1, fx, dEdf, nullptr, dEdx, NegateBwd());
+    case DYHIP_OP_IDENTITY: return ew_launch<1, true, 0>(dev, n, 1, dEdf, nullptr, nullptr, dEdx, AccIn0());
+    default: return fail(DYHIP_ERR_INVALID_ARG, "unknown unary operator %d", op);
+  }
+}
+
+int dyhip_cmult_forward(dyhip_device* dev, size_t n, unsigned bd0, unsigned bd1, const float* a, const float* b,
+                        float* y) {
+  return binary_forward(dev, n, bd0, bd1, a, b, y, Mul2());
+}
+
+int dyhip_csum_forward(dyhip_device* dev, size_t n, unsigned bd0, unsigned bd1, const float* a, const float* b,
+                       float* y) {
+  return binary_forward(dev, n, bd0, bd1, a, b, y, Add2());
+}
+
+int dyhip_cmult_backward(dyhip_device* dev, size_t n, unsigned bd0, unsigned bd1, const float* a, const float* b,
+                         const float* dEdf, unsigned i, float* dEdxi, void* ws, size_t ws_bytes) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_CHECK_STATUS(check_bd(bd0, bd1));
+  DYHIP_REQUIRE(i < 2, "CwiseMultiply has two arguments (i = %u)", i);
+  DYHIP_REQUIRE(n == 0 || (a && b && dEdf && dEdxi), "null tensor pointer");
+  const unsigned bd = bd0 > bd1 ? bd0 : bd1;
+  const float* other = i == 0 ? b : a;
+  const unsigned bd_other = i == 0 ? bd1 : bd0;
+  const unsigned bd_self = i == 0 ? bd0 : bd1;
+  if (bd_self == bd) {
+    if (bd_other == bd) return ew_launch<2, true, 0>(dev, n, bd, dEdf, other, nullptr, dEdxi, AccMul2());
+    return ew_launch<2, true, 2>(dev, n, bd, dEdf, other, nullptr, dEdxi, AccMul2());
+  }
+  // this argument was broadcast over the batch: dxi += sum_b dy * other
+  return batch_reduce(dev, n, bd, dEdf, other, dEdxi, true, ws, ws_bytes);
+}
+
+int dyhip_csum_backward(dyhip_device* dev, size_t n, unsigned bd0, unsigned bd1, const float* dEdf, unsigned i,
+                        float* dEdxi, void* ws, size_t ws_bytes) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_CHECK_STATUS(check_bd(bd0, bd1));
+  DYHIP_REQUIRE(i < 2, "CwiseSum has two arguments (i = %u)", i);
+  DYHIP_REQUIRE(n == 0 || (dEdf && dEdxi), "null tensor pointer");
+  const unsigned bd = bd0 > bd1 ? bd0 : bd1;
+  const unsigned bd_self = i == 0 ? bd0 : bd1;
+  if (bd_self == bd) return ew_launch<1, true, 0>(dev, n, bd, dEdf, nullptr, nullptr, dEdxi, AccIn0());
+  return batch_reduce(dev, n, bd, dEdf, nullptr, dEdxi, true, ws, ws_bytes);
+}
+
+int dyhip_sum_batches_backward(dyhip_device* dev, size_t n, unsigned bd, const float* dEdf, float* dEdx) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(n == 0 || bd == 0 || (dEdf && dEdx), "null tensor pointer");
+  return ew_launch<1, true, 1>(dev, n, bd, dEdf, nullptr, nullptr, dEdx, AccIn0());
+}
+
+int dyhip_constant(dyhip_device* dev, size_t n, float value, float* dst) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(n == 0 || dst, "null tensor pointer");
+  return ew_launch<0, false, 0>(dev, n, 1, nullptr, nullptr, nullptr, dst, ConstFill{value});
+}
+
+int dyhip_accumulate(dyhip_device* dev, size_t n, const float* src, float* dst) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(n == 0 || (src && dst), "null tensor pointer");
+  return ew_launch<1, true, 0>(dev, n, 1, src, nullptr, nullptr, dst, AccIn0());
+}
+
+int dyhip_scale_copy(dyhip_device* dev, size_t n, const float* src, float mult, float* dst) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(n == 0 || (src && dst), "null tensor pointer");
+  if (mult == 1.0f) return ew_launch<1, false, 0>(dev, n, 1, src, nullptr, nullptr, dst, IdentityFwd());
+  return ew_launch<1, false, 0>(dev, n, 1, src, nullptr, nullptr, dst, ScaleCopy{mult});
+}
+
+int dyhip_sgd_update(dyhip_device* dev, size_t n, float* p, const float* g, float lr, float gscale, float wd) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(n == 0 || (p && g), "null tensor pointer");
+  DYHIP_REQUIRE(wd != 0.f, "weight decay scale must be non-zero");
+  return ew_launch<1, true, 0>(dev, n, 1, g, nullptr, nullptr, p, SgdStep{lr * gscale / wd});
+}
+
+}  // extern "C"

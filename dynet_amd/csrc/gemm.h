@@ -1,0 +1,41 @@
+// Internal interface of the fp32 MFMA GEMM (gemm.hip), shared with the fused
+// LSTM gate launcher.
+#pragma once
+
+#include "common.h"
+
+namespace dyhip {
+
+// One K-segment of a GEMM: C += op(A) * op(B) over this segment's K.
+//   a_kmajor == false : A(i,k) = A[i + k*lda]   (contiguous along the output row index)
+//   a_kmajor == true  : A(i,k) = A[k + i*lda]   (contiguous along K, i.e. a transposed operand)
+//   b_kmajor == true  : B(k,j) = B[k + j*ldb]
+//   b_kmajor == false : B(k,j) = B[j + k*ldb]
+struct GemmSeg {
+  const float* A;
+  size_t lda;
+  const float* B;
+  size_t ldb;
+  size_t K;
+};
+
+constexpr int kGemmMaxSeg = 2;
+
+enum GemmEpilogue {
+  kEpiAxpby = 0,      // C = beta*C + sum
+  kEpiLstmGates = 1   // C = act(bias[i] + (H <= i < 2H ? 1 : 0) + sum), logistic rows [0,3H), tanh rows [3H,4H)
+};
+
+struct GemmEpiParams {
+  int kind;
+  float beta;
+  const float* bias;  // kEpiLstmGates
+  unsigned H;         // kEpiLstmGates
+  int logistic_mode;  // kEpiLstmGates
+};
+
+// C is M x N column-major (ldc = M).  Segments share the operand layouts.
+int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N, int nseg, const GemmSeg* segs,
+             float* C, const GemmEpiParams& epi);
+
+}  // namespace dyhip

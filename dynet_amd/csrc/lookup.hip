@@ -1,0 +1,309 @@
+// LookupNode: embedding gather and sorted-index segmented scatter-add.
+//
+// Replaces LookupNode::forward_dev_impl (dynet/param-nodes.cc:304-329) with its
+// one-thread-per-float gather (dynet/gpu-ops.cu:72-90, a division and a modulo
+// per element) and LookupParameterStorage::accumulate_grads_dev
+// (dynet/model.cc:728-743) with its float atomicAdd scatter
+// (dynet/gpu-ops.cu:148-166, order-dependent and serialising on hot rows).
+//
+// Layout: the table is dim x vocab column-major, i.e. row r of the embedding is
+// the contiguous run table[r*dim, (r+1)*dim); fx and g are dim x n_ids.
+//
+// Scatter-add: (id, position) pairs are radix-sorted by id (stable, so equal
+// ids keep ascending position).  The sorted sequence is cut into chunks of
+// kChunk entries; one thread group per chunk walks its entries in order and
+// sums runs of equal ids in registers.  A run that lies inside one chunk is
+// added straight into its gradient row (the chunk is the only writer of that
+// row).  A run that crosses chunk boundaries leaves one partial row per chunk
+// in the workspace, and a second kernel adds the partials of each such run in
+// ascending chunk order.  No atomics anywhere: the result is deterministic and
+// each gradient row is read and written exactly once.
+#include <cstring>
+
+#include <rocprim/rocprim.hpp>
+
+#include "common.h"
+
+namespace dyhip {
+
+constexpr unsigned kNone = 0xFFFFFFFFu;
+constexpr int kChunk = 16;
+constexpr int kLkThreads = 256;
+constexpr int kGatherRowsUnroll = 4;
+
+template <class V>
+__device__ __forceinline__ V vzero();
+template <>
+__device__ __forceinline__ float4 vzero<float4>() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+template <>
+__device__ __forceinline__ float vzero<float>() { return 0.f; }
+__device__ __forceinline__ float4 vadd(const float4 a, const float4 b) {
+  return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w);
+}
+__device__ __forceinline__ float vadd(const float a, const float b) { return a + b; }
+__device__ __forceinline__ float4 vscale(const float4 a, const float m) {
+  return make_float4(a.x * m, a.y * m, a.z * m, a.w * m);
+}
+__device__ __forceinline__ float vscale(const float a, const float m) { return a * m; }
+
+// ---- gather ---------------------------------------------------------------------
+// A group of `tpr` threads owns one id at a time; a block holds 256/tpr groups and
+// each group processes kGatherRowsUnroll ids with all loads issued first.
+template <class V, bool SCALE>
+__global__ __launch_bounds__(kLkThreads) void lookup_gather_kernel(unsigned n_ids, unsigned dimv, unsigned tpr,
+                                                                   unsigned vocab, const unsigned* __restrict__ ids,
+                                                                   const V* __restrict__ table, float mult,
+                                                                   V* __restrict__ fx) {
+  const unsigned groups = kLkThreads / tpr;
+  const unsigned grp = threadIdx.x / tpr, t = threadIdx.x - grp * tpr;
+  const unsigned row0 = (blockIdx.x * groups + grp) * kGatherRowsUnroll;
+  unsigned id[kGatherRowsUnroll];
+#pragma unroll
+  for (int u = 0; u < kGatherRowsUnroll; ++u) id[u] = row0 + u < n_ids ? ids[row0 + u] : kNone;
+  for (unsigned c = t; c < dimv; c += tpr) {
+    V v[kGatherRowsUnroll];
+#pragma unroll
+    for (int u = 0; u < kGatherRowsUnroll; ++u)
+      v[u] = (row0 + u < n_ids && id[u] < vocab) ? table[size_t(id[u]) * dimv + c] : vzero<V>();
+#pragma unroll
+    for (int u = 0; u < kGatherRowsUnroll; ++u)
+      if (row0 + u < n_ids) fx[size_t(row0 + u) * dimv + c] = SCALE ? vscale(v[u], mult) : v[u];
+  }
+}
+
+// ---- segmented scatter-add --------------------------------------------------------
+struct ScatterWs {
+  unsigned* sorted_ids;
+  unsigned* sorted_pos;
+  unsigned* first_row;   // per chunk: row of a first run that began in an earlier chunk, else kNone
+  unsigned* first_cont;  // per chunk: 1 if that run also continues into the next chunk
+  unsigned* last_row;    // per chunk: row of a run that begins here and continues into the next chunk
+  float* part_first;     // [chunks][dim]
+  float* part_last;      // [chunks][dim]
+  void* sort_tmp;
+  size_t sort_tmp_bytes;
+  unsigned chunks;
+};
+
+template <class V>
+__global__ __launch_bounds__(kLkThreads) void scatter_chunk_kernel(unsigned n, unsigned dimv, unsigned tpr,
+                                                                   unsigned vocab, ScatterWs w,
+                                                                   const V* __restrict__ g, V* __restrict__ grads) {
+  const unsigned groups = kLkThreads / tpr;
+  const unsigned grp = threadIdx.x / tpr, t = threadIdx.x - grp * tpr;
+  const unsigned ch = blockIdx.x * groups + grp;
+  if (ch >= w.chunks) return;
+  const unsigned k0 = ch * kChunk;
+  const unsigned cnt = min(n - k0, (unsigned)kChunk);
+  unsigned id[kChunk], pos[kChunk];
+#pragma unroll
+  for (int k = 0; k < kChunk; ++k) {
+    id[k] = k < (int)cnt ? w.sorted_ids[k0 + k] : kNone;
+    pos[k] = k < (int)cnt ? w.sorted_pos[k0 + k] : 0u;
+  }
+  const unsigned prev_id = k0 > 0 ? w.sorted_ids[k0 - 1] : kNone;
+  const unsigned next_id = k0 + cnt < n ? w.sorted_ids[k0 + cnt] : kNone;
+  const unsigned first = id[0], last = id[cnt - 1];
+  const bool single = first == last;
+  const bool open_left = prev_id == first;
+  const bool open_right = next_id == last;
+  if (t == 0) {
+    w.first_row[ch] = open_left ? first : kNone;
+    w.first_cont[ch] = (open_left && single && open_right) ? 1u : 0u;
+    w.last_row[ch] = (open_right && !(single && open_left)) ? last : kNone;
+  }
+  V* part_first = reinterpret_cast<V*>(w.part_first) + size_t(ch) * dimv;
+  V* part_last = reinterpret_cast<V*>(w.part_last) + size_t(ch) * dimv;
+  for (unsigned c = t; c < dimv; c += tpr) {
+    V v[kChunk];
+#pragma unroll
+    for (int k = 0; k < kChunk; ++k) v[k] = k < (int)cnt ? g[size_t(pos[k]) * dimv + c] : vzero<V>();
+    V acc = vzero<V>();
+    unsigned cur = first;
+    // flush the finished run of row `cur`: into a partial if the run crosses a
+    // chunk boundary, else straight into the gradient row (sole writer)
+    auto flush = [&](bool end) {
+      if (open_left && cur == first)
+        part_first[c] = acc;
+      else if (end && open_right)
+        part_last[c] = acc;
+      else if (cur < vocab)
+        grads[size_t(cur) * dimv + c] = vadd(grads[size_t(cur) * dimv + c], acc);
+    };
+#pragma unroll
+    for (int k = 0; k < kChunk; ++k) {
+      if (k < (int)cnt) {
+        if (id[k] != cur) {
+          flush(false);
+          cur = id[k];
+          acc = vzero<V>();
+        }
+        acc = vadd(acc, v[k]);
+      }
+    }
+    flush(true);
+  }
+}
+
+// One thread group per chunk where a boundary-crossing run starts: add its
+// partials in ascending chunk order, then one read-modify-write of the row.
+template <class V>
+__global__ __launch_bounds__(kLkThreads) void scatter_fixup_kernel(unsigned dimv, unsigned tpr, unsigned vocab,
+                                                                   ScatterWs w, V* __restrict__ grads) {
+  const unsigned groups = kLkThreads / tpr;
+  const unsigned grp = threadIdx.x / tpr, t = threadIdx.x - grp * tpr;
+  const unsigned c0 = blockIdx.x * groups + grp;
+  if (c0 >= w.chunks) return;
+  const unsigned row = w.last_row[c0];
+  if (row == kNone || row >= vocab) return;
+  unsigned c1 = c0 + 1;  // one past the last chunk of the run
+  while (c1 < w.chunks && w.first_row[c1] == row) {
+    const bool cont = w.first_cont[c1] != 0;
+    ++c1;
+    if (!cont) break;
+  }
+  const V* pl = reinterpret_cast<const V*>(w.part_last) + size_t(c0) * dimv;
+  const V* pf = reinterpret_cast<const V*>(w.part_first);
+  for (unsigned c = t; c < dimv; c += tpr) {
+    V acc = pl[c];
+    for (unsigned k = c0 + 1; k < c1; ++k) acc = vadd(acc, pf[size_t(k) * dimv + c]);
+    grads[size_t(row) * dimv + c] = vadd(grads[size_t(row) * dimv + c], acc);
+  }
+}
+
+static unsigned threads_per_row(size_t dimv) {
+  unsigned t = 16;
+  while (t < kLkThreads && t < dimv) t <<= 1;
+  return t;
+}
+
+static unsigned key_bits(unsigned vocab) {
+  unsigned bits = 1;
+  while (bits < 32 && (1ull << bits) < (unsigned long long)vocab) ++bits;
+  return bits;
+}
+
+static size_t align256(size_t n) { return (n + 255) / 256 * 256; }
+
+static int sort_tmp_bytes(unsigned n, unsigned vocab, size_t* bytes) {
+  size_t tmp = 0;
+  unsigned* k = nullptr;
+  hipError_t e = rocprim::radix_sort_pairs(nullptr, tmp, static_cast<const unsigned*>(k), k,
+                                           rocprim::counting_iterator<unsigned>(0), k, n, 0, key_bits(vocab));
+  if (e != hipSuccess) return fail(DYHIP_ERR_RUNTIME, "radix sort size query failed: %s", hipGetErrorString(e));
+  *bytes = tmp;
+  return DYHIP_OK;
+}
+
+static int carve(unsigned n, size_t dim, unsigned vocab, void* ws, size_t ws_bytes, ScatterWs* out, size_t* need) {
+  const unsigned chunks = cdiv<unsigned>(n, kChunk);
+  size_t sort_bytes = 0;
+  DYHIP_CHECK_STATUS(sort_tmp_bytes(n, vocab, &sort_bytes));
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    size_t o = off;
+    off += align256(bytes);
+    return o;
+  };
+  const size_t o_ids = take(sizeof(unsigned) * n), o_pos = take(sizeof(unsigned) * n);
+  const size_t o_fr = take(sizeof(unsigned) * chunks), o_fc = take(sizeof(unsigned) * chunks),
+               o_lr = take(sizeof(unsigned) * chunks);
+  const size_t o_pf = take(sizeof(float) * dim * chunks), o_pl = take(sizeof(float) * dim * chunks);
+  const size_t o_tmp = take(sort_bytes);
+  if (need) *need = off;
+  if (out) {
+    if (ws == nullptr || ws_bytes < off)
+      return fail(DYHIP_ERR_INVALID_ARG, "lookup scatter-add needs %zu workspace bytes, got %zu", off, ws_bytes);
+    if (!aligned16(ws)) return fail(DYHIP_ERR_INVALID_ARG, "lookup scatter-add workspace must be 16-byte aligned");
+    char* base = static_cast<char*>(ws);
+    out->sorted_ids = reinterpret_cast<unsigned*>(base + o_ids);
+    out->sorted_pos = reinterpret_cast<unsigned*>(base + o_pos);
+    out->first_row = reinterpret_cast<unsigned*>(base + o_fr);
+    out->first_cont = reinterpret_cast<unsigned*>(base + o_fc);
+    out->last_row = reinterpret_cast<unsigned*>(base + o_lr);
+    out->part_first = reinterpret_cast<float*>(base + o_pf);
+    out->part_last = reinterpret_cast<float*>(base + o_pl);
+    out->sort_tmp = base + o_tmp;
+    out->sort_tmp_bytes = sort_bytes;
+    out->chunks = chunks;
+  }
+  return DYHIP_OK;
+}
+
+}  // namespace dyhip
+
+using namespace dyhip;
+
+extern "C" {
+
+int dyhip_lookup_forward(dyhip_device* dev, unsigned n_ids, const unsigned* ids_host, unsigned* ids_dev, size_t dim,
+                         unsigned vocab, const float* table, float mult, float* fx) {
+  DYHIP_CHECK_DEV(dev);
+  if (n_ids == 0 || dim == 0) return DYHIP_OK;
+  DYHIP_REQUIRE(ids_dev && table && fx, "null pointer in lookup");
+  DYHIP_REQUIRE(dim < (size_t(1) << 31), "lookup dimension too large");
+  if (ids_host != nullptr) {
+    for (unsigned b = 0; b < n_ids; ++b)
+      DYHIP_REQUIRE(ids_host[b] < vocab, "Out-of-bounds attempt to access index %u for LookupParameter of size %u",
+                    ids_host[b], vocab);
+    DYHIP_CHECK_HIP(hipMemcpyAsync(ids_dev, ids_host, sizeof(unsigned) * n_ids, hipMemcpyHostToDevice, dev->stream));
+    DYHIP_CHECK_HIP(hipStreamSynchronize(dev->stream));  // ids_host may be released by the caller on return
+  }
+  const bool vec = dim % 4 == 0 && aligned16(table) && aligned16(fx);
+  const unsigned dimv = static_cast<unsigned>(vec ? dim / 4 : dim);
+  const unsigned tpr = threads_per_row(dimv);
+  const unsigned rows_per_block = (kLkThreads / tpr) * kGatherRowsUnroll;
+  const dim3 grid(cdiv<unsigned>(n_ids, rows_per_block)), block(kLkThreads);
+#define DYHIP_GATHER(V, SCALE)                                                                                \
+  hipLaunchKernelGGL((lookup_gather_kernel<V, SCALE>), grid, block, 0, dev->stream, n_ids, dimv, tpr, vocab, \
+                     ids_dev, reinterpret_cast<const V*>(table), mult, reinterpret_cast<V*>(fx))
+  if (vec) {
+    if (mult == 1.0f) DYHIP_GATHER(float4, false); else DYHIP_GATHER(float4, true);
+  } else {
+    if (mult == 1.0f) DYHIP_GATHER(float, false); else DYHIP_GATHER(float, true);
+  }
+#undef DYHIP_GATHER
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_lookup_accumulate_grads_workspace(unsigned n_ids, size_t dim, unsigned vocab, size_t* ws_bytes) {
+  DYHIP_REQUIRE(ws_bytes != nullptr, "null output pointer");
+  if (n_ids == 0 || dim == 0) {
+    *ws_bytes = 0;
+    return DYHIP_OK;
+  }
+  return carve(n_ids, dim, vocab, nullptr, 0, nullptr, ws_bytes);
+}
+
+int dyhip_lookup_accumulate_grads(dyhip_device* dev, unsigned n_ids, const unsigned* ids_dev, size_t dim,
+                                  unsigned vocab, const float* g, float* all_grads, void* ws, size_t ws_bytes) {
+  DYHIP_CHECK_DEV(dev);
+  if (n_ids == 0 || dim == 0) return DYHIP_OK;
+  DYHIP_REQUIRE(ids_dev && g && all_grads, "null pointer in lookup accumulate_grads");
+  DYHIP_REQUIRE(dim < (size_t(1) << 31), "lookup dimension too large");
+  ScatterWs w;
+  DYHIP_CHECK_STATUS(carve(n_ids, dim, vocab, ws, ws_bytes, &w, nullptr));
+  size_t tmp_bytes = w.sort_tmp_bytes;
+  DYHIP_CHECK_HIP(rocprim::radix_sort_pairs(w.sort_tmp, tmp_bytes, ids_dev, w.sorted_ids,
+                                            rocprim::counting_iterator<unsigned>(0), w.sorted_pos, n_ids, 0,
+                                            key_bits(vocab), dev->stream));
+  const bool vec = dim % 4 == 0 && aligned16(g) && aligned16(all_grads);
+  const unsigned dimv = static_cast<unsigned>(vec ? dim / 4 : dim);
+  const unsigned tpr = threads_per_row(dimv);
+  const dim3 grid(cdiv<unsigned>(w.chunks, kLkThreads / tpr)), block(kLkThreads);
+  if (vec) {
+    hipLaunchKernelGGL(scatter_chunk_kernel<float4>, grid, block, 0, dev->stream, n_ids, dimv, tpr, vocab, w,
+                       reinterpret_cast<const float4*>(g), reinterpret_cast<float4*>(all_grads));
+    hipLaunchKernelGGL(scatter_fixup_kernel<float4>, grid, block, 0, dev->stream, dimv, tpr, vocab, w,
+                       reinterpret_cast<float4*>(all_grads));
+  } else {
+    hipLaunchKernelGGL(scatter_chunk_kernel<float>, grid, block, 0, dev->stream, n_ids, dimv, tpr, vocab, w, g,
+                       all_grads);
+    hipLaunchKernelGGL(scatter_fixup_kernel<float>, grid, block, 0, dev->stream, dimv, tpr, vocab, w, all_grads);
+  }
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,324 @@
+// Fused LSTM nodes: VanillaLSTMGates, VanillaLSTMC, VanillaLSTMH
+// (dynet/nodes-lstm.cc:101-235, 237-527, 562-615, 650-703).
+//
+// Gates forward is ONE GEMM launch over two K segments ([Wx | Wh] * [x ; h])
+// whose epilogue adds the bias and the +1 forget bias and applies logistic to
+// rows [0,3H) and tanh to rows [3H,4H) -- the reference issues a broadcast, a
+// slice add, two cuBLAS calls and six slice/activation launches for the same
+// result.  Backward computes dpre = dEdf * act'(fx) once per call (or takes it
+// precomputed) and feeds the transposed GEMM forms; the bias gradient is a
+// batch reduction.  C and H are single elementwise kernels each way (the
+// reference copies gate slices to scratch first).
+//
+// Layout: gates is 4H x B column-major, gate order i, f, o, g; c, h are H x B.
+#include "gemm.h"
+
+namespace dyhip {
+
+int batch_reduce(dyhip_device* dev, size_t n, unsigned bd, const float* in0, const float* in1, float* out,
+                 bool accumulate, void* ws, size_t ws_bytes);
+
+static size_t align256(size_t n) { return (n + 255) / 256 * 256; }
+
+// dst[b*dst_ld + off + r] = src[b*rows + r] * (mask ? mask[(mask_b ? b : 0)*dst_ld + off + r] : 1)
+__global__ __launch_bounds__(256) void rows_copy_mask_kernel(unsigned rows, unsigned dst_ld, unsigned off,
+                                                             const float* __restrict__ src,
+                                                             const float* __restrict__ mask, int mask_b,
+                                                             float* __restrict__ dst) {
+  const unsigned r = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
+  if (r >= rows) return;
+  float v = src[size_t(b) * rows + r];
+  if (mask) v *= mask[size_t(mask_b ? b : 0) * dst_ld + off + r];
+  dst[size_t(b) * dst_ld + off + r] = v;
+}
+
+// out[b*rows + r] += tmp[b*rows + r] * mask[(mask_b ? b : 0)*mask_ld + off + r]
+__global__ __launch_bounds__(256) void acc_mul_mask_kernel(unsigned rows, unsigned mask_ld, unsigned off,
+                                                           const float* __restrict__ tmp,
+                                                           const float* __restrict__ mask, int mask_b,
+                                                           float* __restrict__ out) {
+  const unsigned r = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
+  if (r >= rows) return;
+  out[size_t(b) * rows + r] += tmp[size_t(b) * rows + r] * mask[size_t(mask_b ? b : 0) * mask_ld + off + r];
+}
+
+// dpre[i, b] = i < 3H ? d*f*(1-f) : d*(1-f*f)      (dynet/nodes-lstm.cc:358-361)
+__global__ __launch_bounds__(256) void lstm_dpre_kernel(unsigned H, const float* __restrict__ fx,
+                                                        const float* __restrict__ dEdf, float* __restrict__ dpre) {
+  const unsigned i = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
+  if (i >= 4 * H) return;
+  const size_t e = size_t(b) * 4 * H + i;
+  const float f = fx[e], d = dEdf[e];
+  dpre[e] = i < 3 * H ? d * f * (1.f - f) : d * (1.f - f * f);
+}
+
+// mode 0: c = i*g + f*c_prev                                   (C forward, :562-589)
+// mode 1: dc_prev += dc*f                                      (C backward i=0, :605-606)
+// mode 2: di += dc*g; df += dc*c_prev; dg += dc*i              (C backward i=1, :607-614)
+// mode 3: h = o*tanh(c)                                        (H forward, :650-668)
+// mode 4: dc += dh*o*(1 - tanh(c)^2)                           (H backward i=0, :684-694)
+// mode 5: do += dh*tanh(c)                                     (H backward i=1, :695-701)
+// `state` is c_prev (modes 0-2) or c (modes 3-5); `d` is dEdf for the backward modes.
+template <int MODE>
+__global__ __launch_bounds__(256) void lstm_pointwise_kernel(unsigned H, const float* __restrict__ state,
+                                                             const float* __restrict__ gates,
+                                                             const float* __restrict__ d, float* __restrict__ out) {
+  const unsigned r = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
+  if (r >= H) return;
+  const size_t s = size_t(b) * H + r;
+  const float* gt = gates + size_t(b) * 4 * H;
+  if (MODE == 0) {
+    out[s] = gt[r] * gt[3 * H + r] + gt[H + r] * state[s];
+  } else if (MODE == 1) {
+    out[s] += d[s] * gt[H + r];
+  } else if (MODE == 2) {
+    float* dg = out + size_t(b) * 4 * H;
+    const float dc = d[s];
+    dg[r] += dc * gt[3 * H + r];
+    dg[H + r] += dc * state[s];
+    dg[3 * H + r] += dc * gt[r];
+  } else if (MODE == 3) {
+    out[s] = gt[2 * H + r] * tanh_accurate(state[s]);
+  } else if (MODE == 4) {
+    const float t = tanh_accurate(state[s]);
+    out[s] += d[s] * gt[2 * H + r] * (1.f - t * t);
+  } else {
+    out[size_t(b) * 4 * H + 2 * H + r] += d[s] * tanh_accurate(state[s]);
+  }
+}
+
+template <int MODE>
+static int launch_pointwise(dyhip_device* dev, unsigned H, unsigned B, const float* state, const float* gates,
+                            const float* d, float* out) {
+  if (H == 0 || B == 0) return DYHIP_OK;
+  DYHIP_REQUIRE(B <= 65535, "LSTM nodes support at most 65535 batch elements per call");
+  hipLaunchKernelGGL(lstm_pointwise_kernel<MODE>, dim3(cdiv<unsigned>(H, 256), B), dim3(256), 0, dev->stream, H, state,
+                     gates, d, out);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+struct GatesInputs {
+  unsigned I;
+  bool dropout;
+};
+
+static int check_gates(unsigned num_inputs, const float* const* xs, const unsigned* x_dims, unsigned H, unsigned B,
+                       const float* mask_x, unsigned mask_x_bd, const float* mask_h, unsigned mask_h_bd,
+                       GatesInputs* out) {
+  DYHIP_REQUIRE(num_inputs >= 1 && xs != nullptr && x_dims != nullptr, "Failed input count check in VanillaLSTMGates");
+  DYHIP_REQUIRE(H >= 1 && B >= 1 && B <= 65535, "VanillaLSTMGates: bad hidden (%u) or batch (%u) size", H, B);
+  unsigned I = 0;
+  for (unsigned k = 0; k < num_inputs; ++k) {
+    DYHIP_REQUIRE(xs[k] != nullptr && x_dims[k] >= 1, "VanillaLSTMGates: x_t[%u] expected to be a vector", k);
+    I += x_dims[k];
+  }
+  DYHIP_REQUIRE((mask_x == nullptr) == (mask_h == nullptr), "VanillaLSTMGates: both dropout masks or none");
+  out->dropout = mask_x != nullptr;
+  if (out->dropout) {
+    DYHIP_REQUIRE(mask_x_bd == B || mask_x_bd == 1,
+                  "VanillaLSTMGates: dropout_mask_x expected to have batch size 1 or %u, was %u", B, mask_x_bd);
+    DYHIP_REQUIRE(mask_h_bd == B || mask_h_bd == 1,
+                  "VanillaLSTMGates: dropout_mask_h expected to have batch size 1 or %u, was %u", B, mask_h_bd);
+  }
+  out->I = I;
+  return DYHIP_OK;
+}
+
+// Builds the effective x_t (concatenated and/or masked) in `buf` when needed;
+// returns the pointer the GEMM should read.
+static int prepare_x(dyhip_device* dev, unsigned num_inputs, const float* const* xs, const unsigned* x_dims,
+                     unsigned I, unsigned B, const float* mask_x, unsigned mask_x_bd, float* buf,
+                     const float** x_eff) {
+  if (num_inputs == 1 && mask_x == nullptr) {
+    *x_eff = xs[0];
+    return DYHIP_OK;
+  }
+  unsigned off = 0;
+  for (unsigned k = 0; k < num_inputs; ++k) {
+    hipLaunchKernelGGL(rows_copy_mask_kernel, dim3(cdiv<unsigned>(x_dims[k], 256), B), dim3(256), 0, dev->stream,
+                       x_dims[k], I, off, xs[k], mask_x, mask_x_bd > 1 ? 1 : 0, buf);
+    off += x_dims[k];
+  }
+  DYHIP_CHECK_LAUNCH();
+  *x_eff = buf;
+  return DYHIP_OK;
+}
+
+static int prepare_h(dyhip_device* dev, unsigned H, unsigned B, const float* h, const float* mask_h,
+                     unsigned mask_h_bd, float* buf, const float** h_eff) {
+  if (mask_h == nullptr) {
+    *h_eff = h;
+    return DYHIP_OK;
+  }
+  hipLaunchKernelGGL(rows_copy_mask_kernel, dim3(cdiv<unsigned>(H, 256), B), dim3(256), 0, dev->stream, H, H, 0u, h,
+                     mask_h, mask_h_bd > 1 ? 1 : 0, buf);
+  DYHIP_CHECK_LAUNCH();
+  *h_eff = buf;
+  return DYHIP_OK;
+}
+
+}  // namespace dyhip
+
+using namespace dyhip;
+
+extern "C" {
+
+int dyhip_lstm_gates_workspace(unsigned num_inputs, unsigned I, unsigned H, unsigned B, int dropout,
+                               size_t* ws_bytes) {
+  DYHIP_REQUIRE(ws_bytes != nullptr, "null output pointer");
+  size_t n = 0;
+  if (num_inputs > 1 || dropout) n += align256(sizeof(float) * size_t(I) * B);
+  if (dropout) n += align256(sizeof(float) * size_t(H) * B);
+  *ws_bytes = n;
+  return DYHIP_OK;
+}
+
+int dyhip_lstm_gates_forward(dyhip_device* dev, unsigned num_inputs, const float* const* xs_host,
+                             const unsigned* x_dims_host, unsigned H, unsigned B, const float* h_tm1,
+                             const float* Wx, const float* Wh, const float* b, const float* mask_x,
+                             unsigned mask_x_bd, const float* mask_h, unsigned mask_h_bd, int logistic_mode,
+                             float* fx, void* ws, size_t ws_bytes) {
+  DYHIP_CHECK_DEV(dev);
+  GatesInputs gi;
+  DYHIP_CHECK_STATUS(check_gates(num_inputs, xs_host, x_dims_host, H, B, mask_x, mask_x_bd, mask_h, mask_h_bd, &gi));
+  DYHIP_REQUIRE(h_tm1 && Wx && Wh && b && fx, "VanillaLSTMGates: null tensor pointer");
+  DYHIP_REQUIRE(logistic_mode == DYHIP_LOGISTIC_PACKET || logistic_mode == DYHIP_LOGISTIC_SCALAR,
+                "unknown logistic mode %d", logistic_mode);
+  size_t need = 0;
+  DYHIP_CHECK_STATUS(dyhip_lstm_gates_workspace(num_inputs, gi.I, H, B, gi.dropout, &need));
+  DYHIP_REQUIRE(need == 0 || (ws != nullptr && ws_bytes >= need), "VanillaLSTMGates needs %zu workspace bytes, got %zu",
+                need, ws_bytes);
+  char* wsp = static_cast<char*>(ws);
+  float* xbuf = reinterpret_cast<float*>(wsp);
+  float* hbuf = reinterpret_cast<float*>(wsp + ((num_inputs > 1 || gi.dropout) ? align256(sizeof(float) * size_t(gi.I) * B) : 0));
+  const float *x_eff = nullptr, *h_eff = nullptr;
+  DYHIP_CHECK_STATUS(prepare_x(dev, num_inputs, xs_host, x_dims_host, gi.I, B, mask_x, mask_x_bd, xbuf, &x_eff));
+  DYHIP_CHECK_STATUS(prepare_h(dev, H, B, h_tm1, mask_h, mask_h_bd, hbuf, &h_eff));
+  const size_t G = size_t(4) * H;
+  GemmSeg segs[2] = {{Wx, G, x_eff, gi.I, gi.I}, {Wh, G, h_eff, H, H}};
+  GemmEpiParams ep{kEpiLstmGates, 0.f, b, H, logistic_mode};
+  return gemm_run(dev, false, true, G, B, 2, segs, fx, ep);
+}
+
+int dyhip_lstm_gates_dpre(dyhip_device* dev, unsigned H, unsigned B, const float* fx, const float* dEdf,
+                          float* dpre) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(fx && dEdf && dpre, "null tensor pointer");
+  if (H == 0 || B == 0) return DYHIP_OK;
+  DYHIP_REQUIRE(B <= 65535, "LSTM nodes support at most 65535 batch elements per call");
+  hipLaunchKernelGGL(lstm_dpre_kernel, dim3(cdiv<unsigned>(4 * H, 256), B), dim3(256), 0, dev->stream, H, fx, dEdf,
+                     dpre);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_lstm_gates_backward_workspace(unsigned num_inputs, unsigned I, unsigned H, unsigned B, int dropout,
+                                        size_t* ws_bytes) {
+  DYHIP_REQUIRE(ws_bytes != nullptr, "null output pointer");
+  (void)num_inputs;
+  (void)dropout;
+  const unsigned big = I > H ? I : H;
+  size_t red = 0;
+  DYHIP_CHECK_STATUS(dyhip_batch_reduce_workspace(size_t(4) * H, B, &red));
+  *ws_bytes = align256(sizeof(float) * size_t(4) * H * B) + align256(sizeof(float) * size_t(big) * B) + align256(red);
+  return DYHIP_OK;
+}
+
+int dyhip_lstm_gates_backward(dyhip_device* dev, unsigned num_inputs, const float* const* xs_host,
+                              const unsigned* x_dims_host, unsigned H, unsigned B, const float* h_tm1,
+                              const float* Wx, const float* Wh, const float* mask_x, unsigned mask_x_bd,
+                              const float* mask_h, unsigned mask_h_bd, const float* fx, const float* dEdf,
+                              const float* dpre, unsigned i, float* dEdxi, void* ws, size_t ws_bytes) {
+  DYHIP_CHECK_DEV(dev);
+  GatesInputs gi;
+  DYHIP_CHECK_STATUS(check_gates(num_inputs, xs_host, x_dims_host, H, B, mask_x, mask_x_bd, mask_h, mask_h_bd, &gi));
+  DYHIP_REQUIRE(i <= num_inputs + 3, "VanillaLSTMGates has %u differentiable arguments (i = %u)", num_inputs + 4, i);
+  DYHIP_REQUIRE(h_tm1 && Wx && Wh && fx && dEdf && dEdxi, "VanillaLSTMGates: null tensor pointer");
+  size_t need = 0;
+  DYHIP_CHECK_STATUS(dyhip_lstm_gates_backward_workspace(num_inputs, gi.I, H, B, gi.dropout, &need));
+  DYHIP_REQUIRE(ws != nullptr && ws_bytes >= need, "VanillaLSTMGates backward needs %zu workspace bytes, got %zu", need,
+                ws_bytes);
+  const size_t G = size_t(4) * H;
+  const unsigned big = gi.I > H ? gi.I : H;
+  char* wsp = static_cast<char*>(ws);
+  float* dpre_buf = reinterpret_cast<float*>(wsp);
+  float* tmp = reinterpret_cast<float*>(wsp + align256(sizeof(float) * G * B));
+  char* red_ws = wsp + align256(sizeof(float) * G * B) + align256(sizeof(float) * size_t(big) * B);
+  const size_t red_bytes = ws_bytes - (red_ws - wsp);
+  if (dpre == nullptr) {
+    DYHIP_CHECK_STATUS(dyhip_lstm_gates_dpre(dev, H, B, fx, dEdf, dpre_buf));
+    dpre = dpre_buf;
+  }
+  const GemmEpiParams acc{kEpiAxpby, 1.0f, nullptr, 0, 0}, ovw{kEpiAxpby, 0.0f, nullptr, 0, 0};
+  if (i <= num_inputs) {
+    // dx_i += Wx[:, slice]^T dpre   or   dh += Wh^T dpre
+    unsigned off = 0, rows = H;
+    const float* W = Wh;
+    const float* mask = mask_h;
+    unsigned mask_ld = H, mask_bd = mask_h_bd;
+    if (i < num_inputs) {
+      for (unsigned j = 0; j < i; ++j) off += x_dims_host[j];
+      rows = x_dims_host[i];
+      W = Wx + size_t(off) * G;
+      mask = mask_x;
+      mask_ld = gi.I;
+      mask_bd = mask_x_bd;
+    } else {
+      off = 0;
+    }
+    GemmSeg s{W, G, dpre, G, G};
+    if (!gi.dropout) return gemm_run(dev, true, true, rows, B, 1, &s, dEdxi, acc);
+    DYHIP_CHECK_STATUS(gemm_run(dev, true, true, rows, B, 1, &s, tmp, ovw));
+    hipLaunchKernelGGL(acc_mul_mask_kernel, dim3(cdiv<unsigned>(rows, 256), B), dim3(256), 0, dev->stream, rows, mask_ld,
+                       off, tmp, mask, mask_bd > 1 ? 1 : 0, dEdxi);
+    DYHIP_CHECK_LAUNCH();
+    return DYHIP_OK;
+  }
+  if (i == num_inputs + 1) {  // dWx += dpre * x_t^T
+    const float* x_eff = nullptr;
+    DYHIP_CHECK_STATUS(prepare_x(dev, num_inputs, xs_host, x_dims_host, gi.I, B, mask_x, mask_x_bd, tmp, &x_eff));
+    GemmSeg s{dpre, G, x_eff, gi.I, B};
+    return gemm_run(dev, false, false, G, gi.I, 1, &s, dEdxi, acc);
+  }
+  if (i == num_inputs + 2) {  // dWh += dpre * h^T
+    const float* h_eff = nullptr;
+    DYHIP_CHECK_STATUS(prepare_h(dev, H, B, h_tm1, mask_h, mask_h_bd, tmp, &h_eff));
+    GemmSeg s{dpre, G, h_eff, H, B};
+    return gemm_run(dev, false, false, G, H, 1, &s, dEdxi, acc);
+  }
+  // db += sum_b dpre
+  return batch_reduce(dev, G, B, dpre, nullptr, dEdxi, true, red_ws, red_bytes);
+}
+
+int dyhip_lstm_c_forward(dyhip_device* dev, unsigned H, unsigned B, const float* c_tm1, const float* gates, float* c) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(c_tm1 && gates && c, "VanillaLSTMC: null tensor pointer");
+  return launch_pointwise<0>(dev, H, B, c_tm1, gates, nullptr, c);
+}
+
+int dyhip_lstm_c_backward(dyhip_device* dev, unsigned H, unsigned B, const float* c_tm1, const float* gates,
+                          const float* dEdf, unsigned i, float* dEdxi) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(c_tm1 && gates && dEdf && dEdxi, "VanillaLSTMC: null tensor pointer");
+  DYHIP_REQUIRE(i < 2, "VanillaLSTMC has two arguments (i = %u)", i);
+  return i == 0 ? launch_pointwise<1>(dev, H, B, c_tm1, gates, dEdf, dEdxi)
+                : launch_pointwise<2>(dev, H, B, c_tm1, gates, dEdf, dEdxi);
+}
+
+int dyhip_lstm_h_forward(dyhip_device* dev, unsigned H, unsigned B, const float* c, const float* gates, float* h) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(c && gates && h, "VanillaLSTMH: null tensor pointer");
+  return launch_pointwise<3>(dev, H, B, c, gates, nullptr, h);
+}
+
+int dyhip_lstm_h_backward(dyhip_device* dev, unsigned H, unsigned B, const float* c, const float* gates,
+                          const float* dEdf, unsigned i, float* dEdxi) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(c && gates && dEdf && dEdxi, "VanillaLSTMH: null tensor pointer");
+  DYHIP_REQUIRE(i < 2, "VanillaLSTMH has two arguments (i = %u)", i);
+  return i == 0 ? launch_pointwise<4>(dev, H, B, c, gates, dEdf, dEdxi)
+                : launch_pointwise<5>(dev, H, B, c, gates, dEdf, dEdxi);
+}
+
+}  // extern "C"

@@ -1,0 +1,214 @@
+// The seven scatter/gather helpers of dynet::gpu (dynet/gpu-ops.h:9-15,
+// gpu-ops.cu:12-166) with their original argument lists, and the squared-norm
+// reduction the trainer's gradient clipping needs (dynet/model.cc:806-848).
+//
+// parallel_memcpy / parallel_accumulate move the ragged per-node tensors of the
+// autobatching executor (dynet/exec.cc:298-411).  The reference maps thread ->
+// sequence (id % num_seqs), so neighbouring lanes touch different sequences; here
+// blockIdx.y is the sequence and lanes walk consecutive floats of it, with
+// 128-bit accesses when both sides are 16-byte aligned.
+#include "common.h"
+
+namespace dyhip {
+
+constexpr int kThreads = 256;
+
+__global__ __launch_bounds__(kThreads) void d2s_assign_kernel(int n, const unsigned* __restrict__ idx,
+                                                              const float* __restrict__ src, float* __restrict__ trg) {
+  const int i = blockIdx.x * kThreads + threadIdx.x;
+  if (i < n) trg[idx[i]] = src[i];
+}
+
+__global__ __launch_bounds__(kThreads) void s2d_assign_kernel(int n, const unsigned* __restrict__ idx,
+                                                              const float* __restrict__ src, float* __restrict__ trg) {
+  const int i = blockIdx.x * kThreads + threadIdx.x;
+  if (i < n) trg[i] = src[idx[i]];
+}
+
+// duplicates in idx are legal, hence the atomic (as in the reference)
+__global__ __launch_bounds__(kThreads) void d2s_subtract_kernel(int n, const unsigned* __restrict__ idx,
+                                                                const float* __restrict__ src,
+                                                                float* __restrict__ trg) {
+  const int i = blockIdx.x * kThreads + threadIdx.x;
+  if (i < n) atomicAdd(trg + idx[i], -src[i]);
+}
+
+// trg[i*bsize + j] = src[idx[i]*bsize + j] * mult : block.y = i, lanes walk j
+__global__ __launch_bounds__(kThreads) void s2d_block_assign_mul_kernel(int bsize, const unsigned* __restrict__ idx,
+                                                                        float mult, const float* __restrict__ src,
+                                                                        float* __restrict__ trg) {
+  const size_t i = blockIdx.y;
+  const float* ps = src + size_t(idx[i]) * bsize;
+  float* pt = trg + i * bsize;
+  for (int j = blockIdx.x * kThreads + threadIdx.x; j < bsize; j += gridDim.x * kThreads) pt[j] = ps[j] * mult;
+}
+
+// trg[idx[i]*bsize + j] += src[i*bsize + j] with duplicates allowed: atomic, like
+// the reference.  (LookupNode gradients use the deterministic sorted path of
+// dyhip_lookup_accumulate_grads instead.)
+__global__ __launch_bounds__(kThreads) void d2s_block_add_kernel(int bsize, const unsigned* __restrict__ idx,
+                                                                 const float* __restrict__ src,
+                                                                 float* __restrict__ trg) {
+  const size_t i = blockIdx.y;
+  const float* ps = src + i * bsize;
+  float* pt = trg + size_t(idx[i]) * bsize;
+  for (int j = blockIdx.x * kThreads + threadIdx.x; j < bsize; j += gridDim.x * kThreads) atomicAdd(pt + j, ps[j]);
+}
+
+template <bool ACC>
+__global__ __launch_bounds__(kThreads) void ragged_move_kernel(float* const* __restrict__ src,
+                                                               float* const* __restrict__ trg,
+                                                               const size_t* __restrict__ len) {
+  const unsigned s = blockIdx.y;
+  const float* ps = src[s];
+  float* pt = trg[s];
+  const size_t n = len[s];
+  const size_t stride = size_t(gridDim.x) * kThreads;
+  const size_t t0 = size_t(blockIdx.x) * kThreads + threadIdx.x;
+  if (!ACC && aligned16(ps) && aligned16(pt)) {
+    const size_t n4 = n >> 2;
+    const float4* s4 = reinterpret_cast<const float4*>(ps);
+    float4* t4 = reinterpret_cast<float4*>(pt);
+    for (size_t i = t0; i < n4; i += stride) t4[i] = s4[i];
+    for (size_t i = (n4 << 2) + t0; i < n; i += stride) pt[i] = ps[i];
+  } else {
+    for (size_t i = t0; i < n; i += stride) {
+      if (ACC)
+        atomicAdd(pt + i, ps[i]);  // several sequences may target the same gradient buffer
+      else
+        pt[i] = ps[i];
+    }
+  }
+}
+
+// stage 1: per-block partial of sum g^2 ; stage 2: one block adds the partials in order
+__global__ __launch_bounds__(kThreads) void sqnorm_partial_kernel(size_t n, const float* __restrict__ g,
+                                                                  float* __restrict__ partial) {
+  __shared__ float red[4];
+  float s = 0.f;
+  const size_t stride = size_t(gridDim.x) * kThreads;
+  for (size_t i = size_t(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride) s += g[i] * g[i];
+  const float t = block_sum<4>(s, red);
+  if (threadIdx.x == 0) partial[blockIdx.x] = t;
+}
+
+__global__ __launch_bounds__(kThreads) void sqnorm_final_kernel(unsigned nparts, const float* __restrict__ partial,
+                                                                float* __restrict__ out) {
+  __shared__ float red[4];
+  float s = 0.f;
+  for (unsigned i = threadIdx.x; i < nparts; i += kThreads) s += partial[i];
+  const float t = block_sum<4>(s, red);
+  if (threadIdx.x == 0) *out = t;
+}
+
+constexpr unsigned kSqnormBlocks = 1024;
+
+static unsigned grid1d(int n) { return static_cast<unsigned>((n + kThreads - 1) / kThreads); }
+
+}  // namespace dyhip
+
+using namespace dyhip;
+
+extern "C" {
+
+int dyhip_dense_to_sparse_assign(dyhip_device* dev, int n, const unsigned* ids, const float* src, float* trg) {
+  DYHIP_CHECK_DEV(dev);
+  if (n <= 0) return DYHIP_OK;
+  DYHIP_REQUIRE(ids && src && trg, "null pointer");
+  hipLaunchKernelGGL(d2s_assign_kernel, dim3(grid1d(n)), dim3(kThreads), 0, dev->stream, n, ids, src, trg);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_sparse_to_dense_assign(dyhip_device* dev, int n, const unsigned* ids, const float* src, float* trg) {
+  DYHIP_CHECK_DEV(dev);
+  if (n <= 0) return DYHIP_OK;
+  DYHIP_REQUIRE(ids && src && trg, "null pointer");
+  hipLaunchKernelGGL(s2d_assign_kernel, dim3(grid1d(n)), dim3(kThreads), 0, dev->stream, n, ids, src, trg);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_dense_to_sparse_subtract(dyhip_device* dev, int n, const unsigned* ids, const float* src, float* trg) {
+  DYHIP_CHECK_DEV(dev);
+  if (n <= 0) return DYHIP_OK;
+  DYHIP_REQUIRE(ids && src && trg, "null pointer");
+  hipLaunchKernelGGL(d2s_subtract_kernel, dim3(grid1d(n)), dim3(kThreads), 0, dev->stream, n, ids, src, trg);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_sparse_to_dense_block_assign_and_multiply(dyhip_device* dev, int n, const unsigned* idx, int bsize,
+                                                    float mult, const float* src, float* trg) {
+  DYHIP_CHECK_DEV(dev);
+  if (n <= 0 || bsize <= 0) return DYHIP_OK;
+  DYHIP_REQUIRE(idx && src && trg, "null pointer");
+  DYHIP_REQUIRE(n <= 65535, "at most 65535 blocks per call (got %d)", n);
+  unsigned gx = grid1d(bsize);
+  if (gx > 64) gx = 64;
+  hipLaunchKernelGGL(s2d_block_assign_mul_kernel, dim3(gx, n), dim3(kThreads), 0, dev->stream, bsize, idx, mult, src,
+                     trg);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_dense_to_sparse_block_add(dyhip_device* dev, int n, const unsigned* ids, int bsize, const float* src,
+                                    float* trg) {
+  DYHIP_CHECK_DEV(dev);
+  if (n <= 0 || bsize <= 0) return DYHIP_OK;
+  DYHIP_REQUIRE(ids && src && trg, "null pointer");
+  DYHIP_REQUIRE(n <= 65535, "at most 65535 blocks per call (got %d)", n);
+  unsigned gx = grid1d(bsize);
+  if (gx > 64) gx = 64;
+  hipLaunchKernelGGL(d2s_block_add_kernel, dim3(gx, n), dim3(kThreads), 0, dev->stream, bsize, ids, src, trg);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+static int ragged_move(dyhip_device* dev, bool acc, int num_seqs, int max_len, float** src, float** trg, size_t* len) {
+  DYHIP_CHECK_DEV(dev);
+  if (num_seqs <= 0 || max_len <= 0) return DYHIP_OK;
+  DYHIP_REQUIRE(src && trg && len, "null pointer");
+  DYHIP_REQUIRE(num_seqs <= 65535, "at most 65535 sequences per call (got %d)", num_seqs);
+  unsigned gx = static_cast<unsigned>((size_t(max_len) + size_t(kThreads) * 4 - 1) / (size_t(kThreads) * 4));
+  if (gx < 1) gx = 1;
+  if (gx > 256) gx = 256;
+  if (acc)
+    hipLaunchKernelGGL(ragged_move_kernel<true>, dim3(gx, num_seqs), dim3(kThreads), 0, dev->stream, src, trg, len);
+  else
+    hipLaunchKernelGGL(ragged_move_kernel<false>, dim3(gx, num_seqs), dim3(kThreads), 0, dev->stream, src, trg, len);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_parallel_memcpy(dyhip_device* dev, int num_seqs, int max_len, float** src, float** trg, size_t* len) {
+  return ragged_move(dev, false, num_seqs, max_len, src, trg, len);
+}
+
+int dyhip_parallel_accumulate(dyhip_device* dev, int num_seqs, int max_len, float** src, float** trg, size_t* len) {
+  return ragged_move(dev, true, num_seqs, max_len, src, trg, len);
+}
+
+int dyhip_squared_l2norm_workspace(size_t n, size_t* ws_bytes) {
+  DYHIP_REQUIRE(ws_bytes != nullptr, "null output pointer");
+  (void)n;
+  *ws_bytes = kSqnormBlocks * sizeof(float);
+  return DYHIP_OK;
+}
+
+int dyhip_squared_l2norm(dyhip_device* dev, size_t n, const float* g, float* out, void* ws, size_t ws_bytes) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(out != nullptr && (n == 0 || g != nullptr), "null pointer");
+  DYHIP_REQUIRE(ws != nullptr && ws_bytes >= kSqnormBlocks * sizeof(float), "squared_l2norm needs %zu workspace bytes",
+                kSqnormBlocks * sizeof(float));
+  unsigned blocks = static_cast<unsigned>((n + size_t(kThreads) * 8 - 1) / (size_t(kThreads) * 8));
+  if (blocks < 1) blocks = 1;
+  if (blocks > kSqnormBlocks) blocks = kSqnormBlocks;
+  float* partial = static_cast<float*>(ws);
+  hipLaunchKernelGGL(sqnorm_partial_kernel, dim3(blocks), dim3(kThreads), 0, dev->stream, n, g, partial);
+  hipLaunchKernelGGL(sqnorm_final_kernel, dim3(1), dim3(kThreads), 0, dev->stream, blocks, partial, out);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+}  // extern "C"

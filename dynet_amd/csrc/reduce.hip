@@ -1,0 +1,611 @@
+// Reductions: sum over the batch dimension (sum_batches and the broadcast-side
+// backward of cmult / csum), mean_elems / std_elems, and the fused LayerNorm.
+//
+// Replaces the Eigen reductions of SumDimension (dynet/nodes-arith-sum.cc:197-248),
+// MomentDimension (dynet/nodes-moments.cc:181-309), StdDimension (:434-555) and the
+// eight-node layer_norm composite of dynet/expr.cc:248-253.
+//
+// All reductions are deterministic: partial sums are combined in a fixed order
+// (lanes by xor-butterfly, waves and grid partials by ascending index), never
+// with floating-point atomics.
+#include "common.h"
+
+namespace dyhip {
+
+// ============================================================================
+// batch reduction: out[j] (+)= sum_b in0[b*n + j] * (in1 ? in1[b*n + j] : 1)
+// ============================================================================
+//
+// Block = 64 column lanes x NW waves.  Lane l owns VEC consecutive columns
+// (VEC = 4: one 128-bit access); wave w of split s sums batch elements
+// s*per_split + w, + NW, ...; the NW wave partials are combined through LDS in
+// ascending w.  With more than one split the block writes its partial row to
+// the workspace and a second kernel adds the splits in ascending s.
+constexpr int kBrWaves = 8;
+constexpr unsigned kBrMaxSplits = 64;
+
+struct BrPlan {
+  unsigned tiles;      // column tiles of 64*VEC columns
+  unsigned splits;     // batch splits
+  unsigned per_split;  // batch elements per split
+  int vec;
+};
+
+static BrPlan br_plan(size_t n, unsigned bd, bool vec_ok) {
+  BrPlan p;
+  p.vec = vec_ok ? 4 : 1;
+  p.tiles = static_cast<unsigned>(cdiv<size_t>(n, size_t(64) * p.vec));
+  unsigned want = p.tiles >= 192 ? 1u : cdiv<unsigned>(512u, p.tiles);
+  unsigned max_by_work = cdiv<unsigned>(bd, kBrWaves * 2);
+  if (want > max_by_work) want = max_by_work;
+  if (want > kBrMaxSplits) want = kBrMaxSplits;
+  if (want < 1) want = 1;
+  p.per_split = cdiv<unsigned>(bd, want);
+  p.splits = cdiv<unsigned>(bd, p.per_split);
+  return p;
+}
+
+template <int VEC, bool MUL>
+__global__ __launch_bounds__(64 * kBrWaves) void batch_reduce_kernel(size_t n, unsigned bd, unsigned per_split,
+                                                                    const float* __restrict__ in0,
+                                                                    const float* __restrict__ in1,
+                                                                    float* __restrict__ out, int accumulate,
+                                                                    float* __restrict__ partial) {
+  __shared__ float lds[kBrWaves][64 * VEC];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const size_t col = (size_t(blockIdx.x) * 64 + lane) * VEC;
+  const unsigned b0 = blockIdx.y * per_split;
+  const unsigned b1 = min(bd, b0 + per_split);
+  float acc[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
+  if (col < n) {
+    constexpr int U = 4;
+    unsigned b = b0 + w;
+    for (; b + (U - 1) * kBrWaves < b1; b += U * kBrWaves) {
+      float x[U][VEC], y[U][VEC];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const size_t off = size_t(b + u * kBrWaves) * n + col;
+        if (VEC == 4) {
+          const float4 t = *reinterpret_cast<const float4*>(in0 + off);
+          x[u][0] = t.x; x[u][1 % VEC] = t.y; x[u][2 % VEC] = t.z; x[u][3 % VEC] = t.w;
+          if (MUL) {
+            const float4 s = *reinterpret_cast<const float4*>(in1 + off);
+            y[u][0] = s.x; y[u][1 % VEC] = s.y; y[u][2 % VEC] = s.z; y[u][3 % VEC] = s.w;
+          }
+        } else {
+          x[u][0] = in0[off];
+          if (MUL) y[u][0] = in1[off];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[v] += MUL ? x[u][v] * y[u][v] : x[u][v];
+    }
+    for (; b < b1; b += kBrWaves) {
+      const size_t off = size_t(b) * n + col;
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) acc[v] += MUL ? in0[off + v] * in1[off + v] : in0[off + v];
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) lds[w][lane * VEC + v] = acc[v];
+  __syncthreads();
+  if (w == 0 && col < n) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      float t = lds[0][lane * VEC + v];
+#pragma unroll
+      for (int k = 1; k < kBrWaves; ++k) t += lds[k][lane * VEC + v];
+      if (partial)
+        partial[size_t(blockIdx.y) * n + col + v] = t;
+      else
+        out[col + v] = accumulate ? out[col + v] + t : t;
+    }
+  }
+}
+
+// out[j] (+)= sum_s partial[s*n + j], ascending s
+__global__ __launch_bounds__(256) void combine_partials_kernel(size_t n, unsigned splits,
+                                                               const float* __restrict__ partial,
+                                                               float* __restrict__ out, int accumulate) {
+  const size_t j = size_t(blockIdx.x) * 256 + threadIdx.x;
+  if (j >= n) return;
+  float t = partial[j];
+  for (unsigned s = 1; s < splits; ++s) t += partial[size_t(s) * n + j];
+  out[j] = accumulate ? out[j] + t : t;
+}
+
+int batch_reduce(dyhip_device* dev, size_t n, unsigned bd, const float* in0, const float* in1, float* out,
+                 bool accumulate, void* ws, size_t ws_bytes) {
+  if (n == 0) return DYHIP_OK;
+  DYHIP_REQUIRE(bd >= 1, "batch reduction over an empty batch");
+  const bool vec_ok = (n % 4 == 0) && aligned16(in0) && (in1 == nullptr || aligned16(in1));
+  const BrPlan p = br_plan(n, bd, vec_ok);
+  float* partial = nullptr;
+  if (p.splits > 1) {
+    const size_t need = size_t(p.splits) * n * sizeof(float);
+    DYHIP_REQUIRE(ws != nullptr && ws_bytes >= need, "batch reduction needs %zu workspace bytes, got %zu", need,
+                  ws_bytes);
+    partial = static_cast<float*>(ws);
+  }
+  const dim3 grid(p.tiles, p.splits), block(64 * kBrWaves);
+  const int acc = accumulate ? 1 : 0;
+#define DYHIP_BR_LAUNCH(VEC, MUL)                                                                          \
+  hipLaunchKernelGGL((batch_reduce_kernel<VEC, MUL>), grid, block, 0, dev->stream, n, bd, p.per_split, in0, \
+                     in1, out, acc, partial)
+  if (p.vec == 4) {
+    if (in1) DYHIP_BR_LAUNCH(4, true); else DYHIP_BR_LAUNCH(4, false);
+  } else {
+    if (in1) DYHIP_BR_LAUNCH(1, true); else DYHIP_BR_LAUNCH(1, false);
+  }
+#undef DYHIP_BR_LAUNCH
+  DYHIP_CHECK_LAUNCH();
+  if (partial) {
+    hipLaunchKernelGGL(combine_partials_kernel, dim3((unsigned)cdiv<size_t>(n, 256)), dim3(256), 0, dev->stream, n,
+                       p.splits, partial, out, acc);
+    DYHIP_CHECK_LAUNCH();
+  }
+  return DYHIP_OK;
+}
+
+// ============================================================================
+// mean_elems / std_elems: one value per batch element (block per batch element)
+// ============================================================================
+template <bool STD>
+__global__ __launch_bounds__(256) void moment_fwd_kernel(size_t n, const float* __restrict__ x,
+                                                         float* __restrict__ y) {
+  __shared__ float red[4];
+  const float* px = x + size_t(blockIdx.x) * n;
+  float s = 0.f;
+  for (size_t j = threadIdx.x; j < n; j += 256) s += px[j];
+  const float mean = block_sum<4>(s, red) / float(n);
+  if (!STD) {
+    if (threadIdx.x == 0) y[blockIdx.x] = mean;
+    return;
+  }
+  float v = 0.f;
+  for (size_t j = threadIdx.x; j < n; j += 256) {
+    const float d = px[j] - mean;
+    v += d * d;
+  }
+  const float var = block_sum<4>(v, red) / float(n);
+  if (threadIdx.x == 0) y[blockIdx.x] = sqrtf(var);
+}
+
+// dx[b, j] += dEdf[b] / n
+__global__ __launch_bounds__(256) void mean_bwd_kernel(size_t n, const float* __restrict__ dEdf,
+                                                       float* __restrict__ dEdx) {
+  const float d = dEdf[blockIdx.y] / float(n);
+  const size_t j = size_t(blockIdx.x) * 256 + threadIdx.x;
+  if (j < n) dEdx[size_t(blockIdx.y) * n + j] += d;
+}
+
+// dx[b, j] += (2/n) * (x - mean_b) * (dEdf[b] / (2 * fx[b]))
+__global__ __launch_bounds__(256) void std_bwd_kernel(size_t n, const float* __restrict__ x,
+                                                      const float* __restrict__ fx, const float* __restrict__ dEdf,
+                                                      float* __restrict__ dEdx) {
+  __shared__ float red[4];
+  const float* px = x + size_t(blockIdx.x) * n;
+  float s = 0.f;
+  for (size_t j = threadIdx.x; j < n; j += 256) s += px[j];
+  const float mean = block_sum<4>(s, red) / float(n);
+  const float sb = dEdf[blockIdx.x] / (2.f * fx[blockIdx.x]);
+  const float c = 2.f / float(n);
+  float* pd = dEdx + size_t(blockIdx.x) * n;
+  for (size_t j = threadIdx.x; j < n; j += 256) pd[j] += c * (px[j] - mean) * sb;
+}
+
+// ============================================================================
+// fused LayerNorm
+// ============================================================================
+//
+// Fast path (n % 4 == 0, n <= 2048, 16-byte aligned): one wavefront per batch
+// element, the whole row held in registers as VPL float4 per lane (lane l owns
+// float4 slots l, l+64, ...), so x (and dy) are read from HBM exactly once.
+// mean and the two-pass population variance are wave-butterfly reductions.
+//
+// Backward keeps per-lane partial sums of dg / db across the rows a wave owns,
+// combines the waves of a block through LDS in ascending wave order, writes one
+// partial row per block to the workspace, and a second kernel adds the block
+// partials in ascending block order into dg / db.
+constexpr int kLnWavesFwd = 4;
+constexpr int kLnWavesBwd = 8;
+constexpr unsigned kLnBwdMaxBlocks = 256;
+constexpr float kLnEps = 1e-8f;
+
+template <int VPL>
+__global__ __launch_bounds__(64 * kLnWavesFwd) void ln_fwd_wave_kernel(unsigned n4, unsigned bd,
+                                                                      const float4* __restrict__ x,
+                                                                      const float4* __restrict__ g,
+                                                                      const float4* __restrict__ b,
+                                                                      float4* __restrict__ y) {
+  const int lane = threadIdx.x & 63;
+  const unsigned row = blockIdx.x * kLnWavesFwd + (threadIdx.x >> 6);
+  if (row >= bd) return;
+  const float fn = float(n4 * 4);
+  const float4* px = x + size_t(row) * n4;
+  float4 v[VPL];
+#pragma unroll
+  for (int u = 0; u < VPL; ++u) {
+    const unsigned idx = lane + 64 * u;
+    v[u] = idx < n4 ? px[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int u = 0; u < VPL; ++u) s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+  const float mean = wave_sum(s) / fn;
+  float ss = 0.f;
+#pragma unroll
+  for (int u = 0; u < VPL; ++u) {
+    if (lane + 64 * u < n4) {
+      const float dx = v[u].x - mean, dy = v[u].y - mean, dz = v[u].z - mean, dw = v[u].w - mean;
+      ss += (dx * dx + dy * dy) + (dz * dz + dw * dw);
+    }
+  }
+  const float sigma = sqrtf(wave_sum(ss) / fn);
+  const float sden = kLnEps + sigma;
+  const float neg = -mean;
+  float4* py = y + size_t(row) * n4;
+#pragma unroll
+  for (int u = 0; u < VPL; ++u) {
+    const unsigned idx = lane + 64 * u;
+    if (idx < n4) {
+      const float4 gg = g[idx], bb = b[idx];
+      float4 r;
+      r.x = gg.x * ((v[u].x + neg) / sden) + bb.x;
+      r.y = gg.y * ((v[u].y + neg) / sden) + bb.y;
+      r.z = gg.z * ((v[u].z + neg) / sden) + bb.z;
+      r.w = gg.w * ((v[u].w + neg) / sden) + bb.w;
+      py[idx] = r;
+    }
+  }
+}
+
+// generic fallback: one block per batch element, three passes over the row
+__global__ __launch_bounds__(256) void ln_fwd_block_kernel(size_t n, const float* __restrict__ x,
+                                                           const float* __restrict__ g,
+                                                           const float* __restrict__ b, float* __restrict__ y) {
+  __shared__ float red[4];
+  const float* px = x + size_t(blockIdx.x) * n;
+  float s = 0.f;
+  for (size_t j = threadIdx.x; j < n; j += 256) s += px[j];
+  const float mean = block_sum<4>(s, red) / float(n);
+  float v = 0.f;
+  for (size_t j = threadIdx.x; j < n; j += 256) {
+    const float d = px[j] - mean;
+    v += d * d;
+  }
+  const float sigma = sqrtf(block_sum<4>(v, red) / float(n));
+  const float sden = kLnEps + sigma, neg = -mean;
+  float* py = y + size_t(blockIdx.x) * n;
+  for (size_t j = threadIdx.x; j < n; j += 256) py[j] = g[j] * ((px[j] + neg) / sden) + b[j];
+}
+
+// accumulate helper for float4 with a per-component functor
+#define DYHIP_F4_EACH(stmt) \
+  { stmt(x) stmt(y) stmt(z) stmt(w) }
+
+template <int VPL>
+__global__ __launch_bounds__(64 * kLnWavesBwd) void ln_bwd_wave_kernel(unsigned n4, unsigned bd,
+                                                                      const float4* __restrict__ x,
+                                                                      const float4* __restrict__ g,
+                                                                      const float4* __restrict__ dEdf,
+                                                                      float4* __restrict__ dx,
+                                                                      float* __restrict__ part_dg,
+                                                                      float* __restrict__ part_db) {
+  extern __shared__ float lds[];  // [kLnWavesBwd][n] when partials are requested
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const float fn = float(n4 * 4);
+  const bool want_g = part_dg != nullptr, want_b = part_db != nullptr;
+  float4 gg[VPL], pdg[VPL], pdb[VPL];
+#pragma unroll
+  for (int u = 0; u < VPL; ++u) {
+    const unsigned idx = lane + 64 * u;
+    gg[u] = idx < n4 ? g[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+    pdg[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    pdb[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  const unsigned wave_global = blockIdx.x * kLnWavesBwd + w;
+  const unsigned wave_count = gridDim.x * kLnWavesBwd;
+  for (unsigned row = wave_global; row < bd; row += wave_count) {
+    const float4* px = x + size_t(row) * n4;
+    const float4* pdy = dEdf + size_t(row) * n4;
+    float4 v[VPL], d[VPL];
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+      const unsigned idx = lane + 64 * u;
+      v[u] = idx < n4 ? px[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+      d[u] = idx < n4 ? pdy[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+    const float mean = wave_sum(s) / fn;
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+      if (lane + 64 * u < n4) {
+        const float ax = v[u].x - mean, ay = v[u].y - mean, az = v[u].z - mean, aw = v[u].w - mean;
+        ss += (ax * ax + ay * ay) + (az * az + aw * aw);
+      }
+    }
+    const float sigma = sqrtf(wave_sum(ss) / fn);
+    const float sden = kLnEps + sigma, neg = -mean, s2 = sden * sden;
+    // per-row sums: ds = -sum dq/s^2 * xc ; dneg = sum dq/s, with dq = dy*g
+    float ds_p = 0.f, dneg_p = 0.f;
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+      if (lane + 64 * u < n4) {
+#define DYHIP_LN_ROW(c)                      \
+  {                                          \
+    const float xc = v[u].c + neg;           \
+    const float dq = d[u].c * gg[u].c;       \
+    ds_p -= dq / s2 * xc;                    \
+    dneg_p += dq / sden;                     \
+    if (want_g) pdg[u].c += d[u].c * (xc / sden); \
+    if (want_b) pdb[u].c += d[u].c;          \
+  }
+        DYHIP_F4_EACH(DYHIP_LN_ROW)
+#undef DYHIP_LN_ROW
+      }
+    }
+    if (dx != nullptr) {
+      const float ds = wave_sum(ds_p);
+      const float dmu = -wave_sum(dneg_p);
+      const float sb = ds / (2.f * sigma);
+      const float c = 2.f / fn;
+      const float dmu_n = dmu / fn;
+      float4* pdx = dx + size_t(row) * n4;
+#pragma unroll
+      for (int u = 0; u < VPL; ++u) {
+        const unsigned idx = lane + 64 * u;
+        if (idx < n4) {
+          float4 o = pdx[idx];
+#define DYHIP_LN_DX(c_)                                            \
+  {                                                                \
+    float acc = o.c_;                                              \
+    acc += c * (v[u].c_ - mean) * sb;                              \
+    acc += (d[u].c_ * gg[u].c_) / sden;                            \
+    acc += dmu_n;                                                  \
+    o.c_ = acc;                                                    \
+  }
+          DYHIP_F4_EACH(DYHIP_LN_DX)
+#undef DYHIP_LN_DX
+          pdx[idx] = o;
+        }
+      }
+    }
+  }
+  if (!want_g && !want_b) return;
+  const unsigned n = n4 * 4;
+  // combine the waves of this block in ascending wave order, one output at a time
+  for (int which = 0; which < 2; ++which) {
+    float* part = which == 0 ? part_dg : part_db;
+    if (part == nullptr) continue;
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+      const unsigned idx = lane + 64 * u;
+      if (idx < n4) reinterpret_cast<float4*>(lds + size_t(w) * n)[idx] = which == 0 ? pdg[u] : pdb[u];
+    }
+    __syncthreads();
+    for (unsigned j = threadIdx.x; j < n; j += 64 * kLnWavesBwd) {
+      float t = lds[j];
+#pragma unroll
+      for (int k = 1; k < kLnWavesBwd; ++k) t += lds[size_t(k) * n + j];
+      part[size_t(blockIdx.x) * n + j] = t;
+    }
+  }
+}
+
+// generic fallback, pass 1: per-row statistics and the dx update.
+// stats[row] = {mean, sden}
+__global__ __launch_bounds__(256) void ln_bwd_block_kernel(size_t n, const float* __restrict__ x,
+                                                           const float* __restrict__ g,
+                                                           const float* __restrict__ dEdf, float* __restrict__ dx,
+                                                           float2* __restrict__ stats) {
+  __shared__ float red[4];
+  const float fn = float(n);
+  const float* px = x + size_t(blockIdx.x) * n;
+  const float* pdy = dEdf + size_t(blockIdx.x) * n;
+  float s = 0.f;
+  for (size_t j = threadIdx.x; j < n; j += 256) s += px[j];
+  const float mean = block_sum<4>(s, red) / fn;
+  float v = 0.f;
+  for (size_t j = threadIdx.x; j < n; j += 256) {
+    const float d = px[j] - mean;
+    v += d * d;
+  }
+  const float sigma = sqrtf(block_sum<4>(v, red) / fn);
+  const float sden = kLnEps + sigma, neg = -mean, s2 = sden * sden;
+  if (stats != nullptr && threadIdx.x == 0) stats[blockIdx.x] = make_float2(mean, sden);
+  if (dx == nullptr) return;
+  float ds_p = 0.f, dneg_p = 0.f;
+  for (size_t j = threadIdx.x; j < n; j += 256) {
+    const float dq = pdy[j] * g[j];
+    ds_p -= dq / s2 * (px[j] + neg);
+    dneg_p += dq / sden;
+  }
+  const float ds = block_sum<4>(ds_p, red);
+  const float dmu = -block_sum<4>(dneg_p, red);
+  const float sb = ds / (2.f * sigma), c = 2.f / fn, dmu_n = dmu / fn;
+  float* pdx = dx + size_t(blockIdx.x) * n;
+  for (size_t j = threadIdx.x; j < n; j += 256) {
+    float acc = pdx[j];
+    acc += c * (px[j] - mean) * sb;
+    acc += (pdy[j] * g[j]) / sden;
+    acc += dmu_n;
+    pdx[j] = acc;
+  }
+}
+
+// generic fallback, pass 2: dg[j] += sum_b dy*(x-mean_b)/sden_b ; db[j] += sum_b dy
+__global__ __launch_bounds__(256) void ln_bwd_cols_kernel(size_t n, unsigned bd, const float* __restrict__ x,
+                                                          const float* __restrict__ dEdf,
+                                                          const float2* __restrict__ stats, float* __restrict__ dg,
+                                                          float* __restrict__ db) {
+  const size_t j = size_t(blockIdx.x) * 256 + threadIdx.x;
+  if (j >= n) return;
+  float sg = 0.f, sb = 0.f;
+  for (unsigned r = 0; r < bd; ++r) {
+    const float2 st = stats[r];
+    const float d = dEdf[size_t(r) * n + j];
+    sg += d * ((x[size_t(r) * n + j] - st.x) / st.y);
+    sb += d;
+  }
+  if (dg) dg[j] += sg;
+  if (db) db[j] += sb;
+}
+
+static bool ln_fast_ok(size_t n, const void* a, const void* b, const void* c, const void* d) {
+  return n % 4 == 0 && n <= 2048 && aligned16(a) && aligned16(b) && (c == nullptr || aligned16(c)) &&
+         (d == nullptr || aligned16(d));
+}
+
+static unsigned ln_bwd_blocks(unsigned bd) {
+  unsigned blocks = cdiv<unsigned>(bd, kLnWavesBwd);
+  return blocks > kLnBwdMaxBlocks ? kLnBwdMaxBlocks : blocks;
+}
+
+}  // namespace dyhip
+
+using namespace dyhip;
+
+extern "C" {
+
+int dyhip_batch_reduce_workspace(size_t n, unsigned bd, size_t* ws_bytes) {
+  DYHIP_REQUIRE(ws_bytes != nullptr, "null output pointer");
+  if (n == 0 || bd == 0) {
+    *ws_bytes = 0;
+    return DYHIP_OK;
+  }
+  // the scalar plan has at least as many tiles, hence at most as many splits
+  const BrPlan p = br_plan(n, bd, n % 4 == 0);
+  const BrPlan q = br_plan(n, bd, false);
+  const unsigned splits = p.splits > q.splits ? p.splits : q.splits;
+  *ws_bytes = splits > 1 ? size_t(splits) * n * sizeof(float) : 0;
+  return DYHIP_OK;
+}
+
+int dyhip_sum_batches_forward(dyhip_device* dev, size_t n, unsigned bd, const float* x, float* y, void* ws,
+                              size_t ws_bytes) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(n == 0 || (x && y), "null tensor pointer");
+  return batch_reduce(dev, n, bd, x, nullptr, y, false, ws, ws_bytes);
+}
+
+int dyhip_mean_elems_forward(dyhip_device* dev, size_t n, unsigned bd, const float* x, float* y) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(n >= 1 && x && y, "mean_elems needs a non-empty tensor");
+  if (bd == 0) return DYHIP_OK;
+  hipLaunchKernelGGL(moment_fwd_kernel<false>, dim3(bd), dim3(256), 0, dev->stream, n, x, y);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_std_elems_forward(dyhip_device* dev, size_t n, unsigned bd, const float* x, float* y) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(n >= 1 && x && y, "std_elems needs a non-empty tensor");
+  if (bd == 0) return DYHIP_OK;
+  hipLaunchKernelGGL(moment_fwd_kernel<true>, dim3(bd), dim3(256), 0, dev->stream, n, x, y);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_mean_elems_backward(dyhip_device* dev, size_t n, unsigned bd, const float* dEdf, float* dEdx) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(n >= 1 && dEdf && dEdx, "mean_elems needs a non-empty tensor");
+  if (bd == 0) return DYHIP_OK;
+  DYHIP_REQUIRE(bd <= 65535, "mean_elems backward supports at most 65535 batch elements");
+  hipLaunchKernelGGL(mean_bwd_kernel, dim3((unsigned)cdiv<size_t>(n, 256), bd), dim3(256), 0, dev->stream, n, dEdf,
+                     dEdx);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_std_elems_backward(dyhip_device* dev, size_t n, unsigned bd, const float* x, const float* fx,
+                             const float* dEdf, float* dEdx) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(n >= 1 && x && fx && dEdf && dEdx, "std_elems needs a non-empty tensor");
+  if (bd == 0) return DYHIP_OK;
+  hipLaunchKernelGGL(std_bwd_kernel, dim3(bd), dim3(256), 0, dev->stream, n, x, fx, dEdf, dEdx);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_layer_norm_forward(dyhip_device* dev, size_t n, unsigned bd, const float* x, const float* g,
+                             const float* b, float* y) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(n >= 1 && x && g && b && y, "layer_norm needs non-empty tensors");
+  if (bd == 0) return DYHIP_OK;
+  if (ln_fast_ok(n, x, g, b, y)) {
+    const unsigned n4 = static_cast<unsigned>(n / 4);
+    const dim3 grid(cdiv<unsigned>(bd, kLnWavesFwd)), block(64 * kLnWavesFwd);
+    const float4 *x4 = reinterpret_cast<const float4*>(x), *g4 = reinterpret_cast<const float4*>(g),
+                 *b4 = reinterpret_cast<const float4*>(b);
+    float4* y4 = reinterpret_cast<float4*>(y);
+    if (n4 <= 64) hipLaunchKernelGGL(ln_fwd_wave_kernel<1>, grid, block, 0, dev->stream, n4, bd, x4, g4, b4, y4);
+    else if (n4 <= 128) hipLaunchKernelGGL(ln_fwd_wave_kernel<2>, grid, block, 0, dev->stream, n4, bd, x4, g4, b4, y4);
+    else if (n4 <= 256) hipLaunchKernelGGL(ln_fwd_wave_kernel<4>, grid, block, 0, dev->stream, n4, bd, x4, g4, b4, y4);
+    else hipLaunchKernelGGL(ln_fwd_wave_kernel<8>, grid, block, 0, dev->stream, n4, bd, x4, g4, b4, y4);
+  } else {
+    hipLaunchKernelGGL(ln_fwd_block_kernel, dim3(bd), dim3(256), 0, dev->stream, n, x, g, b, y);
+  }
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_layer_norm_backward_workspace(size_t n, unsigned bd, size_t* ws_bytes) {
+  DYHIP_REQUIRE(ws_bytes != nullptr, "null output pointer");
+  const size_t fast = size_t(2) * ln_bwd_blocks(bd) * n * sizeof(float);
+  const size_t generic = size_t(bd) * sizeof(float2);
+  *ws_bytes = fast > generic ? fast : generic;
+  return DYHIP_OK;
+}
+
+int dyhip_layer_norm_backward(dyhip_device* dev, size_t n, unsigned bd, const float* x, const float* g,
+                              const float* dEdf, float* dx, float* dg, float* db, void* ws, size_t ws_bytes) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(n >= 1 && x && g && dEdf, "layer_norm needs non-empty tensors");
+  if (bd == 0 || (!dx && !dg && !db)) return DYHIP_OK;
+  const bool cols = dg != nullptr || db != nullptr;
+  size_t need = 0;
+  DYHIP_CHECK_STATUS(dyhip_layer_norm_backward_workspace(n, bd, &need));
+  DYHIP_REQUIRE(!cols || (ws != nullptr && ws_bytes >= need), "layer_norm backward needs %zu workspace bytes, got %zu",
+                need, ws_bytes);
+  if (ln_fast_ok(n, x, g, dEdf, dx)) {
+    const unsigned n4 = static_cast<unsigned>(n / 4);
+    const unsigned blocks = ln_bwd_blocks(bd);
+    float* part_dg = dg ? static_cast<float*>(ws) : nullptr;
+    float* part_db = db ? static_cast<float*>(ws) + size_t(blocks) * n : nullptr;
+    const size_t lds = cols ? size_t(kLnWavesBwd) * n * sizeof(float) : 0;
+    const dim3 grid(blocks), block(64 * kLnWavesBwd);
+    const float4 *x4 = reinterpret_cast<const float4*>(x), *g4 = reinterpret_cast<const float4*>(g),
+                 *d4 = reinterpret_cast<const float4*>(dEdf);
+    float4* dx4 = reinterpret_cast<float4*>(dx);
+    if (n4 <= 64) hipLaunchKernelGGL(ln_bwd_wave_kernel<1>, grid, block, lds, dev->stream, n4, bd, x4, g4, d4, dx4, part_dg, part_db);
+    else if (n4 <= 128) hipLaunchKernelGGL(ln_bwd_wave_kernel<2>, grid, block, lds, dev->stream, n4, bd, x4, g4, d4, dx4, part_dg, part_db);
+    else if (n4 <= 256) hipLaunchKernelGGL(ln_bwd_wave_kernel<4>, grid, block, lds, dev->stream, n4, bd, x4, g4, d4, dx4, part_dg, part_db);
+    else hipLaunchKernelGGL(ln_bwd_wave_kernel<8>, grid, block, lds, dev->stream, n4, bd, x4, g4, d4, dx4, part_dg, part_db);
+    DYHIP_CHECK_LAUNCH();
+    const dim3 cgrid((unsigned)cdiv<size_t>(n, 256));
+    if (dg) hipLaunchKernelGGL(combine_partials_kernel, cgrid, dim3(256), 0, dev->stream, n, blocks, part_dg, dg, 1);
+    if (db) hipLaunchKernelGGL(combine_partials_kernel, cgrid, dim3(256), 0, dev->stream, n, blocks, part_db, db, 1);
+    DYHIP_CHECK_LAUNCH();
+  } else {
+    float2* stats = cols ? static_cast<float2*>(ws) : nullptr;
+    hipLaunchKernelGGL(ln_bwd_block_kernel, dim3(bd), dim3(256), 0, dev->stream, n, x, g, dEdf, dx, stats);
+    DYHIP_CHECK_LAUNCH();
+    if (cols) {
+      hipLaunchKernelGGL(ln_bwd_cols_kernel, dim3((unsigned)cdiv<size_t>(n, 256)), dim3(256), 0, dev->stream, n, bd, x,
+                         dEdf, stats, dg, db);
+      DYHIP_CHECK_LAUNCH();
+    }
+  }
+  return DYHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,380 @@
+// Row-wise log-sum-exp, PickNegLogSoftmax, the LogSumExp node and argmax.
+//
+// Replaces TensorTools::logsumexp_dev (dynet/tensor.cc:468-507: three Eigen
+// launches that read x twice), PickNegLogSoftmax (dynet/nodes-pickneglogsoftmax.cc
+// :79-145, which adds a pick kernel, an Eigen subtract, a full-size exp pass and
+// an atomic subtract), LogSumExp (dynet/nodes-logsumexp.cc:38-97) and
+// TensorTools::argmax_dev (dynet/tensor.cc:527-538).
+//
+// Layout: x is rows x bd, one softmax per batch element (column), contiguous.
+// Forward reads every element exactly once: each thread keeps a running
+// (max, sum of exp(x - max)) pair over its 128-bit slices, pairs are merged by
+// wave butterfly and then across waves through LDS.  Backward is one
+// elementwise read-modify-write pass with the one-hot subtraction folded in.
+#include <cmath>
+#include <vector>
+
+#include "common.h"
+
+namespace dyhip {
+
+constexpr int kLseThreads = 1024;
+constexpr int kLseWaves = kLseThreads / 64;
+
+struct MaxSum {
+  float m, s;
+};
+
+__device__ __forceinline__ void ms_push4(MaxSum& a, const float4 v) {
+  const float cm = fmaxf(fmaxf(v.x, v.y), fmaxf(v.z, v.w));
+  if (cm > a.m) {
+    a.s *= __expf(a.m - cm);
+    a.m = cm;
+  }
+  a.s += (__expf(v.x - a.m) + __expf(v.y - a.m)) + (__expf(v.z - a.m) + __expf(v.w - a.m));
+}
+
+__device__ __forceinline__ void ms_push1(MaxSum& a, const float v) {
+  if (v > a.m) {
+    a.s *= __expf(a.m - v);
+    a.m = v;
+  }
+  a.s += __expf(v - a.m);
+}
+
+__device__ __forceinline__ MaxSum ms_merge(const MaxSum a, const MaxSum b) {
+  MaxSum r;
+  r.m = fmaxf(a.m, b.m);
+  // an empty partial has m = -inf and s = 0; keep it from producing exp(-inf - -inf)
+  const float sa = a.s == 0.f ? 0.f : a.s * __expf(a.m - r.m);
+  const float sb = b.s == 0.f ? 0.f : b.s * __expf(b.m - r.m);
+  r.s = sa + sb;
+  return r;
+}
+
+// One block per batch element.  Writes m[b], z[b]; if ids != nullptr also
+// fx[b] = z[b] - x[ids[b]] (the pick of PickNegLogSoftmax).
+template <bool VEC>
+__global__ __launch_bounds__(kLseThreads) void lse_cols_kernel(size_t rows, const float* __restrict__ x,
+                                                               float* __restrict__ m_out, float* __restrict__ z_out,
+                                                               const unsigned* __restrict__ ids,
+                                                               float* __restrict__ fx) {
+  __shared__ float lm[kLseWaves], ls[kLseWaves];
+  const unsigned b = blockIdx.x;
+  const float* px = x + size_t(b) * rows;
+  MaxSum a;
+  a.m = -INFINITY;
+  a.s = 0.f;
+  if (VEC) {
+    const float4* p4 = reinterpret_cast<const float4*>(px);
+    const size_t n4 = rows >> 2;
+    size_t i = threadIdx.x;
+    for (; i + 3 * kLseThreads < n4; i += 4 * kLseThreads) {
+      const float4 v0 = p4[i], v1 = p4[i + kLseThreads], v2 = p4[i + 2 * kLseThreads], v3 = p4[i + 3 * kLseThreads];
+      ms_push4(a, v0);
+      ms_push4(a, v1);
+      ms_push4(a, v2);
+      ms_push4(a, v3);
+    }
+    for (; i < n4; i += kLseThreads) ms_push4(a, p4[i]);
+  } else {
+    for (size_t i = threadIdx.x; i < rows; i += kLseThreads) ms_push1(a, px[i]);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    MaxSum o;
+    o.m = __shfl_xor(a.m, off, kWave);
+    o.s = __shfl_xor(a.s, off, kWave);
+    a = ms_merge(a, o);
+  }
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  if (lane == 0) {
+    lm[w] = a.m;
+    ls[w] = a.s;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    MaxSum t;
+    t.m = lm[0];
+    t.s = ls[0];
+    for (int k = 1; k < kLseWaves; ++k) {
+      MaxSum o;
+      o.m = lm[k];
+      o.s = ls[k];
+      t = ms_merge(t, o);
+    }
+    const float z = logf(t.s) + t.m;
+    m_out[b] = t.m;
+    z_out[b] = z;
+    if (ids != nullptr) fx[b] = z - x[ids[b]];
+  }
+}
+
+constexpr int kPbThreads = 256;
+constexpr int kPbUnroll = 4;
+
+// dx[:, b] += exp(x[:, b] - z[b]) * dy[b]; dx[ids[b]] -= dy[b]
+template <bool VEC>
+__global__ __launch_bounds__(kPbThreads) void pnls_bwd_kernel(size_t rows, unsigned tiles_per_col,
+                                                              const float* __restrict__ x,
+                                                              const float* __restrict__ z,
+                                                              const unsigned* __restrict__ ids,
+                                                              const float* __restrict__ dEdf,
+                                                              float* __restrict__ dEdx) {
+  const unsigned b = blockIdx.x / tiles_per_col;
+  const unsigned tile = blockIdx.x - b * tiles_per_col;
+  const float zb = z[b], dy = dEdf[b];
+  const size_t col0 = size_t(b) * rows;
+  const size_t hot = size_t(ids[b]) - col0;  // row of the picked element
+  if (VEC) {
+    const size_t n4 = rows >> 2;
+    const float4* x4 = reinterpret_cast<const float4*>(x + col0);
+    float4* d4 = reinterpret_cast<float4*>(dEdx + col0);
+    const size_t j0 = size_t(tile) * (kPbThreads * kPbUnroll) + threadIdx.x;
+    float4 xv[kPbUnroll], dv[kPbUnroll];
+#pragma unroll
+    for (int u = 0; u < kPbUnroll; ++u) {
+      const size_t j = j0 + size_t(u) * kPbThreads;
+      if (j < n4) {
+        xv[u] = x4[j];
+        dv[u] = d4[j];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kPbUnroll; ++u) {
+      const size_t j = j0 + size_t(u) * kPbThreads;
+      if (j < n4) {
+        float4 r;
+        r.x = dv[u].x + __expf(xv[u].x - zb) * dy;
+        r.y = dv[u].y + __expf(xv[u].y - zb) * dy;
+        r.z = dv[u].z + __expf(xv[u].z - zb) * dy;
+        r.w = dv[u].w + __expf(xv[u].w - zb) * dy;
+        if ((hot >> 2) == j) {
+          const unsigned c = hot & 3;
+          if (c == 0) r.x -= dy;
+          else if (c == 1) r.y -= dy;
+          else if (c == 2) r.z -= dy;
+          else r.w -= dy;
+        }
+        d4[j] = r;
+      }
+    }
+  } else {
+    const size_t j0 = size_t(tile) * (kPbThreads * kPbUnroll) + threadIdx.x;
+#pragma unroll
+    for (int u = 0; u < kPbUnroll; ++u) {
+      const size_t j = j0 + size_t(u) * kPbThreads;
+      if (j < rows) {
+        float r = dEdx[col0 + j] + __expf(x[col0 + j] - zb) * dy;
+        if (j == hot) r -= dy;
+        dEdx[col0 + j] = r;
+      }
+    }
+  }
+}
+
+// ---- LogSumExp node over k <= 8 arguments -----------------------------------
+constexpr unsigned kLseNodeMaxArgs = 8;
+struct LseNodeArgs {
+  const float* x[kLseNodeMaxArgs];
+  unsigned bcast[kLseNodeMaxArgs];  // 1 => batch 1, indexed by e % n
+  unsigned k;
+};
+
+__global__ __launch_bounds__(256) void lse_node_fwd_kernel(LseNodeArgs a, size_t n, size_t total,
+                                                           float* __restrict__ fx) {
+  const size_t e = size_t(blockIdx.x) * 256 + threadIdx.x;
+  if (e >= total) return;
+  const size_t j = e % n;
+  float m = a.x[0][a.bcast[0] ? j : e];
+  for (unsigned i = 1; i < a.k; ++i) m = fmaxf(m, a.x[i][a.bcast[i] ? j : e]);
+  float s = 0.f;
+  for (unsigned i = 0; i < a.k; ++i) s += expf(a.x[i][a.bcast[i] ? j : e] - m);
+  fx[e] = logf(s) + m;
+}
+
+// dxi[e] += exp(xi[e] - fx[e]) * dEdf[e]
+__global__ __launch_bounds__(256) void lse_node_bwd_kernel(size_t total, const float* __restrict__ xi,
+                                                           const float* __restrict__ fx,
+                                                           const float* __restrict__ dEdf,
+                                                           float* __restrict__ dEdxi) {
+  const size_t e = size_t(blockIdx.x) * 256 + threadIdx.x;
+  if (e < total) dEdxi[e] += expf(xi[e] - fx[e]) * dEdf[e];
+}
+
+// broadcast argument: tmp[b*n + j] = exp(xi[j] - fx[b*n+j]) * dEdf[b*n+j]
+__global__ __launch_bounds__(256) void lse_node_bwd_bcast_kernel(size_t n, size_t total,
+                                                                 const float* __restrict__ xi,
+                                                                 const float* __restrict__ fx,
+                                                                 const float* __restrict__ dEdf,
+                                                                 float* __restrict__ tmp) {
+  const size_t e = size_t(blockIdx.x) * 256 + threadIdx.x;
+  if (e < total) tmp[e] = expf(xi[e % n] - fx[e]) * dEdf[e];
+}
+
+// ---- argmax along dim 0, first maximum ---------------------------------------
+__global__ __launch_bounds__(256) void argmax_cols_kernel(size_t rows, const float* __restrict__ x,
+                                                          long long* __restrict__ idx) {
+  __shared__ float lv[4];
+  __shared__ unsigned long long li[4];
+  const float* px = x + size_t(blockIdx.x) * rows;
+  float bv = -INFINITY;
+  unsigned long long bi = ~0ull;
+  for (size_t i = threadIdx.x; i < rows; i += 256) {
+    const float v = px[i];
+    if (bi == ~0ull || v > bv) {  // strided ascending i: strict > keeps the first maximum
+      bv = v;
+      bi = i;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, kWave);
+    const unsigned long long oi = __shfl_xor(bi, off, kWave);
+    if (oi != ~0ull && (bi == ~0ull || ov > bv || (ov == bv && oi < bi))) {
+      bv = ov;
+      bi = oi;
+    }
+  }
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  if (lane == 0) {
+    lv[w] = bv;
+    li[w] = bi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int k = 1; k < 4; ++k)
+      if (li[k] != ~0ull && (bi == ~0ull || lv[k] > bv || (lv[k] == bv && li[k] < bi))) {
+        bv = lv[k];
+        bi = li[k];
+      }
+    idx[blockIdx.x] = static_cast<long long>(bi);
+  }
+}
+
+int batch_reduce(dyhip_device* dev, size_t n, unsigned bd, const float* in0, const float* in1, float* out,
+                 bool accumulate, void* ws, size_t ws_bytes);
+
+static int launch_lse(dyhip_device* dev, size_t rows, unsigned bd, const float* x, float* m, float* z,
+                      const unsigned* ids, float* fx) {
+  const bool vec = rows % 4 == 0 && aligned16(x);
+  if (vec)
+    hipLaunchKernelGGL(lse_cols_kernel<true>, dim3(bd), dim3(kLseThreads), 0, dev->stream, rows, x, m, z, ids, fx);
+  else
+    hipLaunchKernelGGL(lse_cols_kernel<false>, dim3(bd), dim3(kLseThreads), 0, dev->stream, rows, x, m, z, ids, fx);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+}  // namespace dyhip
+
+using namespace dyhip;
+
+extern "C" {
+
+int dyhip_logsumexp_cols(dyhip_device* dev, size_t rows, unsigned bd, const float* x, float* m, float* z) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(rows >= 1 && x && m && z, "logsumexp needs a non-empty tensor");
+  if (bd == 0) return DYHIP_OK;
+  return launch_lse(dev, rows, bd, x, m, z, nullptr, nullptr);
+}
+
+int dyhip_pnls_forward(dyhip_device* dev, size_t rows, unsigned bd, const float* x, const unsigned* labels_host,
+                       void* aux, float* fx) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(rows >= 1 && x && labels_host && aux && fx, "PickNegLogSoftmax needs non-empty tensors");
+  if (bd == 0) return DYHIP_OK;
+  DYHIP_REQUIRE(rows * size_t(bd) <= (size_t(1) << 32), "PickNegLogSoftmax: %zu x %u elements overflow 32-bit ids",
+                rows, bd);
+  std::vector<unsigned> ids(bd);
+  for (unsigned b = 0; b < bd; ++b) {
+    DYHIP_REQUIRE(labels_host[b] < rows, "Index error in PickNegLogSoftmax: Index %u out of bounds for input tensor of %zu rows",
+                  labels_host[b], rows);
+    ids[b] = static_cast<unsigned>(rows * b + labels_host[b]);
+  }
+  float* z = static_cast<float*>(aux);
+  float* m = z + bd;
+  unsigned* ids_dev = reinterpret_cast<unsigned*>(m + bd);
+  // pageable source: the copy has been staged by the time the call returns
+  DYHIP_CHECK_HIP(hipMemcpyAsync(ids_dev, ids.data(), sizeof(unsigned) * bd, hipMemcpyHostToDevice, dev->stream));
+  DYHIP_CHECK_HIP(hipStreamSynchronize(dev->stream));
+  return launch_lse(dev, rows, bd, x, m, z, ids_dev, fx);
+}
+
+int dyhip_pnls_backward(dyhip_device* dev, size_t rows, unsigned bd, const float* x, const void* aux,
+                        const float* dEdf, float* dEdx) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(rows >= 1 && x && aux && dEdf && dEdx, "PickNegLogSoftmax needs non-empty tensors");
+  if (bd == 0) return DYHIP_OK;
+  const float* z = static_cast<const float*>(aux);
+  const unsigned* ids = reinterpret_cast<const unsigned*>(z + 2 * size_t(bd));
+  const bool vec = rows % 4 == 0 && aligned16(x) && aligned16(dEdx);
+  const size_t per_tile = size_t(kPbThreads) * kPbUnroll * (vec ? 4 : 1);
+  const size_t tiles = cdiv(rows, per_tile);
+  DYHIP_REQUIRE(tiles * bd < (size_t(1) << 31), "PickNegLogSoftmax backward launch too large");
+  const dim3 grid(static_cast<unsigned>(tiles * bd));
+  if (vec)
+    hipLaunchKernelGGL(pnls_bwd_kernel<true>, grid, dim3(kPbThreads), 0, dev->stream, rows, (unsigned)tiles, x, z, ids, dEdf, dEdx);
+  else
+    hipLaunchKernelGGL(pnls_bwd_kernel<false>, grid, dim3(kPbThreads), 0, dev->stream, rows, (unsigned)tiles, x, z, ids, dEdf, dEdx);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_logsumexp_node_forward(dyhip_device* dev, unsigned k, size_t n, unsigned bd, const float* const* xs_host,
+                                 const unsigned* bds_host, float* fx) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(k >= 1 && k <= kLseNodeMaxArgs, "LogSumExp supports 1..%u arguments (got %u)", kLseNodeMaxArgs, k);
+  DYHIP_REQUIRE(xs_host && bds_host && fx, "null pointer");
+  const size_t total = n * size_t(bd);
+  if (total == 0) return DYHIP_OK;
+  LseNodeArgs a;
+  a.k = k;
+  for (unsigned i = 0; i < k; ++i) {
+    DYHIP_REQUIRE(bds_host[i] == bd || bds_host[i] == 1, "Mismatched input dimensions in LogSumExp");
+    a.x[i] = xs_host[i];
+    a.bcast[i] = (bds_host[i] != bd) ? 1u : 0u;
+  }
+  hipLaunchKernelGGL(lse_node_fwd_kernel, dim3((unsigned)cdiv<size_t>(total, 256)), dim3(256), 0, dev->stream, a, n,
+                     total, fx);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_logsumexp_node_backward(dyhip_device* dev, unsigned k, size_t n, unsigned bd, const float* const* xs_host,
+                                  const unsigned* bds_host, const float* fx, const float* dEdf, unsigned i,
+                                  float* dEdxi, void* ws, size_t ws_bytes) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(k >= 1 && k <= kLseNodeMaxArgs && i < k, "bad argument index %u of %u", i, k);
+  DYHIP_REQUIRE(xs_host && bds_host && fx && dEdf && dEdxi, "null pointer");
+  const size_t total = n * size_t(bd);
+  if (total == 0) return DYHIP_OK;
+  const dim3 grid((unsigned)cdiv<size_t>(total, 256));
+  if (k == 1) return dyhip_accumulate(dev, total, dEdf, dEdxi);
+  if (bds_host[i] == bd) {
+    hipLaunchKernelGGL(lse_node_bwd_kernel, grid, dim3(256), 0, dev->stream, total, xs_host[i], fx, dEdf, dEdxi);
+    DYHIP_CHECK_LAUNCH();
+    return DYHIP_OK;
+  }
+  // broadcast argument: materialise the products, then reduce over the batch
+  size_t red = 0;
+  DYHIP_CHECK_STATUS(dyhip_batch_reduce_workspace(n, bd, &red));
+  const size_t tmp_bytes = cdiv<size_t>(total * sizeof(float), 256) * 256;
+  DYHIP_REQUIRE(ws != nullptr && ws_bytes >= tmp_bytes + red, "LogSumExp backward needs %zu workspace bytes, got %zu",
+                tmp_bytes + red, ws_bytes);
+  float* tmp = static_cast<float*>(ws);
+  hipLaunchKernelGGL(lse_node_bwd_bcast_kernel, grid, dim3(256), 0, dev->stream, n, total, xs_host[i], fx, dEdf, tmp);
+  DYHIP_CHECK_LAUNCH();
+  return batch_reduce(dev, n, bd, tmp, nullptr, dEdxi, true, static_cast<char*>(ws) + tmp_bytes, ws_bytes - tmp_bytes);
+}
+
+int dyhip_argmax_cols(dyhip_device* dev, size_t rows, unsigned bd, const float* x, long long* idx) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(rows >= 1 && x && idx, "argmax needs a non-empty tensor");
+  if (bd == 0) return DYHIP_OK;
+  hipLaunchKernelGGL(argmax_cols_kernel, dim3(bd), dim3(256), 0, dev->stream, rows, x, idx);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,426 @@
+"""Host-side mirror of DyNet's Device / pools / Tensor plumbing over the C-ABI.
+
+``Device`` owns a ``dyhip_device`` (one HIP stream, four bump pools FXS / DEDFS /
+PS / SCS, the three device scalars).  ``DevTensor`` is DyNet's ``Tensor`` reduced
+to what the kernels need: a device pointer plus a shape.  Every method is a
+direct call into ``libdynet_hip.so``; a non-zero status raises ``DyhipError``
+with the library's message (the adapter-side equivalent of rethrowing
+``dynet::cuda_exception`` / ``std::invalid_argument``).
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import lib
+from .lib import cdll
+
+_vp = C.c_void_p
+_sz = C.c_size_t
+_u = C.c_uint
+_f = C.c_float
+_i = C.c_int
+
+
+class DyhipError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__("dyhip status %d: %s" % (status, message))
+        self.status = status
+
+
+def _check(status):
+    if status != lib.OK:
+        raise DyhipError(status, lib.last_error())
+
+
+def device_count():
+    n = _i(0)
+    status = cdll.dyhip_device_count(C.byref(n))
+    if status == lib.ERR_NO_DEVICE:
+        return 0
+    _check(status)
+    return n.value
+
+
+class DevTensor:
+    """A device buffer with a shape (numpy order: batch outermost, DyNet's column-major inside)."""
+
+    __slots__ = ("dev", "ptr", "shape", "dtype")
+
+    def __init__(self, dev, ptr, shape, dtype=np.float32):
+        self.dev = dev
+        self.ptr = int(ptr)
+        self.shape = tuple(int(s) for s in shape)
+        self.dtype = np.dtype(dtype)
+
+    @property
+    def size(self):
+        return int(np.prod(self.shape)) if self.shape else 1
+
+    @property
+    def nbytes(self):
+        return self.size * self.dtype.itemsize
+
+    def numpy(self):
+        out = np.empty(self.shape, self.dtype)
+        if out.nbytes:
+            _check(cdll.dyhip_memcpy_d2h(self.dev.handle, _vp(out.ctypes.data), _vp(self.ptr), _sz(out.nbytes)))
+        return out
+
+    def set(self, array):
+        a = np.ascontiguousarray(array, dtype=self.dtype)
+        assert a.size == self.size, (a.shape, self.shape)
+        if a.nbytes:
+            _check(cdll.dyhip_memcpy_h2d(self.dev.handle, _vp(self.ptr), _vp(a.ctypes.data), _sz(a.nbytes)))
+            self.dev.sync()  # the source array may be a temporary
+        return self
+
+    def offset(self, elems, shape):
+        return DevTensor(self.dev, self.ptr + elems * self.dtype.itemsize, shape, self.dtype)
+
+
+def _p(t):
+    if t is None:
+        return _vp(None)
+    if isinstance(t, DevTensor):
+        return _vp(t.ptr)
+    return _vp(int(t))
+
+
+class Device:
+    """One GPU: stream, pools, scalars.  ``mem_mb`` = MiB for (FXS, DEDFS, PS, SCS)."""
+
+    def __init__(self, ordinal=0, mem_mb=(128, 128, 128, 128)):
+        self.handle = None
+        sizes = (_sz * 4)(*[int(m) for m in mem_mb])
+        h = _vp(None)
+        _check(cdll.dyhip_device_create(_i(ordinal), sizes, C.byref(h)))
+        self.handle = h
+        self.ordinal = ordinal
+
+    def close(self):
+        if self.handle is not None:
+            cdll.dyhip_device_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # ---- plumbing ---------------------------------------------------------
+    def sync(self):
+        _check(cdll.dyhip_device_sync(self.handle))
+
+    def pool(self, which):
+        p = _vp(None)
+        _check(cdll.dyhip_device_pool(self.handle, _i(which), C.byref(p)))
+        return Pool(p, owned=False)
+
+    def scalar_ptr(self, which):
+        p = _vp(None)
+        _check(cdll.dyhip_device_scalar(self.handle, _i(which), C.byref(p)))
+        return p.value
+
+    def alloc(self, nbytes, pool=lib.POOL_FXS):
+        p = _vp(None)
+        _check(cdll.dyhip_device_allocate(self.handle, _i(pool), _sz(int(nbytes)), C.byref(p)))
+        return p.value
+
+    def empty(self, shape, dtype=np.float32, pool=lib.POOL_FXS):
+        shape = (shape,) if np.isscalar(shape) else tuple(shape)
+        n = int(np.prod(shape)) if shape else 1
+        return DevTensor(self, self.alloc(max(n, 1) * np.dtype(dtype).itemsize, pool), shape, dtype)
+
+    def tensor(self, array, dtype=np.float32, pool=lib.POOL_FXS):
+        a = np.ascontiguousarray(array, dtype=dtype)
+        return self.empty(a.shape, dtype, pool).set(a)
+
+    def zeros(self, shape, dtype=np.float32, pool=lib.POOL_FXS):
+        t = self.empty(shape, dtype, pool)
+        _check(cdll.dyhip_zero(self.handle, _vp(t.ptr), _sz(t.nbytes)))
+        return t
+
+    def workspace(self, nbytes):
+        """Scratch from the SCS pool (what a DyNet node takes from pools[SCS])."""
+        nbytes = int(nbytes)
+        if nbytes == 0:
+            return None, 0
+        return self.alloc(nbytes, lib.POOL_SCS), nbytes
+
+    def free_pool(self, which):
+        self.pool(which).free()
+
+    def timer_start(self):
+        _check(cdll.dyhip_timer_start(self.handle))
+
+    def timer_stop(self):
+        ms = _f(0)
+        _check(cdll.dyhip_timer_stop(self.handle, C.byref(ms)))
+        return ms.value
+
+    def copy_d2d(self, dst, src, nbytes):
+        _check(cdll.dyhip_memcpy_d2d(self.handle, _p(dst), _p(src), _sz(int(nbytes))))
+
+    def zero(self, t):
+        _check(cdll.dyhip_zero(self.handle, _p(t), _sz(t.nbytes)))
+
+    def constant(self, t, value):
+        _check(cdll.dyhip_constant(self.handle, _sz(t.size), _f(value), _p(t)))
+
+    def accumulate(self, src, dst):
+        _check(cdll.dyhip_accumulate(self.handle, _sz(src.size), _p(src), _p(dst)))
+
+    # ---- elementwise ------------------------------------------------------
+    def unary_forward(self, op, x, y, logistic_mode=lib.LOGISTIC_PACKET, n=None):
+        _check(cdll.dyhip_unary_forward(self.handle, _i(op), _i(logistic_mode), _sz(x.size if n is None else n), _p(x),
+                                        _p(y)))
+
+    def unary_backward(self, op, fx, dEdf, dEdx, n=None):
+        _check(cdll.dyhip_unary_backward(self.handle, _i(op), _sz(fx.size if n is None else n), _p(fx), _p(dEdf),
+                                         _p(dEdx)))
+
+    def cmult_forward(self, n, bd0, bd1, a, b, y):
+        _check(cdll.dyhip_cmult_forward(self.handle, _sz(n), _u(bd0), _u(bd1), _p(a), _p(b), _p(y)))
+
+    def csum_forward(self, n, bd0, bd1, a, b, y):
+        _check(cdll.dyhip_csum_forward(self.handle, _sz(n), _u(bd0), _u(bd1), _p(a), _p(b), _p(y)))
+
+    def batch_reduce_workspace(self, n, bd):
+        b = _sz(0)
+        _check(cdll.dyhip_batch_reduce_workspace(_sz(n), _u(bd), C.byref(b)))
+        return b.value
+
+    def cmult_backward(self, n, bd0, bd1, a, b, dEdf, i, dEdxi):
+        ws, nb = self.workspace(self.batch_reduce_workspace(n, max(bd0, bd1)))
+        _check(cdll.dyhip_cmult_backward(self.handle, _sz(n), _u(bd0), _u(bd1), _p(a), _p(b), _p(dEdf), _u(i),
+                                         _p(dEdxi), _vp(ws), _sz(nb)))
+
+    def csum_backward(self, n, bd0, bd1, dEdf, i, dEdxi):
+        ws, nb = self.workspace(self.batch_reduce_workspace(n, max(bd0, bd1)))
+        _check(cdll.dyhip_csum_backward(self.handle, _sz(n), _u(bd0), _u(bd1), _p(dEdf), _u(i), _p(dEdxi), _vp(ws),
+                                        _sz(nb)))
+
+    # ---- reductions -------------------------------------------------------
+    def sum_batches_forward(self, n, bd, x, y, ws=None, ws_bytes=None):
+        if ws is None:
+            ws, ws_bytes = self.workspace(self.batch_reduce_workspace(n, bd))
+        _check(cdll.dyhip_sum_batches_forward(self.handle, _sz(n), _u(bd), _p(x), _p(y), _vp(ws), _sz(ws_bytes)))
+
+    def sum_batches_backward(self, n, bd, dEdf, dEdx):
+        _check(cdll.dyhip_sum_batches_backward(self.handle, _sz(n), _u(bd), _p(dEdf), _p(dEdx)))
+
+    def mean_elems_forward(self, n, bd, x, y):
+        _check(cdll.dyhip_mean_elems_forward(self.handle, _sz(n), _u(bd), _p(x), _p(y)))
+
+    def mean_elems_backward(self, n, bd, dEdf, dEdx):
+        _check(cdll.dyhip_mean_elems_backward(self.handle, _sz(n), _u(bd), _p(dEdf), _p(dEdx)))
+
+    def std_elems_forward(self, n, bd, x, y):
+        _check(cdll.dyhip_std_elems_forward(self.handle, _sz(n), _u(bd), _p(x), _p(y)))
+
+    def std_elems_backward(self, n, bd, x, fx, dEdf, dEdx):
+        _check(cdll.dyhip_std_elems_backward(self.handle, _sz(n), _u(bd), _p(x), _p(fx), _p(dEdf), _p(dEdx)))
+
+    # ---- layer norm -------------------------------------------------------
+    def layer_norm_forward(self, n, bd, x, g, b, y):
+        _check(cdll.dyhip_layer_norm_forward(self.handle, _sz(n), _u(bd), _p(x), _p(g), _p(b), _p(y)))
+
+    def layer_norm_backward_workspace(self, n, bd):
+        b = _sz(0)
+        _check(cdll.dyhip_layer_norm_backward_workspace(_sz(n), _u(bd), C.byref(b)))
+        return b.value
+
+    def layer_norm_backward(self, n, bd, x, g, dEdf, dx=None, dg=None, db=None, ws=None, ws_bytes=None):
+        if ws is None:
+            ws, ws_bytes = self.workspace(self.layer_norm_backward_workspace(n, bd))
+        _check(cdll.dyhip_layer_norm_backward(self.handle, _sz(n), _u(bd), _p(x), _p(g), _p(dEdf), _p(dx), _p(dg),
+                                              _p(db), _vp(ws), _sz(ws_bytes)))
+
+    # ---- GEMM -------------------------------------------------------------
+    def gemm_nn(self, M, N, K, l, r, beta, y):
+        _check(cdll.dyhip_gemm_nn(self.handle, _sz(M), _sz(N), _sz(K), _p(l), _p(r), _f(beta), _p(y)))
+
+    def gemm_tn_acc(self, M, N, K, l, r, y):
+        _check(cdll.dyhip_gemm_tn_acc(self.handle, _sz(M), _sz(N), _sz(K), _p(l), _p(r), _p(y)))
+
+    def gemm_nt_acc(self, M, N, K, l, r, y):
+        _check(cdll.dyhip_gemm_nt_acc(self.handle, _sz(M), _sz(N), _sz(K), _p(l), _p(r), _p(y)))
+
+    # ---- LSTM -------------------------------------------------------------
+    @staticmethod
+    def _xs(xs, x_dims):
+        ptrs = (_vp * len(xs))(*[(x.ptr if isinstance(x, DevTensor) else int(x)) for x in xs])
+        dims = (_u * len(xs))(*[int(d) for d in x_dims])
+        return ptrs, dims
+
+    def lstm_gates_forward(self, xs, x_dims, H, B, h_tm1, Wx, Wh, b, fx, mask_x=None, mask_x_bd=0, mask_h=None,
+                           mask_h_bd=0, logistic_mode=lib.LOGISTIC_PACKET):
+        ptrs, dims = self._xs(xs, x_dims)
+        need = _sz(0)
+        _check(cdll.dyhip_lstm_gates_workspace(_u(len(xs)), _u(sum(x_dims)), _u(H), _u(B),
+                                               _i(1 if mask_x is not None else 0), C.byref(need)))
+        ws, nb = self.workspace(need.value)
+        _check(cdll.dyhip_lstm_gates_forward(self.handle, _u(len(xs)), ptrs, dims, _u(H), _u(B), _p(h_tm1), _p(Wx),
+                                             _p(Wh), _p(b), _p(mask_x), _u(mask_x_bd), _p(mask_h), _u(mask_h_bd),
+                                             _i(logistic_mode), _p(fx), _vp(ws), _sz(nb)))
+
+    def lstm_gates_dpre(self, H, B, fx, dEdf, dpre):
+        _check(cdll.dyhip_lstm_gates_dpre(self.handle, _u(H), _u(B), _p(fx), _p(dEdf), _p(dpre)))
+
+    def lstm_gates_backward(self, xs, x_dims, H, B, h_tm1, Wx, Wh, fx, dEdf, i, dEdxi, dpre=None, mask_x=None,
+                            mask_x_bd=0, mask_h=None, mask_h_bd=0):
+        ptrs, dims = self._xs(xs, x_dims)
+        need = _sz(0)
+        _check(cdll.dyhip_lstm_gates_backward_workspace(_u(len(xs)), _u(sum(x_dims)), _u(H), _u(B),
+                                                        _i(1 if mask_x is not None else 0), C.byref(need)))
+        ws, nb = self.workspace(need.value)
+        _check(cdll.dyhip_lstm_gates_backward(self.handle, _u(len(xs)), ptrs, dims, _u(H), _u(B), _p(h_tm1), _p(Wx),
+                                              _p(Wh), _p(mask_x), _u(mask_x_bd), _p(mask_h), _u(mask_h_bd), _p(fx),
+                                              _p(dEdf), _p(dpre), _u(i), _p(dEdxi), _vp(ws), _sz(nb)))
+
+    def lstm_c_forward(self, H, B, c_tm1, gates, c):
+        _check(cdll.dyhip_lstm_c_forward(self.handle, _u(H), _u(B), _p(c_tm1), _p(gates), _p(c)))
+
+    def lstm_c_backward(self, H, B, c_tm1, gates, dEdf, i, dEdxi):
+        _check(cdll.dyhip_lstm_c_backward(self.handle, _u(H), _u(B), _p(c_tm1), _p(gates), _p(dEdf), _u(i),
+                                          _p(dEdxi)))
+
+    def lstm_h_forward(self, H, B, c, gates, h):
+        _check(cdll.dyhip_lstm_h_forward(self.handle, _u(H), _u(B), _p(c), _p(gates), _p(h)))
+
+    def lstm_h_backward(self, H, B, c, gates, dEdf, i, dEdxi):
+        _check(cdll.dyhip_lstm_h_backward(self.handle, _u(H), _u(B), _p(c), _p(gates), _p(dEdf), _u(i), _p(dEdxi)))
+
+    # ---- lookup -----------------------------------------------------------
+    def lookup_forward(self, ids_host, ids_dev, dim, vocab, table, fx, mult=1.0):
+        n = ids_dev.size
+        hp = _vp(None)
+        if ids_host is not None:
+            ids_host = np.ascontiguousarray(ids_host, dtype=np.uint32)
+            assert ids_host.size == n
+            hp = _vp(ids_host.ctypes.data)
+        _check(cdll.dyhip_lookup_forward(self.handle, _u(n), hp, _p(ids_dev), _sz(dim), _u(vocab), _p(table),
+                                         _f(mult), _p(fx)))
+
+    def lookup_accumulate_grads_workspace(self, n_ids, dim, vocab):
+        b = _sz(0)
+        _check(cdll.dyhip_lookup_accumulate_grads_workspace(_u(n_ids), _sz(dim), _u(vocab), C.byref(b)))
+        return b.value
+
+    def lookup_accumulate_grads(self, ids_dev, dim, vocab, g, all_grads, ws=None, ws_bytes=None):
+        n = ids_dev.size
+        if ws is None:
+            ws, ws_bytes = self.workspace(self.lookup_accumulate_grads_workspace(n, dim, vocab))
+        _check(cdll.dyhip_lookup_accumulate_grads(self.handle, _u(n), _p(ids_dev), _sz(dim), _u(vocab), _p(g),
+                                                  _p(all_grads), _vp(ws), _sz(ws_bytes)))
+
+    # ---- logsumexp / pnls -------------------------------------------------
+    def logsumexp_cols(self, rows, bd, x, m, z):
+        _check(cdll.dyhip_logsumexp_cols(self.handle, _sz(rows), _u(bd), _p(x), _p(m), _p(z)))
+
+    def pnls_forward(self, rows, bd, x, labels_host, aux, fx):
+        labels_host = np.ascontiguousarray(labels_host, dtype=np.uint32)
+        assert labels_host.size == bd
+        _check(cdll.dyhip_pnls_forward(self.handle, _sz(rows), _u(bd), _p(x), _vp(labels_host.ctypes.data), _p(aux),
+                                       _p(fx)))
+
+    def pnls_backward(self, rows, bd, x, aux, dEdf, dEdx):
+        _check(cdll.dyhip_pnls_backward(self.handle, _sz(rows), _u(bd), _p(x), _p(aux), _p(dEdf), _p(dEdx)))
+
+    def logsumexp_node_forward(self, n, bd, xs, bds, fx):
+        ptrs, b = self._xs(xs, bds)
+        _check(cdll.dyhip_logsumexp_node_forward(self.handle, _u(len(xs)), _sz(n), _u(bd), ptrs, b, _p(fx)))
+
+    def logsumexp_node_backward(self, n, bd, xs, bds, fx, dEdf, i, dEdxi):
+        ptrs, b = self._xs(xs, bds)
+        ws, nb = self.workspace(n * bd * 4 + 256 + self.batch_reduce_workspace(n, bd))
+        _check(cdll.dyhip_logsumexp_node_backward(self.handle, _u(len(xs)), _sz(n), _u(bd), ptrs, b, _p(fx), _p(dEdf),
+                                                  _u(i), _p(dEdxi), _vp(ws), _sz(nb)))
+
+    def argmax_cols(self, rows, bd, x, idx):
+        _check(cdll.dyhip_argmax_cols(self.handle, _sz(rows), _u(bd), _p(x), _p(idx)))
+
+    # ---- dynet::gpu helpers -----------------------------------------------
+    def dense_to_sparse_assign(self, n, ids, src, trg):
+        _check(cdll.dyhip_dense_to_sparse_assign(self.handle, _i(n), _p(ids), _p(src), _p(trg)))
+
+    def sparse_to_dense_assign(self, n, ids, src, trg):
+        _check(cdll.dyhip_sparse_to_dense_assign(self.handle, _i(n), _p(ids), _p(src), _p(trg)))
+
+    def dense_to_sparse_subtract(self, n, ids, src, trg):
+        _check(cdll.dyhip_dense_to_sparse_subtract(self.handle, _i(n), _p(ids), _p(src), _p(trg)))
+
+    def sparse_to_dense_block_assign_and_multiply(self, n, idx, bsize, mult, src, trg):
+        _check(cdll.dyhip_sparse_to_dense_block_assign_and_multiply(self.handle, _i(n), _p(idx), _i(bsize), _f(mult),
+                                                                    _p(src), _p(trg)))
+
+    def dense_to_sparse_block_add(self, n, ids, bsize, src, trg):
+        _check(cdll.dyhip_dense_to_sparse_block_add(self.handle, _i(n), _p(ids), _i(bsize), _p(src), _p(trg)))
+
+    def parallel_memcpy(self, num_seqs, max_len, src, trg, lens):
+        _check(cdll.dyhip_parallel_memcpy(self.handle, _i(num_seqs), _i(max_len), _p(src), _p(trg), _p(lens)))
+
+    def parallel_accumulate(self, num_seqs, max_len, src, trg, lens):
+        _check(cdll.dyhip_parallel_accumulate(self.handle, _i(num_seqs), _i(max_len), _p(src), _p(trg), _p(lens)))
+
+    # ---- parameter nodes / trainer ----------------------------------------
+    def scale_copy(self, n, src, mult, dst):
+        _check(cdll.dyhip_scale_copy(self.handle, _sz(n), _p(src), _f(mult), _p(dst)))
+
+    def sgd_update(self, n, p, g, lr, gscale=1.0, wd=1.0):
+        _check(cdll.dyhip_sgd_update(self.handle, _sz(n), _p(p), _p(g), _f(lr), _f(gscale), _f(wd)))
+
+    def squared_l2norm(self, n, g, out):
+        need = _sz(0)
+        _check(cdll.dyhip_squared_l2norm_workspace(_sz(n), C.byref(need)))
+        ws, nb = self.workspace(need.value)
+        _check(cdll.dyhip_squared_l2norm(self.handle, _sz(n), _p(g), _p(out), _vp(ws), _sz(nb)))
+
+
+class Pool:
+    """AlignedMemoryPool handle (device pools are borrowed from the Device; host pools are owned)."""
+
+    def __init__(self, handle, owned):
+        self.handle = handle
+        self.owned = owned
+
+    @classmethod
+    def create_host(cls, name, cap_bytes, expanding_unit=1 << 24):
+        h = _vp(None)
+        _check(cdll.dyhip_pool_create_host(name.encode(), _sz(cap_bytes), _sz(expanding_unit), C.byref(h)))
+        return cls(h, owned=True)
+
+    def destroy(self):
+        if self.owned and self.handle is not None:
+            cdll.dyhip_pool_destroy(self.handle)
+            self.handle = None
+
+    def allocate(self, nbytes):
+        p = _vp(None)
+        _check(cdll.dyhip_pool_allocate(self.handle, _sz(nbytes), C.byref(p)))
+        return p.value
+
+    def free(self):
+        _check(cdll.dyhip_pool_free(self.handle))
+
+    def zero_allocated(self):
+        _check(cdll.dyhip_pool_zero_allocated(self.handle))
+
+    def used(self):
+        v = _sz(0)
+        _check(cdll.dyhip_pool_used(self.handle, C.byref(v)))
+        return v.value
+
+    def set_used(self, n):
+        _check(cdll.dyhip_pool_set_used(self.handle, _sz(n)))
+
+    def capacity(self):
+        v = _sz(0)
+        _check(cdll.dyhip_pool_capacity(self.handle, C.byref(v)))
+        return v.value
+
+    def num_blocks(self):
+        v = _i(0)
+        _check(cdll.dyhip_pool_num_blocks(self.handle, C.byref(v)))
+        return v.value

@@ -1,0 +1,239 @@
+/*
+ * dynet_hip.h -- C-ABI of libdynet_hip.so, the MI355X (gfx950) implementation
+ * of the device layer and fused-layer kernels that sit behind DyNet's
+ * Node::forward_dev_impl / backward_dev_impl<Device_GPU>.
+ *
+ * Conventions
+ *  - Every entry point returns an int status (DYHIP_OK == 0), mirroring
+ *    DYNET_C_STATUS / DYNET_C_OK of contrib/c/dynet_c/define.h:42-46; no C++
+ *    exception crosses this boundary.  dyhip_last_error() gives the message of
+ *    the last failure on the calling thread.
+ *  - All tensors are fp32, column-major, batch outermost (dynet/dim.h:34-304):
+ *    element (i, j, b) of a rows x cols tensor is v[i + j*rows + b*rows*cols].
+ *    Indices are 32-bit unsigned.  Pointers are DEVICE pointers unless the
+ *    parameter name ends in _host.
+ *  - forward entry points overwrite their output; backward entry points
+ *    ACCUMULATE (+=) into the gradient buffer, exactly like every
+ *    backward_dev_impl (dynet/exec.cc:207-208 zeroes the buffers once).
+ *  - Kernels never allocate.  Scratch is passed in as (ws, ws_bytes); the size
+ *    needed comes from the matching *_workspace() query.  A DyNet adapter
+ *    takes it from pools[SCS] as the reference's nodes do
+ *    (dynet/nodes-lstm.cc:125,234).
+ *  - Launches are asynchronous on the device's single in-order stream
+ *    (the reference runs everything on the null stream, dynet/devices.cc:113);
+ *    dyhip_device_sync() or a D2H copy synchronises.
+ */
+#ifndef DYNET_HIP_H
+#define DYNET_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status ------------------------------------------------------------- */
+enum {
+  DYHIP_OK = 0,
+  DYHIP_ERR_INVALID_ARG = 1, /* std::invalid_argument in the reference (dynet/except.h:41-46) */
+  DYHIP_ERR_RUNTIME = 2,     /* dynet::cuda_exception / std::runtime_error (dynet/cuda.h:20-52) */
+  DYHIP_ERR_OUT_OF_MEMORY = 3, /* dynet::out_of_memory (dynet/except.h:11-14) */
+  DYHIP_ERR_NO_DEVICE = 4
+};
+const char* dyhip_last_error(void);
+
+/* ---- device: replaces Device_GPU (dynet/devices.h:46-61, devices.cc:91-121)
+ * and initialize_gpu's enumeration (dynet/cuda.cc:15-100) ------------------ */
+typedef struct dyhip_device dyhip_device;
+typedef struct dyhip_pool dyhip_pool;
+
+/* DeviceMempool (dynet/device-structs.h:15) */
+enum { DYHIP_POOL_FXS = 0, DYHIP_POOL_DEDFS = 1, DYHIP_POOL_PS = 2, DYHIP_POOL_SCS = 3 };
+/* the three device-resident scalars (dynet/devices.h:35-37, devices.cc:101-110) */
+enum { DYHIP_SCALAR_MINUSONE = 0, DYHIP_SCALAR_ONE = 1, DYHIP_SCALAR_ZERO = 2 };
+
+int dyhip_device_count(int* count);
+/* pool_mb[4] = FXS, DEDFS, PS, SCS sizes in MiB (DeviceMempoolSizes, devices.cc:17-57) */
+int dyhip_device_create(int ordinal, const size_t pool_mb[4], dyhip_device** out);
+int dyhip_device_destroy(dyhip_device* dev);
+int dyhip_device_sync(dyhip_device* dev);
+int dyhip_device_ordinal(const dyhip_device* dev, int* ordinal);
+int dyhip_device_stream(dyhip_device* dev, void** hip_stream);
+int dyhip_device_pool(dyhip_device* dev, int which, dyhip_pool** pool);
+int dyhip_device_scalar(dyhip_device* dev, int which, const float** ptr);
+/* Device::allocate_tensor (dynet/devices.cc:82-88) */
+int dyhip_device_allocate(dyhip_device* dev, int which_pool, size_t nbytes, void** out);
+
+/* ---- pools: AlignedMemoryPool / InternalMemoryPool
+ * (dynet/aligned-mem-pool.h:11-69, aligned-mem-pool.cc:8-91) over GPUAllocator
+ * (hipMalloc, 256-byte alignment; dynet/mem.h:41-47, mem.cc:71-90) or
+ * CPUAllocator (32-byte alignment; dynet/mem.h:26-31) --------------------- */
+int dyhip_pool_create_host(const char* name, size_t cap_bytes, size_t expanding_unit, dyhip_pool** out);
+int dyhip_pool_destroy(dyhip_pool* pool);
+int dyhip_pool_allocate(dyhip_pool* pool, size_t nbytes, void** out);
+int dyhip_pool_free(dyhip_pool* pool);
+int dyhip_pool_zero_allocated(dyhip_pool* pool);
+int dyhip_pool_used(dyhip_pool* pool, size_t* used);
+int dyhip_pool_set_used(dyhip_pool* pool, size_t used);
+int dyhip_pool_capacity(dyhip_pool* pool, size_t* cap);
+int dyhip_pool_num_blocks(dyhip_pool* pool, int* n);
+
+/* ---- copies: TensorTools::set_elements / as_vector / copy_elements / zero
+ * (dynet/tensor.cc:66-93,106-229) ----------------------------------------- */
+int dyhip_memcpy_h2d(dyhip_device* dev, void* dst, const void* src_host, size_t nbytes);
+int dyhip_memcpy_d2h(dyhip_device* dev, void* dst_host, const void* src, size_t nbytes); /* blocking */
+int dyhip_memcpy_d2d(dyhip_device* dev, void* dst, const void* src, size_t nbytes);
+int dyhip_zero(dyhip_device* dev, void* dst, size_t nbytes);
+int dyhip_constant(dyhip_device* dev, size_t n, float value, float* dst);       /* TensorTools::constant */
+int dyhip_accumulate(dyhip_device* dev, size_t n, const float* src, float* dst); /* TensorTools::accumulate: dst += src */
+
+/* stream-ordered timing for benchmarks (hipEvent pair on the device stream) */
+int dyhip_timer_start(dyhip_device* dev);
+int dyhip_timer_stop(dyhip_device* dev, float* elapsed_ms); /* blocks until the stop event */
+
+/* ---- elementwise nodes -------------------------------------------------- */
+/* operator codes */
+enum {
+  DYHIP_OP_TANH = 0,     /* Tanh            dynet/nodes-trig.cc:312-326 */
+  DYHIP_OP_LOGISTIC = 1, /* LogisticSigmoid dynet/nodes-activations.cc:65-78 */
+  DYHIP_OP_RECTIFY = 2,  /* Rectify         dynet/nodes-activations.cc:31-44 */
+  DYHIP_OP_NEGATE = 3,   /* Negate          dynet/nodes-arith-unary.cc:195-209 */
+  DYHIP_OP_IDENTITY = 4
+};
+/* which form of scalar_logistic_sigmoid_op (dynet/simd-functors.h:74-126) */
+enum {
+  DYHIP_LOGISTIC_PACKET = 0, /* packetOp: clamp +-18 + rational polynomial (what the CPU path runs on full SIMD packets) */
+  DYHIP_LOGISTIC_SCALAR = 1  /* operator(): 1/(1+exp(-x)) */
+};
+int dyhip_unary_forward(dyhip_device* dev, int op, int logistic_mode, size_t n, const float* x, float* y);
+int dyhip_unary_backward(dyhip_device* dev, int op, size_t n, const float* fx, const float* dEdf, float* dEdx);
+
+/* CwiseMultiply (dynet/nodes-arith-cwise.cc:196-307) and CwiseSum (:50-156) for
+ * equal dims; n = elements per batch element, bd0/bd1 = batch counts (equal,
+ * or one of them 1).  backward: i selects the argument. */
+int dyhip_cmult_forward(dyhip_device* dev, size_t n, unsigned bd0, unsigned bd1, const float* a, const float* b, float* y);
+int dyhip_cmult_backward(dyhip_device* dev, size_t n, unsigned bd0, unsigned bd1, const float* a, const float* b,
+                         const float* dEdf, unsigned i, float* dEdxi, void* ws, size_t ws_bytes);
+int dyhip_csum_forward(dyhip_device* dev, size_t n, unsigned bd0, unsigned bd1, const float* a, const float* b, float* y);
+int dyhip_csum_backward(dyhip_device* dev, size_t n, unsigned bd0, unsigned bd1, const float* dEdf, unsigned i,
+                        float* dEdxi, void* ws, size_t ws_bytes);
+
+/* ---- reductions --------------------------------------------------------- */
+/* workspace for every batch reduction of an n x bd tensor (sum_batches fwd,
+ * the broadcast-argument backward of cmult/csum) */
+int dyhip_batch_reduce_workspace(size_t n, unsigned bd, size_t* ws_bytes);
+/* SumDimension({}, include_batch_dim) = sum_batches (dynet/nodes-arith-sum.cc:197-248, expr.cc:218) */
+int dyhip_sum_batches_forward(dyhip_device* dev, size_t n, unsigned bd, const float* x, float* y, void* ws, size_t ws_bytes);
+int dyhip_sum_batches_backward(dyhip_device* dev, size_t n, unsigned bd, const float* dEdf, float* dEdx);
+/* mean_elems / std_elems (dynet/expr.cc:229-238; MomentDimension nodes-moments.cc:181-309,
+ * StdDimension :434-555): one value per batch element over its n elements */
+int dyhip_mean_elems_forward(dyhip_device* dev, size_t n, unsigned bd, const float* x, float* y);
+int dyhip_mean_elems_backward(dyhip_device* dev, size_t n, unsigned bd, const float* dEdf, float* dEdx);
+int dyhip_std_elems_forward(dyhip_device* dev, size_t n, unsigned bd, const float* x, float* y);
+int dyhip_std_elems_backward(dyhip_device* dev, size_t n, unsigned bd, const float* x, const float* fx,
+                             const float* dEdf, float* dEdx);
+
+/* ---- fused LayerNorm: the 8-node composite of dynet/expr.cc:248-253 in one
+ * kernel each way.  y = g * (x - mean) / (std + 1e-8f) + b per batch element.
+ * backward accumulates dx[n*bd], dg[n], db[n]; any of them may be NULL. ---- */
+int dyhip_layer_norm_forward(dyhip_device* dev, size_t n, unsigned bd, const float* x, const float* g,
+                             const float* b, float* y);
+int dyhip_layer_norm_backward_workspace(size_t n, unsigned bd, size_t* ws_bytes);
+int dyhip_layer_norm_backward(dyhip_device* dev, size_t n, unsigned bd, const float* x, const float* g,
+                              const float* dEdf, float* dx, float* dg, float* db, void* ws, size_t ws_bytes);
+
+/* ---- GEMM shim: dynet/matrix-multiply.h, fp32 in / fp32 accumulate on MFMA.
+ * The device-pointer acc_scalar of the reference (kSCALAR_ONE / kSCALAR_ZERO)
+ * becomes the by-value beta. ---------------------------------------------- */
+/* MatrixMultiply (:16-37): y[MxN] = beta*y + l[MxK] * r[KxN] */
+int dyhip_gemm_nn(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float beta, float* y);
+/* MatrixTranspMultiplyAcc (:97-117): y[MxN] += l[KxM]^T * r[KxN] */
+int dyhip_gemm_tn_acc(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float* y);
+/* MatrixMultiplyTranspAcc (:162-180): y[MxN] += l[MxK] * r[NxK]^T */
+int dyhip_gemm_nt_acc(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float* y);
+
+/* ---- fused LSTM nodes (dynet/nodes-lstm.cc) ------------------------------ */
+/* VanillaLSTMGates::forward_dev_impl (:101-235).  xs[k] (HOST array of DEVICE
+ * pointers) has x_dims[k] rows and B columns; mask_x/mask_h NULL = no dropout,
+ * else their batch counts are B or 1.  Gate order i, f, o, g; +1 forget bias
+ * is applied inside.  Workspace is only needed for num_inputs > 1 or dropout. */
+int dyhip_lstm_gates_workspace(unsigned num_inputs, unsigned I, unsigned H, unsigned B, int dropout, size_t* ws_bytes);
+int dyhip_lstm_gates_forward(dyhip_device* dev, unsigned num_inputs, const float* const* xs_host,
+                             const unsigned* x_dims_host, unsigned H, unsigned B, const float* h_tm1,
+                             const float* Wx, const float* Wh, const float* b, const float* mask_x,
+                             unsigned mask_x_bd, const float* mask_h, unsigned mask_h_bd, int logistic_mode,
+                             float* fx, void* ws, size_t ws_bytes);
+/* dpre = [dEdf*fx*(1-fx) rows 0..3H ; dEdf*(1-fx^2) rows 3H..4H] (:358-361), computed once */
+int dyhip_lstm_gates_dpre(dyhip_device* dev, unsigned H, unsigned B, const float* fx, const float* dEdf, float* dpre);
+/* VanillaLSTMGates::backward_dev_impl (:237-527) for argument i (inputs, then
+ * h, Wx, Wh, b).  dpre may be NULL: it is then recomputed into the workspace,
+ * as the reference does on each of its five calls. */
+int dyhip_lstm_gates_backward_workspace(unsigned num_inputs, unsigned I, unsigned H, unsigned B, int dropout, size_t* ws_bytes);
+int dyhip_lstm_gates_backward(dyhip_device* dev, unsigned num_inputs, const float* const* xs_host,
+                              const unsigned* x_dims_host, unsigned H, unsigned B, const float* h_tm1,
+                              const float* Wx, const float* Wh, const float* mask_x, unsigned mask_x_bd,
+                              const float* mask_h, unsigned mask_h_bd, const float* fx, const float* dEdf,
+                              const float* dpre, unsigned i, float* dEdxi, void* ws, size_t ws_bytes);
+/* VanillaLSTMC (:562-615) and VanillaLSTMH (:650-703) */
+int dyhip_lstm_c_forward(dyhip_device* dev, unsigned H, unsigned B, const float* c_tm1, const float* gates, float* c);
+int dyhip_lstm_c_backward(dyhip_device* dev, unsigned H, unsigned B, const float* c_tm1, const float* gates,
+                          const float* dEdf, unsigned i, float* dEdxi);
+int dyhip_lstm_h_forward(dyhip_device* dev, unsigned H, unsigned B, const float* c, const float* gates, float* h);
+int dyhip_lstm_h_backward(dyhip_device* dev, unsigned H, unsigned B, const float* c, const float* gates,
+                          const float* dEdf, unsigned i, float* dEdxi);
+
+/* ---- LookupNode (dynet/param-nodes.cc:304-329) and
+ * LookupParameterStorage::accumulate_grads (dynet/model.cc:728-743) -------- */
+/* fx[:, b] = table[:, ids[b]] * mult; bit-exact gather when mult == 1.0f.
+ * ids_host (may be NULL) is bounds-checked against vocab like the CPU path
+ * (:323) and copied to ids_dev (the node's aux_mem, :318). */
+int dyhip_lookup_forward(dyhip_device* dev, unsigned n_ids, const unsigned* ids_host, unsigned* ids_dev,
+                         size_t dim, unsigned vocab, const float* table, float mult, float* fx);
+/* all_grads[:, ids[b]] += g[:, b], duplicates summed in ascending b by a
+ * sorted-index segmented reduction (no atomics, deterministic). */
+int dyhip_lookup_accumulate_grads_workspace(unsigned n_ids, size_t dim, unsigned vocab, size_t* ws_bytes);
+int dyhip_lookup_accumulate_grads(dyhip_device* dev, unsigned n_ids, const unsigned* ids_dev, size_t dim,
+                                  unsigned vocab, const float* g, float* all_grads, void* ws, size_t ws_bytes);
+
+/* ---- logsumexp / PickNegLogSoftmax / LogSumExp / argmax ------------------ */
+/* TensorTools::logsumexp_dev (dynet/tensor.cc:468-507), vector per batch element */
+int dyhip_logsumexp_cols(dyhip_device* dev, size_t rows, unsigned bd, const float* x, float* m, float* z);
+/* PickNegLogSoftmax (dynet/nodes-pickneglogsoftmax.cc:72-145).  aux (device,
+ * 3*bd*4 bytes, :72-74) = [z | m | ids] with ids[b] = b*rows + label_b;
+ * labels_host are bounds-checked (:100). */
+int dyhip_pnls_forward(dyhip_device* dev, size_t rows, unsigned bd, const float* x, const unsigned* labels_host,
+                       void* aux, float* fx);
+int dyhip_pnls_backward(dyhip_device* dev, size_t rows, unsigned bd, const float* x, const void* aux,
+                        const float* dEdf, float* dEdx);
+/* LogSumExp node over k <= 8 arguments (dynet/nodes-logsumexp.cc:38-97) */
+int dyhip_logsumexp_node_forward(dyhip_device* dev, unsigned k, size_t n, unsigned bd, const float* const* xs_host,
+                                 const unsigned* bds_host, float* fx);
+int dyhip_logsumexp_node_backward(dyhip_device* dev, unsigned k, size_t n, unsigned bd, const float* const* xs_host,
+                                  const unsigned* bds_host, const float* fx, const float* dEdf, unsigned i,
+                                  float* dEdxi, void* ws, size_t ws_bytes);
+/* TensorTools::argmax_dev along dim 0 (dynet/tensor.cc:527-538): first maximum, 64-bit indices */
+int dyhip_argmax_cols(dyhip_device* dev, size_t rows, unsigned bd, const float* x, long long* idx);
+
+/* ---- dynet::gpu::* helpers (dynet/gpu-ops.h:9-15), same argument lists ---- */
+int dyhip_dense_to_sparse_assign(dyhip_device* dev, int n, const unsigned* ids, const float* src, float* trg);
+int dyhip_sparse_to_dense_assign(dyhip_device* dev, int n, const unsigned* ids, const float* src, float* trg);
+int dyhip_dense_to_sparse_subtract(dyhip_device* dev, int n, const unsigned* ids, const float* src, float* trg);
+int dyhip_sparse_to_dense_block_assign_and_multiply(dyhip_device* dev, int n, const unsigned* idx, int bsize,
+                                                    float mult, const float* src, float* trg);
+int dyhip_dense_to_sparse_block_add(dyhip_device* dev, int n, const unsigned* ids, int bsize, const float* src, float* trg);
+int dyhip_parallel_memcpy(dyhip_device* dev, int num_seqs, int max_len, float** src, float** trg, size_t* len);
+int dyhip_parallel_accumulate(dyhip_device* dev, int num_seqs, int max_len, float** src, float** trg, size_t* len);
+
+/* ---- parameter nodes / trainer ------------------------------------------- */
+/* ParameterNode::forward_dev_impl (dynet/param-nodes.cc:201-215): dst = src * mult */
+int dyhip_scale_copy(dyhip_device* dev, size_t n, const float* src, float mult, float* dst);
+/* SimpleSGDTrainer::update_rule_dev (dynet/training.cc:619-622): p -= g * (lr*gscale/wd) */
+int dyhip_sgd_update(dyhip_device* dev, size_t n, float* p, const float* g, float lr, float gscale, float wd);
+/* ParameterStorage::g_squared_l2norm_dev (dynet/model.cc): *out(device) = sum g^2 */
+int dyhip_squared_l2norm_workspace(size_t n, size_t* ws_bytes);
+int dyhip_squared_l2norm(dyhip_device* dev, size_t n, const float* g, float* out, void* ws, size_t ws_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -23,3 +23,24 @@ def golden():
             with open(os.path.join(gdir, name)) as f:
                 out[name[:-5]] = json.load(f)
     return out
+
+
+@pytest.fixture(scope="session")
+def gpu():
+    """One Device for the whole GPU session.  Fails loudly without a GPU: there is no fallback."""
+    from dynet_amd import Device
+
+    dev = Device(0, mem_mb=(3072, 2048, 1024, 1024))
+    yield dev
+    dev.close()
+
+
+@pytest.fixture()
+def dev(gpu):
+    """Per-test view of the device with the graph pools (FXS, DEDFS, SCS) reset."""
+    from dynet_amd import lib
+
+    gpu.sync()
+    for which in (lib.POOL_FXS, lib.POOL_DEDFS, lib.POOL_SCS):
+        gpu.free_pool(which)
+    return gpu

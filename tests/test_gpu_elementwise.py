@@ -1,0 +1,238 @@
+"""GPU parity: elementwise nodes, reductions and the fused LayerNorm against the
+CPU oracle on identical seeded inputs, through the C-ABI.
+
+Sizes: the configuration named by the baseline (a 4096 x 1024 fp32 tensor;
+sum_batches as Dim({64,1024}, bd 64); layer_norm as Dim({1024}, bd 4096) with
+g ~ U(0.5,1.5), b ~ N(0,0.1)) plus ragged / misaligned / tiny edge cases.
+"""
+import numpy as np
+import pytest
+
+from dynet_amd import lib
+from oracle import cpu_oracle as orc
+from util import F32, FWD_RTOL, GRAD_RTOL, assert_close, f32, rms
+
+pytestmark = pytest.mark.gpu
+
+N_BIG = 4096 * 1024
+OPS = [(lib.OP_TANH, "tanh"), (lib.OP_LOGISTIC, "logistic"), (lib.OP_RECTIFY, "rectify"), (lib.OP_NEGATE, "negate")]
+
+
+def _inputs(n, seed):
+    rng = np.random.default_rng(seed)
+    x = f32(rng.standard_normal(n))
+    if n >= 8:
+        x[:8] = [0.0, -0.0, 1e-4, -1e-4, 20.0, -20.0, 9.0, -7.5]  # tails and the zero of ReLU
+    return x, f32(rng.standard_normal(n)), f32(rng.standard_normal(n))
+
+
+@pytest.mark.parametrize("op,name", OPS)
+@pytest.mark.parametrize("n", [N_BIG, 1027, 3, 1])
+def test_unary_forward_backward(dev, op, name, n):
+    x, dy, dx0 = _inputs(n, 100 + op)
+    dx_t = dev.tensor(x)
+    y_t = dev.empty(n)
+    dev.unary_forward(op, dx_t, y_t)
+    y = y_t.numpy()
+    ref = orc.unary_forward(op, x)
+    if op in (lib.OP_RECTIFY, lib.OP_NEGATE):
+        assert y.tobytes() == ref.tobytes()
+    else:
+        assert_close(y, ref, FWD_RTOL, name + " fwd")
+    # backward accumulates into a non-zero gradient buffer, from the oracle's fx
+    g_t = dev.tensor(dx0)
+    dev.unary_backward(op, dev.tensor(ref), dev.tensor(dy), g_t)
+    want = orc.unary_backward(op, ref, dy, dx0.copy())
+    assert_close(g_t.numpy(), want, GRAD_RTOL, name + " bwd", floor=1e-6)
+
+
+def test_logistic_packet_form_is_bit_exact_and_scalar_form_is_accurate(dev):
+    x, _, _ = _inputs(1 << 20, 7)
+    x[8:4096] = np.linspace(-30, 30, 4088)
+    xt, yt = dev.tensor(x), dev.empty(x.size)
+    dev.unary_forward(lib.OP_LOGISTIC, xt, yt, lib.LOGISTIC_PACKET)
+    assert yt.numpy().tobytes() == orc.unary_forward(orc.OP_LOGISTIC, x, orc.LOGISTIC_PACKET).tobytes()
+    dev.unary_forward(lib.OP_LOGISTIC, xt, yt, lib.LOGISTIC_SCALAR)
+    assert_close(yt.numpy(), orc.unary_forward(orc.OP_LOGISTIC, x, orc.LOGISTIC_SCALAR), FWD_RTOL, "logistic scalar")
+
+
+def test_tanh_is_relatively_accurate_everywhere(dev):
+    x = f32(np.concatenate([np.linspace(-12, 12, 200001), np.logspace(-30, 1, 4000), -np.logspace(-30, 1, 4000)]))
+    yt = dev.empty(x.size)
+    dev.unary_forward(lib.OP_TANH, dev.tensor(x), yt)
+    ref = np.tanh(x.astype(np.float64))
+    err = np.abs(yt.numpy() - ref)
+    assert np.max(err / np.maximum(np.abs(ref), 1e-37)) < 1e-6
+
+
+def test_unary_on_a_misaligned_buffer(dev):
+    x, dy, dx0 = _inputs(4099, 11)
+    base = dev.tensor(np.concatenate([[0.0], x]))  # view starting 4 bytes into the allocation
+    xt = base.offset(1, (4099,))
+    ybase = dev.zeros(4100)
+    dev.unary_forward(lib.OP_TANH, xt, ybase.offset(1, (4099,)))
+    out = ybase.numpy()
+    assert out[0] == 0.0
+    assert_close(out[1:], orc.unary_forward(orc.OP_TANH, x), FWD_RTOL, "misaligned tanh")
+
+
+def test_unary_rejects_unknown_operator(dev):
+    from dynet_amd import DyhipError
+
+    t = dev.zeros(4)
+    with pytest.raises(DyhipError) as e:
+        dev.unary_forward(99, t, t)
+    assert e.value.status == lib.ERR_INVALID_ARG
+
+
+@pytest.mark.parametrize("n,bd0,bd1", [(N_BIG // 64, 64, 64), (1024, 4096, 1), (1024, 1, 4096), (7, 5, 1), (5, 1, 1)])
+def test_cmult_and_csum(dev, n, bd0, bd1):
+    rng = np.random.default_rng(21)
+    bd = max(bd0, bd1)
+    a, b = f32(rng.standard_normal((bd0, n))), f32(rng.standard_normal((bd1, n)))
+    dy = f32(rng.standard_normal((bd, n)))
+    at, bt, dyt = dev.tensor(a), dev.tensor(b), dev.tensor(dy)
+    yt = dev.empty((bd, n))
+    dev.cmult_forward(n, bd0, bd1, at, bt, yt)
+    assert yt.numpy().tobytes() == orc.cmult_forward(n, bd0, bd1, a, b).tobytes()
+    dev.csum_forward(n, bd0, bd1, at, bt, yt)
+    assert yt.numpy().tobytes() == orc.csum_forward(n, bd0, bd1, a, b).tobytes()
+    for i, (bdi, other) in enumerate(((bd0, b), (bd1, a))):
+        g0 = f32(rng.standard_normal((bdi, n)))
+        gt = dev.tensor(g0)
+        dev.cmult_backward(n, bd0, bd1, at, bt, dyt, i, gt)
+        want = orc.cmult_backward(n, bd0, bd1, a, b, dy, i, g0.copy())
+        floor = rms(dy) * rms(other) * np.sqrt(bd if bdi != bd else 1)
+        assert_close(gt.numpy(), want, GRAD_RTOL, "cmult bwd %d" % i, floor=floor)
+        gt = dev.tensor(g0)
+        dev.csum_backward(n, bd0, bd1, dyt, i, gt)
+        want = orc.csum_backward(n, bd0, bd1, dy, i, g0.copy())
+        assert_close(gt.numpy(), want, GRAD_RTOL, "csum bwd %d" % i, floor=rms(dy) * np.sqrt(bd if bdi != bd else 1))
+
+
+@pytest.mark.parametrize("n,bd", [(64 * 1024, 64), (1024, 4096), (1027, 33), (3, 2), (5, 1), (4096, 7)])
+def test_sum_batches(dev, n, bd):
+    rng = np.random.default_rng(31)
+    x = f32(rng.standard_normal((bd, n)))
+    yt = dev.empty(n)
+    dev.sum_batches_forward(n, bd, dev.tensor(x), yt)
+    ref = orc.sum_batches_forward(n, bd, x)
+    assert_close(yt.numpy(), ref, FWD_RTOL, "sum_batches fwd", floor=np.sqrt(bd))
+    # the batch order does not matter beyond rounding: compare with fp64 too
+    assert_close(yt.numpy(), x.astype(np.float64).sum(0), FWD_RTOL, "sum_batches vs fp64", floor=np.sqrt(bd))
+    dy, g0 = f32(rng.standard_normal(n)), f32(rng.standard_normal((bd, n)))
+    gt = dev.tensor(g0)
+    dev.sum_batches_backward(n, bd, dev.tensor(dy), gt)
+    assert gt.numpy().tobytes() == orc.sum_batches_backward(n, bd, dy, g0.copy()).tobytes()
+
+
+def test_sum_batches_golden_cadd_broadcast2_neg_val(dev, golden):
+    g = golden["node_values"]
+    x1 = dev.tensor(f32(g["fixture_params"]["param1"]).reshape(1, 3))
+    x2 = dev.tensor(f32(g["fixture_params"]["param4"]).reshape(2, 3))
+    neg, y, z = dev.empty((2, 3)), dev.empty((2, 3)), dev.empty(3)
+    dev.unary_forward(lib.OP_NEGATE, x2, neg)
+    dev.csum_forward(3, 1, 2, x1, neg, y)
+    dev.sum_batches_forward(3, 2, y, z)
+    exp = g["cadd_broadcast2_neg_val"]
+    assert abs(float(z.numpy().astype(np.float64).sum()) - exp["expected"]) <= exp["rel_tol"] * abs(exp["expected"])
+
+
+@pytest.mark.parametrize("n,bd", [(1024, 4096), (9, 3), (1000, 17), (1, 4)])
+def test_mean_std_elems(dev, n, bd):
+    rng = np.random.default_rng(41)
+    x = f32(rng.standard_normal((bd, n)) + 0.5)
+    xt = dev.tensor(x)
+    mt, st = dev.empty(bd), dev.empty(bd)
+    dev.mean_elems_forward(n, bd, xt, mt)
+    dev.std_elems_forward(n, bd, xt, st)
+    assert_close(mt.numpy(), orc.mean_elems_forward(n, bd, x), FWD_RTOL, "mean_elems", floor=1.0 / np.sqrt(n))
+    sd_ref = orc.std_elems_forward(n, bd, x)
+    assert_close(st.numpy(), sd_ref, FWD_RTOL, "std_elems", floor=1e-6)
+    if n > 1:
+        dy, g0 = f32(rng.standard_normal(bd)), f32(rng.standard_normal((bd, n)))
+        gt = dev.tensor(g0)
+        dev.mean_elems_backward(n, bd, dev.tensor(dy), gt)
+        assert_close(gt.numpy(), orc.mean_elems_backward(n, bd, dy, g0.copy()), GRAD_RTOL, "mean bwd", floor=1e-6)
+        gt = dev.tensor(g0)
+        dev.std_elems_backward(n, bd, xt, dev.tensor(sd_ref), dev.tensor(dy), gt)
+        assert_close(gt.numpy(), orc.std_elems_backward(n, bd, x, sd_ref, dy, g0.copy()), GRAD_RTOL, "std bwd",
+                     floor=1e-3)
+
+
+def test_std_golden_std_dim_value(dev, golden):
+    g = golden["node_values"]
+    x = f32(g["fixture_params"]["param_cube1"]).reshape(3, 3, 3)
+    cols = np.ascontiguousarray(np.stack([x[:, j, :].reshape(-1) for j in range(3)]))
+    y, z = dev.empty(3), dev.empty(1)
+    dev.std_elems_forward(9, 3, dev.tensor(cols), y)
+    dev.mean_elems_forward(3, 1, y, z)
+    exp = g["std_dim_value"]
+    assert abs(float(z.numpy()[0]) - exp["expected"]) <= exp["rel_tol"] * exp["expected"]
+
+
+# ---------------------------------------------------------------------------
+# fused LayerNorm
+# ---------------------------------------------------------------------------
+def _ln_case(n, bd, seed):
+    rng = np.random.default_rng(seed)
+    x = f32(rng.standard_normal((bd, n)))
+    g = f32(rng.uniform(0.5, 1.5, n))
+    b = f32(rng.standard_normal(n) * 0.1)
+    dy = f32(rng.standard_normal((bd, n)))
+    return rng, x, g, b, dy
+
+
+@pytest.mark.parametrize("n,bd", [(1024, 4096), (2048, 64), (512, 33), (256, 5), (64, 1), (12, 7), (1027, 9),
+                                  (4096, 6), (3, 1)])
+def test_layer_norm_forward_backward(dev, n, bd):
+    rng, x, g, b, dy = _ln_case(n, bd, 51)
+    xt, gt, bt, dyt = dev.tensor(x), dev.tensor(g), dev.tensor(b), dev.tensor(dy)
+    yt = dev.empty((bd, n))
+    dev.layer_norm_forward(n, bd, xt, gt, bt, yt)
+    ref = orc.layer_norm_forward(n, bd, x, g, b)
+    # y = g*q + b with |g*q| ~ 1: relative to the size of the terms
+    assert_close(yt.numpy(), ref, FWD_RTOL, "layer_norm fwd", floor=1.0)
+    dx0, dg0, db0 = f32(rng.standard_normal((bd, n))), f32(rng.standard_normal(n)), f32(rng.standard_normal(n))
+    dxt, dgt, dbt = dev.tensor(dx0), dev.tensor(dg0), dev.tensor(db0)
+    dev.layer_norm_backward(n, bd, xt, gt, dyt, dxt, dgt, dbt)
+    wx, wg, wb = orc.layer_norm_backward(n, bd, x, g, dy, dx0.copy(), dg0.copy(), db0.copy())
+    assert_close(dxt.numpy(), wx, GRAD_RTOL, "layer_norm dx", floor=1.0)
+    assert_close(dgt.numpy(), wg, GRAD_RTOL, "layer_norm dg", floor=np.sqrt(bd))
+    assert_close(dbt.numpy(), wb, GRAD_RTOL, "layer_norm db", floor=np.sqrt(bd))
+    # one argument at a time, as Node::backward is called
+    dxt2 = dev.tensor(dx0)
+    dev.layer_norm_backward(n, bd, xt, gt, dyt, dx=dxt2)
+    assert dxt2.numpy().tobytes() == dxt.numpy().tobytes()
+    dgt2 = dev.tensor(dg0)
+    dev.layer_norm_backward(n, bd, xt, gt, dyt, dg=dgt2)
+    assert dgt2.numpy().tobytes() == dgt.numpy().tobytes()
+
+
+def test_layer_norm_golden_vectors(dev, golden):
+    g = golden["node_values"]
+    x = f32(g["fixture_params"]["param1"]).reshape(1, 3)
+    yt = dev.empty((1, 3))
+    dev.layer_norm_forward(3, 1, dev.tensor(x), dev.tensor(np.ones(3, F32)), dev.tensor(np.zeros(3, F32)), yt)
+    y = yt.numpy().astype(np.float64)
+    exp = g["layer_norm_forward"]
+    assert abs(y.sum() / 3.0) < exp["mean_abs_max"]
+    assert abs(np.sqrt((y ** 2).sum() / 3.0) - exp["rms"]) <= exp["rms_rel_tol"]
+    exp = g["layer_norm_python"]
+    v = np.arange(exp["n"]).astype(np.float64)
+    vt = dev.tensor(f32(v))
+    yt = dev.empty((1, exp["n"]))
+    dev.layer_norm_forward(exp["n"], 1, vt, vt, vt, yt)
+    assert np.allclose(yt.numpy().reshape(-1), v / v.std() * (v - v.mean()) + v, rtol=exp["rtol"], atol=exp["atol"])
+
+
+def test_layer_norm_invariances_at_full_size(dev):
+    n, bd = 1024, 4096
+    _, x, g, b, _ = _ln_case(n, bd, 52)
+    gt, bt = dev.tensor(g), dev.tensor(b)
+    y0, y1 = dev.empty((bd, n)), dev.empty((bd, n))
+    dev.layer_norm_forward(n, bd, dev.tensor(x), gt, bt, y0)
+    dev.layer_norm_forward(n, bd, dev.tensor(x * F32(4.0)), gt, bt, y1)  # exact power-of-two scaling
+    assert_close(y1.numpy(), y0.numpy(), FWD_RTOL, "LN(4x) == LN(x)", floor=1.0)
+    dev.layer_norm_forward(n, bd, dev.tensor(x + F32(2.0)), gt, bt, y1)
+    assert_close(y1.numpy(), y0.numpy(), 5e-5, "LN(x+2) == LN(x)", floor=1.0)

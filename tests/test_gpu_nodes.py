@@ -1,0 +1,443 @@
+"""GPU parity: GEMM shim, fused LSTM nodes, LookupNode, PickNegLogSoftmax /
+logsumexp / argmax, the dynet::gpu helpers and the trainer kernels against the
+CPU oracle on identical seeded inputs, through the C-ABI.
+"""
+import numpy as np
+import pytest
+
+from dynet_amd import DyhipError, lib
+from oracle import cpu_oracle as orc
+from util import F32, FWD_RTOL, GRAD_RTOL, assert_close, f32, glorot, rms, zipf_ids
+
+pytestmark = pytest.mark.gpu
+
+
+# ---------------------------------------------------------------------------
+# GEMM shim
+# ---------------------------------------------------------------------------
+GEMM_SHAPES = [(1024, 32, 128), (1024, 32, 256), (4096, 128, 1280), (256, 128, 4096), (130, 33, 17), (5, 4, 6),
+               (64, 1, 64), (1000, 128, 1024), (129, 65, 100)]
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+def test_gemm_three_forms(dev, M, N, K):
+    rng = np.random.default_rng(M * 7 + N * 3 + K)
+    y0 = f32(rng.standard_normal((N, M)))
+    floor = np.sqrt(K)  # size of the sum of K products of N(0,1) terms
+    # NN: y = beta*y + l*r
+    l, r = f32(rng.standard_normal((K, M))), f32(rng.standard_normal((N, K)))
+    lt, rt = dev.tensor(l), dev.tensor(r)
+    for beta in (1.0, 0.0):
+        yt = dev.tensor(y0)
+        dev.gemm_nn(M, N, K, lt, rt, beta, yt)
+        assert_close(yt.numpy(), orc.gemm_nn(M, N, K, l, r, beta, y0.copy()), FWD_RTOL, "gemm_nn beta=%g" % beta,
+                     floor=floor)
+    # TN: y += l^T r with l stored K x M
+    l2 = f32(rng.standard_normal((M, K)))
+    yt = dev.tensor(y0)
+    dev.gemm_tn_acc(M, N, K, dev.tensor(l2), rt, yt)
+    assert_close(yt.numpy(), orc.gemm_tn_acc(M, N, K, l2, r, y0.copy()), FWD_RTOL, "gemm_tn", floor=floor)
+    # NT: y += l r^T with r stored N x K
+    r2 = f32(rng.standard_normal((K, N)))
+    yt = dev.tensor(y0)
+    dev.gemm_nt_acc(M, N, K, lt, dev.tensor(r2), yt)
+    assert_close(yt.numpy(), orc.gemm_nt_acc(M, N, K, l, r2, y0.copy()), FWD_RTOL, "gemm_nt", floor=floor)
+
+
+def test_gemm_is_fp32_accurate_against_fp64(dev):
+    """No reduced-precision shortcut on the matrix cores: error vs fp64 stays at fp32 rounding level."""
+    rng = np.random.default_rng(5)
+    M, N, K = 512, 64, 2048
+    l, r = f32(rng.standard_normal((K, M))), f32(rng.standard_normal((N, K)))
+    yt = dev.zeros((N, M))
+    dev.gemm_nn(M, N, K, dev.tensor(l), dev.tensor(r), 0.0, yt)
+    want = r.astype(np.float64) @ l.astype(np.float64)
+    assert np.max(np.abs(yt.numpy() - want)) < 2e-6 * np.sqrt(K) * 10
+
+
+# ---------------------------------------------------------------------------
+# fused LSTM nodes
+# ---------------------------------------------------------------------------
+def test_lstm_golden_vectors(dev, golden):
+    gd = golden["lstm_nodes"]
+    rel = gd["rel_tol"]
+    t = gd["lstm_node_h_fwd"]
+    H, B = t["hidden_dim"], t["batch_size"]
+    out = dev.empty((B, H))
+    dev.lstm_h_forward(H, B, dev.tensor(f32(t["c_t"])), dev.tensor(f32(t["gates_t"])), out)
+    h = out.numpy().reshape(-1)
+    assert abs(h[0]) < t["small_abs"]
+    assert_close(h[1:], np.array(t["h_t"][1:]), rel, "lstm_node_h_fwd")
+    t = gd["lstm_node_c_fwd"]
+    dev.lstm_c_forward(H, B, dev.tensor(f32(t["c_tm1"])), dev.tensor(f32(t["gates_t"])), out)
+    c = out.numpy().reshape(-1)
+    assert np.all(np.abs(c[:3]) < t["small_abs"])
+    assert_close(c[3:], np.array(t["c_t"][3:]), rel, "lstm_node_c_fwd")
+    for name, mode in (("lstm_node_gates_fwd", lib.LOGISTIC_PACKET), ("lstm_node_gates_fwd", lib.LOGISTIC_SCALAR),
+                       ("lstm_node_gates_dropout_fwd", lib.LOGISTIC_PACKET)):
+        t = gd[name]
+        I, H, B = t["input_dim"], t["hidden_dim"], t["batch_size"]
+        fx = dev.empty((B, 4 * H))
+        kw = {}
+        if "mask_x" in t:
+            kw = dict(mask_x=dev.tensor(f32(t["mask_x"])), mask_x_bd=B, mask_h=dev.tensor(f32(t["mask_h"])), mask_h_bd=B)
+        dev.lstm_gates_forward([dev.tensor(f32(t["x_t"]))], [I], H, B, dev.tensor(f32(t["h_tm1"])),
+                               dev.tensor(f32(t["Wx"])), dev.tensor(f32(t["Wh"])), dev.tensor(f32(t["b"])), fx,
+                               logistic_mode=mode, **kw)
+        assert_close(fx.numpy().reshape(-1), np.array(t["gates"]), rel, name)
+
+
+def _lstm_case(rng, I, H, B):
+    x = f32(rng.standard_normal((B, I)))
+    h = f32(rng.standard_normal((B, H)))
+    c = f32(rng.standard_normal((B, H)))
+    Wx, Wh = glorot(rng, 4 * H, I), glorot(rng, 4 * H, H)
+    b = np.zeros(4 * H, F32)
+    return x, h, c, Wx, Wh, b
+
+
+@pytest.mark.parametrize("I,H,B,dims,dropout,mask_full", [
+    (128, 256, 32, None, False, True),      # the single-cell configuration of the baseline
+    (256, 1024, 128, None, False, True),    # layer 1 of the LM configuration
+    (5, 3, 2, None, False, True),           # tests/test-rnn.cc:341-357
+    (3, 5, 2, None, True, True),            # :402-431
+    (3, 5, 2, None, True, False),           # :601-630 (batch-broadcast masks)
+    (4, 5, 2, [1, 3], False, True),         # :433-460 (multi-input)
+    (4, 5, 2, [1, 3], True, True),          # :499-529
+    (37, 19, 7, [5, 32], True, False),
+])
+def test_lstm_cell_forward_backward(dev, I, H, B, dims, dropout, mask_full):
+    rng = np.random.default_rng(I * 100 + H * 10 + B)
+    x, h, c_prev, Wx, Wh, b = _lstm_case(rng, I, H, B)
+    if H < 64:
+        b = f32(rng.standard_normal(4 * H) * 0.1)
+    dims = dims or [I]
+    offs = np.cumsum([0] + dims)
+    xs = [np.ascontiguousarray(x[:, offs[k]:offs[k + 1]]) for k in range(len(dims))]
+    mx = mh = None
+    mbd = 0
+    if dropout:
+        mbd = B if mask_full else 1
+        mx, mh = f32(rng.integers(0, 2, (mbd, I)) * 0.9), f32(rng.integers(0, 2, (mbd, H)) * 0.8)
+    xs_t = [dev.tensor(a) for a in xs]
+    ht, ct, Wxt, Wht, bt = (dev.tensor(a) for a in (h, c_prev, Wx, Wh, b))
+    mxt = dev.tensor(mx) if dropout else None
+    mht = dev.tensor(mh) if dropout else None
+    mask_kw = dict(mask_x=mxt, mask_x_bd=mbd, mask_h=mht, mask_h_bd=mbd)
+    o_mask = dict(mask_x=mx, mask_x_bd=mbd, mask_h=mh, mask_h_bd=mbd)
+    scale = float(np.sqrt(I + H) * max(rms(Wx), rms(Wh)))  # size of the pre-activation terms
+
+    # ---- forward: gates -> c -> h -------------------------------------------
+    fx_t = dev.empty((B, 4 * H))
+    dev.lstm_gates_forward(xs_t, dims, H, B, ht, Wxt, Wht, bt, fx_t, **mask_kw)
+    fx_ref = orc.lstm_gates_forward(xs, dims, H, B, h, Wx, Wh, b, **o_mask)
+    # an fp32 GEMM in another summation order moves the pre-activation by ~1e-7*scale;
+    # the gate moves by at most that (|sigma'|, |tanh'| <= 1)
+    assert_close(fx_t.numpy(), fx_ref, FWD_RTOL, "gates fwd", floor=max(1.0, scale))
+    c_t, h_t = dev.empty((B, H)), dev.empty((B, H))
+    fxo_t = dev.tensor(fx_ref)  # downstream nodes are compared from identical inputs
+    dev.lstm_c_forward(H, B, ct, fxo_t, c_t)
+    c_ref = orc.lstm_c_forward(H, B, c_prev, fx_ref)
+    assert_close(c_t.numpy(), c_ref, FWD_RTOL, "c fwd", floor=1e-3)
+    dev.lstm_h_forward(H, B, dev.tensor(c_ref), fxo_t, h_t)
+    h_ref = orc.lstm_h_forward(H, B, c_ref, fx_ref)
+    assert_close(h_t.numpy(), h_ref, FWD_RTOL, "h fwd", floor=1e-6)
+
+    # ---- backward: h -> c -> gates, every argument, into non-zero buffers ----
+    dh, dc_up = f32(rng.standard_normal((B, H))), f32(rng.standard_normal((B, H)))
+    dht = dev.tensor(dh)
+    cr_t = dev.tensor(c_ref)
+    for i, shape in ((0, (B, H)), (1, (B, 4 * H))):
+        g0 = f32(rng.standard_normal(shape))
+        gt = dev.tensor(g0)
+        dev.lstm_h_backward(H, B, cr_t, fxo_t, dht, i, gt)
+        assert_close(gt.numpy(), orc.lstm_h_backward(H, B, c_ref, fx_ref, dh, i, g0.copy()), GRAD_RTOL, "h bwd %d" % i,
+                     floor=1e-4)
+        gt = dev.tensor(g0)
+        dev.lstm_c_backward(H, B, ct, fxo_t, dev.tensor(dc_up), i, gt)
+        assert_close(gt.numpy(), orc.lstm_c_backward(H, B, c_prev, fx_ref, dc_up, i, g0.copy()), GRAD_RTOL,
+                     "c bwd %d" % i, floor=1e-4)
+    dgates = f32(rng.standard_normal((B, 4 * H)))
+    dgt = dev.tensor(dgates)
+    dpre_t = dev.empty((B, 4 * H))
+    dev.lstm_gates_dpre(H, B, fxo_t, dgt, dpre_t)
+    k_in = len(dims)
+    shapes = [(B, d) for d in dims] + [(B, H), (I, 4 * H), (H, 4 * H), (4 * H,)]
+    floors = [np.sqrt(4 * H) * rms(Wx)] * k_in + [np.sqrt(4 * H) * rms(Wh), np.sqrt(B), np.sqrt(B), np.sqrt(B)]
+    for i, shape in enumerate(shapes):
+        g0 = f32(rng.standard_normal(shape))
+        want = orc.lstm_gates_backward(xs, dims, H, B, h, Wx, Wh, fx_ref, dgates, i, g0.copy(), **o_mask)
+        for cached in (False, True):
+            gt = dev.tensor(g0)
+            dev.lstm_gates_backward(xs_t, dims, H, B, ht, Wxt, Wht, fxo_t, dgt, i, gt,
+                                    dpre=dpre_t if cached else None, **mask_kw)
+            assert_close(gt.numpy(), want, GRAD_RTOL, "gates bwd arg %d cached=%s" % (i, cached),
+                         floor=max(1.0, float(floors[i])))
+
+
+def test_fused_nodes_equal_unfused_path_over_three_steps(dev):
+    """tests/test-rnn.cc:155-184,214-243: gates/C/H equal affine -> logistic/tanh -> cmult."""
+    rng = np.random.default_rng(9)
+    I, H, B = 3, 5, 2
+    x, h, c, Wx, Wh, b = _lstm_case(rng, I, H, B)
+    b = f32(rng.standard_normal(4 * H) * 0.1)
+    xt, Wxt, Wht, bt = dev.tensor(x), dev.tensor(Wx), dev.tensor(Wh), dev.tensor(b)
+    ht, ct = dev.tensor(h), dev.tensor(c)
+    h64, c64 = h.astype(np.float64), c.astype(np.float64)
+    W64x, W64h = Wx.T.astype(np.float64), Wh.T.astype(np.float64)
+    sig = lambda v: 1 / (1 + np.exp(-v))
+    for _ in range(3):
+        fx, c2, h2 = dev.empty((B, 4 * H)), dev.empty((B, H)), dev.empty((B, H))
+        dev.lstm_gates_forward([xt], [I], H, B, ht, Wxt, Wht, bt, fx, logistic_mode=lib.LOGISTIC_SCALAR)
+        dev.lstm_c_forward(H, B, ct, fx, c2)
+        dev.lstm_h_forward(H, B, c2, fx, h2)
+        tmp = x.astype(np.float64) @ W64x.T + h64 @ W64h.T + b
+        i_t, f_t, o_t = sig(tmp[:, :H]), sig(tmp[:, H:2 * H] + 1), sig(tmp[:, 2 * H:3 * H])
+        c64 = f_t * c64 + i_t * np.tanh(tmp[:, 3 * H:])
+        h64 = o_t * np.tanh(c64)
+        assert_close(h2.numpy(), h64, 1e-5, "fused vs unfused", floor=1e-3)
+        ht, ct = h2, c2
+
+
+def test_lstm_rejects_bad_arguments(dev):
+    t = dev.zeros(64)
+    with pytest.raises(DyhipError) as e:
+        dev.lstm_gates_forward([t], [2], 2, 2, t, t, t, t, t, mask_x=t, mask_x_bd=3, mask_h=t, mask_h_bd=2)
+    assert e.value.status == lib.ERR_INVALID_ARG and "dropout_mask_x" in str(e.value)
+    with pytest.raises(DyhipError):
+        dev.lstm_c_backward(2, 2, t, t, t, 2, t)
+
+
+# ---------------------------------------------------------------------------
+# LookupNode
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("vocab,dim,n", [(50000, 512, 256 * 64), (10000, 256, 128), (7, 3, 40), (33, 130, 1000),
+                                         (5, 4, 1)])
+def test_lookup_gather_bit_exact_and_scatter_add(dev, vocab, dim, n):
+    rng = np.random.default_rng(vocab + dim + n)
+    table = f32(rng.uniform(-0.1, 0.1, (vocab, dim)))
+    ids = zipf_ids(rng, n, vocab)
+    tt = dev.tensor(table, pool=lib.POOL_FXS)
+    ids_t = dev.empty(n, np.uint32)
+    fx = dev.empty((n, dim))
+    dev.lookup_forward(ids, ids_t, dim, vocab, tt, fx)
+    assert fx.numpy().tobytes() == table[ids].tobytes()  # bit-exact gather
+    assert ids_t.numpy().tobytes() == ids.tobytes()
+    dev.lookup_forward(None, ids_t, dim, vocab, tt, fx, mult=0.5)  # ids already on the device
+    assert fx.numpy().tobytes() == orc.lookup_forward(ids, dim, vocab, table, 0.5).tobytes()
+    # scatter-add into a non-zero gradient table
+    g = f32(rng.standard_normal((n, dim)))
+    grads0 = f32(rng.standard_normal((vocab, dim)))
+    gt = dev.tensor(grads0)
+    dev.lookup_accumulate_grads(ids_t, dim, vocab, dev.tensor(g), gt)
+    got = gt.numpy()
+    want = orc.lookup_accumulate_grads(ids, dim, vocab, g, grads0.copy())  # sequential fp32, the CPU path
+    counts = np.bincount(ids, minlength=vocab).astype(np.float64)
+    floor = np.sqrt(np.maximum(counts, 1.0))[:, None] * np.ones((1, dim))
+    assert_close(got, want, GRAD_RTOL, "lookup scatter-add", floor=floor)
+    untouched = counts == 0
+    assert got[untouched].tobytes() == grads0[untouched].tobytes()
+    # as close to the fp64 sum as the sequential fp32 path is
+    exact = grads0.astype(np.float64)
+    np.add.at(exact, ids, g.astype(np.float64))
+    assert np.max(np.abs(got - exact)) <= max(4 * np.max(np.abs(want - exact)), 1e-5)
+    # deterministic: the same call gives the same bits
+    gt2 = dev.tensor(grads0)
+    dev.lookup_accumulate_grads(ids_t, dim, vocab, dev.tensor(g), gt2)
+    assert gt2.numpy().tobytes() == got.tobytes()
+
+
+def test_lookup_all_ids_equal_and_all_distinct(dev):
+    rng = np.random.default_rng(3)
+    vocab, dim = 64, 32
+    for ids in (np.full(1000, 5, np.uint32), rng.permutation(vocab).astype(np.uint32)):
+        g = f32(rng.standard_normal((ids.size, dim)))
+        gt = dev.zeros((vocab, dim))
+        dev.lookup_accumulate_grads(dev.tensor(ids, np.uint32), dim, vocab, dev.tensor(g), gt)
+        want = orc.lookup_accumulate_grads(ids, dim, vocab, g, np.zeros((vocab, dim), F32))
+        assert_close(gt.numpy(), want, GRAD_RTOL, "lookup edge", floor=np.sqrt(ids.size))
+
+
+def test_lookup_out_of_range_index_is_an_error(dev):
+    t = dev.zeros((4, 4))
+    with pytest.raises(DyhipError) as e:
+        dev.lookup_forward(np.array([0, 4], np.uint32), dev.empty(2, np.uint32), 4, 4, t, dev.empty((2, 4)))
+    assert e.value.status == lib.ERR_INVALID_ARG and "Out-of-bounds" in str(e.value)
+
+
+# ---------------------------------------------------------------------------
+# logsumexp / PickNegLogSoftmax / LogSumExp / argmax
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("rows,bd", [(50000, 512), (10000, 128), (37, 5), (1027, 3), (1, 4), (4, 1)])
+def test_pnls_forward_backward(dev, rows, bd):
+    rng = np.random.default_rng(rows + bd)
+    x = f32(rng.standard_normal((bd, rows)) * 2.0)
+    labels = rng.integers(0, rows, bd).astype(np.uint32)
+    xt = dev.tensor(x)
+    aux = dev.empty(3 * bd)
+    fx = dev.empty(bd)
+    dev.pnls_forward(rows, bd, xt, labels, aux, fx)
+    ref_fx, ref_aux = orc.pnls_forward(rows, bd, x, labels)
+    a = aux.numpy()
+    assert a.view(np.uint32)[2 * bd:].tobytes() == ref_aux.view(np.uint32)[2 * bd:].tobytes()  # picks: bit exact
+    assert a[bd:2 * bd].tobytes() == ref_aux[bd:2 * bd].tobytes()  # row maxima: bit exact
+    assert_close(a[:bd], ref_aux[:bd], FWD_RTOL, "logsumexp z")
+    assert_close(fx.numpy(), ref_fx, FWD_RTOL, "pnls fwd", floor=1.0)
+    m_t, z_t = dev.empty(bd), dev.empty(bd)
+    dev.logsumexp_cols(rows, bd, xt, m_t, z_t)
+    assert z_t.numpy().tobytes() == a[:bd].tobytes()
+    # backward from the oracle's aux so that both sides see identical z
+    dy = f32(rng.standard_normal(bd))
+    dx0 = f32(rng.standard_normal((bd, rows)) * 0.01)
+    dxt = dev.tensor(dx0)
+    dev.pnls_backward(rows, bd, xt, dev.tensor(ref_aux), dev.tensor(dy), dxt)
+    want = orc.pnls_backward(rows, bd, x, ref_aux, dy, dx0.copy())
+    assert_close(dxt.numpy(), want, GRAD_RTOL, "pnls bwd", floor=1e-4)
+    # sum_v (softmax - onehot) == 0 per row
+    delta = (dxt.numpy().astype(np.float64) - dx0).sum(1)
+    assert np.max(np.abs(delta)) < 1e-4 * max(1.0, np.max(np.abs(dy)))
+
+
+def test_logsumexp_shift_invariance_and_no_overflow(dev):
+    rng = np.random.default_rng(8)
+    rows, bd = 4096, 16
+    x = f32(rng.standard_normal((bd, rows)))
+    m, z, z2 = dev.empty(bd), dev.empty(bd), dev.empty(bd)
+    dev.logsumexp_cols(rows, bd, dev.tensor(x), m, z)
+    dev.logsumexp_cols(rows, bd, dev.tensor(x + F32(64.0)), m, z2)
+    assert np.max(np.abs(z2.numpy() - z.numpy() - 64.0)) < 1e-4
+    big = np.full((1, 8), -1000.0, F32)
+    big[0, :2] = 1000.0
+    dev.logsumexp_cols(8, 1, dev.tensor(big), m, z)
+    assert abs(float(z.numpy()[0]) - (1000.0 + np.log(2.0))) < 1e-3
+
+
+def test_pnls_label_out_of_range_is_an_error(dev):
+    with pytest.raises(DyhipError) as e:
+        dev.pnls_forward(4, 2, dev.zeros((2, 4)), np.array([0, 4], np.uint32), dev.empty(6), dev.empty(2))
+    assert e.value.status == lib.ERR_INVALID_ARG and "Index error in PickNegLogSoftmax" in str(e.value)
+
+
+def test_logsumexp_node(dev):
+    rng = np.random.default_rng(15)
+    n, bd = 600, 4
+    a, b, c1 = f32(rng.standard_normal((bd, n))), f32(rng.standard_normal((bd, n))), f32(rng.standard_normal((1, n)))
+    ts = [dev.tensor(v) for v in (a, b, c1)]
+    bds = [bd, bd, 1]
+    fx = dev.empty((bd, n))
+    dev.logsumexp_node_forward(n, bd, ts, bds, fx)
+    ref = orc.logsumexp_node_forward(n, bd, [a, b, c1], bds)
+    assert_close(fx.numpy(), ref, FWD_RTOL, "LogSumExp fwd", floor=1e-2)
+    dy = f32(rng.standard_normal((bd, n)))
+    for i, shape in ((0, (bd, n)), (2, (1, n))):
+        g0 = f32(rng.standard_normal(shape))
+        gt = dev.tensor(g0)
+        dev.logsumexp_node_backward(n, bd, ts, bds, dev.tensor(ref), dev.tensor(dy), i, gt)
+        want = orc.logsumexp_node_backward(n, bd, [a, b, c1], bds, ref, dy, i, g0.copy())
+        assert_close(gt.numpy(), want, GRAD_RTOL, "LogSumExp bwd %d" % i, floor=1e-2)
+
+
+def test_argmax(dev, golden):
+    t = golden["node_values"]["argmax"]
+    idx = dev.empty(t["bd"], np.int64)
+    dev.argmax_cols(t["rows"], t["bd"], dev.tensor(f32(t["x"])), idx)
+    assert list(idx.numpy()) == t["expected"]
+    rng = np.random.default_rng(4)
+    x = f32(rng.integers(0, 50, (9, 5000)))  # many ties: first maximum wins
+    idx = dev.empty(9, np.int64)
+    dev.argmax_cols(5000, 9, dev.tensor(x), idx)
+    assert idx.numpy().tobytes() == orc.argmax_cols(5000, 9, x).tobytes()
+
+
+# ---------------------------------------------------------------------------
+# dynet::gpu helpers, parameter copy, trainer
+# ---------------------------------------------------------------------------
+def test_gpu_ops_helpers(dev):
+    rng = np.random.default_rng(16)
+    n, size = 1000, 5000
+    src = f32(rng.standard_normal(size))
+    idx = rng.permutation(size)[:n].astype(np.uint32)  # distinct targets
+    it = dev.tensor(idx, np.uint32)
+    out = dev.empty(n)
+    dev.sparse_to_dense_assign(n, it, dev.tensor(src), out)
+    assert out.numpy().tobytes() == orc.sparse_to_dense_assign(idx, src).tobytes()
+    trg = dev.zeros(size)
+    dev.dense_to_sparse_assign(n, it, dev.tensor(src[:n]), trg)
+    assert trg.numpy().tobytes() == orc.dense_to_sparse_assign(idx, src[:n], np.zeros(size, F32)).tobytes()
+    trg = dev.tensor(src)
+    dev.dense_to_sparse_subtract(n, it, dev.tensor(src[:n]), trg)
+    assert trg.numpy().tobytes() == orc.dense_to_sparse_subtract(idx, src[:n], src.copy()).tobytes()
+    table = f32(rng.standard_normal((50, 37)))
+    bidx = rng.integers(0, 50, 64).astype(np.uint32)
+    out = dev.empty((64, 37))
+    dev.sparse_to_dense_block_assign_and_multiply(64, dev.tensor(bidx, np.uint32), 37, 2.0, dev.tensor(table), out)
+    want = orc.sparse_to_dense_block_assign_and_multiply(bidx, 37, 2.0, table)
+    assert out.numpy().tobytes() == want.tobytes()
+    acc = dev.zeros((50, 37))
+    dev.dense_to_sparse_block_add(64, dev.tensor(bidx, np.uint32), 37, dev.tensor(want), acc)
+    assert_close(acc.numpy(), orc.dense_to_sparse_block_add(bidx, 37, want, np.zeros((50, 37), F32)), GRAD_RTOL,
+                 "dense_to_sparse_block_add", floor=1.0)
+
+
+def test_parallel_memcpy_and_accumulate(dev):
+    rng = np.random.default_rng(17)
+    lens = np.array([5, 1024, 0, 333, 4096, 7], np.uint64)
+    srcs = [f32(rng.standard_normal(int(n))) for n in lens]
+    src_t = [dev.tensor(s) if s.size else dev.empty(1) for s in srcs]
+    # ragged targets inside one buffer, deliberately not 16-byte aligned for some
+    total = int(lens.sum()) + len(lens)
+    big = dev.zeros(total)
+    offs = np.concatenate([[0], np.cumsum(lens + 1)[:-1]]).astype(np.int64)
+    ptr_arr = np.array([t.ptr for t in src_t] + [big.ptr + 4 * int(o) for o in offs], np.uint64)
+    ptrs = dev.tensor(ptr_arr, np.uint64)
+    lens_t = dev.tensor(lens, np.uint64)
+    k = len(lens)
+    dev.parallel_memcpy(k, int(lens.max()), ptrs.ptr, ptrs.ptr + 8 * k, lens_t)
+    got = big.numpy()
+    for s, o in zip(srcs, offs):
+        assert got[o:o + s.size].tobytes() == s.tobytes()
+    dev.parallel_accumulate(k, int(lens.max()), ptrs.ptr, ptrs.ptr + 8 * k, lens_t)
+    got = big.numpy()
+    for s, o in zip(srcs, offs):
+        assert got[o:o + s.size].tobytes() == (s + s).tobytes()
+
+
+def test_scale_copy_constant_accumulate_sgd_norm(dev):
+    rng = np.random.default_rng(18)
+    n = 100003
+    p, g = f32(rng.standard_normal(n)), f32(rng.standard_normal(n))
+    pt, gt, out = dev.tensor(p), dev.tensor(g), dev.empty(n)
+    dev.scale_copy(n, pt, 1.0, out)
+    assert out.numpy().tobytes() == p.tobytes()
+    dev.scale_copy(n, pt, 0.25, out)
+    assert out.numpy().tobytes() == orc.scale_copy(p, 0.25).tobytes()
+    dev.constant(out, 3.5)
+    assert np.all(out.numpy() == F32(3.5))
+    dev.accumulate(gt, out)
+    assert out.numpy().tobytes() == (g + F32(3.5)).tobytes()
+    dev.sgd_update(n, pt, gt, 0.1, 0.5, 1.0)
+    assert pt.numpy().tobytes() == orc.sgd_update(p.copy(), g, 0.1, 0.5, 1.0).tobytes()
+    nrm = dev.empty(1)
+    dev.squared_l2norm(n, gt, nrm)
+    assert abs(float(nrm.numpy()[0]) - float((g.astype(np.float64) ** 2).sum())) < 1e-5 * n
+
+
+def test_device_scalars_and_pools(dev):
+    vals = [np.frombuffer(dev_scalar(dev, k), F32)[0] for k in range(3)]
+    assert vals == [-1.0, 1.0, 0.0]
+    pool = dev.pool(lib.POOL_SCS)
+    pool.free()
+    a = pool.allocate(1)
+    b = pool.allocate(1)
+    assert b - a == 256 and a % 256 == 0  # GPUAllocator alignment
+    assert pool.used() == 512
+    z = dev.zeros(1000, pool=lib.POOL_DEDFS)
+    dev.constant(z, 2.0)
+    dev.pool(lib.POOL_DEDFS).zero_allocated()  # what the executor does before backward
+    assert not z.numpy().any()
+
+
+def dev_scalar(dev, which):
+    from dynet_amd.device import DevTensor
+
+    return DevTensor(dev, dev.scalar_ptr(which), (1,)).numpy().tobytes()

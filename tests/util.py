@@ -1,0 +1,53 @@
+"""Shared helpers of the parity tests: seeded inputs, tolerance checks, a GPU fixture."""
+import numpy as np
+
+F32 = np.float32
+
+# parity bar of the hot path: fp32 forward within 1e-5 relative, gradients within
+# 1e-4 relative, gathers / picks / argmax bit exact
+FWD_RTOL = 1e-5
+GRAD_RTOL = 1e-4
+
+
+def f32(a):
+    return np.ascontiguousarray(a, dtype=F32)
+
+
+def assert_close(got, ref, rtol, what, floor=0.0):
+    """|got - ref| <= rtol * max(|ref|, floor), elementwise.
+
+    floor = 0 is a pure relative check.  Operators whose result is a difference
+    or a long sum of terms (LayerNorm, GEMM, batch sums, scatter-add) pass the
+    magnitude of those terms as `floor`, because a relative bound on a value
+    that cancels to ~0 is not meaningful in fp32.
+    """
+    got = np.asarray(got, np.float64)
+    ref = np.asarray(ref, np.float64)
+    assert got.shape == ref.shape, (what, got.shape, ref.shape)
+    assert np.all(np.isfinite(got)), what + ": non-finite output"
+    bound = rtol * np.maximum(np.abs(ref), floor)
+    err = np.abs(got - ref)
+    bad = err > bound
+    if np.any(bad):
+        k = np.argmax(err - bound)
+        raise AssertionError("%s: %d/%d outside tolerance; worst at %d: got %r ref %r (err %g, bound %g)" % (
+            what, int(bad.sum()), bad.size, k, got.flat[k], ref.flat[k], err.flat[k], bound.flat[k]))
+
+
+def rms(a):
+    a = np.asarray(a, np.float64)
+    return float(np.sqrt(np.mean(a * a))) if a.size else 0.0
+
+
+def zipf_ids(rng, n, vocab, s=1.1):
+    """Zipf(s) over [0, vocab): p(k) ~ (k+1)^-s, inverse-CDF sampling."""
+    p = (np.arange(1, vocab + 1, dtype=np.float64)) ** (-s)
+    cdf = np.cumsum(p)
+    cdf /= cdf[-1]
+    return np.minimum(np.searchsorted(cdf, rng.random(n)), vocab - 1).astype(np.uint32)
+
+
+def glorot(rng, rows, cols):
+    """ParameterInitGlorot (dynet/param-init.cc:26-40): U(+-sqrt(6)/sqrt(rows+cols)); column-major rows x cols."""
+    s = np.sqrt(6.0) / np.sqrt(rows + cols)
+    return f32(rng.uniform(-s, s, (cols, rows)))
