@@ -1,0 +1,359 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused-layer hot path on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+Workload (config.workload = "cfg2_elementwise_reduction_sweep"): the
+elementwise / reduction sweep of the baseline on a 4096 x 1024 fp32 tensor with
+values ~ N(0,1): tanh, logistic, rectify, cmult, sum_batches (batch 64 of
+64 x 1024) and layer_norm over the 1024 dim (g ~ U(0.5,1.5), b ~ N(0,0.1)),
+forward and backward.  One "step" is one pass of that sweep (13 kernel
+launches) over one of several rotating buffer sets, so that successive steps
+do not find their inputs in the 256 MB Infinity Cache.  Inputs are resident in
+HBM before the timed region.
+
+Reported: value = algorithmic bytes of one step / step time (GB/s), the
+per-kernel achieved bandwidth of every kernel of the sweep and of the lookup /
+PickNegLogSoftmax kernels (cfg 3 / 4), the latency of one fused LSTM cell step
+(cfg 1), a roofline object for the dominant kernel, and the CPU oracle timed on
+the host cores next to it (a reported baseline, not the target).
+
+Per-kernel durations are measured with HIP events on the library's stream
+around a replayed HIP graph that holds one launch per rotating buffer set, so
+the figure is the back-to-back device time per launch, not Python's launch
+latency.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+S_ELEMS = 4096 * 1024
+S_BYTES = S_ELEMS * 4
+LN_N, LN_BD = 1024, 4096
+SB_N, SB_BD = 64 * 1024, 64
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--sets", type=int, default=24,
+                    help="rotating buffer sets; 24 x 33.5 MB (the smallest kernel footprint) = 3x the Infinity Cache")
+    ap.add_argument("--stream-threshold", type=int, default=None,
+                    help="override the library's non-temporal access threshold in bytes (tuning experiments)")
+    ap.add_argument("--kernel-reps", type=int, default=20, help="graph replays per per-kernel measurement")
+    ap.add_argument("--no-graph", action="store_true", help="time plain back-to-back launches instead of graph replays")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the cfg 1 / 3 / 4 kernel measurements")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="bound on the CPU-baseline leg")
+    return ap.parse_args()
+
+
+class Sweep:
+    """The cfg-2 sweep: buffers for R rotating sets and the list of kernels."""
+
+    def __init__(self, dev, lib, sets, seed=0):
+        self.dev, self.lib, self.R = dev, lib, sets
+        rng = np.random.default_rng(seed)
+        self.g = dev.tensor(rng.uniform(0.5, 1.5, LN_N).astype(np.float32), pool=lib.POOL_PS)
+        self.b = dev.tensor((rng.standard_normal(LN_N) * 0.1).astype(np.float32), pool=lib.POOL_PS)
+        self.dg = dev.zeros(LN_N, pool=lib.POOL_PS)
+        self.db = dev.zeros(LN_N, pool=lib.POOL_PS)
+        self.sets = []
+        for _ in range(sets):
+            s = {
+                "x": dev.tensor(rng.standard_normal(S_ELEMS).astype(np.float32)),
+                "x2": dev.tensor(rng.standard_normal(S_ELEMS).astype(np.float32)),
+                "y": dev.empty(S_ELEMS),
+                "dy": dev.tensor(rng.standard_normal(S_ELEMS).astype(np.float32)),
+                "dx": dev.zeros(S_ELEMS, pool=lib.POOL_DEDFS),
+                "s": dev.empty(SB_N),
+            }
+            self.sets.append(s)
+        self.ws_ln, self.ws_ln_bytes = dev.workspace(dev.layer_norm_backward_workspace(LN_N, LN_BD))
+        self.ws_br, self.ws_br_bytes = dev.workspace(max(dev.batch_reduce_workspace(SB_N, SB_BD), 256))
+        L = lib
+        S = S_BYTES
+        d = dev
+        # (name, algorithmic bytes per launch, launcher taking a buffer set)
+        self.kernels = [
+            ("tanh_fwd", 2 * S, lambda b: d.unary_forward(L.OP_TANH, b["x"], b["y"])),
+            ("tanh_bwd", 4 * S, lambda b: d.unary_backward(L.OP_TANH, b["y"], b["dy"], b["dx"])),
+            ("logistic_fwd", 2 * S, lambda b: d.unary_forward(L.OP_LOGISTIC, b["x"], b["y"])),
+            ("logistic_bwd", 4 * S, lambda b: d.unary_backward(L.OP_LOGISTIC, b["y"], b["dy"], b["dx"])),
+            ("rectify_fwd", 2 * S, lambda b: d.unary_forward(L.OP_RECTIFY, b["x"], b["y"])),
+            ("rectify_bwd", 4 * S, lambda b: d.unary_backward(L.OP_RECTIFY, b["y"], b["dy"], b["dx"])),
+            ("cmult_fwd", 3 * S, lambda b: d.cmult_forward(S_ELEMS, 1, 1, b["x"], b["x2"], b["y"])),
+            ("cmult_bwd_arg0", 4 * S, lambda b: self._cmult_bwd(b, 0)),
+            ("cmult_bwd_arg1", 4 * S, lambda b: self._cmult_bwd(b, 1)),
+            ("sum_batches_fwd", S + S // 64,
+             lambda b: d.sum_batches_forward(SB_N, SB_BD, b["x"], b["s"], self.ws_br, self.ws_br_bytes)),
+            ("sum_batches_bwd", 2 * S + S // 64, lambda b: d.sum_batches_backward(SB_N, SB_BD, b["s"], b["dx"])),
+            ("layer_norm_fwd", 2 * S + 2 * LN_N * 4,
+             lambda b: d.layer_norm_forward(LN_N, LN_BD, b["x"], self.g, self.b, b["y"])),
+            ("layer_norm_bwd", 4 * S + 4 * LN_N * 4,
+             lambda b: d.layer_norm_backward(LN_N, LN_BD, b["x"], self.g, b["dy"], b["dx"], self.dg, self.db,
+                                             self.ws_ln, self.ws_ln_bytes)),
+        ]
+        self.step_bytes = sum(k[1] for k in self.kernels)
+
+    def _cmult_bwd(self, b, i):
+        from dynet_amd.device import _check, _p, _sz, _u, _vp, cdll
+
+        _check(cdll.dyhip_cmult_backward(self.dev.handle, _sz(S_ELEMS), _u(1), _u(1), _p(b["x"]), _p(b["x2"]),
+                                         _p(b["dy"]), _u(i), _p(b["dx"]), _vp(None), _sz(0)))
+
+    def run_step(self, r):
+        b = self.sets[r % self.R]
+        for _, _, fn in self.kernels:
+            fn(b)
+
+
+def time_graph(dev, graph, reps, launches_per_replay):
+    """Average device time per launch (us) of a captured graph replayed `reps` times."""
+    for _ in range(3):
+        graph.launch()
+    dev.sync()
+    dev.timer_start()
+    for _ in range(reps):
+        graph.launch()
+    ms = dev.timer_stop()
+    return ms * 1e3 / (reps * launches_per_replay)
+
+
+def capture(dev, fn_list):
+    dev.graph_begin()
+    try:
+        for fn in fn_list:
+            fn()
+    finally:
+        g = dev.graph_end()
+    return g
+
+
+def time_loop(dev, fns, reps):
+    """Average device time per call (us) of plain back-to-back launches (no graph)."""
+    for fn in fns:
+        fn()
+    dev.sync()
+    dev.timer_start()
+    for _ in range(reps):
+        for fn in fns:
+            fn()
+    ms = dev.timer_stop()
+    return ms * 1e3 / (reps * len(fns))
+
+
+def per_kernel_table(dev, named, sets, reps, use_graph=True):
+    """named: list of (name, bytes, fn(set)); returns a list of dicts with us / GB/s / fraction of peak."""
+    out = []
+    for name, nbytes, fn in named:
+        fns = [(lambda s=s: fn(s)) for s in sets]
+        if use_graph:
+            g = capture(dev, fns)
+            us = time_graph(dev, g, reps, len(sets))
+            g.destroy()
+        else:
+            us = time_loop(dev, fns, reps)
+        gbps = nbytes / us / 1e3
+        out.append({"kernel": name, "bytes": int(nbytes), "us": round(us, 3), "GBps": round(gbps, 1),
+                    "frac_of_8TBps": round(gbps / HBM_PEAK_GBPS, 4)})
+    return out
+
+
+def extras(dev, lib, reps):
+    """cfg 3 (lookup), cfg 4 (PickNegLogSoftmax) kernels and the cfg 1 LSTM cell latency."""
+    from dynet_amd.synth import glorot, zipf_ids
+
+    rng = np.random.default_rng(0)
+    res = {}
+    # ---- cfg 3: lookup 50000 x 512, 16384 Zipf(1.1) ids -----------------------
+    V, D, n = 50000, 512, 256 * 64
+    G = n * D * 4
+    sets = []
+    for _ in range(4):
+        ids = zipf_ids(rng, n, V)
+        sets.append({
+            "table": dev.tensor(rng.uniform(-0.1, 0.1, (V, D)).astype(np.float32)),
+            "grads": dev.zeros((V, D), pool=lib.POOL_DEDFS),
+            "ids": dev.tensor(ids, np.uint32), "fx": dev.empty((n, D)),
+            "g": dev.tensor(rng.standard_normal((n, D)).astype(np.float32)),
+            "uniq": int(np.unique(ids).size),
+        })
+    ws, wsb = dev.workspace(dev.lookup_accumulate_grads_workspace(n, D, V))
+    uniq = sets[0]["uniq"]
+    gather = [("lookup_gather", 2 * G + n * 4,
+               lambda s: dev.lookup_forward(None, s["ids"], D, V, s["table"], s["fx"]))]
+    # the scatter-add is a library sort followed by two kernels: timed as plain launches, outside a graph
+    scatter = [("lookup_scatter_add(sort+segmented)", G + 2 * uniq * D * 4,
+                lambda s: dev.lookup_accumulate_grads(s["ids"], D, V, s["g"], s["grads"], ws, wsb))]
+    res["cfg3_lookup"] = {"vocab": V, "dim": D, "n_ids": n, "unique_ids": uniq,
+                          "kernels": per_kernel_table(dev, gather, sets, reps) +
+                          per_kernel_table(dev, scatter, sets, reps, use_graph=False)}
+    for w in (lib.POOL_FXS, lib.POOL_DEDFS, lib.POOL_SCS):
+        dev.sync()
+        dev.free_pool(w)
+    # ---- cfg 4: PickNegLogSoftmax 50000 x 512 ----------------------------------
+    rows, bd = 50000, 512
+    X = rows * bd * 4
+    sets = []
+    for _ in range(3):
+        labels = rng.integers(0, rows, bd).astype(np.uint32)
+        aux = dev.empty(3 * bd)
+        aux.offset(2 * bd, (bd,)).set((np.arange(bd, dtype=np.uint32) * rows + labels).view(np.float32))
+        sets.append({"x": dev.tensor((rng.standard_normal((bd, rows)) * 2).astype(np.float32)), "aux": aux,
+                     "fx": dev.empty(bd), "dy": dev.tensor(rng.standard_normal(bd).astype(np.float32)),
+                     "dx": dev.zeros((bd, rows), pool=lib.POOL_DEDFS)})
+    for s in sets:
+        dev.pnls_forward_staged(rows, bd, s["x"], s["aux"], s["fx"])
+    named = [
+        ("pnls_fwd", X, lambda s: dev.pnls_forward_staged(rows, bd, s["x"], s["aux"], s["fx"])),
+        ("pnls_bwd", 3 * X, lambda s: dev.pnls_backward(rows, bd, s["x"], s["aux"], s["dy"], s["dx"])),
+    ]
+    res["cfg4_pnls"] = {"rows": rows, "bd": bd, "kernels": per_kernel_table(dev, named, sets, reps)}
+    for w in (lib.POOL_FXS, lib.POOL_DEDFS, lib.POOL_SCS):
+        dev.sync()
+        dev.free_pool(w)
+    # ---- cfg 1: one fused LSTM cell step, fwd + bwd ------------------------------
+    I, H, B = 128, 256, 32
+    t = {k: dev.tensor(v) for k, v in {
+        "x": rng.standard_normal((B, I)), "h": rng.standard_normal((B, H)), "c": rng.standard_normal((B, H)),
+        "Wx": glorot(rng, 4 * H, I), "Wh": glorot(rng, 4 * H, H), "b": np.zeros(4 * H),
+        "dh": rng.standard_normal((B, H)), "dc": rng.standard_normal((B, H))}.items()}
+    fx, c2, h2 = dev.empty((B, 4 * H)), dev.empty((B, H)), dev.empty((B, H))
+    dgates, dcp, dx, dhp = (dev.zeros(s, pool=lib.POOL_DEDFS) for s in ((B, 4 * H), (B, H), (B, I), (B, H)))
+    dWx, dWh, db = (dev.zeros(s, pool=lib.POOL_DEDFS) for s in ((I, 4 * H), (H, 4 * H), (4 * H,)))
+    dct = dev.zeros((B, H), pool=lib.POOL_DEDFS)
+    dpre = dev.empty((B, 4 * H))
+
+    def cell():
+        dev.lstm_gates_forward([t["x"]], [I], H, B, t["h"], t["Wx"], t["Wh"], t["b"], fx)
+        dev.lstm_c_forward(H, B, t["c"], fx, c2)
+        dev.lstm_h_forward(H, B, c2, fx, h2)
+        dev.lstm_h_backward(H, B, c2, fx, t["dh"], 0, dct)
+        dev.lstm_h_backward(H, B, c2, fx, t["dh"], 1, dgates)
+        dev.lstm_c_backward(H, B, t["c"], fx, dct, 0, dcp)
+        dev.lstm_c_backward(H, B, t["c"], fx, dct, 1, dgates)
+        dev.lstm_gates_dpre(H, B, fx, dgates, dpre)
+        for i, out in enumerate((dx, dhp, dWx, dWh, db)):
+            dev.lstm_gates_backward([t["x"]], [I], H, B, t["h"], t["Wx"], t["Wh"], fx, dgates, i, out, dpre=dpre)
+
+    cell()
+    dev.sync()
+    dev.free_pool(lib.POOL_SCS)
+    g = capture(dev, [cell])
+    us = time_graph(dev, g, max(reps, 50), 1)
+    g.destroy()
+    res["cfg1_lstm_cell"] = {"I": I, "H": H, "B": B, "fwd_bwd_us": round(us, 2), "launches": 13 + 5,
+                             "gemm_flops": 3 * 2 * 4 * H * (I + H) * B}
+    return res
+
+
+def cpu_baseline(step_bytes, seconds):
+    """The CPU oracle (plain-C restatement of DyNet's CPU path) on the same sweep, one host core."""
+    from oracle import cpu_oracle as orc
+
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal(S_ELEMS).astype(np.float32)
+    x2 = rng.standard_normal(S_ELEMS).astype(np.float32)
+    dy = rng.standard_normal(S_ELEMS).astype(np.float32)
+    dx = np.zeros(S_ELEMS, np.float32)
+    g = rng.uniform(0.5, 1.5, LN_N).astype(np.float32)
+    b = (rng.standard_normal(LN_N) * 0.1).astype(np.float32)
+    dg, db = np.zeros(LN_N, np.float32), np.zeros(LN_N, np.float32)
+
+    def sweep():
+        for op in (orc.OP_TANH, orc.OP_LOGISTIC, orc.OP_RECTIFY):
+            y = orc.unary_forward(op, x)
+            orc.unary_backward(op, y, dy, dx)
+        orc.cmult_forward(S_ELEMS, 1, 1, x, x2)
+        orc.cmult_backward(S_ELEMS, 1, 1, x, x2, dy, 0, dx)
+        orc.cmult_backward(S_ELEMS, 1, 1, x, x2, dy, 1, dx)
+        s = orc.sum_batches_forward(SB_N, SB_BD, x)
+        orc.sum_batches_backward(SB_N, SB_BD, s, dx)
+        orc.layer_norm_forward(LN_N, LN_BD, x, g, b)
+        orc.layer_norm_backward(LN_N, LN_BD, x, g, dy, dx, dg, db)
+
+    sweep()
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        sweep()
+        reps += 1
+        el = time.perf_counter() - t0
+        if el >= seconds or reps >= 50:
+            break
+    return {"value": round(step_bytes * reps / el / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "%d full passes of the same cfg-2 sweep (4096x1024 fp32) through oracle/libdynet_cpu_oracle.so "
+                      "in %.1f s on one host core of %d" % (reps, el, os.cpu_count() or 0)}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: every box of this build has one, and the hot path has no multi-GPU "
+              "leg (see DESIGN.md, 'How the path would shard'). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    from dynet_amd import Device, lib
+
+    dev = Device(0, mem_mb=(2560, 2048, 64, 256))
+    if args.stream_threshold is not None:
+        dev.set_stream_threshold(args.stream_threshold)
+    sweep = Sweep(dev, lib, args.sets)
+    # ---- whole-step timing: one captured graph per buffer set ---------------------
+    sweep.run_step(0)
+    dev.sync()
+    graphs = [capture(dev, [lambda r=r: sweep.run_step(r)]) for r in range(sweep.R)]
+    for s in range(args.warmup):
+        graphs[s % sweep.R].launch()
+    dev.sync()
+    t0 = time.perf_counter()
+    dev.timer_start()
+    for s in range(args.steps):
+        graphs[s % sweep.R].launch()
+    ms = dev.timer_stop()
+    dev.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_per_step = ms / args.steps
+    value = sweep.step_bytes / (ms_per_step * 1e-3) / 1e9
+    for g in graphs:
+        g.destroy()
+    # ---- per-kernel achieved bandwidth ---------------------------------------------
+    table = per_kernel_table(dev, sweep.kernels, sweep.sets, args.kernel_reps, use_graph=not args.no_graph)
+    dominant = max(table, key=lambda k: k["us"])
+    roofline = {"bound": "hbm", "kernel": dominant["kernel"], "achieved": dominant["GBps"], "peak": HBM_PEAK_GBPS,
+                "unit": "GB/s", "frac": round(dominant["GBps"] / HBM_PEAK_GBPS, 4), "traffic": None,
+                "algorithmic_bytes_per_launch": dominant["bytes"], "avg_launch_us": dominant["us"]}
+    out = {
+        "metric": "fused-kernel HBM GB/s (cfg-2 elementwise/reduction sweep, algorithmic bytes / device time)",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "cfg2_elementwise_reduction_sweep", "tensor": "4096x1024 fp32",
+                   "kernels_per_step": len(sweep.kernels), "rotating_buffer_sets": sweep.R,
+                   "bytes_per_step": int(sweep.step_bytes)},
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
+        "wall_ms_per_step": round(wall_ms / args.steps, 5),
+        "roofline": roofline, "kernels": table, "lstm_lm_tokens_per_s": None,
+    }
+    for w in (lib.POOL_FXS, lib.POOL_DEDFS, lib.POOL_SCS):
+        dev.sync()
+        dev.free_pool(w)
+    if not args.no_extras:
+        out.update(extras(dev, lib, args.kernel_reps))
+    dev.close()
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(sweep.step_bytes, args.cpu_seconds)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

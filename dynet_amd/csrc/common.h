@@ -62,9 +62,15 @@ struct dyhip_device {
   dyhip::MemAllocator* alloc;
   dyhip_pool* pools[4];
   float* scalars;  // device: {-1, 1, 0}
+  size_t stream_threshold;  // tensors at least this large are accessed with streaming (non-temporal) hints
   void* gemm_ws;   // split-K partial tiles (the analogue of a BLAS handle's workspace)
   size_t gemm_ws_bytes;
   hipEvent_t ev_start, ev_stop;
+};
+
+struct dyhip_graph {
+  hipGraph_t graph;
+  hipGraphExec_t exec;
 };
 
 #define DYHIP_CHECK_HIP(expr)                                                                   \
@@ -95,6 +101,44 @@ struct dyhip_device {
 
 #ifdef __HIPCC__
 namespace dyhip {
+
+// ---- streaming (non-temporal) global accesses ------------------------------------
+// Tensors far larger than the 4 MB per-XCD L2 are read once and written once by
+// these kernels; marking those accesses non-temporal keeps them from displacing
+// each other in L2 / Infinity Cache and measurably raises the achieved HBM rate.
+// The read half of a read-modify-write stays a normal load.
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+template <bool NT>
+__device__ __forceinline__ float4 ldg4(const float4* p) {
+  if (NT) {
+    const v4f v = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(p));
+    return make_float4(v.x, v.y, v.z, v.w);
+  }
+  return *p;
+}
+
+template <bool NT>
+__device__ __forceinline__ void stg4(float4* p, const float4 r) {
+  if (NT) {
+    v4f v;
+    v.x = r.x; v.y = r.y; v.z = r.z; v.w = r.w;
+    __builtin_nontemporal_store(v, reinterpret_cast<v4f*>(p));
+  } else {
+    *p = r;
+  }
+}
+
+template <bool NT>
+__device__ __forceinline__ float ldg1(const float* p) {
+  return NT ? __builtin_nontemporal_load(p) : *p;
+}
+
+template <bool NT>
+__device__ __forceinline__ void stg1(float* p, const float v) {
+  if (NT) __builtin_nontemporal_store(v, p);
+  else *p = v;
+}
 
 // ---- wavefront reductions (64 lanes) -----------------------------------------
 __device__ __forceinline__ float wave_sum(float v) {
@@ -167,22 +211,26 @@ __device__ __forceinline__ float logistic(int mode, float x) {
   return mode == DYHIP_LOGISTIC_SCALAR ? logistic_scalar(x) : logistic_packet(x);
 }
 
-// tanh accurate to ~3e-7 relative over the whole range: odd series for
-// |x| < 0.25 (where 1 - e^{-2|x|} would cancel), (1-t)/(1+t) with
-// t = e^{-2|x|} elsewhere.
-__device__ __forceinline__ float tanh_accurate(float x) {
-  const float ax = fabsf(x);
-  if (ax < 0.25f) {
-    const float x2 = x * x;
-    float p = fmaf(x2, -1382.0f / 155925.0f, 62.0f / 2835.0f);
-    p = fmaf(x2, p, -17.0f / 315.0f);
-    p = fmaf(x2, p, 2.0f / 15.0f);
-    p = fmaf(x2, p, -1.0f / 3.0f);
-    return fmaf(x * x2, p, x);
-  }
-  const float t = __expf(-2.0f * ax);
-  const float r = (1.0f - t) / (1.0f + t);
-  return copysignf(r, x);
+// tanh as a clamped odd/even rational function (the form Eigen's vectorised float
+// tanh uses): p(x)/q(x) with p odd, so the result is relatively accurate for small
+// |x| too; max relative error 3.3e-7 against fp64 tanh over the whole range.
+// Branch-free: 9 fused multiply-adds, one reciprocal with a Newton step.
+__device__ __forceinline__ float tanh_accurate(float _x) {
+  const float x = fmaxf(fminf(_x, 9.0f), -9.0f);
+  const float x2 = x * x;
+  float p = fmaf(x2, -2.76076847742355e-16f, 2.00018790482477e-13f);
+  p = fmaf(x2, p, -8.60467152213735e-11f);
+  p = fmaf(x2, p, 5.12229709037114e-08f);
+  p = fmaf(x2, p, 1.48572235717979e-05f);
+  p = fmaf(x2, p, 6.37261928875436e-04f);
+  p = fmaf(x2, p, 4.89352455891786e-03f);
+  p = x * p;
+  float q = fmaf(x2, 1.19825839466702e-06f, 1.18534705686654e-04f);
+  q = fmaf(x2, q, 2.26843463243900e-03f);
+  q = fmaf(x2, q, 4.89352518554385e-03f);
+  float r = __builtin_amdgcn_rcpf(q);
+  r = fmaf(fmaf(-q, r, 1.0f), r, r);  // one Newton step: r ~ 1/q to within 1 ulp
+  return p * r;
 }
 
 }  // namespace dyhip

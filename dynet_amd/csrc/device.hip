@@ -254,6 +254,7 @@ int dyhip_device_create(int ordinal, const size_t pool_mb[4], dyhip_device** out
   dev->alloc = nullptr;
   dev->gemm_ws = nullptr;
   dev->gemm_ws_bytes = 0;
+  dev->stream_threshold = size_t(8) << 20;
   hipError_t e = hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking);
   if (e != hipSuccess) {
     delete dev;
@@ -339,6 +340,12 @@ int dyhip_device_scalar(dyhip_device* dev, int which, const float** ptr) {
   return DYHIP_OK;
 }
 
+int dyhip_device_set_stream_threshold(dyhip_device* dev, size_t bytes) {
+  DYHIP_CHECK_DEV(dev);
+  dev->stream_threshold = bytes;
+  return DYHIP_OK;
+}
+
 int dyhip_device_allocate(dyhip_device* dev, int which_pool, size_t nbytes, void** out) {
   DYHIP_CHECK_DEV(dev);
   DYHIP_REQUIRE(which_pool >= 0 && which_pool < 4, "pool index %d out of range", which_pool);
@@ -378,6 +385,48 @@ int dyhip_zero(dyhip_device* dev, void* dst, size_t nbytes) {
   if (nbytes == 0) return DYHIP_OK;
   DYHIP_REQUIRE(dst != nullptr, "null pointer in zero");
   DYHIP_CHECK_HIP(zero_fill(dst, nbytes, dev->stream));
+  return DYHIP_OK;
+}
+
+// ---------------------------------------------------------------------------
+// HIP graphs
+// ---------------------------------------------------------------------------
+int dyhip_graph_begin_capture(dyhip_device* dev) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_CHECK_HIP(hipStreamBeginCapture(dev->stream, hipStreamCaptureModeThreadLocal));
+  return DYHIP_OK;
+}
+
+int dyhip_graph_end_capture(dyhip_device* dev, dyhip_graph** out) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(out != nullptr, "null output pointer");
+  hipGraph_t graph = nullptr;
+  DYHIP_CHECK_HIP(hipStreamEndCapture(dev->stream, &graph));
+  hipGraphExec_t exec = nullptr;
+  hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  if (e != hipSuccess) {
+    (void)hipGraphDestroy(graph);
+    return fail(DYHIP_ERR_RUNTIME, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+  }
+  dyhip_graph* g = new dyhip_graph();
+  g->graph = graph;
+  g->exec = exec;
+  *out = g;
+  return DYHIP_OK;
+}
+
+int dyhip_graph_launch(dyhip_device* dev, dyhip_graph* graph) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(graph != nullptr, "null graph handle");
+  DYHIP_CHECK_HIP(hipGraphLaunch(graph->exec, dev->stream));
+  return DYHIP_OK;
+}
+
+int dyhip_graph_destroy(dyhip_graph* graph) {
+  DYHIP_REQUIRE(graph != nullptr, "null graph handle");
+  (void)hipGraphExecDestroy(graph->exec);
+  (void)hipGraphDestroy(graph->graph);
+  delete graph;
   return DYHIP_OK;
 }
 

@@ -16,7 +16,7 @@
 // added straight into its gradient row (the chunk is the only writer of that
 // row).  A run that crosses chunk boundaries leaves one partial row per chunk
 // in the workspace, and a second kernel adds the partials of each such run in
-// ascending chunk order.  No atomics anywhere: the result is deterministic and
+// a fixed order.  No atomics anywhere: the result is deterministic and
 // each gradient row is read and written exactly once.
 #include <cstring>
 
@@ -45,11 +45,19 @@ __device__ __forceinline__ float4 vscale(const float4 a, const float m) {
   return make_float4(a.x * m, a.y * m, a.z * m, a.w * m);
 }
 __device__ __forceinline__ float vscale(const float a, const float m) { return a * m; }
+template <bool NT>
+__device__ __forceinline__ float4 vload(const float4* p) { return ldg4<NT>(p); }
+template <bool NT>
+__device__ __forceinline__ float vload(const float* p) { return ldg1<NT>(p); }
+template <bool NT>
+__device__ __forceinline__ void vstore(float4* p, const float4 v) { stg4<NT>(p, v); }
+template <bool NT>
+__device__ __forceinline__ void vstore(float* p, const float v) { stg1<NT>(p, v); }
 
 // ---- gather ---------------------------------------------------------------------
 // A group of `tpr` threads owns one id at a time; a block holds 256/tpr groups and
 // each group processes kGatherRowsUnroll ids with all loads issued first.
-template <class V, bool SCALE>
+template <class V, bool SCALE, bool NT>
 __global__ __launch_bounds__(kLkThreads) void lookup_gather_kernel(unsigned n_ids, unsigned dimv, unsigned tpr,
                                                                    unsigned vocab, const unsigned* __restrict__ ids,
                                                                    const V* __restrict__ table, float mult,
@@ -67,7 +75,7 @@ __global__ __launch_bounds__(kLkThreads) void lookup_gather_kernel(unsigned n_id
       v[u] = (row0 + u < n_ids && id[u] < vocab) ? table[size_t(id[u]) * dimv + c] : vzero<V>();
 #pragma unroll
     for (int u = 0; u < kGatherRowsUnroll; ++u)
-      if (row0 + u < n_ids) fx[size_t(row0 + u) * dimv + c] = SCALE ? vscale(v[u], mult) : v[u];
+      if (row0 + u < n_ids) vstore<NT>(fx + size_t(row0 + u) * dimv + c, SCALE ? vscale(v[u], mult) : v[u]);
   }
 }
 
@@ -75,9 +83,7 @@ __global__ __launch_bounds__(kLkThreads) void lookup_gather_kernel(unsigned n_id
 struct ScatterWs {
   unsigned* sorted_ids;
   unsigned* sorted_pos;
-  unsigned* first_row;   // per chunk: row of a first run that began in an earlier chunk, else kNone
-  unsigned* first_cont;  // per chunk: 1 if that run also continues into the next chunk
-  unsigned* last_row;    // per chunk: row of a run that begins here and continues into the next chunk
+  unsigned* last_row;    // per chunk: row of a run that begins here and continues into the next chunk, else kNone
   float* part_first;     // [chunks][dim]
   float* part_last;      // [chunks][dim]
   void* sort_tmp;
@@ -85,7 +91,7 @@ struct ScatterWs {
   unsigned chunks;
 };
 
-template <class V>
+template <class V, bool NT>
 __global__ __launch_bounds__(kLkThreads) void scatter_chunk_kernel(unsigned n, unsigned dimv, unsigned tpr,
                                                                    unsigned vocab, ScatterWs w,
                                                                    const V* __restrict__ g, V* __restrict__ grads) {
@@ -107,67 +113,101 @@ __global__ __launch_bounds__(kLkThreads) void scatter_chunk_kernel(unsigned n, u
   const bool single = first == last;
   const bool open_left = prev_id == first;
   const bool open_right = next_id == last;
-  if (t == 0) {
-    w.first_row[ch] = open_left ? first : kNone;
-    w.first_cont[ch] = (open_left && single && open_right) ? 1u : 0u;
-    w.last_row[ch] = (open_right && !(single && open_left)) ? last : kNone;
-  }
+  if (t == 0) w.last_row[ch] = (open_right && !(single && open_left)) ? last : kNone;
   V* part_first = reinterpret_cast<V*>(w.part_first) + size_t(ch) * dimv;
   V* part_last = reinterpret_cast<V*>(w.part_last) + size_t(ch) * dimv;
-  for (unsigned c = t; c < dimv; c += tpr) {
-    V v[kChunk];
+  // run_end[k]: entry k is the last of its run inside this chunk; direct[k]: that run
+  // lies wholly inside the chunk, so this thread group is the only writer of the row
+  bool run_end[kChunk], direct[kChunk];
 #pragma unroll
-    for (int k = 0; k < kChunk; ++k) v[k] = k < (int)cnt ? g[size_t(pos[k]) * dimv + c] : vzero<V>();
+  for (int k = 0; k < kChunk; ++k) {
+    const bool last_k = k + 1 >= (int)cnt;
+    run_end[k] = k < (int)cnt && (last_k || id[k + 1 < kChunk ? k + 1 : k] != id[k]);
+    const bool ol = open_left && id[k] == first;
+    const bool orr = open_right && last_k;
+    direct[k] = run_end[k] && !ol && !orr && id[k] < vocab;
+  }
+  for (unsigned c = t; c < dimv; c += tpr) {
+    V v[kChunk], old[kChunk];
+    // every load of the chunk is issued up front: the 16 gradient columns and the
+    // old value of each row that will be updated in place
+#pragma unroll
+    for (int k = 0; k < kChunk; ++k) {
+      v[k] = k < (int)cnt ? vload<NT>(g + size_t(pos[k]) * dimv + c) : vzero<V>();
+      if (direct[k]) old[k] = grads[size_t(id[k]) * dimv + c];
+    }
     V acc = vzero<V>();
-    unsigned cur = first;
-    // flush the finished run of row `cur`: into a partial if the run crosses a
-    // chunk boundary, else straight into the gradient row (sole writer)
-    auto flush = [&](bool end) {
-      if (open_left && cur == first)
-        part_first[c] = acc;
-      else if (end && open_right)
-        part_last[c] = acc;
-      else if (cur < vocab)
-        grads[size_t(cur) * dimv + c] = vadd(grads[size_t(cur) * dimv + c], acc);
-    };
 #pragma unroll
     for (int k = 0; k < kChunk; ++k) {
       if (k < (int)cnt) {
-        if (id[k] != cur) {
-          flush(false);
-          cur = id[k];
+        acc = vadd(acc, v[k]);
+        if (run_end[k]) {
+          if (direct[k])
+            grads[size_t(id[k]) * dimv + c] = vadd(old[k], acc);
+          else if (open_left && id[k] == first)
+            part_first[c] = acc;
+          else if (id[k] < vocab)
+            part_last[c] = acc;
           acc = vzero<V>();
         }
-        acc = vadd(acc, v[k]);
       }
     }
-    flush(true);
   }
 }
 
-// One thread group per chunk where a boundary-crossing run starts: add its
-// partials in ascending chunk order, then one read-modify-write of the row.
+// One block per chunk in which a boundary-crossing run starts.  The end of the run
+// is found by binary search in the sorted ids; the run's partial rows (one per chunk
+// it touches) are split over kFixSlices thread slices that each add every
+// kFixSlices-th partial in ascending order with four loads in flight, and the slices
+// are then added in ascending order: deterministic, and a run of thousands of
+// entries costs a handful of memory round trips instead of one per partial.
+constexpr int kFixThreads = 1024;
+
 template <class V>
-__global__ __launch_bounds__(kLkThreads) void scatter_fixup_kernel(unsigned dimv, unsigned tpr, unsigned vocab,
-                                                                   ScatterWs w, V* __restrict__ grads) {
-  const unsigned groups = kLkThreads / tpr;
-  const unsigned grp = threadIdx.x / tpr, t = threadIdx.x - grp * tpr;
-  const unsigned c0 = blockIdx.x * groups + grp;
-  if (c0 >= w.chunks) return;
+__global__ __launch_bounds__(kFixThreads) void scatter_fixup_kernel(unsigned n, unsigned dimv, unsigned tpr,
+                                                                    unsigned vocab, ScatterWs w,
+                                                                    V* __restrict__ grads) {
+  extern __shared__ __attribute__((aligned(16))) char fix_lds_raw[];
+  V* lds = reinterpret_cast<V*>(fix_lds_raw);
+  const unsigned c0 = blockIdx.x;
   const unsigned row = w.last_row[c0];
-  if (row == kNone || row >= vocab) return;
-  unsigned c1 = c0 + 1;  // one past the last chunk of the run
-  while (c1 < w.chunks && w.first_row[c1] == row) {
-    const bool cont = w.first_cont[c1] != 0;
-    ++c1;
-    if (!cont) break;
+  if (row == kNone || row >= vocab) return;  // uniform over the block
+  // first position after the run: upper bound of `row` in sorted_ids[(c0+1)*kChunk, n)
+  unsigned lo = (c0 + 1) * kChunk, hi = n;
+  while (lo < hi) {
+    const unsigned mid = lo + (hi - lo) / 2;
+    if (w.sorted_ids[mid] <= row) lo = mid + 1;
+    else hi = mid;
   }
+  const unsigned c_last = (lo - 1) / kChunk;  // last chunk holding entries of the run
+  const unsigned slices = kFixThreads / tpr;
+  const unsigned q = threadIdx.x / tpr, t = threadIdx.x - q * tpr;
   const V* pl = reinterpret_cast<const V*>(w.part_last) + size_t(c0) * dimv;
   const V* pf = reinterpret_cast<const V*>(w.part_first);
-  for (unsigned c = t; c < dimv; c += tpr) {
-    V acc = pl[c];
-    for (unsigned k = c0 + 1; k < c1; ++k) acc = vadd(acc, pf[size_t(k) * dimv + c]);
-    grads[size_t(row) * dimv + c] = vadd(grads[size_t(row) * dimv + c], acc);
+  for (unsigned cb = 0; cb < dimv; cb += tpr) {
+    const unsigned c = cb + t;
+    V acc = vzero<V>();
+    if (c < dimv) {
+      // partial index p = 0 is part_last[c0]; p >= 1 is part_first[c0 + p]
+      const unsigned np = c_last - c0 + 1;
+      unsigned p = q;
+      for (; p + 3 * slices < np; p += 4 * slices) {
+        const V a0 = p == 0 ? pl[c] : pf[size_t(c0 + p) * dimv + c];
+        const V a1 = pf[size_t(c0 + p + slices) * dimv + c];
+        const V a2 = pf[size_t(c0 + p + 2 * slices) * dimv + c];
+        const V a3 = pf[size_t(c0 + p + 3 * slices) * dimv + c];
+        acc = vadd(vadd(vadd(vadd(acc, a0), a1), a2), a3);
+      }
+      for (; p < np; p += slices) acc = vadd(acc, p == 0 ? pl[c] : pf[size_t(c0 + p) * dimv + c]);
+    }
+    __syncthreads();
+    lds[q * tpr + t] = acc;
+    __syncthreads();
+    if (q == 0 && c < dimv) {
+      V tot = lds[t];
+      for (unsigned k = 1; k < slices; ++k) tot = vadd(tot, lds[k * tpr + t]);
+      grads[size_t(row) * dimv + c] = vadd(grads[size_t(row) * dimv + c], tot);
+    }
   }
 }
 
@@ -206,8 +246,7 @@ static int carve(unsigned n, size_t dim, unsigned vocab, void* ws, size_t ws_byt
     return o;
   };
   const size_t o_ids = take(sizeof(unsigned) * n), o_pos = take(sizeof(unsigned) * n);
-  const size_t o_fr = take(sizeof(unsigned) * chunks), o_fc = take(sizeof(unsigned) * chunks),
-               o_lr = take(sizeof(unsigned) * chunks);
+  const size_t o_lr = take(sizeof(unsigned) * chunks);
   const size_t o_pf = take(sizeof(float) * dim * chunks), o_pl = take(sizeof(float) * dim * chunks);
   const size_t o_tmp = take(sort_bytes);
   if (need) *need = off;
@@ -218,8 +257,6 @@ static int carve(unsigned n, size_t dim, unsigned vocab, void* ws, size_t ws_byt
     char* base = static_cast<char*>(ws);
     out->sorted_ids = reinterpret_cast<unsigned*>(base + o_ids);
     out->sorted_pos = reinterpret_cast<unsigned*>(base + o_pos);
-    out->first_row = reinterpret_cast<unsigned*>(base + o_fr);
-    out->first_cont = reinterpret_cast<unsigned*>(base + o_fc);
     out->last_row = reinterpret_cast<unsigned*>(base + o_lr);
     out->part_first = reinterpret_cast<float*>(base + o_pf);
     out->part_last = reinterpret_cast<float*>(base + o_pl);
@@ -254,13 +291,17 @@ int dyhip_lookup_forward(dyhip_device* dev, unsigned n_ids, const unsigned* ids_
   const unsigned tpr = threads_per_row(dimv);
   const unsigned rows_per_block = (kLkThreads / tpr) * kGatherRowsUnroll;
   const dim3 grid(cdiv<unsigned>(n_ids, rows_per_block)), block(kLkThreads);
-#define DYHIP_GATHER(V, SCALE)                                                                                \
-  hipLaunchKernelGGL((lookup_gather_kernel<V, SCALE>), grid, block, 0, dev->stream, n_ids, dimv, tpr, vocab, \
+  // the table is read through the caches (hot rows repeat); the output is streamed when large
+  const bool stream = size_t(n_ids) * dim * sizeof(float) >= dev->stream_threshold;
+#define DYHIP_GATHER(V, SCALE, NT)                                                                                \
+  hipLaunchKernelGGL((lookup_gather_kernel<V, SCALE, NT>), grid, block, 0, dev->stream, n_ids, dimv, tpr, vocab, \
                      ids_dev, reinterpret_cast<const V*>(table), mult, reinterpret_cast<V*>(fx))
-  if (vec) {
-    if (mult == 1.0f) DYHIP_GATHER(float4, false); else DYHIP_GATHER(float4, true);
+  if (vec && stream) {
+    if (mult == 1.0f) DYHIP_GATHER(float4, false, true); else DYHIP_GATHER(float4, true, true);
+  } else if (vec) {
+    if (mult == 1.0f) DYHIP_GATHER(float4, false, false); else DYHIP_GATHER(float4, true, false);
   } else {
-    if (mult == 1.0f) DYHIP_GATHER(float, false); else DYHIP_GATHER(float, true);
+    if (mult == 1.0f) DYHIP_GATHER(float, false, false); else DYHIP_GATHER(float, true, false);
   }
 #undef DYHIP_GATHER
   DYHIP_CHECK_LAUNCH();
@@ -292,15 +333,24 @@ int dyhip_lookup_accumulate_grads(dyhip_device* dev, unsigned n_ids, const unsig
   const unsigned dimv = static_cast<unsigned>(vec ? dim / 4 : dim);
   const unsigned tpr = threads_per_row(dimv);
   const dim3 grid(cdiv<unsigned>(w.chunks, kLkThreads / tpr)), block(kLkThreads);
-  if (vec) {
-    hipLaunchKernelGGL(scatter_chunk_kernel<float4>, grid, block, 0, dev->stream, n_ids, dimv, tpr, vocab, w,
+  const dim3 fgrid(w.chunks), fblock(kFixThreads);
+  const size_t flds = size_t(kFixThreads) * (vec ? sizeof(float4) : sizeof(float));
+  const bool stream = size_t(n_ids) * dim * sizeof(float) >= dev->stream_threshold;
+  if (vec && stream) {
+    hipLaunchKernelGGL((scatter_chunk_kernel<float4, true>), grid, block, 0, dev->stream, n_ids, dimv, tpr, vocab, w,
                        reinterpret_cast<const float4*>(g), reinterpret_cast<float4*>(all_grads));
-    hipLaunchKernelGGL(scatter_fixup_kernel<float4>, grid, block, 0, dev->stream, dimv, tpr, vocab, w,
+    hipLaunchKernelGGL(scatter_fixup_kernel<float4>, fgrid, fblock, flds, dev->stream, n_ids, dimv, tpr, vocab, w,
+                       reinterpret_cast<float4*>(all_grads));
+  } else if (vec) {
+    hipLaunchKernelGGL((scatter_chunk_kernel<float4, false>), grid, block, 0, dev->stream, n_ids, dimv, tpr, vocab, w,
+                       reinterpret_cast<const float4*>(g), reinterpret_cast<float4*>(all_grads));
+    hipLaunchKernelGGL(scatter_fixup_kernel<float4>, fgrid, fblock, flds, dev->stream, n_ids, dimv, tpr, vocab, w,
                        reinterpret_cast<float4*>(all_grads));
   } else {
-    hipLaunchKernelGGL(scatter_chunk_kernel<float>, grid, block, 0, dev->stream, n_ids, dimv, tpr, vocab, w, g,
+    hipLaunchKernelGGL((scatter_chunk_kernel<float, false>), grid, block, 0, dev->stream, n_ids, dimv, tpr, vocab, w, g,
                        all_grads);
-    hipLaunchKernelGGL(scatter_fixup_kernel<float>, grid, block, 0, dev->stream, dimv, tpr, vocab, w, all_grads);
+    hipLaunchKernelGGL(scatter_fixup_kernel<float>, fgrid, fblock, flds, dev->stream, n_ids, dimv, tpr, vocab, w,
+                       all_grads);
   }
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;

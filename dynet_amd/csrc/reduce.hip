@@ -21,7 +21,7 @@ namespace dyhip {
 // s*per_split + w, + NW, ...; the NW wave partials are combined through LDS in
 // ascending w.  With more than one split the block writes its partial row to
 // the workspace and a second kernel adds the splits in ascending s.
-constexpr int kBrWaves = 8;
+constexpr int kBrWaves = 16;
 constexpr unsigned kBrMaxSplits = 64;
 
 struct BrPlan {
@@ -45,7 +45,7 @@ static BrPlan br_plan(size_t n, unsigned bd, bool vec_ok) {
   return p;
 }
 
-template <int VEC, bool MUL>
+template <int VEC, bool MUL, bool NT>
 __global__ __launch_bounds__(64 * kBrWaves) void batch_reduce_kernel(size_t n, unsigned bd, unsigned per_split,
                                                                     const float* __restrict__ in0,
                                                                     const float* __restrict__ in1,
@@ -68,10 +68,10 @@ __global__ __launch_bounds__(64 * kBrWaves) void batch_reduce_kernel(size_t n, u
       for (int u = 0; u < U; ++u) {
         const size_t off = size_t(b + u * kBrWaves) * n + col;
         if (VEC == 4) {
-          const float4 t = *reinterpret_cast<const float4*>(in0 + off);
+          const float4 t = ldg4<NT>(reinterpret_cast<const float4*>(in0 + off));
           x[u][0] = t.x; x[u][1 % VEC] = t.y; x[u][2 % VEC] = t.z; x[u][3 % VEC] = t.w;
           if (MUL) {
-            const float4 s = *reinterpret_cast<const float4*>(in1 + off);
+            const float4 s = ldg4<NT>(reinterpret_cast<const float4*>(in1 + off));
             y[u][0] = s.x; y[u][1 % VEC] = s.y; y[u][2 % VEC] = s.z; y[u][3 % VEC] = s.w;
           }
         } else {
@@ -107,15 +107,51 @@ __global__ __launch_bounds__(64 * kBrWaves) void batch_reduce_kernel(size_t n, u
   }
 }
 
-// out[j] (+)= sum_s partial[s*n + j], ascending s
-__global__ __launch_bounds__(256) void combine_partials_kernel(size_t n, unsigned splits,
-                                                               const float* __restrict__ partial,
-                                                               float* __restrict__ out, int accumulate) {
-  const size_t j = size_t(blockIdx.x) * 256 + threadIdx.x;
-  if (j >= n) return;
-  float t = partial[j];
-  for (unsigned s = 1; s < splits; ++s) t += partial[size_t(s) * n + j];
-  out[j] = accumulate ? out[j] + t : t;
+// out[j] (+)= sum_s partial[s*n + j].  Block = 64 columns x kCombSlices slices:
+// slice q adds splits q, q+16, ... in ascending order with four loads in flight,
+// then the slices are added in ascending q.  blockIdx.y selects one of two
+// (partial, out) pairs so that two outputs share a launch.
+constexpr int kCombSlices = 16;
+__global__ __launch_bounds__(64 * kCombSlices) void combine_partials_kernel(size_t n, unsigned splits,
+                                                                           const float* __restrict__ partial0,
+                                                                           float* __restrict__ out0,
+                                                                           const float* __restrict__ partial1,
+                                                                           float* __restrict__ out1,
+                                                                           int accumulate) {
+  __shared__ float lds[kCombSlices][64];
+  const float* partial = blockIdx.y == 0 ? partial0 : partial1;
+  float* out = blockIdx.y == 0 ? out0 : out1;
+  const int lane = threadIdx.x & 63, q = threadIdx.x >> 6;
+  const size_t j = size_t(blockIdx.x) * 64 + lane;
+  float acc = 0.f;
+  if (j < n) {
+    unsigned sp = q;
+    for (; sp + 3 * kCombSlices < splits; sp += 4 * kCombSlices) {
+      const float a0 = partial[size_t(sp) * n + j], a1 = partial[size_t(sp + kCombSlices) * n + j],
+                  a2 = partial[size_t(sp + 2 * kCombSlices) * n + j],
+                  a3 = partial[size_t(sp + 3 * kCombSlices) * n + j];
+      acc += a0;
+      acc += a1;
+      acc += a2;
+      acc += a3;
+    }
+    for (; sp < splits; sp += kCombSlices) acc += partial[size_t(sp) * n + j];
+  }
+  lds[q][lane] = acc;
+  __syncthreads();
+  if (q == 0 && j < n) {
+    float t = lds[0][lane];
+#pragma unroll
+    for (int k = 1; k < kCombSlices; ++k) t += lds[k][lane];
+    out[j] = accumulate ? out[j] + t : t;
+  }
+}
+
+static void launch_combine(dyhip_device* dev, size_t n, unsigned splits, const float* p0, float* o0, const float* p1,
+                           float* o1, int accumulate) {
+  const dim3 grid((unsigned)cdiv<size_t>(n, 64), p1 != nullptr ? 2 : 1);
+  hipLaunchKernelGGL(combine_partials_kernel, grid, dim3(64 * kCombSlices), 0, dev->stream, n, splits, p0, o0, p1, o1,
+                     accumulate);
 }
 
 int batch_reduce(dyhip_device* dev, size_t n, unsigned bd, const float* in0, const float* in1, float* out,
@@ -133,19 +169,23 @@ int batch_reduce(dyhip_device* dev, size_t n, unsigned bd, const float* in0, con
   }
   const dim3 grid(p.tiles, p.splits), block(64 * kBrWaves);
   const int acc = accumulate ? 1 : 0;
-#define DYHIP_BR_LAUNCH(VEC, MUL)                                                                          \
-  hipLaunchKernelGGL((batch_reduce_kernel<VEC, MUL>), grid, block, 0, dev->stream, n, bd, p.per_split, in0, \
+  const bool stream = n * size_t(bd) * sizeof(float) >= dev->stream_threshold;
+#define DYHIP_BR_LAUNCH(VEC, MUL, NT)                                                                           \
+  hipLaunchKernelGGL((batch_reduce_kernel<VEC, MUL, NT>), grid, block, 0, dev->stream, n, bd, p.per_split, in0, \
                      in1, out, acc, partial)
   if (p.vec == 4) {
-    if (in1) DYHIP_BR_LAUNCH(4, true); else DYHIP_BR_LAUNCH(4, false);
+    if (stream) {
+      if (in1) DYHIP_BR_LAUNCH(4, true, true); else DYHIP_BR_LAUNCH(4, false, true);
+    } else {
+      if (in1) DYHIP_BR_LAUNCH(4, true, false); else DYHIP_BR_LAUNCH(4, false, false);
+    }
   } else {
-    if (in1) DYHIP_BR_LAUNCH(1, true); else DYHIP_BR_LAUNCH(1, false);
+    if (in1) DYHIP_BR_LAUNCH(1, true, false); else DYHIP_BR_LAUNCH(1, false, false);
   }
 #undef DYHIP_BR_LAUNCH
   DYHIP_CHECK_LAUNCH();
   if (partial) {
-    hipLaunchKernelGGL(combine_partials_kernel, dim3((unsigned)cdiv<size_t>(n, 256)), dim3(256), 0, dev->stream, n,
-                       p.splits, partial, out, acc);
+    launch_combine(dev, n, p.splits, partial, out, nullptr, nullptr, acc);
     DYHIP_CHECK_LAUNCH();
   }
   return DYHIP_OK;
@@ -216,7 +256,7 @@ constexpr int kLnWavesBwd = 8;
 constexpr unsigned kLnBwdMaxBlocks = 256;
 constexpr float kLnEps = 1e-8f;
 
-template <int VPL>
+template <int VPL, bool NT>
 __global__ __launch_bounds__(64 * kLnWavesFwd) void ln_fwd_wave_kernel(unsigned n4, unsigned bd,
                                                                       const float4* __restrict__ x,
                                                                       const float4* __restrict__ g,
@@ -231,7 +271,7 @@ __global__ __launch_bounds__(64 * kLnWavesFwd) void ln_fwd_wave_kernel(unsigned 
 #pragma unroll
   for (int u = 0; u < VPL; ++u) {
     const unsigned idx = lane + 64 * u;
-    v[u] = idx < n4 ? px[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+    v[u] = idx < n4 ? ldg4<NT>(px + idx) : make_float4(0.f, 0.f, 0.f, 0.f);
   }
   float s = 0.f;
 #pragma unroll
@@ -246,7 +286,8 @@ __global__ __launch_bounds__(64 * kLnWavesFwd) void ln_fwd_wave_kernel(unsigned 
     }
   }
   const float sigma = sqrtf(wave_sum(ss) / fn);
-  const float sden = kLnEps + sigma;
+  // one exact division per row; per element a multiply (within 1.5 ulp of x / (sigma + eps))
+  const float sden = 1.0f / (kLnEps + sigma);
   const float neg = -mean;
   float4* py = y + size_t(row) * n4;
 #pragma unroll
@@ -255,11 +296,11 @@ __global__ __launch_bounds__(64 * kLnWavesFwd) void ln_fwd_wave_kernel(unsigned 
     if (idx < n4) {
       const float4 gg = g[idx], bb = b[idx];
       float4 r;
-      r.x = gg.x * ((v[u].x + neg) / sden) + bb.x;
-      r.y = gg.y * ((v[u].y + neg) / sden) + bb.y;
-      r.z = gg.z * ((v[u].z + neg) / sden) + bb.z;
-      r.w = gg.w * ((v[u].w + neg) / sden) + bb.w;
-      py[idx] = r;
+      r.x = gg.x * ((v[u].x + neg) * sden) + bb.x;
+      r.y = gg.y * ((v[u].y + neg) * sden) + bb.y;
+      r.z = gg.z * ((v[u].z + neg) * sden) + bb.z;
+      r.w = gg.w * ((v[u].w + neg) * sden) + bb.w;
+      stg4<NT>(py + idx, r);
     }
   }
 }
@@ -288,7 +329,26 @@ __global__ __launch_bounds__(256) void ln_fwd_block_kernel(size_t n, const float
 #define DYHIP_F4_EACH(stmt) \
   { stmt(x) stmt(y) stmt(z) stmt(w) }
 
+// Registers of one row: x, dy and (when dx is requested) the old dx.
 template <int VPL>
+struct LnRow {
+  float4 v[VPL], d[VPL], o[VPL];
+};
+
+template <int VPL, bool NT>
+__device__ __forceinline__ void ln_row_load(LnRow<VPL>& r, unsigned n4, int lane, const float4* __restrict__ px,
+                                            const float4* __restrict__ pdy, const float4* __restrict__ pdx) {
+#pragma unroll
+  for (int u = 0; u < VPL; ++u) {
+    const unsigned idx = lane + 64 * u;
+    const bool in = idx < n4;
+    r.v[u] = in ? ldg4<NT>(px + idx) : make_float4(0.f, 0.f, 0.f, 0.f);
+    r.d[u] = in ? ldg4<NT>(pdy + idx) : make_float4(0.f, 0.f, 0.f, 0.f);
+    if (pdx != nullptr) r.o[u] = in ? ldg4<NT>(pdx + idx) : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+}
+
+template <int VPL, bool NT>
 __global__ __launch_bounds__(64 * kLnWavesBwd) void ln_bwd_wave_kernel(unsigned n4, unsigned bd,
                                                                       const float4* __restrict__ x,
                                                                       const float4* __restrict__ g,
@@ -308,54 +368,55 @@ __global__ __launch_bounds__(64 * kLnWavesBwd) void ln_bwd_wave_kernel(unsigned 
     pdg[u] = make_float4(0.f, 0.f, 0.f, 0.f);
     pdb[u] = make_float4(0.f, 0.f, 0.f, 0.f);
   }
-  const unsigned wave_global = blockIdx.x * kLnWavesBwd + w;
   const unsigned wave_count = gridDim.x * kLnWavesBwd;
-  for (unsigned row = wave_global; row < bd; row += wave_count) {
-    const float4* px = x + size_t(row) * n4;
-    const float4* pdy = dEdf + size_t(row) * n4;
-    float4 v[VPL], d[VPL];
-#pragma unroll
-    for (int u = 0; u < VPL; ++u) {
-      const unsigned idx = lane + 64 * u;
-      v[u] = idx < n4 ? px[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
-      d[u] = idx < n4 ? pdy[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
+  unsigned row = blockIdx.x * kLnWavesBwd + w;
+  LnRow<VPL> cur, nxt;
+  if (row < bd)
+    ln_row_load<VPL, NT>(cur, n4, lane, x + size_t(row) * n4, dEdf + size_t(row) * n4,
+                         dx ? dx + size_t(row) * n4 : nullptr);
+  while (row < bd) {
+    // the next row's loads are in flight while this row is reduced and written
+    const unsigned next = row + wave_count;
+    if (next < bd)
+      ln_row_load<VPL, NT>(nxt, n4, lane, x + size_t(next) * n4, dEdf + size_t(next) * n4,
+                           dx ? dx + size_t(next) * n4 : nullptr);
     float s = 0.f;
 #pragma unroll
-    for (int u = 0; u < VPL; ++u) s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+    for (int u = 0; u < VPL; ++u) s += (cur.v[u].x + cur.v[u].y) + (cur.v[u].z + cur.v[u].w);
     const float mean = wave_sum(s) / fn;
     float ss = 0.f;
 #pragma unroll
     for (int u = 0; u < VPL; ++u) {
       if (lane + 64 * u < n4) {
-        const float ax = v[u].x - mean, ay = v[u].y - mean, az = v[u].z - mean, aw = v[u].w - mean;
+        const float ax = cur.v[u].x - mean, ay = cur.v[u].y - mean, az = cur.v[u].z - mean, aw = cur.v[u].w - mean;
         ss += (ax * ax + ay * ay) + (az * az + aw * aw);
       }
     }
     const float sigma = sqrtf(wave_sum(ss) / fn);
-    const float sden = kLnEps + sigma, neg = -mean, s2 = sden * sden;
-    // per-row sums: ds = -sum dq/s^2 * xc ; dneg = sum dq/s, with dq = dy*g
-    float ds_p = 0.f, dneg_p = 0.f;
+    const float rs = 1.0f / (kLnEps + sigma);  // one exact division per row
+    const float neg = -mean;
+    // row sums: sum dq*xc and sum dq, with dq = dy*g
+    float sxq = 0.f, sq = 0.f;
 #pragma unroll
     for (int u = 0; u < VPL; ++u) {
       if (lane + 64 * u < n4) {
-#define DYHIP_LN_ROW(c)                      \
-  {                                          \
-    const float xc = v[u].c + neg;           \
-    const float dq = d[u].c * gg[u].c;       \
-    ds_p -= dq / s2 * xc;                    \
-    dneg_p += dq / sden;                     \
-    if (want_g) pdg[u].c += d[u].c * (xc / sden); \
-    if (want_b) pdb[u].c += d[u].c;          \
+#define DYHIP_LN_ROW(c)                                  \
+  {                                                      \
+    const float xc = cur.v[u].c + neg;                   \
+    const float dq = cur.d[u].c * gg[u].c;               \
+    sxq += dq * xc;                                      \
+    sq += dq;                                            \
+    if (want_g) pdg[u].c += cur.d[u].c * (xc * rs);      \
+    if (want_b) pdb[u].c += cur.d[u].c;                  \
   }
         DYHIP_F4_EACH(DYHIP_LN_ROW)
 #undef DYHIP_LN_ROW
       }
     }
     if (dx != nullptr) {
-      const float ds = wave_sum(ds_p);
-      const float dmu = -wave_sum(dneg_p);
-      const float sb = ds / (2.f * sigma);
+      const float ds = -(wave_sum(sxq) * rs) * rs;   // CwiseQuotient: -sum dq/s^2 * xc
+      const float dmu = -(wave_sum(sq) * rs);        // Negate(CwiseSum): -sum dq/s
+      const float sb = ds / (2.f * sigma);           // StdDimension: d / (2*sigma)
       const float c = 2.f / fn;
       const float dmu_n = dmu / fn;
       float4* pdx = dx + size_t(row) * n4;
@@ -363,21 +424,23 @@ __global__ __launch_bounds__(64 * kLnWavesBwd) void ln_bwd_wave_kernel(unsigned 
       for (int u = 0; u < VPL; ++u) {
         const unsigned idx = lane + 64 * u;
         if (idx < n4) {
-          float4 o = pdx[idx];
+          float4 o = cur.o[u];
 #define DYHIP_LN_DX(c_)                                            \
   {                                                                \
     float acc = o.c_;                                              \
-    acc += c * (v[u].c_ - mean) * sb;                              \
-    acc += (d[u].c_ * gg[u].c_) / sden;                            \
+    acc += c * (cur.v[u].c_ - mean) * sb;                          \
+    acc += (cur.d[u].c_ * gg[u].c_) * rs;                          \
     acc += dmu_n;                                                  \
     o.c_ = acc;                                                    \
   }
           DYHIP_F4_EACH(DYHIP_LN_DX)
 #undef DYHIP_LN_DX
-          pdx[idx] = o;
+          stg4<NT>(pdx + idx, o);
         }
       }
     }
+    if (next < bd) cur = nxt;
+    row = next;
   }
   if (!want_g && !want_b) return;
   const unsigned n = n4 * 4;
@@ -547,10 +610,17 @@ int dyhip_layer_norm_forward(dyhip_device* dev, size_t n, unsigned bd, const flo
     const float4 *x4 = reinterpret_cast<const float4*>(x), *g4 = reinterpret_cast<const float4*>(g),
                  *b4 = reinterpret_cast<const float4*>(b);
     float4* y4 = reinterpret_cast<float4*>(y);
-    if (n4 <= 64) hipLaunchKernelGGL(ln_fwd_wave_kernel<1>, grid, block, 0, dev->stream, n4, bd, x4, g4, b4, y4);
-    else if (n4 <= 128) hipLaunchKernelGGL(ln_fwd_wave_kernel<2>, grid, block, 0, dev->stream, n4, bd, x4, g4, b4, y4);
-    else if (n4 <= 256) hipLaunchKernelGGL(ln_fwd_wave_kernel<4>, grid, block, 0, dev->stream, n4, bd, x4, g4, b4, y4);
-    else hipLaunchKernelGGL(ln_fwd_wave_kernel<8>, grid, block, 0, dev->stream, n4, bd, x4, g4, b4, y4);
+    const bool stream = n * size_t(bd) * sizeof(float) >= dev->stream_threshold;
+#define DYHIP_LN_FWD(VPL)                                                                                       \
+  do {                                                                                                          \
+    if (stream) hipLaunchKernelGGL((ln_fwd_wave_kernel<VPL, true>), grid, block, 0, dev->stream, n4, bd, x4, g4, b4, y4); \
+    else hipLaunchKernelGGL((ln_fwd_wave_kernel<VPL, false>), grid, block, 0, dev->stream, n4, bd, x4, g4, b4, y4);       \
+  } while (0)
+    if (n4 <= 64) DYHIP_LN_FWD(1);
+    else if (n4 <= 128) DYHIP_LN_FWD(2);
+    else if (n4 <= 256) DYHIP_LN_FWD(4);
+    else DYHIP_LN_FWD(8);
+#undef DYHIP_LN_FWD
   } else {
     hipLaunchKernelGGL(ln_fwd_block_kernel, dim3(bd), dim3(256), 0, dev->stream, n, x, g, b, y);
   }
@@ -586,14 +656,25 @@ int dyhip_layer_norm_backward(dyhip_device* dev, size_t n, unsigned bd, const fl
     const float4 *x4 = reinterpret_cast<const float4*>(x), *g4 = reinterpret_cast<const float4*>(g),
                  *d4 = reinterpret_cast<const float4*>(dEdf);
     float4* dx4 = reinterpret_cast<float4*>(dx);
-    if (n4 <= 64) hipLaunchKernelGGL(ln_bwd_wave_kernel<1>, grid, block, lds, dev->stream, n4, bd, x4, g4, d4, dx4, part_dg, part_db);
-    else if (n4 <= 128) hipLaunchKernelGGL(ln_bwd_wave_kernel<2>, grid, block, lds, dev->stream, n4, bd, x4, g4, d4, dx4, part_dg, part_db);
-    else if (n4 <= 256) hipLaunchKernelGGL(ln_bwd_wave_kernel<4>, grid, block, lds, dev->stream, n4, bd, x4, g4, d4, dx4, part_dg, part_db);
-    else hipLaunchKernelGGL(ln_bwd_wave_kernel<8>, grid, block, lds, dev->stream, n4, bd, x4, g4, d4, dx4, part_dg, part_db);
+    const bool stream = n * size_t(bd) * sizeof(float) >= dev->stream_threshold;
+#define DYHIP_LN_BWD(VPL)                                                                                  \
+  do {                                                                                                     \
+    if (stream)                                                                                            \
+      hipLaunchKernelGGL((ln_bwd_wave_kernel<VPL, true>), grid, block, lds, dev->stream, n4, bd, x4, g4, d4, dx4, \
+                         part_dg, part_db);                                                                \
+    else                                                                                                   \
+      hipLaunchKernelGGL((ln_bwd_wave_kernel<VPL, false>), grid, block, lds, dev->stream, n4, bd, x4, g4, d4, dx4, \
+                         part_dg, part_db);                                                                \
+  } while (0)
+    if (n4 <= 64) DYHIP_LN_BWD(1);
+    else if (n4 <= 128) DYHIP_LN_BWD(2);
+    else if (n4 <= 256) DYHIP_LN_BWD(4);
+    else DYHIP_LN_BWD(8);
+#undef DYHIP_LN_BWD
     DYHIP_CHECK_LAUNCH();
-    const dim3 cgrid((unsigned)cdiv<size_t>(n, 256));
-    if (dg) hipLaunchKernelGGL(combine_partials_kernel, cgrid, dim3(256), 0, dev->stream, n, blocks, part_dg, dg, 1);
-    if (db) hipLaunchKernelGGL(combine_partials_kernel, cgrid, dim3(256), 0, dev->stream, n, blocks, part_db, db, 1);
+    if (dg && db) launch_combine(dev, n, blocks, part_dg, dg, part_db, db, 1);
+    else if (dg) launch_combine(dev, n, blocks, part_dg, dg, nullptr, nullptr, 1);
+    else if (db) launch_combine(dev, n, blocks, part_db, db, nullptr, nullptr, 1);
     DYHIP_CHECK_LAUNCH();
   } else {
     float2* stats = cols ? static_cast<float2*>(ws) : nullptr;

@@ -54,7 +54,7 @@ __device__ __forceinline__ MaxSum ms_merge(const MaxSum a, const MaxSum b) {
 
 // One block per batch element.  Writes m[b], z[b]; if ids != nullptr also
 // fx[b] = z[b] - x[ids[b]] (the pick of PickNegLogSoftmax).
-template <bool VEC>
+template <bool VEC, bool NT>
 __global__ __launch_bounds__(kLseThreads) void lse_cols_kernel(size_t rows, const float* __restrict__ x,
                                                                float* __restrict__ m_out, float* __restrict__ z_out,
                                                                const unsigned* __restrict__ ids,
@@ -70,13 +70,14 @@ __global__ __launch_bounds__(kLseThreads) void lse_cols_kernel(size_t rows, cons
     const size_t n4 = rows >> 2;
     size_t i = threadIdx.x;
     for (; i + 3 * kLseThreads < n4; i += 4 * kLseThreads) {
-      const float4 v0 = p4[i], v1 = p4[i + kLseThreads], v2 = p4[i + 2 * kLseThreads], v3 = p4[i + 3 * kLseThreads];
+      const float4 v0 = ldg4<NT>(p4 + i), v1 = ldg4<NT>(p4 + i + kLseThreads),
+                   v2 = ldg4<NT>(p4 + i + 2 * kLseThreads), v3 = ldg4<NT>(p4 + i + 3 * kLseThreads);
       ms_push4(a, v0);
       ms_push4(a, v1);
       ms_push4(a, v2);
       ms_push4(a, v3);
     }
-    for (; i < n4; i += kLseThreads) ms_push4(a, p4[i]);
+    for (; i < n4; i += kLseThreads) ms_push4(a, ldg4<NT>(p4 + i));
   } else {
     for (size_t i = threadIdx.x; i < rows; i += kLseThreads) ms_push1(a, px[i]);
   }
@@ -114,7 +115,7 @@ constexpr int kPbThreads = 256;
 constexpr int kPbUnroll = 4;
 
 // dx[:, b] += exp(x[:, b] - z[b]) * dy[b]; dx[ids[b]] -= dy[b]
-template <bool VEC>
+template <bool VEC, bool NT>
 __global__ __launch_bounds__(kPbThreads) void pnls_bwd_kernel(size_t rows, unsigned tiles_per_col,
                                                               const float* __restrict__ x,
                                                               const float* __restrict__ z,
@@ -136,7 +137,7 @@ __global__ __launch_bounds__(kPbThreads) void pnls_bwd_kernel(size_t rows, unsig
     for (int u = 0; u < kPbUnroll; ++u) {
       const size_t j = j0 + size_t(u) * kPbThreads;
       if (j < n4) {
-        xv[u] = x4[j];
+        xv[u] = ldg4<NT>(x4 + j);
         dv[u] = d4[j];
       }
     }
@@ -156,7 +157,7 @@ __global__ __launch_bounds__(kPbThreads) void pnls_bwd_kernel(size_t rows, unsig
           else if (c == 2) r.z -= dy;
           else r.w -= dy;
         }
-        d4[j] = r;
+        stg4<NT>(d4 + j, r);
       }
     }
   } else {
@@ -258,10 +259,13 @@ int batch_reduce(dyhip_device* dev, size_t n, unsigned bd, const float* in0, con
 static int launch_lse(dyhip_device* dev, size_t rows, unsigned bd, const float* x, float* m, float* z,
                       const unsigned* ids, float* fx) {
   const bool vec = rows % 4 == 0 && aligned16(x);
-  if (vec)
-    hipLaunchKernelGGL(lse_cols_kernel<true>, dim3(bd), dim3(kLseThreads), 0, dev->stream, rows, x, m, z, ids, fx);
+  const bool stream = rows * size_t(bd) * sizeof(float) >= dev->stream_threshold;
+  if (vec && stream)
+    hipLaunchKernelGGL((lse_cols_kernel<true, true>), dim3(bd), dim3(kLseThreads), 0, dev->stream, rows, x, m, z, ids, fx);
+  else if (vec)
+    hipLaunchKernelGGL((lse_cols_kernel<true, false>), dim3(bd), dim3(kLseThreads), 0, dev->stream, rows, x, m, z, ids, fx);
   else
-    hipLaunchKernelGGL(lse_cols_kernel<false>, dim3(bd), dim3(kLseThreads), 0, dev->stream, rows, x, m, z, ids, fx);
+    hipLaunchKernelGGL((lse_cols_kernel<false, false>), dim3(bd), dim3(kLseThreads), 0, dev->stream, rows, x, m, z, ids, fx);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
@@ -301,6 +305,15 @@ int dyhip_pnls_forward(dyhip_device* dev, size_t rows, unsigned bd, const float*
   return launch_lse(dev, rows, bd, x, m, z, ids_dev, fx);
 }
 
+int dyhip_pnls_forward_staged(dyhip_device* dev, size_t rows, unsigned bd, const float* x, void* aux, float* fx) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(rows >= 1 && x && aux && fx, "PickNegLogSoftmax needs non-empty tensors");
+  if (bd == 0) return DYHIP_OK;
+  float* z = static_cast<float*>(aux);
+  float* m = z + bd;
+  return launch_lse(dev, rows, bd, x, m, z, reinterpret_cast<const unsigned*>(m + bd), fx);
+}
+
 int dyhip_pnls_backward(dyhip_device* dev, size_t rows, unsigned bd, const float* x, const void* aux,
                         const float* dEdf, float* dEdx) {
   DYHIP_CHECK_DEV(dev);
@@ -313,10 +326,13 @@ int dyhip_pnls_backward(dyhip_device* dev, size_t rows, unsigned bd, const float
   const size_t tiles = cdiv(rows, per_tile);
   DYHIP_REQUIRE(tiles * bd < (size_t(1) << 31), "PickNegLogSoftmax backward launch too large");
   const dim3 grid(static_cast<unsigned>(tiles * bd));
-  if (vec)
-    hipLaunchKernelGGL(pnls_bwd_kernel<true>, grid, dim3(kPbThreads), 0, dev->stream, rows, (unsigned)tiles, x, z, ids, dEdf, dEdx);
+  const bool stream = rows * size_t(bd) * sizeof(float) >= dev->stream_threshold;
+  if (vec && stream)
+    hipLaunchKernelGGL((pnls_bwd_kernel<true, true>), grid, dim3(kPbThreads), 0, dev->stream, rows, (unsigned)tiles, x, z, ids, dEdf, dEdx);
+  else if (vec)
+    hipLaunchKernelGGL((pnls_bwd_kernel<true, false>), grid, dim3(kPbThreads), 0, dev->stream, rows, (unsigned)tiles, x, z, ids, dEdf, dEdx);
   else
-    hipLaunchKernelGGL(pnls_bwd_kernel<false>, grid, dim3(kPbThreads), 0, dev->stream, rows, (unsigned)tiles, x, z, ids, dEdf, dEdx);
+    hipLaunchKernelGGL((pnls_bwd_kernel<false, false>), grid, dim3(kPbThreads), 0, dev->stream, rows, (unsigned)tiles, x, z, ids, dEdf, dEdx);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }

@@ -112,6 +112,9 @@ class Device:
     def sync(self):
         _check(cdll.dyhip_device_sync(self.handle))
 
+    def set_stream_threshold(self, nbytes):
+        _check(cdll.dyhip_device_set_stream_threshold(self.handle, _sz(int(nbytes))))
+
     def pool(self, which):
         p = _vp(None)
         _check(cdll.dyhip_device_pool(self.handle, _i(which), C.byref(p)))
@@ -150,6 +153,14 @@ class Device:
 
     def free_pool(self, which):
         self.pool(which).free()
+
+    def graph_begin(self):
+        _check(cdll.dyhip_graph_begin_capture(self.handle))
+
+    def graph_end(self):
+        g = _vp(None)
+        _check(cdll.dyhip_graph_end_capture(self.handle, C.byref(g)))
+        return Graph(self, g)
 
     def timer_start(self):
         _check(cdll.dyhip_timer_start(self.handle))
@@ -325,6 +336,9 @@ class Device:
         _check(cdll.dyhip_pnls_forward(self.handle, _sz(rows), _u(bd), _p(x), _vp(labels_host.ctypes.data), _p(aux),
                                        _p(fx)))
 
+    def pnls_forward_staged(self, rows, bd, x, aux, fx):
+        _check(cdll.dyhip_pnls_forward_staged(self.handle, _sz(rows), _u(bd), _p(x), _p(aux), _p(fx)))
+
     def pnls_backward(self, rows, bd, x, aux, dEdf, dEdx):
         _check(cdll.dyhip_pnls_backward(self.handle, _sz(rows), _u(bd), _p(x), _p(aux), _p(dEdf), _p(dEdx)))
 
@@ -376,6 +390,22 @@ class Device:
         _check(cdll.dyhip_squared_l2norm_workspace(_sz(n), C.byref(need)))
         ws, nb = self.workspace(need.value)
         _check(cdll.dyhip_squared_l2norm(self.handle, _sz(n), _p(g), _p(out), _vp(ws), _sz(nb)))
+
+
+class Graph:
+    """A captured launch sequence (HIP graph) bound to its device's stream."""
+
+    def __init__(self, dev, handle):
+        self.dev = dev
+        self.handle = handle
+
+    def launch(self):
+        _check(cdll.dyhip_graph_launch(self.dev.handle, self.handle))
+
+    def destroy(self):
+        if self.handle is not None:
+            cdll.dyhip_graph_destroy(self.handle)
+            self.handle = None
 
 
 class Pool:

@@ -61,6 +61,10 @@ int dyhip_device_ordinal(const dyhip_device* dev, int* ordinal);
 int dyhip_device_stream(dyhip_device* dev, void** hip_stream);
 int dyhip_device_pool(dyhip_device* dev, int which, dyhip_pool** pool);
 int dyhip_device_scalar(dyhip_device* dev, int which, const float** ptr);
+/* Tensors of at least this many bytes are streamed with non-temporal accesses
+ * (default 8 MiB, twice the per-XCD L2); 0 streams everything, SIZE_MAX nothing.
+ * A tuning knob with no counterpart in the reference. */
+int dyhip_device_set_stream_threshold(dyhip_device* dev, size_t bytes);
 /* Device::allocate_tensor (dynet/devices.cc:82-88) */
 int dyhip_device_allocate(dyhip_device* dev, int which_pool, size_t nbytes, void** out);
 
@@ -86,6 +90,17 @@ int dyhip_memcpy_d2d(dyhip_device* dev, void* dst, const void* src, size_t nbyte
 int dyhip_zero(dyhip_device* dev, void* dst, size_t nbytes);
 int dyhip_constant(dyhip_device* dev, size_t n, float value, float* dst);       /* TensorTools::constant */
 int dyhip_accumulate(dyhip_device* dev, size_t n, const float* src, float* dst); /* TensorTools::accumulate: dst += src */
+
+/* Launch-bound inner loops: record the launches issued on the device stream
+ * between begin and end into a HIP graph and replay it with one call.  The
+ * reference has no counterpart (it launches node by node on the null stream);
+ * entry points that copy from host memory or synchronise (those taking *_host
+ * ids/labels) must stay outside a capture. */
+typedef struct dyhip_graph dyhip_graph;
+int dyhip_graph_begin_capture(dyhip_device* dev);
+int dyhip_graph_end_capture(dyhip_device* dev, dyhip_graph** out);
+int dyhip_graph_launch(dyhip_device* dev, dyhip_graph* graph);
+int dyhip_graph_destroy(dyhip_graph* graph);
 
 /* stream-ordered timing for benchmarks (hipEvent pair on the device stream) */
 int dyhip_timer_start(dyhip_device* dev);
@@ -203,6 +218,9 @@ int dyhip_logsumexp_cols(dyhip_device* dev, size_t rows, unsigned bd, const floa
  * labels_host are bounds-checked (:100). */
 int dyhip_pnls_forward(dyhip_device* dev, size_t rows, unsigned bd, const float* x, const unsigned* labels_host,
                        void* aux, float* fx);
+/* same, for callers that have already written ids (b*rows + label_b, validated) into
+ * the third part of aux on the device: no host copy, no synchronisation, capturable */
+int dyhip_pnls_forward_staged(dyhip_device* dev, size_t rows, unsigned bd, const float* x, void* aux, float* fx);
 int dyhip_pnls_backward(dyhip_device* dev, size_t rows, unsigned bd, const float* x, const void* aux,
                         const float* dEdf, float* dEdx);
 /* LogSumExp node over k <= 8 arguments (dynet/nodes-logsumexp.cc:38-97) */

@@ -152,11 +152,11 @@ def test_lstm_cell_forward_backward(dev, I, H, B, dims, dropout, mask_full):
         gt = dev.tensor(g0)
         dev.lstm_h_backward(H, B, cr_t, fxo_t, dht, i, gt)
         assert_close(gt.numpy(), orc.lstm_h_backward(H, B, c_ref, fx_ref, dh, i, g0.copy()), GRAD_RTOL, "h bwd %d" % i,
-                     floor=1e-4)
+                     floor=np.maximum(np.abs(g0), 1e-4))
         gt = dev.tensor(g0)
         dev.lstm_c_backward(H, B, ct, fxo_t, dev.tensor(dc_up), i, gt)
         assert_close(gt.numpy(), orc.lstm_c_backward(H, B, c_prev, fx_ref, dc_up, i, g0.copy()), GRAD_RTOL,
-                     "c bwd %d" % i, floor=1e-4)
+                     "c bwd %d" % i, floor=np.maximum(np.abs(g0), 1e-4))
     dgates = f32(rng.standard_normal((B, 4 * H)))
     dgt = dev.tensor(dgates)
     dpre_t = dev.empty((B, 4 * H))

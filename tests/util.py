@@ -39,15 +39,4 @@ def rms(a):
     return float(np.sqrt(np.mean(a * a))) if a.size else 0.0
 
 
-def zipf_ids(rng, n, vocab, s=1.1):
-    """Zipf(s) over [0, vocab): p(k) ~ (k+1)^-s, inverse-CDF sampling."""
-    p = (np.arange(1, vocab + 1, dtype=np.float64)) ** (-s)
-    cdf = np.cumsum(p)
-    cdf /= cdf[-1]
-    return np.minimum(np.searchsorted(cdf, rng.random(n)), vocab - 1).astype(np.uint32)
-
-
-def glorot(rng, rows, cols):
-    """ParameterInitGlorot (dynet/param-init.cc:26-40): U(+-sqrt(6)/sqrt(rows+cols)); column-major rows x cols."""
-    s = np.sqrt(6.0) / np.sqrt(rows + cols)
-    return f32(rng.uniform(-s, s, (cols, rows)))
+from dynet_amd.synth import glorot, zipf_ids  # noqa: E402,F401
