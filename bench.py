@@ -196,8 +196,14 @@ def extras(dev, lib, reps):
     # the scatter-add is a library sort followed by two kernels: timed as plain launches, outside a graph
     scatter = [("lookup_scatter_add(sort+segmented)", G + 2 * uniq * D * 4,
                 lambda s: dev.lookup_accumulate_grads(s["ids"], D, V, s["g"], s["grads"], ws, wsb))]
+    for s in sets:
+        s["plan"] = dev.lookup_build_plan(s["ids"], V)
+    ws2, wsb2 = dev.workspace(dev.lookup_accumulate_grads_planned_workspace(n, D))
+    planned = [("lookup_scatter_add(ids pre-sorted at forward)", G + 2 * uniq * D * 4,
+                lambda s: dev.lookup_accumulate_grads_planned(n, s["plan"], D, V, s["g"], s["grads"], ws2, wsb2))]
     res["cfg3_lookup"] = {"vocab": V, "dim": D, "n_ids": n, "unique_ids": uniq,
                           "kernels": per_kernel_table(dev, gather, sets, reps) +
+                          per_kernel_table(dev, planned, sets, reps) +
                           per_kernel_table(dev, scatter, sets, reps, use_graph=False)}
     for w in (lib.POOL_FXS, lib.POOL_DEDFS, lib.POOL_SCS):
         dev.sync()

@@ -86,8 +86,6 @@ struct ScatterWs {
   unsigned* last_row;    // per chunk: row of a run that begins here and continues into the next chunk, else kNone
   float* part_first;     // [chunks][dim]
   float* part_last;      // [chunks][dim]
-  void* sort_tmp;
-  size_t sort_tmp_bytes;
   unsigned chunks;
 };
 
@@ -235,35 +233,67 @@ static int sort_tmp_bytes(unsigned n, unsigned vocab, size_t* bytes) {
   return DYHIP_OK;
 }
 
-static int carve(unsigned n, size_t dim, unsigned vocab, void* ws, size_t ws_bytes, ScatterWs* out, size_t* need) {
+// plan = [sorted_ids (n u32) | sorted_pos (n u32)], each part padded to 256 bytes
+static size_t plan_bytes(unsigned n) { return 2 * align256(sizeof(unsigned) * n); }
+
+// scratch of the reduction kernels = [last_row | part_first | part_last]
+static size_t reduce_ws_bytes(unsigned n, size_t dim) {
   const unsigned chunks = cdiv<unsigned>(n, kChunk);
+  return align256(sizeof(unsigned) * chunks) + 2 * align256(sizeof(float) * dim * chunks);
+}
+
+static int build_plan(dyhip_device* dev, unsigned n, const unsigned* ids_dev, unsigned vocab, void* plan,
+                      size_t plan_size, void* ws, size_t ws_bytes) {
   size_t sort_bytes = 0;
   DYHIP_CHECK_STATUS(sort_tmp_bytes(n, vocab, &sort_bytes));
-  size_t off = 0;
-  auto take = [&](size_t bytes) {
-    size_t o = off;
-    off += align256(bytes);
-    return o;
-  };
-  const size_t o_ids = take(sizeof(unsigned) * n), o_pos = take(sizeof(unsigned) * n);
-  const size_t o_lr = take(sizeof(unsigned) * chunks);
-  const size_t o_pf = take(sizeof(float) * dim * chunks), o_pl = take(sizeof(float) * dim * chunks);
-  const size_t o_tmp = take(sort_bytes);
-  if (need) *need = off;
-  if (out) {
-    if (ws == nullptr || ws_bytes < off)
-      return fail(DYHIP_ERR_INVALID_ARG, "lookup scatter-add needs %zu workspace bytes, got %zu", off, ws_bytes);
-    if (!aligned16(ws)) return fail(DYHIP_ERR_INVALID_ARG, "lookup scatter-add workspace must be 16-byte aligned");
-    char* base = static_cast<char*>(ws);
-    out->sorted_ids = reinterpret_cast<unsigned*>(base + o_ids);
-    out->sorted_pos = reinterpret_cast<unsigned*>(base + o_pos);
-    out->last_row = reinterpret_cast<unsigned*>(base + o_lr);
-    out->part_first = reinterpret_cast<float*>(base + o_pf);
-    out->part_last = reinterpret_cast<float*>(base + o_pl);
-    out->sort_tmp = base + o_tmp;
-    out->sort_tmp_bytes = sort_bytes;
-    out->chunks = chunks;
+  DYHIP_REQUIRE(plan != nullptr && plan_size >= plan_bytes(n) && aligned16(plan),
+                "lookup plan needs %zu bytes (16-byte aligned), got %zu", plan_bytes(n), plan_size);
+  DYHIP_REQUIRE(sort_bytes == 0 || (ws != nullptr && ws_bytes >= sort_bytes),
+                "lookup plan needs %zu workspace bytes, got %zu", sort_bytes, ws_bytes);
+  unsigned* sorted_ids = static_cast<unsigned*>(plan);
+  unsigned* sorted_pos = reinterpret_cast<unsigned*>(static_cast<char*>(plan) + align256(sizeof(unsigned) * n));
+  DYHIP_CHECK_HIP(rocprim::radix_sort_pairs(ws, sort_bytes, ids_dev, sorted_ids,
+                                            rocprim::counting_iterator<unsigned>(0), sorted_pos, n, 0, key_bits(vocab),
+                                            dev->stream));
+  return DYHIP_OK;
+}
+
+static int reduce_planned(dyhip_device* dev, unsigned n, const void* plan, size_t dim, unsigned vocab, const float* g,
+                          float* all_grads, void* ws, size_t ws_bytes) {
+  const size_t need = reduce_ws_bytes(n, dim);
+  DYHIP_REQUIRE(ws != nullptr && ws_bytes >= need && aligned16(ws),
+                "lookup scatter-add needs %zu workspace bytes (16-byte aligned), got %zu", need, ws_bytes);
+  ScatterWs w;
+  w.chunks = cdiv<unsigned>(n, kChunk);
+  w.sorted_ids = const_cast<unsigned*>(static_cast<const unsigned*>(plan));
+  w.sorted_pos = reinterpret_cast<unsigned*>(const_cast<char*>(static_cast<const char*>(plan)) +
+                                             align256(sizeof(unsigned) * n));
+  char* base = static_cast<char*>(ws);
+  w.last_row = reinterpret_cast<unsigned*>(base);
+  w.part_first = reinterpret_cast<float*>(base + align256(sizeof(unsigned) * w.chunks));
+  w.part_last = reinterpret_cast<float*>(base + align256(sizeof(unsigned) * w.chunks) +
+                                         align256(sizeof(float) * dim * w.chunks));
+  const bool vec = dim % 4 == 0 && aligned16(g) && aligned16(all_grads);
+  const unsigned dimv = static_cast<unsigned>(vec ? dim / 4 : dim);
+  const unsigned tpr = threads_per_row(dimv);
+  const dim3 grid(cdiv<unsigned>(w.chunks, kLkThreads / tpr)), block(kLkThreads);
+  const dim3 fgrid(w.chunks), fblock(kFixThreads);
+  const size_t flds = size_t(kFixThreads) * (vec ? sizeof(float4) : sizeof(float));
+  const bool stream = size_t(n) * dim * sizeof(float) >= dev->stream_threshold;
+  if (vec) {
+    float4* gr = reinterpret_cast<float4*>(all_grads);
+    const float4* g4 = reinterpret_cast<const float4*>(g);
+    if (stream)
+      hipLaunchKernelGGL((scatter_chunk_kernel<float4, true>), grid, block, 0, dev->stream, n, dimv, tpr, vocab, w, g4, gr);
+    else
+      hipLaunchKernelGGL((scatter_chunk_kernel<float4, false>), grid, block, 0, dev->stream, n, dimv, tpr, vocab, w, g4, gr);
+    hipLaunchKernelGGL(scatter_fixup_kernel<float4>, fgrid, fblock, flds, dev->stream, n, dimv, tpr, vocab, w, gr);
+  } else {
+    hipLaunchKernelGGL((scatter_chunk_kernel<float, false>), grid, block, 0, dev->stream, n, dimv, tpr, vocab, w, g,
+                       all_grads);
+    hipLaunchKernelGGL(scatter_fixup_kernel<float>, fgrid, fblock, flds, dev->stream, n, dimv, tpr, vocab, w, all_grads);
   }
+  DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
 
@@ -308,13 +338,53 @@ int dyhip_lookup_forward(dyhip_device* dev, unsigned n_ids, const unsigned* ids_
   return DYHIP_OK;
 }
 
+int dyhip_lookup_plan_bytes(unsigned n_ids, size_t* bytes) {
+  DYHIP_REQUIRE(bytes != nullptr, "null output pointer");
+  *bytes = n_ids ? plan_bytes(n_ids) : 0;
+  return DYHIP_OK;
+}
+
+int dyhip_lookup_plan_workspace(unsigned n_ids, unsigned vocab, size_t* ws_bytes) {
+  DYHIP_REQUIRE(ws_bytes != nullptr, "null output pointer");
+  *ws_bytes = 0;
+  if (n_ids == 0) return DYHIP_OK;
+  size_t b = 0;
+  DYHIP_CHECK_STATUS(sort_tmp_bytes(n_ids, vocab, &b));
+  *ws_bytes = align256(b);
+  return DYHIP_OK;
+}
+
+int dyhip_lookup_build_plan(dyhip_device* dev, unsigned n_ids, const unsigned* ids_dev, unsigned vocab, void* plan,
+                            size_t plan_size, void* ws, size_t ws_bytes) {
+  DYHIP_CHECK_DEV(dev);
+  if (n_ids == 0) return DYHIP_OK;
+  DYHIP_REQUIRE(ids_dev != nullptr, "null pointer in lookup plan");
+  return build_plan(dev, n_ids, ids_dev, vocab, plan, plan_size, ws, ws_bytes);
+}
+
+int dyhip_lookup_accumulate_grads_planned_workspace(unsigned n_ids, size_t dim, size_t* ws_bytes) {
+  DYHIP_REQUIRE(ws_bytes != nullptr, "null output pointer");
+  *ws_bytes = (n_ids == 0 || dim == 0) ? 0 : reduce_ws_bytes(n_ids, dim);
+  return DYHIP_OK;
+}
+
+int dyhip_lookup_accumulate_grads_planned(dyhip_device* dev, unsigned n_ids, const void* plan, size_t dim,
+                                          unsigned vocab, const float* g, float* all_grads, void* ws, size_t ws_bytes) {
+  DYHIP_CHECK_DEV(dev);
+  if (n_ids == 0 || dim == 0) return DYHIP_OK;
+  DYHIP_REQUIRE(plan && g && all_grads, "null pointer in lookup accumulate_grads");
+  DYHIP_REQUIRE(dim < (size_t(1) << 31), "lookup dimension too large");
+  return reduce_planned(dev, n_ids, plan, dim, vocab, g, all_grads, ws, ws_bytes);
+}
+
 int dyhip_lookup_accumulate_grads_workspace(unsigned n_ids, size_t dim, unsigned vocab, size_t* ws_bytes) {
   DYHIP_REQUIRE(ws_bytes != nullptr, "null output pointer");
-  if (n_ids == 0 || dim == 0) {
-    *ws_bytes = 0;
-    return DYHIP_OK;
-  }
-  return carve(n_ids, dim, vocab, nullptr, 0, nullptr, ws_bytes);
+  *ws_bytes = 0;
+  if (n_ids == 0 || dim == 0) return DYHIP_OK;
+  size_t sort_ws = 0;
+  DYHIP_CHECK_STATUS(dyhip_lookup_plan_workspace(n_ids, vocab, &sort_ws));
+  *ws_bytes = plan_bytes(n_ids) + reduce_ws_bytes(n_ids, dim) + sort_ws;
+  return DYHIP_OK;
 }
 
 int dyhip_lookup_accumulate_grads(dyhip_device* dev, unsigned n_ids, const unsigned* ids_dev, size_t dim,
@@ -323,37 +393,14 @@ int dyhip_lookup_accumulate_grads(dyhip_device* dev, unsigned n_ids, const unsig
   if (n_ids == 0 || dim == 0) return DYHIP_OK;
   DYHIP_REQUIRE(ids_dev && g && all_grads, "null pointer in lookup accumulate_grads");
   DYHIP_REQUIRE(dim < (size_t(1) << 31), "lookup dimension too large");
-  ScatterWs w;
-  DYHIP_CHECK_STATUS(carve(n_ids, dim, vocab, ws, ws_bytes, &w, nullptr));
-  size_t tmp_bytes = w.sort_tmp_bytes;
-  DYHIP_CHECK_HIP(rocprim::radix_sort_pairs(w.sort_tmp, tmp_bytes, ids_dev, w.sorted_ids,
-                                            rocprim::counting_iterator<unsigned>(0), w.sorted_pos, n_ids, 0,
-                                            key_bits(vocab), dev->stream));
-  const bool vec = dim % 4 == 0 && aligned16(g) && aligned16(all_grads);
-  const unsigned dimv = static_cast<unsigned>(vec ? dim / 4 : dim);
-  const unsigned tpr = threads_per_row(dimv);
-  const dim3 grid(cdiv<unsigned>(w.chunks, kLkThreads / tpr)), block(kLkThreads);
-  const dim3 fgrid(w.chunks), fblock(kFixThreads);
-  const size_t flds = size_t(kFixThreads) * (vec ? sizeof(float4) : sizeof(float));
-  const bool stream = size_t(n_ids) * dim * sizeof(float) >= dev->stream_threshold;
-  if (vec && stream) {
-    hipLaunchKernelGGL((scatter_chunk_kernel<float4, true>), grid, block, 0, dev->stream, n_ids, dimv, tpr, vocab, w,
-                       reinterpret_cast<const float4*>(g), reinterpret_cast<float4*>(all_grads));
-    hipLaunchKernelGGL(scatter_fixup_kernel<float4>, fgrid, fblock, flds, dev->stream, n_ids, dimv, tpr, vocab, w,
-                       reinterpret_cast<float4*>(all_grads));
-  } else if (vec) {
-    hipLaunchKernelGGL((scatter_chunk_kernel<float4, false>), grid, block, 0, dev->stream, n_ids, dimv, tpr, vocab, w,
-                       reinterpret_cast<const float4*>(g), reinterpret_cast<float4*>(all_grads));
-    hipLaunchKernelGGL(scatter_fixup_kernel<float4>, fgrid, fblock, flds, dev->stream, n_ids, dimv, tpr, vocab, w,
-                       reinterpret_cast<float4*>(all_grads));
-  } else {
-    hipLaunchKernelGGL((scatter_chunk_kernel<float, false>), grid, block, 0, dev->stream, n_ids, dimv, tpr, vocab, w, g,
-                       all_grads);
-    hipLaunchKernelGGL(scatter_fixup_kernel<float>, fgrid, fblock, flds, dev->stream, n_ids, dimv, tpr, vocab, w,
-                       all_grads);
-  }
-  DYHIP_CHECK_LAUNCH();
-  return DYHIP_OK;
+  size_t need = 0;
+  DYHIP_CHECK_STATUS(dyhip_lookup_accumulate_grads_workspace(n_ids, dim, vocab, &need));
+  DYHIP_REQUIRE(ws != nullptr && ws_bytes >= need && aligned16(ws),
+                "lookup scatter-add needs %zu workspace bytes (16-byte aligned), got %zu", need, ws_bytes);
+  char* base = static_cast<char*>(ws);
+  const size_t pb = plan_bytes(n_ids), rb = reduce_ws_bytes(n_ids, dim);
+  DYHIP_CHECK_STATUS(build_plan(dev, n_ids, ids_dev, vocab, base, pb, base + pb + rb, ws_bytes - pb - rb));
+  return reduce_planned(dev, n_ids, base, dim, vocab, g, all_grads, base + pb, rb);
 }
 
 }  // extern "C"

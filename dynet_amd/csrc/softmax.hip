@@ -69,6 +69,14 @@ __global__ __launch_bounds__(kLseThreads) void lse_cols_kernel(size_t rows, cons
     const float4* p4 = reinterpret_cast<const float4*>(px);
     const size_t n4 = rows >> 2;
     size_t i = threadIdx.x;
+    // eight independent 128-bit loads in flight per thread before the first exp
+    for (; i + 7 * kLseThreads < n4; i += 8 * kLseThreads) {
+      float4 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = ldg4<NT>(p4 + i + u * kLseThreads);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) ms_push4(a, v[u]);
+    }
     for (; i + 3 * kLseThreads < n4; i += 4 * kLseThreads) {
       const float4 v0 = ldg4<NT>(p4 + i), v1 = ldg4<NT>(p4 + i + kLseThreads),
                    v2 = ldg4<NT>(p4 + i + 2 * kLseThreads), v3 = ldg4<NT>(p4 + i + 3 * kLseThreads);

@@ -326,6 +326,29 @@ class Device:
         _check(cdll.dyhip_lookup_accumulate_grads(self.handle, _u(n), _p(ids_dev), _sz(dim), _u(vocab), _p(g),
                                                   _p(all_grads), _vp(ws), _sz(ws_bytes)))
 
+    def lookup_build_plan(self, ids_dev, vocab):
+        """Sorted (id, position) plan of a lookup's ids; returns the plan buffer (FXS pool)."""
+        n = ids_dev.size
+        pb, wb = _sz(0), _sz(0)
+        _check(cdll.dyhip_lookup_plan_bytes(_u(n), C.byref(pb)))
+        _check(cdll.dyhip_lookup_plan_workspace(_u(n), _u(vocab), C.byref(wb)))
+        plan = DevTensor(self, self.alloc(max(pb.value, 1)), (pb.value // 4,), np.uint32)
+        ws, nb = self.workspace(wb.value)
+        _check(cdll.dyhip_lookup_build_plan(self.handle, _u(n), _p(ids_dev), _u(vocab), _p(plan), _sz(pb.value),
+                                            _vp(ws), _sz(nb)))
+        return plan
+
+    def lookup_accumulate_grads_planned_workspace(self, n_ids, dim):
+        b = _sz(0)
+        _check(cdll.dyhip_lookup_accumulate_grads_planned_workspace(_u(n_ids), _sz(dim), C.byref(b)))
+        return b.value
+
+    def lookup_accumulate_grads_planned(self, n_ids, plan, dim, vocab, g, all_grads, ws=None, ws_bytes=None):
+        if ws is None:
+            ws, ws_bytes = self.workspace(self.lookup_accumulate_grads_planned_workspace(n_ids, dim))
+        _check(cdll.dyhip_lookup_accumulate_grads_planned(self.handle, _u(n_ids), _p(plan), _sz(dim), _u(vocab), _p(g),
+                                                          _p(all_grads), _vp(ws), _sz(ws_bytes)))
+
     # ---- logsumexp / pnls -------------------------------------------------
     def logsumexp_cols(self, rows, bd, x, m, z):
         _check(cdll.dyhip_logsumexp_cols(self.handle, _sz(rows), _u(bd), _p(x), _p(m), _p(z)))

@@ -207,6 +207,16 @@ int dyhip_lookup_forward(dyhip_device* dev, unsigned n_ids, const unsigned* ids_
 /* all_grads[:, ids[b]] += g[:, b], duplicates summed in ascending b by a
  * sorted-index segmented reduction (no atomics, deterministic). */
 int dyhip_lookup_accumulate_grads_workspace(unsigned n_ids, size_t dim, unsigned vocab, size_t* ws_bytes);
+/* The same in two phases.  The sorted (id, position) plan depends only on the ids, so
+ * an executor can build it right after the forward gather (the ids sit in the node's
+ * aux_mem from then on) and the backward pass is left with the reduction kernels. */
+int dyhip_lookup_plan_bytes(unsigned n_ids, size_t* plan_bytes);
+int dyhip_lookup_plan_workspace(unsigned n_ids, unsigned vocab, size_t* ws_bytes);
+int dyhip_lookup_build_plan(dyhip_device* dev, unsigned n_ids, const unsigned* ids_dev, unsigned vocab, void* plan,
+                            size_t plan_bytes, void* ws, size_t ws_bytes);
+int dyhip_lookup_accumulate_grads_planned_workspace(unsigned n_ids, size_t dim, size_t* ws_bytes);
+int dyhip_lookup_accumulate_grads_planned(dyhip_device* dev, unsigned n_ids, const void* plan, size_t dim,
+                                          unsigned vocab, const float* g, float* all_grads, void* ws, size_t ws_bytes);
 int dyhip_lookup_accumulate_grads(dyhip_device* dev, unsigned n_ids, const unsigned* ids_dev, size_t dim,
                                   unsigned vocab, const float* g, float* all_grads, void* ws, size_t ws_bytes);
 

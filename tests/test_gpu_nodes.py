@@ -245,6 +245,13 @@ def test_lookup_gather_bit_exact_and_scatter_add(dev, vocab, dim, n):
     gt2 = dev.tensor(grads0)
     dev.lookup_accumulate_grads(ids_t, dim, vocab, dev.tensor(g), gt2)
     assert gt2.numpy().tobytes() == got.tobytes()
+    # two-phase form: plan built once (e.g. at forward time), reduction kernels at backward time
+    plan = dev.lookup_build_plan(ids_t, vocab)
+    sorted_ids = plan.numpy()[:n]
+    assert np.array_equal(sorted_ids, np.sort(ids))
+    gt3 = dev.tensor(grads0)
+    dev.lookup_accumulate_grads_planned(n, plan, dim, vocab, dev.tensor(g), gt3)
+    assert gt3.numpy().tobytes() == got.tobytes()
 
 
 def test_lookup_all_ids_equal_and_all_distinct(dev):
