@@ -52,6 +52,9 @@ def parse_args():
                     help="override the library's non-temporal access threshold in bytes (tuning experiments)")
     ap.add_argument("--kernel-reps", type=int, default=20, help="graph replays per per-kernel measurement")
     ap.add_argument("--no-graph", action="store_true", help="time plain back-to-back launches instead of graph replays")
+    ap.add_argument("--one-pass", action="store_true",
+                    help="counter-collection mode: launch every kernel of the sweep (and a 16.8 MB calibration copy) "
+                         "a few times with plain launches, print nothing but a short note, and exit")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the cfg 1 / 3 / 4 kernel measurements")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="bound on the CPU-baseline leg")
@@ -314,6 +317,16 @@ def main():
     if args.stream_threshold is not None:
         dev.set_stream_threshold(args.stream_threshold)
     sweep = Sweep(dev, lib, args.sets)
+    if args.one_pass:
+        # hardware-counter runs (rocprofv3 --pmc ...): plain launches so that every dispatch is attributed
+        for r in range(min(4, sweep.R)):
+            b = sweep.sets[r]
+            dev.scale_copy(S_ELEMS, b["x"], 1.0, b["y"])  # calibration: reads 16 MiB, writes 16 MiB
+            sweep.run_step(r)
+        dev.sync()
+        dev.close()
+        print(json.dumps({"one_pass": True, "calibration": "ew_vec4_kernel<..IdentityFwd> moves 16384 KiB each way"}))
+        return
     # ---- whole-step timing: one captured graph per buffer set ---------------------
     sweep.run_step(0)
     dev.sync()

@@ -23,7 +23,8 @@ constexpr int kGemmMaxSeg = 2;
 
 enum GemmEpilogue {
   kEpiAxpby = 0,      // C = beta*C + sum
-  kEpiLstmGates = 1   // C = act(bias[i] + (H <= i < 2H ? 1 : 0) + sum), logistic rows [0,3H), tanh rows [3H,4H)
+  kEpiLstmGates = 1,  // C = act(bias[i] + (H <= i < 2H ? 1 : 0) + sum), logistic rows [0,3H), tanh rows [3H,4H)
+  kEpiBias = 2        // C = bias[i] + sum   (AffineTransform: bias broadcast over the columns)
 };
 
 struct GemmEpiParams {

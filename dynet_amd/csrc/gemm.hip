@@ -42,6 +42,7 @@ struct GemmArgs {
   size_t M, N;
   float* C;         // used when partial == nullptr
   float beta;       // used when partial == nullptr
+  const float* bias;  // when set (and partial == nullptr): C = bias[i] + sum
   float* partial;   // [splits][M*N] or nullptr
 };
 
@@ -211,6 +212,12 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_tile_kernel(GemmArgs g, uns
       if (i >= g.M) continue;
       float* p = out + i + j * g.M;
       float4 v = make_float4(acc[t2][4 * q], acc[t2][4 * q + 1], acc[t2][4 * q + 2], acc[t2][4 * q + 3]);
+      if (direct && g.bias != nullptr) {
+        v.x += g.bias[i];
+        if (i + 1 < g.M) v.y += g.bias[i + 1];
+        if (i + 2 < g.M) v.z += g.bias[i + 2];
+        if (i + 3 < g.M) v.w += g.bias[i + 3];
+      }
       if (vec_store && i + 3 < g.M) {
         if (direct && g.beta != 0.f) {
           const float4 o = *reinterpret_cast<const float4*>(p);
@@ -241,6 +248,10 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(size_t M, size_
     float s = partial[e];
     for (unsigned k = 1; k < splits; ++k) s += partial[size_t(k) * total + e];
     C[e] = ep.beta != 0.f ? ep.beta * C[e] + s : s;
+  } else if (EPI == kEpiBias) {
+    float s = ep.bias[e % M];
+    for (unsigned k = 0; k < splits; ++k) s += partial[size_t(k) * total + e];
+    C[e] = s;
   } else {
     const unsigned i = static_cast<unsigned>(e % M);
     float pre = ep.bias[i];
@@ -272,7 +283,8 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
   g.M = M;
   g.N = N;
   g.C = C;
-  g.beta = epi.beta;
+  g.beta = epi.kind == kEpiBias ? 0.f : epi.beta;
+  g.bias = epi.kind == kEpiBias ? epi.bias : nullptr;
   g.ktiles_total = 0;
   bool a_vec = true, b_vec = true;
   for (int s = 0; s < nseg; ++s) {
@@ -301,7 +313,7 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
     if (want > 65535) want = 65535;
     splits = want < 1 ? 1u : static_cast<unsigned>(want);
   }
-  const bool fused_epi = epi.kind != kEpiAxpby;
+  const bool fused_epi = epi.kind == kEpiLstmGates;  // needs the whole sum before the activation
   const bool use_partial = splits > 1 || fused_epi;
   if (use_partial)
     DYHIP_REQUIRE(dev->gemm_ws_bytes >= out_bytes * splits,
@@ -321,6 +333,9 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
     const dim3 grid((unsigned)cdiv<size_t>(total, 256));
     if (fused_epi)
       hipLaunchKernelGGL(gemm_splitk_reduce_kernel<kEpiLstmGates>, grid, dim3(256), 0, dev->stream, M, total, splits,
+                         g.partial, C, epi);
+    else if (epi.kind == kEpiBias)
+      hipLaunchKernelGGL(gemm_splitk_reduce_kernel<kEpiBias>, grid, dim3(256), 0, dev->stream, M, total, splits,
                          g.partial, C, epi);
     else
       hipLaunchKernelGGL(gemm_splitk_reduce_kernel<kEpiAxpby>, grid, dim3(256), 0, dev->stream, M, total, splits,
@@ -342,6 +357,15 @@ int dyhip_gemm_nn(dyhip_device* dev, size_t M, size_t N, size_t K, const float* 
   GemmSeg s{l, M, r, K, K};
   GemmEpiParams ep{kEpiAxpby, beta, nullptr, 0, 0};
   return gemm_run(dev, false, true, M, N, 1, &s, y, ep);
+}
+
+int dyhip_affine_forward(dyhip_device* dev, size_t M, size_t N, size_t K, const float* bias, const float* W,
+                         const float* x, float* fx) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(bias != nullptr, "AffineTransform: null bias");
+  GemmSeg s{W, M, x, K, K};
+  GemmEpiParams ep{kEpiBias, 0.f, bias, 0, 0};
+  return gemm_run(dev, false, true, M, N, 1, &s, fx, ep);
 }
 
 int dyhip_gemm_tn_acc(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float* y) {

@@ -65,6 +65,9 @@ __global__ __launch_bounds__(kLseThreads) void lse_cols_kernel(size_t rows, cons
   MaxSum a;
   a.m = -INFINITY;
   a.s = 0.f;
+  // the picked logit is fetched up front so that its two dependent loads overlap the streaming pass
+  float picked = 0.f;
+  if (ids != nullptr && threadIdx.x == 0) picked = x[ids[b]];
   if (VEC) {
     const float4* p4 = reinterpret_cast<const float4*>(px);
     const size_t n4 = rows >> 2;
@@ -102,20 +105,24 @@ __global__ __launch_bounds__(kLseThreads) void lse_cols_kernel(size_t rows, cons
     ls[w] = a.s;
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
+  if (w == 0) {
+    // wave 0 merges the per-wave pairs with a butterfly over the first kLseWaves lanes
     MaxSum t;
-    t.m = lm[0];
-    t.s = ls[0];
-    for (int k = 1; k < kLseWaves; ++k) {
+    t.m = lane < kLseWaves ? lm[lane] : -INFINITY;
+    t.s = lane < kLseWaves ? ls[lane] : 0.f;
+#pragma unroll
+    for (int off = kLseWaves / 2; off > 0; off >>= 1) {
       MaxSum o;
-      o.m = lm[k];
-      o.s = ls[k];
+      o.m = __shfl_xor(t.m, off, kWave);
+      o.s = __shfl_xor(t.s, off, kWave);
       t = ms_merge(t, o);
     }
-    const float z = logf(t.s) + t.m;
-    m_out[b] = t.m;
-    z_out[b] = z;
-    if (ids != nullptr) fx[b] = z - x[ids[b]];
+    if (lane == 0) {
+      const float z = logf(t.s) + t.m;
+      m_out[b] = t.m;
+      z_out[b] = z;
+      if (ids != nullptr) fx[b] = z - picked;
+    }
   }
 }
 

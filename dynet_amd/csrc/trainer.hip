@@ -1,0 +1,159 @@
+// Trainer kernels: gradient clipping scale on the device, the SimpleSGD rule with a
+// device-resident scale, and the sparse (touched rows only) lookup update.
+//
+// Replaces Trainer::clip_gradients / gradient_l2_norm (dynet/training.cc:173-187,
+// dynet/model.cc:806-848: one device malloc, one blocking device-to-host float copy
+// and one free per parameter per update), SimpleSGDTrainer::update_rule_dev
+// (dynet/training.cc:619-622), the per-row lookup updates of dynet/training.cc:215-226
+// and LookupParameterStorage::clear, which on the GPU zeroes the whole gradient table
+// (dynet/model.cc:175-186).
+#include "common.h"
+
+namespace dyhip {
+
+static size_t align256(size_t n) { return (n + 255) / 256 * 256; }
+
+__global__ void clip_scale_kernel(unsigned n, const float* __restrict__ sqnorms, float threshold,
+                                  float* __restrict__ gscale) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  float s = 0.f;
+  for (unsigned i = 0; i < n; ++i) s += sqnorms[i];
+  const float gg = sqrtf(s);
+  *gscale = (threshold > 0.f && gg > threshold) ? threshold / gg : 1.0f;
+}
+
+template <bool CLEAR>
+__global__ __launch_bounds__(256) void sgd_scaled_kernel(size_t n4, size_t n, float* __restrict__ p,
+                                                         float* __restrict__ g, float lr, float wd,
+                                                         const float* __restrict__ gscale) {
+  const float s = lr * *gscale / wd;
+  const size_t stride = size_t(gridDim.x) * 256;
+  float4* p4 = reinterpret_cast<float4*>(p);
+  float4* g4 = reinterpret_cast<float4*>(g);
+  for (size_t i = size_t(blockIdx.x) * 256 + threadIdx.x; i < n4; i += stride) {
+    float4 pv = p4[i];
+    const float4 gv = g4[i];
+    pv.x -= gv.x * s;
+    pv.y -= gv.y * s;
+    pv.z -= gv.z * s;
+    pv.w -= gv.w * s;
+    p4[i] = pv;
+    if (CLEAR) g4[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  for (size_t i = (n4 << 2) + size_t(blockIdx.x) * 256 + threadIdx.x; i < n; i += stride) {
+    p[i] -= g[i] * s;
+    if (CLEAR) g[i] = 0.f;
+  }
+}
+
+// one block per sorted position; only the first entry of each run of equal ids acts
+__global__ __launch_bounds__(128) void sgd_rows_kernel(unsigned n, const unsigned* __restrict__ sorted_ids,
+                                                       unsigned dim, unsigned vocab, float* __restrict__ values,
+                                                       float* __restrict__ grads, float lr, float wd,
+                                                       const float* __restrict__ gscale) {
+  const unsigned k = blockIdx.x;
+  const unsigned id = sorted_ids[k];
+  if (id >= vocab || (k > 0 && sorted_ids[k - 1] == id)) return;
+  const float s = lr * *gscale / wd;
+  float* pv = values + size_t(id) * dim;
+  float* pg = grads + size_t(id) * dim;
+  for (unsigned j = threadIdx.x; j < dim; j += 128) {
+    pv[j] -= pg[j] * s;
+    pg[j] = 0.f;
+  }
+}
+
+__global__ __launch_bounds__(128) void sqnorm_rows_kernel(unsigned n, const unsigned* __restrict__ sorted_ids,
+                                                          unsigned dim, unsigned vocab,
+                                                          const float* __restrict__ grads,
+                                                          float* __restrict__ partial) {
+  __shared__ float red[2];
+  const unsigned k = blockIdx.x;
+  const unsigned id = sorted_ids[k];
+  const bool head = id < vocab && !(k > 0 && sorted_ids[k - 1] == id);
+  float s = 0.f;
+  if (head) {
+    const float* pg = grads + size_t(id) * dim;
+    for (unsigned j = threadIdx.x; j < dim; j += 128) s += pg[j] * pg[j];
+  }
+  const float t = block_sum<2>(s, red);
+  if (threadIdx.x == 0) partial[k] = t;
+}
+
+__global__ __launch_bounds__(256) void sum_partials_kernel(unsigned n, const float* __restrict__ partial,
+                                                           float* __restrict__ out) {
+  __shared__ float red[4];
+  float s = 0.f;
+  for (unsigned i = threadIdx.x; i < n; i += 256) s += partial[i];
+  const float t = block_sum<4>(s, red);
+  if (threadIdx.x == 0) *out = t;
+}
+
+}  // namespace dyhip
+
+using namespace dyhip;
+
+extern "C" {
+
+int dyhip_clip_scale(dyhip_device* dev, unsigned n, const float* sqnorms, float threshold, float* gscale) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(gscale != nullptr && (n == 0 || sqnorms != nullptr), "null pointer");
+  hipLaunchKernelGGL(clip_scale_kernel, dim3(1), dim3(64), 0, dev->stream, n, sqnorms, threshold, gscale);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_sgd_update_scaled(dyhip_device* dev, size_t n, float* p, float* g, float lr, const float* gscale,
+                            float wd, int clear_grad) {
+  DYHIP_CHECK_DEV(dev);
+  if (n == 0) return DYHIP_OK;
+  DYHIP_REQUIRE(p && g && gscale, "null pointer");
+  DYHIP_REQUIRE(wd != 0.f, "weight decay scale must be non-zero");
+  const bool vec = aligned16(p) && aligned16(g);
+  const size_t n4 = vec ? n / 4 : 0;
+  unsigned blocks = static_cast<unsigned>(cdiv<size_t>(n, size_t(256) * 16));
+  if (blocks < 1) blocks = 1;
+  if (blocks > 4096) blocks = 4096;
+  if (clear_grad)
+    hipLaunchKernelGGL(sgd_scaled_kernel<true>, dim3(blocks), dim3(256), 0, dev->stream, n4, n, p, g, lr, wd, gscale);
+  else
+    hipLaunchKernelGGL(sgd_scaled_kernel<false>, dim3(blocks), dim3(256), 0, dev->stream, n4, n, p, g, lr, wd, gscale);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_sgd_update_rows(dyhip_device* dev, unsigned n_ids, const void* plan, size_t dim, unsigned vocab,
+                          float* values, float* grads, float lr, const float* gscale, float wd) {
+  DYHIP_CHECK_DEV(dev);
+  if (n_ids == 0 || dim == 0) return DYHIP_OK;
+  DYHIP_REQUIRE(plan && values && grads && gscale, "null pointer");
+  DYHIP_REQUIRE(wd != 0.f && dim < (size_t(1) << 31), "bad weight decay scale or dimension");
+  hipLaunchKernelGGL(sgd_rows_kernel, dim3(n_ids), dim3(128), 0, dev->stream, n_ids,
+                     static_cast<const unsigned*>(plan), (unsigned)dim, vocab, values, grads, lr, wd, gscale);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_squared_l2norm_rows_workspace(unsigned n_ids, size_t* ws_bytes) {
+  DYHIP_REQUIRE(ws_bytes != nullptr, "null output pointer");
+  *ws_bytes = align256(sizeof(float) * (n_ids ? n_ids : 1));
+  return DYHIP_OK;
+}
+
+int dyhip_squared_l2norm_rows(dyhip_device* dev, unsigned n_ids, const void* plan, size_t dim, unsigned vocab,
+                              const float* grads, float* out, void* ws, size_t ws_bytes) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(out != nullptr, "null pointer");
+  if (n_ids == 0 || dim == 0) return dyhip_zero(dev, out, sizeof(float));
+  DYHIP_REQUIRE(plan && grads, "null pointer");
+  DYHIP_REQUIRE(ws != nullptr && ws_bytes >= sizeof(float) * n_ids, "squared_l2norm_rows needs %zu workspace bytes",
+                sizeof(float) * n_ids);
+  float* partial = static_cast<float*>(ws);
+  hipLaunchKernelGGL(sqnorm_rows_kernel, dim3(n_ids), dim3(128), 0, dev->stream, n_ids,
+                     static_cast<const unsigned*>(plan), (unsigned)dim, vocab, grads, partial);
+  hipLaunchKernelGGL(sum_partials_kernel, dim3(1), dim3(256), 0, dev->stream, n_ids, partial, out);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+}  // extern "C"

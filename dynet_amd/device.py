@@ -252,6 +252,9 @@ class Device:
     def gemm_nn(self, M, N, K, l, r, beta, y):
         _check(cdll.dyhip_gemm_nn(self.handle, _sz(M), _sz(N), _sz(K), _p(l), _p(r), _f(beta), _p(y)))
 
+    def affine_forward(self, M, N, K, bias, W, x, fx):
+        _check(cdll.dyhip_affine_forward(self.handle, _sz(M), _sz(N), _sz(K), _p(bias), _p(W), _p(x), _p(fx)))
+
     def gemm_tn_acc(self, M, N, K, l, r, y):
         _check(cdll.dyhip_gemm_tn_acc(self.handle, _sz(M), _sz(N), _sz(K), _p(l), _p(r), _p(y)))
 
@@ -338,6 +341,19 @@ class Device:
                                             _vp(ws), _sz(nb)))
         return plan
 
+    def lookup_plan_buffers(self, n_ids, vocab):
+        """(plan, workspace, workspace bytes) for repeated lookup_build_plan_into calls."""
+        pb, wb = _sz(0), _sz(0)
+        _check(cdll.dyhip_lookup_plan_bytes(_u(n_ids), C.byref(pb)))
+        _check(cdll.dyhip_lookup_plan_workspace(_u(n_ids), _u(vocab), C.byref(wb)))
+        plan = DevTensor(self, self.alloc(max(pb.value, 1)), (pb.value // 4,), np.uint32)
+        ws, nb = self.workspace(wb.value)
+        return plan, ws, nb
+
+    def lookup_build_plan_into(self, ids_dev, vocab, plan, ws, ws_bytes):
+        _check(cdll.dyhip_lookup_build_plan(self.handle, _u(ids_dev.size), _p(ids_dev), _u(vocab), _p(plan),
+                                            _sz(plan.nbytes), _vp(ws), _sz(ws_bytes)))
+
     def lookup_accumulate_grads_planned_workspace(self, n_ids, dim):
         b = _sz(0)
         _check(cdll.dyhip_lookup_accumulate_grads_planned_workspace(_u(n_ids), _sz(dim), C.byref(b)))
@@ -407,6 +423,24 @@ class Device:
 
     def sgd_update(self, n, p, g, lr, gscale=1.0, wd=1.0):
         _check(cdll.dyhip_sgd_update(self.handle, _sz(n), _p(p), _p(g), _f(lr), _f(gscale), _f(wd)))
+
+    def clip_scale(self, n, sqnorms, threshold, gscale):
+        _check(cdll.dyhip_clip_scale(self.handle, _u(n), _p(sqnorms), _f(threshold), _p(gscale)))
+
+    def sgd_update_scaled(self, n, p, g, lr, gscale_dev, wd=1.0, clear_grad=True):
+        _check(cdll.dyhip_sgd_update_scaled(self.handle, _sz(n), _p(p), _p(g), _f(lr), _p(gscale_dev), _f(wd),
+                                            _i(1 if clear_grad else 0)))
+
+    def sgd_update_rows(self, n_ids, plan, dim, vocab, values, grads, lr, gscale_dev, wd=1.0):
+        _check(cdll.dyhip_sgd_update_rows(self.handle, _u(n_ids), _p(plan), _sz(dim), _u(vocab), _p(values),
+                                          _p(grads), _f(lr), _p(gscale_dev), _f(wd)))
+
+    def squared_l2norm_rows(self, n_ids, plan, dim, vocab, grads, out):
+        need = _sz(0)
+        _check(cdll.dyhip_squared_l2norm_rows_workspace(_u(n_ids), C.byref(need)))
+        ws, nb = self.workspace(need.value)
+        _check(cdll.dyhip_squared_l2norm_rows(self.handle, _u(n_ids), _p(plan), _sz(dim), _u(vocab), _p(grads),
+                                              _p(out), _vp(ws), _sz(nb)))
 
     def squared_l2norm(self, n, g, out):
         need = _sz(0)

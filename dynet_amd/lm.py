@@ -1,0 +1,203 @@
+"""Batched LSTM language-model training step on the HIP device: the graph of
+examples/batching/rnnlm-batch.h:86-151 (lookup -> CompactVanillaLSTMBuilder, dynet/lstm.cc:905-926,1044-1080
+-> bias + R*h -> pickneglogsoftmax -> sum_batches(sum(errs))) followed by cg.backward and
+SimpleSGDTrainer::update (dynet/training.cc:173-256,619-637), issued as one launch sequence and replayed as a
+HIP graph.
+
+What differs from DyNet's node-at-a-time execution (results agree to fp32 rounding):
+  * the T lookups, the T projections and the T PickNegLogSoftmax nodes of a step run as one call each over
+    T*B columns (what DyNet's autobatching does to them);
+  * with ``time_batched=True`` the weight/bias gradients of the gate GEMMs are formed once per layer over the
+    K = T*B columns of all timesteps instead of T times over B columns;
+  * gradient clipping never leaves the device: squared norms -> clip scale -> update all read device memory.
+"""
+import numpy as np
+
+from . import lib
+from .synth import glorot
+
+
+class LstmLM:
+    """V-word LM: embedding E, L layers of hidden H, batch B, T timesteps per step."""
+
+    def __init__(self, dev, V, E, H, L, B, T, seed=0, lr=0.1, clip=5.0, time_batched=True, params=None):
+        self.dev, self.V, self.E, self.H, self.L, self.B, self.T = dev, V, E, H, L, B, T
+        self.lr, self.clip, self.time_batched = float(lr), float(clip), bool(time_batched)
+        N = self.N = T * B
+        PS, FXS, DE = lib.POOL_PS, lib.POOL_FXS, lib.POOL_DEDFS
+        if params is None:
+            params = self.init_params(V, E, H, L, seed)
+        # parameters and their gradients (PS pool), names as in the reference model
+        self.p, self.g = {}, {}
+        for name, a in params.items():
+            self.p[name] = dev.tensor(a, pool=PS)
+            self.g[name] = dev.zeros(a.shape, pool=PS)
+        self.dense = [n for n in self.p if n != "C"]
+        self.sqnorms = dev.zeros((len(self.dense) + 1,), pool=PS)
+        self.gscale = dev.zeros((1,), pool=PS)
+        # forward values (FXS pool); [t] slices are contiguous so [T, B, *] is one matrix with T*B columns
+        self.ids = dev.empty((N,), np.uint32, pool=FXS)
+        self.emb = dev.empty((T, B, E), pool=FXS)
+        self.h0 = dev.zeros((B, H), pool=FXS)  # zeros(): the initial h and c of every layer
+        self.h = [dev.empty((T, B, H), pool=FXS) for _ in range(L)]
+        self.c = [dev.empty((T, B, H), pool=FXS) for _ in range(L)]
+        self.gates = [dev.empty((T, B, 4 * H), pool=FXS) for _ in range(L)]
+        self.logits = dev.empty((N, V), pool=FXS)
+        self.aux = dev.empty((3 * N,), pool=FXS)  # [z | m | ids] of PickNegLogSoftmax
+        self.errs = dev.empty((N,), pool=FXS)
+        self.loss = dev.empty((1,), pool=FXS)
+        # gradients of the forward values (DEDFS pool), zeroed at the start of every backward pass
+        self.de_begin = dev.pool(DE).used()
+        self.d_errs = dev.empty((N,), pool=DE)
+        self.d_logits = dev.empty((N, V), pool=DE)
+        self.d_emb = dev.empty((T, B, E), pool=DE)
+        self.d_h = [dev.empty((T, B, H), pool=DE) for _ in range(L)]
+        self.d_c = [dev.empty((T, B, H), pool=DE) for _ in range(L)]
+        self.d_gates = [dev.empty((T, B, 4 * H), pool=DE) for _ in range(L)]
+        self.de_bytes = dev.pool(DE).used() - self.de_begin
+        self.d_pre = [dev.empty((T, B, 4 * H), pool=DE) for _ in range(L)]  # overwritten, never accumulated into
+        self.plan, self.plan_ws, self.plan_ws_bytes = dev.lookup_plan_buffers(N, V)
+        self.graph = None
+
+    @staticmethod
+    def init_params(V, E, H, L, seed=0):
+        """ParameterInitGlorot as the reference model's constructors apply it (dynet/param-init.cc:26-40):
+        lookup table scaled by its embedding dimension only, LSTM biases zero (dynet/lstm.cc:916)."""
+        rng = np.random.default_rng(seed)
+        s = np.sqrt(3.0) / np.sqrt(E)
+        p = {"C": rng.uniform(-s, s, (V, E)).astype(np.float32)}
+        d_in = E
+        for l in range(L):
+            p[f"Wx{l}"] = glorot(rng, 4 * H, d_in)
+            p[f"Wh{l}"] = glorot(rng, 4 * H, H)
+            p[f"b{l}"] = np.zeros(4 * H, np.float32)
+            d_in = H
+        p["R"] = glorot(rng, V, H)
+        s = np.sqrt(3.0) / np.sqrt(V)
+        p["bias"] = rng.uniform(-s, s, V).astype(np.float32)
+        return p
+
+    # ---- one step ---------------------------------------------------------------
+    def stage(self, tokens):
+        """Host -> device: tokens[T+1, B]; rows 0..T-1 are the inputs, rows 1..T the words to predict."""
+        tokens = np.ascontiguousarray(tokens, dtype=np.uint32)
+        assert tokens.shape == (self.T + 1, self.B), tokens.shape
+        if tokens.max() >= self.V:
+            raise ValueError("token id out of the vocabulary")
+        self.ids.set(tokens[:-1].reshape(-1))
+        flat = np.arange(self.N, dtype=np.uint64) * self.V + tokens[1:].reshape(-1)
+        if flat.max() >= 2 ** 32:
+            raise ValueError("PickNegLogSoftmax indexes its input with 32-bit offsets")
+        self.aux.offset(2 * self.N, (self.N,)).set(flat.astype(np.uint32).view(np.float32))
+
+    def _t(self, buf, t, width):
+        return buf.offset(t * self.B * width, (self.B, width))
+
+    def forward(self):
+        d, V, E, H, L, B, T, N = self.dev, self.V, self.E, self.H, self.L, self.B, self.T, self.N
+        d.lookup_forward(None, self.ids, E, V, self.p["C"], self.emb)
+        for t in range(T):
+            x, d_in = self._t(self.emb, t, E), E
+            for l in range(L):
+                h_tm1 = self._t(self.h[l], t - 1, H) if t > 0 else self.h0
+                c_tm1 = self._t(self.c[l], t - 1, H) if t > 0 else self.h0
+                g, c, h = self._t(self.gates[l], t, 4 * H), self._t(self.c[l], t, H), self._t(self.h[l], t, H)
+                d.lstm_gates_forward([x], [d_in], H, B, h_tm1, self.p[f"Wx{l}"], self.p[f"Wh{l}"], self.p[f"b{l}"], g)
+                d.lstm_c_forward(H, B, c_tm1, g, c)
+                d.lstm_h_forward(H, B, c, g, h)
+                x, d_in = h, H
+        d.affine_forward(V, N, H, self.p["bias"], self.p["R"], self.h[L - 1], self.logits)
+        d.pnls_forward_staged(V, N, self.logits, self.aux, self.errs)
+        d.sum_batches_forward(1, N, self.errs, self.loss)
+
+    def backward(self):
+        d, V, E, H, L, B, T, N = self.dev, self.V, self.E, self.H, self.L, self.B, self.T, self.N
+        d.zero(lib_tensor(d, self.d_errs.ptr, self.de_bytes))
+        d.constant(self.d_errs, 1.0)  # d loss / d errs[b] through sum_batches(sum(errs))
+        d.pnls_backward(V, N, self.logits, self.aux, self.d_errs, self.d_logits)
+        top = self.h[L - 1]
+        d.csum_backward(V, 1, N, self.d_logits, 0, self.g["bias"])
+        d.gemm_nt_acc(V, H, N, self.d_logits, top, self.g["R"])
+        d.gemm_tn_acc(H, N, V, self.p["R"], self.d_logits, self.d_h[L - 1])
+        for t in reversed(range(T)):
+            for l in reversed(range(L)):
+                g, c = self._t(self.gates[l], t, 4 * H), self._t(self.c[l], t, H)
+                c_tm1 = self._t(self.c[l], t - 1, H) if t > 0 else self.h0
+                h_tm1 = self._t(self.h[l], t - 1, H) if t > 0 else self.h0
+                dh, dc, dg = self._t(self.d_h[l], t, H), self._t(self.d_c[l], t, H), self._t(self.d_gates[l], t, 4 * H)
+                dpre = self._t(self.d_pre[l], t, 4 * H)
+                d.lstm_h_backward(H, B, c, g, dh, 0, dc)
+                d.lstm_h_backward(H, B, c, g, dh, 1, dg)
+                if t > 0:
+                    d.lstm_c_backward(H, B, c_tm1, g, dc, 0, self._t(self.d_c[l], t - 1, H))
+                d.lstm_c_backward(H, B, c_tm1, g, dc, 1, dg)
+                d.lstm_gates_dpre(H, B, g, dg, dpre)
+                if l > 0:
+                    x, d_in, dx = self._t(self.h[l - 1], t, H), H, self._t(self.d_h[l - 1], t, H)
+                else:
+                    x, d_in, dx = self._t(self.emb, t, E), E, self._t(self.d_emb, t, E)
+                d.gemm_tn_acc(d_in, B, 4 * H, self.p[f"Wx{l}"], dpre, dx)
+                if t > 0:
+                    d.gemm_tn_acc(H, B, 4 * H, self.p[f"Wh{l}"], dpre, self._t(self.d_h[l], t - 1, H))
+                if not self.time_batched:
+                    d.gemm_nt_acc(4 * H, d_in, B, dpre, x, self.g[f"Wx{l}"])
+                    if t > 0:  # h_tm1 of the first step is the zero state: its product adds nothing
+                        d.gemm_nt_acc(4 * H, H, B, dpre, h_tm1, self.g[f"Wh{l}"])
+                    d.csum_backward(4 * H, 1, B, dpre, 0, self.g[f"b{l}"])
+        if self.time_batched:
+            for l in range(L):
+                x, d_in = (self.h[l - 1], H) if l > 0 else (self.emb, E)
+                d.gemm_nt_acc(4 * H, d_in, N, self.d_pre[l], x, self.g[f"Wx{l}"])
+                if T > 1:
+                    d.gemm_nt_acc(4 * H, H, N - B, self._t(self.d_pre[l], 1, 4 * H), self.h[l], self.g[f"Wh{l}"])
+                d.csum_backward(4 * H, 1, N, self.d_pre[l], 0, self.g[f"b{l}"])
+        d.lookup_accumulate_grads_planned(N, self.plan, E, V, self.d_emb, self.g["C"])
+
+    def update(self):
+        d = self.dev
+        for k, n in enumerate(self.dense):
+            d.squared_l2norm(self.g[n].size, self.g[n], self.sqnorms.offset(k, (1,)))
+        k = len(self.dense)
+        d.squared_l2norm_rows(self.N, self.plan, self.E, self.V, self.g["C"], self.sqnorms.offset(k, (1,)))
+        d.clip_scale(k + 1, self.sqnorms, self.clip, self.gscale)
+        for n in self.dense:
+            d.sgd_update_scaled(self.p[n].size, self.p[n], self.g[n], self.lr, self.gscale, 1.0, True)
+        d.sgd_update_rows(self.N, self.plan, self.E, self.V, self.p["C"], self.g["C"], self.lr, self.gscale, 1.0)
+
+    def issue(self):
+        """The whole step on the device stream (ids and labels already staged)."""
+        self.dev.lookup_build_plan_into(self.ids, self.V, self.plan, self.plan_ws, self.plan_ws_bytes)
+        self.forward()
+        self.backward()
+        self.update()
+
+    def capture(self):
+        """Record the step once; ``step`` then replays it."""
+        self.dev.sync()
+        self.dev.graph_begin()
+        try:
+            self.issue()
+        finally:
+            self.graph = self.dev.graph_end()
+        return self.graph
+
+    def step(self, tokens, read_loss=True):
+        self.stage(tokens)
+        if self.graph is not None:
+            self.graph.launch()
+        else:
+            self.issue()
+        if read_loss:
+            return float(self.loss.numpy()[0])
+        return None
+
+    def get_params(self):
+        return {n: t.numpy() for n, t in self.p.items()}
+
+    def get_grads(self):
+        return {n: t.numpy() for n, t in self.g.items()}
+
+
+def lib_tensor(dev, ptr, nbytes):
+    from .device import DevTensor
+    return DevTensor(dev, ptr, (nbytes,), np.uint8)

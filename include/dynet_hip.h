@@ -167,6 +167,13 @@ int dyhip_gemm_tn_acc(dyhip_device* dev, size_t M, size_t N, size_t K, const flo
 /* MatrixMultiplyTranspAcc (:162-180): y[MxN] += l[MxK] * r[NxK]^T */
 int dyhip_gemm_nt_acc(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float* y);
 
+/* AffineTransform with one (W, x) pair (dynet/nodes-affinetransform.cc:77-113):
+ * fx[MxN] = bias[M] broadcast over the N columns + W[MxK] * x[KxN], the bias folded into
+ * the GEMM epilogue.  Its backward (:115-156) is dyhip_sum_batches_forward-style reduction
+ * for the bias (dyhip_csum_backward), dyhip_gemm_nt_acc for W and dyhip_gemm_tn_acc for x. */
+int dyhip_affine_forward(dyhip_device* dev, size_t M, size_t N, size_t K, const float* bias, const float* W,
+                         const float* x, float* fx);
+
 /* ---- fused LSTM nodes (dynet/nodes-lstm.cc) ------------------------------ */
 /* VanillaLSTMGates::forward_dev_impl (:101-235).  xs[k] (HOST array of DEVICE
  * pointers) has x_dims[k] rows and B columns; mask_x/mask_h NULL = no dropout,
@@ -257,6 +264,23 @@ int dyhip_parallel_accumulate(dyhip_device* dev, int num_seqs, int max_len, floa
 int dyhip_scale_copy(dyhip_device* dev, size_t n, const float* src, float mult, float* dst);
 /* SimpleSGDTrainer::update_rule_dev (dynet/training.cc:619-622): p -= g * (lr*gscale/wd) */
 int dyhip_sgd_update(dyhip_device* dev, size_t n, float* p, const float* g, float lr, float gscale, float wd);
+/* Trainer::clip_gradients (dynet/training.cc:173-187) without the per-parameter blocking
+ * device-to-host copy of dynet/model.cc:830-842: *gscale (device) = min(1, threshold /
+ * sqrt(sum of the n squared norms)); threshold <= 0 disables clipping (gscale = 1). */
+int dyhip_clip_scale(dyhip_device* dev, unsigned n, const float* sqnorms, float threshold, float* gscale);
+/* the SGD rule with gscale read on the device; clear_grad != 0 also zeroes g (ParameterStorage::clear) */
+int dyhip_sgd_update_scaled(dyhip_device* dev, size_t n, float* p, float* g, float lr, const float* gscale,
+                            float wd, int clear_grad);
+/* Sparse lookup update (dynet/training.cc:215-226,630-637) over the distinct ids of a lookup plan:
+ * values[:, id] -= grads[:, id] * (lr*gscale/wd); grads[:, id] = 0 (LookupParameterStorage::clear
+ * restricted to the touched rows, dynet/model.cc:175-186) */
+int dyhip_sgd_update_rows(dyhip_device* dev, unsigned n_ids, const void* plan, size_t dim, unsigned vocab,
+                          float* values, float* grads, float lr, const float* gscale, float wd);
+/* LookupParameterStorage::g_squared_l2norm_dev over non_zero_grads (dynet/model.cc:664-675): the sum of
+ * squares of the gradient rows named by the plan, each distinct id once */
+int dyhip_squared_l2norm_rows_workspace(unsigned n_ids, size_t* ws_bytes);
+int dyhip_squared_l2norm_rows(dyhip_device* dev, unsigned n_ids, const void* plan, size_t dim, unsigned vocab,
+                              const float* grads, float* out, void* ws, size_t ws_bytes);
 /* ParameterStorage::g_squared_l2norm_dev (dynet/model.cc): *out(device) = sum g^2 */
 int dyhip_squared_l2norm_workspace(size_t n, size_t* ws_bytes);
 int dyhip_squared_l2norm(dyhip_device* dev, size_t n, const float* g, float* out, void* ws, size_t ws_bytes);

@@ -1,0 +1,100 @@
+"""LSTM language-model training step on the GPU against the node-by-node CPU oracle composition
+(examples/batching/rnnlm-batch.h:110-151 + Trainer::update), at sizes the oracle finishes in seconds."""
+import numpy as np
+import pytest
+
+from oracle import lm_oracle
+from dynet_amd.lm import LstmLM
+from dynet_amd.synth import zipf_ids
+from util import assert_close, FWD_RTOL, GRAD_RTOL
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # V, E, H, L, B, T
+    (50, 16, 32, 2, 8, 5),
+    (37, 12, 20, 2, 5, 4),
+    (64, 8, 16, 1, 3, 1),
+    (300, 64, 128, 2, 32, 6),
+]
+
+
+def _tokens(rng, V, B, T):
+    return zipf_ids(rng, (T + 1) * B, V).reshape(T + 1, B)
+
+
+def _grad_floor(ref):
+    # accumulated sums of many signed terms: floor the relative error at a fraction of the tensor's scale
+    return max(float(np.abs(ref).max()) * 1e-2, 1e-6)
+
+
+@pytest.mark.parametrize("time_batched", [False, True])
+@pytest.mark.parametrize("case", CASES)
+def test_lm_step_matches_oracle(dev, case, time_batched):
+    V, E, H, L, B, T = case
+    rng = np.random.default_rng(11)
+    params = LstmLM.init_params(V, E, H, L, seed=3)
+    for l in range(L):  # non-zero biases exercise the bias path
+        params[f"b{l}"] = rng.normal(0, 0.1, 4 * H).astype(np.float32)
+    ref_p = {n: a.copy() for n, a in params.items()}
+    lm = LstmLM(dev, V, E, H, L, B, T, lr=0.1, clip=5.0, time_batched=time_batched, params=params)
+    for it in range(2):
+        tokens = _tokens(rng, V, B, T)
+        ref_loss, ref_g, ref_scale = lm_oracle.step(ref_p, tokens, L, lr=0.1, clip=5.0)
+        lm.stage(tokens)
+        lm.dev.lookup_build_plan_into(lm.ids, V, lm.plan, lm.plan_ws, lm.plan_ws_bytes)
+        lm.forward()
+        lm.backward()
+        loss = lm.loss.numpy()[0]
+        grads = lm.get_grads()
+        lm.update()
+        assert_close(loss, ref_loss, FWD_RTOL * 4, f"loss step {it}")
+        for n in ref_g:
+            assert_close(grads[n], ref_g[n], GRAD_RTOL, f"grad {n} step {it}", floor=_grad_floor(ref_g[n]))
+        assert_close(lm.gscale.numpy()[0], ref_scale, GRAD_RTOL, f"clip scale step {it}")
+        new_p = lm.get_params()
+        for n in ref_p:
+            assert_close(new_p[n], ref_p[n], GRAD_RTOL, f"param {n} step {it}", floor=_grad_floor(ref_p[n]))
+        # the update clears every gradient it consumed (dense: whole tensor, lookup: touched rows)
+        for n, g in lm.get_grads().items():
+            assert not g.any(), n
+        # keep the two trajectories from drifting apart through rounding
+        for n in ref_p:
+            lm.p[n].set(ref_p[n])
+
+
+def test_lm_clipping_engages(dev):
+    V, E, H, L, B, T = 50, 16, 32, 2, 8, 5
+    rng = np.random.default_rng(5)
+    params = LstmLM.init_params(V, E, H, L, seed=1)
+    ref_p = {n: a.copy() for n, a in params.items()}
+    lm = LstmLM(dev, V, E, H, L, B, T, lr=0.1, clip=0.5, params=params)
+    tokens = _tokens(rng, V, B, T)
+    _, _, ref_scale = lm_oracle.step(ref_p, tokens, L, lr=0.1, clip=0.5)
+    lm.step(tokens)
+    assert ref_scale < 1.0
+    assert_close(lm.gscale.numpy()[0], ref_scale, GRAD_RTOL, "clip scale")
+    new_p = lm.get_params()
+    for n in ref_p:
+        assert_close(new_p[n], ref_p[n], GRAD_RTOL, f"param {n}", floor=_grad_floor(ref_p[n]))
+
+
+def test_lm_graph_replay_matches_eager(dev):
+    """The captured step, replayed with fresh tokens each time, follows the eager trajectory bit for bit."""
+    V, E, H, L, B, T = 120, 32, 64, 2, 16, 6
+    rng = np.random.default_rng(7)
+    params = LstmLM.init_params(V, E, H, L, seed=2)
+    eager = LstmLM(dev, V, E, H, L, B, T, params=params)
+    graphed = LstmLM(dev, V, E, H, L, B, T, params=params)
+    batches = [_tokens(rng, V, B, T) for _ in range(4)]
+    graphed.stage(batches[0])
+    graphed.capture()
+    for tok in batches:
+        le = eager.step(tok)
+        lg = graphed.step(tok)
+        dev.sync()
+        assert le == lg
+    pe, pg = eager.get_params(), graphed.get_params()
+    for n in pe:
+        np.testing.assert_array_equal(pe[n], pg[n], err_msg=n)
+    graphed.graph.destroy()

@@ -55,6 +55,19 @@ def test_gemm_is_fp32_accurate_against_fp64(dev):
     assert np.max(np.abs(yt.numpy() - want)) < 2e-6 * np.sqrt(K) * 10
 
 
+@pytest.mark.parametrize("M,N,K", [(1000, 128, 64), (10000, 96, 256), (37, 5, 20), (300, 192, 128), (4096, 4, 1024)])
+def test_affine_forward(dev, M, N, K):
+    """AffineTransform: bias broadcast + W x (direct and split-K routes of the GEMM)."""
+    rng = np.random.default_rng(M + N + K)
+    W, x, b = f32(rng.standard_normal((K, M))), f32(rng.standard_normal((N, K))), f32(rng.standard_normal(M))
+    want = np.ascontiguousarray(np.broadcast_to(b, (N, M))).copy()
+    orc.gemm_nn(M, N, K, W, x, 1.0, want)
+    fx = dev.empty((N, M))
+    dev.constant(fx, 7.0)  # forward overwrites
+    dev.affine_forward(M, N, K, dev.tensor(b), dev.tensor(W), dev.tensor(x), fx)
+    assert_close(fx.numpy(), want, FWD_RTOL, "affine", floor=np.sqrt(K))
+
+
 # ---------------------------------------------------------------------------
 # fused LSTM nodes
 # ---------------------------------------------------------------------------
@@ -427,6 +440,43 @@ def test_scale_copy_constant_accumulate_sgd_norm(dev):
     nrm = dev.empty(1)
     dev.squared_l2norm(n, gt, nrm)
     assert abs(float(nrm.numpy()[0]) - float((g.astype(np.float64) ** 2).sum())) < 1e-5 * n
+
+
+def test_device_side_clipping_and_sparse_rows(dev):
+    rng = np.random.default_rng(19)
+    vocab, dim, n = 500, 48, 700
+    ids = zipf_ids(rng, n, vocab)
+    table, grads = f32(rng.standard_normal((vocab, dim))), np.zeros((vocab, dim), F32)
+    used = np.unique(ids)
+    grads[used] = f32(rng.standard_normal((used.size, dim)))
+    g2 = f32(rng.standard_normal(1000))
+    plan = dev.lookup_build_plan(dev.tensor(ids, np.uint32), vocab)
+    sq = dev.zeros(2)
+    gt, tt, g2t = dev.tensor(grads), dev.tensor(table), dev.tensor(g2)
+    dev.squared_l2norm_rows(n, plan, dim, vocab, gt, sq)
+    dev.squared_l2norm(g2.size, g2t, sq.offset(1, (1,)))
+    want_sq = (grads.astype(np.float64) ** 2).sum()
+    assert abs(float(sq.numpy()[0]) - want_sq) < 1e-5 * want_sq
+    total = np.sqrt(want_sq + (g2.astype(np.float64) ** 2).sum())
+    scale = dev.empty(1)
+    for thr, want in ((5.0, 5.0 / total), (1e9, 1.0), (0.0, 1.0)):
+        dev.clip_scale(2, sq, thr, scale)
+        assert abs(float(scale.numpy()[0]) - want) < 1e-5 * want
+    dev.clip_scale(2, sq, 5.0, scale)
+    s = scale.numpy()[0]
+    dev.sgd_update_rows(n, plan, dim, vocab, tt, gt, 0.1, scale, 1.0)
+    want_t = table.copy()
+    for r in used:
+        orc.sgd_update(want_t[r], grads[r], 0.1, float(s), 1.0)
+    assert tt.numpy().tobytes() == want_t.tobytes()
+    assert not gt.numpy().any()
+    p = f32(rng.standard_normal(1000))
+    pt = dev.tensor(p)
+    dev.sgd_update_scaled(1000, pt, g2t, 0.1, scale, 1.0, clear_grad=False)
+    assert pt.numpy().tobytes() == orc.sgd_update(p.copy(), g2, 0.1, float(s), 1.0).tobytes()
+    assert g2t.numpy().tobytes() == g2.tobytes()
+    dev.sgd_update_scaled(1000, pt, g2t, 0.1, scale, 1.0, clear_grad=True)
+    assert not g2t.numpy().any()
 
 
 def test_device_scalars_and_pools(dev):

@@ -608,3 +608,44 @@ def test_scale_copy_sgd_and_norm():
     want = p - g * F32(F32(0.1) * F32(0.5) / F32(1.0))
     assert np.array_equal(orc.sgd_update(p.copy(), g, 0.1, 0.5, 1.0), want)
     assert abs(orc.squared_l2norm(g) - (g.astype(np.float64) ** 2).sum()) < 1e-4
+
+
+# ---- LM step composition -------------------------------------------------------
+def test_lm_step_gradient_check():
+    """Directional central difference of the LM loss against <grad, direction>: a dropped term, a wrong
+    transpose or a mis-indexed timestep in the backward composition breaks it."""
+    from oracle import lm_oracle
+    from dynet_amd.lm import LstmLM
+    V, E, H, L, B, T = 23, 6, 8, 2, 3, 4
+    rng = np.random.default_rng(0)
+    p = LstmLM.init_params(V, E, H, L, seed=4)
+    for l in range(L):
+        p[f"b{l}"] = rng.normal(0, 0.1, 4 * H).astype(np.float32)
+    tokens = rng.integers(0, V, (T + 1, B)).astype(np.uint32)
+    loss, cache = lm_oracle.forward(p, tokens, L)
+    g = lm_oracle.backward(p, tokens, L, cache)
+    for name in p:
+        d = rng.normal(0, 1, p[name].shape).astype(np.float32)
+        eps = 2e-2
+        plus = {n: (a + eps * d if n == name else a).astype(np.float32) for n, a in p.items()}
+        minus = {n: (a - eps * d if n == name else a).astype(np.float32) for n, a in p.items()}
+        lp, _ = lm_oracle.forward(plus, tokens, L)
+        lmn, _ = lm_oracle.forward(minus, tokens, L)
+        fd = (float(lp) - float(lmn)) / (2 * eps)
+        an = float(np.sum(g[name].astype(np.float64) * d))
+        assert abs(fd - an) <= 2e-2 * max(abs(an), 0.5), (name, fd, an)
+
+
+def test_lm_update_clips_and_touches_only_used_rows():
+    from oracle import lm_oracle
+    from dynet_amd.lm import LstmLM
+    V, E, H, L, B, T = 23, 6, 8, 1, 3, 4
+    rng = np.random.default_rng(1)
+    p = LstmLM.init_params(V, E, H, L, seed=4)
+    before = {n: a.copy() for n, a in p.items()}
+    tokens = rng.integers(0, 5, (T + 1, B)).astype(np.uint32)
+    loss, g, gscale = lm_oracle.step(p, tokens, L, lr=0.1, clip=0.25)
+    norm = np.sqrt(sum(float(np.sum(a.astype(np.float64) ** 2)) for a in g.values()))
+    assert norm > 0.25 and abs(gscale - 0.25 / norm) < 1e-5 * gscale
+    assert np.array_equal(p["C"][5:], before["C"][5:])
+    np.testing.assert_allclose(p["R"], before["R"] - 0.1 * gscale * g["R"], rtol=1e-6, atol=1e-7)
