@@ -1,5 +1,5 @@
 // Internal interface of the fp32 MFMA GEMM (gemm.hip), shared with the fused
-// LSTM gate launcher.
+// LSTM launchers.
 #pragma once
 
 #include "common.h"
@@ -24,15 +24,20 @@ constexpr int kGemmMaxSeg = 2;
 enum GemmEpilogue {
   kEpiAxpby = 0,      // C = beta*C + sum
   kEpiLstmGates = 1,  // C = act(bias[i] + (H <= i < 2H ? 1 : 0) + sum), logistic rows [0,3H), tanh rows [3H,4H)
-  kEpiBias = 2        // C = bias[i] + sum   (AffineTransform: bias broadcast over the columns)
+  kEpiBias = 2,       // C = bias[i] + sum   (AffineTransform: bias broadcast over the columns)
+  kEpiPartials = 3    // no epilogue: the split-K slices stay in the caller's buffer, summed by the consumer
 };
 
 struct GemmEpiParams {
   int kind;
   float beta;
-  const float* bias;  // kEpiLstmGates
+  const float* bias;  // kEpiLstmGates, kEpiBias
   unsigned H;         // kEpiLstmGates
   int logistic_mode;  // kEpiLstmGates
+  // kEpiPartials: slices of M*N floats each are written here; *splits_out receives their number
+  float* partials;
+  size_t partials_bytes;
+  unsigned* splits_out;
 };
 
 // C is M x N column-major (ldc = M).  Segments share the operand layouts.

@@ -3,238 +3,266 @@
 // GEMM shim needs (dynet/matrix-multiply.h:16-37,97-117,162-180), replacing its
 // cublasSgemm calls.
 //
-// Tiling: a 256-thread block (4 wavefronts) owns a 128 x (32*TN) tile of C.
-// Wavefront w owns rows [32w, 32w+32) and TN accumulators of 32x32 (16 VGPRs
-// each).  K advances in steps of 16 through a double-buffered LDS stage: while
-// the matrix cores work on stage s, the global loads of stage s+1 are already
-// in flight in registers.  Operand tiles are kept in LDS in whichever of two
-// layouts makes both the 128-bit global load and the per-lane MFMA operand read
-// conflict-free:
-//   "MN-major" operand (contiguous along the C row/column index):  lds[k][mn]
-//   "K-major"  operand (contiguous along K, i.e. a transposed one): lds[mn][k], pitch 17
-// MFMA 32x32x2 operand mapping: lane l supplies A(i = l%32, k = l/32) and
-// B(k = l/32, j = l%32); accumulator register r of lane l is
-// C(i = 8*(r/4) + 4*(l/32) + r%4, j = l%32).
+// Tiling.  A 256-thread block (4 wavefronts, 2 x 2) owns a 128 x (64*WN) tile of
+// C; each wavefront owns 64 x (32*WN) of it as 2 x WN accumulators of 32x32.  K
+// advances in steps of 32 through a double-buffered LDS stage.  Both operand
+// tiles sit in LDS as lds[k][mn], whatever their orientation in memory, so one
+// lane fetches the operand values of two (WN) neighbouring rows with a single
+// 64-bit LDS read: the rows of a wave's tile are interleaved over its MFMA
+// blocks (tile row 2*i + b belongs to block b), which is only a relabelling of
+// the output rows.  The row pitch is W+4 floats for an operand stored along mn
+// (128-bit LDS writes) and W+2 for one stored along k (transposing 32-bit writes
+// land on 32 distinct banks).
 //
-// Skinny problems (the LSTM gate GEMMs have N = batch) do not have enough
-// tiles to fill 256 CUs, so K is split across blocks; each split writes its
-// partial tile to a device-owned workspace and a second kernel adds the splits
-// in ascending order (deterministic, no atomics) and applies the epilogue:
-// either C = beta*C + sum, or the fused LSTM gate epilogue (bias, +1 forget
-// bias, logistic / tanh).
+// The MFMA "row" index is fed from B and the "column" index (lane % 32) from A,
+// so a lane ends up holding two consecutive rows m of C for each of its columns
+// and a wavefront stores 256 contiguous bytes per column.
+//
+// Schedule per K-tile: issue the global loads of the next tile, run the 16 MFMA
+// steps with the LDS reads of step s+1 in flight under the MFMAs of step s
+// (pinned with scheduling barriers: left alone the compiler waits for every read
+// right before its use), park the next tile in the other LDS buffer three
+// quarters of the way through, barrier.  Two blocks per CU (LDS-limited) cover
+// each other's barrier bubbles; more resident wavefronts per SIMD lower the
+// matrix-core issue rate, fewer expose the bubbles.
+//
+// Tile count rarely divides the 256 CUs, and skinny problems (the LSTM gate
+// GEMMs have N = batch) have far too few tiles, so K is split across blocks when
+// the estimate says it pays: each split writes its partial tile to a workspace
+// and a second kernel adds the splits in ascending order (deterministic, no
+// atomics) and applies the epilogue: C = beta*C + sum, + bias, or the fused LSTM
+// gate epilogue.  The fused LSTM cell kernels consume the unreduced slices.
 #include "gemm.h"
 
 namespace dyhip {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float fvec2 __attribute__((ext_vector_type(2)));
 
 constexpr int kBM = 128;
-constexpr int kBK = 16;
+constexpr int kBK = 32;
 constexpr int kGemmThreads = 256;
-constexpr int kKPitch = kBK + 1;  // row pitch of the K-major LDS layout
+constexpr int kWritePos = (kBK / 2) * 3 / 4;  // MFMA step after which the next tile goes to LDS
 
 struct GemmArgs {
   GemmSeg seg[kGemmMaxSeg];
   int nseg;
-  unsigned ktiles[kGemmMaxSeg];  // k-tiles per segment
+  unsigned ktiles0;  // k-tiles of segment 0
   unsigned ktiles_total;
   unsigned ktiles_per_split;
   size_t M, N;
-  float* C;         // used when partial == nullptr
-  float beta;       // used when partial == nullptr
+  float* C;           // used when partial == nullptr
+  float beta;         // used when partial == nullptr
   const float* bias;  // when set (and partial == nullptr): C = bias[i] + sum
-  float* partial;   // [splits][M*N] or nullptr
+  float* partial;     // [splits][M*N] or nullptr
+  int vec_ok;         // every operand 16-byte aligned with a leading dimension that is a multiple of 4
 };
 
 // ---- global -> register tile loads ------------------------------------------------
-// A tile is W (mn extent) x 16 (k extent) floats = W*4 float4.  Thread t loads
-// float4 number f = t + 256*u.
+// An operand tile is W (mn extent) x 32 (k extent) floats; thread t loads float4 number t + 256*u.
 template <int W>
 struct TileRegs {
-  static constexpr int NV = (W * 4 + kGemmThreads - 1) / kGemmThreads;
+  static constexpr int NV = (W * kBK / 4) / kGemmThreads;
   float4 v[NV];
 };
 
-template <bool KMAJOR, int W>
+// EDGE == false: the whole tile lies inside the matrix and is 16-byte aligned.
+// EDGE == true : branch-free clamped scalar loads, zeros outside the matrix.
+template <bool KMAJOR, int W, bool EDGE>
 __device__ __forceinline__ void load_tile(TileRegs<W>& r, const float* __restrict__ p, size_t ld, size_t mn0,
-                                          size_t k0, size_t MN, size_t K, bool vec_ok) {
+                                          size_t k0, size_t MN, size_t K) {
 #pragma unroll
   for (int u = 0; u < TileRegs<W>::NV; ++u) {
     const int f = threadIdx.x + kGemmThreads * u;
-    float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (f < W * 4) {
-      if (!KMAJOR) {
-        // float4 along mn at fixed k: W/4 float4 per k row
-        const int k = f / (W / 4), m4 = f % (W / 4);
-        const size_t mn = mn0 + size_t(m4) * 4, kk = k0 + k;
-        if (kk < K && mn < MN) {
-          const float* q = p + mn + kk * ld;
-          if (vec_ok && mn + 3 < MN) {
-            val = *reinterpret_cast<const float4*>(q);
-          } else {
-            val.x = q[0];
-            if (mn + 1 < MN) val.y = q[1];
-            if (mn + 2 < MN) val.z = q[2];
-            if (mn + 3 < MN) val.w = q[3];
-          }
-        }
-      } else {
-        // float4 along k at fixed mn: 4 float4 per mn row
-        const int mn_l = f / 4, k4 = f % 4;
-        const size_t mn = mn0 + mn_l, kk = k0 + size_t(k4) * 4;
-        if (mn < MN && kk < K) {
-          const float* q = p + kk + mn * ld;
-          if (vec_ok && kk + 3 < K) {
-            val = *reinterpret_cast<const float4*>(q);
-          } else {
-            val.x = q[0];
-            if (kk + 1 < K) val.y = q[1];
-            if (kk + 2 < K) val.z = q[2];
-            if (kk + 3 < K) val.w = q[3];
-          }
-        }
-      }
+    size_t mn, kk;
+    if (!KMAJOR) {
+      mn = mn0 + size_t(f % (W / 4)) * 4;
+      kk = k0 + f / (W / 4);
+    } else {
+      mn = mn0 + f / (kBK / 4);
+      kk = k0 + size_t(f % (kBK / 4)) * 4;
     }
-    r.v[u] = val;
+    if (!EDGE) {
+      r.v[u] = *reinterpret_cast<const float4*>(KMAJOR ? p + kk + mn * ld : p + mn + kk * ld);
+    } else {
+      float e[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const size_t mi = KMAJOR ? mn : mn + c, ki = KMAJOR ? kk + c : kk;
+        const bool ok = mi < MN && ki < K;
+        const size_t mc = mi < MN ? mi : MN - 1, kc = ki < K ? ki : K - 1;
+        const float x = KMAJOR ? p[kc + mc * ld] : p[mc + kc * ld];
+        e[c] = ok ? x : 0.f;
+      }
+      r.v[u] = make_float4(e[0], e[1], e[2], e[3]);
+    }
   }
+}
+
+template <bool KMAJOR, int W>
+constexpr int lds_pitch() {
+  return KMAJOR ? W + 2 : W + 4;
 }
 
 template <bool KMAJOR, int W>
 __device__ __forceinline__ void store_tile(const TileRegs<W>& r, float* __restrict__ lds) {
+  constexpr int P = lds_pitch<KMAJOR, W>();
 #pragma unroll
   for (int u = 0; u < TileRegs<W>::NV; ++u) {
     const int f = threadIdx.x + kGemmThreads * u;
-    if (f < W * 4) {
-      if (!KMAJOR) {
-        const int k = f / (W / 4), m4 = f % (W / 4);
-        *reinterpret_cast<float4*>(lds + k * W + m4 * 4) = r.v[u];
-      } else {
-        const int mn_l = f / 4, k4 = f % 4;
-        float* q = lds + mn_l * kKPitch + k4 * 4;
-        q[0] = r.v[u].x;
-        q[1] = r.v[u].y;
-        q[2] = r.v[u].z;
-        q[3] = r.v[u].w;
-      }
+    if (!KMAJOR) {
+      const int k = f / (W / 4), m4 = f % (W / 4);
+      *reinterpret_cast<float4*>(lds + k * P + m4 * 4) = r.v[u];
+    } else {
+      const int k4 = f % (kBK / 4), mn_l = f / (kBK / 4);
+      float* q = lds + (k4 * 4) * P + mn_l;
+      q[0] = r.v[u].x;
+      q[P] = r.v[u].y;
+      q[2 * P] = r.v[u].z;
+      q[3 * P] = r.v[u].w;
     }
   }
 }
 
-template <bool KMAJOR, int W>
-__device__ __forceinline__ float lds_operand(const float* __restrict__ lds, int mn, int k) {
-  return KMAJOR ? lds[mn * kKPitch + k] : lds[k * W + mn];
+template <int V>
+__device__ __forceinline__ void lds_read(const float* p, float (&out)[V]) {
+  if constexpr (V == 1) {
+    out[0] = *p;
+  } else {
+    const fvec2 t = *reinterpret_cast<const fvec2*>(p);
+    out[0] = t[0];
+    out[1] = t[1];
+  }
 }
 
-template <bool KMAJOR, int W>
-constexpr int tile_floats() {
-  return KMAJOR ? W * kKPitch : W * kBK;
+// k-tile kt of the (up to two) concatenated K segments -> its segment and offset
+__device__ __forceinline__ void locate_ktile(const GemmArgs& g, unsigned kt, GemmSeg& sg, size_t& k0) {
+  if (g.nseg > 1 && kt >= g.ktiles0) {
+    sg = g.seg[1];
+    k0 = size_t(kt - g.ktiles0) * kBK;
+  } else {
+    sg = g.seg[0];
+    k0 = size_t(kt) * kBK;
+  }
 }
 
-template <bool A_KMAJOR, bool B_KMAJOR, int TN>
-__global__ __launch_bounds__(kGemmThreads) void gemm_tile_kernel(GemmArgs g, unsigned tiles_m, int a_vec, int b_vec) {
-  constexpr int BN = 32 * TN;
-  constexpr int A_FLOATS = tile_floats<A_KMAJOR, kBM>();
-  constexpr int B_FLOATS = tile_floats<B_KMAJOR, BN>();
-  __shared__ __attribute__((aligned(16))) float lds_a[2][A_FLOATS];
-  __shared__ __attribute__((aligned(16))) float lds_b[2][B_FLOATS];
+template <bool A_KMAJOR, bool B_KMAJOR, int WN>
+__device__ __forceinline__ void load_pair(const GemmArgs& g, unsigned kt, bool interior, size_t m0, size_t n0,
+                                          TileRegs<kBM>& ra, TileRegs<64 * WN>& rb) {
+  constexpr int BN = 64 * WN;
+  GemmSeg sg;
+  size_t k0;
+  locate_ktile(g, kt, sg, k0);
+  if (interior && k0 + kBK <= sg.K) {
+    load_tile<A_KMAJOR, kBM, false>(ra, sg.A, sg.lda, m0, k0, g.M, sg.K);
+    load_tile<B_KMAJOR, BN, false>(rb, sg.B, sg.ldb, n0, k0, g.N, sg.K);
+  } else {
+    load_tile<A_KMAJOR, kBM, true>(ra, sg.A, sg.lda, m0, k0, g.M, sg.K);
+    load_tile<B_KMAJOR, BN, true>(rb, sg.B, sg.ldb, n0, k0, g.N, sg.K);
+  }
+}
+
+template <bool A_KMAJOR, bool B_KMAJOR, int WN>
+__global__ __launch_bounds__(kGemmThreads, 2) void gemm_tile_kernel(GemmArgs g, unsigned tiles_m) {
+  constexpr int BN = 64 * WN;
+  constexpr int PA = lds_pitch<A_KMAJOR, kBM>(), PB = lds_pitch<B_KMAJOR, BN>();
+  __shared__ __attribute__((aligned(16))) float lds_a[2][kBK * PA];
+  __shared__ __attribute__((aligned(16))) float lds_b[2][kBK * PB];
 
   const unsigned tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m;
   const unsigned split = blockIdx.y;
   const size_t m0 = size_t(tm) * kBM, n0 = size_t(tn) * BN;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int wm = w & 1, wn = w >> 1;
   const int l32 = lane & 31, lhi = lane >> 5;
 
-  floatx16 acc[TN];
+  floatx16 acc[WN][2];
 #pragma unroll
-  for (int t = 0; t < TN; ++t)
+  for (int a = 0; a < WN; ++a)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
   const unsigned kt_begin = split * g.ktiles_per_split;
   const unsigned kt_end = min(g.ktiles_total, kt_begin + g.ktiles_per_split);
+  const bool interior = g.vec_ok && (m0 + kBM <= g.M) && (n0 + BN <= g.N);
 
-  unsigned seg_first = 0;
-  for (int s = 0; s < g.nseg; ++s) {
-    const unsigned seg_last = seg_first + g.ktiles[s];
-    const unsigned lo = max(kt_begin, seg_first), hi = min(kt_end, seg_last);
-    if (lo < hi) {
-      const GemmSeg sg = g.seg[s];
-      const unsigned nt = hi - lo;
-      TileRegs<kBM> ra;
-      TileRegs<BN> rb;
-      size_t k0 = size_t(lo - seg_first) * kBK;
-      load_tile<A_KMAJOR, kBM>(ra, sg.A, sg.lda, m0, k0, g.M, sg.K, a_vec);
-      load_tile<B_KMAJOR, BN>(rb, sg.B, sg.ldb, n0, k0, g.N, sg.K, b_vec);
-      __syncthreads();  // previous segment's readers are done with buffer 0
-      store_tile<A_KMAJOR, kBM>(ra, lds_a[0]);
-      store_tile<B_KMAJOR, BN>(rb, lds_b[0]);
-      __syncthreads();
-      for (unsigned t = 0; t < nt; ++t) {
-        const int buf = t & 1;
-        if (t + 1 < nt) {
-          k0 += kBK;
-          load_tile<A_KMAJOR, kBM>(ra, sg.A, sg.lda, m0, k0, g.M, sg.K, a_vec);
-          load_tile<B_KMAJOR, BN>(rb, sg.B, sg.ldb, n0, k0, g.N, sg.K, b_vec);
-        }
-        const float* la = lds_a[buf];
-        const float* lb = lds_b[buf];
+  if (kt_begin < kt_end) {
+    TileRegs<kBM> ra;
+    TileRegs<BN> rb;
+    load_pair<A_KMAJOR, B_KMAJOR, WN>(g, kt_begin, interior, m0, n0, ra, rb);
+    store_tile<A_KMAJOR, kBM>(ra, lds_a[0]);
+    store_tile<B_KMAJOR, BN>(rb, lds_b[0]);
+    __syncthreads();
+    for (unsigned kt = kt_begin; kt < kt_end; ++kt) {
+      const int buf = (kt - kt_begin) & 1;
+      const bool more = kt + 1 < kt_end;
+      if (more) load_pair<A_KMAJOR, B_KMAJOR, WN>(g, kt + 1, interior, m0, n0, ra, rb);
+      const float* la = lds_a[buf] + wm * 64 + 2 * l32 + lhi * PA;
+      const float* lb = lds_b[buf] + wn * 32 * WN + WN * l32 + lhi * PB;
+      float av[2][2], bv[2][WN];
+      lds_read<2>(la, av[0]);
+      lds_read<WN>(lb, bv[0]);
 #pragma unroll
-        for (int kk = 0; kk < kBK; kk += 2) {
-          const float a = lds_operand<A_KMAJOR, kBM>(la, 32 * w + l32, kk + lhi);
-#pragma unroll
-          for (int t2 = 0; t2 < TN; ++t2) {
-            const float b = lds_operand<B_KMAJOR, BN>(lb, 32 * t2 + l32, kk + lhi);
-            acc[t2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[t2], 0, 0, 0);
-          }
+      for (int s = 0; s < kBK / 2; ++s) {
+        const int cur = s & 1;
+        if (s + 1 < kBK / 2) {
+          lds_read<2>(la + (2 * s + 2) * PA, av[cur ^ 1]);
+          lds_read<WN>(lb + (2 * s + 2) * PB, bv[cur ^ 1]);
         }
-        if (t + 1 < nt) {
-          // buffer buf^1 was last read in iteration t-1, which every wave has left
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int a = 0; a < WN; ++a)
+#pragma unroll
+          for (int b = 0; b < 2; ++b)
+            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[cur][a], av[cur][b], acc[a][b], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (s == kWritePos && more) {
+          // the other buffer was last read in the previous iteration, which every wave has left
           store_tile<A_KMAJOR, kBM>(ra, lds_a[buf ^ 1]);
           store_tile<B_KMAJOR, BN>(rb, lds_b[buf ^ 1]);
+          __builtin_amdgcn_sched_barrier(0);
         }
-        __syncthreads();
       }
+      __syncthreads();
     }
-    seg_first = seg_last;
   }
 
-  // ---- write back --------------------------------------------------------------
+  // ---- write back ----------------------------------------------------------------
+  // acc[a][b][r] of lane l: row m = m0 + 64*wm + 2*(l%32) + b,
+  //                         column n = n0 + 32*WN*wn + WN*i + a with i = 8*(r/4) + 4*(l/32) + r%4
   float* out = g.partial ? g.partial + size_t(split) * g.M * g.N : g.C;
   const bool direct = g.partial == nullptr;
-  const bool vec_store = (g.M % 4 == 0) && aligned16(out);
+  const size_t m = m0 + wm * 64 + 2 * l32;
+  if (m >= g.M) return;
+  const bool pair = (m + 1 < g.M) && (g.M % 2 == 0) && ((reinterpret_cast<uintptr_t>(out) & 7u) == 0);
+  float bias0 = 0.f, bias1 = 0.f;
+  if (direct && g.bias != nullptr) {
+    bias0 = g.bias[m];
+    if (m + 1 < g.M) bias1 = g.bias[m + 1];
+  }
 #pragma unroll
-  for (int t2 = 0; t2 < TN; ++t2) {
-    const size_t j = n0 + 32 * t2 + l32;
-    if (j >= g.N) continue;
+  for (int a = 0; a < WN; ++a)
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const size_t i = m0 + 32 * w + 8 * q + 4 * lhi;
-      if (i >= g.M) continue;
-      float* p = out + i + j * g.M;
-      float4 v = make_float4(acc[t2][4 * q], acc[t2][4 * q + 1], acc[t2][4 * q + 2], acc[t2][4 * q + 3]);
-      if (direct && g.bias != nullptr) {
-        v.x += g.bias[i];
-        if (i + 1 < g.M) v.y += g.bias[i + 1];
-        if (i + 2 < g.M) v.z += g.bias[i + 2];
-        if (i + 3 < g.M) v.w += g.bias[i + 3];
-      }
-      if (vec_store && i + 3 < g.M) {
+    for (int r = 0; r < 16; ++r) {
+      const int i = 8 * (r / 4) + 4 * lhi + (r % 4);
+      const size_t n = n0 + wn * 32 * WN + WN * i + a;
+      if (n >= g.N) continue;
+      float* p = out + m + n * g.M;
+      float v0 = acc[a][0][r] + bias0, v1 = acc[a][1][r] + bias1;
+      if (pair) {
         if (direct && g.beta != 0.f) {
-          const float4 o = *reinterpret_cast<const float4*>(p);
-          v.x = g.beta * o.x + v.x;
-          v.y = g.beta * o.y + v.y;
-          v.z = g.beta * o.z + v.z;
-          v.w = g.beta * o.w + v.w;
+          const fvec2 o = *reinterpret_cast<const fvec2*>(p);
+          v0 = g.beta * o[0] + v0;
+          v1 = g.beta * o[1] + v1;
         }
-        *reinterpret_cast<float4*>(p) = v;
+        *reinterpret_cast<fvec2*>(p) = fvec2{v0, v1};
       } else {
-        const float vv[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-        for (int c = 0; c < 4; ++c)
-          if (i + c < g.M) p[c] = (direct && g.beta != 0.f) ? g.beta * p[c] + vv[c] : vv[c];
+        p[0] = (direct && g.beta != 0.f) ? g.beta * p[0] + v0 : v0;
+        if (m + 1 < g.M) p[1] = (direct && g.beta != 0.f) ? g.beta * p[1] + v1 : v1;
       }
     }
-  }
 }
 
 // C[e] = epilogue(sum_s partial[s][e]), splits added in ascending order
@@ -263,71 +291,107 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(size_t M, size_
 
 template <bool A_KMAJOR, bool B_KMAJOR>
 static void launch_tiles(dyhip_device* dev, const GemmArgs& g, unsigned tiles_m, unsigned tiles_n, unsigned splits,
-                         int tn, int a_vec, int b_vec) {
+                         int wn) {
   const dim3 grid(tiles_m * tiles_n, splits), block(kGemmThreads);
-  if (tn == 1)
-    hipLaunchKernelGGL((gemm_tile_kernel<A_KMAJOR, B_KMAJOR, 1>), grid, block, 0, dev->stream, g, tiles_m, a_vec, b_vec);
-  else if (tn == 2)
-    hipLaunchKernelGGL((gemm_tile_kernel<A_KMAJOR, B_KMAJOR, 2>), grid, block, 0, dev->stream, g, tiles_m, a_vec, b_vec);
+  if (wn == 1)
+    hipLaunchKernelGGL((gemm_tile_kernel<A_KMAJOR, B_KMAJOR, 1>), grid, block, 0, dev->stream, g, tiles_m);
   else
-    hipLaunchKernelGGL((gemm_tile_kernel<A_KMAJOR, B_KMAJOR, 4>), grid, block, 0, dev->stream, g, tiles_m, a_vec, b_vec);
+    hipLaunchKernelGGL((gemm_tile_kernel<A_KMAJOR, B_KMAJOR, 2>), grid, block, 0, dev->stream, g, tiles_m);
+}
+
+// Tile width and split count by a small cost model.  Measured on MI355X: the matrix cores
+// sustain ~2.0 GHz under this kernel (131 TFLOP/s over 256 CUs); a CU running two blocks
+// keeps them ~95 % busy, a lone block ~77 %; the 64-wide tile reads more LDS per MFMA.
+struct GemmPlan {
+  int wn;
+  unsigned splits;
+};
+
+static GemmPlan plan_gemm(const dyhip_device* dev, size_t M, size_t N, unsigned ktiles, size_t max_splits_ws,
+                          bool must_use_partials) {
+  const double cus = dev->num_cus > 0 ? dev->num_cus : 256;
+  const double peak = cus * 256.0 * 2.0e9, ws_bw = 3.0e12;
+  const double flops = 2.0 * double(M) * double(N) * double(ktiles) * kBK;
+  GemmPlan best{2, 1};
+  double best_t = 1e30;
+  for (int wn = 2; wn >= 1; --wn) {
+    if (wn == 2 && N <= 64) continue;
+    const double tiles = double(cdiv<size_t>(M, kBM)) * double(cdiv<size_t>(N, size_t(64) * wn));
+    for (unsigned s = 1; s <= 32; ++s) {
+      if (s > 1 && (ktiles / s < 2 || s > max_splits_ws)) break;
+      const double blocks = tiles * s;
+      const double rounds = blocks <= cus ? 1.0 : double(cdiv<size_t>(size_t(blocks), size_t(cus)));
+      const double eff = blocks / (rounds * cus);
+      double inloop = blocks >= 2 * cus ? 0.95 : (blocks > cus ? 0.85 : 0.77);
+      if (wn == 1) inloop *= 0.9;
+      double t = flops / (peak * eff * inloop) + rounds * 1.0e-6;
+      if (s > 1 || must_use_partials) t += 2.0 * double(M) * double(N) * 4.0 * s / ws_bw + 2.0e-6;
+      if (t < best_t) {
+        best_t = t;
+        best = GemmPlan{wn, s};
+      }
+    }
+  }
+  return best;
 }
 
 int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N, int nseg, const GemmSeg* segs,
              float* C, const GemmEpiParams& epi) {
+  const bool to_caller = epi.kind == kEpiPartials;
+  if (to_caller) {
+    DYHIP_REQUIRE(epi.partials != nullptr && epi.splits_out != nullptr, "null split-K output");
+    *epi.splits_out = 0;
+  }
   if (M == 0 || N == 0) return DYHIP_OK;
   DYHIP_REQUIRE(nseg >= 1 && nseg <= kGemmMaxSeg, "GEMM supports 1..%d K segments", kGemmMaxSeg);
-  DYHIP_REQUIRE(C != nullptr, "null GEMM output");
+  DYHIP_REQUIRE(to_caller || C != nullptr, "null GEMM output");
   GemmArgs g;
   g.nseg = nseg;
   g.M = M;
   g.N = N;
   g.C = C;
-  g.beta = epi.kind == kEpiBias ? 0.f : epi.beta;
+  g.beta = epi.kind == kEpiAxpby ? epi.beta : 0.f;
   g.bias = epi.kind == kEpiBias ? epi.bias : nullptr;
   g.ktiles_total = 0;
-  bool a_vec = true, b_vec = true;
+  g.ktiles0 = 0;
+  g.seg[1] = GemmSeg{nullptr, 0, nullptr, 0, 0};
+  bool vec = true;
   for (int s = 0; s < nseg; ++s) {
     DYHIP_REQUIRE(segs[s].A != nullptr && segs[s].B != nullptr, "null GEMM operand");
     g.seg[s] = segs[s];
-    g.ktiles[s] = static_cast<unsigned>(cdiv<size_t>(segs[s].K, kBK));
-    g.ktiles_total += g.ktiles[s];
-    a_vec = a_vec && aligned16(segs[s].A) && segs[s].lda % 4 == 0;
-    b_vec = b_vec && aligned16(segs[s].B) && segs[s].ldb % 4 == 0;
+    const unsigned kt = static_cast<unsigned>(cdiv<size_t>(segs[s].K, kBK));
+    if (s == 0) g.ktiles0 = kt;
+    g.ktiles_total += kt;
+    vec = vec && aligned16(segs[s].A) && segs[s].lda % 4 == 0 && aligned16(segs[s].B) && segs[s].ldb % 4 == 0;
   }
-  const int tn = N <= 32 ? 1 : (N <= 64 ? 2 : 4);
-  const size_t tiles_m = cdiv<size_t>(M, kBM), tiles_n = cdiv<size_t>(N, size_t(32) * tn);
-  DYHIP_REQUIRE(tiles_m * tiles_n < (size_t(1) << 31), "GEMM too large");
-  const size_t tiles = tiles_m * tiles_n;
+  g.vec_ok = vec ? 1 : 0;
   const size_t out_bytes = M * N * sizeof(float);
-  // split K only when the tiles alone cannot fill the device
-  unsigned splits = 1;
-  if (g.ktiles_total == 0) {
-    splits = 1;
-  } else if (tiles < size_t(dev->num_cus)) {
-    size_t want = cdiv<size_t>(size_t(2) * dev->num_cus, tiles);
-    const size_t by_k = g.ktiles_total >= 8 ? g.ktiles_total / 4 : 1;
-    const size_t by_ws = dev->gemm_ws_bytes / out_bytes;
-    if (want > by_k) want = by_k;
-    if (want > by_ws) want = by_ws;
-    if (want > 65535) want = 65535;
-    splits = want < 1 ? 1u : static_cast<unsigned>(want);
-  }
+  const size_t ws_bytes = to_caller ? epi.partials_bytes : dev->gemm_ws_bytes;
+  void* ws = to_caller ? static_cast<void*>(epi.partials) : dev->gemm_ws;
   const bool fused_epi = epi.kind == kEpiLstmGates;  // needs the whole sum before the activation
-  const bool use_partial = splits > 1 || fused_epi;
-  if (use_partial)
-    DYHIP_REQUIRE(dev->gemm_ws_bytes >= out_bytes * splits,
-                  "GEMM output of %zu bytes does not fit the %zu-byte split-K workspace", out_bytes,
-                  dev->gemm_ws_bytes);
+  const bool must_partial = fused_epi || to_caller;
+  GemmPlan plan{N <= 64 ? 1 : 2, 1};
+  if (g.ktiles_total > 0) plan = plan_gemm(dev, M, N, g.ktiles_total, ws_bytes / out_bytes, must_partial);
+  unsigned splits = plan.splits;
+  const size_t tiles_m = cdiv<size_t>(M, kBM), tiles_n = cdiv<size_t>(N, size_t(64) * plan.wn);
+  DYHIP_REQUIRE(tiles_m * tiles_n < (size_t(1) << 31), "GEMM too large");
   g.ktiles_per_split = g.ktiles_total == 0 ? 1 : cdiv<unsigned>(g.ktiles_total, splits);
   splits = g.ktiles_total == 0 ? 1 : cdiv<unsigned>(g.ktiles_total, g.ktiles_per_split);
-  g.partial = use_partial ? static_cast<float*>(dev->gemm_ws) : nullptr;
-  const int av = a_vec ? 1 : 0, bv = b_vec ? 1 : 0;
-  if (a_kmajor && b_kmajor) launch_tiles<true, true>(dev, g, (unsigned)tiles_m, (unsigned)tiles_n, splits, tn, av, bv);
-  else if (a_kmajor && !b_kmajor) launch_tiles<true, false>(dev, g, (unsigned)tiles_m, (unsigned)tiles_n, splits, tn, av, bv);
-  else if (!a_kmajor && b_kmajor) launch_tiles<false, true>(dev, g, (unsigned)tiles_m, (unsigned)tiles_n, splits, tn, av, bv);
-  else launch_tiles<false, false>(dev, g, (unsigned)tiles_m, (unsigned)tiles_n, splits, tn, av, bv);
+  const bool use_partial = splits > 1 || must_partial;
+  if (use_partial)
+    DYHIP_REQUIRE(ws != nullptr && ws_bytes >= out_bytes * splits,
+                  "GEMM output of %zu bytes x %u splits does not fit the %zu-byte split-K workspace", out_bytes,
+                  splits, ws_bytes);
+  g.partial = use_partial ? static_cast<float*>(ws) : nullptr;
+  if (a_kmajor && b_kmajor) launch_tiles<true, true>(dev, g, (unsigned)tiles_m, (unsigned)tiles_n, splits, plan.wn);
+  else if (a_kmajor && !b_kmajor) launch_tiles<true, false>(dev, g, (unsigned)tiles_m, (unsigned)tiles_n, splits, plan.wn);
+  else if (!a_kmajor && b_kmajor) launch_tiles<false, true>(dev, g, (unsigned)tiles_m, (unsigned)tiles_n, splits, plan.wn);
+  else launch_tiles<false, false>(dev, g, (unsigned)tiles_m, (unsigned)tiles_n, splits, plan.wn);
   DYHIP_CHECK_LAUNCH();
+  if (to_caller) {
+    *epi.splits_out = splits;
+    return DYHIP_OK;
+  }
   if (use_partial) {
     const size_t total = M * N;
     const dim3 grid((unsigned)cdiv<size_t>(total, 256));
@@ -345,6 +409,13 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
   return DYHIP_OK;
 }
 
+static GemmEpiParams axpby(float beta) {
+  GemmEpiParams ep{};
+  ep.kind = kEpiAxpby;
+  ep.beta = beta;
+  return ep;
+}
+
 }  // namespace dyhip
 
 using namespace dyhip;
@@ -355,8 +426,7 @@ int dyhip_gemm_nn(dyhip_device* dev, size_t M, size_t N, size_t K, const float* 
                   float* y) {
   DYHIP_CHECK_DEV(dev);
   GemmSeg s{l, M, r, K, K};
-  GemmEpiParams ep{kEpiAxpby, beta, nullptr, 0, 0};
-  return gemm_run(dev, false, true, M, N, 1, &s, y, ep);
+  return gemm_run(dev, false, true, M, N, 1, &s, y, axpby(beta));
 }
 
 int dyhip_affine_forward(dyhip_device* dev, size_t M, size_t N, size_t K, const float* bias, const float* W,
@@ -364,22 +434,32 @@ int dyhip_affine_forward(dyhip_device* dev, size_t M, size_t N, size_t K, const 
   DYHIP_CHECK_DEV(dev);
   DYHIP_REQUIRE(bias != nullptr, "AffineTransform: null bias");
   GemmSeg s{W, M, x, K, K};
-  GemmEpiParams ep{kEpiBias, 0.f, bias, 0, 0};
+  GemmEpiParams ep{};
+  ep.kind = kEpiBias;
+  ep.bias = bias;
   return gemm_run(dev, false, true, M, N, 1, &s, fx, ep);
 }
 
-int dyhip_gemm_tn_acc(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float* y) {
+int dyhip_gemm_tn(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float beta,
+                  float* y) {
   DYHIP_CHECK_DEV(dev);
   GemmSeg s{l, K, r, K, K};
-  GemmEpiParams ep{kEpiAxpby, 1.0f, nullptr, 0, 0};
-  return gemm_run(dev, true, true, M, N, 1, &s, y, ep);
+  return gemm_run(dev, true, true, M, N, 1, &s, y, axpby(beta));
+}
+
+int dyhip_gemm_nt(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float beta,
+                  float* y) {
+  DYHIP_CHECK_DEV(dev);
+  GemmSeg s{l, M, r, N, K};
+  return gemm_run(dev, false, false, M, N, 1, &s, y, axpby(beta));
+}
+
+int dyhip_gemm_tn_acc(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float* y) {
+  return dyhip_gemm_tn(dev, M, N, K, l, r, 1.0f, y);
 }
 
 int dyhip_gemm_nt_acc(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float* y) {
-  DYHIP_CHECK_DEV(dev);
-  GemmSeg s{l, M, r, N, K};
-  GemmEpiParams ep{kEpiAxpby, 1.0f, nullptr, 0, 0};
-  return gemm_run(dev, false, false, M, N, 1, &s, y, ep);
+  return dyhip_gemm_nt(dev, M, N, K, l, r, 1.0f, y);
 }
 
 }  // extern "C"

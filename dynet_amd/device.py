@@ -255,6 +255,12 @@ class Device:
     def affine_forward(self, M, N, K, bias, W, x, fx):
         _check(cdll.dyhip_affine_forward(self.handle, _sz(M), _sz(N), _sz(K), _p(bias), _p(W), _p(x), _p(fx)))
 
+    def gemm_tn(self, M, N, K, l, r, beta, y):
+        _check(cdll.dyhip_gemm_tn(self.handle, _sz(M), _sz(N), _sz(K), _p(l), _p(r), _f(beta), _p(y)))
+
+    def gemm_nt(self, M, N, K, l, r, beta, y):
+        _check(cdll.dyhip_gemm_nt(self.handle, _sz(M), _sz(N), _sz(K), _p(l), _p(r), _f(beta), _p(y)))
+
     def gemm_tn_acc(self, M, N, K, l, r, y):
         _check(cdll.dyhip_gemm_tn_acc(self.handle, _sz(M), _sz(N), _sz(K), _p(l), _p(r), _p(y)))
 

@@ -166,6 +166,11 @@ int dyhip_gemm_nn(dyhip_device* dev, size_t M, size_t N, size_t K, const float* 
 int dyhip_gemm_tn_acc(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float* y);
 /* MatrixMultiplyTranspAcc (:162-180): y[MxN] += l[MxK] * r[NxK]^T */
 int dyhip_gemm_nt_acc(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float* y);
+/* the two transposed forms with an explicit beta (beta = 0 overwrites y, which saves zeroing a
+ * gradient buffer that has a single producer); the cublasSgemm calls behind
+ * dynet/matrix-multiply.h:104-113,169-178 take the same scalar */
+int dyhip_gemm_tn(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float beta, float* y);
+int dyhip_gemm_nt(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float beta, float* y);
 
 /* AffineTransform with one (W, x) pair (dynet/nodes-affinetransform.cc:77-113):
  * fx[MxN] = bias[M] broadcast over the N columns + W[MxK] * x[KxN], the bias folded into
