@@ -11,6 +11,8 @@
 // reference copies gate slices to scratch first).
 //
 // Layout: gates is 4H x B column-major, gate order i, f, o, g; c, h are H x B.
+#include <initializer_list>
+
 #include "gemm.h"
 
 namespace dyhip {
@@ -96,6 +98,131 @@ static int launch_pointwise(dyhip_device* dev, unsigned H, unsigned B, const flo
                      gates, d, out);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
+}
+
+
+// ---- fused cell step: gates + C + H in one kernel around the recurrent GEMM ----------
+// The input projection Wx*x of every timestep is one large GEMM up front; a timestep is
+// then (1) the split-K GEMM Wh*h_tm1 whose unreduced slices stay in a workspace and
+// (2) this kernel, which adds the slices, the input projection, the bias and the forget
+// bias, applies the activations and forms c and h.  One thread owns V consecutive hidden
+// units of one batch column and touches the four gate rows j, H+j, 2H+j, 3H+j.
+template <int V>
+struct Pack;
+template <>
+struct Pack<1> {
+  float v[1];
+  __device__ __forceinline__ void load(const float* p) { v[0] = *p; }
+  __device__ __forceinline__ void store(float* p) const { *p = v[0]; }
+};
+template <>
+struct Pack<4> {
+  float v[4];
+  __device__ __forceinline__ void load(const float* p) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  }
+  __device__ __forceinline__ void store(float* p) const { *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]); }
+};
+
+constexpr int kCellThreads = 64;
+
+template <int V>
+__global__ __launch_bounds__(kCellThreads) void lstm_cell_fwd_kernel(unsigned H, unsigned splits, size_t slice,
+                                                                     const float* xproj, const float* __restrict__ rec,
+                                                                     const float* __restrict__ bias,
+                                                                     const float* __restrict__ c_prev, int mode,
+                                                                     float* gates, float* __restrict__ c,
+                                                                     float* __restrict__ h) {
+  const unsigned j = (blockIdx.x * kCellThreads + threadIdx.x) * V, b = blockIdx.y;
+  if (j >= H) return;
+  const size_t g0 = size_t(b) * 4 * H + j, s0 = size_t(b) * H + j;
+  Pack<V> pre[4], cp;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    Pack<V> bq, xq;
+    bq.load(bias + q * H + j);
+    xq.load(xproj + g0 + size_t(q) * H);
+#pragma unroll
+    for (int e = 0; e < V; ++e) pre[q].v[e] = (q == 1 ? bq.v[e] + 1.0f : bq.v[e]) + xq.v[e];
+  }
+  for (unsigned k = 0; k < splits; ++k) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      Pack<V> r;
+      r.load(rec + size_t(k) * slice + g0 + size_t(q) * H);
+#pragma unroll
+      for (int e = 0; e < V; ++e) pre[q].v[e] += r.v[e];
+    }
+  }
+  if (c_prev) cp.load(c_prev + s0);
+  Pack<V> cn, hn;
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    const float gi = logistic(mode, pre[0].v[e]), gf = logistic(mode, pre[1].v[e]), go = logistic(mode, pre[2].v[e]);
+    const float gg = tanh_accurate(pre[3].v[e]);
+    pre[0].v[e] = gi; pre[1].v[e] = gf; pre[2].v[e] = go; pre[3].v[e] = gg;
+    const float cv = c_prev ? gi * gg + gf * cp.v[e] : gi * gg;
+    cn.v[e] = cv;
+    hn.v[e] = go * tanh_accurate(cv);
+  }
+#pragma unroll
+  for (int q = 0; q < 4; ++q) pre[q].store(gates + g0 + size_t(q) * H);
+  cn.store(c + s0);
+  hn.store(h + s0);
+}
+
+// Backward of the same step.  dh = dh_in + sum of the slices of Wh^T * dpre_{t+1}; then the
+// H, C and gate-activation backward formulas of dynet/nodes-lstm.cc:358-361,605-614,684-701
+// in one pass: writes dpre (4H x B) and dc_tm1.
+template <int V>
+__global__ __launch_bounds__(kCellThreads) void lstm_cell_bwd_kernel(unsigned H, unsigned splits, size_t slice,
+                                                                     const float* __restrict__ gates,
+                                                                     const float* __restrict__ c,
+                                                                     const float* __restrict__ c_prev,
+                                                                     const float* __restrict__ dh_in,
+                                                                     const float* __restrict__ rec,
+                                                                     const float* dc_in, float* __restrict__ dpre,
+                                                                     float* dc_prev) {
+  const unsigned j = (blockIdx.x * kCellThreads + threadIdx.x) * V, b = blockIdx.y;
+  if (j >= H) return;
+  const size_t g0 = size_t(b) * 4 * H + j, s0 = size_t(b) * H + j;
+  Pack<V> gt[4], cv, cp, dh, dc;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) gt[q].load(gates + g0 + size_t(q) * H);
+  cv.load(c + s0);
+  dh.load(dh_in + s0);
+  if (c_prev) cp.load(c_prev + s0);
+  if (dc_in) dc.load(dc_in + s0);
+  for (unsigned k = 0; k < splits; ++k) {
+    Pack<V> r;
+    r.load(rec + size_t(k) * slice + s0);
+#pragma unroll
+    for (int e = 0; e < V; ++e) dh.v[e] += r.v[e];
+  }
+  Pack<V> out[4], dcp;
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    const float gi = gt[0].v[e], gf = gt[1].v[e], go = gt[2].v[e], gg = gt[3].v[e];
+    const float t = tanh_accurate(cv.v[e]);
+    const float dcv = (dc_in ? dc.v[e] : 0.f) + dh.v[e] * go * (1.f - t * t);
+    const float d_o = dh.v[e] * t;
+    const float d_i = dcv * gg, d_f = c_prev ? dcv * cp.v[e] : 0.f, d_g = dcv * gi;
+    dcp.v[e] = dcv * gf;
+    out[0].v[e] = d_i * gi * (1.f - gi);
+    out[1].v[e] = d_f * gf * (1.f - gf);
+    out[2].v[e] = d_o * go * (1.f - go);
+    out[3].v[e] = d_g * (1.f - gg * gg);
+  }
+#pragma unroll
+  for (int q = 0; q < 4; ++q) out[q].store(dpre + g0 + size_t(q) * H);
+  if (dc_prev) dcp.store(dc_prev + s0);
+}
+
+static bool all_aligned16(std::initializer_list<const void*> ps) {
+  for (const void* p : ps)
+    if (p != nullptr && !aligned16(p)) return false;
+  return true;
 }
 
 struct GatesInputs {
@@ -319,6 +446,84 @@ int dyhip_lstm_h_backward(dyhip_device* dev, unsigned H, unsigned B, const float
   DYHIP_REQUIRE(i < 2, "VanillaLSTMH has two arguments (i = %u)", i);
   return i == 0 ? launch_pointwise<4>(dev, H, B, c, gates, dEdf, dEdxi)
                 : launch_pointwise<5>(dev, H, B, c, gates, dEdf, dEdxi);
+}
+
+// ---- fused cell path ------------------------------------------------------------------
+static int recurrent_partials(dyhip_device* dev, bool transposed, unsigned H, unsigned B, const float* Wh,
+                              const float* v, void* ws, size_t ws_bytes, unsigned* splits) {
+  DYHIP_REQUIRE(H >= 1 && B >= 1 && B <= 65535, "LSTM cell: bad hidden (%u) or batch (%u) size", H, B);
+  DYHIP_REQUIRE(Wh && v && ws && splits, "LSTM cell: null pointer");
+  const size_t G = size_t(4) * H;
+  GemmEpiParams ep{};
+  ep.kind = kEpiPartials;
+  ep.partials = static_cast<float*>(ws);
+  ep.partials_bytes = ws_bytes;
+  ep.splits_out = splits;
+  if (!transposed) {  // Wh[4H x H] * h[H x B]
+    GemmSeg s{Wh, G, v, H, H};
+    return gemm_run(dev, false, true, G, B, 1, &s, nullptr, ep);
+  }
+  GemmSeg s{Wh, G, v, G, G};  // Wh^T * dpre[4H x B]
+  return gemm_run(dev, true, true, H, B, 1, &s, nullptr, ep);
+}
+
+int dyhip_lstm_cell_workspace(dyhip_device* dev, unsigned H, unsigned B, size_t* fwd_bytes, size_t* bwd_bytes) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(fwd_bytes && bwd_bytes, "null output pointer");
+  // room for the largest split count the GEMM planner considers
+  *fwd_bytes = align256(sizeof(float) * size_t(4) * H * B) * 32;
+  *bwd_bytes = align256(sizeof(float) * size_t(H) * B) * 32;
+  return DYHIP_OK;
+}
+
+int dyhip_lstm_recurrent_forward(dyhip_device* dev, unsigned H, unsigned B, const float* Wh, const float* h_tm1,
+                                 void* ws, size_t ws_bytes, unsigned* splits) {
+  DYHIP_CHECK_DEV(dev);
+  return recurrent_partials(dev, false, H, B, Wh, h_tm1, ws, ws_bytes, splits);
+}
+
+int dyhip_lstm_recurrent_backward(dyhip_device* dev, unsigned H, unsigned B, const float* Wh, const float* dpre,
+                                  void* ws, size_t ws_bytes, unsigned* splits) {
+  DYHIP_CHECK_DEV(dev);
+  return recurrent_partials(dev, true, H, B, Wh, dpre, ws, ws_bytes, splits);
+}
+
+int dyhip_lstm_cell_forward(dyhip_device* dev, unsigned H, unsigned B, const float* xproj, const float* b,
+                            const float* rec, unsigned splits, const float* c_tm1, int logistic_mode, float* gates,
+                            float* c, float* h) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(H >= 1 && B >= 1 && B <= 65535, "LSTM cell: bad hidden (%u) or batch (%u) size", H, B);
+  DYHIP_REQUIRE(xproj && b && gates && c && h, "LSTM cell: null tensor pointer");
+  DYHIP_REQUIRE(splits == 0 || rec != nullptr, "LSTM cell: %u recurrent slices but no buffer", splits);
+  DYHIP_REQUIRE(logistic_mode == DYHIP_LOGISTIC_PACKET || logistic_mode == DYHIP_LOGISTIC_SCALAR,
+                "unknown logistic mode %d", logistic_mode);
+  const size_t slice = size_t(4) * H * B;
+  if (H % 4 == 0 && all_aligned16({xproj, b, rec, c_tm1, gates, c, h}))
+    hipLaunchKernelGGL(lstm_cell_fwd_kernel<4>, dim3(cdiv<unsigned>(H, kCellThreads * 4), B), dim3(kCellThreads), 0,
+                       dev->stream, H, splits, slice, xproj, rec, b, c_tm1, logistic_mode, gates, c, h);
+  else
+    hipLaunchKernelGGL(lstm_cell_fwd_kernel<1>, dim3(cdiv<unsigned>(H, kCellThreads), B), dim3(kCellThreads), 0,
+                       dev->stream, H, splits, slice, xproj, rec, b, c_tm1, logistic_mode, gates, c, h);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_lstm_cell_backward(dyhip_device* dev, unsigned H, unsigned B, const float* gates, const float* c,
+                             const float* c_tm1, const float* dh, const float* rec, unsigned splits, const float* dc,
+                             float* dpre, float* dc_tm1) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(H >= 1 && B >= 1 && B <= 65535, "LSTM cell: bad hidden (%u) or batch (%u) size", H, B);
+  DYHIP_REQUIRE(gates && c && dh && dpre, "LSTM cell: null tensor pointer");
+  DYHIP_REQUIRE(splits == 0 || rec != nullptr, "LSTM cell: %u recurrent slices but no buffer", splits);
+  const size_t slice = size_t(H) * B;
+  if (H % 4 == 0 && all_aligned16({gates, c, c_tm1, dh, rec, dc, dpre, dc_tm1}))
+    hipLaunchKernelGGL(lstm_cell_bwd_kernel<4>, dim3(cdiv<unsigned>(H, kCellThreads * 4), B), dim3(kCellThreads), 0,
+                       dev->stream, H, splits, slice, gates, c, c_tm1, dh, rec, dc, dpre, dc_tm1);
+  else
+    hipLaunchKernelGGL(lstm_cell_bwd_kernel<1>, dim3(cdiv<unsigned>(H, kCellThreads), B), dim3(kCellThreads), 0,
+                       dev->stream, H, splits, slice, gates, c, c_tm1, dh, rec, dc, dpre, dc_tm1);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
 }
 
 }  // extern "C"

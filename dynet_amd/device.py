@@ -312,6 +312,32 @@ class Device:
     def lstm_h_backward(self, H, B, c, gates, dEdf, i, dEdxi):
         _check(cdll.dyhip_lstm_h_backward(self.handle, _u(H), _u(B), _p(c), _p(gates), _p(dEdf), _u(i), _p(dEdxi)))
 
+    # ---- fused cell path --------------------------------------------------
+    def lstm_cell_workspace(self, H, B):
+        f, b = _sz(0), _sz(0)
+        _check(cdll.dyhip_lstm_cell_workspace(self.handle, _u(H), _u(B), C.byref(f), C.byref(b)))
+        return f.value, b.value
+
+    def lstm_recurrent_forward(self, H, B, Wh, h_tm1, ws, ws_bytes):
+        n = _u(0)
+        _check(cdll.dyhip_lstm_recurrent_forward(self.handle, _u(H), _u(B), _p(Wh), _p(h_tm1), _vp(ws), _sz(ws_bytes),
+                                                 C.byref(n)))
+        return n.value
+
+    def lstm_recurrent_backward(self, H, B, Wh, dpre, ws, ws_bytes):
+        n = _u(0)
+        _check(cdll.dyhip_lstm_recurrent_backward(self.handle, _u(H), _u(B), _p(Wh), _p(dpre), _vp(ws), _sz(ws_bytes),
+                                                  C.byref(n)))
+        return n.value
+
+    def lstm_cell_forward(self, H, B, xproj, b, rec, splits, c_tm1, gates, c, h, logistic_mode=lib.LOGISTIC_PACKET):
+        _check(cdll.dyhip_lstm_cell_forward(self.handle, _u(H), _u(B), _p(xproj), _p(b), _vp(rec), _u(splits),
+                                            _p(c_tm1), _i(logistic_mode), _p(gates), _p(c), _p(h)))
+
+    def lstm_cell_backward(self, H, B, gates, c, c_tm1, dh, rec, splits, dc, dpre, dc_tm1):
+        _check(cdll.dyhip_lstm_cell_backward(self.handle, _u(H), _u(B), _p(gates), _p(c), _p(c_tm1), _p(dh), _vp(rec),
+                                             _u(splits), _p(dc), _p(dpre), _p(dc_tm1)))
+
     # ---- lookup -----------------------------------------------------------
     def lookup_forward(self, ids_host, ids_dev, dim, vocab, table, fx, mult=1.0):
         n = ids_dev.size

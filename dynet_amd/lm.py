@@ -7,9 +7,13 @@ HIP graph.
 What differs from DyNet's node-at-a-time execution (results agree to fp32 rounding):
   * the T lookups, the T projections and the T PickNegLogSoftmax nodes of a step run as one call each over
     T*B columns (what DyNet's autobatching does to them);
-  * with ``time_batched=True`` the weight/bias gradients of the gate GEMMs are formed once per layer over the
-    K = T*B columns of all timesteps instead of T times over B columns;
-  * gradient clipping never leaves the device: squared norms -> clip scale -> update all read device memory.
+  * gradient clipping never leaves the device: squared norms -> clip scale -> update all read device memory;
+  * ``path="nodes"`` issues the three fused LSTM nodes per layer and timestep exactly as
+    CompactVanillaLSTMBuilder::add_input_impl does; with ``time_batched=True`` the weight/bias gradients of the
+    gate GEMMs are formed once per layer over the K = T*B columns of all timesteps instead of T times over B;
+  * ``path="fused"`` (default) runs layer by layer: one GEMM forms Wx*x for all timesteps, a timestep is then
+    the recurrent GEMM Wh*h plus one cell kernel (gates + c + h); backward mirrors it, and dx, dWx, dWh, db are
+    GEMMs/reductions over all timesteps.
 """
 import numpy as np
 
@@ -20,9 +24,10 @@ from .synth import glorot
 class LstmLM:
     """V-word LM: embedding E, L layers of hidden H, batch B, T timesteps per step."""
 
-    def __init__(self, dev, V, E, H, L, B, T, seed=0, lr=0.1, clip=5.0, time_batched=True, params=None):
+    def __init__(self, dev, V, E, H, L, B, T, seed=0, lr=0.1, clip=5.0, time_batched=True, params=None, path="fused"):
+        assert path in ("fused", "nodes")
         self.dev, self.V, self.E, self.H, self.L, self.B, self.T = dev, V, E, H, L, B, T
-        self.lr, self.clip, self.time_batched = float(lr), float(clip), bool(time_batched)
+        self.lr, self.clip, self.time_batched, self.path = float(lr), float(clip), bool(time_batched), path
         N = self.N = T * B
         PS, FXS, DE = lib.POOL_PS, lib.POOL_FXS, lib.POOL_DEDFS
         if params is None:
@@ -56,6 +61,9 @@ class LstmLM:
         self.d_gates = [dev.empty((T, B, 4 * H), pool=DE) for _ in range(L)]
         self.de_bytes = dev.pool(DE).used() - self.de_begin
         self.d_pre = [dev.empty((T, B, 4 * H), pool=DE) for _ in range(L)]  # overwritten, never accumulated into
+        fb, bb = dev.lstm_cell_workspace(H, B)
+        self.rec_f, self.rec_f_bytes = dev.workspace(fb)
+        self.rec_b, self.rec_b_bytes = dev.workspace(bb)
         self.plan, self.plan_ws, self.plan_ws_bytes = dev.lookup_plan_buffers(N, V)
         self.graph = None
 
@@ -96,6 +104,32 @@ class LstmLM:
     def forward(self):
         d, V, E, H, L, B, T, N = self.dev, self.V, self.E, self.H, self.L, self.B, self.T, self.N
         d.lookup_forward(None, self.ids, E, V, self.p["C"], self.emb)
+        if self.path == "fused":
+            self._forward_layers_fused()
+        else:
+            self._forward_layers_nodes()
+        d.affine_forward(V, N, H, self.p["bias"], self.p["R"], self.h[L - 1], self.logits)
+        d.pnls_forward_staged(V, N, self.logits, self.aux, self.errs)
+        d.sum_batches_forward(1, N, self.errs, self.loss)
+
+    def _forward_layers_fused(self):
+        d, E, H, L, B, T, N = self.dev, self.E, self.H, self.L, self.B, self.T, self.N
+        for l in range(L):
+            x, d_in = (self.h[l - 1], H) if l > 0 else (self.emb, E)
+            d.gemm_nn(4 * H, N, d_in, self.p[f"Wx{l}"], x, 0.0, self.gates[l])  # Wx*x of every timestep
+            for t in range(T):
+                g = self._t(self.gates[l], t, 4 * H)
+                if t > 0:
+                    n = d.lstm_recurrent_forward(H, B, self.p[f"Wh{l}"], self._t(self.h[l], t - 1, H), self.rec_f,
+                                                 self.rec_f_bytes)
+                    d.lstm_cell_forward(H, B, g, self.p[f"b{l}"], self.rec_f, n, self._t(self.c[l], t - 1, H), g,
+                                        self._t(self.c[l], t, H), self._t(self.h[l], t, H))
+                else:
+                    d.lstm_cell_forward(H, B, g, self.p[f"b{l}"], None, 0, None, g, self._t(self.c[l], t, H),
+                                        self._t(self.h[l], t, H))
+
+    def _forward_layers_nodes(self):
+        d, E, H, L, B, T = self.dev, self.E, self.H, self.L, self.B, self.T
         for t in range(T):
             x, d_in = self._t(self.emb, t, E), E
             for l in range(L):
@@ -106,19 +140,47 @@ class LstmLM:
                 d.lstm_c_forward(H, B, c_tm1, g, c)
                 d.lstm_h_forward(H, B, c, g, h)
                 x, d_in = h, H
-        d.affine_forward(V, N, H, self.p["bias"], self.p["R"], self.h[L - 1], self.logits)
-        d.pnls_forward_staged(V, N, self.logits, self.aux, self.errs)
-        d.sum_batches_forward(1, N, self.errs, self.loss)
 
     def backward(self):
         d, V, E, H, L, B, T, N = self.dev, self.V, self.E, self.H, self.L, self.B, self.T, self.N
-        d.zero(lib_tensor(d, self.d_errs.ptr, self.de_bytes))
+        fused = self.path == "fused"
+        # the node path accumulates into every gradient buffer; the fused path overwrites all but d_logits
+        d.zero(self.d_logits if fused else lib_tensor(d, self.d_errs.ptr, self.de_bytes))
         d.constant(self.d_errs, 1.0)  # d loss / d errs[b] through sum_batches(sum(errs))
         d.pnls_backward(V, N, self.logits, self.aux, self.d_errs, self.d_logits)
         top = self.h[L - 1]
         d.csum_backward(V, 1, N, self.d_logits, 0, self.g["bias"])
         d.gemm_nt_acc(V, H, N, self.d_logits, top, self.g["R"])
-        d.gemm_tn_acc(H, N, V, self.p["R"], self.d_logits, self.d_h[L - 1])
+        d.gemm_tn(H, N, V, self.p["R"], self.d_logits, 0.0 if fused else 1.0, self.d_h[L - 1])
+        if fused:
+            self._backward_layers_fused()
+        else:
+            self._backward_layers_nodes()
+        d.lookup_accumulate_grads_planned(N, self.plan, E, V, self.d_emb, self.g["C"])
+
+    def _backward_layers_fused(self):
+        d, E, H, L, B, T, N = self.dev, self.E, self.H, self.L, self.B, self.T, self.N
+        for l in reversed(range(L)):
+            Wh = self.p[f"Wh{l}"]
+            n = 0
+            for t in reversed(range(T)):
+                last, first = t == T - 1, t == 0
+                dpre = self._t(self.d_pre[l], t, 4 * H)
+                d.lstm_cell_backward(H, B, self._t(self.gates[l], t, 4 * H), self._t(self.c[l], t, H),
+                                     None if first else self._t(self.c[l], t - 1, H), self._t(self.d_h[l], t, H),
+                                     None if last else self.rec_b, n, None if last else self._t(self.d_c[l], t, H),
+                                     dpre, None if first else self._t(self.d_c[l], t - 1, H))
+                if not first:
+                    n = d.lstm_recurrent_backward(H, B, Wh, dpre, self.rec_b, self.rec_b_bytes)
+            x, d_in, dx = (self.h[l - 1], H, self.d_h[l - 1]) if l > 0 else (self.emb, E, self.d_emb)
+            d.gemm_tn(d_in, N, 4 * H, self.p[f"Wx{l}"], self.d_pre[l], 0.0, dx)
+            d.gemm_nt_acc(4 * H, d_in, N, self.d_pre[l], x, self.g[f"Wx{l}"])
+            if T > 1:
+                d.gemm_nt_acc(4 * H, H, N - B, self._t(self.d_pre[l], 1, 4 * H), self.h[l], self.g[f"Wh{l}"])
+            d.csum_backward(4 * H, 1, N, self.d_pre[l], 0, self.g[f"b{l}"])
+
+    def _backward_layers_nodes(self):
+        d, E, H, L, B, T, N = self.dev, self.E, self.H, self.L, self.B, self.T, self.N
         for t in reversed(range(T)):
             for l in reversed(range(L)):
                 g, c = self._t(self.gates[l], t, 4 * H), self._t(self.c[l], t, H)
@@ -151,7 +213,6 @@ class LstmLM:
                 if T > 1:
                     d.gemm_nt_acc(4 * H, H, N - B, self._t(self.d_pre[l], 1, 4 * H), self.h[l], self.g[f"Wh{l}"])
                 d.csum_backward(4 * H, 1, N, self.d_pre[l], 0, self.g[f"b{l}"])
-        d.lookup_accumulate_grads_planned(N, self.plan, E, V, self.d_emb, self.g["C"])
 
     def update(self):
         d = self.dev

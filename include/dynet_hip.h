@@ -209,6 +209,35 @@ int dyhip_lstm_h_forward(dyhip_device* dev, unsigned H, unsigned B, const float*
 int dyhip_lstm_h_backward(dyhip_device* dev, unsigned H, unsigned B, const float* c, const float* gates,
                           const float* dEdf, unsigned i, float* dEdxi);
 
+/* ---- fused cell step: VanillaLSTMGates + VanillaLSTMC + VanillaLSTMH of one timestep
+ * (dynet/nodes-lstm.cc:101-235,562-615,650-703 forward; :237-527,591-615,670-703 backward)
+ * around one recurrent GEMM.  The input projection xproj = Wx * x is formed for all
+ * timesteps at once (dyhip_gemm_nn over T*B columns); a timestep is then
+ *   dyhip_lstm_recurrent_forward : Wh * h_tm1 as unreduced split-K slices in ws
+ *   dyhip_lstm_cell_forward      : gates = act(b + [f: +1] + xproj + sum of slices),
+ *                                  c = i*g + f*c_tm1, h = o*tanh(c)
+ * and backwards, newest timestep first,
+ *   dyhip_lstm_cell_backward     : dh_t = dh + sum of the slices left by the t+1 call below;
+ *                                  writes dpre_t (4H x B, gradient of the pre-activations)
+ *                                  and dc_tm1
+ *   dyhip_lstm_recurrent_backward: Wh^T * dpre_t as slices for the t-1 call.
+ * Weight gradients are then GEMMs over all timesteps (dyhip_gemm_nt with K = T*B), dx is
+ * dyhip_gemm_tn(Wx, dpre) and db a batch reduction of dpre.  No dropout masks on this
+ * path.  gates may alias xproj (each element is read before it is written).  rec/splits
+ * = NULL/0 and c_tm1 = NULL stand for the zero initial state (dynet/lstm.cc:1060-1061);
+ * dc = NULL for the last timestep, dc_tm1 = NULL for the first. */
+int dyhip_lstm_cell_workspace(dyhip_device* dev, unsigned H, unsigned B, size_t* fwd_bytes, size_t* bwd_bytes);
+int dyhip_lstm_recurrent_forward(dyhip_device* dev, unsigned H, unsigned B, const float* Wh, const float* h_tm1,
+                                 void* ws, size_t ws_bytes, unsigned* splits);
+int dyhip_lstm_cell_forward(dyhip_device* dev, unsigned H, unsigned B, const float* xproj, const float* b,
+                            const float* rec, unsigned splits, const float* c_tm1, int logistic_mode, float* gates,
+                            float* c, float* h);
+int dyhip_lstm_recurrent_backward(dyhip_device* dev, unsigned H, unsigned B, const float* Wh, const float* dpre,
+                                  void* ws, size_t ws_bytes, unsigned* splits);
+int dyhip_lstm_cell_backward(dyhip_device* dev, unsigned H, unsigned B, const float* gates, const float* c,
+                             const float* c_tm1, const float* dh, const float* rec, unsigned splits, const float* dc,
+                             float* dpre, float* dc_tm1);
+
 /* ---- LookupNode (dynet/param-nodes.cc:304-329) and
  * LookupParameterStorage::accumulate_grads (dynet/model.cc:728-743) -------- */
 /* fx[:, b] = table[:, ids[b]] * mult; bit-exact gather when mult == 1.0f.

@@ -28,16 +28,16 @@ def _grad_floor(ref):
     return max(float(np.abs(ref).max()) * 1e-2, 1e-6)
 
 
-@pytest.mark.parametrize("time_batched", [False, True])
+@pytest.mark.parametrize("path,time_batched", [("nodes", False), ("nodes", True), ("fused", True)])
 @pytest.mark.parametrize("case", CASES)
-def test_lm_step_matches_oracle(dev, case, time_batched):
+def test_lm_step_matches_oracle(dev, case, path, time_batched):
     V, E, H, L, B, T = case
     rng = np.random.default_rng(11)
     params = LstmLM.init_params(V, E, H, L, seed=3)
     for l in range(L):  # non-zero biases exercise the bias path
         params[f"b{l}"] = rng.normal(0, 0.1, 4 * H).astype(np.float32)
     ref_p = {n: a.copy() for n, a in params.items()}
-    lm = LstmLM(dev, V, E, H, L, B, T, lr=0.1, clip=5.0, time_batched=time_batched, params=params)
+    lm = LstmLM(dev, V, E, H, L, B, T, lr=0.1, clip=5.0, time_batched=time_batched, params=params, path=path)
     for it in range(2):
         tokens = _tokens(rng, V, B, T)
         ref_loss, ref_g, ref_scale = lm_oracle.step(ref_p, tokens, L, lr=0.1, clip=5.0)

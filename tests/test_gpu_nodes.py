@@ -212,6 +212,72 @@ def test_fused_nodes_equal_unfused_path_over_three_steps(dev):
         ht, ct = h2, c2
 
 
+@pytest.mark.parametrize("I,H,B", [(128, 256, 32), (24, 50, 7), (256, 1024, 128), (5, 3, 1)])
+def test_fused_cell_path_equals_node_composition(dev, I, H, B):
+    """dyhip_lstm_recurrent_* + dyhip_lstm_cell_* over two timesteps (the first from the zero state)
+    against the oracle's VanillaLSTMGates -> C -> H nodes and their backward."""
+    rng = np.random.default_rng(I + H + B)
+    Wx, Wh, b = glorot(rng, 4 * H, I), glorot(rng, 4 * H, H), f32(rng.normal(0, 0.1, 4 * H))
+    xs = [f32(rng.standard_normal((B, I))) for _ in range(2)]
+    zeros = np.zeros((B, H), F32)
+    # oracle: node by node
+    ref = []
+    h_prev, c_prev = zeros, zeros
+    for x in xs:
+        g = orc.lstm_gates_forward([x], [I], H, B, h_prev, Wx, Wh, b)
+        c = orc.lstm_c_forward(H, B, c_prev, g)
+        h = orc.lstm_h_forward(H, B, c, g)
+        ref.append((g, c, h, h_prev, c_prev))
+        h_prev, c_prev = h, c
+    # device: xproj for both steps at once, then cell steps
+    Wxt, Wht, bt = dev.tensor(Wx), dev.tensor(Wh), dev.tensor(b)
+    X = dev.tensor(np.stack(xs))
+    gates, cs, hs = dev.empty((2, B, 4 * H)), dev.empty((2, B, H)), dev.empty((2, B, H))
+    fb, bb = dev.lstm_cell_workspace(H, B)
+    wf, wfb = dev.workspace(fb)
+    wb, wbb = dev.workspace(bb)
+    dev.gemm_nn(4 * H, 2 * B, I, Wxt, X, 0.0, gates)
+    sl = lambda t, k, w: t.offset(k * B * w, (B, w))
+    dev.lstm_cell_forward(H, B, sl(gates, 0, 4 * H), bt, None, 0, None, sl(gates, 0, 4 * H), sl(cs, 0, H), sl(hs, 0, H))
+    n = dev.lstm_recurrent_forward(H, B, Wht, sl(hs, 0, H), wf, wfb)
+    assert n >= 1
+    dev.lstm_cell_forward(H, B, sl(gates, 1, 4 * H), bt, wf, n, sl(cs, 0, H), sl(gates, 1, 4 * H), sl(cs, 1, H),
+                          sl(hs, 1, H))
+    # another summation order moves a pre-activation by ~1e-7 * (size of its terms); the gate, c and h
+    # move by at most that (|sigma'|, |tanh'| <= 1)
+    floor = max(1.0, float(np.sqrt(I + H) * max(rms(Wx), rms(Wh))))
+    for k in range(2):
+        assert_close(sl(gates, k, 4 * H).numpy(), ref[k][0], FWD_RTOL, f"gates[{k}]", floor=floor)
+        assert_close(sl(cs, k, H).numpy(), ref[k][1], FWD_RTOL, f"c[{k}]", floor=floor)
+        assert_close(sl(hs, k, H).numpy(), ref[k][2], FWD_RTOL, f"h[{k}]", floor=floor)
+    # backward: gradients arrive at h of both steps
+    dh = [f32(rng.standard_normal((B, H))) for _ in range(2)]
+    r_dh = [d.copy() for d in dh]
+    r_dc = [np.zeros((B, H), F32) for _ in range(2)]
+    r_dpre = [None, None]
+    for k in (1, 0):
+        g, c, h, hp, cp = ref[k]
+        dg = np.zeros((B, 4 * H), F32)
+        orc.lstm_h_backward(H, B, c, g, r_dh[k], 0, r_dc[k])
+        orc.lstm_h_backward(H, B, c, g, r_dh[k], 1, dg)
+        if k > 0:
+            orc.lstm_c_backward(H, B, cp, g, r_dc[k], 0, r_dc[k - 1])
+        orc.lstm_c_backward(H, B, cp, g, r_dc[k], 1, dg)
+        r_dpre[k] = np.where(np.arange(4 * H) < 3 * H, dg * g * (F32(1) - g), dg * (F32(1) - g * g)).astype(F32)
+        if k > 0:
+            orc.lstm_gates_backward([xs[k]], [I], H, B, hp, Wx, Wh, g, dg, 1, r_dh[k - 1])
+    dht = dev.tensor(np.stack(dh))
+    dct, dpre = dev.empty((2, B, H)), dev.empty((2, B, 4 * H))
+    dev.lstm_cell_backward(H, B, sl(gates, 1, 4 * H), sl(cs, 1, H), sl(cs, 0, H), sl(dht, 1, H), None, 0, None,
+                           sl(dpre, 1, 4 * H), sl(dct, 0, H))
+    n = dev.lstm_recurrent_backward(H, B, Wht, sl(dpre, 1, 4 * H), wb, wbb)
+    dev.lstm_cell_backward(H, B, sl(gates, 0, 4 * H), sl(cs, 0, H), None, sl(dht, 0, H), wb, n, sl(dct, 0, H),
+                           sl(dpre, 0, 4 * H), None)
+    for k in range(2):
+        assert_close(sl(dpre, k, 4 * H).numpy(), r_dpre[k], GRAD_RTOL, f"dpre[{k}]",
+                     floor=max(float(np.abs(r_dpre[k]).max()) * 1e-2, 1e-6))
+
+
 def test_lstm_rejects_bad_arguments(dev):
     t = dev.zeros(64)
     with pytest.raises(DyhipError) as e:
