@@ -58,6 +58,8 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the cfg 1 / 3 / 4 kernel measurements")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="bound on the CPU-baseline leg")
+    ap.add_argument("--no-lm", action="store_true", help="skip the cfg 5 LSTM-LM training-step measurement")
+    ap.add_argument("--lm-steps", type=int, default=30)
     return ap.parse_args()
 
 
@@ -267,6 +269,53 @@ def extras(dev, lib, reps):
     return res
 
 
+FP32_MFMA_PEAK_TFLOPS = 157.3
+
+
+def lstm_lm(steps, warmup=3):
+    """cfg 5: whole training step of the 2-layer LSTM LM (forward, backward, clip, SGD update), tokens/s."""
+    from dynet_amd import Device
+    from dynet_amd.lm import LstmLM
+    from dynet_amd.synth import zipf_ids
+
+    V, E, H, L, B, T = 10000, 256, 1024, 2, 128, 35
+    rng = np.random.default_rng(0)
+    batches = [zipf_ids(rng, (T + 1) * B, V).reshape(T + 1, B) for _ in range(8)]
+    flops = 3 * T * (2 * 4 * H * (E + H) * B + 2 * 4 * H * (H + H) * B + 2 * V * H * B)
+    res = {"config": {"V": V, "E": E, "H": H, "layers": L, "B": B, "T": T, "trainer": "SimpleSGD lr 0.1",
+                      "clip_threshold": 5.0, "init": "Glorot (lookup: embedding dim only), LSTM biases 0",
+                      "ids": "Zipf(1.1)"},
+           "tokens_per_step": T * B, "gemm_flop_per_step": flops,
+           "timed_region": "per step: host->device copy of ids and labels, id sort, forward, backward, "
+                           "device-side clipping, update; one HIP-graph replay per step; loss read back after "
+                           "the last step"}
+    for path, tb in (("fused", True), ("nodes", False)):
+        dev = Device(0, mem_mb=(1024, 1024, 512, 1024))
+        lm = LstmLM(dev, V, E, H, L, B, T, lr=0.1, clip=5.0, time_batched=tb, path=path)
+        lm.stage(batches[0])
+        lm.capture()
+        first = None
+        for i in range(warmup):
+            loss = lm.step(batches[i % len(batches)])
+            first = loss if first is None else first
+        dev.sync()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            lm.step(batches[(warmup + i) % len(batches)], read_loss=False)
+        dev.sync()
+        dt = (time.perf_counter() - t0) / steps
+        last = float(lm.loss.numpy()[0])
+        key = "fused_cell_path" if path == "fused" else "node_at_a_time_path"
+        res[key] = {"ms_per_step": round(dt * 1e3, 3), "tokens_per_s": round(T * B / dt, 1),
+                    "gemm_tflops": round(flops / dt / 1e12, 2),
+                    "frac_of_fp32_mfma_peak": round(flops / dt / 1e12 / FP32_MFMA_PEAK_TFLOPS, 4),
+                    "steps": steps, "loss_per_token_first": round(first / (T * B), 4),
+                    "loss_per_token_last": round(last / (T * B), 4)}
+        lm.graph.destroy()
+        dev.close()
+    return res
+
+
 def cpu_baseline(step_bytes, seconds):
     """The CPU oracle (plain-C restatement of DyNet's CPU path) on the same sweep, one host core."""
     from oracle import cpu_oracle as orc
@@ -369,6 +418,9 @@ def main():
     if not args.no_extras:
         out.update(extras(dev, lib, args.kernel_reps))
     dev.close()
+    if not args.no_lm:
+        out["cfg5_lstm_lm"] = lstm_lm(args.lm_steps)
+        out["lstm_lm_tokens_per_s"] = out["cfg5_lstm_lm"]["fused_cell_path"]["tokens_per_s"]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(sweep.step_bytes, args.cpu_seconds)
     print(json.dumps(out))

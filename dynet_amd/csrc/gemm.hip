@@ -34,6 +34,9 @@
 // gate epilogue.  The fused LSTM cell kernels consume the unreduced slices.
 #include "gemm.h"
 
+#include <cstdio>
+#include <cstdlib>
+
 namespace dyhip {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -162,12 +165,57 @@ __device__ __forceinline__ void load_pair(const GemmArgs& g, unsigned kt, bool i
   }
 }
 
-template <bool A_KMAJOR, bool B_KMAJOR, int WN>
+// One K-tile of the main loop: MFMA steps on LDS buffer `buf`, with the global loads of
+// tile i+PF issued first (into register slot S) and the tile i+1 (register slot S^1 for
+// PF == 2, S for PF == 1) parked in the other LDS buffer three quarters of the way through.
+template <bool A_KMAJOR, bool B_KMAJOR, int WN, int PF, int S>
+__device__ __forceinline__ void ktile_iter(const GemmArgs& g, unsigned kt_begin, unsigned n_tiles, unsigned i,
+                                           bool interior, size_t m0, size_t n0, TileRegs<kBM> (&ra)[PF],
+                                           TileRegs<64 * WN> (&rb)[PF], float* lds_a, float* lds_b,
+                                           floatx16 (&acc)[WN][2], int wm, int wn, int l32, int lhi) {
+  constexpr int BN = 64 * WN;
+  constexpr int PA = lds_pitch<A_KMAJOR, kBM>(), PB = lds_pitch<B_KMAJOR, BN>();
+  constexpr int NEXT = PF == 2 ? (S ^ 1) : S;  // register slot holding tile i+1
+  const int buf = i & 1;
+  if (i + PF < n_tiles) load_pair<A_KMAJOR, B_KMAJOR, WN>(g, kt_begin + i + PF, interior, m0, n0, ra[S], rb[S]);
+  const bool more = i + 1 < n_tiles;
+  const float* la = lds_a + buf * (kBK * PA) + wm * 64 + 2 * l32 + lhi * PA;
+  const float* lb = lds_b + buf * (kBK * PB) + wn * 32 * WN + WN * l32 + lhi * PB;
+  float av[2][2], bv[2][WN];
+  lds_read<2>(la, av[0]);
+  lds_read<WN>(lb, bv[0]);
+#pragma unroll
+  for (int s = 0; s < kBK / 2; ++s) {
+    const int cur = s & 1;
+    if (s + 1 < kBK / 2) {
+      lds_read<2>(la + (2 * s + 2) * PA, av[cur ^ 1]);
+      lds_read<WN>(lb + (2 * s + 2) * PB, bv[cur ^ 1]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int a = 0; a < WN; ++a)
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[cur][a], av[cur][b], acc[a][b], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    if (s == kWritePos && more) {
+      // the other buffer was last read in the previous iteration, which every wave has left
+      store_tile<A_KMAJOR, kBM>(ra[NEXT], lds_a + (buf ^ 1) * (kBK * PA));
+      store_tile<B_KMAJOR, BN>(rb[NEXT], lds_b + (buf ^ 1) * (kBK * PB));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  __syncthreads();
+}
+
+// PF = how many K-tiles ahead the global loads run (register stages).  Two for the 64-wide
+// tile: its blocks are the skinny, split-K ones whose few K-tiles are bound by load latency.
+template <bool A_KMAJOR, bool B_KMAJOR, int WN, int PF>
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_tile_kernel(GemmArgs g, unsigned tiles_m) {
   constexpr int BN = 64 * WN;
   constexpr int PA = lds_pitch<A_KMAJOR, kBM>(), PB = lds_pitch<B_KMAJOR, BN>();
-  __shared__ __attribute__((aligned(16))) float lds_a[2][kBK * PA];
-  __shared__ __attribute__((aligned(16))) float lds_b[2][kBK * PB];
+  __shared__ __attribute__((aligned(16))) float lds_a[2 * kBK * PA];
+  __shared__ __attribute__((aligned(16))) float lds_b[2 * kBK * PB];
 
   const unsigned tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m;
   const unsigned split = blockIdx.y;
@@ -189,43 +237,27 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_tile_kernel(GemmArgs g, 
   const bool interior = g.vec_ok && (m0 + kBM <= g.M) && (n0 + BN <= g.N);
 
   if (kt_begin < kt_end) {
-    TileRegs<kBM> ra;
-    TileRegs<BN> rb;
-    load_pair<A_KMAJOR, B_KMAJOR, WN>(g, kt_begin, interior, m0, n0, ra, rb);
-    store_tile<A_KMAJOR, kBM>(ra, lds_a[0]);
-    store_tile<B_KMAJOR, BN>(rb, lds_b[0]);
+    const unsigned n_tiles = kt_end - kt_begin;
+    TileRegs<kBM> ra[PF];
+    TileRegs<BN> rb[PF];
+    load_pair<A_KMAJOR, B_KMAJOR, WN>(g, kt_begin, interior, m0, n0, ra[0], rb[0]);
+    if (PF == 2 && n_tiles > 1)
+      load_pair<A_KMAJOR, B_KMAJOR, WN>(g, kt_begin + 1, interior, m0, n0, ra[PF - 1], rb[PF - 1]);
+    store_tile<A_KMAJOR, kBM>(ra[0], lds_a);
+    store_tile<B_KMAJOR, BN>(rb[0], lds_b);
     __syncthreads();
-    for (unsigned kt = kt_begin; kt < kt_end; ++kt) {
-      const int buf = (kt - kt_begin) & 1;
-      const bool more = kt + 1 < kt_end;
-      if (more) load_pair<A_KMAJOR, B_KMAJOR, WN>(g, kt + 1, interior, m0, n0, ra, rb);
-      const float* la = lds_a[buf] + wm * 64 + 2 * l32 + lhi * PA;
-      const float* lb = lds_b[buf] + wn * 32 * WN + WN * l32 + lhi * PB;
-      float av[2][2], bv[2][WN];
-      lds_read<2>(la, av[0]);
-      lds_read<WN>(lb, bv[0]);
-#pragma unroll
-      for (int s = 0; s < kBK / 2; ++s) {
-        const int cur = s & 1;
-        if (s + 1 < kBK / 2) {
-          lds_read<2>(la + (2 * s + 2) * PA, av[cur ^ 1]);
-          lds_read<WN>(lb + (2 * s + 2) * PB, bv[cur ^ 1]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int a = 0; a < WN; ++a)
-#pragma unroll
-          for (int b = 0; b < 2; ++b)
-            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[cur][a], av[cur][b], acc[a][b], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        if (s == kWritePos && more) {
-          // the other buffer was last read in the previous iteration, which every wave has left
-          store_tile<A_KMAJOR, kBM>(ra, lds_a[buf ^ 1]);
-          store_tile<B_KMAJOR, BN>(rb, lds_b[buf ^ 1]);
-          __builtin_amdgcn_sched_barrier(0);
-        }
+    if (PF == 1) {
+      for (unsigned i = 0; i < n_tiles; ++i)
+        ktile_iter<A_KMAJOR, B_KMAJOR, WN, PF, 0>(g, kt_begin, n_tiles, i, interior, m0, n0, ra, rb, lds_a, lds_b, acc,
+                                                   wm, wn, l32, lhi);
+    } else {
+      for (unsigned i = 0; i < n_tiles; i += 2) {
+        ktile_iter<A_KMAJOR, B_KMAJOR, WN, PF, 0>(g, kt_begin, n_tiles, i, interior, m0, n0, ra, rb, lds_a, lds_b, acc,
+                                                   wm, wn, l32, lhi);
+        if (i + 1 < n_tiles)
+          ktile_iter<A_KMAJOR, B_KMAJOR, WN, PF, PF - 1>(g, kt_begin, n_tiles, i + 1, interior, m0, n0, ra, rb, lds_a,
+                                                          lds_b, acc, wm, wn, l32, lhi);
       }
-      __syncthreads();
     }
   }
 
@@ -294,9 +326,9 @@ static void launch_tiles(dyhip_device* dev, const GemmArgs& g, unsigned tiles_m,
                          int wn) {
   const dim3 grid(tiles_m * tiles_n, splits), block(kGemmThreads);
   if (wn == 1)
-    hipLaunchKernelGGL((gemm_tile_kernel<A_KMAJOR, B_KMAJOR, 1>), grid, block, 0, dev->stream, g, tiles_m);
+    hipLaunchKernelGGL((gemm_tile_kernel<A_KMAJOR, B_KMAJOR, 1, 2>), grid, block, 0, dev->stream, g, tiles_m);
   else
-    hipLaunchKernelGGL((gemm_tile_kernel<A_KMAJOR, B_KMAJOR, 2>), grid, block, 0, dev->stream, g, tiles_m);
+    hipLaunchKernelGGL((gemm_tile_kernel<A_KMAJOR, B_KMAJOR, 2, 1>), grid, block, 0, dev->stream, g, tiles_m);
 }
 
 // Tile width and split count by a small cost model.  Measured on MI355X: the matrix cores
@@ -372,6 +404,10 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
   const bool must_partial = fused_epi || to_caller;
   GemmPlan plan{N <= 64 ? 1 : 2, 1};
   if (g.ktiles_total > 0) plan = plan_gemm(dev, M, N, g.ktiles_total, ws_bytes / out_bytes, must_partial);
+  if (const char* ov = getenv("DYHIP_GEMM_PLAN_DEBUG")) {
+    int wn_o = 0, s_o = 0;
+    if (sscanf(ov, "%d,%d", &wn_o, &s_o) == 2 && N <= 256) plan = GemmPlan{wn_o, (unsigned)s_o};
+  }
   unsigned splits = plan.splits;
   const size_t tiles_m = cdiv<size_t>(M, kBM), tiles_n = cdiv<size_t>(N, size_t(64) * plan.wn);
   DYHIP_REQUIRE(tiles_m * tiles_n < (size_t(1) << 31), "GEMM too large");
