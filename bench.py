@@ -51,7 +51,8 @@ def parse_args():
     ap.add_argument("--stream-threshold", type=int, default=None,
                     help="override the library's non-temporal access threshold in bytes (tuning experiments)")
     ap.add_argument("--kernel-reps", type=int, default=20, help="graph replays per per-kernel measurement")
-    ap.add_argument("--no-graph", action="store_true", help="time plain back-to-back launches instead of graph replays")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="plain back-to-back launches instead of HIP-graph replays everywhere (for profiler runs)")
     ap.add_argument("--one-pass", action="store_true",
                     help="counter-collection mode: launch every kernel of the sweep (and a 16.8 MB calibration copy) "
                          "a few times with plain launches, print nothing but a short note, and exit")
@@ -175,7 +176,7 @@ def per_kernel_table(dev, named, sets, reps, use_graph=True):
     return out
 
 
-def extras(dev, lib, reps):
+def extras(dev, lib, reps, use_graph=True):
     """cfg 3 (lookup), cfg 4 (PickNegLogSoftmax) kernels and the cfg 1 LSTM cell latency."""
     from dynet_amd.synth import glorot, zipf_ids
 
@@ -207,8 +208,8 @@ def extras(dev, lib, reps):
     planned = [("lookup_scatter_add(ids pre-sorted at forward)", G + 2 * uniq * D * 4,
                 lambda s: dev.lookup_accumulate_grads_planned(n, s["plan"], D, V, s["g"], s["grads"], ws2, wsb2))]
     res["cfg3_lookup"] = {"vocab": V, "dim": D, "n_ids": n, "unique_ids": uniq,
-                          "kernels": per_kernel_table(dev, gather, sets, reps) +
-                          per_kernel_table(dev, planned, sets, reps) +
+                          "kernels": per_kernel_table(dev, gather, sets, reps, use_graph=use_graph) +
+                          per_kernel_table(dev, planned, sets, reps, use_graph=use_graph) +
                           per_kernel_table(dev, scatter, sets, reps, use_graph=False)}
     for w in (lib.POOL_FXS, lib.POOL_DEDFS, lib.POOL_SCS):
         dev.sync()
@@ -230,7 +231,7 @@ def extras(dev, lib, reps):
         ("pnls_fwd", X, lambda s: dev.pnls_forward_staged(rows, bd, s["x"], s["aux"], s["fx"])),
         ("pnls_bwd", 3 * X, lambda s: dev.pnls_backward(rows, bd, s["x"], s["aux"], s["dy"], s["dx"])),
     ]
-    res["cfg4_pnls"] = {"rows": rows, "bd": bd, "kernels": per_kernel_table(dev, named, sets, reps)}
+    res["cfg4_pnls"] = {"rows": rows, "bd": bd, "kernels": per_kernel_table(dev, named, sets, reps, use_graph=use_graph)}
     for w in (lib.POOL_FXS, lib.POOL_DEDFS, lib.POOL_SCS):
         dev.sync()
         dev.free_pool(w)
@@ -261,9 +262,12 @@ def extras(dev, lib, reps):
     cell()
     dev.sync()
     dev.free_pool(lib.POOL_SCS)
-    g = capture(dev, [cell])
-    us = time_graph(dev, g, max(reps, 50), 1)
-    g.destroy()
+    if use_graph:
+        g = capture(dev, [cell])
+        us = time_graph(dev, g, max(reps, 50), 1)
+        g.destroy()
+    else:
+        us = time_loop(dev, [cell], max(reps, 50))
     res["cfg1_lstm_cell"] = {"I": I, "H": H, "B": B, "fwd_bwd_us": round(us, 2), "launches": 13 + 5,
                              "gemm_flops": 3 * 2 * 4 * H * (I + H) * B}
     return res
@@ -272,7 +276,7 @@ def extras(dev, lib, reps):
 FP32_MFMA_PEAK_TFLOPS = 157.3
 
 
-def lstm_lm(steps, warmup=3):
+def lstm_lm(steps, warmup=3, use_graph=True):
     """cfg 5: whole training step of the 2-layer LSTM LM (forward, backward, clip, SGD update), tokens/s."""
     from dynet_amd import Device
     from dynet_amd.lm import LstmLM
@@ -293,7 +297,8 @@ def lstm_lm(steps, warmup=3):
         dev = Device(0, mem_mb=(1024, 1024, 512, 1024))
         lm = LstmLM(dev, V, E, H, L, B, T, lr=0.1, clip=5.0, time_batched=tb, path=path)
         lm.stage(batches[0])
-        lm.capture()
+        if use_graph:
+            lm.capture()
         first = None
         for i in range(warmup):
             loss = lm.step(batches[i % len(batches)])
@@ -311,7 +316,8 @@ def lstm_lm(steps, warmup=3):
                     "frac_of_fp32_mfma_peak": round(flops / dt / 1e12 / FP32_MFMA_PEAK_TFLOPS, 4),
                     "steps": steps, "loss_per_token_first": round(first / (T * B), 4),
                     "loss_per_token_last": round(last / (T * B), 4)}
-        lm.graph.destroy()
+        if lm.graph is not None:
+            lm.graph.destroy()
         dev.close()
     return res
 
@@ -379,7 +385,20 @@ def main():
     # ---- whole-step timing: one captured graph per buffer set ---------------------
     sweep.run_step(0)
     dev.sync()
-    graphs = [capture(dev, [lambda r=r: sweep.run_step(r)]) for r in range(sweep.R)]
+    if args.no_graph:
+        class _Eager:
+            def __init__(self, r):
+                self.r = r
+
+            def launch(self):
+                sweep.run_step(self.r)
+
+            def destroy(self):
+                pass
+
+        graphs = [_Eager(r) for r in range(sweep.R)]
+    else:
+        graphs = [capture(dev, [lambda r=r: sweep.run_step(r)]) for r in range(sweep.R)]
     for s in range(args.warmup):
         graphs[s % sweep.R].launch()
     dev.sync()
@@ -416,10 +435,10 @@ def main():
         dev.sync()
         dev.free_pool(w)
     if not args.no_extras:
-        out.update(extras(dev, lib, args.kernel_reps))
+        out.update(extras(dev, lib, args.kernel_reps, use_graph=not args.no_graph))
     dev.close()
     if not args.no_lm:
-        out["cfg5_lstm_lm"] = lstm_lm(args.lm_steps)
+        out["cfg5_lstm_lm"] = lstm_lm(args.lm_steps, use_graph=not args.no_graph)
         out["lstm_lm_tokens_per_s"] = out["cfg5_lstm_lm"]["fused_cell_path"]["tokens_per_s"]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(sweep.step_bytes, args.cpu_seconds)
