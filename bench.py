@@ -275,6 +275,16 @@ def extras(dev, lib, reps, use_graph=True):
 
 FP32_MFMA_PEAK_TFLOPS = 157.3
 
+# HBM bytes per launch measured with hardware counters (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, on
+# `bench.py --one-pass`, each scaled by what the same counter reads for the library's 16 MiB copy kernel:
+# x1.9967 and x0.9997); the table is in profiles/cfg2_sweep_hbm_traffic_pmc.txt.  Keyed by bench kernel name.
+MEASURED_TRAFFIC_BYTES = {
+    "tanh_fwd": 33.58e6, "logistic_fwd": 33.60e6, "rectify_fwd": 33.55e6, "tanh_bwd": 67.05e6,
+    "logistic_bwd": 67.04e6, "rectify_bwd": 67.05e6, "cmult_fwd": 50.30e6, "cmult_bwd_arg0": 67.05e6,
+    "cmult_bwd_arg1": 67.05e6, "sum_batches_fwd": 17.06e6 + 2.14e6, "sum_batches_bwd": 33.81e6,
+    "layer_norm_fwd": 33.62e6, "layer_norm_bwd": 69.27e6 + 2.14e6,
+}
+
 
 def lstm_lm(steps, warmup=3, use_graph=True):
     """cfg 5: whole training step of the 2-layer LSTM LM (forward, backward, clip, SGD update), tokens/s."""
@@ -417,7 +427,8 @@ def main():
     table = per_kernel_table(dev, sweep.kernels, sweep.sets, args.kernel_reps, use_graph=not args.no_graph)
     dominant = max(table, key=lambda k: k["us"])
     roofline = {"bound": "hbm", "kernel": dominant["kernel"], "achieved": dominant["GBps"], "peak": HBM_PEAK_GBPS,
-                "unit": "GB/s", "frac": round(dominant["GBps"] / HBM_PEAK_GBPS, 4), "traffic": None,
+                "unit": "GB/s", "frac": round(dominant["GBps"] / HBM_PEAK_GBPS, 4),
+                "traffic": MEASURED_TRAFFIC_BYTES.get(dominant["kernel"]),
                 "algorithmic_bytes_per_launch": dominant["bytes"], "avg_launch_us": dominant["us"]}
     out = {
         "metric": "fused-kernel HBM GB/s (cfg-2 elementwise/reduction sweep, algorithmic bytes / device time)",
