@@ -300,6 +300,7 @@ def lstm_lm(steps, warmup=3, use_graph=True):
                       "clip_threshold": 5.0, "init": "Glorot (lookup: embedding dim only), LSTM biases 0",
                       "ids": "Zipf(1.1)"},
            "tokens_per_step": T * B, "gemm_flop_per_step": flops,
+           "fused_path_schedule": "layers pipelined over two device queues in chunks of 7 timesteps",
            "timed_region": "per step: host->device copy of ids and labels, id sort, forward, backward, "
                            "device-side clipping, update; one HIP-graph replay per step; loss read back after "
                            "the last step"}

@@ -66,6 +66,10 @@ struct dyhip_device {
   void* gemm_ws;   // split-K partial tiles (the analogue of a BLAS handle's workspace)
   size_t gemm_ws_bytes;
   hipEvent_t ev_start, ev_stop;
+  dyhip_device* parent;                // non-null for a forked queue: pools, scalars and allocator belong to the parent
+  std::vector<hipEvent_t> sync_events; // ring of events recorded on this queue for dyhip_device_wait
+  size_t sync_next;
+  std::vector<dyhip_device*> forks;    // live forked queues (destroyed with the device if still alive)
 };
 
 struct dyhip_graph {

@@ -247,6 +247,8 @@ int dyhip_device_create(int ordinal, const size_t pool_mb[4], dyhip_device** out
   hipDeviceProp_t prop;
   DYHIP_CHECK_HIP(hipGetDeviceProperties(&prop, ordinal));
   dyhip_device* dev = new dyhip_device();
+  dev->parent = nullptr;
+  dev->sync_next = 0;
   dev->ordinal = ordinal;
   dev->num_cus = prop.multiProcessorCount;
   for (auto& p : dev->pools) p = nullptr;
@@ -290,10 +292,76 @@ int dyhip_device_create(int ordinal, const size_t pool_mb[4], dyhip_device** out
   return DYHIP_OK;
 }
 
+int dyhip_device_fork(dyhip_device* parent, dyhip_device** out) {
+  DYHIP_CHECK_DEV(parent);
+  DYHIP_REQUIRE(out != nullptr, "null output pointer");
+  DYHIP_REQUIRE(parent->parent == nullptr, "fork the device itself, not one of its forked queues");
+  DYHIP_CHECK_HIP(hipSetDevice(parent->ordinal));
+  dyhip_device* dev = new dyhip_device(*parent);  // shares pools, scalars, allocator, thresholds
+  dev->parent = parent;
+  dev->sync_events.clear();
+  dev->forks.clear();
+  dev->sync_next = 0;
+  dev->gemm_ws = nullptr;
+  hipError_t e = hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking);
+  if (e != hipSuccess) {
+    delete dev;
+    return fail(DYHIP_ERR_RUNTIME, "hipStreamCreateWithFlags failed: %s", hipGetErrorString(e));
+  }
+  (void)hipEventCreate(&dev->ev_start);
+  (void)hipEventCreate(&dev->ev_stop);
+  dev->gemm_ws = parent->alloc->malloc(dev->gemm_ws_bytes);
+  if (dev->gemm_ws == nullptr) {
+    dyhip_device_destroy(dev);
+    return fail(DYHIP_ERR_OUT_OF_MEMORY, "failed to allocate the GEMM split-K workspace of the forked queue");
+  }
+  parent->forks.push_back(dev);
+  *out = dev;
+  return DYHIP_OK;
+}
+
+int dyhip_device_wait(dyhip_device* dev, dyhip_device* other) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_CHECK_DEV(other);
+  DYHIP_REQUIRE(dev->ordinal == other->ordinal, "both queues must belong to the same GPU");
+  if (dev == other) return DYHIP_OK;
+  // a wait refers to the event's latest record at the time of the call, so a small ring of
+  // events per queue serves any number of waits (eager or captured)
+  constexpr size_t kRing = 16;
+  if (other->sync_events.size() < kRing) {
+    hipEvent_t fresh;
+    DYHIP_CHECK_HIP(hipEventCreateWithFlags(&fresh, hipEventDisableTiming));
+    other->sync_events.push_back(fresh);
+    other->sync_next = other->sync_events.size() - 1;
+  } else {
+    other->sync_next = (other->sync_next + 1) % kRing;
+  }
+  hipEvent_t ev = other->sync_events[other->sync_next];
+  DYHIP_CHECK_HIP(hipEventRecord(ev, other->stream));
+  DYHIP_CHECK_HIP(hipStreamWaitEvent(dev->stream, ev, 0));
+  return DYHIP_OK;
+}
+
 int dyhip_device_destroy(dyhip_device* dev) {
   DYHIP_CHECK_DEV(dev);
   (void)hipSetDevice(dev->ordinal);
   (void)hipStreamSynchronize(dev->stream);
+  for (hipEvent_t ev : dev->sync_events) (void)hipEventDestroy(ev);
+  if (dev->parent != nullptr) {  // a forked queue owns its stream, events and split-K workspace only
+    auto& fl = dev->parent->forks;
+    for (size_t i = 0; i < fl.size(); ++i)
+      if (fl[i] == dev) {
+        fl.erase(fl.begin() + i);
+        break;
+      }
+    if (dev->gemm_ws) dev->alloc->free(dev->gemm_ws);
+    (void)hipEventDestroy(dev->ev_start);
+    (void)hipEventDestroy(dev->ev_stop);
+    (void)hipStreamDestroy(dev->stream);
+    delete dev;
+    return DYHIP_OK;
+  }
+  while (!dev->forks.empty()) dyhip_device_destroy(dev->forks.back());
   for (auto& p : dev->pools)
     if (p) pool_delete(p);
   if (dev->scalars) dev->alloc->free(dev->scalars);

@@ -34,9 +34,6 @@
 // gate epilogue.  The fused LSTM cell kernels consume the unreduced slices.
 #include "gemm.h"
 
-#include <cstdio>
-#include <cstdlib>
-
 namespace dyhip {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -404,10 +401,6 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
   const bool must_partial = fused_epi || to_caller;
   GemmPlan plan{N <= 64 ? 1 : 2, 1};
   if (g.ktiles_total > 0) plan = plan_gemm(dev, M, N, g.ktiles_total, ws_bytes / out_bytes, must_partial);
-  if (const char* ov = getenv("DYHIP_GEMM_PLAN_DEBUG")) {
-    int wn_o = 0, s_o = 0;
-    if (sscanf(ov, "%d,%d", &wn_o, &s_o) == 2 && N <= 256) plan = GemmPlan{wn_o, (unsigned)s_o};
-  }
   unsigned splits = plan.splits;
   const size_t tiles_m = cdiv<size_t>(M, kBM), tiles_n = cdiv<size_t>(N, size_t(64) * plan.wn);
   DYHIP_REQUIRE(tiles_m * tiles_n < (size_t(1) << 31), "GEMM too large");

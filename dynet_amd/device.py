@@ -97,8 +97,24 @@ class Device:
         self.handle = h
         self.ordinal = ordinal
 
+    def fork(self):
+        """A second in-order queue on the same GPU (own stream and split-K workspace, shared pools)."""
+        h = _vp(None)
+        _check(cdll.dyhip_device_fork(self.handle, C.byref(h)))
+        q = Device.__new__(Device)
+        q.handle, q.ordinal, q._parent = h, self.ordinal, self
+        self._forks = getattr(self, "_forks", [])
+        self._forks.append(q)
+        return q
+
+    def wait(self, other):
+        """Work issued on this queue from now on runs after what has been issued on ``other`` so far."""
+        _check(cdll.dyhip_device_wait(self.handle, other.handle))
+
     def close(self):
         if self.handle is not None:
+            for q in getattr(self, "_forks", []):
+                q.handle = None  # the library destroys live forked queues with their device
             cdll.dyhip_device_destroy(self.handle)
             self.handle = None
 

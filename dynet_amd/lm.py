@@ -13,7 +13,11 @@ What differs from DyNet's node-at-a-time execution (results agree to fp32 roundi
     gate GEMMs are formed once per layer over the K = T*B columns of all timesteps instead of T times over B;
   * ``path="fused"`` (default) runs layer by layer: one GEMM forms Wx*x for all timesteps, a timestep is then
     the recurrent GEMM Wh*h plus one cell kernel (gates + c + h); backward mirrors it, and dx, dWx, dWh, db are
-    GEMMs/reductions over all timesteps.
+    GEMMs/reductions over all timesteps;
+  * with ``overlap=True`` (default for more than one layer) the fused path cuts the time axis into chunks and
+    runs the layers as a pipeline on one queue per layer: layer l works on chunk k while layer l-1 is already on
+    chunk k+1 (backward: l on chunk k, l+1 on chunk k-1).  A timestep's recurrent GEMM and cell kernel are
+    latency-bound and leave most of the GPU idle; two such chains side by side fill it.
 """
 import numpy as np
 
@@ -24,8 +28,12 @@ from .synth import glorot
 class LstmLM:
     """V-word LM: embedding E, L layers of hidden H, batch B, T timesteps per step."""
 
-    def __init__(self, dev, V, E, H, L, B, T, seed=0, lr=0.1, clip=5.0, time_batched=True, params=None, path="fused"):
+    def __init__(self, dev, V, E, H, L, B, T, seed=0, lr=0.1, clip=5.0, time_batched=True, params=None, path="fused",
+                 overlap=None, chunk=7):
         assert path in ("fused", "nodes")
+        self.overlap = (L > 1) if overlap is None else bool(overlap)
+        self.overlap = self.overlap and path == "fused" and L > 1
+        self.chunk = max(1, int(chunk))
         self.dev, self.V, self.E, self.H, self.L, self.B, self.T = dev, V, E, H, L, B, T
         self.lr, self.clip, self.time_batched, self.path = float(lr), float(clip), bool(time_batched), path
         N = self.N = T * B
@@ -62,8 +70,11 @@ class LstmLM:
         self.de_bytes = dev.pool(DE).used() - self.de_begin
         self.d_pre = [dev.empty((T, B, 4 * H), pool=DE) for _ in range(L)]  # overwritten, never accumulated into
         fb, bb = dev.lstm_cell_workspace(H, B)
-        self.rec_f, self.rec_f_bytes = dev.workspace(fb)
-        self.rec_b, self.rec_b_bytes = dev.workspace(bb)
+        self.rec_f_bytes, self.rec_b_bytes = fb, bb
+        self.rec_f = [dev.workspace(fb)[0] for _ in range(L)]  # one per layer: layers run side by side
+        self.rec_b = [dev.workspace(bb)[0] for _ in range(L)]
+        # queue l runs layer l; queue 0 is the device itself
+        self.queues = [dev] + ([dev.fork() for _ in range(L - 1)] if self.overlap else [])
         self.plan, self.plan_ws, self.plan_ws_bytes = dev.lookup_plan_buffers(N, V)
         self.graph = None
 
@@ -112,21 +123,46 @@ class LstmLM:
         d.pnls_forward_staged(V, N, self.logits, self.aux, self.errs)
         d.sum_batches_forward(1, N, self.errs, self.loss)
 
+    def _chunks(self):
+        return [(k, min(k + self.chunk, self.T)) for k in range(0, self.T, self.chunk)]
+
+    def _cell_steps_forward(self, q, l, t0, t1):
+        H, B = self.H, self.B
+        for t in range(t0, t1):
+            g = self._t(self.gates[l], t, 4 * H)
+            if t > 0:
+                n = q.lstm_recurrent_forward(H, B, self.p[f"Wh{l}"], self._t(self.h[l], t - 1, H), self.rec_f[l],
+                                             self.rec_f_bytes)
+                q.lstm_cell_forward(H, B, g, self.p[f"b{l}"], self.rec_f[l], n, self._t(self.c[l], t - 1, H), g,
+                                    self._t(self.c[l], t, H), self._t(self.h[l], t, H))
+            else:
+                q.lstm_cell_forward(H, B, g, self.p[f"b{l}"], None, 0, None, g, self._t(self.c[l], t, H),
+                                    self._t(self.h[l], t, H))
+
     def _forward_layers_fused(self):
         d, E, H, L, B, T, N = self.dev, self.E, self.H, self.L, self.B, self.T, self.N
-        for l in range(L):
-            x, d_in = (self.h[l - 1], H) if l > 0 else (self.emb, E)
-            d.gemm_nn(4 * H, N, d_in, self.p[f"Wx{l}"], x, 0.0, self.gates[l])  # Wx*x of every timestep
-            for t in range(T):
-                g = self._t(self.gates[l], t, 4 * H)
-                if t > 0:
-                    n = d.lstm_recurrent_forward(H, B, self.p[f"Wh{l}"], self._t(self.h[l], t - 1, H), self.rec_f,
-                                                 self.rec_f_bytes)
-                    d.lstm_cell_forward(H, B, g, self.p[f"b{l}"], self.rec_f, n, self._t(self.c[l], t - 1, H), g,
-                                        self._t(self.c[l], t, H), self._t(self.h[l], t, H))
-                else:
-                    d.lstm_cell_forward(H, B, g, self.p[f"b{l}"], None, 0, None, g, self._t(self.c[l], t, H),
-                                        self._t(self.h[l], t, H))
+        if not self.overlap:
+            for l in range(L):
+                x, d_in = (self.h[l - 1], H) if l > 0 else (self.emb, E)
+                d.gemm_nn(4 * H, N, d_in, self.p[f"Wx{l}"], x, 0.0, self.gates[l])  # Wx*x of every timestep
+                self._cell_steps_forward(d, l, 0, T)
+            return
+        # pipeline over time chunks: queue l runs layer l, one chunk behind queue l-1
+        qs = self.queues
+        d.gemm_nn(4 * H, N, E, self.p["Wx0"], self.emb, 0.0, self.gates[0])
+        for l in range(1, L):
+            qs[l].wait(d)  # joins the capture; nothing of layer l may start before the step does
+        for (t0, t1) in self._chunks():
+            for l in range(L):
+                q = qs[l]
+                if l > 0:
+                    q.wait(qs[l - 1])  # h of the layer below for this chunk
+                    nb = (t1 - t0) * B
+                    q.gemm_nn(4 * H, nb, H, self.p[f"Wx{l}"], self._t(self.h[l - 1], t0, H),
+                              0.0, self._t(self.gates[l], t0, 4 * H))
+                self._cell_steps_forward(q, l, t0, t1)
+        for l in range(1, L):
+            d.wait(qs[l])
 
     def _forward_layers_nodes(self):
         d, E, H, L, B, T = self.dev, self.E, self.H, self.L, self.B, self.T
@@ -158,26 +194,59 @@ class LstmLM:
             self._backward_layers_nodes()
         d.lookup_accumulate_grads_planned(N, self.plan, E, V, self.d_emb, self.g["C"])
 
+    def _cell_steps_backward(self, q, l, t0, t1):
+        """Timesteps t1-1 .. t0 of layer l; the recurrent slices of step t1 (if any) are in rec_b[l]."""
+        H, B, T = self.H, self.B, self.T
+        Wh = self.p[f"Wh{l}"]
+        for t in reversed(range(t0, t1)):
+            last, first = t == T - 1, t == 0
+            dpre = self._t(self.d_pre[l], t, 4 * H)
+            q.lstm_cell_backward(H, B, self._t(self.gates[l], t, 4 * H), self._t(self.c[l], t, H),
+                                 None if first else self._t(self.c[l], t - 1, H), self._t(self.d_h[l], t, H),
+                                 None if last else self.rec_b[l], 0 if last else self._rec_b_n[l],
+                                 None if last else self._t(self.d_c[l], t, H), dpre,
+                                 None if first else self._t(self.d_c[l], t - 1, H))
+            if not first:
+                self._rec_b_n[l] = q.lstm_recurrent_backward(H, B, Wh, dpre, self.rec_b[l], self.rec_b_bytes)
+
+    def _weight_grads(self, q, l):
+        E, H, B, T, N = self.E, self.H, self.B, self.T, self.N
+        x, d_in = (self.h[l - 1], H) if l > 0 else (self.emb, E)
+        q.gemm_nt_acc(4 * H, d_in, N, self.d_pre[l], x, self.g[f"Wx{l}"])
+        if T > 1:
+            q.gemm_nt_acc(4 * H, H, N - B, self._t(self.d_pre[l], 1, 4 * H), self.h[l], self.g[f"Wh{l}"])
+        q.csum_backward(4 * H, 1, N, self.d_pre[l], 0, self.g[f"b{l}"])
+
     def _backward_layers_fused(self):
         d, E, H, L, B, T, N = self.dev, self.E, self.H, self.L, self.B, self.T, self.N
+        self._rec_b_n = [0] * L
+        if not self.overlap:
+            for l in reversed(range(L)):
+                self._cell_steps_backward(d, l, 0, T)
+                d_in, dx = (H, self.d_h[l - 1]) if l > 0 else (E, self.d_emb)
+                d.gemm_tn(d_in, N, 4 * H, self.p[f"Wx{l}"], self.d_pre[l], 0.0, dx)
+                self._weight_grads(d, l)
+            return
+        # pipeline, newest chunk first: the top layer runs on the device queue (it owns d_h[L-1]),
+        # layer l on queue L-1-l, one chunk behind the layer above
+        qs = self.queues
+        qof = lambda l: qs[L - 1 - l]
+        for l in range(L - 1):
+            qof(l).wait(d)
+        for (t0, t1) in reversed(self._chunks()):
+            for l in reversed(range(L)):
+                q = qof(l)
+                if l < L - 1:
+                    q.wait(qof(l + 1))  # d_h[l] of this chunk
+                self._cell_steps_backward(q, l, t0, t1)
+                nb = (t1 - t0) * B
+                d_in, dx = (H, self.d_h[l - 1]) if l > 0 else (E, self.d_emb)
+                q.gemm_tn(d_in, nb, 4 * H, self.p[f"Wx{l}"], self._t(self.d_pre[l], t0, 4 * H), 0.0,
+                          self._t(dx, t0, d_in))
         for l in reversed(range(L)):
-            Wh = self.p[f"Wh{l}"]
-            n = 0
-            for t in reversed(range(T)):
-                last, first = t == T - 1, t == 0
-                dpre = self._t(self.d_pre[l], t, 4 * H)
-                d.lstm_cell_backward(H, B, self._t(self.gates[l], t, 4 * H), self._t(self.c[l], t, H),
-                                     None if first else self._t(self.c[l], t - 1, H), self._t(self.d_h[l], t, H),
-                                     None if last else self.rec_b, n, None if last else self._t(self.d_c[l], t, H),
-                                     dpre, None if first else self._t(self.d_c[l], t - 1, H))
-                if not first:
-                    n = d.lstm_recurrent_backward(H, B, Wh, dpre, self.rec_b, self.rec_b_bytes)
-            x, d_in, dx = (self.h[l - 1], H, self.d_h[l - 1]) if l > 0 else (self.emb, E, self.d_emb)
-            d.gemm_tn(d_in, N, 4 * H, self.p[f"Wx{l}"], self.d_pre[l], 0.0, dx)
-            d.gemm_nt_acc(4 * H, d_in, N, self.d_pre[l], x, self.g[f"Wx{l}"])
-            if T > 1:
-                d.gemm_nt_acc(4 * H, H, N - B, self._t(self.d_pre[l], 1, 4 * H), self.h[l], self.g[f"Wh{l}"])
-            d.csum_backward(4 * H, 1, N, self.d_pre[l], 0, self.g[f"b{l}"])
+            self._weight_grads(qof(l), l)  # each on its own queue, side by side with the layers still running
+        for l in range(L - 1):
+            d.wait(qof(l))
 
     def _backward_layers_nodes(self):
         d, E, H, L, B, T, N = self.dev, self.E, self.H, self.L, self.B, self.T, self.N

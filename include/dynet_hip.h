@@ -61,6 +61,16 @@ int dyhip_device_ordinal(const dyhip_device* dev, int* ordinal);
 int dyhip_device_stream(dyhip_device* dev, void** hip_stream);
 int dyhip_device_pool(dyhip_device* dev, int which, dyhip_pool** pool);
 int dyhip_device_scalar(dyhip_device* dev, int which, const float** ptr);
+/* A second in-order queue on the same GPU: shares the pools, scalars and settings of
+ * `parent`, has its own HIP stream (default priority) and split-K workspace.  Work issued
+ * on the two handles may overlap on the GPU; dyhip_device_wait orders it: everything
+ * issued on `dev` afterwards runs after everything issued on `other` before the call.
+ * Both calls are legal inside a graph capture begun on the parent (the forked queue joins
+ * the capture with its first wait and must be waited for before the capture ends).
+ * Destroy forked queues before their parent.  No counterpart in the reference, which
+ * issues everything on the null stream. */
+int dyhip_device_fork(dyhip_device* parent, dyhip_device** out);
+int dyhip_device_wait(dyhip_device* dev, dyhip_device* other);
 /* Tensors of at least this many bytes are streamed with non-temporal accesses
  * (default 8 MiB, twice the per-XCD L2); 0 streams everything, SIZE_MAX nothing.
  * A tuning knob with no counterpart in the reference. */

@@ -28,16 +28,18 @@ def _grad_floor(ref):
     return max(float(np.abs(ref).max()) * 1e-2, 1e-6)
 
 
-@pytest.mark.parametrize("path,time_batched", [("nodes", False), ("nodes", True), ("fused", True)])
+@pytest.mark.parametrize("path,time_batched,overlap", [("nodes", False, False), ("nodes", True, False),
+                                                       ("fused", True, False), ("fused", True, True)])
 @pytest.mark.parametrize("case", CASES)
-def test_lm_step_matches_oracle(dev, case, path, time_batched):
+def test_lm_step_matches_oracle(dev, case, path, time_batched, overlap):
     V, E, H, L, B, T = case
     rng = np.random.default_rng(11)
     params = LstmLM.init_params(V, E, H, L, seed=3)
     for l in range(L):  # non-zero biases exercise the bias path
         params[f"b{l}"] = rng.normal(0, 0.1, 4 * H).astype(np.float32)
     ref_p = {n: a.copy() for n, a in params.items()}
-    lm = LstmLM(dev, V, E, H, L, B, T, lr=0.1, clip=5.0, time_batched=time_batched, params=params, path=path)
+    lm = LstmLM(dev, V, E, H, L, B, T, lr=0.1, clip=5.0, time_batched=time_batched, params=params, path=path,
+                overlap=overlap, chunk=2)
     for it in range(2):
         tokens = _tokens(rng, V, B, T)
         ref_loss, ref_g, ref_scale = lm_oracle.step(ref_p, tokens, L, lr=0.1, clip=5.0)
@@ -80,12 +82,13 @@ def test_lm_clipping_engages(dev):
 
 
 def test_lm_graph_replay_matches_eager(dev):
-    """The captured step, replayed with fresh tokens each time, follows the eager trajectory bit for bit."""
+    """The captured step (layers pipelined over two queues), replayed with fresh tokens each time, follows the
+    eagerly issued one bit for bit: same kernels, same data, same order within each queue."""
     V, E, H, L, B, T = 120, 32, 64, 2, 16, 6
     rng = np.random.default_rng(7)
     params = LstmLM.init_params(V, E, H, L, seed=2)
-    eager = LstmLM(dev, V, E, H, L, B, T, params=params)
-    graphed = LstmLM(dev, V, E, H, L, B, T, params=params)
+    eager = LstmLM(dev, V, E, H, L, B, T, params=params, overlap=True, chunk=2)
+    graphed = LstmLM(dev, V, E, H, L, B, T, params=params, overlap=True, chunk=2)
     batches = [_tokens(rng, V, B, T) for _ in range(4)]
     graphed.stage(batches[0])
     graphed.capture()
