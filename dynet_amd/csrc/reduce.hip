@@ -108,7 +108,7 @@ __global__ __launch_bounds__(64 * kBrWaves) void batch_reduce_kernel(size_t n, u
 }
 
 // out[j] (+)= sum_s partial[s*n + j].  Block = 64 columns x kCombSlices slices:
-// slice q adds splits q, q+16, ... in ascending order with four loads in flight,
+// slice q adds splits q, q+16, ... in ascending order with up to sixteen loads in flight,
 // then the slices are added in ascending q.  blockIdx.y selects one of two
 // (partial, out) pairs so that two outputs share a launch.
 constexpr int kCombSlices = 16;
@@ -126,6 +126,14 @@ __global__ __launch_bounds__(64 * kCombSlices) void combine_partials_kernel(size
   float acc = 0.f;
   if (j < n) {
     unsigned sp = q;
+    constexpr int U = 16;  // loads in flight per thread
+    for (; sp + (U - 1) * kCombSlices < splits; sp += U * kCombSlices) {
+      float a[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) a[u] = partial[size_t(sp + u * kCombSlices) * n + j];
+#pragma unroll
+      for (int u = 0; u < U; ++u) acc += a[u];
+    }
     for (; sp + 3 * kCombSlices < splits; sp += 4 * kCombSlices) {
       const float a0 = partial[size_t(sp) * n + j], a1 = partial[size_t(sp + kCombSlices) * n + j],
                   a2 = partial[size_t(sp + 2 * kCombSlices) * n + j],
