@@ -83,7 +83,8 @@ __global__ __launch_bounds__(kLkThreads) void lookup_gather_kernel(unsigned n_id
 struct ScatterWs {
   unsigned* sorted_ids;
   unsigned* sorted_pos;
-  unsigned* last_row;    // per chunk: row of a run that begins here and continues into the next chunk, else kNone
+  unsigned* run_last;    // per chunk (part of the plan): last chunk of the run that begins here and continues
+                         // into the next chunk, else kNone
   float* part_first;     // [chunks][dim]
   float* part_last;      // [chunks][dim]
   unsigned chunks;
@@ -108,10 +109,8 @@ __global__ __launch_bounds__(kLkThreads) void scatter_chunk_kernel(unsigned n, u
   const unsigned prev_id = k0 > 0 ? w.sorted_ids[k0 - 1] : kNone;
   const unsigned next_id = k0 + cnt < n ? w.sorted_ids[k0 + cnt] : kNone;
   const unsigned first = id[0], last = id[cnt - 1];
-  const bool single = first == last;
   const bool open_left = prev_id == first;
   const bool open_right = next_id == last;
-  if (t == 0) w.last_row[ch] = (open_right && !(single && open_left)) ? last : kNone;
   V* part_first = reinterpret_cast<V*>(w.part_first) + size_t(ch) * dimv;
   V* part_last = reinterpret_cast<V*>(w.part_last) + size_t(ch) * dimv;
   // run_end[k]: entry k is the last of its run inside this chunk; direct[k]: that run
@@ -153,13 +152,14 @@ __global__ __launch_bounds__(kLkThreads) void scatter_chunk_kernel(unsigned n, u
   }
 }
 
-// One block per chunk in which a boundary-crossing run starts.  The end of the run
-// is found by binary search in the sorted ids; the run's partial rows (one per chunk
+// One block per chunk in which a boundary-crossing run starts.  The chunk where the run
+// ends comes from the plan; the run's partial rows (one per chunk
 // it touches) are split over kFixSlices thread slices that each add every
 // kFixSlices-th partial in ascending order with four loads in flight, and the slices
 // are then added in ascending order: deterministic, and a run of thousands of
 // entries costs a handful of memory round trips instead of one per partial.
 constexpr int kFixThreads = 1024;
+constexpr int kFixChunks = 1;  // chunks examined per block (runs are independent: one block each keeps them parallel)
 
 template <class V>
 __global__ __launch_bounds__(kFixThreads) void scatter_fixup_kernel(unsigned n, unsigned dimv, unsigned tpr,
@@ -167,44 +167,49 @@ __global__ __launch_bounds__(kFixThreads) void scatter_fixup_kernel(unsigned n, 
                                                                     V* __restrict__ grads) {
   extern __shared__ __attribute__((aligned(16))) char fix_lds_raw[];
   V* lds = reinterpret_cast<V*>(fix_lds_raw);
-  const unsigned c0 = blockIdx.x;
-  const unsigned row = w.last_row[c0];
-  if (row == kNone || row >= vocab) return;  // uniform over the block
-  // first position after the run: upper bound of `row` in sorted_ids[(c0+1)*kChunk, n)
-  unsigned lo = (c0 + 1) * kChunk, hi = n;
-  while (lo < hi) {
-    const unsigned mid = lo + (hi - lo) / 2;
-    if (w.sorted_ids[mid] <= row) lo = mid + 1;
-    else hi = mid;
-  }
-  const unsigned c_last = (lo - 1) / kChunk;  // last chunk holding entries of the run
   const unsigned slices = kFixThreads / tpr;
   const unsigned q = threadIdx.x / tpr, t = threadIdx.x - q * tpr;
-  const V* pl = reinterpret_cast<const V*>(w.part_last) + size_t(c0) * dimv;
   const V* pf = reinterpret_cast<const V*>(w.part_first);
-  for (unsigned cb = 0; cb < dimv; cb += tpr) {
-    const unsigned c = cb + t;
-    V acc = vzero<V>();
-    if (c < dimv) {
-      // partial index p = 0 is part_last[c0]; p >= 1 is part_first[c0 + p]
-      const unsigned np = c_last - c0 + 1;
-      unsigned p = q;
-      for (; p + 3 * slices < np; p += 4 * slices) {
-        const V a0 = p == 0 ? pl[c] : pf[size_t(c0 + p) * dimv + c];
-        const V a1 = pf[size_t(c0 + p + slices) * dimv + c];
-        const V a2 = pf[size_t(c0 + p + 2 * slices) * dimv + c];
-        const V a3 = pf[size_t(c0 + p + 3 * slices) * dimv + c];
-        acc = vadd(vadd(vadd(vadd(acc, a0), a1), a2), a3);
+  // each block looks at kFixChunks consecutive chunks; few of them start a boundary-crossing run
+  const unsigned c_begin = blockIdx.x * kFixChunks, c_end = min(w.chunks, c_begin + kFixChunks);
+  __shared__ unsigned c_lasts[kFixChunks], rows[kFixChunks];
+  if (threadIdx.x < kFixChunks) {
+    const unsigned c = c_begin + threadIdx.x;
+    c_lasts[threadIdx.x] = c < c_end ? w.run_last[c] : kNone;
+    rows[threadIdx.x] = c < c_end ? w.sorted_ids[min(n, (c + 1) * kChunk) - 1] : kNone;
+  }
+  __syncthreads();
+  for (int i = 0; i < kFixChunks; ++i) {
+    const unsigned c0 = c_begin + i;
+    const unsigned c_last = c_lasts[i];  // last chunk holding entries of the run
+    if (c_last == kNone) continue;       // uniform over the block
+    const unsigned row = rows[i];
+    if (row >= vocab) continue;
+    const V* pl = reinterpret_cast<const V*>(w.part_last) + size_t(c0) * dimv;
+    for (unsigned cb = 0; cb < dimv; cb += tpr) {
+      const unsigned c = cb + t;
+      V acc = vzero<V>();
+      if (c < dimv) {
+        // partial index p = 0 is part_last[c0]; p >= 1 is part_first[c0 + p]
+        const unsigned np = c_last - c0 + 1;
+        unsigned p = q;
+        for (; p + 3 * slices < np; p += 4 * slices) {
+          const V a0 = p == 0 ? pl[c] : pf[size_t(c0 + p) * dimv + c];
+          const V a1 = pf[size_t(c0 + p + slices) * dimv + c];
+          const V a2 = pf[size_t(c0 + p + 2 * slices) * dimv + c];
+          const V a3 = pf[size_t(c0 + p + 3 * slices) * dimv + c];
+          acc = vadd(vadd(vadd(vadd(acc, a0), a1), a2), a3);
+        }
+        for (; p < np; p += slices) acc = vadd(acc, p == 0 ? pl[c] : pf[size_t(c0 + p) * dimv + c]);
       }
-      for (; p < np; p += slices) acc = vadd(acc, p == 0 ? pl[c] : pf[size_t(c0 + p) * dimv + c]);
-    }
-    __syncthreads();
-    lds[q * tpr + t] = acc;
-    __syncthreads();
-    if (q == 0 && c < dimv) {
-      V tot = lds[t];
-      for (unsigned k = 1; k < slices; ++k) tot = vadd(tot, lds[k * tpr + t]);
-      grads[size_t(row) * dimv + c] = vadd(grads[size_t(row) * dimv + c], tot);
+      __syncthreads();
+      lds[q * tpr + t] = acc;
+      __syncthreads();
+      if (q == 0 && c < dimv) {
+        V tot = lds[t];
+        for (unsigned k = 1; k < slices; ++k) tot = vadd(tot, lds[k * tpr + t]);
+        grads[size_t(row) * dimv + c] = vadd(grads[size_t(row) * dimv + c], tot);
+      }
     }
   }
 }
@@ -233,13 +238,41 @@ static int sort_tmp_bytes(unsigned n, unsigned vocab, size_t* bytes) {
   return DYHIP_OK;
 }
 
-// plan = [sorted_ids (n u32) | sorted_pos (n u32)], each part padded to 256 bytes
-static size_t plan_bytes(unsigned n) { return 2 * align256(sizeof(unsigned) * n); }
+// Per chunk of the sorted ids: does a run start here (not continuing from the previous chunk,
+// or filling this chunk only partly) and continue into the next chunk?  If so, in which chunk
+// does it end (binary search for the upper bound of its id)?  Part of the plan, so the search
+// is paid when the plan is built, not in the backward pass.
+__global__ __launch_bounds__(256) void plan_runs_kernel(unsigned n, unsigned chunks,
+                                                        const unsigned* __restrict__ sorted_ids,
+                                                        unsigned* __restrict__ run_last) {
+  const unsigned ch = blockIdx.x * 256 + threadIdx.x;
+  if (ch >= chunks) return;
+  const unsigned k0 = ch * kChunk, cnt = min(n - k0, (unsigned)kChunk);
+  const unsigned first = sorted_ids[k0], last = sorted_ids[k0 + cnt - 1];
+  const bool open_left = k0 > 0 && sorted_ids[k0 - 1] == first;
+  const bool open_right = k0 + cnt < n && sorted_ids[k0 + cnt] == last;
+  unsigned out = kNone;
+  if (open_right && !(first == last && open_left)) {
+    unsigned lo = k0 + cnt, hi = n;
+    while (lo < hi) {
+      const unsigned mid = lo + (hi - lo) / 2;
+      if (sorted_ids[mid] <= last) lo = mid + 1;
+      else hi = mid;
+    }
+    out = (lo - 1) / kChunk;
+  }
+  run_last[ch] = out;
+}
 
-// scratch of the reduction kernels = [last_row | part_first | part_last]
+// plan = [sorted_ids (n u32) | sorted_pos (n u32) | run_last (chunks u32)], each part padded to 256 bytes
+static size_t plan_bytes(unsigned n) {
+  return 2 * align256(sizeof(unsigned) * n) + align256(sizeof(unsigned) * cdiv<unsigned>(n, kChunk));
+}
+
+// scratch of the reduction kernels = [part_first | part_last]
 static size_t reduce_ws_bytes(unsigned n, size_t dim) {
   const unsigned chunks = cdiv<unsigned>(n, kChunk);
-  return align256(sizeof(unsigned) * chunks) + 2 * align256(sizeof(float) * dim * chunks);
+  return 2 * align256(sizeof(float) * dim * chunks);
 }
 
 static int build_plan(dyhip_device* dev, unsigned n, const unsigned* ids_dev, unsigned vocab, void* plan,
@@ -255,6 +288,11 @@ static int build_plan(dyhip_device* dev, unsigned n, const unsigned* ids_dev, un
   DYHIP_CHECK_HIP(rocprim::radix_sort_pairs(ws, sort_bytes, ids_dev, sorted_ids,
                                             rocprim::counting_iterator<unsigned>(0), sorted_pos, n, 0, key_bits(vocab),
                                             dev->stream));
+  unsigned* run_last = reinterpret_cast<unsigned*>(static_cast<char*>(plan) + 2 * align256(sizeof(unsigned) * n));
+  const unsigned chunks = cdiv<unsigned>(n, kChunk);
+  hipLaunchKernelGGL(plan_runs_kernel, dim3(cdiv<unsigned>(chunks, 256)), dim3(256), 0, dev->stream, n, chunks,
+                     sorted_ids, run_last);
+  DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
 
@@ -268,16 +306,16 @@ static int reduce_planned(dyhip_device* dev, unsigned n, const void* plan, size_
   w.sorted_ids = const_cast<unsigned*>(static_cast<const unsigned*>(plan));
   w.sorted_pos = reinterpret_cast<unsigned*>(const_cast<char*>(static_cast<const char*>(plan)) +
                                              align256(sizeof(unsigned) * n));
+  w.run_last = reinterpret_cast<unsigned*>(const_cast<char*>(static_cast<const char*>(plan)) +
+                                           2 * align256(sizeof(unsigned) * n));
   char* base = static_cast<char*>(ws);
-  w.last_row = reinterpret_cast<unsigned*>(base);
-  w.part_first = reinterpret_cast<float*>(base + align256(sizeof(unsigned) * w.chunks));
-  w.part_last = reinterpret_cast<float*>(base + align256(sizeof(unsigned) * w.chunks) +
-                                         align256(sizeof(float) * dim * w.chunks));
+  w.part_first = reinterpret_cast<float*>(base);
+  w.part_last = reinterpret_cast<float*>(base + align256(sizeof(float) * dim * w.chunks));
   const bool vec = dim % 4 == 0 && aligned16(g) && aligned16(all_grads);
   const unsigned dimv = static_cast<unsigned>(vec ? dim / 4 : dim);
   const unsigned tpr = threads_per_row(dimv);
   const dim3 grid(cdiv<unsigned>(w.chunks, kLkThreads / tpr)), block(kLkThreads);
-  const dim3 fgrid(w.chunks), fblock(kFixThreads);
+  const dim3 fgrid(cdiv<unsigned>(w.chunks, kFixChunks)), fblock(kFixThreads);
   const size_t flds = size_t(kFixThreads) * (vec ? sizeof(float4) : sizeof(float));
   const bool stream = size_t(n) * dim * sizeof(float) >= dev->stream_threshold;
   if (vec) {
