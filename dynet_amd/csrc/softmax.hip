@@ -285,6 +285,61 @@ static int launch_lse(dyhip_device* dev, size_t rows, unsigned bd, const float* 
   return DYHIP_OK;
 }
 
+// ---- Softmax / LogSoftmax over dim 0 ---------------------------------------------------
+// Column statistics come from lse_cols_kernel (forward) or col_dot_kernel (backward); the
+// element pass is one kernel over (column, tile) with the column's scalars read once per block.
+constexpr int kSmThreads = 256;
+constexpr int kSmUnroll = 4;
+
+// red[c] = sum_i a[i,c] * (b ? b[i,c] : 1), one block per column, fixed summation tree
+__global__ __launch_bounds__(kSmThreads) void col_dot_kernel(size_t rows, const float* __restrict__ a,
+                                                            const float* __restrict__ b, float* __restrict__ red) {
+  __shared__ float sh[kSmThreads / 64];
+  const size_t c0 = size_t(blockIdx.x) * rows;
+  float s = 0.f;
+  for (size_t i = threadIdx.x; i < rows; i += kSmThreads) s += b ? a[c0 + i] * b[c0 + i] : a[c0 + i];
+  const float t = block_sum<kSmThreads / 64>(s, sh);
+  if (threadIdx.x == 0) red[blockIdx.x] = t;
+}
+
+// MODE 0: fx = exp(x - m) * exp(m - z)         softmax forward   (s0 = m, s1 = z = log sum exp)
+// MODE 1: fx = x - z                            log-softmax forward (s0 = z)
+// MODE 2: dx += (d - r) * f                     softmax backward  (a = fx, b = dEdf, s0 = r = sum fx*dEdf)
+// MODE 3: dx += exp(f) * -r + d                 log-softmax backward (a = fx, b = dEdf, s0 = r = sum dEdf)
+template <int MODE>
+__global__ __launch_bounds__(kSmThreads) void col_apply_kernel(size_t rows, unsigned tiles_per_col,
+                                                              const float* __restrict__ a,
+                                                              const float* __restrict__ b,
+                                                              const float* __restrict__ s0,
+                                                              const float* __restrict__ s1, float* __restrict__ out) {
+  const unsigned c = blockIdx.x / tiles_per_col, tile = blockIdx.x - c * tiles_per_col;
+  const size_t c0 = size_t(c) * rows;
+  const float p0 = s0[c];
+  const float p1 = MODE == 0 ? expf(p0 - s1[c]) : 0.f;
+  const size_t i0 = size_t(tile) * kSmThreads * kSmUnroll + threadIdx.x;
+#pragma unroll
+  for (int u = 0; u < kSmUnroll; ++u) {
+    const size_t i = i0 + size_t(u) * kSmThreads;
+    if (i >= rows) break;
+    const size_t e = c0 + i;
+    if (MODE == 0) out[e] = expf(a[e] - p0) * p1;
+    else if (MODE == 1) out[e] = a[e] - p0;
+    else if (MODE == 2) out[e] += (b[e] - p0) * a[e];
+    else out[e] += (expf(a[e]) * -p0) + b[e];
+  }
+}
+
+template <int MODE>
+static int launch_col_apply(dyhip_device* dev, size_t rows, unsigned cols, const float* a, const float* b,
+                            const float* s0, const float* s1, float* out) {
+  const size_t tiles = cdiv<size_t>(rows, size_t(kSmThreads) * kSmUnroll);
+  DYHIP_REQUIRE(tiles * cols < (size_t(1) << 31), "softmax launch too large");
+  hipLaunchKernelGGL(col_apply_kernel<MODE>, dim3(static_cast<unsigned>(tiles * cols)), dim3(kSmThreads), 0, dev->stream,
+                     rows, static_cast<unsigned>(tiles), a, b, s0, s1, out);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
 }  // namespace dyhip
 
 using namespace dyhip;
@@ -406,6 +461,53 @@ int dyhip_argmax_cols(dyhip_device* dev, size_t rows, unsigned bd, const float* 
   hipLaunchKernelGGL(argmax_cols_kernel, dim3(bd), dim3(256), 0, dev->stream, rows, x, idx);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
+}
+
+int dyhip_softmax_forward(dyhip_device* dev, size_t rows, unsigned cols, const float* x, float* fx, void* ws,
+                          size_t ws_bytes) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(rows >= 1 && x && fx, "Softmax needs non-empty tensors");
+  if (cols == 0) return DYHIP_OK;
+  DYHIP_REQUIRE(ws != nullptr && ws_bytes >= 2 * sizeof(float) * cols, "Softmax needs %zu workspace bytes, got %zu",
+                2 * sizeof(float) * cols, ws_bytes);
+  float* z = static_cast<float*>(ws);
+  float* m = z + cols;
+  DYHIP_CHECK_STATUS(launch_lse(dev, rows, cols, x, m, z, nullptr, nullptr));
+  return launch_col_apply<0>(dev, rows, cols, x, nullptr, m, z, fx);
+}
+
+int dyhip_softmax_backward(dyhip_device* dev, size_t rows, unsigned cols, const float* fx, const float* dEdf,
+                           float* dEdx, void* ws, size_t ws_bytes) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(rows >= 1 && fx && dEdf && dEdx, "Softmax needs non-empty tensors");
+  if (cols == 0) return DYHIP_OK;
+  DYHIP_REQUIRE(ws != nullptr && ws_bytes >= sizeof(float) * cols, "Softmax backward needs %zu workspace bytes, got %zu",
+                sizeof(float) * cols, ws_bytes);
+  float* r = static_cast<float*>(ws);
+  hipLaunchKernelGGL(col_dot_kernel, dim3(cols), dim3(kSmThreads), 0, dev->stream, rows, fx, dEdf, r);
+  DYHIP_CHECK_LAUNCH();
+  return launch_col_apply<2>(dev, rows, cols, fx, dEdf, r, nullptr, dEdx);
+}
+
+int dyhip_log_softmax_forward(dyhip_device* dev, size_t rows, unsigned cols, const float* x, void* aux, float* fx) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(rows >= 1 && x && aux && fx, "LogSoftmax needs non-empty tensors");
+  if (cols == 0) return DYHIP_OK;
+  float* z = static_cast<float*>(aux);
+  float* m = z + cols;
+  DYHIP_CHECK_STATUS(launch_lse(dev, rows, cols, x, m, z, nullptr, nullptr));
+  return launch_col_apply<1>(dev, rows, cols, x, nullptr, z, nullptr, fx);
+}
+
+int dyhip_log_softmax_backward(dyhip_device* dev, size_t rows, unsigned cols, const float* fx, const float* dEdf,
+                               void* aux, float* dEdx) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(rows >= 1 && fx && dEdf && aux && dEdx, "LogSoftmax needs non-empty tensors");
+  if (cols == 0) return DYHIP_OK;
+  float* r = static_cast<float*>(aux);  // the reference overwrites z in aux_mem with the column sums of dEdf
+  hipLaunchKernelGGL(col_dot_kernel, dim3(cols), dim3(kSmThreads), 0, dev->stream, rows, dEdf, nullptr, r);
+  DYHIP_CHECK_LAUNCH();
+  return launch_col_apply<3>(dev, rows, cols, fx, dEdf, r, nullptr, dEdx);
 }
 
 }  // extern "C"

@@ -429,6 +429,21 @@ class Device:
     def pnls_backward(self, rows, bd, x, aux, dEdf, dEdx):
         _check(cdll.dyhip_pnls_backward(self.handle, _sz(rows), _u(bd), _p(x), _p(aux), _p(dEdf), _p(dEdx)))
 
+    def softmax_forward(self, rows, cols, x, fx):
+        ws, nb = self.workspace(8 * cols)
+        _check(cdll.dyhip_softmax_forward(self.handle, _sz(rows), _u(cols), _p(x), _p(fx), _vp(ws), _sz(nb)))
+
+    def softmax_backward(self, rows, cols, fx, dEdf, dEdx):
+        ws, nb = self.workspace(4 * cols)
+        _check(cdll.dyhip_softmax_backward(self.handle, _sz(rows), _u(cols), _p(fx), _p(dEdf), _p(dEdx), _vp(ws),
+                                           _sz(nb)))
+
+    def log_softmax_forward(self, rows, cols, x, aux, fx):
+        _check(cdll.dyhip_log_softmax_forward(self.handle, _sz(rows), _u(cols), _p(x), _p(aux), _p(fx)))
+
+    def log_softmax_backward(self, rows, cols, fx, dEdf, aux, dEdx):
+        _check(cdll.dyhip_log_softmax_backward(self.handle, _sz(rows), _u(cols), _p(fx), _p(dEdf), _p(aux), _p(dEdx)))
+
     def logsumexp_node_forward(self, n, bd, xs, bds, fx):
         ptrs, b = self._xs(xs, bds)
         _check(cdll.dyhip_logsumexp_node_forward(self.handle, _u(len(xs)), _sz(n), _u(bd), ptrs, b, _p(fx)))

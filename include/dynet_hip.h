@@ -284,6 +284,18 @@ int dyhip_pnls_forward(dyhip_device* dev, size_t rows, unsigned bd, const float*
 int dyhip_pnls_forward_staged(dyhip_device* dev, size_t rows, unsigned bd, const float* x, void* aux, float* fx);
 int dyhip_pnls_backward(dyhip_device* dev, size_t rows, unsigned bd, const float* x, const void* aux,
                         const float* dEdf, float* dEdx);
+/* Softmax over dim 0 (dynet/nodes-softmaxes.cc:40-87 forward, :89-125 backward): x is rows x cols
+ * with cols = columns x batch.  Forward needs 2*cols floats of scratch (the reference's z and m from
+ * pools[SCS], :45-48), backward cols floats (:97-98).  Softmax along dim 1 is not provided. */
+int dyhip_softmax_forward(dyhip_device* dev, size_t rows, unsigned cols, const float* x, float* fx, void* ws,
+                          size_t ws_bytes);
+int dyhip_softmax_backward(dyhip_device* dev, size_t rows, unsigned cols, const float* fx, const float* dEdf,
+                           float* dEdx, void* ws, size_t ws_bytes);
+/* LogSoftmax (dynet/nodes-softmaxes.cc:141-185 forward, :187-213 backward).  aux = the node's aux_mem,
+ * 2*cols floats [z | m] (:136-138); backward overwrites z with the column sums of dEdf, as the reference does. */
+int dyhip_log_softmax_forward(dyhip_device* dev, size_t rows, unsigned cols, const float* x, void* aux, float* fx);
+int dyhip_log_softmax_backward(dyhip_device* dev, size_t rows, unsigned cols, const float* fx, const float* dEdf,
+                               void* aux, float* dEdx);
 /* LogSumExp node over k <= 8 arguments (dynet/nodes-logsumexp.cc:38-97) */
 int dyhip_logsumexp_node_forward(dyhip_device* dev, unsigned k, size_t n, unsigned bd, const float* const* xs_host,
                                  const unsigned* bds_host, float* fx);

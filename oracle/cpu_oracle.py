@@ -275,6 +275,33 @@ def logsumexp_cols(rows, bd, x):
     return m, z
 
 
+def softmax_forward(rows, cols, x):
+    fx = np.empty((cols, rows), np.float32)
+    _check(_lib.orc_softmax_forward(C.c_size_t(rows), cols, _fp(_f32(x)), _fp(fx)), "softmax_forward")
+    return fx
+
+
+def softmax_backward(rows, cols, fx, dEdf, dEdx):
+    _check(_lib.orc_softmax_backward(C.c_size_t(rows), cols, _fp(_f32(fx)), _fp(_f32(dEdf)), _fp(dEdx)),
+           "softmax_backward")
+    return dEdx
+
+
+def log_softmax_forward(rows, cols, x):
+    """Returns (fx, aux) with aux = [z | m]."""
+    fx = np.empty((cols, rows), np.float32)
+    aux = np.empty(2 * cols, np.float32)
+    _check(_lib.orc_log_softmax_forward(C.c_size_t(rows), cols, _fp(_f32(x)), _fp(aux), _fp(fx)),
+           "log_softmax_forward")
+    return fx, aux
+
+
+def log_softmax_backward(rows, cols, fx, dEdf, dEdx):
+    _check(_lib.orc_log_softmax_backward(C.c_size_t(rows), cols, _fp(_f32(fx)), _fp(_f32(dEdf)), _fp(dEdx)),
+           "log_softmax_backward")
+    return dEdx
+
+
 def pnls_forward(rows, bd, x, labels):
     """Returns (fx[bd], aux) with aux the raw 3*bd*4-byte buffer [z|m|ids]."""
     labels = _u32(labels)

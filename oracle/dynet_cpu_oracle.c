@@ -712,6 +712,63 @@ int orc_logsumexp_cols(size_t rows, unsigned bd, const float* x, float* m, float
   return 0;
 }
 
+/* Softmax::forward_dev_impl, dimension 0, CPU branch (dynet/nodes-softmaxes.cc:58-74):
+ * per column m = max, fx = exp(x - m), z = sum fx, fx = fx / z.
+ * Pinned by fp64 scipy softmax, columns summing to 1 and shift invariance. */
+int orc_softmax_forward(size_t rows, unsigned cols, const float* x, float* fx) {
+  if (rows == 0) return -1;
+  for (unsigned c = 0; c < cols; ++c) {
+    const float* px = x + (size_t)c * rows;
+    float* pf = fx + (size_t)c * rows;
+    float m = px[0];
+    for (size_t i = 1; i < rows; ++i) m = px[i] > m ? px[i] : m;
+    for (size_t i = 0; i < rows; ++i) pf[i] = expf(px[i] - m);
+    float z = 0.f;
+    for (size_t i = 0; i < rows; ++i) z += pf[i];
+    for (size_t i = 0; i < rows; ++i) pf[i] = pf[i] / z;
+  }
+  return 0;
+}
+
+/* Softmax::backward_dev_impl, dimension 0, CPU branch (dynet/nodes-softmaxes.cc:89-113):
+ * z[col] = sum fx*dEdf; dx += (dEdf - z[col]) * fx.  Pinned by central differences. */
+int orc_softmax_backward(size_t rows, unsigned cols, const float* fx, const float* dEdf, float* dEdx) {
+  for (unsigned c = 0; c < cols; ++c) {
+    const float* pf = fx + (size_t)c * rows;
+    const float* pd = dEdf + (size_t)c * rows;
+    float* po = dEdx + (size_t)c * rows;
+    float z = 0.f;
+    for (size_t i = 0; i < rows; ++i) z += pf[i] * pd[i];
+    for (size_t i = 0; i < rows; ++i) po[i] += (pd[i] - z) * pf[i];
+  }
+  return 0;
+}
+
+/* LogSoftmax::forward_dev_impl, CPU branch (dynet/nodes-softmaxes.cc:141-185): aux = [z | m]
+ * (2*cols floats, :136-138) from TensorTools::logsumexp; fx = x - z[col]. */
+int orc_log_softmax_forward(size_t rows, unsigned cols, const float* x, float* aux, float* fx) {
+  float* z = aux;
+  float* m = aux + cols;
+  if (orc_logsumexp_cols(rows, cols, x, m, z)) return -1;
+  for (unsigned c = 0; c < cols; ++c)
+    for (size_t i = 0; i < rows; ++i) fx[(size_t)c * rows + i] = x[(size_t)c * rows + i] - z[c];
+  return 0;
+}
+
+/* LogSoftmax::backward_dev_impl, CPU branch (dynet/nodes-softmaxes.cc:187-213):
+ * z[col] = sum dEdf; dx += exp(fx) * -z[col] + dEdf. */
+int orc_log_softmax_backward(size_t rows, unsigned cols, const float* fx, const float* dEdf, float* dEdx) {
+  for (unsigned c = 0; c < cols; ++c) {
+    const float* pf = fx + (size_t)c * rows;
+    const float* pd = dEdf + (size_t)c * rows;
+    float* po = dEdx + (size_t)c * rows;
+    float z = 0.f;
+    for (size_t i = 0; i < rows; ++i) z += pd[i];
+    for (size_t i = 0; i < rows; ++i) po[i] += (expf(pf[i]) * -z) + pd[i];
+  }
+  return 0;
+}
+
 /* PickNegLogSoftmax::forward_dev_impl, dynet/nodes-pickneglogsoftmax.cc:79-119:
  * aux = [z | m | ids] with ids[b] = b*rows + label_b (:102), labels
  * bounds-checked (:100); fx[b] = z[b] - x[ids[b]] (:113,:115). */

@@ -121,6 +121,10 @@ int orc_lookup_accumulate_grads(unsigned n_ids, const unsigned* ids, size_t dim,
 /* per batch column: m[b] = max, z[b] = log sum exp(x - m) + m */
 int orc_logsumexp_cols(size_t rows, unsigned bd, const float* x, float* m, float* z);
 /* aux = [z(B) | m(B) | ids(B as u32 = b*rows + label)] */
+int orc_softmax_forward(size_t rows, unsigned cols, const float* x, float* fx);
+int orc_softmax_backward(size_t rows, unsigned cols, const float* fx, const float* dEdf, float* dEdx);
+int orc_log_softmax_forward(size_t rows, unsigned cols, const float* x, float* aux, float* fx);
+int orc_log_softmax_backward(size_t rows, unsigned cols, const float* fx, const float* dEdf, float* dEdx);
 int orc_pnls_forward(size_t rows, unsigned bd, const float* x, const unsigned* labels,
                      void* aux, float* fx);
 int orc_pnls_backward(size_t rows, unsigned bd, const float* x, const void* aux,

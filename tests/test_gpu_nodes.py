@@ -404,6 +404,36 @@ def test_pnls_label_out_of_range_is_an_error(dev):
     assert e.value.status == lib.ERR_INVALID_ARG and "Index error in PickNegLogSoftmax" in str(e.value)
 
 
+@pytest.mark.parametrize("rows,cols", [(10000, 128), (37, 5), (1027, 3), (1, 4), (4, 1), (50000, 64)])
+def test_softmax_and_log_softmax(dev, rows, cols):
+    rng = np.random.default_rng(rows + cols)
+    x = f32(rng.standard_normal((cols, rows)) * 2)
+    dy = f32(rng.standard_normal((cols, rows)))
+    g0 = f32(rng.standard_normal((cols, rows)))
+    xt, dyt = dev.tensor(x), dev.tensor(dy)
+    # softmax
+    ref = orc.softmax_forward(rows, cols, x)
+    fx = dev.empty((cols, rows))
+    dev.softmax_forward(rows, cols, xt, fx)
+    assert_close(fx.numpy(), ref, FWD_RTOL, "softmax fwd", floor=1e-30)
+    dx = dev.tensor(g0)
+    dev.softmax_backward(rows, cols, dev.tensor(ref), dyt, dx)
+    want = orc.softmax_backward(rows, cols, ref, dy, g0.copy())
+    assert_close(dx.numpy(), want, GRAD_RTOL, "softmax bwd", floor=np.maximum(np.abs(g0), 1e-4))
+    # log-softmax
+    ref, aux_ref = orc.log_softmax_forward(rows, cols, x)
+    aux = dev.empty(2 * cols)
+    dev.log_softmax_forward(rows, cols, xt, aux, fx)
+    # x - z: an error of 1e-5 relative in z moves every element by 1e-5 * |z|
+    assert_close(fx.numpy(), ref, FWD_RTOL, "log_softmax fwd", floor=float(np.abs(aux_ref[:cols]).max()) + 1.0)
+    assert_close(aux.numpy(), aux_ref, FWD_RTOL, "log_softmax aux")
+    dx = dev.tensor(g0)
+    dev.log_softmax_backward(rows, cols, dev.tensor(ref), dyt, aux, dx)
+    want = orc.log_softmax_backward(rows, cols, ref, dy, g0.copy())
+    scale = np.abs(dy).sum(axis=1, keepdims=True) * np.exp(ref) + np.abs(dy) + np.abs(g0)
+    assert_close(dx.numpy(), want, GRAD_RTOL, "log_softmax bwd", floor=np.maximum(scale, 1e-4))
+
+
 def test_logsumexp_node(dev):
     rng = np.random.default_rng(15)
     n, bd = 600, 4

@@ -649,3 +649,47 @@ def test_lm_update_clips_and_touches_only_used_rows():
     assert norm > 0.25 and abs(gscale - 0.25 / norm) < 1e-5 * gscale
     assert np.array_equal(p["C"][5:], before["C"][5:])
     np.testing.assert_allclose(p["R"], before["R"] - 0.1 * gscale * g["R"], rtol=1e-6, atol=1e-7)
+
+
+# ---- Softmax / LogSoftmax (the reference holds gradient checks only: tests/test-nodes.cc:1083-1160) ----
+def test_softmax_and_log_softmax_closed_forms():
+    from scipy.special import softmax, log_softmax
+    rng = np.random.default_rng(21)
+    for rows, cols in ((3, 1), (37, 5), (1000, 4)):
+        x = (rng.standard_normal((cols, rows)) * 3).astype(np.float32)
+        sm = orc.softmax_forward(rows, cols, x)
+        want = softmax(x.astype(np.float64), axis=1)
+        assert np.max(np.abs(sm - want) / np.maximum(want, 1e-30)) < 2e-6
+        np.testing.assert_allclose(sm.sum(axis=1), 1.0, rtol=0, atol=3e-6)
+        shifted = orc.softmax_forward(rows, cols, x + np.float32(11.5))
+        np.testing.assert_allclose(shifted, sm, rtol=3e-6, atol=0)
+        ls, aux = orc.log_softmax_forward(rows, cols, x)
+        np.testing.assert_allclose(ls, log_softmax(x.astype(np.float64), axis=1), rtol=0, atol=4e-6)
+        m, z = orc.logsumexp_cols(rows, cols, x)
+        assert aux[:cols].tobytes() == z.tobytes() and aux[cols:].tobytes() == m.tobytes()
+    # the values of the reference's gradient-check input {1.1, -2.2, 3.3} (tests/test-nodes.cc:47)
+    x = np.array([[1.1, -2.2, 3.3]], np.float32)
+    e = np.exp(np.array([1.1, -2.2, 3.3]) - 3.3)
+    np.testing.assert_allclose(orc.softmax_forward(3, 1, x)[0], e / e.sum(), rtol=1e-6)
+
+
+def test_softmax_and_log_softmax_backward_central_differences():
+    from scipy.special import softmax, log_softmax
+    rng = np.random.default_rng(22)
+    rows, cols = 7, 3
+    x = rng.standard_normal((cols, rows))
+    dy = rng.standard_normal((cols, rows))
+    for fwd64, fwd, bwd in ((lambda a: softmax(a, axis=1), orc.softmax_forward, orc.softmax_backward),
+                            (lambda a: log_softmax(a, axis=1), lambda r, c, a: orc.log_softmax_forward(r, c, a)[0],
+                             orc.log_softmax_backward)):
+        fx = fwd(rows, cols, x.astype(np.float32))
+        g0 = rng.standard_normal((cols, rows)).astype(np.float32)
+        got = bwd(rows, cols, fx, dy.astype(np.float32), g0.copy())
+        num = np.zeros_like(x)
+        eps = 1e-6
+        for idx in np.ndindex(*x.shape):
+            xp, xm = x.copy(), x.copy()
+            xp[idx] += eps
+            xm[idx] -= eps
+            num[idx] = ((fwd64(xp) - fwd64(xm)) * dy).sum() / (2 * eps)
+        np.testing.assert_allclose(got - g0, num, rtol=2e-4, atol=2e-5)  # backward accumulates onto g0
