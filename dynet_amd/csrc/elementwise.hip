@@ -193,6 +193,23 @@ struct SgdStep {  // p -= g * s
 int batch_reduce(dyhip_device* dev, size_t n, unsigned bd, const float* in0, const float* in1, float* out,
                  bool accumulate, void* ws, size_t ws_bytes);
 
+// ---- Sum node: groups of up to four arguments per launch, in the reference's association order ----
+struct SumArgs {
+  const float* x[4];
+  unsigned bcast[4];  // 1: the argument has batch size 1 and is broadcast over the batch
+  unsigned cnt;
+};
+
+template <bool ACC>
+__global__ __launch_bounds__(256) void sum_group_kernel(SumArgs a, size_t n, size_t total, float* __restrict__ fx) {
+  const size_t e = size_t(blockIdx.x) * 256 + threadIdx.x;
+  if (e >= total) return;
+  const size_t j = e % n;
+  float v = a.x[0][a.bcast[0] ? j : e];
+  for (unsigned i = 1; i < a.cnt; ++i) v = v + a.x[i][a.bcast[i] ? j : e];
+  fx[e] = ACC ? fx[e] + v : v;
+}
+
 static int check_bd(unsigned bd0, unsigned bd1) {
   DYHIP_REQUIRE(bd0 >= 1 && bd1 >= 1 && (bd0 == bd1 || bd0 == 1 || bd1 == 1),
                 "batch size must match or equal 1 (got %u and %u)", bd0, bd1);
@@ -317,6 +334,49 @@ int dyhip_sgd_update(dyhip_device* dev, size_t n, float* p, const float* g, floa
   DYHIP_REQUIRE(n == 0 || (p && g), "null tensor pointer");
   DYHIP_REQUIRE(wd != 0.f, "weight decay scale must be non-zero");
   return ew_launch<1, true, 0>(dev, n, 1, g, nullptr, nullptr, p, SgdStep{lr * gscale / wd});
+}
+
+int dyhip_sum_forward(dyhip_device* dev, unsigned k, size_t n, unsigned bd, const float* const* xs_host,
+                      const unsigned* bds_host, float* fx) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(k >= 1 && xs_host && bds_host && fx, "Sum needs at least one argument");
+  const size_t total = n * size_t(bd);
+  if (total == 0) return DYHIP_OK;
+  bool same = true;
+  for (unsigned i = 0; i < k; ++i) {
+    DYHIP_REQUIRE(xs_host[i] != nullptr, "null argument %u of Sum", i);
+    DYHIP_REQUIRE(bds_host[i] == bd || bds_host[i] == 1, "Mismatched batch dimension in Sum (argument %u)", i);
+    same = same && bds_host[i] == bds_host[0];
+  }
+  DYHIP_REQUIRE(!same || bds_host[0] == bd, "Sum: output batch size %u but every argument has batch size 1", bd);
+  const dim3 grid((unsigned)cdiv<size_t>(total, 256)), block(256);
+  // equal batch sizes: (first four) then the remainder (k - 4) % 4 then groups of four, each group summed
+  // left to right before it is added; mixed batch sizes: one argument at a time onto a zeroed output
+  unsigned at = 0;
+  bool first = true;
+  while (at < k) {
+    unsigned cnt;
+    if (!same) cnt = 1;
+    else if (first) cnt = k < 4 ? k : 4;
+    else if (at == 4 && (k - 4) % 4 != 0) cnt = (k - 4) % 4;
+    else cnt = 4;
+    SumArgs a;
+    a.cnt = cnt;
+    for (unsigned i = 0; i < 4; ++i) {
+      a.x[i] = i < cnt ? xs_host[at + i] : nullptr;
+      a.bcast[i] = (i < cnt && bds_host[at + i] != bd) ? 1u : 0u;
+    }
+    if (first && same)
+      hipLaunchKernelGGL(sum_group_kernel<false>, grid, block, 0, dev->stream, a, n, total, fx);
+    else {
+      if (first) DYHIP_CHECK_STATUS(dyhip_zero(dev, fx, total * sizeof(float)));
+      hipLaunchKernelGGL(sum_group_kernel<true>, grid, block, 0, dev->stream, a, n, total, fx);
+    }
+    first = false;
+    at += cnt;
+  }
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
 }
 
 }  // extern "C"

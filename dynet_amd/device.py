@@ -213,6 +213,11 @@ class Device:
     def csum_forward(self, n, bd0, bd1, a, b, y):
         _check(cdll.dyhip_csum_forward(self.handle, _sz(n), _u(bd0), _u(bd1), _p(a), _p(b), _p(y)))
 
+    def sum_forward(self, n, bd, xs, bds, fx):
+        ptrs = (_vp * len(xs))(*[x.ptr for x in xs])
+        bds_c = (_u * len(xs))(*[int(b) for b in bds])
+        _check(cdll.dyhip_sum_forward(self.handle, _u(len(xs)), _sz(n), _u(bd), ptrs, bds_c, _p(fx)))
+
     def batch_reduce_workspace(self, n, bd):
         b = _sz(0)
         _check(cdll.dyhip_batch_reduce_workspace(_sz(n), _u(bd), C.byref(b)))

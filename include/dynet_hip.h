@@ -143,6 +143,13 @@ int dyhip_csum_forward(dyhip_device* dev, size_t n, unsigned bd0, unsigned bd1, 
 int dyhip_csum_backward(dyhip_device* dev, size_t n, unsigned bd0, unsigned bd1, const float* dEdf, unsigned i,
                         float* dEdxi, void* ws, size_t ws_bytes);
 
+/* Sum node / esum (dynet/nodes-arith-sum.cc:65-129): fx = sum of k same-shaped arguments whose batch
+ * size is bd or 1 (broadcast), added in the reference's association order (groups of four).  xs_host
+ * and bds_host are HOST arrays.  Backward per argument is dyhip_csum_backward (dx_i += dEdf, summed
+ * over the batch for a batch-1 argument, :115-128). */
+int dyhip_sum_forward(dyhip_device* dev, unsigned k, size_t n, unsigned bd, const float* const* xs_host,
+                      const unsigned* bds_host, float* fx);
+
 /* ---- reductions --------------------------------------------------------- */
 /* workspace for every batch reduction of an n x bd tensor (sum_batches fwd,
  * the broadcast-argument backward of cmult/csum) */

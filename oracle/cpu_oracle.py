@@ -275,6 +275,15 @@ def logsumexp_cols(rows, bd, x):
     return m, z
 
 
+def sum_forward(n, bd, xs, bds):
+    """Sum node; its backward per argument is csum_backward (dx_i += dEdf, batch-summed for batch-1 arguments)."""
+    xs = [_f32(x) for x in xs]
+    fx = np.empty((bd, n), np.float32)
+    bds_c = (C.c_uint * len(xs))(*bds)
+    _check(_lib.orc_sum_forward(len(xs), C.c_size_t(n), bd, _ptr_array(xs), bds_c, _fp(fx)), "sum_forward")
+    return fx
+
+
 def softmax_forward(rows, cols, x):
     fx = np.empty((cols, rows), np.float32)
     _check(_lib.orc_softmax_forward(C.c_size_t(rows), cols, _fp(_f32(x)), _fp(fx)), "softmax_forward")

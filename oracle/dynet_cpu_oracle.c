@@ -712,6 +712,48 @@ int orc_logsumexp_cols(size_t rows, unsigned bd, const float* x, float* m, float
   return 0;
 }
 
+/* Sum::forward_dev_impl (dynet/nodes-arith-sum.cc:65-113).  Equal batch sizes: the first
+ * (up to) four arguments are added left to right, then the remainder (num_args - 4) % 4,
+ * then groups of four, each group added left to right before it is added to fx (:67-89).
+ * Mixed batch sizes: fx = 0, then fx += x_i in order, batch-1 arguments broadcast (:91-111).
+ * Pinned by fp64 sums and, for the association order, by a case where it changes the bits. */
+int orc_sum_forward(unsigned k, size_t n, unsigned bd, const float* const* xs, const unsigned* bds, float* fx) {
+  if (k == 0) return -1;
+  size_t tot = n * (size_t)bd;
+  int same = 1;
+  for (unsigned i = 0; i < k; ++i) {
+    if (bds[i] != bd && bds[i] != 1) return -1;
+    if (bds[i] != bds[0]) same = 0;
+  }
+  if (same && bds[0] != bd) return -1;
+  if (same) {
+    unsigned first = k < 4 ? k : 4;
+    for (size_t e = 0; e < tot; ++e) {
+      float v = xs[0][e];
+      for (unsigned i = 1; i < first; ++i) v = v + xs[i][e];
+      fx[e] = v;
+    }
+    if (k <= 4) return 0;
+    unsigned rem = (k - 4) % 4, at = 4;
+    if (rem) {
+      for (size_t e = 0; e < tot; ++e) {
+        float v = xs[at][e];
+        for (unsigned i = 1; i < rem; ++i) v = v + xs[at + i][e];
+        fx[e] += v;
+      }
+      at += rem;
+    }
+    for (; at < k; at += 4)
+      for (size_t e = 0; e < tot; ++e) fx[e] += ((xs[at][e] + xs[at + 1][e]) + xs[at + 2][e]) + xs[at + 3][e];
+    return 0;
+  }
+  for (size_t e = 0; e < tot; ++e) fx[e] = 0.f;
+  for (unsigned i = 0; i < k; ++i)
+    for (unsigned b = 0; b < bd; ++b)
+      for (size_t j = 0; j < n; ++j) fx[(size_t)b * n + j] += xs[i][(bds[i] == bd ? (size_t)b * n : 0) + j];
+  return 0;
+}
+
 /* Softmax::forward_dev_impl, dimension 0, CPU branch (dynet/nodes-softmaxes.cc:58-74):
  * per column m = max, fx = exp(x - m), z = sum fx, fx = fx / z.
  * Pinned by fp64 scipy softmax, columns summing to 1 and shift invariance. */

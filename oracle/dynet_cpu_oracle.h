@@ -121,6 +121,7 @@ int orc_lookup_accumulate_grads(unsigned n_ids, const unsigned* ids, size_t dim,
 /* per batch column: m[b] = max, z[b] = log sum exp(x - m) + m */
 int orc_logsumexp_cols(size_t rows, unsigned bd, const float* x, float* m, float* z);
 /* aux = [z(B) | m(B) | ids(B as u32 = b*rows + label)] */
+int orc_sum_forward(unsigned k, size_t n, unsigned bd, const float* const* xs, const unsigned* bds, float* fx);
 int orc_softmax_forward(size_t rows, unsigned cols, const float* x, float* fx);
 int orc_softmax_backward(size_t rows, unsigned cols, const float* fx, const float* dEdf, float* dEdx);
 int orc_log_softmax_forward(size_t rows, unsigned cols, const float* x, float* aux, float* fx);

@@ -236,3 +236,30 @@ def test_layer_norm_invariances_at_full_size(dev):
     assert_close(y1.numpy(), y0.numpy(), FWD_RTOL, "LN(4x) == LN(x)", floor=1.0)
     dev.layer_norm_forward(n, bd, dev.tensor(x + F32(2.0)), gt, bt, y1)
     assert_close(y1.numpy(), y0.numpy(), 5e-5, "LN(x+2) == LN(x)", floor=1.0)
+
+
+@pytest.mark.parametrize("k", [1, 2, 4, 5, 7, 8, 11])
+def test_sum_node_bit_exact(dev, k):
+    rng = np.random.default_rng(k)
+    n, bd = 1031, 6
+    xs = [f32(rng.standard_normal((bd, n)) * 10.0 ** rng.integers(-2, 3)) for _ in range(k)]
+    fx = dev.empty((bd, n))
+    dev.sum_forward(n, bd, [dev.tensor(x) for x in xs], [bd] * k, fx)
+    assert fx.numpy().tobytes() == orc.sum_forward(n, bd, xs, [bd] * k).tobytes()
+
+
+def test_sum_node_broadcast_and_backward(dev):
+    rng = np.random.default_rng(3)
+    n, bd = 300, 5
+    xs = [f32(rng.standard_normal((bd, n))), f32(rng.standard_normal((1, n))), f32(rng.standard_normal((bd, n)))]
+    bds = [bd, 1, bd]
+    fx = dev.empty((bd, n))
+    dev.sum_forward(n, bd, [dev.tensor(x) for x in xs], bds, fx)
+    assert fx.numpy().tobytes() == orc.sum_forward(n, bd, xs, bds).tobytes()
+    dy = f32(rng.standard_normal((bd, n)))
+    for i, b in enumerate(bds):
+        g0 = f32(rng.standard_normal((b, n)))
+        dx = dev.tensor(g0)
+        dev.csum_backward(n, b, bd, dev.tensor(dy), 0, dx)
+        want = orc.csum_backward(n, b, bd, dy, 0, g0.copy())
+        assert_close(dx.numpy(), want, GRAD_RTOL, f"sum bwd arg {i}", floor=np.sqrt(bd))

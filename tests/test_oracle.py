@@ -693,3 +693,37 @@ def test_softmax_and_log_softmax_backward_central_differences():
             xm[idx] -= eps
             num[idx] = ((fwd64(xp) - fwd64(xm)) * dy).sum() / (2 * eps)
         np.testing.assert_allclose(got - g0, num, rtol=2e-4, atol=2e-5)  # backward accumulates onto g0
+
+
+def test_sum_node_association_order_and_broadcast():
+    rng = np.random.default_rng(23)
+    n, bd = 5, 3
+    for k in (1, 2, 3, 4, 5, 6, 7, 8, 9, 13):
+        xs = [(rng.standard_normal((bd, n)) * 10.0 ** rng.integers(-3, 4)).astype(np.float32) for _ in range(k)]
+        got = orc.sum_forward(n, bd, xs, [bd] * k)
+        np.testing.assert_allclose(got, np.sum([x.astype(np.float64) for x in xs], axis=0), rtol=0,
+                                   atol=1e-6 * max(float(np.abs(x).max()) for x in xs) * k)
+        # groups of four, each summed left to right before it joins fx (dynet/nodes-arith-sum.cc:67-89)
+        want = xs[0].copy()
+        for x in xs[1:4]:
+            want = want + x
+        rem = (k - 4) % 4 if k > 4 else 0
+        at = 4
+        if rem:
+            g = xs[at].copy()
+            for x in xs[at + 1:at + rem]:
+                g = g + x
+            want = want + g
+            at += rem
+        while at < k:
+            want = want + (((xs[at] + xs[at + 1]) + xs[at + 2]) + xs[at + 3])
+            at += 4
+        assert got.tobytes() == want.astype(np.float32).tobytes(), k
+    # a case where the grouping changes the bits: 1e8 + (-1e8 + 1 ...) vs left-to-right
+    xs = [np.full((1, 1), v, np.float32) for v in (1.0, 1e8, -1e8, 1.0, 1.0, 1e8, -1e8, 1.0)]
+    assert orc.sum_forward(1, 1, xs, [1] * 8)[0, 0] == np.float32(np.float32(np.float32(np.float32(1.0) + np.float32(1e8)) + np.float32(-1e8)) + np.float32(1.0)) + np.float32(np.float32(np.float32(np.float32(1.0) + np.float32(1e8)) + np.float32(-1e8)) + np.float32(1.0))
+    # mixed batch sizes: broadcast of batch-1 arguments
+    a, b, c = (rng.standard_normal((bd, n)).astype(np.float32), rng.standard_normal((1, n)).astype(np.float32),
+               rng.standard_normal((bd, n)).astype(np.float32))
+    got = orc.sum_forward(n, bd, [a, b, c], [bd, 1, bd])
+    assert got.tobytes() == (((np.zeros_like(a) + a) + b) + c).tobytes()
