@@ -575,6 +575,40 @@ def test_device_side_clipping_and_sparse_rows(dev):
     assert not g2t.numpy().any()
 
 
+def test_forked_queue_ordering_and_errors(dev):
+    """dyhip_device_fork / dyhip_device_wait: a chain that hops between two queues sees every earlier write."""
+    rng = np.random.default_rng(20)
+    n = 1 << 20
+    x = f32(rng.standard_normal(n))
+    q = dev.fork()
+    a, b, c = dev.tensor(x), dev.empty(n), dev.empty(n)
+    want = x.copy()
+    for _ in range(6):
+        dev.scale_copy(n, a, 0.5, b)      # device queue: b = a / 2
+        q.wait(dev)
+        q.scale_copy(n, b, 3.0, c)        # forked queue: c = 3 b
+        dev.wait(q)
+        dev.scale_copy(n, c, 1.0, a)      # device queue again: a = c
+        want = orc.scale_copy(orc.scale_copy(want, 0.5), 3.0)
+    assert a.numpy().tobytes() == want.tobytes()
+    # a GEMM on each queue at the same time: separate split-K workspaces
+    M, N, K = 256, 64, 2048
+    l, r = f32(rng.standard_normal((K, M))), f32(rng.standard_normal((N, K)))
+    lt, rt = dev.tensor(l), dev.tensor(r)
+    y0, y1 = dev.zeros((N, M)), dev.zeros((N, M))
+    q.wait(dev)
+    for _ in range(4):
+        dev.gemm_nn(M, N, K, lt, rt, 0.0, y0)
+        q.gemm_nn(M, N, K, lt, rt, 0.0, y1)
+    dev.wait(q)
+    ref = orc.gemm_nn(M, N, K, l, r, 0.0, np.zeros((N, M), F32))
+    assert_close(y0.numpy(), ref, FWD_RTOL, "gemm on the device queue", floor=np.sqrt(K))
+    assert y0.numpy().tobytes() == y1.numpy().tobytes()
+    with pytest.raises(DyhipError):
+        q.fork()  # only the device itself can be forked
+    q.close()
+
+
 def test_device_scalars_and_pools(dev):
     vals = [np.frombuffer(dev_scalar(dev, k), F32)[0] for k in range(3)]
     assert vals == [-1.0, 1.0, 0.0]
