@@ -333,6 +333,65 @@ def lstm_lm(steps, warmup=3, use_graph=True):
     return res
 
 
+def lm_kernels(reps, use_graph=True):
+    """The GEMMs and the non-GEMM kernels of the cfg-5 step at their in-situ shapes: TFLOP/s against the fp32
+    MFMA peak, GB/s against the HBM peak."""
+    from dynet_amd import Device, lib
+
+    V, E, H, B, T = 10000, 256, 1024, 128, 35
+    N = T * B
+    dev = Device(0, mem_mb=(2048, 1024, 64, 1024))
+    out = {"gemm": [], "kernels": []}
+    shapes = [("input projection, layer 1 (NN)", "nn", 4 * H, N, H), ("input projection, layer 0 (NN)", "nn", 4 * H, N, E),
+              ("output projection (NN, bias epilogue)", "affine", V, N, H), ("d h_top = R^T dlogits (TN)", "tn", H, N, V),
+              ("dR = dlogits h^T (NT)", "nt", V, H, N), ("dWx1 / dWh = dpre x^T (NT)", "nt", 4 * H, H, N),
+              ("dx = Wx^T dpre (TN)", "tn", H, N, 4 * H), ("dWx0 (NT)", "nt", 4 * H, E, N),
+              ("recurrent Wh h, one timestep (NN, split-K slices)", "rec_f", 4 * H, B, H),
+              ("recurrent Wh^T dpre, one timestep (TN, split-K slices)", "rec_b", H, B, 4 * H)]
+    for name, form, M, Nn, K in shapes:
+        a, b, y = dev.empty((M * K,)), dev.empty((Nn * K,)), dev.empty((M * Nn,))
+        bias = dev.empty((M,))
+        for t in (a, b, bias):
+            dev.constant(t, 0.01)
+        fb, bb = dev.lstm_cell_workspace(H, B)
+        ws, _ = dev.workspace(max(fb, bb))
+        fn = {"nn": lambda: dev.gemm_nn(M, Nn, K, a, b, 0.0, y), "tn": lambda: dev.gemm_tn(M, Nn, K, a, b, 0.0, y),
+              "nt": lambda: dev.gemm_nt(M, Nn, K, a, b, 0.0, y), "affine": lambda: dev.affine_forward(M, Nn, K, bias, a, b, y),
+              "rec_f": lambda: dev.lstm_recurrent_forward(H, B, a, b, ws, fb),
+              "rec_b": lambda: dev.lstm_recurrent_backward(H, B, a, b, ws, bb)}[form]
+        if use_graph:
+            g = capture(dev, [fn] * 4)
+            us = time_graph(dev, g, reps, 4)
+            g.destroy()
+        else:
+            us = time_loop(dev, [fn], reps)
+        tf = 2.0 * M * Nn * K / us / 1e6
+        out["gemm"].append({"gemm": name, "M": M, "N": Nn, "K": K, "us": round(us, 2), "TFLOPs": round(tf, 1),
+                            "frac_of_fp32_mfma_peak": round(tf / FP32_MFMA_PEAK_TFLOPS, 4)})
+        for w in (lib.POOL_FXS, lib.POOL_SCS):
+            dev.sync()
+            dev.free_pool(w)
+    # fused cell kernels at H = 1024, B = 128 with the split counts the recurrent GEMMs produce
+    Wh, h, dpre = dev.empty((H, 4 * H)), dev.empty((B, H)), dev.empty((B, 4 * H))
+    xp, bb_, c, c2, hh, g = (dev.empty(s) for s in ((B, 4 * H), (4 * H,), (B, H), (B, H), (B, H), (B, 4 * H)))
+    dh, dc, dc2 = dev.empty((B, H)), dev.empty((B, H)), dev.empty((B, H))
+    for t in (Wh, h, dpre, xp, bb_, c, dh, dc):
+        dev.constant(t, 0.01)
+    fb, bb = dev.lstm_cell_workspace(H, B)
+    wf, _ = dev.workspace(fb)
+    wb, _ = dev.workspace(bb)
+    nf = dev.lstm_recurrent_forward(H, B, Wh, h, wf, fb)
+    nb = dev.lstm_recurrent_backward(H, B, Wh, dpre, wb, bb)
+    dev.lstm_cell_forward(H, B, xp, bb_, wf, nf, c, g, c2, hh)
+    named = [("lstm_cell_fwd (%d slices)" % nf, (4 * (1 + nf) * H * B + 4 * H + 7 * H * B) * 4,
+              lambda s: dev.lstm_cell_forward(H, B, xp, bb_, wf, nf, c, g, c2, hh)),
+             ("lstm_cell_bwd (%d slices)" % nb, ((4 + 4 + nb + 4 + 1) * H * B) * 4,
+              lambda s: dev.lstm_cell_backward(H, B, g, c2, c, dh, wb, nb, dc, dpre, dc2))]
+    out["kernels"] = per_kernel_table(dev, named, [None] * 4, reps, use_graph=use_graph)
+    dev.close()
+    return out
+
+
 def cpu_baseline(step_bytes, seconds):
     """The CPU oracle (plain-C restatement of DyNet's CPU path) on the same sweep, one host core."""
     from oracle import cpu_oracle as orc
@@ -451,6 +510,7 @@ def main():
     dev.close()
     if not args.no_lm:
         out["cfg5_lstm_lm"] = lstm_lm(args.lm_steps, use_graph=not args.no_graph)
+        out["cfg5_lstm_lm"]["in_situ"] = lm_kernels(args.kernel_reps, use_graph=not args.no_graph)
         out["lstm_lm_tokens_per_s"] = out["cfg5_lstm_lm"]["fused_cell_path"]["tokens_per_s"]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(sweep.step_bytes, args.cpu_seconds)
