@@ -1,0 +1,421 @@
+// C++ host side above the C-ABI: the operator interface DyNet's nodes expose on their GPU
+// path, with the same names, argument meaning and error behaviour, forwarding to
+// libdynet_hip.so.  In a DyNet build these bodies become the Device_GPU instantiations
+// of forward_dev_impl / backward_dev_impl (dynet/nodes-def-macros.h:44-62,
+// dynet/nodes-impl-macros.h:13-61); here they stand on a minimal Dim / Tensor / Device_GPU
+// of their own, because DyNet's headers pull in Eigen, so that the library can be driven
+// and tested from C++ the way the reference's tests drive its nodes.
+//
+//   xs      arguments in the node's own order (dynet/nodes-lstm.cc:101-112 etc.)
+//   fx      forward overwrites it
+//   dEdxi   backward accumulates into it (dynet/exec.cc:207-208 zeroes it once)
+//   errors  std::invalid_argument for bad arguments (DYNET_ARG_CHECK, dynet/except.h:41-46),
+//           dynet_hip::cuda_exception for runtime failures (dynet/cuda.h:20-52),
+//           dynet_hip::out_of_memory (dynet/except.h:11-14)
+#pragma once
+
+#include <cstddef>
+#include <initializer_list>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "dynet_hip.h"
+
+namespace dynet_hip {
+
+typedef float real;  // dynet/tensor.h:36
+
+struct cuda_exception : public std::runtime_error {
+  explicit cuda_exception(const std::string& what) : std::runtime_error(what) {}
+};
+struct out_of_memory : public std::runtime_error {
+  explicit out_of_memory(const std::string& what) : std::runtime_error(what) {}
+};
+
+inline void abi_check(int status) {
+  if (status == DYHIP_OK) return;
+  const std::string msg = dyhip_last_error();
+  if (status == DYHIP_ERR_INVALID_ARG) throw std::invalid_argument(msg);
+  if (status == DYHIP_ERR_OUT_OF_MEMORY) throw out_of_memory(msg);
+  throw cuda_exception(msg);
+}
+
+// dynet/dim.h:34-304, the part the nodes use
+struct Dim {
+  unsigned d[7];
+  unsigned nd;
+  unsigned bd;
+  Dim() : nd(0), bd(1) {}
+  Dim(std::initializer_list<unsigned> x, unsigned b = 1) : nd(0), bd(b) {
+    for (unsigned v : x) d[nd++] = v;
+  }
+  unsigned batch_size() const {
+    unsigned p = 1;
+    for (unsigned i = 0; i < nd; ++i) p *= d[i];
+    return p;
+  }
+  unsigned size() const { return batch_size() * bd; }
+  unsigned rows() const { return nd ? d[0] : 1; }
+  unsigned cols() const { return nd > 1 ? d[1] : 1; }
+  unsigned batch_elems() const { return bd; }
+  unsigned operator[](unsigned i) const { return i < nd ? d[i] : 1; }
+};
+
+enum class DeviceMempool { FXS = 0, DEDFS = 1, PS = 2, SCS = 3, NONE = 4 };  // dynet/device-structs.h:15
+
+// dynet/aligned-mem-pool.h:47-69 over the library's pool
+class AlignedMemoryPool {
+ public:
+  explicit AlignedMemoryPool(dyhip_pool* p) : p_(p) {}
+  void* allocate(size_t n) {
+    void* out = nullptr;
+    abi_check(dyhip_pool_allocate(p_, n, &out));
+    return out;
+  }
+  void free() { abi_check(dyhip_pool_free(p_)); }
+  void zero_allocated_memory() { abi_check(dyhip_pool_zero_allocated(p_)); }
+  size_t used() {
+    size_t u = 0;
+    abi_check(dyhip_pool_used(p_, &u));
+    return u;
+  }
+  void set_used(size_t s) { abi_check(dyhip_pool_set_used(p_, s)); }
+
+ private:
+  dyhip_pool* p_;
+};
+
+struct Device_GPU;
+
+// dynet/tensor.h:46-120, the fields the nodes touch
+struct Tensor {
+  Dim d;
+  float* v;
+  Device_GPU* device;
+  DeviceMempool mem_pool;
+  Tensor() : v(nullptr), device(nullptr), mem_pool(DeviceMempool::NONE) {}
+  Tensor(const Dim& d, float* v, Device_GPU* dev, DeviceMempool mp) : d(d), v(v), device(dev), mem_pool(mp) {}
+};
+
+// dynet/devices.h:46-61, dynet/devices.cc:91-121
+struct Device_GPU {
+  dyhip_device* hip;
+  float *kSCALAR_MINUSONE, *kSCALAR_ONE, *kSCALAR_ZERO;
+  std::vector<AlignedMemoryPool*> pools;
+
+  Device_GPU(int device_id, size_t fxs_mb, size_t dedfs_mb, size_t ps_mb, size_t scs_mb) : hip(nullptr) {
+    const size_t mb[4] = {fxs_mb, dedfs_mb, ps_mb, scs_mb};
+    abi_check(dyhip_device_create(device_id, mb, &hip));
+    const float* s[3];
+    for (int k = 0; k < 3; ++k) abi_check(dyhip_device_scalar(hip, k, &s[k]));
+    kSCALAR_MINUSONE = const_cast<float*>(s[DYHIP_SCALAR_MINUSONE]);
+    kSCALAR_ONE = const_cast<float*>(s[DYHIP_SCALAR_ONE]);
+    kSCALAR_ZERO = const_cast<float*>(s[DYHIP_SCALAR_ZERO]);
+    for (int k = 0; k < 4; ++k) {
+      dyhip_pool* p = nullptr;
+      abi_check(dyhip_device_pool(hip, k, &p));
+      pools.push_back(new AlignedMemoryPool(p));
+    }
+  }
+  ~Device_GPU() {
+    for (AlignedMemoryPool* p : pools) delete p;
+    if (hip) dyhip_device_destroy(hip);
+  }
+  Device_GPU(const Device_GPU&) = delete;
+  Device_GPU& operator=(const Device_GPU&) = delete;
+
+  // Device::allocate_tensor (dynet/devices.cc:82-88)
+  Tensor allocate_tensor(DeviceMempool mp, const Dim& d) {
+    float* v = static_cast<float*>(pools[static_cast<int>(mp)]->allocate(sizeof(float) * d.size()));
+    return Tensor(d, v, this, mp);
+  }
+};
+
+// dynet/tensor.h TensorTools, the calls the tests use (dynet/tensor.cc:66-229)
+struct TensorTools {
+  static void set_elements(Tensor& t, const std::vector<float>& vals) {
+    if (vals.size() != t.d.size()) throw std::invalid_argument("set_elements: size mismatch");
+    abi_check(dyhip_memcpy_h2d(t.device->hip, t.v, vals.data(), sizeof(float) * vals.size()));
+    abi_check(dyhip_device_sync(t.device->hip));
+  }
+  static void zero(Tensor& t) { abi_check(dyhip_zero(t.device->hip, t.v, sizeof(float) * t.d.size())); }
+  static void constant(Tensor& t, float c) { abi_check(dyhip_constant(t.device->hip, t.d.size(), c, t.v)); }
+  static void accumulate(Tensor& t, const Tensor& src) {
+    abi_check(dyhip_accumulate(t.device->hip, t.d.size(), src.v, t.v));
+  }
+};
+inline std::vector<real> as_vector(const Tensor& t) {  // blocking copy, dynet/tensor.cc:66-93
+  std::vector<real> out(t.d.size());
+  abi_check(dyhip_memcpy_d2h(t.device->hip, out.data(), t.v, sizeof(float) * out.size()));
+  return out;
+}
+
+// ---- nodes ---------------------------------------------------------------------------------
+struct Node {
+  virtual ~Node() {}
+  mutable void* aux_mem = nullptr;  // assigned by the executor before forward (dynet/exec.cc:138-147)
+  virtual size_t aux_storage_size() const { return 0; }
+  virtual void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const = 0;
+  virtual void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, const Tensor& fx,
+                                 const Tensor& dEdf, unsigned i, Tensor& dEdxi) const = 0;
+
+ protected:
+  static AlignedMemoryPool* scratch(const Tensor& fx) { return fx.device->pools[static_cast<int>(DeviceMempool::SCS)]; }
+};
+
+// dynet/nodes-lstm.h:9-26, nodes-lstm.cc:101-527.  xs = {x_t[0..k), h_tm1, Wx, Wh, b [, mask_x, mask_h]}
+struct VanillaLSTMGates : public Node {
+  VanillaLSTMGates(bool dropout, real weightnoise_std) : dropout(dropout), weightnoise_std(weightnoise_std) {}
+  bool dropout;
+  real weightnoise_std;
+
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    Args a = unpack(xs);
+    size_t need = 0;
+    abi_check(dyhip_lstm_gates_workspace(a.k, a.I, a.H, a.B, dropout, &need));
+    void* ws = need ? scratch(fx)->allocate(need) : nullptr;
+    abi_check(dyhip_lstm_gates_forward(dev.hip, a.k, a.x.data(), a.xd.data(), a.H, a.B, xs[a.k]->v, xs[a.k + 1]->v,
+                                       xs[a.k + 2]->v, xs[a.k + 3]->v, a.mx, a.mx_bd, a.mh, a.mh_bd,
+                                       DYHIP_LOGISTIC_PACKET, fx.v, ws, need));
+    scratch(fx)->free();
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, const Tensor& fx,
+                         const Tensor& dEdf, unsigned i, Tensor& dEdxi) const override {
+    Args a = unpack(xs);
+    if (i > a.k + 3) return;  // the dropout masks get no gradient (dynet/nodes-lstm.cc:522)
+    size_t need = 0;
+    abi_check(dyhip_lstm_gates_backward_workspace(a.k, a.I, a.H, a.B, dropout, &need));
+    void* ws = scratch(fx)->allocate(need);
+    abi_check(dyhip_lstm_gates_backward(dev.hip, a.k, a.x.data(), a.xd.data(), a.H, a.B, xs[a.k]->v, xs[a.k + 1]->v,
+                                        xs[a.k + 2]->v, a.mx, a.mx_bd, a.mh, a.mh_bd, fx.v, dEdf.v, nullptr, i,
+                                        dEdxi.v, ws, need));
+    scratch(fx)->free();
+  }
+
+ private:
+  struct Args {
+    unsigned k, I, H, B, mx_bd, mh_bd;
+    std::vector<const float*> x;
+    std::vector<unsigned> xd;
+    const float *mx, *mh;
+  };
+  Args unpack(const std::vector<const Tensor*>& xs) const {
+    if (weightnoise_std != 0.f) throw std::invalid_argument("VanillaLSTMGates: weight noise is not supported");
+    if (xs.size() < (dropout ? 7u : 5u)) throw std::invalid_argument("Failed input count check in VanillaLSTMGates");
+    Args a;
+    a.k = static_cast<unsigned>(dropout ? xs.size() - 6 : xs.size() - 4);
+    a.H = xs[a.k]->d[0];
+    a.B = xs[0]->d.bd;
+    a.I = 0;
+    for (unsigned j = 0; j < a.k; ++j) {
+      a.x.push_back(xs[j]->v);
+      a.xd.push_back(xs[j]->d[0]);
+      a.I += xs[j]->d[0];
+    }
+    a.mx = dropout ? xs[a.k + 4]->v : nullptr;
+    a.mh = dropout ? xs[a.k + 5]->v : nullptr;
+    a.mx_bd = dropout ? xs[a.k + 4]->d.bd : 0;
+    a.mh_bd = dropout ? xs[a.k + 5]->d.bd : 0;
+    return a;
+  }
+};
+
+// dynet/nodes-lstm.cc:562-615.  xs = {c_tm1, gates_t}
+struct VanillaLSTMC : public Node {
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    abi_check(dyhip_lstm_c_forward(dev.hip, xs[0]->d[0], xs[0]->d.bd, xs[0]->v, xs[1]->v, fx.v));
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, const Tensor&,
+                         const Tensor& dEdf, unsigned i, Tensor& dEdxi) const override {
+    abi_check(dyhip_lstm_c_backward(dev.hip, xs[0]->d[0], xs[0]->d.bd, xs[0]->v, xs[1]->v, dEdf.v, i, dEdxi.v));
+  }
+};
+
+// dynet/nodes-lstm.cc:650-703.  xs = {c_t, gates_t}
+struct VanillaLSTMH : public Node {
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    abi_check(dyhip_lstm_h_forward(dev.hip, xs[0]->d[0], xs[0]->d.bd, xs[0]->v, xs[1]->v, fx.v));
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, const Tensor&,
+                         const Tensor& dEdf, unsigned i, Tensor& dEdxi) const override {
+    abi_check(dyhip_lstm_h_backward(dev.hip, xs[0]->d[0], xs[0]->d.bd, xs[0]->v, xs[1]->v, dEdf.v, i, dEdxi.v));
+  }
+};
+
+// Tanh (dynet/nodes-trig.cc:312-326), LogisticSigmoid (dynet/nodes-activations.cc:65-78), Rectify (:31-44)
+template <int OP>
+struct UnaryNode : public Node {
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    abi_check(dyhip_unary_forward(dev.hip, OP, DYHIP_LOGISTIC_PACKET, fx.d.size(), xs[0]->v, fx.v));
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>&, const Tensor& fx,
+                         const Tensor& dEdf, unsigned, Tensor& dEdxi) const override {
+    abi_check(dyhip_unary_backward(dev.hip, OP, fx.d.size(), fx.v, dEdf.v, dEdxi.v));
+  }
+};
+typedef UnaryNode<DYHIP_OP_TANH> Tanh;
+typedef UnaryNode<DYHIP_OP_LOGISTIC> LogisticSigmoid;
+typedef UnaryNode<DYHIP_OP_RECTIFY> Rectify;
+
+// CwiseMultiply, same shape or one side with batch size 1 (dynet/nodes-arith-cwise.cc:196-307)
+struct CwiseMultiply : public Node {
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    abi_check(dyhip_cmult_forward(dev.hip, fx.d.batch_size(), xs[0]->d.bd, xs[1]->d.bd, xs[0]->v, xs[1]->v, fx.v));
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, const Tensor& fx,
+                         const Tensor& dEdf, unsigned i, Tensor& dEdxi) const override {
+    size_t need = 0;
+    abi_check(dyhip_batch_reduce_workspace(fx.d.batch_size(), fx.d.bd, &need));
+    void* ws = need ? scratch(fx)->allocate(need) : nullptr;
+    abi_check(dyhip_cmult_backward(dev.hip, fx.d.batch_size(), xs[0]->d.bd, xs[1]->d.bd, xs[0]->v, xs[1]->v, dEdf.v, i,
+                                   dEdxi.v, ws, need));
+    scratch(fx)->free();
+  }
+};
+
+// sum_batches = SumDimension({}, include_batch_dim) (dynet/nodes-arith-sum.cc:197-248, dynet/expr.cc:218)
+struct SumBatches : public Node {
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    size_t need = 0;
+    abi_check(dyhip_batch_reduce_workspace(fx.d.batch_size(), xs[0]->d.bd, &need));
+    void* ws = need ? scratch(fx)->allocate(need) : nullptr;
+    abi_check(dyhip_sum_batches_forward(dev.hip, fx.d.batch_size(), xs[0]->d.bd, xs[0]->v, fx.v, ws, need));
+    scratch(fx)->free();
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, const Tensor& fx,
+                         const Tensor& dEdf, unsigned, Tensor& dEdxi) const override {
+    abi_check(dyhip_sum_batches_backward(dev.hip, fx.d.batch_size(), xs[0]->d.bd, dEdf.v, dEdxi.v));
+  }
+};
+
+// layer_norm(x, g, b) as one node instead of the 8-node composite of dynet/expr.cc:248-253.  xs = {x, g, b}
+struct LayerNorm : public Node {
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    abi_check(dyhip_layer_norm_forward(dev.hip, xs[0]->d.batch_size(), xs[0]->d.bd, xs[0]->v, xs[1]->v, xs[2]->v, fx.v));
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, const Tensor& fx,
+                         const Tensor& dEdf, unsigned i, Tensor& dEdxi) const override {
+    const size_t n = xs[0]->d.batch_size();
+    const unsigned bd = xs[0]->d.bd;
+    size_t need = 0;
+    abi_check(dyhip_layer_norm_backward_workspace(n, bd, &need));
+    void* ws = scratch(fx)->allocate(need);
+    abi_check(dyhip_layer_norm_backward(dev.hip, n, bd, xs[0]->v, xs[1]->v, dEdf.v, i == 0 ? dEdxi.v : nullptr,
+                                        i == 1 ? dEdxi.v : nullptr, i == 2 ? dEdxi.v : nullptr, ws, need));
+    scratch(fx)->free();
+  }
+};
+
+// LookupNode (dynet/param-nodes.cc:304-329) over a table Dim({D}, V) stored as V contiguous rows
+// (dynet/model.cc:130-159); accumulate_grads = LookupParameterStorage::accumulate_grads_dev (:728-743)
+struct LookupNode : public Node {
+  LookupNode(const Tensor* all_values, Tensor* all_grads, const std::vector<unsigned>* pindices)
+      : all_values(all_values), all_grads(all_grads), pindices(pindices) {}
+  const Tensor* all_values;
+  Tensor* all_grads;
+  const std::vector<unsigned>* pindices;
+  size_t aux_storage_size() const override { return sizeof(unsigned) * pindices->size(); }  // :154-156
+
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>&, Tensor& fx) const override {
+    abi_check(dyhip_lookup_forward(dev.hip, static_cast<unsigned>(pindices->size()), pindices->data(),
+                                   static_cast<unsigned*>(aux_mem), all_values->d.batch_size(), all_values->d.bd,
+                                   all_values->v, 1.0f, fx.v));
+  }
+  void backward_dev_impl(const Device_GPU&, const std::vector<const Tensor*>&, const Tensor&, const Tensor&, unsigned,
+                         Tensor&) const override {
+    throw std::runtime_error("called backward() on arity 0 node: i = 0");  // dynet/param-nodes.cc:331-337
+  }
+  void accumulate_grad(const Device_GPU& dev, const Tensor& fx, const Tensor& g) const {
+    const unsigned n = static_cast<unsigned>(pindices->size());
+    const size_t D = all_values->d.batch_size();
+    size_t need = 0;
+    abi_check(dyhip_lookup_accumulate_grads_workspace(n, D, all_values->d.bd, &need));
+    void* ws = scratch(fx)->allocate(need);
+    abi_check(dyhip_lookup_accumulate_grads(dev.hip, n, static_cast<const unsigned*>(aux_mem), D, all_values->d.bd, g.v,
+                                            all_grads->v, ws, need));
+    scratch(fx)->free();
+  }
+};
+
+// PickNegLogSoftmax (dynet/nodes-pickneglogsoftmax.cc:72-145); aux_mem = [z | m | ids]
+struct PickNegLogSoftmax : public Node {
+  explicit PickNegLogSoftmax(const std::vector<unsigned>* pvals) : pvals(pvals) {}
+  const std::vector<unsigned>* pvals;
+  size_t aux_storage_size() const override { return 2 * sizeof(float) * pvals->size() + sizeof(unsigned) * pvals->size(); }
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    if (xs[0]->d.cols() != 1) throw std::invalid_argument("PickNegLogSoftmax::forward not yet implemented for multiple columns");
+    if (pvals->size() != xs[0]->d.bd) throw std::invalid_argument("PickNegLogSoftmax: one index per batch element expected");
+    abi_check(dyhip_pnls_forward(dev.hip, xs[0]->d.rows(), xs[0]->d.bd, xs[0]->v, pvals->data(), aux_mem, fx.v));
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, const Tensor&, const Tensor& dEdf,
+                         unsigned, Tensor& dEdxi) const override {
+    abi_check(dyhip_pnls_backward(dev.hip, xs[0]->d.rows(), xs[0]->d.bd, xs[0]->v, aux_mem, dEdf.v, dEdxi.v));
+  }
+};
+
+// LogSoftmax (dynet/nodes-softmaxes.cc:127-214); aux_mem = [z | m]
+struct LogSoftmax : public Node {
+  explicit LogSoftmax(const Dim& dim) : dim(dim) {}
+  Dim dim;
+  size_t aux_storage_size() const override { return 2 * dim.size() / dim.rows() * sizeof(float); }
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    abi_check(dyhip_log_softmax_forward(dev.hip, xs[0]->d.rows(), xs[0]->d.cols() * xs[0]->d.bd, xs[0]->v, aux_mem, fx.v));
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, const Tensor& fx,
+                         const Tensor& dEdf, unsigned, Tensor& dEdxi) const override {
+    abi_check(dyhip_log_softmax_backward(dev.hip, xs[0]->d.rows(), xs[0]->d.cols() * xs[0]->d.bd, fx.v, dEdf.v, aux_mem,
+                                         dEdxi.v));
+  }
+};
+
+// AffineTransform with one (W, x) pair (dynet/nodes-affinetransform.cc:77-156).  xs = {bias, W, x}
+struct AffineTransform : public Node {
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    if (xs.size() != 3) throw std::invalid_argument("AffineTransform: this device path takes one (W, x) pair");
+    abi_check(dyhip_affine_forward(dev.hip, xs[1]->d.rows(), xs[2]->d.cols() * xs[2]->d.bd, xs[1]->d.cols(), xs[0]->v,
+                                   xs[1]->v, xs[2]->v, fx.v));
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, const Tensor& fx,
+                         const Tensor& dEdf, unsigned i, Tensor& dEdxi) const override {
+    const size_t M = xs[1]->d.rows(), K = xs[1]->d.cols(), N = size_t(xs[2]->d.cols()) * xs[2]->d.bd;
+    if (i == 0) {
+      size_t need = 0;
+      abi_check(dyhip_batch_reduce_workspace(M, static_cast<unsigned>(N), &need));
+      void* ws = need ? scratch(fx)->allocate(need) : nullptr;
+      abi_check(dyhip_csum_backward(dev.hip, M, 1, static_cast<unsigned>(N), dEdf.v, 0, dEdxi.v, ws, need));
+      scratch(fx)->free();
+    } else if (i == 1) {
+      abi_check(dyhip_gemm_nt_acc(dev.hip, M, K, N, dEdf.v, xs[2]->v, dEdxi.v));  // MatrixMultiplyTranspAcc
+    } else {
+      abi_check(dyhip_gemm_tn_acc(dev.hip, K, N, M, xs[1]->v, dEdf.v, dEdxi.v));  // MatrixTranspMultiplyAcc
+    }
+  }
+};
+
+// dynet/matrix-multiply.h:16-37,97-117,162-180 on Device_GPU (unbatched left operand)
+inline void MatrixMultiply(const Device_GPU& dev, const Tensor& l, const Tensor& r, Tensor& y, const float* acc_scalar) {
+  abi_check(dyhip_gemm_nn(dev.hip, l.d.rows(), size_t(r.d.cols()) * r.d.bd, l.d.cols(), l.v, r.v,
+                          acc_scalar == dev.kSCALAR_ONE ? 1.0f : 0.0f, y.v));
+}
+inline void MatrixTranspMultiplyAcc(const Device_GPU& dev, const Tensor& l, const Tensor& r, Tensor& y) {
+  abi_check(dyhip_gemm_tn_acc(dev.hip, l.d.cols(), size_t(r.d.cols()) * r.d.bd, l.d.rows(), l.v, r.v, y.v));
+}
+inline void MatrixMultiplyTranspAcc(const Device_GPU& dev, const Tensor& l, const Tensor& r, Tensor& y) {
+  abi_check(dyhip_gemm_nt_acc(dev.hip, l.d.rows(), r.d.rows(), size_t(l.d.cols()) * l.d.bd, l.v, r.v, y.v));
+}
+
+// dynet::gpu::* (dynet/gpu-ops.h:9-15): same argument lists behind the device
+namespace gpu {
+inline void dense_to_sparse_assign(const Device_GPU& dev, int n, const unsigned* ids, float* src, float* trg) {
+  abi_check(dyhip_dense_to_sparse_assign(dev.hip, n, ids, src, trg));
+}
+inline void sparse_to_dense_assign(const Device_GPU& dev, int n, const unsigned* ids, float* src, float* trg) {
+  abi_check(dyhip_sparse_to_dense_assign(dev.hip, n, ids, src, trg));
+}
+inline void dense_to_sparse_subtract(const Device_GPU& dev, int n, const unsigned* ids, float* src, float* trg) {
+  abi_check(dyhip_dense_to_sparse_subtract(dev.hip, n, ids, src, trg));
+}
+}  // namespace gpu
+
+}  // namespace dynet_hip
