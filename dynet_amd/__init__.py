@@ -8,6 +8,6 @@ importing works anywhere (so that the symbol table can be checked), but creating
 a device without a GPU raises.
 """
 from . import lib  # noqa: F401
-from .device import Device, DevTensor, DyhipError  # noqa: F401
+from .device import Device, DevTensor, DyhipError, PinnedArray  # noqa: F401
 
-__all__ = ["lib", "Device", "DevTensor", "DyhipError"]
+__all__ = ["lib", "Device", "DevTensor", "DyhipError", "PinnedArray"]

@@ -431,6 +431,21 @@ int dyhip_memcpy_h2d(dyhip_device* dev, void* dst, const void* src_host, size_t 
   return DYHIP_OK;
 }
 
+int dyhip_host_alloc(size_t nbytes, void** out) {
+  DYHIP_REQUIRE(out != nullptr && nbytes > 0, "null output pointer or empty allocation");
+  void* p = nullptr;
+  const hipError_t e = hipHostMalloc(&p, nbytes, hipHostMallocDefault);
+  if (e != hipSuccess) return fail(DYHIP_ERR_OUT_OF_MEMORY, "hipHostMalloc(%zu) failed: %s", nbytes, hipGetErrorString(e));
+  *out = p;
+  return DYHIP_OK;
+}
+
+int dyhip_host_free(void* p) {
+  if (p == nullptr) return DYHIP_OK;
+  DYHIP_CHECK_HIP(hipHostFree(p));
+  return DYHIP_OK;
+}
+
 int dyhip_memcpy_d2h(dyhip_device* dev, void* dst_host, const void* src, size_t nbytes) {
   DYHIP_CHECK_DEV(dev);
   if (nbytes == 0) return DYHIP_OK;

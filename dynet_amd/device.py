@@ -86,6 +86,30 @@ def _p(t):
     return _vp(int(t))
 
 
+class PinnedArray:
+    """A page-locked host array (numpy view over dyhip_host_alloc memory) for asynchronous host->device copies."""
+
+    def __init__(self, shape, dtype=np.float32):
+        self.shape, self.dtype = tuple(int(s) for s in shape), np.dtype(dtype)
+        self.nbytes = int(np.prod(self.shape)) * self.dtype.itemsize
+        p = _vp(None)
+        _check(cdll.dyhip_host_alloc(_sz(max(self.nbytes, 1)), C.byref(p)))
+        self.ptr = p.value
+        self.array = np.frombuffer((C.c_char * self.nbytes).from_address(self.ptr), dtype=self.dtype).reshape(self.shape)
+
+    def close(self):
+        if self.ptr:
+            self.array = None
+            cdll.dyhip_host_free(_vp(self.ptr))
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 class Device:
     """One GPU: stream, pools, scalars.  ``mem_mb`` = MiB for (FXS, DEDFS, PS, SCS)."""
 
@@ -185,6 +209,10 @@ class Device:
         ms = _f(0)
         _check(cdll.dyhip_timer_stop(self.handle, C.byref(ms)))
         return ms.value
+
+    def copy_h2d_async(self, dst, pinned):
+        """Queue a copy from a PinnedArray; the array must not change until the copy has run."""
+        _check(cdll.dyhip_memcpy_h2d(self.handle, _p(dst), _vp(pinned.ptr), _sz(pinned.nbytes)))
 
     def copy_d2d(self, dst, src, nbytes):
         _check(cdll.dyhip_memcpy_d2d(self.handle, _p(dst), _p(src), _sz(int(nbytes))))

@@ -77,6 +77,11 @@ class LstmLM:
         self.queues = [dev] + ([dev.fork() for _ in range(L - 1)] if self.overlap else [])
         self.plan, self.plan_ws, self.plan_ws_bytes = dev.lookup_plan_buffers(N, V)
         self.graph = None
+        # page-locked staging for the ids and the flattened label offsets, two sets used in turn: a set is
+        # rewritten only after a device sync that follows the copy that read it
+        from .device import PinnedArray
+        self._stage = [(PinnedArray((N,), np.uint32), PinnedArray((N,), np.uint32)) for _ in range(2)]
+        self._stage_at = 0
 
     @staticmethod
     def init_params(V, E, H, L, seed=0):
@@ -98,16 +103,22 @@ class LstmLM:
 
     # ---- one step ---------------------------------------------------------------
     def stage(self, tokens):
-        """Host -> device: tokens[T+1, B]; rows 0..T-1 are the inputs, rows 1..T the words to predict."""
+        """Host -> device: tokens[T+1, B]; rows 0..T-1 are the inputs, rows 1..T the words to predict.
+        Asynchronous copies from page-locked staging buffers; the host blocks only every second call."""
         tokens = np.ascontiguousarray(tokens, dtype=np.uint32)
         assert tokens.shape == (self.T + 1, self.B), tokens.shape
         if tokens.max() >= self.V:
             raise ValueError("token id out of the vocabulary")
-        self.ids.set(tokens[:-1].reshape(-1))
-        flat = np.arange(self.N, dtype=np.uint64) * self.V + tokens[1:].reshape(-1)
-        if flat.max() >= 2 ** 32:
+        if self.N * self.V > 2 ** 32:
             raise ValueError("PickNegLogSoftmax indexes its input with 32-bit offsets")
-        self.aux.offset(2 * self.N, (self.N,)).set(flat.astype(np.uint32).view(np.float32))
+        if self._stage_at == 0:
+            self.dev.sync()  # both staging sets are free again
+        ids, flat = self._stage[self._stage_at]
+        self._stage_at ^= 1
+        ids.array[:] = tokens[:-1].reshape(-1)
+        flat.array[:] = (np.arange(self.N, dtype=np.uint64) * self.V + tokens[1:].reshape(-1)).astype(np.uint32)
+        self.dev.copy_h2d_async(self.ids, ids)
+        self.dev.copy_h2d_async(self.aux.offset(2 * self.N, (self.N,)), flat)
 
     def _t(self, buf, t, width):
         return buf.offset(t * self.B * width, (self.B, width))

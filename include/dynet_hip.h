@@ -96,6 +96,12 @@ int dyhip_pool_num_blocks(dyhip_pool* pool, int* n);
  * (dynet/tensor.cc:66-93,106-229) ----------------------------------------- */
 int dyhip_memcpy_h2d(dyhip_device* dev, void* dst, const void* src_host, size_t nbytes);
 int dyhip_memcpy_d2h(dyhip_device* dev, void* dst_host, const void* src, size_t nbytes); /* blocking */
+/* Page-locked host staging memory.  dyhip_memcpy_h2d from such a buffer is asynchronous: the buffer
+ * must stay untouched until the copy has run (dyhip_device_sync or any later blocking call).  The
+ * reference stages ids and pointer tables from pageable memory (dynet/param-nodes.cc:318,
+ * dynet/exec.cc:351-355), which makes every such copy a synchronisation point. */
+int dyhip_host_alloc(size_t nbytes, void** out);
+int dyhip_host_free(void* p);
 int dyhip_memcpy_d2d(dyhip_device* dev, void* dst, const void* src, size_t nbytes);
 int dyhip_zero(dyhip_device* dev, void* dst, size_t nbytes);
 int dyhip_constant(dyhip_device* dev, size_t n, float value, float* dst);       /* TensorTools::constant */
