@@ -433,8 +433,8 @@ def cpu_baseline(step_bytes, seconds):
 def main():
     args = parse_args()
     if args.gpus != 1:
-        print("bench.py measures one GPU: every box of this build has one, and the hot path has no multi-GPU "
-              "leg (see DESIGN.md, 'How the path would shard'). Run with --gpus 1.", file=sys.stderr)
+        print("bench.py measures one GPU: the hot path has no multi-GPU leg (it would shard along the batch "
+              "dimension with one gradient all-reduce per step). Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
     from dynet_amd import Device, lib
 
