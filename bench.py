@@ -269,7 +269,34 @@ def extras(dev, lib, reps, use_graph=True):
     else:
         us = time_loop(dev, [cell], max(reps, 50))
     res["cfg1_lstm_cell"] = {"I": I, "H": H, "B": B, "fwd_bwd_us": round(us, 2), "launches": 13 + 5,
-                             "gemm_flops": 3 * 2 * 4 * H * (I + H) * B}
+                             "gemm_flops": 3 * 2 * 4 * H * (I + H) * B,
+                             "path": "VanillaLSTMGates / C / H nodes, every backward argument"}
+    # the same step through the fused cell entry points
+    fb, bb = dev.lstm_cell_workspace(H, B)
+    wf, _ = dev.workspace(fb)
+    wb, _ = dev.workspace(bb)
+    xproj, dcp2 = dev.empty((B, 4 * H)), dev.empty((B, H))
+
+    def cell_fused():
+        dev.gemm_nn(4 * H, B, I, t["Wx"], t["x"], 0.0, xproj)
+        n = dev.lstm_recurrent_forward(H, B, t["Wh"], t["h"], wf, fb)
+        dev.lstm_cell_forward(H, B, xproj, t["b"], wf, n, t["c"], fx, c2, h2)
+        dev.lstm_cell_backward(H, B, fx, c2, t["c"], t["dh"], None, 0, t["dc"], dpre, dcp2)
+        dev.lstm_recurrent_backward(H, B, t["Wh"], dpre, wb, bb)       # d h_prev as split-K slices
+        dev.gemm_tn(I, B, 4 * H, t["Wx"], dpre, 1.0, dx)
+        dev.gemm_nt_acc(4 * H, I, B, dpre, t["x"], dWx)
+        dev.gemm_nt_acc(4 * H, H, B, dpre, t["h"], dWh)
+        dev.csum_backward(4 * H, 1, B, dpre, 0, db)
+
+    cell_fused()
+    dev.sync()
+    if use_graph:
+        g = capture(dev, [cell_fused])
+        us2 = time_graph(dev, g, max(reps, 50), 1)
+        g.destroy()
+    else:
+        us2 = time_loop(dev, [cell_fused], max(reps, 50))
+    res["cfg1_lstm_cell"]["fused_cell_path_fwd_bwd_us"] = round(us2, 2)
     return res
 
 
