@@ -60,6 +60,7 @@ def parse_args():
     ap.add_argument("--no-extras", action="store_true", help="skip the cfg 1 / 3 / 4 kernel measurements")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="bound on the CPU-baseline leg")
     ap.add_argument("--no-lm", action="store_true", help="skip the cfg 5 LSTM-LM training-step measurement")
+    ap.add_argument("--no-large", action="store_true", help="skip the 16x larger repeat of the cfg 2 sweep")
     ap.add_argument("--lm-steps", type=int, default=30)
     return ap.parse_args()
 
@@ -67,20 +68,26 @@ def parse_args():
 class Sweep:
     """The cfg-2 sweep: buffers for R rotating sets and the list of kernels."""
 
-    def __init__(self, dev, lib, sets, seed=0):
+    def __init__(self, dev, lib, sets, seed=0, scale=1):
+        """scale multiplies the number of rows / batch elements (1 = the baseline's 4096 x 1024 tensor)."""
         self.dev, self.lib, self.R = dev, lib, sets
+        S_ELEMS, LN_BD, SB_BD = globals()["S_ELEMS"] * scale, globals()["LN_BD"] * scale, globals()["SB_BD"] * scale
+        S_BYTES = S_ELEMS * 4
+        self.elems = S_ELEMS
         rng = np.random.default_rng(seed)
         self.g = dev.tensor(rng.uniform(0.5, 1.5, LN_N).astype(np.float32), pool=lib.POOL_PS)
         self.b = dev.tensor((rng.standard_normal(LN_N) * 0.1).astype(np.float32), pool=lib.POOL_PS)
         self.dg = dev.zeros(LN_N, pool=lib.POOL_PS)
         self.db = dev.zeros(LN_N, pool=lib.POOL_PS)
         self.sets = []
+        host = [rng.standard_normal(S_ELEMS).astype(np.float32) for _ in range(3)] if scale > 1 else None
         for _ in range(sets):
+            draw = (lambda k: host[k]) if host else (lambda k: rng.standard_normal(S_ELEMS).astype(np.float32))
             s = {
-                "x": dev.tensor(rng.standard_normal(S_ELEMS).astype(np.float32)),
-                "x2": dev.tensor(rng.standard_normal(S_ELEMS).astype(np.float32)),
+                "x": dev.tensor(draw(0)),
+                "x2": dev.tensor(draw(1)),
                 "y": dev.empty(S_ELEMS),
-                "dy": dev.tensor(rng.standard_normal(S_ELEMS).astype(np.float32)),
+                "dy": dev.tensor(draw(2)),
                 "dx": dev.zeros(S_ELEMS, pool=lib.POOL_DEDFS),
                 "s": dev.empty(SB_N),
             }
@@ -115,7 +122,7 @@ class Sweep:
     def _cmult_bwd(self, b, i):
         from dynet_amd.device import _check, _p, _sz, _u, _vp, cdll
 
-        _check(cdll.dyhip_cmult_backward(self.dev.handle, _sz(S_ELEMS), _u(1), _u(1), _p(b["x"]), _p(b["x2"]),
+        _check(cdll.dyhip_cmult_backward(self.dev.handle, _sz(self.elems), _u(1), _u(1), _p(b["x"]), _p(b["x2"]),
                                          _p(b["dy"]), _u(i), _p(b["dx"]), _vp(None), _sz(0)))
 
     def run_step(self, r):
@@ -535,6 +542,18 @@ def main():
     if not args.no_extras:
         out.update(extras(dev, lib, args.kernel_reps, use_graph=not args.no_graph))
     dev.close()
+    if not args.no_large:
+        # the same kernels on tensors 16 times larger (65536 x 1024 fp32, 268 MB each): how much of the gap to the
+        # HBM peak at the baseline's shape is the fixed cost of a launch
+        dev = Device(0, mem_mb=(3584, 1280, 64, 256))
+        if args.stream_threshold is not None:
+            dev.set_stream_threshold(args.stream_threshold)
+        big = Sweep(dev, lib, 2, scale=16)
+        out["cfg2_sweep_16x_larger_tensors"] = {
+            "tensor": "65536x1024 fp32", "rotating_buffer_sets": big.R,
+            "kernels": per_kernel_table(dev, big.kernels, big.sets, max(4, args.kernel_reps // 4),
+                                        use_graph=not args.no_graph)}
+        dev.close()
     if not args.no_lm:
         out["cfg5_lstm_lm"] = lstm_lm(args.lm_steps, use_graph=not args.no_graph)
         out["cfg5_lstm_lm"]["in_situ"] = lm_kernels(args.kernel_reps, use_graph=not args.no_graph)
