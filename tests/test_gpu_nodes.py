@@ -575,6 +575,34 @@ def test_device_side_clipping_and_sparse_rows(dev):
     assert not g2t.numpy().any()
 
 
+def test_zero_sized_calls_are_no_ops(dev):
+    """Empty tensors (a batch of zero columns, zero ids, K = 0) must not launch anything or fail."""
+    sentinel = f32(np.arange(8))
+    t = dev.tensor(sentinel)
+    e = dev.empty((0,))
+    dev.unary_forward(lib.OP_TANH, e, e, n=0)
+    dev.unary_backward(lib.OP_TANH, e, e, e, n=0)
+    dev.cmult_forward(0, 1, 1, e, e, e)
+    dev.scale_copy(0, e, 2.0, e)
+    dev.sgd_update(0, e, e, 0.1)
+    dev.lookup_forward(None, dev.empty((0,), np.uint32), 4, 10, t, e)
+    dev.pnls_forward_staged(5, 0, e, e, e)
+    dev.pnls_backward(5, 0, e, e, e, e)
+    dev.logsumexp_cols(5, 0, e, e, e)
+    dev.gemm_nn(0, 3, 4, e, t, 0.0, e)
+    dev.gemm_nn(3, 0, 4, t, e, 0.0, e)
+    # K = 0: y = beta * y
+    y = dev.tensor(f32([1, 2, 3, 4, 5, 6]))
+    dev.gemm_nn(3, 2, 0, t, t, 1.0, y)
+    assert y.numpy().tobytes() == f32([1, 2, 3, 4, 5, 6]).tobytes()
+    dev.gemm_nn(3, 2, 0, t, t, 0.0, y)
+    assert not y.numpy().any()
+    dev.layer_norm_forward(4, 0, e, t, t, e)
+    dev.sum_forward(0, 3, [e], [3], e)
+    dev.sync()
+    assert t.numpy().tobytes() == sentinel.tobytes()
+
+
 def test_forked_queue_ordering_and_errors(dev):
     """dyhip_device_fork / dyhip_device_wait: a chain that hops between two queues sees every earlier write."""
     rng = np.random.default_rng(20)
