@@ -334,7 +334,8 @@ def lstm_lm(steps, warmup=3, use_graph=True):
                       "clip_threshold": 5.0, "init": "Glorot (lookup: embedding dim only), LSTM biases 0",
                       "ids": "Zipf(1.1)"},
            "tokens_per_step": T * B, "gemm_flop_per_step": flops,
-           "fused_path_schedule": "layers pipelined over two device queues in chunks of 7 timesteps",
+           "fused_path_schedule": "layers pipelined over two device queues in chunks of 7 timesteps; forward "
+                                  "timesteps are one kernel each (recurrent product + cell update)",
            "timed_region": "per step: host->device copy of ids and labels, id sort, forward, backward, "
                            "device-side clipping, update; one HIP-graph replay per step; loss read back after "
                            "the last step"}
@@ -422,6 +423,26 @@ def lm_kernels(reps, use_graph=True):
              ("lstm_cell_bwd (%d slices)" % nb, ((4 + 4 + nb + 4 + 1) * H * B) * 4,
               lambda s: dev.lstm_cell_backward(H, B, g, c2, c, dh, wb, nb, dc, dpre, dc2))]
     out["kernels"] = per_kernel_table(dev, named, [None] * 4, reps, use_graph=use_graph)
+    # single-launch forward timestep: product and cell update in one kernel, Wh read from its packed copy
+    pk = dev.empty((4 * H * H,))
+    dev.lstm_pack_recurrent(H, Wh, pk)
+    step = lambda: dev.lstm_step_forward(H, B, pk, h, xp, bb_, c, g, c2, hh)
+    pack = lambda: dev.lstm_pack_recurrent(H, Wh, pk)
+    for name, fn, flops, nbytes in (("lstm_step_fwd (recurrent product + cell update)", step, 2.0 * 4 * H * H * B,
+                                     (4 * H * H + H * B + 4 * H * B + 4 * H + H * B + 6 * H * B) * 4),
+                                    ("lstm_pack_recurrent (once per layer per step)", pack, 0.0, 2 * 4 * H * H * 4)):
+        if use_graph:
+            gr = capture(dev, [fn] * 4)
+            us = time_graph(dev, gr, reps, 4)
+            gr.destroy()
+        else:
+            us = time_loop(dev, [fn], reps)
+        row = {"kernel": name, "bytes": nbytes, "us": round(us, 3), "GBps": round(nbytes / us / 1e3, 1),
+               "frac_of_8TBps": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+        if flops:
+            row["TFLOPs"] = round(flops / us / 1e6, 1)
+            row["frac_of_fp32_mfma_peak"] = round(flops / us / 1e6 / FP32_MFMA_PEAK_TFLOPS, 4)
+        out["kernels"].append(row)
     dev.close()
     return out
 

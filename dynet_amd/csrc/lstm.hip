@@ -219,6 +219,151 @@ __global__ __launch_bounds__(kCellThreads) void lstm_cell_bwd_kernel(unsigned H,
   if (dc_prev) dcp.store(dc_prev + s0);
 }
 
+// ---- single-launch forward step: recurrent product and cell update in one kernel -------
+// A block owns 8 hidden units x 32 batch columns.  Its 32 weight rows are the four gate
+// rows (i, f, o, g) of those 8 units, so after the product all four pre-activations of a
+// hidden unit sit in the same block and the cell update runs in the epilogue: the 4H x B
+// product never goes to memory.  The four waves split the H-deep sum in quarters, each
+// streaming its quarter through a private double-buffered LDS stage into 32x32x2 MFMAs,
+// and the quarters meet in LDS.
+//
+// The weights are read from a packed copy Wp[H/8][H][32]: tile rt, column k holds the 32
+// rows {g*H + rt*8 + u : g < 4, u < 8} at index g*8 + u, which makes a wave's stage one
+// contiguous 4 KiB run.  Blocks of one row tile are H/8 apart in launch order, so with
+// H/8 a multiple of 8 they land on the same XCD and share that L2's copy of the tile.
+constexpr int kStepBK = 32;                 // k depth of one LDS stage
+constexpr int kStepPitchB = 34;             // B stage: [k][col], 2-way conflicts at most on the transposing write
+constexpr int kStepPitchR = 33;             // quarter-sum exchange: [row][col]
+constexpr int kStepWaveFloats = 2 * 32 * kStepBK + 2 * kStepBK * kStepPitchB;  // per-wave A + B stages
+typedef float stepx16 __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(256) void lstm_pack_recurrent_kernel(unsigned H, const float* __restrict__ Wh,
+                                                                  float* __restrict__ Wp) {
+  const size_t o = size_t(blockIdx.x) * 256 + threadIdx.x;  // output index, (rt*H + k)*32 + g*8 + u
+  if (o >= size_t(4) * H * H) return;
+  const unsigned r = o % 32, g = r / 8, u = r % 8;
+  const size_t tk = o / 32;
+  const unsigned k = tk % H, rt = tk / H;
+  Wp[o] = Wh[size_t(g) * H + rt * 8 + u + size_t(k) * 4 * H];
+}
+
+// orders a wave's LDS writes before the reads its other lanes issue afterwards
+__device__ __forceinline__ void step_wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+__global__ __launch_bounds__(256, 2) void lstm_step_fwd_kernel(unsigned H, unsigned B, const float* __restrict__ Wp,
+                                                               const float* __restrict__ h_prev,
+                                                               const float* xproj,
+                                                               const float* __restrict__ bias,
+                                                               const float* __restrict__ c_prev, int mode,
+                                                               float* gates, float* __restrict__ c,
+                                                               float* __restrict__ h) {
+  __shared__ __attribute__((aligned(16))) float lds[4 * kStepWaveFloats];
+  const unsigned RT = H / 8;
+  const unsigned rt = blockIdx.x % RT, ct = blockIdx.x / RT;
+  const unsigned wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const unsigned l32 = lane % 32, lhi = lane / 32;
+  float* la = lds + wave * kStepWaveFloats;
+  float* lb = la + 2 * 32 * kStepBK;
+  const unsigned kq = H / 4, k0 = wave * kq, nst = kq / kStepBK;
+
+  const float* ga = Wp + (size_t(rt) * H + k0) * 32 + lane * 4;
+  const unsigned bk = 4 * (lane % 8), bc = lane / 8;
+  // columns past the batch are computed on a clamped address and dropped
+  auto column = [&](unsigned i) {
+    const unsigned col = ct * 32 + bc + 8 * i;
+    return h_prev + size_t(col < B ? col : B - 1) * H + k0 + bk;
+  };
+  const float *gb0 = column(0), *gb1 = column(1), *gb2 = column(2), *gb3 = column(3);
+
+  // the epilogue's thread owns hidden unit eu of batch column ecc; its operands are fetched
+  // now so that their latency hides behind the product
+  const unsigned eu = threadIdx.x % 8, ecc = threadIdx.x / 8;
+  const unsigned ecol = ct * 32 + ecc, ej = rt * 8 + eu;
+  float pre[4] = {0.f, 0.f, 0.f, 0.f}, cp = 0.f;
+  if (ecol < B) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float bq = bias[q * H + ej];
+      pre[q] = (q == 1 ? bq + 1.0f : bq) + xproj[size_t(ecol) * 4 * H + ej + size_t(q) * H];
+    }
+    cp = c_prev[size_t(ecol) * H + ej];
+  }
+
+  float4 ra0, ra1, ra2, ra3, rb0, rb1, rb2, rb3;
+#define STEP_LOAD1(i, st)                                                                  \
+  ra##i = *reinterpret_cast<const float4*>(ga + size_t(st) * 32 * kStepBK + i * 256);      \
+  rb##i = *reinterpret_cast<const float4*>(gb##i + (st) * kStepBK);
+#define STEP_LOAD(st) STEP_LOAD1(0, st) STEP_LOAD1(1, st) STEP_LOAD1(2, st) STEP_LOAD1(3, st)
+#define STEP_STORE1(i)                                                                     \
+  *reinterpret_cast<float4*>(a_ + i * 256) = ra##i;                                        \
+  b_[0 * kStepPitchB + 8 * i] = rb##i.x;                                                   \
+  b_[1 * kStepPitchB + 8 * i] = rb##i.y;                                                   \
+  b_[2 * kStepPitchB + 8 * i] = rb##i.z;                                                   \
+  b_[3 * kStepPitchB + 8 * i] = rb##i.w;
+#define STEP_STORE(buf)                                                                    \
+  {                                                                                        \
+    float* a_ = la + (buf) * 32 * kStepBK + lane * 4;                                      \
+    float* b_ = lb + (buf) * kStepBK * kStepPitchB + bk * kStepPitchB + bc;                \
+    STEP_STORE1(0) STEP_STORE1(1) STEP_STORE1(2) STEP_STORE1(3)                            \
+  }
+
+  // The kernel runs at the rate the L2 delivers the operands (every 32x32 output tile pulls
+  // its full-depth strips of both), so one stage of lookahead is enough.
+  stepx16 acc = {0};
+  STEP_LOAD(0)
+  STEP_STORE(0)
+  if (nst > 1) { STEP_LOAD(1) }
+  step_wave_sync();
+  for (unsigned st = 0; st < nst; ++st) {
+    const unsigned cur = st & 1;
+    const float* a = la + cur * 32 * kStepBK + lhi * 32 + l32;
+    const float* b = lb + cur * kStepBK * kStepPitchB + lhi * kStepPitchB + l32;
+#pragma unroll
+    for (int s = 0; s < kStepBK / 2; ++s)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * s * 32], b[2 * s * kStepPitchB], acc, 0, 0, 0);
+    if (st + 1 < nst) {
+      STEP_STORE(cur ^ 1)
+      if (st + 2 < nst) { STEP_LOAD(st + 2) }
+    }
+    step_wave_sync();  // the stages are private to the wave: no block barrier in the loop
+  }
+  __syncthreads();
+#undef STEP_LOAD1
+#undef STEP_LOAD
+#undef STEP_STORE1
+#undef STEP_STORE
+
+  // the four quarter sums meet in LDS (the stages are dead after the last barrier)
+  float* red = lds;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const unsigned row = 8 * (r / 4) + 4 * lhi + (r % 4);
+    red[(wave * 32 + row) * kStepPitchR + l32] = acc[r];
+  }
+  __syncthreads();
+
+  if (ecol >= B) return;
+  const size_t g0 = size_t(ecol) * 4 * H + ej, s0 = size_t(ecol) * H + ej;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+#pragma unroll
+    for (int w = 0; w < 4; ++w) pre[q] += red[(w * 32 + q * 8 + eu) * kStepPitchR + ecc];
+  }
+  const float gi = logistic(mode, pre[0]), gf = logistic(mode, pre[1]), go = logistic(mode, pre[2]);
+  const float gg = tanh_accurate(pre[3]);
+  const float cv = gi * gg + gf * cp;
+  gates[g0] = gi;
+  gates[g0 + H] = gf;
+  gates[g0 + 2 * size_t(H)] = go;
+  gates[g0 + 3 * size_t(H)] = gg;
+  c[s0] = cv;
+  h[s0] = go * tanh_accurate(cv);
+}
+
 static bool all_aligned16(std::initializer_list<const void*> ps) {
   for (const void* p : ps)
     if (p != nullptr && !aligned16(p)) return false;
@@ -522,6 +667,45 @@ int dyhip_lstm_cell_backward(dyhip_device* dev, unsigned H, unsigned B, const fl
   else
     hipLaunchKernelGGL(lstm_cell_bwd_kernel<1>, dim3(cdiv<unsigned>(H, kCellThreads), B), dim3(kCellThreads), 0,
                        dev->stream, H, splits, slice, gates, c, c_tm1, dh, rec, dc, dpre, dc_tm1);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_lstm_step_supported(dyhip_device* dev, unsigned H, unsigned B, int* supported) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(supported, "null output pointer");
+  // quarters of the hidden size in whole 32-deep stages; grid and index ranges in 32 bits
+  *supported = (H >= 128 && H % 128 == 0 && B >= 1 && B <= 65535 && size_t(4) * H * H < (size_t(1) << 32)) ? 1 : 0;
+  return DYHIP_OK;
+}
+
+int dyhip_lstm_pack_recurrent(dyhip_device* dev, unsigned H, const float* Wh, float* packed) {
+  DYHIP_CHECK_DEV(dev);
+  int ok = 0;
+  dyhip_lstm_step_supported(dev, H, 1, &ok);
+  DYHIP_REQUIRE(ok, "LSTM step: hidden size %u is not a multiple of 128", H);
+  DYHIP_REQUIRE(Wh && packed, "LSTM step: null tensor pointer");
+  const size_t n = size_t(4) * H * H;
+  hipLaunchKernelGGL(lstm_pack_recurrent_kernel, dim3(unsigned(cdiv<size_t>(n, 256))), dim3(256), 0, dev->stream, H, Wh,
+                     packed);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_lstm_step_forward(dyhip_device* dev, unsigned H, unsigned B, const float* packed_Wh, const float* h_tm1,
+                            const float* xproj, const float* b, const float* c_tm1, int logistic_mode, float* gates,
+                            float* c, float* h) {
+  DYHIP_CHECK_DEV(dev);
+  int ok = 0;
+  dyhip_lstm_step_supported(dev, H, B, &ok);
+  DYHIP_REQUIRE(ok, "LSTM step: unsupported hidden (%u) or batch (%u) size", H, B);
+  DYHIP_REQUIRE(packed_Wh && h_tm1 && xproj && b && c_tm1 && gates && c && h, "LSTM step: null tensor pointer");
+  DYHIP_REQUIRE(aligned16(packed_Wh) && aligned16(h_tm1), "LSTM step: packed weights and h_tm1 must be 16-byte aligned");
+  DYHIP_REQUIRE(logistic_mode == DYHIP_LOGISTIC_PACKET || logistic_mode == DYHIP_LOGISTIC_SCALAR,
+                "unknown logistic mode %d", logistic_mode);
+  const unsigned blocks = (H / 8) * cdiv<unsigned>(B, 32);
+  hipLaunchKernelGGL(lstm_step_fwd_kernel, dim3(blocks), dim3(256), 0, dev->stream, H, B, packed_Wh, h_tm1, xproj, b,
+                     c_tm1, logistic_mode, gates, c, h);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }

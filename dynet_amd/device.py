@@ -383,6 +383,19 @@ class Device:
         _check(cdll.dyhip_lstm_cell_forward(self.handle, _u(H), _u(B), _p(xproj), _p(b), _vp(rec), _u(splits),
                                             _p(c_tm1), _i(logistic_mode), _p(gates), _p(c), _p(h)))
 
+    def lstm_step_supported(self, H, B):
+        ok = C.c_int(0)
+        _check(cdll.dyhip_lstm_step_supported(self.handle, _u(H), _u(B), C.byref(ok)))
+        return bool(ok.value)
+
+    def lstm_pack_recurrent(self, H, Wh, packed):
+        _check(cdll.dyhip_lstm_pack_recurrent(self.handle, _u(H), _p(Wh), _p(packed)))
+
+    def lstm_step_forward(self, H, B, packed_Wh, h_tm1, xproj, b, c_tm1, gates, c, h,
+                          logistic_mode=lib.LOGISTIC_PACKET):
+        _check(cdll.dyhip_lstm_step_forward(self.handle, _u(H), _u(B), _p(packed_Wh), _p(h_tm1), _p(xproj), _p(b),
+                                            _p(c_tm1), _i(logistic_mode), _p(gates), _p(c), _p(h)))
+
     def lstm_cell_backward(self, H, B, gates, c, c_tm1, dh, rec, splits, dc, dpre, dc_tm1):
         _check(cdll.dyhip_lstm_cell_backward(self.handle, _u(H), _u(B), _p(gates), _p(c), _p(c_tm1), _p(dh), _vp(rec),
                                              _u(splits), _p(dc), _p(dpre), _p(dc_tm1)))

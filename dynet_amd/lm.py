@@ -29,7 +29,7 @@ class LstmLM:
     """V-word LM: embedding E, L layers of hidden H, batch B, T timesteps per step."""
 
     def __init__(self, dev, V, E, H, L, B, T, seed=0, lr=0.1, clip=5.0, time_batched=True, params=None, path="fused",
-                 overlap=None, chunk=7):
+                 overlap=None, chunk=7, single_launch=None):
         assert path in ("fused", "nodes")
         self.overlap = (L > 1) if overlap is None else bool(overlap)
         self.overlap = self.overlap and path == "fused" and L > 1
@@ -73,6 +73,10 @@ class LstmLM:
         self.rec_f_bytes, self.rec_b_bytes = fb, bb
         self.rec_f = [dev.workspace(fb)[0] for _ in range(L)]  # one per layer: layers run side by side
         self.rec_b = [dev.workspace(bb)[0] for _ in range(L)]
+        # forward timesteps as one kernel each (recurrent product + cell update) where the size allows
+        ok = path == "fused" and dev.lstm_step_supported(H, B)
+        self.single_launch = ok if single_launch is None else (bool(single_launch) and ok)
+        self.Wh_packed = [dev.empty((4 * H * H,), pool=PS) for _ in range(L)] if self.single_launch else []
         # queue l runs layer l; queue 0 is the device itself
         self.queues = [dev] + ([dev.fork() for _ in range(L - 1)] if self.overlap else [])
         self.plan, self.plan_ws, self.plan_ws_bytes = dev.lookup_plan_buffers(N, V)
@@ -141,7 +145,10 @@ class LstmLM:
         H, B = self.H, self.B
         for t in range(t0, t1):
             g = self._t(self.gates[l], t, 4 * H)
-            if t > 0:
+            if t > 0 and self.single_launch:
+                q.lstm_step_forward(H, B, self.Wh_packed[l], self._t(self.h[l], t - 1, H), g, self.p[f"b{l}"],
+                                    self._t(self.c[l], t - 1, H), g, self._t(self.c[l], t, H), self._t(self.h[l], t, H))
+            elif t > 0:
                 n = q.lstm_recurrent_forward(H, B, self.p[f"Wh{l}"], self._t(self.h[l], t - 1, H), self.rec_f[l],
                                              self.rec_f_bytes)
                 q.lstm_cell_forward(H, B, g, self.p[f"b{l}"], self.rec_f[l], n, self._t(self.c[l], t - 1, H), g,
@@ -152,6 +159,9 @@ class LstmLM:
 
     def _forward_layers_fused(self):
         d, E, H, L, B, T, N = self.dev, self.E, self.H, self.L, self.B, self.T, self.N
+        if self.single_launch:  # the weights moved in the last update
+            for l in range(L):
+                d.lstm_pack_recurrent(H, self.p[f"Wh{l}"], self.Wh_packed[l])
         if not self.overlap:
             for l in range(L):
                 x, d_in = (self.h[l - 1], H) if l > 0 else (self.emb, E)

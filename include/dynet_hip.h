@@ -261,6 +261,20 @@ int dyhip_lstm_cell_backward(dyhip_device* dev, unsigned H, unsigned B, const fl
                              const float* c_tm1, const float* dh, const float* rec, unsigned splits, const float* dc,
                              float* dpre, float* dc_tm1);
 
+/* Single-launch form of a forward timestep (t >= 1): the recurrent product Wh * h_tm1 and
+ * the cell update of dyhip_lstm_cell_forward in one kernel, the product staying on chip.
+ * A block owns 8 hidden units, i.e. the gate rows j, H+j, 2H+j, 3H+j of the slicing in
+ * dynet/nodes-lstm.cc:213-223, which it reads from a packed copy of Wh laid out
+ * [H/8][H][4 gates x 8 units]: refresh it with dyhip_lstm_pack_recurrent (4*H*H floats)
+ * whenever Wh changes.  Supported when H is a multiple of 128 (dyhip_lstm_step_supported
+ * reports it; the two-call form above covers every other size).  Same results as the
+ * two-call form up to fp32 summation order.  gates may alias xproj. */
+int dyhip_lstm_step_supported(dyhip_device* dev, unsigned H, unsigned B, int* supported);
+int dyhip_lstm_pack_recurrent(dyhip_device* dev, unsigned H, const float* Wh, float* packed);
+int dyhip_lstm_step_forward(dyhip_device* dev, unsigned H, unsigned B, const float* packed_Wh, const float* h_tm1,
+                            const float* xproj, const float* b, const float* c_tm1, int logistic_mode, float* gates,
+                            float* c, float* h);
+
 /* ---- LookupNode (dynet/param-nodes.cc:304-329) and
  * LookupParameterStorage::accumulate_grads (dynet/model.cc:728-743) -------- */
 /* fx[:, b] = table[:, ids[b]] * mult; bit-exact gather when mult == 1.0f.

@@ -29,7 +29,8 @@ def _grad_floor(ref):
 
 
 @pytest.mark.parametrize("path,time_batched,overlap", [("nodes", False, False), ("nodes", True, False),
-                                                       ("fused", True, False), ("fused", True, True)])
+                                                       ("fused", True, False), ("fused", True, True),
+                                                       ("fused_two_call", True, True)])
 @pytest.mark.parametrize("case", CASES)
 def test_lm_step_matches_oracle(dev, case, path, time_batched, overlap):
     V, E, H, L, B, T = case
@@ -38,8 +39,10 @@ def test_lm_step_matches_oracle(dev, case, path, time_batched, overlap):
     for l in range(L):  # non-zero biases exercise the bias path
         params[f"b{l}"] = rng.normal(0, 0.1, 4 * H).astype(np.float32)
     ref_p = {n: a.copy() for n, a in params.items()}
-    lm = LstmLM(dev, V, E, H, L, B, T, lr=0.1, clip=5.0, time_batched=time_batched, params=params, path=path,
-                overlap=overlap, chunk=2)
+    # "fused" takes the single-launch forward step where the hidden size allows it (H = 128 here)
+    lm = LstmLM(dev, V, E, H, L, B, T, lr=0.1, clip=5.0, time_batched=time_batched, params=params,
+                path=path.split("_")[0], overlap=overlap, chunk=2, single_launch=None if path == "fused" else False)
+    assert lm.single_launch == (path == "fused" and H % 128 == 0)
     for it in range(2):
         tokens = _tokens(rng, V, B, T)
         ref_loss, ref_g, ref_scale = lm_oracle.step(ref_p, tokens, L, lr=0.1, clip=5.0)

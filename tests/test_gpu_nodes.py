@@ -278,6 +278,68 @@ def test_fused_cell_path_equals_node_composition(dev, I, H, B):
                      floor=max(float(np.abs(r_dpre[k]).max()) * 1e-2, 1e-6))
 
 
+@pytest.mark.parametrize("I,H,B", [(24, 128, 1), (40, 128, 33), (16, 256, 32), (64, 384, 70), (32, 1024, 128)])
+def test_single_launch_step_equals_node_composition(dev, I, H, B):
+    """dyhip_lstm_step_forward (recurrent product + cell update in one kernel, packed Wh) over three
+    timesteps against the oracle's VanillaLSTMGates -> C -> H nodes and against the two-call form."""
+    rng = np.random.default_rng(7 * I + H + B)
+    Wx, Wh, b = glorot(rng, 4 * H, I), glorot(rng, 4 * H, H), f32(rng.normal(0, 0.1, 4 * H))
+    T = 3
+    xs = [f32(rng.standard_normal((B, I))) for _ in range(T)]
+    zeros = np.zeros((B, H), F32)
+    ref = []
+    h_prev, c_prev = zeros, zeros
+    for x in xs:
+        g = orc.lstm_gates_forward([x], [I], H, B, h_prev, Wx, Wh, b)
+        c = orc.lstm_c_forward(H, B, c_prev, g)
+        h = orc.lstm_h_forward(H, B, c, g)
+        ref.append((g, c, h))
+        h_prev, c_prev = h, c
+    assert dev.lstm_step_supported(H, B)
+    Wxt, Wht, bt = dev.tensor(Wx), dev.tensor(Wh), dev.tensor(b)
+    packed = dev.empty(4 * H * H)
+    dev.lstm_pack_recurrent(H, Wht, packed)
+    # the packed copy is a permutation of Wh: tile rt, column k, slot g*8+u <- row g*H + rt*8 + u
+    want = Wh.reshape(H, 4, H // 8, 8).transpose(2, 0, 1, 3).reshape(-1)   # Wh is stored [k][row]
+    assert np.array_equal(packed.numpy(), want)
+    X = dev.tensor(np.stack(xs))
+    xproj = dev.empty((T, B, 4 * H))
+    dev.gemm_nn(4 * H, T * B, I, Wxt, X, 0.0, xproj)
+    sl = lambda t, k, w: t.offset(k * B * w, (B, w))
+    fb, _ = dev.lstm_cell_workspace(H, B)
+    wf, wfb = dev.workspace(fb)
+    out = {}
+    for name in ("step", "two_call"):
+        gates, cs, hs = dev.empty((T, B, 4 * H)), dev.empty((T, B, H)), dev.empty((T, B, H))
+        dev.lstm_cell_forward(H, B, sl(xproj, 0, 4 * H), bt, None, 0, None, sl(gates, 0, 4 * H), sl(cs, 0, H),
+                              sl(hs, 0, H))
+        for t in range(1, T):
+            if name == "step":
+                dev.lstm_step_forward(H, B, packed, sl(hs, t - 1, H), sl(xproj, t, 4 * H), bt, sl(cs, t - 1, H),
+                                      sl(gates, t, 4 * H), sl(cs, t, H), sl(hs, t, H))
+            else:
+                n = dev.lstm_recurrent_forward(H, B, Wht, sl(hs, t - 1, H), wf, wfb)
+                dev.lstm_cell_forward(H, B, sl(xproj, t, 4 * H), bt, wf, n, sl(cs, t - 1, H), sl(gates, t, 4 * H),
+                                      sl(cs, t, H), sl(hs, t, H))
+        out[name] = (gates.numpy(), cs.numpy(), hs.numpy())
+    floor = max(1.0, float(np.sqrt(I + H) * max(rms(Wx), rms(Wh))))
+    for k in range(T):
+        for q, what in enumerate(("gates", "c", "h")):
+            assert_close(out["step"][q][k], ref[k][q], FWD_RTOL, f"{what}[{k}] vs oracle", floor=floor)
+            assert_close(out["step"][q][k], out["two_call"][q][k], FWD_RTOL, f"{what}[{k}] vs two-call", floor=floor)
+
+
+def test_single_launch_step_rejects_unsupported_sizes(dev):
+    assert not dev.lstm_step_supported(96, 4)
+    assert not dev.lstm_step_supported(130, 4)
+    t = dev.zeros(4 * 96 * 96)
+    with pytest.raises(DyhipError) as e:
+        dev.lstm_pack_recurrent(96, t, t)
+    assert e.value.status == lib.ERR_INVALID_ARG
+    with pytest.raises(DyhipError):
+        dev.lstm_step_forward(96, 4, t, t, t, t, t, t, t, t)
+
+
 def test_lstm_rejects_bad_arguments(dev):
     t = dev.zeros(64)
     with pytest.raises(DyhipError) as e:
