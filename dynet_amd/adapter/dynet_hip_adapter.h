@@ -125,6 +125,9 @@ struct Device_GPU {
   Device_GPU(const Device_GPU&) = delete;
   Device_GPU& operator=(const Device_GPU&) = delete;
 
+  // Device_GPU::reset_rng (dynet/devices.cc:130-135)
+  void reset_rng(unsigned seed) { abi_check(dyhip_reset_rng(hip, seed)); }
+
   // Device::allocate_tensor (dynet/devices.cc:82-88)
   Tensor allocate_tensor(DeviceMempool mp, const Dim& d) {
     float* v = static_cast<float*>(pools[static_cast<int>(mp)]->allocate(sizeof(float) * d.size()));
@@ -143,6 +146,16 @@ struct TensorTools {
   static void constant(Tensor& t, float c) { abi_check(dyhip_constant(t.device->hip, t.d.size(), c, t.v)); }
   static void accumulate(Tensor& t, const Tensor& src) {
     abi_check(dyhip_accumulate(t.device->hip, t.d.size(), src.v, t.v));
+  }
+  // dynet/tensor.cc:261-303 (GPU branches)
+  static void randomize_bernoulli(Tensor& t, real p, real scale = 1.f) {
+    abi_check(dyhip_randomize_bernoulli(t.device->hip, t.d.size(), p, scale, t.v));
+  }
+  static void randomize_normal(Tensor& t, real mean = 0.f, real stddev = 1.f) {
+    abi_check(dyhip_randomize_normal(t.device->hip, t.d.size(), mean, stddev, t.v));
+  }
+  static void randomize_uniform(Tensor& t, real left = 0.f, real right = 1.f) {
+    abi_check(dyhip_randomize_uniform(t.device->hip, t.d.size(), left, right, t.v));
   }
 };
 inline std::vector<real> as_vector(const Tensor& t) {  // blocking copy, dynet/tensor.cc:66-93
@@ -271,6 +284,46 @@ struct CwiseMultiply : public Node {
     abi_check(dyhip_cmult_backward(dev.hip, fx.d.batch_size(), xs[0]->d.bd, xs[1]->d.bd, xs[0]->v, xs[1]->v, dEdf.v, i,
                                    dEdxi.v, ws, need));
     scratch(fx)->free();
+  }
+};
+
+// dynet/nodes-dropout.cc:25-47: the mask lives in aux_mem (dim.size() floats)
+struct Dropout : public Node {
+  Dropout(const Dim& dim, real p) : dim(dim), p(p) {}
+  Dim dim;
+  real p;
+  size_t aux_storage_size() const override { return dim.size() * sizeof(float); }
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    abi_check(dyhip_dropout_forward(dev.hip, fx.d.size(), p, xs[0]->v, static_cast<float*>(aux_mem), fx.v));
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>&, const Tensor& fx, const Tensor& dEdf,
+                         unsigned, Tensor& dEdxi) const override {
+    abi_check(dyhip_dropout_backward(dev.hip, fx.d.size(), static_cast<const float*>(aux_mem), dEdf.v, dEdxi.v));
+  }
+};
+
+// dynet/nodes-random.cc:68-137: nodes without arguments whose forward fills fx
+struct RandomBernoulli : public Node {
+  RandomBernoulli(real p, real scale = 1.f) : p(p), scale(scale) {}
+  real p, scale;
+  void forward_dev_impl(const Device_GPU&, const std::vector<const Tensor*>&, Tensor& fx) const override {
+    TensorTools::randomize_bernoulli(fx, p, scale);
+  }
+  void backward_dev_impl(const Device_GPU&, const std::vector<const Tensor*>&, const Tensor&, const Tensor&, unsigned,
+                         Tensor&) const override {
+    throw std::runtime_error("Called backward() on an arity 0 node");
+  }
+};
+struct RandomNormal : public RandomBernoulli {
+  RandomNormal(real mean = 0.f, real stddev = 1.f) : RandomBernoulli(mean, stddev) {}
+  void forward_dev_impl(const Device_GPU&, const std::vector<const Tensor*>&, Tensor& fx) const override {
+    TensorTools::randomize_normal(fx, p, scale);
+  }
+};
+struct RandomUniform : public RandomBernoulli {
+  RandomUniform(real left, real right) : RandomBernoulli(left, right) {}
+  void forward_dev_impl(const Device_GPU&, const std::vector<const Tensor*>&, Tensor& fx) const override {
+    TensorTools::randomize_uniform(fx, p, scale);
   }
 };
 

@@ -70,6 +70,9 @@ struct dyhip_device {
   std::vector<hipEvent_t> sync_events; // ring of events recorded on this queue for dyhip_device_wait
   size_t sync_next;
   std::vector<dyhip_device*> forks;    // live forked queues (destroyed with the device if still alive)
+  uint64_t* rng_state;                 // device: {Philox key, next counter}; one per queue, see random.hip
+  uint32_t rng_stream;                 // third counter word: 0 for the device, 1.. for its forked queues
+  uint32_t forks_made;                 // forked queues created so far (numbers their random streams)
 };
 
 struct dyhip_graph {

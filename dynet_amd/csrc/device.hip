@@ -253,6 +253,9 @@ int dyhip_device_create(int ordinal, const size_t pool_mb[4], dyhip_device** out
   dev->num_cus = prop.multiProcessorCount;
   for (auto& p : dev->pools) p = nullptr;
   dev->scalars = nullptr;
+  dev->rng_state = nullptr;
+  dev->rng_stream = 0;
+  dev->forks_made = 0;
   dev->alloc = nullptr;
   dev->gemm_ws = nullptr;
   dev->gemm_ws_bytes = 0;
@@ -280,6 +283,11 @@ int dyhip_device_create(int ordinal, const size_t pool_mb[4], dyhip_device** out
       st = fail(DYHIP_ERR_RUNTIME, "failed to initialise the device scalars");
   }
   if (st == DYHIP_OK) {
+    dev->rng_state = static_cast<uint64_t*>(dev->alloc->malloc(256));
+    if (dev->rng_state == nullptr) st = fail(DYHIP_ERR_OUT_OF_MEMORY, "failed to allocate the random generator state");
+  }
+  if (st == DYHIP_OK) st = dyhip_reset_rng(dev, 0);
+  if (st == DYHIP_OK) {
     dev->gemm_ws_bytes = size_t(128) << 20;
     dev->gemm_ws = dev->alloc->malloc(dev->gemm_ws_bytes);
     if (dev->gemm_ws == nullptr) st = fail(DYHIP_ERR_OUT_OF_MEMORY, "failed to allocate the GEMM split-K workspace");
@@ -303,6 +311,7 @@ int dyhip_device_fork(dyhip_device* parent, dyhip_device** out) {
   dev->forks.clear();
   dev->sync_next = 0;
   dev->gemm_ws = nullptr;
+  dev->rng_state = nullptr;
   hipError_t e = hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking);
   if (e != hipSuccess) {
     delete dev;
@@ -311,9 +320,18 @@ int dyhip_device_fork(dyhip_device* parent, dyhip_device** out) {
   (void)hipEventCreate(&dev->ev_start);
   (void)hipEventCreate(&dev->ev_stop);
   dev->gemm_ws = parent->alloc->malloc(dev->gemm_ws_bytes);
-  if (dev->gemm_ws == nullptr) {
+  dev->rng_state = static_cast<uint64_t*>(parent->alloc->malloc(256));
+  dev->rng_stream = ++parent->forks_made;
+  if (dev->gemm_ws == nullptr || dev->rng_state == nullptr) {
     dyhip_device_destroy(dev);
-    return fail(DYHIP_ERR_OUT_OF_MEMORY, "failed to allocate the GEMM split-K workspace of the forked queue");
+    return fail(DYHIP_ERR_OUT_OF_MEMORY, "failed to allocate the workspace of the forked queue");
+  }
+  // the queue draws from its own stream of the parent's generator (same key, own counter)
+  hipError_t ce = hipMemcpy(dev->rng_state, parent->rng_state, 8, hipMemcpyDeviceToDevice);
+  if (ce == hipSuccess) ce = hipMemset(dev->rng_state + 1, 0, 8);
+  if (ce != hipSuccess) {
+    dyhip_device_destroy(dev);
+    return fail(DYHIP_ERR_RUNTIME, "failed to initialise the random generator of the forked queue");
   }
   parent->forks.push_back(dev);
   *out = dev;
@@ -355,6 +373,7 @@ int dyhip_device_destroy(dyhip_device* dev) {
         break;
       }
     if (dev->gemm_ws) dev->alloc->free(dev->gemm_ws);
+    if (dev->rng_state) dev->alloc->free(dev->rng_state);
     (void)hipEventDestroy(dev->ev_start);
     (void)hipEventDestroy(dev->ev_stop);
     (void)hipStreamDestroy(dev->stream);
@@ -365,6 +384,7 @@ int dyhip_device_destroy(dyhip_device* dev) {
   for (auto& p : dev->pools)
     if (p) pool_delete(p);
   if (dev->scalars) dev->alloc->free(dev->scalars);
+  if (dev->rng_state) dev->alloc->free(dev->rng_state);
   if (dev->gemm_ws) dev->alloc->free(dev->gemm_ws);
   delete dev->alloc;
   (void)hipEventDestroy(dev->ev_start);

@@ -400,6 +400,34 @@ class Device:
         _check(cdll.dyhip_lstm_cell_backward(self.handle, _u(H), _u(B), _p(gates), _p(c), _p(c_tm1), _p(dh), _vp(rec),
                                              _u(splits), _p(dc), _p(dpre), _p(dc_tm1)))
 
+    # ---- random tensors ---------------------------------------------------
+    def reset_rng(self, seed):
+        _check(cdll.dyhip_reset_rng(self.handle, _u(seed)))
+
+    def rng_state(self):
+        """(key, position, queue) of this queue's Philox stream; synchronises."""
+        k, pos, q = C.c_ulonglong(0), C.c_ulonglong(0), _u(0)
+        _check(cdll.dyhip_rng_state(self.handle, C.byref(k), C.byref(pos), C.byref(q)))
+        return k.value, pos.value, q.value
+
+    def rng_set_position(self, position):
+        _check(cdll.dyhip_rng_set_position(self.handle, C.c_ulonglong(position)))
+
+    def randomize_uniform(self, out, left=0.0, right=1.0):
+        _check(cdll.dyhip_randomize_uniform(self.handle, _sz(out.size), _f(left), _f(right), _p(out)))
+
+    def randomize_bernoulli(self, out, p, scale=1.0):
+        _check(cdll.dyhip_randomize_bernoulli(self.handle, _sz(out.size), _f(p), _f(scale), _p(out)))
+
+    def randomize_normal(self, out, mean=0.0, stddev=1.0):
+        _check(cdll.dyhip_randomize_normal(self.handle, _sz(out.size), _f(mean), _f(stddev), _p(out)))
+
+    def dropout_forward(self, p, x, mask, fx):
+        _check(cdll.dyhip_dropout_forward(self.handle, _sz(x.size), _f(p), _p(x), _p(mask), _p(fx)))
+
+    def dropout_backward(self, mask, dEdf, dEdxi):
+        _check(cdll.dyhip_dropout_backward(self.handle, _sz(mask.size), _p(mask), _p(dEdf), _p(dEdxi)))
+
     # ---- lookup -----------------------------------------------------------
     def lookup_forward(self, ids_host, ids_dev, dim, vocab, table, fx, mult=1.0):
         n = ids_dev.size

@@ -275,6 +275,30 @@ int dyhip_lstm_step_forward(dyhip_device* dev, unsigned H, unsigned B, const flo
                             const float* xproj, const float* b, const float* c_tm1, int logistic_mode, float* gates,
                             float* c, float* h);
 
+/* ---- random tensors: TensorTools::randomize_{uniform,normal,bernoulli}
+ * (dynet/tensor.cc:261-303), Device_GPU::reset_rng (dynet/devices.cc:130-135), the Dropout
+ * node (dynet/nodes-dropout.cc:32-47); RandomUniform/Normal/Bernoulli nodes
+ * (dynet/nodes-random.cc:68-137) and the LSTM builders' dropout masks
+ * (dynet/lstm.cc:964-982) are single calls of the randomize functions. ----------------
+ * Generator: Philox4x32-10 (the generator the reference asks cuRAND for), key = seed + 1.
+ * Element k of a call is word k % 4 of Philox(counter {lo, hi, queue, 0}, key {key, 0})
+ * with block number hi:lo = position + k / 4; afterwards position += ceil(n / 4).  Key and
+ * position live in device memory (a captured graph draws fresh numbers on every replay);
+ * every forked queue has its own position and queue number, so queues never share numbers.
+ * u = word * 2^-32 + 2^-33 in (0, 1]; uniform = u * (right - left) + left; bernoulli =
+ * floor(u + p) * scale; normal = Box-Muller on word pairs (sin, cos) * stddev + mean.
+ * The order in which cuRAND hands out its Philox words is not reproduced. */
+int dyhip_reset_rng(dyhip_device* dev, unsigned seed);
+int dyhip_rng_state(dyhip_device* dev, unsigned long long* key, unsigned long long* position, unsigned* queue);
+int dyhip_rng_set_position(dyhip_device* dev, unsigned long long position);
+int dyhip_randomize_uniform(dyhip_device* dev, size_t n, float left, float right, float* out);
+int dyhip_randomize_bernoulli(dyhip_device* dev, size_t n, float p, float scale, float* out);
+int dyhip_randomize_normal(dyhip_device* dev, size_t n, float mean, float stddev, float* out);
+/* fx = x (.) m with m = bernoulli(1 - p) / (1 - p) written to mask (the node's aux_mem,
+ * n floats); backward: dEdxi += dEdf (.) mask. */
+int dyhip_dropout_forward(dyhip_device* dev, size_t n, float p, const float* x, float* mask, float* fx);
+int dyhip_dropout_backward(dyhip_device* dev, size_t n, const float* mask, const float* dEdf, float* dEdxi);
+
 /* ---- LookupNode (dynet/param-nodes.cc:304-329) and
  * LookupParameterStorage::accumulate_grads (dynet/model.cc:728-743) -------- */
 /* fx[:, b] = table[:, ids[b]] * mult; bit-exact gather when mult == 1.0f.

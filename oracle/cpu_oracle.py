@@ -403,3 +403,58 @@ def squared_l2norm(g):
     out = C.c_float(0)
     _lib.orc_squared_l2norm(C.c_size_t(g.size), _fp(g), C.byref(out))
     return np.float32(out.value)
+
+
+# ---- random tensors --------------------------------------------------------
+def philox4x32_10(ctr, key):
+    c = (C.c_uint * 4)(*[int(v) & 0xFFFFFFFF for v in ctr])
+    k = (C.c_uint * 2)(*[int(v) & 0xFFFFFFFF for v in key])
+    out = (C.c_uint * 4)()
+    _lib.orc_philox4x32_10(c, k, out)
+    return [int(v) for v in out]
+
+
+def random_words(key, position, queue, n):
+    out = np.empty(n, np.uint32)
+    _lib.orc_random_words(C.c_ulonglong(key), C.c_ulonglong(position), C.c_uint(queue), C.c_size_t(n),
+                          out.ctypes.data_as(C.POINTER(C.c_uint)))
+    return out
+
+
+def _rng_args(key, position, queue, n):
+    return C.c_ulonglong(key), C.c_ulonglong(position), C.c_uint(queue), C.c_size_t(n)
+
+
+def randomize_uniform(key, position, queue, n, left=0.0, right=1.0):
+    out = np.empty(n, np.float32)
+    _check(_lib.orc_randomize_uniform(*_rng_args(key, position, queue, n), C.c_float(left), C.c_float(right),
+                                     _fp(out)), "randomize_uniform")
+    return out
+
+
+def randomize_bernoulli(key, position, queue, n, p, scale=1.0):
+    out = np.empty(n, np.float32)
+    _check(_lib.orc_randomize_bernoulli(*_rng_args(key, position, queue, n), C.c_float(p), C.c_float(scale),
+                                       _fp(out)), "randomize_bernoulli")
+    return out
+
+
+def randomize_normal(key, position, queue, n, mean=0.0, stddev=1.0):
+    out = np.empty(n, np.float32)
+    _check(_lib.orc_randomize_normal(*_rng_args(key, position, queue, n), C.c_float(mean), C.c_float(stddev),
+                                    _fp(out)), "randomize_normal")
+    return out
+
+
+def dropout_forward(key, position, queue, p, x):
+    x = _f32(x)
+    mask, fx = np.empty_like(x), np.empty_like(x)
+    _check(_lib.orc_dropout_forward(*_rng_args(key, position, queue, x.size), C.c_float(p), _fp(x), _fp(mask),
+                                   _fp(fx)), "dropout_forward")
+    return mask, fx
+
+
+def dropout_backward(mask, dEdf, dEdxi):
+    _check(_lib.orc_dropout_backward(C.c_size_t(mask.size), _fp(_f32(mask)), _fp(_f32(dEdf)), _fp(dEdxi)),
+           "dropout_backward")
+    return dEdxi

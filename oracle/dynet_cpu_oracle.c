@@ -975,3 +975,129 @@ int orc_squared_l2norm(size_t n, const float* g, float* out) {
   *out = s;
   return 0;
 }
+
+/* ======================================================================== */
+/* random tensors                                                            */
+/* ======================================================================== */
+
+/* The reference's GPU device draws from cuRAND's Philox4x32-10 keyed with seed + 1
+ * (dynet/devices.cc:130-135); its CPU device from std::mt19937.  Neither stream is
+ * reproduced: what is restated here is the generator itself (Salmon et al.,
+ * "Parallel random numbers: as easy as 1, 2, 3", SC'11: ten rounds of two 32x32->64
+ * multiplies with the Weyl-bumped key) and the reference's conversions
+ * (dynet/tensor.cc:261-303,446-448).  Pinned by the Random123 known-answer vectors
+ * for philox4x32-10; the assignment of counters to tensor elements is this
+ * build's own (stated in orc_random_words), parity unpinned against cuRAND's. */
+void orc_philox4x32_10(const unsigned ctr[4], const unsigned key[2], unsigned out[4]) {
+  unsigned c[4] = {ctr[0], ctr[1], ctr[2], ctr[3]};
+  unsigned k[2] = {key[0], key[1]};
+  for (int round = 0; round < 10; ++round) {
+    if (round > 0) {
+      k[0] += 0x9E3779B9u; /* golden ratio */
+      k[1] += 0xBB67AE85u; /* sqrt(3) - 1 */
+    }
+    unsigned long long a = 0xD2511F53ull * c[0];
+    unsigned long long b = 0xCD9E8D57ull * c[2];
+    unsigned hi_a = (unsigned)(a >> 32), lo_a = (unsigned)a;
+    unsigned hi_b = (unsigned)(b >> 32), lo_b = (unsigned)b;
+    unsigned n0 = hi_b ^ c[1] ^ k[0];
+    unsigned n2 = hi_a ^ c[3] ^ k[1];
+    c[0] = n0;
+    c[1] = lo_b;
+    c[2] = n2;
+    c[3] = lo_a;
+  }
+  for (int i = 0; i < 4; ++i) out[i] = c[i];
+}
+
+/* words[k] = word k % 4 of Philox(counter {lo, hi, queue, 0}, key {key_lo, key_hi})
+ * where hi:lo = position + k / 4. */
+int orc_random_words(unsigned long long key, unsigned long long position, unsigned queue, size_t n,
+                     unsigned* words) {
+  unsigned kk[2] = {(unsigned)key, (unsigned)(key >> 32)};
+  for (size_t k0 = 0; k0 < n; k0 += 4) {
+    unsigned long long blk = position + k0 / 4;
+    unsigned ctr[4] = {(unsigned)blk, (unsigned)(blk >> 32), queue, 0u}, out[4];
+    orc_philox4x32_10(ctr, kk, out);
+    for (size_t e = 0; e < 4 && k0 + e < n; ++e) words[k0 + e] = out[e];
+  }
+  return 0;
+}
+
+/* cuRAND's uniform conversion: (0, 1] */
+static float unit_interval(unsigned x) {
+  float f = (float)x;
+  f = f * 2.3283064365386963e-10f; /* 2^-32 */
+  return f + 1.1641532182693481e-10f; /* 2^-33 */
+}
+
+/* TensorTools::randomize_uniform, GPU branch, dynet/tensor.cc:290-303: uniform in
+ * (0, 1], then scale_dev(val, right - left, left) unless the range is (0, 1). */
+int orc_randomize_uniform(unsigned long long key, unsigned long long position, unsigned queue, size_t n,
+                          float left, float right, float* out) {
+  unsigned w[4];
+  for (size_t k = 0; k < n; ++k) {
+    if (k % 4 == 0) orc_random_words(key, position + k / 4, queue, 4, w);
+    float u = unit_interval(w[k % 4]);
+    if (left != 0.f || right != 1.f) {
+      float a = right - left;
+      u = u * a;
+      u = u + left;
+    }
+    out[k] = u;
+  }
+  return 0;
+}
+
+/* TensorTools::randomize_bernoulli, GPU branch, dynet/tensor.cc:261-275:
+ * floor(u + p) (uniform_to_bernoulli_dev, :446-448) then * scale. */
+int orc_randomize_bernoulli(unsigned long long key, unsigned long long position, unsigned queue, size_t n,
+                            float p, float scale, float* out) {
+  if (!(p >= 0.f && p <= 1.f)) return -1;
+  unsigned w[4];
+  for (size_t k = 0; k < n; ++k) {
+    if (k % 4 == 0) orc_random_words(key, position + k / 4, queue, 4, w);
+    float u = unit_interval(w[k % 4]);
+    float s = u + p;
+    out[k] = floorf(s) * scale;
+  }
+  return 0;
+}
+
+/* TensorTools::randomize_normal, dynet/tensor.cc:277-288 (curandGenerateNormal):
+ * Box-Muller on consecutive word pairs, sine first, as cuRAND does. */
+int orc_randomize_normal(unsigned long long key, unsigned long long position, unsigned queue, size_t n,
+                         float mean, float stddev, float* out) {
+  unsigned w[4];
+  for (size_t k = 0; k < n; k += 2) {
+    if (k % 4 == 0) orc_random_words(key, position + k / 4, queue, 4, w);
+    float u = unit_interval(w[k % 4]);
+    float ang = (float)w[k % 4 + 1] * 1.4629180792671596e-9f; /* 2 pi 2^-32 */
+    ang = ang + 7.3145903963357980e-10f;                      /* 2 pi 2^-33 */
+    float s = sqrtf(-2.0f * logf(u));
+    float z0 = s * sinf(ang), z1 = s * cosf(ang);
+    z0 = z0 * stddev;
+    z1 = z1 * stddev;
+    out[k] = z0 + mean;
+    if (k + 1 < n) out[k + 1] = z1 + mean;
+  }
+  return 0;
+}
+
+/* Dropout::forward_dev_impl / backward_dev_impl, dynet/nodes-dropout.cc:32-47:
+ * m = bernoulli(1 - p) * 1/(1 - p); fx = x (.) m; dEdxi += dEdf (.) m. */
+int orc_dropout_forward(unsigned long long key, unsigned long long position, unsigned queue, size_t n, float p,
+                        const float* x, float* mask, float* fx) {
+  if (!(p >= 0.f && p < 1.f)) return -1;
+  float keep = 1.f - p;
+  float scale = 1.f / keep;
+  int st = orc_randomize_bernoulli(key, position, queue, n, keep, scale, mask);
+  if (st) return st;
+  for (size_t k = 0; k < n; ++k) fx[k] = x[k] * mask[k];
+  return 0;
+}
+
+int orc_dropout_backward(size_t n, const float* mask, const float* dEdf, float* dEdxi) {
+  for (size_t k = 0; k < n; ++k) dEdxi[k] += dEdf[k] * mask[k];
+  return 0;
+}

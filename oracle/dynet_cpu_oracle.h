@@ -155,6 +155,20 @@ int orc_scale_copy(size_t n, const float* src, float mult, float* dst);
 int orc_sgd_update(size_t n, float* p, const float* g, float lr, float gscale, float wd);
 int orc_squared_l2norm(size_t n, const float* g, float* out);
 
+/* ---- random tensors (Philox4x32-10; key = seed + 1) ----------------------- */
+void orc_philox4x32_10(const unsigned ctr[4], const unsigned key[2], unsigned out[4]);
+int orc_random_words(unsigned long long key, unsigned long long position, unsigned queue, size_t n,
+                     unsigned* words);
+int orc_randomize_uniform(unsigned long long key, unsigned long long position, unsigned queue, size_t n,
+                          float left, float right, float* out);
+int orc_randomize_bernoulli(unsigned long long key, unsigned long long position, unsigned queue, size_t n,
+                            float p, float scale, float* out);
+int orc_randomize_normal(unsigned long long key, unsigned long long position, unsigned queue, size_t n,
+                         float mean, float stddev, float* out);
+int orc_dropout_forward(unsigned long long key, unsigned long long position, unsigned queue, size_t n, float p,
+                        const float* x, float* mask, float* fx);
+int orc_dropout_backward(size_t n, const float* mask, const float* dEdf, float* dEdxi);
+
 #ifdef __cplusplus
 }
 #endif

@@ -362,6 +362,73 @@ static void lookup_and_softmax(Fixture& F) {
   }
 }
 
+// tests/test-nodes.cc:1236-1272 only run these nodes ("noise is random, so it cannot be tested
+// simply"); here the values are checked against what the node's definition fixes.
+static void random_nodes(Fixture& F) {
+  g_case = "dropout_forward";
+  {
+    F.dev.reset_rng(3);
+    const Dim d({64}, 8);
+    vector<float> xv(d.size());
+    for (size_t i = 0; i < xv.size(); ++i) xv[i] = 0.25f + 0.01f * float(i);
+    Tensor x = F.input(d, xv);
+    Dropout node(d, 0.5f);
+    node.aux_mem = F.dev.pools[0]->allocate(node.aux_storage_size());
+    Tensor fx = F.dev.allocate_tensor(DeviceMempool::FXS, d);
+    node.forward_dev_impl(F.dev, {&x}, fx);
+    const vector<float> y = as_vector(fx);
+    Tensor mask(d, static_cast<float*>(node.aux_mem), &F.dev, DeviceMempool::FXS);
+    const vector<float> m = as_vector(mask);
+    size_t kept = 0;
+    for (size_t i = 0; i < y.size(); ++i) {
+      CHECK(m[i] == 0.f || m[i] == 2.f);  // bernoulli(1 - p) * 1 / (1 - p)
+      CHECK(y[i] == xv[i] * m[i]);
+      kept += m[i] != 0.f;
+    }
+    CHECK(kept > y.size() * 2 / 5 && kept < y.size() * 3 / 5);
+    // backward accumulates dEdf (.) mask
+    vector<float> gv(d.size(), 1.5f);
+    Tensor dEdf = F.input(d, gv, DeviceMempool::DEDFS);
+    Tensor dEdx = F.zeros(d);
+    TensorTools::constant(dEdx, 1.f);
+    node.backward_dev_impl(F.dev, {&x}, fx, dEdf, 0, dEdx);
+    const vector<float> g = as_vector(dEdx);
+    for (size_t i = 0; i < g.size(); ++i) CHECK(g[i] == 1.f + 1.5f * m[i]);
+    // the same seed gives the same mask again; the next draw differs
+    F.dev.reset_rng(3);
+    node.forward_dev_impl(F.dev, {&x}, fx);
+    CHECK(as_vector(mask) == m);
+    node.forward_dev_impl(F.dev, {&x}, fx);
+    CHECK(as_vector(mask) != m);
+  }
+  g_case = "random_nodes";
+  {
+    F.dev.reset_rng(1);
+    const Dim d({1000}, 4);
+    Tensor fx = F.dev.allocate_tensor(DeviceMempool::FXS, d);
+    RandomNormal(2.f, 0.5f).forward_dev_impl(F.dev, {}, fx);
+    vector<float> v = as_vector(fx);
+    double s = 0, ss = 0;
+    for (float e : v) { s += e; ss += double(e) * e; }
+    const double mean = s / v.size(), var = ss / v.size() - mean * mean;
+    CHECK_SMALL(mean - 2.0, 0.05);
+    CHECK_SMALL(std::sqrt(var) - 0.5, 0.05);
+    RandomUniform(-1.f, 3.f).forward_dev_impl(F.dev, {}, fx);
+    v = as_vector(fx);
+    s = 0;
+    for (float e : v) { CHECK(e > -1.f && e <= 3.f); s += e; }
+    CHECK_SMALL(s / v.size() - 1.0, 0.1);
+    RandomBernoulli(0.25f, 4.f).forward_dev_impl(F.dev, {}, fx);
+    v = as_vector(fx);
+    size_t ones = 0;
+    for (float e : v) { CHECK(e == 0.f || e == 4.f); ones += e != 0.f; }
+    CHECK_SMALL(double(ones) / v.size() - 0.25, 0.03);
+    bool threw = false;
+    try { RandomBernoulli(1.5f).forward_dev_impl(F.dev, {}, fx); } catch (const std::invalid_argument&) { threw = true; }
+    CHECK(threw);
+  }
+}
+
 int main(int argc, char** argv) {
   if (argc > 1 && std::strcmp(argv[1], "--no-gpu") == 0) {
     try {
@@ -376,7 +443,7 @@ int main(int argc, char** argv) {
   Fixture F;
   const std::vector<std::function<void(Fixture&)>> cases = {lstm_node_h_fwd,      lstm_node_c_fwd, lstm_node_gates_fwd,
                                                              lstm_node_gradients,  elementwise_gradients, layer_norm,
-                                                             lookup_and_softmax};
+                                                             lookup_and_softmax,   random_nodes};
   for (const auto& c : cases) {
     c(F);
     F.reset();

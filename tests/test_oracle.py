@@ -727,3 +727,93 @@ def test_sum_node_association_order_and_broadcast():
                rng.standard_normal((bd, n)).astype(np.float32))
     got = orc.sum_forward(n, bd, [a, b, c], [bd, 1, bd])
     assert got.tobytes() == (((np.zeros_like(a) + a) + b) + c).tobytes()
+
+
+# ---- random tensors ---------------------------------------------------------------------------
+# Known-answer vectors of philox4x32-10 published with the generator (Random123 kat_vectors):
+# counter words, key words -> output words.
+PHILOX_KAT = [
+    ([0, 0, 0, 0], [0, 0], [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]),
+    ([0xFFFFFFFF] * 4, [0xFFFFFFFF] * 2, [0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD]),
+    ([0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344], [0xA4093822, 0x299F31D0],
+     [0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1]),
+]
+
+
+def _philox_python(ctr, key):
+    """The published algorithm written a second time, straight from its definition (bijection of rounds:
+    L' = mullo(R, M), R' = mulhi(R, M) ^ k ^ L on the two counter halves, then the word permutation)."""
+    M = (0xD2511F53, 0xCD9E8D57)
+    W = (0x9E3779B9, 0xBB67AE85)
+    c, k = list(ctr), list(key)
+    for r in range(10):
+        hi0, lo0 = divmod(M[0] * c[0], 1 << 32)
+        hi1, lo1 = divmod(M[1] * c[2], 1 << 32)
+        c = [hi1 ^ c[1] ^ k[0], lo1, hi0 ^ c[3] ^ k[1], lo0]
+        k = [(k[0] + W[0]) & 0xFFFFFFFF, (k[1] + W[1]) & 0xFFFFFFFF]
+    return c
+
+
+@pytest.mark.parametrize("ctr,key,want", PHILOX_KAT)
+def test_philox_known_answers(ctr, key, want):
+    assert orc.philox4x32_10(ctr, key) == want
+    assert _philox_python(ctr, key) == want
+
+
+def test_philox_words_follow_the_stated_counter_layout():
+    rng = np.random.default_rng(0)
+    for _ in range(20):
+        key = int(rng.integers(0, 1 << 63)) * 2 + int(rng.integers(0, 2))
+        pos = int(rng.integers(0, 1 << 40)) + (1 << 32) - 3  # crosses the 32-bit carry of the block number
+        queue, n = int(rng.integers(0, 5)), int(rng.integers(1, 40))
+        words = orc.random_words(key, pos, queue, n)
+        for k in range(n):
+            blk = pos + k // 4
+            ref = _philox_python([blk & 0xFFFFFFFF, blk >> 32, queue, 0], [key & 0xFFFFFFFF, key >> 32])
+            assert int(words[k]) == ref[k % 4]
+
+
+def test_uniform_conversion_and_range():
+    # u = w * 2^-32 + 2^-33 evaluated in fp32, in (0, 1]; the extreme words map to 2^-33 and 1
+    words = orc.random_words(1, 0, 0, 4096)
+    u = orc.randomize_uniform(1, 0, 0, 4096)
+    want = (words.astype(np.float32) * np.float32(2.0 ** -32) + np.float32(2.0 ** -33)).astype(np.float32)
+    assert np.array_equal(u, want)
+    assert u.min() > 0 and u.max() <= 1
+    v = orc.randomize_uniform(1, 0, 0, 4096, -3.0, 5.0)
+    assert np.array_equal(v, (u * np.float32(8.0) + np.float32(-3.0)).astype(np.float32))
+
+
+def test_random_distributions():
+    from scipy import stats
+
+    n = 400000
+    u = orc.randomize_uniform(123, 77, 0, n).astype(np.float64)
+    assert stats.kstest(u, "uniform").pvalue > 1e-3
+    # successive words are uncorrelated
+    assert abs(np.corrcoef(u[:-1], u[1:])[0, 1]) < 5e-3
+    z = orc.randomize_normal(123, 77, 0, n, 2.0, 0.5).astype(np.float64)
+    assert stats.kstest((z - 2.0) / 0.5, "norm").pvalue > 1e-3
+    assert abs(np.corrcoef(z[0::2], z[1::2])[0, 1]) < 5e-3  # the two outputs of one Box-Muller pair
+    for p in (0.0, 0.1, 0.5, 0.9, 1.0):
+        b = orc.randomize_bernoulli(123, 77, 0, n, p, 3.0)
+        assert set(np.unique(b)) <= {np.float32(0), np.float32(3)}
+        rate = (b != 0).mean()
+        assert abs(rate - p) < 4 * np.sqrt(max(p * (1 - p), 1e-12) / n) + 1e-6, (p, rate)
+    # floor(u + p) is 1 exactly when u >= 1 - p (up to the rounding of the fp32 sum)
+    u32 = orc.randomize_uniform(123, 77, 0, 1000)
+    b = orc.randomize_bernoulli(123, 77, 0, 1000, 0.3)
+    assert np.array_equal(b, np.floor(u32 + np.float32(0.3)).astype(np.float32))
+
+
+def test_dropout_oracle():
+    rng = np.random.default_rng(4)
+    x, dy = f32(rng.standard_normal(1001)), f32(rng.standard_normal(1001))
+    mask, fx = orc.dropout_forward(9, 0, 0, 0.2, x)
+    keep_scale = np.float32(1.0) / np.float32(0.8)
+    assert np.array_equal(mask, orc.randomize_bernoulli(9, 0, 0, 1001, 0.8, float(keep_scale)))
+    assert np.array_equal(fx, x * mask)
+    dx = orc.dropout_backward(mask, dy, np.ones(1001, np.float32))
+    assert np.array_equal(dx, (np.float32(1) + dy * mask).astype(np.float32))
+    with pytest.raises(ValueError):
+        orc.dropout_forward(9, 0, 0, 1.0, x)
