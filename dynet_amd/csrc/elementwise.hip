@@ -20,6 +20,8 @@
 // 16.8 MB-per-tensor copy from about 4.6 to 5.8 TB/s and a three-read-one-write
 // update from 4.7 to 5.6 TB/s.  Tensors whose n is not a multiple of 4, or whose base is not
 // 16-byte aligned, take the scalar variant of the same kernel.
+#include <algorithm>
+
 #include "common.h"
 
 namespace dyhip {
@@ -228,6 +230,40 @@ static int binary_forward(dyhip_device* dev, size_t n, unsigned bd0, unsigned bd
   return ew_launch<2, false, 2>(dev, n, bd, a, b, nullptr, y, f);
 }
 
+// PickRange (dynet/nodes-select.cc:230-259): slicing dimension `dim` of a column-major tensor is a
+// strided copy of `outer` contiguous runs: with inner = product of the dimensions before `dim`,
+// run o is src[o*inner*len + start*inner, +inner*(end-start)).  blockIdx.y walks runs, lanes walk a run.
+template <bool ACC>
+__global__ __launch_bounds__(256) void pick_range_kernel(size_t run, size_t small_stride, size_t big_stride,
+                                                         size_t big_offset, unsigned outer,
+                                                         const float* __restrict__ src, float* __restrict__ dst) {
+  for (unsigned o = blockIdx.y; o < outer; o += gridDim.y) {
+    // forward: dst is the slice (small), src the whole tensor (big); backward: the other way round
+    const float* s = ACC ? src + o * small_stride : src + o * big_stride + big_offset;
+    float* d = ACC ? dst + o * big_stride + big_offset : dst + o * small_stride;
+    for (size_t e = size_t(blockIdx.x) * 256 + threadIdx.x; e < run; e += size_t(gridDim.x) * 256)
+      d[e] = ACC ? d[e] + s[e] : s[e];
+  }
+}
+
+static int pick_range(dyhip_device* dev, bool backward, size_t inner, size_t len, size_t outer, size_t start,
+                      size_t end, const float* src, float* dst) {
+  DYHIP_REQUIRE(start < end && end <= len, "PickRange: bad range [%zu, %zu) for a dimension of %zu", start, end, len);
+  if (inner == 0 || outer == 0) return DYHIP_OK;
+  DYHIP_REQUIRE(src && dst, "PickRange: null tensor pointer");
+  DYHIP_REQUIRE(outer <= 0xffffffffu, "PickRange: too many slices");
+  const size_t run = inner * (end - start);
+  const dim3 grid(unsigned(std::min<size_t>(cdiv<size_t>(run, 256), 4096)), unsigned(std::min<size_t>(outer, 65535)));
+  if (backward)
+    hipLaunchKernelGGL(pick_range_kernel<true>, grid, dim3(256), 0, dev->stream, run, run, inner * len, start * inner,
+                       unsigned(outer), src, dst);
+  else
+    hipLaunchKernelGGL(pick_range_kernel<false>, grid, dim3(256), 0, dev->stream, run, run, inner * len, start * inner,
+                       unsigned(outer), src, dst);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
 }  // namespace dyhip
 
 using namespace dyhip;
@@ -377,6 +413,18 @@ int dyhip_sum_forward(dyhip_device* dev, unsigned k, size_t n, unsigned bd, cons
   }
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
+}
+
+int dyhip_pick_range_forward(dyhip_device* dev, size_t inner, size_t len, size_t outer, size_t start, size_t end,
+                             const float* x, float* fx) {
+  DYHIP_CHECK_DEV(dev);
+  return pick_range(dev, false, inner, len, outer, start, end, x, fx);
+}
+
+int dyhip_pick_range_backward(dyhip_device* dev, size_t inner, size_t len, size_t outer, size_t start, size_t end,
+                              const float* dEdf, float* dEdxi) {
+  DYHIP_CHECK_DEV(dev);
+  return pick_range(dev, true, inner, len, outer, start, end, dEdf, dEdxi);
 }
 
 }  // extern "C"

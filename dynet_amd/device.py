@@ -400,6 +400,14 @@ class Device:
         _check(cdll.dyhip_lstm_cell_backward(self.handle, _u(H), _u(B), _p(gates), _p(c), _p(c_tm1), _p(dh), _vp(rec),
                                              _u(splits), _p(dc), _p(dpre), _p(dc_tm1)))
 
+    def pick_range_forward(self, inner, length, outer, start, end, x, fx):
+        _check(cdll.dyhip_pick_range_forward(self.handle, _sz(inner), _sz(length), _sz(outer), _sz(start), _sz(end),
+                                             _p(x), _p(fx)))
+
+    def pick_range_backward(self, inner, length, outer, start, end, dEdf, dEdxi):
+        _check(cdll.dyhip_pick_range_backward(self.handle, _sz(inner), _sz(length), _sz(outer), _sz(start), _sz(end),
+                                              _p(dEdf), _p(dEdxi)))
+
     # ---- random tensors ---------------------------------------------------
     def reset_rng(self, seed):
         _check(cdll.dyhip_reset_rng(self.handle, _u(seed)))

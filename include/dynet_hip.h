@@ -149,6 +149,15 @@ int dyhip_csum_forward(dyhip_device* dev, size_t n, unsigned bd0, unsigned bd1, 
 int dyhip_csum_backward(dyhip_device* dev, size_t n, unsigned bd0, unsigned bd1, const float* dEdf, unsigned i,
                         float* dEdxi, void* ws, size_t ws_bytes);
 
+/* PickRange (dynet/nodes-select.cc:230-259): fx = x sliced to [start, end) along one dimension.
+ * The tensor is described as inner x len x outer, column-major: inner = product of the dimensions
+ * before the sliced one, len = its size, outer = product of the later ones times the batch size.
+ * Forward copies (bit-exact); backward accumulates dEdf into the slice of dEdxi (:258). */
+int dyhip_pick_range_forward(dyhip_device* dev, size_t inner, size_t len, size_t outer, size_t start, size_t end,
+                             const float* x, float* fx);
+int dyhip_pick_range_backward(dyhip_device* dev, size_t inner, size_t len, size_t outer, size_t start, size_t end,
+                              const float* dEdf, float* dEdxi);
+
 /* Sum node / esum (dynet/nodes-arith-sum.cc:65-129): fx = sum of k same-shaped arguments whose batch
  * size is bd or 1 (broadcast), added in the reference's association order (groups of four).  xs_host
  * and bds_host are HOST arrays.  Backward per argument is dyhip_csum_backward (dx_i += dEdf, summed

@@ -458,3 +458,18 @@ def dropout_backward(mask, dEdf, dEdxi):
     _check(_lib.orc_dropout_backward(C.c_size_t(mask.size), _fp(_f32(mask)), _fp(_f32(dEdf)), _fp(dEdxi)),
            "dropout_backward")
     return dEdxi
+
+
+# ---- PickRange -------------------------------------------------------------
+def pick_range_forward(inner, length, outer, start, end, x):
+    x = _f32(x)
+    fx = np.empty(inner * max(end - start, 0) * outer, np.float32)
+    _check(_lib.orc_pick_range_forward(C.c_size_t(inner), C.c_size_t(length), C.c_size_t(outer), C.c_size_t(start),
+                                       C.c_size_t(end), _fp(x), _fp(fx)), "pick_range_forward")
+    return fx
+
+
+def pick_range_backward(inner, length, outer, start, end, dEdf, dEdxi):
+    _check(_lib.orc_pick_range_backward(C.c_size_t(inner), C.c_size_t(length), C.c_size_t(outer), C.c_size_t(start),
+                                        C.c_size_t(end), _fp(_f32(dEdf)), _fp(dEdxi)), "pick_range_backward")
+    return dEdxi

@@ -1101,3 +1101,30 @@ int orc_dropout_backward(size_t n, const float* mask, const float* dEdf, float* 
   for (size_t k = 0; k < n; ++k) dEdxi[k] += dEdf[k] * mask[k];
   return 0;
 }
+
+/* ======================================================================== */
+/* PickRange                                                                 */
+/* ======================================================================== */
+
+/* PickRange::forward_dev_impl / backward_dev_impl, dynet/nodes-select.cc:230-259:
+ * fx = x.slice(start along dim, end - start); dEdxi.slice(...) += dEdf.  The tensor
+ * is given as inner x len x outer (column-major), the sliced dimension being len. */
+int orc_pick_range_forward(size_t inner, size_t len, size_t outer, size_t start, size_t end, const float* x,
+                           float* fx) {
+  if (!(start < end && end <= len)) return -1;
+  size_t w = end - start;
+  for (size_t o = 0; o < outer; ++o)
+    for (size_t k = 0; k < w; ++k)
+      for (size_t i = 0; i < inner; ++i) fx[i + inner * (k + w * o)] = x[i + inner * (start + k + len * o)];
+  return 0;
+}
+
+int orc_pick_range_backward(size_t inner, size_t len, size_t outer, size_t start, size_t end, const float* dEdf,
+                            float* dEdxi) {
+  if (!(start < end && end <= len)) return -1;
+  size_t w = end - start;
+  for (size_t o = 0; o < outer; ++o)
+    for (size_t k = 0; k < w; ++k)
+      for (size_t i = 0; i < inner; ++i) dEdxi[i + inner * (start + k + len * o)] += dEdf[i + inner * (k + w * o)];
+  return 0;
+}

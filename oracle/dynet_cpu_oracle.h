@@ -155,6 +155,12 @@ int orc_scale_copy(size_t n, const float* src, float mult, float* dst);
 int orc_sgd_update(size_t n, float* p, const float* g, float lr, float gscale, float wd);
 int orc_squared_l2norm(size_t n, const float* g, float* out);
 
+/* ---- PickRange ---------------------------------------------------------- */
+int orc_pick_range_forward(size_t inner, size_t len, size_t outer, size_t start, size_t end, const float* x,
+                           float* fx);
+int orc_pick_range_backward(size_t inner, size_t len, size_t outer, size_t start, size_t end, const float* dEdf,
+                            float* dEdxi);
+
 /* ---- random tensors (Philox4x32-10; key = seed + 1) ----------------------- */
 void orc_philox4x32_10(const unsigned ctr[4], const unsigned key[2], unsigned out[4]);
 int orc_random_words(unsigned long long key, unsigned long long position, unsigned queue, size_t n,

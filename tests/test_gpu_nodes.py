@@ -718,3 +718,122 @@ def dev_scalar(dev, which):
     from dynet_amd.device import DevTensor
 
     return DevTensor(dev, dev.scalar_ptr(which), (1,)).numpy().tobytes()
+
+
+# ---- PickRange and the unfused builder step ---------------------------------------------------
+@pytest.mark.parametrize("inner,length,outer,start,end", [(1, 8, 5, 2, 6), (1, 4096, 128, 1024, 2048), (7, 5, 3, 0, 5),
+                                                          (3, 9, 70000, 4, 5), (33, 4, 1, 1, 3)])
+def test_pick_range(dev, inner, length, outer, start, end):
+    rng = np.random.default_rng(inner + length)
+    x = f32(rng.standard_normal(inner * length * outer))
+    want = orc.pick_range_forward(inner, length, outer, start, end, x)
+    fx = dev.empty(want.size)
+    dev.pick_range_forward(inner, length, outer, start, end, dev.tensor(x), fx)
+    assert np.array_equal(fx.numpy(), want)
+    dy, dx0 = f32(rng.standard_normal(want.size)), f32(rng.standard_normal(x.size))
+    dxt = dev.tensor(dx0)
+    dev.pick_range_backward(inner, length, outer, start, end, dev.tensor(dy), dxt)
+    assert np.array_equal(dxt.numpy(), orc.pick_range_backward(inner, length, outer, start, end, dy, dx0.copy()))
+    with pytest.raises(DyhipError):
+        dev.pick_range_forward(inner, length, outer, end, end, dxt, fx)
+
+
+def _builder_step(dev, H, B, x_in, d_in, h_prev, c_prev, P, ln):
+    """One layer of VanillaLSTMBuilder::add_input_impl (dynet/lstm.cc:477-546) issued op by op:
+    affine_transform (or bias + layer_norm(Wx x) + layer_norm(Wh h)), pick_range x4, logistic / tanh
+    (forget gate through ConstantPlusX 1.0), cmult / sum, tanh (of layer_norm(c) under ln_lstm), cmult."""
+    G = 4 * H
+    tmp = dev.empty((B, G))
+    if ln:
+        a, an = dev.empty((B, G)), dev.empty((B, G))
+        b_, bn = dev.empty((B, G)), dev.empty((B, G))
+        dev.gemm_nn(G, B, d_in, P["Wx"], x_in, 0.0, a)
+        dev.layer_norm_forward(G, B, a, P["gx"], P["bx"], an)
+        dev.gemm_nn(G, B, H, P["Wh"], h_prev, 0.0, b_)
+        dev.layer_norm_forward(G, B, b_, P["gh"], P["bh"], bn)
+        dev.sum_forward(G, B, [P["b"], an, bn], [1, B, B], tmp)
+    else:
+        dev.affine_forward(G, B, d_in, P["b"], P["Wx"], x_in, tmp)
+        dev.gemm_nn(G, B, H, P["Wh"], h_prev, 1.0, tmp)
+    parts = []
+    for q in range(4):
+        t = dev.empty((B, H))
+        dev.pick_range_forward(1, G, B, q * H, (q + 1) * H, tmp, t)
+        parts.append(t)
+    a_i, a_f, a_o, a_g = parts
+    one = dev.empty((H,))
+    dev.constant(one, 1.0)
+    a_f1 = dev.empty((B, H))
+    dev.csum_forward(H, B, 1, a_f, one, a_f1)  # i_aft + forget_bias
+    i_t, f_t, o_t, g_t = (dev.empty((B, H)) for _ in range(4))
+    for src, dst in ((a_i, i_t), (a_f1, f_t), (a_o, o_t)):
+        dev.unary_forward(lib.OP_LOGISTIC, src, dst)
+    dev.unary_forward(lib.OP_TANH, a_g, g_t)
+    fc, ig, c = dev.empty((B, H)), dev.empty((B, H)), dev.empty((B, H))
+    dev.cmult_forward(H, B, B, f_t, c_prev, fc)
+    dev.cmult_forward(H, B, B, i_t, g_t, ig)
+    dev.sum_forward(H, B, [fc, ig], [B, B], c)
+    tc, h = dev.empty((B, H)), dev.empty((B, H))
+    if ln:
+        cn = dev.empty((B, H))
+        dev.layer_norm_forward(H, B, c, P["gc"], P["bc"], cn)
+        dev.unary_forward(lib.OP_TANH, cn, tc)
+    else:
+        dev.unary_forward(lib.OP_TANH, c, tc)
+    dev.cmult_forward(H, B, B, o_t, tc, h)
+    return h, c
+
+
+def test_unfused_builder_step_equals_fused_nodes(dev):
+    """tests/test-rnn.cc:155-184: VanillaLSTMBuilder (unfused ops) and the fused gates/C/H nodes agree over
+    three timesteps to 1e-5, here with both sides running on the device."""
+    rng = np.random.default_rng(21)
+    I, H, B = 6, 8, 4
+    Wx, Wh, b = glorot(rng, 4 * H, I), glorot(rng, 4 * H, H), f32(rng.normal(0, 0.1, 4 * H))
+    P = {"Wx": dev.tensor(Wx), "Wh": dev.tensor(Wh), "b": dev.tensor(b)}
+    h_u = h_f = dev.tensor(f32(rng.standard_normal((B, H)) * 0.5))
+    c_u = c_f = dev.tensor(f32(rng.standard_normal((B, H)) * 0.5))
+    for t in range(3):
+        x = dev.tensor(f32(rng.standard_normal((B, I))))
+        h_u, c_u = _builder_step(dev, H, B, x, I, h_u, c_u, P, ln=False)
+        g, c2, h2 = dev.empty((B, 4 * H)), dev.empty((B, H)), dev.empty((B, H))
+        dev.lstm_gates_forward([x], [I], H, B, h_f, P["Wx"], P["Wh"], P["b"], g)
+        dev.lstm_c_forward(H, B, c_f, g, c2)
+        dev.lstm_h_forward(H, B, c2, g, h2)
+        h_f, c_f = h2, c2
+        assert_close(h_u.numpy(), h_f.numpy(), 1e-5, f"h step {t}", floor=1e-2)
+        assert_close(c_u.numpy(), c_f.numpy(), 1e-5, f"c step {t}", floor=1e-2)
+
+
+def test_ln_lstm_builder_step(dev):
+    """The ln_lstm variant (dynet/lstm.cc:513-518,540-542), the in-tree consumer of layer_norm, against
+    the same step composed from the oracle's nodes."""
+    rng = np.random.default_rng(22)
+    I, H, B = 10, 12, 5
+    G = 4 * H
+    Wx, Wh, b = glorot(rng, G, I), glorot(rng, G, H), f32(rng.normal(0, 0.1, G))
+    ln = {k: f32(rng.uniform(0.5, 1.5, n)) if k[0] == "g" else f32(rng.normal(0, 0.1, n))
+          for k, n in (("gx", G), ("bx", G), ("gh", G), ("bh", G), ("gc", H), ("bc", H))}
+    P = {"Wx": dev.tensor(Wx), "Wh": dev.tensor(Wh), "b": dev.tensor(b)}
+    P.update({k: dev.tensor(v) for k, v in ln.items()})
+    h, c = f32(rng.standard_normal((B, H)) * 0.5), f32(rng.standard_normal((B, H)) * 0.5)
+    ht, ct = dev.tensor(h), dev.tensor(c)
+    for t in range(2):
+        x = f32(rng.standard_normal((B, I)))
+        ht, ct = _builder_step(dev, H, B, dev.tensor(x), I, ht, ct, P, ln=True)
+        # oracle composition of the same nodes
+        a = orc.gemm_nn(G, B, I, Wx, x, 0.0, np.zeros((B, G), F32))
+        bb = orc.gemm_nn(G, B, H, Wh, h, 0.0, np.zeros((B, G), F32))
+        tmp = orc.sum_forward(G, B, [b, orc.layer_norm_forward(G, B, a, ln["gx"], ln["bx"]),
+                                     orc.layer_norm_forward(G, B, bb, ln["gh"], ln["bh"])], [1, B, B]).reshape(B, G)
+        pick = lambda q: np.ascontiguousarray(tmp[:, q * H:(q + 1) * H])
+        i_t = orc.unary_forward(orc.OP_LOGISTIC, pick(0))
+        f_t = orc.unary_forward(orc.OP_LOGISTIC, pick(1) + F32(1.0))
+        o_t = orc.unary_forward(orc.OP_LOGISTIC, pick(2))
+        g_t = orc.unary_forward(orc.OP_TANH, pick(3))
+        c = (f_t * c + i_t * g_t).astype(F32)
+        h = (o_t * orc.unary_forward(orc.OP_TANH, orc.layer_norm_forward(H, B, c, ln["gc"], ln["bc"]).reshape(B, H))
+             ).astype(F32)
+        # layer_norm divides by sigma of a GEMM output: differences of 1e-7 in it come back scaled by g / sigma
+        assert_close(ct.numpy(), c, FWD_RTOL, f"c step {t}", floor=1.0)
+        assert_close(ht.numpy(), h, FWD_RTOL, f"h step {t}", floor=1.0)

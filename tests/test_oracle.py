@@ -817,3 +817,31 @@ def test_dropout_oracle():
     assert np.array_equal(dx, (np.float32(1) + dy * mask).astype(np.float32))
     with pytest.raises(ValueError):
         orc.dropout_forward(9, 0, 0, 1.0, x)
+
+
+# ---- PickRange ----------------------------------------------------------------------------------
+@pytest.mark.parametrize("dim", [0, 1, 2])
+def test_pick_range_is_a_numpy_slice(dim):
+    rng = np.random.default_rng(dim)
+    d = (4, 5, 3)
+    bd = 2
+    # batch outermost, column-major: numpy shape (bd, d2, d1, d0)
+    x = f32(rng.standard_normal((bd, d[2], d[1], d[0])))
+    start, end = 1, 3
+    inner = int(np.prod(d[:dim]))
+    outer = int(np.prod(d[dim + 1:])) * bd
+    got = orc.pick_range_forward(inner, d[dim], outer, start, end, x)
+    sl = [slice(None)] * 4
+    sl[3 - dim] = slice(start, end)
+    assert np.array_equal(got, x[tuple(sl)].ravel())
+    # backward is the adjoint: accumulates into the slice and nothing else
+    dy = f32(rng.standard_normal(got.size))
+    dx = np.ones(x.size, np.float32)
+    orc.pick_range_backward(inner, d[dim], outer, start, end, dy, dx)
+    want = np.ones_like(x)
+    want[tuple(sl)] += dy.reshape(want[tuple(sl)].shape)
+    assert np.array_equal(dx, want.ravel())
+    with pytest.raises(ValueError):
+        orc.pick_range_forward(inner, d[dim], outer, 3, 3, x)
+    with pytest.raises(ValueError):
+        orc.pick_range_forward(inner, d[dim], outer, 0, d[dim] + 1, x)
