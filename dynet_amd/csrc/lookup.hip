@@ -85,6 +85,9 @@ struct ScatterWs {
   unsigned* sorted_pos;
   unsigned* run_last;    // per chunk (part of the plan): last chunk of the run that begins here and continues
                          // into the next chunk, else kNone
+  uint4* fix_list;       // part of the plan: {first chunk, last chunk, row, -} of every run that crosses a chunk
+                         // boundary, in no particular order
+  unsigned* fix_count;   // part of the plan: how many
   float* part_first;     // [chunks][dim]
   float* part_last;      // [chunks][dim]
   unsigned chunks;
@@ -152,14 +155,12 @@ __global__ __launch_bounds__(kLkThreads) void scatter_chunk_kernel(unsigned n, u
   }
 }
 
-// One block per chunk in which a boundary-crossing run starts.  The chunk where the run
-// ends comes from the plan; the run's partial rows (one per chunk
-// it touches) are split over kFixSlices thread slices that each add every
-// kFixSlices-th partial in ascending order with four loads in flight, and the slices
-// are then added in ascending order: deterministic, and a run of thousands of
-// entries costs a handful of memory round trips instead of one per partial.
+// One block per boundary-crossing run (the plan lists the chunks in which such runs start and
+// where each ends).  The run's partial rows (one per chunk it touches) are split over
+// kFixThreads / tpr thread slices that each add every slices-th partial in ascending order with
+// four loads in flight, and the slices are then added in ascending order: deterministic, and a
+// run of thousands of entries costs a handful of memory round trips instead of one per partial.
 constexpr int kFixThreads = 1024;
-constexpr int kFixChunks = 1;  // chunks examined per block (runs are independent: one block each keeps them parallel)
 
 template <class V>
 __global__ __launch_bounds__(kFixThreads) void scatter_fixup_kernel(unsigned n, unsigned dimv, unsigned tpr,
@@ -170,25 +171,18 @@ __global__ __launch_bounds__(kFixThreads) void scatter_fixup_kernel(unsigned n, 
   const unsigned slices = kFixThreads / tpr;
   const unsigned q = threadIdx.x / tpr, t = threadIdx.x - q * tpr;
   const V* pf = reinterpret_cast<const V*>(w.part_first);
-  // each block looks at kFixChunks consecutive chunks; few of them start a boundary-crossing run
-  const unsigned c_begin = blockIdx.x * kFixChunks, c_end = min(w.chunks, c_begin + kFixChunks);
-  __shared__ unsigned c_lasts[kFixChunks], rows[kFixChunks];
-  if (threadIdx.x < kFixChunks) {
-    const unsigned c = c_begin + threadIdx.x;
-    c_lasts[threadIdx.x] = c < c_end ? w.run_last[c] : kNone;
-    rows[threadIdx.x] = c < c_end ? w.sorted_ids[min(n, (c + 1) * kChunk) - 1] : kNone;
-  }
-  __syncthreads();
-  for (int i = 0; i < kFixChunks; ++i) {
-    const unsigned c0 = c_begin + i;
-    const unsigned c_last = c_lasts[i];  // last chunk holding entries of the run
-    if (c_last == kNone) continue;       // uniform over the block
-    const unsigned row = rows[i];
+  // count and the block's first entry are fetched together (entries past count are never used)
+  uint4 e = w.fix_list[blockIdx.x];
+  const unsigned count = *w.fix_count;
+  for (unsigned i = blockIdx.x; i < count; i += gridDim.x) {  // uniform over the block
+    if (i != blockIdx.x) e = w.fix_list[i];
+    const unsigned c0 = e.x, c_last = e.y, row = e.z;
     if (row >= vocab) continue;
     const V* pl = reinterpret_cast<const V*>(w.part_last) + size_t(c0) * dimv;
     for (unsigned cb = 0; cb < dimv; cb += tpr) {
       const unsigned c = cb + t;
-      V acc = vzero<V>();
+      V acc = vzero<V>(), old = vzero<V>();
+      if (q == 0 && c < dimv) old = grads[size_t(row) * dimv + c];  // in flight beside the partials
       if (c < dimv) {
         // partial index p = 0 is part_last[c0]; p >= 1 is part_first[c0 + p]
         const unsigned np = c_last - c0 + 1;
@@ -208,7 +202,7 @@ __global__ __launch_bounds__(kFixThreads) void scatter_fixup_kernel(unsigned n, 
       if (q == 0 && c < dimv) {
         V tot = lds[t];
         for (unsigned k = 1; k < slices; ++k) tot = vadd(tot, lds[k * tpr + t]);
-        grads[size_t(row) * dimv + c] = vadd(grads[size_t(row) * dimv + c], tot);
+        grads[size_t(row) * dimv + c] = vadd(old, tot);
       }
     }
   }
@@ -242,9 +236,12 @@ static int sort_tmp_bytes(unsigned n, unsigned vocab, size_t* bytes) {
 // or filling this chunk only partly) and continue into the next chunk?  If so, in which chunk
 // does it end (binary search for the upper bound of its id)?  Part of the plan, so the search
 // is paid when the plan is built, not in the backward pass.
+__global__ void plan_reset_kernel(unsigned* fix_count) { *fix_count = 0; }
+
 __global__ __launch_bounds__(256) void plan_runs_kernel(unsigned n, unsigned chunks,
                                                         const unsigned* __restrict__ sorted_ids,
-                                                        unsigned* __restrict__ run_last) {
+                                                        unsigned* __restrict__ run_last,
+                                                        uint4* __restrict__ fix_list, unsigned* fix_count) {
   const unsigned ch = blockIdx.x * 256 + threadIdx.x;
   if (ch >= chunks) return;
   const unsigned k0 = ch * kChunk, cnt = min(n - k0, (unsigned)kChunk);
@@ -262,11 +259,26 @@ __global__ __launch_bounds__(256) void plan_runs_kernel(unsigned n, unsigned chu
     out = (lo - 1) / kChunk;
   }
   run_last[ch] = out;
+  // the order of the list does not matter: the runs are independent of each other
+  if (out != kNone) fix_list[atomicAdd(fix_count, 1u)] = make_uint4(ch, out, last, 0u);
 }
 
-// plan = [sorted_ids (n u32) | sorted_pos (n u32) | run_last (chunks u32)], each part padded to 256 bytes
+// plan = [sorted_ids (n u32) | sorted_pos (n u32) | run_last (chunks u32) | fix_list (chunks uint4) | fix_count],
+// each part padded to 256 bytes
 static size_t plan_bytes(unsigned n) {
-  return 2 * align256(sizeof(unsigned) * n) + align256(sizeof(unsigned) * cdiv<unsigned>(n, kChunk));
+  const unsigned chunks = cdiv<unsigned>(n, kChunk);
+  return 2 * align256(sizeof(unsigned) * n) + align256(sizeof(unsigned) * chunks) + align256(sizeof(uint4) * chunks) + 256;
+}
+
+static void plan_parts(const void* plan, unsigned n, ScatterWs* w) {
+  char* p = const_cast<char*>(static_cast<const char*>(plan));
+  const size_t ids_b = align256(sizeof(unsigned) * n), ch_b = align256(sizeof(unsigned) * cdiv<unsigned>(n, kChunk));
+  w->chunks = cdiv<unsigned>(n, kChunk);
+  w->sorted_ids = reinterpret_cast<unsigned*>(p);
+  w->sorted_pos = reinterpret_cast<unsigned*>(p + ids_b);
+  w->run_last = reinterpret_cast<unsigned*>(p + 2 * ids_b);
+  w->fix_list = reinterpret_cast<uint4*>(p + 2 * ids_b + ch_b);
+  w->fix_count = reinterpret_cast<unsigned*>(p + 2 * ids_b + ch_b + align256(sizeof(uint4) * w->chunks));
 }
 
 // scratch of the reduction kernels = [part_first | part_last]
@@ -288,10 +300,11 @@ static int build_plan(dyhip_device* dev, unsigned n, const unsigned* ids_dev, un
   DYHIP_CHECK_HIP(rocprim::radix_sort_pairs(ws, sort_bytes, ids_dev, sorted_ids,
                                             rocprim::counting_iterator<unsigned>(0), sorted_pos, n, 0, key_bits(vocab),
                                             dev->stream));
-  unsigned* run_last = reinterpret_cast<unsigned*>(static_cast<char*>(plan) + 2 * align256(sizeof(unsigned) * n));
-  const unsigned chunks = cdiv<unsigned>(n, kChunk);
-  hipLaunchKernelGGL(plan_runs_kernel, dim3(cdiv<unsigned>(chunks, 256)), dim3(256), 0, dev->stream, n, chunks,
-                     sorted_ids, run_last);
+  ScatterWs w;
+  plan_parts(plan, n, &w);
+  hipLaunchKernelGGL(plan_reset_kernel, dim3(1), dim3(1), 0, dev->stream, w.fix_count);
+  hipLaunchKernelGGL(plan_runs_kernel, dim3(cdiv<unsigned>(w.chunks, 256)), dim3(256), 0, dev->stream, n, w.chunks,
+                     sorted_ids, w.run_last, w.fix_list, w.fix_count);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
@@ -302,12 +315,7 @@ static int reduce_planned(dyhip_device* dev, unsigned n, const void* plan, size_
   DYHIP_REQUIRE(ws != nullptr && ws_bytes >= need && aligned16(ws),
                 "lookup scatter-add needs %zu workspace bytes (16-byte aligned), got %zu", need, ws_bytes);
   ScatterWs w;
-  w.chunks = cdiv<unsigned>(n, kChunk);
-  w.sorted_ids = const_cast<unsigned*>(static_cast<const unsigned*>(plan));
-  w.sorted_pos = reinterpret_cast<unsigned*>(const_cast<char*>(static_cast<const char*>(plan)) +
-                                             align256(sizeof(unsigned) * n));
-  w.run_last = reinterpret_cast<unsigned*>(const_cast<char*>(static_cast<const char*>(plan)) +
-                                           2 * align256(sizeof(unsigned) * n));
+  plan_parts(plan, n, &w);
   char* base = static_cast<char*>(ws);
   w.part_first = reinterpret_cast<float*>(base);
   w.part_last = reinterpret_cast<float*>(base + align256(sizeof(float) * dim * w.chunks));
@@ -315,16 +323,14 @@ static int reduce_planned(dyhip_device* dev, unsigned n, const void* plan, size_
   const unsigned dimv = static_cast<unsigned>(vec ? dim / 4 : dim);
   const unsigned tpr = threads_per_row(dimv);
   const dim3 grid(cdiv<unsigned>(w.chunks, kLkThreads / tpr)), block(kLkThreads);
-  const dim3 fgrid(cdiv<unsigned>(w.chunks, kFixChunks)), fblock(kFixThreads);
+  // enough blocks for every CU; a block walks the plan's list of boundary-crossing runs
+  const dim3 fgrid(std::min<unsigned>(w.chunks, 2u * unsigned(dev->num_cus))), fblock(kFixThreads);
   const size_t flds = size_t(kFixThreads) * (vec ? sizeof(float4) : sizeof(float));
-  const bool stream = size_t(n) * dim * sizeof(float) >= dev->stream_threshold;
   if (vec) {
     float4* gr = reinterpret_cast<float4*>(all_grads);
     const float4* g4 = reinterpret_cast<const float4*>(g);
-    if (stream)
-      hipLaunchKernelGGL((scatter_chunk_kernel<float4, true>), grid, block, 0, dev->stream, n, dimv, tpr, vocab, w, g4, gr);
-    else
-      hipLaunchKernelGGL((scatter_chunk_kernel<float4, false>), grid, block, 0, dev->stream, n, dimv, tpr, vocab, w, g4, gr);
+    // plain loads: streaming (non-temporal) hints make this random-row gather slower, not faster
+    hipLaunchKernelGGL((scatter_chunk_kernel<float4, false>), grid, block, 0, dev->stream, n, dimv, tpr, vocab, w, g4, gr);
     hipLaunchKernelGGL(scatter_fixup_kernel<float4>, fgrid, fblock, flds, dev->stream, n, dimv, tpr, vocab, w, gr);
   } else {
     hipLaunchKernelGGL((scatter_chunk_kernel<float, false>), grid, block, 0, dev->stream, n, dimv, tpr, vocab, w, g,
