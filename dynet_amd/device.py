@@ -173,7 +173,12 @@ class Device:
     def empty(self, shape, dtype=np.float32, pool=lib.POOL_FXS):
         shape = (shape,) if np.isscalar(shape) else tuple(shape)
         n = int(np.prod(shape)) if shape else 1
-        return DevTensor(self, self.alloc(max(n, 1) * np.dtype(dtype).itemsize, pool), shape, dtype)
+        t = DevTensor(self, self.alloc(max(n, 1) * np.dtype(dtype).itemsize, pool), shape, dtype)
+        if getattr(self, "poison_empty", False) and n > 0 and np.dtype(dtype) == np.float32:
+            # debugging aid for tests: an element a kernel forgets to write shows up as NaN instead of
+            # whatever the pool held before (fresh pools are zero-filled, which hides such gaps)
+            _check(cdll.dyhip_constant(self.handle, _sz(n), _f(float("nan")), _vp(t.ptr)))
+        return t
 
     def tensor(self, array, dtype=np.float32, pool=lib.POOL_FXS):
         a = np.ascontiguousarray(array, dtype=dtype)
