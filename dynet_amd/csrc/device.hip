@@ -26,20 +26,23 @@ int fail(int code, const char* fmt, ...) {
 }
 
 // Zero-fill as a kernel rather than a memset node, so that callers may capture
-// it into a HIP graph.  Handles any byte count: 16-byte body + byte tail.
+// it into a HIP graph.  Handles any address and byte count: byte head up to the
+// first 16-byte boundary, 16-byte body, byte tail.
 __global__ __launch_bounds__(256) void zero_fill_kernel(char* p, size_t nbytes) {
-  const size_t n16 = nbytes >> 4;
-  uint4* p16 = reinterpret_cast<uint4*>(p);
+  const size_t gid = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
   const size_t stride = size_t(gridDim.x) * blockDim.x;
-  for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n16; i += stride)
-    p16[i] = make_uint4(0u, 0u, 0u, 0u);
-  const size_t tail0 = n16 << 4;
-  for (size_t i = tail0 + size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < nbytes; i += stride) p[i] = 0;
+  size_t head = (16 - (reinterpret_cast<uintptr_t>(p) & 15u)) & 15u;
+  if (head > nbytes) head = nbytes;
+  if (gid < head) p[gid] = 0;
+  char* body = p + head;
+  const size_t rest = nbytes - head, n16 = rest >> 4;
+  uint4* p16 = reinterpret_cast<uint4*>(body);
+  for (size_t i = gid; i < n16; i += stride) p16[i] = make_uint4(0u, 0u, 0u, 0u);
+  for (size_t i = (n16 << 4) + gid; i < rest; i += stride) body[i] = 0;
 }
 
 hipError_t zero_fill(void* p, size_t nbytes, hipStream_t stream) {
   if (nbytes == 0) return hipSuccess;
-  if (!aligned16(p)) return hipMemsetAsync(p, 0, nbytes, stream);
   size_t blocks = cdiv<size_t>(nbytes >> 4, 256 * 8);
   if (blocks < 1) blocks = 1;
   if (blocks > 4096) blocks = 4096;

@@ -225,6 +225,10 @@ class Device:
     def zero(self, t):
         _check(cdll.dyhip_zero(self.handle, _p(t), _sz(t.nbytes)))
 
+    def zero_bytes(self, ptr, nbytes):
+        """dyhip_zero on a raw device address (any alignment)."""
+        _check(cdll.dyhip_zero(self.handle, _vp(ptr), _sz(nbytes)))
+
     def constant(self, t, value):
         _check(cdll.dyhip_constant(self.handle, _sz(t.size), _f(value), _p(t)))
 

@@ -837,3 +837,29 @@ def test_ln_lstm_builder_step(dev):
         # layer_norm divides by sigma of a GEMM output: differences of 1e-7 in it come back scaled by g / sigma
         assert_close(ct.numpy(), c, FWD_RTOL, f"c step {t}", floor=1.0)
         assert_close(ht.numpy(), h, FWD_RTOL, f"h step {t}", floor=1.0)
+
+
+def test_zero_any_alignment_and_inside_a_graph(dev):
+    """dyhip_zero is a kernel for every address and size (no memset node), so it can be captured."""
+    n = 4096
+    buf = dev.empty(n, np.uint32)
+    ones = np.full(n, 0xFFFFFFFF, np.uint32)
+    for off, nbytes in [(0, 16), (1, 1), (3, 13), (5, 64), (15, 17), (16, 4000), (7, 4001), (9, 2), (2, 0)]:
+        buf.set(ones)
+        dev.zero_bytes(buf.ptr + off, nbytes)
+        got = buf.numpy().view(np.uint8)
+        want = ones.view(np.uint8).copy()
+        want[off:off + nbytes] = 0
+        assert np.array_equal(got, want), (off, nbytes)
+    buf.set(ones)
+    dev.graph_begin()
+    dev.zero_bytes(buf.ptr + 6, 999)
+    g = dev.graph_end()
+    for _ in range(2):
+        buf.set(ones)
+        g.launch()
+        dev.sync()
+        want = ones.view(np.uint8).copy()
+        want[6:6 + 999] = 0
+        assert np.array_equal(buf.numpy().view(np.uint8), want)
+    g.destroy()
