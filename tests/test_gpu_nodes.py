@@ -16,7 +16,9 @@ pytestmark = pytest.mark.gpu
 # GEMM shim
 # ---------------------------------------------------------------------------
 GEMM_SHAPES = [(1024, 32, 128), (1024, 32, 256), (4096, 128, 1280), (256, 128, 4096), (130, 33, 17), (5, 4, 6),
-               (64, 1, 64), (1000, 128, 1024), (129, 65, 100)]
+               (64, 1, 64), (1000, 128, 1024), (129, 65, 100),
+               # more tiles than two per CU with a thin last round: the trailing tile columns run as a GEMM of their own
+               (4096, 2304, 40), (4100, 2310, 33)]
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
@@ -55,7 +57,8 @@ def test_gemm_is_fp32_accurate_against_fp64(dev):
     assert np.max(np.abs(yt.numpy() - want)) < 2e-6 * np.sqrt(K) * 10
 
 
-@pytest.mark.parametrize("M,N,K", [(1000, 128, 64), (10000, 96, 256), (37, 5, 20), (300, 192, 128), (4096, 4, 1024)])
+@pytest.mark.parametrize("M,N,K", [(1000, 128, 64), (10000, 96, 256), (37, 5, 20), (300, 192, 128), (4096, 4, 1024),
+                                   (4100, 2310, 24)])
 def test_affine_forward(dev, M, N, K):
     """AffineTransform: bias broadcast + W x (direct and split-K routes of the GEMM)."""
     rng = np.random.default_rng(M + N + K)
