@@ -56,6 +56,7 @@ struct GemmArgs {
   const float* bias;  // when set (and partial == nullptr): C = bias[i] + sum
   float* partial;     // [splits][M*N] or nullptr
   int vec_ok;         // every operand 16-byte aligned with a leading dimension that is a multiple of 4
+  int edge4_ok;       // vec_ok, and no 128-bit group of any operand straddles the matrix edge
 };
 
 // ---- global -> register tile loads ------------------------------------------------
@@ -66,9 +67,11 @@ struct TileRegs {
   float4 v[NV];
 };
 
-// EDGE == false: the whole tile lies inside the matrix and is 16-byte aligned.
-// EDGE == true : branch-free clamped scalar loads, zeros outside the matrix.
-template <bool KMAJOR, int W, bool EDGE>
+// EDGE == 0: the whole tile lies inside the matrix and is 16-byte aligned.
+// EDGE == 1: 16-byte aligned operands whose extent along the vectorised direction is a multiple of 4,
+//            so every 128-bit group is wholly inside or wholly outside: branch-free clamped 128-bit loads.
+// EDGE == 2: branch-free clamped scalar loads, zeros outside the matrix.
+template <bool KMAJOR, int W, int EDGE>
 __device__ __forceinline__ void load_tile(TileRegs<W>& r, const float* __restrict__ p, size_t ld, size_t mn0,
                                           size_t k0, size_t MN, size_t K) {
 #pragma unroll
@@ -82,8 +85,13 @@ __device__ __forceinline__ void load_tile(TileRegs<W>& r, const float* __restric
       mn = mn0 + f / (kBK / 4);
       kk = k0 + size_t(f % (kBK / 4)) * 4;
     }
-    if (!EDGE) {
+    if (EDGE == 0) {
       r.v[u] = *reinterpret_cast<const float4*>(KMAJOR ? p + kk + mn * ld : p + mn + kk * ld);
+    } else if (EDGE == 1) {
+      const bool ok = mn < MN && kk < K;
+      const size_t mc = ok ? mn : 0, kc = ok ? kk : 0;
+      const float4 x = *reinterpret_cast<const float4*>(KMAJOR ? p + kc + mc * ld : p + mc + kc * ld);
+      r.v[u] = make_float4(ok ? x.x : 0.f, ok ? x.y : 0.f, ok ? x.z : 0.f, ok ? x.w : 0.f);
     } else {
       float e[4];
 #pragma unroll
@@ -154,11 +162,14 @@ __device__ __forceinline__ void load_pair(const GemmArgs& g, unsigned kt, bool i
   size_t k0;
   locate_ktile(g, kt, sg, k0);
   if (interior && k0 + kBK <= sg.K) {
-    load_tile<A_KMAJOR, kBM, false>(ra, sg.A, sg.lda, m0, k0, g.M, sg.K);
-    load_tile<B_KMAJOR, BN, false>(rb, sg.B, sg.ldb, n0, k0, g.N, sg.K);
+    load_tile<A_KMAJOR, kBM, 0>(ra, sg.A, sg.lda, m0, k0, g.M, sg.K);
+    load_tile<B_KMAJOR, BN, 0>(rb, sg.B, sg.ldb, n0, k0, g.N, sg.K);
+  } else if (g.edge4_ok) {
+    load_tile<A_KMAJOR, kBM, 1>(ra, sg.A, sg.lda, m0, k0, g.M, sg.K);
+    load_tile<B_KMAJOR, BN, 1>(rb, sg.B, sg.ldb, n0, k0, g.N, sg.K);
   } else {
-    load_tile<A_KMAJOR, kBM, true>(ra, sg.A, sg.lda, m0, k0, g.M, sg.K);
-    load_tile<B_KMAJOR, BN, true>(rb, sg.B, sg.ldb, n0, k0, g.N, sg.K);
+    load_tile<A_KMAJOR, kBM, 2>(ra, sg.A, sg.lda, m0, k0, g.M, sg.K);
+    load_tile<B_KMAJOR, BN, 2>(rb, sg.B, sg.ldb, n0, k0, g.N, sg.K);
   }
 }
 
@@ -394,6 +405,10 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
     vec = vec && aligned16(segs[s].A) && segs[s].lda % 4 == 0 && aligned16(segs[s].B) && segs[s].ldb % 4 == 0;
   }
   g.vec_ok = vec ? 1 : 0;
+  // a group of four runs along k for a k-major operand and along m (or n) otherwise
+  bool edge4 = vec && (a_kmajor || M % 4 == 0) && (b_kmajor || N % 4 == 0);
+  for (int s = 0; s < nseg; ++s) edge4 = edge4 && (!(a_kmajor || b_kmajor) || segs[s].K % 4 == 0);
+  g.edge4_ok = edge4 ? 1 : 0;
   const size_t out_bytes = M * N * sizeof(float);
   const size_t ws_bytes = to_caller ? epi.partials_bytes : dev->gemm_ws_bytes;
   void* ws = to_caller ? static_cast<void*>(epi.partials) : dev->gemm_ws;
