@@ -56,6 +56,22 @@ def test_logistic_packet_form_is_bit_exact_and_scalar_form_is_accurate(dev):
     assert_close(yt.numpy(), orc.unary_forward(orc.OP_LOGISTIC, x, orc.LOGISTIC_SCALAR), FWD_RTOL, "logistic scalar")
 
 
+def test_logistic_packet_form_is_bit_exact_on_a_dense_sweep(dev):
+    """Every float in [-19, 19] at a stride of 64 bit patterns, every 4096-th float elsewhere (infinities, NaN
+    patterns and denormals included): the same bits as the oracle's IEEE division."""
+    pos = np.arange(0, 0x80000000, 4096, dtype=np.uint64)
+    lo, hi = f32(2.0 ** -40).view(np.uint32), f32(19.0).view(np.uint32)
+    dense = np.arange(int(lo.item()), int(hi.item()), 64, dtype=np.uint64)
+    bits = np.concatenate([pos, dense]).astype(np.uint32)
+    bits = np.concatenate([bits, bits | np.uint32(0x80000000)])
+    x = bits.view(np.float32)
+    yt = dev.empty(x.size)
+    dev.unary_forward(lib.OP_LOGISTIC, dev.tensor(x), yt, lib.LOGISTIC_PACKET)
+    got, want = yt.numpy(), orc.unary_forward(orc.OP_LOGISTIC, x, orc.LOGISTIC_PACKET)
+    same = (got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))
+    assert same.all(), (x[~same][:5], got[~same][:5], want[~same][:5])
+
+
 def test_tanh_is_relatively_accurate_everywhere(dev):
     x = f32(np.concatenate([np.linspace(-12, 12, 200001), np.logspace(-30, 1, 4000), -np.logspace(-30, 1, 4000)]))
     yt = dev.empty(x.size)
