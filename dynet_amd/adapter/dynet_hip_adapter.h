@@ -368,12 +368,27 @@ struct LookupNode : public Node {
   const Tensor* all_values;
   Tensor* all_grads;
   const std::vector<unsigned>* pindices;
-  size_t aux_storage_size() const override { return sizeof(unsigned) * pindices->size(); }  // :154-156
+  // aux_mem = [ids | sorted (id, position) plan].  The reference keeps only the ids there (:154-156); the
+  // plan depends on nothing but the ids, so forward builds it and the backward pass starts at the reduction.
+  static size_t ids_bytes(size_t n) { return (sizeof(unsigned) * n + 255) / 256 * 256; }
+  size_t aux_storage_size() const override {
+    size_t plan = 0;
+    abi_check(dyhip_lookup_plan_bytes(static_cast<unsigned>(pindices->size()), &plan));
+    return ids_bytes(pindices->size()) + plan;
+  }
 
   void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>&, Tensor& fx) const override {
-    abi_check(dyhip_lookup_forward(dev.hip, static_cast<unsigned>(pindices->size()), pindices->data(),
-                                   static_cast<unsigned*>(aux_mem), all_values->d.batch_size(), all_values->d.bd,
+    const unsigned n = static_cast<unsigned>(pindices->size());
+    unsigned* ids_dev = static_cast<unsigned*>(aux_mem);
+    abi_check(dyhip_lookup_forward(dev.hip, n, pindices->data(), ids_dev, all_values->d.batch_size(), all_values->d.bd,
                                    all_values->v, 1.0f, fx.v));
+    size_t plan = 0, need = 0;
+    abi_check(dyhip_lookup_plan_bytes(n, &plan));
+    abi_check(dyhip_lookup_plan_workspace(n, all_values->d.bd, &need));
+    void* ws = need ? scratch(fx)->allocate(need) : nullptr;
+    abi_check(dyhip_lookup_build_plan(dev.hip, n, ids_dev, all_values->d.bd, static_cast<char*>(aux_mem) + ids_bytes(n),
+                                      plan, ws, need));
+    scratch(fx)->free();
   }
   void backward_dev_impl(const Device_GPU&, const std::vector<const Tensor*>&, const Tensor&, const Tensor&, unsigned,
                          Tensor&) const override {
@@ -383,10 +398,10 @@ struct LookupNode : public Node {
     const unsigned n = static_cast<unsigned>(pindices->size());
     const size_t D = all_values->d.batch_size();
     size_t need = 0;
-    abi_check(dyhip_lookup_accumulate_grads_workspace(n, D, all_values->d.bd, &need));
-    void* ws = scratch(fx)->allocate(need);
-    abi_check(dyhip_lookup_accumulate_grads(dev.hip, n, static_cast<const unsigned*>(aux_mem), D, all_values->d.bd, g.v,
-                                            all_grads->v, ws, need));
+    abi_check(dyhip_lookup_accumulate_grads_planned_workspace(n, D, &need));
+    void* ws = need ? scratch(fx)->allocate(need) : nullptr;
+    abi_check(dyhip_lookup_accumulate_grads_planned(dev.hip, n, static_cast<const char*>(aux_mem) + ids_bytes(n), D,
+                                                    all_values->d.bd, g.v, all_grads->v, ws, need));
     scratch(fx)->free();
   }
 };
