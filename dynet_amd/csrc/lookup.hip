@@ -83,8 +83,6 @@ __global__ __launch_bounds__(kLkThreads) void lookup_gather_kernel(unsigned n_id
 struct ScatterWs {
   unsigned* sorted_ids;
   unsigned* sorted_pos;
-  unsigned* run_last;    // per chunk (part of the plan): last chunk of the run that begins here and continues
-                         // into the next chunk, else kNone
   uint4* fix_list;       // part of the plan: {first chunk, last chunk, row, -} of every run that crosses a chunk
                          // boundary, in no particular order
   unsigned* fix_count;   // part of the plan: how many
@@ -232,15 +230,15 @@ static int sort_tmp_bytes(unsigned n, unsigned vocab, size_t* bytes) {
   return DYHIP_OK;
 }
 
+__global__ void plan_reset_kernel(unsigned* fix_count) { *fix_count = 0; }
+
 // Per chunk of the sorted ids: does a run start here (not continuing from the previous chunk,
 // or filling this chunk only partly) and continue into the next chunk?  If so, in which chunk
-// does it end (binary search for the upper bound of its id)?  Part of the plan, so the search
-// is paid when the plan is built, not in the backward pass.
-__global__ void plan_reset_kernel(unsigned* fix_count) { *fix_count = 0; }
+// does it end (binary search for the upper bound of its id)?  Every such run becomes one entry
+// of the plan's fix-up list, so the search is paid when the plan is built, not in the backward pass.
 
 __global__ __launch_bounds__(256) void plan_runs_kernel(unsigned n, unsigned chunks,
                                                         const unsigned* __restrict__ sorted_ids,
-                                                        unsigned* __restrict__ run_last,
                                                         uint4* __restrict__ fix_list, unsigned* fix_count) {
   const unsigned ch = blockIdx.x * 256 + threadIdx.x;
   if (ch >= chunks) return;
@@ -258,27 +256,23 @@ __global__ __launch_bounds__(256) void plan_runs_kernel(unsigned n, unsigned chu
     }
     out = (lo - 1) / kChunk;
   }
-  run_last[ch] = out;
   // the order of the list does not matter: the runs are independent of each other
   if (out != kNone) fix_list[atomicAdd(fix_count, 1u)] = make_uint4(ch, out, last, 0u);
 }
 
-// plan = [sorted_ids (n u32) | sorted_pos (n u32) | run_last (chunks u32) | fix_list (chunks uint4) | fix_count],
-// each part padded to 256 bytes
+// plan = [sorted_ids (n u32) | sorted_pos (n u32) | fix_list (chunks uint4) | fix_count], each part padded to 256 bytes
 static size_t plan_bytes(unsigned n) {
-  const unsigned chunks = cdiv<unsigned>(n, kChunk);
-  return 2 * align256(sizeof(unsigned) * n) + align256(sizeof(unsigned) * chunks) + align256(sizeof(uint4) * chunks) + 256;
+  return 2 * align256(sizeof(unsigned) * n) + align256(sizeof(uint4) * cdiv<unsigned>(n, kChunk)) + 256;
 }
 
 static void plan_parts(const void* plan, unsigned n, ScatterWs* w) {
   char* p = const_cast<char*>(static_cast<const char*>(plan));
-  const size_t ids_b = align256(sizeof(unsigned) * n), ch_b = align256(sizeof(unsigned) * cdiv<unsigned>(n, kChunk));
+  const size_t ids_b = align256(sizeof(unsigned) * n);
   w->chunks = cdiv<unsigned>(n, kChunk);
   w->sorted_ids = reinterpret_cast<unsigned*>(p);
   w->sorted_pos = reinterpret_cast<unsigned*>(p + ids_b);
-  w->run_last = reinterpret_cast<unsigned*>(p + 2 * ids_b);
-  w->fix_list = reinterpret_cast<uint4*>(p + 2 * ids_b + ch_b);
-  w->fix_count = reinterpret_cast<unsigned*>(p + 2 * ids_b + ch_b + align256(sizeof(uint4) * w->chunks));
+  w->fix_list = reinterpret_cast<uint4*>(p + 2 * ids_b);
+  w->fix_count = reinterpret_cast<unsigned*>(p + 2 * ids_b + align256(sizeof(uint4) * w->chunks));
 }
 
 // scratch of the reduction kernels = [part_first | part_last]
@@ -304,7 +298,7 @@ static int build_plan(dyhip_device* dev, unsigned n, const unsigned* ids_dev, un
   plan_parts(plan, n, &w);
   hipLaunchKernelGGL(plan_reset_kernel, dim3(1), dim3(1), 0, dev->stream, w.fix_count);
   hipLaunchKernelGGL(plan_runs_kernel, dim3(cdiv<unsigned>(w.chunks, 256)), dim3(256), 0, dev->stream, n, w.chunks,
-                     sorted_ids, w.run_last, w.fix_list, w.fix_count);
+                     sorted_ids, w.fix_list, w.fix_count);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
