@@ -129,8 +129,8 @@ __global__ __launch_bounds__(kLseThreads) void lse_cols_kernel(size_t rows, cons
 constexpr int kPbThreads = 256;
 constexpr int kPbUnroll = 4;
 
-// dx[:, b] += exp(x[:, b] - z[b]) * dy[b]; dx[ids[b]] -= dy[b]
-template <bool VEC, bool NT>
+// dx[:, b] += exp(x[:, b] - z[b]) * dy[b]; dx[ids[b]] -= dy[b]   (ACC == false: = instead of +=)
+template <bool VEC, bool NT, bool ACC>
 __global__ __launch_bounds__(kPbThreads) void pnls_bwd_kernel(size_t rows, unsigned tiles_per_col,
                                                               const float* __restrict__ x,
                                                               const float* __restrict__ z,
@@ -153,7 +153,7 @@ __global__ __launch_bounds__(kPbThreads) void pnls_bwd_kernel(size_t rows, unsig
       const size_t j = j0 + size_t(u) * kPbThreads;
       if (j < n4) {
         xv[u] = ldg4<NT>(x4 + j);
-        dv[u] = d4[j];
+        dv[u] = ACC ? d4[j] : make_float4(0.f, 0.f, 0.f, 0.f);
       }
     }
 #pragma unroll
@@ -181,7 +181,7 @@ __global__ __launch_bounds__(kPbThreads) void pnls_bwd_kernel(size_t rows, unsig
     for (int u = 0; u < kPbUnroll; ++u) {
       const size_t j = j0 + size_t(u) * kPbThreads;
       if (j < rows) {
-        float r = dEdx[col0 + j] + __expf(x[col0 + j] - zb) * dy;
+        float r = (ACC ? dEdx[col0 + j] : 0.f) + __expf(x[col0 + j] - zb) * dy;
         if (j == hot) r -= dy;
         dEdx[col0 + j] = r;
       }
@@ -340,6 +340,29 @@ static int launch_col_apply(dyhip_device* dev, size_t rows, unsigned cols, const
   return DYHIP_OK;
 }
 
+template <bool ACC>
+static int pnls_backward(dyhip_device* dev, size_t rows, unsigned bd, const float* x, const void* aux, const float* dEdf,
+                         float* dEdx) {
+  DYHIP_REQUIRE(rows >= 1 && x && aux && dEdf && dEdx, "PickNegLogSoftmax needs non-empty tensors");
+  if (bd == 0) return DYHIP_OK;
+  const float* z = static_cast<const float*>(aux);
+  const unsigned* ids = reinterpret_cast<const unsigned*>(z + 2 * size_t(bd));
+  const bool vec = rows % 4 == 0 && aligned16(x) && aligned16(dEdx);
+  const size_t per_tile = size_t(kPbThreads) * kPbUnroll * (vec ? 4 : 1);
+  const size_t tiles = cdiv(rows, per_tile);
+  DYHIP_REQUIRE(tiles * bd < (size_t(1) << 31), "PickNegLogSoftmax backward launch too large");
+  const dim3 grid(static_cast<unsigned>(tiles * bd));
+  const bool stream = rows * size_t(bd) * sizeof(float) >= dev->stream_threshold;
+  if (vec && stream)
+    hipLaunchKernelGGL((pnls_bwd_kernel<true, true, ACC>), grid, dim3(kPbThreads), 0, dev->stream, rows, (unsigned)tiles, x, z, ids, dEdf, dEdx);
+  else if (vec)
+    hipLaunchKernelGGL((pnls_bwd_kernel<true, false, ACC>), grid, dim3(kPbThreads), 0, dev->stream, rows, (unsigned)tiles, x, z, ids, dEdf, dEdx);
+  else
+    hipLaunchKernelGGL((pnls_bwd_kernel<false, false, ACC>), grid, dim3(kPbThreads), 0, dev->stream, rows, (unsigned)tiles, x, z, ids, dEdf, dEdx);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
 }  // namespace dyhip
 
 using namespace dyhip;
@@ -387,24 +410,13 @@ int dyhip_pnls_forward_staged(dyhip_device* dev, size_t rows, unsigned bd, const
 int dyhip_pnls_backward(dyhip_device* dev, size_t rows, unsigned bd, const float* x, const void* aux,
                         const float* dEdf, float* dEdx) {
   DYHIP_CHECK_DEV(dev);
-  DYHIP_REQUIRE(rows >= 1 && x && aux && dEdf && dEdx, "PickNegLogSoftmax needs non-empty tensors");
-  if (bd == 0) return DYHIP_OK;
-  const float* z = static_cast<const float*>(aux);
-  const unsigned* ids = reinterpret_cast<const unsigned*>(z + 2 * size_t(bd));
-  const bool vec = rows % 4 == 0 && aligned16(x) && aligned16(dEdx);
-  const size_t per_tile = size_t(kPbThreads) * kPbUnroll * (vec ? 4 : 1);
-  const size_t tiles = cdiv(rows, per_tile);
-  DYHIP_REQUIRE(tiles * bd < (size_t(1) << 31), "PickNegLogSoftmax backward launch too large");
-  const dim3 grid(static_cast<unsigned>(tiles * bd));
-  const bool stream = rows * size_t(bd) * sizeof(float) >= dev->stream_threshold;
-  if (vec && stream)
-    hipLaunchKernelGGL((pnls_bwd_kernel<true, true>), grid, dim3(kPbThreads), 0, dev->stream, rows, (unsigned)tiles, x, z, ids, dEdf, dEdx);
-  else if (vec)
-    hipLaunchKernelGGL((pnls_bwd_kernel<true, false>), grid, dim3(kPbThreads), 0, dev->stream, rows, (unsigned)tiles, x, z, ids, dEdf, dEdx);
-  else
-    hipLaunchKernelGGL((pnls_bwd_kernel<false, false>), grid, dim3(kPbThreads), 0, dev->stream, rows, (unsigned)tiles, x, z, ids, dEdf, dEdx);
-  DYHIP_CHECK_LAUNCH();
-  return DYHIP_OK;
+  return pnls_backward<true>(dev, rows, bd, x, aux, dEdf, dEdx);
+}
+
+int dyhip_pnls_backward_assign(dyhip_device* dev, size_t rows, unsigned bd, const float* x, const void* aux,
+                               const float* dEdf, float* dEdx) {
+  DYHIP_CHECK_DEV(dev);
+  return pnls_backward<false>(dev, rows, bd, x, aux, dEdf, dEdx);
 }
 
 int dyhip_logsumexp_node_forward(dyhip_device* dev, unsigned k, size_t n, unsigned bd, const float* const* xs_host,

@@ -517,8 +517,9 @@ class Device:
     def pnls_forward_staged(self, rows, bd, x, aux, fx):
         _check(cdll.dyhip_pnls_forward_staged(self.handle, _sz(rows), _u(bd), _p(x), _p(aux), _p(fx)))
 
-    def pnls_backward(self, rows, bd, x, aux, dEdf, dEdx):
-        _check(cdll.dyhip_pnls_backward(self.handle, _sz(rows), _u(bd), _p(x), _p(aux), _p(dEdf), _p(dEdx)))
+    def pnls_backward(self, rows, bd, x, aux, dEdf, dEdx, assign=False):
+        fn = cdll.dyhip_pnls_backward_assign if assign else cdll.dyhip_pnls_backward
+        _check(fn(self.handle, _sz(rows), _u(bd), _p(x), _p(aux), _p(dEdf), _p(dEdx)))
 
     def softmax_forward(self, rows, cols, x, fx):
         ws, nb = self.workspace(8 * cols)

@@ -42,11 +42,23 @@ class LstmLM:
             params = self.init_params(V, E, H, L, seed)
         # parameters and their gradients (PS pool), names as in the reference model
         self.p, self.g = {}, {}
-        for name, a in params.items():
-            self.p[name] = dev.tensor(a, pool=PS)
-            self.g[name] = dev.zeros(a.shape, pool=PS)
-        self.dense = [n for n in self.p if n != "C"]
-        self.sqnorms = dev.zeros((len(self.dense) + 1,), pool=PS)
+        # The dense parameters sit in one slab and their gradients in another (each tensor starts on a
+        # 256-byte boundary, the gaps stay zero), so that the trainer's norm and update are one launch each
+        # over the slab instead of one per parameter.  The lookup table is updated by rows and stays apart.
+        self.dense = [n for n in params if n != "C"]
+        pad = lambda k: (k + 63) // 64 * 64
+        self.dense_elems = sum(pad(params[n].size) for n in self.dense)
+        self.p_dense = dev.zeros((self.dense_elems,), pool=PS)
+        self.g_dense = dev.zeros((self.dense_elems,), pool=PS)
+        off = 0
+        for name in self.dense:
+            a = params[name]
+            self.p[name] = self.p_dense.offset(off, a.shape).set(np.ascontiguousarray(a, dtype=np.float32))
+            self.g[name] = self.g_dense.offset(off, a.shape)
+            off += pad(a.size)
+        self.p["C"] = dev.tensor(params["C"], pool=PS)
+        self.g["C"] = dev.zeros(params["C"].shape, pool=PS)
+        self.sqnorms = dev.zeros((2,), pool=PS)  # [dense slab, touched lookup rows]
         self.gscale = dev.zeros((1,), pool=PS)
         # forward values (FXS pool); [t] slices are contiguous so [T, B, *] is one matrix with T*B columns
         self.ids = dev.empty((N,), np.uint32, pool=FXS)
@@ -201,10 +213,12 @@ class LstmLM:
     def backward(self):
         d, V, E, H, L, B, T, N = self.dev, self.V, self.E, self.H, self.L, self.B, self.T, self.N
         fused = self.path == "fused"
-        # the node path accumulates into every gradient buffer; the fused path overwrites all but d_logits
-        d.zero(self.d_logits if fused else lib_tensor(d, self.d_errs.ptr, self.de_bytes))
+        # the node path accumulates into every gradient buffer (zeroed first, as the executor does); the fused
+        # path overwrites them all
+        if not fused:
+            d.zero(lib_tensor(d, self.d_errs.ptr, self.de_bytes))
         d.constant(self.d_errs, 1.0)  # d loss / d errs[b] through sum_batches(sum(errs))
-        d.pnls_backward(V, N, self.logits, self.aux, self.d_errs, self.d_logits)
+        d.pnls_backward(V, N, self.logits, self.aux, self.d_errs, self.d_logits, assign=fused)
         top = self.h[L - 1]
         d.csum_backward(V, 1, N, self.d_logits, 0, self.g["bias"])
         d.gemm_nt_acc(V, H, N, self.d_logits, top, self.g["R"])
@@ -306,13 +320,10 @@ class LstmLM:
 
     def update(self):
         d = self.dev
-        for k, n in enumerate(self.dense):
-            d.squared_l2norm(self.g[n].size, self.g[n], self.sqnorms.offset(k, (1,)))
-        k = len(self.dense)
-        d.squared_l2norm_rows(self.N, self.plan, self.E, self.V, self.g["C"], self.sqnorms.offset(k, (1,)))
-        d.clip_scale(k + 1, self.sqnorms, self.clip, self.gscale)
-        for n in self.dense:
-            d.sgd_update_scaled(self.p[n].size, self.p[n], self.g[n], self.lr, self.gscale, 1.0, True)
+        d.squared_l2norm(self.dense_elems, self.g_dense, self.sqnorms.offset(0, (1,)))
+        d.squared_l2norm_rows(self.N, self.plan, self.E, self.V, self.g["C"], self.sqnorms.offset(1, (1,)))
+        d.clip_scale(2, self.sqnorms, self.clip, self.gscale)
+        d.sgd_update_scaled(self.dense_elems, self.p_dense, self.g_dense, self.lr, self.gscale, 1.0, True)
         d.sgd_update_rows(self.N, self.plan, self.E, self.V, self.p["C"], self.g["C"], self.lr, self.gscale, 1.0)
 
     def issue(self):

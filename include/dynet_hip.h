@@ -344,6 +344,11 @@ int dyhip_pnls_forward(dyhip_device* dev, size_t rows, unsigned bd, const float*
 int dyhip_pnls_forward_staged(dyhip_device* dev, size_t rows, unsigned bd, const float* x, void* aux, float* fx);
 int dyhip_pnls_backward(dyhip_device* dev, size_t rows, unsigned bd, const float* x, const void* aux,
                         const float* dEdf, float* dEdx);
+/* The same with dEdx overwritten instead of accumulated into: for an executor that knows this
+ * node is the first consumer to contribute to dEdx, it saves zero-filling the buffer
+ * (dynet/exec.cc:207-208) and reading it back, two passes over a rows x bd tensor. */
+int dyhip_pnls_backward_assign(dyhip_device* dev, size_t rows, unsigned bd, const float* x, const void* aux,
+                               const float* dEdf, float* dEdx);
 /* Softmax over dim 0 (dynet/nodes-softmaxes.cc:40-87 forward, :89-125 backward): x is rows x cols
  * with cols = columns x batch.  Forward needs 2*cols floats of scratch (the reference's z and m from
  * pools[SCS], :45-48), backward cols floats (:97-98).  Softmax along dim 1 is not provided. */

@@ -447,6 +447,12 @@ def test_pnls_forward_backward(dev, rows, bd):
     # sum_v (softmax - onehot) == 0 per row
     delta = (dxt.numpy().astype(np.float64) - dx0).sum(1)
     assert np.max(np.abs(delta)) < 1e-4 * max(1.0, np.max(np.abs(dy)))
+    # the overwriting form: the same as accumulating into zeros, whatever the buffer held before
+    dxa = dev.empty((bd, rows))
+    dev.pnls_backward(rows, bd, xt, dev.tensor(ref_aux), dev.tensor(dy), dxa, assign=True)
+    dxz = dev.zeros((bd, rows))
+    dev.pnls_backward(rows, bd, xt, dev.tensor(ref_aux), dev.tensor(dy), dxz)
+    assert dxa.numpy().tobytes() == dxz.numpy().tobytes()
 
 
 def test_logsumexp_shift_invariance_and_no_overflow(dev):
