@@ -356,7 +356,11 @@ def test_lstm_rejects_bad_arguments(dev):
 # LookupNode
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize("vocab,dim,n", [(50000, 512, 256 * 64), (10000, 256, 128), (7, 3, 40), (33, 130, 1000),
-                                         (5, 4, 1)])
+                                         (5, 4, 1),
+                                         # id counts around powers of two, key widths from 9 to 18 bits, a vocabulary that is
+                                         # a power of two
+                                         (4096, 8, 2048), (4096, 8, 2049), (300, 4, 4097), (70000, 4, 8193),
+                                         (1 << 16, 4, 16383), (200000, 4, 16385), (1000, 16, 40000)])
 def test_lookup_gather_bit_exact_and_scatter_add(dev, vocab, dim, n):
     rng = np.random.default_rng(vocab + dim + n)
     table = f32(rng.uniform(-0.1, 0.1, (vocab, dim)))
@@ -393,6 +397,8 @@ def test_lookup_gather_bit_exact_and_scatter_add(dev, vocab, dim, n):
     plan = dev.lookup_build_plan(ids_t, vocab)
     sorted_ids = plan.numpy()[:n]
     assert np.array_equal(sorted_ids, np.sort(ids))
+    pos0 = (4 * n + 255) // 256 * 256 // 4  # each part of the plan starts on a 256-byte boundary
+    assert np.array_equal(plan.numpy()[pos0:pos0 + n], np.argsort(ids, kind="stable"))  # stable: positions ascend in a run
     gt3 = dev.tensor(grads0)
     dev.lookup_accumulate_grads_planned(n, plan, dim, vocab, dev.tensor(g), gt3)
     assert gt3.numpy().tobytes() == got.tobytes()
