@@ -304,6 +304,40 @@ def extras(dev, lib, reps, use_graph=True):
     else:
         us2 = time_loop(dev, [cell_fused], max(reps, 50))
     res["cfg1_lstm_cell"]["fused_cell_path_fwd_bwd_us"] = round(us2, 2)
+    # forward in one launch (input product, recurrent product and cell update from packed weights); the two
+    # packed copies are made once outside the timed region, as a caller does per weight update, not per timestep
+    pWx, pWh = dev.empty(4 * H * I), dev.empty(4 * H * H)
+    dev.lstm_pack_input(I, H, t["Wx"], pWx)
+    dev.lstm_pack_recurrent(H, t["Wh"], pWh)
+
+    def fwd_single():
+        dev.lstm_step_forward_x(I, H, B, pWx, t["x"], pWh, t["h"], t["b"], t["c"], fx, c2, h2)
+
+    def fwd_nodes():
+        dev.lstm_gates_forward([t["x"]], [I], H, B, t["h"], t["Wx"], t["Wh"], t["b"], fx)
+        dev.lstm_c_forward(H, B, t["c"], fx, c2)
+        dev.lstm_h_forward(H, B, c2, fx, h2)
+
+    def cell_single():
+        fwd_single()
+        dev.lstm_cell_backward(H, B, fx, c2, t["c"], t["dh"], None, 0, t["dc"], dpre, dcp2)
+        dev.lstm_recurrent_backward(H, B, t["Wh"], dpre, wb, bb)
+        dev.gemm_tn(I, B, 4 * H, t["Wx"], dpre, 1.0, dx)
+        dev.gemm_nt_acc(4 * H, I, B, dpre, t["x"], dWx)
+        dev.gemm_nt_acc(4 * H, H, B, dpre, t["h"], dWh)
+        dev.csum_backward(4 * H, 1, B, dpre, 0, db)
+
+    for key, fn in (("forward_only_nodes_us", fwd_nodes), ("forward_only_single_launch_us", fwd_single),
+                    ("single_launch_forward_fwd_bwd_us", cell_single)):
+        fn()
+        dev.sync()
+        if use_graph:
+            g = capture(dev, [fn] * 4)
+            us3 = time_graph(dev, g, max(reps, 50), 4)
+            g.destroy()
+        else:
+            us3 = time_loop(dev, [fn], max(reps, 50))
+        res["cfg1_lstm_cell"][key] = round(us3, 2)
     return res
 
 

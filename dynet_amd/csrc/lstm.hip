@@ -237,14 +237,15 @@ constexpr int kStepPitchR = 33;             // quarter-sum exchange: [row][col]
 constexpr int kStepWaveFloats = 2 * 32 * kStepBK + 2 * kStepBK * kStepPitchB;  // per-wave A + B stages
 typedef float stepx16 __attribute__((ext_vector_type(16)));
 
-__global__ __launch_bounds__(256) void lstm_pack_recurrent_kernel(unsigned H, const float* __restrict__ Wh,
+// W is 4H x K (Wh: K = H, Wx: K = the input size)
+__global__ __launch_bounds__(256) void lstm_pack_recurrent_kernel(unsigned H, unsigned K, const float* __restrict__ W,
                                                                   float* __restrict__ Wp) {
-  const size_t o = size_t(blockIdx.x) * 256 + threadIdx.x;  // output index, (rt*H + k)*32 + g*8 + u
-  if (o >= size_t(4) * H * H) return;
+  const size_t o = size_t(blockIdx.x) * 256 + threadIdx.x;  // output index, (rt*K + k)*32 + g*8 + u
+  if (o >= size_t(4) * H * K) return;
   const unsigned r = o % 32, g = r / 8, u = r % 8;
   const size_t tk = o / 32;
-  const unsigned k = tk % H, rt = tk / H;
-  Wp[o] = Wh[size_t(g) * H + rt * 8 + u + size_t(k) * 4 * H];
+  const unsigned k = tk % K, rt = tk / K;
+  Wp[o] = W[size_t(g) * H + rt * 8 + u + size_t(k) * 4 * H];
 }
 
 // orders a wave's LDS writes before the reads its other lanes issue afterwards
@@ -254,8 +255,15 @@ __device__ __forceinline__ void step_wave_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-__global__ __launch_bounds__(256, 2) void lstm_step_fwd_kernel(unsigned H, unsigned B, const float* __restrict__ Wp,
-                                                               const float* __restrict__ h_prev,
+// Up to two products feed the pre-activations: Wx * x (packed Wx, depth I) and Wh * h_tm1 (packed Wh,
+// depth H); either may be absent (null), and Wx * x may instead arrive precomputed in xproj.
+struct StepOperand {
+  const float* Wp;  // packed weights [H/8][K][32]
+  const float* v;   // K x B, column-major
+  unsigned K;
+};
+
+__global__ __launch_bounds__(256, 2) void lstm_step_fwd_kernel(unsigned H, unsigned B, StepOperand op0, StepOperand op1,
                                                                const float* xproj,
                                                                const float* __restrict__ bias,
                                                                const float* __restrict__ c_prev, int mode,
@@ -268,16 +276,7 @@ __global__ __launch_bounds__(256, 2) void lstm_step_fwd_kernel(unsigned H, unsig
   const unsigned l32 = lane % 32, lhi = lane / 32;
   float* la = lds + wave * kStepWaveFloats;
   float* lb = la + 2 * 32 * kStepBK;
-  const unsigned kq = H / 4, k0 = wave * kq, nst = kq / kStepBK;
-
-  const float* ga = Wp + (size_t(rt) * H + k0) * 32 + lane * 4;
   const unsigned bk = 4 * (lane % 8), bc = lane / 8;
-  // columns past the batch are computed on a clamped address and dropped
-  auto column = [&](unsigned i) {
-    const unsigned col = ct * 32 + bc + 8 * i;
-    return h_prev + size_t(col < B ? col : B - 1) * H + k0 + bk;
-  };
-  const float *gb0 = column(0), *gb1 = column(1), *gb2 = column(2), *gb3 = column(3);
 
   // the epilogue's thread owns hidden unit eu of batch column ecc; its operands are fetched
   // now so that their latency hides behind the product
@@ -288,9 +287,10 @@ __global__ __launch_bounds__(256, 2) void lstm_step_fwd_kernel(unsigned H, unsig
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const float bq = bias[q * H + ej];
-      pre[q] = (q == 1 ? bq + 1.0f : bq) + xproj[size_t(ecol) * 4 * H + ej + size_t(q) * H];
+      pre[q] = q == 1 ? bq + 1.0f : bq;
+      if (xproj != nullptr) pre[q] += xproj[size_t(ecol) * 4 * H + ej + size_t(q) * H];
     }
-    cp = c_prev[size_t(ecol) * H + ej];
+    if (c_prev != nullptr) cp = c_prev[size_t(ecol) * H + ej];
   }
 
   float4 ra0, ra1, ra2, ra3, rb0, rb1, rb2, rb3;
@@ -314,22 +314,38 @@ __global__ __launch_bounds__(256, 2) void lstm_step_fwd_kernel(unsigned H, unsig
   // The kernel runs at the rate the L2 delivers the operands (every 32x32 output tile pulls
   // its full-depth strips of both), so one stage of lookahead is enough.
   stepx16 acc = {0};
-  STEP_LOAD(0)
-  STEP_STORE(0)
-  if (nst > 1) { STEP_LOAD(1) }
-  step_wave_sync();
-  for (unsigned st = 0; st < nst; ++st) {
-    const unsigned cur = st & 1;
-    const float* a = la + cur * 32 * kStepBK + lhi * 32 + l32;
-    const float* b = lb + cur * kStepBK * kStepPitchB + lhi * kStepPitchB + l32;
+  const float *ga = nullptr, *gb0 = nullptr, *gb1 = nullptr, *gb2 = nullptr, *gb3 = nullptr;
+  for (int which = 0; which < 2; ++which) {
+    const StepOperand op = which == 0 ? op0 : op1;
+    if (op.Wp == nullptr) continue;  // uniform over the grid
+    const unsigned kq = op.K / 4, k0 = wave * kq, nst = kq / kStepBK;
+    ga = op.Wp + (size_t(rt) * op.K + k0) * 32 + lane * 4;
+    // columns past the batch are computed on a clamped address and dropped
+    auto column = [&](unsigned i) {
+      const unsigned col = ct * 32 + bc + 8 * i;
+      return op.v + size_t(col < B ? col : B - 1) * op.K + k0 + bk;
+    };
+    gb0 = column(0);
+    gb1 = column(1);
+    gb2 = column(2);
+    gb3 = column(3);
+    STEP_LOAD(0)
+    STEP_STORE(0)
+    if (nst > 1) { STEP_LOAD(1) }
+    step_wave_sync();
+    for (unsigned st = 0; st < nst; ++st) {
+      const unsigned cur = st & 1;
+      const float* a = la + cur * 32 * kStepBK + lhi * 32 + l32;
+      const float* b = lb + cur * kStepBK * kStepPitchB + lhi * kStepPitchB + l32;
 #pragma unroll
-    for (int s = 0; s < kStepBK / 2; ++s)
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * s * 32], b[2 * s * kStepPitchB], acc, 0, 0, 0);
-    if (st + 1 < nst) {
-      STEP_STORE(cur ^ 1)
-      if (st + 2 < nst) { STEP_LOAD(st + 2) }
+      for (int s = 0; s < kStepBK / 2; ++s)
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * s * 32], b[2 * s * kStepPitchB], acc, 0, 0, 0);
+      if (st + 1 < nst) {
+        STEP_STORE(cur ^ 1)
+        if (st + 2 < nst) { STEP_LOAD(st + 2) }
+      }
+      step_wave_sync();  // the stages are private to the wave: no block barrier in the loop
     }
-    step_wave_sync();  // the stages are private to the wave: no block barrier in the loop
   }
   __syncthreads();
 #undef STEP_LOAD1
@@ -355,7 +371,7 @@ __global__ __launch_bounds__(256, 2) void lstm_step_fwd_kernel(unsigned H, unsig
   }
   const float gi = logistic(mode, pre[0]), gf = logistic(mode, pre[1]), go = logistic(mode, pre[2]);
   const float gg = tanh_accurate(pre[3]);
-  const float cv = gi * gg + gf * cp;
+  const float cv = c_prev != nullptr ? gi * gg + gf * cp : gi * gg;
   gates[g0] = gi;
   gates[g0 + H] = gf;
   gates[g0 + 2 * size_t(H)] = go;
@@ -671,23 +687,54 @@ int dyhip_lstm_cell_backward(dyhip_device* dev, unsigned H, unsigned B, const fl
   return DYHIP_OK;
 }
 
+static bool step_depth_ok(unsigned K) { return K >= 128 && K % 128 == 0; }  // quarters in whole 32-deep stages
+
 int dyhip_lstm_step_supported(dyhip_device* dev, unsigned H, unsigned B, int* supported) {
   DYHIP_CHECK_DEV(dev);
   DYHIP_REQUIRE(supported, "null output pointer");
-  // quarters of the hidden size in whole 32-deep stages; grid and index ranges in 32 bits
-  *supported = (H >= 128 && H % 128 == 0 && B >= 1 && B <= 65535 && size_t(4) * H * H < (size_t(1) << 32)) ? 1 : 0;
+  // grid and index ranges in 32 bits
+  *supported = (step_depth_ok(H) && B >= 1 && B <= 65535 && size_t(4) * H * H < (size_t(1) << 32)) ? 1 : 0;
+  return DYHIP_OK;
+}
+
+static int pack_weights(dyhip_device* dev, unsigned H, unsigned K, const float* W, float* packed) {
+  DYHIP_REQUIRE(step_depth_ok(H) && step_depth_ok(K) && size_t(4) * H * K < (size_t(1) << 32),
+                "LSTM step: hidden size %u and product depth %u must be multiples of 128", H, K);
+  DYHIP_REQUIRE(W && packed, "LSTM step: null tensor pointer");
+  const size_t n = size_t(4) * H * K;
+  hipLaunchKernelGGL(lstm_pack_recurrent_kernel, dim3(unsigned(cdiv<size_t>(n, 256))), dim3(256), 0, dev->stream, H, K, W,
+                     packed);
+  DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
 
 int dyhip_lstm_pack_recurrent(dyhip_device* dev, unsigned H, const float* Wh, float* packed) {
   DYHIP_CHECK_DEV(dev);
+  return pack_weights(dev, H, H, Wh, packed);
+}
+
+int dyhip_lstm_pack_input(dyhip_device* dev, unsigned I, unsigned H, const float* Wx, float* packed) {
+  DYHIP_CHECK_DEV(dev);
+  return pack_weights(dev, H, I, Wx, packed);
+}
+
+static int step_forward(dyhip_device* dev, unsigned I, unsigned H, unsigned B, const float* packed_Wx, const float* x,
+                        const float* packed_Wh, const float* h_tm1, const float* xproj, const float* b,
+                        const float* c_tm1, int logistic_mode, float* gates, float* c, float* h) {
   int ok = 0;
-  dyhip_lstm_step_supported(dev, H, 1, &ok);
-  DYHIP_REQUIRE(ok, "LSTM step: hidden size %u is not a multiple of 128", H);
-  DYHIP_REQUIRE(Wh && packed, "LSTM step: null tensor pointer");
-  const size_t n = size_t(4) * H * H;
-  hipLaunchKernelGGL(lstm_pack_recurrent_kernel, dim3(unsigned(cdiv<size_t>(n, 256))), dim3(256), 0, dev->stream, H, Wh,
-                     packed);
+  dyhip_lstm_step_supported(dev, H, B, &ok);
+  DYHIP_REQUIRE(ok, "LSTM step: unsupported hidden (%u) or batch (%u) size", H, B);
+  DYHIP_REQUIRE(b && gates && c && h, "LSTM step: null tensor pointer");
+  DYHIP_REQUIRE((packed_Wx == nullptr) == (x == nullptr) && (packed_Wh == nullptr) == (h_tm1 == nullptr),
+                "LSTM step: packed weights and their operand come together");
+  DYHIP_REQUIRE(packed_Wx == nullptr || step_depth_ok(I), "LSTM step: input size %u is not a multiple of 128", I);
+  DYHIP_REQUIRE(all_aligned16({packed_Wx, x, packed_Wh, h_tm1}), "LSTM step: weights and operands must be 16-byte aligned");
+  DYHIP_REQUIRE(logistic_mode == DYHIP_LOGISTIC_PACKET || logistic_mode == DYHIP_LOGISTIC_SCALAR,
+                "unknown logistic mode %d", logistic_mode);
+  const StepOperand op0{packed_Wx, x, I}, op1{packed_Wh, h_tm1, H};
+  const unsigned blocks = (H / 8) * cdiv<unsigned>(B, 32);
+  hipLaunchKernelGGL(lstm_step_fwd_kernel, dim3(blocks), dim3(256), 0, dev->stream, H, B, op0, op1, xproj, b, c_tm1,
+                     logistic_mode, gates, c, h);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
@@ -696,18 +743,16 @@ int dyhip_lstm_step_forward(dyhip_device* dev, unsigned H, unsigned B, const flo
                             const float* xproj, const float* b, const float* c_tm1, int logistic_mode, float* gates,
                             float* c, float* h) {
   DYHIP_CHECK_DEV(dev);
-  int ok = 0;
-  dyhip_lstm_step_supported(dev, H, B, &ok);
-  DYHIP_REQUIRE(ok, "LSTM step: unsupported hidden (%u) or batch (%u) size", H, B);
-  DYHIP_REQUIRE(packed_Wh && h_tm1 && xproj && b && c_tm1 && gates && c && h, "LSTM step: null tensor pointer");
-  DYHIP_REQUIRE(aligned16(packed_Wh) && aligned16(h_tm1), "LSTM step: packed weights and h_tm1 must be 16-byte aligned");
-  DYHIP_REQUIRE(logistic_mode == DYHIP_LOGISTIC_PACKET || logistic_mode == DYHIP_LOGISTIC_SCALAR,
-                "unknown logistic mode %d", logistic_mode);
-  const unsigned blocks = (H / 8) * cdiv<unsigned>(B, 32);
-  hipLaunchKernelGGL(lstm_step_fwd_kernel, dim3(blocks), dim3(256), 0, dev->stream, H, B, packed_Wh, h_tm1, xproj, b,
-                     c_tm1, logistic_mode, gates, c, h);
-  DYHIP_CHECK_LAUNCH();
-  return DYHIP_OK;
+  DYHIP_REQUIRE(packed_Wh && h_tm1 && xproj && c_tm1, "LSTM step: null tensor pointer");
+  return step_forward(dev, 0, H, B, nullptr, nullptr, packed_Wh, h_tm1, xproj, b, c_tm1, logistic_mode, gates, c, h);
+}
+
+int dyhip_lstm_step_forward_x(dyhip_device* dev, unsigned I, unsigned H, unsigned B, const float* packed_Wx,
+                              const float* x, const float* packed_Wh, const float* h_tm1, const float* b,
+                              const float* c_tm1, int logistic_mode, float* gates, float* c, float* h) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(packed_Wx && x, "LSTM step: null tensor pointer");
+  return step_forward(dev, I, H, B, packed_Wx, x, packed_Wh, h_tm1, nullptr, b, c_tm1, logistic_mode, gates, c, h);
 }
 
 }  // extern "C"

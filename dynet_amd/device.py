@@ -405,6 +405,14 @@ class Device:
         _check(cdll.dyhip_lstm_step_forward(self.handle, _u(H), _u(B), _p(packed_Wh), _p(h_tm1), _p(xproj), _p(b),
                                             _p(c_tm1), _i(logistic_mode), _p(gates), _p(c), _p(h)))
 
+    def lstm_pack_input(self, I, H, Wx, packed):
+        _check(cdll.dyhip_lstm_pack_input(self.handle, _u(I), _u(H), _p(Wx), _p(packed)))
+
+    def lstm_step_forward_x(self, I, H, B, packed_Wx, x, packed_Wh, h_tm1, b, c_tm1, gates, c, h,
+                            logistic_mode=lib.LOGISTIC_PACKET):
+        _check(cdll.dyhip_lstm_step_forward_x(self.handle, _u(I), _u(H), _u(B), _p(packed_Wx), _p(x), _p(packed_Wh),
+                                              _p(h_tm1), _p(b), _p(c_tm1), _i(logistic_mode), _p(gates), _p(c), _p(h)))
+
     def lstm_cell_backward(self, H, B, gates, c, c_tm1, dh, rec, splits, dc, dpre, dc_tm1):
         _check(cdll.dyhip_lstm_cell_backward(self.handle, _u(H), _u(B), _p(gates), _p(c), _p(c_tm1), _p(dh), _vp(rec),
                                              _u(splits), _p(dc), _p(dpre), _p(dc_tm1)))

@@ -283,6 +283,15 @@ int dyhip_lstm_pack_recurrent(dyhip_device* dev, unsigned H, const float* Wh, fl
 int dyhip_lstm_step_forward(dyhip_device* dev, unsigned H, unsigned B, const float* packed_Wh, const float* h_tm1,
                             const float* xproj, const float* b, const float* c_tm1, int logistic_mode, float* gates,
                             float* c, float* h);
+/* The whole forward of a timestep in one launch, input product included: gates = act(b + [f: +1] +
+ * Wx * x + Wh * h_tm1) from packed copies of both weight matrices (dyhip_lstm_pack_input: Wx is
+ * 4H x I, I a multiple of 128), then c and h.  For callers that see one timestep at a time
+ * (decoding, the single-step configuration).  packed_Wh / h_tm1 / c_tm1 = NULL stand for the
+ * zero initial state. */
+int dyhip_lstm_pack_input(dyhip_device* dev, unsigned I, unsigned H, const float* Wx, float* packed);
+int dyhip_lstm_step_forward_x(dyhip_device* dev, unsigned I, unsigned H, unsigned B, const float* packed_Wx,
+                              const float* x, const float* packed_Wh, const float* h_tm1, const float* b,
+                              const float* c_tm1, int logistic_mode, float* gates, float* c, float* h);
 
 /* ---- random tensors: TensorTools::randomize_{uniform,normal,bernoulli}
  * (dynet/tensor.cc:261-303), Device_GPU::reset_rng (dynet/devices.cc:130-135), the Dropout

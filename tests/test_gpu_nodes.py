@@ -332,6 +332,41 @@ def test_single_launch_step_equals_node_composition(dev, I, H, B):
             assert_close(out["step"][q][k], out["two_call"][q][k], FWD_RTOL, f"{what}[{k}] vs two-call", floor=floor)
 
 
+@pytest.mark.parametrize("I,H,B", [(128, 256, 32), (256, 128, 1), (128, 128, 45), (384, 256, 70)])
+def test_single_launch_step_with_input_product(dev, I, H, B):
+    """dyhip_lstm_step_forward_x: Wx*x, Wh*h_tm1, bias, activations, c and h in one launch, from the zero state
+    (no recurrent operand) and from a given state, against the oracle's gates -> C -> H nodes."""
+    rng = np.random.default_rng(I + 3 * H + B)
+    Wx, Wh, b = glorot(rng, 4 * H, I), glorot(rng, 4 * H, H), f32(rng.normal(0, 0.1, 4 * H))
+    Wxt, Wht, bt = dev.tensor(Wx), dev.tensor(Wh), dev.tensor(b)
+    pWx, pWh = dev.empty(4 * H * I), dev.empty(4 * H * H)
+    dev.lstm_pack_input(I, H, Wxt, pWx)
+    dev.lstm_pack_recurrent(H, Wht, pWh)
+    assert np.array_equal(pWx.numpy(), Wx.reshape(I, 4, H // 8, 8).transpose(2, 0, 1, 3).reshape(-1))
+    zeros = np.zeros((B, H), F32)
+    h_prev, c_prev = zeros, zeros
+    ht = ct = None
+    floor = max(1.0, float(np.sqrt(I + H) * max(rms(Wx), rms(Wh))))
+    for t in range(3):
+        x = f32(rng.standard_normal((B, I)))
+        g_ref = orc.lstm_gates_forward([x], [I], H, B, h_prev, Wx, Wh, b)
+        c_ref = orc.lstm_c_forward(H, B, c_prev, g_ref)
+        h_ref = orc.lstm_h_forward(H, B, c_ref, g_ref)
+        g2, c2, h2 = dev.empty((B, 4 * H)), dev.empty((B, H)), dev.empty((B, H))
+        if t == 0:
+            dev.lstm_step_forward_x(I, H, B, pWx, dev.tensor(x), None, None, bt, None, g2, c2, h2)
+        else:
+            dev.lstm_step_forward_x(I, H, B, pWx, dev.tensor(x), pWh, ht, bt, ct, g2, c2, h2)
+        assert_close(g2.numpy(), g_ref, FWD_RTOL, f"gates[{t}]", floor=floor)
+        assert_close(c2.numpy(), c_ref, FWD_RTOL, f"c[{t}]", floor=floor)
+        assert_close(h2.numpy(), h_ref, FWD_RTOL, f"h[{t}]", floor=floor)
+        ht, ct, h_prev, c_prev = h2, c2, h_ref, c_ref
+    with pytest.raises(DyhipError):
+        dev.lstm_step_forward_x(96, H, B, pWx, ht, pWh, ht, bt, ct, g2, c2, h2)
+    with pytest.raises(DyhipError):
+        dev.lstm_step_forward_x(I, H, B, pWx, ht, pWh, None, bt, ct, g2, c2, h2)
+
+
 def test_single_launch_step_rejects_unsupported_sizes(dev):
     assert not dev.lstm_step_supported(96, 4)
     assert not dev.lstm_step_supported(130, 4)
