@@ -230,7 +230,8 @@ __device__ __forceinline__ float logistic(int mode, float x) {
 // tanh uses): p(x)/q(x) with p odd, so the result is relatively accurate for small
 // |x| too; max relative error 4e-7 against fp64 tanh over the whole range.
 // Branch-free: one median-of-three clamp, 9 fused multiply-adds, one hardware
-// reciprocal (1 ulp; q >= 4.89e-3, no special cases).
+// reciprocal (1 ulp; q >= 4.89e-3), and one select that hands a NaN input through
+// (the clamp alone would turn it into -9, i.e. tanh(NaN) = -1; tanhf returns NaN).
 __device__ __forceinline__ float tanh_accurate(float _x) {
   const float x = __builtin_amdgcn_fmed3f(_x, -9.0f, 9.0f);
   const float x2 = x * x;
@@ -244,7 +245,8 @@ __device__ __forceinline__ float tanh_accurate(float _x) {
   float q = fmaf(x2, 1.19825839466702e-06f, 1.18534705686654e-04f);
   q = fmaf(x2, q, 2.26843463243900e-03f);
   q = fmaf(x2, q, 4.89352518554385e-03f);
-  return p * __builtin_amdgcn_rcpf(q);
+  const float r = p * __builtin_amdgcn_rcpf(q);
+  return _x != _x ? _x : r;
 }
 
 }  // namespace dyhip

@@ -25,6 +25,13 @@ struct MaxSum {
   float m, s;
 };
 
+// The running maximum starts at the most negative finite float, never at -inf: a thread whose first
+// values are all -inf (masked logits) then adds exp(-inf - finite) = 0 instead of exp(-inf + inf) = NaN.
+// Any finite input is >= this start value, so the final maximum is exact; a column that holds nothing
+// but -inf ends with s == 0 and is given the reference's result (m = -inf, z = NaN: its
+// exp(x - m) is exp(NaN), dynet/tensor.cc:468-507) when the block writes its outputs.
+constexpr float kLseStartMax = -3.402823466e+38f;
+
 __device__ __forceinline__ void ms_push4(MaxSum& a, const float4 v) {
   const float cm = fmaxf(fmaxf(v.x, v.y), fmaxf(v.z, v.w));
   if (cm > a.m) {
@@ -45,10 +52,8 @@ __device__ __forceinline__ void ms_push1(MaxSum& a, const float v) {
 __device__ __forceinline__ MaxSum ms_merge(const MaxSum a, const MaxSum b) {
   MaxSum r;
   r.m = fmaxf(a.m, b.m);
-  // an empty partial has m = -inf and s = 0; keep it from producing exp(-inf - -inf)
-  const float sa = a.s == 0.f ? 0.f : a.s * __expf(a.m - r.m);
-  const float sb = b.s == 0.f ? 0.f : b.s * __expf(b.m - r.m);
-  r.s = sa + sb;
+  // both maxima are finite (see kLseStartMax), so neither exponent can be inf - inf
+  r.s = a.s * __expf(a.m - r.m) + b.s * __expf(b.m - r.m);
   return r;
 }
 
@@ -63,7 +68,7 @@ __global__ __launch_bounds__(kLseThreads) void lse_cols_kernel(size_t rows, cons
   const unsigned b = blockIdx.x;
   const float* px = x + size_t(b) * rows;
   MaxSum a;
-  a.m = -INFINITY;
+  a.m = kLseStartMax;
   a.s = 0.f;
   // the picked logit is fetched up front so that its two dependent loads overlap the streaming pass
   float picked = 0.f;
@@ -108,7 +113,7 @@ __global__ __launch_bounds__(kLseThreads) void lse_cols_kernel(size_t rows, cons
   if (w == 0) {
     // wave 0 merges the per-wave pairs with a butterfly over the first kLseWaves lanes
     MaxSum t;
-    t.m = lane < kLseWaves ? lm[lane] : -INFINITY;
+    t.m = lane < kLseWaves ? lm[lane] : kLseStartMax;
     t.s = lane < kLseWaves ? ls[lane] : 0.f;
 #pragma unroll
     for (int off = kLseWaves / 2; off > 0; off >>= 1) {
@@ -118,7 +123,9 @@ __global__ __launch_bounds__(kLseThreads) void lse_cols_kernel(size_t rows, cons
       t = ms_merge(t, o);
     }
     if (lane == 0) {
-      const float z = logf(t.s) + t.m;
+      const bool empty = t.s == 0.f;  // every input was -inf
+      const float z = empty ? NAN : logf(t.s) + t.m;
+      if (empty) t.m = -INFINITY;
       m_out[b] = t.m;
       z_out[b] = z;
       if (ids != nullptr) fx[b] = z - picked;

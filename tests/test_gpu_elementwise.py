@@ -81,6 +81,18 @@ def test_tanh_is_relatively_accurate_everywhere(dev):
     assert np.max(err / np.maximum(np.abs(ref), 1e-37)) < 1e-6
 
 
+def test_tanh_special_values(dev):
+    """NaN goes through (tanhf(NaN) = NaN, as on the reference's CPU and GPU paths), infinities saturate."""
+    x = f32([np.nan, -np.nan, np.inf, -np.inf, 0.0, -0.0, 1e-40, 100.0] * 65)
+    yt = dev.empty(x.size)
+    dev.unary_forward(lib.OP_TANH, dev.tensor(x), yt)
+    got, want = yt.numpy(), orc.unary_forward(orc.OP_TANH, x)
+    assert np.array_equal(np.isnan(got), np.isnan(want)) and np.isnan(got[:2]).all()
+    ok = ~np.isnan(want)
+    assert np.max(np.abs(got[ok] - want[ok])) <= 1e-6
+    assert abs(got[2] - 1.0) < 1e-7 and abs(got[3] + 1.0) < 1e-7 and got[4] == 0.0  # saturates within one ulp
+
+
 def test_unary_on_a_misaligned_buffer(dev):
     x, dy, dx0 = _inputs(4099, 11)
     base = dev.tensor(np.concatenate([[0.0], x]))  # view starting 4 bytes into the allocation

@@ -68,6 +68,52 @@ def test_lm_step_matches_oracle(dev, case, path, time_batched, overlap):
             lm.p[n].set(ref_p[n])
 
 
+@pytest.fixture(scope="module")
+def wide_case():
+    """The LM configuration's layer widths (E = 256, H = 1024, two layers, B = 128: the sizes that select the
+    production kernels - 128-wide GEMM tiles, the single-launch timestep, split-K recurrent products) with a
+    vocabulary and a sequence length small enough for one CPU core: the oracle step takes ~10 s, once."""
+    V, E, H, L, B, T = 300, 256, 1024, 2, 128, 3
+    rng = np.random.default_rng(23)
+    params = LstmLM.init_params(V, E, H, L, seed=5)
+    for l in range(L):
+        params[f"b{l}"] = rng.normal(0, 0.1, 4 * H).astype(np.float32)
+    tokens = _tokens(rng, V, B, T)
+    ref_p = {n: a.copy() for n, a in params.items()}
+    ref_loss, ref_g, ref_scale = lm_oracle.step(ref_p, tokens, L, lr=0.1, clip=5.0)
+    return (V, E, H, L, B, T), params, tokens, ref_loss, ref_g, ref_scale, ref_p
+
+
+@pytest.mark.parametrize("path,time_batched,overlap", [("nodes", False, False), ("fused", True, False),
+                                                       ("fused", True, True)])
+def test_lm_step_matches_oracle_at_production_width(dev, wide_case, path, time_batched, overlap):
+    (V, E, H, L, B, T), params, tokens, ref_loss, ref_g, ref_scale, ref_p = wide_case
+    lm = LstmLM(dev, V, E, H, L, B, T, lr=0.1, clip=5.0, time_batched=time_batched,
+                params={n: a.copy() for n, a in params.items()}, path=path, overlap=overlap, chunk=2)
+    assert lm.single_launch == (path == "fused")
+    lm.stage(tokens)
+    lm.dev.lookup_build_plan_into(lm.ids, V, lm.plan, lm.plan_ws, lm.plan_ws_bytes)
+    lm.forward()
+    lm.backward()
+    loss = lm.loss.numpy()[0]
+    grads = lm.get_grads()
+    lm.update()
+    assert_close(loss, ref_loss, FWD_RTOL * 4, "loss")
+    for n in ref_g:
+        assert_close(grads[n], ref_g[n], GRAD_RTOL, f"grad {n}", floor=_grad_floor(ref_g[n]))
+    # The clip scale is 5 / |g| over 13 M gradient elements.  The CPU oracle adds their squares one by one in
+    # fp32, which stagnates at this length (each addend is about one ulp of the running sum): it is 3e-4 off
+    # the fp64 norm of its own gradients, and the reference's Eigen reduction is a blocked tree, not that
+    # chain.  The yardstick is therefore the fp64 norm of the oracle's gradients.
+    exact = min(1.0, 5.0 / np.sqrt(sum(float((a.astype(np.float64) ** 2).sum()) for a in ref_g.values())))
+    assert abs(ref_scale - exact) < 1e-3 * exact
+    assert_close(lm.gscale.numpy()[0], exact, GRAD_RTOL, "clip scale")
+    new_p = lm.get_params()
+    for n in ref_p:  # SimpleSGD with that scale: p -= lr * scale * g
+        want = params[n].astype(np.float64) - 0.1 * exact * ref_g[n].astype(np.float64)
+        assert_close(new_p[n], want, GRAD_RTOL, f"param {n}", floor=_grad_floor(ref_p[n]))
+
+
 def test_lm_clipping_engages(dev):
     V, E, H, L, B, T = 50, 16, 32, 2, 8, 5
     rng = np.random.default_rng(5)

@@ -7,7 +7,7 @@ import pytest
 
 from dynet_amd import DyhipError, lib
 from oracle import cpu_oracle as orc
-from util import F32, FWD_RTOL, GRAD_RTOL, assert_close, f32, glorot, rms, zipf_ids
+from util import F32, FWD_RTOL, GRAD_RTOL, assert_close, assert_shadow, f32, glorot, rms, zipf_ids
 
 pytestmark = pytest.mark.gpu
 
@@ -103,6 +103,34 @@ def test_lstm_golden_vectors(dev, golden):
         assert_close(fx.numpy().reshape(-1), np.array(t["gates"]), rel, name)
 
 
+def _sig64(v):
+    return 1.0 / (1.0 + np.exp(-v))
+
+
+def _lstm_exact_step(x, h_prev, c_prev, Wx, Wh, b, mask_x=None, mask_h=None):
+    """One VanillaLSTMGates -> C -> H step in fp64 from fp32 inputs (true sigmoid / tanh): the yardstick
+    for assert_shadow.  Weights are stored [k][row], so the pre-activation is x Wx + h Wh + b (+1 on f)."""
+    f64 = lambda a: np.asarray(a, np.float64)
+    H = h_prev.shape[1]
+    xm = f64(x) * (f64(mask_x) if mask_x is not None else 1.0)
+    hm = f64(h_prev) * (f64(mask_h) if mask_h is not None else 1.0)
+    pre = xm @ f64(Wx) + hm @ f64(Wh) + f64(b)
+    pre[:, H:2 * H] += 1.0
+    g = np.concatenate([_sig64(pre[:, :3 * H]), np.tanh(pre[:, 3 * H:])], axis=1)
+    c = g[:, :H] * g[:, 3 * H:] + g[:, H:2 * H] * f64(c_prev)
+    h = g[:, 2 * H:3 * H] * np.tanh(c)
+    return g, c, h
+
+
+def _assert_gates_shadow(got, ref, exact, H, what):
+    """Sigmoid gates: relative everywhere (a small gate has a large negative pre-activation, so its relative
+    error is the absolute error of that sum).  The tanh gate, c and h pass through zero, where a relative
+    error measures nothing (tanh(s) ~ s for a sum s of O(1) terms that cancels): absolute everywhere,
+    relative above 0.1."""
+    assert_shadow(got[:, :3 * H], ref[:, :3 * H], exact[:, :3 * H], what + " (i,f,o)")
+    assert_shadow(got[:, 3 * H:], ref[:, 3 * H:], exact[:, 3 * H:], what + " (g)", rel_min=0.1)
+
+
 def _lstm_case(rng, I, H, B):
     x = f32(rng.standard_normal((B, I)))
     h = f32(rng.standard_normal((B, H)))
@@ -150,14 +178,21 @@ def test_lstm_cell_forward_backward(dev, I, H, B, dims, dropout, mask_full):
     # an fp32 GEMM in another summation order moves the pre-activation by ~1e-7*scale;
     # the gate moves by at most that (|sigma'|, |tanh'| <= 1)
     assert_close(fx_t.numpy(), fx_ref, FWD_RTOL, "gates fwd", floor=max(1.0, scale))
+    # ... and every gate, however small, is as close to the fp64 value as the CPU path is
+    g64, _, _ = _lstm_exact_step(x, h, c_prev, Wx, Wh, b, mx, mh)
+    _assert_gates_shadow(fx_t.numpy(), fx_ref, g64, H, "gates fwd")
     c_t, h_t = dev.empty((B, H)), dev.empty((B, H))
     fxo_t = dev.tensor(fx_ref)  # downstream nodes are compared from identical inputs
     dev.lstm_c_forward(H, B, ct, fxo_t, c_t)
     c_ref = orc.lstm_c_forward(H, B, c_prev, fx_ref)
     assert_close(c_t.numpy(), c_ref, FWD_RTOL, "c fwd", floor=1e-3)
+    f64 = lambda a: a.astype(np.float64)
+    c64 = f64(fx_ref[:, :H]) * f64(fx_ref[:, 3 * H:]) + f64(fx_ref[:, H:2 * H]) * f64(c_prev)
+    assert_shadow(c_t.numpy(), c_ref, c64, "c fwd", rel_min=0.1)
     dev.lstm_h_forward(H, B, dev.tensor(c_ref), fxo_t, h_t)
     h_ref = orc.lstm_h_forward(H, B, c_ref, fx_ref)
     assert_close(h_t.numpy(), h_ref, FWD_RTOL, "h fwd", floor=1e-6)
+    assert_shadow(h_t.numpy(), h_ref, f64(fx_ref[:, 2 * H:3 * H]) * np.tanh(f64(c_ref)), "h fwd", rel_min=1e-6)
 
     # ---- backward: h -> c -> gates, every argument, into non-zero buffers ----
     dh, dc_up = f32(rng.standard_normal((B, H))), f32(rng.standard_normal((B, H)))
@@ -249,10 +284,15 @@ def test_fused_cell_path_equals_node_composition(dev, I, H, B):
     # another summation order moves a pre-activation by ~1e-7 * (size of its terms); the gate, c and h
     # move by at most that (|sigma'|, |tanh'| <= 1)
     floor = max(1.0, float(np.sqrt(I + H) * max(rms(Wx), rms(Wh))))
+    h64, c64 = zeros, zeros
     for k in range(2):
         assert_close(sl(gates, k, 4 * H).numpy(), ref[k][0], FWD_RTOL, f"gates[{k}]", floor=floor)
         assert_close(sl(cs, k, H).numpy(), ref[k][1], FWD_RTOL, f"c[{k}]", floor=floor)
         assert_close(sl(hs, k, H).numpy(), ref[k][2], FWD_RTOL, f"h[{k}]", floor=floor)
+        g64, c64, h64 = _lstm_exact_step(xs[k], h64, c64, Wx, Wh, b)
+        _assert_gates_shadow(sl(gates, k, 4 * H).numpy(), ref[k][0], g64, H, f"gates[{k}]")
+        assert_shadow(sl(cs, k, H).numpy(), ref[k][1], c64, f"c[{k}]", rel_min=0.1)
+        assert_shadow(sl(hs, k, H).numpy(), ref[k][2], h64, f"h[{k}]", rel_min=0.1)
     # backward: gradients arrive at h of both steps
     dh = [f32(rng.standard_normal((B, H))) for _ in range(2)]
     r_dh = [d.copy() for d in dh]
@@ -326,10 +366,17 @@ def test_single_launch_step_equals_node_composition(dev, I, H, B):
                                       sl(cs, t, H), sl(hs, t, H))
         out[name] = (gates.numpy(), cs.numpy(), hs.numpy())
     floor = max(1.0, float(np.sqrt(I + H) * max(rms(Wx), rms(Wh))))
+    h64, c64 = zeros, zeros
     for k in range(T):
         for q, what in enumerate(("gates", "c", "h")):
             assert_close(out["step"][q][k], ref[k][q], FWD_RTOL, f"{what}[{k}] vs oracle", floor=floor)
             assert_close(out["step"][q][k], out["two_call"][q][k], FWD_RTOL, f"{what}[{k}] vs two-call", floor=floor)
+        exact = _lstm_exact_step(xs[k], h64, c64, Wx, Wh, b)
+        _, c64, h64 = exact
+        for name in ("step", "two_call"):
+            _assert_gates_shadow(out[name][0][k], ref[k][0], exact[0], H, f"gates[{k}] {name}")
+            assert_shadow(out[name][1][k], ref[k][1], exact[1], f"c[{k}] {name}", rel_min=0.1)
+            assert_shadow(out[name][2][k], ref[k][2], exact[2], f"h[{k}] {name}", rel_min=0.1)
 
 
 @pytest.mark.parametrize("I,H,B", [(128, 256, 32), (256, 128, 1), (128, 128, 45), (384, 256, 70)])
@@ -352,6 +399,7 @@ def test_single_launch_step_with_input_product(dev, I, H, B):
         g_ref = orc.lstm_gates_forward([x], [I], H, B, h_prev, Wx, Wh, b)
         c_ref = orc.lstm_c_forward(H, B, c_prev, g_ref)
         h_ref = orc.lstm_h_forward(H, B, c_ref, g_ref)
+        g64, c64, h64 = _lstm_exact_step(x, h_prev, c_prev, Wx, Wh, b)  # both sides start the step from h_ref, c_ref
         g2, c2, h2 = dev.empty((B, 4 * H)), dev.empty((B, H)), dev.empty((B, H))
         if t == 0:
             dev.lstm_step_forward_x(I, H, B, pWx, dev.tensor(x), None, None, bt, None, g2, c2, h2)
@@ -360,6 +408,13 @@ def test_single_launch_step_with_input_product(dev, I, H, B):
         assert_close(g2.numpy(), g_ref, FWD_RTOL, f"gates[{t}]", floor=floor)
         assert_close(c2.numpy(), c_ref, FWD_RTOL, f"c[{t}]", floor=floor)
         assert_close(h2.numpy(), h_ref, FWD_RTOL, f"h[{t}]", floor=floor)
+        if t > 0:
+            ht.set(h_prev)   # the device step starts from the CPU path's state, as the fp64 yardstick does
+            ct.set(c_prev)
+            dev.lstm_step_forward_x(I, H, B, pWx, dev.tensor(x), pWh, ht, bt, ct, g2, c2, h2)
+        _assert_gates_shadow(g2.numpy(), g_ref, g64, H, f"gates[{t}]")
+        assert_shadow(c2.numpy(), c_ref, c64, f"c[{t}]", rel_min=0.1)
+        assert_shadow(h2.numpy(), h_ref, h64, f"h[{t}]", rel_min=0.1)
         ht, ct, h_prev, c_prev = h2, c2, h_ref, c_ref
     with pytest.raises(DyhipError):
         dev.lstm_step_forward_x(96, H, B, pWx, ht, pWh, ht, bt, ct, g2, c2, h2)
@@ -484,16 +539,63 @@ def test_pnls_forward_backward(dev, rows, bd):
     dxt = dev.tensor(dx0)
     dev.pnls_backward(rows, bd, xt, dev.tensor(ref_aux), dev.tensor(dy), dxt)
     want = orc.pnls_backward(rows, bd, x, ref_aux, dy, dx0.copy())
-    assert_close(dxt.numpy(), want, GRAD_RTOL, "pnls bwd", floor=1e-4)
+    assert_close(dxt.numpy(), want, GRAD_RTOL, "pnls bwd", floor=np.maximum(np.abs(dx0), 1e-7))
     # sum_v (softmax - onehot) == 0 per row
     delta = (dxt.numpy().astype(np.float64) - dx0).sum(1)
     assert np.max(np.abs(delta)) < 1e-4 * max(1.0, np.max(np.abs(dy)))
-    # the overwriting form: the same as accumulating into zeros, whatever the buffer held before
-    dxa = dev.empty((bd, rows))
-    dev.pnls_backward(rows, bd, xt, dev.tensor(ref_aux), dev.tensor(dy), dxa, assign=True)
+    # the gradient itself, without a buffer that hides its small terms: accumulate into zeros and the
+    # overwriting form, each against the oracle element by element.  Every softmax term exp(x - z) * dy is
+    # held to 1e-4 relative down to p = 1e-7 (the floor |dy| * 1e-7); the picked element is p*dy - dy.
+    want0 = orc.pnls_backward(rows, bd, x, ref_aux, dy, np.zeros((bd, rows), F32))
+    floor0 = np.abs(dy)[:, None] * 1e-7 * np.ones((1, rows))
+    floor0[np.arange(bd), labels] = np.abs(dy)
     dxz = dev.zeros((bd, rows))
     dev.pnls_backward(rows, bd, xt, dev.tensor(ref_aux), dev.tensor(dy), dxz)
+    assert_close(dxz.numpy(), want0, GRAD_RTOL, "pnls bwd into zeros", floor=floor0)
+    # the overwriting form: the same, whatever the buffer held before
+    dxa = dev.empty((bd, rows))
+    dev.pnls_backward(rows, bd, xt, dev.tensor(ref_aux), dev.tensor(dy), dxa, assign=True)
+    assert_close(dxa.numpy(), want0, GRAD_RTOL, "pnls bwd assign", floor=floor0)
     assert dxa.numpy().tobytes() == dxz.numpy().tobytes()
+
+
+@pytest.mark.parametrize("rows", [64, 4099, 13])
+def test_logsumexp_with_minus_infinity_entries(dev, rows):
+    """Masked logits: -inf entries contribute exp(-inf - m) = 0, as in the reference's max-first form
+    (dynet/tensor.cc:468-507), wherever they sit: the first 128-bit group of a thread, the scalar tail of a
+    row count that is not a multiple of four, whole wavefronts.  A column of nothing but -inf gives NaN there
+    (exp(-inf + inf)) and here."""
+    rng = np.random.default_rng(rows)
+    bd = 7
+    x = f32(rng.standard_normal((bd, rows)) * 2.0)
+    x[0, :4] = -np.inf                      # a thread's first float4
+    x[1, :min(rows, 4096)] = -np.inf        # every thread's first group (all of the column when rows <= 4096)
+    x[1, -1] = 0.5
+    x[2, ::2] = -np.inf
+    x[3, 1:] = -np.inf                      # a single finite entry
+    x[4, :] = -np.inf                       # nothing finite at all
+    x[5, -3:] = -np.inf                     # the scalar tail
+    labels = rng.integers(0, rows, bd).astype(np.uint32)
+    labels[3] = 0
+    xt = dev.tensor(x)
+    m_t, z_t = dev.empty(bd), dev.empty(bd)
+    dev.logsumexp_cols(rows, bd, xt, m_t, z_t)
+    aux, fx = dev.empty(3 * bd), dev.empty(bd)
+    dev.pnls_forward(rows, bd, xt, labels, aux, fx)
+    ref_fx, ref_aux = orc.pnls_forward(rows, bd, x, labels)
+    ref_z, ref_m = ref_aux[:bd], ref_aux[bd:2 * bd]
+    assert np.isnan(ref_z[4]) and np.isnan(z_t.numpy()[4]) and np.isnan(fx.numpy()[4])
+    ok = np.arange(bd) != 4
+    assert m_t.numpy().tobytes() == ref_m.tobytes()
+    assert_close(z_t.numpy()[ok], ref_z[ok], FWD_RTOL, "logsumexp with -inf", floor=1e-3)
+    fin = ok & np.isfinite(ref_fx)
+    assert np.array_equal(np.isfinite(fx.numpy()[ok]), np.isfinite(ref_fx[ok]))
+    assert_close(fx.numpy()[fin], ref_fx[fin], FWD_RTOL, "pnls fwd with -inf", floor=1.0)
+    keep = np.array([0, 1, 2, 3, 5, 6])
+    xs = np.ascontiguousarray(x[keep])
+    sm = dev.empty((keep.size, rows))
+    dev.softmax_forward(rows, keep.size, dev.tensor(xs), sm)
+    assert_close(sm.numpy(), orc.softmax_forward(rows, keep.size, xs), FWD_RTOL, "softmax with -inf", floor=1e-30)
 
 
 def test_logsumexp_shift_invariance_and_no_overflow(dev):
