@@ -73,7 +73,13 @@ struct dyhip_device {
   uint64_t* rng_state;                 // device: {Philox key, next counter}; one per queue, see random.hip
   uint32_t rng_stream;                 // third counter word: 0 for the device, 1.. for its forked queues
   uint32_t forks_made;                 // forked queues created so far (numbers their random streams)
+  void* ln_scratch;                    // this GPU's copy of the static scratch array of dyhip_layer_norm_backward_static
 };
+
+namespace dyhip {
+// reduce.hip: looks up, on the current device, the address of the static scratch array (once per device handle)
+int ln_static_scratch_setup(dyhip_device* dev);
+}  // namespace dyhip
 
 struct dyhip_graph {
   hipGraph_t graph;

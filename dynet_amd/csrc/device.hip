@@ -262,6 +262,7 @@ int dyhip_device_create(int ordinal, const size_t pool_mb[4], dyhip_device** out
   dev->alloc = nullptr;
   dev->gemm_ws = nullptr;
   dev->gemm_ws_bytes = 0;
+  dev->ln_scratch = nullptr;
   dev->stream_threshold = size_t(8) << 20;
   hipError_t e = hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking);
   if (e != hipSuccess) {
@@ -290,6 +291,7 @@ int dyhip_device_create(int ordinal, const size_t pool_mb[4], dyhip_device** out
     if (dev->rng_state == nullptr) st = fail(DYHIP_ERR_OUT_OF_MEMORY, "failed to allocate the random generator state");
   }
   if (st == DYHIP_OK) st = dyhip_reset_rng(dev, 0);
+  if (st == DYHIP_OK) st = ln_static_scratch_setup(dev);  // this device is current (hipSetDevice above)
   if (st == DYHIP_OK) {
     dev->gemm_ws_bytes = size_t(128) << 20;
     dev->gemm_ws = dev->alloc->malloc(dev->gemm_ws_bytes);

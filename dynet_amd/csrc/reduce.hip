@@ -541,6 +541,21 @@ static unsigned ln_bwd_blocks(unsigned bd) {
   return blocks > kLnBwdMaxBlocks ? kLnBwdMaxBlocks : blocks;
 }
 
+// Scratch of dyhip_layer_norm_backward_static: the per-block dg / db partial rows (or the per-row
+// statistics of the generic path) live in this array instead of a caller-provided workspace, so that
+// entry point allocates nothing.  Every GPU the library runs on holds its own copy at its own address
+// until the process ends.  Host code never uses the array's name as an address (on the host it is only
+// a stand-in for the device symbol): ln_static_scratch_setup asks the runtime for the address on the
+// current device once, when the device handle is created, and every later use goes through that pointer.
+static __device__ __align__(256) unsigned char scratch[DYHIP_LN_STATIC_SCRATCH_BYTES];
+
+int ln_static_scratch_setup(dyhip_device* dev) {
+  void* ptr = nullptr;
+  DYHIP_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+  dev->ln_scratch = ptr;
+  return DYHIP_OK;
+}
+
 }  // namespace dyhip
 
 using namespace dyhip;
@@ -642,6 +657,19 @@ int dyhip_layer_norm_backward_workspace(size_t n, unsigned bd, size_t* ws_bytes)
   const size_t generic = size_t(bd) * sizeof(float2);
   *ws_bytes = fast > generic ? fast : generic;
   return DYHIP_OK;
+}
+
+int dyhip_layer_norm_backward_static(dyhip_device* dev, size_t n, unsigned bd, const float* x, const float* g,
+                                     const float* dEdf, float* dx, float* dg, float* db) {
+  DYHIP_CHECK_DEV(dev);
+  size_t need = 0;
+  DYHIP_CHECK_STATUS(dyhip_layer_norm_backward_workspace(n, bd, &need));
+  DYHIP_REQUIRE(need <= size_t(DYHIP_LN_STATIC_SCRATCH_BYTES),
+                "layer_norm backward without a workspace is limited to %zu scratch bytes; n = %zu, bd = %u needs %zu",
+                size_t(DYHIP_LN_STATIC_SCRATCH_BYTES), n, bd, need);
+  DYHIP_REQUIRE(dev->ln_scratch != nullptr, "the static scratch array of this device was not set up");
+  return dyhip_layer_norm_backward(dev, n, bd, x, g, dEdf, dx, dg, db, dev->ln_scratch,
+                                   size_t(DYHIP_LN_STATIC_SCRATCH_BYTES));
 }
 
 int dyhip_layer_norm_backward(dyhip_device* dev, size_t n, unsigned bd, const float* x, const float* g,

@@ -306,6 +306,11 @@ class Device:
         _check(cdll.dyhip_layer_norm_backward(self.handle, _sz(n), _u(bd), _p(x), _p(g), _p(dEdf), _p(dx), _p(dg),
                                               _p(db), _vp(ws), _sz(ws_bytes)))
 
+    def layer_norm_backward_static(self, n, bd, x, g, dEdf, dx=None, dg=None, db=None):
+        """No workspace argument and no allocation: the scratch is a static device array of the library."""
+        _check(cdll.dyhip_layer_norm_backward_static(self.handle, _sz(n), _u(bd), _p(x), _p(g), _p(dEdf), _p(dx),
+                                                     _p(dg), _p(db)))
+
     # ---- GEMM -------------------------------------------------------------
     def gemm_nn(self, M, N, K, l, r, beta, y):
         _check(cdll.dyhip_gemm_nn(self.handle, _sz(M), _sz(N), _sz(K), _p(l), _p(r), _f(beta), _p(y)))

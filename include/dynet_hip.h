@@ -188,6 +188,16 @@ int dyhip_layer_norm_forward(dyhip_device* dev, size_t n, unsigned bd, const flo
 int dyhip_layer_norm_backward_workspace(size_t n, unsigned bd, size_t* ws_bytes);
 int dyhip_layer_norm_backward(dyhip_device* dev, size_t n, unsigned bd, const float* x, const float* g,
                               const float* dEdf, float* dx, float* dg, float* db, void* ws, size_t ws_bytes);
+/* The same without a workspace argument, for callers that cannot allocate or carry one: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference (whose nodes take scratch from pools[SCS]).  The scratch is a static device array of
+ * DYHIP_LN_STATIC_SCRATCH_BYTES that each GPU holds until the process ends; the call allocates nothing and
+ * fails with DYHIP_ERR_INVALID_ARG when dyhip_layer_norm_backward_workspace(n, bd) exceeds that size
+ * (n <= 2048 on the fast path: any bd; otherwise bd <= 524288).  All calls on one GPU share the array:
+ * calls that overlap on one GPU (two queues, two threads) race; calls on one queue are ordered. */
+#define DYHIP_LN_STATIC_SCRATCH_BYTES (4u << 20)
+int dyhip_layer_norm_backward_static(dyhip_device* dev, size_t n, unsigned bd, const float* x, const float* g,
+                                     const float* dEdf, float* dx, float* dg, float* db);
 
 /* ---- GEMM shim: dynet/matrix-multiply.h, fp32 in / fp32 accumulate on MFMA.
  * The device-pointer acc_scalar of the reference (kSCALAR_ONE / kSCALAR_ZERO)
