@@ -9,15 +9,12 @@
 // Layout: the table is dim x vocab column-major, i.e. row r of the embedding is
 // the contiguous run table[r*dim, (r+1)*dim); fx and g are dim x n_ids.
 //
-// Scatter-add: (id, position) pairs are radix-sorted by id (stable, so equal
-// ids keep ascending position).  The sorted sequence is cut into chunks of
-// kChunk entries; one thread group per chunk walks its entries in order and
-// sums runs of equal ids in registers.  A run that lies inside one chunk is
-// added straight into its gradient row (the chunk is the only writer of that
-// row).  A run that crosses chunk boundaries leaves one partial row per chunk
-// in the workspace, and a second kernel adds the partials of each such run in
-// a fixed order.  No atomics anywhere: the result is deterministic and
-// each gradient row is read and written exactly once.
+// Scatter-add: the ids are grouped by value (a "plan": equal ids consecutive, ascending
+// position inside each run, see below) and one kernel sums each run: short runs by one
+// thread group in the CPU path's order, long runs split by columns over several thread
+// groups.  No atomics on floats and no partial rows: the result is deterministic, each
+// gradient row is read and written exactly once, and rows with short runs are bit-identical
+// to the sequential CPU sum.
 #include <cstring>
 
 #include <rocprim/rocprim.hpp>
@@ -27,7 +24,6 @@
 namespace dyhip {
 
 constexpr unsigned kNone = 0xFFFFFFFFu;
-constexpr int kChunk = 16;
 constexpr int kLkThreads = 256;
 constexpr int kGatherRowsUnroll = 4;
 
@@ -53,6 +49,32 @@ template <bool NT>
 __device__ __forceinline__ void vstore(float4* p, const float4 v) { stg4<NT>(p, v); }
 template <bool NT>
 __device__ __forceinline__ void vstore(float* p, const float v) { stg1<NT>(p, v); }
+// Stores and loads that bypass the caches that are private to a part of the chip (used for the few values that
+// thread groups on different L2s hand to each other inside one kernel).
+__device__ __forceinline__ void vstore_through(float* p, const float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+__device__ __forceinline__ void vstore_through(float4* p, const float4 v) {
+  unsigned long long* q = reinterpret_cast<unsigned long long*>(p);
+  const unsigned long long lo = (unsigned long long)__float_as_uint(v.x) | ((unsigned long long)__float_as_uint(v.y) << 32);
+  const unsigned long long hi = (unsigned long long)__float_as_uint(v.z) | ((unsigned long long)__float_as_uint(v.w) << 32);
+  __hip_atomic_store(q, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  __hip_atomic_store(q + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+__device__ __forceinline__ float vload_through(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+__device__ __forceinline__ float4 vload_through(const float4* p) {
+  const unsigned long long* q = reinterpret_cast<const unsigned long long*>(p);
+  const unsigned long long lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  const unsigned long long hi = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  return make_float4(__uint_as_float(unsigned(lo)), __uint_as_float(unsigned(lo >> 32)), __uint_as_float(unsigned(hi)),
+                     __uint_as_float(unsigned(hi >> 32)));
+}
+__device__ __forceinline__ float vshfl(const float v, int src) { return __shfl(v, src, kWave); }
+__device__ __forceinline__ float4 vshfl(const float4 v, int src) {
+  return make_float4(__shfl(v.x, src, kWave), __shfl(v.y, src, kWave), __shfl(v.z, src, kWave), __shfl(v.w, src, kWave));
+}
 
 // ---- gather ---------------------------------------------------------------------
 // A group of `tpr` threads owns one id at a time; a block holds 256/tpr groups and
@@ -79,128 +101,661 @@ __global__ __launch_bounds__(kLkThreads) void lookup_gather_kernel(unsigned n_id
   }
 }
 
-// ---- segmented scatter-add --------------------------------------------------------
-struct ScatterWs {
-  unsigned* sorted_ids;
-  unsigned* sorted_pos;
-  uint4* fix_list;       // part of the plan: {first chunk, last chunk, row, -} of every run that crosses a chunk
-                         // boundary, in no particular order
-  unsigned* fix_count;   // part of the plan: how many
-  float* part_first;     // [chunks][dim]
-  float* part_last;      // [chunks][dim]
-  unsigned chunks;
+// ---- the plan: ids grouped by value ------------------------------------------------
+// plan = [gid | gpos | roff | rrem | arrivals | status], each part padded to 256 bytes:
+//   gid[k]   id of the k-th entry in grouped order: entries of one id are consecutive (a "run"),
+//            ids >= vocab are replaced by vocab (one run that the reduction skips)
+//   gpos[k]  position of that entry in the caller's id vector; ascending inside a run
+//   roff[k]  entries of the run before k        (0 at the head of a run)
+//   rrem[k]  entries of the run from k onwards  (1 at its last entry)
+//   arrivals one counter per 8 entries, zero whenever no reduction is running: the groups that share one
+//            slice of a very long run count themselves here so that the last one adds their partial sums up
+//   status   [0] = number of ids >= vocab
+// The order of the runs does not matter to anything that consumes a plan (the segmented sum below and
+// the trainer's row kernels), so the ids are grouped, not fully sorted:
+// bucket = id mod 256, inside a bucket ascending id / 256, inside a run ascending position.
+struct Plan {
+  unsigned* gid;
+  unsigned* gpos;
+  unsigned* roff;
+  unsigned* rrem;
+  unsigned* arrivals;
+  unsigned* status;
 };
 
-template <class V, bool NT>
-__global__ __launch_bounds__(kLkThreads) void scatter_chunk_kernel(unsigned n, unsigned dimv, unsigned tpr,
-                                                                   unsigned vocab, ScatterWs w,
-                                                                   const V* __restrict__ g, V* __restrict__ grads) {
-  const unsigned groups = kLkThreads / tpr;
-  const unsigned grp = threadIdx.x / tpr, t = threadIdx.x - grp * tpr;
-  const unsigned ch = blockIdx.x * groups + grp;
-  if (ch >= w.chunks) return;
-  const unsigned k0 = ch * kChunk;
-  const unsigned cnt = min(n - k0, (unsigned)kChunk);
-  unsigned id[kChunk], pos[kChunk];
+constexpr int kChunk = 8;  // entries per thread group of the segmented sum (see there)
+
+static size_t align256(size_t n) { return (n + 255) / 256 * 256; }
+
+static size_t plan_bytes(unsigned n) {
+  return 4 * align256(sizeof(unsigned) * n) + align256(sizeof(unsigned) * cdiv<unsigned>(n, kChunk)) + 256;
+}
+
+static void plan_parts(const void* plan, unsigned n, Plan* w) {
+  char* p = const_cast<char*>(static_cast<const char*>(plan));
+  const size_t b = align256(sizeof(unsigned) * n);
+  w->gid = reinterpret_cast<unsigned*>(p);
+  w->gpos = reinterpret_cast<unsigned*>(p + b);
+  w->roff = reinterpret_cast<unsigned*>(p + 2 * b);
+  w->rrem = reinterpret_cast<unsigned*>(p + 3 * b);
+  w->arrivals = reinterpret_cast<unsigned*>(p + 4 * b);
+  w->status = reinterpret_cast<unsigned*>(p + 4 * b + align256(sizeof(unsigned) * cdiv<unsigned>(n, kChunk)));
+}
+
+static unsigned key_bits(unsigned max_key) {
+  unsigned bits = 1;
+  while (bits < 32 && (1ull << bits) <= (unsigned long long)max_key) ++bits;
+  return bits;
+}
+
+// ---- one-launch plan for up to 65535 ids ---------------------------------------------
+// 256 blocks, one per bucket (id mod 256).  Every block reads the whole id vector (64 KB at
+// 16384 ids, from L2 after the first block of an XCD), so no block waits for another:
+//   1. thread t owns a contiguous piece of the positions and counts, in registers, the ids of smaller
+//      buckets (their sum is where this bucket starts in the output) and of this bucket (their prefix
+//      over the threads is where the thread's matches go: the bucket is compacted in ascending position);
+//   2. stable counting sort of the bucket by the higher id bits, 8 bits per pass, in LDS: wave-private
+//      digit counters, ranks inside a 64-entry step from ballots, so no atomic decides an order;
+//   3. run offsets: head flags per 64-entry step, the last head before / first head after each step from
+//      a scan over the steps, written out together with ids and positions in coalesced order.
+// A bucket of more than kPlanCap entries (a heavily skewed id vector) takes the same steps in a
+// global-memory buffer instead of LDS.
+constexpr int kPlanThreads = 1024;
+constexpr int kPlanWaves = kPlanThreads / 64;
+constexpr unsigned kPlanSmallMax = 65535;
+constexpr int kPlanMaxQuads = (kPlanSmallMax + 4 * kPlanThreads - 1) / (4 * kPlanThreads);  // 128-bit loads per thread: 16
+constexpr unsigned kPlanCap = 8192;
+constexpr unsigned kPlanBuckets = 256;
+constexpr unsigned kPlanMaxSteps = (kPlanSmallMax + 63) / 64;  // 64-entry steps of the largest bucket: 1024
+// LDS words: digit counters [256][16] | scratch [128] | per-step last / first head [2][1024] | four buffers of kPlanCap
+constexpr unsigned kPlanLdsCnt = 0;
+constexpr unsigned kPlanLdsTmp = kPlanLdsCnt + 256 * kPlanWaves;
+constexpr unsigned kPlanLdsStep = kPlanLdsTmp + 128;
+constexpr unsigned kPlanLdsBuf = kPlanLdsStep + 2 * kPlanMaxSteps;
+constexpr unsigned kPlanLdsWords = kPlanLdsBuf + 4 * kPlanCap;
+
+__device__ __forceinline__ unsigned long long lanes_below(int lane) { return (1ull << lane) - 1ull; }
+
+// inclusive prefix sum over the lanes of a wavefront
+__device__ __forceinline__ unsigned wave_scan_add(unsigned v, int lane) {
 #pragma unroll
-  for (int k = 0; k < kChunk; ++k) {
-    id[k] = k < (int)cnt ? w.sorted_ids[k0 + k] : kNone;
-    pos[k] = k < (int)cnt ? w.sorted_pos[k0 + k] : 0u;
+  for (int off = 1; off < 64; off <<= 1) {
+    const unsigned u = __shfl_up(v, off, kWave);
+    if (lane >= off) v += u;
   }
-  const unsigned prev_id = k0 > 0 ? w.sorted_ids[k0 - 1] : kNone;
-  const unsigned next_id = k0 + cnt < n ? w.sorted_ids[k0 + cnt] : kNone;
-  const unsigned first = id[0], last = id[cnt - 1];
-  const bool open_left = prev_id == first;
-  const bool open_right = next_id == last;
-  V* part_first = reinterpret_cast<V*>(w.part_first) + size_t(ch) * dimv;
-  V* part_last = reinterpret_cast<V*>(w.part_last) + size_t(ch) * dimv;
-  // run_end[k]: entry k is the last of its run inside this chunk; direct[k]: that run
-  // lies wholly inside the chunk, so this thread group is the only writer of the row
-  bool run_end[kChunk], direct[kChunk];
+  return v;
+}
+
+// Exclusive prefix sum of one value per thread over the whole block (1024 threads), and the total.
+// tmp = kPlanWaves LDS words; a barrier separates the call from earlier uses of tmp.
+__device__ __forceinline__ unsigned block_scan_excl(unsigned v, unsigned* tmp, unsigned* total) {
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const unsigned inc = wave_scan_add(v, lane);
+  if (lane == 63) tmp[w] = inc;
+  __syncthreads();
+  unsigned before = 0, all = 0;
 #pragma unroll
-  for (int k = 0; k < kChunk; ++k) {
-    const bool last_k = k + 1 >= (int)cnt;
-    run_end[k] = k < (int)cnt && (last_k || id[k + 1 < kChunk ? k + 1 : k] != id[k]);
-    const bool ol = open_left && id[k] == first;
-    const bool orr = open_right && last_k;
-    direct[k] = run_end[k] && !ol && !orr && id[k] < vocab;
+  for (int k = 0; k < kPlanWaves; ++k) {
+    const unsigned x = tmp[k];
+    all += x;
+    if (k < w) before += x;
   }
-  for (unsigned c = t; c < dimv; c += tpr) {
-    V v[kChunk], old[kChunk];
-    // every load of the chunk is issued up front: the 16 gradient columns and the
-    // old value of each row that will be updated in place
+  *total = all;
+  return before + inc - v;
+}
+
+// lanes of the wavefront (among `valid` ones) that hold the same 8-bit digit as this lane
+__device__ __forceinline__ unsigned long long same_digit_lanes(unsigned dig, bool valid) {
+  unsigned long long same = __ballot(valid);
 #pragma unroll
-    for (int k = 0; k < kChunk; ++k) {
-      v[k] = k < (int)cnt ? vload<NT>(g + size_t(pos[k]) * dimv + c) : vzero<V>();
-      if (direct[k]) old[k] = grads[size_t(id[k]) * dimv + c];
+  for (int b = 0; b < 8; ++b) {
+    const bool bit = (dig >> b) & 1u;
+    const unsigned long long bal = __ballot(valid && bit);
+    same &= bit ? bal : ~bal;
+  }
+  return same;
+}
+
+// One stable counting-sort pass over the m entries (key, pos) of a bucket on digit (key >> shift) & 255.
+// cnt[digit * 16 + wave] must be zero on entry and is zero again on return.  Wavefront w owns a contiguous
+// piece of the input.  A: it counts its digits; B: exclusive prefix over (digit, wavefront) in that
+// order; C: it walks its piece 64 entries at a time, ranks equal digits inside the step with ballots and
+// advances its own counters, so entries with equal digits keep their input order.
+__device__ __forceinline__ void plan_sort_pass(unsigned m, unsigned shift, const unsigned* kin, const unsigned* pin,
+                                               unsigned* kout, unsigned* pout, unsigned* cnt, unsigned* tmp) {
+  const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+  const unsigned per_wave = cdiv<unsigned>(cdiv<unsigned>(m, kPlanWaves), 64u) * 64u;
+  const unsigned wb = min(m, w * per_wave), we = min(m, wb + per_wave);
+  for (unsigned j0 = wb; j0 < we; j0 += 64) {  // uniform over the wavefront
+    const unsigned j = j0 + lane;
+    const bool valid = j < we;
+    const unsigned dig = valid ? (kin[j] >> shift) & 255u : 0u;
+    const unsigned long long same = same_digit_lanes(dig, valid);
+    if (valid && (same & lanes_below(lane)) == 0) cnt[dig * kPlanWaves + w] += __popcll(same);
+  }
+  __syncthreads();
+  // B: thread t scans counters [4t, 4t + 4)
+  uint4 c4 = reinterpret_cast<uint4*>(cnt)[t];
+  unsigned tot_unused;
+  const unsigned sum4 = c4.x + c4.y + c4.z + c4.w;
+  const unsigned base = block_scan_excl(sum4, tmp, &tot_unused);
+  uint4 e4;
+  e4.x = base;
+  e4.y = e4.x + c4.x;
+  e4.z = e4.y + c4.y;
+  e4.w = e4.z + c4.z;
+  reinterpret_cast<uint4*>(cnt)[t] = e4;
+  __syncthreads();
+  for (unsigned j0 = wb; j0 < we; j0 += 64) {
+    const unsigned j = j0 + lane;
+    const bool valid = j < we;
+    const unsigned key = valid ? kin[j] : 0u;
+    const unsigned pos = valid ? pin[j] : 0u;
+    const unsigned dig = (key >> shift) & 255u;
+    const unsigned long long same = same_digit_lanes(dig, valid);
+    const unsigned rank = __popcll(same & lanes_below(lane));
+    // every lane reads its digit's counter before the first lane of each digit advances it: the
+    // wavefront issues the load for all its lanes, then the store, and LDS keeps that order
+    unsigned at = 0;
+    if (valid) at = cnt[dig * kPlanWaves + w];
+    __builtin_amdgcn_wave_barrier();
+    if (valid && rank == 0) cnt[dig * kPlanWaves + w] = at + __popcll(same);
+    __builtin_amdgcn_wave_barrier();
+    if (valid) {
+      kout[at + rank] = key;
+      pout[at + rank] = pos;
     }
-    V acc = vzero<V>();
+  }
+  __syncthreads();
+  reinterpret_cast<uint4*>(cnt)[t] = make_uint4(0u, 0u, 0u, 0u);
+  __syncthreads();
+}
+
+// Steps 2 and 3 on buffers in LDS or in global memory (same code, two address spaces).
+__device__ __forceinline__ void plan_finish_bucket(unsigned m, unsigned passes, unsigned bstart, unsigned* kA,
+                                                   unsigned* pA, unsigned* kB, unsigned* pB, unsigned* cnt,
+                                                   unsigned* tmp, int* step_last, int* step_first, const Plan out) {
+  const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+  for (unsigned p = 0; p < passes; ++p) {
+    plan_sort_pass(m, 8u + 8u * p, kA, pA, kB, pB, cnt, tmp);
+    unsigned* s;
+    s = kA; kA = kB; kB = s;
+    s = pA; pA = pB; pB = s;
+  }
+  // grouped entries are in (kA, pA).  Step q = entries [64q, 64q + 64), taken by wavefront q mod 16.
+  const unsigned steps = cdiv<unsigned>(m, 64u);
+  for (unsigned q = w; q < steps; q += kPlanWaves) {
+    const unsigned j = q * 64 + lane;
+    const bool head = j < m && (j == 0 || kA[j - 1] != kA[j]);
+    const unsigned long long hm = __ballot(head);
+    if (lane == 0) {
+      step_last[q] = hm ? int(q * 64) + 63 - __clzll(hm) : -1;
+      step_first[q] = hm ? int(q * 64) + __ffsll((long long)hm) - 1 : int(m);
+    }
+  }
+  __syncthreads();
+  // running maximum of step_last (ascending) and running minimum of step_first (descending), by wavefront 0:
+  // afterwards step_last[q] = last head in steps <= q, step_first[q] = first head in steps >= q (m if none)
+  if (w == 0) {
+    int carry_l = -1, carry_f = int(m);
+    for (unsigned q0 = 0; q0 < steps; q0 += 64) {
+      const unsigned q = q0 + lane;
+      int l = q < steps ? step_last[q] : -1;
 #pragma unroll
-    for (int k = 0; k < kChunk; ++k) {
-      if (k < (int)cnt) {
-        acc = vadd(acc, v[k]);
-        if (run_end[k]) {
-          if (direct[k])
-            grads[size_t(id[k]) * dimv + c] = vadd(old[k], acc);
-          else if (open_left && id[k] == first)
-            part_first[c] = acc;
-          else if (id[k] < vocab)
-            part_last[c] = acc;
-          acc = vzero<V>();
-        }
+      for (int off = 1; off < 64; off <<= 1) {
+        const int u = __shfl_up(l, off, kWave);
+        if (lane >= off) l = max(l, u);
       }
+      l = max(l, carry_l);
+      if (q < steps) step_last[q] = l;
+      carry_l = __shfl(l, 63, kWave);
+    }
+    for (unsigned r0 = 0; r0 < steps; r0 += 64) {  // from the top step down
+      const unsigned r = r0 + lane;                // reversed index
+      const bool in = r < steps;
+      const unsigned q = in ? steps - 1 - r : 0;
+      int f = in ? step_first[q] : int(m);
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int u = __shfl_up(f, off, kWave);
+        if (lane >= off) f = min(f, u);
+      }
+      f = min(f, carry_f);
+      if (in) step_first[q] = f;
+      carry_f = __shfl(f, 63, kWave);
+    }
+  }
+  __syncthreads();
+  for (unsigned q = w; q < steps; q += kPlanWaves) {
+    const unsigned j = q * 64 + lane;
+    const bool in = j < m;
+    const unsigned key = in ? kA[j] : 0u;
+    const bool head = in && (j == 0 || kA[j - 1] != key);
+    const unsigned long long hm = __ballot(head);
+    // last head at or before j: inside this step, else carried from the steps before
+    const unsigned long long le = hm & (lanes_below(lane) | (1ull << lane));
+    const int lh = le ? int(q * 64) + 63 - __clzll(le) : (q > 0 ? step_last[q - 1] : 0);
+    // first head after j: inside this step, else carried from the steps after
+    const unsigned long long gt = lane == 63 ? 0ull : hm & ~(lanes_below(lane + 1));
+    const int nh = gt ? int(q * 64) + __ffsll((long long)gt) - 1 : (q + 1 < steps ? step_first[q + 1] : int(m));
+    if (in) {
+      out.gid[bstart + j] = key;
+      out.gpos[bstart + j] = pA[j];
+      out.roff[bstart + j] = j - unsigned(lh);
+      out.rrem[bstart + j] = unsigned(nh) - j;
+      if ((bstart + j) % kChunk == 0) out.arrivals[(bstart + j) / kChunk] = 0;
     }
   }
 }
 
-// One block per boundary-crossing run (the plan lists the chunks in which such runs start and
-// where each ends).  The run's partial rows (one per chunk it touches) are split over
-// kFixThreads / tpr thread slices that each add every slices-th partial in ascending order with
-// four loads in flight, and the slices are then added in ascending order: deterministic, and a
-// run of thousands of entries costs a handful of memory round trips instead of one per partial.
-constexpr int kFixThreads = 1024;
-
-template <class V>
-__global__ __launch_bounds__(kFixThreads) void scatter_fixup_kernel(unsigned n, unsigned dimv, unsigned tpr,
-                                                                    unsigned vocab, ScatterWs w,
-                                                                    V* __restrict__ grads) {
-  extern __shared__ __attribute__((aligned(16))) char fix_lds_raw[];
-  V* lds = reinterpret_cast<V*>(fix_lds_raw);
-  const unsigned slices = kFixThreads / tpr;
-  const unsigned q = threadIdx.x / tpr, t = threadIdx.x - q * tpr;
-  const V* pf = reinterpret_cast<const V*>(w.part_first);
-  // count and the block's first entry are fetched together (entries past count are never used)
-  uint4 e = w.fix_list[blockIdx.x];
-  const unsigned count = *w.fix_count;
-  for (unsigned i = blockIdx.x; i < count; i += gridDim.x) {  // uniform over the block
-    if (i != blockIdx.x) e = w.fix_list[i];
-    const unsigned c0 = e.x, c_last = e.y, row = e.z;
-    if (row >= vocab) continue;
-    const V* pl = reinterpret_cast<const V*>(w.part_last) + size_t(c0) * dimv;
-    for (unsigned cb = 0; cb < dimv; cb += tpr) {
-      const unsigned c = cb + t;
-      V acc = vzero<V>(), old = vzero<V>();
-      if (q == 0 && c < dimv) old = grads[size_t(row) * dimv + c];  // in flight beside the partials
-      if (c < dimv) {
-        // partial index p = 0 is part_last[c0]; p >= 1 is part_first[c0 + p]
-        const unsigned np = c_last - c0 + 1;
-        unsigned p = q;
-        for (; p + 3 * slices < np; p += 4 * slices) {
-          const V a0 = p == 0 ? pl[c] : pf[size_t(c0 + p) * dimv + c];
-          const V a1 = pf[size_t(c0 + p + slices) * dimv + c];
-          const V a2 = pf[size_t(c0 + p + 2 * slices) * dimv + c];
-          const V a3 = pf[size_t(c0 + p + 3 * slices) * dimv + c];
-          acc = vadd(vadd(vadd(vadd(acc, a0), a1), a2), a3);
-        }
-        for (; p < np; p += slices) acc = vadd(acc, p == 0 ? pl[c] : pf[size_t(c0 + p) * dimv + c]);
+template <bool VEC>
+__global__ __launch_bounds__(kPlanThreads) void plan_group_kernel(unsigned n, unsigned vocab, unsigned passes,
+                                                                  const unsigned* __restrict__ ids, const Plan out,
+                                                                  unsigned* __restrict__ gbuf) {
+  extern __shared__ __attribute__((aligned(16))) unsigned plan_lds[];
+  unsigned* cnt = plan_lds + kPlanLdsCnt;
+  unsigned* tmp = plan_lds + kPlanLdsTmp;
+  int* step_last = reinterpret_cast<int*>(plan_lds + kPlanLdsStep);
+  int* step_first = step_last + kPlanMaxSteps;
+  const unsigned d = blockIdx.x;
+  const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+  reinterpret_cast<uint4*>(cnt)[t] = make_uint4(0u, 0u, 0u, 0u);  // 4096 counters, 4 per thread
+  // ---- 1. thread t reads positions [t * 4 * quads, (t + 1) * 4 * quads); keys stay in registers ------
+  const unsigned quads = cdiv<unsigned>(n, 4u * kPlanThreads);  // 128-bit loads per thread (uniform)
+  const unsigned p_first = unsigned(t) * 4u * quads;
+  unsigned key[kPlanMaxQuads][4];
+  unsigned lt = 0, eq = 0, bad = 0;
+#pragma unroll
+  for (int i = 0; i < kPlanMaxQuads; ++i) {
+    if (unsigned(i) < quads) {  // uniform
+      const unsigned p0 = p_first + 4u * i;
+      unsigned raw[4] = {kNone, kNone, kNone, kNone};
+      if (VEC && p0 + 3 < n) {
+        const uint4 v = *reinterpret_cast<const uint4*>(ids + p0);
+        raw[0] = v.x; raw[1] = v.y; raw[2] = v.z; raw[3] = v.w;
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          if (p0 + c < n) raw[c] = ids[p0 + c];
       }
-      __syncthreads();
-      lds[q * tpr + t] = acc;
-      __syncthreads();
-      if (q == 0 && c < dimv) {
-        V tot = lds[t];
-        for (unsigned k = 1; k < slices; ++k) tot = vadd(tot, lds[k * tpr + t]);
-        grads[size_t(row) * dimv + c] = vadd(old, tot);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const bool in = p0 + c < n;
+        const unsigned k = in ? min(raw[c], vocab) : kNone;
+        key[i][c] = k;
+        const unsigned dg = k & 255u;
+        lt += in && dg < d ? 1u : 0u;
+        eq += in && dg == d ? 1u : 0u;
+        bad += in && raw[c] >= vocab ? 1u : 0u;
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) key[i][c] = kNone;
+    }
+  }
+  // one scan for both counts: eq in the low half (its total is at most 65535), lt in the high half
+  unsigned both = 0, nbad = 0;
+  const unsigned my_at = block_scan_excl(eq | (lt << 16), tmp, &both) & 0xFFFFu;
+  const unsigned m = both & 0xFFFFu, bstart = both >> 16;
+  if (d == kPlanBuckets - 1) {  // the ids >= vocab are counted by one block, not the one of the (often hottest) bucket 0
+    (void)block_scan_excl(bad, tmp + 32, &nbad);
+    if (t == 0) out.status[0] = nbad;
+  }
+  if (m == 0) return;  // uniform over the block
+  const bool in_lds = m <= kPlanCap;
+  unsigned* kA = in_lds ? plan_lds + kPlanLdsBuf : gbuf + bstart;
+  unsigned* pA = in_lds ? plan_lds + kPlanLdsBuf + kPlanCap : gbuf + size_t(n) + bstart;
+  // ---- compaction of this bucket's entries, ascending position ------------------------------
+  if (eq) {
+    unsigned at = my_at;
+#pragma unroll
+    for (int i = 0; i < kPlanMaxQuads; ++i) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        if (unsigned(i) < quads && key[i][c] != kNone && (key[i][c] & 255u) == d) {
+          if (in_lds) {
+            plan_lds[kPlanLdsBuf + at] = key[i][c];
+            plan_lds[kPlanLdsBuf + kPlanCap + at] = p_first + 4u * i + c;
+          } else {
+            kA[at] = key[i][c];
+            pA[at] = p_first + 4u * i + c;
+          }
+          ++at;
+        }
+      }
+    }
+  }
+  __syncthreads();
+  if (in_lds)
+    plan_finish_bucket(m, passes, bstart, plan_lds + kPlanLdsBuf, plan_lds + kPlanLdsBuf + kPlanCap,
+                       plan_lds + kPlanLdsBuf + 2 * kPlanCap, plan_lds + kPlanLdsBuf + 3 * kPlanCap, cnt, tmp,
+                       step_last, step_first, out);
+  else
+    plan_finish_bucket(m, passes, bstart, kA, pA, gbuf + 2 * size_t(n) + bstart, gbuf + 3 * size_t(n) + bstart, cnt,
+                       tmp, step_last, step_first, out);
+}
+
+// ---- plan for more ids than that: device-wide radix sort, then the run offsets by binary search -----
+__global__ __launch_bounds__(256) void plan_clamp_kernel(unsigned n, unsigned vocab, const unsigned* __restrict__ ids,
+                                                         unsigned* __restrict__ keys, unsigned* status) {
+  const unsigned k = blockIdx.x * 256 + threadIdx.x;
+  if (k == 0) *status = 0;  // the count itself is taken by plan_runs_sorted_kernel
+  if (k < n) keys[k] = min(ids[k], vocab);
+}
+
+__global__ __launch_bounds__(256) void plan_runs_sorted_kernel(unsigned n, unsigned vocab, const Plan out) {
+  const unsigned k = blockIdx.x * 256 + threadIdx.x;
+  if (k >= n) return;
+  const unsigned id = out.gid[k];
+  unsigned lo = 0, hi = k;  // first index holding id
+  while (lo < hi) {
+    const unsigned mid = lo + (hi - lo) / 2;
+    if (out.gid[mid] < id) lo = mid + 1;
+    else hi = mid;
+  }
+  const unsigned first = lo;
+  lo = k + 1, hi = n;  // first index holding a larger id
+  while (lo < hi) {
+    const unsigned mid = lo + (hi - lo) / 2;
+    if (out.gid[mid] <= id) lo = mid + 1;
+    else hi = mid;
+  }
+  out.roff[k] = k - first;
+  out.rrem[k] = lo - k;
+  if (k % kChunk == 0) out.arrivals[k / kChunk] = 0;
+  if (id >= vocab && k == first) out.status[0] = lo - first;  // one writer: the head of the run of clamped ids
+}
+
+static int sort_tmp_bytes(unsigned n, unsigned bits, size_t* bytes) {
+  size_t tmp = 0;
+  unsigned* k = nullptr;
+  hipError_t e = rocprim::radix_sort_pairs(nullptr, tmp, static_cast<const unsigned*>(k), k,
+                                           rocprim::counting_iterator<unsigned>(0), k, n, 0, bits);
+  if (e != hipSuccess) return fail(DYHIP_ERR_RUNTIME, "radix sort size query failed: %s", hipGetErrorString(e));
+  *bytes = tmp;
+  return DYHIP_OK;
+}
+
+static int plan_ws_bytes(unsigned n, unsigned vocab, size_t* bytes) {
+  if (n <= kPlanSmallMax) {
+    *bytes = align256(4 * sizeof(unsigned) * size_t(n));
+    return DYHIP_OK;
+  }
+  size_t sort_b = 0;
+  DYHIP_CHECK_STATUS(sort_tmp_bytes(n, key_bits(vocab), &sort_b));
+  *bytes = align256(sizeof(unsigned) * size_t(n)) + align256(sort_b);
+  return DYHIP_OK;
+}
+
+static int build_plan(dyhip_device* dev, unsigned n, const unsigned* ids_dev, unsigned vocab, void* plan,
+                      size_t plan_size, void* ws, size_t ws_bytes) {
+  DYHIP_REQUIRE(vocab >= 1 && vocab < 0x7FFFFFFFu, "lookup vocabulary size %u out of range", vocab);
+  size_t need = 0;
+  DYHIP_CHECK_STATUS(plan_ws_bytes(n, vocab, &need));
+  DYHIP_REQUIRE(plan != nullptr && plan_size >= plan_bytes(n) && aligned16(plan),
+                "lookup plan needs %zu bytes (16-byte aligned), got %zu", plan_bytes(n), plan_size);
+  DYHIP_REQUIRE(ws != nullptr && ws_bytes >= need && aligned16(ws), "lookup plan needs %zu workspace bytes, got %zu", need,
+                ws_bytes);
+  Plan out;
+  plan_parts(plan, n, &out);
+  const unsigned bits = key_bits(vocab);  // keys are min(id, vocab) <= vocab
+  if (n <= kPlanSmallMax) {
+    const unsigned passes = bits <= 8 ? 0u : (bits - 8 + 7) / 8;
+    const size_t lds = sizeof(unsigned) * kPlanLdsWords;
+    static bool attr_set[2] = {false, false};
+    const bool vec = aligned16(ids_dev);
+    if (!attr_set[vec]) {
+      if (vec)
+        DYHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&plan_group_kernel<true>),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)));
+      else
+        DYHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&plan_group_kernel<false>),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)));
+      attr_set[vec] = true;
+    }
+    if (vec)
+      hipLaunchKernelGGL(plan_group_kernel<true>, dim3(kPlanBuckets), dim3(kPlanThreads), lds, dev->stream, n, vocab,
+                         passes, ids_dev, out, static_cast<unsigned*>(ws));
+    else
+      hipLaunchKernelGGL(plan_group_kernel<false>, dim3(kPlanBuckets), dim3(kPlanThreads), lds, dev->stream, n, vocab,
+                         passes, ids_dev, out, static_cast<unsigned*>(ws));
+    DYHIP_CHECK_LAUNCH();
+    return DYHIP_OK;
+  }
+  unsigned* keys = static_cast<unsigned*>(ws);
+  const size_t keys_b = align256(sizeof(unsigned) * size_t(n));
+  size_t sort_b = 0;
+  DYHIP_CHECK_STATUS(sort_tmp_bytes(n, bits, &sort_b));
+  const dim3 grid(cdiv<unsigned>(n, 256)), block(256);
+  hipLaunchKernelGGL(plan_clamp_kernel, grid, block, 0, dev->stream, n, vocab, ids_dev, keys, out.status);
+  DYHIP_CHECK_LAUNCH();
+  DYHIP_CHECK_HIP(rocprim::radix_sort_pairs(static_cast<char*>(ws) + keys_b, sort_b, static_cast<const unsigned*>(keys),
+                                            out.gid, rocprim::counting_iterator<unsigned>(0), out.gpos, n, 0, bits,
+                                            dev->stream));
+  hipLaunchKernelGGL(plan_runs_sorted_kernel, grid, block, 0, dev->stream, n, vocab, out);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+// ---- segmented sum over the runs of a plan -----------------------------------------
+// One thread group per chunk of kChunk consecutive grouped entries; a group is `tpr` threads that
+// cover the row width (one block = one group when tpr >= 64, else 64 / tpr groups inside one wavefront).
+//   * A run of fewer than kHeavyMin entries is summed by the group whose chunk holds its head, to its
+//     end (into the following chunks if need be): acc = old row, += each gradient row in ascending
+//     position, store.  That is the CPU path's order, so such rows come out bit-identical to it.
+//     A group's runs hold at most kItemMax entries together.
+//   * A run of kHeavyMin or more entries covers at least one whole chunk; the groups of the chunks
+//     it covers entirely have no run of their own and share the run by COLUMNS: each sums every entry
+//     of the run for a slice of the row, entry slots in parallel across the group's threads, slots
+//     added in ascending order.  A slice is at least one 128-byte line wide; a run long enough to give
+//     every slice several groups is also cut into parts of consecutive entries, whose sums the last
+//     group to finish adds up in ascending order (arrival counters in the plan, partial sums in the
+//     workspace).  Either way a thread's share of a run of any length is a few batches.
+// Loads go out in batches of kBatch rows per thread (nearly every group needs one batch); the kernel keeps
+// few enough registers for every block of the grid to be resident at once.  Updated rows are written with
+// streaming stores, so they drain while the kernel runs instead of when it ends.
+// No second launch, no float atomics, and no group ever waits for another: the result does not depend on timing.
+constexpr int kBatch = 11;
+constexpr unsigned kHeavyMin = 2 * kChunk - 1;         // shortest run that must contain a whole chunk
+constexpr int kItemMax = 3 * kChunk - 2;               // own chunk after its first entry (7) + the longest short run (14) <= 22
+constexpr int kItemBatches = (kItemMax + kBatch - 1) / kBatch;
+static_assert(kChunk - 1 + int(kHeavyMin) - 1 <= kItemMax, "a group's short runs fit kItemBatches batches");
+static_assert(3 * kChunk <= 64 && kItemMax <= 32 && kBatch >= kChunk, "plan entries of an item sit in the lanes of one "
+              "wavefront / two 16-lane rounds; every head of an item is in its first batch");
+
+template <class V, bool WIDE>
+__global__ __launch_bounds__(256) void scatter_runs_kernel(unsigned n, unsigned dimv, unsigned tpr, unsigned vocab,
+                                                           const Plan p, const V* __restrict__ g,
+                                                           V* __restrict__ grads, V* partials) {
+  extern __shared__ __attribute__((aligned(16))) char scatter_lds_raw[];
+  V* lds = reinterpret_cast<V*>(scatter_lds_raw);
+  const unsigned groups = blockDim.x / tpr;
+  const unsigned grp = threadIdx.x / tpr, t = threadIdx.x - grp * tpr;
+  const unsigned ch = blockIdx.x * groups + grp;
+  const unsigned k0 = ch * kChunk;
+  if (k0 >= n) return;  // whole groups leave; with tpr >= 64 the group is the block
+  const int lane = threadIdx.x & 63;
+  // Plan entries k0 + l, one per lane.  WIDE: lanes 0..23 of every wavefront of the group hold the chunk and
+  // the two after it (as far as a short run that starts here can reach).  Narrow groups (16 or 32
+  // threads) hold entries k0 .. k0+15 in each 16-lane cluster and fetch an item's entries afterwards.
+  const unsigned l = WIDE ? unsigned(lane) : (threadIdx.x & 15u);
+  const bool l_in = (WIDE ? l < 3u * kChunk : true) && k0 + l < n;
+  const unsigned e_off = l_in ? p.roff[k0 + l] : 1u;
+  const unsigned e_rem = l_in ? p.rrem[k0 + l] : 0u;
+  const unsigned e_id = l_in ? p.gid[k0 + l] : kNone;
+  const unsigned e_pos = l_in ? p.gpos[k0 + l] : kNone;
+  const unsigned o0 = WIDE ? __builtin_amdgcn_readfirstlane(e_off) : __shfl(e_off, 0, 16);
+  const unsigned r0 = WIDE ? __builtin_amdgcn_readfirstlane(e_rem) : __shfl(e_rem, 0, 16);
+  if (o0 + r0 >= kHeavyMin && r0 >= unsigned(kChunk)) {
+    // ---- this chunk lies inside a long run: take a slice of its columns --------------------
+    const unsigned start = k0 - o0, R = o0 + r0;
+    const unsigned cf = (start + kChunk - 1) / kChunk;       // first chunk the run covers entirely
+    const unsigned W = (start + R) / kChunk - cf;            // how many it covers entirely (>= 1)
+    const unsigned idx = ch - cf;
+    const unsigned row = WIDE ? __builtin_amdgcn_readfirstlane(e_id) : __shfl(e_id, 0, 16);
+    if (row >= vocab) return;
+    // Slice width w in vector elements: whole 128-byte lines (narrower slices make several L2s fetch
+    // the same line), wider if the run covers too few chunks to give every line-wide slice a group.
+    const unsigned line = min(128u / unsigned(sizeof(V)), dimv);
+    const unsigned w = min(tpr, max(cdiv<unsigned>(dimv, W), line));
+    const unsigned S = cdiv<unsigned>(dimv, w), E = tpr / w;  // slices; entry slots per slice (threads >= E * w idle)
+    const unsigned slot = t / w, cin = t - slot * w;
+    const bool busy = slot < E;
+    // A run that covers at least two groups per slice is also cut into P parts of consecutive entries: group
+    // idx takes slice idx mod S of part idx / S.  The parts of a slice meet through `partials` (one 128-byte
+    // line per chunk): each writes its sum there, counts itself in the slice's arrival counter, and the one
+    // that arrives last adds all P up in ascending part order: the same sum whoever is last.
+    const unsigned P = (WIDE && w * unsigned(sizeof(V)) <= 128u && W >= 2 * S) ? W / S : 1u;
+    const unsigned per_part = cdiv<unsigned>(R, P);
+    for (unsigned s0 = idx; s0 < S * P; s0 += W) {            // uniform over the group; one trip unless dimv > tpr * W
+      const unsigned s = s0 % S, q = s0 / S;
+      const unsigned eb = q * per_part, ee = min(R, eb + per_part);  // this part's entries of the run
+      const unsigned c = s * w + cin;
+      const bool cok = busy && c < dimv;
+      V old = vzero<V>();
+      if (cok && slot == 0) old = grads[size_t(row) * dimv + c];
+      V acc = vzero<V>();
+      for (unsigned e0 = eb + slot; e0 < ee; e0 += E * kBatch) {
+        unsigned pos[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+          const unsigned e = e0 + u * E;
+          pos[u] = (cok && e < ee) ? p.gpos[start + e] : kNone;
+        }
+        V v[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u)
+          v[u] = pos[u] != kNone ? g[size_t(pos[u]) * dimv + c] : vzero<V>();
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) acc = vadd(acc, v[u]);
+      }
+      if (WIDE) {
+        // slots are added in ascending order: first every eighth slot by eight threads per column, then those
+        __syncthreads();
+        lds[t] = acc;
+        __syncthreads();
+        const unsigned fan = E >= 16 ? 8u : 1u;
+        V part = vzero<V>();
+        if (slot < fan && cok) {
+          part = acc;
+          for (unsigned qq = slot + fan; qq < E; qq += fan) part = vadd(part, lds[qq * w + cin]);
+        }
+        if (fan > 1) {
+          __syncthreads();
+          if (slot < fan) lds[slot * w + cin] = part;
+          __syncthreads();
+          if (slot == 0)
+            for (unsigned qq = 1; qq < fan; ++qq) part = vadd(part, lds[qq * w + cin]);
+        }
+        if (P == 1) {
+          if (slot == 0 && cok) vstore<true>(grads + size_t(row) * dimv + c, vadd(old, part));
+        } else {
+          // The partial sum goes to memory past the L2 of this block (each L2 serves one eighth of the chip
+          // and does not see the others' lines); when the stores have been acknowledged the group counts
+          // itself.  Nobody waits for anybody: whichever group finds P - 1 arrivals before it does the rest.
+          const unsigned line_v = 128u / unsigned(sizeof(V));
+          if (slot == 0 && cok) vstore_through(partials + size_t(ch) * line_v + cin, part);
+          // every store of this wavefront has been acknowledged by memory before the barrier lets thread 0 count
+          // (a workgroup-scope fence does not wait for global stores, an agent-scope one would also write the L2 back)
+          __builtin_amdgcn_s_waitcnt(0);
+          __syncthreads();
+          unsigned* flag = reinterpret_cast<unsigned*>(lds);
+          if (t == 0)
+            *flag = __hip_atomic_fetch_add(p.arrivals + cf + s, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == P - 1;
+          __syncthreads();
+          const bool last = *flag != 0;
+          __syncthreads();
+          if (last) {
+            if (slot == 0 && cok) {
+              V tot = vload_through(partials + size_t(cf + s) * line_v + cin);
+              for (unsigned qq = 1; qq < P; ++qq)
+                tot = vadd(tot, vload_through(partials + size_t(cf + qq * S + s) * line_v + cin));
+              vstore<true>(grads + size_t(row) * dimv + c, vadd(old, tot));
+            }
+            if (t == 0) __hip_atomic_store(p.arrivals + cf + s, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+        }
+      } else {
+        // the group sits inside one wavefront: slots are fetched from their lanes in ascending order
+        const int lane0 = lane - int(t);
+        V tot = acc;
+        for (unsigned qq = 1; qq < E; ++qq) {
+          const V o = vshfl(acc, lane0 + int(qq * w + cin));
+          tot = vadd(tot, o);
+        }
+        if (slot == 0 && cok) vstore<true>(grads + size_t(row) * dimv + c, vadd(old, tot));
+      }
+    }
+    return;
+  }
+  // ---- short runs whose head lies in this chunk ------------------------------------------------
+  // first such head and the end of the last such run (a long run that starts here takes the rest of the chunk)
+  const bool own = l < unsigned(kChunk) && l_in && e_off == 0 && e_rem < kHeavyMin;
+  unsigned long long own_mask = __ballot(own);
+  if (!WIDE) own_mask = (own_mask >> (lane & 48)) & 0xFFFFull;  // this group's 16-lane cluster
+  if (own_mask == 0) return;
+  const unsigned first_l = __ffsll((long long)own_mask) - 1, last_l = 63 - __clzll(own_mask);
+  const unsigned ks = k0 + first_l;
+  const unsigned ke = k0 + last_l + (WIDE ? __builtin_amdgcn_readlane(e_rem, last_l) : __shfl(e_rem, last_l, 16));
+  // WIDE: entry ks + j sits in lane first_l + j (< 24) of every wavefront.  Narrow groups fetch entry ks + j
+  // with lane j mod 16 of their 16-lane cluster (two rounds) and hand it around.
+  const unsigned my_flags = (e_off == 0 ? 1u : 0u) | (e_rem == 1 ? 2u : 0u);
+  unsigned b_pos[2] = {kNone, kNone}, b_id[2] = {kNone, kNone}, b_fl[2] = {0u, 0u};
+  if (!WIDE) {
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      const unsigned k = ks + 16u * r + (threadIdx.x & 15u);
+      const bool in = k < ke;
+      b_pos[r] = in ? p.gpos[k] : kNone;
+      b_id[r] = in ? p.gid[k] : kNone;
+      b_fl[r] = in ? (p.roff[k] == 0 ? 1u : 0u) | (p.rrem[k] == 1 ? 2u : 0u) : 0u;
+    }
+  }
+  for (unsigned c0 = 0; c0 < dimv; c0 += tpr) {
+    const unsigned c = c0 + t;
+    const bool cok = c < dimv;
+    V acc = vzero<V>();
+#pragma unroll
+    for (int r = 0; r < kItemBatches; ++r) {
+      if (ks + unsigned(r * kBatch) >= ke) break;  // uniform over the group
+      unsigned id[kBatch], pos[kBatch];
+      bool head[kBatch], tail[kBatch];
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        const int j = r * kBatch + u;
+        if (j >= kItemMax) {
+          pos[u] = kNone; id[u] = kNone; head[u] = false; tail[u] = false;
+        } else if (WIDE) {
+          const bool in = ks + j < ke;
+          const unsigned src = in ? first_l + j : 0u;
+          pos[u] = in ? __builtin_amdgcn_readlane(e_pos, src) : kNone;
+          id[u] = __builtin_amdgcn_readlane(e_id, src);
+          const unsigned fl = __builtin_amdgcn_readlane(my_flags, src);
+          head[u] = in && (fl & 1u);
+          tail[u] = in && (fl & 2u);
+        } else {
+          pos[u] = __shfl(b_pos[j / 16], j % 16, 16);
+          id[u] = __shfl(b_id[j / 16], j % 16, 16);
+          const unsigned fl = __shfl(b_fl[j / 16], j % 16, 16);
+          head[u] = fl & 1u;
+          tail[u] = fl & 2u;
+        }
+      }
+      // every load of the batch is issued before the first add; heads lie in the own chunk, i.e. in batch 0
+      V v[kBatch], old[kChunk];
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        v[u] = (cok && pos[u] != kNone) ? g[size_t(pos[u]) * dimv + c] : vzero<V>();
+        if (r == 0 && u < kChunk)
+          old[u] = (cok && head[u] && id[u] < vocab) ? grads[size_t(id[u]) * dimv + c] : vzero<V>();
+      }
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        if (pos[u] != kNone) {
+          if (r == 0 && u < kChunk && head[u]) acc = old[u];
+          acc = vadd(acc, v[u]);
+          if (cok && tail[u] && id[u] < vocab) vstore<true>(grads + size_t(id[u]) * dimv + c, acc);
+        }
       }
     }
   }
@@ -212,125 +767,31 @@ static unsigned threads_per_row(size_t dimv) {
   return t;
 }
 
-static unsigned key_bits(unsigned vocab) {
-  unsigned bits = 1;
-  while (bits < 32 && (1ull << bits) < (unsigned long long)vocab) ++bits;
-  return bits;
-}
-
-static size_t align256(size_t n) { return (n + 255) / 256 * 256; }
-
-static int sort_tmp_bytes(unsigned n, unsigned vocab, size_t* bytes) {
-  size_t tmp = 0;
-  unsigned* k = nullptr;
-  hipError_t e = rocprim::radix_sort_pairs(nullptr, tmp, static_cast<const unsigned*>(k), k,
-                                           rocprim::counting_iterator<unsigned>(0), k, n, 0, key_bits(vocab));
-  if (e != hipSuccess) return fail(DYHIP_ERR_RUNTIME, "radix sort size query failed: %s", hipGetErrorString(e));
-  *bytes = tmp;
-  return DYHIP_OK;
-}
-
-__global__ void plan_reset_kernel(unsigned* fix_count) { *fix_count = 0; }
-
-// Per chunk of the sorted ids: does a run start here (not continuing from the previous chunk,
-// or filling this chunk only partly) and continue into the next chunk?  If so, in which chunk
-// does it end (binary search for the upper bound of its id)?  Every such run becomes one entry
-// of the plan's fix-up list, so the search is paid when the plan is built, not in the backward pass.
-
-__global__ __launch_bounds__(256) void plan_runs_kernel(unsigned n, unsigned chunks,
-                                                        const unsigned* __restrict__ sorted_ids,
-                                                        uint4* __restrict__ fix_list, unsigned* fix_count) {
-  const unsigned ch = blockIdx.x * 256 + threadIdx.x;
-  if (ch >= chunks) return;
-  const unsigned k0 = ch * kChunk, cnt = min(n - k0, (unsigned)kChunk);
-  const unsigned first = sorted_ids[k0], last = sorted_ids[k0 + cnt - 1];
-  const bool open_left = k0 > 0 && sorted_ids[k0 - 1] == first;
-  const bool open_right = k0 + cnt < n && sorted_ids[k0 + cnt] == last;
-  unsigned out = kNone;
-  if (open_right && !(first == last && open_left)) {
-    unsigned lo = k0 + cnt, hi = n;
-    while (lo < hi) {
-      const unsigned mid = lo + (hi - lo) / 2;
-      if (sorted_ids[mid] <= last) lo = mid + 1;
-      else hi = mid;
-    }
-    out = (lo - 1) / kChunk;
-  }
-  // the order of the list does not matter: the runs are independent of each other
-  if (out != kNone) fix_list[atomicAdd(fix_count, 1u)] = make_uint4(ch, out, last, 0u);
-}
-
-// plan = [sorted_ids (n u32) | sorted_pos (n u32) | fix_list (chunks uint4) | fix_count], each part padded to 256 bytes
-static size_t plan_bytes(unsigned n) {
-  return 2 * align256(sizeof(unsigned) * n) + align256(sizeof(uint4) * cdiv<unsigned>(n, kChunk)) + 256;
-}
-
-static void plan_parts(const void* plan, unsigned n, ScatterWs* w) {
-  char* p = const_cast<char*>(static_cast<const char*>(plan));
-  const size_t ids_b = align256(sizeof(unsigned) * n);
-  w->chunks = cdiv<unsigned>(n, kChunk);
-  w->sorted_ids = reinterpret_cast<unsigned*>(p);
-  w->sorted_pos = reinterpret_cast<unsigned*>(p + ids_b);
-  w->fix_list = reinterpret_cast<uint4*>(p + 2 * ids_b);
-  w->fix_count = reinterpret_cast<unsigned*>(p + 2 * ids_b + align256(sizeof(uint4) * w->chunks));
-}
-
-// scratch of the reduction kernels = [part_first | part_last]
-static size_t reduce_ws_bytes(unsigned n, size_t dim) {
-  const unsigned chunks = cdiv<unsigned>(n, kChunk);
-  return 2 * align256(sizeof(float) * dim * chunks);
-}
-
-static int build_plan(dyhip_device* dev, unsigned n, const unsigned* ids_dev, unsigned vocab, void* plan,
-                      size_t plan_size, void* ws, size_t ws_bytes) {
-  size_t sort_bytes = 0;
-  DYHIP_CHECK_STATUS(sort_tmp_bytes(n, vocab, &sort_bytes));
-  DYHIP_REQUIRE(plan != nullptr && plan_size >= plan_bytes(n) && aligned16(plan),
-                "lookup plan needs %zu bytes (16-byte aligned), got %zu", plan_bytes(n), plan_size);
-  DYHIP_REQUIRE(sort_bytes == 0 || (ws != nullptr && ws_bytes >= sort_bytes),
-                "lookup plan needs %zu workspace bytes, got %zu", sort_bytes, ws_bytes);
-  unsigned* sorted_ids = static_cast<unsigned*>(plan);
-  unsigned* sorted_pos = reinterpret_cast<unsigned*>(static_cast<char*>(plan) + align256(sizeof(unsigned) * n));
-  DYHIP_CHECK_HIP(rocprim::radix_sort_pairs(ws, sort_bytes, ids_dev, sorted_ids,
-                                            rocprim::counting_iterator<unsigned>(0), sorted_pos, n, 0, key_bits(vocab),
-                                            dev->stream));
-  ScatterWs w;
-  plan_parts(plan, n, &w);
-  hipLaunchKernelGGL(plan_reset_kernel, dim3(1), dim3(1), 0, dev->stream, w.fix_count);
-  hipLaunchKernelGGL(plan_runs_kernel, dim3(cdiv<unsigned>(w.chunks, 256)), dim3(256), 0, dev->stream, n, w.chunks,
-                     sorted_ids, w.fix_list, w.fix_count);
-  DYHIP_CHECK_LAUNCH();
-  return DYHIP_OK;
-}
+// scratch of the segmented sum: one 128-byte line per chunk (partial sums of the parts of very long runs)
+static size_t reduce_ws_bytes(unsigned n) { return size_t(128) * cdiv<unsigned>(n, kChunk); }
 
 static int reduce_planned(dyhip_device* dev, unsigned n, const void* plan, size_t dim, unsigned vocab, const float* g,
                           float* all_grads, void* ws, size_t ws_bytes) {
-  const size_t need = reduce_ws_bytes(n, dim);
-  DYHIP_REQUIRE(ws != nullptr && ws_bytes >= need && aligned16(ws),
-                "lookup scatter-add needs %zu workspace bytes (16-byte aligned), got %zu", need, ws_bytes);
-  ScatterWs w;
+  DYHIP_REQUIRE(ws != nullptr && ws_bytes >= reduce_ws_bytes(n) && aligned16(ws),
+                "lookup scatter-add needs %zu workspace bytes (16-byte aligned), got %zu", reduce_ws_bytes(n), ws_bytes);
+  Plan w;
   plan_parts(plan, n, &w);
-  char* base = static_cast<char*>(ws);
-  w.part_first = reinterpret_cast<float*>(base);
-  w.part_last = reinterpret_cast<float*>(base + align256(sizeof(float) * dim * w.chunks));
   const bool vec = dim % 4 == 0 && aligned16(g) && aligned16(all_grads);
   const unsigned dimv = static_cast<unsigned>(vec ? dim / 4 : dim);
   const unsigned tpr = threads_per_row(dimv);
-  const dim3 grid(cdiv<unsigned>(w.chunks, kLkThreads / tpr)), block(kLkThreads);
-  // enough blocks for every CU; a block walks the plan's list of boundary-crossing runs
-  const dim3 fgrid(std::min<unsigned>(w.chunks, 2u * unsigned(dev->num_cus))), fblock(kFixThreads);
-  const size_t flds = size_t(kFixThreads) * (vec ? sizeof(float4) : sizeof(float));
+  const unsigned threads = tpr >= 64 ? tpr : 64;
+  const unsigned chunks = cdiv<unsigned>(n, kChunk);
+  const dim3 grid(cdiv<unsigned>(chunks, threads / tpr)), block(threads);
+  const size_t lds = tpr >= 64 ? size_t(threads) * (vec ? sizeof(float4) : sizeof(float)) : 0;
+#define DYHIP_SCATTER(V, WIDE)                                                                                    \
+  hipLaunchKernelGGL((scatter_runs_kernel<V, WIDE>), grid, block, lds, dev->stream, n, dimv, tpr, vocab, w,     \
+                     reinterpret_cast<const V*>(g), reinterpret_cast<V*>(all_grads), reinterpret_cast<V*>(ws))
   if (vec) {
-    float4* gr = reinterpret_cast<float4*>(all_grads);
-    const float4* g4 = reinterpret_cast<const float4*>(g);
-    // plain loads: streaming (non-temporal) hints make this random-row gather slower, not faster
-    hipLaunchKernelGGL((scatter_chunk_kernel<float4, false>), grid, block, 0, dev->stream, n, dimv, tpr, vocab, w, g4, gr);
-    hipLaunchKernelGGL(scatter_fixup_kernel<float4>, fgrid, fblock, flds, dev->stream, n, dimv, tpr, vocab, w, gr);
+    if (tpr >= 64) DYHIP_SCATTER(float4, true); else DYHIP_SCATTER(float4, false);
   } else {
-    hipLaunchKernelGGL((scatter_chunk_kernel<float, false>), grid, block, 0, dev->stream, n, dimv, tpr, vocab, w, g,
-                       all_grads);
-    hipLaunchKernelGGL(scatter_fixup_kernel<float>, fgrid, fblock, flds, dev->stream, n, dimv, tpr, vocab, w, all_grads);
+    if (tpr >= 64) DYHIP_SCATTER(float, true); else DYHIP_SCATTER(float, false);
   }
+#undef DYHIP_SCATTER
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
@@ -386,10 +847,7 @@ int dyhip_lookup_plan_workspace(unsigned n_ids, unsigned vocab, size_t* ws_bytes
   DYHIP_REQUIRE(ws_bytes != nullptr, "null output pointer");
   *ws_bytes = 0;
   if (n_ids == 0) return DYHIP_OK;
-  size_t b = 0;
-  DYHIP_CHECK_STATUS(sort_tmp_bytes(n_ids, vocab, &b));
-  *ws_bytes = align256(b);
-  return DYHIP_OK;
+  return plan_ws_bytes(n_ids, vocab, ws_bytes);
 }
 
 int dyhip_lookup_build_plan(dyhip_device* dev, unsigned n_ids, const unsigned* ids_dev, unsigned vocab, void* plan,
@@ -400,9 +858,23 @@ int dyhip_lookup_build_plan(dyhip_device* dev, unsigned n_ids, const unsigned* i
   return build_plan(dev, n_ids, ids_dev, vocab, plan, plan_size, ws, ws_bytes);
 }
 
+int dyhip_lookup_plan_invalid_ids(dyhip_device* dev, unsigned n_ids, const void* plan, unsigned* count) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(count != nullptr, "null output pointer");
+  *count = 0;
+  if (n_ids == 0) return DYHIP_OK;
+  DYHIP_REQUIRE(plan != nullptr, "null pointer in lookup plan");
+  Plan w;
+  plan_parts(plan, n_ids, &w);
+  DYHIP_CHECK_HIP(hipMemcpyAsync(count, w.status, sizeof(unsigned), hipMemcpyDeviceToHost, dev->stream));
+  DYHIP_CHECK_HIP(hipStreamSynchronize(dev->stream));
+  return DYHIP_OK;
+}
+
 int dyhip_lookup_accumulate_grads_planned_workspace(unsigned n_ids, size_t dim, size_t* ws_bytes) {
   DYHIP_REQUIRE(ws_bytes != nullptr, "null output pointer");
-  *ws_bytes = (n_ids == 0 || dim == 0) ? 0 : reduce_ws_bytes(n_ids, dim);
+  (void)dim;
+  *ws_bytes = n_ids ? reduce_ws_bytes(n_ids) : 0;
   return DYHIP_OK;
 }
 
@@ -419,9 +891,9 @@ int dyhip_lookup_accumulate_grads_workspace(unsigned n_ids, size_t dim, unsigned
   DYHIP_REQUIRE(ws_bytes != nullptr, "null output pointer");
   *ws_bytes = 0;
   if (n_ids == 0 || dim == 0) return DYHIP_OK;
-  size_t sort_ws = 0;
-  DYHIP_CHECK_STATUS(dyhip_lookup_plan_workspace(n_ids, vocab, &sort_ws));
-  *ws_bytes = plan_bytes(n_ids) + reduce_ws_bytes(n_ids, dim) + sort_ws;
+  size_t plan_ws = 0;
+  DYHIP_CHECK_STATUS(plan_ws_bytes(n_ids, vocab, &plan_ws));
+  *ws_bytes = plan_bytes(n_ids) + align256(reduce_ws_bytes(n_ids)) + plan_ws;
   return DYHIP_OK;
 }
 
@@ -436,7 +908,7 @@ int dyhip_lookup_accumulate_grads(dyhip_device* dev, unsigned n_ids, const unsig
   DYHIP_REQUIRE(ws != nullptr && ws_bytes >= need && aligned16(ws),
                 "lookup scatter-add needs %zu workspace bytes (16-byte aligned), got %zu", need, ws_bytes);
   char* base = static_cast<char*>(ws);
-  const size_t pb = plan_bytes(n_ids), rb = reduce_ws_bytes(n_ids, dim);
+  const size_t pb = plan_bytes(n_ids), rb = align256(reduce_ws_bytes(n_ids));
   DYHIP_CHECK_STATUS(build_plan(dev, n_ids, ids_dev, vocab, base, pb, base + pb + rb, ws_bytes - pb - rb));
   return reduce_planned(dev, n_ids, base, dim, vocab, g, all_grads, base + pb, rb);
 }

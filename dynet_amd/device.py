@@ -481,8 +481,21 @@ class Device:
         _check(cdll.dyhip_lookup_accumulate_grads(self.handle, _u(n), _p(ids_dev), _sz(dim), _u(vocab), _p(g),
                                                   _p(all_grads), _vp(ws), _sz(ws_bytes)))
 
+    @staticmethod
+    def lookup_plan_parts(plan_words, n):
+        """Splits a plan read back as uint32 words into (gid, gpos, roff, rrem): ids grouped by value,
+        their positions, entries of the run before / from each entry.  Each part starts on a 256-byte boundary."""
+        part = (4 * n + 255) // 256 * 256 // 4
+        return tuple(plan_words[q * part:q * part + n] for q in range(4))
+
+    def lookup_plan_invalid_ids(self, n_ids, plan):
+        """How many ids of the plan were >= vocab (the reduction skips them); synchronises."""
+        c = C.c_uint(0)
+        _check(cdll.dyhip_lookup_plan_invalid_ids(self.handle, _u(n_ids), _p(plan), C.byref(c)))
+        return c.value
+
     def lookup_build_plan(self, ids_dev, vocab):
-        """Sorted (id, position) plan of a lookup's ids; returns the plan buffer (FXS pool)."""
+        """Plan of a lookup's ids (ids grouped by value with run offsets); returns the plan buffer (FXS pool)."""
         n = ids_dev.size
         pb, wb = _sz(0), _sz(0)
         _check(cdll.dyhip_lookup_plan_bytes(_u(n), C.byref(pb)))

@@ -334,16 +334,24 @@ int dyhip_dropout_backward(dyhip_device* dev, size_t n, const float* mask, const
  * (:323) and copied to ids_dev (the node's aux_mem, :318). */
 int dyhip_lookup_forward(dyhip_device* dev, unsigned n_ids, const unsigned* ids_host, unsigned* ids_dev,
                          size_t dim, unsigned vocab, const float* table, float mult, float* fx);
-/* all_grads[:, ids[b]] += g[:, b], duplicates summed in ascending b by a
- * sorted-index segmented reduction (no atomics, deterministic). */
+/* all_grads[:, ids[b]] += g[:, b] without float atomics: the ids are grouped by value (the "plan") and one
+ * kernel sums each run of equal ids.  Deterministic; a row that fewer than 15 ids name is summed in
+ * ascending b starting from its old value, i.e. bit-identical to the CPU path (:735-741); a row named
+ * more often is summed by several thread groups (entries interleaved over a fixed number of slots, slots
+ * added in ascending order).  ids >= vocab are skipped (the reference throws on the host,
+ * dynet/param-nodes.cc:323, and does not check device-resident ids); dyhip_lookup_plan_invalid_ids
+ * tells how many there were. */
 int dyhip_lookup_accumulate_grads_workspace(unsigned n_ids, size_t dim, unsigned vocab, size_t* ws_bytes);
-/* The same in two phases.  The sorted (id, position) plan depends only on the ids, so
- * an executor can build it right after the forward gather (the ids sit in the node's
- * aux_mem from then on) and the backward pass is left with the reduction kernels. */
+/* The same in two phases.  The plan depends only on the ids, so an executor can build it right after the
+ * forward gather (the ids sit in the node's aux_mem from then on) and the backward pass is left with the
+ * reduction kernel.  Up to 65535 ids the plan is built by one kernel; beyond that by a device-wide radix
+ * sort.  The plan is opaque; vocab must be below 2^31 - 1.  dyhip_lookup_accumulate_grads_planned takes no
+ * workspace any more (its size query returns 0; ws may be NULL). */
 int dyhip_lookup_plan_bytes(unsigned n_ids, size_t* plan_bytes);
 int dyhip_lookup_plan_workspace(unsigned n_ids, unsigned vocab, size_t* ws_bytes);
 int dyhip_lookup_build_plan(dyhip_device* dev, unsigned n_ids, const unsigned* ids_dev, unsigned vocab, void* plan,
                             size_t plan_bytes, void* ws, size_t ws_bytes);
+int dyhip_lookup_plan_invalid_ids(dyhip_device* dev, unsigned n_ids, const void* plan, unsigned* count);
 int dyhip_lookup_accumulate_grads_planned_workspace(unsigned n_ids, size_t dim, size_t* ws_bytes);
 int dyhip_lookup_accumulate_grads_planned(dyhip_device* dev, unsigned n_ids, const void* plan, size_t dim,
                                           unsigned vocab, const float* g, float* all_grads, void* ws, size_t ws_bytes);
