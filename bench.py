@@ -57,6 +57,10 @@ def parse_args():
                     help="counter-collection mode: launch every kernel of the sweep (and a 16.8 MB calibration copy) "
                          "a few times with plain launches, print nothing but a short note, and exit")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-summary", nargs=2, metavar=("FETCH_DB", "WRITE_DB"),
+                    help="print the hardware-counter summary of two --one-pass runs under rocprofv3 --pmc and exit")
+    ap.add_argument("--unique-ids", type=int, default=None,
+                    help="with --pmc-summary: distinct ids of the cfg-3 id vector (the bench prints it as unique_ids)")
     ap.add_argument("--no-extras", action="store_true", help="skip the cfg 1 / 3 / 4 kernel measurements")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="bound on the CPU-baseline leg")
     ap.add_argument("--no-lm", action="store_true", help="skip the cfg 5 LSTM-LM training-step measurement")
@@ -183,17 +187,18 @@ def per_kernel_table(dev, named, sets, reps, use_graph=True):
     return out
 
 
-def extras(dev, lib, reps, use_graph=True):
-    """cfg 3 (lookup), cfg 4 (PickNegLogSoftmax) kernels and the cfg 1 LSTM cell latency."""
-    from dynet_amd.synth import glorot, zipf_ids
+def extras_kernels(dev, lib, n_sets=None):
+    """cfg 3 (lookup) and cfg 4 (PickNegLogSoftmax): yields (name, info, [(kernel, bytes, launcher)], buffer sets),
+    one configuration at a time (the caller frees the pools in between).  Enough rotating buffer sets that a
+    kernel's working set over one rotation exceeds the 256 MB Infinity Cache."""
+    from dynet_amd.synth import zipf_ids
 
     rng = np.random.default_rng(0)
-    res = {}
     # ---- cfg 3: lookup 50000 x 512, 16384 Zipf(1.1) ids -----------------------
-    V, D, n = 50000, 512, 256 * 64
+    V, D, n = CFG3["V"], CFG3["D"], CFG3["n"]
     G = n * D * 4
     sets = []
-    for _ in range(4):
+    for _ in range(n_sets or 8):  # 8 x (33.5 MB of gradient rows + ~8 MB of touched table rows) = 335 MB
         ids = zipf_ids(rng, n, V)
         sets.append({
             "table": dev.tensor(rng.uniform(-0.1, 0.1, (V, D)).astype(np.float32)),
@@ -204,28 +209,26 @@ def extras(dev, lib, reps, use_graph=True):
         })
     ws, wsb = dev.workspace(dev.lookup_accumulate_grads_workspace(n, D, V))
     uniq = sets[0]["uniq"]
-    gather = [("lookup_gather", 2 * G + n * 4,
-               lambda s: dev.lookup_forward(None, s["ids"], D, V, s["table"], s["fx"]))]
-    # the scatter-add is a library sort followed by two kernels: timed as plain launches, outside a graph
-    scatter = [("lookup_scatter_add(sort+segmented)", G + 2 * uniq * D * 4,
-                lambda s: dev.lookup_accumulate_grads(s["ids"], D, V, s["g"], s["grads"], ws, wsb))]
     for s in sets:
-        s["plan"] = dev.lookup_build_plan(s["ids"], V)
+        s["plan"], s["plan_ws"], s["plan_wsb"] = dev.lookup_plan_buffers(n, V)
+        dev.lookup_build_plan_into(s["ids"], V, s["plan"], s["plan_ws"], s["plan_wsb"])
     ws2, wsb2 = dev.workspace(dev.lookup_accumulate_grads_planned_workspace(n, D))
-    planned = [("lookup_scatter_add(ids pre-sorted at forward)", G + 2 * uniq * D * 4,
-                lambda s: dev.lookup_accumulate_grads_planned(n, s["plan"], D, V, s["g"], s["grads"], ws2, wsb2))]
-    res["cfg3_lookup"] = {"vocab": V, "dim": D, "n_ids": n, "unique_ids": uniq,
-                          "kernels": per_kernel_table(dev, gather, sets, reps, use_graph=use_graph) +
-                          per_kernel_table(dev, planned, sets, reps, use_graph=use_graph) +
-                          per_kernel_table(dev, scatter, sets, reps, use_graph=False)}
-    for w in (lib.POOL_FXS, lib.POOL_DEDFS, lib.POOL_SCS):
-        dev.sync()
-        dev.free_pool(w)
+    scatter_bytes = G + 2 * uniq * D * 4
+    named = [
+        ("lookup_gather", 2 * G + n * 4, lambda s: dev.lookup_forward(None, s["ids"], D, V, s["table"], s["fx"])),
+        ("lookup_scatter_add(plan built at forward)", scatter_bytes,
+         lambda s: dev.lookup_accumulate_grads_planned(n, s["plan"], D, V, s["g"], s["grads"], ws2, wsb2)),
+        ("lookup_scatter_add(plan + segmented sum)", scatter_bytes,
+         lambda s: dev.lookup_accumulate_grads(s["ids"], D, V, s["g"], s["grads"], ws, wsb)),
+        ("lookup_plan (one kernel; no float data moved, bytes as for the scatter-add)", scatter_bytes,
+         lambda s: dev.lookup_build_plan_into(s["ids"], V, s["plan"], s["plan_ws"], s["plan_wsb"])),
+    ]
+    yield "cfg3_lookup", {"vocab": V, "dim": D, "n_ids": n, "unique_ids": uniq, "rotating_buffer_sets": len(sets)}, named, sets
     # ---- cfg 4: PickNegLogSoftmax 50000 x 512 ----------------------------------
-    rows, bd = 50000, 512
+    rows, bd = CFG4["rows"], CFG4["bd"]
     X = rows * bd * 4
     sets = []
-    for _ in range(3):
+    for _ in range(n_sets or 3):
         labels = rng.integers(0, rows, bd).astype(np.uint32)
         aux = dev.empty(3 * bd)
         aux.offset(2 * bd, (bd,)).set((np.arange(bd, dtype=np.uint32) * rows + labels).view(np.float32))
@@ -238,10 +241,21 @@ def extras(dev, lib, reps, use_graph=True):
         ("pnls_fwd", X, lambda s: dev.pnls_forward_staged(rows, bd, s["x"], s["aux"], s["fx"])),
         ("pnls_bwd", 3 * X, lambda s: dev.pnls_backward(rows, bd, s["x"], s["aux"], s["dy"], s["dx"])),
     ]
-    res["cfg4_pnls"] = {"rows": rows, "bd": bd, "kernels": per_kernel_table(dev, named, sets, reps, use_graph=use_graph)}
-    for w in (lib.POOL_FXS, lib.POOL_DEDFS, lib.POOL_SCS):
-        dev.sync()
-        dev.free_pool(w)
+    yield "cfg4_pnls", {"rows": rows, "bd": bd, "rotating_buffer_sets": len(sets)}, named, sets
+
+
+def extras(dev, lib, reps, use_graph=True):
+    """cfg 3 (lookup), cfg 4 (PickNegLogSoftmax) kernels and the cfg 1 LSTM cell latency."""
+    from dynet_amd.synth import glorot
+
+    rng = np.random.default_rng(1)
+    res = {}
+    for name, info, named, sets in extras_kernels(dev, lib):
+        info["kernels"] = per_kernel_table(dev, named, sets, reps, use_graph=use_graph)
+        res[name] = info
+        for w in (lib.POOL_FXS, lib.POOL_DEDFS, lib.POOL_SCS):
+            dev.sync()
+            dev.free_pool(w)
     # ---- cfg 1: one fused LSTM cell step, fwd + bwd ------------------------------
     I, H, B = 128, 256, 32
     t = {k: dev.tensor(v) for k, v in {
@@ -343,15 +357,123 @@ def extras(dev, lib, reps, use_graph=True):
 
 FP32_MFMA_PEAK_TFLOPS = 157.3
 
-# HBM bytes per launch measured with hardware counters (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, on
-# `bench.py --one-pass`, each scaled by what the same counter reads for the library's 16 MiB copy kernel:
-# x1.9967 and x0.9997); the table is in profiles/cfg2_sweep_hbm_traffic_pmc.txt.  Keyed by bench kernel name.
-MEASURED_TRAFFIC_BYTES = {
-    "tanh_fwd": 33.58e6, "logistic_fwd": 33.60e6, "rectify_fwd": 33.55e6, "tanh_bwd": 67.05e6,
-    "logistic_bwd": 67.04e6, "rectify_bwd": 67.05e6, "cmult_fwd": 50.30e6, "cmult_bwd_arg0": 67.05e6,
-    "cmult_bwd_arg1": 67.05e6, "sum_batches_fwd": 17.06e6 + 2.14e6, "sum_batches_bwd": 33.81e6,
-    "layer_norm_fwd": 33.62e6, "layer_norm_bwd": 69.27e6 + 2.14e6,
-}
+PMC_PROFILE = os.path.join(ROOT, "profiles", "hbm_traffic_pmc_all_kernels.txt")
+
+
+def measured_traffic():
+    """HBM bytes per launch from the committed hardware-counter summary (rocprofv3 --pmc FETCH_SIZE, then
+    WRITE_SIZE, on `bench.py --one-pass`, scaled as the summary says; written by `bench.py --pmc-summary`).
+    The counters are not read in this run: the figures belong to the commit that wrote the file.  {} if absent."""
+    out = {}
+    try:
+        with open(PMC_PROFILE) as f:
+            for line in f:
+                parts = line.split()
+                if len(parts) == 3 and parts[0] == "TRAFFIC":
+                    out[parts[1]] = float(parts[2])
+    except OSError:
+        pass
+    return out
+
+
+# device kernel (substring of its name) -> entry of the counter summary
+PMC_KERNELS = [
+    ("TanhFwd", "tanh_fwd"), ("TanhBwd", "tanh_bwd"), ("LogisticPacketFwd", "logistic_fwd"),
+    ("LogisticBwd", "logistic_bwd"), ("RectifyFwd", "rectify_fwd"), ("RectifyBwd", "rectify_bwd"),
+    ("AccMul2", "cmult_bwd"), ("Mul2", "cmult_fwd"), ("AccIn0", "sum_batches_bwd"),
+    ("batch_reduce_kernel", "sum_batches_fwd"), ("ln_fwd_wave_kernel", "layer_norm_fwd"),
+    ("ln_bwd_wave_kernel", "layer_norm_bwd_main"), ("combine_partials", "layer_norm_bwd_combine"),
+    ("lookup_gather_kernel", "lookup_gather"), ("plan_group_kernel", "lookup_plan"),
+    ("scatter_runs_kernel", "lookup_scatter_runs"), ("lse_cols_kernel", "pnls_fwd"), ("pnls_bwd_kernel", "pnls_bwd"),
+]
+CFG3 = {"V": 50000, "D": 512, "n": 256 * 64}
+CFG4 = {"rows": 50000, "bd": 512}
+
+
+def print_pmc_summary(fetch_db, write_db, unique_ids):
+    """Text summary of two rocprofv3 --pmc runs of `bench.py --one-pass` (rocpd databases): KiB per dispatch of
+    FETCH_SIZE and WRITE_SIZE per kernel, the scale factors from the calibration copies, and TRAFFIC lines
+    (bench entry, HBM bytes per launch) that measured_traffic() reads back."""
+    import re
+    import sqlite3
+
+    def table(path):
+        cur = sqlite3.connect(path).cursor()
+        rows = cur.execute("select kernel_name, count(*), avg(value) from counters_collection group by kernel_name")
+        return {k: (c, a) for k, c, a in rows}
+
+    def entry(kname):
+        if "IdentityFwd" in kname:  # the calibration copy: 4th template argument = streaming accesses or not
+            m = re.search(r"ew_vec4_kernel<\s*\d+,\s*\w+,\s*\d+,\s*(true|false)", kname)
+            return "copy_streaming" if (m and m.group(1) == "true") else "copy_plain"
+        for sub, name in PMC_KERNELS:
+            if sub in kname:
+                return name
+        return None
+
+    f, w = table(fetch_db), table(write_db)
+    rows = {}
+    for k in f:
+        e = entry(k)
+        if e is None:
+            continue
+        calls, fk = f[k]
+        wk = w.get(k, (0, 0.0))[1]
+        r = rows.setdefault(e, [0, 0.0, 0.0])
+        r[1] = (r[1] * r[0] + fk * calls) / (r[0] + calls)
+        r[2] = (r[2] * r[0] + wk * calls) / (r[0] + calls)
+        r[0] += calls
+    S = S_BYTES
+    G = CFG3["n"] * CFG3["D"] * 4
+    X = CFG4["rows"] * CFG4["bd"] * 4
+    algo = {"tanh_fwd": 2 * S, "logistic_fwd": 2 * S, "rectify_fwd": 2 * S, "tanh_bwd": 4 * S, "logistic_bwd": 4 * S,
+            "rectify_bwd": 4 * S, "cmult_fwd": 3 * S, "cmult_bwd": 4 * S, "sum_batches_fwd": S + S // 64,
+            "sum_batches_bwd": 2 * S + S // 64, "layer_norm_fwd": 2 * S + 2 * LN_N * 4,
+            "layer_norm_bwd_main": 4 * S + 4 * LN_N * 4, "lookup_gather": 2 * G + CFG3["n"] * 4,
+            "lookup_scatter_runs": G + 2 * unique_ids * CFG3["D"] * 4, "pnls_fwd": X, "pnls_bwd": 3 * X}
+    kib = S / 1024.0
+    cs, cp = rows.get("copy_streaming"), rows.get("copy_plain")
+    ff = kib / cs[1]
+    fw = kib / cs[2]
+    print("HBM traffic per launch from hardware counters, one MI355X")
+    print()
+    print("commands (each from /tmp with TMPDIR=/tmp, one counter per run):")
+    print("  timeout -s KILL 120 rocprofv3 --pmc FETCH_SIZE -d <out> -o pmc -- python3 bench.py --one-pass --sets 4")
+    print("  timeout -s KILL 120 rocprofv3 --pmc WRITE_SIZE -d <out> -o pmc -- python3 bench.py --one-pass --sets 4")
+    print("  python3 bench.py --pmc-summary <FETCH run>/pmc_results.db <WRITE run>/pmc_results.db --unique-ids %d" % unique_ids)
+    print("(--one-pass: plain launches of the cfg-2 sweep over 4 buffer sets, each preceded by the library's copy kernel on a")
+    print(" 16 MiB tensor, once with streaming (non-temporal) and once with plain accesses; then the cfg-3 lookup kernels and")
+    print(" the cfg-4 PickNegLogSoftmax kernels on 4 buffer sets each.  KiB per dispatch, averaged, from the rocpd database.)")
+    print()
+    print("calibration: the copy kernel moves %.0f KiB each way." % kib)
+    print("  streaming accesses: FETCH_SIZE reads %.1f, WRITE_SIZE reads %.1f" % (cs[1], cs[2]))
+    if cp:
+        print("  plain accesses:     FETCH_SIZE reads %.1f, WRITE_SIZE reads %.1f" % (cp[1], cp[2]))
+        print("  -> the FETCH_SIZE ratio to the bytes moved is %.4f with streaming loads and %.4f with plain loads: the counter's"
+              % (cs[1] / kib, cp[1] / kib))
+        print("     scale does not depend on the kind of load, so one factor applies to every kernel below.")
+    print("  -> scale factors: FETCH x %.4f, WRITE x %.4f" % (ff, fw))
+    print()
+    print("%-28s %6s %12s %12s %12s %15s %8s" % ("kernel", "calls", "FETCH KiB", "WRITE KiB", "scaled MB", "algorithmic MB", "ratio"))
+    traffic = {}
+    for name in sorted(rows):
+        calls, fk, wk = rows[name]
+        scaled = (fk * ff + wk * fw) * 1024.0
+        traffic[name] = scaled
+        al = algo.get(name)
+        print("%-28s %6d %12.1f %12.1f %12.2f %15s %8s" % (name, calls, fk, wk, scaled / 1e6,
+                                                         "%.2f" % (al / 1e6) if al else "-",
+                                                         "%.3f" % (scaled / al) if al else "-"))
+    print()
+    print("bench entries (layer_norm_bwd = main kernel + its combine launch; both cmult_bwd calls launch one kernel):")
+    t = dict(traffic)
+    if "layer_norm_bwd_main" in t:
+        t["layer_norm_bwd"] = t.pop("layer_norm_bwd_main") + t.pop("layer_norm_bwd_combine", 0.0)
+    if "cmult_bwd" in t:
+        t["cmult_bwd_arg0"] = t["cmult_bwd_arg1"] = t.pop("cmult_bwd")
+    for name in sorted(t):
+        if not name.startswith("copy_"):
+            print("TRAFFIC %s %.0f" % (name, t[name]))
 
 
 def lstm_lm(steps, warmup=3, use_graph=True):
@@ -482,45 +604,72 @@ def lm_kernels(reps, use_graph=True):
 
 
 def cpu_baseline(step_bytes, seconds):
-    """The CPU oracle (plain-C restatement of DyNet's CPU path) on the same sweep, one host core."""
+    """The CPU oracle (plain-C restatement of DyNet's CPU path) on the same sweep: one host core (the process is
+    pinned to it for the duration), the C functions called directly into preallocated outputs."""
+    import ctypes as C
+
     from oracle import cpu_oracle as orc
 
+    L = orc._lib
     rng = np.random.default_rng(0)
     x = rng.standard_normal(S_ELEMS).astype(np.float32)
     x2 = rng.standard_normal(S_ELEMS).astype(np.float32)
     dy = rng.standard_normal(S_ELEMS).astype(np.float32)
-    dx = np.zeros(S_ELEMS, np.float32)
+    dx, y = np.zeros(S_ELEMS, np.float32), np.empty(S_ELEMS, np.float32)
+    s_out = np.empty(SB_N, np.float32)
     g = rng.uniform(0.5, 1.5, LN_N).astype(np.float32)
     b = (rng.standard_normal(LN_N) * 0.1).astype(np.float32)
     dg, db = np.zeros(LN_N, np.float32), np.zeros(LN_N, np.float32)
+    fp = lambda a: a.ctypes.data_as(C.POINTER(C.c_float))  # noqa: E731
+    X, X2, DY, DX, Y, SO, G, B, DG, DB = (fp(a) for a in (x, x2, dy, dx, y, s_out, g, b, dg, db))
+    n, one = C.c_size_t(S_ELEMS), C.c_uint(1)
 
     def sweep():
         for op in (orc.OP_TANH, orc.OP_LOGISTIC, orc.OP_RECTIFY):
-            y = orc.unary_forward(op, x)
-            orc.unary_backward(op, y, dy, dx)
-        orc.cmult_forward(S_ELEMS, 1, 1, x, x2)
-        orc.cmult_backward(S_ELEMS, 1, 1, x, x2, dy, 0, dx)
-        orc.cmult_backward(S_ELEMS, 1, 1, x, x2, dy, 1, dx)
-        s = orc.sum_batches_forward(SB_N, SB_BD, x)
-        orc.sum_batches_backward(SB_N, SB_BD, s, dx)
-        orc.layer_norm_forward(LN_N, LN_BD, x, g, b)
-        orc.layer_norm_backward(LN_N, LN_BD, x, g, dy, dx, dg, db)
+            L.orc_unary_forward(op, orc.LOGISTIC_PACKET, n, X, Y)
+            L.orc_unary_backward(op, n, Y, DY, DX)
+        L.orc_cmult_forward(n, one, one, X, X2, Y)
+        L.orc_cmult_backward(n, one, one, X, X2, DY, C.c_uint(0), DX)
+        L.orc_cmult_backward(n, one, one, X, X2, DY, C.c_uint(1), DX)
+        L.orc_sum_batches_forward(C.c_size_t(SB_N), C.c_uint(SB_BD), X, SO)
+        L.orc_sum_batches_backward(C.c_size_t(SB_N), C.c_uint(SB_BD), SO, DX)
+        L.orc_layer_norm_forward(C.c_size_t(LN_N), C.c_uint(LN_BD), X, G, B, Y)
+        L.orc_layer_norm_backward(C.c_size_t(LN_N), C.c_uint(LN_BD), X, G, DY, DX, DG, DB)
 
-    sweep()
-    reps, t0 = 0, time.perf_counter()
-    while True:
+    pinned = None
+    try:
+        allowed = sorted(os.sched_getaffinity(0))
+        pinned = allowed[len(allowed) // 2]
+        os.sched_setaffinity(0, {pinned})
+    except (AttributeError, OSError):
+        allowed = None
+    try:
         sweep()
-        reps += 1
-        el = time.perf_counter() - t0
-        if el >= seconds or reps >= 50:
-            break
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            sweep()
+            reps += 1
+            el = time.perf_counter() - t0
+            if el >= seconds or reps >= 50:
+                break
+    finally:
+        if allowed is not None:
+            os.sched_setaffinity(0, set(allowed))
     return {"value": round(step_bytes * reps / el / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": "%d full passes of the same cfg-2 sweep (4096x1024 fp32) through oracle/libdynet_cpu_oracle.so "
-                      "in %.1f s on one host core of %d" % (reps, el, os.cpu_count() or 0)}
+                      "in %.1f s on one host core (pinned to cpu %s) of %d" % (reps, el, pinned, os.cpu_count() or 0)}
 
 
 def main():
     args = parse_args()
+    if args.pmc_summary:
+        uniq = args.unique_ids
+        if uniq is None:
+            from dynet_amd.synth import zipf_ids
+
+            uniq = int(np.unique(zipf_ids(np.random.default_rng(0), CFG3["n"], CFG3["V"])).size)
+        print_pmc_summary(args.pmc_summary[0], args.pmc_summary[1], uniq)
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU: the hot path has no multi-GPU leg (it would shard along the batch "
               "dimension with one gradient all-reduce per step). Run with --gpus 1.", file=sys.stderr)
@@ -533,17 +682,32 @@ def main():
         # been replayed in one process; the per-dispatch durations it records do not need graphs anyway
         print("bench.py: running under rocprofiler, switching to plain launches (--no-graph)", file=sys.stderr)
         args.no_graph = True
-    dev = Device(0, mem_mb=(2560, 2048, 64, 256))
+    dev = Device(0, mem_mb=(2560, 2048, 64, 256))  # pools grow on demand (cfg 3 takes ~1.4 GB + 0.8 GB)
     if args.stream_threshold is not None:
         dev.set_stream_threshold(args.stream_threshold)
     sweep = Sweep(dev, lib, args.sets)
     if args.one_pass:
         # hardware-counter runs (rocprofv3 --pmc ...): plain launches so that every dispatch is attributed
+        default_threshold = 8 << 20
         for r in range(min(4, sweep.R)):
             b = sweep.sets[r]
-            dev.scale_copy(S_ELEMS, b["x"], 1.0, b["y"])  # calibration: reads 16 MiB, writes 16 MiB
+            # calibration: reads 16 MiB, writes 16 MiB; with streaming accesses, then with plain ones
+            dev.scale_copy(S_ELEMS, b["x"], 1.0, b["y"])
+            dev.set_stream_threshold(1 << 62)
+            dev.scale_copy(S_ELEMS, b["x"], 1.0, b["y"])
+            dev.set_stream_threshold(args.stream_threshold if args.stream_threshold is not None else default_threshold)
             sweep.run_step(r)
         dev.sync()
+        for w in (lib.POOL_FXS, lib.POOL_DEDFS, lib.POOL_SCS):
+            dev.free_pool(w)
+        for _, _, fns, sets in extras_kernels(dev, lib, n_sets=4):
+            for st in sets:
+                for kname, _, fn in fns:
+                    if "plan + segmented" not in kname:  # the combined call repeats the two kernels timed apart
+                        fn(st)
+            dev.sync()
+            for w in (lib.POOL_FXS, lib.POOL_DEDFS, lib.POOL_SCS):
+                dev.free_pool(w)
         dev.close()
         print(json.dumps({"one_pass": True, "calibration": "ew_vec4_kernel<..IdentityFwd> moves 16384 KiB each way"}))
         return
@@ -580,6 +744,14 @@ def main():
         g.destroy()
     # ---- per-kernel achieved bandwidth ---------------------------------------------
     table = per_kernel_table(dev, sweep.kernels, sweep.sets, args.kernel_reps, use_graph=not args.no_graph)
+    # The ceiling a kernel of this size can reach here: the library's plain copy (streaming 128-bit loads and stores,
+    # nothing else) on the same 16.8 MB tensors, measured in the same way.  Every entry is also given as a fraction
+    # of it: what is left above that fraction is the memory system and the fixed cost of a launch, not the kernel.
+    copy = per_kernel_table(dev, [("copy", 2 * S_BYTES, lambda b: dev.scale_copy(S_ELEMS, b["x"], 1.0, b["y"]))],
+                            sweep.sets, args.kernel_reps, use_graph=not args.no_graph)[0]
+    for k in table:
+        k["frac_of_copy_ceiling"] = round(k["GBps"] / copy["GBps"], 4)
+    traffic_table = measured_traffic()
     # Dominant kernel = the device kernel with the largest share of the sweep's device time, as the first row
     # of a kernel-trace summary of the sweep would name it.  cmult_bwd_arg0 and cmult_bwd_arg1 launch the same
     # device kernel (ew_vec4_kernel<.., AccMul2>); every other row is a device kernel of its own, except
@@ -593,10 +765,11 @@ def main():
         us = sum(r["us"] for r in rows) / len(rows)
         nbytes = sum(r["bytes"] for r in rows) / len(rows)
         gbps = nbytes / us / 1e3
-        traffic = [MEASURED_TRAFFIC_BYTES.get(r["kernel"]) for r in rows]
+        traffic = [traffic_table.get(r["kernel"]) for r in rows]
         return {"bound": "hbm", "kernel": name, "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(gbps / HBM_PEAK_GBPS, 4),
                 "traffic": None if None in traffic else sum(traffic) / len(traffic),
+                "traffic_source": "profiles/" + os.path.basename(PMC_PROFILE) + " (offline counter runs, not this run)",
                 "algorithmic_bytes_per_launch": int(nbytes), "avg_launch_us": round(us, 3),
                 "launches_per_step": len(rows),
                 "share_of_step_device_time": round(sum(r["us"] for r in rows) / sum(k["us"] for k in table), 4)}
@@ -615,8 +788,13 @@ def main():
                    "bytes_per_step": int(sweep.step_bytes)},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
         "wall_ms_per_step": round(wall_ms / args.steps, 5),
-        "roofline": roofline, "roofline_longest_entry": roofline_slowest, "kernels": table,
-        "lstm_lm_tokens_per_s": None,
+        "roofline": roofline, "roofline_longest_entry": roofline_slowest,
+        "hbm_copy_ceiling": {"kernel": "copy of one 4096x1024 fp32 tensor (streaming loads and stores)", "bytes": 2 * S_BYTES,
+                             "us": copy["us"], "GBps": copy["GBps"], "frac_of_8TBps": copy["frac_of_8TBps"]},
+        "kernels": table,
+        # cfg 5, both paths named: the drop-in one (DyNet's nodes called one at a time, as its executor does) and the
+        # time-batched / fused one, which needs the builder-level call sequence INTEGRATION.md describes
+        "lstm_lm_tokens_per_s_node_api": None, "lstm_lm_tokens_per_s_fused_path": None,
     }
     for w in (lib.POOL_FXS, lib.POOL_DEDFS, lib.POOL_SCS):
         dev.sync()
@@ -639,7 +817,8 @@ def main():
     if not args.no_lm:
         out["cfg5_lstm_lm"] = lstm_lm(args.lm_steps, use_graph=not args.no_graph)
         out["cfg5_lstm_lm"]["in_situ"] = lm_kernels(args.kernel_reps, use_graph=not args.no_graph)
-        out["lstm_lm_tokens_per_s"] = out["cfg5_lstm_lm"]["fused_cell_path"]["tokens_per_s"]
+        out["lstm_lm_tokens_per_s_node_api"] = out["cfg5_lstm_lm"]["node_at_a_time_path"]["tokens_per_s"]
+        out["lstm_lm_tokens_per_s_fused_path"] = out["cfg5_lstm_lm"]["fused_cell_path"]["tokens_per_s"]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(sweep.step_bytes, args.cpu_seconds)
     print(json.dumps(out))

@@ -154,16 +154,33 @@ __device__ __forceinline__ void stg1(float* p, const float v) {
 }
 
 // ---- wavefront reductions (64 lanes) -----------------------------------------
+// Cross-lane steps are DPP modifiers of the adding instruction itself (no trip through the LDS crossbar):
+// pairs, quads, half rows and rows of 16 lanes by quad permutes and row mirrors, then lane 15 of a
+// row into the next row and lane 31 into the upper half; lane 63 ends up with the total, which every
+// lane reads back through a scalar register.  Summation order: fixed, the same for every call.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_move(float v, float fill) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(fill), __float_as_int(v), CTRL, ROW_MASK, 0xF, false));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-  return v;
+  v += dpp_move<0xB1, 0xF>(v, 0.f);   // quad_perm [1,0,3,2]
+  v += dpp_move<0x4E, 0xF>(v, 0.f);   // quad_perm [2,3,0,1]
+  v += dpp_move<0x141, 0xF>(v, 0.f);  // row_half_mirror
+  v += dpp_move<0x140, 0xF>(v, 0.f);  // row_mirror: every lane of a row holds the row's sum
+  v += dpp_move<0x142, 0xA>(v, 0.f);  // row_bcast:15 into rows 1 and 3
+  v += dpp_move<0x143, 0xC>(v, 0.f);  // row_bcast:31 into rows 2 and 3
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
-  return v;
+  v = fmaxf(v, dpp_move<0xB1, 0xF>(v, v));
+  v = fmaxf(v, dpp_move<0x4E, 0xF>(v, v));
+  v = fmaxf(v, dpp_move<0x141, 0xF>(v, v));
+  v = fmaxf(v, dpp_move<0x140, 0xF>(v, v));
+  v = fmaxf(v, dpp_move<0x142, 0xA>(v, v));
+  v = fmaxf(v, dpp_move<0x143, 0xC>(v, v));
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
 // Block-wide sum for blockDim.x = 64 * NW.  Every thread gets the result.

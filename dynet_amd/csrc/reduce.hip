@@ -155,8 +155,75 @@ __global__ __launch_bounds__(64 * kCombSlices) void combine_partials_kernel(size
   }
 }
 
+// The same for rows of float4 with many more blocks: a block owns 8 float4 columns (one 128-byte line of every
+// partial row) and 32 row slots; slot q adds rows q, q+32, ... in ascending order with four loads in flight,
+// then eight threads per column add every eighth slot and one adds those eight: a fixed order again.
+constexpr int kCombVecSlots = 32;
+constexpr int kCombVecCols = 8;
+__global__ __launch_bounds__(kCombVecCols * kCombVecSlots) void combine_partials_vec_kernel(unsigned n4, unsigned splits,
+                                                                               const float4* __restrict__ partial0,
+                                                                               float4* __restrict__ out0,
+                                                                               const float4* __restrict__ partial1,
+                                                                               float4* __restrict__ out1,
+                                                                               int accumulate) {
+  __shared__ float4 lds[kCombVecSlots][kCombVecCols];
+  const float4* partial = blockIdx.y == 0 ? partial0 : partial1;
+  float4* out = blockIdx.y == 0 ? out0 : out1;
+  const unsigned c = threadIdx.x % kCombVecCols, q = threadIdx.x / kCombVecCols;
+  const unsigned col = blockIdx.x * kCombVecCols + c;
+  const bool in = col < n4;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  float4 old = acc;
+  if (in && q == 0 && accumulate) old = out[col];
+  if (in) {
+    unsigned sp = q;
+    for (; sp + 3 * kCombVecSlots < splits; sp += 4 * kCombVecSlots) {
+      const float4 a0 = partial[size_t(sp) * n4 + col], a1 = partial[size_t(sp + kCombVecSlots) * n4 + col],
+                   a2 = partial[size_t(sp + 2 * kCombVecSlots) * n4 + col],
+                   a3 = partial[size_t(sp + 3 * kCombVecSlots) * n4 + col];
+      acc.x += a0.x; acc.y += a0.y; acc.z += a0.z; acc.w += a0.w;
+      acc.x += a1.x; acc.y += a1.y; acc.z += a1.z; acc.w += a1.w;
+      acc.x += a2.x; acc.y += a2.y; acc.z += a2.z; acc.w += a2.w;
+      acc.x += a3.x; acc.y += a3.y; acc.z += a3.z; acc.w += a3.w;
+    }
+    for (; sp < splits; sp += kCombVecSlots) {
+      const float4 a = partial[size_t(sp) * n4 + col];
+      acc.x += a.x; acc.y += a.y; acc.z += a.z; acc.w += a.w;
+    }
+  }
+  lds[q][c] = acc;
+  __syncthreads();
+  if (q < 8) {
+    float4 t = lds[q][c];
+    for (int k = q + 8; k < kCombVecSlots; k += 8) {
+      const float4 a = lds[k][c];
+      t.x += a.x; t.y += a.y; t.z += a.z; t.w += a.w;
+    }
+    acc = t;
+  }
+  __syncthreads();
+  if (q < 8) lds[q][c] = acc;
+  __syncthreads();
+  if (q == 0 && in) {
+    float4 t = lds[0][c];
+    for (int k = 1; k < 8; ++k) {
+      const float4 a = lds[k][c];
+      t.x += a.x; t.y += a.y; t.z += a.z; t.w += a.w;
+    }
+    out[col] = make_float4(old.x + t.x, old.y + t.y, old.z + t.z, old.w + t.w);
+  }
+}
+
 static void launch_combine(dyhip_device* dev, size_t n, unsigned splits, const float* p0, float* o0, const float* p1,
                            float* o1, int accumulate) {
+  if (n % 4 == 0 && splits >= 32 && aligned16(p0) && aligned16(o0) && (p1 == nullptr || (aligned16(p1) && aligned16(o1)))) {
+    const unsigned n4 = static_cast<unsigned>(n / 4);
+    hipLaunchKernelGGL(combine_partials_vec_kernel, dim3(cdiv<unsigned>(n4, kCombVecCols), p1 != nullptr ? 2 : 1),
+                       dim3(kCombVecCols * kCombVecSlots), 0, dev->stream, n4, splits, reinterpret_cast<const float4*>(p0),
+                       reinterpret_cast<float4*>(o0), reinterpret_cast<const float4*>(p1), reinterpret_cast<float4*>(o1),
+                       accumulate);
+    return;
+  }
   const dim3 grid((unsigned)cdiv<size_t>(n, 64), p1 != nullptr ? 2 : 1);
   hipLaunchKernelGGL(combine_partials_kernel, grid, dim3(64 * kCombSlices), 0, dev->stream, n, splits, p0, o0, p1, o1,
                      accumulate);
@@ -356,15 +423,15 @@ __device__ __forceinline__ void ln_row_load(LnRow<VPL>& r, unsigned n4, int lane
   }
 }
 
-template <int VPL, bool NT>
-__global__ __launch_bounds__(64 * kLnWavesBwd) void ln_bwd_wave_kernel(unsigned n4, unsigned bd,
+template <int VPL, bool NT, int WAVES, bool PREFETCH>
+__global__ __launch_bounds__(64 * WAVES) void ln_bwd_wave_kernel(unsigned n4, unsigned bd,
                                                                       const float4* __restrict__ x,
                                                                       const float4* __restrict__ g,
                                                                       const float4* __restrict__ dEdf,
                                                                       float4* __restrict__ dx,
                                                                       float* __restrict__ part_dg,
                                                                       float* __restrict__ part_db) {
-  extern __shared__ float lds[];  // [kLnWavesBwd][n] when partials are requested
+  extern __shared__ float lds[];  // [WAVES][n] when partials are requested
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const float fn = float(n4 * 4);
   const bool want_g = part_dg != nullptr, want_b = part_db != nullptr;
@@ -376,16 +443,19 @@ __global__ __launch_bounds__(64 * kLnWavesBwd) void ln_bwd_wave_kernel(unsigned 
     pdg[u] = make_float4(0.f, 0.f, 0.f, 0.f);
     pdb[u] = make_float4(0.f, 0.f, 0.f, 0.f);
   }
-  const unsigned wave_count = gridDim.x * kLnWavesBwd;
-  unsigned row = blockIdx.x * kLnWavesBwd + w;
+  const unsigned wave_count = gridDim.x * WAVES;
+  unsigned row = blockIdx.x * WAVES + w;
   LnRow<VPL> cur, nxt;
-  if (row < bd)
+  if (PREFETCH && row < bd)
     ln_row_load<VPL, NT>(cur, n4, lane, x + size_t(row) * n4, dEdf + size_t(row) * n4,
                          dx ? dx + size_t(row) * n4 : nullptr);
   while (row < bd) {
     // the next row's loads are in flight while this row is reduced and written
     const unsigned next = row + wave_count;
-    if (next < bd)
+    if (!PREFETCH)
+      ln_row_load<VPL, NT>(cur, n4, lane, x + size_t(row) * n4, dEdf + size_t(row) * n4,
+                           dx ? dx + size_t(row) * n4 : nullptr);
+    if (PREFETCH && next < bd)
       ln_row_load<VPL, NT>(nxt, n4, lane, x + size_t(next) * n4, dEdf + size_t(next) * n4,
                            dx ? dx + size_t(next) * n4 : nullptr);
     float s = 0.f;
@@ -412,9 +482,9 @@ __global__ __launch_bounds__(64 * kLnWavesBwd) void ln_bwd_wave_kernel(unsigned 
   {                                                      \
     const float xc = cur.v[u].c + neg;                   \
     const float dq = cur.d[u].c * gg[u].c;               \
-    sxq += dq * xc;                                      \
+    sxq = fmaf(dq, xc, sxq);                             \
     sq += dq;                                            \
-    if (want_g) pdg[u].c += cur.d[u].c * (xc * rs);      \
+    if (want_g) pdg[u].c = fmaf(cur.d[u].c, xc * rs, pdg[u].c); \
     if (want_b) pdb[u].c += cur.d[u].c;                  \
   }
         DYHIP_F4_EACH(DYHIP_LN_ROW)
@@ -447,28 +517,36 @@ __global__ __launch_bounds__(64 * kLnWavesBwd) void ln_bwd_wave_kernel(unsigned 
         }
       }
     }
-    if (next < bd) cur = nxt;
+    if (PREFETCH && next < bd) cur = nxt;
     row = next;
   }
   if (!want_g && !want_b) return;
   const unsigned n = n4 * 4;
-  // combine the waves of this block in ascending wave order, one output at a time
-  for (int which = 0; which < 2; ++which) {
+  // combine the waves of this block in ascending wave order: both outputs in one pass through LDS
+  // (layout [which][wave][n]), the block's partial rows leave with 128-bit stores
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < VPL; ++u) {
+    const unsigned idx = lane + 64 * u;
+    if (idx < n4) {
+      if (want_g) reinterpret_cast<float4*>(lds + size_t(w) * n)[idx] = pdg[u];
+      if (want_b) reinterpret_cast<float4*>(lds + size_t(WAVES + w) * n)[idx] = pdb[u];
+    }
+  }
+  __syncthreads();
+  for (unsigned j4 = threadIdx.x; j4 < 2 * n4; j4 += 64 * WAVES) {
+    const unsigned which = j4 >= n4 ? 1u : 0u;
     float* part = which == 0 ? part_dg : part_db;
     if (part == nullptr) continue;
-    __syncthreads();
+    const unsigned c4 = j4 - which * n4;
+    const float4* src = reinterpret_cast<const float4*>(lds + size_t(which) * WAVES * n) + c4;
+    float4 t = src[0];
 #pragma unroll
-    for (int u = 0; u < VPL; ++u) {
-      const unsigned idx = lane + 64 * u;
-      if (idx < n4) reinterpret_cast<float4*>(lds + size_t(w) * n)[idx] = which == 0 ? pdg[u] : pdb[u];
+    for (int k = 1; k < WAVES; ++k) {
+      const float4 a = src[size_t(k) * n4];
+      t.x += a.x; t.y += a.y; t.z += a.z; t.w += a.w;
     }
-    __syncthreads();
-    for (unsigned j = threadIdx.x; j < n; j += 64 * kLnWavesBwd) {
-      float t = lds[j];
-#pragma unroll
-      for (int k = 1; k < kLnWavesBwd; ++k) t += lds[size_t(k) * n + j];
-      part[size_t(blockIdx.x) * n + j] = t;
-    }
+    reinterpret_cast<float4*>(part + size_t(blockIdx.x) * n)[c4] = t;
   }
 }
 
@@ -687,7 +765,7 @@ int dyhip_layer_norm_backward(dyhip_device* dev, size_t n, unsigned bd, const fl
     const unsigned blocks = ln_bwd_blocks(bd);
     float* part_dg = dg ? static_cast<float*>(ws) : nullptr;
     float* part_db = db ? static_cast<float*>(ws) + size_t(blocks) * n : nullptr;
-    const size_t lds = cols ? size_t(kLnWavesBwd) * n * sizeof(float) : 0;
+    const size_t lds = cols ? size_t(2) * kLnWavesBwd * n * sizeof(float) : 0;  // [dg | db][wave][n]
     const dim3 grid(blocks), block(64 * kLnWavesBwd);
     const float4 *x4 = reinterpret_cast<const float4*>(x), *g4 = reinterpret_cast<const float4*>(g),
                  *d4 = reinterpret_cast<const float4*>(dEdf);
@@ -695,11 +773,19 @@ int dyhip_layer_norm_backward(dyhip_device* dev, size_t n, unsigned bd, const fl
     const bool stream = n * size_t(bd) * sizeof(float) >= dev->stream_threshold;
 #define DYHIP_LN_BWD(VPL)                                                                                  \
   do {                                                                                                     \
+    static bool big_lds_ok = false;                                                                        \
+    if (lds > (size_t(64) << 10) && !big_lds_ok) {                                                          \
+      DYHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&ln_bwd_wave_kernel<VPL, true, kLnWavesBwd, true>),   \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 128 << 10));          \
+      DYHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&ln_bwd_wave_kernel<VPL, false, kLnWavesBwd, true>),  \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 128 << 10));          \
+      big_lds_ok = true;                                                                                   \
+    }                                                                                                      \
     if (stream)                                                                                            \
-      hipLaunchKernelGGL((ln_bwd_wave_kernel<VPL, true>), grid, block, lds, dev->stream, n4, bd, x4, g4, d4, dx4, \
+      hipLaunchKernelGGL((ln_bwd_wave_kernel<VPL, true, kLnWavesBwd, true>), grid, block, lds, dev->stream, n4, bd, x4, g4, d4, dx4, \
                          part_dg, part_db);                                                                \
     else                                                                                                   \
-      hipLaunchKernelGGL((ln_bwd_wave_kernel<VPL, false>), grid, block, lds, dev->stream, n4, bd, x4, g4, d4, dx4, \
+      hipLaunchKernelGGL((ln_bwd_wave_kernel<VPL, false, kLnWavesBwd, true>), grid, block, lds, dev->stream, n4, bd, x4, g4, d4, dx4, \
                          part_dg, part_db);                                                                \
   } while (0)
     if (n4 <= 64) DYHIP_LN_BWD(1);
