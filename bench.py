@@ -242,6 +242,21 @@ def extras_kernels(dev, lib, n_sets=None):
         ("pnls_bwd", 3 * X, lambda s: dev.pnls_backward(rows, bd, s["x"], s["aux"], s["dy"], s["dx"])),
     ]
     yield "cfg4_pnls", {"rows": rows, "bd": bd, "rotating_buffer_sets": len(sets)}, named, sets
+    # ---- layer_norm over rows wider than the one-wave-per-row kernels take (> 2048 floats) ---------------------
+    n, bd = 4096, 1024
+    S = n * bd * 4
+    sets = [{"x": dev.tensor(rng.standard_normal((bd, n)).astype(np.float32)), "y": dev.empty((bd, n)),
+             "dy": dev.tensor(rng.standard_normal((bd, n)).astype(np.float32)),
+             "dx": dev.zeros((bd, n), pool=lib.POOL_DEDFS)} for _ in range(n_sets or 6)]
+    g, b = dev.tensor(rng.uniform(0.5, 1.5, n).astype(np.float32)), dev.tensor(np.zeros(n, np.float32))
+    dg, db = dev.zeros(n, pool=lib.POOL_DEDFS), dev.zeros(n, pool=lib.POOL_DEDFS)
+    ws_ln, ws_lnb = dev.workspace(dev.layer_norm_backward_workspace(n, bd))
+    named = [
+        ("layer_norm_fwd(n=4096)", 2 * S + 2 * n * 4, lambda s: dev.layer_norm_forward(n, bd, s["x"], g, b, s["y"])),
+        ("layer_norm_bwd(n=4096)", 4 * S + 4 * n * 4,
+         lambda s: dev.layer_norm_backward(n, bd, s["x"], g, s["dy"], s["dx"], dg, db, ws_ln, ws_lnb)),
+    ]
+    yield "layer_norm_wide_rows", {"n": n, "bd": bd, "rotating_buffer_sets": len(sets)}, named, sets
 
 
 def extras(dev, lib, reps, use_graph=True):

@@ -1,0 +1,400 @@
+// CwiseSum / CwiseMultiply / CwiseQuotient with broadcast over any dimension (and the batch), and the
+// scalar-constant nodes ConstantPlusX / ConstantMinusX.
+//
+// Replaces the Eigen broadcast / reduce statements of dynet/nodes-arith-cwise.cc (forward :50-97, :196-243,
+// :338-351; backward and backward_helper :99-156, :245-307, :353-421) and dynet/nodes-arith-const.cc:33-75.
+// The batch-only cases keep their streaming kernels (elementwise.hip); this file adds the general case, which
+// the unfused layer_norm composite needs (x - mean, (x - mean) / (sigma + eps): Dim({n}, bd) against Dim({1}, bd)).
+//
+// Layout: a tensor is dims[5] = {d0, d1, d2, d3, bd}, column-major with the batch outermost; on every axis
+// the two arguments agree or one of them is 1.
+//   forward / backward without reduction: one thread per 4 consecutive elements along d0 (128-bit accesses
+//     when d0 % 4 == 0), operands that are 1 along an axis are indexed with stride 0;
+//   backward of an argument that was broadcast: dEdxi[o] += sum of the terms over the broadcast axes.
+//     kept axes = a prefix and the other operand is full size: the batch reduction of reduce.hip (coalesced);
+//     otherwise one wavefront per output element (>= 64 terms, lanes walk the broadcast axes fastest-first,
+//     fixed summation order) or one thread per output element (fewer terms).
+#include "common.h"
+
+namespace dyhip {
+
+int batch_reduce(dyhip_device* dev, size_t n, unsigned bd, const float* in0, const float* in1, float* out,
+                 bool accumulate, void* ws, size_t ws_bytes);
+
+struct CwShape {
+  unsigned d[5];      // dimensions of the full (output-sized) index space
+  size_t s[3][5];     // element strides of the three operands; 0 on an axis the operand is broadcast over
+};
+
+// FN: 0: p0 + p1   1: p0 * p1   2: p0 / p1                                   (forward, overwrite)
+//     3: out + p0  4: out + p0 * p1   5: out + p0 / p1   6: out - p0 / (p1 * p1) * p2   (backward, accumulate)
+template <int FN>
+__device__ __forceinline__ float cw_apply(float p0, float p1, float p2, float old) {
+  if (FN == 0) return p0 + p1;
+  if (FN == 1) return p0 * p1;
+  if (FN == 2) return p0 / p1;
+  if (FN == 3) return old + p0;
+  if (FN == 4) return old + p0 * p1;
+  if (FN == 5) return old + p0 / p1;
+  return old - p0 / (p1 * p1) * p2;
+}
+template <int FN>
+__device__ __forceinline__ float cw_term(float p0, float p1, float p2) {  // what a reduction sums (added to the output)
+  if (FN == 3) return p0;
+  if (FN == 4) return p0 * p1;
+  return -(p0 / (p1 * p1) * p2);
+}
+constexpr int cw_inputs(int fn) { return fn == 3 ? 1 : fn == 6 ? 3 : 2; }
+
+// ---- no reduction: out[e] = f(operands at the broadcast index of e) ------------------------------
+template <int FN, int W>  // W = 4: d0 % 4 == 0 and every pointer 16-byte aligned; W = 1 otherwise
+__global__ __launch_bounds__(256) void cwise_bcast_kernel(CwShape sh, const float* __restrict__ p0,
+                                                          const float* __restrict__ p1, const float* __restrict__ p2,
+                                                          float* __restrict__ out, size_t groups) {
+  constexpr int NIN = cw_inputs(FN);
+  constexpr bool ACC = FN >= 3;
+  const unsigned d0g = sh.d[0] / W;
+  for (size_t g = size_t(blockIdx.x) * 256 + threadIdx.x; g < groups; g += size_t(gridDim.x) * 256) {
+    size_t r = g / d0g;
+    unsigned idx[5];
+    idx[0] = unsigned(g - r * d0g) * W;
+#pragma unroll
+    for (int j = 1; j < 4; ++j) {
+      const size_t q = r / sh.d[j];
+      idx[j] = unsigned(r - q * sh.d[j]);
+      r = q;
+    }
+    idx[4] = unsigned(r);
+    const float* ps[3] = {p0, p1, p2};
+    float v[3][W];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+      if (k < NIN) {
+        size_t off = 0;
+#pragma unroll
+        for (int j = 0; j < 5; ++j) off += size_t(idx[j]) * sh.s[k][j];
+        if (W == 4 && sh.s[k][0] == 1) {
+          const float4 t = *reinterpret_cast<const float4*>(ps[k] + off);
+          v[k][0] = t.x; v[k][1 % W] = t.y; v[k][2 % W] = t.z; v[k][3 % W] = t.w;
+        } else {
+#pragma unroll
+          for (int e = 0; e < W; ++e) v[k][e] = ps[k][off + size_t(e) * sh.s[k][0]];
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < W; ++e) v[k][e] = 0.f;
+      }
+    }
+    float* po = out + g * W;
+    float o[W];
+    if (W == 4) {
+      float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (ACC) t = *reinterpret_cast<const float4*>(po);
+      o[0] = t.x; o[1 % W] = t.y; o[2 % W] = t.z; o[3 % W] = t.w;
+    } else {
+      o[0] = ACC ? po[0] : 0.f;
+    }
+#pragma unroll
+    for (int e = 0; e < W; ++e) o[e] = cw_apply<FN>(v[0][e], v[1][e], v[2][e], o[e]);
+    if (W == 4) *reinterpret_cast<float4*>(po) = make_float4(o[0], o[1 % W], o[2 % W], o[3 % W]);
+    else po[0] = o[0];
+  }
+}
+
+// ---- reduction over the broadcast axes ------------------------------------------------------------
+struct CwReduce {
+  unsigned kd[5], rd[5];   // sizes of the kept / reduced axes, in axis order, padded with 1
+  size_t ks[3][5];         // strides of the three operands along the kept axes (same order)
+  size_t rs[3][5];         // ... along the reduced axes
+  size_t n_out, n_red;
+};
+
+template <int FN>
+__device__ __forceinline__ float cw_reduce_one(const CwReduce& c, size_t o, size_t q0, size_t qstep, const float* p0,
+                                               const float* p1, const float* p2) {
+  constexpr int NIN = cw_inputs(FN);
+  size_t base[3] = {0, 0, 0};
+  {
+    size_t r = o;
+#pragma unroll
+    for (int j = 0; j < 5; ++j) {
+      const size_t q = r / c.kd[j];
+      const size_t i = r - q * c.kd[j];
+      r = q;
+#pragma unroll
+      for (int k = 0; k < NIN; ++k) base[k] += i * c.ks[k][j];
+    }
+  }
+  float acc = 0.f;
+  for (size_t q = q0; q < c.n_red; q += qstep) {
+    size_t off[3] = {base[0], base[1], base[2]};
+    size_t r = q;
+#pragma unroll
+    for (int j = 0; j < 5; ++j) {
+      const size_t t = r / c.rd[j];
+      const size_t i = r - t * c.rd[j];
+      r = t;
+#pragma unroll
+      for (int k = 0; k < NIN; ++k) off[k] += i * c.rs[k][j];
+    }
+    acc += cw_term<FN>(p0[off[0]], NIN > 1 ? p1[off[1]] : 0.f, NIN > 2 ? p2[off[2]] : 0.f);
+  }
+  return acc;
+}
+
+template <int FN>
+__global__ __launch_bounds__(256) void cwise_reduce_wave_kernel(CwReduce c, const float* __restrict__ p0,
+                                                                const float* __restrict__ p1,
+                                                                const float* __restrict__ p2, float* __restrict__ out) {
+  const int lane = threadIdx.x & 63;
+  for (size_t o = size_t(blockIdx.x) * 4 + (threadIdx.x >> 6); o < c.n_out; o += size_t(gridDim.x) * 4) {
+    const float t = wave_sum(cw_reduce_one<FN>(c, o, size_t(lane), 64, p0, p1, p2));
+    if (lane == 0) out[o] += t;
+  }
+}
+
+template <int FN>
+__global__ __launch_bounds__(256) void cwise_reduce_thread_kernel(CwReduce c, const float* __restrict__ p0,
+                                                                  const float* __restrict__ p1,
+                                                                  const float* __restrict__ p2,
+                                                                  float* __restrict__ out) {
+  for (size_t o = size_t(blockIdx.x) * 256 + threadIdx.x; o < c.n_out; o += size_t(gridDim.x) * 256)
+    out[o] += cw_reduce_one<FN>(c, o, 0, 1, p0, p1, p2);
+}
+
+// ---- host side ---------------------------------------------------------------------------------------
+static int cw_check(int op, const unsigned* da, const unsigned* db, const char* what) {
+  DYHIP_REQUIRE(op >= DYHIP_CWISE_SUM && op <= DYHIP_CWISE_QUOTIENT, "%s: unknown operator %d", what, op);
+  DYHIP_REQUIRE(da != nullptr && db != nullptr, "%s: null dimension array", what);
+  for (int j = 0; j < 5; ++j) {
+    DYHIP_REQUIRE(da[j] >= 1 && db[j] >= 1, "%s: empty dimension %d", what, j);
+    if (op == DYHIP_CWISE_QUOTIENT)
+      DYHIP_REQUIRE(da[j] == db[j] || db[j] == 1,
+                    "CwiseQuotient: For each dimension, the dim size needs to match or the right side needs to equal 1 "
+                    "(axis %d: %u and %u)", j, da[j], db[j]);
+    else
+      DYHIP_REQUIRE(da[j] == db[j] || da[j] == 1 || db[j] == 1,
+                    "%s: For each dimension, the dim size needs to match or equal 1 (axis %d: %u and %u)", what, j, da[j],
+                    db[j]);
+  }
+  return DYHIP_OK;
+}
+
+static void cw_strides(const unsigned* dims, const unsigned* full, size_t* s) {
+  size_t stride = 1;
+  for (int j = 0; j < 5; ++j) {
+    s[j] = (dims[j] == 1 && full[j] > 1) ? 0 : stride;
+    stride *= dims[j];
+  }
+}
+
+static size_t cw_size(const unsigned* d) { return size_t(d[0]) * d[1] * d[2] * d[3] * d[4]; }
+
+static unsigned cw_grid(size_t work_items, unsigned per_block, const dyhip_device* dev) {
+  const size_t want = cdiv<size_t>(work_items, per_block);
+  const size_t cap = size_t(dev->num_cus) * 16;
+  return static_cast<unsigned>(want < cap ? (want ? want : 1) : cap);
+}
+
+template <int FN>
+static int cw_launch_bcast(dyhip_device* dev, const CwShape& sh, const float* p0, const float* p1, const float* p2,
+                           float* out) {
+  const size_t total = cw_size(sh.d);
+  if (total == 0) return DYHIP_OK;
+  bool vec = sh.d[0] % 4 == 0 && aligned16(out);
+  const float* ps[3] = {p0, p1, p2};
+  for (int k = 0; k < cw_inputs(FN); ++k) {
+    if (sh.s[k][0] == 1) {  // 128-bit loads of an operand that follows d0
+      vec = vec && aligned16(ps[k]);
+      for (int j = 1; j < 5; ++j) vec = vec && sh.s[k][j] % 4 == 0;
+    }
+  }
+  if (vec) {
+    const size_t groups = total / 4;
+    hipLaunchKernelGGL((cwise_bcast_kernel<FN, 4>), dim3(cw_grid(groups, 256, dev)), dim3(256), 0, dev->stream, sh, p0, p1,
+                       p2, out, groups);
+  } else {
+    hipLaunchKernelGGL((cwise_bcast_kernel<FN, 1>), dim3(cw_grid(total, 256, dev)), dim3(256), 0, dev->stream, sh, p0, p1,
+                       p2, out, total);
+  }
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+template <int FN>
+static int cw_launch_reduce(dyhip_device* dev, const unsigned* full, const unsigned* dself, const size_t s[3][5],
+                            const float* p0, const float* p1, const float* p2, float* out) {
+  CwReduce c;
+  int nk = 0, nr = 0;
+  for (int j = 0; j < 5; ++j) {
+    c.kd[j] = c.rd[j] = 1;
+    for (int k = 0; k < 3; ++k) c.ks[k][j] = c.rs[k][j] = 0;
+  }
+  for (int j = 0; j < 5; ++j) {
+    const bool reduced = dself[j] == 1 && full[j] > 1;
+    if (reduced) {
+      c.rd[nr] = full[j];
+      for (int k = 0; k < 3; ++k) c.rs[k][nr] = s[k][j];
+      ++nr;
+    } else {
+      c.kd[nk] = full[j];
+      for (int k = 0; k < 3; ++k) c.ks[k][nk] = s[k][j];
+      ++nk;
+    }
+  }
+  c.n_out = cw_size(c.kd);
+  c.n_red = cw_size(c.rd);
+  if (c.n_red >= 64)
+    hipLaunchKernelGGL(cwise_reduce_wave_kernel<FN>, dim3(cw_grid(c.n_out, 4, dev)), dim3(256), 0, dev->stream, c, p0, p1, p2,
+                       out);
+  else
+    hipLaunchKernelGGL(cwise_reduce_thread_kernel<FN>, dim3(cw_grid(c.n_out, 256, dev)), dim3(256), 0, dev->stream, c, p0,
+                       p1, p2, out);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+// kept axes form a prefix of the axes and every later axis is reduced (or has size 1)?  Then the reduction is
+// out[j] += sum_b in[b * n + j] with n = the prefix's size: the coalesced batch reduction.
+static bool cw_prefix_split(const unsigned* full, const unsigned* dself, size_t* n, size_t* bd) {
+  int first_red = 5;
+  for (int j = 0; j < 5; ++j)
+    if (dself[j] == 1 && full[j] > 1) {
+      first_red = j;
+      break;
+    }
+  *n = 1;
+  *bd = 1;
+  for (int j = 0; j < 5; ++j) {
+    if (j < first_red) *n *= full[j];
+    else {
+      if (dself[j] != 1) return false;
+      *bd *= full[j];
+    }
+  }
+  return first_red < 5;
+}
+
+struct AddConst {
+  float c;
+  __device__ float operator()(float x) const { return c + x; }
+};
+struct SubFromConst {
+  float c;
+  __device__ float operator()(float x) const { return c - x; }
+};
+
+template <class F>
+__global__ __launch_bounds__(256) void const_op_kernel(size_t n, const float* __restrict__ x, float* __restrict__ y, F f) {
+  for (size_t j = size_t(blockIdx.x) * 256 + threadIdx.x; j < n; j += size_t(gridDim.x) * 256) y[j] = f(x[j]);
+}
+
+}  // namespace dyhip
+
+using namespace dyhip;
+
+extern "C" {
+
+int dyhip_cwise_forward(dyhip_device* dev, int op, const unsigned* dims_a, const unsigned* dims_b, const float* a,
+                        const float* b, float* fx) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_CHECK_STATUS(cw_check(op, dims_a, dims_b, "cwise forward"));
+  DYHIP_REQUIRE(a && b && fx, "null tensor pointer");
+  bool dims_equal = true;
+  for (int j = 0; j < 4; ++j) dims_equal = dims_equal && dims_a[j] == dims_b[j];
+  const size_t n = size_t(dims_a[0]) * dims_a[1] * dims_a[2] * dims_a[3];
+  if (dims_equal && op == DYHIP_CWISE_SUM) return dyhip_csum_forward(dev, n, dims_a[4], dims_b[4], a, b, fx);
+  if (dims_equal && op == DYHIP_CWISE_MULT) return dyhip_cmult_forward(dev, n, dims_a[4], dims_b[4], a, b, fx);
+  CwShape sh;
+  for (int j = 0; j < 5; ++j) sh.d[j] = dims_a[j] > dims_b[j] ? dims_a[j] : dims_b[j];
+  cw_strides(dims_a, sh.d, sh.s[0]);
+  cw_strides(dims_b, sh.d, sh.s[1]);
+  for (int j = 0; j < 5; ++j) sh.s[2][j] = 0;
+  if (op == DYHIP_CWISE_SUM) return cw_launch_bcast<0>(dev, sh, a, b, nullptr, fx);
+  if (op == DYHIP_CWISE_MULT) return cw_launch_bcast<1>(dev, sh, a, b, nullptr, fx);
+  return cw_launch_bcast<2>(dev, sh, a, b, nullptr, fx);
+}
+
+int dyhip_cwise_backward_workspace(const unsigned* dims_a, const unsigned* dims_b, unsigned i, size_t* ws_bytes) {
+  DYHIP_REQUIRE(ws_bytes != nullptr && dims_a != nullptr && dims_b != nullptr && i < 2, "bad argument");
+  unsigned full[5];
+  for (int j = 0; j < 5; ++j) full[j] = dims_a[j] > dims_b[j] ? dims_a[j] : dims_b[j];
+  size_t n = 0, bd = 0;
+  *ws_bytes = 0;
+  if (cw_prefix_split(full, i == 0 ? dims_a : dims_b, &n, &bd) && bd <= 0xFFFFFFFFull)
+    return dyhip_batch_reduce_workspace(n, static_cast<unsigned>(bd), ws_bytes);
+  return DYHIP_OK;
+}
+
+int dyhip_cwise_backward(dyhip_device* dev, int op, const unsigned* dims_a, const unsigned* dims_b, const float* a,
+                         const float* b, const float* dEdf, unsigned i, float* dEdxi, void* ws, size_t ws_bytes) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_CHECK_STATUS(cw_check(op, dims_a, dims_b, "cwise backward"));
+  DYHIP_REQUIRE(i < 2, "the operator has two arguments (i = %u)", i);
+  DYHIP_REQUIRE(a && b && dEdf && dEdxi, "null tensor pointer");
+  unsigned full[5];
+  for (int j = 0; j < 5; ++j) full[j] = dims_a[j] > dims_b[j] ? dims_a[j] : dims_b[j];
+  const unsigned* dself = i == 0 ? dims_a : dims_b;
+  const unsigned* dother = i == 0 ? dims_b : dims_a;
+  const float* other = i == 0 ? b : a;
+  bool reduces = false, other_full = true;
+  for (int j = 0; j < 5; ++j) {
+    reduces = reduces || (dself[j] == 1 && full[j] > 1);
+    other_full = other_full && dother[j] == full[j];
+  }
+  // operands of the term: p0 = dEdf (full size); sum: -, multiply: p1 = other, quotient: p1 = b, p2 = a
+  size_t s[3][5];
+  cw_strides(full, full, s[0]);
+  const float *p1 = nullptr, *p2 = nullptr;
+  for (int j = 0; j < 5; ++j) s[1][j] = s[2][j] = 0;
+  if (op == DYHIP_CWISE_MULT) {
+    p1 = other;
+    cw_strides(dother, full, s[1]);
+  } else if (op == DYHIP_CWISE_QUOTIENT) {
+    p1 = b;
+    cw_strides(dims_b, full, s[1]);
+    p2 = a;
+    cw_strides(dims_a, full, s[2]);
+  }
+  if (!reduces) {
+    CwShape sh;
+    for (int j = 0; j < 5; ++j) {
+      sh.d[j] = full[j];
+      for (int k = 0; k < 3; ++k) sh.s[k][j] = s[k][j];
+    }
+    if (op == DYHIP_CWISE_SUM) return cw_launch_bcast<3>(dev, sh, dEdf, nullptr, nullptr, dEdxi);
+    if (op == DYHIP_CWISE_MULT) return cw_launch_bcast<4>(dev, sh, dEdf, p1, nullptr, dEdxi);
+    if (i == 0) return cw_launch_bcast<5>(dev, sh, dEdf, p1, nullptr, dEdxi);
+    return cw_launch_bcast<6>(dev, sh, dEdf, p1, p2, dEdxi);
+  }
+  DYHIP_REQUIRE(!(op == DYHIP_CWISE_QUOTIENT && i == 0), "CwiseQuotient: the left argument is never broadcast");
+  size_t n = 0, bd = 0;
+  if (op != DYHIP_CWISE_QUOTIENT && cw_prefix_split(full, dself, &n, &bd) && bd <= 0xFFFFFFFFull &&
+      (op == DYHIP_CWISE_SUM || other_full))
+    return batch_reduce(dev, n, static_cast<unsigned>(bd), dEdf, op == DYHIP_CWISE_MULT ? other : nullptr, dEdxi, true, ws,
+                        ws_bytes);
+  if (op == DYHIP_CWISE_SUM) return cw_launch_reduce<3>(dev, full, dself, s, dEdf, nullptr, nullptr, dEdxi);
+  if (op == DYHIP_CWISE_MULT) return cw_launch_reduce<4>(dev, full, dself, s, dEdf, p1, nullptr, dEdxi);
+  return cw_launch_reduce<6>(dev, full, dself, s, dEdf, p1, p2, dEdxi);
+}
+
+int dyhip_const_plus_x_forward(dyhip_device* dev, size_t n, float c, const float* x, float* fx) {
+  DYHIP_CHECK_DEV(dev);
+  if (n == 0) return DYHIP_OK;
+  DYHIP_REQUIRE(x && fx, "null tensor pointer");
+  hipLaunchKernelGGL(const_op_kernel<AddConst>, dim3(cw_grid(n, 256, dev)), dim3(256), 0, dev->stream, n, x, fx, AddConst{c});
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_const_minus_x_forward(dyhip_device* dev, size_t n, float c, const float* x, float* fx) {
+  DYHIP_CHECK_DEV(dev);
+  if (n == 0) return DYHIP_OK;
+  DYHIP_REQUIRE(x && fx, "null tensor pointer");
+  hipLaunchKernelGGL(const_op_kernel<SubFromConst>, dim3(cw_grid(n, 256, dev)), dim3(256), 0, dev->stream, n, x, fx,
+                     SubFromConst{c});
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+}  // extern "C"

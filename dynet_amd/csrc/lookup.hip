@@ -358,7 +358,7 @@ __global__ __launch_bounds__(kPlanThreads) void plan_group_kernel(unsigned n, un
   int* step_last = reinterpret_cast<int*>(plan_lds + kPlanLdsStep);
   int* step_first = step_last + kPlanMaxSteps;
   const unsigned d = blockIdx.x;
-  const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+  const int t = threadIdx.x;
   reinterpret_cast<uint4*>(cnt)[t] = make_uint4(0u, 0u, 0u, 0u);  // 4096 counters, 4 per thread
   // ---- 1. thread t reads positions [t * 4 * quads, (t + 1) * 4 * quads); keys stay in registers ------
   const unsigned quads = cdiv<unsigned>(n, 4u * kPlanThreads);  // 128-bit loads per thread (uniform)

@@ -22,36 +22,45 @@ int batch_reduce(dyhip_device* dev, size_t n, unsigned bd, const float* in0, con
 
 static size_t align256(size_t n) { return (n + 255) / 256 * 256; }
 
+// blocks along the grid's second dimension for B batch elements (kernels stride over the rest)
+static unsigned grid_y(unsigned B) { return B < 65535u ? B : 65535u; }
+
 // dst[b*dst_ld + off + r] = src[b*rows + r] * (mask ? mask[(mask_b ? b : 0)*dst_ld + off + r] : 1)
 __global__ __launch_bounds__(256) void rows_copy_mask_kernel(unsigned rows, unsigned dst_ld, unsigned off,
                                                              const float* __restrict__ src,
                                                              const float* __restrict__ mask, int mask_b,
-                                                             float* __restrict__ dst) {
-  const unsigned r = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
+                                                             float* __restrict__ dst, unsigned B) {
+  const unsigned r = blockIdx.x * 256 + threadIdx.x;
   if (r >= rows) return;
-  float v = src[size_t(b) * rows + r];
-  if (mask) v *= mask[size_t(mask_b ? b : 0) * dst_ld + off + r];
-  dst[size_t(b) * dst_ld + off + r] = v;
+  for (unsigned b = blockIdx.y; b < B; b += gridDim.y) {  // the grid's second dimension holds at most 65535 blocks
+    float v = src[size_t(b) * rows + r];
+    if (mask) v *= mask[size_t(mask_b ? b : 0) * dst_ld + off + r];
+    dst[size_t(b) * dst_ld + off + r] = v;
+  }
 }
 
 // out[b*rows + r] += tmp[b*rows + r] * mask[(mask_b ? b : 0)*mask_ld + off + r]
 __global__ __launch_bounds__(256) void acc_mul_mask_kernel(unsigned rows, unsigned mask_ld, unsigned off,
                                                            const float* __restrict__ tmp,
                                                            const float* __restrict__ mask, int mask_b,
-                                                           float* __restrict__ out) {
-  const unsigned r = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
+                                                           float* __restrict__ out, unsigned B) {
+  const unsigned r = blockIdx.x * 256 + threadIdx.x;
   if (r >= rows) return;
-  out[size_t(b) * rows + r] += tmp[size_t(b) * rows + r] * mask[size_t(mask_b ? b : 0) * mask_ld + off + r];
+  for (unsigned b = blockIdx.y; b < B; b += gridDim.y)
+    out[size_t(b) * rows + r] += tmp[size_t(b) * rows + r] * mask[size_t(mask_b ? b : 0) * mask_ld + off + r];
 }
 
 // dpre[i, b] = i < 3H ? d*f*(1-f) : d*(1-f*f)      (dynet/nodes-lstm.cc:358-361)
 __global__ __launch_bounds__(256) void lstm_dpre_kernel(unsigned H, const float* __restrict__ fx,
-                                                        const float* __restrict__ dEdf, float* __restrict__ dpre) {
-  const unsigned i = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
+                                                        const float* __restrict__ dEdf, float* __restrict__ dpre,
+                                                        unsigned B) {
+  const unsigned i = blockIdx.x * 256 + threadIdx.x;
   if (i >= 4 * H) return;
-  const size_t e = size_t(b) * 4 * H + i;
-  const float f = fx[e], d = dEdf[e];
-  dpre[e] = i < 3 * H ? d * f * (1.f - f) : d * (1.f - f * f);
+  for (unsigned b = blockIdx.y; b < B; b += gridDim.y) {
+    const size_t e = size_t(b) * 4 * H + i;
+    const float f = fx[e], d = dEdf[e];
+    dpre[e] = i < 3 * H ? d * f * (1.f - f) : d * (1.f - f * f);
+  }
 }
 
 // mode 0: c = i*g + f*c_prev                                   (C forward, :562-589)
@@ -64,9 +73,11 @@ __global__ __launch_bounds__(256) void lstm_dpre_kernel(unsigned H, const float*
 template <int MODE>
 __global__ __launch_bounds__(256) void lstm_pointwise_kernel(unsigned H, const float* __restrict__ state,
                                                              const float* __restrict__ gates,
-                                                             const float* __restrict__ d, float* __restrict__ out) {
-  const unsigned r = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
+                                                             const float* __restrict__ d, float* __restrict__ out,
+                                                             unsigned B) {
+  const unsigned r = blockIdx.x * 256 + threadIdx.x;
   if (r >= H) return;
+  for (unsigned b = blockIdx.y; b < B; b += gridDim.y) {
   const size_t s = size_t(b) * H + r;
   const float* gt = gates + size_t(b) * 4 * H;
   if (MODE == 0) {
@@ -88,14 +99,14 @@ __global__ __launch_bounds__(256) void lstm_pointwise_kernel(unsigned H, const f
     out[size_t(b) * 4 * H + 2 * H + r] += d[s] * tanh_accurate(state[s]);
   }
 }
+}
 
 template <int MODE>
 static int launch_pointwise(dyhip_device* dev, unsigned H, unsigned B, const float* state, const float* gates,
                             const float* d, float* out) {
   if (H == 0 || B == 0) return DYHIP_OK;
-  DYHIP_REQUIRE(B <= 65535, "LSTM nodes support at most 65535 batch elements per call");
-  hipLaunchKernelGGL(lstm_pointwise_kernel<MODE>, dim3(cdiv<unsigned>(H, 256), B), dim3(256), 0, dev->stream, H, state,
-                     gates, d, out);
+  hipLaunchKernelGGL(lstm_pointwise_kernel<MODE>, dim3(cdiv<unsigned>(H, 256), grid_y(B)), dim3(256), 0, dev->stream, H,
+                     state, gates, d, out, B);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
@@ -133,8 +144,8 @@ __global__ __launch_bounds__(kCellThreads) void lstm_cell_fwd_kernel(unsigned H,
                                                                      const float* __restrict__ bias,
                                                                      const float* __restrict__ c_prev, int mode,
                                                                      float* gates, float* __restrict__ c,
-                                                                     float* __restrict__ h) {
-  const unsigned j = (blockIdx.x * kCellThreads + threadIdx.x) * V, b = blockIdx.y;
+                                                                     float* __restrict__ h, unsigned b_first) {
+  const unsigned j = (blockIdx.x * kCellThreads + threadIdx.x) * V, b = b_first + blockIdx.y;
   if (j >= H) return;
   const size_t g0 = size_t(b) * 4 * H + j, s0 = size_t(b) * H + j;
   Pack<V> pre[4], cp;
@@ -183,8 +194,8 @@ __global__ __launch_bounds__(kCellThreads) void lstm_cell_bwd_kernel(unsigned H,
                                                                      const float* __restrict__ dh_in,
                                                                      const float* __restrict__ rec,
                                                                      const float* dc_in, float* __restrict__ dpre,
-                                                                     float* dc_prev) {
-  const unsigned j = (blockIdx.x * kCellThreads + threadIdx.x) * V, b = blockIdx.y;
+                                                                     float* dc_prev, unsigned b_first) {
+  const unsigned j = (blockIdx.x * kCellThreads + threadIdx.x) * V, b = b_first + blockIdx.y;
   if (j >= H) return;
   const size_t g0 = size_t(b) * 4 * H + j, s0 = size_t(b) * H + j;
   Pack<V> gt[4], cv, cp, dh, dc;
@@ -395,7 +406,7 @@ static int check_gates(unsigned num_inputs, const float* const* xs, const unsign
                        const float* mask_x, unsigned mask_x_bd, const float* mask_h, unsigned mask_h_bd,
                        GatesInputs* out) {
   DYHIP_REQUIRE(num_inputs >= 1 && xs != nullptr && x_dims != nullptr, "Failed input count check in VanillaLSTMGates");
-  DYHIP_REQUIRE(H >= 1 && B >= 1 && B <= 65535, "VanillaLSTMGates: bad hidden (%u) or batch (%u) size", H, B);
+  DYHIP_REQUIRE(H >= 1 && B >= 1, "VanillaLSTMGates: bad hidden (%u) or batch (%u) size", H, B);
   unsigned I = 0;
   for (unsigned k = 0; k < num_inputs; ++k) {
     DYHIP_REQUIRE(xs[k] != nullptr && x_dims[k] >= 1, "VanillaLSTMGates: x_t[%u] expected to be a vector", k);
@@ -424,8 +435,8 @@ static int prepare_x(dyhip_device* dev, unsigned num_inputs, const float* const*
   }
   unsigned off = 0;
   for (unsigned k = 0; k < num_inputs; ++k) {
-    hipLaunchKernelGGL(rows_copy_mask_kernel, dim3(cdiv<unsigned>(x_dims[k], 256), B), dim3(256), 0, dev->stream,
-                       x_dims[k], I, off, xs[k], mask_x, mask_x_bd > 1 ? 1 : 0, buf);
+    hipLaunchKernelGGL(rows_copy_mask_kernel, dim3(cdiv<unsigned>(x_dims[k], 256), grid_y(B)), dim3(256), 0, dev->stream,
+                       x_dims[k], I, off, xs[k], mask_x, mask_x_bd > 1 ? 1 : 0, buf, B);
     off += x_dims[k];
   }
   DYHIP_CHECK_LAUNCH();
@@ -439,8 +450,8 @@ static int prepare_h(dyhip_device* dev, unsigned H, unsigned B, const float* h, 
     *h_eff = h;
     return DYHIP_OK;
   }
-  hipLaunchKernelGGL(rows_copy_mask_kernel, dim3(cdiv<unsigned>(H, 256), B), dim3(256), 0, dev->stream, H, H, 0u, h,
-                     mask_h, mask_h_bd > 1 ? 1 : 0, buf);
+  hipLaunchKernelGGL(rows_copy_mask_kernel, dim3(cdiv<unsigned>(H, 256), grid_y(B)), dim3(256), 0, dev->stream, H, H, 0u,
+                     h, mask_h, mask_h_bd > 1 ? 1 : 0, buf, B);
   DYHIP_CHECK_LAUNCH();
   *h_eff = buf;
   return DYHIP_OK;
@@ -494,9 +505,8 @@ int dyhip_lstm_gates_dpre(dyhip_device* dev, unsigned H, unsigned B, const float
   DYHIP_CHECK_DEV(dev);
   DYHIP_REQUIRE(fx && dEdf && dpre, "null tensor pointer");
   if (H == 0 || B == 0) return DYHIP_OK;
-  DYHIP_REQUIRE(B <= 65535, "LSTM nodes support at most 65535 batch elements per call");
-  hipLaunchKernelGGL(lstm_dpre_kernel, dim3(cdiv<unsigned>(4 * H, 256), B), dim3(256), 0, dev->stream, H, fx, dEdf,
-                     dpre);
+  hipLaunchKernelGGL(lstm_dpre_kernel, dim3(cdiv<unsigned>(4 * H, 256), grid_y(B)), dim3(256), 0, dev->stream, H, fx, dEdf,
+                     dpre, B);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
@@ -558,8 +568,8 @@ int dyhip_lstm_gates_backward(dyhip_device* dev, unsigned num_inputs, const floa
     GemmSeg s{W, G, dpre, G, G};
     if (!gi.dropout) return gemm_run(dev, true, true, rows, B, 1, &s, dEdxi, acc);
     DYHIP_CHECK_STATUS(gemm_run(dev, true, true, rows, B, 1, &s, tmp, ovw));
-    hipLaunchKernelGGL(acc_mul_mask_kernel, dim3(cdiv<unsigned>(rows, 256), B), dim3(256), 0, dev->stream, rows, mask_ld,
-                       off, tmp, mask, mask_bd > 1 ? 1 : 0, dEdxi);
+    hipLaunchKernelGGL(acc_mul_mask_kernel, dim3(cdiv<unsigned>(rows, 256), grid_y(B)), dim3(256), 0, dev->stream, rows,
+                       mask_ld, off, tmp, mask, mask_bd > 1 ? 1 : 0, dEdxi, B);
     DYHIP_CHECK_LAUNCH();
     return DYHIP_OK;
   }
@@ -612,7 +622,7 @@ int dyhip_lstm_h_backward(dyhip_device* dev, unsigned H, unsigned B, const float
 // ---- fused cell path ------------------------------------------------------------------
 static int recurrent_partials(dyhip_device* dev, bool transposed, unsigned H, unsigned B, const float* Wh,
                               const float* v, void* ws, size_t ws_bytes, unsigned* splits) {
-  DYHIP_REQUIRE(H >= 1 && B >= 1 && B <= 65535, "LSTM cell: bad hidden (%u) or batch (%u) size", H, B);
+  DYHIP_REQUIRE(H >= 1 && B >= 1, "LSTM cell: bad hidden (%u) or batch (%u) size", H, B);
   DYHIP_REQUIRE(Wh && v && ws && splits, "LSTM cell: null pointer");
   const size_t G = size_t(4) * H;
   GemmEpiParams ep{};
@@ -653,18 +663,22 @@ int dyhip_lstm_cell_forward(dyhip_device* dev, unsigned H, unsigned B, const flo
                             const float* rec, unsigned splits, const float* c_tm1, int logistic_mode, float* gates,
                             float* c, float* h) {
   DYHIP_CHECK_DEV(dev);
-  DYHIP_REQUIRE(H >= 1 && B >= 1 && B <= 65535, "LSTM cell: bad hidden (%u) or batch (%u) size", H, B);
+  DYHIP_REQUIRE(H >= 1 && B >= 1, "LSTM cell: bad hidden (%u) or batch (%u) size", H, B);
   DYHIP_REQUIRE(xproj && b && gates && c && h, "LSTM cell: null tensor pointer");
   DYHIP_REQUIRE(splits == 0 || rec != nullptr, "LSTM cell: %u recurrent slices but no buffer", splits);
   DYHIP_REQUIRE(logistic_mode == DYHIP_LOGISTIC_PACKET || logistic_mode == DYHIP_LOGISTIC_SCALAR,
                 "unknown logistic mode %d", logistic_mode);
   const size_t slice = size_t(4) * H * B;
-  if (H % 4 == 0 && all_aligned16({xproj, b, rec, c_tm1, gates, c, h}))
-    hipLaunchKernelGGL(lstm_cell_fwd_kernel<4>, dim3(cdiv<unsigned>(H, kCellThreads * 4), B), dim3(kCellThreads), 0,
-                       dev->stream, H, splits, slice, xproj, rec, b, c_tm1, logistic_mode, gates, c, h);
-  else
-    hipLaunchKernelGGL(lstm_cell_fwd_kernel<1>, dim3(cdiv<unsigned>(H, kCellThreads), B), dim3(kCellThreads), 0,
-                       dev->stream, H, splits, slice, xproj, rec, b, c_tm1, logistic_mode, gates, c, h);
+  const bool vec = H % 4 == 0 && all_aligned16({xproj, b, rec, c_tm1, gates, c, h});
+  for (unsigned b0 = 0; b0 < B; b0 += 65535u) {  // the grid's second dimension holds at most 65535 blocks
+    const unsigned nb = B - b0 < 65535u ? B - b0 : 65535u;
+    if (vec)
+      hipLaunchKernelGGL(lstm_cell_fwd_kernel<4>, dim3(cdiv<unsigned>(H, kCellThreads * 4), nb), dim3(kCellThreads), 0,
+                         dev->stream, H, splits, slice, xproj, rec, b, c_tm1, logistic_mode, gates, c, h, b0);
+    else
+      hipLaunchKernelGGL(lstm_cell_fwd_kernel<1>, dim3(cdiv<unsigned>(H, kCellThreads), nb), dim3(kCellThreads), 0,
+                         dev->stream, H, splits, slice, xproj, rec, b, c_tm1, logistic_mode, gates, c, h, b0);
+  }
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
@@ -673,16 +687,20 @@ int dyhip_lstm_cell_backward(dyhip_device* dev, unsigned H, unsigned B, const fl
                              const float* c_tm1, const float* dh, const float* rec, unsigned splits, const float* dc,
                              float* dpre, float* dc_tm1) {
   DYHIP_CHECK_DEV(dev);
-  DYHIP_REQUIRE(H >= 1 && B >= 1 && B <= 65535, "LSTM cell: bad hidden (%u) or batch (%u) size", H, B);
+  DYHIP_REQUIRE(H >= 1 && B >= 1, "LSTM cell: bad hidden (%u) or batch (%u) size", H, B);
   DYHIP_REQUIRE(gates && c && dh && dpre, "LSTM cell: null tensor pointer");
   DYHIP_REQUIRE(splits == 0 || rec != nullptr, "LSTM cell: %u recurrent slices but no buffer", splits);
   const size_t slice = size_t(H) * B;
-  if (H % 4 == 0 && all_aligned16({gates, c, c_tm1, dh, rec, dc, dpre, dc_tm1}))
-    hipLaunchKernelGGL(lstm_cell_bwd_kernel<4>, dim3(cdiv<unsigned>(H, kCellThreads * 4), B), dim3(kCellThreads), 0,
-                       dev->stream, H, splits, slice, gates, c, c_tm1, dh, rec, dc, dpre, dc_tm1);
-  else
-    hipLaunchKernelGGL(lstm_cell_bwd_kernel<1>, dim3(cdiv<unsigned>(H, kCellThreads), B), dim3(kCellThreads), 0,
-                       dev->stream, H, splits, slice, gates, c, c_tm1, dh, rec, dc, dpre, dc_tm1);
+  const bool vec = H % 4 == 0 && all_aligned16({gates, c, c_tm1, dh, rec, dc, dpre, dc_tm1});
+  for (unsigned b0 = 0; b0 < B; b0 += 65535u) {
+    const unsigned nb = B - b0 < 65535u ? B - b0 : 65535u;
+    if (vec)
+      hipLaunchKernelGGL(lstm_cell_bwd_kernel<4>, dim3(cdiv<unsigned>(H, kCellThreads * 4), nb), dim3(kCellThreads), 0,
+                         dev->stream, H, splits, slice, gates, c, c_tm1, dh, rec, dc, dpre, dc_tm1, b0);
+    else
+      hipLaunchKernelGGL(lstm_cell_bwd_kernel<1>, dim3(cdiv<unsigned>(H, kCellThreads), nb), dim3(kCellThreads), 0,
+                         dev->stream, H, splits, slice, gates, c, c_tm1, dh, rec, dc, dpre, dc_tm1, b0);
+  }
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }

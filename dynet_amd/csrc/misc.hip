@@ -34,32 +34,35 @@ __global__ __launch_bounds__(kThreads) void d2s_subtract_kernel(int n, const uns
 }
 
 // trg[i*bsize + j] = src[idx[i]*bsize + j] * mult : block.y = i, lanes walk j
-__global__ __launch_bounds__(kThreads) void s2d_block_assign_mul_kernel(int bsize, const unsigned* __restrict__ idx,
-                                                                        float mult, const float* __restrict__ src,
+__global__ __launch_bounds__(kThreads) void s2d_block_assign_mul_kernel(int n, int bsize,
+                                                                        const unsigned* __restrict__ idx, float mult,
+                                                                        const float* __restrict__ src,
                                                                         float* __restrict__ trg) {
-  const size_t i = blockIdx.y;
-  const float* ps = src + size_t(idx[i]) * bsize;
-  float* pt = trg + i * bsize;
-  for (int j = blockIdx.x * kThreads + threadIdx.x; j < bsize; j += gridDim.x * kThreads) pt[j] = ps[j] * mult;
+  for (size_t i = blockIdx.y; i < size_t(n); i += gridDim.y) {  // the grid's second dimension holds at most 65535 blocks
+    const float* ps = src + size_t(idx[i]) * bsize;
+    float* pt = trg + i * bsize;
+    for (int j = blockIdx.x * kThreads + threadIdx.x; j < bsize; j += gridDim.x * kThreads) pt[j] = ps[j] * mult;
+  }
 }
 
 // trg[idx[i]*bsize + j] += src[i*bsize + j] with duplicates allowed: atomic, like
 // the reference.  (LookupNode gradients use the deterministic sorted path of
 // dyhip_lookup_accumulate_grads instead.)
-__global__ __launch_bounds__(kThreads) void d2s_block_add_kernel(int bsize, const unsigned* __restrict__ idx,
+__global__ __launch_bounds__(kThreads) void d2s_block_add_kernel(int n, int bsize, const unsigned* __restrict__ idx,
                                                                  const float* __restrict__ src,
                                                                  float* __restrict__ trg) {
-  const size_t i = blockIdx.y;
-  const float* ps = src + i * bsize;
-  float* pt = trg + size_t(idx[i]) * bsize;
-  for (int j = blockIdx.x * kThreads + threadIdx.x; j < bsize; j += gridDim.x * kThreads) atomicAdd(pt + j, ps[j]);
+  for (size_t i = blockIdx.y; i < size_t(n); i += gridDim.y) {
+    const float* ps = src + i * bsize;
+    float* pt = trg + size_t(idx[i]) * bsize;
+    for (int j = blockIdx.x * kThreads + threadIdx.x; j < bsize; j += gridDim.x * kThreads) atomicAdd(pt + j, ps[j]);
+  }
 }
 
 template <bool ACC>
-__global__ __launch_bounds__(kThreads) void ragged_move_kernel(float* const* __restrict__ src,
+__global__ __launch_bounds__(kThreads) void ragged_move_kernel(int num_seqs, float* const* __restrict__ src,
                                                                float* const* __restrict__ trg,
                                                                const size_t* __restrict__ len) {
-  const unsigned s = blockIdx.y;
+  for (unsigned s = blockIdx.y; s < unsigned(num_seqs); s += gridDim.y) {
   const float* ps = src[s];
   float* pt = trg[s];
   const size_t n = len[s];
@@ -78,6 +81,7 @@ __global__ __launch_bounds__(kThreads) void ragged_move_kernel(float* const* __r
       else
         pt[i] = ps[i];
     }
+  }
   }
 }
 
@@ -143,11 +147,10 @@ int dyhip_sparse_to_dense_block_assign_and_multiply(dyhip_device* dev, int n, co
   DYHIP_CHECK_DEV(dev);
   if (n <= 0 || bsize <= 0) return DYHIP_OK;
   DYHIP_REQUIRE(idx && src && trg, "null pointer");
-  DYHIP_REQUIRE(n <= 65535, "at most 65535 blocks per call (got %d)", n);
   unsigned gx = grid1d(bsize);
   if (gx > 64) gx = 64;
-  hipLaunchKernelGGL(s2d_block_assign_mul_kernel, dim3(gx, n), dim3(kThreads), 0, dev->stream, bsize, idx, mult, src,
-                     trg);
+  hipLaunchKernelGGL(s2d_block_assign_mul_kernel, dim3(gx, n < 65535 ? n : 65535), dim3(kThreads), 0, dev->stream, n,
+                     bsize, idx, mult, src, trg);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
@@ -157,10 +160,10 @@ int dyhip_dense_to_sparse_block_add(dyhip_device* dev, int n, const unsigned* id
   DYHIP_CHECK_DEV(dev);
   if (n <= 0 || bsize <= 0) return DYHIP_OK;
   DYHIP_REQUIRE(ids && src && trg, "null pointer");
-  DYHIP_REQUIRE(n <= 65535, "at most 65535 blocks per call (got %d)", n);
   unsigned gx = grid1d(bsize);
   if (gx > 64) gx = 64;
-  hipLaunchKernelGGL(d2s_block_add_kernel, dim3(gx, n), dim3(kThreads), 0, dev->stream, bsize, ids, src, trg);
+  hipLaunchKernelGGL(d2s_block_add_kernel, dim3(gx, n < 65535 ? n : 65535), dim3(kThreads), 0, dev->stream, n, bsize, ids,
+                     src, trg);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
@@ -169,14 +172,15 @@ static int ragged_move(dyhip_device* dev, bool acc, int num_seqs, int max_len, f
   DYHIP_CHECK_DEV(dev);
   if (num_seqs <= 0 || max_len <= 0) return DYHIP_OK;
   DYHIP_REQUIRE(src && trg && len, "null pointer");
-  DYHIP_REQUIRE(num_seqs <= 65535, "at most 65535 sequences per call (got %d)", num_seqs);
   unsigned gx = static_cast<unsigned>((size_t(max_len) + size_t(kThreads) * 4 - 1) / (size_t(kThreads) * 4));
   if (gx < 1) gx = 1;
   if (gx > 256) gx = 256;
   if (acc)
-    hipLaunchKernelGGL(ragged_move_kernel<true>, dim3(gx, num_seqs), dim3(kThreads), 0, dev->stream, src, trg, len);
+    hipLaunchKernelGGL(ragged_move_kernel<true>, dim3(gx, num_seqs < 65535 ? num_seqs : 65535), dim3(kThreads), 0,
+                       dev->stream, num_seqs, src, trg, len);
   else
-    hipLaunchKernelGGL(ragged_move_kernel<false>, dim3(gx, num_seqs), dim3(kThreads), 0, dev->stream, src, trg, len);
+    hipLaunchKernelGGL(ragged_move_kernel<false>, dim3(gx, num_seqs < 65535 ? num_seqs : 65535), dim3(kThreads), 0,
+                       dev->stream, num_seqs, src, trg, len);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }

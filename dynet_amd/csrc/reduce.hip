@@ -291,11 +291,12 @@ __global__ __launch_bounds__(256) void moment_fwd_kernel(size_t n, const float* 
 }
 
 // dx[b, j] += dEdf[b] / n
-__global__ __launch_bounds__(256) void mean_bwd_kernel(size_t n, const float* __restrict__ dEdf,
+__global__ __launch_bounds__(256) void mean_bwd_kernel(size_t n, unsigned bd, const float* __restrict__ dEdf,
                                                        float* __restrict__ dEdx) {
-  const float d = dEdf[blockIdx.y] / float(n);
   const size_t j = size_t(blockIdx.x) * 256 + threadIdx.x;
-  if (j < n) dEdx[size_t(blockIdx.y) * n + j] += d;
+  if (j >= n) return;
+  for (unsigned b = blockIdx.y; b < bd; b += gridDim.y)  // the grid's second dimension holds at most 65535 blocks
+    dEdx[size_t(b) * n + j] += dEdf[b] / float(n);
 }
 
 // dx[b, j] += (2/n) * (x - mean_b) * (dEdf[b] / (2 * fx[b]))
@@ -368,6 +369,67 @@ __global__ __launch_bounds__(64 * kLnWavesFwd) void ln_fwd_wave_kernel(unsigned 
 #pragma unroll
   for (int u = 0; u < VPL; ++u) {
     const unsigned idx = lane + 64 * u;
+    if (idx < n4) {
+      const float4 gg = g[idx], bb = b[idx];
+      float4 r;
+      r.x = gg.x * ((v[u].x + neg) * sden) + bb.x;
+      r.y = gg.y * ((v[u].y + neg) * sden) + bb.y;
+      r.z = gg.z * ((v[u].z + neg) * sden) + bb.z;
+      r.w = gg.w * ((v[u].w + neg) * sden) + bb.w;
+      stg4<NT>(py + idx, r);
+    }
+  }
+}
+
+// Rows of 2052..16384 floats: a team of WPT waves holds one row in registers (four float4 per thread) and
+// reduces through LDS, one barrier per reduction (each reduction has its own slots).
+constexpr int kLnTeamVpt = 4;
+
+template <int WPT>
+__device__ __forceinline__ float team_sum(float v, float* slot, int w, int team) {
+  v = wave_sum(v);
+  if ((threadIdx.x & 63) == 0) slot[w] = v;
+  __syncthreads();
+  float t = slot[team * WPT];
+#pragma unroll
+  for (int k = 1; k < WPT; ++k) t += slot[team * WPT + k];
+  return t;
+}
+
+template <int WPT, bool NT>
+__global__ __launch_bounds__(64 * WPT) void ln_fwd_team_kernel(unsigned n4, const float4* __restrict__ x,
+                                                               const float4* __restrict__ g,
+                                                               const float4* __restrict__ b, float4* __restrict__ y) {
+  __shared__ float red[2][16];
+  constexpr int TEAM = 64 * WPT;
+  const int w = threadIdx.x >> 6;
+  const float fn = float(n4 * 4);
+  const float4* px = x + size_t(blockIdx.x) * n4;
+  float4 v[kLnTeamVpt];
+#pragma unroll
+  for (int u = 0; u < kLnTeamVpt; ++u) {
+    const unsigned idx = threadIdx.x + TEAM * u;
+    v[u] = idx < n4 ? ldg4<NT>(px + idx) : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int u = 0; u < kLnTeamVpt; ++u) s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+  const float mean = team_sum<WPT>(s, red[0], w, 0) / fn;
+  float ss = 0.f;
+#pragma unroll
+  for (int u = 0; u < kLnTeamVpt; ++u) {
+    if (threadIdx.x + TEAM * u < n4) {
+      const float dx = v[u].x - mean, dy = v[u].y - mean, dz = v[u].z - mean, dw = v[u].w - mean;
+      ss += (dx * dx + dy * dy) + (dz * dz + dw * dw);
+    }
+  }
+  const float sigma = sqrtf(team_sum<WPT>(ss, red[1], w, 0) / fn);
+  const float sden = 1.0f / (kLnEps + sigma);
+  const float neg = -mean;
+  float4* py = y + size_t(blockIdx.x) * n4;
+#pragma unroll
+  for (int u = 0; u < kLnTeamVpt; ++u) {
+    const unsigned idx = threadIdx.x + TEAM * u;
     if (idx < n4) {
       const float4 gg = g[idx], bb = b[idx];
       float4 r;
@@ -550,6 +612,154 @@ __global__ __launch_bounds__(64 * WAVES) void ln_bwd_wave_kernel(unsigned n4, un
   }
 }
 
+// Backward for rows of 2052..16384 floats: a 1024-thread block is 16/WPT teams of WPT waves; a team owns rows
+// blockIdx.x*T + team, + gridDim.x*T, ... and keeps its dg / db partial sums in registers.  All teams of a block
+// run the same number of iterations (rows past the end are all-zero rows that store nothing), so the barriers of
+// the team reductions match.  At the end the teams are added in ascending order through LDS ([which][team][n]);
+// the block's partial rows go to the workspace.
+template <int WPT, bool NT>
+__global__ __launch_bounds__(1024) void ln_bwd_team_kernel(unsigned n4, unsigned bd, const float4* __restrict__ x,
+                                                           const float4* __restrict__ g,
+                                                           const float4* __restrict__ dEdf, float4* __restrict__ dx,
+                                                           float* __restrict__ part_dg, float* __restrict__ part_db) {
+  extern __shared__ float lds[];
+  __shared__ float red[4][16];
+  constexpr int T = 16 / WPT, TEAM = 64 * WPT, VPT = kLnTeamVpt;
+  const int w = threadIdx.x >> 6, team = w / WPT, tl = threadIdx.x - team * TEAM;
+  const float fn = float(n4 * 4);
+  const bool want_g = part_dg != nullptr, want_b = part_db != nullptr;
+  float4 gg[VPT], pdg[VPT], pdb[VPT];
+#pragma unroll
+  for (int u = 0; u < VPT; ++u) {
+    const unsigned idx = tl + TEAM * u;
+    gg[u] = idx < n4 ? g[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+    pdg[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    pdb[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  for (unsigned base = blockIdx.x * T; base < bd; base += gridDim.x * T) {
+    const unsigned row = base + team;
+    const bool live = row < bd;
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 v[VPT], d[VPT], o[VPT];
+#pragma unroll
+    for (int u = 0; u < VPT; ++u) {
+      const unsigned idx = tl + TEAM * u;
+      const bool in = live && idx < n4;
+      v[u] = in ? ldg4<NT>(x + size_t(row) * n4 + idx) : zero;
+      d[u] = in ? ldg4<NT>(dEdf + size_t(row) * n4 + idx) : zero;
+      if (dx != nullptr) o[u] = in ? ldg4<NT>(dx + size_t(row) * n4 + idx) : zero;
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int u = 0; u < VPT; ++u) s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+    const float mean = team_sum<WPT>(s, red[0], w, team) / fn;
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < VPT; ++u) {
+      if (tl + TEAM * u < n4) {
+        const float ax = v[u].x - mean, ay = v[u].y - mean, az = v[u].z - mean, aw = v[u].w - mean;
+        ss += (ax * ax + ay * ay) + (az * az + aw * aw);
+      }
+    }
+    const float sigma = sqrtf(team_sum<WPT>(ss, red[1], w, team) / fn);
+    const float rs = 1.0f / (kLnEps + sigma);
+    const float neg = -mean;
+    float sxq = 0.f, sq = 0.f;
+#pragma unroll
+    for (int u = 0; u < VPT; ++u) {
+      if (live && tl + TEAM * u < n4) {
+#define DYHIP_LN_ROW(c)                                        \
+  {                                                            \
+    const float xc = v[u].c + neg;                             \
+    const float dq = d[u].c * gg[u].c;                         \
+    sxq = fmaf(dq, xc, sxq);                                   \
+    sq += dq;                                                  \
+    if (want_g) pdg[u].c = fmaf(d[u].c, xc * rs, pdg[u].c);    \
+    if (want_b) pdb[u].c += d[u].c;                            \
+  }
+        DYHIP_F4_EACH(DYHIP_LN_ROW)
+#undef DYHIP_LN_ROW
+      }
+    }
+    if (dx != nullptr) {
+      // both row sums cross the team behind one barrier
+      sxq = wave_sum(sxq);
+      sq = wave_sum(sq);
+      if ((threadIdx.x & 63) == 0) {
+        red[2][w] = sxq;
+        red[3][w] = sq;
+      }
+      __syncthreads();
+      float txq = red[2][team * WPT], tq = red[3][team * WPT];
+#pragma unroll
+      for (int k = 1; k < WPT; ++k) {
+        txq += red[2][team * WPT + k];
+        tq += red[3][team * WPT + k];
+      }
+      const float ds = -(txq * rs) * rs;
+      const float dmu = -(tq * rs);
+      const float sb = ds / (2.f * sigma);
+      const float c = 2.f / fn;
+      const float dmu_n = dmu / fn;
+#pragma unroll
+      for (int u = 0; u < VPT; ++u) {
+        const unsigned idx = tl + TEAM * u;
+        if (live && idx < n4) {
+          float4 r = o[u];
+#define DYHIP_LN_DX(c_)                           \
+  {                                               \
+    float acc = r.c_;                             \
+    acc += c * (v[u].c_ - mean) * sb;             \
+    acc += (d[u].c_ * gg[u].c_) * rs;             \
+    acc += dmu_n;                                 \
+    r.c_ = acc;                                   \
+  }
+          DYHIP_F4_EACH(DYHIP_LN_DX)
+#undef DYHIP_LN_DX
+          stg4<NT>(dx + size_t(row) * n4 + idx, r);
+        }
+      }
+    }
+  }
+  if (!want_g && !want_b) return;
+  const unsigned n = n4 * 4;
+  if (T == 1) {
+#pragma unroll
+    for (int u = 0; u < VPT; ++u) {
+      const unsigned idx = tl + TEAM * u;
+      if (idx < n4) {
+        if (want_g) reinterpret_cast<float4*>(part_dg + size_t(blockIdx.x) * n)[idx] = pdg[u];
+        if (want_b) reinterpret_cast<float4*>(part_db + size_t(blockIdx.x) * n)[idx] = pdb[u];
+      }
+    }
+    return;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < VPT; ++u) {
+    const unsigned idx = tl + TEAM * u;
+    if (idx < n4) {
+      if (want_g) reinterpret_cast<float4*>(lds + size_t(team) * n)[idx] = pdg[u];
+      if (want_b) reinterpret_cast<float4*>(lds + size_t(T + team) * n)[idx] = pdb[u];
+    }
+  }
+  __syncthreads();
+  for (unsigned j4 = threadIdx.x; j4 < 2 * n4; j4 += 1024) {
+    const unsigned which = j4 >= n4 ? 1u : 0u;
+    float* part = which == 0 ? part_dg : part_db;
+    if (part == nullptr) continue;
+    const unsigned c4 = j4 - which * n4;
+    const float4* src = reinterpret_cast<const float4*>(lds + size_t(which) * T * n) + c4;
+    float4 t = src[0];
+#pragma unroll
+    for (int k = 1; k < T; ++k) {
+      const float4 a = src[size_t(k) * n4];
+      t.x += a.x; t.y += a.y; t.z += a.z; t.w += a.w;
+    }
+    reinterpret_cast<float4*>(part + size_t(blockIdx.x) * n)[c4] = t;
+  }
+}
+
 // generic fallback, pass 1: per-row statistics and the dx update.
 // stats[row] = {mean, sden}
 __global__ __launch_bounds__(256) void ln_bwd_block_kernel(size_t n, const float* __restrict__ x,
@@ -591,31 +801,88 @@ __global__ __launch_bounds__(256) void ln_bwd_block_kernel(size_t n, const float
   }
 }
 
-// generic fallback, pass 2: dg[j] += sum_b dy*(x-mean_b)/sden_b ; db[j] += sum_b dy
-__global__ __launch_bounds__(256) void ln_bwd_cols_kernel(size_t n, unsigned bd, const float* __restrict__ x,
-                                                          const float* __restrict__ dEdf,
-                                                          const float2* __restrict__ stats, float* __restrict__ dg,
-                                                          float* __restrict__ db) {
-  const size_t j = size_t(blockIdx.x) * 256 + threadIdx.x;
-  if (j >= n) return;
+// generic fallback, pass 2: dg[j] += sum_b dy*(x-mean_b)/sden_b ; db[j] += sum_b dy.
+// Row-parallel like batch_reduce_kernel: a block is 64 column lanes x 16 waves, wave w of split s walks rows
+// s*per_split + w, + 16, ... with four rows in flight; waves are combined through LDS in ascending order and the
+// block's partial rows go to the workspace, where combine_partials adds the splits in ascending order.
+constexpr int kLnColsWaves = 16;
+__global__ __launch_bounds__(64 * kLnColsWaves) void ln_bwd_cols_kernel(size_t n, unsigned bd, unsigned per_split,
+                                                                       const float* __restrict__ x,
+                                                                       const float* __restrict__ dEdf,
+                                                                       const float2* __restrict__ stats,
+                                                                       float* __restrict__ part_dg,
+                                                                       float* __restrict__ part_db) {
+  __shared__ float lds[2][kLnColsWaves][64];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const size_t j = size_t(blockIdx.x) * 64 + lane;
+  const unsigned b0 = blockIdx.y * per_split, b1 = min(bd, b0 + per_split);
   float sg = 0.f, sb = 0.f;
-  for (unsigned r = 0; r < bd; ++r) {
-    const float2 st = stats[r];
-    const float d = dEdf[size_t(r) * n + j];
-    sg += d * ((x[size_t(r) * n + j] - st.x) / st.y);
-    sb += d;
+  if (j < n) {
+    constexpr int U = 4;
+    unsigned r = b0 + w;
+    for (; r + (U - 1) * kLnColsWaves < b1; r += U * kLnColsWaves) {
+      float xv[U], dv[U];
+      float2 st[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const unsigned rr = r + u * kLnColsWaves;
+        xv[u] = x[size_t(rr) * n + j];
+        dv[u] = dEdf[size_t(rr) * n + j];
+        st[u] = stats[rr];
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        sg += dv[u] * ((xv[u] - st[u].x) / st[u].y);
+        sb += dv[u];
+      }
+    }
+    for (; r < b1; r += kLnColsWaves) {
+      const float2 st = stats[r];
+      const float d = dEdf[size_t(r) * n + j];
+      sg += d * ((x[size_t(r) * n + j] - st.x) / st.y);
+      sb += d;
+    }
   }
-  if (dg) dg[j] += sg;
-  if (db) db[j] += sb;
+  lds[0][w][lane] = sg;
+  lds[1][w][lane] = sb;
+  __syncthreads();
+  if (w < 2 && j < n) {
+    float t = lds[w][0][lane];
+#pragma unroll
+    for (int k = 1; k < kLnColsWaves; ++k) t += lds[w][k][lane];
+    float* part = w == 0 ? part_dg : part_db;
+    if (part) part[size_t(blockIdx.y) * n + j] = t;
+  }
 }
+
+static unsigned ln_cols_splits(size_t n, unsigned bd) {
+  const unsigned tiles = static_cast<unsigned>(cdiv<size_t>(n, 64));
+  unsigned want = tiles >= 512 ? 1u : cdiv<unsigned>(512u, tiles);
+  const unsigned max_by_work = cdiv<unsigned>(bd, 2 * kLnColsWaves);
+  if (want > max_by_work) want = max_by_work;
+  if (want > 64) want = 64;
+  if (want < 1) want = 1;
+  return cdiv<unsigned>(bd, cdiv<unsigned>(bd, want));
+}
+
+static size_t ln_stats_bytes(unsigned bd) { return cdiv<size_t>(size_t(bd) * sizeof(float2), 256) * 256; }
 
 static bool ln_fast_ok(size_t n, const void* a, const void* b, const void* c, const void* d) {
   return n % 4 == 0 && n <= 2048 && aligned16(a) && aligned16(b) && (c == nullptr || aligned16(c)) &&
          (d == nullptr || aligned16(d));
 }
 
-static unsigned ln_bwd_blocks(unsigned bd) {
-  unsigned blocks = cdiv<unsigned>(bd, kLnWavesBwd);
+static bool ln_team_ok(size_t n, const void* a, const void* b, const void* c, const void* d) {
+  return n % 4 == 0 && n > 2048 && n <= 16384 && aligned16(a) && aligned16(b) && (c == nullptr || aligned16(c)) &&
+         (d == nullptr || aligned16(d));
+}
+
+// waves per team of the wide-row kernels: the team's 64*WPT threads hold 16 floats each
+static int ln_team_waves(size_t n) { return n <= 4096 ? 4 : n <= 8192 ? 8 : 16; }
+
+static unsigned ln_bwd_blocks(size_t n, unsigned bd) {
+  const unsigned per_block = n <= 2048 ? unsigned(kLnWavesBwd) : unsigned(16 / ln_team_waves(n));
+  unsigned blocks = cdiv<unsigned>(bd, per_block);
   return blocks > kLnBwdMaxBlocks ? kLnBwdMaxBlocks : blocks;
 }
 
@@ -683,9 +950,8 @@ int dyhip_mean_elems_backward(dyhip_device* dev, size_t n, unsigned bd, const fl
   DYHIP_CHECK_DEV(dev);
   DYHIP_REQUIRE(n >= 1 && dEdf && dEdx, "mean_elems needs a non-empty tensor");
   if (bd == 0) return DYHIP_OK;
-  DYHIP_REQUIRE(bd <= 65535, "mean_elems backward supports at most 65535 batch elements");
-  hipLaunchKernelGGL(mean_bwd_kernel, dim3((unsigned)cdiv<size_t>(n, 256), bd), dim3(256), 0, dev->stream, n, dEdf,
-                     dEdx);
+  hipLaunchKernelGGL(mean_bwd_kernel, dim3((unsigned)cdiv<size_t>(n, 256), bd < 65535u ? bd : 65535u), dim3(256), 0,
+                     dev->stream, n, bd, dEdf, dEdx);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
@@ -722,6 +988,23 @@ int dyhip_layer_norm_forward(dyhip_device* dev, size_t n, unsigned bd, const flo
     else if (n4 <= 256) DYHIP_LN_FWD(4);
     else DYHIP_LN_FWD(8);
 #undef DYHIP_LN_FWD
+  } else if (ln_team_ok(n, x, g, b, y)) {
+    const unsigned n4 = static_cast<unsigned>(n / 4);
+    const float4 *x4 = reinterpret_cast<const float4*>(x), *g4 = reinterpret_cast<const float4*>(g),
+                 *b4 = reinterpret_cast<const float4*>(b);
+    float4* y4 = reinterpret_cast<float4*>(y);
+    const bool stream = n * size_t(bd) * sizeof(float) >= dev->stream_threshold;
+#define DYHIP_LN_FWD(WPT)                                                                                         \
+  do {                                                                                                            \
+    if (stream) hipLaunchKernelGGL((ln_fwd_team_kernel<WPT, true>), dim3(bd), dim3(64 * WPT), 0, dev->stream, n4, x4, g4, b4, y4); \
+    else hipLaunchKernelGGL((ln_fwd_team_kernel<WPT, false>), dim3(bd), dim3(64 * WPT), 0, dev->stream, n4, x4, g4, b4, y4);       \
+  } while (0)
+    switch (ln_team_waves(n)) {
+      case 4: DYHIP_LN_FWD(4); break;
+      case 8: DYHIP_LN_FWD(8); break;
+      default: DYHIP_LN_FWD(16); break;
+    }
+#undef DYHIP_LN_FWD
   } else {
     hipLaunchKernelGGL(ln_fwd_block_kernel, dim3(bd), dim3(256), 0, dev->stream, n, x, g, b, y);
   }
@@ -731,8 +1014,9 @@ int dyhip_layer_norm_forward(dyhip_device* dev, size_t n, unsigned bd, const flo
 
 int dyhip_layer_norm_backward_workspace(size_t n, unsigned bd, size_t* ws_bytes) {
   DYHIP_REQUIRE(ws_bytes != nullptr, "null output pointer");
-  const size_t fast = size_t(2) * ln_bwd_blocks(bd) * n * sizeof(float);
-  const size_t generic = size_t(bd) * sizeof(float2);
+  const size_t fast = n <= 16384 ? size_t(2) * ln_bwd_blocks(n, bd) * n * sizeof(float) : 0;
+  // generic path: per-row statistics, then one partial row per output and batch split
+  const size_t generic = ln_stats_bytes(bd) + size_t(2) * ln_cols_splits(n, bd ? bd : 1) * n * sizeof(float);
   *ws_bytes = fast > generic ? fast : generic;
   return DYHIP_OK;
 }
@@ -762,7 +1046,7 @@ int dyhip_layer_norm_backward(dyhip_device* dev, size_t n, unsigned bd, const fl
                 need, ws_bytes);
   if (ln_fast_ok(n, x, g, dEdf, dx)) {
     const unsigned n4 = static_cast<unsigned>(n / 4);
-    const unsigned blocks = ln_bwd_blocks(bd);
+    const unsigned blocks = ln_bwd_blocks(n, bd);
     float* part_dg = dg ? static_cast<float*>(ws) : nullptr;
     float* part_db = db ? static_cast<float*>(ws) + size_t(blocks) * n : nullptr;
     const size_t lds = cols ? size_t(2) * kLnWavesBwd * n * sizeof(float) : 0;  // [dg | db][wave][n]
@@ -798,13 +1082,59 @@ int dyhip_layer_norm_backward(dyhip_device* dev, size_t n, unsigned bd, const fl
     else if (dg) launch_combine(dev, n, blocks, part_dg, dg, nullptr, nullptr, 1);
     else if (db) launch_combine(dev, n, blocks, part_db, db, nullptr, nullptr, 1);
     DYHIP_CHECK_LAUNCH();
+  } else if (ln_team_ok(n, x, g, dEdf, dx)) {
+    const unsigned n4 = static_cast<unsigned>(n / 4);
+    const unsigned blocks = ln_bwd_blocks(n, bd);
+    const int wpt = ln_team_waves(n), teams = 16 / wpt;
+    float* part_dg = dg ? static_cast<float*>(ws) : nullptr;
+    float* part_db = db ? static_cast<float*>(ws) + size_t(blocks) * n : nullptr;
+    const size_t lds = cols && teams > 1 ? size_t(2) * teams * n * sizeof(float) : 0;  // [dg | db][team][n], <= 128 KB
+    const float4 *x4 = reinterpret_cast<const float4*>(x), *g4 = reinterpret_cast<const float4*>(g),
+                 *d4 = reinterpret_cast<const float4*>(dEdf);
+    float4* dx4 = reinterpret_cast<float4*>(dx);
+    const bool stream = n * size_t(bd) * sizeof(float) >= dev->stream_threshold;
+#define DYHIP_LN_BWD(WPT)                                                                                       \
+  do {                                                                                                          \
+    static bool big_lds_ok = false;                                                                             \
+    if (lds > (size_t(64) << 10) && !big_lds_ok) {                                                               \
+      DYHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&ln_bwd_team_kernel<WPT, true>),        \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 128 << 10));               \
+      DYHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&ln_bwd_team_kernel<WPT, false>),       \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 128 << 10));               \
+      big_lds_ok = true;                                                                                        \
+    }                                                                                                           \
+    if (stream)                                                                                                 \
+      hipLaunchKernelGGL((ln_bwd_team_kernel<WPT, true>), dim3(blocks), dim3(1024), lds, dev->stream, n4, bd, x4, g4, \
+                         d4, dx4, part_dg, part_db);                                                            \
+    else                                                                                                        \
+      hipLaunchKernelGGL((ln_bwd_team_kernel<WPT, false>), dim3(blocks), dim3(1024), lds, dev->stream, n4, bd, x4, g4, \
+                         d4, dx4, part_dg, part_db);                                                            \
+  } while (0)
+    switch (wpt) {
+      case 4: DYHIP_LN_BWD(4); break;
+      case 8: DYHIP_LN_BWD(8); break;
+      default: DYHIP_LN_BWD(16); break;
+    }
+#undef DYHIP_LN_BWD
+    DYHIP_CHECK_LAUNCH();
+    if (dg && db) launch_combine(dev, n, blocks, part_dg, dg, part_db, db, 1);
+    else if (dg) launch_combine(dev, n, blocks, part_dg, dg, nullptr, nullptr, 1);
+    else if (db) launch_combine(dev, n, blocks, part_db, db, nullptr, nullptr, 1);
+    DYHIP_CHECK_LAUNCH();
   } else {
     float2* stats = cols ? static_cast<float2*>(ws) : nullptr;
     hipLaunchKernelGGL(ln_bwd_block_kernel, dim3(bd), dim3(256), 0, dev->stream, n, x, g, dEdf, dx, stats);
     DYHIP_CHECK_LAUNCH();
     if (cols) {
-      hipLaunchKernelGGL(ln_bwd_cols_kernel, dim3((unsigned)cdiv<size_t>(n, 256)), dim3(256), 0, dev->stream, n, bd, x,
-                         dEdf, stats, dg, db);
+      const unsigned splits = ln_cols_splits(n, bd), per_split = cdiv<unsigned>(bd, splits);
+      float* part_dg = reinterpret_cast<float*>(static_cast<char*>(ws) + ln_stats_bytes(bd));
+      float* part_db = part_dg + size_t(splits) * n;
+      hipLaunchKernelGGL(ln_bwd_cols_kernel, dim3((unsigned)cdiv<size_t>(n, 64), splits), dim3(64 * kLnColsWaves), 0,
+                         dev->stream, n, bd, per_split, x, dEdf, stats, dg ? part_dg : nullptr, db ? part_db : nullptr);
+      DYHIP_CHECK_LAUNCH();
+      if (dg && db) launch_combine(dev, n, splits, part_dg, dg, part_db, db, 1);
+      else if (dg) launch_combine(dev, n, splits, part_dg, dg, nullptr, nullptr, 1);
+      else launch_combine(dev, n, splits, part_db, db, nullptr, nullptr, 1);
       DYHIP_CHECK_LAUNCH();
     }
   }

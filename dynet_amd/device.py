@@ -306,6 +306,30 @@ class Device:
         _check(cdll.dyhip_layer_norm_backward(self.handle, _sz(n), _u(bd), _p(x), _p(g), _p(dEdf), _p(dx), _p(dg),
                                               _p(db), _vp(ws), _sz(ws_bytes)))
 
+    # ---- cwise ops with dimension broadcast ---------------------------------------
+    @staticmethod
+    def _dims5(d):
+        d = list(d) + [1] * (5 - len(d))
+        return (C.c_uint * 5)(*d)
+
+    def cwise_forward(self, op, dims_a, dims_b, a, b, fx):
+        """dims: (d0, d1, d2, d3, bd), column-major with the batch outermost (numpy shape = reversed dims)."""
+        _check(cdll.dyhip_cwise_forward(self.handle, _i(op), self._dims5(dims_a), self._dims5(dims_b), _p(a), _p(b), _p(fx)))
+
+    def cwise_backward(self, op, dims_a, dims_b, a, b, dEdf, i, dEdxi):
+        nb = _sz(0)
+        da, db = self._dims5(dims_a), self._dims5(dims_b)
+        _check(cdll.dyhip_cwise_backward_workspace(da, db, _u(i), C.byref(nb)))
+        ws, nbytes = self.workspace(nb.value)
+        _check(cdll.dyhip_cwise_backward(self.handle, _i(op), da, db, _p(a), _p(b), _p(dEdf), _u(i), _p(dEdxi), _vp(ws),
+                                         _sz(nbytes)))
+
+    def const_plus_x_forward(self, c, x, fx):
+        _check(cdll.dyhip_const_plus_x_forward(self.handle, _sz(x.size), C.c_float(c), _p(x), _p(fx)))
+
+    def const_minus_x_forward(self, c, x, fx):
+        _check(cdll.dyhip_const_minus_x_forward(self.handle, _sz(x.size), C.c_float(c), _p(x), _p(fx)))
+
     def layer_norm_backward_static(self, n, bd, x, g, dEdf, dx=None, dg=None, db=None):
         """No workspace argument and no allocation: the scratch is a static device array of the library."""
         _check(cdll.dyhip_layer_norm_backward_static(self.handle, _sz(n), _u(bd), _p(x), _p(g), _p(dEdf), _p(dx),

@@ -14,6 +14,7 @@ POOL_FXS, POOL_DEDFS, POOL_PS, POOL_SCS = range(4)
 SCALAR_MINUSONE, SCALAR_ONE, SCALAR_ZERO = range(3)
 OP_TANH, OP_LOGISTIC, OP_RECTIFY, OP_NEGATE, OP_IDENTITY = range(5)
 LOGISTIC_PACKET, LOGISTIC_SCALAR = 0, 1
+CWISE_SUM, CWISE_MULT, CWISE_QUOTIENT = range(3)
 LN_STATIC_SCRATCH_BYTES = 4 << 20  # DYHIP_LN_STATIC_SCRATCH_BYTES
 
 

@@ -169,6 +169,27 @@ int dyhip_sum_forward(dyhip_device* dev, unsigned k, size_t n, unsigned bd, cons
 /* workspace for every batch reduction of an n x bd tensor (sum_batches fwd,
  * the broadcast-argument backward of cmult/csum) */
 int dyhip_batch_reduce_workspace(size_t n, unsigned bd, size_t* ws_bytes);
+/* ---- CwiseSum / CwiseMultiply / CwiseQuotient with broadcast over dimensions as well as the batch
+ * (dynet/nodes-arith-cwise.cc:50-156, :196-307, :338-421, backward_helper included) and the constant
+ * nodes of dynet/nodes-arith-const.cc:33-75.  A tensor is dims[5] = {d0, d1, d2, d3, bd}, column-major,
+ * batch outermost, missing dimensions 1; on every axis the two arguments agree or one of them is 1
+ * (CwiseQuotient: only the right one); the result takes the larger.  backward accumulates into dEdxi
+ * (argument i's own shape), summing over the axes it was broadcast over:
+ *   sum: dEdf    multiply: dEdf * other    quotient: i = 0: dEdf / b, i = 1: -(dEdf / (b*b) * a).
+ * The batch-only cases are the streaming kernels of dyhip_csum_* / dyhip_cmult_*. ------------------- */
+#define DYHIP_CWISE_SUM 0
+#define DYHIP_CWISE_MULT 1
+#define DYHIP_CWISE_QUOTIENT 2
+int dyhip_cwise_forward(dyhip_device* dev, int op, const unsigned* dims_a, const unsigned* dims_b, const float* a,
+                        const float* b, float* fx);
+int dyhip_cwise_backward_workspace(const unsigned* dims_a, const unsigned* dims_b, unsigned i, size_t* ws_bytes);
+int dyhip_cwise_backward(dyhip_device* dev, int op, const unsigned* dims_a, const unsigned* dims_b, const float* a,
+                         const float* b, const float* dEdf, unsigned i, float* dEdxi, void* ws, size_t ws_bytes);
+/* ConstantPlusX: fx = c + x, backward dEdx += dEdf (dyhip_accumulate); ConstantMinusX: fx = c - x, backward
+ * dEdx -= dEdf (dyhip_unary_backward with DYHIP_OP_NEGATE). */
+int dyhip_const_plus_x_forward(dyhip_device* dev, size_t n, float c, const float* x, float* fx);
+int dyhip_const_minus_x_forward(dyhip_device* dev, size_t n, float c, const float* x, float* fx);
+
 /* SumDimension({}, include_batch_dim) = sum_batches (dynet/nodes-arith-sum.cc:197-248, expr.cc:218) */
 int dyhip_sum_batches_forward(dyhip_device* dev, size_t n, unsigned bd, const float* x, float* y, void* ws, size_t ws_bytes);
 int dyhip_sum_batches_backward(dyhip_device* dev, size_t n, unsigned bd, const float* dEdf, float* dEdx);
@@ -193,7 +214,8 @@ int dyhip_layer_norm_backward(dyhip_device* dev, size_t n, unsigned bd, const fl
  * reference (whose nodes take scratch from pools[SCS]).  The scratch is a static device array of
  * DYHIP_LN_STATIC_SCRATCH_BYTES that each GPU holds until the process ends; the call allocates nothing and
  * fails with DYHIP_ERR_INVALID_ARG when dyhip_layer_norm_backward_workspace(n, bd) exceeds that size
- * (n <= 2048 on the fast path: any bd; otherwise bd <= 524288).  All calls on one GPU share the array:
+ * (rows of up to 2048 floats on the fast path: any bd; wider or unaligned rows: 8 bytes per row plus up
+ * to 64 partial rows of dg and db).  All calls on one GPU share the array:
  * calls that overlap on one GPU (two queues, two threads) race; calls on one queue are ordered. */
 #define DYHIP_LN_STATIC_SCRATCH_BYTES (4u << 20)
 int dyhip_layer_norm_backward_static(dyhip_device* dev, size_t n, unsigned bd, const float* x, const float* g,

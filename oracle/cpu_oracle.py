@@ -128,6 +128,43 @@ def csum_backward(n, bd0, bd1, dEdf, i, dEdxi):
     return dEdxi
 
 
+CWISE_SUM, CWISE_MULT, CWISE_QUOTIENT = range(3)
+
+
+def _dims5(d):
+    d = list(d) + [1] * (5 - len(d))
+    return (C.c_uint * 5)(*d)
+
+
+def cwise_forward(op, dims_a, dims_b, a, b):
+    """dims: (d0, d1, d2, d3, bd), column-major with the batch outermost; numpy shape = reversed dims."""
+    a, b = _f32(a), _f32(b)
+    full = [max(x, y) for x, y in zip(dims_a, dims_b)]
+    fx = np.empty(tuple(reversed(full)), np.float32)
+    _check(_lib.orc_cwise_forward(op, _dims5(dims_a), _dims5(dims_b), _fp(a), _fp(b), _fp(fx)), "cwise_forward")
+    return fx
+
+
+def cwise_backward(op, dims_a, dims_b, a, b, dEdf, i, dEdxi):
+    _check(_lib.orc_cwise_backward(op, _dims5(dims_a), _dims5(dims_b), _fp(_f32(a)), _fp(_f32(b)), _fp(_f32(dEdf)), i,
+                                   _fp(dEdxi)), "cwise_backward")
+    return dEdxi
+
+
+def const_plus_x_forward(c, x):
+    x = _f32(x)
+    y = np.empty_like(x)
+    _check(_lib.orc_const_plus_x_forward(C.c_size_t(x.size), C.c_float(c), _fp(x), _fp(y)), "const_plus_x")
+    return y
+
+
+def const_minus_x_forward(c, x):
+    x = _f32(x)
+    y = np.empty_like(x)
+    _check(_lib.orc_const_minus_x_forward(C.c_size_t(x.size), C.c_float(c), _fp(x), _fp(y)), "const_minus_x")
+    return y
+
+
 # ---- reductions ------------------------------------------------------------
 def sum_batches_forward(n, bd, x):
     x = _f32(x)

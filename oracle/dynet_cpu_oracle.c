@@ -198,6 +198,108 @@ int orc_csum_backward(size_t n, unsigned bd0, unsigned bd1, const float* dEdf, u
   return 0;
 }
 
+/* ---- CwiseSum / CwiseMultiply / CwiseQuotient with broadcast over dimensions and batch --------------
+ * dynet/nodes-arith-cwise.cc: forward :50-97 (sum), :196-243 (multiply), :338-351 (quotient); backward
+ * :99-156, :245-307, :353-421.  A tensor is given by dims[5] = {d0, d1, d2, d3, bd} (column-major, batch
+ * outermost; missing dimensions are 1).  For every axis the two arguments agree or one of them is 1
+ * (CwiseQuotient: only the right one may be 1, :320-325); the output takes the larger.
+ * Forward: fx[e] = a[bcast e] op b[bcast e].
+ * Backward of argument i: dEdxi[o] (+/-)= sum over the axes where argument i is 1 and the output is not of
+ *   sum:       dEdf                                  (:141-156, Eigen .sum(red_axis))
+ *   multiply:  dEdf * other                          (:284-307)
+ *   quotient:  i = 0: dEdf / b                       (:363-374, no axis is ever reduced)
+ *              i = 1: -(dEdf / (b*b) * a)            (:376-421; b squared first, as the reference does)
+ * summed here sequentially in the order of the output's linear index (parity unpinned at the Eigen boundary
+ * for the order of a reduction).  Pinned in tests/test_oracle.py by numpy broadcasting in fp64, by central
+ * differences, and by the batch-only cases agreeing with orc_csum_* / orc_cmult_*. */
+static int cw_dims_ok(const unsigned* da, const unsigned* db, int quotient) {
+  for (int j = 0; j < 5; ++j) {
+    if (da[j] == 0 || db[j] == 0) return 0;
+    if (da[j] != db[j] && da[j] != 1 && db[j] != 1) return 0;
+    if (quotient && da[j] != db[j] && db[j] != 1) return 0;
+  }
+  return 1;
+}
+
+static size_t cw_offset(const unsigned* idx, const unsigned* dims) {
+  size_t off = 0, stride = 1;
+  for (int j = 0; j < 5; ++j) {
+    off += (dims[j] == 1 ? 0 : idx[j]) * stride;
+    stride *= dims[j];
+  }
+  return off;
+}
+
+int orc_cwise_forward(int op, const unsigned* da, const unsigned* db, const float* a, const float* b, float* fx) {
+  if (op < 0 || op > 2 || !cw_dims_ok(da, db, op == 2)) return -1;
+  unsigned df[5], idx[5];
+  for (int j = 0; j < 5; ++j) df[j] = da[j] > db[j] ? da[j] : db[j];
+  size_t e = 0;
+  for (idx[4] = 0; idx[4] < df[4]; ++idx[4])
+    for (idx[3] = 0; idx[3] < df[3]; ++idx[3])
+      for (idx[2] = 0; idx[2] < df[2]; ++idx[2])
+        for (idx[1] = 0; idx[1] < df[1]; ++idx[1])
+          for (idx[0] = 0; idx[0] < df[0]; ++idx[0], ++e) {
+            const float x = a[cw_offset(idx, da)], y = b[cw_offset(idx, db)];
+            fx[e] = op == 0 ? x + y : op == 1 ? x * y : x / y;
+          }
+  return 0;
+}
+
+int orc_cwise_backward(int op, const unsigned* da, const unsigned* db, const float* a, const float* b,
+                       const float* dEdf, unsigned i, float* dEdxi) {
+  if (op < 0 || op > 2 || i > 1 || !cw_dims_ok(da, db, op == 2)) return -1;
+  unsigned df[5], idx[5];
+  for (int j = 0; j < 5; ++j) df[j] = da[j] > db[j] ? da[j] : db[j];
+  const unsigned* di = i == 0 ? da : db;
+  /* the reference forms the reduced tensor first (`.sum(red_axis)`) and then adds it to dEdxi; without a
+   * reduction the terms go straight into dEdxi */
+  int reduces = 0;
+  size_t n_self = 1;
+  for (int j = 0; j < 5; ++j) {
+    reduces |= di[j] == 1 && df[j] > 1;
+    n_self *= di[j];
+  }
+  float* acc = dEdxi;
+  if (reduces) {
+    acc = (float*)calloc(n_self, sizeof(float));
+    if (!acc) return -1;
+  }
+  size_t e = 0;
+  for (idx[4] = 0; idx[4] < df[4]; ++idx[4])
+    for (idx[3] = 0; idx[3] < df[3]; ++idx[3])
+      for (idx[2] = 0; idx[2] < df[2]; ++idx[2])
+        for (idx[1] = 0; idx[1] < df[1]; ++idx[1])
+          for (idx[0] = 0; idx[0] < df[0]; ++idx[0], ++e) {
+            const float x = a[cw_offset(idx, da)], y = b[cw_offset(idx, db)], d = dEdf[e];
+            float* out = acc + cw_offset(idx, di);
+            if (op == 0) *out += d;
+            else if (op == 1) *out += d * (i == 0 ? y : x);
+            else if (i == 0) *out += d / y;
+            else if (reduces) *out += d / (y * y) * x;
+            else *out -= d / (y * y) * x;
+          }
+  if (reduces) {
+    for (size_t j = 0; j < n_self; ++j) {
+      if (op == 2) dEdxi[j] -= acc[j];
+      else dEdxi[j] += acc[j];
+    }
+    free(acc);
+  }
+  return 0;
+}
+
+/* ConstantPlusX / ConstantMinusX, dynet/nodes-arith-const.cc:33-75: fx = c + x (c - x); backward
+ * dEdx += dEdf (-= dEdf). */
+int orc_const_plus_x_forward(size_t n, float c, const float* x, float* fx) {
+  for (size_t j = 0; j < n; ++j) fx[j] = c + x[j];
+  return 0;
+}
+int orc_const_minus_x_forward(size_t n, float c, const float* x, float* fx) {
+  for (size_t j = 0; j < n; ++j) fx[j] = c - x[j];
+  return 0;
+}
+
 /* ======================================================================== */
 /* reductions                                                                */
 /* ======================================================================== */

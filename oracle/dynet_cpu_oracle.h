@@ -65,6 +65,14 @@ int orc_cmult_backward(size_t n, unsigned bd0, unsigned bd1, const float* a, con
 int orc_csum_forward(size_t n, unsigned bd0, unsigned bd1, const float* a, const float* b, float* y);
 int orc_csum_backward(size_t n, unsigned bd0, unsigned bd1, const float* dEdf, unsigned i, float* dEdxi);
 
+/* the same three operators with broadcast over any of {d0, d1, d2, d3, bd}: dims arrays of 5;
+ * op 0 = sum, 1 = multiply, 2 = quotient (only the right argument may be broadcast) */
+int orc_cwise_forward(int op, const unsigned* dims_a, const unsigned* dims_b, const float* a, const float* b, float* fx);
+int orc_cwise_backward(int op, const unsigned* dims_a, const unsigned* dims_b, const float* a, const float* b,
+                       const float* dEdf, unsigned i, float* dEdxi);
+int orc_const_plus_x_forward(size_t n, float c, const float* x, float* fx);
+int orc_const_minus_x_forward(size_t n, float c, const float* x, float* fx);
+
 /* ---- reductions --------------------------------------------------------- */
 int orc_sum_batches_forward(size_t n, unsigned bd, const float* x, float* y);
 int orc_sum_batches_backward(size_t n, unsigned bd, const float* dEdf, float* dEdx);

@@ -212,7 +212,8 @@ def _ln_case(n, bd, seed):
 
 
 @pytest.mark.parametrize("n,bd", [(1024, 4096), (2048, 64), (512, 33), (256, 5), (64, 1), (12, 7), (1027, 9),
-                                  (4096, 6), (3, 1)])
+                                  (4096, 6), (3, 1), (4096, 1024), (4100, 300), (37, 1000), (70, 2051),
+                                  (8192, 70), (16384, 33), (2052, 19), (12288, 5), (16388, 9)])
 def test_layer_norm_forward_backward(dev, n, bd):
     rng, x, g, b, dy = _ln_case(n, bd, 51)
     xt, gt, bt, dyt = dev.tensor(x), dev.tensor(g), dev.tensor(b), dev.tensor(dy)
@@ -235,6 +236,110 @@ def test_layer_norm_forward_backward(dev, n, bd):
     dgt2 = dev.tensor(dg0)
     dev.layer_norm_backward(n, bd, xt, gt, dyt, dg=dgt2)
     assert dgt2.numpy().tobytes() == dgt.numpy().tobytes()
+
+
+CWISE_SHAPES = [
+    # dims_a, dims_b as (d0, d1, d2, d3, bd)
+    ((1024, 1, 1, 1, 4096), (1, 1, 1, 1, 4096)),  # x - mean and x / sigma of the layer_norm composite, baseline shape
+    ((1024, 1, 1, 1, 33), (1, 1, 1, 1, 33)),
+    ((5, 3, 1, 1, 4), (5, 1, 1, 1, 1)),
+    ((5, 3, 1, 1, 4), (1, 3, 1, 1, 4)),
+    ((4, 3, 2, 1, 3), (4, 1, 2, 1, 1)),
+    ((2, 3, 4, 5, 2), (1, 3, 1, 5, 1)),
+    ((128, 70, 1, 1, 9), (128, 1, 1, 1, 1)),      # kept axes are a prefix: the coalesced batch reduction
+    ((64, 100, 1, 1, 3), (1, 100, 1, 1, 3)),      # 64 terms per output: one wavefront each
+    ((7, 1, 1, 1, 3), (7, 1, 1, 1, 3)),           # nothing broadcast
+    ((6, 2, 1, 1, 5), (6, 2, 1, 1, 1)),           # batch only: the streaming kernels
+    ((1023, 3, 1, 1, 2), (1, 3, 1, 1, 1)),        # d0 not a multiple of 4
+]
+
+
+@pytest.mark.parametrize("op", [lib.CWISE_SUM, lib.CWISE_MULT, lib.CWISE_QUOTIENT])
+@pytest.mark.parametrize("da,db", CWISE_SHAPES)
+def test_cwise_with_dimension_broadcast(dev, op, da, db):
+    """CwiseSum / CwiseMultiply / CwiseQuotient with broadcast over dimensions (dynet/nodes-arith-cwise.cc incl. the
+    backward_helper reductions), both argument orders, against the oracle."""
+    from dynet_amd import DyhipError
+
+    rng = np.random.default_rng(sum(da) + 3 * sum(db) + op)
+    for swap in (False, True):
+        d0, d1 = (db, da) if swap else (da, db)
+        if op == lib.CWISE_QUOTIENT and any(x != y and y != 1 for x, y in zip(d0, d1)):
+            t = dev.zeros(4)
+            with pytest.raises(DyhipError) as e:
+                dev.cwise_forward(op, d0, d1, t, t, t)
+            assert e.value.status == lib.ERR_INVALID_ARG and "CwiseQuotient" in str(e.value)
+            continue
+        a = f32(rng.standard_normal(d0[::-1]))
+        b = f32(rng.standard_normal(d1[::-1]))
+        if op == lib.CWISE_QUOTIENT:
+            b = f32(np.sign(b) * (np.abs(b) + 0.5))  # keep the divisor away from zero
+        at, bt = dev.tensor(a), dev.tensor(b)
+        want = orc.cwise_forward(op, d0, d1, a, b)
+        fx = dev.empty(want.shape)
+        dev.cwise_forward(op, d0, d1, at, bt, fx)
+        if op == lib.CWISE_QUOTIENT:
+            assert_close(fx.numpy(), want, FWD_RTOL, "cwise fwd")  # one correctly rounded division each
+        else:
+            assert fx.numpy().tobytes() == want.tobytes()
+        dy = f32(rng.standard_normal(want.shape))
+        dyt = dev.tensor(dy)
+        for i, x in enumerate((a, b)):
+            g0 = f32(rng.standard_normal(x.shape))
+            gt = dev.tensor(g0)
+            dev.cwise_backward(op, d0, d1, at, bt, dyt, i, gt)
+            ref = orc.cwise_backward(op, d0, d1, a, b, dy, i, g0.copy())
+            terms = want.size / x.size  # terms summed into one output element
+            other = np.abs(b if i == 0 else a).max() if op != lib.CWISE_SUM else 1.0
+            if op == lib.CWISE_QUOTIENT:
+                other = (1.0 / np.abs(b).min()) * (1.0 if i == 0 else np.abs(a).max() / np.abs(b).min())
+            assert_close(gt.numpy(), ref, GRAD_RTOL, "cwise bwd op %d arg %d" % (op, i),
+                         floor=np.maximum(np.abs(g0), rms(dy) * other * np.sqrt(terms)))
+
+
+def test_layer_norm_composite_of_eight_nodes_on_the_device(dev):
+    """dynet/expr.cc:248-253 issued node by node through the C-ABI (mean_elems, Negate, CwiseSum, std_elems,
+    ConstantPlusX, CwiseQuotient, CwiseMultiply, CwiseSum; forward and backward) at the baseline's shape, against
+    the fused kernels and against the oracle's layer_norm."""
+    n, bd = 1024, 4096
+    rng, x, g, b, dy = _ln_case(n, bd, 77)
+    X, S, G = (n, 1, 1, 1, bd), (1, 1, 1, 1, bd), (n, 1, 1, 1, 1)
+    xt, gt, bt, dyt = dev.tensor(x), dev.tensor(g), dev.tensor(b), dev.tensor(dy)
+    e = lambda *s: dev.empty(s)
+    z = lambda *s: dev.zeros(s, pool=lib.POOL_DEDFS)
+    mu, neg, xc, sigma, se, q, gq, y = e(bd), e(bd), e(bd, n), e(bd), e(bd), e(bd, n), e(bd, n), e(bd, n)
+    dev.mean_elems_forward(n, bd, xt, mu)
+    dev.unary_forward(lib.OP_NEGATE, mu, neg)
+    dev.cwise_forward(lib.CWISE_SUM, X, S, xt, neg, xc)
+    dev.std_elems_forward(n, bd, xt, sigma)
+    dev.const_plus_x_forward(1e-8, sigma, se)
+    dev.cwise_forward(lib.CWISE_QUOTIENT, X, S, xc, se, q)
+    dev.cwise_forward(lib.CWISE_MULT, G, X, gt, q, gq)
+    dev.cwise_forward(lib.CWISE_SUM, X, G, gq, bt, y)
+    fused = e(bd, n)
+    dev.layer_norm_forward(n, bd, xt, gt, bt, fused)
+    ref = orc.layer_norm_forward(n, bd, x, g, b).reshape(bd, n)
+    assert_close(y.numpy(), ref, FWD_RTOL, "composite fwd vs oracle", floor=1.0)
+    assert_close(y.numpy(), fused.numpy(), FWD_RTOL, "composite fwd vs fused", floor=1.0)
+    # backward, in reverse topological order; every node accumulates into its arguments' gradients
+    d_gq, d_b, d_g, d_q, d_xc, d_se, d_x, d_neg, d_mu = z(bd, n), z(n), z(n), z(bd, n), z(bd, n), z(bd), z(bd, n), z(bd), z(bd)
+    dev.cwise_backward(lib.CWISE_SUM, X, G, gq, bt, dyt, 0, d_gq)
+    dev.cwise_backward(lib.CWISE_SUM, X, G, gq, bt, dyt, 1, d_b)
+    dev.cwise_backward(lib.CWISE_MULT, G, X, gt, q, d_gq, 0, d_g)
+    dev.cwise_backward(lib.CWISE_MULT, G, X, gt, q, d_gq, 1, d_q)
+    dev.cwise_backward(lib.CWISE_QUOTIENT, X, S, xc, se, d_q, 0, d_xc)
+    dev.cwise_backward(lib.CWISE_QUOTIENT, X, S, xc, se, d_q, 1, d_se)
+    dev.std_elems_backward(n, bd, xt, sigma, d_se, d_x)            # ConstantPlusX: d_sigma += d_se, same buffer
+    dev.cwise_backward(lib.CWISE_SUM, X, S, xt, neg, d_xc, 0, d_x)
+    dev.cwise_backward(lib.CWISE_SUM, X, S, xt, neg, d_xc, 1, d_neg)
+    dev.unary_backward(lib.OP_NEGATE, neg, d_neg, d_mu)
+    dev.mean_elems_backward(n, bd, d_mu, d_x)
+    fx_, fg_, fb_ = z(bd, n), z(n), z(n)
+    dev.layer_norm_backward(n, bd, xt, gt, dyt, fx_, fg_, fb_)
+    wx, wg, wb = orc.layer_norm_backward(n, bd, x, g, dy, np.zeros((bd, n), F32), np.zeros(n, F32), np.zeros(n, F32))
+    for got, fusedv, want, fl, what in ((d_x, fx_, wx, 1.0, "dx"), (d_g, fg_, wg, np.sqrt(bd), "dg"), (d_b, fb_, wb, np.sqrt(bd), "db")):
+        assert_close(got.numpy(), want.reshape(got.shape), GRAD_RTOL, "composite %s vs oracle" % what, floor=fl)
+        assert_close(got.numpy(), fusedv.numpy(), GRAD_RTOL, "composite %s vs fused" % what, floor=fl)
 
 
 def test_layer_norm_golden_vectors(dev, golden):

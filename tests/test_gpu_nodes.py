@@ -433,6 +433,50 @@ def test_single_launch_step_rejects_unsupported_sizes(dev):
         dev.lstm_step_forward(96, 4, t, t, t, t, t, t, t, t)
 
 
+def test_more_than_65535_batch_elements(dev):
+    """The grid's second dimension holds 65535 blocks; kernels that put a batch element (or a block / sequence of
+    the gpu-ops helpers) there stride over the rest, as the reference's launches do (dynet/cuda.h:82-103)."""
+    rng = np.random.default_rng(70)
+    B, H = 70000, 4
+    c_prev, gates = f32(rng.standard_normal((B, H))), f32(rng.uniform(0.1, 0.9, (B, 4 * H)))
+    ct, gt = dev.tensor(c_prev), dev.tensor(gates)
+    c2, h2 = dev.empty((B, H)), dev.empty((B, H))
+    dev.lstm_c_forward(H, B, ct, gt, c2)
+    c_ref = orc.lstm_c_forward(H, B, c_prev, gates)
+    assert_close(c2.numpy(), c_ref, FWD_RTOL, "c fwd", floor=1e-3)
+    dev.lstm_h_forward(H, B, dev.tensor(c_ref), gt, h2)
+    assert_close(h2.numpy(), orc.lstm_h_forward(H, B, c_ref, gates), FWD_RTOL, "h fwd", floor=1e-6)
+    dg = f32(rng.standard_normal((B, 4 * H)))
+    dpre = dev.empty((B, 4 * H))
+    dev.lstm_gates_dpre(H, B, gt, dev.tensor(dg), dpre)
+    want = np.where(np.arange(4 * H) < 3 * H, dg * gates * (F32(1) - gates), dg * (F32(1) - gates * gates)).astype(F32)
+    assert_close(dpre.numpy(), want, GRAD_RTOL, "dpre", floor=1e-6)
+    # mean_elems backward over 70000 batch elements
+    d, dx0 = f32(rng.standard_normal(B)), f32(rng.standard_normal((B, 3)))
+    dxt = dev.tensor(dx0)
+    dev.mean_elems_backward(3, B, dev.tensor(d), dxt)
+    assert_close(dxt.numpy(), orc.mean_elems_backward(3, B, d, dx0.copy()), GRAD_RTOL, "mean_elems bwd", floor=1e-3)
+    # block gather / scatter helpers with 70000 blocks
+    table = f32(rng.standard_normal((100, 5)))
+    bidx = rng.integers(0, 100, B).astype(np.uint32)
+    out = dev.empty((B, 5))
+    dev.sparse_to_dense_block_assign_and_multiply(B, dev.tensor(bidx, np.uint32), 5, 2.0, dev.tensor(table), out)
+    want = orc.sparse_to_dense_block_assign_and_multiply(bidx, 5, 2.0, table)
+    assert out.numpy().tobytes() == want.tobytes()
+    acc = dev.zeros((100, 5))
+    dev.dense_to_sparse_block_add(B, dev.tensor(bidx, np.uint32), 5, dev.tensor(want), acc)
+    assert_close(acc.numpy(), orc.dense_to_sparse_block_add(bidx, 5, want, np.zeros((100, 5), F32)), GRAD_RTOL,
+                 "dense_to_sparse_block_add", floor=np.sqrt(B / 100) * 2)
+    # ragged movers with 70000 sequences of 2 floats
+    src = dev.tensor(f32(rng.standard_normal((B, 2))))
+    dst = dev.zeros((B, 2))
+    ptrs = dev.tensor(np.concatenate([src.ptr + 8 * np.arange(B, dtype=np.uint64), dst.ptr + 8 * np.arange(B, dtype=np.uint64)]),
+                      np.uint64)
+    lens = dev.tensor(np.full(B, 2, np.uint64), np.uint64)
+    dev.parallel_memcpy(B, 2, ptrs.ptr, ptrs.ptr + 8 * B, lens)
+    assert dst.numpy().tobytes() == src.numpy().tobytes()
+
+
 def test_lstm_rejects_bad_arguments(dev):
     t = dev.zeros(64)
     with pytest.raises(DyhipError) as e:

@@ -13,6 +13,7 @@ import pytest
 from scipy.special import logsumexp as sp_logsumexp
 
 from oracle import cpu_oracle as orc
+from util import assert_close
 
 F32 = np.float32
 
@@ -119,6 +120,104 @@ def test_cmult_and_csum_broadcast_forward_backward():
 # ---------------------------------------------------------------------------
 # reductions (golden: cadd_broadcast2_neg_val, std_dim_value)
 # ---------------------------------------------------------------------------
+CWISE_SHAPES = [
+    # dims_a, dims_b as (d0, d1, d2, d3, bd)
+    ((1024, 1, 1, 1, 6), (1, 1, 1, 1, 6)),      # x - mean, x / sigma of the layer_norm composite
+    ((5, 3, 1, 1, 4), (5, 1, 1, 1, 1)),         # a column vector against a matrix batch
+    ((5, 3, 1, 1, 4), (1, 3, 1, 1, 4)),
+    ((4, 3, 2, 1, 3), (4, 1, 2, 1, 1)),         # kept axes on both sides of a broadcast one
+    ((2, 3, 4, 5, 2), (1, 3, 1, 5, 1)),
+    ((7, 1, 1, 1, 3), (7, 1, 1, 1, 3)),         # nothing broadcast
+    ((6, 2, 1, 1, 5), (6, 2, 1, 1, 1)),         # batch only
+]
+
+
+@pytest.mark.parametrize("op", [orc.CWISE_SUM, orc.CWISE_MULT, orc.CWISE_QUOTIENT])
+@pytest.mark.parametrize("da,db", CWISE_SHAPES)
+def test_cwise_broadcast_against_numpy_broadcasting(op, da, db):
+    """orc_cwise_*: numpy's own broadcasting in fp64 is the yardstick (shape = reversed dims), both argument
+    orders; the backward is the broadcast-reduced product rule, summed with np.sum over the broadcast axes."""
+    rng = np.random.default_rng(sum(da) + 7 * sum(db) + op)
+    for swap in (False, True):
+        d0, d1 = (db, da) if swap else (da, db)
+        if op == orc.CWISE_QUOTIENT and any(x != y and y != 1 for x, y in zip(d0, d1)):
+            with pytest.raises(ValueError):
+                orc.cwise_forward(op, d0, d1, np.zeros(d0[::-1], F32), np.ones(d1[::-1], F32))
+            continue
+        a = f32(rng.standard_normal(d0[::-1]))
+        b = f32(rng.standard_normal(d1[::-1]) + (3.0 if op == orc.CWISE_QUOTIENT else 0.0))
+        a64, b64 = a.astype(np.float64), b.astype(np.float64)
+        want = a64 + b64 if op == orc.CWISE_SUM else a64 * b64 if op == orc.CWISE_MULT else a64 / b64
+        fx = orc.cwise_forward(op, d0, d1, a, b)
+        assert fx.shape == want.shape
+        assert_close(fx, want, 1e-6, "cwise fwd", floor=1e-3)
+        dy = f32(rng.standard_normal(want.shape))
+        for i, (x, dims) in enumerate(((a, d0), (b, d1))):
+            if op == orc.CWISE_SUM:
+                term = dy.astype(np.float64) * np.ones_like(want)
+            elif op == orc.CWISE_MULT:
+                term = dy * (b64 if i == 0 else a64) * np.ones_like(want)
+            else:
+                term = dy / b64 if i == 0 else -(dy * a64 / (b64 * b64))
+            axes = tuple(k for k, (n_x, n_f) in enumerate(zip(x.shape, want.shape)) if n_x == 1 and n_f > 1)
+            red = term.sum(axis=axes, keepdims=True) if axes else term
+            g0 = f32(rng.standard_normal(x.shape))
+            got = orc.cwise_backward(op, d0, d1, a, b, dy, i, g0.copy())
+            assert_close(got, g0 + red, 1e-5, "cwise bwd %d" % i, floor=np.sqrt(want.size / x.size))
+
+
+def test_cwise_broadcast_reduces_to_the_batch_only_operators():
+    rng = np.random.default_rng(3)
+    n, bd = 12, 5
+    a, b, dy = f32(rng.standard_normal((bd, n))), f32(rng.standard_normal((1, n))), f32(rng.standard_normal((bd, n)))
+    da, db = (n, 1, 1, 1, bd), (n, 1, 1, 1, 1)
+    assert orc.cwise_forward(orc.CWISE_SUM, da, db, a, b).reshape(bd, n).tobytes() == orc.csum_forward(n, bd, 1, a, b).tobytes()
+    assert orc.cwise_forward(orc.CWISE_MULT, da, db, a, b).reshape(bd, n).tobytes() == orc.cmult_forward(n, bd, 1, a, b).tobytes()
+    for i, shape in ((0, (bd, n)), (1, (1, n))):
+        g0 = f32(rng.standard_normal(shape))
+        # bitwise without a reduction; with one the general form sums first and then adds (backward_helper's
+        # `+= (...).sum(red_axis)`), the batch-only CPU branch adds term by term
+        same = (lambda u, v: u.tobytes() == v.tobytes()) if i == 0 else (lambda u, v: np.allclose(u, v, rtol=1e-6, atol=1e-6))
+        assert same(orc.cwise_backward(orc.CWISE_MULT, da, db, a, b, dy, i, g0.copy()),
+                    orc.cmult_backward(n, bd, 1, a, b, dy, i, g0.copy()))
+        assert same(orc.cwise_backward(orc.CWISE_SUM, da, db, a, b, dy, i, g0.copy()),
+                    orc.csum_backward(n, bd, 1, dy, i, g0.copy()))
+
+
+def test_layer_norm_composite_of_eight_nodes_equals_the_layer_norm_oracle():
+    """dynet/expr.cc:248-253 node by node through the oracle's own node functions - mean_elems, Negate + CwiseSum,
+    std_elems, ConstantPlusX, CwiseQuotient, CwiseMultiply, CwiseSum - forward and backward, against
+    orc_layer_norm_* (which restates the same graph in one function)."""
+    rng = np.random.default_rng(12)
+    n, bd = 24, 5
+    x, g, b = f32(rng.standard_normal((bd, n))), f32(rng.uniform(0.5, 1.5, n)), f32(rng.standard_normal(n) * 0.1)
+    dy = f32(rng.standard_normal((bd, n)))
+    X, S, G = (n, 1, 1, 1, bd), (1, 1, 1, 1, bd), (n, 1, 1, 1, 1)
+    mu = orc.mean_elems_forward(n, bd, x)
+    neg = orc.unary_forward(orc.OP_NEGATE, mu)
+    xc = orc.cwise_forward(orc.CWISE_SUM, X, S, x, neg)
+    sigma = orc.std_elems_forward(n, bd, x)
+    se = orc.const_plus_x_forward(1e-8, sigma)
+    q = orc.cwise_forward(orc.CWISE_QUOTIENT, X, S, xc, se)
+    gq = orc.cwise_forward(orc.CWISE_MULT, G, X, g, q)
+    y = orc.cwise_forward(orc.CWISE_SUM, X, G, gq, b)
+    assert_close(y.reshape(bd, n), orc.layer_norm_forward(n, bd, x, g, b).reshape(bd, n), 1e-6, "composite fwd", floor=1.0)
+    z = lambda *s: np.zeros(s, F32)
+    d_gq, d_b = orc.cwise_backward(orc.CWISE_SUM, X, G, gq, b, dy, 0, z(bd, n)), orc.cwise_backward(orc.CWISE_SUM, X, G, gq, b, dy, 1, z(n))
+    d_g, d_q = orc.cwise_backward(orc.CWISE_MULT, G, X, g, q, d_gq, 0, z(n)), orc.cwise_backward(orc.CWISE_MULT, G, X, g, q, d_gq, 1, z(bd, n))
+    d_xc = orc.cwise_backward(orc.CWISE_QUOTIENT, X, S, xc, se, d_q, 0, z(bd, n))
+    d_se = orc.cwise_backward(orc.CWISE_QUOTIENT, X, S, xc, se, d_q, 1, z(bd))
+    d_x = orc.std_elems_backward(n, bd, x, sigma, d_se, z(bd, n))            # ConstantPlusX passes d_se through
+    d_x = orc.cwise_backward(orc.CWISE_SUM, X, S, x, neg, d_xc, 0, d_x)
+    d_neg = orc.cwise_backward(orc.CWISE_SUM, X, S, x, neg, d_xc, 1, z(bd))
+    d_mu = orc.unary_backward(orc.OP_NEGATE, neg, d_neg, z(bd))
+    d_x = orc.mean_elems_backward(n, bd, d_mu, d_x)
+    wx, wg, wb = orc.layer_norm_backward(n, bd, x, g, dy, z(bd, n), z(n), z(n))
+    assert_close(d_x, wx, 1e-5, "composite dx", floor=1.0)
+    assert_close(d_g, wg, 1e-5, "composite dg", floor=np.sqrt(bd))
+    assert_close(d_b, wb, 1e-5, "composite db", floor=np.sqrt(bd))
+
+
 def test_sum_batches_golden_cadd_broadcast2_neg_val(golden):
     g = golden["node_values"]
     x1 = f32(g["fixture_params"]["param1"]).reshape(1, 3)
