@@ -367,6 +367,55 @@ def extras(dev, lib, reps, use_graph=True):
         else:
             us3 = time_loop(dev, [fn], max(reps, 50))
         res["cfg1_lstm_cell"][key] = round(us3, 2)
+    res["combine_tensors"] = movers(dev, lib, reps, use_graph)
+    return res
+
+
+def movers(dev, lib, reps, use_graph=True):
+    """The batched executor's combine_tensors / accumulate_tensors on 128 nodes of 1024 floats each: the mover
+    kernels alone (pointer table resident), and the whole host path per call (table written into page-locked
+    memory, queued copy, kernel; no synchronisation between calls)."""
+    from dynet_amd.device import PinnedArray
+
+    rng = np.random.default_rng(2)
+    k, sz = 128, 1024
+    parts = [dev.tensor(rng.standard_normal(sz).astype(np.float32)) for _ in range(k)]
+    grads = [dev.zeros(sz, pool=lib.POOL_DEDFS) for _ in range(k)]
+    out = dev.empty(k * sz)
+    table = dev.empty(3 * k, np.uint64)
+    lens = np.full(k, sz, np.uint64)
+    fwd = np.concatenate([np.array([t.ptr for t in parts], np.uint64), out.ptr + 4 * sz * np.arange(k, dtype=np.uint64), lens])
+    bwd = np.concatenate([out.ptr + 4 * sz * np.arange(k, dtype=np.uint64), np.array([t.ptr for t in grads], np.uint64), lens])
+    ring = [PinnedArray((3 * k,), np.uint64) for _ in range(64)]
+    res = {"nodes": k, "floats_per_node": sz}
+    for name, tab, call, nbytes in (("combine_tensors", fwd, dev.parallel_memcpy, 2 * k * sz * 4),
+                                    ("accumulate_tensors", bwd, dev.parallel_accumulate, 3 * k * sz * 4)):
+        table.set(tab)
+        fn = lambda: call(k, sz, table.ptr, table.ptr + 8 * k, table.ptr + 16 * k)
+        fn()
+        dev.sync()
+        if use_graph:
+            g = capture(dev, [fn] * 8)
+            us = time_graph(dev, g, max(reps, 50), 8)
+            g.destroy()
+        else:
+            us = time_loop(dev, [fn], max(reps, 50))
+        # host path: 64 calls back to back, each with its own slice of page-locked staging memory
+        for p in ring:
+            p.array[:] = tab
+        dev.sync()
+        t0 = time.perf_counter()
+        for p in ring:
+            dev.copy_h2d_async(table, p)
+            fn()
+        t_issue = time.perf_counter() - t0
+        dev.sync()
+        t_all = time.perf_counter() - t0
+        res[name] = {"bytes": nbytes, "kernel_us": round(us, 2), "kernel_GBps": round(nbytes / us / 1e3, 1),
+                     "host_path_us_per_call": round(t_all / len(ring) * 1e6, 2),
+                     "host_issue_us_per_call": round(t_issue / len(ring) * 1e6, 2)}
+    for p in ring:
+        p.close()
     return res
 
 

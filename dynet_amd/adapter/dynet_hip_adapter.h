@@ -99,12 +99,58 @@ struct Tensor {
 };
 
 // dynet/devices.h:46-61, dynet/devices.cc:91-121
+// Page-locked staging ring for the small host tables a call hands to the GPU (pointer / length tables of the
+// batched executor, dynet/exec.cc:319-355).  A copy from it is asynchronous, so a slice may only be reused once
+// the copies issued from it have run: the ring synchronises the device when it wraps, which with 24-byte entries
+// is once per ~10^4 staged tensors, and never otherwise.
+class PinnedStaging {
+ public:
+  explicit PinnedStaging(dyhip_device* dev, size_t bytes = size_t(256) << 10) : dev_(dev), cap_(0), cur_(0), base_(nullptr) {
+    grow(bytes);
+  }
+  ~PinnedStaging() {
+    if (base_) {
+      dyhip_device_sync(dev_);
+      dyhip_host_free(base_);
+    }
+  }
+  PinnedStaging(const PinnedStaging&) = delete;
+  PinnedStaging& operator=(const PinnedStaging&) = delete;
+  void* take(size_t bytes) {
+    bytes = (bytes + 63) & ~size_t(63);
+    if (bytes > cap_) grow(2 * bytes);
+    if (cur_ + bytes > cap_) {
+      abi_check(dyhip_device_sync(dev_));
+      cur_ = 0;
+    }
+    void* out = static_cast<char*>(base_) + cur_;
+    cur_ += bytes;
+    return out;
+  }
+
+ private:
+  void grow(size_t bytes) {
+    if (base_) {
+      abi_check(dyhip_device_sync(dev_));
+      abi_check(dyhip_host_free(base_));
+      base_ = nullptr;
+    }
+    abi_check(dyhip_host_alloc(bytes, &base_));
+    cap_ = bytes;
+    cur_ = 0;
+  }
+  dyhip_device* dev_;
+  size_t cap_, cur_;
+  void* base_;
+};
+
 struct Device_GPU {
   dyhip_device* hip;
   float *kSCALAR_MINUSONE, *kSCALAR_ONE, *kSCALAR_ZERO;
   std::vector<AlignedMemoryPool*> pools;
+  PinnedStaging* staging;
 
-  Device_GPU(int device_id, size_t fxs_mb, size_t dedfs_mb, size_t ps_mb, size_t scs_mb) : hip(nullptr) {
+  Device_GPU(int device_id, size_t fxs_mb, size_t dedfs_mb, size_t ps_mb, size_t scs_mb) : hip(nullptr), staging(nullptr) {
     const size_t mb[4] = {fxs_mb, dedfs_mb, ps_mb, scs_mb};
     abi_check(dyhip_device_create(device_id, mb, &hip));
     const float* s[3];
@@ -117,8 +163,10 @@ struct Device_GPU {
       abi_check(dyhip_device_pool(hip, k, &p));
       pools.push_back(new AlignedMemoryPool(p));
     }
+    staging = new PinnedStaging(hip);
   }
   ~Device_GPU() {
+    delete staging;
     for (AlignedMemoryPool* p : pools) delete p;
     if (hip) dyhip_device_destroy(hip);
   }
@@ -270,20 +318,81 @@ struct UnaryNode : public Node {
 typedef UnaryNode<DYHIP_OP_TANH> Tanh;
 typedef UnaryNode<DYHIP_OP_LOGISTIC> LogisticSigmoid;
 typedef UnaryNode<DYHIP_OP_RECTIFY> Rectify;
+typedef UnaryNode<DYHIP_OP_NEGATE> Negate;
 
-// CwiseMultiply, same shape or one side with batch size 1 (dynet/nodes-arith-cwise.cc:196-307)
-struct CwiseMultiply : public Node {
+// CwiseSum / CwiseMultiply / CwiseQuotient (dynet/nodes-arith-cwise.cc:51-126, 197-306, 339-419): every
+// dimension and the batch of either argument may be 1 against the other's size (the reference's
+// get_broadcasting_bits rule); backward sums over the dimensions argument i was broadcast over.
+inline void dims5(const Dim& d, unsigned out[5]) {
+  if (d.nd > 4) throw std::invalid_argument("component-wise nodes take tensors of at most 4 dimensions");
+  for (unsigned k = 0; k < 4; ++k) out[k] = d[k];
+  out[4] = d.bd;
+}
+template <int OP>
+struct CwiseNode : public Node {
   void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
-    abi_check(dyhip_cmult_forward(dev.hip, fx.d.batch_size(), xs[0]->d.bd, xs[1]->d.bd, xs[0]->v, xs[1]->v, fx.v));
+    unsigned da[5], db[5];
+    dims5(xs[0]->d, da);
+    dims5(xs[1]->d, db);
+    abi_check(dyhip_cwise_forward(dev.hip, OP, da, db, xs[0]->v, xs[1]->v, fx.v));
   }
   void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, const Tensor& fx,
                          const Tensor& dEdf, unsigned i, Tensor& dEdxi) const override {
+    unsigned da[5], db[5];
+    dims5(xs[0]->d, da);
+    dims5(xs[1]->d, db);
     size_t need = 0;
-    abi_check(dyhip_batch_reduce_workspace(fx.d.batch_size(), fx.d.bd, &need));
+    abi_check(dyhip_cwise_backward_workspace(da, db, i, &need));
     void* ws = need ? scratch(fx)->allocate(need) : nullptr;
-    abi_check(dyhip_cmult_backward(dev.hip, fx.d.batch_size(), xs[0]->d.bd, xs[1]->d.bd, xs[0]->v, xs[1]->v, dEdf.v, i,
-                                   dEdxi.v, ws, need));
+    abi_check(dyhip_cwise_backward(dev.hip, OP, da, db, xs[0]->v, xs[1]->v, dEdf.v, i, dEdxi.v, ws, need));
     scratch(fx)->free();
+  }
+};
+typedef CwiseNode<DYHIP_CWISE_SUM> CwiseSum;
+typedef CwiseNode<DYHIP_CWISE_MULT> CwiseMultiply;
+typedef CwiseNode<DYHIP_CWISE_QUOTIENT> CwiseQuotient;
+
+// ConstantPlusX / ConstantMinusX (dynet/nodes-arith-const.cc:30-44, 63-77)
+struct ConstantPlusX : public Node {
+  explicit ConstantPlusX(real c) : c(c) {}
+  real c;
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    abi_check(dyhip_const_plus_x_forward(dev.hip, fx.d.size(), c, xs[0]->v, fx.v));
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>&, const Tensor&, const Tensor& dEdf,
+                         unsigned, Tensor& dEdxi) const override {
+    abi_check(dyhip_accumulate(dev.hip, dEdf.d.size(), dEdf.v, dEdxi.v));
+  }
+};
+struct ConstantMinusX : public Node {
+  explicit ConstantMinusX(real c) : c(c) {}
+  real c;
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    abi_check(dyhip_const_minus_x_forward(dev.hip, fx.d.size(), c, xs[0]->v, fx.v));
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>&, const Tensor& fx, const Tensor& dEdf,
+                         unsigned, Tensor& dEdxi) const override {
+    abi_check(dyhip_unary_backward(dev.hip, DYHIP_OP_NEGATE, fx.d.size(), fx.v, dEdf.v, dEdxi.v));
+  }
+};
+
+// mean_elems / std_elems: MomentElements with order 1 and StdElements (dynet/nodes-moments.cc:121-148, 380-400)
+struct MeanElements : public Node {
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    abi_check(dyhip_mean_elems_forward(dev.hip, xs[0]->d.batch_size(), xs[0]->d.bd, xs[0]->v, fx.v));
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, const Tensor&, const Tensor& dEdf,
+                         unsigned, Tensor& dEdxi) const override {
+    abi_check(dyhip_mean_elems_backward(dev.hip, xs[0]->d.batch_size(), xs[0]->d.bd, dEdf.v, dEdxi.v));
+  }
+};
+struct StdElements : public Node {
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    abi_check(dyhip_std_elems_forward(dev.hip, xs[0]->d.batch_size(), xs[0]->d.bd, xs[0]->v, fx.v));
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, const Tensor& fx,
+                         const Tensor& dEdf, unsigned, Tensor& dEdxi) const override {
+    abi_check(dyhip_std_elems_backward(dev.hip, xs[0]->d.batch_size(), xs[0]->d.bd, xs[0]->v, fx.v, dEdf.v, dEdxi.v));
   }
 };
 
@@ -484,6 +593,87 @@ inline void sparse_to_dense_assign(const Device_GPU& dev, int n, const unsigned*
 inline void dense_to_sparse_subtract(const Device_GPU& dev, int n, const unsigned* ids, float* src, float* trg) {
   abi_check(dyhip_dense_to_sparse_subtract(dev.hip, n, ids, src, trg));
 }
+inline void sparse_to_dense_block_assign_and_multiply(const Device_GPU& dev, int n, const unsigned* idx, int bsize,
+                                                      float mult, float* src, float* trg) {
+  abi_check(dyhip_sparse_to_dense_block_assign_and_multiply(dev.hip, n, idx, bsize, mult, src, trg));
+}
+inline void dense_to_sparse_block_add(const Device_GPU& dev, int n, const unsigned* ids, int bsize, float* src, float* trg) {
+  abi_check(dyhip_dense_to_sparse_block_add(dev.hip, n, ids, bsize, src, trg));
+}
+inline void parallel_memcpy(const Device_GPU& dev, int num_seqs, int max_len, float** src, float** trg, size_t* len) {
+  abi_check(dyhip_parallel_memcpy(dev.hip, num_seqs, max_len, src, trg, len));
+}
+inline void parallel_accumulate(const Device_GPU& dev, int num_seqs, int max_len, float** src, float** trg, size_t* len) {
+  abi_check(dyhip_parallel_accumulate(dev.hip, num_seqs, max_len, src, trg, len));
+}
 }  // namespace gpu
+
+// The GPU branches of BatchedExecutionEngine::combine_tensors / accumulate_tensors (dynet/exec.cc:298-361,
+// 363-409) without the executor around them: the caller names the tensors.  The [src | trg | len] table is
+// written into page-locked staging memory, so its copy to the device queues behind earlier work instead of
+// stalling the host the way the reference's copy from a pageable std::vector does.
+namespace detail {
+inline void stage_and_move(Device_GPU& dev, DeviceMempool table_pool, const std::vector<float*>& srcs,
+                           const std::vector<float*>& trgs, const std::vector<size_t>& lens, bool accumulate) {
+  const size_t n = srcs.size();
+  if (n == 0) return;
+  static_assert(sizeof(float*) == sizeof(size_t), "pointer and length entries share one table");
+  size_t* host = static_cast<size_t*>(dev.staging->take(3 * n * sizeof(size_t)));
+  size_t max_len = 0;
+  for (size_t k = 0; k < n; ++k) {
+    host[k] = reinterpret_cast<size_t>(srcs[k]);
+    host[n + k] = reinterpret_cast<size_t>(trgs[k]);
+    host[2 * n + k] = lens[k];
+    if (lens[k] > max_len) max_len = lens[k];
+  }
+  void* table = dev.pools[static_cast<int>(table_pool)]->allocate(3 * n * sizeof(size_t));
+  abi_check(dyhip_memcpy_h2d(dev.hip, table, host, 3 * n * sizeof(size_t)));
+  float** d_src = static_cast<float**>(table);
+  float** d_trg = d_src + n;
+  size_t* d_len = static_cast<size_t*>(table) + 2 * n;
+  if (accumulate) gpu::parallel_accumulate(dev, static_cast<int>(n), static_cast<int>(max_len), d_src, d_trg, d_len);
+  else gpu::parallel_memcpy(dev, static_cast<int>(n), static_cast<int>(max_len), d_src, d_trg, d_len);
+}
+}  // namespace detail
+
+// tout becomes one contiguous tensor Dim({sum of sizes}) allocated from pools[FXS], holding the tensors of
+// `parts` back to back (dynet/exec.cc:298-361)
+inline void combine_tensors(Device_GPU& dev, const std::vector<const Tensor*>& parts, Tensor& tout) {
+  size_t total = 0;
+  for (const Tensor* t : parts) total += t->d.size();
+  if (total > 0xffffffffu) throw std::invalid_argument("combine_tensors: more than 2^32 - 1 elements");
+  tout.d = Dim({static_cast<unsigned>(total)});
+  tout.device = &dev;
+  tout.mem_pool = DeviceMempool::FXS;
+  tout.v = static_cast<float*>(dev.pools[static_cast<int>(DeviceMempool::FXS)]->allocate(total * sizeof(float)));
+  std::vector<float*> srcs, trgs;
+  std::vector<size_t> lens;
+  float* dest = tout.v;
+  for (const Tensor* t : parts) {
+    srcs.push_back(t->v);
+    trgs.push_back(dest);
+    lens.push_back(t->d.size());
+    dest += t->d.size();
+  }
+  detail::stage_and_move(dev, DeviceMempool::FXS, srcs, trgs, lens, false);
+}
+
+// every tensor of `grads` += its slice of tin, slices back to back in the order given (dynet/exec.cc:363-409);
+// two entries must not name the same memory, as the reference's one-thread-per-element kernel assumes
+inline void accumulate_tensors(Device_GPU& dev, const Tensor& tin, const std::vector<Tensor*>& grads) {
+  std::vector<float*> srcs, trgs;
+  std::vector<size_t> lens;
+  float* src = tin.v;
+  size_t total = 0;
+  for (Tensor* t : grads) {
+    srcs.push_back(src);
+    trgs.push_back(t->v);
+    lens.push_back(t->d.size());
+    src += t->d.size();
+    total += t->d.size();
+  }
+  if (total != tin.d.size()) throw std::invalid_argument("accumulate_tensors: the slices do not cover the input tensor");
+  detail::stage_and_move(dev, DeviceMempool::DEDFS, srcs, trgs, lens, true);
+}
 
 }  // namespace dynet_hip

@@ -429,6 +429,180 @@ static void random_nodes(Fixture& F) {
   }
 }
 
+// ---- component-wise nodes with dimension broadcast (tests/test-nodes.cc:177-212, 583-608, 1457-1484, 384-391) ----
+static void cwise_broadcast(Fixture& F) {
+  const vector<float> param1 = {1.1f, -2.2f, 3.3f}, param4 = {1.1f, 2.2f, 3.3f, -1.2f, 2.1f, 3.4f};
+  const vector<float> cube1 = {.051f, .062f, .073f, .052f, .062f, .072f, .053f, .063f, .073f,
+                               .111f, -.122f, -.033f, -.112f, -.022f, -.132f, -.113f, -.123f, -.133f,
+                               .211f, .222f, .233f, .212f, .222f, .232f, .213f, .223f, .233f};
+  const Dim two[] = {Dim({3, 1}, 2), Dim({3, 2}, 1)};
+  const Dim three[] = {Dim({3, 3, 3}, 1), Dim({3, 3, 1}, 3), Dim({1, 3, 3}, 3), Dim({9, 3, 1}, 1), Dim({1, 3, 9}, 1),
+                       Dim({1, 3, 1}, 9)};
+  auto both_orders = [&](const Node& node, const Dim& d1, const vector<float>& v1, const Dim& d2,
+                         const vector<float>& v2, bool swap_too) {
+    { vector<Tensor> a = {F.input(d1, v1), F.input(d2, v2)}; CHECK(check_grad(F, node, a, d2, {true, true})); }
+    if (swap_too) { vector<Tensor> a = {F.input(d2, v2), F.input(d1, v1)}; CHECK(check_grad(F, node, a, d2, {true, true})); }
+    F.reset();
+  };
+  for (const Dim& d : two) {
+    g_case = "cadd_broadcast2_gradient";
+    both_orders(CwiseSum(), Dim({3, 1}), param1, d, param4, true);
+    g_case = "cmult_broadcast2_gradient";
+    both_orders(CwiseMultiply(), Dim({3, 1}), param1, d, param4, true);
+    g_case = "cdiv_broadcast2_gradient";  // cdiv(x2, x1): the denominator is the broadcast side
+    { vector<Tensor> a = {F.input(d, param4), F.input(Dim({3, 1}), param1)}; CHECK(check_grad(F, CwiseQuotient(), a, d, {true, true})); }
+    F.reset();
+  }
+  for (const Dim& d : three) {
+    g_case = "cadd_broadcast3_gradient";
+    both_orders(CwiseSum(), Dim({1, 3, 1}), param1, d, cube1, true);
+    g_case = "cmult_broadcast3_gradient";
+    both_orders(CwiseMultiply(), Dim({1, 3, 1}), param1, d, cube1, true);
+    g_case = "cdiv_broadcast3_gradient";
+    { vector<Tensor> a = {F.input(d, cube1), F.input(Dim({1, 3, 1}), param1)}; CHECK(check_grad(F, CwiseQuotient(), a, d, {true, true})); }
+    F.reset();
+  }
+  g_case = "cadd_broadcast2_neg_val";  // tests/test-nodes.cc:206-213: sum of x1 - x2 is -6.5
+  {
+    Tensor x1 = F.input(Dim({3, 1}), param1), x2 = F.input(Dim({3, 1}, 2), param4);
+    Tensor nx2 = F.dev.allocate_tensor(DeviceMempool::FXS, x2.d), y = F.dev.allocate_tensor(DeviceMempool::FXS, x2.d);
+    Negate().forward_dev_impl(F.dev, {&x2}, nx2);
+    CwiseSum().forward_dev_impl(F.dev, {&x1, &nx2}, y);
+    double z = 0;
+    for (float e : as_vector(y)) z += e;
+    CHECK_CLOSE(z, -6.5, 0.001);
+  }
+  g_case = "addscalar_gradient";
+  { vector<Tensor> a = {F.input(Dim({3}), param1)}; CHECK(check_grad(F, ConstantPlusX(2.0f), a, Dim({3}), {true})); }
+  g_case = "scalarsubtract_gradient";
+  { vector<Tensor> a = {F.input(Dim({3}), param1)}; CHECK(check_grad(F, ConstantMinusX(2.0f), a, Dim({3}), {true})); }
+  g_case = "mean_std_elems_gradient";
+  {
+    vector<Tensor> a = {F.input(Dim({3}, 2), param4)};
+    CHECK(check_grad(F, MeanElements(), a, Dim({1}, 2), {true}));
+    CHECK(check_grad(F, StdElements(), a, Dim({1}, 2), {true}));
+  }
+}
+
+// ---- layer_norm as the reference composes it from eight nodes (dynet/expr.cc:248-253) against the fused node ----
+static void layer_norm_composite(Fixture& F) {
+  g_case = "layer_norm_composite";
+  const unsigned n = 64, bd = 5;
+  vector<float> xv(n * bd), gv(n), bv(n), wv(n * bd);
+  for (size_t k = 0; k < xv.size(); ++k) xv[k] = std::sin(0.37f * float(k)) * 2.f + 0.01f * float(k % 11);
+  for (size_t k = 0; k < n; ++k) { gv[k] = 0.5f + 0.01f * float(k); bv[k] = 0.1f * std::cos(float(k)); }
+  for (size_t k = 0; k < wv.size(); ++k) wv[k] = 0.3f + 0.1f * float(k % 7) - 0.05f * float(k % 3);
+  const Dim dx({n}, bd), dp({n}), ds({1}, bd);
+  Tensor x = F.input(dx, xv), g = F.input(dp, gv), b = F.input(dp, bv), dEdf = F.input(dx, wv, DeviceMempool::DEDFS);
+  auto fx = [&](const Dim& d) { return F.dev.allocate_tensor(DeviceMempool::FXS, d); };
+  Tensor mu = fx(ds), nmu = fx(ds), xc = fx(dx), sigma = fx(ds), se = fx(ds), q = fx(dx), gq = fx(dx), y = fx(dx), fused = fx(dx);
+  const MeanElements mean_n; const Negate neg_n; const CwiseSum sum_n; const StdElements std_n;
+  const ConstantPlusX eps_n(1e-8f); const CwiseQuotient div_n; const CwiseMultiply mul_n;
+  mean_n.forward_dev_impl(F.dev, {&x}, mu);
+  neg_n.forward_dev_impl(F.dev, {&mu}, nmu);
+  sum_n.forward_dev_impl(F.dev, {&x, &nmu}, xc);
+  std_n.forward_dev_impl(F.dev, {&x}, sigma);
+  eps_n.forward_dev_impl(F.dev, {&sigma}, se);
+  div_n.forward_dev_impl(F.dev, {&xc, &se}, q);
+  mul_n.forward_dev_impl(F.dev, {&g, &q}, gq);
+  sum_n.forward_dev_impl(F.dev, {&gq, &b}, y);
+  LayerNorm().forward_dev_impl(F.dev, {&x, &g, &b}, fused);
+  const vector<float> yc = as_vector(y), yf = as_vector(fused);
+  for (size_t k = 0; k < yc.size(); ++k) CHECK_SMALL(yc[k] - yf[k], 2e-6 * (1.0 + std::fabs(yf[k])));
+  // backward through the eight nodes in reverse order
+  Tensor d_gq = F.zeros(dx), d_b = F.zeros(dp), d_g = F.zeros(dp), d_q = F.zeros(dx), d_xc = F.zeros(dx), d_se = F.zeros(ds),
+         d_sigma = F.zeros(ds), d_x = F.zeros(dx), d_nmu = F.zeros(ds), d_mu = F.zeros(ds);
+  sum_n.backward_dev_impl(F.dev, {&gq, &b}, y, dEdf, 0, d_gq);
+  sum_n.backward_dev_impl(F.dev, {&gq, &b}, y, dEdf, 1, d_b);
+  mul_n.backward_dev_impl(F.dev, {&g, &q}, gq, d_gq, 0, d_g);
+  mul_n.backward_dev_impl(F.dev, {&g, &q}, gq, d_gq, 1, d_q);
+  div_n.backward_dev_impl(F.dev, {&xc, &se}, q, d_q, 0, d_xc);
+  div_n.backward_dev_impl(F.dev, {&xc, &se}, q, d_q, 1, d_se);
+  eps_n.backward_dev_impl(F.dev, {&sigma}, se, d_se, 0, d_sigma);
+  std_n.backward_dev_impl(F.dev, {&x}, sigma, d_sigma, 0, d_x);
+  sum_n.backward_dev_impl(F.dev, {&x, &nmu}, xc, d_xc, 0, d_x);
+  sum_n.backward_dev_impl(F.dev, {&x, &nmu}, xc, d_xc, 1, d_nmu);
+  neg_n.backward_dev_impl(F.dev, {&mu}, nmu, d_nmu, 0, d_mu);
+  mean_n.backward_dev_impl(F.dev, {&x}, mu, d_mu, 0, d_x);
+  Tensor f_x = F.zeros(dx), f_g = F.zeros(dp), f_b = F.zeros(dp);
+  const LayerNorm ln;
+  ln.forward_dev_impl(F.dev, {&x, &g, &b}, fused);
+  ln.backward_dev_impl(F.dev, {&x, &g, &b}, fused, dEdf, 0, f_x);
+  ln.backward_dev_impl(F.dev, {&x, &g, &b}, fused, dEdf, 1, f_g);
+  ln.backward_dev_impl(F.dev, {&x, &g, &b}, fused, dEdf, 2, f_b);
+  const vector<float> cx = as_vector(d_x), cg = as_vector(d_g), cb = as_vector(d_b), rx = as_vector(f_x), rg = as_vector(f_g),
+                      rb = as_vector(f_b);
+  for (size_t k = 0; k < cx.size(); ++k) CHECK_SMALL(cx[k] - rx[k], 1e-5 * (1.0 + std::fabs(rx[k])));
+  for (size_t k = 0; k < n; ++k) {
+    CHECK_SMALL(cg[k] - rg[k], 1e-5 * (1.0 + std::fabs(rg[k])));
+    CHECK_SMALL(cb[k] - rb[k], 1e-5 * (1.0 + std::fabs(rb[k])));
+  }
+}
+
+// ---- BatchedExecutionEngine::combine_tensors / accumulate_tensors (dynet/exec.cc:298-409) ----
+static void combine_and_accumulate(Fixture& F) {
+  g_case = "combine_tensors";
+  // 128 nodes of 1024 floats, then a ragged tail (sizes 1, 7, 1000, 3)
+  vector<unsigned> sizes(128, 1024);
+  for (unsigned s : {1u, 7u, 1000u, 3u}) sizes.push_back(s);
+  vector<Tensor> parts;
+  vector<vector<float>> host;
+  vector<float> expect;
+  unsigned seed = 1;
+  for (unsigned sz : sizes) {
+    vector<float> v(sz);
+    for (float& e : v) { seed = seed * 1664525u + 1013904223u; e = float(seed >> 8) * (1.f / 16777216.f) - 0.5f; }
+    expect.insert(expect.end(), v.begin(), v.end());
+    parts.push_back(F.input(Dim({sz}), v));
+    host.push_back(v);
+  }
+  vector<const Tensor*> ptrs;
+  for (const Tensor& t : parts) ptrs.push_back(&t);
+  for (int rep = 0; rep < 3; ++rep) {  // repeated calls walk the staging ring
+    Tensor tout;
+    combine_tensors(F.dev, ptrs, tout);
+    CHECK(tout.d.size() == expect.size());
+    CHECK(as_vector(tout) == expect);
+  }
+  g_case = "accumulate_tensors";
+  vector<Tensor> grads;
+  for (size_t k = 0; k < sizes.size(); ++k) {
+    vector<float> init(sizes[k]);
+    for (size_t e = 0; e < init.size(); ++e) init[e] = 0.25f * float((k + e) % 5);
+    grads.push_back(F.input(Dim({sizes[k]}), init, DeviceMempool::DEDFS));
+  }
+  Tensor tin = F.input(Dim({static_cast<unsigned>(expect.size())}), expect, DeviceMempool::DEDFS);
+  vector<Tensor*> gp;
+  for (Tensor& t : grads) gp.push_back(&t);
+  accumulate_tensors(F.dev, tin, gp);
+  accumulate_tensors(F.dev, tin, gp);
+  for (size_t k = 0; k < sizes.size(); ++k) {
+    const vector<float> got = as_vector(grads[k]);
+    bool same = true;
+    for (size_t e = 0; e < got.size(); ++e) same = same && got[e] == (0.25f * float((k + e) % 5) + host[k][e]) + host[k][e];
+    CHECK(same);
+  }
+  bool threw = false;
+  gp.pop_back();
+  try { accumulate_tensors(F.dev, tin, gp); } catch (const std::invalid_argument&) { threw = true; }
+  CHECK(threw);
+  g_case = "staging_ring_wraps";  // more staged bytes than the ring holds: the wrap must not corrupt earlier tables
+  {
+    vector<const Tensor*> two = {&parts[0], &parts[1]};
+    vector<float> want(host[0]);
+    want.insert(want.end(), host[1].begin(), host[1].end());
+    bool ok = true;
+    for (int rep = 0; rep < 6000; ++rep) {  // 6000 x 64 bytes > 256 KiB
+      const size_t used = F.dev.pools[0]->used();
+      Tensor tout;
+      combine_tensors(F.dev, two, tout);
+      if (rep % 1500 == 0) ok = ok && as_vector(tout) == want;
+      F.dev.pools[0]->set_used(used);
+    }
+    CHECK(ok);
+  }
+}
+
 int main(int argc, char** argv) {
   if (argc > 1 && std::strcmp(argv[1], "--no-gpu") == 0) {
     try {
@@ -443,7 +617,8 @@ int main(int argc, char** argv) {
   Fixture F;
   const std::vector<std::function<void(Fixture&)>> cases = {lstm_node_h_fwd,      lstm_node_c_fwd, lstm_node_gates_fwd,
                                                              lstm_node_gradients,  elementwise_gradients, layer_norm,
-                                                             lookup_and_softmax,   random_nodes};
+                                                             lookup_and_softmax,   random_nodes,    cwise_broadcast,       layer_norm_composite,
+                                                             combine_and_accumulate};
   for (const auto& c : cases) {
     c(F);
     F.reset();
