@@ -546,6 +546,53 @@ struct LogSoftmax : public Node {
   }
 };
 
+// Softmax along dimension 0 or 1 (dynet/nodes-softmaxes.cc:40-125)
+struct Softmax : public Node {
+  explicit Softmax(unsigned dimension = 0) : dimension(dimension) {}
+  unsigned dimension;
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    const Dim& d = xs[0]->d;
+    if (dimension == 0) {
+      const unsigned cols = d.cols() * d.bd;
+      void* ws = scratch(fx)->allocate(2 * sizeof(float) * cols);
+      abi_check(dyhip_softmax_forward(dev.hip, d.rows(), cols, xs[0]->v, fx.v, ws, 2 * sizeof(float) * cols));
+      scratch(fx)->free();
+    } else {
+      abi_check(dyhip_softmax_rows_forward(dev.hip, d.rows(), d.cols(), d.bd, xs[0]->v, fx.v));
+    }
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, const Tensor& fx,
+                         const Tensor& dEdf, unsigned, Tensor& dEdxi) const override {
+    const Dim& d = xs[0]->d;
+    if (dimension == 0) {
+      const unsigned cols = d.cols() * d.bd;
+      void* ws = scratch(fx)->allocate(sizeof(float) * cols);
+      abi_check(dyhip_softmax_backward(dev.hip, d.rows(), cols, fx.v, dEdf.v, dEdxi.v, ws, sizeof(float) * cols));
+      scratch(fx)->free();
+    } else {
+      abi_check(dyhip_softmax_rows_backward(dev.hip, d.rows(), d.cols(), d.bd, fx.v, dEdf.v, dEdxi.v));
+    }
+  }
+};
+
+// LogSumExpDimension (dynet/nodes-logsumexp.cc:126-145); the maxima go to scratch as in the reference
+struct LogSumExpDimension : public Node {
+  explicit LogSumExpDimension(unsigned dimension = 0) : dimension(dimension) {}
+  unsigned dimension;
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    const Dim& d = xs[0]->d;
+    if (d.nd > 2) throw std::invalid_argument("LogSumExpDimension supports tensors of dimension <= 2");
+    float* ms = static_cast<float*>(scratch(fx)->allocate(sizeof(float) * fx.d.size()));
+    abi_check(dyhip_logsumexp_dim_forward(dev.hip, d.rows(), d.cols(), d.bd, xs[0]->v, dimension, ms, fx.v));
+    scratch(fx)->free();
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, const Tensor& fx,
+                         const Tensor& dEdf, unsigned, Tensor& dEdxi) const override {
+    const Dim& d = xs[0]->d;
+    abi_check(dyhip_logsumexp_dim_backward(dev.hip, d.rows(), d.cols(), d.bd, xs[0]->v, fx.v, dEdf.v, dimension, dEdxi.v));
+  }
+};
+
 // AffineTransform with one (W, x) pair (dynet/nodes-affinetransform.cc:77-156).  xs = {bias, W, x}
 struct AffineTransform : public Node {
   void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
@@ -570,16 +617,32 @@ struct AffineTransform : public Node {
   }
 };
 
-// dynet/matrix-multiply.h:16-37,97-117,162-180 on Device_GPU (unbatched left operand)
+// dynet/matrix-multiply.h:16-37,97-117,162-180 on Device_GPU: one GEMM over all columns when the left operand
+// is shared by the batch, the strided-batched form otherwise (same branch conditions as the reference)
+inline size_t batch_stride(const Tensor& t) { return t.d.bd > 1 ? t.d.batch_size() : 0; }
 inline void MatrixMultiply(const Device_GPU& dev, const Tensor& l, const Tensor& r, Tensor& y, const float* acc_scalar) {
-  abi_check(dyhip_gemm_nn(dev.hip, l.d.rows(), size_t(r.d.cols()) * r.d.bd, l.d.cols(), l.v, r.v,
-                          acc_scalar == dev.kSCALAR_ONE ? 1.0f : 0.0f, y.v));
+  const float beta = acc_scalar == dev.kSCALAR_ONE ? 1.0f : 0.0f;
+  if (l.d.bd == 1 && r.d.bd == y.d.bd)
+    abi_check(dyhip_gemm_nn(dev.hip, y.d.rows(), size_t(y.d.cols()) * y.d.bd, l.d.cols(), l.v, r.v, beta, y.v));
+  else
+    abi_check(dyhip_gemm_strided_batched(dev.hip, 0, 0, y.d.rows(), y.d.cols(), l.d.cols(), l.v, batch_stride(l), r.v,
+                                         batch_stride(r), beta, y.v, y.d.batch_size(), y.d.bd));
 }
 inline void MatrixTranspMultiplyAcc(const Device_GPU& dev, const Tensor& l, const Tensor& r, Tensor& y) {
-  abi_check(dyhip_gemm_tn_acc(dev.hip, l.d.cols(), size_t(r.d.cols()) * r.d.bd, l.d.rows(), l.v, r.v, y.v));
+  const unsigned max_b = l.d.bd > r.d.bd ? l.d.bd : r.d.bd;
+  if (l.d.bd == 1 && y.d.bd == r.d.bd)
+    abi_check(dyhip_gemm_tn_acc(dev.hip, y.d.rows(), size_t(y.d.cols()) * y.d.bd, l.d.rows(), l.v, r.v, y.v));
+  else
+    abi_check(dyhip_gemm_strided_batched(dev.hip, 1, 0, y.d.rows(), y.d.cols(), l.d.rows(), l.v, batch_stride(l), r.v,
+                                         batch_stride(r), 1.0f, y.v, y.d.batch_size(), max_b));
 }
 inline void MatrixMultiplyTranspAcc(const Device_GPU& dev, const Tensor& l, const Tensor& r, Tensor& y) {
-  abi_check(dyhip_gemm_nt_acc(dev.hip, l.d.rows(), r.d.rows(), size_t(l.d.cols()) * l.d.bd, l.v, r.v, y.v));
+  const unsigned max_b = l.d.bd > r.d.bd ? l.d.bd : r.d.bd;
+  if (y.d.bd == 1 && l.d.bd == r.d.bd)
+    abi_check(dyhip_gemm_nt_acc(dev.hip, y.d.rows(), y.d.cols(), size_t(l.d.cols()) * l.d.bd, l.v, r.v, y.v));
+  else
+    abi_check(dyhip_gemm_strided_batched(dev.hip, 0, 1, y.d.rows(), y.d.cols(), l.d.cols(), l.v, batch_stride(l), r.v,
+                                         batch_stride(r), 1.0f, y.v, y.d.batch_size(), max_b));
 }
 
 // dynet::gpu::* (dynet/gpu-ops.h:9-15): same argument lists behind the device

@@ -40,8 +40,15 @@ struct GemmEpiParams {
   unsigned* splits_out;
 };
 
+// `count` independent products in one launch: item b uses A + b*stride_a, B + b*stride_b, C + b*stride_c
+// (strides in floats; 0 shares an operand between the items).  One K segment, axpby epilogue, no split-K.
+struct GemmBatch {
+  unsigned count;
+  size_t stride_a, stride_b, stride_c;
+};
+
 // C is M x N column-major (ldc = M).  Segments share the operand layouts.
 int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N, int nseg, const GemmSeg* segs,
-             float* C, const GemmEpiParams& epi);
+             float* C, const GemmEpiParams& epi, const GemmBatch* batch = nullptr);
 
 }  // namespace dyhip

@@ -55,6 +55,7 @@ struct GemmArgs {
   float beta;         // used when partial == nullptr
   const float* bias;  // when set (and partial == nullptr): C = bias[i] + sum
   float* partial;     // [splits][M*N] or nullptr
+  size_t stride_a, stride_b, stride_c;  // floats between consecutive batch items (blockIdx.z); 0 = shared operand
   int vec_ok;         // every operand 16-byte aligned with a leading dimension that is a multiple of 4
   int edge4_ok;       // vec_ok, and no 128-bit group of any operand straddles the matrix edge
 };
@@ -221,6 +222,11 @@ __device__ __forceinline__ void ktile_iter(const GemmArgs& g, unsigned kt_begin,
 template <bool A_KMAJOR, bool B_KMAJOR, int WN, int PF>
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_tile_kernel(GemmArgs g, unsigned tiles_m) {
   constexpr int BN = 64 * WN;
+  if (gridDim.z > 1) {  // strided batch: item blockIdx.z of every operand (single K segment, no split)
+    g.seg[0].A += size_t(blockIdx.z) * g.stride_a;
+    g.seg[0].B += size_t(blockIdx.z) * g.stride_b;
+    g.C += size_t(blockIdx.z) * g.stride_c;
+  }
   constexpr int PA = lds_pitch<A_KMAJOR, kBM>(), PB = lds_pitch<B_KMAJOR, BN>();
   __shared__ __attribute__((aligned(16))) float lds_a[2 * kBK * PA];
   __shared__ __attribute__((aligned(16))) float lds_b[2 * kBK * PB];
@@ -331,8 +337,8 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(size_t M, size_
 
 template <bool A_KMAJOR, bool B_KMAJOR>
 static void launch_tiles(dyhip_device* dev, const GemmArgs& g, unsigned tiles_m, unsigned tiles_n, unsigned splits,
-                         int wn) {
-  const dim3 grid(tiles_m * tiles_n, splits), block(kGemmThreads);
+                         int wn, unsigned batch = 1) {
+  const dim3 grid(tiles_m * tiles_n, splits, batch), block(kGemmThreads);
   if (wn == 1)
     hipLaunchKernelGGL((gemm_tile_kernel<A_KMAJOR, B_KMAJOR, 1, 2>), grid, block, 0, dev->stream, g, tiles_m);
   else
@@ -376,7 +382,7 @@ static GemmPlan plan_gemm(const dyhip_device* dev, size_t M, size_t N, unsigned 
 }
 
 int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N, int nseg, const GemmSeg* segs,
-             float* C, const GemmEpiParams& epi) {
+             float* C, const GemmEpiParams& epi, const GemmBatch* batch) {
   const bool to_caller = epi.kind == kEpiPartials;
   if (to_caller) {
     DYHIP_REQUIRE(epi.partials != nullptr && epi.splits_out != nullptr, "null split-K output");
@@ -395,7 +401,17 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
   g.ktiles_total = 0;
   g.ktiles0 = 0;
   g.seg[1] = GemmSeg{nullptr, 0, nullptr, 0, 0};
+  const unsigned items = batch ? batch->count : 1;
+  g.stride_a = g.stride_b = g.stride_c = 0;
   bool vec = true;
+  if (items > 1) {
+    DYHIP_REQUIRE(nseg == 1 && epi.kind == kEpiAxpby, "a strided-batched GEMM has one K segment and the axpby epilogue");
+    DYHIP_REQUIRE(batch->stride_c >= M * N, "batch items of the GEMM output overlap");
+    g.stride_a = batch->stride_a;
+    g.stride_b = batch->stride_b;
+    g.stride_c = batch->stride_c;
+    vec = g.stride_a % 4 == 0 && g.stride_b % 4 == 0;
+  }
   for (int s = 0; s < nseg; ++s) {
     DYHIP_REQUIRE(segs[s].A != nullptr && segs[s].B != nullptr, "null GEMM operand");
     g.seg[s] = segs[s];
@@ -415,7 +431,8 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
   const bool fused_epi = epi.kind == kEpiLstmGates;  // needs the whole sum before the activation
   const bool must_partial = fused_epi || to_caller;
   GemmPlan plan{N <= 64 ? 1 : 2, 1};
-  if (g.ktiles_total > 0) plan = plan_gemm(dev, M, N, g.ktiles_total, ws_bytes / out_bytes, must_partial);
+  if (g.ktiles_total > 0)
+    plan = plan_gemm(dev, M, N, g.ktiles_total, items > 1 ? 1 : ws_bytes / out_bytes, must_partial);
   unsigned splits = plan.splits;
   const size_t tiles_m = cdiv<size_t>(M, kBM), tiles_n = cdiv<size_t>(N, size_t(64) * plan.wn);
   DYHIP_REQUIRE(tiles_m * tiles_n < (size_t(1) << 31), "GEMM too large");
@@ -427,10 +444,18 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
                   "GEMM output of %zu bytes x %u splits does not fit the %zu-byte split-K workspace", out_bytes,
                   splits, ws_bytes);
   g.partial = use_partial ? static_cast<float*>(ws) : nullptr;
-  if (a_kmajor && b_kmajor) launch_tiles<true, true>(dev, g, (unsigned)tiles_m, (unsigned)tiles_n, splits, plan.wn);
-  else if (a_kmajor && !b_kmajor) launch_tiles<true, false>(dev, g, (unsigned)tiles_m, (unsigned)tiles_n, splits, plan.wn);
-  else if (!a_kmajor && b_kmajor) launch_tiles<false, true>(dev, g, (unsigned)tiles_m, (unsigned)tiles_n, splits, plan.wn);
-  else launch_tiles<false, false>(dev, g, (unsigned)tiles_m, (unsigned)tiles_n, splits, plan.wn);
+  // grid z holds at most 65535 batch items per launch
+  for (unsigned first = 0; first < items; first += 65535u) {
+    const unsigned nb = items - first < 65535u ? items - first : 65535u;
+    GemmArgs h = g;
+    h.seg[0].A += size_t(first) * g.stride_a;
+    h.seg[0].B += size_t(first) * g.stride_b;
+    if (h.C != nullptr) h.C += size_t(first) * g.stride_c;
+    if (a_kmajor && b_kmajor) launch_tiles<true, true>(dev, h, (unsigned)tiles_m, (unsigned)tiles_n, splits, plan.wn, nb);
+    else if (a_kmajor && !b_kmajor) launch_tiles<true, false>(dev, h, (unsigned)tiles_m, (unsigned)tiles_n, splits, plan.wn, nb);
+    else if (!a_kmajor && b_kmajor) launch_tiles<false, true>(dev, h, (unsigned)tiles_m, (unsigned)tiles_n, splits, plan.wn, nb);
+    else launch_tiles<false, false>(dev, h, (unsigned)tiles_m, (unsigned)tiles_n, splits, plan.wn, nb);
+  }
   DYHIP_CHECK_LAUNCH();
   if (to_caller) {
     *epi.splits_out = splits;
@@ -496,6 +521,17 @@ int dyhip_gemm_nt(dyhip_device* dev, size_t M, size_t N, size_t K, const float* 
   DYHIP_CHECK_DEV(dev);
   GemmSeg s{l, M, r, N, K};
   return gemm_run(dev, false, false, M, N, 1, &s, y, axpby(beta));
+}
+
+int dyhip_gemm_strided_batched(dyhip_device* dev, int trans_l, int trans_r, size_t M, size_t N, size_t K,
+                               const float* l, size_t stride_l, const float* r, size_t stride_r, float beta, float* y,
+                               size_t stride_y, unsigned batch) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(!(trans_l && trans_r), "the strided-batched GEMM has the forms l*r, l^T*r and l*r^T");
+  if (batch == 0) return DYHIP_OK;
+  GemmSeg s{l, trans_l ? K : M, r, trans_r ? N : K, K};
+  GemmBatch b{batch, stride_l, stride_r, stride_y};
+  return gemm_run(dev, trans_l != 0, trans_r == 0, M, N, 1, &s, y, axpby(beta), &b);
 }
 
 int dyhip_gemm_tn_acc(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float* y) {

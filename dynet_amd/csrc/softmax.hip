@@ -347,6 +347,94 @@ static int launch_col_apply(dyhip_device* dev, size_t rows, unsigned cols, const
   return DYHIP_OK;
 }
 
+// ---- reductions along dim 1 (Softmax with dimension 1, LogSumExpDimension) --------------------------------
+// x is rows x cols column-major per batch element.  A block is 64 lanes (consecutive rows: coalesced) x
+// kRowWaves waves (wave w takes columns w, w + kRowWaves, ...); the per-row maximum, then the per-row sum of
+// exp(x - max), cross the waves through LDS, the sum in ascending wave order.  The second read of x comes
+// from cache for all but very large matrices.
+constexpr int kRowWaves = 8;
+
+// MODE 0: m_out = max, z_out = log(sum) + max     (TensorTools::logsumexp_dev along axis 1)
+// MODE 1: out = exp(x - max) / sum                (Softmax forward, dimension 1)
+// MODE 2: out += (b - sum_j a*b) * a              (Softmax backward, dimension 1; a = fx, b = dEdf)
+template <int MODE>
+__global__ __launch_bounds__(64 * kRowWaves) void rowwise_kernel(unsigned rows, unsigned cols, unsigned bd,
+                                                                 const float* __restrict__ a,
+                                                                 const float* __restrict__ b,
+                                                                 float* __restrict__ m_out, float* __restrict__ out) {
+  __shared__ float red[kRowWaves][64];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const unsigned row = blockIdx.x * 64 + lane;
+  const bool live = row < rows;
+  for (unsigned bi = blockIdx.y; bi < bd; bi += gridDim.y) {
+    const size_t base = size_t(bi) * rows * cols + row;
+    float mx = -INFINITY;
+    if (MODE != 2) {
+      if (live)
+        for (unsigned j = w; j < cols; j += kRowWaves) {
+          const float v = a[base + size_t(j) * rows];
+          mx = v > mx ? v : mx;  // a NaN entry is skipped here and turns the row's sum into NaN below
+        }
+      red[w][lane] = mx;
+      __syncthreads();
+      mx = red[0][lane];
+#pragma unroll
+      for (int k = 1; k < kRowWaves; ++k) {
+        const float o = red[k][lane];
+        mx = o > mx ? o : mx;
+      }
+      __syncthreads();
+    }
+    float s = 0.f;
+    if (live)
+      for (unsigned j = w; j < cols; j += kRowWaves) {
+        const size_t e = base + size_t(j) * rows;
+        s += MODE == 2 ? a[e] * b[e] : expf(a[e] - mx);
+      }
+    red[w][lane] = s;
+    __syncthreads();
+    s = red[0][lane];
+#pragma unroll
+    for (int k = 1; k < kRowWaves; ++k) s += red[k][lane];
+    __syncthreads();
+    if (!live) continue;
+    if (MODE == 0) {
+      if (w == 0) {
+        m_out[size_t(bi) * rows + row] = mx;
+        out[size_t(bi) * rows + row] = logf(s) + mx;
+      }
+    } else {
+      for (unsigned j = w; j < cols; j += kRowWaves) {
+        const size_t e = base + size_t(j) * rows;
+        if (MODE == 1) out[e] = expf(a[e] - mx) / s;
+        else out[e] += (b[e] - s) * a[e];
+      }
+    }
+  }
+}
+
+template <int MODE>
+static int launch_rowwise(dyhip_device* dev, size_t rows, size_t cols, unsigned bd, const float* a, const float* b,
+                          float* m_out, float* out) {
+  DYHIP_REQUIRE(rows < (size_t(1) << 31) && cols < (size_t(1) << 31), "matrix dimension too large");
+  const dim3 grid(static_cast<unsigned>(cdiv<size_t>(rows, 64)), bd < 65535u ? bd : 65535u);
+  hipLaunchKernelGGL(rowwise_kernel<MODE>, grid, dim3(64 * kRowWaves), 0, dev->stream, static_cast<unsigned>(rows),
+                     static_cast<unsigned>(cols), bd, a, b, m_out, out);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+// LogSumExpDimension backward: dx[i,j,b] += exp(x[i,j,b] - fx[o,b]) * dEdf[o,b], o = j (dim 0) or i (dim 1)
+__global__ __launch_bounds__(256) void lse_dim_bwd_kernel(unsigned rows, unsigned cols, size_t total, unsigned dim,
+                                                          const float* __restrict__ x, const float* __restrict__ fx,
+                                                          const float* __restrict__ dEdf, float* __restrict__ dEdx) {
+  for (size_t e = size_t(blockIdx.x) * 256 + threadIdx.x; e < total; e += size_t(gridDim.x) * 256) {
+    const size_t col = e / rows;  // column index over (cols x batch)
+    const size_t o = dim == 0 ? col : (col / cols) * rows + (e - col * rows);
+    dEdx[e] += expf(x[e] - fx[o]) * dEdf[o];
+  }
+}
+
 template <bool ACC>
 static int pnls_backward(dyhip_device* dev, size_t rows, unsigned bd, const float* x, const void* aux, const float* dEdf,
                          float* dEdx) {
@@ -506,6 +594,49 @@ int dyhip_softmax_backward(dyhip_device* dev, size_t rows, unsigned cols, const 
   hipLaunchKernelGGL(col_dot_kernel, dim3(cols), dim3(kSmThreads), 0, dev->stream, rows, fx, dEdf, r);
   DYHIP_CHECK_LAUNCH();
   return launch_col_apply<2>(dev, rows, cols, fx, dEdf, r, nullptr, dEdx);
+}
+
+int dyhip_softmax_rows_forward(dyhip_device* dev, size_t rows, size_t cols, unsigned bd, const float* x, float* fx) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(rows >= 1 && cols >= 1 && x && fx, "Softmax needs non-empty tensors");
+  if (bd == 0) return DYHIP_OK;
+  return launch_rowwise<1>(dev, rows, cols, bd, x, nullptr, nullptr, fx);
+}
+
+int dyhip_softmax_rows_backward(dyhip_device* dev, size_t rows, size_t cols, unsigned bd, const float* fx,
+                                const float* dEdf, float* dEdx) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(rows >= 1 && cols >= 1 && fx && dEdf && dEdx, "Softmax needs non-empty tensors");
+  if (bd == 0) return DYHIP_OK;
+  return launch_rowwise<2>(dev, rows, cols, bd, fx, dEdf, nullptr, dEdx);
+}
+
+int dyhip_logsumexp_dim_forward(dyhip_device* dev, size_t rows, size_t cols, unsigned bd, const float* x, unsigned dim,
+                                float* m, float* fx) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(dim <= 1, "LogSumExpDimension reduces dimension 0 or 1, got %u", dim);
+  DYHIP_REQUIRE(rows >= 1 && cols >= 1 && x && m && fx, "LogSumExpDimension needs non-empty tensors");
+  if (bd == 0) return DYHIP_OK;
+  if (dim == 0) {
+    DYHIP_REQUIRE(cols * size_t(bd) <= 0xffffffffu, "too many columns");
+    return launch_lse(dev, rows, static_cast<unsigned>(cols * bd), x, m, fx, nullptr, nullptr);
+  }
+  return launch_rowwise<0>(dev, rows, cols, bd, x, nullptr, m, fx);
+}
+
+int dyhip_logsumexp_dim_backward(dyhip_device* dev, size_t rows, size_t cols, unsigned bd, const float* x,
+                                 const float* fx, const float* dEdf, unsigned dim, float* dEdx) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(dim <= 1, "LogSumExpDimension reduces dimension 0 or 1, got %u", dim);
+  DYHIP_REQUIRE(rows >= 1 && cols >= 1 && rows < (size_t(1) << 31) && cols < (size_t(1) << 31) && x && fx && dEdf && dEdx,
+                "LogSumExpDimension needs non-empty tensors");
+  const size_t total = rows * cols * bd;
+  if (total == 0) return DYHIP_OK;
+  const size_t blocks = cdiv<size_t>(total, 256);
+  hipLaunchKernelGGL(lse_dim_bwd_kernel, dim3(static_cast<unsigned>(blocks < 65536 * 16 ? blocks : 65536 * 16)), dim3(256), 0,
+                     dev->stream, static_cast<unsigned>(rows), static_cast<unsigned>(cols), total, dim, x, fx, dEdf, dEdx);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
 }
 
 int dyhip_log_softmax_forward(dyhip_device* dev, size_t rows, unsigned cols, const float* x, void* aux, float* fx) {

@@ -348,6 +348,11 @@ class Device:
     def gemm_nt(self, M, N, K, l, r, beta, y):
         _check(cdll.dyhip_gemm_nt(self.handle, _sz(M), _sz(N), _sz(K), _p(l), _p(r), _f(beta), _p(y)))
 
+    def gemm_strided_batched(self, trans_l, trans_r, M, N, K, l, stride_l, r, stride_r, beta, y, stride_y, batch):
+        _check(cdll.dyhip_gemm_strided_batched(self.handle, _i(trans_l), _i(trans_r), _sz(M), _sz(N), _sz(K), _p(l),
+                                               _sz(stride_l), _p(r), _sz(stride_r), _f(beta), _p(y), _sz(stride_y),
+                                               _u(batch)))
+
     def gemm_tn_acc(self, M, N, K, l, r, y):
         _check(cdll.dyhip_gemm_tn_acc(self.handle, _sz(M), _sz(N), _sz(K), _p(l), _p(r), _p(y)))
 
@@ -579,6 +584,19 @@ class Device:
         ws, nb = self.workspace(4 * cols)
         _check(cdll.dyhip_softmax_backward(self.handle, _sz(rows), _u(cols), _p(fx), _p(dEdf), _p(dEdx), _vp(ws),
                                            _sz(nb)))
+
+    def softmax_rows_forward(self, rows, cols, bd, x, fx):
+        _check(cdll.dyhip_softmax_rows_forward(self.handle, _sz(rows), _sz(cols), _u(bd), _p(x), _p(fx)))
+
+    def softmax_rows_backward(self, rows, cols, bd, fx, dEdf, dEdx):
+        _check(cdll.dyhip_softmax_rows_backward(self.handle, _sz(rows), _sz(cols), _u(bd), _p(fx), _p(dEdf), _p(dEdx)))
+
+    def logsumexp_dim_forward(self, rows, cols, bd, x, dim, m, fx):
+        _check(cdll.dyhip_logsumexp_dim_forward(self.handle, _sz(rows), _sz(cols), _u(bd), _p(x), _u(dim), _p(m), _p(fx)))
+
+    def logsumexp_dim_backward(self, rows, cols, bd, x, fx, dEdf, dim, dEdx):
+        _check(cdll.dyhip_logsumexp_dim_backward(self.handle, _sz(rows), _sz(cols), _u(bd), _p(x), _p(fx), _p(dEdf),
+                                                 _u(dim), _p(dEdx)))
 
     def log_softmax_forward(self, rows, cols, x, aux, fx):
         _check(cdll.dyhip_log_softmax_forward(self.handle, _sz(rows), _u(cols), _p(x), _p(aux), _p(fx)))

@@ -230,6 +230,15 @@ int dyhip_gemm_nn(dyhip_device* dev, size_t M, size_t N, size_t K, const float* 
 int dyhip_gemm_tn_acc(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float* y);
 /* MatrixMultiplyTranspAcc (:162-180): y[MxN] += l[MxK] * r[NxK]^T */
 int dyhip_gemm_nt_acc(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float* y);
+/* The cublasSgemmStridedBatched branches of the three shims (dynet/matrix-multiply.h:27-34, 110-117,
+ * 175-182), taken when the left operand is batched: for b in [0, batch)
+ *   y_b[MxN] = beta*y_b + op(l_b) * op(r_b),   x_b = x + b*stride_x (strides in floats),
+ * with op = transpose where trans_l / trans_r is non-zero (not both) and the operand shapes of the
+ * three calls above.  A stride of 0 shares an operand between the items, as the reference passes for
+ * an operand whose batch size is 1; stride_y must be at least M*N.  One launch for all items. */
+int dyhip_gemm_strided_batched(dyhip_device* dev, int trans_l, int trans_r, size_t M, size_t N, size_t K,
+                               const float* l, size_t stride_l, const float* r, size_t stride_r, float beta, float* y,
+                               size_t stride_y, unsigned batch);
 /* the two transposed forms with an explicit beta (beta = 0 overwrites y, which saves zeroing a
  * gradient buffer that has a single producer); the cublasSgemm calls behind
  * dynet/matrix-multiply.h:104-113,169-178 take the same scalar */
@@ -400,11 +409,25 @@ int dyhip_pnls_backward_assign(dyhip_device* dev, size_t rows, unsigned bd, cons
                                const float* dEdf, float* dEdx);
 /* Softmax over dim 0 (dynet/nodes-softmaxes.cc:40-87 forward, :89-125 backward): x is rows x cols
  * with cols = columns x batch.  Forward needs 2*cols floats of scratch (the reference's z and m from
- * pools[SCS], :45-48), backward cols floats (:97-98).  Softmax along dim 1 is not provided. */
+ * pools[SCS], :45-48), backward cols floats (:97-98). */
 int dyhip_softmax_forward(dyhip_device* dev, size_t rows, unsigned cols, const float* x, float* fx, void* ws,
                           size_t ws_bytes);
 int dyhip_softmax_backward(dyhip_device* dev, size_t rows, unsigned cols, const float* fx, const float* dEdf,
                            float* dEdx, void* ws, size_t ws_bytes);
+/* Softmax over dim 1 (dynet/nodes-softmaxes.cc:74-85 forward, :114-122 backward): x is rows x cols per batch
+ * element, each row is normalised over its columns.  One kernel each, no scratch (the reference takes z and
+ * m, rows x bd floats each, from pools[SCS]). */
+int dyhip_softmax_rows_forward(dyhip_device* dev, size_t rows, size_t cols, unsigned bd, const float* x, float* fx);
+int dyhip_softmax_rows_backward(dyhip_device* dev, size_t rows, size_t cols, unsigned bd, const float* fx,
+                                const float* dEdf, float* dEdx);
+/* LogSumExpDimension (dynet/nodes-logsumexp.cc:126-145) through TensorTools::logsumexp_dev's GPU branch
+ * (dynet/tensor.cc:487-496): x is rows x cols per batch element, dim in {0, 1} is the reduced dimension;
+ * m (the reference's scratch tensor ms) and fx hold cols x bd values for dim 0, rows x bd for dim 1.
+ * backward: dEdx[i,j,b] += exp(x[i,j,b] - fx[o,b]) * dEdf[o,b], o = j for dim 0, i for dim 1. */
+int dyhip_logsumexp_dim_forward(dyhip_device* dev, size_t rows, size_t cols, unsigned bd, const float* x, unsigned dim,
+                                float* m, float* fx);
+int dyhip_logsumexp_dim_backward(dyhip_device* dev, size_t rows, size_t cols, unsigned bd, const float* x,
+                                 const float* fx, const float* dEdf, unsigned dim, float* dEdx);
 /* LogSoftmax (dynet/nodes-softmaxes.cc:141-185 forward, :187-213 backward).  aux = the node's aux_mem,
  * 2*cols floats [z | m] (:136-138); backward overwrites z with the column sums of dEdf, as the reference does. */
 int dyhip_log_softmax_forward(dyhip_device* dev, size_t rows, unsigned cols, const float* x, void* aux, float* fx);

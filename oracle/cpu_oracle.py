@@ -333,6 +333,35 @@ def softmax_backward(rows, cols, fx, dEdf, dEdx):
     return dEdx
 
 
+def softmax_rows_forward(rows, cols, bd, x):
+    """Softmax along dim 1; x and the result are (bd, cols, rows) arrays (column-major matrices per batch element)."""
+    fx = np.empty((bd, cols, rows), np.float32)
+    _check(_lib.orc_softmax_rows_forward(C.c_size_t(rows), C.c_size_t(cols), bd, _fp(_f32(x)), _fp(fx)),
+           "softmax_rows_forward")
+    return fx
+
+
+def softmax_rows_backward(rows, cols, bd, fx, dEdf, dEdx):
+    _check(_lib.orc_softmax_rows_backward(C.c_size_t(rows), C.c_size_t(cols), bd, _fp(_f32(fx)), _fp(_f32(dEdf)),
+                                          _fp(dEdx)), "softmax_rows_backward")
+    return dEdx
+
+
+def logsumexp_dim_forward(rows, cols, bd, x, dim):
+    """Returns (m, z), each (bd, cols) for dim 0 and (bd, rows) for dim 1."""
+    others = cols if dim == 0 else rows
+    m, z = np.empty((bd, others), np.float32), np.empty((bd, others), np.float32)
+    _check(_lib.orc_logsumexp_dim_forward(C.c_size_t(rows), C.c_size_t(cols), bd, _fp(_f32(x)), dim, _fp(m), _fp(z)),
+           "logsumexp_dim_forward")
+    return m, z
+
+
+def logsumexp_dim_backward(rows, cols, bd, x, fx, dEdf, dim, dEdx):
+    _check(_lib.orc_logsumexp_dim_backward(C.c_size_t(rows), C.c_size_t(cols), bd, _fp(_f32(x)), _fp(_f32(fx)),
+                                           _fp(_f32(dEdf)), dim, _fp(dEdx)), "logsumexp_dim_backward")
+    return dEdx
+
+
 def log_softmax_forward(rows, cols, x):
     """Returns (fx, aux) with aux = [z | m]."""
     fx = np.empty((cols, rows), np.float32)

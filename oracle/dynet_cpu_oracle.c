@@ -895,6 +895,76 @@ int orc_softmax_backward(size_t rows, unsigned cols, const float* fx, const floa
   return 0;
 }
 
+/* Softmax::forward_dev_impl, dimension 1 (dynet/nodes-softmaxes.cc:74-85): x is rows x cols per batch
+ * element; per (row, batch) m = max over the columns, fx = exp(x - m), z = sum over the columns, fx /= z.
+ * Pinned by scipy.special.softmax and by equality with the dimension-0 routine on the transposed matrix. */
+int orc_softmax_rows_forward(size_t rows, size_t cols, unsigned bd, const float* x, float* fx) {
+  if (rows == 0 || cols == 0) return -1;
+  for (unsigned b = 0; b < bd; ++b)
+    for (size_t i = 0; i < rows; ++i) {
+      const float* px = x + (size_t)b * rows * cols + i;
+      float* pf = fx + (size_t)b * rows * cols + i;
+      float m = px[0];
+      for (size_t j = 1; j < cols; ++j) m = px[j * rows] > m ? px[j * rows] : m;
+      for (size_t j = 0; j < cols; ++j) pf[j * rows] = expf(px[j * rows] - m);
+      float z = 0.f;
+      for (size_t j = 0; j < cols; ++j) z += pf[j * rows];
+      for (size_t j = 0; j < cols; ++j) pf[j * rows] = pf[j * rows] / z;
+    }
+  return 0;
+}
+
+/* Softmax::backward_dev_impl, dimension 1 (dynet/nodes-softmaxes.cc:114-122): per (row, batch)
+ * z = sum_j fx*dEdf; dx += (dEdf - z) * fx.  Pinned by central differences. */
+int orc_softmax_rows_backward(size_t rows, size_t cols, unsigned bd, const float* fx, const float* dEdf, float* dEdx) {
+  for (unsigned b = 0; b < bd; ++b)
+    for (size_t i = 0; i < rows; ++i) {
+      const size_t o = (size_t)b * rows * cols + i;
+      float z = 0.f;
+      for (size_t j = 0; j < cols; ++j) z += fx[o + j * rows] * dEdf[o + j * rows];
+      for (size_t j = 0; j < cols; ++j) dEdx[o + j * rows] += (dEdf[o + j * rows] - z) * fx[o + j * rows];
+    }
+  return 0;
+}
+
+/* LogSumExpDimension::forward_dev_impl (dynet/nodes-logsumexp.cc:126-132) through TensorTools::logsumexp_dev,
+ * GPU branch (dynet/tensor.cc:487-496): m = max along `dim`, z = log(sum exp(x - m)) + m.  The result has
+ * cols x bd entries for dim 0 and rows x bd for dim 1.  (The reference's CPU branch, :498-504, walks x.d[1]
+ * entries whatever the axis and is only right for square matrices; the GPU branch is the one restated.)
+ * Pinned by scipy.special.logsumexp. */
+int orc_logsumexp_dim_forward(size_t rows, size_t cols, unsigned bd, const float* x, unsigned dim, float* m, float* z) {
+  if (rows == 0 || cols == 0 || dim > 1) return -1;
+  const size_t len = dim == 0 ? rows : cols, others = dim == 0 ? cols : rows;
+  const size_t step = dim == 0 ? 1 : rows, ostep = dim == 0 ? rows : 1;
+  for (unsigned b = 0; b < bd; ++b)
+    for (size_t o = 0; o < others; ++o) {
+      const float* px = x + (size_t)b * rows * cols + o * ostep;
+      float mx = px[0];
+      for (size_t k = 1; k < len; ++k) mx = px[k * step] > mx ? px[k * step] : mx;
+      float s = 0.f;
+      for (size_t k = 0; k < len; ++k) s += expf(px[k * step] - mx);
+      m[(size_t)b * others + o] = mx;
+      z[(size_t)b * others + o] = logf(s) + mx;
+    }
+  return 0;
+}
+
+/* LogSumExpDimension::backward_dev_impl (dynet/nodes-logsumexp.cc:134-145):
+ * dx[i,j,b] += exp(x[i,j,b] - fx[o,b]) * dEdf[o,b] with o = j for dim 0 and o = i for dim 1.
+ * Pinned by central differences. */
+int orc_logsumexp_dim_backward(size_t rows, size_t cols, unsigned bd, const float* x, const float* fx,
+                               const float* dEdf, unsigned dim, float* dEdx) {
+  if (dim > 1) return -1;
+  const size_t others = dim == 0 ? cols : rows;
+  for (unsigned b = 0; b < bd; ++b)
+    for (size_t j = 0; j < cols; ++j)
+      for (size_t i = 0; i < rows; ++i) {
+        const size_t e = ((size_t)b * cols + j) * rows + i, o = (size_t)b * others + (dim == 0 ? j : i);
+        dEdx[e] += expf(x[e] - fx[o]) * dEdf[o];
+      }
+  return 0;
+}
+
 /* LogSoftmax::forward_dev_impl, CPU branch (dynet/nodes-softmaxes.cc:141-185): aux = [z | m]
  * (2*cols floats, :136-138) from TensorTools::logsumexp; fx = x - z[col]. */
 int orc_log_softmax_forward(size_t rows, unsigned cols, const float* x, float* aux, float* fx) {

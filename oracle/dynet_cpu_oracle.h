@@ -132,6 +132,11 @@ int orc_logsumexp_cols(size_t rows, unsigned bd, const float* x, float* m, float
 int orc_sum_forward(unsigned k, size_t n, unsigned bd, const float* const* xs, const unsigned* bds, float* fx);
 int orc_softmax_forward(size_t rows, unsigned cols, const float* x, float* fx);
 int orc_softmax_backward(size_t rows, unsigned cols, const float* fx, const float* dEdf, float* dEdx);
+int orc_softmax_rows_forward(size_t rows, size_t cols, unsigned bd, const float* x, float* fx);
+int orc_softmax_rows_backward(size_t rows, size_t cols, unsigned bd, const float* fx, const float* dEdf, float* dEdx);
+int orc_logsumexp_dim_forward(size_t rows, size_t cols, unsigned bd, const float* x, unsigned dim, float* m, float* z);
+int orc_logsumexp_dim_backward(size_t rows, size_t cols, unsigned bd, const float* x, const float* fx,
+                               const float* dEdf, unsigned dim, float* dEdx);
 int orc_log_softmax_forward(size_t rows, unsigned cols, const float* x, float* aux, float* fx);
 int orc_log_softmax_backward(size_t rows, unsigned cols, const float* fx, const float* dEdf, float* dEdx);
 int orc_pnls_forward(size_t rows, unsigned bd, const float* x, const unsigned* labels,

@@ -472,6 +472,34 @@ static void cwise_broadcast(Fixture& F) {
     for (float e : as_vector(y)) z += e;
     CHECK_CLOSE(z, -6.5, 0.001);
   }
+  g_case = "softmax_logsumexp_dims_gradient";  // tests/test-nodes.cc: softmax_cols_gradient, logsumexp_dim_gradient
+  for (unsigned dim : {0u, 1u}) {
+    const vector<float> sq = {1.1f, 2.2f, 3.4f, 1.2f, 2.5f, 3.2f, 5.3f, 2.3f, 3.3f, -0.4f, 0.6f, 1.7f};
+    { vector<Tensor> a = {F.input(Dim({3, 2}, 2), sq)}; CHECK(check_grad(F, Softmax(dim), a, Dim({3, 2}, 2), {true})); }
+    { vector<Tensor> a = {F.input(Dim({3, 2}, 2), sq)};
+      CHECK(check_grad(F, LogSumExpDimension(dim), a, dim == 0 ? Dim({2}, 2) : Dim({3}, 2), {true})); }
+    F.reset();
+  }
+  g_case = "matmul_batched_left_gradient";  // MatrixMultiply with a batched left operand, all three shims
+  {
+    struct MatMul : public Node {
+      void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+        MatrixMultiply(dev, *xs[0], *xs[1], fx, dev.kSCALAR_ZERO);
+      }
+      void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, const Tensor&, const Tensor& dEdf,
+                             unsigned i, Tensor& dEdxi) const override {
+        if (i == 0) MatrixMultiplyTranspAcc(dev, dEdf, *xs[1], dEdxi);
+        else MatrixTranspMultiplyAcc(dev, *xs[0], dEdf, dEdxi);
+      }
+    };
+    const vector<float> lv = {1.1f, -2.2f, 3.3f, 0.4f, 0.5f, -0.6f, 0.7f, 0.8f, -0.9f, 1.0f, 1.2f, -1.3f};
+    const vector<float> rv = {0.3f, -0.2f, 0.5f, 0.7f, -1.1f, 0.9f, 0.2f, 0.4f};
+    { vector<Tensor> a = {F.input(Dim({3, 2}, 2), lv), F.input(Dim({2, 2}, 2), rv)};
+      CHECK(check_grad(F, MatMul(), a, Dim({3, 2}, 2), {true, true})); }
+    { vector<Tensor> a = {F.input(Dim({3, 2}, 2), lv), F.input(Dim({2, 2}), {0.3f, -0.2f, 0.5f, 0.7f})};
+      CHECK(check_grad(F, MatMul(), a, Dim({3, 2}, 2), {true, false})); }
+    F.reset();
+  }
   g_case = "addscalar_gradient";
   { vector<Tensor> a = {F.input(Dim({3}), param1)}; CHECK(check_grad(F, ConstantPlusX(2.0f), a, Dim({3}), {true})); }
   g_case = "scalarsubtract_gradient";

@@ -46,6 +46,42 @@ def test_gemm_three_forms(dev, M, N, K):
     assert_close(yt.numpy(), orc.gemm_nt_acc(M, N, K, l, r2, y0.copy()), FWD_RTOL, "gemm_nt", floor=floor)
 
 
+@pytest.mark.parametrize("M,N,K,B", [(64, 48, 32, 5), (130, 70, 33, 3), (7, 5, 3, 17), (256, 128, 256, 4), (31, 1, 9, 2)])
+def test_gemm_strided_batched(dev, M, N, K, B):
+    """The batched-left-operand branches of the three GEMM shims: per batch item the plain product, as the
+    reference's CPU path loops it (dynet/matrix-multiply.h:90-93, 148-150, 213-215)."""
+    rng = np.random.default_rng(M + 3 * N + 5 * K + B)
+    floor = np.sqrt(K)
+    y0 = f32(rng.standard_normal((B, N, M)))
+    l, r = f32(rng.standard_normal((B, K, M))), f32(rng.standard_normal((B, N, K)))
+    lT, rT = f32(rng.standard_normal((B, M, K))), f32(rng.standard_normal((B, K, N)))
+    # l * r, both batched, beta 0 and 1; then with r shared by the items (stride 0)
+    for beta in (0.0, 1.0):
+        yt = dev.tensor(y0)
+        dev.gemm_strided_batched(0, 0, M, N, K, dev.tensor(l), M * K, dev.tensor(r), K * N, beta, yt, M * N, B)
+        want = np.stack([orc.gemm_nn(M, N, K, l[b], r[b], beta, y0[b].copy()) for b in range(B)])
+        assert_close(yt.numpy(), want, FWD_RTOL, "batched l*r beta=%g" % beta, floor=floor)
+    yt = dev.tensor(y0)
+    dev.gemm_strided_batched(0, 0, M, N, K, dev.tensor(l), M * K, dev.tensor(r[0]), 0, 1.0, yt, M * N, B)
+    want = np.stack([orc.gemm_nn(M, N, K, l[b], r[0], 1.0, y0[b].copy()) for b in range(B)])
+    assert_close(yt.numpy(), want, FWD_RTOL, "batched l*r, shared r", floor=floor)
+    # l^T * r
+    yt = dev.tensor(y0)
+    dev.gemm_strided_batched(1, 0, M, N, K, dev.tensor(lT), M * K, dev.tensor(r), K * N, 1.0, yt, M * N, B)
+    want = np.stack([orc.gemm_tn_acc(M, N, K, lT[b], r[b], y0[b].copy()) for b in range(B)])
+    assert_close(yt.numpy(), want, FWD_RTOL, "batched l^T*r", floor=floor)
+    # l * r^T with l shared
+    yt = dev.tensor(y0)
+    dev.gemm_strided_batched(0, 1, M, N, K, dev.tensor(l[1]), 0, dev.tensor(rT), K * N, 1.0, yt, M * N, B)
+    want = np.stack([orc.gemm_nt_acc(M, N, K, l[1], rT[b], y0[b].copy()) for b in range(B)])
+    assert_close(yt.numpy(), want, FWD_RTOL, "batched l*r^T, shared l", floor=floor)
+    # overlapping outputs and the doubly transposed form are refused
+    with pytest.raises(DyhipError):
+        dev.gemm_strided_batched(0, 0, M, N, K, dev.tensor(l), M * K, dev.tensor(r), K * N, 0.0, yt, M * N - 1, B)
+    with pytest.raises(DyhipError):
+        dev.gemm_strided_batched(1, 1, M, N, K, dev.tensor(l), M * K, dev.tensor(r), K * N, 0.0, yt, M * N, B)
+
+
 def test_gemm_is_fp32_accurate_against_fp64(dev):
     """No reduced-precision shortcut on the matrix cores: error vs fp64 stays at fp32 rounding level."""
     rng = np.random.default_rng(5)
@@ -1134,3 +1170,35 @@ def test_zero_any_alignment_and_inside_a_graph(dev):
         want[6:6 + 999] = 0
         assert np.array_equal(buf.numpy().view(np.uint8), want)
     g.destroy()
+
+
+@pytest.mark.parametrize("rows,cols,bd", [(7, 5, 3), (64, 100, 2), (130, 9, 1), (1, 300, 4), (1000, 33, 2), (3, 1, 5)])
+def test_softmax_and_logsumexp_along_dim_1(dev, rows, cols, bd):
+    rng = np.random.default_rng(rows + cols + bd)
+    x = f32(rng.standard_normal((bd, cols, rows)) * 3)
+    xt = dev.tensor(x)
+    fx = dev.empty((bd, cols, rows))
+    dev.softmax_rows_forward(rows, cols, bd, xt, fx)
+    ref = orc.softmax_rows_forward(rows, cols, bd, x)
+    assert_close(fx.numpy(), ref, FWD_RTOL, "softmax dim 1", floor=1.0 / cols)
+    np.testing.assert_allclose(fx.numpy().sum(axis=1), 1.0, rtol=1e-5)
+    dy = f32(rng.standard_normal((bd, cols, rows)))
+    dx0 = f32(rng.standard_normal((bd, cols, rows)))
+    dxt = dev.tensor(dx0)
+    dev.softmax_rows_backward(rows, cols, bd, dev.tensor(ref), dev.tensor(dy), dxt)
+    assert_close(dxt.numpy(), orc.softmax_rows_backward(rows, cols, bd, ref, dy, dx0.copy()), GRAD_RTOL, "softmax dim 1 bwd",
+                 floor=1.0)
+    for dim in (0, 1):
+        others = cols if dim == 0 else rows
+        m, z = dev.empty((bd, others)), dev.empty((bd, others))
+        dev.logsumexp_dim_forward(rows, cols, bd, xt, dim, m, z)
+        rm, rz = orc.logsumexp_dim_forward(rows, cols, bd, x, dim)
+        assert m.numpy().tobytes() == rm.tobytes()
+        assert_close(z.numpy(), rz, FWD_RTOL, "logsumexp dim %d" % dim, floor=1.0)
+        dz = f32(rng.standard_normal((bd, others)))
+        dxt = dev.tensor(dx0)
+        dev.logsumexp_dim_backward(rows, cols, bd, xt, dev.tensor(rz), dev.tensor(dz), dim, dxt)
+        assert_close(dxt.numpy(), orc.logsumexp_dim_backward(rows, cols, bd, x, rz, dz, dim, dx0.copy()), GRAD_RTOL,
+                     "logsumexp dim %d bwd" % dim, floor=1.0)
+    with pytest.raises(DyhipError):
+        dev.logsumexp_dim_forward(rows, cols, bd, xt, 2, m, z)

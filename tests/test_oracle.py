@@ -944,3 +944,47 @@ def test_pick_range_is_a_numpy_slice(dim):
         orc.pick_range_forward(inner, d[dim], outer, 3, 3, x)
     with pytest.raises(ValueError):
         orc.pick_range_forward(inner, d[dim], outer, 0, d[dim] + 1, x)
+
+
+def test_softmax_along_dim_1_and_logsumexp_dim_against_scipy():
+    """Pins: scipy.special.softmax / logsumexp in fp64; the dimension-1 softmax equals the dimension-0 routine
+    on the transposed matrices; backward by central differences in fp64."""
+    from scipy.special import logsumexp, softmax
+
+    rng = np.random.default_rng(77)
+    rows, cols, bd = 7, 5, 3
+    x = (rng.standard_normal((bd, cols, rows)) * 3).astype(np.float32)  # [b][j][i]: column-major matrices
+    fx = orc.softmax_rows_forward(rows, cols, bd, x)
+    np.testing.assert_allclose(fx, softmax(x.astype(np.float64), axis=1), rtol=2e-6, atol=1e-9)
+    xt = np.ascontiguousarray(x.transpose(0, 2, 1))  # rows <-> cols
+    via_dim0 = orc.softmax_forward(cols, rows * bd, xt.reshape(bd * rows, cols)).reshape(bd, rows, cols)
+    assert np.array_equal(fx, via_dim0.transpose(0, 2, 1))
+    for dim, axis in ((0, 2), (1, 1)):
+        m, z = orc.logsumexp_dim_forward(rows, cols, bd, x, dim)
+        np.testing.assert_allclose(z, logsumexp(x.astype(np.float64), axis=axis), rtol=2e-6)
+        assert np.array_equal(m, x.max(axis=axis))
+    m0, z0 = orc.logsumexp_dim_forward(rows, cols, bd, x, 0)
+    m_c, z_c = orc.logsumexp_cols(rows, cols * bd, x.reshape(bd * cols, rows))
+    assert np.array_equal(z0.ravel(), z_c) and np.array_equal(m0.ravel(), m_c)
+    # gradients: loss = sum w * f(x), central differences in fp64
+    w = rng.standard_normal((bd, cols, rows))
+    g = orc.softmax_rows_backward(rows, cols, bd, fx, w.astype(np.float32), np.zeros((bd, cols, rows), np.float32))
+    x64, h = x.astype(np.float64), 1e-6
+    num = np.zeros_like(x64)
+    for idx in np.ndindex(x64.shape):
+        xp, xm = x64.copy(), x64.copy()
+        xp[idx] += h
+        xm[idx] -= h
+        num[idx] = ((softmax(xp, axis=1) - softmax(xm, axis=1)) * w.astype(np.float32)).sum() / (2 * h)
+    np.testing.assert_allclose(g, num, rtol=2e-4, atol=2e-5)
+    for dim, axis in ((0, 2), (1, 1)):
+        m, z = orc.logsumexp_dim_forward(rows, cols, bd, x, dim)
+        wz = rng.standard_normal(z.shape).astype(np.float32)
+        g = orc.logsumexp_dim_backward(rows, cols, bd, x, z, wz, dim, np.zeros((bd, cols, rows), np.float32))
+        num = np.zeros_like(x64)
+        for idx in np.ndindex(x64.shape):
+            xp, xm = x64.copy(), x64.copy()
+            xp[idx] += h
+            xm[idx] -= h
+            num[idx] = ((logsumexp(xp, axis=axis) - logsumexp(xm, axis=axis)) * wz).sum() / (2 * h)
+        np.testing.assert_allclose(g, num, rtol=2e-4, atol=2e-5)
