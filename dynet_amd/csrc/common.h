@@ -35,6 +35,7 @@ struct MemAllocator {
   virtual bool zero(void* p, size_t n) = 0;
   size_t round_up_align(size_t n) const { return align < 2 ? n : ((n + align - 1) / align) * align; }
   const size_t align;
+  const char* refusal = nullptr;  // set by malloc when it declines for a reason other than exhaustion
 };
 
 }  // namespace dyhip

@@ -55,7 +55,17 @@ struct HipAllocator : MemAllocator {
   HipAllocator(int ordinal, hipStream_t stream) : MemAllocator(256), ordinal(ordinal), stream(stream) {}
   void* malloc(size_t n) override {
     void* p = nullptr;
+    refusal = nullptr;
     if (hipSetDevice(ordinal) != hipSuccess) return nullptr;
+    // A block allocated while a graph is being recorded would be zeroed and freed outside the recorded
+    // order (and the queues forked from this device record into the same capture): pools are sized before
+    // a capture begins, growth inside one is refused.
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess) (void)hipGetLastError();
+    if (cap != hipStreamCaptureStatusNone) {
+      refusal = "a memory pool cannot grow while a graph capture is in progress; allocate before the capture";
+      return nullptr;
+    }
     if (hipMalloc(&p, n) != hipSuccess) {
       (void)hipGetLastError();
       return nullptr;
@@ -63,7 +73,15 @@ struct HipAllocator : MemAllocator {
     return p;
   }
   void free(void* p) override { (void)hipFree(p); }
-  bool zero(void* p, size_t n) override { return zero_fill(p, n, stream) == hipSuccess; }
+  // The fill runs on the device's own stream; queues forked from the device share the pools, so the call
+  // returns only once the block is zero: whatever any queue launches afterwards finds it cleared.
+  bool zero(void* p, size_t n) override {
+    if (zero_fill(p, n, stream) != hipSuccess) return false;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess) (void)hipGetLastError();
+    if (cap != hipStreamCaptureStatusNone) return true;  // pool_zero_allocated inside a capture: recorded in order
+    return hipStreamSynchronize(stream) == hipSuccess;
+  }
   int ordinal;
   hipStream_t stream;
 };
@@ -88,8 +106,10 @@ static int pool_add_block(dyhip_pool* pool, size_t cap) {
   blk.capacity = pool->alloc->round_up_align(cap);
   blk.mem = static_cast<char*>(pool->alloc->malloc(blk.capacity));
   blk.used = 0;
-  if (blk.mem == nullptr)
+  if (blk.mem == nullptr) {
+    if (pool->alloc->refusal != nullptr) return fail(DYHIP_ERR_RUNTIME, "%s: %s", pool->name.c_str(), pool->alloc->refusal);
     return fail(DYHIP_ERR_OUT_OF_MEMORY, "%s failed to allocate %zu bytes", pool->name.c_str(), blk.capacity);
+  }
   if (!pool->alloc->zero(blk.mem, blk.capacity)) {
     pool->alloc->free(blk.mem);
     return fail(DYHIP_ERR_RUNTIME, "%s failed to zero %zu bytes", pool->name.c_str(), blk.capacity);
@@ -172,9 +192,18 @@ int dyhip_pool_free(dyhip_pool* pool) {
   if (pool->blocks.size() > 1) {
     // consolidate: one block of the total capacity, so that the next graph of
     // the same size fits without growing again
-    for (auto& b : pool->blocks) pool->alloc->free(b.mem);
-    pool->blocks.clear();
-    DYHIP_CHECK_STATUS(pool_add_block(pool, pool->cap));
+    // The consolidated block is allocated before the old ones are released: if that fails the pool
+    // keeps its blocks (emptied) and stays usable.
+    std::vector<dyhip_pool::Block> old;
+    old.swap(pool->blocks);
+    const int st = pool_add_block(pool, pool->cap);
+    if (st != DYHIP_OK) {
+      pool->blocks.swap(old);
+      for (auto& b : pool->blocks) b.used = 0;
+      // allocation continues from the newest block, as after growth
+      return st;
+    }
+    for (auto& b : old) pool->alloc->free(b.mem);
   }
   pool->blocks[0].used = 0;
   return DYHIP_OK;

@@ -13,35 +13,44 @@ namespace dyhip {
 
 static size_t align256(size_t n) { return (n + 255) / 256 * 256; }
 
+// A gradient norm that is NaN or infinite gives scale 0, which the update kernels below read as "leave the
+// parameters alone": Trainer::clip_gradients throws in that case (dynet/training.cc:176-180), a kernel cannot,
+// so the step is skipped on the device and the norm slot lets the host raise the error when it looks.
 __global__ void clip_scale_kernel(unsigned n, const float* __restrict__ sqnorms, float threshold,
-                                  float* __restrict__ gscale) {
+                                  float* __restrict__ gscale, float* __restrict__ norm) {
   if (threadIdx.x != 0 || blockIdx.x != 0) return;
   float s = 0.f;
   for (unsigned i = 0; i < n; ++i) s += sqnorms[i];
   const float gg = sqrtf(s);
-  *gscale = (threshold > 0.f && gg > threshold) ? threshold / gg : 1.0f;
+  const bool finite = gg - gg == 0.f;
+  *gscale = !finite ? 0.0f : (threshold > 0.f && gg > threshold) ? threshold / gg : 1.0f;
+  if (norm != nullptr) *norm = gg;
 }
 
 template <bool CLEAR>
 __global__ __launch_bounds__(256) void sgd_scaled_kernel(size_t n4, size_t n, float* __restrict__ p,
                                                          float* __restrict__ g, float lr, float wd,
                                                          const float* __restrict__ gscale) {
-  const float s = lr * *gscale / wd;
+  const float gs = *gscale;
+  const bool skip = gs == 0.f;  // non-finite gradient norm: the parameters stay as they are
+  const float s = lr * gs / wd;
   const size_t stride = size_t(gridDim.x) * 256;
   float4* p4 = reinterpret_cast<float4*>(p);
   float4* g4 = reinterpret_cast<float4*>(g);
   for (size_t i = size_t(blockIdx.x) * 256 + threadIdx.x; i < n4; i += stride) {
-    float4 pv = p4[i];
-    const float4 gv = g4[i];
-    pv.x -= gv.x * s;
-    pv.y -= gv.y * s;
-    pv.z -= gv.z * s;
-    pv.w -= gv.w * s;
-    p4[i] = pv;
+    if (!skip) {
+      float4 pv = p4[i];
+      const float4 gv = g4[i];
+      pv.x -= gv.x * s;
+      pv.y -= gv.y * s;
+      pv.z -= gv.z * s;
+      pv.w -= gv.w * s;
+      p4[i] = pv;
+    }
     if (CLEAR) g4[i] = make_float4(0.f, 0.f, 0.f, 0.f);
   }
   for (size_t i = (n4 << 2) + size_t(blockIdx.x) * 256 + threadIdx.x; i < n; i += stride) {
-    p[i] -= g[i] * s;
+    if (!skip) p[i] -= g[i] * s;
     if (CLEAR) g[i] = 0.f;
   }
 }
@@ -54,11 +63,12 @@ __global__ __launch_bounds__(128) void sgd_rows_kernel(unsigned n, const unsigne
   const unsigned k = blockIdx.x;
   const unsigned id = sorted_ids[k];
   if (id >= vocab || (k > 0 && sorted_ids[k - 1] == id)) return;
-  const float s = lr * *gscale / wd;
+  const float gs = *gscale;
+  const float s = lr * gs / wd;
   float* pv = values + size_t(id) * dim;
   float* pg = grads + size_t(id) * dim;
   for (unsigned j = threadIdx.x; j < dim; j += 128) {
-    pv[j] -= pg[j] * s;
+    if (gs != 0.f) pv[j] -= pg[j] * s;
     pg[j] = 0.f;
   }
 }
@@ -95,12 +105,17 @@ using namespace dyhip;
 
 extern "C" {
 
-int dyhip_clip_scale(dyhip_device* dev, unsigned n, const float* sqnorms, float threshold, float* gscale) {
+int dyhip_clip_scale_norm(dyhip_device* dev, unsigned n, const float* sqnorms, float threshold, float* gscale,
+                          float* norm) {
   DYHIP_CHECK_DEV(dev);
   DYHIP_REQUIRE(gscale != nullptr && (n == 0 || sqnorms != nullptr), "null pointer");
-  hipLaunchKernelGGL(clip_scale_kernel, dim3(1), dim3(64), 0, dev->stream, n, sqnorms, threshold, gscale);
+  hipLaunchKernelGGL(clip_scale_kernel, dim3(1), dim3(64), 0, dev->stream, n, sqnorms, threshold, gscale, norm);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
+}
+
+int dyhip_clip_scale(dyhip_device* dev, unsigned n, const float* sqnorms, float threshold, float* gscale) {
+  return dyhip_clip_scale_norm(dev, n, sqnorms, threshold, gscale, nullptr);
 }
 
 int dyhip_sgd_update_scaled(dyhip_device* dev, size_t n, float* p, float* g, float lr, const float* gscale,

@@ -647,8 +647,8 @@ class Device:
     def sgd_update(self, n, p, g, lr, gscale=1.0, wd=1.0):
         _check(cdll.dyhip_sgd_update(self.handle, _sz(n), _p(p), _p(g), _f(lr), _f(gscale), _f(wd)))
 
-    def clip_scale(self, n, sqnorms, threshold, gscale):
-        _check(cdll.dyhip_clip_scale(self.handle, _u(n), _p(sqnorms), _f(threshold), _p(gscale)))
+    def clip_scale(self, n, sqnorms, threshold, gscale, norm=None):
+        _check(cdll.dyhip_clip_scale_norm(self.handle, _u(n), _p(sqnorms), _f(threshold), _p(gscale), _p(norm)))
 
     def sgd_update_scaled(self, n, p, g, lr, gscale_dev, wd=1.0, clear_grad=True):
         _check(cdll.dyhip_sgd_update_scaled(self.handle, _sz(n), _p(p), _p(g), _f(lr), _p(gscale_dev), _f(wd),

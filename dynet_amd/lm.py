@@ -60,6 +60,7 @@ class LstmLM:
         self.g["C"] = dev.zeros(params["C"].shape, pool=PS)
         self.sqnorms = dev.zeros((2,), pool=PS)  # [dense slab, touched lookup rows]
         self.gscale = dev.zeros((1,), pool=PS)
+        self.gnorm = dev.zeros((1,), pool=PS)  # gradient norm of the last step, for the host to check
         # forward values (FXS pool); [t] slices are contiguous so [T, B, *] is one matrix with T*B columns
         self.ids = dev.empty((N,), np.uint32, pool=FXS)
         self.emb = dev.empty((T, B, E), pool=FXS)
@@ -322,7 +323,7 @@ class LstmLM:
         d = self.dev
         d.squared_l2norm(self.dense_elems, self.g_dense, self.sqnorms.offset(0, (1,)))
         d.squared_l2norm_rows(self.N, self.plan, self.E, self.V, self.g["C"], self.sqnorms.offset(1, (1,)))
-        d.clip_scale(2, self.sqnorms, self.clip, self.gscale)
+        d.clip_scale(2, self.sqnorms, self.clip, self.gscale, self.gnorm)
         d.sgd_update_scaled(self.dense_elems, self.p_dense, self.g_dense, self.lr, self.gscale, 1.0, True)
         d.sgd_update_rows(self.N, self.plan, self.E, self.V, self.p["C"], self.g["C"], self.lr, self.gscale, 1.0)
 
@@ -350,8 +351,17 @@ class LstmLM:
         else:
             self.issue()
         if read_loss:
+            self.check_gradient_norm()
             return float(self.loss.numpy()[0])
         return None
+
+    def check_gradient_norm(self):
+        """Trainer::clip_gradients's check (dynet/training.cc:176-180), made when the host looks: a step whose
+        gradient norm was NaN or infinite has already been dropped on the device."""
+        nrm = float(self.gnorm.numpy()[0])
+        if not np.isfinite(nrm):
+            raise RuntimeError("Magnitude of gradient is bad: %r" % nrm)
+        return nrm
 
     def get_params(self):
         return {n: t.numpy() for n, t in self.p.items()}

@@ -461,6 +461,13 @@ int dyhip_sgd_update(dyhip_device* dev, size_t n, float* p, const float* g, floa
  * device-to-host copy of dynet/model.cc:830-842: *gscale (device) = min(1, threshold /
  * sqrt(sum of the n squared norms)); threshold <= 0 disables clipping (gscale = 1). */
 int dyhip_clip_scale(dyhip_device* dev, unsigned n, const float* sqnorms, float threshold, float* gscale);
+/* The same, also storing the gradient norm in *norm (device, may be null).  Where the reference throws
+ * "Magnitude of gradient is bad" for a NaN or infinite norm (dynet/training.cc:176-180), both forms set
+ * *gscale = 0, and dyhip_sgd_update_scaled / dyhip_sgd_update_rows given a scale of 0 leave the parameters
+ * untouched (gradients are still cleared): the diverged step is dropped on the device, and the host raises
+ * the reference's error when it reads a non-finite *norm. */
+int dyhip_clip_scale_norm(dyhip_device* dev, unsigned n, const float* sqnorms, float threshold, float* gscale,
+                          float* norm);
 /* the SGD rule with gscale read on the device; clear_grad != 0 also zeroes g (ParameterStorage::clear) */
 int dyhip_sgd_update_scaled(dyhip_device* dev, size_t n, float* p, float* g, float lr, const float* gscale,
                             float wd, int clear_grad);

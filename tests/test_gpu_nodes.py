@@ -942,6 +942,21 @@ def test_device_side_clipping_and_sparse_rows(dev):
     assert g2t.numpy().tobytes() == g2.tobytes()
     dev.sgd_update_scaled(1000, pt, g2t, 0.1, scale, 1.0, clear_grad=True)
     assert not g2t.numpy().any()
+    # a NaN or infinite gradient norm: scale 0, the norm is reported, and the updates leave the parameters alone
+    norm = dev.empty(1)
+    dev.clip_scale(2, sq, 5.0, scale, norm)
+    assert abs(float(norm.numpy()[0]) - total) < 1e-5 * total and scale.numpy()[0] == s
+    for bad in (np.nan, np.inf):
+        dev.clip_scale(2, dev.tensor(np.array([1.0, bad], F32)), 5.0, scale, norm)
+        assert scale.numpy()[0] == 0.0
+        assert np.isnan(norm.numpy()[0]) if np.isnan(bad) else np.isinf(norm.numpy()[0])
+        before, before_t = pt.numpy().copy(), tt.numpy().copy()
+        g_bad = dev.tensor(np.full(1000, bad, F32))
+        dev.sgd_update_scaled(1000, pt, g_bad, 0.1, scale, 1.0, clear_grad=True)
+        assert pt.numpy().tobytes() == before.tobytes() and not g_bad.numpy().any()
+        gt.set(np.full((vocab, dim), bad, F32))
+        dev.sgd_update_rows(n, plan, dim, vocab, tt, gt, 0.1, scale, 1.0)
+        assert tt.numpy().tobytes() == before_t.tobytes()
 
 
 def test_zero_sized_calls_are_no_ops(dev):
@@ -1202,3 +1217,37 @@ def test_softmax_and_logsumexp_along_dim_1(dev, rows, cols, bd):
                      "logsumexp dim %d bwd" % dim, floor=1.0)
     with pytest.raises(DyhipError):
         dev.logsumexp_dim_forward(rows, cols, bd, xt, 2, m, z)
+
+
+def test_pool_growth_is_ordered_with_forked_queues_and_refused_inside_a_capture(gpu):
+    """A pool that grows zero-fills its new block before any queue can use it; growth while a graph is being
+    recorded is refused with a clear error and leaves the capture usable."""
+    from dynet_amd import Device
+
+    gpu.sync()
+    d = Device(0, mem_mb=(1, 1, 1, 1))
+    try:
+        small = d.empty(100)
+        d.graph_begin()
+        with pytest.raises(DyhipError, match="capture"):
+            d.empty(1 << 20)  # 4 MB from a 1 MB pool: would have to grow
+        d.constant(small, 2.0)
+        g = d.graph_end()
+        g.launch()
+        d.sync()
+        assert np.all(small.numpy() == F32(2.0))
+        g.destroy()
+        q = d.fork()
+        big = q.empty(1 << 21)  # the shared pool grows through the forked queue ...
+        q.constant(big, 1.0)    # ... whose next kernel must find the block already cleared
+        q.sync()
+        d.sync()
+        assert np.all(big.numpy() == F32(1.0))
+        fresh = d.empty(1 << 22)
+        assert not fresh.numpy().any()
+        d.sync()
+        d.free_pool(lib.POOL_FXS)  # consolidates the blocks into one
+        again = d.empty(1 << 22)
+        assert not again.numpy().any()
+    finally:
+        d.close()
