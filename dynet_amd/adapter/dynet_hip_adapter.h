@@ -226,12 +226,22 @@ struct Node {
 };
 
 // dynet/nodes-lstm.h:9-26, nodes-lstm.cc:101-527.  xs = {x_t[0..k), h_tm1, Wx, Wh, b [, mask_x, mask_h]}
+//
+// The executor calls backward once per differentiable argument with the same dEdf; the activation
+// derivative dpre = dEdf * act'(fx) (dynet/nodes-lstm.cc:358-361) is the same for all of them.  When the
+// node was given aux_mem (aux_storage_size() = one fx-sized tensor, requested by passing the output
+// dimension to the constructor), the first backward call stores dpre there and the others reuse it;
+// forward invalidates it.  Without aux_mem every call recomputes dpre.
 struct VanillaLSTMGates : public Node {
-  VanillaLSTMGates(bool dropout, real weightnoise_std) : dropout(dropout), weightnoise_std(weightnoise_std) {}
+  VanillaLSTMGates(bool dropout, real weightnoise_std, const Dim& dim = Dim())
+      : dropout(dropout), weightnoise_std(weightnoise_std), dim(dim) {}
   bool dropout;
   real weightnoise_std;
+  Dim dim;  // the node's output dimension ({4H}, B) when the dpre cache is wanted
+  size_t aux_storage_size() const override { return dim.nd ? dim.size() * sizeof(float) : 0; }
 
   void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    dpre_of_ = nullptr;
     Args a = unpack(xs);
     size_t need = 0;
     abi_check(dyhip_lstm_gates_workspace(a.k, a.I, a.H, a.B, dropout, &need));
@@ -248,13 +258,22 @@ struct VanillaLSTMGates : public Node {
     size_t need = 0;
     abi_check(dyhip_lstm_gates_backward_workspace(a.k, a.I, a.H, a.B, dropout, &need));
     void* ws = scratch(fx)->allocate(need);
+    const float* dpre = nullptr;
+    if (aux_mem != nullptr && dim.nd && dim.size() == fx.d.size()) {
+      if (dpre_of_ != dEdf.v) {
+        abi_check(dyhip_lstm_gates_dpre(dev.hip, a.H, a.B, fx.v, dEdf.v, static_cast<float*>(aux_mem)));
+        dpre_of_ = dEdf.v;
+      }
+      dpre = static_cast<const float*>(aux_mem);
+    }
     abi_check(dyhip_lstm_gates_backward(dev.hip, a.k, a.x.data(), a.xd.data(), a.H, a.B, xs[a.k]->v, xs[a.k + 1]->v,
-                                        xs[a.k + 2]->v, a.mx, a.mx_bd, a.mh, a.mh_bd, fx.v, dEdf.v, nullptr, i,
+                                        xs[a.k + 2]->v, a.mx, a.mx_bd, a.mh, a.mh_bd, fx.v, dEdf.v, dpre, i,
                                         dEdxi.v, ws, need));
     scratch(fx)->free();
   }
 
  private:
+  mutable const float* dpre_of_ = nullptr;  // the dEdf whose dpre sits in aux_mem
   struct Args {
     unsigned k, I, H, B, mx_bd, mh_bd;
     std::vector<const float*> x;

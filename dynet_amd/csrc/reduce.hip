@@ -33,6 +33,15 @@ struct BrPlan {
 
 static BrPlan br_plan(size_t n, unsigned bd, bool vec_ok) {
   BrPlan p;
+  // A reduction of at most 4 MB is bound by launches, not bytes: one launch of scalar tiles (four times as
+  // many blocks as vector tiles) beats split partial sums plus a combining launch when there are enough of them.
+  if (n * size_t(bd) <= (size_t(1) << 20) && n >= 32 * 64) {
+    p.vec = 1;
+    p.tiles = static_cast<unsigned>(cdiv<size_t>(n, 64));
+    p.splits = 1;
+    p.per_split = bd;
+    return p;
+  }
   p.vec = vec_ok ? 4 : 1;
   p.tiles = static_cast<unsigned>(cdiv<size_t>(n, size_t(64) * p.vec));
   unsigned want = p.tiles >= 192 ? 1u : cdiv<unsigned>(512u, p.tiles);

@@ -203,6 +203,27 @@ static void lstm_node_gradients(Fixture& F) {
                         F.input(Dim({hidden_dim * 4, input_dim}), Wx60), F.input(Dim({hidden_dim * 4, hidden_dim}), Wh36),
                         F.input(Dim({hidden_dim * 4}), b12)};
     CHECK(check_grad(F, VanillaLSTMGates(false, 0.f), a, Dim({hidden_dim * 4}, batch_size), {true, true, true, true, true}));
+    // the same with the activation derivative cached in aux_mem across the five backward calls
+    g_case = "lstm_node_gates_bwd_cached_dpre";
+    const Dim gd({hidden_dim * 4}, batch_size);
+    VanillaLSTMGates cached(false, 0.f, gd);
+    CHECK(cached.aux_storage_size() == gd.size() * sizeof(float));
+    Tensor aux = F.dev.allocate_tensor(DeviceMempool::FXS, gd);
+    cached.aux_mem = aux.v;
+    CHECK(check_grad(F, cached, a, gd, {true, true, true, true, true}));
+    // and call by call against the uncached node, bit for bit
+    VanillaLSTMGates plain(false, 0.f);
+    vector<const Tensor*> xs;
+    for (Tensor& t : a) xs.push_back(&t);
+    Tensor fx = F.dev.allocate_tensor(DeviceMempool::FXS, gd), dEdf = F.input(gd, cycle(gd.size(), {0.3f, -0.2f, 0.5f, 0.1f, -0.4f}), DeviceMempool::DEDFS);
+    plain.forward_dev_impl(F.dev, xs, fx);
+    cached.forward_dev_impl(F.dev, xs, fx);
+    for (unsigned i = 0; i < 5; ++i) {
+      Tensor g0 = F.zeros(a[i].d), g1 = F.zeros(a[i].d);
+      plain.backward_dev_impl(F.dev, xs, fx, dEdf, i, g0);
+      cached.backward_dev_impl(F.dev, xs, fx, dEdf, i, g1);
+      CHECK(as_vector(g0) == as_vector(g1));
+    }
   }
   g_case = "lstm_node_gates_dropout_bwd";
   {
