@@ -554,8 +554,9 @@ def lstm_lm(steps, warmup=3, use_graph=True):
                       "clip_threshold": 5.0, "init": "Glorot (lookup: embedding dim only), LSTM biases 0",
                       "ids": "Zipf(1.1)"},
            "tokens_per_step": T * B, "gemm_flop_per_step": flops,
-           "fused_path_schedule": "layers pipelined over two device queues in chunks of 7 timesteps; forward "
-                                  "timesteps are one kernel each (recurrent product + cell update)",
+           "fused_path_schedule": "one device queue, layer by layer; a forward timestep is one kernel (recurrent "
+                                  "product + cell update), a backward timestep two (cell update, Wh^T dpre), "
+                                  "operands handed from timestep to timestep in matrix-core fragment order",
            "timed_region": "per step: host->device copy of ids and labels, id sort, forward, backward, "
                            "device-side clipping, update; one HIP-graph replay per step; loss read back after "
                            "the last step"}
@@ -646,10 +647,24 @@ def lm_kernels(reps, use_graph=True):
     # single-launch forward timestep: product and cell update in one kernel, Wh read from its packed copy
     pk = dev.empty((4 * H * H,))
     dev.lstm_pack_recurrent(H, Wh, pk)
-    step = lambda: dev.lstm_step_forward(H, B, pk, h, xp, bb_, c, g, c2, hh)
+    nh, nd = dev.lstm_packed_state_floats(H, B), dev.lstm_packed_state_floats(4 * H, B)
+    hp_in, hp_out, dpp = dev.empty((nh,)), dev.empty((nh,)), dev.empty((nd,))
+    dev.lstm_pack_state(H, B, h, hp_in)
+    step = lambda: dev.lstm_step_forward_packed(H, B, pk, hp_in, xp, bb_, c, g, c2, hh, hp_out)
     pack = lambda: dev.lstm_pack_recurrent(H, Wh, pk)
+    # backward timestep over packed operands: cell kernel (dpre plain and packed), then the slices of Wh^T dpre
+    pkT = dev.empty((4 * H * H,))
+    dev.lstm_pack_recurrent_transposed(H, Wh, pkT)
+    dev.lstm_cell_backward_packed(H, B, g, c2, c, dh, None, 0, dc, dpre, dc2, dpp)
+    nbp = dev.lstm_recurrent_backward_packed(H, B, pkT, dpp, wb, bb)
+    rec_bwd = lambda: dev.lstm_recurrent_backward_packed(H, B, pkT, dpp, wb, bb)
+    cell_bwd = lambda: dev.lstm_cell_backward_packed(H, B, g, c2, c, dh, wb, nbp, dc, dpre, dc2, dpp)
     for name, fn, flops, nbytes in (("lstm_step_fwd (recurrent product + cell update)", step, 2.0 * 4 * H * H * B,
-                                     (4 * H * H + H * B + 4 * H * B + 4 * H + H * B + 6 * H * B) * 4),
+                                     (4 * H * H + H * B + 4 * H * B + 4 * H + H * B + 7 * H * B) * 4),
+                                    ("lstm_rec_bwd (Wh^T dpre from packed operands, %d slices)" % nbp, rec_bwd,
+                                     2.0 * 4 * H * H * B, (4 * H * H + 4 * H * B + nbp * H * B) * 4),
+                                    ("lstm_cell_bwd_packed (%d slices, dpre plain + packed)" % nbp, cell_bwd, 0.0,
+                                     ((4 + 4 + nbp + 4 + 4 + 1) * H * B) * 4),
                                     ("lstm_pack_recurrent (once per layer per step)", pack, 0.0, 2 * 4 * H * H * 4)):
         if use_graph:
             gr = capture(dev, [fn] * 4)

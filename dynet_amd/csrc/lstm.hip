@@ -194,7 +194,8 @@ __global__ __launch_bounds__(kCellThreads) void lstm_cell_bwd_kernel(unsigned H,
                                                                      const float* __restrict__ dh_in,
                                                                      const float* __restrict__ rec,
                                                                      const float* dc_in, float* __restrict__ dpre,
-                                                                     float* dc_prev, unsigned b_first) {
+                                                                     float* dc_prev, unsigned b_first,
+                                                                     float* __restrict__ dpre_packed) {
   const unsigned j = (blockIdx.x * kCellThreads + threadIdx.x) * V, b = b_first + blockIdx.y;
   if (j >= H) return;
   const size_t g0 = size_t(b) * 4 * H + j, s0 = size_t(b) * H + j;
@@ -228,167 +229,243 @@ __global__ __launch_bounds__(kCellThreads) void lstm_cell_bwd_kernel(unsigned H,
 #pragma unroll
   for (int q = 0; q < 4; ++q) out[q].store(dpre + g0 + size_t(q) * H);
   if (dc_prev) dcp.store(dc_prev + s0);
+  // dpre again in the fragment order of the next recurrent product (depth 4H): see lstm_pack_state_kernel
+  if (dpre_packed != nullptr) {
+    const size_t tile = size_t(b / 32) * (H / 2) * 256 + (b % 32) * 4;  // column tile of 4H/8 groups of 256 floats
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const unsigned k = q * H + j + e;
+        dpre_packed[tile + size_t(k / 8) * 256 + (k % 2) * 128 + (k % 8) / 2] = out[q].v[e];
+      }
+  }
 }
 
 // ---- single-launch forward step: recurrent product and cell update in one kernel -------
-// A block owns 8 hidden units x 32 batch columns.  Its 32 weight rows are the four gate
-// rows (i, f, o, g) of those 8 units, so after the product all four pre-activations of a
-// hidden unit sit in the same block and the cell update runs in the epilogue: the 4H x B
-// product never goes to memory.  The four waves split the H-deep sum in quarters, each
-// streaming its quarter through a private double-buffered LDS stage into 32x32x2 MFMAs,
-// and the quarters meet in LDS.
+// A block owns 16 hidden units x 32 batch columns.  Its 64 weight rows are the four gate rows
+// (i, f, o, g) of those units, so after the product all four pre-activations of a hidden unit
+// sit in the same block and the cell update runs in the epilogue: the 4H x B product never goes
+// to memory.  The four waves split the depth of the sum in quarters and meet in LDS; each wave
+// multiplies two 32-row tiles by one 32-column tile, so a fragment of the state feeds two MFMAs.
 //
-// The weights are read from a packed copy Wp[H/8][H][32]: tile rt, column k holds the 32
-// rows {g*H + rt*8 + u : g < 4, u < 8} at index g*8 + u, which makes a wave's stage one
-// contiguous 4 KiB run.  Blocks of one row tile are H/8 apart in launch order, so with
-// H/8 a multiple of 8 they land on the same XCD and share that L2's copy of the tile.
-constexpr int kStepBK = 32;                 // k depth of one LDS stage
-constexpr int kStepPitchB = 34;             // B stage: [k][col], 2-way conflicts at most on the transposing write
-constexpr int kStepPitchR = 33;             // quarter-sum exchange: [row][col]
-constexpr int kStepWaveFloats = 2 * 32 * kStepBK + 2 * kStepBK * kStepPitchB;  // per-wave A + B stages
+// What bounds the kernel is the rate at which one CU can pull operands through its vector memory
+// path (about 26 GB/s whether they come from L2 or from HBM), so the tile is chosen for the fewest
+// operand bytes per CU that still gives every CU a block at H = 1024, B = 128: (64 + 32) rows and
+// columns of depth H per block.  Both operands are read in MFMA fragment order straight into
+// registers (no LDS stage, no barrier in the loop): for a 32-wide tile and a group of 8 consecutive
+// k, lane l = 32*lhi + l32 holds k = 8*kg + 2*s + lhi, s = 0..3, of row (or column) l32 as one
+// float4, and a group of a tile is 1 KiB contiguous.
+//   weights  Wp[rows/32][K/8][64][4]   forward: row g*H + rt*8 + u of W at l32 = g*8 + u of tile rt;
+//                                      backward: row rt*32 + l32 of W^T (dyhip_lstm_pack_*)
+//   state    vp[ceil(B/32)][K/8][64][4]   column ct*32 + l32 (dyhip_lstm_pack_state, or the packed h /
+//            dpre the step kernels write for the next timestep); columns past B hold zeros or stale
+//            values and only feed output columns that are dropped
+// Blocks that share weight rows are a multiple of 8 apart in launch order, so they land on the same
+// XCD and share that L2's copy of the rows.
+constexpr int kStepPitchR = 33;  // partial-sum exchange: [row][col]
 typedef float stepx16 __attribute__((ext_vector_type(16)));
 
-// W is 4H x K (Wh: K = H, Wx: K = the input size)
-__global__ __launch_bounds__(256) void lstm_pack_recurrent_kernel(unsigned H, unsigned K, const float* __restrict__ W,
-                                                                  float* __restrict__ Wp) {
-  const size_t o = size_t(blockIdx.x) * 256 + threadIdx.x;  // output index, (rt*K + k)*32 + g*8 + u
+// W is 4H x K column-major (Wh: K = H, Wx: K = the input size): gate-interleaved row tiles
+__global__ __launch_bounds__(256) void lstm_pack_weights_kernel(unsigned H, unsigned K, const float* __restrict__ W,
+                                                                float* __restrict__ Wp) {
+  const size_t o = size_t(blockIdx.x) * 256 + threadIdx.x;  // ((rt*(K/8) + kg)*64 + lane)*4 + s
   if (o >= size_t(4) * H * K) return;
-  const unsigned r = o % 32, g = r / 8, u = r % 8;
-  const size_t tk = o / 32;
-  const unsigned k = tk % K, rt = tk / K;
+  const unsigned s = o % 4, lane = (o / 4) % 64, l32 = lane % 32, lhi = lane / 32;
+  const size_t tg = o / 256;
+  const unsigned kg = tg % (K / 8), rt = tg / (K / 8);
+  const unsigned g = l32 / 8, u = l32 % 8, k = 8 * kg + 2 * s + lhi;
   Wp[o] = W[size_t(g) * H + rt * 8 + u + size_t(k) * 4 * H];
 }
 
-// orders a wave's LDS writes before the reads its other lanes issue afterwards
-__device__ __forceinline__ void step_wave_sync() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+// Wh is 4H x H column-major; the packed matrix is Wh^T (H rows, depth 4H) in plain 32-row tiles
+__global__ __launch_bounds__(256) void lstm_pack_transposed_kernel(unsigned H, const float* __restrict__ W,
+                                                                   float* __restrict__ Wp) {
+  const size_t o = size_t(blockIdx.x) * 256 + threadIdx.x;  // ((rt*(4H/8) + kg)*64 + lane)*4 + s
+  if (o >= size_t(4) * H * H) return;
+  const unsigned s = o % 4, lane = (o / 4) % 64, l32 = lane % 32, lhi = lane / 32;
+  const size_t tg = o / 256;
+  const unsigned kg = tg % (H / 2), rt = tg / (H / 2);
+  Wp[o] = W[size_t(rt * 32 + l32) * 4 * H + 8 * kg + 2 * s + lhi];
 }
 
-// Up to two products feed the pre-activations: Wx * x (packed Wx, depth I) and Wh * h_tm1 (packed Wh,
-// depth H); either may be absent (null), and Wx * x may instead arrive precomputed in xproj.
+// v is K x B column-major
+__global__ __launch_bounds__(256) void lstm_pack_state_kernel(unsigned K, unsigned B, const float* __restrict__ v,
+                                                              float* __restrict__ vp) {
+  const size_t o = size_t(blockIdx.x) * 256 + threadIdx.x;  // ((ct*(K/8) + kg)*64 + lane)*4 + s
+  if (o >= size_t(K) * cdiv<unsigned>(B, 32) * 32) return;
+  const unsigned s = o % 4, lane = (o / 4) % 64, l32 = lane % 32, lhi = lane / 32;
+  const size_t tg = o / 256;
+  const unsigned kg = tg % (K / 8), ct = tg / (K / 8);
+  const unsigned col = ct * 32 + l32, k = 8 * kg + 2 * s + lhi;
+  vp[o] = col < B ? v[size_t(col) * K + k] : 0.f;
+}
+
+// acc0 / acc1 += (two 32-row tiles of packed weights) x (one 32-column tile of packed state) over `groups`
+// groups of 8 k (a multiple of 4), starting at the group the pointers name.  Eight groups at a time run as a
+// branch-free double buffer: four groups are multiplied while the next four are in flight (the last round
+// re-reads its own groups instead of branching around the loads, so the compiler counts the outstanding
+// loads exactly; the scheduling barriers keep it from sinking the loads down to their uses).
+__device__ __forceinline__ void step_product(stepx16& acc0, stepx16& acc1, const float4* __restrict__ pa0,
+                                             const float4* __restrict__ pa1, const float4* __restrict__ pb,
+                                             unsigned groups) {
+  float4 a0[4], a1[4], b0[4], c0[4], c1[4], d0[4];
+#define STEP_LOAD(A0, A1, BB, grp)                 \
+  _Pragma("unroll") for (int u = 0; u < 4; ++u) {  \
+    A0[u] = pa0[size_t((grp) + u) * 64];           \
+    A1[u] = pa1[size_t((grp) + u) * 64];           \
+    BB[u] = pb[size_t((grp) + u) * 64];            \
+  }                                                \
+  __builtin_amdgcn_sched_barrier(0);
+#define STEP_MMA1(x, y, acc) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, acc, 0, 0, 0);
+#define STEP_MMA(A0, A1, BB)                       \
+  _Pragma("unroll") for (int u = 0; u < 4; ++u) {  \
+    STEP_MMA1(A0[u].x, BB[u].x, acc0)              \
+    STEP_MMA1(A1[u].x, BB[u].x, acc1)              \
+    STEP_MMA1(A0[u].y, BB[u].y, acc0)              \
+    STEP_MMA1(A1[u].y, BB[u].y, acc1)              \
+    STEP_MMA1(A0[u].z, BB[u].z, acc0)              \
+    STEP_MMA1(A1[u].z, BB[u].z, acc1)              \
+    STEP_MMA1(A0[u].w, BB[u].w, acc0)              \
+    STEP_MMA1(A1[u].w, BB[u].w, acc1)              \
+  }                                                \
+  __builtin_amdgcn_sched_barrier(0);
+  const unsigned full = groups / 8 * 8;
+  if (full > 0) {
+    STEP_LOAD(a0, a1, b0, 0u)
+    for (unsigned g = 0; g < full; g += 8) {
+      const unsigned nx = g + 8 < full ? g + 8 : g;  // the last round's prefetch lands on its own groups
+      STEP_LOAD(c0, c1, d0, g + 4)
+      STEP_MMA(a0, a1, b0)
+      STEP_LOAD(a0, a1, b0, nx)
+      STEP_MMA(c0, c1, d0)
+    }
+  }
+  if (full < groups) {
+    STEP_LOAD(a0, a1, b0, full)
+    STEP_MMA(a0, a1, b0)
+  }
+#undef STEP_LOAD
+#undef STEP_MMA1
+#undef STEP_MMA
+}
+
+// Up to two products feed the pre-activations: Wx * x (depth I) and Wh * h_tm1 (depth H), both operands
+// packed; either product may be absent (null), and Wx * x may instead arrive precomputed in xproj.
 struct StepOperand {
-  const float* Wp;  // packed weights [H/8][K][32]
-  const float* v;   // K x B, column-major
+  const float* Wp;
+  const float* vp;
   unsigned K;
 };
 
-__global__ __launch_bounds__(256, 2) void lstm_step_fwd_kernel(unsigned H, unsigned B, StepOperand op0, StepOperand op1,
-                                                               const float* xproj,
-                                                               const float* __restrict__ bias,
-                                                               const float* __restrict__ c_prev, int mode,
-                                                               float* gates, float* __restrict__ c,
-                                                               float* __restrict__ h) {
-  __shared__ __attribute__((aligned(16))) float lds[4 * kStepWaveFloats];
-  const unsigned RT = H / 8;
-  const unsigned rt = blockIdx.x % RT, ct = blockIdx.x / RT;
+__global__ __launch_bounds__(256) void lstm_step_fwd_kernel(unsigned H, unsigned B, StepOperand op0, StepOperand op1,
+                                                            const float* xproj, const float* __restrict__ bias,
+                                                            const float* __restrict__ c_prev, int mode, float* gates,
+                                                            float* __restrict__ c, float* __restrict__ h,
+                                                            float* __restrict__ hp) {
+  __shared__ float red[4 * 64 * kStepPitchR];
+  const unsigned RP = H / 16;  // pairs of row tiles = groups of 16 hidden units
+  const unsigned rp = blockIdx.x % RP, ct = blockIdx.x / RP;
   const unsigned wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const unsigned l32 = lane % 32, lhi = lane / 32;
-  float* la = lds + wave * kStepWaveFloats;
-  float* lb = la + 2 * 32 * kStepBK;
-  const unsigned bk = 4 * (lane % 8), bc = lane / 8;
 
-  // the epilogue's thread owns hidden unit eu of batch column ecc; its operands are fetched
-  // now so that their latency hides behind the product
-  const unsigned eu = threadIdx.x % 8, ecc = threadIdx.x / 8;
-  const unsigned ecol = ct * 32 + ecc, ej = rt * 8 + eu;
-  float pre[4] = {0.f, 0.f, 0.f, 0.f}, cp = 0.f;
-  if (ecol < B) {
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const float bq = bias[q * H + ej];
-      pre[q] = q == 1 ? bq + 1.0f : bq;
-      if (xproj != nullptr) pre[q] += xproj[size_t(ecol) * 4 * H + ej + size_t(q) * H];
-    }
-    if (c_prev != nullptr) cp = c_prev[size_t(ecol) * H + ej];
-  }
-
-  float4 ra0, ra1, ra2, ra3, rb0, rb1, rb2, rb3;
-#define STEP_LOAD1(i, st)                                                                  \
-  ra##i = *reinterpret_cast<const float4*>(ga + size_t(st) * 32 * kStepBK + i * 256);      \
-  rb##i = *reinterpret_cast<const float4*>(gb##i + (st) * kStepBK);
-#define STEP_LOAD(st) STEP_LOAD1(0, st) STEP_LOAD1(1, st) STEP_LOAD1(2, st) STEP_LOAD1(3, st)
-#define STEP_STORE1(i)                                                                     \
-  *reinterpret_cast<float4*>(a_ + i * 256) = ra##i;                                        \
-  b_[0 * kStepPitchB + 8 * i] = rb##i.x;                                                   \
-  b_[1 * kStepPitchB + 8 * i] = rb##i.y;                                                   \
-  b_[2 * kStepPitchB + 8 * i] = rb##i.z;                                                   \
-  b_[3 * kStepPitchB + 8 * i] = rb##i.w;
-#define STEP_STORE(buf)                                                                    \
-  {                                                                                        \
-    float* a_ = la + (buf) * 32 * kStepBK + lane * 4;                                      \
-    float* b_ = lb + (buf) * kStepBK * kStepPitchB + bk * kStepPitchB + bc;                \
-    STEP_STORE1(0) STEP_STORE1(1) STEP_STORE1(2) STEP_STORE1(3)                            \
-  }
-
-  // The kernel runs at the rate the L2 delivers the operands (every 32x32 output tile pulls
-  // its full-depth strips of both), so one stage of lookahead is enough.
-  stepx16 acc = {0};
-  const float *ga = nullptr, *gb0 = nullptr, *gb1 = nullptr, *gb2 = nullptr, *gb3 = nullptr;
+  stepx16 acc0 = {0}, acc1 = {0};
   for (int which = 0; which < 2; ++which) {
     const StepOperand op = which == 0 ? op0 : op1;
     if (op.Wp == nullptr) continue;  // uniform over the grid
-    const unsigned kq = op.K / 4, k0 = wave * kq, nst = kq / kStepBK;
-    ga = op.Wp + (size_t(rt) * op.K + k0) * 32 + lane * 4;
-    // columns past the batch are computed on a clamped address and dropped
-    auto column = [&](unsigned i) {
-      const unsigned col = ct * 32 + bc + 8 * i;
-      return op.v + size_t(col < B ? col : B - 1) * op.K + k0 + bk;
-    };
-    gb0 = column(0);
-    gb1 = column(1);
-    gb2 = column(2);
-    gb3 = column(3);
-    STEP_LOAD(0)
-    STEP_STORE(0)
-    if (nst > 1) { STEP_LOAD(1) }
-    step_wave_sync();
-    for (unsigned st = 0; st < nst; ++st) {
-      const unsigned cur = st & 1;
-      const float* a = la + cur * 32 * kStepBK + lhi * 32 + l32;
-      const float* b = lb + cur * kStepBK * kStepPitchB + lhi * kStepPitchB + l32;
+    const unsigned G = op.K / 8, gq = G / 4, g0 = wave * gq;
+    const float4* pa = reinterpret_cast<const float4*>(op.Wp) + (size_t(2 * rp) * G + g0) * 64 + lane;
+    step_product(acc0, acc1, pa, pa + size_t(G) * 64,
+                 reinterpret_cast<const float4*>(op.vp) + (size_t(ct) * G + g0) * 64 + lane, gq);
+  }
+
+  // The epilogue's thread owns hidden unit eu (of 16) of batch columns ecc and ecc + 16.  Its operands are
+  // requested only now: loads return in order, so asking for them before the product would hold up the
+  // product's first fragments; here their latency hides behind the exchange of the partial sums.
+  const unsigned eu = threadIdx.x % 16, ecc = threadIdx.x / 16, ej = rp * 16 + eu;
+  float pre[2][4], cp[2] = {0.f, 0.f};
 #pragma unroll
-      for (int s = 0; s < kStepBK / 2; ++s)
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * s * 32], b[2 * s * kStepPitchB], acc, 0, 0, 0);
-      if (st + 1 < nst) {
-        STEP_STORE(cur ^ 1)
-        if (st + 2 < nst) { STEP_LOAD(st + 2) }
+  for (int i = 0; i < 2; ++i) {
+    const unsigned ecol = ct * 32 + ecc + 16 * i;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) pre[i][q] = 0.f;
+    if (ecol < B) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float bq = bias[q * H + ej];
+        pre[i][q] = q == 1 ? bq + 1.0f : bq;
+        if (xproj != nullptr) pre[i][q] += xproj[size_t(ecol) * 4 * H + ej + size_t(q) * H];
       }
-      step_wave_sync();  // the stages are private to the wave: no block barrier in the loop
+      if (c_prev != nullptr) cp[i] = c_prev[size_t(ecol) * H + ej];
     }
   }
-  __syncthreads();
-#undef STEP_LOAD1
-#undef STEP_LOAD
-#undef STEP_STORE1
-#undef STEP_STORE
 
-  // the four quarter sums meet in LDS (the stages are dead after the last barrier)
-  float* red = lds;
+  // the four quarter sums meet in LDS: rows 0..31 = first tile of the pair, 32..63 = second
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const unsigned row = 8 * (r / 4) + 4 * lhi + (r % 4);
-    red[(wave * 32 + row) * kStepPitchR + l32] = acc[r];
+    red[(wave * 64 + row) * kStepPitchR + l32] = acc0[r];
+    red[(wave * 64 + 32 + row) * kStepPitchR + l32] = acc1[r];
   }
   __syncthreads();
 
-  if (ecol >= B) return;
-  const size_t g0 = size_t(ecol) * 4 * H + ej, s0 = size_t(ecol) * H + ej;
+  const unsigned tile = eu / 8, u = eu % 8;
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {
+  for (int i = 0; i < 2; ++i) {
+    const unsigned col = ecc + 16 * i, ecol = ct * 32 + col;
+    if (ecol >= B) continue;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) pre[q] += red[(w * 32 + q * 8 + eu) * kStepPitchR + ecc];
+    for (int q = 0; q < 4; ++q) {
+#pragma unroll
+      for (int w = 0; w < 4; ++w) pre[i][q] += red[(w * 64 + tile * 32 + q * 8 + u) * kStepPitchR + col];
+    }
+    const float gi = logistic(mode, pre[i][0]), gf = logistic(mode, pre[i][1]), go = logistic(mode, pre[i][2]);
+    const float gg = tanh_accurate(pre[i][3]);
+    const float cv = c_prev != nullptr ? gi * gg + gf * cp[i] : gi * gg;
+    const float hv = go * tanh_accurate(cv);
+    const size_t g0 = size_t(ecol) * 4 * H + ej, s0 = size_t(ecol) * H + ej;
+    gates[g0] = gi;
+    gates[g0 + H] = gf;
+    gates[g0 + 2 * size_t(H)] = go;
+    gates[g0 + 3 * size_t(H)] = gg;
+    c[s0] = cv;
+    h[s0] = hv;
+    // h again, as the next timestep's packed operand: unit ej is k = 8*(2*rp + tile) + u
+    if (hp != nullptr) hp[((size_t(ct) * (H / 8) + 2 * rp + tile) * 64 + (u % 2) * 32 + col) * 4 + u / 2] = hv;
   }
-  const float gi = logistic(mode, pre[0]), gf = logistic(mode, pre[1]), go = logistic(mode, pre[2]);
-  const float gg = tanh_accurate(pre[3]);
-  const float cv = c_prev != nullptr ? gi * gg + gf * cp : gi * gg;
-  gates[g0] = gi;
-  gates[g0 + H] = gf;
-  gates[g0 + 2 * size_t(H)] = go;
-  gates[g0 + 3 * size_t(H)] = gg;
-  c[s0] = cv;
-  h[s0] = go * tanh_accurate(cv);
+}
+
+// Recurrent product of the backward timestep: slice[split] = (Wh^T)[64 hidden units, depth range] x dpre[depth
+// range, 32 columns], the same tile and operand order as the forward kernel; the depth 4H is cut into
+// gridDim.y ranges so that every CU has a block, and the cell kernel adds the slices in ascending order.
+__global__ __launch_bounds__(256) void lstm_rec_bwd_kernel(unsigned H, unsigned B, const float* __restrict__ WpT,
+                                                           const float* __restrict__ dpp, float* __restrict__ slices) {
+  __shared__ float red[4 * 64 * kStepPitchR];
+  const unsigned RP = H / 64;
+  const unsigned rp = blockIdx.x % RP, ct = blockIdx.x / RP, split = blockIdx.y;
+  const unsigned wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const unsigned l32 = lane % 32, lhi = lane / 32;
+  const unsigned G = H / 2, gq = G / (4 * gridDim.y), g0 = (split * 4 + wave) * gq;
+  stepx16 acc0 = {0}, acc1 = {0};
+  const float4* pa = reinterpret_cast<const float4*>(WpT) + (size_t(2 * rp) * G + g0) * 64 + lane;
+  step_product(acc0, acc1, pa, pa + size_t(G) * 64, reinterpret_cast<const float4*>(dpp) + (size_t(ct) * G + g0) * 64 + lane,
+               gq);
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const unsigned row = 8 * (r / 4) + 4 * lhi + (r % 4);
+    red[(wave * 64 + row) * kStepPitchR + l32] = acc0[r];
+    red[(wave * 64 + 32 + row) * kStepPitchR + l32] = acc1[r];
+  }
+  __syncthreads();
+  float* out = slices + size_t(split) * H * B;
+  for (unsigned o = threadIdx.x; o < 64 * 32; o += 256) {
+    const unsigned row = o % 64, col = o / 64, ecol = ct * 32 + col;
+    if (ecol >= B) continue;
+    float s = red[row * kStepPitchR + col];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) s += red[(w * 64 + row) * kStepPitchR + col];
+    out[size_t(ecol) * H + rp * 64 + row] = s;
+  }
 }
 
 static bool all_aligned16(std::initializer_list<const void*> ps) {
@@ -683,10 +760,9 @@ int dyhip_lstm_cell_forward(dyhip_device* dev, unsigned H, unsigned B, const flo
   return DYHIP_OK;
 }
 
-int dyhip_lstm_cell_backward(dyhip_device* dev, unsigned H, unsigned B, const float* gates, const float* c,
-                             const float* c_tm1, const float* dh, const float* rec, unsigned splits, const float* dc,
-                             float* dpre, float* dc_tm1) {
-  DYHIP_CHECK_DEV(dev);
+static int cell_backward(dyhip_device* dev, unsigned H, unsigned B, const float* gates, const float* c,
+                         const float* c_tm1, const float* dh, const float* rec, unsigned splits, const float* dc,
+                         float* dpre, float* dc_tm1, float* dpre_packed) {
   DYHIP_REQUIRE(H >= 1 && B >= 1, "LSTM cell: bad hidden (%u) or batch (%u) size", H, B);
   DYHIP_REQUIRE(gates && c && dh && dpre, "LSTM cell: null tensor pointer");
   DYHIP_REQUIRE(splits == 0 || rec != nullptr, "LSTM cell: %u recurrent slices but no buffer", splits);
@@ -696,16 +772,23 @@ int dyhip_lstm_cell_backward(dyhip_device* dev, unsigned H, unsigned B, const fl
     const unsigned nb = B - b0 < 65535u ? B - b0 : 65535u;
     if (vec)
       hipLaunchKernelGGL(lstm_cell_bwd_kernel<4>, dim3(cdiv<unsigned>(H, kCellThreads * 4), nb), dim3(kCellThreads), 0,
-                         dev->stream, H, splits, slice, gates, c, c_tm1, dh, rec, dc, dpre, dc_tm1, b0);
+                         dev->stream, H, splits, slice, gates, c, c_tm1, dh, rec, dc, dpre, dc_tm1, b0, dpre_packed);
     else
       hipLaunchKernelGGL(lstm_cell_bwd_kernel<1>, dim3(cdiv<unsigned>(H, kCellThreads), nb), dim3(kCellThreads), 0,
-                         dev->stream, H, splits, slice, gates, c, c_tm1, dh, rec, dc, dpre, dc_tm1, b0);
+                         dev->stream, H, splits, slice, gates, c, c_tm1, dh, rec, dc, dpre, dc_tm1, b0, dpre_packed);
   }
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
 
-static bool step_depth_ok(unsigned K) { return K >= 128 && K % 128 == 0; }  // quarters in whole 32-deep stages
+int dyhip_lstm_cell_backward(dyhip_device* dev, unsigned H, unsigned B, const float* gates, const float* c,
+                             const float* c_tm1, const float* dh, const float* rec, unsigned splits, const float* dc,
+                             float* dpre, float* dc_tm1) {
+  DYHIP_CHECK_DEV(dev);
+  return cell_backward(dev, H, B, gates, c, c_tm1, dh, rec, splits, dc, dpre, dc_tm1, nullptr);
+}
+
+static bool step_depth_ok(unsigned K) { return K >= 128 && K % 128 == 0; }  // quarters in whole sets of 4 groups of 8
 
 int dyhip_lstm_step_supported(dyhip_device* dev, unsigned H, unsigned B, int* supported) {
   DYHIP_CHECK_DEV(dev);
@@ -720,7 +803,19 @@ static int pack_weights(dyhip_device* dev, unsigned H, unsigned K, const float* 
                 "LSTM step: hidden size %u and product depth %u must be multiples of 128", H, K);
   DYHIP_REQUIRE(W && packed, "LSTM step: null tensor pointer");
   const size_t n = size_t(4) * H * K;
-  hipLaunchKernelGGL(lstm_pack_recurrent_kernel, dim3(unsigned(cdiv<size_t>(n, 256))), dim3(256), 0, dev->stream, H, K, W,
+  hipLaunchKernelGGL(lstm_pack_weights_kernel, dim3(unsigned(cdiv<size_t>(n, 256))), dim3(256), 0, dev->stream, H, K, W,
+                     packed);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+static size_t packed_state_floats(unsigned K, unsigned B) { return size_t(K) * cdiv<unsigned>(B, 32) * 32; }
+
+static int pack_state(dyhip_device* dev, unsigned K, unsigned B, const float* v, float* packed) {
+  DYHIP_REQUIRE(step_depth_ok(K) && B >= 1 && B <= 65535, "LSTM step: state of %u rows x %u columns cannot be packed", K, B);
+  DYHIP_REQUIRE(v && packed, "LSTM step: null tensor pointer");
+  const size_t n = packed_state_floats(K, B);
+  hipLaunchKernelGGL(lstm_pack_state_kernel, dim3(unsigned(cdiv<size_t>(n, 256))), dim3(256), 0, dev->stream, K, B, v,
                      packed);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
@@ -736,9 +831,34 @@ int dyhip_lstm_pack_input(dyhip_device* dev, unsigned I, unsigned H, const float
   return pack_weights(dev, H, I, Wx, packed);
 }
 
+int dyhip_lstm_pack_recurrent_transposed(dyhip_device* dev, unsigned H, const float* Wh, float* packed) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(step_depth_ok(H) && size_t(4) * H * H < (size_t(1) << 32), "LSTM step: hidden size %u must be a multiple of 128", H);
+  DYHIP_REQUIRE(Wh && packed, "LSTM step: null tensor pointer");
+  const size_t n = size_t(4) * H * H;
+  hipLaunchKernelGGL(lstm_pack_transposed_kernel, dim3(unsigned(cdiv<size_t>(n, 256))), dim3(256), 0, dev->stream, H, Wh,
+                     packed);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_lstm_packed_state_floats(unsigned rows, unsigned B, size_t* floats) {
+  DYHIP_REQUIRE(floats != nullptr, "null output pointer");
+  *floats = packed_state_floats(rows, B);
+  return DYHIP_OK;
+}
+
+int dyhip_lstm_pack_state(dyhip_device* dev, unsigned rows, unsigned B, const float* v, float* packed) {
+  DYHIP_CHECK_DEV(dev);
+  return pack_state(dev, rows, B, v, packed);
+}
+
+// x and h_tm1 arrive packed (x_packed / h_packed true) or plain; a plain operand is packed into the queue's
+// GEMM workspace first (one more launch; nothing else of this queue uses the workspace meanwhile).
 static int step_forward(dyhip_device* dev, unsigned I, unsigned H, unsigned B, const float* packed_Wx, const float* x,
-                        const float* packed_Wh, const float* h_tm1, const float* xproj, const float* b,
-                        const float* c_tm1, int logistic_mode, float* gates, float* c, float* h) {
+                        bool x_packed, const float* packed_Wh, const float* h_tm1, bool h_packed, const float* xproj,
+                        const float* b, const float* c_tm1, int logistic_mode, float* gates, float* c, float* h,
+                        float* hp_out) {
   int ok = 0;
   dyhip_lstm_step_supported(dev, H, B, &ok);
   DYHIP_REQUIRE(ok, "LSTM step: unsupported hidden (%u) or batch (%u) size", H, B);
@@ -746,13 +866,30 @@ static int step_forward(dyhip_device* dev, unsigned I, unsigned H, unsigned B, c
   DYHIP_REQUIRE((packed_Wx == nullptr) == (x == nullptr) && (packed_Wh == nullptr) == (h_tm1 == nullptr),
                 "LSTM step: packed weights and their operand come together");
   DYHIP_REQUIRE(packed_Wx == nullptr || step_depth_ok(I), "LSTM step: input size %u is not a multiple of 128", I);
-  DYHIP_REQUIRE(all_aligned16({packed_Wx, x, packed_Wh, h_tm1}), "LSTM step: weights and operands must be 16-byte aligned");
+  DYHIP_REQUIRE(all_aligned16({packed_Wx, x, packed_Wh, h_tm1, hp_out}),
+                "LSTM step: weights and operands must be 16-byte aligned");
   DYHIP_REQUIRE(logistic_mode == DYHIP_LOGISTIC_PACKET || logistic_mode == DYHIP_LOGISTIC_SCALAR,
                 "unknown logistic mode %d", logistic_mode);
+  float* scratch = static_cast<float*>(dev->gemm_ws);
+  size_t scratch_floats = dev->gemm_ws_bytes / sizeof(float);
+  if (x != nullptr && !x_packed) {
+    const size_t n = packed_state_floats(I, B);
+    DYHIP_REQUIRE(scratch != nullptr && n <= scratch_floats, "LSTM step: no room to pack the input");
+    DYHIP_CHECK_STATUS(pack_state(dev, I, B, x, scratch));
+    x = scratch;
+    scratch += n;
+    scratch_floats -= n;
+  }
+  if (h_tm1 != nullptr && !h_packed) {
+    const size_t n = packed_state_floats(H, B);
+    DYHIP_REQUIRE(scratch != nullptr && n <= scratch_floats, "LSTM step: no room to pack the state");
+    DYHIP_CHECK_STATUS(pack_state(dev, H, B, h_tm1, scratch));
+    h_tm1 = scratch;
+  }
   const StepOperand op0{packed_Wx, x, I}, op1{packed_Wh, h_tm1, H};
-  const unsigned blocks = (H / 8) * cdiv<unsigned>(B, 32);
+  const unsigned blocks = (H / 16) * cdiv<unsigned>(B, 32);
   hipLaunchKernelGGL(lstm_step_fwd_kernel, dim3(blocks), dim3(256), 0, dev->stream, H, B, op0, op1, xproj, b, c_tm1,
-                     logistic_mode, gates, c, h);
+                     logistic_mode, gates, c, h, hp_out);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
@@ -762,7 +899,19 @@ int dyhip_lstm_step_forward(dyhip_device* dev, unsigned H, unsigned B, const flo
                             float* c, float* h) {
   DYHIP_CHECK_DEV(dev);
   DYHIP_REQUIRE(packed_Wh && h_tm1 && xproj && c_tm1, "LSTM step: null tensor pointer");
-  return step_forward(dev, 0, H, B, nullptr, nullptr, packed_Wh, h_tm1, xproj, b, c_tm1, logistic_mode, gates, c, h);
+  return step_forward(dev, 0, H, B, nullptr, nullptr, false, packed_Wh, h_tm1, false, xproj, b, c_tm1, logistic_mode,
+                      gates, c, h, nullptr);
+}
+
+int dyhip_lstm_step_forward_packed(dyhip_device* dev, unsigned H, unsigned B, const float* packed_Wh,
+                                   const float* h_tm1_packed, const float* xproj, const float* b, const float* c_tm1,
+                                   int logistic_mode, float* gates, float* c, float* h, float* h_packed) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(xproj != nullptr, "LSTM step: null tensor pointer");
+  DYHIP_REQUIRE((packed_Wh == nullptr) == (h_tm1_packed == nullptr) && (packed_Wh == nullptr) == (c_tm1 == nullptr),
+                "LSTM step: the recurrent weights, the packed state and c_tm1 come together (all null = zero state)");
+  return step_forward(dev, 0, H, B, nullptr, nullptr, false, packed_Wh, h_tm1_packed, true, xproj, b, c_tm1,
+                      logistic_mode, gates, c, h, h_packed);
 }
 
 int dyhip_lstm_step_forward_x(dyhip_device* dev, unsigned I, unsigned H, unsigned B, const float* packed_Wx,
@@ -770,7 +919,42 @@ int dyhip_lstm_step_forward_x(dyhip_device* dev, unsigned I, unsigned H, unsigne
                               const float* c_tm1, int logistic_mode, float* gates, float* c, float* h) {
   DYHIP_CHECK_DEV(dev);
   DYHIP_REQUIRE(packed_Wx && x, "LSTM step: null tensor pointer");
-  return step_forward(dev, I, H, B, packed_Wx, x, packed_Wh, h_tm1, nullptr, b, c_tm1, logistic_mode, gates, c, h);
+  return step_forward(dev, I, H, B, packed_Wx, x, false, packed_Wh, h_tm1, false, nullptr, b, c_tm1, logistic_mode, gates,
+                      c, h, nullptr);
+}
+
+// depth ranges of the backward product: enough blocks for every CU, whole sets of four groups per wave
+static unsigned rec_bwd_splits(unsigned H, unsigned B) {
+  const unsigned tiles = (H / 64) * cdiv<unsigned>(B, 32);
+  unsigned s = 1;
+  while (s < 8 && tiles * s < 256 && (H / 2) % (s * 2 * 16) == 0) s *= 2;
+  return s;
+}
+
+int dyhip_lstm_recurrent_backward_packed(dyhip_device* dev, unsigned H, unsigned B, const float* packed_WhT,
+                                         const float* dpre_packed, void* ws, size_t ws_bytes, unsigned* splits) {
+  DYHIP_CHECK_DEV(dev);
+  int ok = 0;
+  dyhip_lstm_step_supported(dev, H, B, &ok);
+  DYHIP_REQUIRE(ok, "LSTM step: unsupported hidden (%u) or batch (%u) size", H, B);
+  DYHIP_REQUIRE(packed_WhT && dpre_packed && ws && splits, "LSTM step: null pointer");
+  DYHIP_REQUIRE(all_aligned16({packed_WhT, dpre_packed}), "LSTM step: weights and operands must be 16-byte aligned");
+  const unsigned s = rec_bwd_splits(H, B);
+  DYHIP_REQUIRE(ws_bytes >= sizeof(float) * size_t(H) * B * s, "LSTM step: %u slices of %u x %u floats do not fit %zu bytes", s, H,
+                B, ws_bytes);
+  hipLaunchKernelGGL(lstm_rec_bwd_kernel, dim3((H / 64) * cdiv<unsigned>(B, 32), s), dim3(256), 0, dev->stream, H, B,
+                     packed_WhT, dpre_packed, static_cast<float*>(ws));
+  DYHIP_CHECK_LAUNCH();
+  *splits = s;
+  return DYHIP_OK;
+}
+
+int dyhip_lstm_cell_backward_packed(dyhip_device* dev, unsigned H, unsigned B, const float* gates, const float* c,
+                                    const float* c_tm1, const float* dh, const float* rec, unsigned splits,
+                                    const float* dc, float* dpre, float* dc_tm1, float* dpre_packed) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(dpre_packed == nullptr || (H % 8 == 0 && aligned16(dpre_packed)), "LSTM cell: packed dpre needs H %% 8 == 0");
+  return cell_backward(dev, H, B, gates, c, c_tm1, dh, rec, splits, dc, dpre, dc_tm1, dpre_packed);
 }
 
 }  // extern "C"

@@ -439,6 +439,33 @@ class Device:
         _check(cdll.dyhip_lstm_step_forward(self.handle, _u(H), _u(B), _p(packed_Wh), _p(h_tm1), _p(xproj), _p(b),
                                             _p(c_tm1), _i(logistic_mode), _p(gates), _p(c), _p(h)))
 
+    def lstm_packed_state_floats(self, rows, B):
+        n = C.c_size_t(0)
+        _check(cdll.dyhip_lstm_packed_state_floats(_u(rows), _u(B), C.byref(n)))
+        return n.value
+
+    def lstm_pack_state(self, rows, B, v, packed):
+        _check(cdll.dyhip_lstm_pack_state(self.handle, _u(rows), _u(B), _p(v), _p(packed)))
+
+    def lstm_step_forward_packed(self, H, B, packed_Wh, h_tm1_packed, xproj, b, c_tm1, gates, c, h, h_packed,
+                                 logistic_mode=lib.LOGISTIC_PACKET):
+        _check(cdll.dyhip_lstm_step_forward_packed(self.handle, _u(H), _u(B), _p(packed_Wh), _p(h_tm1_packed), _p(xproj),
+                                                   _p(b), _p(c_tm1), _i(logistic_mode), _p(gates), _p(c), _p(h),
+                                                   _p(h_packed)))
+
+    def lstm_pack_recurrent_transposed(self, H, Wh, packed):
+        _check(cdll.dyhip_lstm_pack_recurrent_transposed(self.handle, _u(H), _p(Wh), _p(packed)))
+
+    def lstm_recurrent_backward_packed(self, H, B, packed_WhT, dpre_packed, ws, ws_bytes):
+        n = _u(0)
+        _check(cdll.dyhip_lstm_recurrent_backward_packed(self.handle, _u(H), _u(B), _p(packed_WhT), _p(dpre_packed),
+                                                         _vp(ws), _sz(ws_bytes), C.byref(n)))
+        return n.value
+
+    def lstm_cell_backward_packed(self, H, B, gates, c, c_tm1, dh, rec, splits, dc, dpre, dc_tm1, dpre_packed):
+        _check(cdll.dyhip_lstm_cell_backward_packed(self.handle, _u(H), _u(B), _p(gates), _p(c), _p(c_tm1), _p(dh),
+                                                    _vp(rec), _u(splits), _p(dc), _p(dpre), _p(dc_tm1), _p(dpre_packed)))
+
     def lstm_pack_input(self, I, H, Wx, packed):
         _check(cdll.dyhip_lstm_pack_input(self.handle, _u(I), _u(H), _p(Wx), _p(packed)))
 

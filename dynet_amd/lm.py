@@ -14,10 +14,13 @@ What differs from DyNet's node-at-a-time execution (results agree to fp32 roundi
   * ``path="fused"`` (default) runs layer by layer: one GEMM forms Wx*x for all timesteps, a timestep is then
     the recurrent GEMM Wh*h plus one cell kernel (gates + c + h); backward mirrors it, and dx, dWx, dWh, db are
     GEMMs/reductions over all timesteps;
-  * with ``overlap=True`` (default for more than one layer) the fused path cuts the time axis into chunks and
-    runs the layers as a pipeline on one queue per layer: layer l works on chunk k while layer l-1 is already on
-    chunk k+1 (backward: l on chunk k, l+1 on chunk k-1).  A timestep's recurrent GEMM and cell kernel are
-    latency-bound and leave most of the GPU idle; two such chains side by side fill it.
+  * a timestep of the fused path is one kernel forward (recurrent product + cell update) and two backward (cell
+    update, then the slices of Wh^T * dpre), all reading their operands from packed copies in matrix-core fragment
+    order that the previous timestep's kernel wrote (``single_launch``, where the sizes allow);
+  * with ``overlap=True`` the fused path cuts the time axis into chunks and runs the layers as a pipeline on one
+    queue per layer: layer l works on chunk k while layer l-1 is already on chunk k+1 (backward: l on chunk k, l+1
+    on chunk k-1).  It paid off while a timestep's kernels left most of the GPU idle; the packed kernels are bound by
+    what one CU can load, two of them side by side only slow each other, and the default is one queue.
 """
 import numpy as np
 
@@ -31,7 +34,7 @@ class LstmLM:
     def __init__(self, dev, V, E, H, L, B, T, seed=0, lr=0.1, clip=5.0, time_batched=True, params=None, path="fused",
                  overlap=None, chunk=7, single_launch=None):
         assert path in ("fused", "nodes")
-        self.overlap = (L > 1) if overlap is None else bool(overlap)
+        self.overlap = False if overlap is None else bool(overlap)
         self.overlap = self.overlap and path == "fused" and L > 1
         self.chunk = max(1, int(chunk))
         self.dev, self.V, self.E, self.H, self.L, self.B, self.T = dev, V, E, H, L, B, T
@@ -90,6 +93,12 @@ class LstmLM:
         ok = path == "fused" and dev.lstm_step_supported(H, B)
         self.single_launch = ok if single_launch is None else (bool(single_launch) and ok)
         self.Wh_packed = [dev.empty((4 * H * H,), pool=PS) for _ in range(L)] if self.single_launch else []
+        self.WhT_packed = [dev.empty((4 * H * H,), pool=PS) for _ in range(L)] if self.single_launch else []
+        # packed copies of h and of dpre for the next timestep's recurrent product, two per layer used in turn
+        nh = dev.lstm_packed_state_floats(H, B) if self.single_launch else 0
+        nd = dev.lstm_packed_state_floats(4 * H, B) if self.single_launch else 0
+        self.h_packed = [[dev.empty((nh,), pool=FXS) for _ in range(2)] for _ in range(L)] if self.single_launch else []
+        self.dpre_packed = [[dev.empty((nd,), pool=DE) for _ in range(2)] for _ in range(L)] if self.single_launch else []
         # queue l runs layer l; queue 0 is the device itself
         self.queues = [dev] + ([dev.fork() for _ in range(L - 1)] if self.overlap else [])
         self.plan, self.plan_ws, self.plan_ws_bytes = dev.lookup_plan_buffers(N, V)
@@ -158,9 +167,12 @@ class LstmLM:
         H, B = self.H, self.B
         for t in range(t0, t1):
             g = self._t(self.gates[l], t, 4 * H)
-            if t > 0 and self.single_launch:
-                q.lstm_step_forward(H, B, self.Wh_packed[l], self._t(self.h[l], t - 1, H), g, self.p[f"b{l}"],
-                                    self._t(self.c[l], t - 1, H), g, self._t(self.c[l], t, H), self._t(self.h[l], t, H))
+            if self.single_launch:
+                hp = self.h_packed[l]
+                q.lstm_step_forward_packed(H, B, self.Wh_packed[l] if t > 0 else None, hp[(t - 1) % 2] if t > 0 else None,
+                                           g, self.p[f"b{l}"], self._t(self.c[l], t - 1, H) if t > 0 else None, g,
+                                           self._t(self.c[l], t, H), self._t(self.h[l], t, H),
+                                           hp[t % 2] if t + 1 < self.T else None)
             elif t > 0:
                 n = q.lstm_recurrent_forward(H, B, self.p[f"Wh{l}"], self._t(self.h[l], t - 1, H), self.rec_f[l],
                                              self.rec_f_bytes)
@@ -175,6 +187,7 @@ class LstmLM:
         if self.single_launch:  # the weights moved in the last update
             for l in range(L):
                 d.lstm_pack_recurrent(H, self.p[f"Wh{l}"], self.Wh_packed[l])
+                d.lstm_pack_recurrent_transposed(H, self.p[f"Wh{l}"], self.WhT_packed[l])
         if not self.overlap:
             for l in range(L):
                 x, d_in = (self.h[l - 1], H) if l > 0 else (self.emb, E)
@@ -237,11 +250,18 @@ class LstmLM:
         for t in reversed(range(t0, t1)):
             last, first = t == T - 1, t == 0
             dpre = self._t(self.d_pre[l], t, 4 * H)
-            q.lstm_cell_backward(H, B, self._t(self.gates[l], t, 4 * H), self._t(self.c[l], t, H),
-                                 None if first else self._t(self.c[l], t - 1, H), self._t(self.d_h[l], t, H),
-                                 None if last else self.rec_b[l], 0 if last else self._rec_b_n[l],
-                                 None if last else self._t(self.d_c[l], t, H), dpre,
-                                 None if first else self._t(self.d_c[l], t - 1, H))
+            args = (H, B, self._t(self.gates[l], t, 4 * H), self._t(self.c[l], t, H),
+                    None if first else self._t(self.c[l], t - 1, H), self._t(self.d_h[l], t, H),
+                    None if last else self.rec_b[l], 0 if last else self._rec_b_n[l],
+                    None if last else self._t(self.d_c[l], t, H), dpre, None if first else self._t(self.d_c[l], t - 1, H))
+            if self.single_launch:  # dpre also in the operand order of the recurrent product below
+                dpp = self.dpre_packed[l][t % 2]
+                q.lstm_cell_backward_packed(*args, None if first else dpp)
+                if not first:
+                    self._rec_b_n[l] = q.lstm_recurrent_backward_packed(H, B, self.WhT_packed[l], dpp, self.rec_b[l],
+                                                                        self.rec_b_bytes)
+                continue
+            q.lstm_cell_backward(*args)
             if not first:
                 self._rec_b_n[l] = q.lstm_recurrent_backward(H, B, Wh, dpre, self.rec_b[l], self.rec_b_bytes)
 

@@ -311,24 +311,45 @@ int dyhip_lstm_cell_backward(dyhip_device* dev, unsigned H, unsigned B, const fl
                              const float* c_tm1, const float* dh, const float* rec, unsigned splits, const float* dc,
                              float* dpre, float* dc_tm1);
 
-/* Single-launch form of a forward timestep (t >= 1): the recurrent product Wh * h_tm1 and
- * the cell update of dyhip_lstm_cell_forward in one kernel, the product staying on chip.
- * A block owns 8 hidden units, i.e. the gate rows j, H+j, 2H+j, 3H+j of the slicing in
- * dynet/nodes-lstm.cc:213-223, which it reads from a packed copy of Wh laid out
- * [H/8][H][4 gates x 8 units]: refresh it with dyhip_lstm_pack_recurrent (4*H*H floats)
- * whenever Wh changes.  Supported when H is a multiple of 128 (dyhip_lstm_step_supported
- * reports it; the two-call form above covers every other size).  Same results as the
- * two-call form up to fp32 summation order.  gates may alias xproj. */
+/* Single-launch form of a forward timestep: the recurrent product Wh * h_tm1 and the cell update of
+ * dyhip_lstm_cell_forward in one kernel, the product staying on chip.  A block owns 16 hidden units,
+ * i.e. the gate rows j, H+j, 2H+j, 3H+j of the slicing in dynet/nodes-lstm.cc:213-223, and reads both
+ * operands in matrix-core fragment order: the weights from a packed copy of Wh (4*H*H floats; refresh
+ * it with dyhip_lstm_pack_recurrent whenever Wh changes), the state from a packed copy of h_tm1
+ * (dyhip_lstm_packed_state_floats(H, B) floats).  Supported when H is a multiple of 128
+ * (dyhip_lstm_step_supported reports it; the two-call form above covers every other size).  Same
+ * results as the two-call form up to fp32 summation order.  gates may alias xproj.
+ *   dyhip_lstm_step_forward         h_tm1 plain (H x B): packed internally by one extra launch
+ *   dyhip_lstm_step_forward_packed  h_tm1 packed; also writes h_packed (may be null), the packed copy of
+ *                                   the new h, so a chain of timesteps never repacks; packed_Wh =
+ *                                   h_tm1_packed = c_tm1 = NULL stand for the zero initial state
+ *   dyhip_lstm_pack_state           packs a rows x B state that did not come from a step (a non-zero h_0) */
 int dyhip_lstm_step_supported(dyhip_device* dev, unsigned H, unsigned B, int* supported);
 int dyhip_lstm_pack_recurrent(dyhip_device* dev, unsigned H, const float* Wh, float* packed);
+int dyhip_lstm_packed_state_floats(unsigned rows, unsigned B, size_t* floats);
+int dyhip_lstm_pack_state(dyhip_device* dev, unsigned rows, unsigned B, const float* v, float* packed);
 int dyhip_lstm_step_forward(dyhip_device* dev, unsigned H, unsigned B, const float* packed_Wh, const float* h_tm1,
                             const float* xproj, const float* b, const float* c_tm1, int logistic_mode, float* gates,
                             float* c, float* h);
+int dyhip_lstm_step_forward_packed(dyhip_device* dev, unsigned H, unsigned B, const float* packed_Wh,
+                                   const float* h_tm1_packed, const float* xproj, const float* b, const float* c_tm1,
+                                   int logistic_mode, float* gates, float* c, float* h, float* h_packed);
+/* The backward timestep over the same packed operands: dyhip_lstm_recurrent_backward_packed forms the
+ * slices of Wh^T * dpre (what dyhip_lstm_recurrent_backward does) from a packed copy of Wh^T
+ * (dyhip_lstm_pack_recurrent_transposed, 4*H*H floats) and the packed dpre of the timestep above
+ * (dyhip_lstm_packed_state_floats(4*H, B) floats), which dyhip_lstm_cell_backward_packed writes next to
+ * the plain dpre.  ws holds the slices (the bwd_bytes of dyhip_lstm_cell_workspace suffice). */
+int dyhip_lstm_pack_recurrent_transposed(dyhip_device* dev, unsigned H, const float* Wh, float* packed);
+int dyhip_lstm_recurrent_backward_packed(dyhip_device* dev, unsigned H, unsigned B, const float* packed_WhT,
+                                         const float* dpre_packed, void* ws, size_t ws_bytes, unsigned* splits);
+int dyhip_lstm_cell_backward_packed(dyhip_device* dev, unsigned H, unsigned B, const float* gates, const float* c,
+                                    const float* c_tm1, const float* dh, const float* rec, unsigned splits,
+                                    const float* dc, float* dpre, float* dc_tm1, float* dpre_packed);
 /* The whole forward of a timestep in one launch, input product included: gates = act(b + [f: +1] +
  * Wx * x + Wh * h_tm1) from packed copies of both weight matrices (dyhip_lstm_pack_input: Wx is
- * 4H x I, I a multiple of 128), then c and h.  For callers that see one timestep at a time
- * (decoding, the single-step configuration).  packed_Wh / h_tm1 / c_tm1 = NULL stand for the
- * zero initial state. */
+ * 4H x I, I a multiple of 128), then c and h; x and h_tm1 are plain and packed internally.  For callers
+ * that see one timestep at a time (decoding, the single-step configuration).  packed_Wh / h_tm1 /
+ * c_tm1 = NULL stand for the zero initial state. */
 int dyhip_lstm_pack_input(dyhip_device* dev, unsigned I, unsigned H, const float* Wx, float* packed);
 int dyhip_lstm_step_forward_x(dyhip_device* dev, unsigned I, unsigned H, unsigned B, const float* packed_Wx,
                               const float* x, const float* packed_Wh, const float* h_tm1, const float* b,

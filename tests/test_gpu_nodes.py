@@ -357,6 +357,12 @@ def test_fused_cell_path_equals_node_composition(dev, I, H, B):
                      floor=max(float(np.abs(r_dpre[k]).max()) * 1e-2, 1e-6))
 
 
+def lib_slices(dev, ws, n, size):
+    """The n split slices of `size` floats a recurrent product left in the workspace `ws`."""
+    from dynet_amd.device import DevTensor
+    return DevTensor(dev, ws, (n, size), np.float32).numpy()
+
+
 @pytest.mark.parametrize("I,H,B", [(24, 128, 1), (40, 128, 33), (16, 256, 32), (64, 384, 70), (32, 1024, 128)])
 def test_single_launch_step_equals_node_composition(dev, I, H, B):
     """dyhip_lstm_step_forward (recurrent product + cell update in one kernel, packed Wh) over three
@@ -378,9 +384,20 @@ def test_single_launch_step_equals_node_composition(dev, I, H, B):
     Wxt, Wht, bt = dev.tensor(Wx), dev.tensor(Wh), dev.tensor(b)
     packed = dev.empty(4 * H * H)
     dev.lstm_pack_recurrent(H, Wht, packed)
-    # the packed copy is a permutation of Wh: tile rt, column k, slot g*8+u <- row g*H + rt*8 + u
-    want = Wh.reshape(H, 4, H // 8, 8).transpose(2, 0, 1, 3).reshape(-1)   # Wh is stored [k][row]
+    # the packed copy is a permutation of Wh (stored [k][row]): tile rt, group kg, lane 32*lhi + g*8 + u, slot s
+    # <- row g*H + rt*8 + u, k = 8*kg + 2*s + lhi
+    want = Wh.reshape(H // 8, 4, 2, 4, H // 8, 8).transpose(4, 0, 2, 3, 5, 1).reshape(-1)
     assert np.array_equal(packed.numpy(), want)
+    # and the packed state of h (stored [col][k]): tile ct, group kg, lane 32*lhi + l32, slot s, zero past B
+    Bp = (B + 31) // 32 * 32
+    assert dev.lstm_packed_state_floats(H, B) == H * Bp
+    hv = f32(rng.standard_normal((B, H)))
+    hp_t = dev.empty(H * Bp)
+    dev.lstm_pack_state(H, B, dev.tensor(hv), hp_t)
+    hpad = np.zeros((Bp, H), F32)
+    hpad[:B] = hv
+    pack_cols = lambda a, K: a.reshape(Bp // 32, 32, K // 8, 4, 2).transpose(0, 2, 4, 1, 3).reshape(-1)
+    assert np.array_equal(hp_t.numpy(), pack_cols(hpad, H))
     X = dev.tensor(np.stack(xs))
     xproj = dev.empty((T, B, 4 * H))
     dev.gemm_nn(4 * H, T * B, I, Wxt, X, 0.0, xproj)
@@ -388,8 +405,18 @@ def test_single_launch_step_equals_node_composition(dev, I, H, B):
     fb, _ = dev.lstm_cell_workspace(H, B)
     wf, wfb = dev.workspace(fb)
     out = {}
-    for name in ("step", "two_call"):
+    for name in ("step", "chain", "two_call"):
         gates, cs, hs = dev.empty((T, B, 4 * H)), dev.empty((T, B, H)), dev.empty((T, B, H))
+        if name == "chain":  # every timestep one launch, the packed h handed from step to step
+            hp = [dev.empty(H * Bp), dev.empty(H * Bp)]
+            dev.lstm_step_forward_packed(H, B, None, None, sl(xproj, 0, 4 * H), bt, None, sl(gates, 0, 4 * H),
+                                         sl(cs, 0, H), sl(hs, 0, H), hp[0])
+            for t in range(1, T):
+                dev.lstm_step_forward_packed(H, B, packed, hp[(t - 1) % 2], sl(xproj, t, 4 * H), bt, sl(cs, t - 1, H),
+                                             sl(gates, t, 4 * H), sl(cs, t, H), sl(hs, t, H),
+                                             hp[t % 2] if t + 1 < T else None)
+            out[name] = (gates.numpy(), cs.numpy(), hs.numpy())
+            continue
         dev.lstm_cell_forward(H, B, sl(xproj, 0, 4 * H), bt, None, 0, None, sl(gates, 0, 4 * H), sl(cs, 0, H),
                               sl(hs, 0, H))
         for t in range(1, T):
@@ -409,10 +436,61 @@ def test_single_launch_step_equals_node_composition(dev, I, H, B):
             assert_close(out["step"][q][k], out["two_call"][q][k], FWD_RTOL, f"{what}[{k}] vs two-call", floor=floor)
         exact = _lstm_exact_step(xs[k], h64, c64, Wx, Wh, b)
         _, c64, h64 = exact
-        for name in ("step", "two_call"):
+        assert out["chain"][0][k].tobytes() == out["step"][0][k].tobytes()  # same kernel, same operands
+        for name in ("step", "chain", "two_call"):
             _assert_gates_shadow(out[name][0][k], ref[k][0], exact[0], H, f"gates[{k}] {name}")
             assert_shadow(out[name][1][k], ref[k][1], exact[1], f"c[{k}] {name}", rel_min=0.1)
             assert_shadow(out[name][2][k], ref[k][2], exact[2], f"h[{k}] {name}", rel_min=0.1)
+
+
+@pytest.mark.parametrize("H,B", [(128, 1), (128, 33), (256, 32), (384, 70), (1024, 128)])
+def test_packed_backward_timestep_equals_the_two_call_form(dev, H, B):
+    """dyhip_lstm_cell_backward_packed + dyhip_lstm_recurrent_backward_packed (packed Wh^T and dpre) against
+    dyhip_lstm_cell_backward + dyhip_lstm_recurrent_backward and against fp64."""
+    rng = np.random.default_rng(3 * H + B)
+    Wh = glorot(rng, 4 * H, H)
+    gates = f32(rng.uniform(0.05, 0.95, (B, 4 * H)))
+    gates[:, 3 * H:] = f32(rng.uniform(-0.9, 0.9, (B, H)))
+    c, c_tm1 = f32(rng.standard_normal((B, H))), f32(rng.standard_normal((B, H)))
+    dh, dc = f32(rng.standard_normal((B, H))), f32(rng.standard_normal((B, H)))
+    Wht = dev.tensor(Wh)
+    packedT = dev.empty(4 * H * H)
+    dev.lstm_pack_recurrent_transposed(H, Wht, packedT)
+    # Wh is stored [j][r] (column j of the 4H x H matrix): tile rt of Wh^T, group kg, lane 32*lhi + l32, slot s
+    # <- Wh[r = 8*kg + 2*s + lhi, j = rt*32 + l32]
+    want = Wh.reshape(H // 32, 32, 4 * H // 8, 4, 2).transpose(0, 2, 4, 1, 3).reshape(-1)
+    assert np.array_equal(packedT.numpy(), want)
+    _, bb = dev.lstm_cell_workspace(H, B)
+    ws, wsb = dev.workspace(bb)
+    Bp = (B + 31) // 32 * 32
+    gt, ct, cpt, dht, dct = (dev.tensor(a) for a in (gates, c, c_tm1, dh, dc))
+    # plain form
+    dpre0, dcp0 = dev.empty((B, 4 * H)), dev.empty((B, H))
+    dev.lstm_cell_backward(H, B, gt, ct, cpt, dht, None, 0, dct, dpre0, dcp0)
+    n0 = dev.lstm_recurrent_backward(H, B, Wht, dpre0, ws, wsb)
+    rec0 = lib_slices(dev, ws, n0, H * B).sum(axis=0, dtype=np.float64)
+    # packed form
+    dpre1, dcp1 = dev.empty((B, 4 * H)), dev.empty((B, H))
+    dpp = dev.empty(4 * H * Bp)
+    dev.zero(dpp)
+    dev.lstm_cell_backward_packed(H, B, gt, ct, cpt, dht, None, 0, dct, dpre1, dcp1, dpp)
+    assert dpre1.numpy().tobytes() == dpre0.numpy().tobytes() and dcp1.numpy().tobytes() == dcp0.numpy().tobytes()
+    pad = np.zeros((Bp, 4 * H), F32)
+    pad[:B] = dpre1.numpy()
+    assert np.array_equal(dpp.numpy(), pad.reshape(Bp // 32, 32, 4 * H // 8, 4, 2).transpose(0, 2, 4, 1, 3).reshape(-1))
+    n1 = dev.lstm_recurrent_backward_packed(H, B, packedT, dpp, ws, wsb)
+    rec1 = lib_slices(dev, ws, n1, H * B).sum(axis=0, dtype=np.float64)
+    exact = dpre1.numpy().astype(np.float64) @ Wh.astype(np.float64).T  # (B, 4H) x (4H, H)
+    floor = np.sqrt(4 * H) * rms(Wh) * rms(dpre1.numpy())
+    assert_close(rec1.reshape(B, H), exact, FWD_RTOL, "packed Wh^T dpre vs fp64", floor=floor)
+    assert_close(rec1.reshape(B, H), rec0.reshape(B, H), FWD_RTOL, "packed vs plain recurrent product", floor=floor)
+    # the next timestep down consumes the slices exactly like the plain ones
+    dpre2, dcp2 = dev.empty((B, 4 * H)), dev.empty((B, H))
+    dev.lstm_cell_backward_packed(H, B, gt, ct, cpt, dht, ws, n1, dct, dpre2, dcp2, None)
+    want_dh = dh.astype(np.float64) + rec1.reshape(B, H)
+    t = np.tanh(c.astype(np.float64))
+    dcv = dc + want_dh * gates[:, 2 * H:3 * H] * (1 - t * t)
+    assert_close(dcp2.numpy(), dcv * gates[:, H:2 * H], GRAD_RTOL, "dc_tm1 after the packed product", floor=1.0)
 
 
 @pytest.mark.parametrize("I,H,B", [(128, 256, 32), (256, 128, 1), (128, 128, 45), (384, 256, 70)])
@@ -425,7 +503,7 @@ def test_single_launch_step_with_input_product(dev, I, H, B):
     pWx, pWh = dev.empty(4 * H * I), dev.empty(4 * H * H)
     dev.lstm_pack_input(I, H, Wxt, pWx)
     dev.lstm_pack_recurrent(H, Wht, pWh)
-    assert np.array_equal(pWx.numpy(), Wx.reshape(I, 4, H // 8, 8).transpose(2, 0, 1, 3).reshape(-1))
+    assert np.array_equal(pWx.numpy(), Wx.reshape(I // 8, 4, 2, 4, H // 8, 8).transpose(4, 0, 2, 3, 5, 1).reshape(-1))
     zeros = np.zeros((B, H), F32)
     h_prev, c_prev = zeros, zeros
     ht = ct = None
