@@ -540,7 +540,7 @@ def print_pmc_summary(fetch_db, write_db, unique_ids):
             print("TRAFFIC %s %.0f" % (name, t[name]))
 
 
-def lstm_lm(steps, warmup=3, use_graph=True):
+def lstm_lm(steps, warmup=12, use_graph=True):
     """cfg 5: whole training step of the 2-layer LSTM LM (forward, backward, clip, SGD update), tokens/s."""
     from dynet_amd import Device
     from dynet_amd.lm import LstmLM

@@ -306,28 +306,38 @@ __global__ __launch_bounds__(256) void lstm_pack_state_kernel(unsigned K, unsign
 // branch-free double buffer: four groups are multiplied while the next four are in flight (the last round
 // re-reads its own groups instead of branching around the loads, so the compiler counts the outstanding
 // loads exactly; the scheduling barriers keep it from sinking the loads down to their uses).
+// With PLAIN the state is not packed: pb points at this lane's column of the K x B matrix, at the first k of its
+// depth range plus lane / 32, and a fragment is four strided scalar loads (for callers that hold a plain state
+// and run one timestep at a time; a long chain hands packed states from step to step instead).
+// TILES = 1 leaves the second row tile out (pa1 and acc1 unused): small problems get twice the blocks.
+template <bool PLAIN, int TILES = 2>
 __device__ __forceinline__ void step_product(stepx16& acc0, stepx16& acc1, const float4* __restrict__ pa0,
-                                             const float4* __restrict__ pa1, const float4* __restrict__ pb,
+                                             const float4* __restrict__ pa1, const float* __restrict__ pb,
                                              unsigned groups) {
   float4 a0[4], a1[4], b0[4], c0[4], c1[4], d0[4];
-#define STEP_LOAD(A0, A1, BB, grp)                 \
-  _Pragma("unroll") for (int u = 0; u < 4; ++u) {  \
-    A0[u] = pa0[size_t((grp) + u) * 64];           \
-    A1[u] = pa1[size_t((grp) + u) * 64];           \
-    BB[u] = pb[size_t((grp) + u) * 64];            \
-  }                                                \
+#define STEP_LOAD(A0, A1, BB, grp)                                                                   \
+  _Pragma("unroll") for (int u = 0; u < 4; ++u) {                                                    \
+    A0[u] = pa0[size_t((grp) + u) * 64];                                                             \
+    if (TILES == 2) A1[u] = pa1[size_t((grp) + u) * 64];                                             \
+    if (PLAIN) {                                                                                     \
+      const float* q = pb + size_t((grp) + u) * 8;                                                   \
+      BB[u] = make_float4(q[0], q[2], q[4], q[6]);                                                   \
+    } else {                                                                                         \
+      BB[u] = reinterpret_cast<const float4*>(pb)[size_t((grp) + u) * 64];                           \
+    }                                                                                                \
+  }                                                                                                  \
   __builtin_amdgcn_sched_barrier(0);
 #define STEP_MMA1(x, y, acc) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, acc, 0, 0, 0);
 #define STEP_MMA(A0, A1, BB)                       \
   _Pragma("unroll") for (int u = 0; u < 4; ++u) {  \
     STEP_MMA1(A0[u].x, BB[u].x, acc0)              \
-    STEP_MMA1(A1[u].x, BB[u].x, acc1)              \
+    if (TILES == 2) STEP_MMA1(A1[u].x, BB[u].x, acc1) \
     STEP_MMA1(A0[u].y, BB[u].y, acc0)              \
-    STEP_MMA1(A1[u].y, BB[u].y, acc1)              \
+    if (TILES == 2) STEP_MMA1(A1[u].y, BB[u].y, acc1) \
     STEP_MMA1(A0[u].z, BB[u].z, acc0)              \
-    STEP_MMA1(A1[u].z, BB[u].z, acc1)              \
+    if (TILES == 2) STEP_MMA1(A1[u].z, BB[u].z, acc1) \
     STEP_MMA1(A0[u].w, BB[u].w, acc0)              \
-    STEP_MMA1(A1[u].w, BB[u].w, acc1)              \
+    if (TILES == 2) STEP_MMA1(A1[u].w, BB[u].w, acc1) \
   }                                                \
   __builtin_amdgcn_sched_barrier(0);
   const unsigned full = groups / 8 * 8;
@@ -358,35 +368,30 @@ struct StepOperand {
   unsigned K;
 };
 
+template <bool PLAIN, int TILES>
 __global__ __launch_bounds__(256) void lstm_step_fwd_kernel(unsigned H, unsigned B, StepOperand op0, StepOperand op1,
                                                             const float* xproj, const float* __restrict__ bias,
                                                             const float* __restrict__ c_prev, int mode, float* gates,
                                                             float* __restrict__ c, float* __restrict__ h,
                                                             float* __restrict__ hp) {
-  __shared__ float red[4 * 64 * kStepPitchR];
-  const unsigned RP = H / 16;  // pairs of row tiles = groups of 16 hidden units
+  constexpr int UB = 8 * TILES;       // hidden units of a block (its 32*TILES weight rows are their four gate rows)
+  constexpr int ROWS = 32 * TILES;
+  constexpr int CSTEP = 256 / UB;     // columns an epilogue thread strides by
+  __shared__ float red[4 * ROWS * kStepPitchR];
+  const unsigned RP = H / UB;
   const unsigned rp = blockIdx.x % RP, ct = blockIdx.x / RP;
   const unsigned wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const unsigned l32 = lane % 32, lhi = lane / 32;
 
-  stepx16 acc0 = {0}, acc1 = {0};
-  for (int which = 0; which < 2; ++which) {
-    const StepOperand op = which == 0 ? op0 : op1;
-    if (op.Wp == nullptr) continue;  // uniform over the grid
-    const unsigned G = op.K / 8, gq = G / 4, g0 = wave * gq;
-    const float4* pa = reinterpret_cast<const float4*>(op.Wp) + (size_t(2 * rp) * G + g0) * 64 + lane;
-    step_product(acc0, acc1, pa, pa + size_t(G) * 64,
-                 reinterpret_cast<const float4*>(op.vp) + (size_t(ct) * G + g0) * 64 + lane, gq);
-  }
-
-  // The epilogue's thread owns hidden unit eu (of 16) of batch columns ecc and ecc + 16.  Its operands are
-  // requested only now: loads return in order, so asking for them before the product would hold up the
-  // product's first fragments; here their latency hides behind the exchange of the partial sums.
-  const unsigned eu = threadIdx.x % 16, ecc = threadIdx.x / 16, ej = rp * 16 + eu;
-  float pre[2][4], cp[2] = {0.f, 0.f};
+  // The epilogue's thread owns hidden unit eu (of UB) of batch columns ecc + CSTEP*i; its operands are fetched
+  // now so that their latency hides behind the product (it matters for small problems, which are one chain of
+  // latencies; at H = 1024, B = 128 fetching them after the product measures the same).
+  const unsigned eu = threadIdx.x % UB, ecc = threadIdx.x / UB, ej = rp * UB + eu;
+  float pre[TILES][4], cp[TILES];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const unsigned ecol = ct * 32 + ecc + 16 * i;
+  for (int i = 0; i < TILES; ++i) {
+    const unsigned ecol = ct * 32 + ecc + CSTEP * i;
+    cp[i] = 0.f;
 #pragma unroll
     for (int q = 0; q < 4; ++q) pre[i][q] = 0.f;
     if (ecol < B) {
@@ -400,24 +405,36 @@ __global__ __launch_bounds__(256) void lstm_step_fwd_kernel(unsigned H, unsigned
     }
   }
 
-  // the four quarter sums meet in LDS: rows 0..31 = first tile of the pair, 32..63 = second
+  stepx16 acc0 = {0}, acc1 = {0};
+  for (int which = 0; which < 2; ++which) {
+    const StepOperand op = which == 0 ? op0 : op1;
+    if (op.Wp == nullptr) continue;  // uniform over the grid
+    const unsigned G = op.K / 8, gq = G / 4, g0 = wave * gq;
+    const float4* pa = reinterpret_cast<const float4*>(op.Wp) + (size_t(TILES * rp) * G + g0) * 64 + lane;
+    // plain state: columns past the batch are computed on a clamped address and dropped
+    const unsigned pcol = ct * 32 + l32 < B ? ct * 32 + l32 : B - 1;
+    const float* pb = PLAIN ? op.vp + size_t(pcol) * op.K + size_t(g0) * 8 + lhi : op.vp + ((size_t(ct) * G + g0) * 64 + lane) * 4;
+    step_product<PLAIN, TILES>(acc0, acc1, pa, pa + size_t(G) * 64, pb, gq);
+  }
+
+  // the four quarter sums meet in LDS: rows 0..31 = first tile, 32..63 = second
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const unsigned row = 8 * (r / 4) + 4 * lhi + (r % 4);
-    red[(wave * 64 + row) * kStepPitchR + l32] = acc0[r];
-    red[(wave * 64 + 32 + row) * kStepPitchR + l32] = acc1[r];
+    red[(wave * ROWS + row) * kStepPitchR + l32] = acc0[r];
+    if (TILES == 2) red[(wave * ROWS + 32 + row) * kStepPitchR + l32] = acc1[r];
   }
   __syncthreads();
 
   const unsigned tile = eu / 8, u = eu % 8;
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const unsigned col = ecc + 16 * i, ecol = ct * 32 + col;
+  for (int i = 0; i < TILES; ++i) {
+    const unsigned col = ecc + CSTEP * i, ecol = ct * 32 + col;
     if (ecol >= B) continue;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
 #pragma unroll
-      for (int w = 0; w < 4; ++w) pre[i][q] += red[(w * 64 + tile * 32 + q * 8 + u) * kStepPitchR + col];
+      for (int w = 0; w < 4; ++w) pre[i][q] += red[(w * ROWS + tile * 32 + q * 8 + u) * kStepPitchR + col];
     }
     const float gi = logistic(mode, pre[i][0]), gf = logistic(mode, pre[i][1]), go = logistic(mode, pre[i][2]);
     const float gg = tanh_accurate(pre[i][3]);
@@ -430,8 +447,8 @@ __global__ __launch_bounds__(256) void lstm_step_fwd_kernel(unsigned H, unsigned
     gates[g0 + 3 * size_t(H)] = gg;
     c[s0] = cv;
     h[s0] = hv;
-    // h again, as the next timestep's packed operand: unit ej is k = 8*(2*rp + tile) + u
-    if (hp != nullptr) hp[((size_t(ct) * (H / 8) + 2 * rp + tile) * 64 + (u % 2) * 32 + col) * 4 + u / 2] = hv;
+    // h again, as the next timestep's packed operand: unit ej is k = 8*(TILES*rp + tile) + u
+    if (hp != nullptr) hp[((size_t(ct) * (H / 8) + TILES * rp + tile) * 64 + (u % 2) * 32 + col) * 4 + u / 2] = hv;
   }
 }
 
@@ -448,8 +465,7 @@ __global__ __launch_bounds__(256) void lstm_rec_bwd_kernel(unsigned H, unsigned 
   const unsigned G = H / 2, gq = G / (4 * gridDim.y), g0 = (split * 4 + wave) * gq;
   stepx16 acc0 = {0}, acc1 = {0};
   const float4* pa = reinterpret_cast<const float4*>(WpT) + (size_t(2 * rp) * G + g0) * 64 + lane;
-  step_product(acc0, acc1, pa, pa + size_t(G) * 64, reinterpret_cast<const float4*>(dpp) + (size_t(ct) * G + g0) * 64 + lane,
-               gq);
+  step_product<false>(acc0, acc1, pa, pa + size_t(G) * 64, dpp + ((size_t(ct) * G + g0) * 64 + lane) * 4, gq);
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const unsigned row = 8 * (r / 4) + 4 * lhi + (r % 4);
@@ -853,10 +869,9 @@ int dyhip_lstm_pack_state(dyhip_device* dev, unsigned rows, unsigned B, const fl
   return pack_state(dev, rows, B, v, packed);
 }
 
-// x and h_tm1 arrive packed (x_packed / h_packed true) or plain; a plain operand is packed into the queue's
-// GEMM workspace first (one more launch; nothing else of this queue uses the workspace meanwhile).
+// x and h_tm1 are both packed or both plain (the plain form reads them with strided loads, no extra launch).
 static int step_forward(dyhip_device* dev, unsigned I, unsigned H, unsigned B, const float* packed_Wx, const float* x,
-                        bool x_packed, const float* packed_Wh, const float* h_tm1, bool h_packed, const float* xproj,
+                        const float* packed_Wh, const float* h_tm1, bool states_packed, const float* xproj,
                         const float* b, const float* c_tm1, int logistic_mode, float* gates, float* c, float* h,
                         float* hp_out) {
   int ok = 0;
@@ -870,26 +885,22 @@ static int step_forward(dyhip_device* dev, unsigned I, unsigned H, unsigned B, c
                 "LSTM step: weights and operands must be 16-byte aligned");
   DYHIP_REQUIRE(logistic_mode == DYHIP_LOGISTIC_PACKET || logistic_mode == DYHIP_LOGISTIC_SCALAR,
                 "unknown logistic mode %d", logistic_mode);
-  float* scratch = static_cast<float*>(dev->gemm_ws);
-  size_t scratch_floats = dev->gemm_ws_bytes / sizeof(float);
-  if (x != nullptr && !x_packed) {
-    const size_t n = packed_state_floats(I, B);
-    DYHIP_REQUIRE(scratch != nullptr && n <= scratch_floats, "LSTM step: no room to pack the input");
-    DYHIP_CHECK_STATUS(pack_state(dev, I, B, x, scratch));
-    x = scratch;
-    scratch += n;
-    scratch_floats -= n;
-  }
-  if (h_tm1 != nullptr && !h_packed) {
-    const size_t n = packed_state_floats(H, B);
-    DYHIP_REQUIRE(scratch != nullptr && n <= scratch_floats, "LSTM step: no room to pack the state");
-    DYHIP_CHECK_STATUS(pack_state(dev, H, B, h_tm1, scratch));
-    h_tm1 = scratch;
-  }
   const StepOperand op0{packed_Wx, x, I}, op1{packed_Wh, h_tm1, H};
-  const unsigned blocks = (H / 16) * cdiv<unsigned>(B, 32);
-  hipLaunchKernelGGL(lstm_step_fwd_kernel, dim3(blocks), dim3(256), 0, dev->stream, H, B, op0, op1, xproj, b, c_tm1,
-                     logistic_mode, gates, c, h, hp_out);
+  // 64-row tiles (fewest operand bytes per CU) once they give half the CUs a block, 32-row tiles below that
+  const unsigned blocks2 = (H / 16) * cdiv<unsigned>(B, 32);
+  const bool two = blocks2 * 2 >= unsigned(dev->num_cus > 0 ? dev->num_cus : 256);
+  const dim3 grid(two ? blocks2 : blocks2 * 2), block(256);
+#define DYHIP_STEP(PLAIN, TILES)                                                                                     \
+  hipLaunchKernelGGL((lstm_step_fwd_kernel<PLAIN, TILES>), grid, block, 0, dev->stream, H, B, op0, op1, xproj, b, c_tm1, \
+                     logistic_mode, gates, c, h, hp_out)
+  if (states_packed) {
+    if (two) DYHIP_STEP(false, 2);
+    else DYHIP_STEP(false, 1);
+  } else {
+    if (two) DYHIP_STEP(true, 2);
+    else DYHIP_STEP(true, 1);
+  }
+#undef DYHIP_STEP
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
@@ -899,8 +910,8 @@ int dyhip_lstm_step_forward(dyhip_device* dev, unsigned H, unsigned B, const flo
                             float* c, float* h) {
   DYHIP_CHECK_DEV(dev);
   DYHIP_REQUIRE(packed_Wh && h_tm1 && xproj && c_tm1, "LSTM step: null tensor pointer");
-  return step_forward(dev, 0, H, B, nullptr, nullptr, false, packed_Wh, h_tm1, false, xproj, b, c_tm1, logistic_mode,
-                      gates, c, h, nullptr);
+  return step_forward(dev, 0, H, B, nullptr, nullptr, packed_Wh, h_tm1, false, xproj, b, c_tm1, logistic_mode, gates, c,
+                      h, nullptr);
 }
 
 int dyhip_lstm_step_forward_packed(dyhip_device* dev, unsigned H, unsigned B, const float* packed_Wh,
@@ -910,8 +921,8 @@ int dyhip_lstm_step_forward_packed(dyhip_device* dev, unsigned H, unsigned B, co
   DYHIP_REQUIRE(xproj != nullptr, "LSTM step: null tensor pointer");
   DYHIP_REQUIRE((packed_Wh == nullptr) == (h_tm1_packed == nullptr) && (packed_Wh == nullptr) == (c_tm1 == nullptr),
                 "LSTM step: the recurrent weights, the packed state and c_tm1 come together (all null = zero state)");
-  return step_forward(dev, 0, H, B, nullptr, nullptr, false, packed_Wh, h_tm1_packed, true, xproj, b, c_tm1,
-                      logistic_mode, gates, c, h, h_packed);
+  return step_forward(dev, 0, H, B, nullptr, nullptr, packed_Wh, h_tm1_packed, true, xproj, b, c_tm1, logistic_mode,
+                      gates, c, h, h_packed);
 }
 
 int dyhip_lstm_step_forward_x(dyhip_device* dev, unsigned I, unsigned H, unsigned B, const float* packed_Wx,
@@ -919,8 +930,8 @@ int dyhip_lstm_step_forward_x(dyhip_device* dev, unsigned I, unsigned H, unsigne
                               const float* c_tm1, int logistic_mode, float* gates, float* c, float* h) {
   DYHIP_CHECK_DEV(dev);
   DYHIP_REQUIRE(packed_Wx && x, "LSTM step: null tensor pointer");
-  return step_forward(dev, I, H, B, packed_Wx, x, false, packed_Wh, h_tm1, false, nullptr, b, c_tm1, logistic_mode, gates,
-                      c, h, nullptr);
+  return step_forward(dev, I, H, B, packed_Wx, x, packed_Wh, h_tm1, false, nullptr, b, c_tm1, logistic_mode, gates, c, h,
+                      nullptr);
 }
 
 // depth ranges of the backward product: enough blocks for every CU, whole sets of four groups per wave

@@ -319,7 +319,7 @@ int dyhip_lstm_cell_backward(dyhip_device* dev, unsigned H, unsigned B, const fl
  * (dyhip_lstm_packed_state_floats(H, B) floats).  Supported when H is a multiple of 128
  * (dyhip_lstm_step_supported reports it; the two-call form above covers every other size).  Same
  * results as the two-call form up to fp32 summation order.  gates may alias xproj.
- *   dyhip_lstm_step_forward         h_tm1 plain (H x B): packed internally by one extra launch
+ *   dyhip_lstm_step_forward         h_tm1 plain (H x B), read with strided loads: for single timesteps
  *   dyhip_lstm_step_forward_packed  h_tm1 packed; also writes h_packed (may be null), the packed copy of
  *                                   the new h, so a chain of timesteps never repacks; packed_Wh =
  *                                   h_tm1_packed = c_tm1 = NULL stand for the zero initial state
@@ -347,7 +347,7 @@ int dyhip_lstm_cell_backward_packed(dyhip_device* dev, unsigned H, unsigned B, c
                                     const float* dc, float* dpre, float* dc_tm1, float* dpre_packed);
 /* The whole forward of a timestep in one launch, input product included: gates = act(b + [f: +1] +
  * Wx * x + Wh * h_tm1) from packed copies of both weight matrices (dyhip_lstm_pack_input: Wx is
- * 4H x I, I a multiple of 128), then c and h; x and h_tm1 are plain and packed internally.  For callers
+ * 4H x I, I a multiple of 128), then c and h; x and h_tm1 are plain.  For callers
  * that see one timestep at a time (decoding, the single-step configuration).  packed_Wh / h_tm1 /
  * c_tm1 = NULL stand for the zero initial state. */
 int dyhip_lstm_pack_input(dyhip_device* dev, unsigned I, unsigned H, const float* Wx, float* packed);
