@@ -233,12 +233,10 @@ __global__ __launch_bounds__(kCellThreads) void lstm_cell_bwd_kernel(unsigned H,
   if (dpre_packed != nullptr) {
     const size_t tile = size_t(b / 32) * (H / 2) * 256 + (b % 32) * 4;  // column tile of 4H/8 groups of 256 floats
 #pragma unroll
-    for (int q = 0; q < 4; ++q)
-#pragma unroll
-      for (int e = 0; e < V; ++e) {
-        const unsigned k = q * H + j + e;
-        dpre_packed[tile + size_t(k / 8) * 256 + (k % 2) * 128 + (k % 8) / 2] = out[q].v[e];
-      }
+    for (int q = 0; q < 4; ++q) {
+      const unsigned k = q * H + j;  // k .. k+V-1 are the slots of one lane: k = 8*kg + 4*lhi + s
+      out[q].store(dpre_packed + tile + size_t(k / 8) * 256 + ((k % 8) / 4) * 128 + k % 4);
+    }
   }
 }
 
@@ -254,8 +252,9 @@ __global__ __launch_bounds__(kCellThreads) void lstm_cell_bwd_kernel(unsigned H,
 // operand bytes per CU that still gives every CU a block at H = 1024, B = 128: (64 + 32) rows and
 // columns of depth H per block.  Both operands are read in MFMA fragment order straight into
 // registers (no LDS stage, no barrier in the loop): for a 32-wide tile and a group of 8 consecutive
-// k, lane l = 32*lhi + l32 holds k = 8*kg + 2*s + lhi, s = 0..3, of row (or column) l32 as one
-// float4, and a group of a tile is 1 KiB contiguous.
+// k, lane l = 32*lhi + l32 holds k = 8*kg + 4*lhi + s, s = 0..3, of row (or column) l32 as one
+// float4 (MFMA step s of the group multiplies k = 8*kg + s and 8*kg + 4 + s; the order inside a
+// group is free as long as both operands agree), and a group of a tile is 1 KiB contiguous.
 //   weights  Wp[rows/32][K/8][64][4]   forward: row g*H + rt*8 + u of W at l32 = g*8 + u of tile rt;
 //                                      backward: row rt*32 + l32 of W^T (dyhip_lstm_pack_*)
 //   state    vp[ceil(B/32)][K/8][64][4]   column ct*32 + l32 (dyhip_lstm_pack_state, or the packed h /
@@ -274,7 +273,7 @@ __global__ __launch_bounds__(256) void lstm_pack_weights_kernel(unsigned H, unsi
   const unsigned s = o % 4, lane = (o / 4) % 64, l32 = lane % 32, lhi = lane / 32;
   const size_t tg = o / 256;
   const unsigned kg = tg % (K / 8), rt = tg / (K / 8);
-  const unsigned g = l32 / 8, u = l32 % 8, k = 8 * kg + 2 * s + lhi;
+  const unsigned g = l32 / 8, u = l32 % 8, k = 8 * kg + 4 * lhi + s;
   Wp[o] = W[size_t(g) * H + rt * 8 + u + size_t(k) * 4 * H];
 }
 
@@ -286,7 +285,7 @@ __global__ __launch_bounds__(256) void lstm_pack_transposed_kernel(unsigned H, c
   const unsigned s = o % 4, lane = (o / 4) % 64, l32 = lane % 32, lhi = lane / 32;
   const size_t tg = o / 256;
   const unsigned kg = tg % (H / 2), rt = tg / (H / 2);
-  Wp[o] = W[size_t(rt * 32 + l32) * 4 * H + 8 * kg + 2 * s + lhi];
+  Wp[o] = W[size_t(rt * 32 + l32) * 4 * H + 8 * kg + 4 * lhi + s];
 }
 
 // v is K x B column-major
@@ -297,7 +296,7 @@ __global__ __launch_bounds__(256) void lstm_pack_state_kernel(unsigned K, unsign
   const unsigned s = o % 4, lane = (o / 4) % 64, l32 = lane % 32, lhi = lane / 32;
   const size_t tg = o / 256;
   const unsigned kg = tg % (K / 8), ct = tg / (K / 8);
-  const unsigned col = ct * 32 + l32, k = 8 * kg + 2 * s + lhi;
+  const unsigned col = ct * 32 + l32, k = 8 * kg + 4 * lhi + s;
   vp[o] = col < B ? v[size_t(col) * K + k] : 0.f;
 }
 
@@ -307,8 +306,8 @@ __global__ __launch_bounds__(256) void lstm_pack_state_kernel(unsigned K, unsign
 // re-reads its own groups instead of branching around the loads, so the compiler counts the outstanding
 // loads exactly; the scheduling barriers keep it from sinking the loads down to their uses).
 // With PLAIN the state is not packed: pb points at this lane's column of the K x B matrix, at the first k of its
-// depth range plus lane / 32, and a fragment is four strided scalar loads (for callers that hold a plain state
-// and run one timestep at a time; a long chain hands packed states from step to step instead).
+// depth range plus 4 * (lane / 32); a fragment is then the 128-bit load of four consecutive k of that column
+// (32 segments of 32 bytes per wave and load where the packed form has 1 KiB contiguous).
 // TILES = 1 leaves the second row tile out (pa1 and acc1 unused): small problems get twice the blocks.
 template <bool PLAIN, int TILES = 2>
 __device__ __forceinline__ void step_product(stepx16& acc0, stepx16& acc1, const float4* __restrict__ pa0,
@@ -320,8 +319,7 @@ __device__ __forceinline__ void step_product(stepx16& acc0, stepx16& acc1, const
     A0[u] = pa0[size_t((grp) + u) * 64];                                                             \
     if (TILES == 2) A1[u] = pa1[size_t((grp) + u) * 64];                                             \
     if (PLAIN) {                                                                                     \
-      const float* q = pb + size_t((grp) + u) * 8;                                                   \
-      BB[u] = make_float4(q[0], q[2], q[4], q[6]);                                                   \
+      BB[u] = *reinterpret_cast<const float4*>(pb + size_t((grp) + u) * 8);                          \
     } else {                                                                                         \
       BB[u] = reinterpret_cast<const float4*>(pb)[size_t((grp) + u) * 64];                           \
     }                                                                                                \
@@ -413,7 +411,7 @@ __global__ __launch_bounds__(256) void lstm_step_fwd_kernel(unsigned H, unsigned
     const float4* pa = reinterpret_cast<const float4*>(op.Wp) + (size_t(TILES * rp) * G + g0) * 64 + lane;
     // plain state: columns past the batch are computed on a clamped address and dropped
     const unsigned pcol = ct * 32 + l32 < B ? ct * 32 + l32 : B - 1;
-    const float* pb = PLAIN ? op.vp + size_t(pcol) * op.K + size_t(g0) * 8 + lhi : op.vp + ((size_t(ct) * G + g0) * 64 + lane) * 4;
+    const float* pb = PLAIN ? op.vp + size_t(pcol) * op.K + size_t(g0) * 8 + 4 * lhi : op.vp + ((size_t(ct) * G + g0) * 64 + lane) * 4;
     step_product<PLAIN, TILES>(acc0, acc1, pa, pa + size_t(G) * 64, pb, gq);
   }
 
@@ -448,7 +446,7 @@ __global__ __launch_bounds__(256) void lstm_step_fwd_kernel(unsigned H, unsigned
     c[s0] = cv;
     h[s0] = hv;
     // h again, as the next timestep's packed operand: unit ej is k = 8*(TILES*rp + tile) + u
-    if (hp != nullptr) hp[((size_t(ct) * (H / 8) + TILES * rp + tile) * 64 + (u % 2) * 32 + col) * 4 + u / 2] = hv;
+    if (hp != nullptr) hp[((size_t(ct) * (H / 8) + TILES * rp + tile) * 64 + (u / 4) * 32 + col) * 4 + u % 4] = hv;
   }
 }
 

@@ -319,7 +319,7 @@ int dyhip_lstm_cell_backward(dyhip_device* dev, unsigned H, unsigned B, const fl
  * (dyhip_lstm_packed_state_floats(H, B) floats).  Supported when H is a multiple of 128
  * (dyhip_lstm_step_supported reports it; the two-call form above covers every other size).  Same
  * results as the two-call form up to fp32 summation order.  gates may alias xproj.
- *   dyhip_lstm_step_forward         h_tm1 plain (H x B), read with strided loads: for single timesteps
+ *   dyhip_lstm_step_forward         h_tm1 plain (H x B): for single timesteps
  *   dyhip_lstm_step_forward_packed  h_tm1 packed; also writes h_packed (may be null), the packed copy of
  *                                   the new h, so a chain of timesteps never repacks; packed_Wh =
  *                                   h_tm1_packed = c_tm1 = NULL stand for the zero initial state

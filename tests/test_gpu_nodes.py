@@ -385,8 +385,8 @@ def test_single_launch_step_equals_node_composition(dev, I, H, B):
     packed = dev.empty(4 * H * H)
     dev.lstm_pack_recurrent(H, Wht, packed)
     # the packed copy is a permutation of Wh (stored [k][row]): tile rt, group kg, lane 32*lhi + g*8 + u, slot s
-    # <- row g*H + rt*8 + u, k = 8*kg + 2*s + lhi
-    want = Wh.reshape(H // 8, 4, 2, 4, H // 8, 8).transpose(4, 0, 2, 3, 5, 1).reshape(-1)
+    # <- row g*H + rt*8 + u, k = 8*kg + 4*lhi + s
+    want = Wh.reshape(H // 8, 2, 4, 4, H // 8, 8).transpose(4, 0, 1, 3, 5, 2).reshape(-1)
     assert np.array_equal(packed.numpy(), want)
     # and the packed state of h (stored [col][k]): tile ct, group kg, lane 32*lhi + l32, slot s, zero past B
     Bp = (B + 31) // 32 * 32
@@ -396,7 +396,7 @@ def test_single_launch_step_equals_node_composition(dev, I, H, B):
     dev.lstm_pack_state(H, B, dev.tensor(hv), hp_t)
     hpad = np.zeros((Bp, H), F32)
     hpad[:B] = hv
-    pack_cols = lambda a, K: a.reshape(Bp // 32, 32, K // 8, 4, 2).transpose(0, 2, 4, 1, 3).reshape(-1)
+    pack_cols = lambda a, K: a.reshape(Bp // 32, 32, K // 8, 2, 4).transpose(0, 2, 3, 1, 4).reshape(-1)
     assert np.array_equal(hp_t.numpy(), pack_cols(hpad, H))
     X = dev.tensor(np.stack(xs))
     xproj = dev.empty((T, B, 4 * H))
@@ -457,8 +457,8 @@ def test_packed_backward_timestep_equals_the_two_call_form(dev, H, B):
     packedT = dev.empty(4 * H * H)
     dev.lstm_pack_recurrent_transposed(H, Wht, packedT)
     # Wh is stored [j][r] (column j of the 4H x H matrix): tile rt of Wh^T, group kg, lane 32*lhi + l32, slot s
-    # <- Wh[r = 8*kg + 2*s + lhi, j = rt*32 + l32]
-    want = Wh.reshape(H // 32, 32, 4 * H // 8, 4, 2).transpose(0, 2, 4, 1, 3).reshape(-1)
+    # <- Wh[r = 8*kg + 4*lhi + s, j = rt*32 + l32]
+    want = Wh.reshape(H // 32, 32, 4 * H // 8, 2, 4).transpose(0, 2, 3, 1, 4).reshape(-1)
     assert np.array_equal(packedT.numpy(), want)
     _, bb = dev.lstm_cell_workspace(H, B)
     ws, wsb = dev.workspace(bb)
@@ -477,7 +477,7 @@ def test_packed_backward_timestep_equals_the_two_call_form(dev, H, B):
     assert dpre1.numpy().tobytes() == dpre0.numpy().tobytes() and dcp1.numpy().tobytes() == dcp0.numpy().tobytes()
     pad = np.zeros((Bp, 4 * H), F32)
     pad[:B] = dpre1.numpy()
-    assert np.array_equal(dpp.numpy(), pad.reshape(Bp // 32, 32, 4 * H // 8, 4, 2).transpose(0, 2, 4, 1, 3).reshape(-1))
+    assert np.array_equal(dpp.numpy(), pad.reshape(Bp // 32, 32, 4 * H // 8, 2, 4).transpose(0, 2, 3, 1, 4).reshape(-1))
     n1 = dev.lstm_recurrent_backward_packed(H, B, packedT, dpp, ws, wsb)
     rec1 = lib_slices(dev, ws, n1, H * B).sum(axis=0, dtype=np.float64)
     exact = dpre1.numpy().astype(np.float64) @ Wh.astype(np.float64).T  # (B, 4H) x (4H, H)
@@ -503,7 +503,7 @@ def test_single_launch_step_with_input_product(dev, I, H, B):
     pWx, pWh = dev.empty(4 * H * I), dev.empty(4 * H * H)
     dev.lstm_pack_input(I, H, Wxt, pWx)
     dev.lstm_pack_recurrent(H, Wht, pWh)
-    assert np.array_equal(pWx.numpy(), Wx.reshape(I // 8, 4, 2, 4, H // 8, 8).transpose(4, 0, 2, 3, 5, 1).reshape(-1))
+    assert np.array_equal(pWx.numpy(), Wx.reshape(I // 8, 2, 4, 4, H // 8, 8).transpose(4, 0, 1, 3, 5, 2).reshape(-1))
     zeros = np.zeros((B, H), F32)
     h_prev, c_prev = zeros, zeros
     ht = ct = None
