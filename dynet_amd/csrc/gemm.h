@@ -51,4 +51,9 @@ struct GemmBatch {
 int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N, int nseg, const GemmSeg* segs,
              float* C, const GemmEpiParams& epi, const GemmBatch* batch = nullptr);
 
+// lstm.hip: C = beta * C + A^T B by the fragment-order product for small outputs with deep sums (A is K x M, B is
+// K x N, k contiguous); *taken tells whether it ran or the shape should go to gemm_run.
+int skinny_tn_gemm(dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B,
+                   size_t ldb, float beta, float* C, bool* taken);
+
 }  // namespace dyhip

@@ -512,6 +512,11 @@ int dyhip_affine_forward(dyhip_device* dev, size_t M, size_t N, size_t K, const 
 int dyhip_gemm_tn(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float beta,
                   float* y) {
   DYHIP_CHECK_DEV(dev);
+  if (l != nullptr && r != nullptr && y != nullptr) {
+    bool taken = false;
+    DYHIP_CHECK_STATUS(skinny_tn_gemm(dev, M, N, K, l, K, r, K, beta, y, &taken));
+    if (taken) return DYHIP_OK;
+  }
   GemmSeg s{l, K, r, K, K};
   return gemm_run(dev, true, true, M, N, 1, &s, y, axpby(beta));
 }

@@ -305,24 +305,22 @@ __global__ __launch_bounds__(256) void lstm_pack_state_kernel(unsigned K, unsign
 // branch-free double buffer: four groups are multiplied while the next four are in flight (the last round
 // re-reads its own groups instead of branching around the loads, so the compiler counts the outstanding
 // loads exactly; the scheduling barriers keep it from sinking the loads down to their uses).
-// With PLAIN the state is not packed: pb points at this lane's column of the K x B matrix, at the first k of its
-// depth range plus 4 * (lane / 32); a fragment is then the 128-bit load of four consecutive k of that column
+// Every pointer names this lane's fragment of the first group; the next group is 256 floats on for a packed
+// operand and 8 floats on for a plain one (PLAIN_A / PLAIN_B): a matrix stored with k contiguous per row (or
+// column) needs no packing, its fragment is the 128-bit load of four consecutive k at row l32, offset 4 * lhi
 // (32 segments of 32 bytes per wave and load where the packed form has 1 KiB contiguous).
 // TILES = 1 leaves the second row tile out (pa1 and acc1 unused): small problems get twice the blocks.
-template <bool PLAIN, int TILES = 2>
-__device__ __forceinline__ void step_product(stepx16& acc0, stepx16& acc1, const float4* __restrict__ pa0,
-                                             const float4* __restrict__ pa1, const float* __restrict__ pb,
+template <bool PLAIN_A, bool PLAIN_B, int TILES = 2>
+__device__ __forceinline__ void step_product(stepx16& acc0, stepx16& acc1, const float* __restrict__ pa0,
+                                             const float* __restrict__ pa1, const float* __restrict__ pb,
                                              unsigned groups) {
+  constexpr size_t SA = PLAIN_A ? 8 : 256, SB = PLAIN_B ? 8 : 256;
   float4 a0[4], a1[4], b0[4], c0[4], c1[4], d0[4];
 #define STEP_LOAD(A0, A1, BB, grp)                                                                   \
   _Pragma("unroll") for (int u = 0; u < 4; ++u) {                                                    \
-    A0[u] = pa0[size_t((grp) + u) * 64];                                                             \
-    if (TILES == 2) A1[u] = pa1[size_t((grp) + u) * 64];                                             \
-    if (PLAIN) {                                                                                     \
-      BB[u] = *reinterpret_cast<const float4*>(pb + size_t((grp) + u) * 8);                          \
-    } else {                                                                                         \
-      BB[u] = reinterpret_cast<const float4*>(pb)[size_t((grp) + u) * 64];                           \
-    }                                                                                                \
+    A0[u] = *reinterpret_cast<const float4*>(pa0 + size_t((grp) + u) * SA);                          \
+    if (TILES == 2) A1[u] = *reinterpret_cast<const float4*>(pa1 + size_t((grp) + u) * SA);          \
+    BB[u] = *reinterpret_cast<const float4*>(pb + size_t((grp) + u) * SB);                           \
   }                                                                                                  \
   __builtin_amdgcn_sched_barrier(0);
 #define STEP_MMA1(x, y, acc) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, acc, 0, 0, 0);
@@ -408,11 +406,11 @@ __global__ __launch_bounds__(256) void lstm_step_fwd_kernel(unsigned H, unsigned
     const StepOperand op = which == 0 ? op0 : op1;
     if (op.Wp == nullptr) continue;  // uniform over the grid
     const unsigned G = op.K / 8, gq = G / 4, g0 = wave * gq;
-    const float4* pa = reinterpret_cast<const float4*>(op.Wp) + (size_t(TILES * rp) * G + g0) * 64 + lane;
+    const float* pa = op.Wp + ((size_t(TILES * rp) * G + g0) * 64 + lane) * 4;
     // plain state: columns past the batch are computed on a clamped address and dropped
     const unsigned pcol = ct * 32 + l32 < B ? ct * 32 + l32 : B - 1;
     const float* pb = PLAIN ? op.vp + size_t(pcol) * op.K + size_t(g0) * 8 + 4 * lhi : op.vp + ((size_t(ct) * G + g0) * 64 + lane) * 4;
-    step_product<PLAIN, TILES>(acc0, acc1, pa, pa + size_t(G) * 64, pb, gq);
+    step_product<false, PLAIN, TILES>(acc0, acc1, pa, pa + size_t(G) * 256, pb, gq);
   }
 
   // the four quarter sums meet in LDS: rows 0..31 = first tile, 32..63 = second
@@ -450,20 +448,39 @@ __global__ __launch_bounds__(256) void lstm_step_fwd_kernel(unsigned H, unsigned
   }
 }
 
-// Recurrent product of the backward timestep: slice[split] = (Wh^T)[64 hidden units, depth range] x dpre[depth
-// range, 32 columns], the same tile and operand order as the forward kernel; the depth 4H is cut into
-// gridDim.y ranges so that every CU has a block, and the cell kernel adds the slices in ascending order.
-__global__ __launch_bounds__(256) void lstm_rec_bwd_kernel(unsigned H, unsigned B, const float* __restrict__ WpT,
-                                                           const float* __restrict__ dpp, float* __restrict__ slices) {
+// Skinny transposed product: slice[split] = A^T[M rows, depth range] x B[depth range, N columns] for M x N small
+// and the depth K large (the backward timestep's Wh^T * dpre, and dx = Wx^T * dpre of the gates node): the same
+// 64x32 tile and operand order as the forward kernel; K is cut into gridDim.y ranges so that every CU has a block,
+// and whoever consumes the slices adds them in ascending order.  A is K x M and B is K x N, both with k contiguous
+// (leading dimensions lda, ldb), read plain, or packed in fragment order.  Rows and columns past M and N are
+// computed on clamped addresses and dropped.
+template <bool PLAIN_A, bool PLAIN_B>
+__global__ __launch_bounds__(256) void skinny_tn_kernel(unsigned M, unsigned N, unsigned K, const float* __restrict__ A,
+                                                        size_t lda, const float* __restrict__ Bm, size_t ldb,
+                                                        float* __restrict__ slices) {
   __shared__ float red[4 * 64 * kStepPitchR];
-  const unsigned RP = H / 64;
+  const unsigned RP = cdiv<unsigned>(M, 64);
   const unsigned rp = blockIdx.x % RP, ct = blockIdx.x / RP, split = blockIdx.y;
   const unsigned wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const unsigned l32 = lane % 32, lhi = lane / 32;
-  const unsigned G = H / 2, gq = G / (4 * gridDim.y), g0 = (split * 4 + wave) * gq;
+  const unsigned G = K / 8, gq = G / (4 * gridDim.y), g0 = (split * 4 + wave) * gq;
   stepx16 acc0 = {0}, acc1 = {0};
-  const float4* pa = reinterpret_cast<const float4*>(WpT) + (size_t(2 * rp) * G + g0) * 64 + lane;
-  step_product<false>(acc0, acc1, pa, pa + size_t(G) * 64, dpp + ((size_t(ct) * G + g0) * 64 + lane) * 4, gq);
+  const float *pa0, *pa1, *pb;
+  if (PLAIN_A) {
+    const unsigned r0 = rp * 64 + l32, r1 = r0 + 32;
+    pa0 = A + size_t(r0 < M ? r0 : M - 1) * lda + size_t(g0) * 8 + 4 * lhi;
+    pa1 = A + size_t(r1 < M ? r1 : M - 1) * lda + size_t(g0) * 8 + 4 * lhi;
+  } else {
+    pa0 = A + ((size_t(2 * rp) * G + g0) * 64 + lane) * 4;
+    pa1 = pa0 + size_t(G) * 256;
+  }
+  if (PLAIN_B) {
+    const unsigned c0 = ct * 32 + l32;
+    pb = Bm + size_t(c0 < N ? c0 : N - 1) * ldb + size_t(g0) * 8 + 4 * lhi;
+  } else {
+    pb = Bm + ((size_t(ct) * G + g0) * 64 + lane) * 4;
+  }
+  step_product<PLAIN_A, PLAIN_B, 2>(acc0, acc1, pa0, pa1, pb, gq);
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const unsigned row = 8 * (r / 4) + 4 * lhi + (r % 4);
@@ -471,15 +488,26 @@ __global__ __launch_bounds__(256) void lstm_rec_bwd_kernel(unsigned H, unsigned 
     red[(wave * 64 + 32 + row) * kStepPitchR + l32] = acc1[r];
   }
   __syncthreads();
-  float* out = slices + size_t(split) * H * B;
+  float* out = slices + size_t(split) * M * N;
   for (unsigned o = threadIdx.x; o < 64 * 32; o += 256) {
-    const unsigned row = o % 64, col = o / 64, ecol = ct * 32 + col;
-    if (ecol >= B) continue;
+    const unsigned row = o % 64, col = o / 64, erow = rp * 64 + row, ecol = ct * 32 + col;
+    if (erow >= M || ecol >= N) continue;
     float s = red[row * kStepPitchR + col];
 #pragma unroll
     for (int w = 1; w < 4; ++w) s += red[(w * 64 + row) * kStepPitchR + col];
-    out[size_t(ecol) * H + rp * 64 + row] = s;
+    out[size_t(ecol) * M + erow] = s;
   }
+}
+
+// out[e] = beta * out[e] + (slices[0][e] + slices[1][e] + ...), slices added in ascending order
+__global__ __launch_bounds__(256) void slices_accumulate_kernel(size_t total, unsigned splits,
+                                                                const float* __restrict__ slices, float beta,
+                                                                float* __restrict__ out) {
+  const size_t e = size_t(blockIdx.x) * 256 + threadIdx.x;
+  if (e >= total) return;
+  float s = slices[e];
+  for (unsigned k = 1; k < splits; ++k) s += slices[size_t(k) * total + e];
+  out[e] = beta != 0.f ? beta * out[e] + s : s;
 }
 
 static bool all_aligned16(std::initializer_list<const void*> ps) {
@@ -545,6 +573,59 @@ static int prepare_h(dyhip_device* dev, unsigned H, unsigned B, const float* h, 
                      h, mask_h, mask_h_bd > 1 ? 1 : 0, buf, B);
   DYHIP_CHECK_LAUNCH();
   *h_eff = buf;
+  return DYHIP_OK;
+}
+
+// Depth ranges of a skinny transposed product: enough blocks for every CU, whole sets of four groups of 8 k per
+// wave.  0 when the depth does not divide that way (the caller then takes the general GEMM).
+static unsigned skinny_tn_splits(unsigned M, unsigned N, unsigned K) {
+  if (K < 128 || K % 128 != 0) return 0;
+  const unsigned tiles = cdiv<unsigned>(M, 64) * cdiv<unsigned>(N, 32);
+  unsigned s = 1;
+  while (s < 16 && tiles * s < 256 && (K / 8) % (s * 2 * 16) == 0) s *= 2;
+  return s;
+}
+
+// slices[s] = A^T B over depth range s (s < *splits); see skinny_tn_kernel for the operand forms
+static int skinny_tn(dyhip_device* dev, unsigned M, unsigned N, unsigned K, const float* A, size_t lda, bool plain_a,
+                     const float* B, size_t ldb, bool plain_b, float* slices, size_t slices_bytes, unsigned* splits) {
+  const unsigned s = skinny_tn_splits(M, N, K);
+  DYHIP_REQUIRE(s >= 1, "skinny product: depth %u is not a multiple of 128", K);
+  DYHIP_REQUIRE(aligned16(A) && aligned16(B) && lda % 4 == 0 && ldb % 4 == 0, "skinny product: operands must be 16-byte aligned");
+  DYHIP_REQUIRE(slices != nullptr && slices_bytes >= sizeof(float) * size_t(M) * N * s,
+                "skinny product: %u slices of %u x %u floats do not fit %zu bytes", s, M, N, slices_bytes);
+  const dim3 grid(cdiv<unsigned>(M, 64) * cdiv<unsigned>(N, 32), s), block(256);
+#define DYHIP_SKINNY(PA, PB) \
+  hipLaunchKernelGGL((skinny_tn_kernel<PA, PB>), grid, block, 0, dev->stream, M, N, K, A, lda, B, ldb, slices)
+  if (plain_a && plain_b) DYHIP_SKINNY(true, true);
+  else if (plain_a) DYHIP_SKINNY(true, false);
+  else if (plain_b) DYHIP_SKINNY(false, true);
+  else DYHIP_SKINNY(false, false);
+#undef DYHIP_SKINNY
+  DYHIP_CHECK_LAUNCH();
+  *splits = s;
+  return DYHIP_OK;
+}
+
+// C[M x N] = beta * C + A^T B for a small output with a deep sum, A (K x M) and B (K x N) plain with k contiguous:
+// the fragment-order product leaves a few slices in the queue's GEMM workspace and a second launch folds them into
+// C.  *taken = false (nothing launched) when the shape is not one this form is faster on.
+int skinny_tn_gemm(dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B,
+                   size_t ldb, float beta, float* C, bool* taken) {
+  *taken = false;
+  if (M == 0 || N == 0 || M > 4096 || N > 256 || K < 1024 || K > (size_t(1) << 24)) return DYHIP_OK;
+  if (M * N > (size_t(1) << 19) || lda % 4 != 0 || ldb % 4 != 0 || !aligned16(A) || !aligned16(B)) return DYHIP_OK;
+  const unsigned m = unsigned(M), n = unsigned(N), k = unsigned(K);
+  if (skinny_tn_splits(m, n, k) == 0 || dev->gemm_ws == nullptr || dev->gemm_ws_bytes < sizeof(float) * M * N * 16)
+    return DYHIP_OK;
+  unsigned splits = 0;
+  DYHIP_CHECK_STATUS(skinny_tn(dev, m, n, k, A, lda, true, B, ldb, true, static_cast<float*>(dev->gemm_ws),
+                               dev->gemm_ws_bytes, &splits));
+  const size_t total = M * N;
+  hipLaunchKernelGGL(slices_accumulate_kernel, dim3(unsigned(cdiv<size_t>(total, 256))), dim3(256), 0, dev->stream, total,
+                     splits, static_cast<const float*>(dev->gemm_ws), beta, C);
+  DYHIP_CHECK_LAUNCH();
+  *taken = true;
   return DYHIP_OK;
 }
 
@@ -657,6 +738,11 @@ int dyhip_lstm_gates_backward(dyhip_device* dev, unsigned num_inputs, const floa
       off = 0;
     }
     GemmSeg s{W, G, dpre, G, G};
+    if (!gi.dropout) {  // a small output with a 4H-deep sum: the fragment-order product when the shape suits it
+      bool taken = false;
+      DYHIP_CHECK_STATUS(skinny_tn_gemm(dev, rows, B, G, W, G, dpre, G, 1.0f, dEdxi, &taken));
+      if (taken) return DYHIP_OK;
+    }
     if (!gi.dropout) return gemm_run(dev, true, true, rows, B, 1, &s, dEdxi, acc);
     DYHIP_CHECK_STATUS(gemm_run(dev, true, true, rows, B, 1, &s, tmp, ovw));
     hipLaunchKernelGGL(acc_mul_mask_kernel, dim3(cdiv<unsigned>(rows, 256), grid_y(B)), dim3(256), 0, dev->stream, rows,
@@ -932,14 +1018,6 @@ int dyhip_lstm_step_forward_x(dyhip_device* dev, unsigned I, unsigned H, unsigne
                       nullptr);
 }
 
-// depth ranges of the backward product: enough blocks for every CU, whole sets of four groups per wave
-static unsigned rec_bwd_splits(unsigned H, unsigned B) {
-  const unsigned tiles = (H / 64) * cdiv<unsigned>(B, 32);
-  unsigned s = 1;
-  while (s < 8 && tiles * s < 256 && (H / 2) % (s * 2 * 16) == 0) s *= 2;
-  return s;
-}
-
 int dyhip_lstm_recurrent_backward_packed(dyhip_device* dev, unsigned H, unsigned B, const float* packed_WhT,
                                          const float* dpre_packed, void* ws, size_t ws_bytes, unsigned* splits) {
   DYHIP_CHECK_DEV(dev);
@@ -947,15 +1025,7 @@ int dyhip_lstm_recurrent_backward_packed(dyhip_device* dev, unsigned H, unsigned
   dyhip_lstm_step_supported(dev, H, B, &ok);
   DYHIP_REQUIRE(ok, "LSTM step: unsupported hidden (%u) or batch (%u) size", H, B);
   DYHIP_REQUIRE(packed_WhT && dpre_packed && ws && splits, "LSTM step: null pointer");
-  DYHIP_REQUIRE(all_aligned16({packed_WhT, dpre_packed}), "LSTM step: weights and operands must be 16-byte aligned");
-  const unsigned s = rec_bwd_splits(H, B);
-  DYHIP_REQUIRE(ws_bytes >= sizeof(float) * size_t(H) * B * s, "LSTM step: %u slices of %u x %u floats do not fit %zu bytes", s, H,
-                B, ws_bytes);
-  hipLaunchKernelGGL(lstm_rec_bwd_kernel, dim3((H / 64) * cdiv<unsigned>(B, 32), s), dim3(256), 0, dev->stream, H, B,
-                     packed_WhT, dpre_packed, static_cast<float*>(ws));
-  DYHIP_CHECK_LAUNCH();
-  *splits = s;
-  return DYHIP_OK;
+  return skinny_tn(dev, H, B, 4 * H, packed_WhT, 0, false, dpre_packed, 0, false, static_cast<float*>(ws), ws_bytes, splits);
 }
 
 int dyhip_lstm_cell_backward_packed(dyhip_device* dev, unsigned H, unsigned B, const float* gates, const float* c,
