@@ -17,6 +17,9 @@ pytestmark = pytest.mark.gpu
 # ---------------------------------------------------------------------------
 GEMM_SHAPES = [(1024, 32, 128), (1024, 32, 256), (4096, 128, 1280), (256, 128, 4096), (130, 33, 17), (5, 4, 6),
                (64, 1, 64), (1000, 128, 1024), (129, 65, 100),
+               # small outputs with deep sums: the transposed form takes the fragment-order product (ragged edges,
+               # one and several depth ranges)
+               (100, 37, 1152), (64, 1, 2048), (33, 256, 1024), (2048, 200, 2560),
                # more tiles than two per CU with a thin last round: the trailing tile columns run as a GEMM of their own
                (4096, 2304, 40), (4100, 2310, 33)]
 
@@ -39,6 +42,9 @@ def test_gemm_three_forms(dev, M, N, K):
     yt = dev.tensor(y0)
     dev.gemm_tn_acc(M, N, K, dev.tensor(l2), rt, yt)
     assert_close(yt.numpy(), orc.gemm_tn_acc(M, N, K, l2, r, y0.copy()), FWD_RTOL, "gemm_tn", floor=floor)
+    yt = dev.tensor(y0)
+    dev.gemm_tn(M, N, K, dev.tensor(l2), rt, 0.0, yt)  # overwrites
+    assert_close(yt.numpy(), orc.gemm_tn_acc(M, N, K, l2, r, np.zeros_like(y0)), FWD_RTOL, "gemm_tn beta=0", floor=floor)
     # NT: y += l r^T with r stored N x K
     r2 = f32(rng.standard_normal((K, N)))
     yt = dev.tensor(y0)
