@@ -811,7 +811,11 @@ static int recurrent_partials(dyhip_device* dev, bool transposed, unsigned H, un
     GemmSeg s{Wh, G, v, H, H};
     return gemm_run(dev, false, true, G, B, 1, &s, nullptr, ep);
   }
-  GemmSeg s{Wh, G, v, G, G};  // Wh^T * dpre[4H x B]
+  // Wh^T * dpre[4H x B]: a small output with a deep sum, both operands with k contiguous as they lie
+  if (B <= 512 && skinny_tn_splits(H, B, unsigned(G)) >= 1 && aligned16(Wh) && aligned16(v) &&
+      ws_bytes >= sizeof(float) * size_t(H) * B * skinny_tn_splits(H, B, unsigned(G)))
+    return skinny_tn(dev, H, B, unsigned(G), Wh, G, true, v, G, true, static_cast<float*>(ws), ws_bytes, splits);
+  GemmSeg s{Wh, G, v, G, G};
   return gemm_run(dev, true, true, H, B, 1, &s, nullptr, ep);
 }
 
