@@ -309,17 +309,28 @@ __global__ __launch_bounds__(256) void lstm_pack_state_kernel(unsigned K, unsign
 // operand and 8 floats on for a plain one (PLAIN_A / PLAIN_B): a matrix stored with k contiguous per row (or
 // column) needs no packing, its fragment is the 128-bit load of four consecutive k at row l32, offset 4 * lhi
 // (32 segments of 32 bytes per wave and load where the packed form has 1 KiB contiguous).
+// A_MODE 2 is a matrix stored with the ROW index contiguous (leading dimension lda between consecutive k, e.g.
+// DyNet's 4H x K weights as they lie): the four k of a fragment are four 32-bit loads, each one 128-byte run
+// over the 32 rows of the tile; pa then points at row l32 of k = first k + 4 * lhi.
 // TILES = 1 leaves the second row tile out (pa1 and acc1 unused): small problems get twice the blocks.
-template <bool PLAIN_A, bool PLAIN_B, int TILES = 2>
+enum { kFragPacked = 0, kFragAlongK = 1, kFragAlongRows = 2 };
+template <int A_MODE, bool PLAIN_B, int TILES = 2>
 __device__ __forceinline__ void step_product(stepx16& acc0, stepx16& acc1, const float* __restrict__ pa0,
                                              const float* __restrict__ pa1, const float* __restrict__ pb,
-                                             unsigned groups) {
-  constexpr size_t SA = PLAIN_A ? 8 : 256, SB = PLAIN_B ? 8 : 256;
+                                             unsigned groups, size_t lda = 0) {
+  constexpr size_t SA = A_MODE == kFragAlongK ? 8 : 256, SB = PLAIN_B ? 8 : 256;
   float4 a0[4], a1[4], b0[4], c0[4], c1[4], d0[4];
+#define STEP_LOAD_A(dst, p, g_)                                                                      \
+  if (A_MODE == kFragAlongRows) {                                                                    \
+    const float* q_ = p + size_t(g_) * 8 * lda;                                                      \
+    dst = make_float4(q_[0], q_[lda], q_[2 * lda], q_[3 * lda]);                                     \
+  } else {                                                                                           \
+    dst = *reinterpret_cast<const float4*>(p + size_t(g_) * SA);                                     \
+  }
 #define STEP_LOAD(A0, A1, BB, grp)                                                                   \
   _Pragma("unroll") for (int u = 0; u < 4; ++u) {                                                    \
-    A0[u] = *reinterpret_cast<const float4*>(pa0 + size_t((grp) + u) * SA);                          \
-    if (TILES == 2) A1[u] = *reinterpret_cast<const float4*>(pa1 + size_t((grp) + u) * SA);          \
+    STEP_LOAD_A(A0[u], pa0, (grp) + u)                                                               \
+    if (TILES == 2) { STEP_LOAD_A(A1[u], pa1, (grp) + u) }                                           \
     BB[u] = *reinterpret_cast<const float4*>(pb + size_t((grp) + u) * SB);                           \
   }                                                                                                  \
   __builtin_amdgcn_sched_barrier(0);
@@ -351,6 +362,7 @@ __device__ __forceinline__ void step_product(stepx16& acc0, stepx16& acc1, const
     STEP_LOAD(a0, a1, b0, full)
     STEP_MMA(a0, a1, b0)
   }
+#undef STEP_LOAD_A
 #undef STEP_LOAD
 #undef STEP_MMA1
 #undef STEP_MMA
@@ -410,7 +422,7 @@ __global__ __launch_bounds__(256) void lstm_step_fwd_kernel(unsigned H, unsigned
     // plain state: columns past the batch are computed on a clamped address and dropped
     const unsigned pcol = ct * 32 + l32 < B ? ct * 32 + l32 : B - 1;
     const float* pb = PLAIN ? op.vp + size_t(pcol) * op.K + size_t(g0) * 8 + 4 * lhi : op.vp + ((size_t(ct) * G + g0) * 64 + lane) * 4;
-    step_product<false, PLAIN, TILES>(acc0, acc1, pa, pa + size_t(G) * 256, pb, gq);
+    step_product<kFragPacked, PLAIN, TILES>(acc0, acc1, pa, pa + size_t(G) * 256, pb, gq);
   }
 
   // the four quarter sums meet in LDS: rows 0..31 = first tile, 32..63 = second
@@ -480,7 +492,7 @@ __global__ __launch_bounds__(256) void skinny_tn_kernel(unsigned M, unsigned N, 
   } else {
     pb = Bm + ((size_t(ct) * G + g0) * 64 + lane) * 4;
   }
-  step_product<PLAIN_A, PLAIN_B, 2>(acc0, acc1, pa0, pa1, pb, gq);
+  step_product<PLAIN_A ? kFragAlongK : kFragPacked, PLAIN_B, 2>(acc0, acc1, pa0, pa1, pb, gq);
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const unsigned row = 8 * (r / 4) + 4 * lhi + (r % 4);
@@ -496,6 +508,51 @@ __global__ __launch_bounds__(256) void skinny_tn_kernel(unsigned M, unsigned N, 
 #pragma unroll
     for (int w = 1; w < 4; ++w) s += red[(w * 64 + row) * kStepPitchR + col];
     out[size_t(ecol) * M + erow] = s;
+  }
+}
+
+// VanillaLSTMGates forward for a batch that is a few 32-column tiles wide: fx = act(b + [f: +1] + Wx x + Wh h) with
+// the weights as DyNet stores them (4H x K, rows contiguous) and x, h plain (k contiguous per column).  A block owns
+// 64 consecutive gate rows x 32 columns over the full depth of both products (4H / 64 x B / 32 blocks: one per CU at
+// H = 1024, B = 128), its four waves split each depth in quarters and meet in LDS; nothing goes through a workspace.
+struct NnOperand {
+  const float* W;  // M x K, leading dimension M (rows contiguous)
+  const float* v;  // K x N, leading dimension K
+  unsigned K;
+};
+
+__global__ __launch_bounds__(256) void lstm_gates_skinny_kernel(unsigned H, unsigned B, NnOperand op0, NnOperand op1,
+                                                                const float* __restrict__ bias, int mode,
+                                                                float* __restrict__ fx) {
+  __shared__ float red[4 * 64 * kStepPitchR];
+  const unsigned M = 4 * H, RP = M / 64;
+  const unsigned rp = blockIdx.x % RP, ct = blockIdx.x / RP;
+  const unsigned wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const unsigned l32 = lane % 32, lhi = lane / 32;
+  stepx16 acc0 = {0}, acc1 = {0};
+  const unsigned pcol = ct * 32 + l32 < B ? ct * 32 + l32 : B - 1;
+  for (int which = 0; which < 2; ++which) {
+    const NnOperand op = which == 0 ? op0 : op1;
+    const unsigned G = op.K / 8, gq = G / 4, g0 = wave * gq;
+    const float* pa = op.W + size_t(rp) * 64 + l32 + (size_t(g0) * 8 + 4 * lhi) * M;
+    const float* pb = op.v + size_t(pcol) * op.K + size_t(g0) * 8 + 4 * lhi;
+    step_product<kFragAlongRows, true, 2>(acc0, acc1, pa, pa + 32, pb, gq, M);
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const unsigned row = 8 * (r / 4) + 4 * lhi + (r % 4);
+    red[(wave * 64 + row) * kStepPitchR + l32] = acc0[r];
+    red[(wave * 64 + 32 + row) * kStepPitchR + l32] = acc1[r];
+  }
+  __syncthreads();
+  for (unsigned o = threadIdx.x; o < 64 * 32; o += 256) {
+    const unsigned row = o % 64, col = o / 64, erow = rp * 64 + row, ecol = ct * 32 + col;
+    if (ecol >= B) continue;
+    float pre = bias[erow];
+    if (erow >= H && erow < 2 * H) pre += 1.0f;  // forget-gate bias
+#pragma unroll
+    for (int w = 0; w < 4; ++w) pre += red[(w * 64 + row) * kStepPitchR + col];
+    fx[size_t(ecol) * M + erow] = erow < 3 * H ? logistic(mode, pre) : tanh_accurate(pre);
   }
 }
 
@@ -667,6 +724,15 @@ int dyhip_lstm_gates_forward(dyhip_device* dev, unsigned num_inputs, const float
   DYHIP_CHECK_STATUS(prepare_x(dev, num_inputs, xs_host, x_dims_host, gi.I, B, mask_x, mask_x_bd, xbuf, &x_eff));
   DYHIP_CHECK_STATUS(prepare_h(dev, H, B, h_tm1, mask_h, mask_h_bd, hbuf, &h_eff));
   const size_t G = size_t(4) * H;
+  // a batch of a few column tiles: one launch of the fragment-order kernel on the operands as they lie
+  if (B <= 256 && H % 16 == 0 && gi.I % 128 == 0 && H % 128 == 0 && G < (size_t(1) << 31) &&
+      all_aligned16({Wx, Wh, x_eff, h_eff}) && (G / 64) * cdiv<unsigned>(B, 32) >= unsigned(dev->num_cus > 0 ? dev->num_cus : 256) / 2) {
+    const NnOperand op0{Wx, x_eff, gi.I}, op1{Wh, h_eff, H};
+    hipLaunchKernelGGL(lstm_gates_skinny_kernel, dim3(unsigned(G / 64) * cdiv<unsigned>(B, 32)), dim3(256), 0, dev->stream, H,
+                       B, op0, op1, b, logistic_mode, fx);
+    DYHIP_CHECK_LAUNCH();
+    return DYHIP_OK;
+  }
   GemmSeg segs[2] = {{Wx, G, x_eff, gi.I, gi.I}, {Wh, G, h_eff, H, H}};
   GemmEpiParams ep{kEpiLstmGates, 0.f, b, H, logistic_mode};
   return gemm_run(dev, false, true, G, B, 2, segs, fx, ep);
