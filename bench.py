@@ -603,7 +603,7 @@ def lm_kernels(reps, use_graph=True):
               ("dR = dlogits h^T (NT)", "nt", V, H, N), ("dWx1 / dWh = dpre x^T (NT)", "nt", 4 * H, H, N),
               ("dx = Wx^T dpre (TN)", "tn", H, N, 4 * H), ("dWx0 (NT)", "nt", 4 * H, E, N),
               ("recurrent Wh h, one timestep (NN, split-K slices)", "rec_f", 4 * H, B, H),
-              ("recurrent Wh^T dpre, one timestep (TN, split-K slices)", "rec_b", H, B, 4 * H)]
+              ("recurrent Wh^T dpre, one timestep (TN, depth-range slices, plain operands)", "rec_b", H, B, 4 * H)]
     for name, form, M, Nn, K in shapes:
         a, b, y = dev.empty((M * K,)), dev.empty((Nn * K,)), dev.empty((M * Nn,))
         bias = dev.empty((M,))
