@@ -66,6 +66,7 @@ struct dyhip_device {
   size_t stream_threshold;  // tensors at least this large are accessed with streaming (non-temporal) hints
   void* gemm_ws;   // split-K partial tiles (the analogue of a BLAS handle's workspace)
   size_t gemm_ws_bytes;
+  unsigned wide_gemm_ready;  // gemm_wide.hip: kernels whose dynamic-LDS limit has been raised on this device
   hipEvent_t ev_start, ev_stop;
   dyhip_device* parent;                // non-null for a forked queue: pools, scalars and allocator belong to the parent
   std::vector<hipEvent_t> sync_events; // ring of events recorded on this queue for dyhip_device_wait

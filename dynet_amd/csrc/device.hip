@@ -291,6 +291,7 @@ int dyhip_device_create(int ordinal, const size_t pool_mb[4], dyhip_device** out
   dev->alloc = nullptr;
   dev->gemm_ws = nullptr;
   dev->gemm_ws_bytes = 0;
+  dev->wide_gemm_ready = 0;
   dev->ln_scratch = nullptr;
   dev->stream_threshold = size_t(8) << 20;
   hipError_t e = hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking);

@@ -51,6 +51,14 @@ struct GemmBatch {
 int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N, int nseg, const GemmSeg* segs,
              float* C, const GemmEpiParams& epi, const GemmBatch* batch = nullptr);
 
+// gemm_wide.hip: the 256 x 256-tile kernel for large outputs.  gemm_wide_eligible tells whether a one-segment,
+// unbatched product qualifies; gemm_wide_run computes C = beta*C + sum (or bias[i] + sum when bias is set) over the
+// first K32 (a multiple of 32) of the depth.
+bool gemm_wide_eligible(const dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N, size_t K,
+                        const float* A, size_t lda, const float* B, size_t ldb, const float* C);
+int gemm_wide_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N, size_t K32, const float* A,
+                  size_t lda, const float* B, size_t ldb, float* C, float beta, const float* bias);
+
 // lstm.hip: C = beta * C + A^T B by the fragment-order product for small outputs with deep sums (A is K x M, B is
 // K x N, k contiguous); *taken tells whether it ran or the shape should go to gemm_run.
 int skinny_tn_gemm(dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B,

@@ -391,6 +391,23 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
   if (M == 0 || N == 0) return DYHIP_OK;
   DYHIP_REQUIRE(nseg >= 1 && nseg <= kGemmMaxSeg, "GEMM supports 1..%d K segments", kGemmMaxSeg);
   DYHIP_REQUIRE(to_caller || C != nullptr, "null GEMM output");
+  // large outputs: the 256 x 256-tile kernel over the depth's multiple of 32, the rest of the depth added by the
+  // kernel below
+  if (nseg == 1 && (batch == nullptr || batch->count <= 1) && segs[0].A != nullptr && segs[0].B != nullptr &&
+      (epi.kind == kEpiAxpby || (epi.kind == kEpiBias && epi.bias != nullptr && aligned16(epi.bias))) &&
+      gemm_wide_eligible(dev, a_kmajor, b_kmajor, M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, segs[0].ldb, C)) {
+    const GemmSeg& s0 = segs[0];
+    const size_t K32 = s0.K / kBK * kBK;
+    DYHIP_CHECK_STATUS(gemm_wide_run(dev, a_kmajor, b_kmajor, M, N, K32, s0.A, s0.lda, s0.B, s0.ldb, C,
+                                     epi.kind == kEpiAxpby ? epi.beta : 0.f, epi.kind == kEpiBias ? epi.bias : nullptr));
+    if (K32 == s0.K) return DYHIP_OK;
+    GemmSeg tail{s0.A + (a_kmajor ? K32 : K32 * s0.lda), s0.lda, s0.B + (b_kmajor ? K32 : K32 * s0.ldb), s0.ldb,
+                 s0.K - K32};
+    GemmEpiParams acc{};
+    acc.kind = kEpiAxpby;
+    acc.beta = 1.f;
+    return gemm_run(dev, a_kmajor, b_kmajor, M, N, 1, &tail, C, acc, nullptr);
+  }
   GemmArgs g;
   g.nseg = nseg;
   g.M = M;
@@ -537,6 +554,20 @@ int dyhip_gemm_strided_batched(dyhip_device* dev, int trans_l, int trans_r, size
   GemmSeg s{l, trans_l ? K : M, r, trans_r ? N : K, K};
   GemmBatch b{batch, stride_l, stride_r, stride_y};
   return gemm_run(dev, trans_l != 0, trans_r == 0, M, N, 1, &s, y, axpby(beta), &b);
+}
+
+int dyhip_gemm_uses_wide_tiles(dyhip_device* dev, int trans_l, int trans_r, size_t M, size_t N, size_t K,
+                               int* wide_tiles) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(wide_tiles != nullptr, "null output");
+  DYHIP_REQUIRE(!(trans_l && trans_r), "the GEMM has the forms l*r, l^T*r and l*r^T");
+  // any 16-byte aligned address stands for the operands: only alignment is looked at
+  const float* aligned = reinterpret_cast<const float*>(uintptr_t(256));
+  *wide_tiles = gemm_wide_eligible(dev, trans_l != 0, trans_r == 0, M, N, K, aligned, trans_l ? K : M, aligned,
+                                   trans_r ? N : K, aligned)
+                    ? 1
+                    : 0;
+  return DYHIP_OK;
 }
 
 int dyhip_gemm_tn_acc(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float* y) {

@@ -353,6 +353,12 @@ class Device:
                                                _sz(stride_l), _p(r), _sz(stride_r), _f(beta), _p(y), _sz(stride_y),
                                                _u(batch)))
 
+    def gemm_uses_wide_tiles(self, trans_l, trans_r, M, N, K):
+        out = C.c_int(0)
+        _check(cdll.dyhip_gemm_uses_wide_tiles(self.handle, _i(trans_l), _i(trans_r), _sz(M), _sz(N), _sz(K),
+                                               C.byref(out)))
+        return bool(out.value)
+
     def gemm_tn_acc(self, M, N, K, l, r, y):
         _check(cdll.dyhip_gemm_tn_acc(self.handle, _sz(M), _sz(N), _sz(K), _p(l), _p(r), _p(y)))
 

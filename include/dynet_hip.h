@@ -230,6 +230,11 @@ int dyhip_gemm_nn(dyhip_device* dev, size_t M, size_t N, size_t K, const float* 
 int dyhip_gemm_tn_acc(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float* y);
 /* MatrixMultiplyTranspAcc (:162-180): y[MxN] += l[MxK] * r[NxK]^T */
 int dyhip_gemm_nt_acc(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float* y);
+/* Which kernel the three calls above take for a problem with packed leading dimensions and 16-byte aligned
+ * operands: *wide_tiles = 1 for the 256 x 256-tile kernel (large outputs with enough depth per CU), 0 for the
+ * 128-wide kernel or the fragment-order product.  trans_l / trans_r as in dyhip_gemm_strided_batched.  No
+ * counterpart in the reference (cuBLAS picks its kernels silently); for tests and tuning. */
+int dyhip_gemm_uses_wide_tiles(dyhip_device* dev, int trans_l, int trans_r, size_t M, size_t N, size_t K, int* wide_tiles);
 /* The cublasSgemmStridedBatched branches of the three shims (dynet/matrix-multiply.h:27-34, 110-117,
  * 175-182), taken when the left operand is batched: for b in [0, batch)
  *   y_b[MxN] = beta*y_b + op(l_b) * op(r_b),   x_b = x + b*stride_x (strides in floats),

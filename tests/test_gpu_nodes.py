@@ -52,6 +52,43 @@ def test_gemm_three_forms(dev, M, N, K):
     assert_close(yt.numpy(), orc.gemm_nt_acc(M, N, K, l, r2, y0.copy()), FWD_RTOL, "gemm_nt", floor=floor)
 
 
+# Large outputs go to the 256 x 256-tile kernel: (a) fewer tiles than CUs, every tile cut into runs of k-tiles whose
+# partial tiles a second kernel adds, ragged edges and a depth that is not a multiple of 32 (the rest of the depth
+# is added by the 128-wide kernel); (b) one full round of whole tiles plus a remainder dealt in runs; (c) a
+# remainder too large to be worth cutting; (d) a transposed left operand whose row count is not a multiple of 4.
+# Checked against the fp64 product of the same fp32 inputs (the oracle's triple loop is the same sum, too slow here).
+WIDE_GEMM_SHAPES = [(1000, 1000, 8200), (4352, 4096, 512), (7936, 4096, 256), (1001, 1000, 8192), (2048, 2304, 2080)]
+
+
+@pytest.mark.parametrize("M,N,K", WIDE_GEMM_SHAPES)
+def test_gemm_wide_tiles_three_forms(dev, M, N, K):
+    assert dev.gemm_uses_wide_tiles(1, 0, M, N, K) and (M % 4 != 0 or dev.gemm_uses_wide_tiles(0, 0, M, N, K))
+    rng = np.random.default_rng(M + 3 * N + 7 * K)
+    y0 = f32(rng.standard_normal((N, M)))
+    floor = np.sqrt(K)
+    l, r = f32(rng.standard_normal((K, M))), f32(rng.standard_normal((N, K)))  # l: M x K, r: K x N, column-major
+    exact = r.astype(np.float64) @ l.astype(np.float64)                        # (N, M) = column-major M x N
+    lt, rt = dev.tensor(l), dev.tensor(r)
+    if M % 4 == 0:
+        for beta in (1.0, 0.0):
+            yt = dev.tensor(y0)
+            dev.gemm_nn(M, N, K, lt, rt, beta, yt)
+            assert_close(yt.numpy(), beta * y0 + exact, FWD_RTOL, "wide gemm_nn beta=%g" % beta, floor=floor)
+        r2 = f32(r.T)  # N x K column-major = (K, N) row-major
+        yt = dev.tensor(y0)
+        dev.gemm_nt_acc(M, N, K, lt, dev.tensor(r2), yt)
+        assert_close(yt.numpy(), y0 + exact, FWD_RTOL, "wide gemm_nt", floor=floor)
+        bias = f32(rng.standard_normal(M))
+        yt = dev.empty((N, M))
+        dev.affine_forward(M, N, K, dev.tensor(bias), lt, rt, yt)
+        assert_close(yt.numpy(), bias[None, :] + exact, FWD_RTOL, "wide affine", floor=floor)
+    l2 = f32(l.T)  # K x M column-major
+    for beta in (1.0, 0.0):
+        yt = dev.tensor(y0)
+        dev.gemm_tn(M, N, K, dev.tensor(l2), rt, beta, yt)
+        assert_close(yt.numpy(), beta * y0 + exact, FWD_RTOL, "wide gemm_tn beta=%g" % beta, floor=floor)
+
+
 @pytest.mark.parametrize("M,N,K,B", [(64, 48, 32, 5), (130, 70, 33, 3), (7, 5, 3, 17), (256, 128, 256, 4), (31, 1, 9, 2)])
 def test_gemm_strided_batched(dev, M, N, K, B):
     """The batched-left-operand branches of the three GEMM shims: per batch item the plain product, as the
