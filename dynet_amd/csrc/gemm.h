@@ -59,6 +59,13 @@ bool gemm_wide_eligible(const dyhip_device* dev, bool a_kmajor, bool b_kmajor, s
 int gemm_wide_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N, size_t K32, const float* A,
                   size_t lda, const float* B, size_t ldb, float* C, float beta, const float* bias);
 
+// gemm_wide.hip: C[M x N] = beta*C + A[M x K] * B[N x K]^T for a depth of at most 128 (both operands contiguous
+// along the output index): operand tiles fetched whole, one latency per block.
+bool gemm_shallow_nt_eligible(const dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda,
+                              const float* B, size_t ldb, const float* C);
+int gemm_shallow_nt_run(dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B,
+                        size_t ldb, float* C, float beta);
+
 // lstm.hip: C = beta * C + A^T B by the fragment-order product for small outputs with deep sums (A is K x M, B is
 // K x N, k contiguous); *taken tells whether it ran or the shape should go to gemm_run.
 int skinny_tn_gemm(dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B,

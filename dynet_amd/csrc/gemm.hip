@@ -408,6 +408,10 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
     acc.beta = 1.f;
     return gemm_run(dev, a_kmajor, b_kmajor, M, N, 1, &tail, C, acc, nullptr);
   }
+  if (nseg == 1 && (batch == nullptr || batch->count <= 1) && !a_kmajor && !b_kmajor && epi.kind == kEpiAxpby &&
+      segs[0].A != nullptr && segs[0].B != nullptr &&
+      gemm_shallow_nt_eligible(dev, M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, segs[0].ldb, C))
+    return gemm_shallow_nt_run(dev, M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, segs[0].ldb, C, epi.beta);
   GemmArgs g;
   g.nseg = nseg;
   g.M = M;

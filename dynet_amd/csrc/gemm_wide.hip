@@ -320,6 +320,139 @@ __global__ __launch_bounds__(256) void gemm_wide_fixup_kernel(WideArgs g) {
   }
 }
 
+// ---- shallow products: C[M x N] = beta*C + A[M x K] * B[N x K]^T with K <= 128 (the weight gradient of one timestep:
+// K is the batch) -----------------------------------------------------------------------------------------------
+// With four k-tiles a pipelined loop never fills: set-up, the exposed latency of each k-tile and the read-modify-write
+// of C add up to more than the MFMAs.  Here a 512-thread block owns a 128 x 128 tile and fetches BOTH operand tiles
+// whole (2 x 64 KiB, straight into LDS) plus its part of the old C in one burst at the start, so the block pays one
+// memory latency, then 128 MFMAs per wave, then stores.  Wave w (2 x 4 over the tile) owns 64 m x 32 n.
+// LDS: [half h of the depth][wave w][A 4 KiB][B 4 KiB]; the 1 KiB chunk u of wave w in half h holds rows
+// k = 64h + 8w + 2u + {0, 1} of the operand tile (128 floats each), so that each half is one M0 window per wave.
+struct ShallowArgs {
+  const float* A;
+  const float* B;
+  float* C;
+  unsigned lda, ldb;
+  unsigned M, N, K;
+  unsigned tiles_m;
+  float beta;
+};
+
+constexpr size_t kShallowLdsBytes = sizeof(float) * 2 * kStageFloats;
+
+__global__ __launch_bounds__(kWideThreads, 1) void gemm_shallow_nt_kernel(ShallowArgs g) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const unsigned lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const unsigned wm = w & 1, wn = w >> 1, l32 = lane & 31, lhi = lane >> 5;
+  const unsigned tm = blockIdx.x % g.tiles_m, tn = blockIdx.x / g.tiles_m;
+  const unsigned m0 = tm * 128, n0 = tn * 128;
+
+  // old C of this lane's outputs: m = m0 + 64 wm + 2 l32 + {0, 1}, n = n0 + 32 wn + i, i = 8 (r/4) + 4 lhi + r%4
+  const unsigned m = m0 + wm * 64 + 2 * l32;
+  fvec2 cold[16];
+  if (g.beta != 0.f) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const unsigned n = n0 + wn * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+      cold[r] = fvec2{0.f, 0.f};
+      if (m < g.M && n < g.N) cold[r] = *reinterpret_cast<const fvec2*>(g.C + m + size_t(n) * g.M);
+    }
+  }
+  // operand tiles: rows past the depth are not fetched (nor read), groups of four past the edge are clamped
+  unsigned am = m0 + 4 * l32, bn = n0 + 4 * l32;
+  am = am < g.M ? am : g.M - 4;
+  bn = bn < g.N ? bn : g.N - 4;
+#define DYHIP_SHALLOW_LOADS(h)                                                                                     \
+  {                                                                                                                \
+    float* window = lds + (h) * kStageFloats + w * 2048 + 1024;                                                    \
+    const unsigned k0 = 64 * (h) + 8 * w + lhi;                                                                    \
+    const float* pa = g.A + am + size_t(k0) * g.lda;                                                               \
+    const float* pb = g.B + bn + size_t(k0) * g.ldb;                                                               \
+    if (64 * (h) + 8 * w + 0 < g.K) {                                                                              \
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(pa + 1024), (lds_ptr_t)window, 16, -4096, 0);                \
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(pb), (lds_ptr_t)window, 16, 0, 0);                           \
+    }                                                                                                              \
+    if (64 * (h) + 8 * w + 2 < g.K) {                                                                              \
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(pa + 2 * size_t(g.lda) + 768), (lds_ptr_t)window, 16, -3072, 0); \
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(pb + 2 * size_t(g.ldb) - 256), (lds_ptr_t)window, 16, 1024, 0);  \
+    }                                                                                                              \
+    if (64 * (h) + 8 * w + 4 < g.K) {                                                                              \
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(pa + 4 * size_t(g.lda) + 512), (lds_ptr_t)window, 16, -2048, 0); \
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(pb + 4 * size_t(g.ldb) - 512), (lds_ptr_t)window, 16, 2048, 0);  \
+    }                                                                                                              \
+    if (64 * (h) + 8 * w + 6 < g.K) {                                                                              \
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(pa + 6 * size_t(g.lda) + 256), (lds_ptr_t)window, 16, -1024, 0); \
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(pb + 6 * size_t(g.ldb) - 768), (lds_ptr_t)window, 16, 3072, 0);  \
+    }                                                                                                              \
+  }
+  DYHIP_SHALLOW_LOADS(0)
+  DYHIP_SHALLOW_LOADS(1)
+#undef DYHIP_SHALLOW_LOADS
+
+  floatx16 acc[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+  // group kg (8 k) of half h: step s of lane half lhi is row k = 8 kg + 4 lhi + s, i.e. chunk 2 lhi + s/2 of wave kg%8
+  const float* la = lds + lhi * 512 + wm * 64 + 2 * l32;
+  const float* lb = lds + 1024 + lhi * 512 + wn * 32 + l32;
+  const unsigned groups = g.K / 8;
+  fvec2 a[2][4];
+  float b[2][4];
+#define DYHIP_SHALLOW_READ(buf, kg)                                                        \
+  _Pragma("unroll") for (int s = 0; s < 4; ++s) {                                          \
+    const unsigned o = ((kg) / 8) * kStageFloats + ((kg) % 8) * 2048 + (s / 2) * 256 + (s % 2) * 128; \
+    a[buf][s] = *reinterpret_cast<const fvec2*>(la + o);                                   \
+    b[buf][s] = lb[o];                                                                     \
+  }
+#define DYHIP_SHALLOW_MMA(buf)                                                                          \
+  __builtin_amdgcn_sched_barrier(0);                                                                    \
+  _Pragma("unroll") for (int s = 0; s < 4; ++s) {                                                       \
+    acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(b[buf][s], a[buf][s][0], acc[0], 0, 0, 0);            \
+    acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(b[buf][s], a[buf][s][1], acc[1], 0, 0, 0);            \
+  }                                                                                                     \
+  __builtin_amdgcn_sched_barrier(0);
+  // the first half of the depth can start while the second is still on its way (only when the whole second half
+  // was asked for, so that every wave has the same number of loads in flight)
+  const bool two_phase = g.K == 128;
+  if (two_phase) __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): the eight loads of the second half may be in flight
+  else __builtin_amdgcn_s_waitcnt(0x0F70);
+  __syncthreads();
+  const unsigned first = two_phase ? 8 : groups;
+  DYHIP_SHALLOW_READ(0, 0u)
+  for (unsigned kg = 0; kg < first; kg += 2) {
+    const unsigned k1 = kg + 1 < first ? kg + 1 : kg, k2 = kg + 2 < first ? kg + 2 : kg;
+    DYHIP_SHALLOW_READ(1, k1)
+    DYHIP_SHALLOW_MMA(0)
+    DYHIP_SHALLOW_READ(0, k2)
+    if (kg + 1 < first) { DYHIP_SHALLOW_MMA(1) }
+  }
+  if (two_phase) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    DYHIP_SHALLOW_READ(0, 8u)
+    for (unsigned kg = 8; kg < 16; kg += 2) {
+      const unsigned k2 = kg + 2 < 16 ? kg + 2 : kg;
+      DYHIP_SHALLOW_READ(1, kg + 1)
+      DYHIP_SHALLOW_MMA(0)
+      DYHIP_SHALLOW_READ(0, k2)
+      DYHIP_SHALLOW_MMA(1)
+    }
+  }
+#undef DYHIP_SHALLOW_READ
+#undef DYHIP_SHALLOW_MMA
+  if (m >= g.M) return;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const unsigned n = n0 + wn * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+    if (n >= g.N) continue;
+    fvec2 v = fvec2{acc[0][r], acc[1][r]};
+    if (g.beta != 0.f) v += g.beta * cold[r];
+    *reinterpret_cast<fvec2*>(g.C + m + size_t(n) * g.M) = v;
+  }
+}
+
 template <bool AK, bool BKM>
 int launch_wide(dyhip_device* dev, const WideArgs& g, unsigned blocks, unsigned bit) {
   const void* fn = reinterpret_cast<const void*>(&gemm_wide_kernel<AK, BKM>);
@@ -414,6 +547,40 @@ int gemm_wide_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, siz
     hipLaunchKernelGGL(gemm_wide_fixup_kernel, dim3(p.rem, kWT / 16), dim3(256), 0, dev->stream, g);
     DYHIP_CHECK_LAUNCH();
   }
+  return DYHIP_OK;
+}
+
+bool gemm_shallow_nt_eligible(const dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda,
+                              const float* B, size_t ldb, const float* C) {
+  if (K < 32 || K > 128 || K % 8 != 0 || M % 4 != 0 || N % 4 != 0 || M < 128 || N < 128) return false;
+  if (!aligned16(A) || !aligned16(B) || lda % 4 != 0 || ldb % 4 != 0 || (reinterpret_cast<uintptr_t>(C) & 7u) != 0)
+    return false;
+  if (K * lda >= (size_t(1) << 31) || K * ldb >= (size_t(1) << 31) || M * N >= (size_t(1) << 31)) return false;
+  const size_t cus = dev->num_cus > 0 ? size_t(dev->num_cus) : 256;
+  return cdiv<size_t>(M, 128) * cdiv<size_t>(N, 128) * 2 >= cus;  // fewer tiles: the 128-wide kernel cuts the depth
+}
+
+int gemm_shallow_nt_run(dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B,
+                        size_t ldb, float* C, float beta) {
+  ShallowArgs g;
+  g.A = A;
+  g.B = B;
+  g.C = C;
+  g.lda = unsigned(lda);
+  g.ldb = unsigned(ldb);
+  g.M = unsigned(M);
+  g.N = unsigned(N);
+  g.K = unsigned(K);
+  g.tiles_m = unsigned(cdiv<size_t>(M, 128));
+  g.beta = beta;
+  if ((dev->wide_gemm_ready & (1u << 4)) == 0) {
+    DYHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_shallow_nt_kernel),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, int(kShallowLdsBytes)));
+    dev->wide_gemm_ready |= 1u << 4;
+  }
+  const unsigned blocks = g.tiles_m * unsigned(cdiv<size_t>(N, 128));
+  hipLaunchKernelGGL(gemm_shallow_nt_kernel, dim3(blocks), dim3(kWideThreads), kShallowLdsBytes, dev->stream, g);
+  DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
 

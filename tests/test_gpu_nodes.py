@@ -52,6 +52,27 @@ def test_gemm_three_forms(dev, M, N, K):
     assert_close(yt.numpy(), orc.gemm_nt_acc(M, N, K, l, r2, y0.copy()), FWD_RTOL, "gemm_nt", floor=floor)
 
 
+# Shallow products l * r^T (the weight gradient of one timestep, depth = batch <= 128) fetch both operand tiles whole:
+# full depth (two halves), half depth, a depth with an odd number of groups of 8, ragged edges.
+@pytest.mark.parametrize("M,N,K", [(4096, 1024, 128), (2052, 1028, 96), (4096, 512, 40), (1024, 4096, 64), (2048, 2048, 32)])
+def test_gemm_nt_shallow(dev, M, N, K):
+    rng = np.random.default_rng(M + N + K)
+    y0 = f32(rng.standard_normal((N, M)))
+    l, r2 = f32(rng.standard_normal((K, M))), f32(rng.standard_normal((K, N)))
+    lt, rt = dev.tensor(l), dev.tensor(r2)
+    yt = dev.tensor(y0)
+    dev.gemm_nt_acc(M, N, K, lt, rt, yt)
+    assert_close(yt.numpy(), orc.gemm_nt_acc(M, N, K, l, r2, y0.copy()), FWD_RTOL, "shallow gemm_nt_acc", floor=np.sqrt(K))
+    yt = dev.tensor(y0)
+    dev.gemm_nt(M, N, K, lt, rt, 0.0, yt)
+    assert_close(yt.numpy(), orc.gemm_nt_acc(M, N, K, l, r2, np.zeros_like(y0)), FWD_RTOL, "shallow gemm_nt beta=0",
+                 floor=np.sqrt(K))
+    yt = dev.tensor(y0)
+    dev.gemm_nt(M, N, K, lt, rt, 0.5, yt)
+    assert_close(yt.numpy(), orc.gemm_nt_acc(M, N, K, l, r2, f32(0.5 * y0)), FWD_RTOL, "shallow gemm_nt beta=0.5",
+                 floor=np.sqrt(K))
+
+
 # Large outputs go to the 256 x 256-tile kernel: (a) fewer tiles than CUs, every tile cut into runs of k-tiles whose
 # partial tiles a second kernel adds, ragged edges and a depth that is not a multiple of 32 (the rest of the depth
 # is added by the 128-wide kernel); (b) one full round of whole tiles plus a remainder dealt in runs; (c) a
