@@ -602,13 +602,15 @@ def lm_kernels(reps, use_graph=True):
               ("output projection (NN, bias epilogue)", "affine", V, N, H), ("d h_top = R^T dlogits (TN)", "tn", H, N, V),
               ("dR = dlogits h^T (NT)", "nt", V, H, N), ("dWx1 / dWh = dpre x^T (NT)", "nt", 4 * H, H, N),
               ("dx = Wx^T dpre (TN)", "tn", H, N, 4 * H), ("dWx0 (NT)", "nt", 4 * H, E, N),
+              ("dWh of one timestep = dpre h^T (NT, depth = batch; node-at-a-time path)", "nt", 4 * H, H, B),
               ("recurrent Wh h, one timestep (NN, split-K slices)", "rec_f", 4 * H, B, H),
               ("recurrent Wh^T dpre, one timestep (TN, depth-range slices, plain operands)", "rec_b", H, B, 4 * H)]
     for name, form, M, Nn, K in shapes:
         a, b, y = dev.empty((M * K,)), dev.empty((Nn * K,)), dev.empty((M * Nn,))
         bias = dev.empty((M,))
+        # random operands: constant fills switch few bits in the matrix cores, and the clock under them is ~10 % higher
         for t in (a, b, bias):
-            dev.constant(t, 0.01)
+            dev.randomize_normal(t, 0.0, 0.1)
         fb, bb = dev.lstm_cell_workspace(H, B)
         ws, _ = dev.workspace(max(fb, bb))
         fn = {"nn": lambda: dev.gemm_nn(M, Nn, K, a, b, 0.0, y), "tn": lambda: dev.gemm_tn(M, Nn, K, a, b, 0.0, y),
