@@ -392,25 +392,18 @@ __global__ __launch_bounds__(256) void lstm_step_fwd_kernel(unsigned H, unsigned
   const unsigned l32 = lane % 32, lhi = lane / 32;
 
   // The epilogue's thread owns hidden unit eu (of UB) of batch columns ecc + CSTEP*i; its operands are fetched
-  // now so that their latency hides behind the product (it matters for small problems, which are one chain of
-  // latencies; at H = 1024, B = 128 fetching them after the product measures the same).
+  // now so that their latency hides behind the product, and kept as loaded: any arithmetic on them here would
+  // make the wave wait for them before its first MFMA (1.3 us at H = 1024, B = 128).
   const unsigned eu = threadIdx.x % UB, ecc = threadIdx.x / UB, ej = rp * UB + eu;
-  float pre[TILES][4], cp[TILES];
+  float bq[4], xq[TILES][4], cp[TILES];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) bq[q] = bias[q * H + ej];
 #pragma unroll
   for (int i = 0; i < TILES; ++i) {
-    const unsigned ecol = ct * 32 + ecc + CSTEP * i;
-    cp[i] = 0.f;
+    const unsigned ecol = ct * 32 + ecc + CSTEP * i, lcol = ecol < B ? ecol : B - 1;  // past the batch: clamped, dropped
 #pragma unroll
-    for (int q = 0; q < 4; ++q) pre[i][q] = 0.f;
-    if (ecol < B) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const float bq = bias[q * H + ej];
-        pre[i][q] = q == 1 ? bq + 1.0f : bq;
-        if (xproj != nullptr) pre[i][q] += xproj[size_t(ecol) * 4 * H + ej + size_t(q) * H];
-      }
-      if (c_prev != nullptr) cp[i] = c_prev[size_t(ecol) * H + ej];
-    }
+    for (int q = 0; q < 4; ++q) xq[i][q] = xproj != nullptr ? xproj[size_t(lcol) * 4 * H + ej + size_t(q) * H] : 0.f;
+    cp[i] = c_prev != nullptr ? c_prev[size_t(lcol) * H + ej] : 0.f;
   }
 
   stepx16 acc0 = {0}, acc1 = {0};
@@ -439,13 +432,15 @@ __global__ __launch_bounds__(256) void lstm_step_fwd_kernel(unsigned H, unsigned
   for (int i = 0; i < TILES; ++i) {
     const unsigned col = ecc + CSTEP * i, ecol = ct * 32 + col;
     if (ecol >= B) continue;
+    float pre[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
+      pre[q] = (q == 1 ? bq[q] + 1.0f : bq[q]) + xq[i][q];
 #pragma unroll
-      for (int w = 0; w < 4; ++w) pre[i][q] += red[(w * ROWS + tile * 32 + q * 8 + u) * kStepPitchR + col];
+      for (int w = 0; w < 4; ++w) pre[q] += red[(w * ROWS + tile * 32 + q * 8 + u) * kStepPitchR + col];
     }
-    const float gi = logistic(mode, pre[i][0]), gf = logistic(mode, pre[i][1]), go = logistic(mode, pre[i][2]);
-    const float gg = tanh_accurate(pre[i][3]);
+    const float gi = logistic(mode, pre[0]), gf = logistic(mode, pre[1]), go = logistic(mode, pre[2]);
+    const float gg = tanh_accurate(pre[3]);
     const float cv = c_prev != nullptr ? gi * gg + gf * cp[i] : gi * gg;
     const float hv = go * tanh_accurate(cv);
     const size_t g0 = size_t(ecol) * 4 * H + ej, s0 = size_t(ecol) * H + ej;
@@ -531,6 +526,8 @@ __global__ __launch_bounds__(256) void lstm_gates_skinny_kernel(unsigned H, unsi
   const unsigned l32 = lane % 32, lhi = lane / 32;
   stepx16 acc0 = {0}, acc1 = {0};
   const unsigned pcol = ct * 32 + l32 < B ? ct * 32 + l32 : B - 1;
+  // every output of this thread lies in gate row rp*64 + threadIdx.x % 64: its bias is fetched under the product
+  const float bias_row = bias[rp * 64 + threadIdx.x % 64];
   for (int which = 0; which < 2; ++which) {
     const NnOperand op = which == 0 ? op0 : op1;
     const unsigned G = op.K / 8, gq = G / 4, g0 = wave * gq;
@@ -548,7 +545,7 @@ __global__ __launch_bounds__(256) void lstm_gates_skinny_kernel(unsigned H, unsi
   for (unsigned o = threadIdx.x; o < 64 * 32; o += 256) {
     const unsigned row = o % 64, col = o / 64, erow = rp * 64 + row, ecol = ct * 32 + col;
     if (ecol >= B) continue;
-    float pre = bias[erow];
+    float pre = bias_row;
     if (erow >= H && erow < 2 * H) pre += 1.0f;  // forget-gate bias
 #pragma unroll
     for (int w = 0; w < 4; ++w) pre += red[(w * 64 + row) * kStepPitchR + col];
