@@ -376,83 +376,81 @@ struct StepOperand {
   unsigned K;
 };
 
+// Waves 0..3 form the product.  The cell update has one thread per (hidden unit, column) of the block, 32 * UB of
+// them: with 64-row tiles that is eight waves, and the four that take no part in the product wait at the barrier
+// (one wavefront per SIMD issues dependent VALU work at a fraction of the rate two can).
 template <bool PLAIN, int TILES>
-__global__ __launch_bounds__(256) void lstm_step_fwd_kernel(unsigned H, unsigned B, StepOperand op0, StepOperand op1,
-                                                            const float* xproj, const float* __restrict__ bias,
-                                                            const float* __restrict__ c_prev, int mode, float* gates,
-                                                            float* __restrict__ c, float* __restrict__ h,
-                                                            float* __restrict__ hp) {
+__global__ __launch_bounds__(256 * TILES) void lstm_step_fwd_kernel(unsigned H, unsigned B, StepOperand op0,
+                                                                    StepOperand op1, const float* xproj,
+                                                                    const float* __restrict__ bias,
+                                                                    const float* __restrict__ c_prev, int mode,
+                                                                    float* gates, float* __restrict__ c,
+                                                                    float* __restrict__ h, float* __restrict__ hp) {
   constexpr int UB = 8 * TILES;       // hidden units of a block (its 32*TILES weight rows are their four gate rows)
   constexpr int ROWS = 32 * TILES;
-  constexpr int CSTEP = 256 / UB;     // columns an epilogue thread strides by
   __shared__ float red[4 * ROWS * kStepPitchR];
   const unsigned RP = H / UB;
   const unsigned rp = blockIdx.x % RP, ct = blockIdx.x / RP;
   const unsigned wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const unsigned l32 = lane % 32, lhi = lane / 32;
 
-  // The epilogue's thread owns hidden unit eu (of UB) of batch columns ecc + CSTEP*i; its operands are fetched
-  // now so that their latency hides behind the product, and kept as loaded: any arithmetic on them here would
-  // make the wave wait for them before its first MFMA (1.3 us at H = 1024, B = 128).
-  const unsigned eu = threadIdx.x % UB, ecc = threadIdx.x / UB, ej = rp * UB + eu;
-  float bq[4], xq[TILES][4], cp[TILES];
+  // The epilogue's thread owns hidden unit eu (of UB) of batch column col; its operands are fetched now so that
+  // their latency hides behind the product, and kept as loaded: any arithmetic on them here would make the wave
+  // wait for them before its first MFMA (1.3 us at H = 1024, B = 128).
+  const unsigned eu = threadIdx.x % UB, col = threadIdx.x / UB, ej = rp * UB + eu;
+  const unsigned ecol = ct * 32 + col, lcol = ecol < B ? ecol : B - 1;  // past the batch: clamped, dropped
+  float bq[4], xq[4];
 #pragma unroll
-  for (int q = 0; q < 4; ++q) bq[q] = bias[q * H + ej];
-#pragma unroll
-  for (int i = 0; i < TILES; ++i) {
-    const unsigned ecol = ct * 32 + ecc + CSTEP * i, lcol = ecol < B ? ecol : B - 1;  // past the batch: clamped, dropped
-#pragma unroll
-    for (int q = 0; q < 4; ++q) xq[i][q] = xproj != nullptr ? xproj[size_t(lcol) * 4 * H + ej + size_t(q) * H] : 0.f;
-    cp[i] = c_prev != nullptr ? c_prev[size_t(lcol) * H + ej] : 0.f;
+  for (int q = 0; q < 4; ++q) {
+    bq[q] = bias[q * H + ej];
+    xq[q] = xproj != nullptr ? xproj[size_t(lcol) * 4 * H + ej + size_t(q) * H] : 0.f;
   }
+  const float cp = c_prev != nullptr ? c_prev[size_t(lcol) * H + ej] : 0.f;
 
-  stepx16 acc0 = {0}, acc1 = {0};
-  for (int which = 0; which < 2; ++which) {
-    const StepOperand op = which == 0 ? op0 : op1;
-    if (op.Wp == nullptr) continue;  // uniform over the grid
-    const unsigned G = op.K / 8, gq = G / 4, g0 = wave * gq;
-    const float* pa = op.Wp + ((size_t(TILES * rp) * G + g0) * 64 + lane) * 4;
-    // plain state: columns past the batch are computed on a clamped address and dropped
-    const unsigned pcol = ct * 32 + l32 < B ? ct * 32 + l32 : B - 1;
-    const float* pb = PLAIN ? op.vp + size_t(pcol) * op.K + size_t(g0) * 8 + 4 * lhi : op.vp + ((size_t(ct) * G + g0) * 64 + lane) * 4;
-    step_product<kFragPacked, PLAIN, TILES>(acc0, acc1, pa, pa + size_t(G) * 256, pb, gq);
-  }
-
-  // the four quarter sums meet in LDS: rows 0..31 = first tile, 32..63 = second
+  if (wave < 4) {
+    stepx16 acc0 = {0}, acc1 = {0};
+    for (int which = 0; which < 2; ++which) {
+      const StepOperand op = which == 0 ? op0 : op1;
+      if (op.Wp == nullptr) continue;  // uniform over the grid
+      const unsigned G = op.K / 8, gq = G / 4, g0 = wave * gq;
+      const float* pa = op.Wp + ((size_t(TILES * rp) * G + g0) * 64 + lane) * 4;
+      // plain state: columns past the batch are computed on a clamped address and dropped
+      const unsigned pcol = ct * 32 + l32 < B ? ct * 32 + l32 : B - 1;
+      const float* pb = PLAIN ? op.vp + size_t(pcol) * op.K + size_t(g0) * 8 + 4 * lhi : op.vp + ((size_t(ct) * G + g0) * 64 + lane) * 4;
+      step_product<kFragPacked, PLAIN, TILES>(acc0, acc1, pa, pa + size_t(G) * 256, pb, gq);
+    }
+    // the four quarter sums meet in LDS: rows 0..31 = first tile, 32..63 = second
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const unsigned row = 8 * (r / 4) + 4 * lhi + (r % 4);
-    red[(wave * ROWS + row) * kStepPitchR + l32] = acc0[r];
-    if (TILES == 2) red[(wave * ROWS + 32 + row) * kStepPitchR + l32] = acc1[r];
+    for (int r = 0; r < 16; ++r) {
+      const unsigned row = 8 * (r / 4) + 4 * lhi + (r % 4);
+      red[(wave * ROWS + row) * kStepPitchR + l32] = acc0[r];
+      if (TILES == 2) red[(wave * ROWS + 32 + row) * kStepPitchR + l32] = acc1[r];
+    }
   }
   __syncthreads();
+  if (ecol >= B) return;
 
   const unsigned tile = eu / 8, u = eu % 8;
+  float pre[4];
 #pragma unroll
-  for (int i = 0; i < TILES; ++i) {
-    const unsigned col = ecc + CSTEP * i, ecol = ct * 32 + col;
-    if (ecol >= B) continue;
-    float pre[4];
+  for (int q = 0; q < 4; ++q) {
+    pre[q] = (q == 1 ? bq[q] + 1.0f : bq[q]) + xq[q];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      pre[q] = (q == 1 ? bq[q] + 1.0f : bq[q]) + xq[i][q];
-#pragma unroll
-      for (int w = 0; w < 4; ++w) pre[q] += red[(w * ROWS + tile * 32 + q * 8 + u) * kStepPitchR + col];
-    }
-    const float gi = logistic(mode, pre[0]), gf = logistic(mode, pre[1]), go = logistic(mode, pre[2]);
-    const float gg = tanh_accurate(pre[3]);
-    const float cv = c_prev != nullptr ? gi * gg + gf * cp[i] : gi * gg;
-    const float hv = go * tanh_accurate(cv);
-    const size_t g0 = size_t(ecol) * 4 * H + ej, s0 = size_t(ecol) * H + ej;
-    gates[g0] = gi;
-    gates[g0 + H] = gf;
-    gates[g0 + 2 * size_t(H)] = go;
-    gates[g0 + 3 * size_t(H)] = gg;
-    c[s0] = cv;
-    h[s0] = hv;
-    // h again, as the next timestep's packed operand: unit ej is k = 8*(TILES*rp + tile) + u
-    if (hp != nullptr) hp[((size_t(ct) * (H / 8) + TILES * rp + tile) * 64 + (u / 4) * 32 + col) * 4 + u % 4] = hv;
+    for (int w = 0; w < 4; ++w) pre[q] += red[(w * ROWS + tile * 32 + q * 8 + u) * kStepPitchR + col];
   }
+  const float gi = logistic(mode, pre[0]), gf = logistic(mode, pre[1]), go = logistic(mode, pre[2]);
+  const float gg = tanh_accurate(pre[3]);
+  const float cv = c_prev != nullptr ? gi * gg + gf * cp : gi * gg;
+  const float hv = go * tanh_accurate(cv);
+  const size_t g0 = size_t(ecol) * 4 * H + ej, s0 = size_t(ecol) * H + ej;
+  gates[g0] = gi;
+  gates[g0 + H] = gf;
+  gates[g0 + 2 * size_t(H)] = go;
+  gates[g0 + 3 * size_t(H)] = gg;
+  c[s0] = cv;
+  h[s0] = hv;
+  // h again, as the next timestep's packed operand: unit ej is k = 8*(TILES*rp + tile) + u
+  if (hp != nullptr) hp[((size_t(ct) * (H / 8) + TILES * rp + tile) * 64 + (u / 4) * 32 + col) * 4 + u % 4] = hv;
 }
 
 // Skinny transposed product: slice[split] = A^T[M rows, depth range] x B[depth range, N columns] for M x N small
@@ -1040,7 +1038,7 @@ static int step_forward(dyhip_device* dev, unsigned I, unsigned H, unsigned B, c
   // 64-row tiles (fewest operand bytes per CU) once they give half the CUs a block, 32-row tiles below that
   const unsigned blocks2 = (H / 16) * cdiv<unsigned>(B, 32);
   const bool two = blocks2 * 2 >= unsigned(dev->num_cus > 0 ? dev->num_cus : 256);
-  const dim3 grid(two ? blocks2 : blocks2 * 2), block(256);
+  const dim3 grid(two ? blocks2 : blocks2 * 2), block(two ? 512 : 256);
 #define DYHIP_STEP(PLAIN, TILES)                                                                                     \
   hipLaunchKernelGGL((lstm_step_fwd_kernel<PLAIN, TILES>), grid, block, 0, dev->stream, H, B, op0, op1, xproj, b, c_tm1, \
                      logistic_mode, gates, c, h, hp_out)
