@@ -56,6 +56,10 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
 // first K32 (a multiple of 32) of the depth.
 bool gemm_wide_eligible(const dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N, size_t K,
                         const float* A, size_t lda, const float* B, size_t ldb, const float* C);
+// For a product that does not qualify as a whole: the number of leading columns that form full rounds of one tile per
+// CU and qualify on their own (0 if none); the caller hands the remaining columns to whatever kernel suits them.
+size_t gemm_wide_whole_rounds_columns(const dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N, size_t K,
+                                      const float* A, size_t lda, const float* B, size_t ldb, const float* C);
 int gemm_wide_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N, size_t K32, const float* A,
                   size_t lda, const float* B, size_t ldb, float* C, float beta, const float* bias);
 

@@ -392,21 +392,32 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
   DYHIP_REQUIRE(nseg >= 1 && nseg <= kGemmMaxSeg, "GEMM supports 1..%d K segments", kGemmMaxSeg);
   DYHIP_REQUIRE(to_caller || C != nullptr, "null GEMM output");
   // large outputs: the 256 x 256-tile kernel over the depth's multiple of 32, the rest of the depth added by the
-  // kernel below
+  // kernel below; when only the leading columns form full rounds of tiles, those columns, and the rest as a product
+  // of its own
   if (nseg == 1 && (batch == nullptr || batch->count <= 1) && segs[0].A != nullptr && segs[0].B != nullptr &&
-      (epi.kind == kEpiAxpby || (epi.kind == kEpiBias && epi.bias != nullptr && aligned16(epi.bias))) &&
-      gemm_wide_eligible(dev, a_kmajor, b_kmajor, M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, segs[0].ldb, C)) {
+      (epi.kind == kEpiAxpby || (epi.kind == kEpiBias && epi.bias != nullptr && aligned16(epi.bias)))) {
     const GemmSeg& s0 = segs[0];
-    const size_t K32 = s0.K / kBK * kBK;
-    DYHIP_CHECK_STATUS(gemm_wide_run(dev, a_kmajor, b_kmajor, M, N, K32, s0.A, s0.lda, s0.B, s0.ldb, C,
-                                     epi.kind == kEpiAxpby ? epi.beta : 0.f, epi.kind == kEpiBias ? epi.bias : nullptr));
-    if (K32 == s0.K) return DYHIP_OK;
-    GemmSeg tail{s0.A + (a_kmajor ? K32 : K32 * s0.lda), s0.lda, s0.B + (b_kmajor ? K32 : K32 * s0.ldb), s0.ldb,
-                 s0.K - K32};
-    GemmEpiParams acc{};
-    acc.kind = kEpiAxpby;
-    acc.beta = 1.f;
-    return gemm_run(dev, a_kmajor, b_kmajor, M, N, 1, &tail, C, acc, nullptr);
+    // leading full rounds first: the 128-wide kernel finishes a few remaining tile columns (96 of its tiles) sooner
+    // than runs of k-tiles with their partial tiles do (4096x4480x512: 184 against 204 us)
+    size_t cols = gemm_wide_whole_rounds_columns(dev, a_kmajor, b_kmajor, M, N, s0.K, s0.A, s0.lda, s0.B, s0.ldb, C);
+    if (cols == 0 && gemm_wide_eligible(dev, a_kmajor, b_kmajor, M, N, s0.K, s0.A, s0.lda, s0.B, s0.ldb, C)) cols = N;
+    if (cols > 0) {
+      const size_t K32 = s0.K / kBK * kBK;
+      DYHIP_CHECK_STATUS(gemm_wide_run(dev, a_kmajor, b_kmajor, M, cols, K32, s0.A, s0.lda, s0.B, s0.ldb, C,
+                                       epi.kind == kEpiAxpby ? epi.beta : 0.f,
+                                       epi.kind == kEpiBias ? epi.bias : nullptr));
+      if (K32 < s0.K) {
+        GemmSeg tail{s0.A + (a_kmajor ? K32 : K32 * s0.lda), s0.lda, s0.B + (b_kmajor ? K32 : K32 * s0.ldb), s0.ldb,
+                     s0.K - K32};
+        GemmEpiParams acc{};
+        acc.kind = kEpiAxpby;
+        acc.beta = 1.f;
+        DYHIP_CHECK_STATUS(gemm_run(dev, a_kmajor, b_kmajor, M, cols, 1, &tail, C, acc, nullptr));
+      }
+      if (cols == N) return DYHIP_OK;
+      GemmSeg rest{s0.A, s0.lda, s0.B + (b_kmajor ? cols * s0.ldb : cols), s0.ldb, s0.K};
+      return gemm_run(dev, a_kmajor, b_kmajor, M, N - cols, 1, &rest, C + cols * M, epi, nullptr);
+    }
   }
   if (nseg == 1 && (batch == nullptr || batch->count <= 1) && !a_kmajor && !b_kmajor && epi.kind == kEpiAxpby &&
       segs[0].A != nullptr && segs[0].B != nullptr &&
@@ -567,10 +578,11 @@ int dyhip_gemm_uses_wide_tiles(dyhip_device* dev, int trans_l, int trans_r, size
   DYHIP_REQUIRE(!(trans_l && trans_r), "the GEMM has the forms l*r, l^T*r and l*r^T");
   // any 16-byte aligned address stands for the operands: only alignment is looked at
   const float* aligned = reinterpret_cast<const float*>(uintptr_t(256));
-  *wide_tiles = gemm_wide_eligible(dev, trans_l != 0, trans_r == 0, M, N, K, aligned, trans_l ? K : M, aligned,
-                                   trans_r ? N : K, aligned)
-                    ? 1
-                    : 0;
+  const size_t lda = trans_l ? K : M, ldb = trans_r ? N : K;
+  if (gemm_wide_whole_rounds_columns(dev, trans_l != 0, trans_r == 0, M, N, K, aligned, lda, aligned, ldb, aligned) > 0)
+    *wide_tiles = 2;
+  else if (gemm_wide_eligible(dev, trans_l != 0, trans_r == 0, M, N, K, aligned, lda, aligned, ldb, aligned)) *wide_tiles = 1;
+  else *wide_tiles = 0;
   return DYHIP_OK;
 }
 

@@ -493,9 +493,10 @@ static WidePlan plan_wide(const dyhip_device* dev, size_t M, size_t N, size_t K3
   // Measured against the 128-wide kernel: a block's set-up, its 256 KiB of output and the second kernel cost about
   // three k-tiles, so runs must be long (a problem of fewer tiles than CUs is nothing but runs), and a cut remainder
   // after full rounds pays only under deep tiles.
+  // A last round of whole tiles is only worth a round when it is mostly full.
   const bool split = p.per < p.nt;
   if (p.direct_tiles == 0) p.ok = split ? p.per >= 16 : p.nt >= 16 && p.rem * 4 >= cus * 3;
-  else p.ok = split ? p.nt >= 16 : p.nt >= 8;
+  else p.ok = split ? p.nt >= 16 : p.nt >= 8 && (p.rem == 0 || p.rem * 4 >= cus * 3);
   return p;
 }
 
@@ -514,6 +515,16 @@ bool gemm_wide_eligible(const dyhip_device* dev, bool a_kmajor, bool b_kmajor, s
   if (double(M) * double(N) < 0.8 * double(tiles) * double(kSlotFloats)) return false;
   if (dev->gemm_ws == nullptr || dev->gemm_ws_bytes < (2 * cus) * kSlotFloats * sizeof(float)) return false;
   return plan_wide(dev, M, N, K32).ok;
+}
+
+size_t gemm_wide_whole_rounds_columns(const dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N, size_t K,
+                                      const float* A, size_t lda, const float* B, size_t ldb, const float* C) {
+  const size_t cus = dev->num_cus > 0 ? size_t(dev->num_cus) : 256;
+  const size_t tiles_m = cdiv<size_t>(M, kWT), tiles = tiles_m * cdiv<size_t>(N, kWT);
+  const size_t direct = tiles / cus * cus;
+  if (direct == 0 || direct == tiles || direct % tiles_m != 0) return 0;
+  const size_t cols = direct / tiles_m * kWT;
+  return cols < N && gemm_wide_eligible(dev, a_kmajor, b_kmajor, M, cols, K, A, lda, B, ldb, C) ? cols : 0;
 }
 
 int gemm_wide_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N, size_t K32, const float* A,

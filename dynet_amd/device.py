@@ -357,7 +357,7 @@ class Device:
         out = C.c_int(0)
         _check(cdll.dyhip_gemm_uses_wide_tiles(self.handle, _i(trans_l), _i(trans_r), _sz(M), _sz(N), _sz(K),
                                                C.byref(out)))
-        return bool(out.value)
+        return int(out.value)  # 0: no, 1: the whole product, 2: its leading full-round columns
 
     def gemm_tn_acc(self, M, N, K, l, r, y):
         _check(cdll.dyhip_gemm_tn_acc(self.handle, _sz(M), _sz(N), _sz(K), _p(l), _p(r), _p(y)))

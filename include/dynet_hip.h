@@ -231,9 +231,11 @@ int dyhip_gemm_tn_acc(dyhip_device* dev, size_t M, size_t N, size_t K, const flo
 /* MatrixMultiplyTranspAcc (:162-180): y[MxN] += l[MxK] * r[NxK]^T */
 int dyhip_gemm_nt_acc(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float* y);
 /* Which kernel the three calls above take for a problem with packed leading dimensions and 16-byte aligned
- * operands: *wide_tiles = 1 for the 256 x 256-tile kernel (large outputs with enough depth per CU), 0 for the
- * 128-wide kernel or the fragment-order product.  trans_l / trans_r as in dyhip_gemm_strided_batched.  No
- * counterpart in the reference (cuBLAS picks its kernels silently); for tests and tuning. */
+ * operands: *wide_tiles = 1 when the 256 x 256-tile kernel takes the whole product (large outputs with enough
+ * depth per CU), 2 when it takes the leading columns that form full rounds of one tile per CU and the rest runs
+ * as a product of its own, 0 for the 128-wide kernel or the fragment-order product.  trans_l / trans_r as in
+ * dyhip_gemm_strided_batched.  No counterpart in the reference (cuBLAS picks its kernels silently); for tests
+ * and tuning. */
 int dyhip_gemm_uses_wide_tiles(dyhip_device* dev, int trans_l, int trans_r, size_t M, size_t N, size_t K, int* wide_tiles);
 /* The cublasSgemmStridedBatched branches of the three shims (dynet/matrix-multiply.h:27-34, 110-117,
  * 175-182), taken when the left operand is batched: for b in [0, batch)

@@ -78,12 +78,16 @@ def test_gemm_nt_shallow(dev, M, N, K):
 # is added by the 128-wide kernel); (b) one full round of whole tiles plus a remainder dealt in runs; (c) a
 # remainder too large to be worth cutting; (d) a transposed left operand whose row count is not a multiple of 4.
 # Checked against the fp64 product of the same fp32 inputs (the oracle's triple loop is the same sum, too slow here).
-WIDE_GEMM_SHAPES = [(1000, 1000, 8200), (4352, 4096, 512), (7936, 4096, 256), (1001, 1000, 8192), (2048, 2304, 2080)]
+# (e) a shallow product whose leading 4096 columns are one full round of tiles: those go to the 256-wide kernel, the
+# other 384 columns run as a product of their own.
+WIDE_GEMM_SHAPES = [(1000, 1000, 8200), (4352, 4096, 512), (7936, 4096, 256), (1001, 1000, 8192), (2048, 2304, 2080),
+                    (4096, 4480, 264)]
 
 
 @pytest.mark.parametrize("M,N,K", WIDE_GEMM_SHAPES)
 def test_gemm_wide_tiles_three_forms(dev, M, N, K):
-    assert dev.gemm_uses_wide_tiles(1, 0, M, N, K) and (M % 4 != 0 or dev.gemm_uses_wide_tiles(0, 0, M, N, K))
+    want = 2 if (M, N) == (4096, 4480) else 1
+    assert dev.gemm_uses_wide_tiles(1, 0, M, N, K) == want and (M % 4 != 0 or dev.gemm_uses_wide_tiles(0, 0, M, N, K) == want)
     rng = np.random.default_rng(M + 3 * N + 7 * K)
     y0 = f32(rng.standard_normal((N, M)))
     floor = np.sqrt(K)
