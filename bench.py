@@ -24,6 +24,7 @@ the figure is the back-to-back device time per launch, not Python's launch
 latency.
 """
 import argparse
+import gc
 import json
 import os
 import sys
@@ -560,32 +561,44 @@ def lstm_lm(steps, warmup=12, use_graph=True):
            "timed_region": "per step: host->device copy of ids and labels, id sort, forward, backward, "
                            "device-side clipping, update; one HIP-graph replay per step; loss read back after "
                            "the last step"}
+    # Each path is measured on two instances (device, model and graph built afresh); both times are reported and
+    # ms_per_step is the faster one.  The collector is off inside the timed loop: in this process, which holds the
+    # tables of every earlier leg, one full collection is a 5-10 ms pause of the host thread that launches the steps
+    # (7.1 instead of 6.6 ms per step over 30 steps; a kernel trace shows equal kernel durations either way).
     for path, tb in (("fused", True), ("nodes", False)):
-        dev = Device(0, mem_mb=(1024, 1024, 512, 1024))
-        lm = LstmLM(dev, V, E, H, L, B, T, lr=0.1, clip=5.0, time_batched=tb, path=path)
-        lm.stage(batches[0])
-        if use_graph:
-            lm.capture()
-        first = None
-        for i in range(warmup):
-            loss = lm.step(batches[i % len(batches)])
-            first = loss if first is None else first
-        dev.sync()
-        t0 = time.perf_counter()
-        for i in range(steps):
-            lm.step(batches[(warmup + i) % len(batches)], read_loss=False)
-        dev.sync()
-        dt = (time.perf_counter() - t0) / steps
-        last = float(lm.loss.numpy()[0])
+        runs = []
+        for _ in range(2):
+            dev = Device(0, mem_mb=(1024, 1024, 512, 1024))
+            lm = LstmLM(dev, V, E, H, L, B, T, lr=0.1, clip=5.0, time_batched=tb, path=path)
+            lm.stage(batches[0])
+            if use_graph:
+                lm.capture()
+            first = None
+            for i in range(warmup):
+                loss = lm.step(batches[i % len(batches)])
+                first = loss if first is None else first
+            dev.sync()
+            gc.collect()
+            gc.disable()
+            t0 = time.perf_counter()
+            for i in range(steps):
+                lm.step(batches[(warmup + i) % len(batches)], read_loss=False)
+            dev.sync()
+            dt = (time.perf_counter() - t0) / steps
+            gc.enable()
+            last = float(lm.loss.numpy()[0])
+            runs.append((dt, first, last))
+            if lm.graph is not None:
+                lm.graph.destroy()
+            dev.close()
+        dt, first, last = min(runs)
         key = "fused_cell_path" if path == "fused" else "node_at_a_time_path"
         res[key] = {"ms_per_step": round(dt * 1e3, 3), "tokens_per_s": round(T * B / dt, 1),
+                    "ms_per_step_of_each_instance": [round(r[0] * 1e3, 3) for r in runs],
                     "gemm_tflops": round(flops / dt / 1e12, 2),
                     "frac_of_fp32_mfma_peak": round(flops / dt / 1e12 / FP32_MFMA_PEAK_TFLOPS, 4),
                     "steps": steps, "loss_per_token_first": round(first / (T * B), 4),
                     "loss_per_token_last": round(last / (T * B), 4)}
-        if lm.graph is not None:
-            lm.graph.destroy()
-        dev.close()
     return res
 
 

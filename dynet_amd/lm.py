@@ -355,13 +355,22 @@ class LstmLM:
         self.update()
 
     def capture(self):
-        """Record the step once; ``step`` then replays it."""
-        self.dev.sync()
-        self.dev.graph_begin()
-        try:
-            self.issue()
-        finally:
-            self.graph = self.dev.graph_end()
+        """Record the step; ``step`` then replays it.
+
+        The step is recorded and instantiated twice and the first graph thrown away: in a process that has built and
+        destroyed many small graphs before, the first large graph replays ~3 % slower than one instantiated after
+        it (6.77 against 6.55 ms per step here; kernel durations are the same, the time goes between the nodes).
+        """
+        for attempt in range(2):
+            self.dev.sync()
+            self.dev.graph_begin()
+            try:
+                self.issue()
+            finally:
+                graph = self.dev.graph_end()
+            if attempt == 0:
+                graph.destroy()
+        self.graph = graph
         return self.graph
 
     def step(self, tokens, read_loss=True):
