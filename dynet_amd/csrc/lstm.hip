@@ -526,12 +526,18 @@ __global__ __launch_bounds__(256) void lstm_gates_skinny_kernel(unsigned H, unsi
   const unsigned pcol = ct * 32 + l32 < B ? ct * 32 + l32 : B - 1;
   // every output of this thread lies in gate row rp*64 + threadIdx.x % 64: its bias is fetched under the product
   const float bias_row = bias[rp * 64 + threadIdx.x % 64];
+  // The four waves split the depth of BOTH products taken together into quarters (with I = H two waves multiply by
+  // Wx and two by Wh): one run of the load pipeline per wave instead of one per product (its start costs ~1.5 us).
+  const unsigned G0 = op0.K / 8, Gt = G0 + op1.K / 8, lo = wave * (Gt / 4), hi = lo + Gt / 4;
   for (int which = 0; which < 2; ++which) {
     const NnOperand op = which == 0 ? op0 : op1;
-    const unsigned G = op.K / 8, gq = G / 4, g0 = wave * gq;
+    const unsigned base = which == 0 ? 0 : G0, G = op.K / 8;
+    const unsigned glo = lo > base ? lo : base, ghi = hi < base + G ? hi : base + G;
+    if (glo >= ghi) continue;
+    const unsigned g0 = glo - base;
     const float* pa = op.W + size_t(rp) * 64 + l32 + (size_t(g0) * 8 + 4 * lhi) * M;
     const float* pb = op.v + size_t(pcol) * op.K + size_t(g0) * 8 + 4 * lhi;
-    step_product<kFragAlongRows, true, 2>(acc0, acc1, pa, pa + 32, pb, gq, M);
+    step_product<kFragAlongRows, true, 2>(acc0, acc1, pa, pa + 32, pb, ghi - glo, M);
   }
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
