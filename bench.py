@@ -450,6 +450,9 @@ PMC_KERNELS = [
     ("ln_bwd_wave_kernel", "layer_norm_bwd_main"), ("combine_partials", "layer_norm_bwd_combine"),
     ("lookup_gather_kernel", "lookup_gather"), ("plan_group_kernel", "lookup_plan"),
     ("scatter_runs_kernel", "lookup_scatter_runs"), ("lse_cols_kernel", "pnls_fwd"), ("pnls_bwd_kernel", "pnls_bwd"),
+    ("lstm_step_fwd_kernel", "lstm_step_fwd"), ("skinny_tn_kernel<false, false>", "lstm_rec_bwd_packed"),
+    ("lstm_cell_bwd_kernel", "lstm_cell_bwd_packed"), ("gemm_wide_kernel<false, false>", "gemm_wide_nt_dW"),
+    ("gemm_wide_fixup_kernel", "gemm_wide_nt_dW_fixup"),
 ]
 CFG3 = {"V": 50000, "D": 512, "n": 256 * 64}
 CFG4 = {"rows": 50000, "bd": 512}
@@ -495,7 +498,13 @@ def print_pmc_summary(fetch_db, write_db, unique_ids):
             "rectify_bwd": 4 * S, "cmult_fwd": 3 * S, "cmult_bwd": 4 * S, "sum_batches_fwd": S + S // 64,
             "sum_batches_bwd": 2 * S + S // 64, "layer_norm_fwd": 2 * S + 2 * LN_N * 4,
             "layer_norm_bwd_main": 4 * S + 4 * LN_N * 4, "lookup_gather": 2 * G + CFG3["n"] * 4,
-            "lookup_scatter_runs": G + 2 * unique_ids * CFG3["D"] * 4, "pnls_fwd": X, "pnls_bwd": 3 * X}
+            "lookup_scatter_runs": G + 2 * unique_ids * CFG3["D"] * 4, "pnls_fwd": X, "pnls_bwd": 3 * X,
+            # cfg-5 timestep at H = 1024, B = 128 (HB = H*B floats): packed Wh once + 13 HB; packed Wh^T once + 4 HB
+            # in + 4 slices of HB out; 4+4+4+4+1 HB in and out of the packed cell backward
+            "lstm_step_fwd": (4 * 1024 * 1024 + 13 * 1024 * 128) * 4, "lstm_rec_bwd_packed": (4 * 1024 * 1024 + 8 * 1024 * 128) * 4,
+            "lstm_cell_bwd_packed": 21 * 1024 * 128 * 4,
+            # operands once + the output read and written (the partial tiles of its runs are traffic on top)
+            "gemm_wide_nt_dW": (4096 * 4480 + 1024 * 4480 + 2 * 4096 * 1024) * 4}
     kib = S / 1024.0
     cs, cp = rows.get("copy_streaming"), rows.get("copy_plain")
     ff = kib / cs[1]
@@ -508,7 +517,8 @@ def print_pmc_summary(fetch_db, write_db, unique_ids):
     print("  python3 bench.py --pmc-summary <FETCH run>/pmc_results.db <WRITE run>/pmc_results.db --unique-ids %d" % unique_ids)
     print("(--one-pass: plain launches of the cfg-2 sweep over 4 buffer sets, each preceded by the library's copy kernel on a")
     print(" 16 MiB tensor, once with streaming (non-temporal) and once with plain accesses; then the cfg-3 lookup kernels and")
-    print(" the cfg-4 PickNegLogSoftmax kernels on 4 buffer sets each.  KiB per dispatch, averaged, from the rocpd database.)")
+    print(" the cfg-4 PickNegLogSoftmax kernels on 4 buffer sets each; then the kernels of one cfg-5 timestep (H = 1024, B = 128,")
+    print(" packed operands) and the weight-gradient GEMM 4096x1024x4480.  KiB per dispatch, averaged, from the rocpd database.)")
     print()
     print("calibration: the copy kernel moves %.0f KiB each way." % kib)
     print("  streaming accesses: FETCH_SIZE reads %.1f, WRITE_SIZE reads %.1f" % (cs[1], cs[2]))
@@ -539,6 +549,39 @@ def print_pmc_summary(fetch_db, write_db, unique_ids):
     for name in sorted(t):
         if not name.startswith("copy_"):
             print("TRAFFIC %s %.0f" % (name, t[name]))
+
+
+def lstm_one_pass(dev, launches=4):
+    """For the counter runs: the kernels of one cfg-5 timestep (H = 1024, B = 128) on packed operands and the
+    weight-gradient GEMM over all timesteps (4096 x 1024 x 4480, accumulating), `launches` plain launches each."""
+    H, B, T = 1024, 128, 35
+    Wh = dev.empty((H, 4 * H))
+    h, c, c2, hh, dh, dc, dc2 = (dev.empty((B, H)) for _ in range(7))
+    xp, g, dpre = (dev.empty((B, 4 * H)) for _ in range(3))
+    bias = dev.empty((4 * H,))
+    for t in (Wh, h, c, dh, dc, xp, bias):
+        dev.randomize_normal(t, 0.0, 0.1)
+    pk, pkT = dev.empty((4 * H * H,)), dev.empty((4 * H * H,))
+    dev.lstm_pack_recurrent(H, Wh, pk)
+    dev.lstm_pack_recurrent_transposed(H, Wh, pkT)
+    nh, nd = dev.lstm_packed_state_floats(H, B), dev.lstm_packed_state_floats(4 * H, B)
+    hp_in, hp_out, dpp = dev.empty((nh,)), dev.empty((nh,)), dev.empty((nd,))
+    dev.lstm_pack_state(H, B, h, hp_in)
+    _, bb = dev.lstm_cell_workspace(H, B)
+    wb, _ = dev.workspace(bb)
+    dev.lstm_step_forward_packed(H, B, pk, hp_in, xp, bias, c, g, c2, hh, hp_out)
+    nb = 0
+    for _ in range(launches):
+        dev.lstm_step_forward_packed(H, B, pk, hp_in, xp, bias, c, g, c2, hh, hp_out)
+        dev.lstm_cell_backward_packed(H, B, g, c2, c, dh, wb if nb else None, nb, dc, dpre, dc2, dpp)
+        nb = dev.lstm_recurrent_backward_packed(H, B, pkT, dpp, wb, bb)
+    N = T * B
+    a, b, y = dev.empty((N, 4 * H)), dev.empty((N, H)), dev.empty((H, 4 * H))
+    for t in (a, b, y):
+        dev.randomize_normal(t, 0.0, 0.1)
+    for _ in range(launches):
+        dev.gemm_nt_acc(4 * H, H, N, a, b, y)
+    dev.sync()
 
 
 def lstm_lm(steps, warmup=12, use_graph=True):
@@ -802,6 +845,7 @@ def main():
             dev.sync()
             for w in (lib.POOL_FXS, lib.POOL_DEDFS, lib.POOL_SCS):
                 dev.free_pool(w)
+        lstm_one_pass(dev)
         dev.close()
         print(json.dumps({"one_pass": True, "calibration": "ew_vec4_kernel<..IdentityFwd> moves 16384 KiB each way"}))
         return
@@ -887,7 +931,7 @@ def main():
                              "us": copy["us"], "GBps": copy["GBps"], "frac_of_8TBps": copy["frac_of_8TBps"]},
         "kernels": table,
         # cfg 5, both paths named: the drop-in one (DyNet's nodes called one at a time, as its executor does) and the
-        # time-batched / fused one, which needs the builder-level call sequence INTEGRATION.md describes
+        # time-batched / fused one, which needs a builder-level call sequence (the timesteps of a layer issued together)
         "lstm_lm_tokens_per_s_node_api": None, "lstm_lm_tokens_per_s_fused_path": None,
     }
     for w in (lib.POOL_FXS, lib.POOL_DEDFS, lib.POOL_SCS):
