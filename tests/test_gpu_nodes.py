@@ -114,6 +114,36 @@ def test_gemm_wide_tiles_three_forms(dev, M, N, K):
         assert_close(yt.numpy(), beta * y0 + exact, FWD_RTOL, "wide gemm_tn beta=%g" % beta, floor=floor)
 
 
+def test_gemm_wide_tiles_first_used_inside_a_graph_and_scaled_accumulate():
+    """A device whose first large product is recorded into a graph (the kernel's dynamic-LDS opt-in then happens
+    during the capture), replayed with eager work between the replays; and beta other than 0 or 1."""
+    from dynet_amd import Device
+
+    d = Device(0, mem_mb=(256, 64, 64, 64))
+    try:
+        M, N, K = 1024, 1024, 8192
+        assert d.gemm_uses_wide_tiles(0, 0, M, N, K) == 1
+        rng = np.random.default_rng(5)
+        l, r = f32(rng.standard_normal((K, M))), f32(rng.standard_normal((N, K)))
+        y0 = f32(rng.standard_normal((N, M)))
+        exact = r.astype(np.float64) @ l.astype(np.float64)
+        lt, rt, yt, y0t = d.tensor(l), d.tensor(r), d.empty((N, M)), d.tensor(y0)
+        d.graph_begin()
+        d.scale_copy(M * N, y0t, 1.0, yt)
+        d.gemm_nn(M, N, K, lt, rt, 0.5, yt)
+        g = d.graph_end()
+        for replay in range(3):
+            g.launch()
+            d.sync()
+            assert_close(yt.numpy(), 0.5 * y0 + exact, FWD_RTOL, "wide gemm in a graph, replay %d" % replay,
+                         floor=np.sqrt(K))
+            d.constant(yt, 7.0)  # eager work between the replays
+            d.sync()
+        g.destroy()
+    finally:
+        d.close()
+
+
 @pytest.mark.parametrize("M,N,K,B", [(64, 48, 32, 5), (130, 70, 33, 3), (7, 5, 3, 17), (256, 128, 256, 4), (31, 1, 9, 2)])
 def test_gemm_strided_batched(dev, M, N, K, B):
     """The batched-left-operand branches of the three GEMM shims: per batch item the plain product, as the
