@@ -15,6 +15,12 @@ pytestmark = pytest.mark.gpu
 # ---------------------------------------------------------------------------
 # GEMM shim
 # ---------------------------------------------------------------------------
+def lib_pools():
+    from dynet_amd import lib
+
+    return (lib.POOL_FXS, lib.POOL_DEDFS, lib.POOL_SCS)
+
+
 GEMM_SHAPES = [(1024, 32, 128), (1024, 32, 256), (4096, 128, 1280), (256, 128, 4096), (130, 33, 17), (5, 4, 6),
                (64, 1, 64), (1000, 128, 1024), (129, 65, 100),
                # small outputs with deep sums: the transposed form takes the fragment-order product (ragged edges,
@@ -112,6 +118,48 @@ def test_gemm_wide_tiles_three_forms(dev, M, N, K):
         yt = dev.tensor(y0)
         dev.gemm_tn(M, N, K, dev.tensor(l2), rt, beta, yt)
         assert_close(yt.numpy(), beta * y0 + exact, FWD_RTOL, "wide gemm_tn beta=%g" % beta, floor=floor)
+
+
+def test_gemm_wide_tiles_random_shapes(dev):
+    """Seeded random shapes of the four classes the planner of the 256 x 256-tile kernel tells apart -- fewer tiles
+    than CUs (nothing but runs of k-tiles, which end inside tiles), full rounds plus a remainder cut into runs, full
+    rounds plus leading-column split, full rounds plus a remainder large enough to run whole -- with ragged edges
+    and depths with and without a remainder of 32; all three forms against the fp64 product."""
+    rng = np.random.default_rng(2024)
+    r4 = lambda lo, hi: 4 * int(rng.integers(lo, hi))
+    shapes = []
+    for _ in range(4):  # few tiles, deep
+        a, b = int(rng.integers(2, 5)), int(rng.integers(2, 5))
+        nt = -(-4096 // (a * b)) + int(rng.integers(0, 8))
+        shapes.append((256 * a - r4(0, 10), 256 * b - r4(0, 10), 32 * nt + r4(0, 8)))
+    for _ in range(2):  # one round and a few tile columns more, cut into runs
+        shapes.append((256 * 17 - r4(0, 10), 256 * int(rng.integers(17, 19)) - r4(0, 10), 32 * int(rng.integers(16, 22)) + r4(0, 8)))
+    for _ in range(2):  # one exact round of tile columns and some columns more
+        shapes.append((4096, 4096 + r4(10, 100), 32 * int(rng.integers(8, 12)) + r4(0, 8)))
+    shapes.append((256 * 19 - r4(0, 10), 256 * 24 - r4(0, 10), 256 + r4(0, 8)))  # 456 tiles: the last 200 run whole
+    taken = set()
+    for M, N, K in shapes:
+        kind = dev.gemm_uses_wide_tiles(0, 0, M, N, K)
+        taken.add(kind)
+        l, r = f32(rng.standard_normal((K, M))), f32(rng.standard_normal((N, K)))
+        y0 = f32(rng.standard_normal((N, M)))
+        exact = r.astype(np.float64) @ l.astype(np.float64)
+        lt, rt = dev.tensor(l), dev.tensor(r)
+        what = "M=%d N=%d K=%d kernel choice %d" % (M, N, K, kind)
+        assert kind != 0, what
+        yt = dev.tensor(y0)
+        dev.gemm_nn(M, N, K, lt, rt, 1.0, yt)
+        assert_close(yt.numpy(), y0 + exact, FWD_RTOL, "gemm_nn " + what, floor=np.sqrt(K))
+        yt = dev.tensor(y0)
+        dev.gemm_nt(M, N, K, lt, dev.tensor(f32(r.T)), 0.0, yt)
+        assert_close(yt.numpy(), exact, FWD_RTOL, "gemm_nt " + what, floor=np.sqrt(K))
+        yt = dev.tensor(y0)
+        dev.gemm_tn(M, N, K, dev.tensor(f32(l.T)), rt, 1.0, yt)
+        assert_close(yt.numpy(), y0 + exact, FWD_RTOL, "gemm_tn " + what, floor=np.sqrt(K))
+        for w in lib_pools():
+            dev.sync()
+            dev.free_pool(w)
+    assert taken == {1, 2}
 
 
 def test_gemm_wide_tiles_first_used_inside_a_graph_and_scaled_accumulate():
