@@ -86,12 +86,32 @@ __global__ __launch_bounds__(kThreads) void ragged_move_kernel(int num_seqs, flo
 }
 
 // stage 1: per-block partial of sum g^2 ; stage 2: one block adds the partials in order
+// partial[block] = sum of squares of the block's share.  The 16-byte aligned middle of the array goes through
+// 128-bit loads, four in flight per thread (plain ones: the update that follows reads the same gradient); the few floats before and after it are added by block 0.
 __global__ __launch_bounds__(kThreads) void sqnorm_partial_kernel(size_t n, const float* __restrict__ g,
                                                                   float* __restrict__ partial) {
   __shared__ float red[4];
+  const size_t head = min(n, (size_t(4) - ((reinterpret_cast<uintptr_t>(g) >> 2) & 3u)) & 3u);  // floats before alignment
+  const size_t n4 = (n - head) / 4;
+  const float4* g4 = reinterpret_cast<const float4*>(g + head);
   float s = 0.f;
   const size_t stride = size_t(gridDim.x) * kThreads;
-  for (size_t i = size_t(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride) s += g[i] * g[i];
+  size_t i = size_t(blockIdx.x) * kThreads + threadIdx.x;
+  for (; i + 3 * stride < n4; i += 4 * stride) {
+    const float4 a = ldg4<false>(g4 + i), b = ldg4<false>(g4 + i + stride), c = ldg4<false>(g4 + i + 2 * stride),
+                 d = ldg4<false>(g4 + i + 3 * stride);
+    s += ((a.x * a.x + a.y * a.y) + (a.z * a.z + a.w * a.w)) + ((b.x * b.x + b.y * b.y) + (b.z * b.z + b.w * b.w));
+    s += ((c.x * c.x + c.y * c.y) + (c.z * c.z + c.w * c.w)) + ((d.x * d.x + d.y * d.y) + (d.z * d.z + d.w * d.w));
+  }
+  for (; i < n4; i += stride) {
+    const float4 a = ldg4<false>(g4 + i);
+    s += (a.x * a.x + a.y * a.y) + (a.z * a.z + a.w * a.w);
+  }
+  if (blockIdx.x == 0) {
+    const size_t tail0 = head + 4 * n4;
+    for (size_t j = threadIdx.x; j < head; j += kThreads) s += g[j] * g[j];
+    for (size_t j = tail0 + threadIdx.x; j < n; j += kThreads) s += g[j] * g[j];
+  }
   const float t = block_sum<4>(s, red);
   if (threadIdx.x == 0) partial[blockIdx.x] = t;
 }
@@ -205,7 +225,7 @@ int dyhip_squared_l2norm(dyhip_device* dev, size_t n, const float* g, float* out
   DYHIP_REQUIRE(out != nullptr && (n == 0 || g != nullptr), "null pointer");
   DYHIP_REQUIRE(ws != nullptr && ws_bytes >= kSqnormBlocks * sizeof(float), "squared_l2norm needs %zu workspace bytes",
                 kSqnormBlocks * sizeof(float));
-  unsigned blocks = static_cast<unsigned>((n + size_t(kThreads) * 8 - 1) / (size_t(kThreads) * 8));
+  unsigned blocks = static_cast<unsigned>((n + size_t(kThreads) * 16 - 1) / (size_t(kThreads) * 16));
   if (blocks < 1) blocks = 1;
   if (blocks > kSqnormBlocks) blocks = kSqnormBlocks;
   float* partial = static_cast<float*>(ws);

@@ -1131,6 +1131,19 @@ def test_scale_copy_constant_accumulate_sgd_norm(dev):
     assert abs(float(nrm.numpy()[0]) - float((g.astype(np.float64) ** 2).sum())) < 1e-5 * n
 
 
+@pytest.mark.parametrize("n,shift", [(1, 0), (3, 1), (1000003, 0), (1000003, 1), (1000003, 3), (4096, 2), (24 * 1024 * 1024 + 5, 0)])
+def test_squared_l2norm_any_length_and_alignment(dev, n, shift):
+    """The vector body of the squared norm starts at the first 16-byte boundary: lengths that are not multiples of 4
+    and inputs that start 4, 8 or 12 bytes past one; the largest case takes the full grid."""
+    rng = np.random.default_rng(n + shift)
+    g = f32(rng.standard_normal(n + shift))
+    gt = dev.tensor(g).offset(shift, (n,))
+    nrm = dev.empty(1)
+    dev.squared_l2norm(n, gt, nrm)
+    want = float((g[shift:].astype(np.float64) ** 2).sum())
+    assert abs(float(nrm.numpy()[0]) - want) <= 2e-6 * want + 1e-6
+
+
 def test_device_side_clipping_and_sparse_rows(dev):
     rng = np.random.default_rng(19)
     vocab, dim, n = 500, 48, 700
