@@ -59,6 +59,7 @@ struct dyhip_pool {
 struct dyhip_device {
   int ordinal;
   int num_cus;
+  size_t max_lds_per_block;  // what a block may opt in to (dynamic LDS); 0 if unknown
   hipStream_t stream;
   dyhip::MemAllocator* alloc;
   dyhip_pool* pools[4];

@@ -283,6 +283,7 @@ int dyhip_device_create(int ordinal, const size_t pool_mb[4], dyhip_device** out
   dev->sync_next = 0;
   dev->ordinal = ordinal;
   dev->num_cus = prop.multiProcessorCount;
+  dev->max_lds_per_block = prop.sharedMemPerBlockOptin > 0 ? prop.sharedMemPerBlockOptin : prop.sharedMemPerBlock;
   for (auto& p : dev->pools) p = nullptr;
   dev->scalars = nullptr;
   dev->rng_state = nullptr;

@@ -503,7 +503,7 @@ static WidePlan plan_wide(const dyhip_device* dev, size_t M, size_t N, size_t K3
 bool gemm_wide_eligible(const dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N, size_t K,
                         const float* A, size_t lda, const float* B, size_t ldb, const float* C) {
   const size_t K32 = K / kWK * kWK;
-  if (K32 < 256 || M < 192 || N < 192) return false;
+  if (K32 < 256 || M < 192 || N < 192 || dev->max_lds_per_block < kWideLdsBytes) return false;
   if (!aligned16(A) || !aligned16(B) || !aligned16(C) || lda % 4 != 0 || ldb % 4 != 0) return false;
   if ((!a_kmajor && M % 4 != 0) || (!b_kmajor && N % 4 != 0)) return false;
   // 32-bit element offsets inside the kernel
@@ -564,6 +564,7 @@ int gemm_wide_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, siz
 bool gemm_shallow_nt_eligible(const dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda,
                               const float* B, size_t ldb, const float* C) {
   if (K < 32 || K > 128 || K % 8 != 0 || M % 4 != 0 || N % 4 != 0 || M < 128 || N < 128) return false;
+  if (dev->max_lds_per_block < kShallowLdsBytes) return false;
   if (!aligned16(A) || !aligned16(B) || lda % 4 != 0 || ldb % 4 != 0 || (reinterpret_cast<uintptr_t>(C) & 7u) != 0)
     return false;
   if (K * lda >= (size_t(1) << 31) || K * ldb >= (size_t(1) << 31) || M * N >= (size_t(1) << 31)) return false;
