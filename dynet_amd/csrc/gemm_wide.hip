@@ -3,10 +3,10 @@
 // (v_mfma_f32_32x32x2_f32, fp32 in and out) as gemm.hip, which keeps the small, skinny, ragged, segmented and batched
 // problems (dynet/matrix-multiply.h:16-37,97-117,162-180 are the callers this replaces cublasSgemm for).
 //
-// Why a second kernel.  A 128 x 128 tile pulls 32 KiB of operands through the CU's vector memory path per 1 MFLOP;
-// with two such blocks per CU that path is two thirds busy and the loads, their LDS writes and the address arithmetic
-// share issue slots with the MFMAs.  A 256 x 256 tile halves the bytes per flop, and `global_load_lds_dwordx4` moves
-// them without passing through registers: the main loop is MFMAs, 24 LDS reads and 8 load issues per 128 MFMAs.
+// Why a second kernel.  A 128 x 128 tile needs 32 KiB of operands per MFLOP, and gemm.hip stages them through
+// registers into LDS: the loads, the LDS writes and the address arithmetic share issue slots with the MFMAs, and the
+// staging registers are what limits its tile.  A 256 x 256 tile halves the bytes per flop, and `global_load_lds_dwordx4`
+// moves them without passing through registers: the main loop is MFMAs, 24 LDS reads and 8 load issues per 128 MFMAs.
 //
 // LDS.  Two stages of 64 KiB.  A stage holds the 256 x 32 tiles of both operands as 64 chunks of 1 KiB, one per
 // wave-wide load (64 lanes x 16 bytes; lane j fills bytes 16 j.. of its chunk).  Wave w issues chunks 4w..4w+3 of each

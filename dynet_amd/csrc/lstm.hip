@@ -247,10 +247,11 @@ __global__ __launch_bounds__(kCellThreads) void lstm_cell_bwd_kernel(unsigned H,
 // to memory.  The four waves split the depth of the sum in quarters and meet in LDS; each wave
 // multiplies two 32-row tiles by one 32-column tile, so a fragment of the state feeds two MFMAs.
 //
-// What bounds the kernel is the rate at which one CU can pull operands through its vector memory
-// path (about 26 GB/s whether they come from L2 or from HBM), so the tile is chosen for the fewest
-// operand bytes per CU that still gives every CU a block at H = 1024, B = 128: (64 + 32) rows and
-// columns of depth H per block.  Both operands are read in MFMA fragment order straight into
+// The kernel is bound by the MFMA issue of its one wavefront per SIMD (256 MFMAs per wave at H = 1024);
+// the tile is the one with the fewest operand bytes per block that still gives every CU a block at
+// H = 1024, B = 128, (64 + 32) rows and columns of depth H.  Blocks b and b + 8k run on the same XCD,
+// so the column tiles of one row pair share its L2 and the weights arrive from beyond it once per
+// launch, not once per block.  Both operands are read in MFMA fragment order straight into
 // registers (no LDS stage, no barrier in the loop): for a 32-wide tile and a group of 8 consecutive
 // k, lane l = 32*lhi + l32 holds k = 8*kg + 4*lhi + s, s = 0..3, of row (or column) l32 as one
 // float4 (MFMA step s of the group multiplies k = 8*kg + s and 8*kg + 4 + s; the order inside a

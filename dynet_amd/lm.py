@@ -19,8 +19,9 @@ What differs from DyNet's node-at-a-time execution (results agree to fp32 roundi
     order that the previous timestep's kernel wrote (``single_launch``, where the sizes allow);
   * with ``overlap=True`` the fused path cuts the time axis into chunks and runs the layers as a pipeline on one
     queue per layer: layer l works on chunk k while layer l-1 is already on chunk k+1 (backward: l on chunk k, l+1
-    on chunk k-1).  It paid off while a timestep's kernels left most of the GPU idle; the packed kernels are bound by
-    what one CU can load, two of them side by side only slow each other, and the default is one queue.
+    on chunk k-1).  It paid off while a timestep's kernels left most of the GPU idle; the packed kernels keep the
+    matrix cores of every CU busy on their own, two of them side by side only slow each other, and the default is
+    one queue.
 """
 import numpy as np
 
