@@ -599,8 +599,9 @@ def lstm_lm(steps, warmup=12, use_graph=True):
                       "ids": "Zipf(1.1)"},
            "tokens_per_step": T * B, "gemm_flop_per_step": flops,
            "fused_path_schedule": "one device queue, layer by layer; a forward timestep is one kernel (recurrent "
-                                  "product + cell update), a backward timestep two (cell update, Wh^T dpre), "
-                                  "operands handed from timestep to timestep in matrix-core fragment order",
+                                  "product + cell update) and so is a backward one (Wh^T dpre of the step above + "
+                                  "cell backward), operands handed from timestep to timestep in matrix-core "
+                                  "fragment order",
            "timed_region": "per step: host->device copy of ids and labels, id sort, forward, backward, "
                            "device-side clipping, update; one HIP-graph replay per step; loss read back after "
                            "the last step"}
@@ -716,9 +717,18 @@ def lm_kernels(reps, use_graph=True):
     dev.lstm_cell_backward_packed(H, B, g, c2, c, dh, None, 0, dc, dpre, dc2, dpp)
     nbp = dev.lstm_recurrent_backward_packed(H, B, pkT, dpp, wb, bb)
     rec_bwd = lambda: dev.lstm_recurrent_backward_packed(H, B, pkT, dpp, wb, bb)
+    # the same backward timestep as one launch (what the fused path issues): 16x16x4 fragment order
+    pkT16 = dev.empty((4 * H * H,))
+    dev.lstm_pack_recurrent_transposed16(H, Wh, pkT16)
+    nd16 = dev.lstm_packed_state16_floats(4 * H, B)
+    dp16_in, dp16_out = dev.empty((nd16,)), dev.empty((nd16,))
+    dev.lstm_pack_state16(4 * H, B, dpre, dp16_in)
+    step_bwd = lambda: dev.lstm_step_backward_packed(H, B, pkT16, dp16_in, g, c2, c, dh, dc, dpre, dc2, dp16_out)
     cell_bwd = lambda: dev.lstm_cell_backward_packed(H, B, g, c2, c, dh, wb, nbp, dc, dpre, dc2, dpp)
     for name, fn, flops, nbytes in (("lstm_step_fwd (recurrent product + cell update)", step, 2.0 * 4 * H * H * B,
                                      (4 * H * H + H * B + 4 * H * B + 4 * H + H * B + 7 * H * B) * 4),
+                                    ("lstm_step_bwd (Wh^T dpre over the whole depth + cell backward, one launch)", step_bwd,
+                                     2.0 * 4 * H * H * B, (4 * H * H + 4 * H * B + 17 * H * B) * 4),
                                     ("lstm_rec_bwd (Wh^T dpre from packed operands, %d slices)" % nbp, rec_bwd,
                                      2.0 * 4 * H * H * B, (4 * H * H + 4 * H * B + nbp * H * B) * 4),
                                     ("lstm_cell_bwd_packed (%d slices, dpre plain + packed)" % nbp, cell_bwd, 0.0,

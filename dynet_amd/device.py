@@ -472,6 +472,25 @@ class Device:
         _check(cdll.dyhip_lstm_cell_backward_packed(self.handle, _u(H), _u(B), _p(gates), _p(c), _p(c_tm1), _p(dh),
                                                     _vp(rec), _u(splits), _p(dc), _p(dpre), _p(dc_tm1), _p(dpre_packed)))
 
+    def lstm_pack_recurrent_transposed16(self, H, Wh, packed):
+        _check(cdll.dyhip_lstm_pack_recurrent_transposed16(self.handle, _u(H), _p(Wh), _p(packed)))
+
+    @staticmethod
+    def lstm_packed_state16_floats(rows, B):
+        n = C.c_size_t(0)
+        _check(cdll.dyhip_lstm_packed_state16_floats(_u(rows), _u(B), C.byref(n)))
+        return n.value
+
+    def lstm_pack_state16(self, rows, B, v, packed):
+        _check(cdll.dyhip_lstm_pack_state16(self.handle, _u(rows), _u(B), _p(v), _p(packed)))
+
+    def lstm_step_backward_packed(self, H, B, packed_WhT16, dpre_next_packed16, gates, c, c_tm1, dh, dc, dpre, dc_tm1,
+                                  dpre_packed16):
+        """One launch per backward timestep: Wh^T * dpre_{t+1} over its whole depth and the cell backward of step t."""
+        _check(cdll.dyhip_lstm_step_backward_packed(self.handle, _u(H), _u(B), _p(packed_WhT16),
+                                                    _p(dpre_next_packed16), _p(gates), _p(c), _p(c_tm1), _p(dh), _p(dc),
+                                                    _p(dpre), _p(dc_tm1), _p(dpre_packed16)))
+
     def lstm_pack_input(self, I, H, Wx, packed):
         _check(cdll.dyhip_lstm_pack_input(self.handle, _u(I), _u(H), _p(Wx), _p(packed)))
 

@@ -14,9 +14,9 @@ What differs from DyNet's node-at-a-time execution (results agree to fp32 roundi
   * ``path="fused"`` (default) runs layer by layer: one GEMM forms Wx*x for all timesteps, a timestep is then
     the recurrent GEMM Wh*h plus one cell kernel (gates + c + h); backward mirrors it, and dx, dWx, dWh, db are
     GEMMs/reductions over all timesteps;
-  * a timestep of the fused path is one kernel forward (recurrent product + cell update) and two backward (cell
-    update, then the slices of Wh^T * dpre), all reading their operands from packed copies in matrix-core fragment
-    order that the previous timestep's kernel wrote (``single_launch``, where the sizes allow);
+  * a timestep of the fused path is one kernel forward (recurrent product + cell update) and one backward (Wh^T *
+    dpre of the step above + cell backward), both reading their operands from packed copies in matrix-core
+    fragment order that the previous timestep's kernel wrote (``single_launch``, where the sizes allow);
   * with ``overlap=True`` the fused path cuts the time axis into chunks and runs the layers as a pipeline on one
     queue per layer: layer l works on chunk k while layer l-1 is already on chunk k+1 (backward: l on chunk k, l+1
     on chunk k-1).  It paid off while a timestep's kernels left most of the GPU idle; the packed kernels keep the
@@ -97,7 +97,7 @@ class LstmLM:
         self.WhT_packed = [dev.empty((4 * H * H,), pool=PS) for _ in range(L)] if self.single_launch else []
         # packed copies of h and of dpre for the next timestep's recurrent product, two per layer used in turn
         nh = dev.lstm_packed_state_floats(H, B) if self.single_launch else 0
-        nd = dev.lstm_packed_state_floats(4 * H, B) if self.single_launch else 0
+        nd = dev.lstm_packed_state16_floats(4 * H, B) if self.single_launch else 0
         self.h_packed = [[dev.empty((nh,), pool=FXS) for _ in range(2)] for _ in range(L)] if self.single_launch else []
         self.dpre_packed = [[dev.empty((nd,), pool=DE) for _ in range(2)] for _ in range(L)] if self.single_launch else []
         # queue l runs layer l; queue 0 is the device itself
@@ -188,7 +188,7 @@ class LstmLM:
         if self.single_launch:  # the weights moved in the last update
             for l in range(L):
                 d.lstm_pack_recurrent(H, self.p[f"Wh{l}"], self.Wh_packed[l])
-                d.lstm_pack_recurrent_transposed(H, self.p[f"Wh{l}"], self.WhT_packed[l])
+                d.lstm_pack_recurrent_transposed16(H, self.p[f"Wh{l}"], self.WhT_packed[l])
         if not self.overlap:
             for l in range(L):
                 x, d_in = (self.h[l - 1], H) if l > 0 else (self.emb, E)
@@ -251,17 +251,20 @@ class LstmLM:
         for t in reversed(range(t0, t1)):
             last, first = t == T - 1, t == 0
             dpre = self._t(self.d_pre[l], t, 4 * H)
+            if self.single_launch:
+                # one launch: Wh^T * dpre of the step above (from the fragment-order copy that step's launch wrote)
+                # and this step's cell backward, which writes dpre plain and in fragment order for the step below
+                q.lstm_step_backward_packed(H, B, self.WhT_packed[l], None if last else self.dpre_packed[l][(t + 1) % 2],
+                                            self._t(self.gates[l], t, 4 * H), self._t(self.c[l], t, H),
+                                            None if first else self._t(self.c[l], t - 1, H), self._t(self.d_h[l], t, H),
+                                            None if last else self._t(self.d_c[l], t, H), dpre,
+                                            None if first else self._t(self.d_c[l], t - 1, H),
+                                            None if first else self.dpre_packed[l][t % 2])
+                continue
             args = (H, B, self._t(self.gates[l], t, 4 * H), self._t(self.c[l], t, H),
                     None if first else self._t(self.c[l], t - 1, H), self._t(self.d_h[l], t, H),
                     None if last else self.rec_b[l], 0 if last else self._rec_b_n[l],
                     None if last else self._t(self.d_c[l], t, H), dpre, None if first else self._t(self.d_c[l], t - 1, H))
-            if self.single_launch:  # dpre also in the operand order of the recurrent product below
-                dpp = self.dpre_packed[l][t % 2]
-                q.lstm_cell_backward_packed(*args, None if first else dpp)
-                if not first:
-                    self._rec_b_n[l] = q.lstm_recurrent_backward_packed(H, B, self.WhT_packed[l], dpp, self.rec_b[l],
-                                                                        self.rec_b_bytes)
-                continue
             q.lstm_cell_backward(*args)
             if not first:
                 self._rec_b_n[l] = q.lstm_recurrent_backward(H, B, Wh, dpre, self.rec_b[l], self.rec_b_bytes)

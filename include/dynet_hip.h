@@ -352,6 +352,24 @@ int dyhip_lstm_recurrent_backward_packed(dyhip_device* dev, unsigned H, unsigned
 int dyhip_lstm_cell_backward_packed(dyhip_device* dev, unsigned H, unsigned B, const float* gates, const float* c,
                                     const float* c_tm1, const float* dh, const float* rec, unsigned splits,
                                     const float* dc, float* dpre, float* dc_tm1, float* dpre_packed);
+/* The backward timestep in ONE launch (the mirror of dyhip_lstm_step_forward_packed; no counterpart in the
+ * reference, whose backward is the three nodes' backward_dev_impl, dynet/nodes-lstm.cc:238-372,605-614,684-701):
+ *   dh_t  = dh + Wh^T * dpre_{t+1}                       (the product over its whole depth 4H, inside the kernel)
+ *   dpre_t, dc_tm1 = cell backward(gates_t, c_t, c_tm1, dh_t, dc)   (the formulas of dyhip_lstm_cell_backward)
+ * Wh^T and dpre_{t+1} are read in the fragment order of the 16x16x4 matrix-core instruction:
+ * dyhip_lstm_pack_recurrent_transposed16 packs Wh (4*H*H floats, once per weight update); the kernel itself writes
+ * dpre_t in that order to dpre_packed16 (dyhip_lstm_packed_state16_floats(4*H, B) floats) for the launch of
+ * timestep t-1, next to the plain dpre (4H x B) that the weight-gradient products over all timesteps read.
+ * dpre_next_packed16 null: the last timestep, no recurrent term; c_tm1, dc, dc_tm1, dpre_packed16 may be null
+ * as in dyhip_lstm_cell_backward.  dyhip_lstm_pack_state16 packs a 4H x B dpre that did not come from a launch of
+ * this kernel.  Sizes as dyhip_lstm_step_supported says. */
+int dyhip_lstm_pack_recurrent_transposed16(dyhip_device* dev, unsigned H, const float* Wh, float* packed);
+int dyhip_lstm_packed_state16_floats(unsigned rows, unsigned B, size_t* floats);
+int dyhip_lstm_pack_state16(dyhip_device* dev, unsigned rows, unsigned B, const float* v, float* packed);
+int dyhip_lstm_step_backward_packed(dyhip_device* dev, unsigned H, unsigned B, const float* packed_WhT16,
+                                    const float* dpre_next_packed16, const float* gates, const float* c,
+                                    const float* c_tm1, const float* dh, const float* dc, float* dpre, float* dc_tm1,
+                                    float* dpre_packed16);
 /* The whole forward of a timestep in one launch, input product included: gates = act(b + [f: +1] +
  * Wx * x + Wh * h_tm1) from packed copies of both weight matrices (dyhip_lstm_pack_input: Wx is
  * 4H x I, I a multiple of 128), then c and h; x and h_tm1 are plain.  For callers

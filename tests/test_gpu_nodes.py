@@ -639,6 +639,69 @@ def test_packed_backward_timestep_equals_the_two_call_form(dev, H, B):
     assert_close(dcp2.numpy(), dcv * gates[:, H:2 * H], GRAD_RTOL, "dc_tm1 after the packed product", floor=1.0)
 
 
+@pytest.mark.parametrize("H,B", [(128, 1), (128, 33), (256, 32), (384, 70), (1024, 128)])
+def test_single_launch_backward_timestep(dev, H, B):
+    """dyhip_lstm_step_backward_packed over three timesteps (T-1: no recurrent term; T-2 and T-3: Wh^T * dpre of the
+    step above from the fragment-order copy the launch above wrote) against the cell-backward + recurrent-product
+    entry points on plain operands, the packed layouts against their definition, and the product against fp64."""
+    rng = np.random.default_rng(5 * H + B)
+    Wh = glorot(rng, 4 * H, H)
+    Wht = dev.tensor(Wh)
+    pT = dev.empty(4 * H * H)
+    dev.lstm_pack_recurrent_transposed16(H, Wht, pT)
+    # Wh is stored [unit j][depth k]: tile rt of Wh^T, group kg, lane 16*lq + l16, slot s <- Wh[k = 16kg + 4lq + s, j = 16rt + l16]
+    want = Wh.reshape(H // 16, 16, 4 * H // 16, 4, 4).transpose(0, 2, 3, 1, 4).reshape(-1)
+    assert np.array_equal(pT.numpy(), want)
+    n16 = dev.lstm_packed_state16_floats(4 * H, B)
+    Bp = (B + 31) // 32 * 32
+    assert n16 == 4 * H * Bp
+    _, bb = dev.lstm_cell_workspace(H, B)
+    ws, wsb = dev.workspace(bb)
+    steps = []
+    for t in range(3):
+        gates = f32(rng.uniform(0.05, 0.95, (B, 4 * H)))
+        gates[:, 3 * H:] = f32(rng.uniform(-0.9, 0.9, (B, H)))
+        steps.append(tuple(dev.tensor(a) for a in (gates, f32(rng.standard_normal((B, H))), f32(rng.standard_normal((B, H))),
+                                                   f32(rng.standard_normal((B, H))))))
+    dpp = [dev.empty(n16), dev.empty(n16)]
+    for q in dpp:
+        dev.zero(q)
+    dc_new, dc_ref = None, None
+    prev_packed, n_slices, dpre_ref_prev = None, 0, None
+    for t, (gt, ct, cpt, dht) in enumerate(steps):
+        dpre1, dcp1 = dev.empty((B, 4 * H)), dev.empty((B, H))
+        dev.lstm_step_backward_packed(H, B, pT, prev_packed, gt, ct, cpt, dht, dc_new, dpre1, dcp1, dpp[t % 2])
+        # reference: slices of Wh^T * dpre of the step above (plain operands), then the cell backward
+        dpre0, dcp0 = dev.empty((B, 4 * H)), dev.empty((B, H))
+        if dpre_ref_prev is not None:
+            n_slices = dev.lstm_recurrent_backward(H, B, Wht, dpre_ref_prev, ws, wsb)
+        dev.lstm_cell_backward(H, B, gt, ct, cpt, dht, ws if n_slices else None, n_slices, dc_ref, dpre0, dcp0)
+        what = "H=%d B=%d step %d" % (H, B, t)
+        if t == 0:  # no product: the same arithmetic on the same values
+            assert dpre1.numpy().tobytes() == dpre0.numpy().tobytes() and dcp1.numpy().tobytes() == dcp0.numpy().tobytes(), what
+        else:
+            floor = max(1.0, float(np.sqrt(4 * H) * rms(Wh) * rms(dpre_ref_prev.numpy())))
+            assert_close(dpre1.numpy(), dpre0.numpy(), GRAD_RTOL, "dpre " + what, floor=floor)
+            assert_close(dcp1.numpy(), dcp0.numpy(), GRAD_RTOL, "dc_tm1 " + what, floor=floor)
+            # the product inside the launch against fp64: recover it from dc_tm1 = (dc + (dh + rec) o (1 - tanh^2 c)) f
+            g = gt.numpy().astype(np.float64)
+            tc = np.tanh(ct.numpy().astype(np.float64))
+            rec = dpre_ref_prev.numpy().astype(np.float64) @ Wh.astype(np.float64).T
+            dcv = dc_ref.numpy() + (dht.numpy() + rec) * g[:, 2 * H:3 * H] * (1 - tc * tc)
+            assert_close(dcp1.numpy(), dcv * g[:, H:2 * H], GRAD_RTOL, "dc_tm1 vs fp64 " + what, floor=floor)
+        pad = np.zeros((Bp, 4 * H), F32)
+        pad[:B] = dpre1.numpy()
+        assert np.array_equal(dpp[t % 2].numpy(),
+                              pad.reshape(Bp // 16, 16, 4 * H // 16, 4, 4).transpose(0, 2, 3, 1, 4).reshape(-1)), what
+        prev_packed, dpre_ref_prev, dc_new, dc_ref = dpp[t % 2], dpre0, dcp1, dcp0
+    # a dpre that did not come from a launch of the kernel
+    other = dev.empty(n16)
+    dev.lstm_pack_state16(4 * H, B, dpre_ref_prev, other)
+    pad = np.zeros((Bp, 4 * H), F32)
+    pad[:B] = dpre_ref_prev.numpy()
+    assert np.array_equal(other.numpy(), pad.reshape(Bp // 16, 16, 4 * H // 16, 4, 4).transpose(0, 2, 3, 1, 4).reshape(-1))
+
+
 @pytest.mark.parametrize("I,H,B", [(128, 256, 32), (256, 128, 1), (128, 128, 45), (384, 256, 70)])
 def test_single_launch_step_with_input_product(dev, I, H, B):
     """dyhip_lstm_step_forward_x: Wx*x, Wh*h_tm1, bias, activations, c and h in one launch, from the zero state
