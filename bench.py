@@ -450,7 +450,8 @@ PMC_KERNELS = [
     ("ln_bwd_wave_kernel", "layer_norm_bwd_main"), ("combine_partials", "layer_norm_bwd_combine"),
     ("lookup_gather_kernel", "lookup_gather"), ("plan_group_kernel", "lookup_plan"),
     ("scatter_runs_kernel", "lookup_scatter_runs"), ("lse_cols_kernel", "pnls_fwd"), ("pnls_bwd_kernel", "pnls_bwd"),
-    ("lstm_step_fwd_kernel", "lstm_step_fwd"), ("skinny_tn_kernel<false, false>", "lstm_rec_bwd_packed"),
+    ("lstm_step_fwd_kernel", "lstm_step_fwd"), ("lstm_step_bwd_kernel", "lstm_step_bwd"),
+    ("skinny_tn_kernel<false, false>", "lstm_rec_bwd_packed"),
     ("lstm_cell_bwd_kernel", "lstm_cell_bwd_packed"), ("gemm_wide_kernel<false, false>", "gemm_wide_nt_dW"),
     ("gemm_wide_fixup_kernel", "gemm_wide_nt_dW_fixup"),
 ]
@@ -503,6 +504,8 @@ def print_pmc_summary(fetch_db, write_db, unique_ids):
             # in + 4 slices of HB out; 4+4+4+4+1 HB in and out of the packed cell backward
             "lstm_step_fwd": (4 * 1024 * 1024 + 13 * 1024 * 128) * 4, "lstm_rec_bwd_packed": (4 * 1024 * 1024 + 8 * 1024 * 128) * 4,
             "lstm_cell_bwd_packed": 21 * 1024 * 128 * 4,
+            # packed Wh^T once + dpre of the step above (4 HB) + gates 4, c, c_tm1, dh, dc in + dpre twice and dc_tm1 out
+            "lstm_step_bwd": (4 * 1024 * 1024 + 21 * 1024 * 128) * 4,
             # operands once + the output read and written (the partial tiles of its runs are traffic on top)
             "gemm_wide_nt_dW": (4096 * 4480 + 1024 * 4480 + 2 * 4096 * 1024) * 4}
     kib = S / 1024.0
@@ -575,6 +578,13 @@ def lstm_one_pass(dev, launches=4):
         dev.lstm_step_forward_packed(H, B, pk, hp_in, xp, bias, c, g, c2, hh, hp_out)
         dev.lstm_cell_backward_packed(H, B, g, c2, c, dh, wb if nb else None, nb, dc, dpre, dc2, dpp)
         nb = dev.lstm_recurrent_backward_packed(H, B, pkT, dpp, wb, bb)
+    pkT16 = dev.empty((4 * H * H,))
+    dev.lstm_pack_recurrent_transposed16(H, Wh, pkT16)
+    nd16 = dev.lstm_packed_state16_floats(4 * H, B)
+    dp_in, dp_out = dev.empty((nd16,)), dev.empty((nd16,))
+    dev.lstm_pack_state16(4 * H, B, dpre, dp_in)
+    for _ in range(launches):
+        dev.lstm_step_backward_packed(H, B, pkT16, dp_in, g, c2, c, dh, dc, dpre, dc2, dp_out)
     N = T * B
     a, b, y = dev.empty((N, 4 * H)), dev.empty((N, H)), dev.empty((H, 4 * H))
     for t in (a, b, y):
