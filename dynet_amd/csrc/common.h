@@ -17,6 +17,7 @@ namespace dyhip {
 int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 
 constexpr int kWave = 64;  // CDNA wavefront width
+constexpr unsigned kGemmFlagWords = 1024;  // per queue: one flag per segment of the 256x256-tile GEMM + a counter
 
 // ceil(a / b) for positive integers
 template <class T>
@@ -68,6 +69,8 @@ struct dyhip_device {
   void* gemm_ws;   // split-K partial tiles (the analogue of a BLAS handle's workspace)
   size_t gemm_ws_bytes;
   unsigned wide_gemm_ready;  // gemm_wide.hip: kernels whose dynamic-LDS limit has been raised on this device
+  unsigned* gemm_flags;      // gemm_wide.hip: kGemmFlagWords words behind gemm_ws that no other kernel touches, zero between launches
+  bool gemm_flags_used;      // a launch since the last dyhip_device_sync may have counted a wait that gave up
   hipEvent_t ev_start, ev_stop;
   dyhip_device* parent;                // non-null for a forked queue: pools, scalars and allocator belong to the parent
   std::vector<hipEvent_t> sync_events; // ring of events recorded on this queue for dyhip_device_wait

@@ -267,6 +267,14 @@ int dyhip_device_count(int* count) {
   return DYHIP_OK;
 }
 
+// The flag words of the 256 x 256-tile GEMM sit behind the split-K workspace, outside the size that other kernels
+// are told, and start out zero.
+static int gemm_flags_setup(dyhip_device* dev) {
+  dev->gemm_flags = reinterpret_cast<unsigned*>(static_cast<char*>(dev->gemm_ws) + dev->gemm_ws_bytes);
+  DYHIP_CHECK_HIP(hipMemset(dev->gemm_flags, 0, kGemmFlagWords * sizeof(unsigned)));
+  return DYHIP_OK;
+}
+
 int dyhip_device_create(int ordinal, const size_t pool_mb[4], dyhip_device** out) {
   DYHIP_REQUIRE(out != nullptr && pool_mb != nullptr, "null output pointer or pool sizes");
   int n = 0;
@@ -293,6 +301,8 @@ int dyhip_device_create(int ordinal, const size_t pool_mb[4], dyhip_device** out
   dev->gemm_ws = nullptr;
   dev->gemm_ws_bytes = 0;
   dev->wide_gemm_ready = 0;
+  dev->gemm_flags = nullptr;
+  dev->gemm_flags_used = false;
   dev->ln_scratch = nullptr;
   dev->stream_threshold = size_t(8) << 20;
   hipError_t e = hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking);
@@ -325,8 +335,9 @@ int dyhip_device_create(int ordinal, const size_t pool_mb[4], dyhip_device** out
   if (st == DYHIP_OK) st = ln_static_scratch_setup(dev);  // this device is current (hipSetDevice above)
   if (st == DYHIP_OK) {
     dev->gemm_ws_bytes = size_t(128) << 20;
-    dev->gemm_ws = dev->alloc->malloc(dev->gemm_ws_bytes);
+    dev->gemm_ws = dev->alloc->malloc(dev->gemm_ws_bytes + kGemmFlagWords * sizeof(unsigned));
     if (dev->gemm_ws == nullptr) st = fail(DYHIP_ERR_OUT_OF_MEMORY, "failed to allocate the GEMM split-K workspace");
+    else st = gemm_flags_setup(dev);
   }
   if (st != DYHIP_OK) {
     dyhip_device_destroy(dev);
@@ -355,12 +366,18 @@ int dyhip_device_fork(dyhip_device* parent, dyhip_device** out) {
   }
   (void)hipEventCreate(&dev->ev_start);
   (void)hipEventCreate(&dev->ev_stop);
-  dev->gemm_ws = parent->alloc->malloc(dev->gemm_ws_bytes);
+  dev->gemm_flags = nullptr;
+  dev->gemm_flags_used = false;
+  dev->gemm_ws = parent->alloc->malloc(dev->gemm_ws_bytes + kGemmFlagWords * sizeof(unsigned));
   dev->rng_state = static_cast<uint64_t*>(parent->alloc->malloc(256));
   dev->rng_stream = ++parent->forks_made;
   if (dev->gemm_ws == nullptr || dev->rng_state == nullptr) {
     dyhip_device_destroy(dev);
     return fail(DYHIP_ERR_OUT_OF_MEMORY, "failed to allocate the workspace of the forked queue");
+  }
+  if (gemm_flags_setup(dev) != DYHIP_OK) {
+    dyhip_device_destroy(dev);
+    return DYHIP_ERR_RUNTIME;
   }
   // the queue draws from its own stream of the parent's generator (same key, own counter)
   hipError_t ce = hipMemcpy(dev->rng_state, parent->rng_state, 8, hipMemcpyDeviceToDevice);
@@ -433,6 +450,17 @@ int dyhip_device_destroy(dyhip_device* dev) {
 int dyhip_device_sync(dyhip_device* dev) {
   DYHIP_CHECK_DEV(dev);
   DYHIP_CHECK_HIP(hipStreamSynchronize(dev->stream));
+  if (dev->gemm_flags_used) {
+    // the 256 x 256-tile GEMM counts the blocks that gave up waiting for another block's partial tile
+    dev->gemm_flags_used = false;
+    unsigned gave_up = 0;
+    DYHIP_CHECK_HIP(hipMemcpy(&gave_up, dev->gemm_flags + kGemmFlagWords - 1, sizeof(unsigned), hipMemcpyDeviceToHost));
+    if (gave_up != 0) {
+      (void)hipMemset(dev->gemm_flags, 0, kGemmFlagWords * sizeof(unsigned));
+      return fail(DYHIP_ERR_RUNTIME, "GEMM: %u blocks gave up waiting for a partial tile; the products since the last "
+                                     "synchronisation are incomplete", gave_up);
+    }
+  }
   return DYHIP_OK;
 }
 

@@ -26,10 +26,25 @@
 // from there the stage just consumed is refilled two k-tiles ahead and the next k-tile's first fragments are fetched,
 // both under the remaining MFMAs.
 //
-// Work distribution.  Tiles beyond the last full round of one tile per CU would leave most CUs idle for a whole
-// round, so the k-tiles of those remaining tiles are dealt to the CUs in equal runs; a run that does not cover a
-// whole tile leaves a partial tile in the workspace, and a second kernel adds the partial tiles of each tile in run
-// order (deterministic, no atomics) and applies the epilogue.
+// Work distribution.  The tile count rarely divides the CU count, and a round of one tile per CU that is not full
+// leaves CUs idle for the whole round.  So the units of work are k-tiles: all k-tiles of all tiles, tile by tile, form
+// one sequence that is cut into one equal segment per CU, and a block walks its segment, loads running two k-tiles
+// ahead of the MFMAs straight across tile boundaries (the next tile's operands arrive under the stores of the one
+// just finished).  A tile that lies wholly inside a segment is written out by that block.  A tile cut by segment
+// boundaries is completed in one of two ways:
+//   * segments at least a tile long (more tiles than CUs): a tile is cut at most once.  The block that holds its later
+//     k-tiles (the start of its segment) leaves a partial tile in the workspace and raises a flag; the block that
+//     holds its first k-tiles (the end of its segment, hundreds of microseconds later) adds that partial tile to its
+//     own, applies the epilogue and stores.  No second kernel, no float atomics, a fixed order of additions.
+//     Segments are dealt in descending block order, so a block only ever waits for a block dispatched before it,
+//     which itself waits for nobody before it raises its flag; the wait is bounded anyway, and a wait that gave up is
+//     counted and reported by dyhip_device_sync.
+//   * shorter segments (fewer tiles than CUs, or little more): a tile spans several segments, one CU adding all their
+//     partial tiles would take longer than its share of the product (256 KiB per partial tile at one CU's ~30 GB/s
+//     from beyond its L2), so every part goes to the workspace and a second kernel, 16 blocks per tile, adds them in
+//     segment order and applies the epilogue.
+// When the tiles are a whole number of rounds plus a few tile columns, the caller gives this kernel the leading
+// columns (whole rounds, nothing cut) and the rest to the 128-wide kernel.
 #include "gemm.h"
 
 namespace dyhip {
@@ -47,20 +62,23 @@ constexpr int kWK = 32;                   // k-tile
 constexpr int kStageFloats = 16384;       // 64 KiB
 constexpr size_t kWideLdsBytes = sizeof(float) * 2 * kStageFloats;
 constexpr size_t kSlotFloats = size_t(kWT) * kWT;
+constexpr unsigned kWideMinSegment = 8;  // k-tiles per block below which the kernel is not used
 
 struct WideArgs {
   const float* A;
   const float* B;
   float* C;
-  const float* bias;      // C = bias[m] + sum when set (beta unused)
-  float* slots;           // partial tiles [slot][256 n][256 m]
+  const float* bias;    // C = bias[m] + sum when set (beta unused)
+  float* slots;         // partial tiles, [32][512 threads][4] in the order the threads hold them: slot = segment when
+                        // tiles are finished in the kernel, else 2 x segment + (0: the segment's first item, 1: its last)
+  unsigned* flags;      // one per segment, zero between launches; the last of the kGemmFlagWords counts waits that gave up
   unsigned lda, ldb;
   unsigned M, N;
-  unsigned nt;            // k-tiles
+  unsigned nt;          // k-tiles of a tile
   unsigned tiles_m;
-  unsigned direct_tiles;  // tiles [0, direct_tiles) are computed whole, one per block
-  unsigned rem_units;     // k-tiles of the remaining tiles, dealt to the blocks that follow in runs of `per`
-  unsigned per;
+  unsigned units;       // tiles x nt, dealt to the blocks in equal segments
+  unsigned spin_limit;  // polls (about a microsecond apart) before a wait for another block gives up
+  int finish_in_kernel; // a cut tile is finished by the block that holds its first k-tiles; else by the second kernel
   float beta;
 };
 
@@ -94,6 +112,16 @@ __device__ __forceinline__ void load_chunks(const float* __restrict__ base, cons
 #define DYHIP_LOAD_CHUNK(u)                                                                                        \
   __builtin_amdgcn_global_load_lds((global_ptr_t)(base + off[u] - (I0 + u * 1024) / 4), (lds_ptr_t)wave_stage, 16, \
                                    I0 + u * 1024, 0);
+  DYHIP_LOAD_CHUNK(0) DYHIP_LOAD_CHUNK(1) DYHIP_LOAD_CHUNK(2) DYHIP_LOAD_CHUNK(3)
+#undef DYHIP_LOAD_CHUNK
+}
+
+// the same with the four global addresses formed ahead of time (biased back by the instruction offset already)
+template <int OP>
+__device__ __forceinline__ void load_chunks_at(const float* const (&ptr)[4], float* wave_stage) {
+  constexpr int I0 = OP == 0 ? -4096 : 0;
+#define DYHIP_LOAD_CHUNK(u) \
+  __builtin_amdgcn_global_load_lds((global_ptr_t)(ptr[u]), (lds_ptr_t)wave_stage, 16, I0 + u * 1024, 0);
   DYHIP_LOAD_CHUNK(0) DYHIP_LOAD_CHUNK(1) DYHIP_LOAD_CHUNK(2) DYHIP_LOAD_CHUNK(3)
 #undef DYHIP_LOAD_CHUNK
 }
@@ -133,6 +161,30 @@ __device__ __forceinline__ void read_b(float (&b)[4][2], const float* __restrict
   }
 }
 
+// Values that blocks on different L2s hand to each other inside one launch go past those caches (each L2 serves one
+// eighth of the chip and does not see the others' lines).
+__device__ __forceinline__ void store_through(float* p, float x, float y, float z, float w) {
+  unsigned long long* q = reinterpret_cast<unsigned long long*>(p);
+  __hip_atomic_store(q, (unsigned long long)__float_as_uint(x) | ((unsigned long long)__float_as_uint(y) << 32),
+                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  __hip_atomic_store(q + 1, (unsigned long long)__float_as_uint(z) | ((unsigned long long)__float_as_uint(w) << 32),
+                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+__device__ __forceinline__ float4 load_through(const float* p) {
+  const unsigned long long* q = reinterpret_cast<const unsigned long long*>(p);
+  const unsigned long long lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  const unsigned long long hi = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  return make_float4(__uint_as_float(unsigned(lo)), __uint_as_float(unsigned(lo >> 32)), __uint_as_float(unsigned(hi)),
+                     __uint_as_float(unsigned(hi >> 32)));
+}
+
+// first unit of segment s when `units` k-tiles are dealt to `segments` blocks: floor(s * units / segments) in 32-bit
+// arithmetic (segments <= 65536)
+__device__ __forceinline__ unsigned segment_start(unsigned s, unsigned units, unsigned segments) {
+  const unsigned q = units / segments, rm = units - q * segments;
+  return s * q + s * rm / segments;
+}
+
 // AK: A(m,k) = A[k + m*lda], else A[m + k*lda].  BKM: B(k,n) = B[k + n*ldb], else B[n + k*ldb].
 template <bool AK, bool BKM>
 __global__ __launch_bounds__(kWideThreads, 1) void gemm_wide_kernel(WideArgs g) {
@@ -149,23 +201,67 @@ __global__ __launch_bounds__(kWideThreads, 1) void gemm_wide_kernel(WideArgs g) 
   const unsigned nt = g.nt;
   const size_t stepa = AK ? kWK : size_t(kWK) * g.lda, stepb = BKM ? kWK : size_t(kWK) * g.ldb;
 
-  // work of this block: one whole tile, or a run of k-tiles that may cross from one tile into the next
-  unsigned u0, u1, tile_base, run = 0;
-  if (blockIdx.x < g.direct_tiles) {
-    tile_base = blockIdx.x;
-    u0 = 0;
-    u1 = nt;
-  } else {
-    run = blockIdx.x - g.direct_tiles;
-    tile_base = g.direct_tiles;
-    u0 = run * g.per;
-    u1 = min(g.rem_units, u0 + g.per);
+  // this block's segment of the unit sequence (tile-major, k-tiles ascending inside a tile).  Segments are handed out
+  // in descending order of block index: the blocks that a block may have to wait for (below) have lower indices and
+  // were therefore dispatched before it.
+  const unsigned segments = gridDim.x, seg = segments - 1 - blockIdx.x;
+  const unsigned u0 = segment_start(seg, g.units, segments), u1 = segment_start(seg + 1, g.units, segments);
+  if (u0 == u1) return;
+
+  // Loads run two units ahead of the product, across tile boundaries (a unit two ahead lies in this tile or the next:
+  // a tile has at least two k-tiles), and repeat the segment's last unit at its end: unconditional loads and selects
+  // keep the loop one basic block.
+  const unsigned last = u1 - 1, tiles = g.units / nt;
+  unsigned offa[4], offb[4], offa_n[4], offb_n[4];
+  {
+    const unsigned t0 = u0 / nt;
+    load_offsets<AK>(offa_n, g.lda, (t0 % g.tiles_m) * kWT, g.M);
+    load_offsets<BKM>(offb_n, g.ldb, (t0 / g.tiles_m) * kWT, g.N);
   }
-  for (unsigned ti = u0 / nt; ti * nt < u1; ++ti) {
-    const unsigned tile = tile_base + ti;
-    const unsigned kt0 = max(u0, ti * nt) - ti * nt, kt1 = min(u1, (ti + 1) * nt) - ti * nt;
-    const unsigned tm = tile % g.tiles_m, tn = tile / g.tiles_m;
-    const unsigned m0 = tm * kWT, n0 = tn * kWT;
+  // DYHIP_WIDE_AIM forms the eight addresses of a unit's loads (early in a k-tile, under its MFMAs: in front of the
+  // loads themselves the arithmetic would hold up both wavefronts of a SIMD right after their barrier),
+  // DYHIP_WIDE_FIRE issues the loads.
+  const float *pa_[4], *pb_[4];
+#define DYHIP_WIDE_AIM(unit, ub)                                                        \
+  {                                                                                     \
+    const unsigned p_ = min((unit), last);                                              \
+    const bool nxt_ = p_ >= (ub) + nt;                                                  \
+    const unsigned kk_ = p_ - (ub) - (nxt_ ? nt : 0u);                                  \
+    _Pragma("unroll") for (int u_ = 0; u_ < 4; ++u_) {                                  \
+      pa_[u_] = g.A + kk_ * stepa + (nxt_ ? offa_n[u_] : offa[u_]) - (-4096 + u_ * 1024) / 4; \
+      pb_[u_] = g.B + kk_ * stepb + (nxt_ ? offb_n[u_] : offb[u_]) - (u_ * 1024) / 4;   \
+      asm volatile("" : "+v"(pa_[u_]), "+v"(pb_[u_]));                                  \
+    }                                                                                   \
+  }
+#define DYHIP_WIDE_FIRE(stage)         \
+  load_chunks_at<0>(pa_, (stage));     \
+  load_chunks_at<1>(pb_, (stage));
+  float a[2][4][4], b[2][4][2];
+  int buf = 0;
+
+  for (unsigned pos = u0; pos < u1;) {
+    const unsigned tile = pos / nt, ub = tile * nt, kt0 = pos - ub, kt1 = min(nt, u1 - ub);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      offa[u] = offa_n[u];
+      offb[u] = offb_n[u];
+    }
+    {
+      const unsigned tn_ = min(tile + 1, tiles - 1);
+      load_offsets<AK>(offa_n, g.lda, (tn_ % g.tiles_m) * kWT, g.M);
+      load_offsets<BKM>(offb_n, g.ldb, (tn_ / g.tiles_m) * kWT, g.N);
+    }
+    if (pos == u0) {
+      DYHIP_WIDE_AIM(pos, ub)
+      DYHIP_WIDE_FIRE(wave_stage)
+      DYHIP_WIDE_AIM(pos + 1, ub)
+      DYHIP_WIDE_FIRE(wave_stage + kStageFloats)
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+      __syncthreads();
+      read_a<AK>(a[0], lds + oa, 0, sw);
+      read_b<BKM>(b[0], lds + ob, 0, sw);
+    }
+    pos += kt1 - kt0;
     floatx16 acc[2][4];
 #pragma unroll
     for (int u = 0; u < 2; ++u)
@@ -173,25 +269,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void gemm_wide_kernel(WideArgs g) 
       for (int t = 0; t < 4; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[u][t][r] = 0.f;
-    unsigned offa[4], offb[4];
-    load_offsets<AK>(offa, g.lda, m0, g.M);
-    load_offsets<BKM>(offb, g.ldb, n0, g.N);
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): loads of the previous tile still on their way into LDS
-    __syncthreads();                     // and every wave has left its stages
-    {
-      const unsigned second = kt0 + 1 < kt1 ? kt0 + 1 : kt0;
-      load_chunks<0>(g.A + kt0 * stepa, offa, wave_stage);
-      load_chunks<1>(g.B + kt0 * stepb, offb, wave_stage);
-      load_chunks<0>(g.A + second * stepa, offa, wave_stage + kStageFloats);
-      load_chunks<1>(g.B + second * stepb, offb, wave_stage + kStageFloats);
-    }
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
-    float a[2][4][4], b[2][4][2];
-    read_a<AK>(a[0], lds + oa, 0, sw);
-    read_b<BKM>(b[0], lds + ob, 0, sw);
-    for (unsigned i = kt0; i < kt1; ++i) {
-      const int buf = (i - kt0) & 1;
+    for (unsigned i = kt0; i < kt1; ++i, buf ^= 1) {
       const float* la = lds + buf * kStageFloats + oa;
       const float* lb = lds + buf * kStageFloats + ob;
 #pragma unroll
@@ -212,12 +290,11 @@ __global__ __launch_bounds__(kWideThreads, 1) void gemm_wide_kernel(WideArgs g) 
         if (kg < 3) {
           read_a<AK>(a[cur ^ 1], la, kg + 1, sw);
           read_b<BKM>(b[cur ^ 1], lb, kg + 1, sw);
+          if (kg == 0) DYHIP_WIDE_AIM(ub + i + 2, ub)
         } else {
-          // refill this stage two k-tiles ahead (the last two iterations reload the last k-tile, unconditional loads
-          // keep the loop free of branches) and fetch the next k-tile's first fragments
-          const unsigned nx = i + 2 < kt1 ? i + 2 : kt1 - 1;
-          load_chunks<0>(g.A + nx * stepa, offa, wave_stage + buf * kStageFloats);
-          load_chunks<1>(g.B + nx * stepb, offb, wave_stage + buf * kStageFloats);
+          // refill this stage two units ahead and fetch the next unit's first fragments (after the block's last unit
+          // both are idle repeats)
+          DYHIP_WIDE_FIRE(wave_stage + buf * kStageFloats)
           read_a<AK>(a[0], lds + (buf ^ 1) * kStageFloats + oa, 0, sw);
           read_b<BKM>(b[0], lds + (buf ^ 1) * kStageFloats + ob, 0, sw);
         }
@@ -233,88 +310,176 @@ __global__ __launch_bounds__(kWideThreads, 1) void gemm_wide_kernel(WideArgs g) 
       }
     }
 
-    // write back.  acc[u][t][r] of lane l: m = AK ? 32 t + l%32 : 4 (l%32) + t (+ 128 wm),
-    // n = BKM ? 32 u + i : 2 i + u (+ 64 wn) with i = 8 (r/4) + 4 (l/32) + r%4
-    const bool whole = kt0 == 0 && kt1 == nt;
-    float* out = whole ? g.C + m0 + size_t(n0) * g.M : g.slots + size_t(run + ti) * kSlotFloats;
-    const unsigned ldo = whole ? g.M : kWT;
-    const unsigned mlim = whole ? g.M - m0 : kWT, nlim = whole ? g.N - n0 : kWT;
-    const float beta = whole && g.bias == nullptr ? g.beta : 0.f;
-    const bool add_bias = whole && g.bias != nullptr;
+    // the thread index as the compiler cannot see through: the addresses below are formed here, after the loop,
+    // instead of being computed ahead of it and parked in scratch memory
+    unsigned tid_e = threadIdx.x;
+    asm volatile("" : "+v"(tid_e));
+    // acc[u][t][r] of lane l: m = AK ? 32 t + l%32 : 4 (l%32) + t (+ 128 wm),
+    // n = BKM ? 32 u + i : 2 i + u (+ 64 wn) with i = 8 (r/4) + 4 (l/32) + r%4.
+    // A partial tile is stored as [u][r][thread][t]: one 128-bit access per thread and (u, r), whoever reads it.
+    if (kt0 > 0 || (kt1 < nt && !g.finish_in_kernel)) {
+      // Not the whole tile, and not this block's to finish: leave the partial tile in a slot.
+      if (g.finish_in_kernel) {
+        // past the L2, for a block on another one; the segment's flag goes up once memory has acknowledged every store
+        float* slot = g.slots + size_t(seg) * kSlotFloats + 4 * tid_e;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            store_through(slot + size_t(u * 16 + r) * (4 * kWideThreads), acc[u][0][r], acc[u][1][r], acc[u][2][r],
+                          acc[u][3][r]);
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        if (tid_e == 0) __hip_atomic_store(g.flags + seg, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      } else {
+        float* slot = g.slots + size_t(2 * seg + (tile == u0 / nt ? 0 : 1)) * kSlotFloats + 4 * tid_e;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            *reinterpret_cast<float4*>(slot + size_t(u * 16 + r) * (4 * kWideThreads)) =
+                make_float4(acc[u][0][r], acc[u][1][r], acc[u][2][r], acc[u][3][r]);
+      }
+      continue;
+    }
+    // This block holds the tile's first k-tiles (or all of them) and finishes the tile.  The segments that start inside
+    // the tile computed their partial tiles first thing, long ago by now; the wait is bounded all the same, and a wait
+    // that gives up is counted for the host to report.  Partial tiles are added in segment order.
+    unsigned s_end = seg + 1;
+    if (kt1 < nt) {
+      while (s_end < segments && segment_start(s_end, g.units, segments) < ub + nt) ++s_end;
+      if (tid_e == 0) {
+        for (unsigned s2 = seg + 1; s2 < s_end; ++s2) {
+          unsigned spins = 0;
+          while (__hip_atomic_load(g.flags + s2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u) {
+            if (spins++ >= g.spin_limit) {
+              atomicAdd(g.flags + kGemmFlagWords - 1, 1u);
+              break;
+            }
+            __builtin_amdgcn_s_sleep(32);
+          }
+          __hip_atomic_store(g.flags + s2, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+        }
+      }
+      __syncthreads();
+    }
+    const unsigned lane_e = tid_e & 63, wm_e = (tid_e >> 6) & 1, wn_e = tid_e >> 7, l32_e = lane_e & 31, lhi_e = lane_e >> 5;
+    const unsigned m0 = (tile % g.tiles_m) * kWT, n0 = (tile / g.tiles_m) * kWT;
+    float* out = g.C + m0 + size_t(n0) * g.M;
+    const unsigned mlim = g.M - m0, nlim = g.N - n0;
+    const float beta = g.bias == nullptr ? g.beta : 0.f;
+    const bool add_bias = g.bias != nullptr;
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int i = 8 * (r / 4) + 4 * lhi + (r % 4);
-        const unsigned n = wn * 64 + (BKM ? 32 * u + i : 2 * i + u);
-        if (n >= nlim) continue;
-        if (!AK) {
-          const unsigned m = wm * 128 + 4 * l32;
-          if (m >= mlim) continue;
-          float* p = out + m + size_t(n) * ldo;
-          float4 v = make_float4(acc[u][0][r], acc[u][1][r], acc[u][2][r], acc[u][3][r]);
-          if (add_bias) {
-            const float4 o = *reinterpret_cast<const float4*>(g.bias + m0 + m);
-            v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
-          } else if (beta != 0.f) {
-            const float4 o = *reinterpret_cast<const float4*>(p);
-            v.x += beta * o.x; v.y += beta * o.y; v.z += beta * o.z; v.w += beta * o.w;
-          }
-          *reinterpret_cast<float4*>(p) = v;
-        } else {
+      for (int r0 = 0; r0 < 16; r0 += 8) {
+        float4 v[8];
 #pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const unsigned m = wm * 128 + 32 * t + l32;
+        for (int q = 0; q < 8; ++q) v[q] = make_float4(acc[u][0][r0 + q], acc[u][1][r0 + q], acc[u][2][r0 + q], acc[u][3][r0 + q]);
+        for (unsigned s2 = seg + 1; s2 < s_end; ++s2) {  // eight loads in flight
+          const float* slot = g.slots + size_t(s2) * kSlotFloats + 4 * tid_e + size_t(u * 16 + r0) * (4 * kWideThreads);
+          float4 o[8];
+#pragma unroll
+          for (int q = 0; q < 8; ++q) o[q] = load_through(slot + size_t(q) * (4 * kWideThreads));
+#pragma unroll
+          for (int q = 0; q < 8; ++q) {
+            v[q].x += o[q].x; v[q].y += o[q].y; v[q].z += o[q].z; v[q].w += o[q].w;
+          }
+        }
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+          const int r = r0 + q;
+          const int i = 8 * (r / 4) + 4 * lhi_e + (r % 4);
+          const unsigned n = wn_e * 64 + (BKM ? 32 * u + i : 2 * i + u);
+          if (n >= nlim) continue;
+          if (!AK) {
+            const unsigned m = wm_e * 128 + 4 * l32_e;
             if (m >= mlim) continue;
-            float* p = out + m + size_t(n) * ldo;
-            float v = acc[u][t][r];
-            if (add_bias) v += g.bias[m0 + m];
-            else if (beta != 0.f) v += beta * *p;
-            *p = v;
+            float* p = out + m + size_t(n) * g.M;
+            float4 x = v[q];
+            if (add_bias) {
+              const float4 o = *reinterpret_cast<const float4*>(g.bias + m0 + m);
+              x.x += o.x; x.y += o.y; x.z += o.z; x.w += o.w;
+            } else if (beta != 0.f) {
+              const float4 o = *reinterpret_cast<const float4*>(p);
+              x.x += beta * o.x; x.y += beta * o.y; x.z += beta * o.z; x.w += beta * o.w;
+            }
+            *reinterpret_cast<float4*>(p) = x;
+          } else {
+            const float xs[4] = {v[q].x, v[q].y, v[q].z, v[q].w};
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+              const unsigned m = wm_e * 128 + 32 * t + l32_e;
+              if (m >= mlim) continue;
+              float* p = out + m + size_t(n) * g.M;
+              float x = xs[t];
+              if (add_bias) x += g.bias[m0 + m];
+              else if (beta != 0.f) x += beta * *p;
+              *p = x;
+            }
           }
         }
       }
   }
+#undef DYHIP_WIDE_AIM
+#undef DYHIP_WIDE_FIRE
 }
 
-// C tile = epilogue(sum of the partial tiles of its runs, in run order).  Block (x, y): 16 columns y of remaining
-// tile x, one thread per four consecutive m (scalar when M is not a multiple of 4).
-__global__ __launch_bounds__(256) void gemm_wide_fixup_kernel(WideArgs g) {
-  const unsigned nt = g.nt, ti = blockIdx.x;
-  const unsigned r0 = (ti * nt) / g.per, r1 = min(((ti + 1) * nt - 1) / g.per, (g.rem_units - 1) / g.per);
-  if (r0 == r1) return;  // one run had the whole tile and wrote it itself
-  const unsigned tile = g.direct_tiles + ti, tm = tile % g.tiles_m, tn = tile / g.tiles_m;
-  const unsigned ml = (threadIdx.x % 64) * 4, m = tm * kWT + ml;
-  const bool vec = g.M % 4 == 0;
+// Second kernel for products whose tiles span several segments each (fewer tiles than CUs, or little more): C tile =
+// epilogue(sum of the tile's partial tiles in segment order).  Block (x, y) takes tile x and two of its 32 (u, r)
+// groups, its threads standing for the threads of the main kernel (a partial tile is stored in their order).
+template <bool AK, bool BKM>
+__global__ __launch_bounds__(kWideThreads) void gemm_wide_fixup_kernel(WideArgs g, unsigned segments) {
+  const unsigned nt = g.nt, tile = blockIdx.x, ub = tile * nt;
+  // segments that hold k-tiles of this tile: s_lo holds its first, s_hi its last
+  unsigned s_lo = min(ub / (g.units / segments), segments - 1);
+  while (s_lo + 1 < segments && segment_start(s_lo + 1, g.units, segments) <= ub) ++s_lo;
+  while (segment_start(s_lo, g.units, segments) > ub) --s_lo;
+  unsigned s_hi = s_lo;
+  while (s_hi + 1 < segments && segment_start(s_hi + 1, g.units, segments) < ub + nt) ++s_hi;
+  if (s_lo == s_hi) return;  // one block had the whole tile and wrote it itself
+  const unsigned tid = threadIdx.x, lane = tid & 63, wm = (tid >> 6) & 1, wn = tid >> 7, l32 = lane & 31, lhi = lane >> 5;
+  const unsigned m0 = (tile % g.tiles_m) * kWT, n0 = (tile / g.tiles_m) * kWT;
+  float* out = g.C + m0 + size_t(n0) * g.M;
+  const unsigned mlim = g.M - m0, nlim = g.N - n0;
 #pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    const unsigned nl = blockIdx.y * 16 + (threadIdx.x / 64) * 4 + c, n = tn * kWT + nl;
-    if (m >= g.M || n >= g.N) continue;
-    const size_t e = ml + size_t(nl) * kWT;
-    float4 s = *reinterpret_cast<const float4*>(g.slots + size_t(r0 + ti) * kSlotFloats + e);
-    for (unsigned r = r0 + 1; r <= r1; ++r) {
-      const float4 v = *reinterpret_cast<const float4*>(g.slots + size_t(r + ti) * kSlotFloats + e);
-      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+  for (int j = 0; j < 2; ++j) {
+    const unsigned ur = blockIdx.y * 2 + j, u = ur / 16, r = ur % 16;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (unsigned s2 = s_lo; s2 <= s_hi; ++s2) {
+      // the tile is the first item of every segment but the one that holds its first k-tiles (unless that segment
+      // starts with it)
+      const unsigned first_tile = segment_start(s2, g.units, segments) / nt;
+      const float4 o = *reinterpret_cast<const float4*>(g.slots + size_t(2 * s2 + (first_tile == tile ? 0 : 1)) * kSlotFloats +
+                                                        size_t(ur) * (4 * kWideThreads) + 4 * tid);
+      v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
     }
-    float* p = g.C + m + size_t(n) * g.M;
-    float sv[4] = {s.x, s.y, s.z, s.w};
-    if (vec) {
+    const unsigned i = 8 * (r / 4) + 4 * lhi + (r % 4);
+    const unsigned n = wn * 64 + (BKM ? 32 * u + i : 2 * i + u);
+    if (n >= nlim) continue;
+    if (!AK) {
+      const unsigned m = wm * 128 + 4 * l32;
+      if (m >= mlim) continue;
+      float* p = out + m + size_t(n) * g.M;
       if (g.bias != nullptr) {
-        const float4 o = *reinterpret_cast<const float4*>(g.bias + m);
-        s.x += o.x; s.y += o.y; s.z += o.z; s.w += o.w;
+        const float4 o = *reinterpret_cast<const float4*>(g.bias + m0 + m);
+        v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
       } else if (g.beta != 0.f) {
         const float4 o = *reinterpret_cast<const float4*>(p);
-        s.x += g.beta * o.x; s.y += g.beta * o.y; s.z += g.beta * o.z; s.w += g.beta * o.w;
+        v.x += g.beta * o.x; v.y += g.beta * o.y; v.z += g.beta * o.z; v.w += g.beta * o.w;
       }
-      *reinterpret_cast<float4*>(p) = s;
+      *reinterpret_cast<float4*>(p) = v;
     } else {
+      const float xs[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        if (m + j >= g.M) break;
-        float v = sv[j];
-        if (g.bias != nullptr) v += g.bias[m + j];
-        else if (g.beta != 0.f) v += g.beta * p[j];
-        p[j] = v;
+      for (int t = 0; t < 4; ++t) {
+        const unsigned m = wm * 128 + 32 * t + l32;
+        if (m >= mlim) continue;
+        float* p = out + m + size_t(n) * g.M;
+        float x = xs[t];
+        if (g.bias != nullptr) x += g.bias[m0 + m];
+        else if (g.beta != 0.f) x += g.beta * *p;
+        *p = x;
       }
     }
   }
@@ -466,10 +631,11 @@ int launch_wide(dyhip_device* dev, const WideArgs& g, unsigned blocks, unsigned 
 
 }  // namespace
 
-// How the tiles are dealt to the blocks.  ok = false: leave the problem to the 128-wide kernel.
+// How the k-tiles are dealt to the blocks.  ok = false: leave the problem to the 128-wide kernel.
 struct WidePlan {
   bool ok;
-  unsigned tiles_m, nt, direct_tiles, rem, per, runs;
+  bool finish_in_kernel;  // segments at least a tile long: a tile is cut at most once, and finished inside the kernel
+  unsigned tiles_m, tiles, nt, units, segments;
 };
 
 static WidePlan plan_wide(const dyhip_device* dev, size_t M, size_t N, size_t K32) {
@@ -477,26 +643,15 @@ static WidePlan plan_wide(const dyhip_device* dev, size_t M, size_t N, size_t K3
   WidePlan p{};
   p.tiles_m = unsigned(cdiv<size_t>(M, kWT));
   p.nt = unsigned(K32 / kWK);
-  const unsigned tiles = p.tiles_m * unsigned(cdiv<size_t>(N, kWT));
-  p.direct_tiles = tiles / cus * cus;
-  p.rem = tiles - p.direct_tiles;
-  p.per = p.nt;
-  p.runs = p.rem;
-  if (p.rem > 0) {
-    const unsigned units = p.rem * p.nt, per = cdiv<unsigned>(units, cus), runs = cdiv<unsigned>(units, per);
-    // a run costs `per` k-tiles (~7.5 us each); a partial tile is written and read once more (~0.2 us over the GPU)
-    if (per + (runs + p.rem) / 40 < p.nt) {
-      p.per = per;
-      p.runs = runs;
-    }
-  }
-  // Measured against the 128-wide kernel: a block's set-up, its 256 KiB of output and the second kernel cost about
-  // three k-tiles, so runs must be long (a problem of fewer tiles than CUs is nothing but runs), and a cut remainder
-  // after full rounds pays only under deep tiles.
-  // A last round of whole tiles is only worth a round when it is mostly full.
-  const bool split = p.per < p.nt;
-  if (p.direct_tiles == 0) p.ok = split ? p.per >= 16 : p.nt >= 16 && p.rem * 4 >= cus * 3;
-  else p.ok = split ? p.nt >= 16 : p.nt >= 8 && (p.rem == 0 || p.rem * 4 >= cus * 3);
+  const size_t tiles = size_t(p.tiles_m) * cdiv<size_t>(N, kWT), units = tiles * p.nt;
+  p.tiles = unsigned(tiles);
+  p.units = unsigned(units);
+  p.segments = cus;
+  const size_t per = units / cus;
+  p.finish_in_kernel = per >= p.nt;
+  // Measured against the 128-wide kernel: a block's set-up, its share of partial tiles and of the second kernel cost
+  // about three k-tiles, so a problem of fewer tiles than CUs (nothing but cut tiles) needs long segments.
+  p.ok = units < (size_t(1) << 31) && (p.finish_in_kernel ? p.nt >= 8 : per >= 16);
   return p;
 }
 
@@ -513,7 +668,9 @@ bool gemm_wide_eligible(const dyhip_device* dev, bool a_kmajor, bool b_kmajor, s
   const size_t cus = dev->num_cus > 0 ? size_t(dev->num_cus) : 256;
   // edge tiles compute whole 256 x 256 tiles: ragged shapes stay with the 128-wide kernel
   if (double(M) * double(N) < 0.8 * double(tiles) * double(kSlotFloats)) return false;
-  if (dev->gemm_ws == nullptr || dev->gemm_ws_bytes < (2 * cus) * kSlotFloats * sizeof(float)) return false;
+  if (dev->gemm_ws == nullptr || dev->gemm_flags == nullptr || dev->gemm_ws_bytes < (2 * cus) * kSlotFloats * sizeof(float) ||
+      cus + 1 > size_t(kGemmFlagWords))
+    return false;
   return plan_wide(dev, M, N, K32).ok;
 }
 
@@ -522,7 +679,7 @@ size_t gemm_wide_whole_rounds_columns(const dyhip_device* dev, bool a_kmajor, bo
   const size_t cus = dev->num_cus > 0 ? size_t(dev->num_cus) : 256;
   const size_t tiles_m = cdiv<size_t>(M, kWT), tiles = tiles_m * cdiv<size_t>(N, kWT);
   const size_t direct = tiles / cus * cus;
-  if (direct == 0 || direct == tiles || direct % tiles_m != 0) return 0;
+  if (direct == 0 || direct == tiles || direct % tiles_m != 0 || tiles - direct > cus / 4) return 0;
   const size_t cols = direct / tiles_m * kWT;
   return cols < N && gemm_wide_eligible(dev, a_kmajor, b_kmajor, M, cols, K, A, lda, B, ldb, C) ? cols : 0;
 }
@@ -536,26 +693,32 @@ int gemm_wide_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, siz
   g.C = C;
   g.bias = bias;
   g.slots = static_cast<float*>(dev->gemm_ws);
+  g.flags = dev->gemm_flags;
   g.lda = unsigned(lda);
   g.ldb = unsigned(ldb);
   g.M = unsigned(M);
   g.N = unsigned(N);
   g.nt = p.nt;
   g.tiles_m = p.tiles_m;
+  g.units = p.units;
+  g.finish_in_kernel = p.finish_in_kernel ? 1 : 0;
+  g.spin_limit = 1u << 22;  // seconds; a partial tile is normally there hundreds of microseconds before it is asked for
   g.beta = beta;
-  g.direct_tiles = p.direct_tiles;
-  g.rem_units = p.rem * p.nt;
-  g.per = p.per;
-  const unsigned blocks = p.direct_tiles + p.runs;
   int st;
-  if (a_kmajor && b_kmajor) st = launch_wide<true, true>(dev, g, blocks, 0);
-  else if (a_kmajor) st = launch_wide<true, false>(dev, g, blocks, 1);
-  else if (b_kmajor) st = launch_wide<false, true>(dev, g, blocks, 2);
-  else st = launch_wide<false, false>(dev, g, blocks, 3);
+  if (a_kmajor && b_kmajor) st = launch_wide<true, true>(dev, g, p.segments, 0);
+  else if (a_kmajor) st = launch_wide<true, false>(dev, g, p.segments, 1);
+  else if (b_kmajor) st = launch_wide<false, true>(dev, g, p.segments, 2);
+  else st = launch_wide<false, false>(dev, g, p.segments, 3);
   DYHIP_CHECK_STATUS(st);
   DYHIP_CHECK_LAUNCH();
-  if (g.per < g.nt) {
-    hipLaunchKernelGGL(gemm_wide_fixup_kernel, dim3(p.rem, kWT / 16), dim3(256), 0, dev->stream, g);
+  if (p.finish_in_kernel) {
+    dev->gemm_flags_used = true;
+  } else {
+    const dim3 grid(p.tiles, 16);
+    if (a_kmajor && b_kmajor) hipLaunchKernelGGL((gemm_wide_fixup_kernel<true, true>), grid, dim3(kWideThreads), 0, dev->stream, g, p.segments);
+    else if (a_kmajor) hipLaunchKernelGGL((gemm_wide_fixup_kernel<true, false>), grid, dim3(kWideThreads), 0, dev->stream, g, p.segments);
+    else if (b_kmajor) hipLaunchKernelGGL((gemm_wide_fixup_kernel<false, true>), grid, dim3(kWideThreads), 0, dev->stream, g, p.segments);
+    else hipLaunchKernelGGL((gemm_wide_fixup_kernel<false, false>), grid, dim3(kWideThreads), 0, dev->stream, g, p.segments);
     DYHIP_CHECK_LAUNCH();
   }
   return DYHIP_OK;

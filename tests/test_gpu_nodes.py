@@ -79,15 +79,18 @@ def test_gemm_nt_shallow(dev, M, N, K):
                  floor=np.sqrt(K))
 
 
-# Large outputs go to the 256 x 256-tile kernel: (a) fewer tiles than CUs, every tile cut into runs of k-tiles whose
-# partial tiles a second kernel adds, ragged edges and a depth that is not a multiple of 32 (the rest of the depth
-# is added by the 128-wide kernel); (b) one full round of whole tiles plus a remainder dealt in runs; (c) a
-# remainder too large to be worth cutting; (d) a transposed left operand whose row count is not a multiple of 4.
+# Large outputs go to the 256 x 256-tile kernel, which deals the k-tiles of all tiles to the CUs in equal segments:
+# (a) fewer tiles than CUs: every tile spans several segments, whose partial tiles a second kernel adds; ragged edges
+# and a depth that is not a multiple of 32 (the rest of the depth is added by the 128-wide kernel); (b), (c) a little
+# more than one tile, and about two shallow tiles, per CU: a cut tile is finished inside the kernel; (d) a transposed
+# left operand whose row count is not a multiple of 4.
 # Checked against the fp64 product of the same fp32 inputs (the oracle's triple loop is the same sum, too slow here).
 # (e) a shallow product whose leading 4096 columns are one full round of tiles: those go to the 256-wide kernel, the
 # other 384 columns run as a product of their own.
+# (f) more tiles than CUs with ragged edges and a depth remainder: every block finishes one cut tile from another
+# block's partial tile inside the kernel; (g) the cfg-5 output projection.
 WIDE_GEMM_SHAPES = [(1000, 1000, 8200), (4352, 4096, 512), (7936, 4096, 256), (1001, 1000, 8192), (2048, 2304, 2080),
-                    (4096, 4480, 264)]
+                    (4096, 4480, 264), (5000, 4400, 520), (10000, 4480, 1024)]
 
 
 @pytest.mark.parametrize("M,N,K", WIDE_GEMM_SHAPES)
@@ -105,6 +108,9 @@ def test_gemm_wide_tiles_three_forms(dev, M, N, K):
             yt = dev.tensor(y0)
             dev.gemm_nn(M, N, K, lt, rt, beta, yt)
             assert_close(yt.numpy(), beta * y0 + exact, FWD_RTOL, "wide gemm_nn beta=%g" % beta, floor=floor)
+        again = dev.tensor(y0)  # partial tiles are added in a fixed order: the same bits every time
+        dev.gemm_nn(M, N, K, lt, rt, 0.0, again)
+        assert again.numpy().tobytes() == yt.numpy().tobytes()
         r2 = f32(r.T)  # N x K column-major = (K, N) row-major
         yt = dev.tensor(y0)
         dev.gemm_nt_acc(M, N, K, lt, dev.tensor(r2), yt)
@@ -121,10 +127,10 @@ def test_gemm_wide_tiles_three_forms(dev, M, N, K):
 
 
 def test_gemm_wide_tiles_random_shapes(dev):
-    """Seeded random shapes of the four classes the planner of the 256 x 256-tile kernel tells apart -- fewer tiles
-    than CUs (nothing but runs of k-tiles, which end inside tiles), full rounds plus a remainder cut into runs, full
-    rounds plus leading-column split, full rounds plus a remainder large enough to run whole -- with ragged edges
-    and depths with and without a remainder of 32; all three forms against the fp64 product."""
+    """Seeded random shapes -- fewer tiles than CUs (every tile spans several segments of k-tiles; a second kernel
+    adds the parts), a little more than one tile per CU (a cut tile is finished inside the kernel), whole rounds plus
+    a few tile columns that run as a product of their own, many shallow tiles -- with ragged edges and depths with
+    and without a remainder of 32; all three forms against the fp64 product."""
     rng = np.random.default_rng(2024)
     r4 = lambda lo, hi: 4 * int(rng.integers(lo, hi))
     shapes = []
@@ -132,11 +138,11 @@ def test_gemm_wide_tiles_random_shapes(dev):
         a, b = int(rng.integers(2, 5)), int(rng.integers(2, 5))
         nt = -(-4096 // (a * b)) + int(rng.integers(0, 8))
         shapes.append((256 * a - r4(0, 10), 256 * b - r4(0, 10), 32 * nt + r4(0, 8)))
-    for _ in range(2):  # one round and a few tile columns more, cut into runs
+    for _ in range(2):  # one round and a few tile columns more
         shapes.append((256 * 17 - r4(0, 10), 256 * int(rng.integers(17, 19)) - r4(0, 10), 32 * int(rng.integers(16, 22)) + r4(0, 8)))
     for _ in range(2):  # one exact round of tile columns and some columns more
         shapes.append((4096, 4096 + r4(10, 100), 32 * int(rng.integers(8, 12)) + r4(0, 8)))
-    shapes.append((256 * 19 - r4(0, 10), 256 * 24 - r4(0, 10), 256 + r4(0, 8)))  # 456 tiles: the last 200 run whole
+    shapes.append((256 * 19 - r4(0, 10), 256 * 24 - r4(0, 10), 256 + r4(0, 8)))  # 456 tiles of 8 k-tiles
     taken = set()
     for M, N, K in shapes:
         kind = dev.gemm_uses_wide_tiles(0, 0, M, N, K)
