@@ -56,6 +56,9 @@ int dyhip_device_count(int* count);
 /* pool_mb[4] = FXS, DEDFS, PS, SCS sizes in MiB (DeviceMempoolSizes, devices.cc:17-57) */
 int dyhip_device_create(int ordinal, const size_t pool_mb[4], dyhip_device** out);
 int dyhip_device_destroy(dyhip_device* dev);
+/* Waits for everything queued on the device.  Also the point where a failure inside an earlier asynchronous launch
+ * surfaces: DYHIP_ERR_RUNTIME if blocks of a large GEMM gave up waiting for each other's partial tiles (their bounded
+ * wait, seconds long, ran out), in which case the products since the last synchronisation are incomplete. */
 int dyhip_device_sync(dyhip_device* dev);
 int dyhip_device_ordinal(const dyhip_device* dev, int* ordinal);
 int dyhip_device_stream(dyhip_device* dev, void** hip_stream);
