@@ -27,17 +27,44 @@ __global__ void clip_scale_kernel(unsigned n, const float* __restrict__ sqnorms,
   if (norm != nullptr) *norm = gg;
 }
 
-template <bool CLEAR>
+// p -= (lr * gscale / wd) * g over one slab, optionally clearing g in the same pass.  Four 128-bit groups per thread
+// and array in flight; streaming accesses when the slab is far larger than the caches (it is read and written once).
+template <bool CLEAR, bool NT>
 __global__ __launch_bounds__(256) void sgd_scaled_kernel(size_t n4, size_t n, float* __restrict__ p,
                                                          float* __restrict__ g, float lr, float wd,
                                                          const float* __restrict__ gscale) {
+  constexpr int U = 4;
   const float gs = *gscale;
   const bool skip = gs == 0.f;  // non-finite gradient norm: the parameters stay as they are
   const float s = lr * gs / wd;
-  const size_t stride = size_t(gridDim.x) * 256;
   float4* p4 = reinterpret_cast<float4*>(p);
   float4* g4 = reinterpret_cast<float4*>(g);
-  for (size_t i = size_t(blockIdx.x) * 256 + threadIdx.x; i < n4; i += stride) {
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  const size_t chunks = n4 / (256 * U);  // whole chunks of 256 * U groups, dealt to the blocks in turn
+  for (size_t c = blockIdx.x; c < chunks; c += gridDim.x) {
+    const size_t i = c * (256 * U) + threadIdx.x;
+    if (!skip) {
+      float4 pv[U], gv[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        pv[u] = ldg4<NT>(p4 + i + 256 * u);
+        gv[u] = ldg4<NT>(g4 + i + 256 * u);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        pv[u].x -= gv[u].x * s;
+        pv[u].y -= gv[u].y * s;
+        pv[u].z -= gv[u].z * s;
+        pv[u].w -= gv[u].w * s;
+        stg4<NT>(p4 + i + 256 * u, pv[u]);
+      }
+    }
+    if (CLEAR) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) stg4<NT>(g4 + i + 256 * u, zero);
+    }
+  }
+  for (size_t i = chunks * (256 * U) + size_t(blockIdx.x) * 256 + threadIdx.x; i < n4; i += size_t(gridDim.x) * 256) {
     if (!skip) {
       float4 pv = p4[i];
       const float4 gv = g4[i];
@@ -47,11 +74,11 @@ __global__ __launch_bounds__(256) void sgd_scaled_kernel(size_t n4, size_t n, fl
       pv.w -= gv.w * s;
       p4[i] = pv;
     }
-    if (CLEAR) g4[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (CLEAR) g4[i] = zero;
   }
-  for (size_t i = (n4 << 2) + size_t(blockIdx.x) * 256 + threadIdx.x; i < n; i += stride) {
-    if (!skip) p[i] -= g[i] * s;
-    if (CLEAR) g[i] = 0.f;
+  for (size_t k = (n4 << 2) + size_t(blockIdx.x) * 256 + threadIdx.x; k < n; k += size_t(gridDim.x) * 256) {
+    if (!skip) p[k] -= g[k] * s;
+    if (CLEAR) g[k] = 0.f;
   }
 }
 
@@ -126,13 +153,20 @@ int dyhip_sgd_update_scaled(dyhip_device* dev, size_t n, float* p, float* g, flo
   DYHIP_REQUIRE(wd != 0.f, "weight decay scale must be non-zero");
   const bool vec = aligned16(p) && aligned16(g);
   const size_t n4 = vec ? n / 4 : 0;
-  unsigned blocks = static_cast<unsigned>(cdiv<size_t>(n, size_t(256) * 16));
-  if (blocks < 1) blocks = 1;
-  if (blocks > 4096) blocks = 4096;
-  if (clear_grad)
-    hipLaunchKernelGGL(sgd_scaled_kernel<true>, dim3(blocks), dim3(256), 0, dev->stream, n4, n, p, g, lr, wd, gscale);
-  else
-    hipLaunchKernelGGL(sgd_scaled_kernel<false>, dim3(blocks), dim3(256), 0, dev->stream, n4, n, p, g, lr, wd, gscale);
+  // a block takes whole chunks of 256 x 4 groups in turn: as many blocks as give each the same number of chunks
+  const size_t chunks = cdiv<size_t>(n, size_t(256) * 16), per = cdiv<size_t>(chunks, 2048);
+  const unsigned blocks = static_cast<unsigned>(cdiv<size_t>(chunks, per));
+  const bool nt = n * sizeof(float) >= dev->stream_threshold;
+#define DYHIP_SGD(CLEAR, NT) \
+  hipLaunchKernelGGL((sgd_scaled_kernel<CLEAR, NT>), dim3(blocks), dim3(256), 0, dev->stream, n4, n, p, g, lr, wd, gscale)
+  if (clear_grad) {
+    if (nt) DYHIP_SGD(true, true);
+    else DYHIP_SGD(true, false);
+  } else {
+    if (nt) DYHIP_SGD(false, true);
+    else DYHIP_SGD(false, false);
+  }
+#undef DYHIP_SGD
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }

@@ -1265,6 +1265,29 @@ def test_device_side_clipping_and_sparse_rows(dev):
         assert tt.numpy().tobytes() == before_t.tobytes()
 
 
+@pytest.mark.parametrize("n", [4 * 1024 * 3 + 5, 5_000_003])
+def test_sgd_update_of_a_large_slab(dev, n):
+    """The slab update's unrolled and streaming forms (whole chunks of 1024 groups of four, the remaining groups, the
+    last odd floats; 20 MB takes the streaming accesses), with and without clearing the gradient, and from an address
+    that is not 16-byte aligned: the oracle's p -= g * (lr * scale / wd), bit for bit."""
+    rng = np.random.default_rng(n)
+    for shift in (0, 1):
+        p, g = f32(rng.standard_normal(n + shift)), f32(rng.standard_normal(n + shift))
+        pt, gt = dev.tensor(p), dev.tensor(g)
+        scale = dev.tensor(np.array([0.37], F32))
+        pv, gv = pt.offset(shift, (n,)), gt.offset(shift, (n,))
+        want = orc.sgd_update(p[shift:].copy(), g[shift:], 0.1, 0.37, 1.0)
+        dev.sgd_update_scaled(n, pv, gv, 0.1, scale, 1.0, clear_grad=False)
+        assert pt.numpy()[shift:].tobytes() == want.tobytes() and gt.numpy().tobytes() == g.tobytes()
+        dev.sgd_update_scaled(n, pv, gv, 0.1, scale, 1.0, clear_grad=True)
+        assert pt.numpy()[shift:].tobytes() == orc.sgd_update(want.copy(), g[shift:], 0.1, 0.37, 1.0).tobytes()
+        assert not gt.numpy()[shift:].any() and gt.numpy()[:shift].tobytes() == g[:shift].tobytes()
+        assert pt.numpy()[:shift].tobytes() == p[:shift].tobytes()
+        for w in lib_pools():
+            dev.sync()
+            dev.free_pool(w)
+
+
 def test_zero_sized_calls_are_no_ops(dev):
     """Empty tensors (a batch of zero columns, zero ids, K = 0) must not launch anything or fail."""
     sentinel = f32(np.arange(8))
