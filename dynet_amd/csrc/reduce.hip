@@ -481,9 +481,21 @@ struct LnRow {
   float4 v[VPL], d[VPL], o[VPL];
 };
 
-template <int VPL, bool NT>
+// FULL: the row fills every lane's groups and pdx is set, so the loads are unconditional.  Loads inside branches
+// cannot be counted by the compiler, which then waits for everything in flight (the row fetched ahead included)
+// before the first use of any of them.
+template <int VPL, bool NT, bool FULL = false>
 __device__ __forceinline__ void ln_row_load(LnRow<VPL>& r, unsigned n4, int lane, const float4* __restrict__ px,
                                             const float4* __restrict__ pdy, const float4* __restrict__ pdx) {
+  if (FULL) {
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+      r.v[u] = ldg4<NT>(px + lane + 64 * u);
+      r.d[u] = ldg4<NT>(pdy + lane + 64 * u);
+      r.o[u] = ldg4<NT>(pdx + lane + 64 * u);
+    }
+    return;
+  }
 #pragma unroll
   for (int u = 0; u < VPL; ++u) {
     const unsigned idx = lane + 64 * u;
@@ -494,7 +506,9 @@ __device__ __forceinline__ void ln_row_load(LnRow<VPL>& r, unsigned n4, int lane
   }
 }
 
-template <int VPL, bool NT, int WAVES, bool PREFETCH>
+// FULL: n4 == 64 * VPL and dx is wanted (the usual case): no per-lane bounds, and the row fetched ahead is always a
+// valid one (the last iteration fetches its own row again), so the kernel's main loop has no branch around a load.
+template <int VPL, bool NT, int WAVES, bool PREFETCH, bool FULL = false>
 __global__ __launch_bounds__(64 * WAVES) void ln_bwd_wave_kernel(unsigned n4, unsigned bd,
                                                                       const float4* __restrict__ x,
                                                                       const float4* __restrict__ g,
@@ -517,79 +531,99 @@ __global__ __launch_bounds__(64 * WAVES) void ln_bwd_wave_kernel(unsigned n4, un
   const unsigned wave_count = gridDim.x * WAVES;
   unsigned row = blockIdx.x * WAVES + w;
   LnRow<VPL> cur, nxt;
-  if (PREFETCH && row < bd)
-    ln_row_load<VPL, NT>(cur, n4, lane, x + size_t(row) * n4, dEdf + size_t(row) * n4,
-                         dx ? dx + size_t(row) * n4 : nullptr);
-  while (row < bd) {
-    // the next row's loads are in flight while this row is reduced and written
-    const unsigned next = row + wave_count;
-    if (!PREFETCH)
-      ln_row_load<VPL, NT>(cur, n4, lane, x + size_t(row) * n4, dEdf + size_t(row) * n4,
-                           dx ? dx + size_t(row) * n4 : nullptr);
-    if (PREFETCH && next < bd)
-      ln_row_load<VPL, NT>(nxt, n4, lane, x + size_t(next) * n4, dEdf + size_t(next) * n4,
-                           dx ? dx + size_t(next) * n4 : nullptr);
-    float s = 0.f;
+  // one row: the row sums, dx, and this wave's dg / db partial sums
+  auto process = [&](const LnRow<VPL>& cur, unsigned row) __attribute__((always_inline)) {
+  float s = 0.f;
 #pragma unroll
-    for (int u = 0; u < VPL; ++u) s += (cur.v[u].x + cur.v[u].y) + (cur.v[u].z + cur.v[u].w);
-    const float mean = wave_sum(s) / fn;
-    float ss = 0.f;
+  for (int u = 0; u < VPL; ++u) s += (cur.v[u].x + cur.v[u].y) + (cur.v[u].z + cur.v[u].w);
+  const float mean = wave_sum(s) / fn;
+  float ss = 0.f;
 #pragma unroll
-    for (int u = 0; u < VPL; ++u) {
-      if (lane + 64 * u < n4) {
-        const float ax = cur.v[u].x - mean, ay = cur.v[u].y - mean, az = cur.v[u].z - mean, aw = cur.v[u].w - mean;
-        ss += (ax * ax + ay * ay) + (az * az + aw * aw);
-      }
+  for (int u = 0; u < VPL; ++u) {
+    if (FULL || lane + 64 * u < n4) {
+      const float ax = cur.v[u].x - mean, ay = cur.v[u].y - mean, az = cur.v[u].z - mean, aw = cur.v[u].w - mean;
+      ss += (ax * ax + ay * ay) + (az * az + aw * aw);
     }
-    const float sigma = sqrtf(wave_sum(ss) / fn);
-    const float rs = 1.0f / (kLnEps + sigma);  // one exact division per row
-    const float neg = -mean;
-    // row sums: sum dq*xc and sum dq, with dq = dy*g
-    float sxq = 0.f, sq = 0.f;
+  }
+  const float sigma = sqrtf(wave_sum(ss) / fn);
+  const float rs = 1.0f / (kLnEps + sigma);  // one exact division per row
+  const float neg = -mean;
+  // row sums: sum dq*xc and sum dq, with dq = dy*g
+  float sxq = 0.f, sq = 0.f;
 #pragma unroll
-    for (int u = 0; u < VPL; ++u) {
-      if (lane + 64 * u < n4) {
+  for (int u = 0; u < VPL; ++u) {
+    if (FULL || lane + 64 * u < n4) {
 #define DYHIP_LN_ROW(c)                                  \
   {                                                      \
-    const float xc = cur.v[u].c + neg;                   \
-    const float dq = cur.d[u].c * gg[u].c;               \
-    sxq = fmaf(dq, xc, sxq);                             \
-    sq += dq;                                            \
-    if (want_g) pdg[u].c = fmaf(cur.d[u].c, xc * rs, pdg[u].c); \
-    if (want_b) pdb[u].c += cur.d[u].c;                  \
+  const float xc = cur.v[u].c + neg;                   \
+  const float dq = cur.d[u].c * gg[u].c;               \
+  sxq = fmaf(dq, xc, sxq);                             \
+  sq += dq;                                            \
+  if (want_g) pdg[u].c = fmaf(cur.d[u].c, xc * rs, pdg[u].c); \
+  if (want_b) pdb[u].c += cur.d[u].c;                  \
   }
-        DYHIP_F4_EACH(DYHIP_LN_ROW)
+      DYHIP_F4_EACH(DYHIP_LN_ROW)
 #undef DYHIP_LN_ROW
-      }
     }
-    if (dx != nullptr) {
-      const float ds = -(wave_sum(sxq) * rs) * rs;   // CwiseQuotient: -sum dq/s^2 * xc
-      const float dmu = -(wave_sum(sq) * rs);        // Negate(CwiseSum): -sum dq/s
-      const float sb = ds / (2.f * sigma);           // StdDimension: d / (2*sigma)
-      const float c = 2.f / fn;
-      const float dmu_n = dmu / fn;
-      float4* pdx = dx + size_t(row) * n4;
+  }
+  if (FULL || dx != nullptr) {
+    const float ds = -(wave_sum(sxq) * rs) * rs;   // CwiseQuotient: -sum dq/s^2 * xc
+    const float dmu = -(wave_sum(sq) * rs);        // Negate(CwiseSum): -sum dq/s
+    const float sb = ds / (2.f * sigma);           // StdDimension: d / (2*sigma)
+    const float c = 2.f / fn;
+    const float dmu_n = dmu / fn;
+    float4* pdx = dx + size_t(row) * n4;
 #pragma unroll
-      for (int u = 0; u < VPL; ++u) {
-        const unsigned idx = lane + 64 * u;
-        if (idx < n4) {
-          float4 o = cur.o[u];
+    for (int u = 0; u < VPL; ++u) {
+      const unsigned idx = lane + 64 * u;
+      if (FULL || idx < n4) {
+        float4 o = cur.o[u];
 #define DYHIP_LN_DX(c_)                                            \
   {                                                                \
-    float acc = o.c_;                                              \
-    acc += c * (cur.v[u].c_ - mean) * sb;                          \
-    acc += (cur.d[u].c_ * gg[u].c_) * rs;                          \
-    acc += dmu_n;                                                  \
-    o.c_ = acc;                                                    \
+  float acc = o.c_;                                              \
+  acc += c * (cur.v[u].c_ - mean) * sb;                          \
+  acc += (cur.d[u].c_ * gg[u].c_) * rs;                          \
+  acc += dmu_n;                                                  \
+  o.c_ = acc;                                                    \
   }
-          DYHIP_F4_EACH(DYHIP_LN_DX)
+        DYHIP_F4_EACH(DYHIP_LN_DX)
 #undef DYHIP_LN_DX
-          stg4<NT>(pdx + idx, o);
-        }
+        stg4<NT>(pdx + idx, o);
       }
     }
-    if (PREFETCH && next < bd) cur = nxt;
-    row = next;
+  }
+  };
+  if (FULL) {
+    // Straight-line loads only: the row after this one is fetched before this one is reduced, and the last row is
+    // processed after the loop, so that no load sits inside a branch.  The row index is the same in every lane.
+    unsigned r = __builtin_amdgcn_readfirstlane(row);
+    if (r < bd) {
+      ln_row_load<VPL, NT, true>(cur, n4, lane, x + size_t(r) * n4, dEdf + size_t(r) * n4, dx + size_t(r) * n4);
+      for (unsigned next = r + wave_count; next < bd; next += wave_count) {
+        ln_row_load<VPL, NT, true>(nxt, n4, lane, x + size_t(next) * n4, dEdf + size_t(next) * n4, dx + size_t(next) * n4);
+        process(cur, r);
+        cur = nxt;
+        r = next;
+      }
+      process(cur, r);
+    }
+  } else {
+    if (PREFETCH && row < bd)
+      ln_row_load<VPL, NT>(cur, n4, lane, x + size_t(row) * n4, dEdf + size_t(row) * n4,
+                           dx ? dx + size_t(row) * n4 : nullptr);
+    while (row < bd) {
+      // the next row's loads are in flight while this row is reduced and written
+      const unsigned next = row + wave_count;
+      if (!PREFETCH)
+        ln_row_load<VPL, NT>(cur, n4, lane, x + size_t(row) * n4, dEdf + size_t(row) * n4,
+                             dx ? dx + size_t(row) * n4 : nullptr);
+      if (PREFETCH && next < bd)
+        ln_row_load<VPL, NT>(nxt, n4, lane, x + size_t(next) * n4, dEdf + size_t(next) * n4,
+                             dx ? dx + size_t(next) * n4 : nullptr);
+      process(cur, row);
+      if (PREFETCH && next < bd) cur = nxt;
+      row = next;
+    }
   }
   if (!want_g && !want_b) return;
   const unsigned n = n4 * 4;
@@ -1055,37 +1089,45 @@ int dyhip_layer_norm_backward(dyhip_device* dev, size_t n, unsigned bd, const fl
                 need, ws_bytes);
   if (ln_fast_ok(n, x, g, dEdf, dx)) {
     const unsigned n4 = static_cast<unsigned>(n / 4);
+    const unsigned waves = kLnWavesBwd;
     const unsigned blocks = ln_bwd_blocks(n, bd);
     float* part_dg = dg ? static_cast<float*>(ws) : nullptr;
     float* part_db = db ? static_cast<float*>(ws) + size_t(blocks) * n : nullptr;
-    const size_t lds = cols ? size_t(2) * kLnWavesBwd * n * sizeof(float) : 0;  // [dg | db][wave][n]
-    const dim3 grid(blocks), block(64 * kLnWavesBwd);
+    const size_t lds = cols ? size_t(2) * waves * n * sizeof(float) : 0;  // [dg | db][wave][n]
+    const dim3 grid(blocks), block(64 * waves);
     const float4 *x4 = reinterpret_cast<const float4*>(x), *g4 = reinterpret_cast<const float4*>(g),
                  *d4 = reinterpret_cast<const float4*>(dEdf);
     float4* dx4 = reinterpret_cast<float4*>(dx);
     const bool stream = n * size_t(bd) * sizeof(float) >= dev->stream_threshold;
+#define DYHIP_LN_BWD_LAUNCH(VPL, NT, WAVES, FULL)                                                           \
+  hipLaunchKernelGGL((ln_bwd_wave_kernel<VPL, NT, WAVES, true, FULL>), grid, block, lds, dev->stream, n4, bd, x4, g4, \
+                     d4, dx4, part_dg, part_db)
+#define DYHIP_LN_BWD_LDS(VPL, NT, WAVES, FULL)                                                              \
+  DYHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&ln_bwd_wave_kernel<VPL, NT, WAVES, true, FULL>), \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 128 << 10))
 #define DYHIP_LN_BWD(VPL)                                                                                  \
   do {                                                                                                     \
     static bool big_lds_ok = false;                                                                        \
     if (lds > (size_t(64) << 10) && !big_lds_ok) {                                                          \
-      DYHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&ln_bwd_wave_kernel<VPL, true, kLnWavesBwd, true>),   \
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, 128 << 10));          \
-      DYHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&ln_bwd_wave_kernel<VPL, false, kLnWavesBwd, true>),  \
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, 128 << 10));          \
+      DYHIP_LN_BWD_LDS(VPL, true, kLnWavesBwd, true);                                                      \
+      DYHIP_LN_BWD_LDS(VPL, false, kLnWavesBwd, true);                                                     \
+      DYHIP_LN_BWD_LDS(VPL, true, kLnWavesBwd, false);                                                     \
+      DYHIP_LN_BWD_LDS(VPL, false, kLnWavesBwd, false);                                                    \
       big_lds_ok = true;                                                                                   \
     }                                                                                                      \
-    if (stream)                                                                                            \
-      hipLaunchKernelGGL((ln_bwd_wave_kernel<VPL, true, kLnWavesBwd, true>), grid, block, lds, dev->stream, n4, bd, x4, g4, d4, dx4, \
-                         part_dg, part_db);                                                                \
-    else                                                                                                   \
-      hipLaunchKernelGGL((ln_bwd_wave_kernel<VPL, false, kLnWavesBwd, true>), grid, block, lds, dev->stream, n4, bd, x4, g4, d4, dx4, \
-                         part_dg, part_db);                                                                \
+    const bool full = dx4 != nullptr && n4 == 64u * VPL;                                                   \
+    if (stream && full) DYHIP_LN_BWD_LAUNCH(VPL, true, kLnWavesBwd, true);                            \
+    else if (stream) DYHIP_LN_BWD_LAUNCH(VPL, true, kLnWavesBwd, false);                                   \
+    else if (full) DYHIP_LN_BWD_LAUNCH(VPL, false, kLnWavesBwd, true);                                     \
+    else DYHIP_LN_BWD_LAUNCH(VPL, false, kLnWavesBwd, false);                                              \
   } while (0)
     if (n4 <= 64) DYHIP_LN_BWD(1);
     else if (n4 <= 128) DYHIP_LN_BWD(2);
     else if (n4 <= 256) DYHIP_LN_BWD(4);
     else DYHIP_LN_BWD(8);
 #undef DYHIP_LN_BWD
+#undef DYHIP_LN_BWD_LAUNCH
+#undef DYHIP_LN_BWD_LDS
     DYHIP_CHECK_LAUNCH();
     if (dg && db) launch_combine(dev, n, blocks, part_dg, dg, part_db, db, 1);
     else if (dg) launch_combine(dev, n, blocks, part_dg, dg, nullptr, nullptr, 1);
