@@ -39,16 +39,29 @@ struct EwArgs {
 // NIN: number of inputs read; ACC: also read the output (old value).
 // BMASK: bit k set => input k has batch 1 and is indexed by the in-batch offset.
 // U: 128-bit accesses per thread and stream; NT: stream with non-temporal accesses.
+// Whether a functor's kernels take the branch-free path for tiles that lie wholly inside the tensor.  Measured per
+// kernel on 4096 x 1024 floats (same GPU, same run): it helps the three-stream backward kernels (12.3 -> 12.1 us) and
+// the logistic (7.2 -> 6.7 us, whose loads the bounds checks had serialised), and costs the lightest one- and
+// two-stream kernels (rectify 6.2 -> 7.0 us, cmult 9.0 -> 9.8 us), which therefore keep the bounds-checked form.
+template <class F>
+struct EwStraightLoads {
+  static constexpr bool value = false;
+};
+
 template <int NIN, bool ACC, int BMASK, bool NT, int U, class F>
 struct EwTile {
   float4 v[NIN > 0 ? NIN : 1][U];
   float4 o[U];
 
+  // FULL: the whole tile lies inside the tensor.  Without the per-access bounds the loads are straight-line code;
+  // under a bound each load sits in a branch of its own, into which the compiler may pull part of the arithmetic
+  // (it did for the logistic), and then every load waits for the one before it.
+  template <bool FULL>
   __device__ __forceinline__ void load(const EwArgs& a, size_t base4, size_t j0, size_t n4) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const size_t j = j0 + size_t(u) * kEwThreads;
-      if (j < n4) {
+      if (FULL || j < n4) {
 #pragma unroll
         for (int k = 0; k < NIN; ++k) {
           const float4* p = reinterpret_cast<const float4*>(a.in[k]);
@@ -61,23 +74,34 @@ struct EwTile {
     }
   }
 
+  // Phases: every load of the tile, then all the arithmetic, then every store (scheduling barriers keep them apart:
+  // left alone the compiler stores each group as soon as its loads have arrived, and a tile whose reads and writes
+  // alternate measured 5-15 % slower on the one- and two-stream kernels).
+  template <bool FULL>
   __device__ __forceinline__ void compute_store(const EwArgs& a, size_t base4, size_t j0, size_t n4, const F& f) {
+    float4 r[U];
+    if (FULL) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const size_t j = j0 + size_t(u) * kEwThreads;
-      if (j < n4) {
+      if (FULL || j < n4) {
         const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
         const float4 x0 = NIN > 0 ? v[0][u] : z;
         const float4 x1 = NIN > 1 ? v[NIN > 1 ? 1 : 0][u] : z;
         const float4 x2 = NIN > 2 ? v[NIN > 2 ? 2 : 0][u] : z;
         const float4 od = ACC ? o[u] : z;
-        float4 r;
-        r.x = f(x0.x, x1.x, x2.x, od.x);
-        r.y = f(x0.y, x1.y, x2.y, od.y);
-        r.z = f(x0.z, x1.z, x2.z, od.z);
-        r.w = f(x0.w, x1.w, x2.w, od.w);
-        stg4<NT>(reinterpret_cast<float4*>(a.out) + base4 + j, r);
+        r[u].x = f(x0.x, x1.x, x2.x, od.x);
+        r[u].y = f(x0.y, x1.y, x2.y, od.y);
+        r[u].z = f(x0.z, x1.z, x2.z, od.z);
+        r[u].w = f(x0.w, x1.w, x2.w, od.w);
+        if (!FULL) stg4<NT>(reinterpret_cast<float4*>(a.out) + base4 + j, r[u]);
       }
+    }
+    if (FULL) {
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        stg4<NT>(reinterpret_cast<float4*>(a.out) + base4 + j0 + size_t(u) * kEwThreads, r[u]);
     }
   }
 };
@@ -91,8 +115,13 @@ __global__ __launch_bounds__(kEwThreads) void ew_vec4_kernel(EwArgs a, F f) {
   const size_t base4 = size_t(batch) * n4;
   const size_t j0 = size_t(tile) * (kEwThreads * U) + threadIdx.x;
   EwTile<NIN, ACC, BMASK, NT, U, F> t;
-  t.load(a, base4, j0, n4);
-  t.compute_store(a, base4, j0, n4, f);
+  if (EwStraightLoads<F>::value && size_t(tile + 1) * (kEwThreads * U) <= n4) {  // the same for every thread of the block
+    t.template load<true>(a, base4, j0, n4);
+    t.template compute_store<true>(a, base4, j0, n4, f);
+  } else {
+    t.template load<false>(a, base4, j0, n4);
+    t.template compute_store<false>(a, base4, j0, n4, f);
+  }
 }
 
 template <int NIN, bool ACC, int BMASK, class F>
@@ -263,6 +292,12 @@ static int pick_range(dyhip_device* dev, bool backward, size_t inner, size_t len
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
+
+template <> struct EwStraightLoads<LogisticPacketFwd> { static constexpr bool value = true; };
+template <> struct EwStraightLoads<TanhBwd> { static constexpr bool value = true; };
+template <> struct EwStraightLoads<LogisticBwd> { static constexpr bool value = true; };
+template <> struct EwStraightLoads<RectifyBwd> { static constexpr bool value = true; };
+template <> struct EwStraightLoads<AccMul2> { static constexpr bool value = true; };
 
 }  // namespace dyhip
 
