@@ -667,9 +667,18 @@ __global__ __launch_bounds__(256) void scatter_runs_kernel(unsigned n, unsigned 
           __syncthreads();
           if (last) {
             if (slot == 0 && cok) {
-              V tot = vload_through(partials + size_t(cf + s) * line_v + cin);
-              for (unsigned qq = 1; qq < P; ++qq)
-                tot = vadd(tot, vload_through(partials + size_t(cf + qq * S + s) * line_v + cin));
+              // sixteen partial sums in flight at a time (the loads go past the caches; issued one by one between
+              // the additions, each would be a round trip of its own), added in ascending part order
+              V tot = vzero<V>();
+              for (unsigned q0 = 0; q0 < P; q0 += 16) {
+                V part16[16];
+#pragma unroll
+                for (int u = 0; u < 16; ++u)
+                  part16[u] = vload_through(partials + size_t(cf + min(q0 + u, P - 1) * S + s) * line_v + cin);
+#pragma unroll
+                for (int u = 0; u < 16; ++u)
+                  if (q0 + u < P) tot = q0 + u == 0 ? part16[u] : vadd(tot, part16[u]);
+              }
               vstore<true>(grads + size_t(row) * dimv + c, vadd(old, tot));
             }
             if (t == 0) __hip_atomic_store(p.arrivals + cf + s, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -749,6 +758,10 @@ __global__ __launch_bounds__(256) void scatter_runs_kernel(unsigned n, unsigned 
         if (r == 0 && u < kChunk)
           old[u] = (cok && head[u] && id[u] < vocab) ? grads[size_t(id[u]) * dimv + c] : vzero<V>();
       }
+      // One explicit wait for the batch.  The loads sit in per-entry branches, so the compiler cannot count them and
+      // waits for everything in flight before each use of a loaded row: after the first finished run that includes
+      // the run's own store, and the stores of a group went out one acknowledged round trip at a time.
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
 #pragma unroll
       for (int u = 0; u < kBatch; ++u) {
         if (pos[u] != kNone) {
