@@ -163,19 +163,26 @@ __device__ __forceinline__ void read_b(float (&b)[4][2], const float* __restrict
 
 // Values that blocks on different L2s hand to each other inside one launch go past those caches (each L2 serves one
 // eighth of the chip and does not see the others' lines).
+// 128 bits per instruction, with the scope bits of a system-scope access (what the compiler emits for a relaxed
+// system-scope atomic, which it only offers up to 64 bits).  The compiler does not know that the loads are in flight:
+// wait_through() is the wait, and takes the loaded values through it so that no use can move in front of it.
+typedef float wide_v4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void store_through(float* p, float x, float y, float z, float w) {
-  unsigned long long* q = reinterpret_cast<unsigned long long*>(p);
-  __hip_atomic_store(q, (unsigned long long)__float_as_uint(x) | ((unsigned long long)__float_as_uint(y) << 32),
-                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-  __hip_atomic_store(q + 1, (unsigned long long)__float_as_uint(z) | ((unsigned long long)__float_as_uint(w) << 32),
-                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  const wide_v4 v = {x, y, z, w};
+  // the wait states that a store of more than 64 bits needs before its data registers may be written again are the
+  // compiler's to insert for its own stores; it does not look inside this one
+  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 2" : : "v"(p), "v"(v) : "memory");
 }
-__device__ __forceinline__ float4 load_through(const float* p) {
-  const unsigned long long* q = reinterpret_cast<const unsigned long long*>(p);
-  const unsigned long long lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-  const unsigned long long hi = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-  return make_float4(__uint_as_float(unsigned(lo)), __uint_as_float(unsigned(lo >> 32)), __uint_as_float(unsigned(hi)),
-                     __uint_as_float(unsigned(hi >> 32)));
+__device__ __forceinline__ wide_v4 load_through_issue(const float* p) {
+  wide_v4 v;
+  asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
+__device__ __forceinline__ void wait_through(wide_v4 (&v)[8]) {
+  asm volatile("s_waitcnt vmcnt(0)"
+               : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7])
+               :
+               : "memory");
 }
 
 // first unit of segment s when `units` k-tiles are dealt to `segments` blocks: floor(s * units / segments) in 32-bit
@@ -378,12 +385,13 @@ __global__ __launch_bounds__(kWideThreads, 1) void gemm_wide_kernel(WideArgs g) 
         for (int q = 0; q < 8; ++q) v[q] = make_float4(acc[u][0][r0 + q], acc[u][1][r0 + q], acc[u][2][r0 + q], acc[u][3][r0 + q]);
         for (unsigned s2 = seg + 1; s2 < s_end; ++s2) {  // eight loads in flight
           const float* slot = g.slots + size_t(s2) * kSlotFloats + 4 * tid_e + size_t(u * 16 + r0) * (4 * kWideThreads);
-          float4 o[8];
+          wide_v4 o[8];
 #pragma unroll
-          for (int q = 0; q < 8; ++q) o[q] = load_through(slot + size_t(q) * (4 * kWideThreads));
+          for (int q = 0; q < 8; ++q) o[q] = load_through_issue(slot + size_t(q) * (4 * kWideThreads));
+          wait_through(o);
 #pragma unroll
           for (int q = 0; q < 8; ++q) {
-            v[q].x += o[q].x; v[q].y += o[q].y; v[q].z += o[q].z; v[q].w += o[q].w;
+            v[q].x += o[q][0]; v[q].y += o[q][1]; v[q].z += o[q][2]; v[q].w += o[q][3];
           }
         }
 #pragma unroll
