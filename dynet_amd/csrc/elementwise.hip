@@ -39,13 +39,18 @@ struct EwArgs {
 // NIN: number of inputs read; ACC: also read the output (old value).
 // BMASK: bit k set => input k has batch 1 and is indexed by the in-batch offset.
 // U: 128-bit accesses per thread and stream; NT: stream with non-temporal accesses.
-// Whether a functor's kernels take the branch-free path for tiles that lie wholly inside the tensor.  Measured per
-// kernel on 4096 x 1024 floats (same GPU, same run): it helps the three-stream backward kernels (12.3 -> 12.1 us) and
-// the logistic (7.2 -> 6.7 us, whose loads the bounds checks had serialised), and costs the lightest one- and
-// two-stream kernels (rectify 6.2 -> 7.0 us, cmult 9.0 -> 9.8 us), which therefore keep the bounds-checked form.
+// Which form a functor's kernels take for tiles that lie wholly inside the tensor, chosen per kernel by measurement
+// on 4096 x 1024 floats (same GPU, same run; why the forms differ this way is not understood beyond the first point):
+//   0  the bounds-checked form.  Each load sits in a branch of its own, so the compiler cannot count what is in
+//      flight and waits for everything before each use: in effect every store waits for the one before it.
+//   1  branch-free, in three phases: every load, all the arithmetic, every store.  Best for the three-stream backward
+//      kernels (12.3 -> 12.1 us); costs the light forward kernels (rectify 6.2 -> 7.0 us, cmult 9.0 -> 9.8 us).
+//   2  as 1, and each store waits for the one before it.  Brings every one-stream forward kernel to the copy's own
+//      time whatever its arithmetic (tanh 6.8, logistic 7.2 (whose loads form 0 had serialised) -> 6.2 us); costs the
+//      others (backward 12.5 us, cmult 9.3 us).
 template <class F>
-struct EwStraightLoads {
-  static constexpr bool value = false;
+struct EwTileForm {
+  static constexpr int value = 0;
 };
 
 template <int NIN, bool ACC, int BMASK, bool NT, int U, class F>
@@ -100,8 +105,10 @@ struct EwTile {
     if (FULL) {
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int u = 0; u < U; ++u)
+      for (int u = 0; u < U; ++u) {
         stg4<NT>(reinterpret_cast<float4*>(a.out) + base4 + j0 + size_t(u) * kEwThreads, r[u]);
+        if (EwTileForm<F>::value == 2 && u + 1 < U) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+      }
     }
   }
 };
@@ -115,7 +122,7 @@ __global__ __launch_bounds__(kEwThreads) void ew_vec4_kernel(EwArgs a, F f) {
   const size_t base4 = size_t(batch) * n4;
   const size_t j0 = size_t(tile) * (kEwThreads * U) + threadIdx.x;
   EwTile<NIN, ACC, BMASK, NT, U, F> t;
-  if (EwStraightLoads<F>::value && size_t(tile + 1) * (kEwThreads * U) <= n4) {  // the same for every thread of the block
+  if (EwTileForm<F>::value != 0 && size_t(tile + 1) * (kEwThreads * U) <= n4) {  // the same for every thread of the block
     t.template load<true>(a, base4, j0, n4);
     t.template compute_store<true>(a, base4, j0, n4, f);
   } else {
@@ -293,11 +300,14 @@ static int pick_range(dyhip_device* dev, bool backward, size_t inner, size_t len
   return DYHIP_OK;
 }
 
-template <> struct EwStraightLoads<LogisticPacketFwd> { static constexpr bool value = true; };
-template <> struct EwStraightLoads<TanhBwd> { static constexpr bool value = true; };
-template <> struct EwStraightLoads<LogisticBwd> { static constexpr bool value = true; };
-template <> struct EwStraightLoads<RectifyBwd> { static constexpr bool value = true; };
-template <> struct EwStraightLoads<AccMul2> { static constexpr bool value = true; };
+template <> struct EwTileForm<TanhFwd> { static constexpr int value = 2; };
+template <> struct EwTileForm<LogisticPacketFwd> { static constexpr int value = 2; };
+template <> struct EwTileForm<LogisticScalarFwd> { static constexpr int value = 2; };
+template <> struct EwTileForm<RectifyFwd> { static constexpr int value = 2; };
+template <> struct EwTileForm<TanhBwd> { static constexpr int value = 1; };
+template <> struct EwTileForm<LogisticBwd> { static constexpr int value = 1; };
+template <> struct EwTileForm<RectifyBwd> { static constexpr int value = 1; };
+template <> struct EwTileForm<AccMul2> { static constexpr int value = 1; };
 
 }  // namespace dyhip
 
