@@ -398,7 +398,7 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
       (epi.kind == kEpiAxpby || (epi.kind == kEpiBias && epi.bias != nullptr && aligned16(epi.bias)))) {
     const GemmSeg& s0 = segs[0];
     // leading full rounds first: the 128-wide kernel finishes a few remaining tile columns (96 of its tiles) sooner
-    // than runs of k-tiles with their partial tiles do (4096x4480x512: 184 against 204 us)
+    // than one sequence of k-tiles over all tiles does (4096x4480x1024: 335 against 349 us)
     size_t cols = gemm_wide_whole_rounds_columns(dev, a_kmajor, b_kmajor, M, N, s0.K, s0.A, s0.lda, s0.B, s0.ldb, C);
     if (cols == 0 && gemm_wide_eligible(dev, a_kmajor, b_kmajor, M, N, s0.K, s0.A, s0.lda, s0.B, s0.ldb, C)) cols = N;
     if (cols > 0) {

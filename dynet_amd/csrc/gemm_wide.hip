@@ -62,7 +62,6 @@ constexpr int kWK = 32;                   // k-tile
 constexpr int kStageFloats = 16384;       // 64 KiB
 constexpr size_t kWideLdsBytes = sizeof(float) * 2 * kStageFloats;
 constexpr size_t kSlotFloats = size_t(kWT) * kWT;
-constexpr unsigned kWideMinSegment = 8;  // k-tiles per block below which the kernel is not used
 
 struct WideArgs {
   const float* A;
