@@ -586,6 +586,8 @@ int dyhip_graph_launch(dyhip_device* dev, dyhip_graph* graph) {
   DYHIP_CHECK_DEV(dev);
   DYHIP_REQUIRE(graph != nullptr, "null graph handle");
   DYHIP_CHECK_HIP(hipGraphLaunch(graph->exec, dev->stream));
+  // a recorded large GEMM runs again with every replay: the next synchronisation looks at its give-up counter
+  if (dev->wide_gemm_ready != 0) dev->gemm_flags_used = true;
   return DYHIP_OK;
 }
 
