@@ -522,7 +522,7 @@ __global__ __launch_bounds__(512) void lstm_step_bwd_kernel(unsigned H, unsigned
     const float4* pb0 = reinterpret_cast<const float4*>(dpre_next_p) + (size_t(2 * ct) * G + g_first) * 64 + lane;
     const float4* pb1 = pb0 + size_t(G) * 64;
     stepx4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
-    float4 a[2][4], b0[2][4], b1[2][4];
+    float4 a[3][4], b0[3][4], b1[3][4];
 #define BWD_LOAD(buf, grp)                                   \
   _Pragma("unroll") for (int u = 0; u < 4; ++u) {            \
     a[buf][u] = pa[size_t((grp) + u) * 64];                  \
@@ -539,14 +539,20 @@ __global__ __launch_bounds__(512) void lstm_step_bwd_kernel(unsigned H, unsigned
     BWD_MMA1(a[buf][u].w, b0[buf][u].w, acc0) BWD_MMA1(a[buf][u].w, b1[buf][u].w, acc1)         \
   }                                                                                             \
   __builtin_amdgcn_sched_barrier(0);
-    // eight groups a round: four are multiplied while the next four are in flight (the last round re-reads its own)
+    // Rounds of four groups through three register buffers: one is multiplied while the next two are in flight.  A
+    // wave's 3 KiB per group against 8 MFMAs is twice the forward kernel's bytes per MFMA cycle, about what a CU gets
+    // from its L2, so the bytes in flight, not the MFMAs, set the pace.  Loads past the quarter's end re-read its last
+    // round (unconditional: the compiler counts what is in flight only in straight-line code).
+    const unsigned last_round = gq - 4;
     BWD_LOAD(0, 0u)
-    for (unsigned g = 0; g < gq; g += 8) {
-      const unsigned nx = g + 8 < gq ? g + 8 : g;
-      BWD_LOAD(1, g + 4)
+    BWD_LOAD(1, min(4u, last_round))
+    for (unsigned g = 0; g < gq; g += 12) {
+      BWD_LOAD(2, min(g + 8, last_round))
       BWD_MMA(0)
-      BWD_LOAD(0, nx)
-      BWD_MMA(1)
+      BWD_LOAD(0, min(g + 12, last_round))
+      if (g + 4 < gq) { BWD_MMA(1) }
+      BWD_LOAD(1, min(g + 16, last_round))
+      if (g + 8 < gq) { BWD_MMA(2) }
     }
 #undef BWD_LOAD
 #undef BWD_MMA1
