@@ -63,6 +63,9 @@ size_t gemm_wide_whole_rounds_columns(const dyhip_device* dev, bool a_kmajor, bo
 int gemm_wide_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N, size_t K32, const float* A,
                   size_t lda, const float* B, size_t ldb, float* C, float beta, const float* bias);
 
+void gemm_wide_describe(size_t M, size_t N, size_t K, unsigned segments, unsigned* starts, unsigned* k_tiles_per_tile,
+                        int* finish_in_kernel);
+
 // gemm_wide.hip: C[M x N] = beta*C + A[M x K] * B[N x K]^T for a depth of at most 128 (both operands contiguous
 // along the output index): operand tiles fetched whole, one latency per block.
 bool gemm_shallow_nt_eligible(const dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda,

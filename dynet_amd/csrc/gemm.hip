@@ -586,6 +586,15 @@ int dyhip_gemm_uses_wide_tiles(dyhip_device* dev, int trans_l, int trans_r, size
   return DYHIP_OK;
 }
 
+int dyhip_gemm_wide_segments(size_t M, size_t N, size_t K, unsigned segments, unsigned* starts,
+                             unsigned* k_tiles_per_tile, int* finish_in_kernel) {
+  DYHIP_REQUIRE(starts && k_tiles_per_tile && finish_in_kernel, "null output");
+  DYHIP_REQUIRE(segments >= 1 && segments <= 65536 && M >= 1 && N >= 1 && K >= 32, "bad shape or segment count");
+  DYHIP_REQUIRE(cdiv<size_t>(M, 256) * cdiv<size_t>(N, 256) * (K / 32) < (size_t(1) << 31), "too many k-tiles");
+  gemm_wide_describe(M, N, K, segments, starts, k_tiles_per_tile, finish_in_kernel);
+  return DYHIP_OK;
+}
+
 int dyhip_gemm_tn_acc(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float* y) {
   return dyhip_gemm_tn(dev, M, N, K, l, r, 1.0f, y);
 }

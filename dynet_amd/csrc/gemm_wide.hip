@@ -186,7 +186,7 @@ __device__ __forceinline__ void wait_through(wide_v4 (&v)[8]) {
 
 // first unit of segment s when `units` k-tiles are dealt to `segments` blocks: floor(s * units / segments) in 32-bit
 // arithmetic (segments <= 65536)
-__device__ __forceinline__ unsigned segment_start(unsigned s, unsigned units, unsigned segments) {
+__host__ __device__ __forceinline__ unsigned segment_start(unsigned s, unsigned units, unsigned segments) {
   const unsigned q = units / segments, rm = units - q * segments;
   return s * q + s * rm / segments;
 }
@@ -764,6 +764,18 @@ int gemm_shallow_nt_run(dyhip_device* dev, size_t M, size_t N, size_t K, const f
   hipLaunchKernelGGL(gemm_shallow_nt_kernel, dim3(blocks), dim3(kWideThreads), kShallowLdsBytes, dev->stream, g);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
+}
+
+// For tests of the hand-off between blocks without a GPU: the first unit of every segment (segments + 1 values, the
+// last one = units) when the k-tiles of an M x N x K product are dealt to `segments` blocks, and how cut tiles are
+// finished.  The same function as the kernels use.
+void gemm_wide_describe(size_t M, size_t N, size_t K, unsigned segments, unsigned* starts, unsigned* k_tiles_per_tile,
+                        int* finish_in_kernel) {
+  const unsigned nt = unsigned(K / kWK);
+  const size_t units = cdiv<size_t>(M, kWT) * cdiv<size_t>(N, kWT) * nt;
+  for (unsigned s2 = 0; s2 <= segments; ++s2) starts[s2] = segment_start(s2, unsigned(units), segments);
+  *k_tiles_per_tile = nt;
+  *finish_in_kernel = units / segments >= nt ? 1 : 0;
 }
 
 }  // namespace dyhip

@@ -359,6 +359,14 @@ class Device:
                                                C.byref(out)))
         return int(out.value)  # 0: no, 1: the whole product, 2: its leading full-round columns
 
+    @staticmethod
+    def gemm_wide_segments(M, N, K, segments):
+        """(starts, k_tiles_per_tile, finish_in_kernel) of the 256 x 256-tile GEMM's work distribution; needs no GPU."""
+        starts = (C.c_uint * (segments + 1))()
+        nt, fin = C.c_uint(0), C.c_int(0)
+        _check(cdll.dyhip_gemm_wide_segments(_sz(M), _sz(N), _sz(K), _u(segments), starts, C.byref(nt), C.byref(fin)))
+        return list(starts), int(nt.value), bool(fin.value)
+
     def gemm_tn_acc(self, M, N, K, l, r, y):
         _check(cdll.dyhip_gemm_tn_acc(self.handle, _sz(M), _sz(N), _sz(K), _p(l), _p(r), _p(y)))
 

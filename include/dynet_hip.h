@@ -240,6 +240,14 @@ int dyhip_gemm_nt_acc(dyhip_device* dev, size_t M, size_t N, size_t K, const flo
  * dyhip_gemm_strided_batched.  No counterpart in the reference (cuBLAS picks its kernels silently); for tests
  * and tuning. */
 int dyhip_gemm_uses_wide_tiles(dyhip_device* dev, int trans_l, int trans_r, size_t M, size_t N, size_t K, int* wide_tiles);
+/* How the 256 x 256-tile kernel deals an M x N x K product (K rounded down to a multiple of 32) to `segments`
+ * blocks: starts[s], s = 0..segments, is the first k-tile of block segment s in the sequence of all k-tiles of all
+ * tiles (tile by tile, k ascending; starts[segments] = their number), *k_tiles_per_tile the k-tiles of one tile, and
+ * *finish_in_kernel whether a tile cut by a segment boundary is finished inside the kernel (by the block that holds its
+ * first k-tiles, from the partial tiles of the blocks that hold the rest) or by a second kernel.  Needs no device.
+ * No counterpart in the reference; for tests of the hand-off's invariants. */
+int dyhip_gemm_wide_segments(size_t M, size_t N, size_t K, unsigned segments, unsigned* starts,
+                             unsigned* k_tiles_per_tile, int* finish_in_kernel);
 /* The cublasSgemmStridedBatched branches of the three shims (dynet/matrix-multiply.h:27-34, 110-117,
  * 175-182), taken when the left operand is batched: for b in [0, batch)
  *   y_b[MxN] = beta*y_b + op(l_b) * op(r_b),   x_b = x + b*stride_x (strides in floats),
