@@ -266,16 +266,32 @@ __global__ __launch_bounds__(kCellThreads) void lstm_cell_bwd_kernel(unsigned H,
 constexpr int kStepPitchR = 33;  // partial-sum exchange: [row][col]
 typedef float stepx16 __attribute__((ext_vector_type(16)));
 
-// W is 4H x K column-major (Wh: K = H, Wx: K = the input size): gate-interleaved row tiles
+// W is 4H x K column-major (Wh: K = H, Wx: K = the input size): gate-interleaved row tiles.  A block packs the
+// tiles rt0 .. rt0 + 7 of one group of 8 k: for a gate and a k their 64 units are one 256-byte run of W, which goes
+// through LDS ([gate][k][unit]) into the eight 1 KiB fragment groups (H is a multiple of 64).
 __global__ __launch_bounds__(256) void lstm_pack_weights_kernel(unsigned H, unsigned K, const float* __restrict__ W,
                                                                 float* __restrict__ Wp) {
-  const size_t o = size_t(blockIdx.x) * 256 + threadIdx.x;  // ((rt*(K/8) + kg)*64 + lane)*4 + s
-  if (o >= size_t(4) * H * K) return;
-  const unsigned s = o % 4, lane = (o / 4) % 64, l32 = lane % 32, lhi = lane / 32;
-  const size_t tg = o / 256;
-  const unsigned kg = tg % (K / 8), rt = tg / (K / 8);
-  const unsigned g = l32 / 8, u = l32 % 8, k = 8 * kg + 4 * lhi + s;
-  Wp[o] = W[size_t(g) * H + rt * 8 + u + size_t(k) * 4 * H];
+  __shared__ float tile[4 * 8 * 65];
+  const unsigned kg = blockIdx.x % (K / 8), rt0 = (blockIdx.x / (K / 8)) * 8;
+  const unsigned t = threadIdx.x;
+#pragma unroll
+  for (int pass = 0; pass < 8; ++pass) {
+    const unsigned pair = pass * 4 + t / 64, g = pair / 8, k = pair % 8, unit = t % 64;
+    tile[(g * 8 + k) * 65 + unit] = W[size_t(g) * H + rt0 * 8 + unit + size_t(8 * kg + k) * 4 * H];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const unsigned q = j * 256 + t, r = q / 64, lane = q % 64, l32 = lane % 32, lhi = lane / 32;
+    const unsigned g = l32 / 8, unit = r * 8 + l32 % 8;
+    float4 v;
+    v.x = tile[(g * 8 + 4 * lhi + 0) * 65 + unit];
+    v.y = tile[(g * 8 + 4 * lhi + 1) * 65 + unit];
+    v.z = tile[(g * 8 + 4 * lhi + 2) * 65 + unit];
+    v.w = tile[(g * 8 + 4 * lhi + 3) * 65 + unit];
+    float* dst = Wp + ((size_t(rt0 + r) * (K / 8) + kg) * 64 + lane) * 4;  // packed buffers are 16-byte aligned or not:
+    dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;              // four stores the compiler may merge
+  }
 }
 
 // Wh is 4H x H column-major; the packed matrix is Wh^T (H rows, depth 4H) in plain 32-row tiles
@@ -469,14 +485,22 @@ __global__ __launch_bounds__(256 * TILES) void lstm_step_fwd_kernel(unsigned H, 
 // fragment order (for the next launch), and dc_tm1.  Per block the product reads (16 + 32) x 4H floats, twice the
 // forward kernel's bytes per flop: 12.5 us for the bare product against 11.4 us forward, but one launch instead of
 // two and no slices through memory.
-__global__ void lstm_pack_transposed16_kernel(unsigned H, const float* __restrict__ W, float* __restrict__ Wp) {
-  const size_t o = size_t(blockIdx.x) * 256 + threadIdx.x;  // ((rt*(4H/16) + kg)*64 + lane)*4 + s
-  if (o >= size_t(4) * H * H) return;
-  const unsigned s = o % 4, lane = (o / 4) % 64, l16 = lane % 16, lq = lane / 16;
-  const size_t tg = o / 256;
+// One 128-bit group per thread: the four k of a lane's fragment are consecutive in Wh's column as well.  When the
+// operands are not 16-byte aligned the group is moved float by float.
+__global__ void lstm_pack_transposed16_kernel(unsigned H, const float* __restrict__ W, float* __restrict__ Wp, int vec) {
+  const size_t o4 = size_t(blockIdx.x) * 256 + threadIdx.x;  // (rt*(4H/16) + kg)*64 + lane
+  if (o4 >= size_t(H) * H) return;
+  const unsigned lane = o4 % 64, l16 = lane % 16, lq = lane / 16;
+  const size_t tg = o4 / 64;
   const unsigned G = H / 4, kg = tg % G, rt = tg / G;
-  const unsigned unit = rt * 16 + l16, k = 16 * kg + 4 * lq + s;
-  Wp[o] = W[k + size_t(unit) * 4 * H];  // Wh is 4H x H, column-major: Wh^T(unit, k) = Wh(k, unit)
+  const unsigned unit = rt * 16 + l16, k = 16 * kg + 4 * lq;
+  const float* src = W + k + size_t(unit) * 4 * H;  // Wh is 4H x H, column-major: Wh^T(unit, k) = Wh(k, unit)
+  if (vec) {
+    reinterpret_cast<float4*>(Wp)[o4] = *reinterpret_cast<const float4*>(src);
+  } else {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) Wp[o4 * 4 + q] = src[q];
+  }
 }
 
 __global__ void lstm_pack_state16_kernel(unsigned K, unsigned B, const float* __restrict__ v, float* __restrict__ vp) {
@@ -1120,8 +1144,7 @@ static int pack_weights(dyhip_device* dev, unsigned H, unsigned K, const float* 
                 "LSTM step: hidden size %u and product depth %u must be multiples of 128", H, K);
   DYHIP_REQUIRE(W && packed, "LSTM step: null tensor pointer");
   const size_t n = size_t(4) * H * K;
-  hipLaunchKernelGGL(lstm_pack_weights_kernel, dim3(unsigned(cdiv<size_t>(n, 256))), dim3(256), 0, dev->stream, H, K, W,
-                     packed);
+  hipLaunchKernelGGL(lstm_pack_weights_kernel, dim3(unsigned(n / 2048)), dim3(256), 0, dev->stream, H, K, W, packed);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
@@ -1164,8 +1187,8 @@ int dyhip_lstm_pack_recurrent_transposed16(dyhip_device* dev, unsigned H, const 
   DYHIP_REQUIRE(step_depth_ok(H) && size_t(4) * H * H < (size_t(1) << 32), "LSTM step: hidden size %u must be a multiple of 128", H);
   DYHIP_REQUIRE(Wh && packed, "LSTM step: null tensor pointer");
   const size_t n = size_t(4) * H * H;
-  hipLaunchKernelGGL(lstm_pack_transposed16_kernel, dim3(unsigned(cdiv<size_t>(n, 256))), dim3(256), 0, dev->stream, H, Wh,
-                     packed);
+  hipLaunchKernelGGL(lstm_pack_transposed16_kernel, dim3(unsigned(cdiv<size_t>(n / 4, 256))), dim3(256), 0, dev->stream, H,
+                     Wh, packed, aligned16(Wh) && aligned16(packed) ? 1 : 0);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
