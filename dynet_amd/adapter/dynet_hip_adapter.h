@@ -230,8 +230,13 @@ struct Node {
 // The executor calls backward once per differentiable argument with the same dEdf; the activation
 // derivative dpre = dEdf * act'(fx) (dynet/nodes-lstm.cc:358-361) is the same for all of them.  When the
 // node was given aux_mem (aux_storage_size() = one fx-sized tensor, requested by passing the output
-// dimension to the constructor), the first backward call stores dpre there and the others reuse it;
-// forward invalidates it.  Without aux_mem every call recomputes dpre.
+// dimension to the constructor), the first backward call of a backward pass stores dpre there and the
+// others reuse it.  A pass is recognised by the executor's own order: it visits the arguments of a node
+// in ascending order (dynet/exec.cc:247-262), so a call whose argument index does not exceed the last
+// one served starts a new pass -- the executor frees and refills pools[DEDFS] at the start of every
+// backward (dynet/exec.cc:178), so a second backward on the same forward can present the same dEdf
+// address with other contents.  forward invalidates the cache too.  Without aux_mem every call
+// recomputes dpre.
 struct VanillaLSTMGates : public Node {
   VanillaLSTMGates(bool dropout, real weightnoise_std, const Dim& dim = Dim())
       : dropout(dropout), weightnoise_std(weightnoise_std), dim(dim) {}
@@ -242,6 +247,7 @@ struct VanillaLSTMGates : public Node {
 
   void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
     dpre_of_ = nullptr;
+    last_i_ = -1;
     Args a = unpack(xs);
     size_t need = 0;
     abi_check(dyhip_lstm_gates_workspace(a.k, a.I, a.H, a.B, dropout, &need));
@@ -260,10 +266,11 @@ struct VanillaLSTMGates : public Node {
     void* ws = scratch(fx)->allocate(need);
     const float* dpre = nullptr;
     if (aux_mem != nullptr && dim.nd && dim.size() == fx.d.size()) {
-      if (dpre_of_ != dEdf.v) {
+      if (dpre_of_ != dEdf.v || int(i) <= last_i_) {
         abi_check(dyhip_lstm_gates_dpre(dev.hip, a.H, a.B, fx.v, dEdf.v, static_cast<float*>(aux_mem)));
         dpre_of_ = dEdf.v;
       }
+      last_i_ = int(i);
       dpre = static_cast<const float*>(aux_mem);
     }
     abi_check(dyhip_lstm_gates_backward(dev.hip, a.k, a.x.data(), a.xd.data(), a.H, a.B, xs[a.k]->v, xs[a.k + 1]->v,
@@ -274,6 +281,7 @@ struct VanillaLSTMGates : public Node {
 
  private:
   mutable const float* dpre_of_ = nullptr;  // the dEdf whose dpre sits in aux_mem
+  mutable int last_i_ = -1;                 // the argument served by the latest backward call
   struct Args {
     unsigned k, I, H, B, mx_bd, mh_bd;
     std::vector<const float*> x;

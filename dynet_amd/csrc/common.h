@@ -70,7 +70,9 @@ struct dyhip_device {
   size_t gemm_ws_bytes;
   unsigned wide_gemm_ready;  // gemm_wide.hip: kernels whose dynamic-LDS limit has been raised on this device
   unsigned* gemm_flags;      // gemm_wide.hip: kGemmFlagWords words behind gemm_ws that no other kernel touches, zero between launches
-  bool gemm_flags_used;      // a launch since the last dyhip_device_sync may have counted a wait that gave up
+  bool gemm_flags_used;      // a launch since the last host synchronisation may have counted a wait that gave up
+  unsigned gemm_spin_limit;  // polls before a block's wait for another block's partial tile gives up
+  int gemm_raise_flags;      // 0 only in tests of the give-up path: producers leave their flags down
   hipEvent_t ev_start, ev_stop;
   dyhip_device* parent;                // non-null for a forked queue: pools, scalars and allocator belong to the parent
   std::vector<hipEvent_t> sync_events; // ring of events recorded on this queue for dyhip_device_wait
@@ -85,6 +87,8 @@ struct dyhip_device {
 namespace dyhip {
 // reduce.hip: looks up, on the current device, the address of the static scratch array (once per device handle)
 int ln_static_scratch_setup(dyhip_device* dev);
+// device.hip: after a host synchronisation of dev's stream, reports waits that gave up inside a large GEMM
+int gemm_check_giveups(dyhip_device* dev);
 }  // namespace dyhip
 
 struct dyhip_graph {

@@ -150,6 +150,55 @@ static void pool_delete(dyhip_pool* pool) {
 
 using namespace dyhip;
 
+// The flag words of the 256 x 256-tile GEMM sit behind the split-K workspace, outside the size that other kernels
+// are told, and start out zero.
+// The fill runs on the queue's own stream (a non-blocking stream is not ordered against the null stream) and has
+// finished when the call returns.
+static int gemm_flags_clear(dyhip_device* dev) {
+  DYHIP_CHECK_HIP(hipMemsetAsync(dev->gemm_flags, 0, kGemmFlagWords * sizeof(unsigned), dev->stream));
+  DYHIP_CHECK_HIP(hipStreamSynchronize(dev->stream));
+  return DYHIP_OK;
+}
+
+static int gemm_flags_setup(dyhip_device* dev) {
+  dev->gemm_flags = reinterpret_cast<unsigned*>(static_cast<char*>(dev->gemm_ws) + dev->gemm_ws_bytes);
+  dev->gemm_spin_limit = 1u << 22;  // polls about a microsecond apart: seconds
+  dev->gemm_raise_flags = 1;
+  return gemm_flags_clear(dev);
+}
+
+// One queue's give-up counter; the queue's stream has been synchronised.
+static int gemm_giveups_of_queue(dyhip_device* q, unsigned* gave_up) {
+  *gave_up = 0;
+  if (!q->gemm_flags_used || q->gemm_flags == nullptr) return DYHIP_OK;
+  q->gemm_flags_used = false;
+  DYHIP_CHECK_HIP(hipMemcpyAsync(gave_up, q->gemm_flags + kGemmFlagWords - 1, sizeof(unsigned), hipMemcpyDeviceToHost,
+                                 q->stream));
+  DYHIP_CHECK_HIP(hipStreamSynchronize(q->stream));
+  // a waiter that gave up cleared a flag that its late producer raised afterwards: start the next launch clean
+  if (*gave_up != 0) DYHIP_CHECK_STATUS(gemm_flags_clear(q));
+  return DYHIP_OK;
+}
+
+// Called by every entry point that has just synchronised dev's stream and hands results to the host: turns waits
+// that gave up inside a 256 x 256-tile GEMM (on this queue, or on a queue forked from it: a graph launched here may
+// hold products recorded there) into an error.
+int dyhip::gemm_check_giveups(dyhip_device* dev) {
+  unsigned total = 0, n = 0;
+  DYHIP_CHECK_STATUS(gemm_giveups_of_queue(dev, &n));
+  total += n;
+  for (dyhip_device* f : dev->forks) {
+    if (!f->gemm_flags_used) continue;
+    DYHIP_CHECK_HIP(hipStreamSynchronize(f->stream));
+    DYHIP_CHECK_STATUS(gemm_giveups_of_queue(f, &n));
+    total += n;
+  }
+  if (total != 0)
+    return fail(DYHIP_ERR_RUNTIME, "GEMM: %u blocks gave up waiting for a partial tile; the products since the last "
+                                   "synchronisation are incomplete", total);
+  return DYHIP_OK;
+}
+
 extern "C" {
 
 const char* dyhip_last_error(void) { return g_last_error; }
@@ -264,14 +313,6 @@ int dyhip_device_count(int* count) {
     return fail(DYHIP_ERR_NO_DEVICE, "hipGetDeviceCount failed: %s", hipGetErrorString(e));
   }
   *count = n;
-  return DYHIP_OK;
-}
-
-// The flag words of the 256 x 256-tile GEMM sit behind the split-K workspace, outside the size that other kernels
-// are told, and start out zero.
-static int gemm_flags_setup(dyhip_device* dev) {
-  dev->gemm_flags = reinterpret_cast<unsigned*>(static_cast<char*>(dev->gemm_ws) + dev->gemm_ws_bytes);
-  DYHIP_CHECK_HIP(hipMemset(dev->gemm_flags, 0, kGemmFlagWords * sizeof(unsigned)));
   return DYHIP_OK;
 }
 
@@ -450,17 +491,13 @@ int dyhip_device_destroy(dyhip_device* dev) {
 int dyhip_device_sync(dyhip_device* dev) {
   DYHIP_CHECK_DEV(dev);
   DYHIP_CHECK_HIP(hipStreamSynchronize(dev->stream));
-  if (dev->gemm_flags_used) {
-    // the 256 x 256-tile GEMM counts the blocks that gave up waiting for another block's partial tile
-    dev->gemm_flags_used = false;
-    unsigned gave_up = 0;
-    DYHIP_CHECK_HIP(hipMemcpy(&gave_up, dev->gemm_flags + kGemmFlagWords - 1, sizeof(unsigned), hipMemcpyDeviceToHost));
-    if (gave_up != 0) {
-      (void)hipMemset(dev->gemm_flags, 0, kGemmFlagWords * sizeof(unsigned));
-      return fail(DYHIP_ERR_RUNTIME, "GEMM: %u blocks gave up waiting for a partial tile; the products since the last "
-                                     "synchronisation are incomplete", gave_up);
-    }
-  }
+  return gemm_check_giveups(dev);
+}
+
+int dyhip_device_set_gemm_handoff(dyhip_device* dev, unsigned spin_limit, int raise_flags) {
+  DYHIP_CHECK_DEV(dev);
+  dev->gemm_spin_limit = spin_limit;
+  dev->gemm_raise_flags = raise_flags ? 1 : 0;
   return DYHIP_OK;
 }
 
@@ -536,7 +573,7 @@ int dyhip_memcpy_d2h(dyhip_device* dev, void* dst_host, const void* src, size_t 
   DYHIP_REQUIRE(dst_host != nullptr && src != nullptr, "null pointer in d2h copy");
   DYHIP_CHECK_HIP(hipMemcpyAsync(dst_host, src, nbytes, hipMemcpyDeviceToHost, dev->stream));
   DYHIP_CHECK_HIP(hipStreamSynchronize(dev->stream));
-  return DYHIP_OK;
+  return gemm_check_giveups(dev);  // the bytes may be the output of a product that is incomplete
 }
 
 int dyhip_memcpy_d2d(dyhip_device* dev, void* dst, const void* src, size_t nbytes) {
@@ -586,8 +623,11 @@ int dyhip_graph_launch(dyhip_device* dev, dyhip_graph* graph) {
   DYHIP_CHECK_DEV(dev);
   DYHIP_REQUIRE(graph != nullptr, "null graph handle");
   DYHIP_CHECK_HIP(hipGraphLaunch(graph->exec, dev->stream));
-  // a recorded large GEMM runs again with every replay: the next synchronisation looks at its give-up counter
+  // a recorded large GEMM runs again with every replay, on this queue or on one forked from it: the next
+  // synchronisation looks at their give-up counters
   if (dev->wide_gemm_ready != 0) dev->gemm_flags_used = true;
+  for (dyhip_device* f : dev->forks)
+    if (f->wide_gemm_ready != 0) f->gemm_flags_used = true;
   return DYHIP_OK;
 }
 

@@ -77,6 +77,7 @@ struct WideArgs {
   unsigned tiles_m;
   unsigned units;       // tiles x nt, dealt to the blocks in equal segments
   unsigned spin_limit;  // polls (about a microsecond apart) before a wait for another block gives up
+  int raise_flags;      // 1; 0 only in tests of the give-up path (the partial tile is stored, its flag stays down)
   int finish_in_kernel; // a cut tile is finished by the block that holds its first k-tiles; else by the second kernel
   float beta;
 };
@@ -161,27 +162,25 @@ __device__ __forceinline__ void read_b(float (&b)[4][2], const float* __restrict
 }
 
 // Values that blocks on different L2s hand to each other inside one launch go past those caches (each L2 serves one
-// eighth of the chip and does not see the others' lines).
-// 128 bits per instruction, with the scope bits of a system-scope access (what the compiler emits for a relaxed
-// system-scope atomic, which it only offers up to 64 bits).  The compiler does not know that the loads are in flight:
-// wait_through() is the wait, and takes the loaded values through it so that no use can move in front of it.
+// eighth of the chip and does not see the others' lines): relaxed system-scope atomic accesses, which the compiler
+// offers up to 64 bits, two per 128-bit group.  They are ordinary accesses to the compiler: it counts them, waits for
+// them before their values are used and pads the stores' data registers itself.
 typedef float wide_v4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ unsigned long long pack_through(float lo, float hi) {
+  return (unsigned long long)__float_as_uint(lo) | ((unsigned long long)__float_as_uint(hi) << 32);
+}
 __device__ __forceinline__ void store_through(float* p, float x, float y, float z, float w) {
-  const wide_v4 v = {x, y, z, w};
-  // the wait states that a store of more than 64 bits needs before its data registers may be written again are the
-  // compiler's to insert for its own stores; it does not look inside this one
-  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 2" : : "v"(p), "v"(v) : "memory");
+  unsigned long long* q = reinterpret_cast<unsigned long long*>(p);
+  __hip_atomic_store(q, pack_through(x, y), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  __hip_atomic_store(q + 1, pack_through(z, w), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
-__device__ __forceinline__ wide_v4 load_through_issue(const float* p) {
-  wide_v4 v;
-  asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(v) : "v"(p) : "memory");
+__device__ __forceinline__ wide_v4 load_through(const float* p) {
+  const unsigned long long* q = reinterpret_cast<const unsigned long long*>(p);
+  const unsigned long long lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  const unsigned long long hi = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  const wide_v4 v = {__uint_as_float(unsigned(lo)), __uint_as_float(unsigned(lo >> 32)), __uint_as_float(unsigned(hi)),
+                     __uint_as_float(unsigned(hi >> 32))};
   return v;
-}
-__device__ __forceinline__ void wait_through(wide_v4 (&v)[8]) {
-  asm volatile("s_waitcnt vmcnt(0)"
-               : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7])
-               :
-               : "memory");
 }
 
 // first unit of segment s when `units` k-tiles are dealt to `segments` blocks: floor(s * units / segments) in 32-bit
@@ -336,7 +335,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void gemm_wide_kernel(WideArgs g) 
                           acc[u][3][r]);
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
-        if (tid_e == 0) __hip_atomic_store(g.flags + seg, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid_e == 0 && g.raise_flags) __hip_atomic_store(g.flags + seg, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       } else {
         float* slot = g.slots + size_t(2 * seg + (tile == u0 / nt ? 0 : 1)) * kSlotFloats + 4 * tid_e;
 #pragma unroll
@@ -386,8 +385,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void gemm_wide_kernel(WideArgs g) 
           const float* slot = g.slots + size_t(s2) * kSlotFloats + 4 * tid_e + size_t(u * 16 + r0) * (4 * kWideThreads);
           wide_v4 o[8];
 #pragma unroll
-          for (int q = 0; q < 8; ++q) o[q] = load_through_issue(slot + size_t(q) * (4 * kWideThreads));
-          wait_through(o);
+          for (int q = 0; q < 8; ++q) o[q] = load_through(slot + size_t(q) * (4 * kWideThreads));
 #pragma unroll
           for (int q = 0; q < 8; ++q) {
             v[q].x += o[q][0]; v[q].y += o[q][1]; v[q].z += o[q][2]; v[q].w += o[q][3];
@@ -709,7 +707,8 @@ int gemm_wide_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, siz
   g.tiles_m = p.tiles_m;
   g.units = p.units;
   g.finish_in_kernel = p.finish_in_kernel ? 1 : 0;
-  g.spin_limit = 1u << 22;  // seconds; a partial tile is normally there hundreds of microseconds before it is asked for
+  g.spin_limit = dev->gemm_spin_limit;  // seconds by default; a partial tile is normally there hundreds of microseconds before it is asked for
+  g.raise_flags = dev->gemm_raise_flags;
   g.beta = beta;
   int st;
   if (a_kmajor && b_kmajor) st = launch_wide<true, true>(dev, g, p.segments, 0);

@@ -881,7 +881,7 @@ int dyhip_lookup_plan_invalid_ids(dyhip_device* dev, unsigned n_ids, const void*
   plan_parts(plan, n_ids, &w);
   DYHIP_CHECK_HIP(hipMemcpyAsync(count, w.status, sizeof(unsigned), hipMemcpyDeviceToHost, dev->stream));
   DYHIP_CHECK_HIP(hipStreamSynchronize(dev->stream));
-  return DYHIP_OK;
+  return gemm_check_giveups(dev);
 }
 
 int dyhip_lookup_accumulate_grads_planned_workspace(unsigned n_ids, size_t dim, size_t* ws_bytes) {

@@ -1055,11 +1055,23 @@ int dyhip_layer_norm_forward(dyhip_device* dev, size_t n, unsigned bd, const flo
   return DYHIP_OK;
 }
 
+// Scratch of the backward pass by the path it takes: the register-resident kernels need one partial row of dg and of
+// db per block, the generic path per-row statistics and one partial row per output and batch split; nothing at all
+// when neither dg nor db is asked for.
+static size_t ln_bwd_ws_fast(size_t n, unsigned bd) { return size_t(2) * ln_bwd_blocks(n, bd) * n * sizeof(float); }
+static size_t ln_bwd_ws_generic(size_t n, unsigned bd) {
+  return ln_stats_bytes(bd) + size_t(2) * ln_cols_splits(n, bd ? bd : 1) * n * sizeof(float);
+}
+static size_t ln_bwd_ws_of_call(size_t n, unsigned bd, const float* x, const float* g, const float* dEdf, const float* dx,
+                                bool cols) {
+  if (!cols || bd == 0) return 0;
+  return ln_fast_ok(n, x, g, dEdf, dx) || ln_team_ok(n, x, g, dEdf, dx) ? ln_bwd_ws_fast(n, bd) : ln_bwd_ws_generic(n, bd);
+}
+
 int dyhip_layer_norm_backward_workspace(size_t n, unsigned bd, size_t* ws_bytes) {
   DYHIP_REQUIRE(ws_bytes != nullptr, "null output pointer");
-  const size_t fast = n <= 16384 ? size_t(2) * ln_bwd_blocks(n, bd) * n * sizeof(float) : 0;
-  // generic path: per-row statistics, then one partial row per output and batch split
-  const size_t generic = ln_stats_bytes(bd) + size_t(2) * ln_cols_splits(n, bd ? bd : 1) * n * sizeof(float);
+  // the pointers are not known here: enough for whichever path the call takes
+  const size_t fast = n <= 16384 ? ln_bwd_ws_fast(n, bd) : 0, generic = ln_bwd_ws_generic(n, bd);
   *ws_bytes = fast > generic ? fast : generic;
   return DYHIP_OK;
 }
@@ -1067,8 +1079,8 @@ int dyhip_layer_norm_backward_workspace(size_t n, unsigned bd, size_t* ws_bytes)
 int dyhip_layer_norm_backward_static(dyhip_device* dev, size_t n, unsigned bd, const float* x, const float* g,
                                      const float* dEdf, float* dx, float* dg, float* db) {
   DYHIP_CHECK_DEV(dev);
-  size_t need = 0;
-  DYHIP_CHECK_STATUS(dyhip_layer_norm_backward_workspace(n, bd, &need));
+  // what the path this call takes needs (its pointers are known here), not the larger of the two paths
+  const size_t need = ln_bwd_ws_of_call(n, bd, x, g, dEdf, dx, dg != nullptr || db != nullptr);
   DYHIP_REQUIRE(need <= size_t(DYHIP_LN_STATIC_SCRATCH_BYTES),
                 "layer_norm backward without a workspace is limited to %zu scratch bytes; n = %zu, bd = %u needs %zu",
                 size_t(DYHIP_LN_STATIC_SCRATCH_BYTES), n, bd, need);
@@ -1083,8 +1095,7 @@ int dyhip_layer_norm_backward(dyhip_device* dev, size_t n, unsigned bd, const fl
   DYHIP_REQUIRE(n >= 1 && x && g && dEdf, "layer_norm needs non-empty tensors");
   if (bd == 0 || (!dx && !dg && !db)) return DYHIP_OK;
   const bool cols = dg != nullptr || db != nullptr;
-  size_t need = 0;
-  DYHIP_CHECK_STATUS(dyhip_layer_norm_backward_workspace(n, bd, &need));
+  const size_t need = ln_bwd_ws_of_call(n, bd, x, g, dEdf, dx, cols);
   DYHIP_REQUIRE(!cols || (ws != nullptr && ws_bytes >= need), "layer_norm backward needs %zu workspace bytes, got %zu",
                 need, ws_bytes);
   if (ln_fast_ok(n, x, g, dEdf, dx)) {

@@ -13,9 +13,11 @@ namespace dyhip {
 
 static size_t align256(size_t n) { return (n + 255) / 256 * 256; }
 
-// A gradient norm that is NaN or infinite gives scale 0, which the update kernels below read as "leave the
-// parameters alone": Trainer::clip_gradients throws in that case (dynet/training.cc:176-180), a kernel cannot,
-// so the step is skipped on the device and the norm slot lets the host raise the error when it looks.
+// With clipping enabled (threshold > 0), a gradient norm that is NaN or infinite gives scale 0, which the update
+// kernels below read as "leave the parameters alone": Trainer::clip_gradients throws in that case
+// (dynet/training.cc:176-180), a kernel cannot, so the step is skipped on the device and the norm slot lets the host
+// raise the error when it looks.  With clipping disabled the reference neither looks at the norm nor throws
+// (dynet/training.cc:174 returns 1 before the check): the scale is 1 whatever the norm, as there.
 __global__ void clip_scale_kernel(unsigned n, const float* __restrict__ sqnorms, float threshold,
                                   float* __restrict__ gscale, float* __restrict__ norm) {
   if (threadIdx.x != 0 || blockIdx.x != 0) return;
@@ -23,7 +25,7 @@ __global__ void clip_scale_kernel(unsigned n, const float* __restrict__ sqnorms,
   for (unsigned i = 0; i < n; ++i) s += sqnorms[i];
   const float gg = sqrtf(s);
   const bool finite = gg - gg == 0.f;
-  *gscale = !finite ? 0.0f : (threshold > 0.f && gg > threshold) ? threshold / gg : 1.0f;
+  *gscale = !(threshold > 0.f) ? 1.0f : !finite ? 0.0f : gg > threshold ? threshold / gg : 1.0f;
   if (norm != nullptr) *norm = gg;
 }
 

@@ -152,6 +152,10 @@ class Device:
     def sync(self):
         _check(cdll.dyhip_device_sync(self.handle))
 
+    def set_gemm_handoff(self, spin_limit=1 << 22, raise_flags=True):
+        """Bounded wait of the large GEMM's hand-off between blocks (a test hook for its error path)."""
+        _check(cdll.dyhip_device_set_gemm_handoff(self.handle, _u(int(spin_limit)), _i(1 if raise_flags else 0)))
+
     def set_stream_threshold(self, nbytes):
         _check(cdll.dyhip_device_set_stream_threshold(self.handle, _sz(int(nbytes))))
 

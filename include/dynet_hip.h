@@ -56,10 +56,17 @@ int dyhip_device_count(int* count);
 /* pool_mb[4] = FXS, DEDFS, PS, SCS sizes in MiB (DeviceMempoolSizes, devices.cc:17-57) */
 int dyhip_device_create(int ordinal, const size_t pool_mb[4], dyhip_device** out);
 int dyhip_device_destroy(dyhip_device* dev);
-/* Waits for everything queued on the device.  Also the point where a failure inside an earlier asynchronous launch
+/* Waits for everything queued on the device.  Also a point where a failure inside an earlier asynchronous launch
  * surfaces: DYHIP_ERR_RUNTIME if blocks of a large GEMM gave up waiting for each other's partial tiles (their bounded
- * wait, seconds long, ran out), in which case the products since the last synchronisation are incomplete. */
+ * wait, seconds long, ran out), in which case the products since the last synchronisation are incomplete.  Every
+ * entry point that synchronises and hands device results to the host reports it the same way (dyhip_memcpy_d2h,
+ * dyhip_lookup_plan_invalid_ids), for the queue itself and for the queues forked from it. */
 int dyhip_device_sync(dyhip_device* dev);
+/* The bounded wait of that hand-off: spin_limit polls (about a microsecond apart; default 1 << 22) before a block gives
+ * up; raise_flags = 0 makes the producing blocks store their partial tiles without raising their flags, so that with
+ * spin_limit = 0 every consumer gives up at once while every kernel still runs to its end: the host-driven test of
+ * the error path.  Applies to products issued afterwards on this queue.  No counterpart in the reference. */
+int dyhip_device_set_gemm_handoff(dyhip_device* dev, unsigned spin_limit, int raise_flags);
 int dyhip_device_ordinal(const dyhip_device* dev, int* ordinal);
 int dyhip_device_stream(dyhip_device* dev, void** hip_stream);
 int dyhip_device_pool(dyhip_device* dev, int which, dyhip_pool** pool);
@@ -216,9 +223,11 @@ int dyhip_layer_norm_backward(dyhip_device* dev, size_t n, unsigned bd, const fl
  * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
  * reference (whose nodes take scratch from pools[SCS]).  The scratch is a static device array of
  * DYHIP_LN_STATIC_SCRATCH_BYTES that each GPU holds until the process ends; the call allocates nothing and
- * fails with DYHIP_ERR_INVALID_ARG when dyhip_layer_norm_backward_workspace(n, bd) exceeds that size
- * (rows of up to 2048 floats on the fast path: any bd; wider or unaligned rows: 8 bytes per row plus up
- * to 64 partial rows of dg and db).  All calls on one GPU share the array:
+ * fails with DYHIP_ERR_INVALID_ARG when the scratch that this call's path needs exceeds that size: nothing when
+ * dg and db are both NULL; rows of up to 2048 floats, a multiple of 4, 16-byte aligned: at most 256 partial
+ * rows of dg and db, any bd; such rows of up to 16384 floats: the same, so n = 4096 fits up to 128 blocks of
+ * rows; any other row: 8 bytes per row of the batch plus up to 64 partial rows of dg and db (never more than
+ * dyhip_layer_norm_backward_workspace(n, bd)).  All calls on one GPU share the array:
  * calls that overlap on one GPU (two queues, two threads) race; calls on one queue are ordered. */
 #define DYHIP_LN_STATIC_SCRATCH_BYTES (4u << 20)
 int dyhip_layer_norm_backward_static(dyhip_device* dev, size_t n, unsigned bd, const float* x, const float* g,
@@ -519,10 +528,12 @@ int dyhip_sgd_update(dyhip_device* dev, size_t n, float* p, const float* g, floa
  * sqrt(sum of the n squared norms)); threshold <= 0 disables clipping (gscale = 1). */
 int dyhip_clip_scale(dyhip_device* dev, unsigned n, const float* sqnorms, float threshold, float* gscale);
 /* The same, also storing the gradient norm in *norm (device, may be null).  Where the reference throws
- * "Magnitude of gradient is bad" for a NaN or infinite norm (dynet/training.cc:176-180), both forms set
- * *gscale = 0, and dyhip_sgd_update_scaled / dyhip_sgd_update_rows given a scale of 0 leave the parameters
- * untouched (gradients are still cleared): the diverged step is dropped on the device, and the host raises
- * the reference's error when it reads a non-finite *norm. */
+ * "Magnitude of gradient is bad" for a NaN or infinite norm (dynet/training.cc:176-180: only with clipping
+ * enabled, threshold > 0), both forms set *gscale = 0, and dyhip_sgd_update_scaled / dyhip_sgd_update_rows
+ * given a scale of 0 leave the parameters untouched (gradients are still cleared): the diverged step is dropped
+ * on the device.  Nothing else reports it: a caller that wants the reference's error must read the norm slot
+ * (this form) and raise it when the value is not finite.  With threshold <= 0 the scale is 1 whatever the norm,
+ * as in the reference (dynet/training.cc:174). */
 int dyhip_clip_scale_norm(dyhip_device* dev, unsigned n, const float* sqnorms, float threshold, float* gscale,
                           float* norm);
 /* the SGD rule with gscale read on the device; clear_grad != 0 also zeroes g (ParameterStorage::clear) */

@@ -224,6 +224,25 @@ static void lstm_node_gradients(Fixture& F) {
       cached.backward_dev_impl(F.dev, xs, fx, dEdf, i, g1);
       CHECK(as_vector(g0) == as_vector(g1));
     }
+    // a second backward pass on the same forward: the executor refills pools[DEDFS], so the same dEdf address
+    // comes back with other contents (dynet/exec.cc:178-208); the cached derivative must not be reused
+    g_case = "lstm_node_gates_bwd_second_pass_same_dEdf_address";
+    TensorTools::set_elements(dEdf, cycle(gd.size(), {-0.7f, 0.4f, 0.2f, -0.1f, 0.6f, 0.3f, -0.5f}));
+    for (unsigned i = 0; i < 5; ++i) {
+      Tensor g0 = F.zeros(a[i].d), g1 = F.zeros(a[i].d);
+      plain.backward_dev_impl(F.dev, xs, fx, dEdf, i, g0);
+      cached.backward_dev_impl(F.dev, xs, fx, dEdf, i, g1);
+      CHECK(as_vector(g0) == as_vector(g1));
+    }
+    // a pass that asks for some of the arguments only (needs_derivative), then a new one starting at a later index
+    TensorTools::set_elements(dEdf, cycle(gd.size(), {0.9f, -0.3f, 0.1f}));
+    for (unsigned i : {1u, 3u, 2u, 4u}) {  // 1, 3 = one pass; 2, 4 = the next (2 <= 3)
+      if (i == 2u) TensorTools::set_elements(dEdf, cycle(gd.size(), {0.2f, 0.8f, -0.6f, 0.5f}));
+      Tensor g0 = F.zeros(a[i].d), g1 = F.zeros(a[i].d);
+      plain.backward_dev_impl(F.dev, xs, fx, dEdf, i, g0);
+      cached.backward_dev_impl(F.dev, xs, fx, dEdf, i, g1);
+      CHECK(as_vector(g0) == as_vector(g1));
+    }
   }
   g_case = "lstm_node_gates_dropout_bwd";
   {

@@ -18,7 +18,7 @@ def _random_shapes():
             for _ in range(40)]
 
 
-@pytest.mark.parametrize("segments", [256, 304, 64])
+@pytest.mark.parametrize("segments", [256, 304, 64, 1, 2, 255, 257])
 @pytest.mark.parametrize("M,N,K", SHAPES + _random_shapes())
 def test_every_flag_is_raised_once_and_waited_for_once(M, N, K, segments):
     starts, nt, in_kernel = Device.gemm_wide_segments(M, N, K, segments)

@@ -168,6 +168,39 @@ def test_gemm_wide_tiles_random_shapes(dev):
     assert taken == {1, 2}
 
 
+def test_gemm_wide_give_up_is_reported_by_every_synchronising_call_and_leaves_clean_flags():
+    """The error path of the hand-off between blocks, forced from the host: producers store their partial tiles but
+    leave their flags down and the consumers' bounded wait is set to zero polls, so every cut tile's consumer gives
+    up at once and every kernel still runs to its end.  dyhip_device_sync and dyhip_memcpy_d2h must both report it,
+    and the next product (defaults restored) must be right: no stale flag."""
+    from dynet_amd import Device
+    from dynet_amd.device import DyhipError
+
+    d = Device(0, mem_mb=(512, 64, 64, 64))
+    try:
+        M, N, K = 4352, 4096, 512  # 272 tiles of 16 k-tiles on 256 segments: cut tiles are finished inside the kernel
+        assert d.gemm_uses_wide_tiles(0, 0, M, N, K) == 1
+        assert Device.gemm_wide_segments(M, N, K, 256)[2]
+        rng = np.random.default_rng(11)
+        l, r = f32(rng.standard_normal((K, M))), f32(rng.standard_normal((N, K)))
+        exact = r.astype(np.float64) @ l.astype(np.float64)
+        lt, rt, yt = d.tensor(l), d.tensor(r), d.empty((N, M))
+        d.set_gemm_handoff(0, False)
+        d.gemm_nn(M, N, K, lt, rt, 0.0, yt)
+        with pytest.raises(DyhipError, match="gave up"):
+            d.sync()
+        d.sync()  # reported once; the queue is usable again
+        d.gemm_nn(M, N, K, lt, rt, 0.0, yt)
+        with pytest.raises(DyhipError, match="gave up"):
+            yt.numpy()
+        d.set_gemm_handoff()
+        d.gemm_nn(M, N, K, lt, rt, 0.0, yt)
+        d.sync()
+        assert_close(yt.numpy(), exact, FWD_RTOL, "wide gemm after a reported give-up", floor=np.sqrt(K))
+    finally:
+        d.close()
+
+
 def test_gemm_wide_tiles_first_used_inside_a_graph_and_scaled_accumulate():
     """A device whose first large product is recorded into a graph (the kernel's dynamic-LDS opt-in then happens
     during the capture), replayed with eager work between the replays; and beta other than 0 or 1."""
@@ -1263,6 +1296,11 @@ def test_device_side_clipping_and_sparse_rows(dev):
         gt.set(np.full((vocab, dim), bad, F32))
         dev.sgd_update_rows(n, plan, dim, vocab, tt, gt, 0.1, scale, 1.0)
         assert tt.numpy().tobytes() == before_t.tobytes()
+        # clipping disabled: the reference does not look at the norm (dynet/training.cc:174), the scale is 1
+        for off in (0.0, -1.0):
+            dev.clip_scale(2, dev.tensor(np.array([1.0, bad], F32)), off, scale, norm)
+            assert scale.numpy()[0] == 1.0
+            assert np.isnan(norm.numpy()[0]) if np.isnan(bad) else np.isinf(norm.numpy()[0])
 
 
 @pytest.mark.parametrize("n", [4 * 1024 * 3 + 5, 5_000_003])
