@@ -64,6 +64,8 @@ def parse_args():
                     help="with --pmc-summary: distinct ids of the cfg-3 id vector (the bench prints it as unique_ids)")
     ap.add_argument("--no-extras", action="store_true", help="skip the cfg 1 / 3 / 4 kernel measurements")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="bound on the CPU-baseline leg")
+    ap.add_argument("--cpu-config-seconds", type=float, default=3.0,
+                    help="bound on each leg of the per-configuration CPU baseline (cfg 1, 3, 4 and the reduced cfg 5)")
     ap.add_argument("--no-lm", action="store_true", help="skip the cfg 5 LSTM-LM training-step measurement")
     ap.add_argument("--no-large", action="store_true", help="skip the 16x larger repeat of the cfg 2 sweep")
     ap.add_argument("--lm-steps", type=int, default=30)
@@ -760,6 +762,128 @@ def lm_kernels(reps, use_graph=True):
     return out
 
 
+class _OneCore:
+    """Pins the process to one host core for the duration (the CPU legs are single-threaded C)."""
+
+    def __enter__(self):
+        self.allowed, self.cpu = None, None
+        try:
+            self.allowed = sorted(os.sched_getaffinity(0))
+            self.cpu = self.allowed[len(self.allowed) // 2]
+            os.sched_setaffinity(0, {self.cpu})
+        except (AttributeError, OSError):
+            self.allowed = None
+        return self
+
+    def __exit__(self, *exc):
+        if self.allowed is not None:
+            os.sched_setaffinity(0, set(self.allowed))
+        return False
+
+
+def _time_cpu(fn, seconds, max_reps):
+    fn()
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        fn()
+        reps += 1
+        el = time.perf_counter() - t0
+        if el >= seconds or reps >= max_reps:
+            return el / reps, reps
+
+
+def cpu_baseline_per_config(seconds):
+    """The CPU oracle on configurations 1, 3, 4 at their full sizes and on a reduced configuration 5, each on one
+    pinned host core, the C functions called into preallocated outputs; `seconds` bounds each leg."""
+    import ctypes as C
+
+    from dynet_amd.synth import glorot, zipf_ids
+    from oracle import cpu_oracle as orc
+    from oracle import lm_oracle
+
+    L = orc._lib
+    rng = np.random.default_rng(0)
+    f = lambda a: np.ascontiguousarray(a, dtype=np.float32)  # noqa: E731
+    fp = lambda a: a.ctypes.data_as(C.POINTER(C.c_float))  # noqa: E731
+    up = lambda a: a.ctypes.data_as(C.POINTER(C.c_uint))  # noqa: E731
+    out = {"cores": 1, "kind": "port", "library": "oracle/libdynet_cpu_oracle.so"}
+    with _OneCore() as core:
+        out["pinned_to_cpu"] = core.cpu
+        # ---- cfg 1: VanillaLSTMGates + C + H, forward and every backward argument ------------------------------
+        I, H, B = 128, 256, 32
+        x, h, c, dh = (f(rng.standard_normal((B, d))) for d in (I, H, H, H))
+        Wx, Wh, b = f(glorot(rng, 4 * H, I)), f(glorot(rng, 4 * H, H)), np.zeros(4 * H, np.float32)
+        fx, c2, h2 = np.empty((B, 4 * H), np.float32), np.empty((B, H), np.float32), np.empty((B, H), np.float32)
+        dgates, dct, dcp = np.zeros((B, 4 * H), np.float32), np.zeros((B, H), np.float32), np.zeros((B, H), np.float32)
+        outs = [np.zeros(sh, np.float32) for sh in ((B, I), (B, H), (I, 4 * H), (H, 4 * H), (4 * H,))]
+        xs = (C.POINTER(C.c_float) * 1)(fp(x))
+        dims = (C.c_uint * 1)(I)
+        none = C.POINTER(C.c_float)()
+
+        def cell():
+            L.orc_lstm_gates_forward(1, xs, dims, H, B, fp(h), fp(Wx), fp(Wh), fp(b), none, 0, none, 0,
+                                     orc.LOGISTIC_PACKET, fp(fx))
+            L.orc_lstm_c_forward(H, B, fp(c), fp(fx), fp(c2))
+            L.orc_lstm_h_forward(H, B, fp(c2), fp(fx), fp(h2))
+            L.orc_lstm_h_backward(H, B, fp(c2), fp(fx), fp(dh), 0, fp(dct))
+            L.orc_lstm_h_backward(H, B, fp(c2), fp(fx), fp(dh), 1, fp(dgates))
+            L.orc_lstm_c_backward(H, B, fp(c), fp(fx), fp(dct), 0, fp(dcp))
+            L.orc_lstm_c_backward(H, B, fp(c), fp(fx), fp(dct), 1, fp(dgates))
+            for i, o in enumerate(outs):
+                L.orc_lstm_gates_backward(1, xs, dims, H, B, fp(h), fp(Wx), fp(Wh), none, 0, none, 0, fp(fx), fp(dgates),
+                                          i, fp(o))
+
+        dt, reps = _time_cpu(cell, seconds, 2000)
+        out["cfg1_lstm_cell"] = {"I": I, "H": H, "B": B, "fwd_bwd_us": round(dt * 1e6, 1), "reps": reps,
+                                 "what": "gates, C, H forward; H and C backward (both arguments); gates backward for all "
+                                         "five arguments, each recomputing the activation derivative as the reference does"}
+        # ---- cfg 3: gather + scatter-add -----------------------------------------------------------------------
+        V, D, n = CFG3["V"], CFG3["D"], CFG3["n"]
+        ids = np.ascontiguousarray(zipf_ids(rng, n, V), dtype=np.uint32)
+        table, g = f(rng.uniform(-0.1, 0.1, (V, D))), f(rng.standard_normal((n, D)))
+        fxl, grads = np.empty((n, D), np.float32), np.zeros((V, D), np.float32)
+        G, uniq = n * D * 4, int(np.unique(ids).size)
+        dt_g, r1 = _time_cpu(lambda: L.orc_lookup_forward(n, up(ids), C.c_size_t(D), V, fp(table), C.c_float(1.0), fp(fxl)),
+                             seconds / 2, 200)
+        dt_s, r2 = _time_cpu(lambda: L.orc_lookup_accumulate_grads(n, up(ids), C.c_size_t(D), V, fp(g), fp(grads)),
+                             seconds / 2, 200)
+        out["cfg3_lookup"] = {"vocab": V, "dim": D, "n_ids": n, "unique_ids": uniq,
+                              "gather_ms": round(dt_g * 1e3, 3), "gather_GBps": round((2 * G + 4 * n) / dt_g / 1e9, 2),
+                              "scatter_add_ms": round(dt_s * 1e3, 3),
+                              "scatter_add_GBps": round((G + 2 * uniq * D * 4) / dt_s / 1e9, 2), "reps": [r1, r2]}
+        del table, g, fxl, grads
+        # ---- cfg 4: PickNegLogSoftmax forward + backward -------------------------------------------------------
+        rows, bd = CFG4["rows"], CFG4["bd"]
+        xl = f(rng.standard_normal((bd, rows)) * 2)
+        labels = rng.integers(0, rows, bd).astype(np.uint32)
+        aux, err, dy = np.empty(3 * bd, np.float32), np.empty(bd, np.float32), f(rng.standard_normal(bd))
+        dxl = np.zeros((bd, rows), np.float32)
+        X = rows * bd * 4
+        vp = lambda a: a.ctypes.data_as(C.c_void_p)  # noqa: E731
+        dt_f, r1 = _time_cpu(lambda: L.orc_pnls_forward(C.c_size_t(rows), bd, fp(xl), up(labels), vp(aux), fp(err)),
+                             seconds / 2, 50)
+        dt_b, r2 = _time_cpu(lambda: L.orc_pnls_backward(C.c_size_t(rows), bd, fp(xl), vp(aux), fp(dy), fp(dxl)),
+                             seconds / 2, 50)
+        out["cfg4_pnls"] = {"rows": rows, "bd": bd, "fwd_ms": round(dt_f * 1e3, 2), "fwd_GBps": round(X / dt_f / 1e9, 2),
+                            "bwd_ms": round(dt_b * 1e3, 2), "bwd_GBps": round(3 * X / dt_b / 1e9, 2), "reps": [r1, r2]}
+        del xl, dxl
+        # ---- cfg 5 at a reduced size (the oracle's matrix products are plain triple loops) ----------------------
+        V5, E5, H5, L5, B5, T5 = 1000, 64, 128, 2, 16, 8
+        from dynet_amd.lm import LstmLM
+
+        params = LstmLM.init_params(V5, E5, H5, L5, seed=3)
+        tokens = zipf_ids(rng, (T5 + 1) * B5, V5).reshape(T5 + 1, B5).astype(np.uint32)
+        dt5, r5 = _time_cpu(lambda: lm_oracle.step(params, tokens, L5), seconds, 20)
+        flops = 3 * T5 * (2 * 4 * H5 * (E5 + H5) * B5 + 2 * 4 * H5 * (H5 + H5) * B5 + 2 * V5 * H5 * B5)
+        out["cfg5_lstm_lm_reduced"] = {
+            "V": V5, "E": E5, "H": H5, "layers": L5, "B": B5, "T": T5, "ms_per_step": round(dt5 * 1e3, 2),
+            "tokens_per_s": round(T5 * B5 / dt5, 1), "gemm_gflops": round(flops / dt5 / 1e9, 2), "reps": r5,
+            "note": "timed at this reduced size; the full configuration (V 10000, E 256, H 1024, B 128, T 35) has %.0f "
+                    "times the matrix-product work" % (3 * 35 * (2 * 4 * 1024 * 1280 * 128 + 2 * 4 * 1024 * 2048 * 128
+                                                                   + 2 * 10000 * 1024 * 128) / flops)}
+    return out
+
+
 def cpu_baseline(step_bytes, seconds):
     """The CPU oracle (plain-C restatement of DyNet's CPU path) on the same sweep: one host core (the process is
     pinned to it for the duration), the C functions called directly into preallocated outputs."""
@@ -793,25 +917,10 @@ def cpu_baseline(step_bytes, seconds):
         L.orc_layer_norm_forward(C.c_size_t(LN_N), C.c_uint(LN_BD), X, G, B, Y)
         L.orc_layer_norm_backward(C.c_size_t(LN_N), C.c_uint(LN_BD), X, G, DY, DX, DG, DB)
 
-    pinned = None
-    try:
-        allowed = sorted(os.sched_getaffinity(0))
-        pinned = allowed[len(allowed) // 2]
-        os.sched_setaffinity(0, {pinned})
-    except (AttributeError, OSError):
-        allowed = None
-    try:
-        sweep()
-        reps, t0 = 0, time.perf_counter()
-        while True:
-            sweep()
-            reps += 1
-            el = time.perf_counter() - t0
-            if el >= seconds or reps >= 50:
-                break
-    finally:
-        if allowed is not None:
-            os.sched_setaffinity(0, set(allowed))
+    with _OneCore() as core:
+        pinned = core.cpu
+        dt, reps = _time_cpu(sweep, seconds, 50)
+        el = dt * reps
     return {"value": round(step_bytes * reps / el / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": "%d full passes of the same cfg-2 sweep (4096x1024 fp32) through oracle/libdynet_cpu_oracle.so "
                       "in %.1f s on one host core (pinned to cpu %s) of %d" % (reps, el, pinned, os.cpu_count() or 0)}
@@ -978,8 +1087,16 @@ def main():
         out["lstm_lm_tokens_per_s_node_api"] = out["cfg5_lstm_lm"]["node_at_a_time_path"]["tokens_per_s"]
         out["lstm_lm_tokens_per_s_fused_path"] = out["cfg5_lstm_lm"]["fused_cell_path"]["tokens_per_s"]
     if not args.no_cpu_baseline:
+        out["cpu_baseline_per_config"] = cpu_baseline_per_config(args.cpu_config_seconds)
         out["cpu_baseline"] = cpu_baseline(sweep.step_bytes, args.cpu_seconds)
-    print(json.dumps(out))
+    # the long tables first, the headline fields last: a reader who keeps only the end of the line keeps those
+    head = ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+            "vs_baseline", "dtype", "data", "config", "frac_of_hbm_peak", "wall_ms_per_step", "hbm_copy_ceiling",
+            "lstm_lm_tokens_per_s_node_api", "lstm_lm_tokens_per_s_fused_path", "roofline_longest_entry", "roofline",
+            "cpu_baseline")
+    ordered = {k: v for k, v in out.items() if k not in head}
+    ordered.update({k: out[k] for k in head if k in out})
+    print(json.dumps(ordered))
 
 
 if __name__ == "__main__":
