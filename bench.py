@@ -176,11 +176,14 @@ def time_loop(dev, fns, reps):
 def per_kernel_table(dev, named, sets, reps, use_graph=True):
     """named: list of (name, bytes, fn(set)); returns a list of dicts with us / GB/s / fraction of peak."""
     out = []
+    # One replay holds at least 24 launches (the set list repeated if need be): the boundary between two replays of a
+    # graph costs about 5 us on this GPU, which a graph of 8 launches would add to every launch as 0.6 us.
+    rounds = max(1, -(-24 // max(len(sets), 1)))
     for name, nbytes, fn in named:
-        fns = [(lambda s=s: fn(s)) for s in sets]
+        fns = [(lambda s=s: fn(s)) for s in sets] * rounds
         if use_graph:
             g = capture(dev, fns)
-            us = time_graph(dev, g, reps, len(sets))
+            us = time_graph(dev, g, reps, len(fns))
             g.destroy()
         else:
             us = time_loop(dev, fns, reps)

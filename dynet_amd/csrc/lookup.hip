@@ -102,12 +102,13 @@ __global__ __launch_bounds__(kLkThreads) void lookup_gather_kernel(unsigned n_id
 }
 
 // ---- the plan: ids grouped by value ------------------------------------------------
-// plan = [gid | gpos | roff | rrem | arrivals | status], each part padded to 256 bytes:
-//   gid[k]   id of the k-th entry in grouped order: entries of one id are consecutive (a "run"),
-//            ids >= vocab are replaced by vocab (one run that the reduction skips)
-//   gpos[k]  position of that entry in the caller's id vector; ascending inside a run
-//   roff[k]  entries of the run before k        (0 at the head of a run)
-//   rrem[k]  entries of the run from k onwards  (1 at its last entry)
+// plan = [entries | arrivals | status], each part padded to 256 bytes.  Entry k of the grouped order is one
+// 16-byte record, so that a consumer's first (and only) dependent load per entry is a single 128-bit access:
+//   .x  id of the entry: entries of one id are consecutive (a "run"); ids >= vocab are replaced by vocab
+//       (one run that the reduction skips)
+//   .y  position of that entry in the caller's id vector; ascending inside a run
+//   .z  entries of the run before k        (0 at the head of a run)
+//   .w  entries of the run from k onwards  (1 at its last entry)
 //   arrivals one counter per 8 entries, zero whenever no reduction is running: the groups that share one
 //            slice of a very long run count themselves here so that the last one adds their partial sums up
 //   status   [0] = number of ids >= vocab
@@ -115,10 +116,7 @@ __global__ __launch_bounds__(kLkThreads) void lookup_gather_kernel(unsigned n_id
 // the trainer's row kernels), so the ids are grouped, not fully sorted:
 // bucket = id mod 256, inside a bucket ascending id / 256, inside a run ascending position.
 struct Plan {
-  unsigned* gid;
-  unsigned* gpos;
-  unsigned* roff;
-  unsigned* rrem;
+  uint4* ent;
   unsigned* arrivals;
   unsigned* status;
 };
@@ -128,18 +126,15 @@ constexpr int kChunk = 8;  // entries per thread group of the segmented sum (see
 static size_t align256(size_t n) { return (n + 255) / 256 * 256; }
 
 static size_t plan_bytes(unsigned n) {
-  return 4 * align256(sizeof(unsigned) * n) + align256(sizeof(unsigned) * cdiv<unsigned>(n, kChunk)) + 256;
+  return align256(sizeof(uint4) * size_t(n)) + align256(sizeof(unsigned) * cdiv<unsigned>(n, kChunk)) + 256;
 }
 
 static void plan_parts(const void* plan, unsigned n, Plan* w) {
   char* p = const_cast<char*>(static_cast<const char*>(plan));
-  const size_t b = align256(sizeof(unsigned) * n);
-  w->gid = reinterpret_cast<unsigned*>(p);
-  w->gpos = reinterpret_cast<unsigned*>(p + b);
-  w->roff = reinterpret_cast<unsigned*>(p + 2 * b);
-  w->rrem = reinterpret_cast<unsigned*>(p + 3 * b);
-  w->arrivals = reinterpret_cast<unsigned*>(p + 4 * b);
-  w->status = reinterpret_cast<unsigned*>(p + 4 * b + align256(sizeof(unsigned) * cdiv<unsigned>(n, kChunk)));
+  const size_t b = align256(sizeof(uint4) * size_t(n));
+  w->ent = reinterpret_cast<uint4*>(p);
+  w->arrivals = reinterpret_cast<unsigned*>(p + b);
+  w->status = reinterpret_cast<unsigned*>(p + b + align256(sizeof(unsigned) * cdiv<unsigned>(n, kChunk)));
 }
 
 static unsigned key_bits(unsigned max_key) {
@@ -148,9 +143,11 @@ static unsigned key_bits(unsigned max_key) {
   return bits;
 }
 
-// ---- one-launch plan for up to 65535 ids ---------------------------------------------
+// ---- one-launch plan for up to 65535 ids -----------------------------------------------
 // 256 blocks, one per bucket (id mod 256).  Every block reads the whole id vector (64 KB at
-// 16384 ids, from L2 after the first block of an XCD), so no block waits for another:
+// 16384 ids, from L2 after the first block of an XCD), so no block waits for another.
+// Two kernels: plan_direct_kernel (further down) when the keys fit 16 bits, which needs neither a
+// compaction nor sort passes, and this general one for wider keys:
 //   1. thread t owns a contiguous piece of the positions and counts, in registers, the ids of smaller
 //      buckets (their sum is where this bucket starts in the output) and of this bucket (their prefix
 //      over the threads is where the thread's matches go: the bucket is compacted in ascending position);
@@ -176,13 +173,21 @@ constexpr unsigned kPlanLdsWords = kPlanLdsBuf + 4 * kPlanCap;
 
 __device__ __forceinline__ unsigned long long lanes_below(int lane) { return (1ull << lane) - 1ull; }
 
-// inclusive prefix sum over the lanes of a wavefront
+// Inclusive prefix sum over the lanes of a wavefront.  The cross-lane steps are DPP modifiers (shifts inside a row of
+// 16 lanes, then lane 15 of a row into the next row and lane 31 into the upper half), not trips through the LDS
+// crossbar: six dependent adds of a few cycles each instead of six round trips.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ unsigned dpp_from(unsigned v) {  // 0 where the source lane does not exist or the row is masked
+  return unsigned(__builtin_amdgcn_update_dpp(0, int(v), CTRL, ROW_MASK, 0xF, false));
+}
 __device__ __forceinline__ unsigned wave_scan_add(unsigned v, int lane) {
-#pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    const unsigned u = __shfl_up(v, off, kWave);
-    if (lane >= off) v += u;
-  }
+  (void)lane;
+  v += dpp_from<0x111, 0xF>(v);  // row_shr:1
+  v += dpp_from<0x112, 0xF>(v);  // row_shr:2
+  v += dpp_from<0x114, 0xF>(v);  // row_shr:4
+  v += dpp_from<0x118, 0xF>(v);  // row_shr:8: every row holds its own inclusive prefix
+  v += dpp_from<0x142, 0xA>(v);  // row_bcast:15 into rows 1 and 3
+  v += dpp_from<0x143, 0xC>(v);  // row_bcast:31 into rows 2 and 3
   return v;
 }
 
@@ -206,14 +211,29 @@ __device__ __forceinline__ unsigned block_scan_excl(unsigned v, unsigned* tmp, u
 
 // lanes of the wavefront (among `valid` ones) that hold the same 8-bit digit as this lane
 __device__ __forceinline__ unsigned long long same_digit_lanes(unsigned dig, bool valid) {
-  unsigned long long same = __ballot(valid);
-#pragma unroll
-  for (int b = 0; b < 8; ++b) {
-    const bool bit = (dig >> b) & 1u;
-    const unsigned long long bal = __ballot(valid && bit);
-    same &= bit ? bal : ~bal;
+  // One ballot per distinct digit for the first few digits: a step mostly holds the odd id of a bucket, or many
+  // copies of one hot id and little else.  Lanes left after that (many distinct digits in one step) are matched bit
+  // by bit, eight ballots whatever their number.
+  unsigned long long todo = __ballot(valid), mine = 0ull;
+#pragma unroll 1
+  for (int it = 0; it < 4 && todo != 0ull; ++it) {  // uniform
+    const unsigned d0 = unsigned(__builtin_amdgcn_readlane(int(dig), __ffsll((long long)todo) - 1));
+    const unsigned long long eq = __ballot(valid && dig == d0);
+    if (valid && dig == d0) mine = eq;
+    todo &= ~eq;
   }
-  return same;
+  if (todo != 0ull) {
+    const bool rest = valid && ((todo >> (threadIdx.x & 63)) & 1ull) != 0ull;
+    unsigned long long same = todo;
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      const bool bit = (dig >> b) & 1u;
+      const unsigned long long bal = __ballot(rest && bit);
+      same &= bit ? bal : ~bal;
+    }
+    if (rest) mine = same;
+  }
+  return mine;
 }
 
 // One stable counting-sort pass over the m entries (key, pos) of a bucket on digit (key >> shift) & 255.
@@ -339,10 +359,7 @@ __device__ __forceinline__ void plan_finish_bucket(unsigned m, unsigned passes, 
     const unsigned long long gt = lane == 63 ? 0ull : hm & ~(lanes_below(lane + 1));
     const int nh = gt ? int(q * 64) + __ffsll((long long)gt) - 1 : (q + 1 < steps ? step_first[q + 1] : int(m));
     if (in) {
-      out.gid[bstart + j] = key;
-      out.gpos[bstart + j] = pA[j];
-      out.roff[bstart + j] = j - unsigned(lh);
-      out.rrem[bstart + j] = unsigned(nh) - j;
+      out.ent[bstart + j] = make_uint4(key, pA[j], j - unsigned(lh), unsigned(nh) - j);
       if ((bstart + j) % kChunk == 0) out.arrivals[(bstart + j) / kChunk] = 0;
     }
   }
@@ -435,6 +452,170 @@ __global__ __launch_bounds__(kPlanThreads) void plan_group_kernel(unsigned n, un
                        tmp, step_last, step_first, out);
 }
 
+// ---- one-launch plan when the keys fit 16 bits (vocab <= 65535): no compaction, no sort passes -------------
+// The bucket digit is the low byte, and what is left of a key is one more byte, which names the id inside its
+// bucket: a run IS a bin of that byte.  Wavefront w owns the positions [w * per_wave, (w + 1) * per_wave), 64 at a
+// step, and keeps their keys in registers.
+//   pass 1  counts per (high byte, wavefront) in LDS: the lanes of a step that hold the same byte are found with
+//           ballots, the first of them adds their number to the wavefront's own counter (no atomics, nothing
+//           depends on timing); also the ids of smaller buckets (where this bucket starts in the output);
+//   scan    exclusive prefix over the 4096 counters in (byte, wavefront) order: counter (b, w) becomes the place of
+//           the first entry with byte b that wavefront w holds, and (b, 0) the start of the run;
+//   pass 2  the same walk again: an entry's place is its wavefront's counter plus its rank among the equal bytes of
+//           its step, the counter advances by the step's count; place, run start and run end give the whole record,
+//           which goes straight to global memory.
+// Entries of a run end up in ascending position because wavefronts own ascending position ranges and walk them in
+// ascending order.  A bucket of any size takes the same path (nothing is staged in LDS but the counters).
+template <int STEPS>
+__global__ __launch_bounds__(kPlanThreads) void plan_direct_kernel(unsigned n, unsigned vocab,
+                                                                   const unsigned* __restrict__ ids, const Plan out) {
+  __shared__ __attribute__((aligned(16))) unsigned cnt[256 * kPlanWaves];  // [high byte][wavefront]
+  __shared__ unsigned run_start[257];
+  __shared__ unsigned tmp[kPlanWaves], lt_tot[kPlanWaves], bad_tot[kPlanWaves];
+  const unsigned d = blockIdx.x;
+  const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+  reinterpret_cast<uint4*>(cnt)[t] = make_uint4(0u, 0u, 0u, 0u);
+  const unsigned per_wave = cdiv<unsigned>(cdiv<unsigned>(n, kPlanWaves), 64u) * 64u;
+  const unsigned base = unsigned(w) * per_wave;
+  // A slot (wavefront, step, lane) that stands for no position holds a key that is in no bucket's way: its low byte
+  // is not d, so it never counts as this bucket's; it may count as a smaller bucket's, which is taken off again below.
+  // What a wavefront-step costs is its vector instructions (16 wavefronts share 4 SIMDs): the first walk is kept to
+  // six per step.
+  const unsigned none_key = 0x80000000u | ((d + 1u) & 255u);
+  const unsigned slots = unsigned(kPlanWaves) * 64u * unsigned(STEPS);
+  const unsigned left = n > base + lane ? n - base - lane : 0u;          // positions from this lane's first one on
+  const unsigned lim = min(cdiv<unsigned>(left, 64u), per_wave / 64u);   // steps in which this lane holds a position
+  unsigned key[STEPS];
+#pragma unroll
+  for (int i = 0; i < STEPS; ++i) {
+    // unconditional loads (a slot past the end reads the last id and is masked): loads inside branches are waited
+    // for one by one
+    const unsigned p = base + 64u * i + lane;
+    key[i] = ids[min(p, n - 1u)];
+  }
+  __syncthreads();  // the counters are zero
+  // Each wavefront "tracks" one high byte, the first of this bucket that it meets: in the bucket of a hot id that is
+  // the hot id.  Entries with the tracked byte are counted and ranked in scalar registers (one ballot a step); only
+  // the others go through the wavefront's LDS counters, a round trip per step that holds any.
+  unsigned lt = 0;
+  unsigned tracked = kNone, run = 0;  // uniform over the wavefront
+  // which steps hold an id of this bucket at all: both walks skip the other steps (most of them) with a scalar test
+  unsigned long long active = 0ull;  // uniform; STEPS <= 64
+#pragma unroll
+  for (int i = 0; i < STEPS; ++i) {
+    const unsigned k = unsigned(i) < lim ? min(key[i], vocab) : none_key;
+    key[i] = k;
+    lt += (k & 255u) < d ? 1u : 0u;
+    active |= __ballot((k & 255u) == d) != 0ull ? 1ull << i : 0ull;
+  }
+  unsigned bad = 0;
+  if (d == kPlanBuckets - 1) {  // one block counts the ids >= vocab (not the one of the often hottest bucket 0)
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i) bad += key[i] == vocab ? 1u : 0u;
+  }
+#pragma unroll
+  for (int i = 0; i < STEPS; ++i) {
+    if (((active >> i) & 1ull) != 0ull) {  // uniform over the wavefront
+      unsigned k = key[i];
+      asm volatile("" : "+v"(k));  // a value of its own: the lane masks of the loop above are recomputed, not kept
+      const bool mine = (k & 255u) == d;
+      unsigned long long todo = __ballot(mine);
+      const unsigned hi = mine ? k >> 8 : kNone;
+      if (tracked == kNone) tracked = unsigned(__builtin_amdgcn_readlane(int(hi), __ffsll((long long)todo) - 1));
+      const unsigned long long eq = __ballot(hi == tracked);
+      run += unsigned(__popcll(eq));
+      todo &= ~eq;
+      if (todo != 0ull) {
+        // the wavefront's own counters: LDS adds that return nothing, so the walk does not wait for them
+        const bool rest = mine && hi != tracked;
+        if ((todo & (todo - 1ull)) == 0ull) {  // one more entry, the usual case in a sparse bucket: nothing to match
+          if (rest) atomicAdd(&cnt[hi * kPlanWaves + w], 1u);
+        } else {
+          const unsigned long long same = same_digit_lanes(hi, rest);
+          if (rest && (same & lanes_below(lane)) == 0) atomicAdd(&cnt[hi * kPlanWaves + w], unsigned(__popcll(same)));
+        }
+      }
+    }
+  }
+  if (tracked != kNone && lane == 0) atomicAdd(&cnt[tracked * kPlanWaves + w], run);
+  lt = wave_scan_add(lt, lane);
+  bad = wave_scan_add(bad, lane);
+  if (lane == 63) {
+    lt_tot[w] = lt;
+    bad_tot[w] = bad;
+  }
+  __syncthreads();
+  // thread t scans counters [4t, 4t + 4): bytes in ascending order, wavefronts in ascending order inside a byte
+  uint4 c4 = reinterpret_cast<uint4*>(cnt)[t];
+  unsigned m = 0;
+  const unsigned e0 = block_scan_excl(c4.x + c4.y + c4.z + c4.w, tmp, &m);
+  uint4 e4;
+  e4.x = e0;
+  e4.y = e4.x + c4.x;
+  e4.z = e4.y + c4.y;
+  e4.w = e4.z + c4.z;
+  reinterpret_cast<uint4*>(cnt)[t] = e4;
+  if ((t & 3) == 0) run_start[t >> 2] = e0;  // counter (byte, wavefront 0)
+  if (t == 0) run_start[256] = m;
+  unsigned bstart = 0, nbad = 0;
+#pragma unroll
+  for (int k = 0; k < kPlanWaves; ++k) {
+    bstart += lt_tot[k];
+    nbad += bad_tot[k];
+  }
+  if ((none_key & 255u) < d) bstart -= slots - n;  // the slots that stand for no position were counted as a smaller bucket's
+  if (d == kPlanBuckets - 1 && t == 0) out.status[0] = nbad;
+  if (m == 0) return;  // uniform over the block
+  __syncthreads();
+  unsigned at_tracked = 0, first_tracked = 0, end_tracked = 0;
+  if (tracked != kNone) {
+    at_tracked = unsigned(__builtin_amdgcn_readfirstlane(int(cnt[tracked * kPlanWaves + w])));
+    first_tracked = unsigned(__builtin_amdgcn_readfirstlane(int(run_start[tracked])));
+    end_tracked = unsigned(__builtin_amdgcn_readfirstlane(int(run_start[tracked + 1])));
+  }
+#pragma unroll
+  for (int i = 0; i < STEPS; ++i) {
+    if (((active >> i) & 1ull) != 0ull) {
+      unsigned k = key[i];
+      asm volatile("" : "+v"(k));  // a value of its own: the first walk's lane masks are recomputed, not kept in registers
+      const bool mine = (k & 255u) == d;
+      unsigned long long todo = __ballot(mine);
+      const unsigned hi = mine ? k >> 8 : kNone;
+      const unsigned pos = base + 64u * i + lane;
+      const unsigned long long eq = __ballot(hi == tracked);
+      if (hi == tracked) {
+        const unsigned j = at_tracked + __builtin_amdgcn_mbcnt_hi(unsigned(eq >> 32), __builtin_amdgcn_mbcnt_lo(unsigned(eq), 0u));
+        out.ent[bstart + j] = make_uint4(k, pos, j - first_tracked, end_tracked - j);
+      }
+      at_tracked += unsigned(__popcll(eq));
+      todo &= ~eq;
+      if (todo != 0ull && (todo & (todo - 1ull)) == 0ull) {  // one more entry: its counter is its place
+        if (mine && hi != tracked) {
+          const unsigned j = atomicAdd(&cnt[hi * kPlanWaves + w], 1u);
+          out.ent[bstart + j] = make_uint4(k, pos, j - run_start[hi], run_start[hi + 1] - j);
+        }
+      } else if (todo != 0ull) {
+        const bool rest = mine && hi != tracked;
+        const unsigned long long same = same_digit_lanes(hi, rest);
+        const unsigned rank = __popcll(same & lanes_below(lane));
+        // every lane reads its byte's counter before the first lane of each byte advances it: the wavefront issues
+        // the load for all its lanes, then the store, and LDS keeps that order
+        unsigned at = 0;
+        if (rest) at = cnt[hi * kPlanWaves + w];
+        __builtin_amdgcn_wave_barrier();
+        if (rest && rank == 0) cnt[hi * kPlanWaves + w] = at + __popcll(same);
+        __builtin_amdgcn_wave_barrier();
+        if (rest) {
+          const unsigned j = at + rank;
+          out.ent[bstart + j] = make_uint4(k, pos, j - run_start[hi], run_start[hi + 1] - j);
+        }
+      }
+    }
+  }
+  // the arrival counters of the chunks that start inside this bucket's part of the output
+  for (unsigned c = cdiv<unsigned>(bstart, kChunk) + t; c * kChunk < bstart + m; c += kPlanThreads) out.arrivals[c] = 0;
+}
+
 // ---- plan for more ids than that: device-wide radix sort, then the run offsets by binary search -----
 __global__ __launch_bounds__(256) void plan_clamp_kernel(unsigned n, unsigned vocab, const unsigned* __restrict__ ids,
                                                          unsigned* __restrict__ keys, unsigned* status) {
@@ -443,25 +624,26 @@ __global__ __launch_bounds__(256) void plan_clamp_kernel(unsigned n, unsigned vo
   if (k < n) keys[k] = min(ids[k], vocab);
 }
 
-__global__ __launch_bounds__(256) void plan_runs_sorted_kernel(unsigned n, unsigned vocab, const Plan out) {
+__global__ __launch_bounds__(256) void plan_runs_sorted_kernel(unsigned n, unsigned vocab,
+                                                               const unsigned* __restrict__ sid,
+                                                               const unsigned* __restrict__ spos, const Plan out) {
   const unsigned k = blockIdx.x * 256 + threadIdx.x;
   if (k >= n) return;
-  const unsigned id = out.gid[k];
+  const unsigned id = sid[k];
   unsigned lo = 0, hi = k;  // first index holding id
   while (lo < hi) {
     const unsigned mid = lo + (hi - lo) / 2;
-    if (out.gid[mid] < id) lo = mid + 1;
+    if (sid[mid] < id) lo = mid + 1;
     else hi = mid;
   }
   const unsigned first = lo;
   lo = k + 1, hi = n;  // first index holding a larger id
   while (lo < hi) {
     const unsigned mid = lo + (hi - lo) / 2;
-    if (out.gid[mid] <= id) lo = mid + 1;
+    if (sid[mid] <= id) lo = mid + 1;
     else hi = mid;
   }
-  out.roff[k] = k - first;
-  out.rrem[k] = lo - k;
+  out.ent[k] = make_uint4(id, spos[k], k - first, lo - k);
   if (k % kChunk == 0) out.arrivals[k / kChunk] = 0;
   if (id >= vocab && k == first) out.status[0] = lo - first;  // one writer: the head of the run of clamped ids
 }
@@ -478,12 +660,13 @@ static int sort_tmp_bytes(unsigned n, unsigned bits, size_t* bytes) {
 
 static int plan_ws_bytes(unsigned n, unsigned vocab, size_t* bytes) {
   if (n <= kPlanSmallMax) {
+    // only a bucket too large for LDS on the route for keys wider than 16 bits uses it
     *bytes = align256(4 * sizeof(unsigned) * size_t(n));
     return DYHIP_OK;
   }
   size_t sort_b = 0;
   DYHIP_CHECK_STATUS(sort_tmp_bytes(n, key_bits(vocab), &sort_b));
-  *bytes = align256(sizeof(unsigned) * size_t(n)) + align256(sort_b);
+  *bytes = 3 * align256(sizeof(unsigned) * size_t(n)) + align256(sort_b);  // keys, sorted keys, sorted positions
   return DYHIP_OK;
 }
 
@@ -499,6 +682,15 @@ static int build_plan(dyhip_device* dev, unsigned n, const unsigned* ids_dev, un
   Plan out;
   plan_parts(plan, n, &out);
   const unsigned bits = key_bits(vocab);  // keys are min(id, vocab) <= vocab
+  if (n <= kPlanSmallMax && bits <= 16) {
+    const unsigned per_wave = cdiv<unsigned>(cdiv<unsigned>(n, kPlanWaves), 64u);  // 64-entry steps of a wavefront
+    const dim3 grid(kPlanBuckets), block(kPlanThreads);
+    if (per_wave <= 4) hipLaunchKernelGGL(plan_direct_kernel<4>, grid, block, 0, dev->stream, n, vocab, ids_dev, out);
+    else if (per_wave <= 16) hipLaunchKernelGGL(plan_direct_kernel<16>, grid, block, 0, dev->stream, n, vocab, ids_dev, out);
+    else hipLaunchKernelGGL(plan_direct_kernel<64>, grid, block, 0, dev->stream, n, vocab, ids_dev, out);
+    DYHIP_CHECK_LAUNCH();
+    return DYHIP_OK;
+  }
   if (n <= kPlanSmallMax) {
     const unsigned passes = bits <= 8 ? 0u : (bits - 8 + 7) / 8;
     const size_t lds = sizeof(unsigned) * kPlanLdsWords;
@@ -522,17 +714,18 @@ static int build_plan(dyhip_device* dev, unsigned n, const unsigned* ids_dev, un
     DYHIP_CHECK_LAUNCH();
     return DYHIP_OK;
   }
-  unsigned* keys = static_cast<unsigned*>(ws);
   const size_t keys_b = align256(sizeof(unsigned) * size_t(n));
+  unsigned* keys = static_cast<unsigned*>(ws);
+  unsigned* sid = reinterpret_cast<unsigned*>(static_cast<char*>(ws) + keys_b);
+  unsigned* spos = reinterpret_cast<unsigned*>(static_cast<char*>(ws) + 2 * keys_b);
   size_t sort_b = 0;
   DYHIP_CHECK_STATUS(sort_tmp_bytes(n, bits, &sort_b));
   const dim3 grid(cdiv<unsigned>(n, 256)), block(256);
   hipLaunchKernelGGL(plan_clamp_kernel, grid, block, 0, dev->stream, n, vocab, ids_dev, keys, out.status);
   DYHIP_CHECK_LAUNCH();
-  DYHIP_CHECK_HIP(rocprim::radix_sort_pairs(static_cast<char*>(ws) + keys_b, sort_b, static_cast<const unsigned*>(keys),
-                                            out.gid, rocprim::counting_iterator<unsigned>(0), out.gpos, n, 0, bits,
-                                            dev->stream));
-  hipLaunchKernelGGL(plan_runs_sorted_kernel, grid, block, 0, dev->stream, n, vocab, out);
+  DYHIP_CHECK_HIP(rocprim::radix_sort_pairs(static_cast<char*>(ws) + 3 * keys_b, sort_b, static_cast<const unsigned*>(keys),
+                                            sid, rocprim::counting_iterator<unsigned>(0), spos, n, 0, bits, dev->stream));
+  hipLaunchKernelGGL(plan_runs_sorted_kernel, grid, block, 0, dev->stream, n, vocab, sid, spos, out);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
@@ -550,18 +743,73 @@ static int build_plan(dyhip_device* dev, unsigned n, const unsigned* ids_dev, un
 //     added in ascending order.  A slice is at least one 128-byte line wide; a run long enough to give
 //     every slice several groups is also cut into parts of consecutive entries, whose sums the last
 //     group to finish adds up in ascending order (arrival counters in the plan, partial sums in the
-//     workspace).  Either way a thread's share of a run of any length is a few batches.
-// Loads go out in batches of kBatch rows per thread (nearly every group needs one batch); the kernel keeps
-// few enough registers for every block of the grid to be resident at once.  Updated rows are written with
-// streaming stores, so they drain while the kernel runs instead of when it ends.
+//     workspace).  Either way a thread's share of a run is one batch of loads at the usual row widths.
+// The kernel keeps few enough registers for every block of the grid to be resident at once.  Updated rows are
+// written with streaming stores, so they drain while the kernel runs instead of when it ends; the old rows are read
+// with streaming loads (each is read once, and a line left in the L2 would only stand in the store's way).
 // No second launch, no float atomics, and no group ever waits for another: the result does not depend on timing.
-constexpr int kBatch = 11;
+constexpr int kBatch = 11;                              // narrow groups: rows per thread and batch
+constexpr int kBatchLong = 16;                          // wide groups inside a long run: rows per thread and batch
 constexpr unsigned kHeavyMin = 2 * kChunk - 1;         // shortest run that must contain a whole chunk
 constexpr int kItemMax = 3 * kChunk - 2;               // own chunk after its first entry (7) + the longest short run (14) <= 22
 constexpr int kItemBatches = (kItemMax + kBatch - 1) / kBatch;
 static_assert(kChunk - 1 + int(kHeavyMin) - 1 <= kItemMax, "a group's short runs fit kItemBatches batches");
 static_assert(3 * kChunk <= 64 && kItemMax <= 32 && kBatch >= kChunk, "plan entries of an item sit in the lanes of one "
               "wavefront / two 16-lane rounds; every head of an item is in its first batch");
+
+// Wide groups sum the short runs of their item as one stream of rows per thread, straight-line code without a
+// branch around any load: the old rows of the (at most kChunk) runs that start in the chunk and the first kBatch
+// gradient rows are requested at once; an item of more than kBatch entries refills the register of each row it has
+// consumed with the row kBatch further on, so its later rows never wait for a whole batch to come back.  A slot
+// without an entry loads a row that is in flight anyway and is not added.  Because nothing is conditional the compiler
+// can count the loads in flight and waits for exactly the row it needs; loads issued inside per-entry branches made
+// it wait for everything before every use.
+constexpr unsigned kSlotValid = 1u, kSlotHead = 2u, kSlotLast = 4u;
+
+__device__ __forceinline__ unsigned lane_get(unsigned v, unsigned src_lane) {
+  return unsigned(__builtin_amdgcn_readlane(int(v), int(src_lane)));
+}
+__device__ __forceinline__ float4 vsel(bool c, const float4 a, const float4 b) {
+  return make_float4(c ? a.x : b.x, c ? a.y : b.y, c ? a.z : b.z, c ? a.w : b.w);
+}
+__device__ __forceinline__ float vsel(bool c, const float a, const float b) { return c ? a : b; }
+
+// Entry j of the item sits in lane first_l + j: e_pos its position (row of g), e_id its id (row of grads), e_fl its
+// kSlot* flags (0 = no such entry, or an entry of the run of ids >= vocab, which is skipped).  NE = entries walked.
+template <class V, int NE>
+__device__ __forceinline__ void stream_item(unsigned e_pos, unsigned e_id, unsigned e_fl, unsigned first_l,
+                                            unsigned dimv, unsigned c, bool cok, const V* __restrict__ g,
+                                            V* __restrict__ grads) {
+  const unsigned cc = cok ? c : 0u;
+  const unsigned dummy_pos = lane_get(e_pos, first_l);  // a row of g that exists and is requested anyway
+  V old[kChunk], v[kBatch];
+#pragma unroll
+  for (int j = 0; j < kChunk; ++j) {  // a run of the item starts inside the chunk
+    const unsigned fl = lane_get(e_fl, first_l + j);
+    const bool head = (fl & kSlotHead) != 0;
+    const V* src = head ? grads + size_t(lane_get(e_id, first_l + j)) * dimv : g + size_t(dummy_pos) * dimv;
+    old[j] = vload<true>(src + cc);
+  }
+#define DYHIP_ENTRY_LOAD(dst, j2)                                                                  \
+  do {                                                                                             \
+    const unsigned fl_ = lane_get(e_fl, first_l + (j2));                                           \
+    const unsigned row_ = (fl_ & kSlotValid) ? lane_get(e_pos, first_l + (j2)) : dummy_pos;        \
+    (dst) = vload<false>(g + size_t(row_) * dimv + cc);                                            \
+  } while (0)
+#pragma unroll
+  for (int j = 0; j < kBatch; ++j) DYHIP_ENTRY_LOAD(v[j], j);
+  V acc = vzero<V>();
+#pragma unroll
+  for (int j = 0; j < NE; ++j) {
+    const unsigned fl = lane_get(e_fl, first_l + j);
+    const V x = v[j % kBatch];
+    if (j + kBatch < NE) DYHIP_ENTRY_LOAD(v[j % kBatch], j + kBatch);
+    const V from = j < kChunk ? vsel((fl & kSlotHead) != 0, old[j < kChunk ? j : 0], acc) : acc;
+    acc = vsel((fl & kSlotValid) != 0, vadd(from, x), acc);
+    if ((fl & kSlotLast) && cok) vstore<true>(grads + size_t(lane_get(e_id, first_l + j)) * dimv + c, acc);
+  }
+#undef DYHIP_ENTRY_LOAD
+}
 
 template <class V, bool WIDE>
 __global__ __launch_bounds__(256) void scatter_runs_kernel(unsigned n, unsigned dimv, unsigned tpr, unsigned vocab,
@@ -580,14 +828,13 @@ __global__ __launch_bounds__(256) void scatter_runs_kernel(unsigned n, unsigned 
   // threads) hold entries k0 .. k0+15 in each 16-lane cluster and fetch an item's entries afterwards.
   const unsigned l = WIDE ? unsigned(lane) : (threadIdx.x & 15u);
   const bool l_in = (WIDE ? l < 3u * kChunk : true) && k0 + l < n;
-  const unsigned e_off = l_in ? p.roff[k0 + l] : 1u;
-  const unsigned e_rem = l_in ? p.rrem[k0 + l] : 0u;
-  const unsigned e_id = l_in ? p.gid[k0 + l] : kNone;
-  const unsigned e_pos = l_in ? p.gpos[k0 + l] : kNone;
+  const uint4 ent = l_in ? p.ent[k0 + l] : make_uint4(kNone, kNone, 1u, 0u);
+  const unsigned e_id = ent.x, e_pos = ent.y, e_off = ent.z, e_rem = ent.w;
   const unsigned o0 = WIDE ? __builtin_amdgcn_readfirstlane(e_off) : __shfl(e_off, 0, 16);
   const unsigned r0 = WIDE ? __builtin_amdgcn_readfirstlane(e_rem) : __shfl(e_rem, 0, 16);
   if (o0 + r0 >= kHeavyMin && r0 >= unsigned(kChunk)) {
     // ---- this chunk lies inside a long run: take a slice of its columns --------------------
+    constexpr int kB = WIDE ? kBatchLong : kBatch;
     const unsigned start = k0 - o0, R = o0 + r0;
     const unsigned cf = (start + kChunk - 1) / kChunk;       // first chunk the run covers entirely
     const unsigned W = (start + R) / kChunk - cf;            // how many it covers entirely (>= 1)
@@ -613,21 +860,21 @@ __global__ __launch_bounds__(256) void scatter_runs_kernel(unsigned n, unsigned 
       const unsigned c = s * w + cin;
       const bool cok = busy && c < dimv;
       V old = vzero<V>();
-      if (cok && slot == 0) old = grads[size_t(row) * dimv + c];
+      if (cok && slot == 0) old = vload<true>(grads + size_t(row) * dimv + c);
       V acc = vzero<V>();
-      for (unsigned e0 = eb + slot; e0 < ee; e0 += E * kBatch) {
-        unsigned pos[kBatch];
+      for (unsigned e0 = eb + slot; e0 < ee; e0 += E * kB) {
+        unsigned pos[kB];
 #pragma unroll
-        for (int u = 0; u < kBatch; ++u) {
+        for (int u = 0; u < kB; ++u) {
           const unsigned e = e0 + u * E;
-          pos[u] = (cok && e < ee) ? p.gpos[start + e] : kNone;
+          pos[u] = (cok && e < ee) ? p.ent[start + e].y : kNone;
         }
-        V v[kBatch];
+        V v[kB];
 #pragma unroll
-        for (int u = 0; u < kBatch; ++u)
+        for (int u = 0; u < kB; ++u)
           v[u] = pos[u] != kNone ? g[size_t(pos[u]) * dimv + c] : vzero<V>();
 #pragma unroll
-        for (int u = 0; u < kBatch; ++u) acc = vadd(acc, v[u]);
+        for (int u = 0; u < kB; ++u) acc = vadd(acc, v[u]);
       }
       if (WIDE) {
         // slots are added in ascending order: first every eighth slot by eight threads per column, then those
@@ -706,68 +953,65 @@ __global__ __launch_bounds__(256) void scatter_runs_kernel(unsigned n, unsigned 
   const unsigned first_l = __ffsll((long long)own_mask) - 1, last_l = 63 - __clzll(own_mask);
   const unsigned ks = k0 + first_l;
   const unsigned ke = k0 + last_l + (WIDE ? __builtin_amdgcn_readlane(e_rem, last_l) : __shfl(e_rem, last_l, 16));
-  // WIDE: entry ks + j sits in lane first_l + j (< 24) of every wavefront.  Narrow groups fetch entry ks + j
-  // with lane j mod 16 of their 16-lane cluster (two rounds) and hand it around.
-  const unsigned my_flags = (e_off == 0 ? 1u : 0u) | (e_rem == 1 ? 2u : 0u);
-  unsigned b_pos[2] = {kNone, kNone}, b_id[2] = {kNone, kNone}, b_fl[2] = {0u, 0u};
-  if (!WIDE) {
+  if constexpr (WIDE) {
+    // entry ks + j sits in lane first_l + j (< 24) of every wavefront of the group
+    const bool live = l >= first_l && k0 + l < ke && e_id < vocab;  // ids >= vocab form one run that is skipped
+    const unsigned e_fl = live ? (kSlotValid | (e_off == 0 ? kSlotHead : 0u) | (e_rem == 1 ? kSlotLast : 0u)) : 0u;
+    for (unsigned c0 = 0; c0 < dimv; c0 += tpr) {
+      const unsigned c = c0 + t;
+      if (ke - ks <= unsigned(kBatch)) stream_item<V, kBatch>(e_pos, e_id, e_fl, first_l, dimv, c, c < dimv, g, grads);
+      else stream_item<V, kItemMax>(e_pos, e_id, e_fl, first_l, dimv, c, c < dimv, g, grads);
+    }
+  } else {
+    // Narrow groups fetch entry ks + j with lane j mod 16 of their 16-lane cluster (two rounds) and hand it around.
+    unsigned b_pos[2] = {kNone, kNone}, b_id[2] = {kNone, kNone}, b_fl[2] = {0u, 0u};
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
       const unsigned k = ks + 16u * r + (threadIdx.x & 15u);
       const bool in = k < ke;
-      b_pos[r] = in ? p.gpos[k] : kNone;
-      b_id[r] = in ? p.gid[k] : kNone;
-      b_fl[r] = in ? (p.roff[k] == 0 ? 1u : 0u) | (p.rrem[k] == 1 ? 2u : 0u) : 0u;
+      const uint4 e2 = in ? p.ent[k] : make_uint4(kNone, kNone, 1u, 0u);
+      b_pos[r] = e2.y;
+      b_id[r] = e2.x;
+      b_fl[r] = in ? (e2.z == 0 ? 1u : 0u) | (e2.w == 1 ? 2u : 0u) : 0u;
     }
-  }
-  for (unsigned c0 = 0; c0 < dimv; c0 += tpr) {
-    const unsigned c = c0 + t;
-    const bool cok = c < dimv;
-    V acc = vzero<V>();
+    for (unsigned c0 = 0; c0 < dimv; c0 += tpr) {
+      const unsigned c = c0 + t;
+      const bool cok = c < dimv;
+      V acc = vzero<V>();
 #pragma unroll
-    for (int r = 0; r < kItemBatches; ++r) {
-      if (ks + unsigned(r * kBatch) >= ke) break;  // uniform over the group
-      unsigned id[kBatch], pos[kBatch];
-      bool head[kBatch], tail[kBatch];
+      for (int r = 0; r < kItemBatches; ++r) {
+        if (ks + unsigned(r * kBatch) >= ke) break;  // uniform over the group
+        unsigned id[kBatch], pos[kBatch];
+        bool head[kBatch], tail[kBatch];
 #pragma unroll
-      for (int u = 0; u < kBatch; ++u) {
-        const int j = r * kBatch + u;
-        if (j >= kItemMax) {
-          pos[u] = kNone; id[u] = kNone; head[u] = false; tail[u] = false;
-        } else if (WIDE) {
-          const bool in = ks + j < ke;
-          const unsigned src = in ? first_l + j : 0u;
-          pos[u] = in ? __builtin_amdgcn_readlane(e_pos, src) : kNone;
-          id[u] = __builtin_amdgcn_readlane(e_id, src);
-          const unsigned fl = __builtin_amdgcn_readlane(my_flags, src);
-          head[u] = in && (fl & 1u);
-          tail[u] = in && (fl & 2u);
-        } else {
-          pos[u] = __shfl(b_pos[j / 16], j % 16, 16);
-          id[u] = __shfl(b_id[j / 16], j % 16, 16);
-          const unsigned fl = __shfl(b_fl[j / 16], j % 16, 16);
-          head[u] = fl & 1u;
-          tail[u] = fl & 2u;
+        for (int u = 0; u < kBatch; ++u) {
+          const int j = r * kBatch + u;
+          if (j >= kItemMax) {
+            pos[u] = kNone; id[u] = kNone; head[u] = false; tail[u] = false;
+          } else {
+            pos[u] = __shfl(b_pos[j / 16], j % 16, 16);
+            id[u] = __shfl(b_id[j / 16], j % 16, 16);
+            const unsigned fl = __shfl(b_fl[j / 16], j % 16, 16);
+            head[u] = fl & 1u;
+            tail[u] = fl & 2u;
+          }
         }
-      }
-      // every load of the batch is issued before the first add; heads lie in the own chunk, i.e. in batch 0
-      V v[kBatch], old[kChunk];
+        // every load of the batch is issued before the first add; heads lie in the own chunk, i.e. in batch 0
+        V v[kBatch], old[kChunk];
 #pragma unroll
-      for (int u = 0; u < kBatch; ++u) {
-        v[u] = (cok && pos[u] != kNone) ? g[size_t(pos[u]) * dimv + c] : vzero<V>();
-        if (r == 0 && u < kChunk)
-          old[u] = (cok && head[u] && id[u] < vocab) ? grads[size_t(id[u]) * dimv + c] : vzero<V>();
-      }
-      // One explicit wait for the batch.  The loads sit in per-entry branches, so the compiler cannot count them and
-      // waits for everything in flight before each use of a loaded row: after the first finished run that includes
-      // the run's own store, and the stores of a group went out one acknowledged round trip at a time.
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        for (int u = 0; u < kBatch; ++u) {
+          v[u] = (cok && pos[u] != kNone) ? g[size_t(pos[u]) * dimv + c] : vzero<V>();
+          if (r == 0 && u < kChunk)
+            old[u] = (cok && head[u] && id[u] < vocab) ? vload<true>(grads + size_t(id[u]) * dimv + c) : vzero<V>();
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): one explicit wait for the batch
 #pragma unroll
-      for (int u = 0; u < kBatch; ++u) {
-        if (pos[u] != kNone) {
-          if (r == 0 && u < kChunk && head[u]) acc = old[u];
-          acc = vadd(acc, v[u]);
-          if (cok && tail[u] && id[u] < vocab) vstore<true>(grads + size_t(id[u]) * dimv + c, acc);
+        for (int u = 0; u < kBatch; ++u) {
+          if (pos[u] != kNone) {
+            if (r == 0 && u < kChunk && head[u]) acc = old[u];
+            acc = vadd(acc, v[u]);
+            if (cok && tail[u] && id[u] < vocab) vstore<true>(grads + size_t(id[u]) * dimv + c, acc);
+          }
         }
       }
     }

@@ -84,14 +84,17 @@ __global__ __launch_bounds__(256) void sgd_scaled_kernel(size_t n4, size_t n, fl
   }
 }
 
-// one block per sorted position; only the first entry of each run of equal ids acts
-__global__ __launch_bounds__(128) void sgd_rows_kernel(unsigned n, const unsigned* __restrict__ sorted_ids,
+// The entries of a lookup plan (lookup.hip): one 16-byte record per grouped position, .x = id (ids >= vocab replaced
+// by vocab), .z = entries of its run before it (0 at the head of a run).
+// One block per grouped position; only the first entry of each run of equal ids acts.
+__global__ __launch_bounds__(128) void sgd_rows_kernel(unsigned n, const uint4* __restrict__ entries,
                                                        unsigned dim, unsigned vocab, float* __restrict__ values,
                                                        float* __restrict__ grads, float lr, float wd,
                                                        const float* __restrict__ gscale) {
   const unsigned k = blockIdx.x;
-  const unsigned id = sorted_ids[k];
-  if (id >= vocab || (k > 0 && sorted_ids[k - 1] == id)) return;
+  const uint4 e = entries[k];
+  const unsigned id = e.x;
+  if (id >= vocab || e.z != 0) return;
   const float gs = *gscale;
   const float s = lr * gs / wd;
   float* pv = values + size_t(id) * dim;
@@ -102,14 +105,15 @@ __global__ __launch_bounds__(128) void sgd_rows_kernel(unsigned n, const unsigne
   }
 }
 
-__global__ __launch_bounds__(128) void sqnorm_rows_kernel(unsigned n, const unsigned* __restrict__ sorted_ids,
+__global__ __launch_bounds__(128) void sqnorm_rows_kernel(unsigned n, const uint4* __restrict__ entries,
                                                           unsigned dim, unsigned vocab,
                                                           const float* __restrict__ grads,
                                                           float* __restrict__ partial) {
   __shared__ float red[2];
   const unsigned k = blockIdx.x;
-  const unsigned id = sorted_ids[k];
-  const bool head = id < vocab && !(k > 0 && sorted_ids[k - 1] == id);
+  const uint4 e = entries[k];
+  const unsigned id = e.x;
+  const bool head = id < vocab && e.z == 0;
   float s = 0.f;
   if (head) {
     const float* pg = grads + size_t(id) * dim;
@@ -180,7 +184,7 @@ int dyhip_sgd_update_rows(dyhip_device* dev, unsigned n_ids, const void* plan, s
   DYHIP_REQUIRE(plan && values && grads && gscale, "null pointer");
   DYHIP_REQUIRE(wd != 0.f && dim < (size_t(1) << 31), "bad weight decay scale or dimension");
   hipLaunchKernelGGL(sgd_rows_kernel, dim3(n_ids), dim3(128), 0, dev->stream, n_ids,
-                     static_cast<const unsigned*>(plan), (unsigned)dim, vocab, values, grads, lr, wd, gscale);
+                     static_cast<const uint4*>(plan), (unsigned)dim, vocab, values, grads, lr, wd, gscale);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
@@ -201,7 +205,7 @@ int dyhip_squared_l2norm_rows(dyhip_device* dev, unsigned n_ids, const void* pla
                 sizeof(float) * n_ids);
   float* partial = static_cast<float*>(ws);
   hipLaunchKernelGGL(sqnorm_rows_kernel, dim3(n_ids), dim3(128), 0, dev->stream, n_ids,
-                     static_cast<const unsigned*>(plan), (unsigned)dim, vocab, grads, partial);
+                     static_cast<const uint4*>(plan), (unsigned)dim, vocab, grads, partial);
   hipLaunchKernelGGL(sum_partials_kernel, dim3(1), dim3(256), 0, dev->stream, n_ids, partial, out);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;

@@ -577,9 +577,10 @@ class Device:
     @staticmethod
     def lookup_plan_parts(plan_words, n):
         """Splits a plan read back as uint32 words into (gid, gpos, roff, rrem): ids grouped by value,
-        their positions, entries of the run before / from each entry.  Each part starts on a 256-byte boundary."""
-        part = (4 * n + 255) // 256 * 256 // 4
-        return tuple(plan_words[q * part:q * part + n] for q in range(4))
+        their positions, entries of the run before / from each entry.  The plan starts with one 16-byte
+        record (id, position, before, from) per grouped entry."""
+        rec = np.asarray(plan_words[:4 * n]).reshape(n, 4)
+        return tuple(np.ascontiguousarray(rec[:, q]) for q in range(4))
 
     def lookup_plan_invalid_ids(self, n_ids, plan):
         """How many ids of the plan were >= vocab (the reduction skips them); synchronises."""
