@@ -230,6 +230,39 @@ def extras_kernels(dev, lib, n_sets=None):
          lambda s: dev.lookup_build_plan_into(s["ids"], V, s["plan"], s["plan_ws"], s["plan_wsb"])),
     ]
     yield "cfg3_lookup", {"vocab": V, "dim": D, "n_ids": n, "unique_ids": uniq, "rotating_buffer_sets": len(sets)}, named, sets
+    # ---- the plan beyond 65535 ids (device-wide radix sort + run offsets) and for keys wider than 16 bits ---------
+    big_n, wide_v = 262144, 200000
+    sets = []
+    for _ in range(n_sets or 4):
+        sets.append({"ids_big": dev.tensor(zipf_ids(rng, big_n, V), np.uint32), "ids_wide": dev.tensor(zipf_ids(rng, n, wide_v), np.uint32)})
+    pb, pbw, pbb = dev.lookup_plan_buffers(big_n, V)
+    pw, pww, pwb = dev.lookup_plan_buffers(n, wide_v)
+    named = [
+        ("lookup_plan, 262144 ids (radix sort + run offsets; bytes = ids read + plan written)", big_n * 20,
+         lambda s: dev.lookup_build_plan_into(s["ids_big"], V, pb, pbw, pbb)),
+        ("lookup_plan, 16384 ids over a vocabulary of 200000 (one kernel, keys of 18 bits)", n * 20,
+         lambda s: dev.lookup_build_plan_into(s["ids_wide"], wide_v, pw, pww, pwb)),
+    ]
+    yield "lookup_plan_other_routes", {"rotating_buffer_sets": len(sets)}, named, sets
+    # ---- cwise with a dimension broadcast at the layer_norm composite's shape (x - mean, x / sigma) ----------------
+    cn, cbd = LN_N, LN_BD
+    da, db_ = (cn, 1, 1, 1, cbd), (1, 1, 1, 1, cbd)
+    S = cn * cbd * 4
+    sets = [{"a": dev.tensor(rng.standard_normal((cbd, cn)).astype(np.float32)),
+             "b": dev.tensor(rng.uniform(0.5, 1.5, cbd).astype(np.float32)), "y": dev.empty((cbd, cn)),
+             "dy": dev.tensor(rng.standard_normal((cbd, cn)).astype(np.float32)),
+             "da": dev.zeros((cbd, cn), pool=lib.POOL_DEDFS), "db": dev.zeros(cbd, pool=lib.POOL_DEDFS)}
+            for _ in range(n_sets or 12)]
+    wsc, wscb = dev.workspace(max(dev.cwise_backward_workspace(da, db_, 1), 256))
+    named = [
+        ("cwise_quotient_fwd(1024 x 4096 by 1 x 4096)", 2 * S + cbd * 4,
+         lambda s: dev.cwise_forward(lib.CWISE_QUOTIENT, da, db_, s["a"], s["b"], s["y"])),
+        ("cwise_quotient_bwd_arg0", 3 * S + cbd * 4,
+         lambda s: dev.cwise_backward(lib.CWISE_QUOTIENT, da, db_, s["a"], s["b"], s["dy"], 0, s["da"], wsc, wscb)),
+        ("cwise_quotient_bwd_arg1(sum over the 1024 dim)", 2 * S + 3 * cbd * 4,
+         lambda s: dev.cwise_backward(lib.CWISE_QUOTIENT, da, db_, s["a"], s["b"], s["dy"], 1, s["db"], wsc, wscb)),
+    ]
+    yield "cwise_dimension_broadcast", {"dims_a": list(da), "dims_b": list(db_), "rotating_buffer_sets": len(sets)}, named, sets
     # ---- cfg 4: PickNegLogSoftmax 50000 x 512 ----------------------------------
     rows, bd = CFG4["rows"], CFG4["bd"]
     X = rows * bd * 4
@@ -1021,6 +1054,10 @@ def main():
                             sweep.sets, args.kernel_reps, use_graph=not args.no_graph)[0]
     for k in table:
         k["frac_of_copy_ceiling"] = round(k["GBps"] / copy["GBps"], 4)
+    # the runtime's own device-to-device copy (hipMemcpyAsync through dyhip_memcpy_d2d: not one of this library's
+    # kernels) on the same tensors, as a ceiling that does not share code with what it is a ceiling for
+    copy_rt = per_kernel_table(dev, [("hipMemcpyAsync", 2 * S_BYTES, lambda b: dev.copy_d2d(b["y"], b["x"], S_BYTES))],
+                               sweep.sets, args.kernel_reps, use_graph=not args.no_graph)[0]
     traffic_table = measured_traffic()
     # Dominant kernel = the device kernel with the largest share of the sweep's device time, as the first row
     # of a kernel-trace summary of the sweep would name it.  cmult_bwd_arg0 and cmult_bwd_arg1 launch the same
@@ -1060,7 +1097,10 @@ def main():
         "wall_ms_per_step": round(wall_ms / args.steps, 5),
         "roofline": roofline, "roofline_longest_entry": roofline_slowest,
         "hbm_copy_ceiling": {"kernel": "copy of one 4096x1024 fp32 tensor (streaming loads and stores)", "bytes": 2 * S_BYTES,
-                             "us": copy["us"], "GBps": copy["GBps"], "frac_of_8TBps": copy["frac_of_8TBps"]},
+                             "us": copy["us"], "GBps": copy["GBps"], "frac_of_8TBps": copy["frac_of_8TBps"],
+                             "runtime_memcpy_d2d": {"what": "hipMemcpyAsync device-to-device on the same rotating tensors",
+                                                    "us": copy_rt["us"], "GBps": copy_rt["GBps"],
+                                                    "frac_of_8TBps": copy_rt["frac_of_8TBps"]}},
         "kernels": table,
         # cfg 5, both paths named: the drop-in one (DyNet's nodes called one at a time, as its executor does) and the
         # time-batched / fused one, which needs a builder-level call sequence (the timesteps of a layer issued together)

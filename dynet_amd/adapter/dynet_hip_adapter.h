@@ -558,6 +558,28 @@ struct PickNegLogSoftmax : public Node {
   }
 };
 
+// Argmax over a vector per batch element (dynet/nodes-argmax.h, dynet/nodes-argmax.cc:26-68); aux_mem = one 64-bit
+// index per batch element (:37-39).  fx is one-hot; backward copies the gradient through when straight_through is set
+// and contributes nothing otherwise.
+struct Argmax : public Node {
+  Argmax(const Dim& dim, unsigned d, bool straight_through) : dim(dim), d(d), straight_through(straight_through) {
+    if (dim.nd != 1) throw std::invalid_argument("Argmax only supports vectors for now");
+    if (d >= dim.nd) throw std::invalid_argument("Cannot compute argmax along that dimension");
+  }
+  Dim dim;
+  unsigned d;
+  bool straight_through;
+  size_t aux_storage_size() const override { return dim.size() / dim[d] * sizeof(long long); }
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    abi_check(dyhip_argmax_onehot_forward(dev.hip, xs[0]->d[d], xs[0]->d.bd, xs[0]->v, static_cast<long long*>(aux_mem),
+                                          fx.v));
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>&, const Tensor&, const Tensor& dEdf,
+                         unsigned, Tensor& dEdxi) const override {
+    if (straight_through) abi_check(dyhip_accumulate(dev.hip, dEdf.d.size(), dEdf.v, dEdxi.v));
+  }
+};
+
 // LogSoftmax (dynet/nodes-softmaxes.cc:127-214); aux_mem = [z | m]
 struct LogSoftmax : public Node {
   explicit LogSoftmax(const Dim& dim) : dim(dim) {}

@@ -235,6 +235,14 @@ __global__ __launch_bounds__(256) void lse_node_bwd_bcast_kernel(size_t n, size_
   if (e < total) tmp[e] = expf(xi[e % n] - fx[e]) * dEdf[e];
 }
 
+// The Argmax node's output (dynet/nodes-argmax.cc:44-55): 1 at each batch element's argmax, 0 elsewhere.  The
+// reference copies the indices to the host and sets the ones one element at a time; here they never leave the device.
+__global__ __launch_bounds__(256) void onehot_kernel(size_t rows, size_t total, const long long* __restrict__ idx,
+                                                     float* __restrict__ fx) {
+  const size_t e = size_t(blockIdx.x) * 256 + threadIdx.x;
+  if (e < total) fx[e] = (long long)(e % rows) == idx[e / rows] ? 1.0f : 0.0f;
+}
+
 // ---- argmax along dim 0, first maximum ---------------------------------------
 __global__ __launch_bounds__(256) void argmax_cols_kernel(size_t rows, const float* __restrict__ x,
                                                           long long* __restrict__ idx) {
@@ -566,6 +574,18 @@ int dyhip_argmax_cols(dyhip_device* dev, size_t rows, unsigned bd, const float* 
   DYHIP_REQUIRE(rows >= 1 && x && idx, "argmax needs a non-empty tensor");
   if (bd == 0) return DYHIP_OK;
   hipLaunchKernelGGL(argmax_cols_kernel, dim3(bd), dim3(256), 0, dev->stream, rows, x, idx);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
+int dyhip_argmax_onehot_forward(dyhip_device* dev, size_t rows, unsigned bd, const float* x, long long* idx, float* fx) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(rows >= 1 && x && idx && fx, "argmax needs a non-empty tensor");
+  if (bd == 0) return DYHIP_OK;
+  hipLaunchKernelGGL(argmax_cols_kernel, dim3(bd), dim3(256), 0, dev->stream, rows, x, idx);
+  DYHIP_CHECK_LAUNCH();
+  const size_t total = rows * size_t(bd);
+  hipLaunchKernelGGL(onehot_kernel, dim3((unsigned)cdiv<size_t>(total, 256)), dim3(256), 0, dev->stream, rows, total, idx, fx);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }

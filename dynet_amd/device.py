@@ -320,11 +320,15 @@ class Device:
         """dims: (d0, d1, d2, d3, bd), column-major with the batch outermost (numpy shape = reversed dims)."""
         _check(cdll.dyhip_cwise_forward(self.handle, _i(op), self._dims5(dims_a), self._dims5(dims_b), _p(a), _p(b), _p(fx)))
 
-    def cwise_backward(self, op, dims_a, dims_b, a, b, dEdf, i, dEdxi):
+    def cwise_backward_workspace(self, dims_a, dims_b, i):
         nb = _sz(0)
+        _check(cdll.dyhip_cwise_backward_workspace(self._dims5(dims_a), self._dims5(dims_b), _u(i), C.byref(nb)))
+        return nb.value
+
+    def cwise_backward(self, op, dims_a, dims_b, a, b, dEdf, i, dEdxi, ws=None, nbytes=None):
         da, db = self._dims5(dims_a), self._dims5(dims_b)
-        _check(cdll.dyhip_cwise_backward_workspace(da, db, _u(i), C.byref(nb)))
-        ws, nbytes = self.workspace(nb.value)
+        if ws is None:
+            ws, nbytes = self.workspace(self.cwise_backward_workspace(dims_a, dims_b, i))
         _check(cdll.dyhip_cwise_backward(self.handle, _i(op), da, db, _p(a), _p(b), _p(dEdf), _u(i), _p(dEdxi), _vp(ws),
                                          _sz(nbytes)))
 
@@ -681,6 +685,9 @@ class Device:
 
     def argmax_cols(self, rows, bd, x, idx):
         _check(cdll.dyhip_argmax_cols(self.handle, _sz(rows), _u(bd), _p(x), _p(idx)))
+
+    def argmax_onehot_forward(self, rows, bd, x, idx, fx):
+        _check(cdll.dyhip_argmax_onehot_forward(self.handle, _sz(rows), _u(bd), _p(x), _p(idx), _p(fx)))
 
     # ---- dynet::gpu helpers -----------------------------------------------
     def dense_to_sparse_assign(self, n, ids, src, trg):

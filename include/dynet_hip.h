@@ -507,6 +507,11 @@ int dyhip_logsumexp_node_backward(dyhip_device* dev, unsigned k, size_t n, unsig
                                   float* dEdxi, void* ws, size_t ws_bytes);
 /* TensorTools::argmax_dev along dim 0 (dynet/tensor.cc:527-538): first maximum, 64-bit indices */
 int dyhip_argmax_cols(dyhip_device* dev, size_t rows, unsigned bd, const float* x, long long* idx);
+/* Argmax::forward_dev_impl over a vector per batch element (dynet/nodes-argmax.cc:44-55): idx (the node's aux_mem,
+ * bd 64-bit indices, :37-39) = argmax along dim 0, fx = 1 at each batch element's argmax and 0 elsewhere.  Nothing is
+ * copied to the host (the reference reads the indices back and sets the ones element by element).  backward
+ * (:57-68) is dyhip_accumulate(dEdf -> dEdxi) for the straight-through estimator and nothing otherwise. */
+int dyhip_argmax_onehot_forward(dyhip_device* dev, size_t rows, unsigned bd, const float* x, long long* idx, float* fx);
 
 /* ---- dynet::gpu::* helpers (dynet/gpu-ops.h:9-15), same argument lists ---- */
 int dyhip_dense_to_sparse_assign(dyhip_device* dev, int n, const unsigned* ids, const float* src, float* trg);

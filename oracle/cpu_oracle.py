@@ -417,6 +417,15 @@ def argmax_cols(rows, bd, x):
     return idx
 
 
+def argmax_onehot_forward(rows, bd, x):
+    """Argmax node: (indices, one-hot output)."""
+    idx = np.empty(bd, np.int64)
+    fx = np.empty((bd, rows), np.float32)
+    _check(_lib.orc_argmax_onehot_forward(C.c_size_t(rows), bd, _fp(_f32(x)), idx.ctypes.data_as(C.POINTER(C.c_longlong)),
+                                          _fp(fx)), "argmax_onehot_forward")
+    return idx, fx
+
+
 # ---- scatter / gather helpers ---------------------------------------------
 def dense_to_sparse_assign(idx, src, trg):
     idx = _u32(idx)

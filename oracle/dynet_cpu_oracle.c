@@ -1082,6 +1082,15 @@ int orc_argmax_cols(size_t rows, unsigned bd, const float* x, long long* idx) {
   return 0;
 }
 
+/* Argmax::forward_dev_impl, dynet/nodes-argmax.cc:44-55: the indices, then fx = 0 with a 1 at
+ * idx[b] + b * rows.  Pinned by tests/test-nodes.cc:1277-1288 ({1.1,2.6,3.3 | 4.0,5.1,6.6} -> 0,0,1,0,0,1). */
+int orc_argmax_onehot_forward(size_t rows, unsigned bd, const float* x, long long* idx, float* fx) {
+  if (orc_argmax_cols(rows, bd, x, idx) != 0) return -1;
+  for (size_t e = 0; e < rows * (size_t)bd; ++e) fx[e] = 0.0f;
+  for (unsigned b = 0; b < bd; ++b) fx[(size_t)idx[b] + (size_t)b * rows] = 1.0f;
+  return 0;
+}
+
 /* ======================================================================== */
 /* scatter/gather helpers: what dynet/gpu-ops.cu:12-166 computes, restated  */
 /* sequentially (the atomics there make the result order-dependent; the     */

@@ -150,6 +150,7 @@ int orc_logsumexp_node_backward(unsigned k, size_t n, unsigned bd, const float* 
                                 const unsigned* bds, const float* fx, const float* dEdf,
                                 unsigned i, float* dEdxi);
 int orc_argmax_cols(size_t rows, unsigned bd, const float* x, long long* idx);
+int orc_argmax_onehot_forward(size_t rows, unsigned bd, const float* x, long long* idx, float* fx);
 
 /* ---- scatter/gather helpers (dynet::gpu::*) ------------------------------ */
 int orc_dense_to_sparse_assign(int n, const unsigned* idx, const float* src, float* trg);

@@ -265,6 +265,35 @@ static void lstm_node_gradients(Fixture& F) {
   }
 }
 
+// ---- tests/test-nodes.cc:1277-1321: argmax_forward, argmax_backward, straight_through_backward ----
+static void argmax_node(Fixture& F) {
+  g_case = "argmax_node";
+  const vector<float> batch_vals = {1.1f, 2.6f, 3.3f, 4.0f, 5.1f, 6.6f};
+  const Dim xd({3}, 2);
+  Tensor x = F.input(xd, batch_vals);
+  vector<const Tensor*> xs = {&x};
+  for (bool st : {false, true}) {
+    Argmax node(xd, 0, st);
+    CHECK(node.aux_storage_size() == 2 * sizeof(long long));
+    Tensor aux = F.dev.allocate_tensor(DeviceMempool::FXS, Dim({4}));  // 16 bytes
+    node.aux_mem = aux.v;
+    Tensor fx = F.dev.allocate_tensor(DeviceMempool::FXS, xd);
+    node.forward_dev_impl(F.dev, xs, fx);
+    CHECK(as_vector(fx) == (vector<float>{0.f, 0.f, 1.f, 0.f, 0.f, 1.f}));
+    // z = sum_batches(dot_product(y, x_)) with x_ = batch_vals: dz/dy = batch_vals
+    Tensor dEdf = F.input(xd, batch_vals, DeviceMempool::DEDFS), dx = F.zeros(xd);
+    node.backward_dev_impl(F.dev, xs, fx, dEdf, 0, dx);
+    CHECK(as_vector(dx) == (st ? batch_vals : vector<float>(6, 0.f)));
+  }
+  bool threw = false;
+  try {
+    Argmax bad(Dim({3, 2}), 0, false);
+  } catch (const std::invalid_argument&) {
+    threw = true;
+  }
+  CHECK(threw);
+}
+
 // ---- tests/test-nodes.cc:854-860 (tanh), :944-960 (rectify, logistic), :1408-1484 (cmult) on {1.1,-2.2,3.3} ----
 static void elementwise_gradients(Fixture& F) {
   const vector<float> param_vals = {1.1f, -2.2f, 3.3f}, param2_vals = {2.2f, 3.4f, -1.2f};
@@ -686,7 +715,7 @@ int main(int argc, char** argv) {
   const std::vector<std::function<void(Fixture&)>> cases = {lstm_node_h_fwd,      lstm_node_c_fwd, lstm_node_gates_fwd,
                                                              lstm_node_gradients,  elementwise_gradients, layer_norm,
                                                              lookup_and_softmax,   random_nodes,    cwise_broadcast,       layer_norm_composite,
-                                                             combine_and_accumulate};
+                                                             combine_and_accumulate, argmax_node};
   for (const auto& c : cases) {
     c(F);
     F.reset();

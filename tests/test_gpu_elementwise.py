@@ -10,7 +10,7 @@ import pytest
 
 from dynet_amd import lib
 from oracle import cpu_oracle as orc
-from util import F32, FWD_RTOL, GRAD_RTOL, assert_close, f32, rms
+from util import assert_shadow, F32, FWD_RTOL, GRAD_RTOL, assert_close, f32, rms
 
 pytestmark = pytest.mark.gpu
 
@@ -211,6 +211,21 @@ def _ln_case(n, bd, seed):
     return rng, x, g, b, dy
 
 
+def _ln_fp64(x, g, b, dy):
+    """y = g (x - mean) / (std + 1e-8) + b per row in fp64 and its analytic gradients: with s = std + eps, q = xc / s,
+    dq = dy g:  dx = dq / s - mean(dq) / s - xc * sum(dq xc) / (n s^2 std);  dg = sum_b dy q;  db = sum_b dy."""
+    x, g, b, dy = (np.asarray(a, np.float64) for a in (x, g, b, dy))
+    n = x.shape[1]
+    xc = x - x.mean(axis=1, keepdims=True)
+    std = np.sqrt((xc * xc).mean(axis=1, keepdims=True))
+    s = std + np.float64(np.float32(1e-8))
+    q = xc / s
+    dq = dy * g
+    dxc = dq / s - xc * (dq * xc).sum(axis=1, keepdims=True) / (n * s * s * std)
+    dx = dxc - dxc.mean(axis=1, keepdims=True)
+    return g * q + b, dx, (dy * q).sum(axis=0), dy.sum(axis=0)
+
+
 @pytest.mark.parametrize("n,bd", [(1024, 4096), (2048, 64), (512, 33), (256, 5), (64, 1), (12, 7), (1027, 9),
                                   (4096, 6), (3, 1), (4096, 1024), (4100, 300), (37, 1000), (70, 2051),
                                   (8192, 70), (16384, 33), (2052, 19), (12288, 5), (16388, 9)])
@@ -229,6 +244,13 @@ def test_layer_norm_forward_backward(dev, n, bd):
     assert_close(dxt.numpy(), wx, GRAD_RTOL, "layer_norm dx", floor=1.0)
     assert_close(dgt.numpy(), wg, GRAD_RTOL, "layer_norm dg", floor=np.sqrt(bd))
     assert_close(dbt.numpy(), wb, GRAD_RTOL, "layer_norm db", floor=np.sqrt(bd))
+    # and per element against the fp64 value of the same fp32 inputs: the device result must be as close to it as
+    # the CPU path is (within a small factor), so that no kernel hides behind the floor of the relative bars above
+    y64, dx64, dg64, db64 = _ln_fp64(x, g, b, dy)
+    assert_shadow(yt.numpy(), ref, y64, "layer_norm fwd vs fp64", rel_min=1e-3)
+    assert_shadow(dxt.numpy(), wx, dx0.astype(np.float64) + dx64, "layer_norm dx vs fp64", rel_min=1e-2)
+    assert_shadow(dgt.numpy(), wg, dg0.astype(np.float64) + dg64, "layer_norm dg vs fp64", k=6.0, rel_min=1.0)
+    assert_shadow(dbt.numpy(), wb, db0.astype(np.float64) + db64, "layer_norm db vs fp64", k=6.0, rel_min=1.0)
     # one argument at a time, as Node::backward is called
     dxt2 = dev.tensor(dx0)
     dev.layer_norm_backward(n, bd, xt, gt, dyt, dx=dxt2)

@@ -1160,6 +1160,24 @@ def test_argmax(dev, golden):
     assert idx.numpy().tobytes() == orc.argmax_cols(5000, 9, x).tobytes()
 
 
+def test_argmax_node(dev, golden):
+    """The Argmax node (dynet/nodes-argmax.cc:44-68): one-hot forward with the reference test's vector, bit-exact against
+    the oracle on a larger case with ties, straight-through backward = accumulate."""
+    t = golden["node_values"]["argmax_node"]
+    idx, fx = dev.empty(t["bd"], np.int64), dev.empty((t["bd"], t["rows"]))
+    dev.argmax_onehot_forward(t["rows"], t["bd"], dev.tensor(f32(t["x"])), idx, fx)
+    assert list(fx.numpy().ravel()) == t["expected"]
+    dx = dev.zeros((t["bd"], t["rows"]), pool=lib.POOL_DEDFS)
+    dev.accumulate(dev.tensor(f32(t["x"])), dx)        # straight-through: dEdxi += dEdf, with dEdf = x_ = batch_vals
+    assert list(dx.numpy().ravel()) == list(f32(t["straight_through_dx"]))
+    rng = np.random.default_rng(13)
+    x = f32(np.round(rng.standard_normal((300, 1001)) * 2))  # many ties: the first maximum wins
+    idx, fx = dev.empty(300, np.int64), dev.empty((300, 1001))
+    dev.argmax_onehot_forward(1001, 300, dev.tensor(x), idx, fx)
+    want_idx, want_fx = orc.argmax_onehot_forward(1001, 300, x)
+    assert idx.numpy().tobytes() == want_idx.tobytes() and fx.numpy().tobytes() == want_fx.tobytes()
+
+
 # ---------------------------------------------------------------------------
 # dynet::gpu helpers, parameter copy, trainer
 # ---------------------------------------------------------------------------

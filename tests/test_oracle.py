@@ -677,6 +677,16 @@ def test_argmax_golden(golden):
     assert list(orc.argmax_cols(4, 1, f32([3, 7, 7, 1]))) == [1]  # first maximum on ties
 
 
+def test_argmax_node_golden(golden):
+    t = golden["node_values"]["argmax_node"]
+    idx, fx = orc.argmax_onehot_forward(t["rows"], t["bd"], f32(t["x"]))
+    assert list(fx.ravel()) == t["expected"] and list(idx) == [2, 2]
+    rng = np.random.default_rng(12)
+    x = f32(rng.standard_normal((7, 13)))
+    idx, fx = orc.argmax_onehot_forward(13, 7, x)
+    assert np.array_equal(idx, np.argmax(x, axis=1)) and np.array_equal(fx, np.eye(13, dtype=np.float32)[idx])
+
+
 # ---------------------------------------------------------------------------
 # scatter/gather helpers, parameter copy, trainer
 # ---------------------------------------------------------------------------
