@@ -402,7 +402,8 @@ __global__ __launch_bounds__(256 * TILES) void lstm_step_fwd_kernel(unsigned H, 
                                                                     const float* __restrict__ bias,
                                                                     const float* __restrict__ c_prev, int mode,
                                                                     float* gates, float* __restrict__ c,
-                                                                    float* __restrict__ h, float* __restrict__ hp) {
+                                                                    float* __restrict__ h, float* __restrict__ hp,
+                                                                    const float* __restrict__ mask_h) {
   constexpr int UB = 8 * TILES;       // hidden units of a block (its 32*TILES weight rows are their four gate rows)
   constexpr int ROWS = 32 * TILES;
   __shared__ float red[4 * ROWS * kStepPitchR];
@@ -423,6 +424,9 @@ __global__ __launch_bounds__(256 * TILES) void lstm_step_fwd_kernel(unsigned H, 
     xq[q] = xproj != nullptr ? xproj[size_t(lcol) * 4 * H + ej + size_t(q) * H] : 0.f;
   }
   const float cp = c_prev != nullptr ? c_prev[size_t(lcol) * H + ej] : 0.f;
+  // the recurrent dropout mask of the sequence (H x B): the next timestep multiplies Wh by h (.) mask_h, so the packed
+  // copy of h that it reads is written masked; the plain h (the layer's output) is not
+  const float mh = mask_h != nullptr ? mask_h[size_t(lcol) * H + ej] : 1.f;
 
   if (wave < 4) {
     stepx16 acc0 = {0}, acc1 = {0};
@@ -467,7 +471,7 @@ __global__ __launch_bounds__(256 * TILES) void lstm_step_fwd_kernel(unsigned H, 
   c[s0] = cv;
   h[s0] = hv;
   // h again, as the next timestep's packed operand: unit ej is k = 8*(TILES*rp + tile) + u
-  if (hp != nullptr) hp[((size_t(ct) * (H / 8) + TILES * rp + tile) * 64 + (u / 4) * 32 + col) * 4 + u % 4] = hv;
+  if (hp != nullptr) hp[((size_t(ct) * (H / 8) + TILES * rp + tile) * 64 + (u / 4) * 32 + col) * 4 + u % 4] = hv * mh;
 }
 
 // ---- single-launch backward step: recurrent product Wh^T * dpre_{t+1} and the cell backward of step t -----------
@@ -523,7 +527,8 @@ __global__ __launch_bounds__(512) void lstm_step_bwd_kernel(unsigned H, unsigned
                                                             const float* __restrict__ c_prev,
                                                             const float* __restrict__ dh_in, const float* dc_in,
                                                             float* __restrict__ dpre, float* dc_prev,
-                                                            float* __restrict__ dpre_p) {
+                                                            float* __restrict__ dpre_p,
+                                                            const float* __restrict__ mask_h) {
   __shared__ float red[4 * 16 * kStepPitchR];
   const unsigned RT = H / 16;
   const unsigned rt = blockIdx.x % RT, ct = blockIdx.x / RT;  // ct: pair of 16-column tiles
@@ -539,6 +544,8 @@ __global__ __launch_bounds__(512) void lstm_step_bwd_kernel(unsigned H, unsigned
   const float cv = c[s0], dhv = dh_in[s0];
   const float cpv = c_prev != nullptr ? c_prev[s0] : 0.f;
   const float dcv_in = dc_in != nullptr ? dc_in[s0] : 0.f;
+  // recurrent dropout: timestep t+1 multiplied Wh by h_t (.) mask_h, so its gradient reaches h_t through the mask
+  const float mh = mask_h != nullptr ? mask_h[s0] : 1.f;
 
   if (wave < 4 && dpre_next_p != nullptr) {
     const unsigned G = H / 4, gq = G / 4, g_first = wave * gq;  // groups of 16 k; a quarter of the depth per wave
@@ -597,7 +604,7 @@ __global__ __launch_bounds__(512) void lstm_step_bwd_kernel(unsigned H, unsigned
     float rec = red[eu * kStepPitchR + col];
 #pragma unroll
     for (int w = 1; w < 4; ++w) rec += red[(w * 16 + eu) * kStepPitchR + col];
-    dh += rec;
+    dh += mask_h != nullptr ? rec * mh : rec;
   }
   const float gi = gt[0], gf = gt[1], go = gt[2], gg = gt[3];
   const float t = tanh_accurate(cv);
@@ -1215,6 +1222,14 @@ int dyhip_lstm_step_backward_packed(dyhip_device* dev, unsigned H, unsigned B, c
                                     const float* dpre_next_packed16, const float* gates, const float* c,
                                     const float* c_tm1, const float* dh, const float* dc, float* dpre, float* dc_tm1,
                                     float* dpre_packed16) {
+  return dyhip_lstm_step_backward_packed_dropout(dev, H, B, packed_WhT16, dpre_next_packed16, gates, c, c_tm1, dh, dc,
+                                                 nullptr, dpre, dc_tm1, dpre_packed16);
+}
+
+int dyhip_lstm_step_backward_packed_dropout(dyhip_device* dev, unsigned H, unsigned B, const float* packed_WhT16,
+                                            const float* dpre_next_packed16, const float* gates, const float* c,
+                                            const float* c_tm1, const float* dh, const float* dc, const float* mask_h,
+                                            float* dpre, float* dc_tm1, float* dpre_packed16) {
   DYHIP_CHECK_DEV(dev);
   int ok = 0;
   dyhip_lstm_step_supported(dev, H, B, &ok);
@@ -1223,7 +1238,7 @@ int dyhip_lstm_step_backward_packed(dyhip_device* dev, unsigned H, unsigned B, c
   DYHIP_REQUIRE(dpre_next_packed16 == nullptr || packed_WhT16 != nullptr, "LSTM step: packed weights and their operand come together");
   DYHIP_REQUIRE(all_aligned16({packed_WhT16, dpre_next_packed16}), "LSTM step: weights and operands must be 16-byte aligned");
   hipLaunchKernelGGL(lstm_step_bwd_kernel, dim3((H / 16) * cdiv<unsigned>(B, 32)), dim3(512), 0, dev->stream, H, B,
-                     packed_WhT16, dpre_next_packed16, gates, c, c_tm1, dh, dc, dpre, dc_tm1, dpre_packed16);
+                     packed_WhT16, dpre_next_packed16, gates, c, c_tm1, dh, dc, dpre, dc_tm1, dpre_packed16, mask_h);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
@@ -1243,7 +1258,7 @@ int dyhip_lstm_pack_state(dyhip_device* dev, unsigned rows, unsigned B, const fl
 static int step_forward(dyhip_device* dev, unsigned I, unsigned H, unsigned B, const float* packed_Wx, const float* x,
                         const float* packed_Wh, const float* h_tm1, bool states_packed, const float* xproj,
                         const float* b, const float* c_tm1, int logistic_mode, float* gates, float* c, float* h,
-                        float* hp_out) {
+                        float* hp_out, const float* mask_h = nullptr) {
   int ok = 0;
   dyhip_lstm_step_supported(dev, H, B, &ok);
   DYHIP_REQUIRE(ok, "LSTM step: unsupported hidden (%u) or batch (%u) size", H, B);
@@ -1262,7 +1277,7 @@ static int step_forward(dyhip_device* dev, unsigned I, unsigned H, unsigned B, c
   const dim3 grid(two ? blocks2 : blocks2 * 2), block(two ? 512 : 256);
 #define DYHIP_STEP(PLAIN, TILES)                                                                                     \
   hipLaunchKernelGGL((lstm_step_fwd_kernel<PLAIN, TILES>), grid, block, 0, dev->stream, H, B, op0, op1, xproj, b, c_tm1, \
-                     logistic_mode, gates, c, h, hp_out)
+                     logistic_mode, gates, c, h, hp_out, mask_h)
   if (states_packed) {
     if (two) DYHIP_STEP(false, 2);
     else DYHIP_STEP(false, 1);
@@ -1293,6 +1308,18 @@ int dyhip_lstm_step_forward_packed(dyhip_device* dev, unsigned H, unsigned B, co
                 "LSTM step: the recurrent weights, the packed state and c_tm1 come together (all null = zero state)");
   return step_forward(dev, 0, H, B, nullptr, nullptr, packed_Wh, h_tm1_packed, true, xproj, b, c_tm1, logistic_mode,
                       gates, c, h, h_packed);
+}
+
+int dyhip_lstm_step_forward_packed_dropout(dyhip_device* dev, unsigned H, unsigned B, const float* packed_Wh,
+                                           const float* h_tm1_packed, const float* xproj, const float* b,
+                                           const float* c_tm1, const float* mask_h, int logistic_mode, float* gates,
+                                           float* c, float* h, float* h_packed) {
+  DYHIP_CHECK_DEV(dev);
+  DYHIP_REQUIRE(xproj != nullptr, "LSTM step: null tensor pointer");
+  DYHIP_REQUIRE((packed_Wh == nullptr) == (h_tm1_packed == nullptr) && (packed_Wh == nullptr) == (c_tm1 == nullptr),
+                "LSTM step: the recurrent weights, the packed state and c_tm1 come together (all null = zero state)");
+  return step_forward(dev, 0, H, B, nullptr, nullptr, packed_Wh, h_tm1_packed, true, xproj, b, c_tm1, logistic_mode,
+                      gates, c, h, h_packed, mask_h);
 }
 
 int dyhip_lstm_step_forward_x(dyhip_device* dev, unsigned I, unsigned H, unsigned B, const float* packed_Wx,

@@ -470,7 +470,12 @@ class Device:
         _check(cdll.dyhip_lstm_pack_state(self.handle, _u(rows), _u(B), _p(v), _p(packed)))
 
     def lstm_step_forward_packed(self, H, B, packed_Wh, h_tm1_packed, xproj, b, c_tm1, gates, c, h, h_packed,
-                                 logistic_mode=lib.LOGISTIC_PACKET):
+                                 logistic_mode=lib.LOGISTIC_PACKET, mask_h=None):
+        if mask_h is not None:  # recurrent dropout: h_packed = h (.) mask_h
+            _check(cdll.dyhip_lstm_step_forward_packed_dropout(self.handle, _u(H), _u(B), _p(packed_Wh), _p(h_tm1_packed),
+                                                               _p(xproj), _p(b), _p(c_tm1), _p(mask_h), _i(logistic_mode),
+                                                               _p(gates), _p(c), _p(h), _p(h_packed)))
+            return
         _check(cdll.dyhip_lstm_step_forward_packed(self.handle, _u(H), _u(B), _p(packed_Wh), _p(h_tm1_packed), _p(xproj),
                                                    _p(b), _p(c_tm1), _i(logistic_mode), _p(gates), _p(c), _p(h),
                                                    _p(h_packed)))
@@ -501,8 +506,14 @@ class Device:
         _check(cdll.dyhip_lstm_pack_state16(self.handle, _u(rows), _u(B), _p(v), _p(packed)))
 
     def lstm_step_backward_packed(self, H, B, packed_WhT16, dpre_next_packed16, gates, c, c_tm1, dh, dc, dpre, dc_tm1,
-                                  dpre_packed16):
+                                  dpre_packed16, mask_h=None):
         """One launch per backward timestep: Wh^T * dpre_{t+1} over its whole depth and the cell backward of step t."""
+        if mask_h is not None:  # recurrent dropout: the product reaches dh through the mask
+            _check(cdll.dyhip_lstm_step_backward_packed_dropout(self.handle, _u(H), _u(B), _p(packed_WhT16),
+                                                                _p(dpre_next_packed16), _p(gates), _p(c), _p(c_tm1),
+                                                                _p(dh), _p(dc), _p(mask_h), _p(dpre), _p(dc_tm1),
+                                                                _p(dpre_packed16)))
+            return
         _check(cdll.dyhip_lstm_step_backward_packed(self.handle, _u(H), _u(B), _p(packed_WhT16),
                                                     _p(dpre_next_packed16), _p(gates), _p(c), _p(c_tm1), _p(dh), _p(dc),
                                                     _p(dpre), _p(dc_tm1), _p(dpre_packed16)))

@@ -22,6 +22,14 @@ What differs from DyNet's node-at-a-time execution (results agree to fp32 roundi
     on chunk k-1).  It paid off while a timestep's kernels left most of the GPU idle; the packed kernels keep the
     matrix cores of every CU busy on their own, two of them side by side only slow each other, and the default is
     one queue.
+
+Dropout (``dropout`` / ``dropout_h`` > 0) is CompactVanillaLSTMBuilder's (dynet/lstm.cc:964-982,1068-1073): per layer
+one input mask (d_in x B) and one recurrent mask (H x B), Bernoulli(retention) / retention, drawn once per sequence,
+i.e. once per step here, on the device; the gates see x (.) mask_x and h_tm1 (.) mask_h at every timestep.  The node
+path hands the masks to the gates node.  The fused path multiplies the layer's input by mask_x once for all
+timesteps before the input product (and dx by it after the transposed product), the one-launch timesteps take mask_h
+as an argument (the packed copy of h for the next timestep is written masked; the recurrent gradient passes through
+the mask), and the weight gradients over all timesteps read the masked copies.
 """
 import numpy as np
 
@@ -33,10 +41,14 @@ class LstmLM:
     """V-word LM: embedding E, L layers of hidden H, batch B, T timesteps per step."""
 
     def __init__(self, dev, V, E, H, L, B, T, seed=0, lr=0.1, clip=5.0, time_batched=True, params=None, path="fused",
-                 overlap=None, chunk=7, single_launch=None):
+                 overlap=None, chunk=7, single_launch=None, dropout=0.0, dropout_h=None):
         assert path in ("fused", "nodes")
+        self.dropout = float(dropout)
+        self.dropout_h = self.dropout if dropout_h is None else float(dropout_h)
+        assert 0.0 <= self.dropout < 1.0 and 0.0 <= self.dropout_h < 1.0
+        self.use_dropout = self.dropout > 0.0 or self.dropout_h > 0.0
         self.overlap = False if overlap is None else bool(overlap)
-        self.overlap = self.overlap and path == "fused" and L > 1
+        self.overlap = self.overlap and path == "fused" and L > 1 and not self.use_dropout
         self.chunk = max(1, int(chunk))
         self.dev, self.V, self.E, self.H, self.L, self.B, self.T = dev, V, E, H, L, B, T
         self.lr, self.clip, self.time_batched, self.path = float(lr), float(clip), bool(time_batched), path
@@ -76,6 +88,17 @@ class LstmLM:
         self.aux = dev.empty((3 * N,), pool=FXS)  # [z | m | ids] of PickNegLogSoftmax
         self.errs = dev.empty((N,), pool=FXS)
         self.loss = dev.empty((1,), pool=FXS)
+        # dropout masks of the sequence, and the masked copies of every layer's input and state that the weight
+        # gradients over all timesteps (and the fused path's input product) read
+        self.mask_x, self.mask_h, self.xm, self.hm = [], [], [], []
+        if self.use_dropout:
+            for l in range(L):
+                d_in = E if l == 0 else H
+                self.mask_x.append(dev.empty((B, d_in), pool=FXS))
+                self.mask_h.append(dev.empty((B, H), pool=FXS))
+                self.xm.append(dev.empty((T, B, d_in), pool=FXS))
+                self.hm.append(dev.empty((T, B, H), pool=FXS))
+            self.dh_rec = dev.empty((B, H), pool=FXS)  # (Wh^T dpre) of one timestep where no one-launch step exists
         # gradients of the forward values (DEDFS pool), zeroed at the start of every backward pass
         self.de_begin = dev.pool(DE).used()
         self.d_errs = dev.empty((N,), pool=DE)
@@ -150,6 +173,24 @@ class LstmLM:
     def _t(self, buf, t, width):
         return buf.offset(t * self.B * width, (self.B, width))
 
+    def draw_masks(self):
+        """set_dropout_masks (dynet/lstm.cc:964-982): per layer the input mask, then the recurrent mask, each
+        random_bernoulli(retention, 1 / retention) with one column per batch element."""
+        for l in range(self.L):
+            self.dev.randomize_bernoulli(self.mask_x[l], 1.0 - self.dropout, 1.0 / (1.0 - self.dropout))
+            self.dev.randomize_bernoulli(self.mask_h[l], 1.0 - self.dropout_h, 1.0 / (1.0 - self.dropout_h))
+
+    def _x_of(self, l):
+        """(input of layer l over all timesteps as the gates see it, its width)."""
+        if self.use_dropout:
+            return self.xm[l], (self.H if l > 0 else self.E)
+        return (self.h[l - 1], self.H) if l > 0 else (self.emb, self.E)
+
+    def _mask_inputs(self, q, l):
+        """xm[l] = input of layer l (.) mask_x[l], the mask broadcast over the timesteps."""
+        x, d_in = (self.h[l - 1], self.H) if l > 0 else (self.emb, self.E)
+        q.cmult_forward(self.B * d_in, self.T, 1, x, self.mask_x[l], self.xm[l])
+
     def forward(self):
         d, V, E, H, L, B, T, N = self.dev, self.V, self.E, self.H, self.L, self.B, self.T, self.N
         d.lookup_forward(None, self.ids, E, V, self.p["C"], self.emb)
@@ -173,9 +214,14 @@ class LstmLM:
                 q.lstm_step_forward_packed(H, B, self.Wh_packed[l] if t > 0 else None, hp[(t - 1) % 2] if t > 0 else None,
                                            g, self.p[f"b{l}"], self._t(self.c[l], t - 1, H) if t > 0 else None, g,
                                            self._t(self.c[l], t, H), self._t(self.h[l], t, H),
-                                           hp[t % 2] if t + 1 < self.T else None)
+                                           hp[t % 2] if t + 1 < self.T else None,
+                                           mask_h=self.mask_h[l] if self.use_dropout else None)
             elif t > 0:
-                n = q.lstm_recurrent_forward(H, B, self.p[f"Wh{l}"], self._t(self.h[l], t - 1, H), self.rec_f[l],
+                h_tm1 = self._t(self.h[l], t - 1, H)
+                if self.use_dropout:  # the recurrent product reads h_tm1 (.) mask_h
+                    q.cmult_forward(B * H, 1, 1, h_tm1, self.mask_h[l], self._t(self.hm[l], t - 1, H))
+                    h_tm1 = self._t(self.hm[l], t - 1, H)
+                n = q.lstm_recurrent_forward(H, B, self.p[f"Wh{l}"], h_tm1, self.rec_f[l],
                                              self.rec_f_bytes)
                 q.lstm_cell_forward(H, B, g, self.p[f"b{l}"], self.rec_f[l], n, self._t(self.c[l], t - 1, H), g,
                                     self._t(self.c[l], t, H), self._t(self.h[l], t, H))
@@ -191,9 +237,13 @@ class LstmLM:
                 d.lstm_pack_recurrent_transposed16(H, self.p[f"Wh{l}"], self.WhT_packed[l])
         if not self.overlap:
             for l in range(L):
-                x, d_in = (self.h[l - 1], H) if l > 0 else (self.emb, E)
+                if self.use_dropout:
+                    self._mask_inputs(d, l)
+                x, d_in = self._x_of(l)
                 d.gemm_nn(4 * H, N, d_in, self.p[f"Wx{l}"], x, 0.0, self.gates[l])  # Wx*x of every timestep
                 self._cell_steps_forward(d, l, 0, T)
+                if self.use_dropout and self.single_launch and T > 1:  # for dWh: h (.) mask_h of every timestep
+                    d.cmult_forward(B * H, T, 1, self.h[l], self.mask_h[l], self.hm[l])
             return
         # pipeline over time chunks: queue l runs layer l, one chunk behind queue l-1
         qs = self.queues
@@ -220,10 +270,21 @@ class LstmLM:
                 h_tm1 = self._t(self.h[l], t - 1, H) if t > 0 else self.h0
                 c_tm1 = self._t(self.c[l], t - 1, H) if t > 0 else self.h0
                 g, c, h = self._t(self.gates[l], t, 4 * H), self._t(self.c[l], t, H), self._t(self.h[l], t, H)
-                d.lstm_gates_forward([x], [d_in], H, B, h_tm1, self.p[f"Wx{l}"], self.p[f"Wh{l}"], self.p[f"b{l}"], g)
+                d.lstm_gates_forward([x], [d_in], H, B, h_tm1, self.p[f"Wx{l}"], self.p[f"Wh{l}"], self.p[f"b{l}"], g,
+                                     **self._node_masks(l))
                 d.lstm_c_forward(H, B, c_tm1, g, c)
                 d.lstm_h_forward(H, B, c, g, h)
                 x, d_in = h, H
+        if self.use_dropout and self.time_batched:  # the masked copies for the weight gradients over all timesteps
+            for l in range(L):
+                self._mask_inputs(d, l)
+                if T > 1:
+                    d.cmult_forward(B * H, T, 1, self.h[l], self.mask_h[l], self.hm[l])
+
+    def _node_masks(self, l):
+        if not self.use_dropout:
+            return {}
+        return {"mask_x": self.mask_x[l], "mask_x_bd": self.B, "mask_h": self.mask_h[l], "mask_h_bd": self.B}
 
     def backward(self):
         d, V, E, H, L, B, T, N = self.dev, self.V, self.E, self.H, self.L, self.B, self.T, self.N
@@ -259,7 +320,19 @@ class LstmLM:
                                             None if first else self._t(self.c[l], t - 1, H), self._t(self.d_h[l], t, H),
                                             None if last else self._t(self.d_c[l], t, H), dpre,
                                             None if first else self._t(self.d_c[l], t - 1, H),
-                                            None if first else self.dpre_packed[l][t % 2])
+                                            None if first else self.dpre_packed[l][t % 2],
+                                            mask_h=self.mask_h[l] if self.use_dropout else None)
+                continue
+            if self.use_dropout:
+                # no one-launch step at this size: (Wh^T dpre) as a plain product, through the mask, into d_h[t-1]
+                q.lstm_cell_backward(H, B, self._t(self.gates[l], t, 4 * H), self._t(self.c[l], t, H),
+                                     None if first else self._t(self.c[l], t - 1, H), self._t(self.d_h[l], t, H), None, 0,
+                                     None if last else self._t(self.d_c[l], t, H), dpre,
+                                     None if first else self._t(self.d_c[l], t - 1, H))
+                if not first:
+                    q.gemm_tn(H, B, 4 * H, Wh, dpre, 0.0, self.dh_rec)
+                    q.cmult_forward(B * H, 1, 1, self.dh_rec, self.mask_h[l], self.dh_rec)
+                    q.accumulate(self.dh_rec, self._t(self.d_h[l], t - 1, H))
                 continue
             args = (H, B, self._t(self.gates[l], t, 4 * H), self._t(self.c[l], t, H),
                     None if first else self._t(self.c[l], t - 1, H), self._t(self.d_h[l], t, H),
@@ -271,10 +344,11 @@ class LstmLM:
 
     def _weight_grads(self, q, l):
         E, H, B, T, N = self.E, self.H, self.B, self.T, self.N
-        x, d_in = (self.h[l - 1], H) if l > 0 else (self.emb, E)
+        x, d_in = self._x_of(l)
         q.gemm_nt_acc(4 * H, d_in, N, self.d_pre[l], x, self.g[f"Wx{l}"])
         if T > 1:
-            q.gemm_nt_acc(4 * H, H, N - B, self._t(self.d_pre[l], 1, 4 * H), self.h[l], self.g[f"Wh{l}"])
+            q.gemm_nt_acc(4 * H, H, N - B, self._t(self.d_pre[l], 1, 4 * H), self.hm[l] if self.use_dropout else self.h[l],
+                          self.g[f"Wh{l}"])
         q.csum_backward(4 * H, 1, N, self.d_pre[l], 0, self.g[f"b{l}"])
 
     def _backward_layers_fused(self):
@@ -285,6 +359,8 @@ class LstmLM:
                 self._cell_steps_backward(d, l, 0, T)
                 d_in, dx = (H, self.d_h[l - 1]) if l > 0 else (E, self.d_emb)
                 d.gemm_tn(d_in, N, 4 * H, self.p[f"Wx{l}"], self.d_pre[l], 0.0, dx)
+                if self.use_dropout:  # the gradient reaches the layer's input through mask_x
+                    d.cmult_forward(B * d_in, T, 1, dx, self.mask_x[l], dx)
                 self._weight_grads(d, l)
             return
         # pipeline, newest chunk first: the top layer runs on the device queue (it owns d_h[L-1]),
@@ -327,6 +403,19 @@ class LstmLM:
                     x, d_in, dx = self._t(self.h[l - 1], t, H), H, self._t(self.d_h[l - 1], t, H)
                 else:
                     x, d_in, dx = self._t(self.emb, t, E), E, self._t(self.d_emb, t, E)
+                if self.use_dropout:
+                    # the gates node's own backward: it applies the masks to dx / dh and to the operands of dWx / dWh
+                    mk = self._node_masks(l)
+                    args = ([x], [d_in], H, B, h_tm1, self.p[f"Wx{l}"], self.p[f"Wh{l}"], g, dg)
+                    d.lstm_gates_backward(*args, 0, dx, dpre=dpre, **mk)
+                    if t > 0:
+                        d.lstm_gates_backward(*args, 1, self._t(self.d_h[l], t - 1, H), dpre=dpre, **mk)
+                    if not self.time_batched:
+                        d.lstm_gates_backward(*args, 2, self.g[f"Wx{l}"], dpre=dpre, **mk)
+                        if t > 0:
+                            d.lstm_gates_backward(*args, 3, self.g[f"Wh{l}"], dpre=dpre, **mk)
+                        d.lstm_gates_backward(*args, 4, self.g[f"b{l}"], dpre=dpre, **mk)
+                    continue
                 d.gemm_tn_acc(d_in, B, 4 * H, self.p[f"Wx{l}"], dpre, dx)
                 if t > 0:
                     d.gemm_tn_acc(H, B, 4 * H, self.p[f"Wh{l}"], dpre, self._t(self.d_h[l], t - 1, H))
@@ -337,10 +426,11 @@ class LstmLM:
                     d.csum_backward(4 * H, 1, B, dpre, 0, self.g[f"b{l}"])
         if self.time_batched:
             for l in range(L):
-                x, d_in = (self.h[l - 1], H) if l > 0 else (self.emb, E)
+                x, d_in = self._x_of(l)
                 d.gemm_nt_acc(4 * H, d_in, N, self.d_pre[l], x, self.g[f"Wx{l}"])
                 if T > 1:
-                    d.gemm_nt_acc(4 * H, H, N - B, self._t(self.d_pre[l], 1, 4 * H), self.h[l], self.g[f"Wh{l}"])
+                    d.gemm_nt_acc(4 * H, H, N - B, self._t(self.d_pre[l], 1, 4 * H),
+                                  self.hm[l] if self.use_dropout else self.h[l], self.g[f"Wh{l}"])
                 d.csum_backward(4 * H, 1, N, self.d_pre[l], 0, self.g[f"b{l}"])
 
     def update(self):
@@ -354,6 +444,8 @@ class LstmLM:
     def issue(self):
         """The whole step on the device stream (ids and labels already staged)."""
         self.dev.lookup_build_plan_into(self.ids, self.V, self.plan, self.plan_ws, self.plan_ws_bytes)
+        if self.use_dropout:
+            self.draw_masks()
         self.forward()
         self.backward()
         self.update()
@@ -395,6 +487,12 @@ class LstmLM:
         if not np.isfinite(nrm):
             raise RuntimeError("Magnitude of gradient is bad: %r" % nrm)
         return nrm
+
+    def get_masks(self):
+        """The dropout masks of the last step, per layer (mask_x[B, d_in], mask_h[B, H]); None without dropout."""
+        if not self.use_dropout:
+            return None
+        return [(self.mask_x[l].numpy(), self.mask_h[l].numpy()) for l in range(self.L)]
 
     def get_params(self):
         return {n: t.numpy() for n, t in self.p.items()}

@@ -322,8 +322,10 @@ int dyhip_lstm_h_backward(dyhip_device* dev, unsigned H, unsigned B, const float
  *                                  and dc_tm1
  *   dyhip_lstm_recurrent_backward: Wh^T * dpre_t as slices for the t-1 call.
  * Weight gradients are then GEMMs over all timesteps (dyhip_gemm_nt with K = T*B), dx is
- * dyhip_gemm_tn(Wx, dpre) and db a batch reduction of dpre.  No dropout masks on this
- * path.  gates may alias xproj (each element is read before it is written).  rec/splits
+ * dyhip_gemm_tn(Wx, dpre) and db a batch reduction of dpre.  These two-call entry points take
+ * no dropout masks (a caller applies the builder's masks around them: h_tm1 (.) mask_h before
+ * dyhip_lstm_recurrent_forward, the product of dyhip_gemm_tn(Wh, dpre) times mask_h into dh;
+ * the one-launch timesteps further down take the recurrent mask as an argument).  gates may alias xproj (each element is read before it is written).  rec/splits
  * = NULL/0 and c_tm1 = NULL stand for the zero initial state (dynet/lstm.cc:1060-1061);
  * dc = NULL for the last timestep, dc_tm1 = NULL for the first. */
 int dyhip_lstm_cell_workspace(dyhip_device* dev, unsigned H, unsigned B, size_t* fwd_bytes, size_t* bwd_bytes);
@@ -390,6 +392,20 @@ int dyhip_lstm_step_backward_packed(dyhip_device* dev, unsigned H, unsigned B, c
                                     const float* dpre_next_packed16, const float* gates, const float* c,
                                     const float* c_tm1, const float* dh, const float* dc, float* dpre, float* dc_tm1,
                                     float* dpre_packed16);
+/* The two single-launch timesteps with the recurrent dropout mask of CompactVanillaLSTMBuilder (dynet/lstm.cc:964-982:
+ * one mask per layer and sequence, H x B, already scaled by 1 / retention; the node applies it as h_tm1 (.) mask_h,
+ * dynet/nodes-lstm.cc:178-198, and hands the gradient back through it, :448-470).  Forward: h is written plain,
+ * h_packed = h (.) mask_h, which is what the next timestep multiplies Wh by.  Backward: dh_t = dh + (Wh^T * dpre_{t+1})
+ * (.) mask_h.  mask_h = NULL: the calls above.  The input mask is applied by the caller to x before the product over
+ * all timesteps (dyhip_cmult_forward with the mask as the batch-1 argument) and to dx after it. */
+int dyhip_lstm_step_forward_packed_dropout(dyhip_device* dev, unsigned H, unsigned B, const float* packed_Wh,
+                                           const float* h_tm1_packed, const float* xproj, const float* b,
+                                           const float* c_tm1, const float* mask_h, int logistic_mode, float* gates,
+                                           float* c, float* h, float* h_packed);
+int dyhip_lstm_step_backward_packed_dropout(dyhip_device* dev, unsigned H, unsigned B, const float* packed_WhT16,
+                                            const float* dpre_next_packed16, const float* gates, const float* c,
+                                            const float* c_tm1, const float* dh, const float* dc, const float* mask_h,
+                                            float* dpre, float* dc_tm1, float* dpre_packed16);
 /* The whole forward of a timestep in one launch, input product included: gates = act(b + [f: +1] +
  * Wx * x + Wh * h_tm1) from packed copies of both weight matrices (dyhip_lstm_pack_input: Wx is
  * 4H x I, I a multiple of 128), then c and h; x and h_tm1 are plain.  For callers

@@ -18,8 +18,17 @@ import numpy as np
 from . import cpu_oracle as orc
 
 
-def forward(p, tokens, L):
-    """tokens[T+1, B].  Returns (loss, cache)."""
+def _mask_args(masks, l, B):
+    """Keyword arguments of the gates node for layer l: the sequence's dropout masks (dynet/lstm.cc:964-982), or none."""
+    if masks is None:
+        return {}
+    mx, mh = masks[l]
+    return {"mask_x": mx, "mask_x_bd": B, "mask_h": mh, "mask_h_bd": B}
+
+
+def forward(p, tokens, L, masks=None):
+    """tokens[T+1, B]; masks = per layer (mask_x[B, d_in], mask_h[B, H]) for vanilla_lstm_gates_dropout
+    (dynet/lstm.cc:1068-1073), or None.  Returns (loss, cache)."""
     T, B = tokens.shape[0] - 1, tokens.shape[1]
     V, E = p["C"].shape
     H = p["Wh0"].shape[0]
@@ -33,7 +42,8 @@ def forward(p, tokens, L):
         for l in range(L):
             h_tm1 = cache["h"][t - 1][l] if t > 0 else zeros
             c_tm1 = cache["c"][t - 1][l] if t > 0 else zeros
-            g = orc.lstm_gates_forward([x], [d_in], H, B, h_tm1, p[f"Wx{l}"], p[f"Wh{l}"], p[f"b{l}"])
+            g = orc.lstm_gates_forward([x], [d_in], H, B, h_tm1, p[f"Wx{l}"], p[f"Wh{l}"], p[f"b{l}"],
+                                       **_mask_args(masks, l, B))
             c = orc.lstm_c_forward(H, B, c_tm1, g)
             h = orc.lstm_h_forward(H, B, c, g)
             cache["gates"][t][l], cache["c"][t][l], cache["h"][t][l] = g, c, h
@@ -52,7 +62,7 @@ def forward(p, tokens, L):
     return loss, cache
 
 
-def backward(p, tokens, L, cache):
+def backward(p, tokens, L, cache, masks=None):
     T, B = tokens.shape[0] - 1, tokens.shape[1]
     V, E = p["C"].shape
     H = p["Wh0"].shape[0]
@@ -83,11 +93,12 @@ def backward(p, tokens, L, cache):
             d_x = d_h[t][l - 1] if l > 0 else np.zeros((B, E), np.float32)
             d_h_tm1 = d_h[t - 1][l] if t > 0 else np.zeros((B, H), np.float32)
             args = ([x], [d_in], H, B, h_tm1, p[f"Wx{l}"], p[f"Wh{l}"], gates, d_g)
-            orc.lstm_gates_backward(*args, 0, d_x)
-            orc.lstm_gates_backward(*args, 1, d_h_tm1)
-            orc.lstm_gates_backward(*args, 2, g[f"Wx{l}"])
-            orc.lstm_gates_backward(*args, 3, g[f"Wh{l}"])
-            orc.lstm_gates_backward(*args, 4, g[f"b{l}"])
+            mk = _mask_args(masks, l, B)
+            orc.lstm_gates_backward(*args, 0, d_x, **mk)
+            orc.lstm_gates_backward(*args, 1, d_h_tm1, **mk)
+            orc.lstm_gates_backward(*args, 2, g[f"Wx{l}"], **mk)
+            orc.lstm_gates_backward(*args, 3, g[f"Wh{l}"], **mk)
+            orc.lstm_gates_backward(*args, 4, g[f"b{l}"], **mk)
             if l == 0:
                 d_x_below = d_x
         orc.lookup_accumulate_grads(tokens[t], E, V, d_x_below, g["C"])
@@ -114,10 +125,10 @@ def update(p, g, tokens, lr, clip):
     return gscale
 
 
-def step(p, tokens, L, lr=0.1, clip=5.0):
+def step(p, tokens, L, lr=0.1, clip=5.0, masks=None):
     """One training step; p is updated in place.  Returns (loss, grads before the update, clip scale)."""
     tokens = np.ascontiguousarray(tokens, dtype=np.uint32)
-    loss, cache = forward(p, tokens, L)
-    g = backward(p, tokens, L, cache)
+    loss, cache = forward(p, tokens, L, masks)
+    g = backward(p, tokens, L, cache, masks)
     gscale = update(p, g, tokens, lr, clip)
     return loss, g, gscale

@@ -68,6 +68,77 @@ def test_lm_step_matches_oracle(dev, case, path, time_batched, overlap):
             lm.p[n].set(ref_p[n])
 
 
+@pytest.mark.parametrize("path,time_batched", [("fused", True), ("fused_two_call", True), ("nodes", True), ("nodes", False)])
+@pytest.mark.parametrize("case,rates", [((300, 64, 128, 2, 32, 6), (0.3, 0.3)), ((200, 128, 256, 2, 64, 4), (0.25, 0.4)),
+                                        ((50, 16, 32, 2, 8, 5), (0.5, 0.2)), ((37, 12, 20, 1, 5, 4), (0.3, 0.0))])
+def test_lm_step_with_dropout_matches_oracle(dev, case, rates, path, time_batched):
+    """CompactVanillaLSTMBuilder's dropout (dynet/lstm.cc:964-982,1068-1073): masks drawn on the device once per
+    step, in the builder's order, from the generator (recomputed here on the host from seed and position); the step
+    against the oracle's node-by-node composition with the same masks.  The fused path takes its one-launch
+    timesteps with the recurrent mask where the size allows (H = 128, 256), the plain products elsewhere."""
+    from oracle import cpu_oracle as orc
+
+    V, E, H, L, B, T = case
+    rng = np.random.default_rng(31)
+    params = LstmLM.init_params(V, E, H, L, seed=4)
+    for l in range(L):
+        params[f"b{l}"] = rng.normal(0, 0.1, 4 * H).astype(np.float32)
+    ref_p = {n: a.copy() for n, a in params.items()}
+    lm = LstmLM(dev, V, E, H, L, B, T, lr=0.1, clip=5.0, time_batched=time_batched, params=params,
+                path=path.split("_")[0], single_launch=None if path == "fused" else False, dropout=rates[0],
+                dropout_h=rates[1])
+    assert lm.single_launch == (path == "fused" and H % 128 == 0 and B % 32 == 0)
+    dev.reset_rng(41)
+    for it in range(2):
+        tokens = _tokens(rng, V, B, T)
+        key, pos, queue = dev.rng_state()
+        lm.stage(tokens)
+        lm.dev.lookup_build_plan_into(lm.ids, V, lm.plan, lm.plan_ws, lm.plan_ws_bytes)
+        lm.draw_masks()
+        lm.forward()
+        lm.backward()
+        masks = lm.get_masks()
+        # the masks are the generator's words at the positions the builder's drawing order gives them
+        at = pos
+        for l in range(L):
+            for m, rate in zip(masks[l], rates):
+                want = orc.randomize_bernoulli(key, at, queue, m.size, 1.0 - rate, 1.0 / (1.0 - rate)).reshape(m.shape)
+                assert np.array_equal(m, want), (l, rate)
+                at += (m.size + 3) // 4
+        if rates[1] > 0:
+            assert 0.0 in masks[0][1] and masks[0][1].max() > 1.0  # something is dropped, the rest is scaled up
+        ref_loss, ref_g, ref_scale = lm_oracle.step(ref_p, tokens, L, lr=0.1, clip=5.0, masks=masks)
+        loss = lm.loss.numpy()[0]
+        grads = lm.get_grads()
+        lm.update()
+        assert_close(loss, ref_loss, FWD_RTOL * 4, f"loss step {it}")
+        for n in ref_g:
+            assert_close(grads[n], ref_g[n], GRAD_RTOL, f"grad {n} step {it}", floor=_grad_floor(ref_g[n]))
+        assert_close(lm.gscale.numpy()[0], ref_scale, GRAD_RTOL, f"clip scale step {it}")
+        new_p = lm.get_params()
+        for n in ref_p:  # p - lr * scale * g: the update term carries the gradient's and the clip scale's tolerance
+            assert_close(new_p[n], ref_p[n], GRAD_RTOL, f"param {n} step {it}",
+                         floor=_grad_floor(ref_p[n]) + 0.1 * float(np.abs(ref_g[n]).max()))
+        for n in ref_p:
+            lm.p[n].set(ref_p[n])
+
+
+def test_lm_dropout_inside_a_captured_step_draws_new_masks_on_every_replay(dev):
+    V, E, H, L, B, T = 300, 64, 128, 2, 32, 4
+    rng = np.random.default_rng(6)
+    lm = LstmLM(dev, V, E, H, L, B, T, dropout=0.3)
+    lm.stage(_tokens(rng, V, B, T))
+    lm.capture()
+    seen = []
+    for _ in range(3):
+        lm.step(_tokens(rng, V, B, T))
+        seen.append(lm.get_masks()[1][1].copy())
+        dev.constant(lm.errs, 0.0)  # eager work between the replays
+        dev.sync()
+    assert not np.array_equal(seen[0], seen[1]) and not np.array_equal(seen[1], seen[2])
+    lm.graph.destroy()
+
+
 @pytest.fixture(scope="module")
 def wide_case():
     """The LM configuration's layer widths (E = 256, H = 1024, two layers, B = 128: the sizes that select the
