@@ -650,6 +650,12 @@ def lstm_lm(steps, warmup=12, use_graph=True):
                                   "product + cell update) and so is a backward one (Wh^T dpre of the step above + "
                                   "cell backward), operands handed from timestep to timestep in matrix-core "
                                   "fragment order",
+           "node_path_schedule": "the three fused LSTM nodes per layer and timestep, every backward argument its own "
+                                 "call; the gates nodes' backward calls for Wx, Wh and b record their operands and the "
+                                 "T recorded products of a parameter are formed as one product over the gathered "
+                                 "operands where the executor hands the gradient to the parameter "
+                                 "(node_at_a_time_path); node_at_a_time_path_weight_gradients_per_node forms them "
+                                 "node by node, T products of depth B each",
            "timed_region": "per step: host->device copy of ids and labels, id sort, forward, backward, "
                            "device-side clipping, update; one HIP-graph replay per step; loss read back after "
                            "the last step"}
@@ -657,11 +663,12 @@ def lstm_lm(steps, warmup=12, use_graph=True):
     # ms_per_step is the faster one.  The collector is off inside the timed loop: in this process, which holds the
     # tables of every earlier leg, one full collection is a 5-10 ms pause of the host thread that launches the steps
     # (7.1 instead of 6.6 ms per step over 30 steps; a kernel trace shows equal kernel durations either way).
-    for path, tb in (("fused", True), ("nodes", False)):
+    for path, tb in (("fused", True), ("nodes", False), ("nodes_eager", False)):
         runs = []
         for _ in range(2):
             dev = Device(0, mem_mb=(1024, 1024, 512, 1024))
-            lm = LstmLM(dev, V, E, H, L, B, T, lr=0.1, clip=5.0, time_batched=tb, path=path)
+            lm = LstmLM(dev, V, E, H, L, B, T, lr=0.1, clip=5.0, time_batched=tb, path=path.split("_")[0],
+                        defer_weight_grads=path == "nodes")
             lm.stage(batches[0])
             if use_graph:
                 lm.capture()
@@ -684,7 +691,8 @@ def lstm_lm(steps, warmup=12, use_graph=True):
                 lm.graph.destroy()
             dev.close()
         dt, first, last = min(runs)
-        key = "fused_cell_path" if path == "fused" else "node_at_a_time_path"
+        key = {"fused": "fused_cell_path", "nodes": "node_at_a_time_path",
+               "nodes_eager": "node_at_a_time_path_weight_gradients_per_node"}[path]
         res[key] = {"ms_per_step": round(dt * 1e3, 3), "tokens_per_s": round(T * B / dt, 1),
                     "ms_per_step_of_each_instance": [round(r[0] * 1e3, 3) for r in runs],
                     "gemm_tflops": round(flops / dt / 1e12, 2),

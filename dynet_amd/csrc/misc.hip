@@ -85,6 +85,37 @@ __global__ __launch_bounds__(kThreads) void ragged_move_kernel(int num_seqs, flo
   }
 }
 
+// Equal-length segments copied one behind the other: dst[s * len, (s + 1) * len) = src_s.  The segment addresses
+// travel in the kernel's argument block, not in a device table, so the call needs no staging copy, no synchronisation
+// and may be recorded into a graph.  blockIdx.y = segment; a tile of 256 x 4 groups of four floats per block, all its
+// loads issued before the first store.
+constexpr int kGatherSegs = 32;
+struct GatherArgs {
+  const float* src[kGatherSegs];
+};
+
+template <bool VEC, bool NT>
+__global__ __launch_bounds__(kThreads) void gather_segments_kernel(GatherArgs a, size_t len, float* __restrict__ dst) {
+  const float* ps = a.src[blockIdx.y];
+  float* pt = dst + size_t(blockIdx.y) * len;
+  if (VEC) {
+    const size_t n4 = len >> 2;
+    const float4* s4 = reinterpret_cast<const float4*>(ps);
+    float4* t4 = reinterpret_cast<float4*>(pt);
+    const size_t i0 = size_t(blockIdx.x) * (kThreads * 4) + threadIdx.x;
+    float4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = ldg4<NT>(s4 + min(i0 + size_t(u) * kThreads, n4 - 1));
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (i0 + size_t(u) * kThreads < n4) stg4<NT>(t4 + i0 + size_t(u) * kThreads, v[u]);
+  } else {
+    for (size_t i = size_t(blockIdx.x) * (kThreads * 16) + threadIdx.x, e = min(len, (size_t(blockIdx.x) + 1) * (kThreads * 16));
+         i < e; i += kThreads)
+      pt[i] = ps[i];
+  }
+}
+
 // stage 1: per-block partial of sum g^2 ; stage 2: one block adds the partials in order
 // partial[block] = sum of squares of the block's share.  The 16-byte aligned middle of the array goes through
 // 128-bit loads, four in flight per thread (plain ones: the update that follows reads the same gradient); the few floats before and after it are added by block 0.
@@ -211,6 +242,32 @@ int dyhip_parallel_memcpy(dyhip_device* dev, int num_seqs, int max_len, float** 
 
 int dyhip_parallel_accumulate(dyhip_device* dev, int num_seqs, int max_len, float** src, float** trg, size_t* len) {
   return ragged_move(dev, true, num_seqs, max_len, src, trg, len);
+}
+
+int dyhip_gather_segments(dyhip_device* dev, unsigned n_seg, size_t len, const float* const* src_host, float* dst) {
+  DYHIP_CHECK_DEV(dev);
+  if (n_seg == 0 || len == 0) return DYHIP_OK;
+  DYHIP_REQUIRE(src_host != nullptr && dst != nullptr, "null pointer in gather_segments");
+  DYHIP_REQUIRE(len < (size_t(1) << 40), "segment too long");
+  bool vec = len % 4 == 0 && aligned16(dst);
+  for (unsigned s2 = 0; s2 < n_seg; ++s2) {
+    DYHIP_REQUIRE(src_host[s2] != nullptr, "null segment %u in gather_segments", s2);
+    vec = vec && aligned16(src_host[s2]);
+  }
+  const bool nt = size_t(n_seg) * len * sizeof(float) >= dev->stream_threshold;
+  const unsigned gx = static_cast<unsigned>(cdiv<size_t>(len, size_t(kThreads) * 16));
+  for (unsigned s0 = 0; s0 < n_seg; s0 += kGatherSegs) {
+    const unsigned cnt = n_seg - s0 < unsigned(kGatherSegs) ? n_seg - s0 : unsigned(kGatherSegs);
+    GatherArgs a;
+    for (unsigned k = 0; k < unsigned(kGatherSegs); ++k) a.src[k] = src_host[s0 + (k < cnt ? k : 0)];
+    float* out = dst + size_t(s0) * len;
+    const dim3 grid(gx, cnt), block(kThreads);
+    if (vec && nt) hipLaunchKernelGGL((gather_segments_kernel<true, true>), grid, block, 0, dev->stream, a, len, out);
+    else if (vec) hipLaunchKernelGGL((gather_segments_kernel<true, false>), grid, block, 0, dev->stream, a, len, out);
+    else hipLaunchKernelGGL((gather_segments_kernel<false, false>), grid, block, 0, dev->stream, a, len, out);
+    DYHIP_CHECK_LAUNCH();
+  }
+  return DYHIP_OK;
 }
 
 int dyhip_squared_l2norm_workspace(size_t n, size_t* ws_bytes) {

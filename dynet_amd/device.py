@@ -518,6 +518,11 @@ class Device:
                                                     _p(dpre_next_packed16), _p(gates), _p(c), _p(c_tm1), _p(dh), _p(dc),
                                                     _p(dpre), _p(dc_tm1), _p(dpre_packed16)))
 
+    def gather_segments(self, segments, length, dst):
+        """dst = the equal-length tensors `segments` one behind the other (pointers travel as kernel arguments)."""
+        ptrs = (C.c_void_p * len(segments))(*[t.ptr if isinstance(t, DevTensor) else int(t) for t in segments])
+        _check(cdll.dyhip_gather_segments(self.handle, _u(len(segments)), _sz(int(length)), ptrs, _p(dst)))
+
     def lstm_pack_input(self, I, H, Wx, packed):
         _check(cdll.dyhip_lstm_pack_input(self.handle, _u(I), _u(H), _p(Wx), _p(packed)))
 

@@ -11,6 +11,11 @@ What differs from DyNet's node-at-a-time execution (results agree to fp32 roundi
   * ``path="nodes"`` issues the three fused LSTM nodes per layer and timestep exactly as
     CompactVanillaLSTMBuilder::add_input_impl does; with ``time_batched=True`` the weight/bias gradients of the
     gate GEMMs are formed once per layer over the K = T*B columns of all timesteps instead of T times over B;
+    with ``defer_weight_grads=True`` every gates node's backward call for Wx, Wh and b only records its operands
+    (they stay alive until the graph is freed), and the recorded products of a parameter are formed as one
+    product over the gathered operands at the point where the executor hands the gradient to the parameter: what
+    an adapter behind the unchanged node API can do (it sees one node at a time and does not know that its
+    operands sit in one array here, so it gathers them);
   * ``path="fused"`` (default) runs layer by layer: one GEMM forms Wx*x for all timesteps, a timestep is then
     the recurrent GEMM Wh*h plus one cell kernel (gates + c + h); backward mirrors it, and dx, dWx, dWh, db are
     GEMMs/reductions over all timesteps;
@@ -41,8 +46,12 @@ class LstmLM:
     """V-word LM: embedding E, L layers of hidden H, batch B, T timesteps per step."""
 
     def __init__(self, dev, V, E, H, L, B, T, seed=0, lr=0.1, clip=5.0, time_batched=True, params=None, path="fused",
-                 overlap=None, chunk=7, single_launch=None, dropout=0.0, dropout_h=None):
+                 overlap=None, chunk=7, single_launch=None, dropout=0.0, dropout_h=None, defer_weight_grads=False):
         assert path in ("fused", "nodes")
+        # node path: the weight and bias gradients of the gates nodes are not formed node by node (T products of
+        # depth B into the same parameter gradient) but recorded and formed once, where the executor hands the
+        # gradient to the parameter (ParameterNode::accumulate_grad, dynet/exec.cc:274-280)
+        self.defer = bool(defer_weight_grads) and path == "nodes" and not time_batched
         self.dropout = float(dropout)
         self.dropout_h = self.dropout if dropout_h is None else float(dropout_h)
         assert 0.0 <= self.dropout < 1.0 and 0.0 <= self.dropout_h < 1.0
@@ -108,6 +117,10 @@ class LstmLM:
         self.d_c = [dev.empty((T, B, H), pool=DE) for _ in range(L)]
         self.d_gates = [dev.empty((T, B, 4 * H), pool=DE) for _ in range(L)]
         self.de_bytes = dev.pool(DE).used() - self.de_begin
+        if self.defer:  # the gathered operands of a layer's recorded products
+            self.gath_dpre = dev.empty((T, B, 4 * H), pool=DE)
+            self.gath_x = dev.empty((T, B, max(E, H)), pool=DE)
+            self.gath_h = dev.empty((T, B, H), pool=DE)
         self.d_pre = [dev.empty((T, B, 4 * H), pool=DE) for _ in range(L)]  # overwritten, never accumulated into
         fb, bb = dev.lstm_cell_workspace(H, B)
         self.rec_f_bytes, self.rec_b_bytes = fb, bb
@@ -384,8 +397,42 @@ class LstmLM:
         for l in range(L - 1):
             d.wait(qof(l))
 
+    def _flush_recorded(self):
+        """The recorded products of every parameter as one product each: the operands of the T backward calls are
+        gathered in ascending timestep order (the addresses go to the kernel as arguments), then
+        dWx += dpre x^T, dWh += dpre[1:] h[:-1]^T, db += sum over the columns of dpre, each over all timesteps."""
+        d, E, H, B, T = self.dev, self.E, self.H, self.B, self.T
+        for l in range(self.L):
+            rec = sorted(self._recorded[l], key=lambda r: r[0])
+            d_in = H if l > 0 else E
+            n = len(rec) * B
+            gx = self.gath_x.offset(0, (len(rec), B, d_in))
+            d.gather_segments([r[1] for r in rec], 4 * H * B, self.gath_dpre)
+            d.gather_segments([r[2] for r in rec], d_in * B, gx)
+            if self.use_dropout:  # the gates saw x (.) mask_x and h_tm1 (.) mask_h
+                d.cmult_forward(B * d_in, len(rec), 1, gx, self.mask_x[l], gx)
+            d.gemm_nt_acc(4 * H, d_in, n, self.gath_dpre, gx, self.g[f"Wx{l}"])
+            later = [r for r in rec if r[0] > 0]  # h_tm1 of the first step is the zero state: its product adds nothing
+            if later:
+                assert rec[0][0] == 0 and len(later) == len(rec) - 1
+                gh = self.gath_h.offset(0, (len(later), B, H))
+                d.gather_segments([r[3] for r in later], H * B, gh)
+                if self.use_dropout:
+                    d.cmult_forward(B * H, len(later), 1, gh, self.mask_h[l], gh)
+                d.gemm_nt_acc(4 * H, H, len(later) * B, self._t(self.gath_dpre, 1, 4 * H), gh, self.g[f"Wh{l}"])
+            d.csum_backward(4 * H, 1, n, self.gath_dpre, 0, self.g[f"b{l}"])
+            if l == 0:
+                # the T recorded products Wx^T dpre_t into the lookup nodes' gradients as one product over the gathered
+                # dpre (here the T gradients are one array; an executor's are T tensors, which the product's columns
+                # are added to with one dyhip_parallel_accumulate)
+                assert len(rec) == T
+                d.gemm_tn_acc(E, n, 4 * H, self.p["Wx0"], self.gath_dpre, self.d_emb)
+                if self.use_dropout:
+                    d.cmult_forward(B * E, T, 1, self.d_emb, self.mask_x[0], self.d_emb)
+
     def _backward_layers_nodes(self):
         d, E, H, L, B, T, N = self.dev, self.E, self.H, self.L, self.B, self.T, self.N
+        self._recorded = [[] for _ in range(L)]
         for t in reversed(range(T)):
             for l in reversed(range(L)):
                 g, c = self._t(self.gates[l], t, 4 * H), self._t(self.c[l], t, H)
@@ -403,27 +450,38 @@ class LstmLM:
                     x, d_in, dx = self._t(self.h[l - 1], t, H), H, self._t(self.d_h[l - 1], t, H)
                 else:
                     x, d_in, dx = self._t(self.emb, t, E), E, self._t(self.d_emb, t, E)
+                # The gradient of layer 0's input belongs to a lookup node, an arity-0 node whose gradient nobody reads
+                # before the executor hands it over at the end of backward: its product is recorded as well.
+                lazy_dx = self.defer and l == 0
                 if self.use_dropout:
                     # the gates node's own backward: it applies the masks to dx / dh and to the operands of dWx / dWh
                     mk = self._node_masks(l)
                     args = ([x], [d_in], H, B, h_tm1, self.p[f"Wx{l}"], self.p[f"Wh{l}"], g, dg)
-                    d.lstm_gates_backward(*args, 0, dx, dpre=dpre, **mk)
+                    if not lazy_dx:
+                        d.lstm_gates_backward(*args, 0, dx, dpre=dpre, **mk)
                     if t > 0:
                         d.lstm_gates_backward(*args, 1, self._t(self.d_h[l], t - 1, H), dpre=dpre, **mk)
-                    if not self.time_batched:
+                    if self.defer:
+                        self._recorded[l].append((t, dpre, x, h_tm1))
+                    elif not self.time_batched:
                         d.lstm_gates_backward(*args, 2, self.g[f"Wx{l}"], dpre=dpre, **mk)
                         if t > 0:
                             d.lstm_gates_backward(*args, 3, self.g[f"Wh{l}"], dpre=dpre, **mk)
                         d.lstm_gates_backward(*args, 4, self.g[f"b{l}"], dpre=dpre, **mk)
                     continue
-                d.gemm_tn_acc(d_in, B, 4 * H, self.p[f"Wx{l}"], dpre, dx)
+                if not lazy_dx:
+                    d.gemm_tn_acc(d_in, B, 4 * H, self.p[f"Wx{l}"], dpre, dx)
                 if t > 0:
                     d.gemm_tn_acc(H, B, 4 * H, self.p[f"Wh{l}"], dpre, self._t(self.d_h[l], t - 1, H))
-                if not self.time_batched:
+                if self.defer:
+                    self._recorded[l].append((t, dpre, x, h_tm1))
+                elif not self.time_batched:
                     d.gemm_nt_acc(4 * H, d_in, B, dpre, x, self.g[f"Wx{l}"])
                     if t > 0:  # h_tm1 of the first step is the zero state: its product adds nothing
                         d.gemm_nt_acc(4 * H, H, B, dpre, h_tm1, self.g[f"Wh{l}"])
                     d.csum_backward(4 * H, 1, B, dpre, 0, self.g[f"b{l}"])
+        if self.defer:
+            self._flush_recorded()
         if self.time_batched:
             for l in range(L):
                 x, d_in = self._x_of(l)

@@ -30,7 +30,7 @@ def _grad_floor(ref):
 
 @pytest.mark.parametrize("path,time_batched,overlap", [("nodes", False, False), ("nodes", True, False),
                                                        ("fused", True, False), ("fused", True, True),
-                                                       ("fused_two_call", True, True)])
+                                                       ("fused_two_call", True, True), ("nodes_deferred", False, False)])
 @pytest.mark.parametrize("case", CASES)
 def test_lm_step_matches_oracle(dev, case, path, time_batched, overlap):
     V, E, H, L, B, T = case
@@ -41,8 +41,9 @@ def test_lm_step_matches_oracle(dev, case, path, time_batched, overlap):
     ref_p = {n: a.copy() for n, a in params.items()}
     # "fused" takes the single-launch forward step where the hidden size allows it (H = 128 here)
     lm = LstmLM(dev, V, E, H, L, B, T, lr=0.1, clip=5.0, time_batched=time_batched, params=params,
-                path=path.split("_")[0], overlap=overlap, chunk=2, single_launch=None if path == "fused" else False)
-    assert lm.single_launch == (path == "fused" and H % 128 == 0)
+                path=path.split("_")[0], overlap=overlap, chunk=2, single_launch=None if path == "fused" else False,
+                defer_weight_grads=path == "nodes_deferred")
+    assert lm.single_launch == (path == "fused" and H % 128 == 0) and lm.defer == (path == "nodes_deferred")
     for it in range(2):
         tokens = _tokens(rng, V, B, T)
         ref_loss, ref_g, ref_scale = lm_oracle.step(ref_p, tokens, L, lr=0.1, clip=5.0)
@@ -68,7 +69,8 @@ def test_lm_step_matches_oracle(dev, case, path, time_batched, overlap):
             lm.p[n].set(ref_p[n])
 
 
-@pytest.mark.parametrize("path,time_batched", [("fused", True), ("fused_two_call", True), ("nodes", True), ("nodes", False)])
+@pytest.mark.parametrize("path,time_batched", [("fused", True), ("fused_two_call", True), ("nodes", True), ("nodes", False),
+                                               ("nodes_deferred", False)])
 @pytest.mark.parametrize("case,rates", [((300, 64, 128, 2, 32, 6), (0.3, 0.3)), ((200, 128, 256, 2, 64, 4), (0.25, 0.4)),
                                         ((50, 16, 32, 2, 8, 5), (0.5, 0.2)), ((37, 12, 20, 1, 5, 4), (0.3, 0.0))])
 def test_lm_step_with_dropout_matches_oracle(dev, case, rates, path, time_batched):
@@ -86,7 +88,7 @@ def test_lm_step_with_dropout_matches_oracle(dev, case, rates, path, time_batche
     ref_p = {n: a.copy() for n, a in params.items()}
     lm = LstmLM(dev, V, E, H, L, B, T, lr=0.1, clip=5.0, time_batched=time_batched, params=params,
                 path=path.split("_")[0], single_launch=None if path == "fused" else False, dropout=rates[0],
-                dropout_h=rates[1])
+                dropout_h=rates[1], defer_weight_grads=path == "nodes_deferred")
     assert lm.single_launch == (path == "fused" and H % 128 == 0 and B % 32 == 0)
     dev.reset_rng(41)
     for it in range(2):
@@ -156,11 +158,12 @@ def wide_case():
 
 
 @pytest.mark.parametrize("path,time_batched,overlap", [("nodes", False, False), ("fused", True, False),
-                                                       ("fused", True, True)])
+                                                       ("fused", True, True), ("nodes_deferred", False, False)])
 def test_lm_step_matches_oracle_at_production_width(dev, wide_case, path, time_batched, overlap):
     (V, E, H, L, B, T), params, tokens, ref_loss, ref_g, ref_scale, ref_p = wide_case
     lm = LstmLM(dev, V, E, H, L, B, T, lr=0.1, clip=5.0, time_batched=time_batched,
-                params={n: a.copy() for n, a in params.items()}, path=path, overlap=overlap, chunk=2)
+                params={n: a.copy() for n, a in params.items()}, path=path.split("_")[0], overlap=overlap, chunk=2,
+                defer_weight_grads=path == "nodes_deferred")
     assert lm.single_launch == (path == "fused")
     lm.stage(tokens)
     lm.dev.lookup_build_plan_into(lm.ids, V, lm.plan, lm.plan_ws, lm.plan_ws_bytes)
