@@ -16,6 +16,7 @@
 
 #include <cstddef>
 #include <initializer_list>
+#include <map>
 #include <stdexcept>
 #include <string>
 #include <vector>
@@ -144,13 +145,102 @@ class PinnedStaging {
   void* base_;
 };
 
+// Products that nodes add into the gradient of an arity-0 node (a parameter or a lookup), recorded instead of
+// formed.  The executor visits a node's arguments one at a time (dynet/exec.cc:247-262), so the T gates nodes of an
+// unrolled LSTM add T products of depth B (the batch) into the same dEdf of the ParameterNode of Wx: T launches that
+// each read and rewrite the whole gradient for a product too shallow to fill the matrix cores.  Nobody reads such a
+// gradient before the executor hands it to the parameter (ParameterNode::accumulate_grad, dynet/exec.cc:274-280),
+// and the operands (node outputs in pools[FXS], the cached activation derivative in the node's aux_mem) stay alive
+// until the graph is freed.  So a node may record (operands, shape) here, and the recorded products of one gradient
+// are formed as ONE product over the gathered operands when the gradient is first read: by accumulate_grad, by
+// as_vector / TensorTools of this adapter, or by flush_all.
+//
+// The executor's part (three lines in ExecutionEngine::backward): after ndEdfs is allocated, call clear() and then
+// allow(ndEdfs[i].v) for every i in cg.parameter_nodes; gradients of other nodes are never deferred, because the
+// executor reads them (as dEdf of that node's own backward) right after its consumers have run.
+class DeferredGrads {
+ public:
+  explicit DeferredGrads(dyhip_device* dev, std::vector<AlignedMemoryPool*>* pools) : dev_(dev), pools_(pools) {}
+  void clear() {
+    allowed_.clear();
+    pending_.clear();
+  }
+  void allow(const float* dst) { allowed_[dst] = true; }
+  bool allowed(const float* dst) const { return allowed_.count(dst) != 0; }
+  bool pending(const float* dst) const {
+    auto it = pending_.find(dst);
+    return it != pending_.end() && !it->second.empty();
+  }
+  // dst[M x N] += l[M x K] * r[N x K]^T (MatrixMultiplyTranspAcc); with r == nullptr: dst[M] += sum of l's K columns
+  void record(float* dst, unsigned M, unsigned N, unsigned K, const float* l, const float* r) {
+    pending_[dst].push_back(Product{M, N, K, l, r});
+  }
+  void flush(const float* dst) {
+    auto it = pending_.find(dst);
+    if (it == pending_.end() || it->second.empty()) return;
+    std::vector<Product> list;
+    list.swap(it->second);
+    float* out = const_cast<float*>(dst);
+    bool same = true;
+    for (const Product& p : list) same = same && p.M == list[0].M && p.N == list[0].N && p.K == list[0].K && (p.r == nullptr) == (list[0].r == nullptr);
+    AlignedMemoryPool* scs = (*pools_)[static_cast<int>(DeviceMempool::SCS)];
+    if (!same || list.size() == 1) {  // nothing to merge: form them one by one
+      for (const Product& p : list) form(out, p.M, p.N, p.K, p.l, p.r, scs);
+      scs->free();
+      return;
+    }
+    const unsigned n = static_cast<unsigned>(list.size()), M = list[0].M, N = list[0].N, K = list[0].K;
+    std::vector<const float*> ls, rs;
+    for (const Product& p : list) {
+      ls.push_back(p.l);
+      rs.push_back(p.r);
+    }
+    float* gl = static_cast<float*>(scs->allocate(sizeof(float) * size_t(M) * K * n));
+    abi_check(dyhip_gather_segments(dev_, n, size_t(M) * K, ls.data(), gl));
+    float* gr = nullptr;
+    if (list[0].r != nullptr) {
+      gr = static_cast<float*>(scs->allocate(sizeof(float) * size_t(N) * K * n));
+      abi_check(dyhip_gather_segments(dev_, n, size_t(N) * K, rs.data(), gr));
+    }
+    form(out, M, N, K * n, gl, gr, scs);
+    scs->free();
+  }
+  void flush_all() {
+    std::vector<const float*> keys;
+    for (auto& kv : pending_) keys.push_back(kv.first);
+    for (const float* k : keys) flush(k);
+  }
+
+ private:
+  struct Product {
+    unsigned M, N, K;
+    const float *l, *r;
+  };
+  void form(float* out, unsigned M, unsigned N, unsigned K, const float* l, const float* r, AlignedMemoryPool* scs) {
+    if (r != nullptr) {
+      abi_check(dyhip_gemm_nt_acc(dev_, M, N, K, l, r, out));
+    } else {
+      size_t need = 0;
+      abi_check(dyhip_batch_reduce_workspace(M, K, &need));
+      void* ws = need ? scs->allocate(need) : nullptr;
+      abi_check(dyhip_csum_backward(dev_, M, 1, K, l, 0, out, ws, need));
+    }
+  }
+  dyhip_device* dev_;
+  std::vector<AlignedMemoryPool*>* pools_;
+  std::map<const float*, bool> allowed_;
+  std::map<const float*, std::vector<Product>> pending_;
+};
+
 struct Device_GPU {
   dyhip_device* hip;
   float *kSCALAR_MINUSONE, *kSCALAR_ONE, *kSCALAR_ZERO;
   std::vector<AlignedMemoryPool*> pools;
   PinnedStaging* staging;
+  DeferredGrads* deferred;
 
-  Device_GPU(int device_id, size_t fxs_mb, size_t dedfs_mb, size_t ps_mb, size_t scs_mb) : hip(nullptr), staging(nullptr) {
+  Device_GPU(int device_id, size_t fxs_mb, size_t dedfs_mb, size_t ps_mb, size_t scs_mb)
+      : hip(nullptr), staging(nullptr), deferred(nullptr) {
     const size_t mb[4] = {fxs_mb, dedfs_mb, ps_mb, scs_mb};
     abi_check(dyhip_device_create(device_id, mb, &hip));
     const float* s[3];
@@ -164,8 +254,10 @@ struct Device_GPU {
       pools.push_back(new AlignedMemoryPool(p));
     }
     staging = new PinnedStaging(hip);
+    deferred = new DeferredGrads(hip, &pools);
   }
   ~Device_GPU() {
+    delete deferred;
     delete staging;
     for (AlignedMemoryPool* p : pools) delete p;
     if (hip) dyhip_device_destroy(hip);
@@ -193,6 +285,7 @@ struct TensorTools {
   static void zero(Tensor& t) { abi_check(dyhip_zero(t.device->hip, t.v, sizeof(float) * t.d.size())); }
   static void constant(Tensor& t, float c) { abi_check(dyhip_constant(t.device->hip, t.d.size(), c, t.v)); }
   static void accumulate(Tensor& t, const Tensor& src) {
+    src.device->deferred->flush(src.v);
     abi_check(dyhip_accumulate(t.device->hip, t.d.size(), src.v, t.v));
   }
   // dynet/tensor.cc:261-303 (GPU branches)
@@ -207,6 +300,7 @@ struct TensorTools {
   }
 };
 inline std::vector<real> as_vector(const Tensor& t) {  // blocking copy, dynet/tensor.cc:66-93
+  t.device->deferred->flush(t.v);  // a gradient with recorded products is complete before anyone sees it
   std::vector<real> out(t.d.size());
   abi_check(dyhip_memcpy_d2h(t.device->hip, out.data(), t.v, sizeof(float) * out.size()));
   return out;
@@ -272,6 +366,16 @@ struct VanillaLSTMGates : public Node {
       }
       last_i_ = int(i);
       dpre = static_cast<const float*>(aux_mem);
+    }
+    // Wx (one input, no dropout), Wh and b of a node whose activation derivative is cached: when the destination is
+    // the gradient of an arity-0 node, the product is recorded and formed together with those of the other timesteps
+    // (dynet/nodes-lstm.cc:472-500: dWx += dpre x^T, dWh += dpre h_tm1^T, db += sum of dpre's columns)
+    if (dpre != nullptr && !dropout && a.k == 1 && i >= a.k + 1 && dev.deferred->allowed(dEdxi.v)) {
+      const float* r = i == a.k + 1 ? xs[0]->v : i == a.k + 2 ? xs[a.k]->v : nullptr;
+      const unsigned N = i == a.k + 1 ? a.I : i == a.k + 2 ? a.H : 1;
+      dev.deferred->record(dEdxi.v, 4 * a.H, N, a.B, dpre, r);
+      scratch(fx)->free();
+      return;
     }
     abi_check(dyhip_lstm_gates_backward(dev.hip, a.k, a.x.data(), a.xd.data(), a.H, a.B, xs[a.k]->v, xs[a.k + 1]->v,
                                         xs[a.k + 2]->v, a.mx, a.mx_bd, a.mh, a.mh_bd, fx.v, dEdf.v, dpre, i,
@@ -555,6 +659,39 @@ struct PickNegLogSoftmax : public Node {
   void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, const Tensor&, const Tensor& dEdf,
                          unsigned, Tensor& dEdxi) const override {
     abi_check(dyhip_pnls_backward(dev.hip, xs[0]->d.rows(), xs[0]->d.bd, xs[0]->v, aux_mem, dEdf.v, dEdxi.v));
+  }
+};
+
+// ParameterStorage reduced to what the node needs (dynet/model.h:76-118): values and gradient on the device
+struct ParameterStorage {
+  Tensor values, g;
+  bool nonzero_grad = false;
+  // ParameterStorage::accumulate_grad (dynet/model.cc:556-571): g += d
+  void accumulate_grad(const Tensor& d) {
+    nonzero_grad = true;
+    abi_check(dyhip_accumulate(values.device->hip, g.d.size(), d.v, g.v));
+  }
+};
+
+// ParameterNode over a dense parameter (dynet/param-nodes.h:40-58, dynet/param-nodes.cc:43-50,201-225): forward copies
+// the values times the current weight decay; backward must never be called (arity 0); accumulate_grad is where the
+// executor hands the node's gradient to the parameter (dynet/exec.cc:274-280) -- and where the products recorded into
+// that gradient are formed.
+struct ParameterNode : public Node {
+  ParameterNode(ParameterStorage* params, real weight_decay = 1.f) : params(params), weight_decay(weight_decay) {}
+  ParameterStorage* params;
+  real weight_decay;
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    if (!xs.empty()) throw std::invalid_argument("Failed dimension check in ParameterNode");
+    abi_check(dyhip_scale_copy(dev.hip, fx.d.size(), params->values.v, weight_decay, fx.v));
+  }
+  void backward_dev_impl(const Device_GPU&, const std::vector<const Tensor*>&, const Tensor&, const Tensor&, unsigned i,
+                         Tensor&) const override {
+    throw std::runtime_error("called backward() on arity 0 node: i = " + std::to_string(i));
+  }
+  void accumulate_grad(const Tensor& g) const {
+    g.device->deferred->flush(g.v);
+    params->accumulate_grad(g);
   }
 };
 

@@ -265,6 +265,107 @@ static void lstm_node_gradients(Fixture& F) {
   }
 }
 
+// ---- the executor's accumulation of a parameter gradient over the timesteps of an unrolled LSTM
+// (dynet/exec.cc:247-280): T gates nodes add their products into the dEdf of the same ParameterNode.  With the
+// gradients of the parameter nodes registered as deferrable, the nodes record, and the gradient is formed as one
+// product when it is first read -- which every way of reading it through this adapter does.
+static void deferred_parameter_gradients(Fixture& F) {
+  g_case = "deferred_parameter_gradients";
+  const unsigned H = 8, I = 12, B = 16, T = 3;
+  auto ramp = [](size_t n, float a, float b) {
+    vector<float> v(n);
+    for (size_t k = 0; k < n; ++k) v[k] = a * std::sin(0.37f * float(k) + b);
+    return v;
+  };
+  ParameterStorage pWx, pWh, pb;
+  pWx.values = F.input(Dim({4 * H, I}), ramp(4 * H * I, 0.3f, 0.1f), DeviceMempool::PS);
+  pWh.values = F.input(Dim({4 * H, H}), ramp(4 * H * H, 0.3f, 0.7f), DeviceMempool::PS);
+  pb.values = F.input(Dim({4 * H}), ramp(4 * H, 0.1f, 0.3f), DeviceMempool::PS);
+  for (ParameterStorage* ps : {&pWx, &pWh, &pb}) ps->g = F.zeros(ps->values.d, DeviceMempool::PS);
+  ParameterNode nWx(&pWx), nWh(&pWh, 0.5f), nb(&pb);
+  Tensor Wx = F.dev.allocate_tensor(DeviceMempool::FXS, pWx.values.d), Wh = F.dev.allocate_tensor(DeviceMempool::FXS, pWh.values.d),
+         b = F.dev.allocate_tensor(DeviceMempool::FXS, pb.values.d);
+  nWx.forward_dev_impl(F.dev, {}, Wx);
+  nWh.forward_dev_impl(F.dev, {}, Wh);
+  nb.forward_dev_impl(F.dev, {}, b);
+  {  // forward = values * weight decay
+    const vector<float> v = as_vector(pWh.values), w = as_vector(Wh);
+    bool ok = true;
+    for (size_t k = 0; k < v.size(); ++k) ok = ok && w[k] == 0.5f * v[k];
+    CHECK(ok);
+  }
+  bool threw = false;
+  try {
+    Tensor dummy;
+    nWx.backward_dev_impl(F.dev, {}, Wx, Wx, 0, dummy);
+  } catch (const std::runtime_error&) {
+    threw = true;
+  }
+  CHECK(threw);
+  const Dim gd({4 * H}, B);
+  vector<Tensor> x, h, fx, dEdf, aux;
+  vector<VanillaLSTMGates> nodes;
+  for (unsigned t = 0; t < T; ++t) {
+    x.push_back(F.input(Dim({I}, B), ramp(I * B, 0.8f, 0.2f * t)));
+    h.push_back(F.input(Dim({H}, B), ramp(H * B, 0.6f, 1.0f + 0.3f * t)));
+    fx.push_back(F.dev.allocate_tensor(DeviceMempool::FXS, gd));
+    aux.push_back(F.dev.allocate_tensor(DeviceMempool::FXS, gd));
+    dEdf.push_back(F.input(gd, ramp(gd.size(), 0.5f, 2.0f + t), DeviceMempool::DEDFS));
+    nodes.emplace_back(false, 0.f, gd);
+  }
+  auto run_backward = [&](Tensor& dWx, Tensor& dWh, Tensor& db) {
+    for (int t = int(T) - 1; t >= 0; --t) {  // reverse topological order
+      vector<const Tensor*> xs = {&x[t], &h[t], &Wx, &Wh, &b};
+      nodes[t].aux_mem = aux[t].v;
+      nodes[t].forward_dev_impl(F.dev, xs, fx[t]);
+      nodes[t].backward_dev_impl(F.dev, xs, fx[t], dEdf[t], 2, dWx);
+      nodes[t].backward_dev_impl(F.dev, xs, fx[t], dEdf[t], 3, dWh);
+      nodes[t].backward_dev_impl(F.dev, xs, fx[t], dEdf[t], 4, db);
+    }
+  };
+  // node by node, as without the registry
+  F.dev.deferred->clear();
+  Tensor eWx = F.zeros(Wx.d), eWh = F.zeros(Wh.d), eb = F.zeros(b.d);
+  run_backward(eWx, eWh, eb);
+  CHECK(!F.dev.deferred->pending(eWx.v) && !F.dev.deferred->pending(eWh.v) && !F.dev.deferred->pending(eb.v));
+  const vector<float> wantWx = as_vector(eWx), wantWh = as_vector(eWh), wantb = as_vector(eb);
+  // recorded: the executor registers the parameter nodes' gradients at the start of backward
+  Tensor dWx = F.zeros(Wx.d), dWh = F.zeros(Wh.d), db = F.zeros(b.d);
+  F.dev.deferred->clear();
+  for (Tensor* g : {&dWx, &dWh, &db}) F.dev.deferred->allow(g->v);
+  run_backward(dWx, dWh, db);
+  CHECK(F.dev.deferred->pending(dWx.v) && F.dev.deferred->pending(dWh.v) && F.dev.deferred->pending(db.v));
+  auto close = [](const vector<float>& a, const vector<float>& w) {
+    if (a.size() != w.size()) return false;
+    double scale = 0;
+    for (float v : w) scale = std::fmax(scale, std::fabs(v));
+    for (size_t k = 0; k < a.size(); ++k)
+      if (std::fabs(double(a[k]) - w[k]) > 1e-5 * scale) return false;
+    return scale > 0;
+  };
+  // (1) as_vector: whoever looks at the gradient sees all of it
+  CHECK(close(as_vector(dWx), wantWx));
+  CHECK(!F.dev.deferred->pending(dWx.v));
+  // (2) the executor's hand-over to the parameter
+  nWh.accumulate_grad(dWh);
+  CHECK(!F.dev.deferred->pending(dWh.v) && pWh.nonzero_grad);
+  CHECK(close(as_vector(pWh.g), wantWh));
+  // (3) everything that is left
+  F.dev.deferred->flush_all();
+  CHECK(!F.dev.deferred->pending(db.v));
+  CHECK(close(as_vector(db), wantb));
+  // a second backward pass records afresh and adds to what the gradient holds
+  F.dev.deferred->clear();
+  F.dev.deferred->allow(dWx.v);
+  Tensor d2Wh = F.zeros(Wh.d), d2b = F.zeros(b.d);
+  run_backward(dWx, d2Wh, d2b);  // dWh and db not registered: formed at once
+  CHECK(!F.dev.deferred->pending(d2Wh.v) && close(as_vector(d2Wh), wantWh));
+  vector<float> twice = wantWx;
+  for (float& v : twice) v *= 2.f;
+  CHECK(close(as_vector(dWx), twice));
+  F.dev.deferred->clear();
+}
+
 // ---- tests/test-nodes.cc:1277-1321: argmax_forward, argmax_backward, straight_through_backward ----
 static void argmax_node(Fixture& F) {
   g_case = "argmax_node";
@@ -715,7 +816,7 @@ int main(int argc, char** argv) {
   const std::vector<std::function<void(Fixture&)>> cases = {lstm_node_h_fwd,      lstm_node_c_fwd, lstm_node_gates_fwd,
                                                              lstm_node_gradients,  elementwise_gradients, layer_norm,
                                                              lookup_and_softmax,   random_nodes,    cwise_broadcast,       layer_norm_composite,
-                                                             combine_and_accumulate, argmax_node};
+                                                             combine_and_accumulate, argmax_node, deferred_parameter_gradients};
   for (const auto& c : cases) {
     c(F);
     F.reset();
