@@ -101,6 +101,66 @@ __global__ __launch_bounds__(256) void cwise_bcast_kernel(CwShape sh, const floa
   }
 }
 
+// The same when the index space collapses to two axes (the usual case: a matrix against a row or a column of it, e.g.
+// x - mean and x / sigma of the layer_norm composite): no index arithmetic beyond the block's own coordinates, kRows
+// rows of the outer axis per block with all their loads issued first, streaming accesses for large tensors.
+struct CwShape2 {
+  unsigned d0g, d1;   // groups of W elements along the inner axis; extent of the outer axis
+  size_t s0[3], s1[3];  // element strides of the three operands along the two axes (0 = broadcast)
+};
+constexpr int kCwRows = 4;
+
+template <int FN, int W, bool NT>
+__global__ __launch_bounds__(256) void cwise_bcast2_kernel(CwShape2 sh, const float* __restrict__ p0,
+                                                           const float* __restrict__ p1, const float* __restrict__ p2,
+                                                           float* __restrict__ out) {
+  constexpr int NIN = cw_inputs(FN);
+  constexpr bool ACC = FN >= 3;
+  const unsigned gx = blockIdx.x * 256 + threadIdx.x;
+  if (gx >= sh.d0g) return;
+  const float* ps[3] = {p0, p1, p2};
+  for (unsigned y0 = blockIdx.y * kCwRows; y0 < sh.d1; y0 += gridDim.y * kCwRows) {
+    float v[kCwRows][3][W], o[kCwRows][W];
+#pragma unroll
+    for (int r = 0; r < kCwRows; ++r) {
+      const unsigned y = min(y0 + r, sh.d1 - 1);  // rows past the end repeat the last one and are not stored
+#pragma unroll
+      for (int k = 0; k < 3; ++k) {
+        if (k < NIN) {
+          const float* q = ps[k] + size_t(y) * sh.s1[k] + size_t(gx) * W * sh.s0[k];
+          if (W == 4 && sh.s0[k] == 1) {
+            const float4 t = ldg4<NT>(reinterpret_cast<const float4*>(q));
+            v[r][k][0] = t.x; v[r][k][1 % W] = t.y; v[r][k][2 % W] = t.z; v[r][k][3 % W] = t.w;
+          } else {
+#pragma unroll
+            for (int e = 0; e < W; ++e) v[r][k][e] = q[size_t(e) * sh.s0[k]];
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < W; ++e) v[r][k][e] = 0.f;
+        }
+      }
+      const float* po = out + (size_t(y) * sh.d0g + gx) * W;
+      if (ACC && W == 4) {
+        const float4 t = *reinterpret_cast<const float4*>(po);  // read-modify-write: a plain load
+        o[r][0] = t.x; o[r][1 % W] = t.y; o[r][2 % W] = t.z; o[r][3 % W] = t.w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < W; ++e) o[r][e] = ACC ? po[e] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < kCwRows; ++r) {
+      if (y0 + r >= sh.d1) break;
+      float* po = out + (size_t(y0 + r) * sh.d0g + gx) * W;
+#pragma unroll
+      for (int e = 0; e < W; ++e) o[r][e] = cw_apply<FN>(v[r][0][e], v[r][1][e], v[r][2][e], o[r][e]);
+      if (W == 4) stg4<NT>(reinterpret_cast<float4*>(po), make_float4(o[r][0], o[r][1 % W], o[r][2 % W], o[r][3 % W]));
+      else po[0] = o[r][0];
+    }
+  }
+}
+
 // ---- reduction over the broadcast axes ------------------------------------------------------------
 struct CwReduce {
   unsigned kd[5], rd[5];   // sizes of the kept / reduced axes, in axis order, padded with 1
@@ -153,6 +213,74 @@ __global__ __launch_bounds__(256) void cwise_reduce_wave_kernel(CwReduce c, cons
   }
 }
 
+// The reduced axes collapse to one (the usual case: the sum over the row of a matrix): the kept index is decomposed
+// once per output, the walk along the reduced axis needs no division, and four terms per lane are in flight.
+// VEC: every operand runs along the reduced axis with stride 1 (128-bit loads) or stride 0.
+template <int FN, bool VEC>
+__global__ __launch_bounds__(256) void cwise_reduce_row_kernel(CwReduce c, const float* __restrict__ p0,
+                                                               const float* __restrict__ p1,
+                                                               const float* __restrict__ p2, float* __restrict__ out) {
+  constexpr int NIN = cw_inputs(FN);
+  const unsigned lane = threadIdx.x & 63;
+  const float* ps[3] = {p0, p1, p2};
+  for (size_t o = size_t(blockIdx.x) * 4 + (threadIdx.x >> 6); o < c.n_out; o += size_t(gridDim.x) * 4) {
+    size_t base[3] = {0, 0, 0};
+    size_t r = o;
+#pragma unroll
+    for (int j = 0; j < 5; ++j) {
+      const size_t q = r / c.kd[j];
+      const size_t i = r - q * c.kd[j];
+      r = q;
+#pragma unroll
+      for (int k = 0; k < NIN; ++k) base[k] += i * c.ks[k][j];
+    }
+    const unsigned nr = unsigned(c.n_red);
+    float acc = 0.f;
+    if (VEC) {
+      for (unsigned q0 = 0; q0 < nr; q0 += 4 * 64 * 4) {
+        float4 v[4][3];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const unsigned q = min(q0 + 4 * (lane + 64 * u), nr - 4);  // clamped, masked below
+#pragma unroll
+          for (int k = 0; k < 3; ++k) {
+            if (k >= NIN) v[u][k] = make_float4(0.f, 0.f, 0.f, 0.f);
+            else if (c.rs[k][0] == 1) v[u][k] = *reinterpret_cast<const float4*>(ps[k] + base[k] + q);
+            else {
+              const float b = ps[k][base[k]];
+              v[u][k] = make_float4(b, b, b, b);
+            }
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          if (q0 + 4 * (lane + 64 * u) < nr) {
+            acc += cw_term<FN>(v[u][0].x, v[u][1].x, v[u][2].x);
+            acc += cw_term<FN>(v[u][0].y, v[u][1].y, v[u][2].y);
+            acc += cw_term<FN>(v[u][0].z, v[u][1].z, v[u][2].z);
+            acc += cw_term<FN>(v[u][0].w, v[u][1].w, v[u][2].w);
+          }
+        }
+      }
+    } else {
+      for (unsigned q0 = 0; q0 < nr; q0 += 64 * 4) {
+        float v[4][3];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const unsigned q = min(q0 + lane + 64 * u, nr - 1);
+#pragma unroll
+          for (int k = 0; k < 3; ++k) v[u][k] = k < NIN ? ps[k][base[k] + size_t(q) * c.rs[k][0]] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (q0 + lane + 64 * u < nr) acc += cw_term<FN>(v[u][0], v[u][1], v[u][2]);
+      }
+    }
+    const float t = wave_sum(acc);
+    if (lane == 0) out[o] += t;
+  }
+}
+
 template <int FN>
 __global__ __launch_bounds__(256) void cwise_reduce_thread_kernel(CwReduce c, const float* __restrict__ p0,
                                                                   const float* __restrict__ p1,
@@ -196,11 +324,39 @@ static unsigned cw_grid(size_t work_items, unsigned per_block, const dyhip_devic
   return static_cast<unsigned>(want < cap ? (want ? want : 1) : cap);
 }
 
+// Axes of extent 1 dropped, neighbouring axes merged when every operand treats them alike (broadcast over both, or
+// laid out contiguously across both).  Returns the number of axes left; d / s are padded with 1 / 0.
+static int cw_collapse(const unsigned* d_in, const size_t s_in[3][5], int nin, unsigned* d, size_t s[3][5]) {
+  int r = 0;
+  for (int j = 0; j < 5; ++j) {
+    if (d_in[j] == 1) continue;
+    if (r > 0 && size_t(d[r - 1]) * d_in[j] <= 0xFFFFFFFFull) {
+      bool ok = true;
+      for (int k = 0; k < nin; ++k)
+        ok = ok && ((s[k][r - 1] == 0 && s_in[k][j] == 0) || (s[k][r - 1] != 0 && s_in[k][j] == s[k][r - 1] * d[r - 1]));
+      if (ok) {
+        d[r - 1] *= d_in[j];
+        continue;
+      }
+    }
+    d[r] = d_in[j];
+    for (int k = 0; k < 3; ++k) s[k][r] = k < nin ? s_in[k][j] : 0;
+    ++r;
+  }
+  for (int j = r; j < 5; ++j) {
+    d[j] = 1;
+    for (int k = 0; k < 3; ++k) s[k][j] = 0;
+  }
+  return r;
+}
+
 template <int FN>
-static int cw_launch_bcast(dyhip_device* dev, const CwShape& sh, const float* p0, const float* p1, const float* p2,
+static int cw_launch_bcast(dyhip_device* dev, const CwShape& sh_in, const float* p0, const float* p1, const float* p2,
                            float* out) {
-  const size_t total = cw_size(sh.d);
+  const size_t total = cw_size(sh_in.d);
   if (total == 0) return DYHIP_OK;
+  CwShape sh;
+  const int rank = cw_collapse(sh_in.d, sh_in.s, cw_inputs(FN), sh.d, sh.s);
   bool vec = sh.d[0] % 4 == 0 && aligned16(out);
   const float* ps[3] = {p0, p1, p2};
   for (int k = 0; k < cw_inputs(FN); ++k) {
@@ -209,7 +365,21 @@ static int cw_launch_bcast(dyhip_device* dev, const CwShape& sh, const float* p0
       for (int j = 1; j < 5; ++j) vec = vec && sh.s[k][j] % 4 == 0;
     }
   }
-  if (vec) {
+  if (rank <= 2) {  // the two-axis kernel: no index arithmetic, several rows in flight per block
+    CwShape2 s2;
+    s2.d0g = sh.d[0] / (vec ? 4 : 1);
+    s2.d1 = sh.d[1];
+    for (int k = 0; k < 3; ++k) {
+      s2.s0[k] = sh.s[k][0];
+      s2.s1[k] = sh.s[k][1];
+    }
+    const unsigned gy = cdiv<unsigned>(s2.d1, kCwRows);
+    const dim3 grid(cdiv<unsigned>(s2.d0g, 256), gy < 65535u ? gy : 65535u), block(256);
+    const bool nt = total * sizeof(float) >= dev->stream_threshold;
+    if (vec && nt) hipLaunchKernelGGL((cwise_bcast2_kernel<FN, 4, true>), grid, block, 0, dev->stream, s2, p0, p1, p2, out);
+    else if (vec) hipLaunchKernelGGL((cwise_bcast2_kernel<FN, 4, false>), grid, block, 0, dev->stream, s2, p0, p1, p2, out);
+    else hipLaunchKernelGGL((cwise_bcast2_kernel<FN, 1, false>), grid, block, 0, dev->stream, s2, p0, p1, p2, out);
+  } else if (vec) {
     const size_t groups = total / 4;
     hipLaunchKernelGGL((cwise_bcast_kernel<FN, 4>), dim3(cw_grid(groups, 256, dev)), dim3(256), 0, dev->stream, sh, p0, p1,
                        p2, out, groups);
@@ -244,6 +414,33 @@ static int cw_launch_reduce(dyhip_device* dev, const unsigned* full, const unsig
   }
   c.n_out = cw_size(c.kd);
   c.n_red = cw_size(c.rd);
+  {
+    // the reduced axes as one axis, if every operand walks them alike
+    unsigned rd2[5];
+    size_t rs2[3][5], rs_in[3][5];
+    for (int k = 0; k < 3; ++k)
+      for (int j = 0; j < 5; ++j) rs_in[k][j] = c.rs[k][j];
+    if (c.n_red >= 64 && c.n_red <= 0xFFFFFFFFull && cw_collapse(c.rd, rs_in, cw_inputs(FN), rd2, rs2) == 1) {
+      const float* ps[3] = {p0, p1, p2};
+      bool vec = c.n_red % 4 == 0;
+      for (int k = 0; k < cw_inputs(FN); ++k) {
+        vec = vec && (rs2[k][0] == 0 || rs2[k][0] == 1);
+        if (rs2[k][0] == 1) {
+          vec = vec && aligned16(ps[k]);
+          for (int j = 0; j < 5; ++j) vec = vec && c.ks[k][j] % 4 == 0;
+        }
+      }
+      for (int j = 0; j < 5; ++j) {
+        c.rd[j] = rd2[j];
+        for (int k = 0; k < 3; ++k) c.rs[k][j] = rs2[k][j];
+      }
+      const dim3 grid(cw_grid(c.n_out, 4, dev)), block(256);
+      if (vec) hipLaunchKernelGGL((cwise_reduce_row_kernel<FN, true>), grid, block, 0, dev->stream, c, p0, p1, p2, out);
+      else hipLaunchKernelGGL((cwise_reduce_row_kernel<FN, false>), grid, block, 0, dev->stream, c, p0, p1, p2, out);
+      DYHIP_CHECK_LAUNCH();
+      return DYHIP_OK;
+    }
+  }
   if (c.n_red >= 64)
     hipLaunchKernelGGL(cwise_reduce_wave_kernel<FN>, dim3(cw_grid(c.n_out, 4, dev)), dim3(256), 0, dev->stream, c, p0, p1, p2,
                        out);
