@@ -176,9 +176,12 @@ def time_loop(dev, fns, reps):
 def per_kernel_table(dev, named, sets, reps, use_graph=True):
     """named: list of (name, bytes, fn(set)); returns a list of dicts with us / GB/s / fraction of peak."""
     out = []
-    # One replay holds at least 24 launches (the set list repeated if need be): the boundary between two replays of a
-    # graph costs about 5 us on this GPU, which a graph of 8 launches would add to every launch as 0.6 us.
-    rounds = max(1, -(-24 // max(len(sets), 1)))
+    # One replay holds at least 192 launches (the set list repeated): the boundary between two replays of a graph
+    # costs about 5 us on this GPU (measured from inside the kernels: 6.5 us from the last block of one replay to the
+    # first block of the next, against 1.5 us between two launches of one replay), which a graph of 8 launches would
+    # add to every launch as 0.6 us and one of 24 as 0.2 us.  The figure is then what a launch costs inside a long
+    # graph, such as the 2500-node LSTM-LM step.
+    rounds = max(1, -(-192 // max(len(sets), 1)))
     for name, nbytes, fn in named:
         fns = [(lambda s=s: fn(s)) for s in sets] * rounds
         if use_graph:
@@ -1039,19 +1042,31 @@ def main():
         graphs = [_Eager(r) for r in range(sweep.R)]
     else:
         graphs = [capture(dev, [lambda r=r: sweep.run_step(r)]) for r in range(sweep.R)]
+    # Eight consecutive steps per graph where the step count allows: the boundary between two graph replays costs
+    # about 5 us here (see per_kernel_table), 4 % of a 127 us step if every step is a replay of its own.  The rest of
+    # the K steps, and the warmup, are single-step replays.
+    G = 8
+    multi = [] if args.no_graph or sweep.R % G else [
+        capture(dev, [lambda r=r: sweep.run_step(r) for r in range(k, k + G)]) for k in range(0, sweep.R, G)]
     for s in range(args.warmup):
         graphs[s % sweep.R].launch()
+    for g in multi:
+        g.launch()
     dev.sync()
     t0 = time.perf_counter()
     dev.timer_start()
-    for s in range(args.steps):
+    s = 0
+    while multi and args.steps - s >= G:
+        multi[(s // G) % len(multi)].launch()
+        s += G
+    for s in range(s, args.steps):
         graphs[s % sweep.R].launch()
     ms = dev.timer_stop()
     dev.sync()
     wall_ms = (time.perf_counter() - t0) * 1e3
     ms_per_step = ms / args.steps
     value = sweep.step_bytes / (ms_per_step * 1e-3) / 1e9
-    for g in graphs:
+    for g in graphs + multi:
         g.destroy()
     # ---- per-kernel achieved bandwidth ---------------------------------------------
     table = per_kernel_table(dev, sweep.kernels, sweep.sets, args.kernel_reps, use_graph=not args.no_graph)
@@ -1100,6 +1115,7 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "cfg2_elementwise_reduction_sweep", "tensor": "4096x1024 fp32",
                    "kernels_per_step": len(sweep.kernels), "rotating_buffer_sets": sweep.R,
+                   "steps_per_graph_replay": G if multi else 1,
                    "bytes_per_step": int(sweep.step_bytes)},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
         "wall_ms_per_step": round(wall_ms / args.steps, 5),

@@ -151,6 +151,52 @@ __global__ __launch_bounds__(kEwThreads) void ew_scalar_kernel(EwArgs a, F f) {
   }
 }
 
+// A batch-broadcast launch whose batch elements are shorter than a tile: a thread keeps one in-batch offset and walks
+// U consecutive batch elements, so the broadcast inputs are loaded once per thread and every thread still has U
+// accesses per stream in flight (with one tile per batch element a 1024-float element left three quarters of each
+// tile masked off: one access per thread and 4096 blocks).  Loads are unconditional on clamped addresses; only the
+// stores are guarded.
+template <int NIN, bool ACC, int BMASK, bool NT, int U, class F>
+__global__ __launch_bounds__(kEwThreads) void ew_bcast_vec4_kernel(EwArgs a, unsigned bd, F f) {
+  const size_t n4 = a.n >> 2;
+  const size_t j = size_t(blockIdx.x) * kEwThreads + threadIdx.x;
+  const bool live = j < n4;
+  const size_t jc = live ? j : n4 - 1;
+  const unsigned b0 = blockIdx.y * U;
+  float4 v[NIN > 0 ? NIN : 1][U];
+  float4 o[U];
+#pragma unroll
+  for (int k = 0; k < NIN; ++k)
+    if ((BMASK >> k) & 1) v[k][0] = reinterpret_cast<const float4*>(a.in[k])[jc];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const unsigned b = b0 + u < bd ? b0 + u : bd - 1;
+    const size_t at = size_t(b) * n4 + jc;
+#pragma unroll
+    for (int k = 0; k < NIN; ++k)
+      if (!((BMASK >> k) & 1)) v[k][u] = ldg4<NT>(reinterpret_cast<const float4*>(a.in[k]) + at);
+    if (ACC) o[u] = ldg4<NT>(reinterpret_cast<const float4*>(a.out) + at);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  float4 r[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+    const float4 x0 = NIN > 0 ? v[0][(BMASK & 1) ? 0 : u] : z;
+    const float4 x1 = NIN > 1 ? v[NIN > 1 ? 1 : 0][(BMASK & 2) ? 0 : u] : z;
+    const float4 x2 = NIN > 2 ? v[NIN > 2 ? 2 : 0][(BMASK & 4) ? 0 : u] : z;
+    const float4 od = ACC ? o[u] : z;
+    r[u].x = f(x0.x, x1.x, x2.x, od.x);
+    r[u].y = f(x0.y, x1.y, x2.y, od.y);
+    r[u].z = f(x0.z, x1.z, x2.z, od.z);
+    r[u].w = f(x0.w, x1.w, x2.w, od.w);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+    if (live && b0 + u < bd) stg4<NT>(reinterpret_cast<float4*>(a.out) + size_t(b0 + u) * n4 + j, r[u]);
+}
+
 // Launch over an (n x bd) output.  Inputs whose bit is set in BMASK have batch 1.
 template <int NIN, bool ACC, int BMASK, class F>
 int ew_launch(dyhip_device* dev, size_t n, unsigned bd, const float* in0, const float* in1, const float* in2,
@@ -177,7 +223,13 @@ int ew_launch(dyhip_device* dev, size_t n, unsigned bd, const float* in0, const 
   a.tiles_per_batch = static_cast<unsigned>(tiles);
   const dim3 grid(static_cast<unsigned>(tiles * bd)), block(kEwThreads);
   const bool stream = n * bd * sizeof(float) >= dev->stream_threshold;
-  if (!vec) {
+  if (BMASK != 0 && vec && n / 4 < size_t(kEwThreads) * U && cdiv<size_t>(bd, U) <= 65535) {
+    const dim3 g2(static_cast<unsigned>(cdiv<size_t>(n / 4, kEwThreads)), static_cast<unsigned>(cdiv<size_t>(bd, U)));
+    if (stream)
+      hipLaunchKernelGGL((ew_bcast_vec4_kernel<NIN, ACC, BMASK, true, U, F>), g2, block, 0, dev->stream, a, bd, f);
+    else
+      hipLaunchKernelGGL((ew_bcast_vec4_kernel<NIN, ACC, BMASK, false, U, F>), g2, block, 0, dev->stream, a, bd, f);
+  } else if (!vec) {
     hipLaunchKernelGGL((ew_scalar_kernel<NIN, ACC, BMASK, F>), grid, block, 0, dev->stream, a, f);
   } else if (stream) {
     hipLaunchKernelGGL((ew_vec4_kernel<NIN, ACC, BMASK, true, U, F>), grid, block, 0, dev->stream, a, f);
