@@ -165,10 +165,12 @@ __global__ __launch_bounds__(64 * kCombSlices) void combine_partials_kernel(size
 }
 
 // The same for rows of float4 with many more blocks: a block owns 8 float4 columns (one 128-byte line of every
-// partial row) and 32 row slots; slot q adds rows q, q+32, ... in ascending order with four loads in flight,
-// then eight threads per column add every eighth slot and one adds those eight: a fixed order again.
-constexpr int kCombVecSlots = 32;
+// partial row) and kCombVecSlots row slots (32, or 64 for more than 128 partial rows, so that 256 rows are one batch of
+// four loads per thread, all in flight at once, instead of two dependent batches); slot q adds rows q, q+slots, ...
+// in ascending order, then eight threads per column add every eighth slot and one adds those eight: a fixed order
+// again for a given number of partial rows.
 constexpr int kCombVecCols = 8;
+template <int kCombVecSlots>
 __global__ __launch_bounds__(kCombVecCols * kCombVecSlots) void combine_partials_vec_kernel(unsigned n4, unsigned splits,
                                                                                const float4* __restrict__ partial0,
                                                                                float4* __restrict__ out0,
@@ -227,10 +229,15 @@ static void launch_combine(dyhip_device* dev, size_t n, unsigned splits, const f
                            float* o1, int accumulate) {
   if (n % 4 == 0 && splits >= 32 && aligned16(p0) && aligned16(o0) && (p1 == nullptr || (aligned16(p1) && aligned16(o1)))) {
     const unsigned n4 = static_cast<unsigned>(n / 4);
-    hipLaunchKernelGGL(combine_partials_vec_kernel, dim3(cdiv<unsigned>(n4, kCombVecCols), p1 != nullptr ? 2 : 1),
-                       dim3(kCombVecCols * kCombVecSlots), 0, dev->stream, n4, splits, reinterpret_cast<const float4*>(p0),
-                       reinterpret_cast<float4*>(o0), reinterpret_cast<const float4*>(p1), reinterpret_cast<float4*>(o1),
-                       accumulate);
+    const dim3 grid(cdiv<unsigned>(n4, kCombVecCols), p1 != nullptr ? 2 : 1);
+    if (splits > 128)
+      hipLaunchKernelGGL(combine_partials_vec_kernel<64>, grid, dim3(kCombVecCols * 64), 0, dev->stream, n4, splits,
+                         reinterpret_cast<const float4*>(p0), reinterpret_cast<float4*>(o0),
+                         reinterpret_cast<const float4*>(p1), reinterpret_cast<float4*>(o1), accumulate);
+    else
+      hipLaunchKernelGGL(combine_partials_vec_kernel<32>, grid, dim3(kCombVecCols * 32), 0, dev->stream, n4, splits,
+                         reinterpret_cast<const float4*>(p0), reinterpret_cast<float4*>(o0),
+                         reinterpret_cast<const float4*>(p1), reinterpret_cast<float4*>(o1), accumulate);
     return;
   }
   const dim3 grid((unsigned)cdiv<size_t>(n, 64), p1 != nullptr ? 2 : 1);
@@ -926,7 +933,12 @@ static int ln_team_waves(size_t n) { return n <= 4096 ? 4 : n <= 8192 ? 8 : 16; 
 static unsigned ln_bwd_blocks(size_t n, unsigned bd) {
   const unsigned per_block = n <= 2048 ? unsigned(kLnWavesBwd) : unsigned(16 / ln_team_waves(n));
   unsigned blocks = cdiv<unsigned>(bd, per_block);
-  return blocks > kLnBwdMaxBlocks ? kLnBwdMaxBlocks : blocks;
+  // one block per CU keeps the partial rows few; once every wave of those blocks would own eight rows or more the
+  // partial rows no longer matter and a second block per CU (its 64 KB of LDS fits beside the first up to n = 1024)
+  // hides the row reductions (65536 rows of 1024: 192 -> 188 us)
+  const unsigned cap =
+      n <= 1024 && bd / (kLnBwdMaxBlocks * per_block) >= 8 ? 2 * kLnBwdMaxBlocks : kLnBwdMaxBlocks;
+  return blocks > cap ? cap : blocks;
 }
 
 // Scratch of dyhip_layer_norm_backward_static: the per-block dg / db partial rows (or the per-row
