@@ -489,7 +489,9 @@ PMC_KERNELS = [
     ("AccMul2", "cmult_bwd"), ("Mul2", "cmult_fwd"), ("AccIn0", "sum_batches_bwd"),
     ("batch_reduce_kernel", "sum_batches_fwd"), ("ln_fwd_wave_kernel", "layer_norm_fwd"),
     ("ln_bwd_wave_kernel", "layer_norm_bwd_main"), ("combine_partials", "layer_norm_bwd_combine"),
-    ("lookup_gather_kernel", "lookup_gather"), ("plan_group_kernel", "lookup_plan"),
+    ("lookup_gather_kernel", "lookup_gather"), ("plan_direct_kernel", "lookup_plan"),
+    ("cwise_bcast2_kernel<2,", "cwise_quotient_fwd"), ("cwise_bcast2_kernel<5,", "cwise_quotient_bwd_arg0"),
+    ("cwise_reduce_row_kernel<6,", "cwise_quotient_bwd_arg1"),
     ("scatter_runs_kernel", "lookup_scatter_runs"), ("lse_cols_kernel", "pnls_fwd"), ("pnls_bwd_kernel", "pnls_bwd"),
     ("lstm_step_fwd_kernel", "lstm_step_fwd"), ("lstm_step_bwd_kernel", "lstm_step_bwd"),
     ("skinny_tn_kernel<false, false>", "lstm_rec_bwd_packed"),
@@ -541,6 +543,9 @@ def print_pmc_summary(fetch_db, write_db, unique_ids):
             "sum_batches_bwd": 2 * S + S // 64, "layer_norm_fwd": 2 * S + 2 * LN_N * 4,
             "layer_norm_bwd_main": 4 * S + 4 * LN_N * 4, "lookup_gather": 2 * G + CFG3["n"] * 4,
             "lookup_scatter_runs": G + 2 * unique_ids * CFG3["D"] * 4, "pnls_fwd": X, "pnls_bwd": 3 * X,
+            # 1024 x 4096 by 1 x 4096: S in and out + the divisor row; dy, the row and dx in and out; dy, both operands
+            "cwise_quotient_fwd": 2 * S + 4096 * 4, "cwise_quotient_bwd_arg0": 3 * S + 4096 * 4,
+            "cwise_quotient_bwd_arg1": 2 * S + 3 * 4096 * 4,
             # cfg-5 timestep at H = 1024, B = 128 (HB = H*B floats): packed Wh once + 13 HB; packed Wh^T once + 4 HB
             # in + 4 slices of HB out; 4+4+4+4+1 HB in and out of the packed cell backward
             "lstm_step_fwd": (4 * 1024 * 1024 + 13 * 1024 * 128) * 4, "lstm_rec_bwd_packed": (4 * 1024 * 1024 + 8 * 1024 * 128) * 4,
