@@ -489,6 +489,7 @@ PMC_KERNELS = [
     ("AccMul2", "cmult_bwd"), ("Mul2", "cmult_fwd"), ("AccIn0", "sum_batches_bwd"),
     ("batch_reduce_kernel", "sum_batches_fwd"), ("ln_fwd_wave_kernel", "layer_norm_fwd"),
     ("ln_bwd_wave_kernel", "layer_norm_bwd_main"), ("combine_partials", "layer_norm_bwd_combine"),
+    ("ln_fwd_team_kernel", "layer_norm_wide_fwd"), ("ln_bwd_team_kernel", "layer_norm_wide_bwd_main"),
     ("lookup_gather_kernel", "lookup_gather"), ("plan_direct_kernel", "lookup_plan"),
     ("cwise_bcast2_kernel<2,", "cwise_quotient_fwd"), ("cwise_bcast2_kernel<5,", "cwise_quotient_bwd_arg0"),
     ("cwise_reduce_row_kernel<6,", "cwise_quotient_bwd_arg1"),
@@ -510,14 +511,31 @@ def print_pmc_summary(fetch_db, write_db, unique_ids):
     import sqlite3
 
     def table(path):
+        # per kernel name; the combine kernel of the LayerNorm backward runs at two shapes (the sweep's 4096 rows of
+        # 1024 and the wide-row extra's 1024 rows of 4096): its launches are told apart by grid size, the smaller
+        # grid being the sweep's
         cur = sqlite3.connect(path).cursor()
-        rows = cur.execute("select kernel_name, count(*), avg(value) from counters_collection group by kernel_name")
-        return {k: (c, a) for k, c, a in rows}
+        cols = [r[1] for r in cur.execute("pragma table_info(counters_collection)")]
+        grid = next((c for c in ("grid_size", "grid_size_x", "grid_x") if c in cols), None)
+        if grid is None:
+            rows = cur.execute("select kernel_name, count(*), avg(value) from counters_collection group by kernel_name")
+            return {k: (c, a) for k, c, a in rows}
+        rows = cur.execute("select kernel_name, %s, count(*), avg(value) from counters_collection group by kernel_name, %s"
+                           % (grid, grid)).fetchall()
+        small = min((g for k, g, _, _ in rows if "combine_partials" in k), default=None)
+        out = {}
+        for k, g, c, a in rows:
+            key = k + " [wide rows]" if "combine_partials" in k and g != small else k
+            c0, a0 = out.get(key, (0, 0.0))
+            out[key] = (c0 + c, (a0 * c0 + a * c) / (c0 + c))
+        return out
 
     def entry(kname):
         if "IdentityFwd" in kname:  # the calibration copy: 4th template argument = streaming accesses or not
             m = re.search(r"ew_vec4_kernel<\s*\d+,\s*\w+,\s*\d+,\s*(true|false)", kname)
             return "copy_streaming" if (m and m.group(1) == "true") else "copy_plain"
+        if "combine_partials" in kname and kname.endswith("[wide rows]"):
+            return "layer_norm_wide_bwd_combine"
         for sub, name in PMC_KERNELS:
             if sub in kname:
                 return name
@@ -541,7 +559,8 @@ def print_pmc_summary(fetch_db, write_db, unique_ids):
     algo = {"tanh_fwd": 2 * S, "logistic_fwd": 2 * S, "rectify_fwd": 2 * S, "tanh_bwd": 4 * S, "logistic_bwd": 4 * S,
             "rectify_bwd": 4 * S, "cmult_fwd": 3 * S, "cmult_bwd": 4 * S, "sum_batches_fwd": S + S // 64,
             "sum_batches_bwd": 2 * S + S // 64, "layer_norm_fwd": 2 * S + 2 * LN_N * 4,
-            "layer_norm_bwd_main": 4 * S + 4 * LN_N * 4, "lookup_gather": 2 * G + CFG3["n"] * 4,
+            "layer_norm_bwd_main": 4 * S + 4 * LN_N * 4, "layer_norm_wide_fwd": 2 * S + 2 * 4096 * 4,
+            "layer_norm_wide_bwd_main": 4 * S + 4 * 4096 * 4, "lookup_gather": 2 * G + CFG3["n"] * 4,
             "lookup_scatter_runs": G + 2 * unique_ids * CFG3["D"] * 4, "pnls_fwd": X, "pnls_bwd": 3 * X,
             # 1024 x 4096 by 1 x 4096: S in and out + the divisor row; dy, the row and dx in and out; dy, both operands
             "cwise_quotient_fwd": 2 * S + 4096 * 4, "cwise_quotient_bwd_arg0": 3 * S + 4096 * 4,
@@ -593,6 +612,8 @@ def print_pmc_summary(fetch_db, write_db, unique_ids):
     t = dict(traffic)
     if "layer_norm_bwd_main" in t:
         t["layer_norm_bwd"] = t.pop("layer_norm_bwd_main") + t.pop("layer_norm_bwd_combine", 0.0)
+    if "layer_norm_wide_bwd_main" in t:
+        t["layer_norm_wide_bwd"] = t.pop("layer_norm_wide_bwd_main") + t.pop("layer_norm_wide_bwd_combine", 0.0)
     if "cmult_bwd" in t:
         t["cmult_bwd_arg0"] = t["cmult_bwd_arg1"] = t.pop("cmult_bwd")
     for name in sorted(t):
@@ -671,12 +692,13 @@ def lstm_lm(steps, warmup=12, use_graph=True):
     # ms_per_step is the faster one.  The collector is off inside the timed loop: in this process, which holds the
     # tables of every earlier leg, one full collection is a 5-10 ms pause of the host thread that launches the steps
     # (7.1 instead of 6.6 ms per step over 30 steps; a kernel trace shows equal kernel durations either way).
-    for path, tb in (("fused", True), ("nodes", False), ("nodes_eager", False)):
+    for path, tb in (("fused", True), ("fused_dropout", True), ("nodes", False), ("nodes_eager", False)):
         runs = []
-        for _ in range(2):
+        for _ in range(1 if path == "fused_dropout" else 2):
             dev = Device(0, mem_mb=(1024, 1024, 512, 1024))
+            drop = 0.5 if path == "fused_dropout" else 0.0  # CompactVanillaLSTMBuilder::set_dropout(d, d_h)
             lm = LstmLM(dev, V, E, H, L, B, T, lr=0.1, clip=5.0, time_batched=tb, path=path.split("_")[0],
-                        defer_weight_grads=path == "nodes")
+                        defer_weight_grads=path == "nodes", dropout=drop, dropout_h=drop)
             lm.stage(batches[0])
             if use_graph:
                 lm.capture()
@@ -699,7 +721,7 @@ def lstm_lm(steps, warmup=12, use_graph=True):
                 lm.graph.destroy()
             dev.close()
         dt, first, last = min(runs)
-        key = {"fused": "fused_cell_path", "nodes": "node_at_a_time_path",
+        key = {"fused": "fused_cell_path", "fused_dropout": "fused_cell_path_with_dropout_0.5_0.5", "nodes": "node_at_a_time_path",
                "nodes_eager": "node_at_a_time_path_weight_gradients_per_node"}[path]
         res[key] = {"ms_per_step": round(dt * 1e3, 3), "tokens_per_s": round(T * B / dt, 1),
                     "ms_per_step_of_each_instance": [round(r[0] * 1e3, 3) for r in runs],
