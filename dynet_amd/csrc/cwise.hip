@@ -216,7 +216,7 @@ __global__ __launch_bounds__(256) void cwise_reduce_wave_kernel(CwReduce c, cons
 // The reduced axes collapse to one (the usual case: the sum over the row of a matrix): the kept index is decomposed
 // once per output, the walk along the reduced axis needs no division, and four terms per lane are in flight.
 // VEC: every operand runs along the reduced axis with stride 1 (128-bit loads) or stride 0.
-template <int FN, bool VEC>
+template <int FN, bool VEC, bool NT>
 __global__ __launch_bounds__(256) void cwise_reduce_row_kernel(CwReduce c, const float* __restrict__ p0,
                                                                const float* __restrict__ p1,
                                                                const float* __restrict__ p2, float* __restrict__ out) {
@@ -225,16 +225,31 @@ __global__ __launch_bounds__(256) void cwise_reduce_row_kernel(CwReduce c, const
   const float* ps[3] = {p0, p1, p2};
   for (size_t o = size_t(blockIdx.x) * 4 + (threadIdx.x >> 6); o < c.n_out; o += size_t(gridDim.x) * 4) {
     size_t base[3] = {0, 0, 0};
-    size_t r = o;
+    size_t r = o;  // the same in every lane of the wave: the branches below are uniform
 #pragma unroll
     for (int j = 0; j < 5; ++j) {
-      const size_t q = r / c.kd[j];
-      const size_t i = r - q * c.kd[j];
+      const unsigned kd = c.kd[j];
+      if (kd == 1) continue;
+      // no division once the rest fits the axis (always so with one kept axis: the kernel's loads used to start
+      // behind five 64-bit divisions), a 32-bit one while it fits 32 bits
+      size_t q, i;
+      if (r < kd) {
+        q = 0;
+        i = r;
+      } else if (r <= 0xFFFFFFFFull) {
+        const unsigned r32 = unsigned(r), q32 = r32 / kd;
+        q = q32;
+        i = r32 - q32 * kd;
+      } else {
+        q = r / kd;
+        i = r - q * kd;
+      }
       r = q;
 #pragma unroll
       for (int k = 0; k < NIN; ++k) base[k] += i * c.ks[k][j];
     }
     const unsigned nr = unsigned(c.n_red);
+    const float old = lane == 0 ? out[o] : 0.f;  // fetched beside the terms, not after the sum
     float acc = 0.f;
     if (VEC) {
       for (unsigned q0 = 0; q0 < nr; q0 += 4 * 64 * 4) {
@@ -245,7 +260,7 @@ __global__ __launch_bounds__(256) void cwise_reduce_row_kernel(CwReduce c, const
 #pragma unroll
           for (int k = 0; k < 3; ++k) {
             if (k >= NIN) v[u][k] = make_float4(0.f, 0.f, 0.f, 0.f);
-            else if (c.rs[k][0] == 1) v[u][k] = *reinterpret_cast<const float4*>(ps[k] + base[k] + q);
+            else if (c.rs[k][0] == 1) v[u][k] = ldg4<NT>(reinterpret_cast<const float4*>(ps[k] + base[k] + q));
             else {
               const float b = ps[k][base[k]];
               v[u][k] = make_float4(b, b, b, b);
@@ -277,7 +292,7 @@ __global__ __launch_bounds__(256) void cwise_reduce_row_kernel(CwReduce c, const
       }
     }
     const float t = wave_sum(acc);
-    if (lane == 0) out[o] += t;
+    if (lane == 0) out[o] = old + t;
   }
 }
 
@@ -435,8 +450,11 @@ static int cw_launch_reduce(dyhip_device* dev, const unsigned* full, const unsig
         for (int k = 0; k < 3; ++k) c.rs[k][j] = rs2[k][j];
       }
       const dim3 grid(cw_grid(c.n_out, 4, dev)), block(256);
-      if (vec) hipLaunchKernelGGL((cwise_reduce_row_kernel<FN, true>), grid, block, 0, dev->stream, c, p0, p1, p2, out);
-      else hipLaunchKernelGGL((cwise_reduce_row_kernel<FN, false>), grid, block, 0, dev->stream, c, p0, p1, p2, out);
+      // operands far larger than the caches are read once: streaming loads
+      const bool nt = vec && c.n_out * c.n_red * sizeof(float) >= dev->stream_threshold;
+      if (nt) hipLaunchKernelGGL((cwise_reduce_row_kernel<FN, true, true>), grid, block, 0, dev->stream, c, p0, p1, p2, out);
+      else if (vec) hipLaunchKernelGGL((cwise_reduce_row_kernel<FN, true, false>), grid, block, 0, dev->stream, c, p0, p1, p2, out);
+      else hipLaunchKernelGGL((cwise_reduce_row_kernel<FN, false, false>), grid, block, 0, dev->stream, c, p0, p1, p2, out);
       DYHIP_CHECK_LAUNCH();
       return DYHIP_OK;
     }

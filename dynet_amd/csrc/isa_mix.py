@@ -22,7 +22,7 @@ FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950", "-ffp-contract=off", "-Xc
 HOT = ["ew_vec4_kernel<2, true, 0, true, 2, dyhip::AccMul2", "ew_vec4_kernel<1, false, 0, true, 4, dyhip::TanhFwd",
        "ew_bcast_vec4_kernel<1, true, 1, true, 4, dyhip::AccIn0", "batch_reduce_kernel<4, false, true>",
        "ln_fwd_wave_kernel<4, true>", "ln_bwd_wave_kernel<4, true, 8, true, true>", "ln_bwd_team_kernel<4, true>",
-       "combine_partials_vec_kernel<64>", "cwise_bcast2_kernel<2, 4, true>", "cwise_reduce_row_kernel<6, true>",
+       "combine_partials_vec_kernel<64>", "cwise_bcast2_kernel<2, 4, true>", "cwise_reduce_row_kernel<6, true, true>",
        "lookup_gather_kernel<HIP_vector_type<float, 4u>, false, true>", "plan_direct_kernel<16>", "plan_group_kernel<true>",
        "scatter_runs_kernel<HIP_vector_type<float, 4u>, true>", "lse_cols_kernel<true, true>", "pnls_bwd_kernel<true, true, true>",
        "lstm_step_fwd_kernel<false, 2>", "lstm_step_bwd_kernel", "skinny_tn_kernel<true, true>", "lstm_gates_skinny_kernel",
