@@ -682,12 +682,15 @@ static int build_plan(dyhip_device* dev, unsigned n, const unsigned* ids_dev, un
   Plan out;
   plan_parts(plan, n, &out);
   const unsigned bits = key_bits(vocab);  // keys are min(id, vocab) <= vocab
-  if (n <= kPlanSmallMax && bits <= 16) {
-    const unsigned per_wave = cdiv<unsigned>(cdiv<unsigned>(n, kPlanWaves), 64u);  // 64-entry steps of a wavefront
+  // 64-entry steps of a wavefront; a wavefront keeps its keys in registers, and 64 of them do not fit beside the
+  // rest (the 64-step form spilled and took 122 us for 32 768 ids): beyond 32 steps the route below takes over
+  const unsigned per_wave = cdiv<unsigned>(cdiv<unsigned>(n, kPlanWaves), 64u);
+  if (n <= kPlanSmallMax && bits <= 16 && per_wave <= 32) {
     const dim3 grid(kPlanBuckets), block(kPlanThreads);
     if (per_wave <= 4) hipLaunchKernelGGL(plan_direct_kernel<4>, grid, block, 0, dev->stream, n, vocab, ids_dev, out);
+    else if (per_wave <= 8) hipLaunchKernelGGL(plan_direct_kernel<8>, grid, block, 0, dev->stream, n, vocab, ids_dev, out);
     else if (per_wave <= 16) hipLaunchKernelGGL(plan_direct_kernel<16>, grid, block, 0, dev->stream, n, vocab, ids_dev, out);
-    else hipLaunchKernelGGL(plan_direct_kernel<64>, grid, block, 0, dev->stream, n, vocab, ids_dev, out);
+    else hipLaunchKernelGGL(plan_direct_kernel<32>, grid, block, 0, dev->stream, n, vocab, ids_dev, out);
     DYHIP_CHECK_LAUNCH();
     return DYHIP_OK;
   }

@@ -926,6 +926,9 @@ def _check_plan(dev, plan, ids, vocab):
 
 @pytest.mark.parametrize("vocab,n,kind", [
     (50000, 65535, "zipf"),        # the largest id vector of the one-kernel plan
+    (50000, 4480, "zipf"),         # 16-bit keys, 5 steps of 64 ids per wavefront: the 8-step form of the direct kernel
+    (50000, 32768, "zipf"),        # ... 32 steps: the longest the direct kernel takes
+    (50000, 32769, "zipf"),        # ... 33: the compact-and-sort kernel although the keys fit 16 bits
     (50000, 65536, "zipf"),        # the first size of the radix-sort plan
     (300000, 70001, "zipf"),
     (1 << 20, 30000, "uniform"),   # 21-bit ids: two sort passes beyond the bucket digit
