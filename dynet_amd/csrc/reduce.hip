@@ -1156,11 +1156,15 @@ int dyhip_layer_norm_backward(dyhip_device* dev, size_t n, unsigned bd, const fl
                  *d4 = reinterpret_cast<const float4*>(dEdf);
     float4* dx4 = reinterpret_cast<float4*>(dx);
     const bool stream = n * size_t(bd) * sizeof(float) >= dev->stream_threshold;
+// The row after the current one is fetched ahead, except for rows of 1028..2044 floats: two rows of eight groups a
+// lane do not fit the registers beside the partial sums, and with the bounds-checked loads of a row that does not
+// fill every lane the spills cost more than the prefetch gains (2048 rows of 1536: 32.1 -> 15.4 us without it; rows
+// of exactly 2048 floats keep it: 18.1 against 23.9 us).
 #define DYHIP_LN_BWD_LAUNCH(VPL, NT, WAVES, FULL)                                                           \
-  hipLaunchKernelGGL((ln_bwd_wave_kernel<VPL, NT, WAVES, true, FULL>), grid, block, lds, dev->stream, n4, bd, x4, g4, \
-                     d4, dx4, part_dg, part_db)
+  hipLaunchKernelGGL((ln_bwd_wave_kernel<VPL, NT, WAVES, (VPL < 8 || FULL), FULL>), grid, block, lds, dev->stream, n4, bd, x4, \
+                     g4, d4, dx4, part_dg, part_db)
 #define DYHIP_LN_BWD_LDS(VPL, NT, WAVES, FULL)                                                              \
-  DYHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&ln_bwd_wave_kernel<VPL, NT, WAVES, true, FULL>), \
+  DYHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&ln_bwd_wave_kernel<VPL, NT, WAVES, (VPL < 8 || FULL), FULL>), \
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 128 << 10))
 #define DYHIP_LN_BWD(VPL)                                                                                  \
   do {                                                                                                     \
