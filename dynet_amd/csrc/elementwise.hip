@@ -129,6 +129,15 @@ __global__ __launch_bounds__(kEwThreads) void ew_vec4_kernel(EwArgs a, F f) {
     t.template load<false>(a, base4, j0, n4);
     t.template compute_store<false>(a, base4, j0, n4, f);
   }
+  // A flat tensor (nothing broadcast) whose length is not a multiple of four: its last one to three elements.
+  if (BMASK == 0 && blockIdx.x == 0 && threadIdx.x < (a.n & 3)) {
+    const size_t e = (n4 << 2) + threadIdx.x;
+    const float x0 = NIN > 0 ? a.in[0][e] : 0.f;
+    const float x1 = NIN > 1 ? a.in[NIN > 1 ? 1 : 0][e] : 0.f;
+    const float x2 = NIN > 2 ? a.in[NIN > 2 ? 2 : 0][e] : 0.f;
+    const float od = ACC ? a.out[e] : 0.f;
+    a.out[e] = f(x0, x1, x2, od);
+  }
 }
 
 template <int NIN, bool ACC, int BMASK, class F>
@@ -215,10 +224,12 @@ int ew_launch(dyhip_device* dev, size_t n, unsigned bd, const float* in0, const 
   a.in[2] = in2;
   a.out = out;
   a.n = n;
-  bool vec = (n % 4 == 0) && aligned16(out);
+  // 128-bit accesses need 16-byte aligned pointers and, when an input is broadcast, batch elements that keep that
+  // alignment; a flat tensor of any length >= 4 qualifies (its last n % 4 elements are done one by one)
+  bool vec = (BMASK == 0 ? n >= 4 : n % 4 == 0) && aligned16(out);
   for (int k = 0; k < NIN; ++k) vec = vec && aligned16(a.in[k]);
   const size_t per_tile = vec ? size_t(kEwThreads) * U * 4 : size_t(kEwThreads) * 4;
-  const size_t tiles = cdiv(n, per_tile);
+  const size_t tiles = cdiv(vec ? n - n % 4 : n, per_tile);
   DYHIP_REQUIRE(tiles * bd < (size_t(1) << 31), "elementwise launch too large: %zu tiles x %u batches", tiles, bd);
   a.tiles_per_batch = static_cast<unsigned>(tiles);
   const dim3 grid(static_cast<unsigned>(tiles * bd)), block(kEwThreads);

@@ -74,8 +74,17 @@ __global__ __launch_bounds__(kLseThreads) void lse_cols_kernel(size_t rows, cons
   float picked = 0.f;
   if (ids != nullptr && threadIdx.x == 0) picked = x[ids[b]];
   if (VEC) {
-    const float4* p4 = reinterpret_cast<const float4*>(px);
-    const size_t n4 = rows >> 2;
+    // A column starts wherever b * rows falls: up to three leading elements bring it to a 16-byte boundary, the body
+    // runs in 128-bit groups, up to three elements trail (taken by the last threads of the block).  With rows a
+    // multiple of four and an aligned x there is only the body.
+    const size_t head = min(size_t((4u - unsigned((reinterpret_cast<uintptr_t>(px) >> 2) & 3u)) & 3u), rows);
+    const size_t n4 = (rows - head) >> 2;
+    if (threadIdx.x < head) ms_push1(a, px[threadIdx.x]);
+    {
+      const size_t e = head + (n4 << 2) + (kLseThreads - 1 - threadIdx.x);
+      if (e < rows) ms_push1(a, px[e]);
+    }
+    const float4* p4 = reinterpret_cast<const float4*>(px + head);
     size_t i = threadIdx.x;
     // eight independent 128-bit loads in flight per thread before the first exp
     for (; i + 7 * kLseThreads < n4; i += 8 * kLseThreads) {
@@ -133,6 +142,109 @@ __global__ __launch_bounds__(kLseThreads) void lse_cols_kernel(size_t rows, cons
   }
 }
 
+// Short columns (rows <= 64 * U): one wavefront per column, four columns per block, every load of a column in flight
+// at once.  A 1024-thread block per column of 33 rows (a tagger's label set over a large batch) is 1023 idle threads
+// and a barrier per column: 337 us for 100 000 columns against 8 us here.
+template <int U>
+__global__ __launch_bounds__(256) void lse_cols_wave_kernel(unsigned rows, unsigned bd, const float* __restrict__ x,
+                                                            float* __restrict__ m_out, float* __restrict__ z_out,
+                                                            const unsigned* __restrict__ ids, float* __restrict__ fx) {
+  const unsigned b = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (b >= bd) return;  // whole wavefronts leave; the kernel has no barrier
+  const int lane = threadIdx.x & 63;
+  const float* px = x + size_t(b) * rows;
+  float picked = 0.f;
+  if (ids != nullptr && lane == 0) picked = x[ids[b]];
+  float v[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const unsigned i = lane + 64 * u;
+    v[u] = px[i < rows ? i : rows - 1];  // unconditional loads; a lane past the end does not push its value
+  }
+  MaxSum a;
+  a.m = kLseStartMax;
+  a.s = 0.f;
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+    if (lane + 64 * u < rows) ms_push1(a, v[u]);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    MaxSum o;
+    o.m = __shfl_xor(a.m, off, kWave);
+    o.s = __shfl_xor(a.s, off, kWave);
+    a = ms_merge(a, o);
+  }
+  if (lane == 0) {
+    const bool empty = a.s == 0.f;  // every input was -inf
+    const float z = empty ? NAN : logf(a.s) + a.m;
+    m_out[b] = empty ? -INFINITY : a.m;
+    z_out[b] = z;
+    if (ids != nullptr) fx[b] = z - picked;
+  }
+}
+
+// Columns of at most 64 rows: one thread per column, eight loads in flight, no cross-lane step at all (with a
+// wavefront per column the six merge steps of the butterfly, two exp each, cost more than the column's own terms:
+// 23 us for 100 000 columns of 33 rows, vector-instruction bound).  A wavefront reads 64 neighbouring columns, i.e.
+// one contiguous span, line by line through its L1.
+__global__ __launch_bounds__(256) void lse_cols_thread_kernel(unsigned rows, unsigned bd, const float* __restrict__ x,
+                                                              float* __restrict__ m_out, float* __restrict__ z_out,
+                                                              const unsigned* __restrict__ ids, float* __restrict__ fx) {
+  const unsigned b = blockIdx.x * 256 + threadIdx.x;
+  if (b >= bd) return;
+  const float* px = x + size_t(b) * rows;
+  float picked = 0.f;
+  if (ids != nullptr) picked = x[ids[b]];
+  MaxSum a;
+  a.m = kLseStartMax;
+  a.s = 0.f;
+  unsigned i = 0;
+  for (; i + 8 <= rows; i += 8) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = px[i + u];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) ms_push1(a, v[u]);
+  }
+  for (; i < rows; ++i) ms_push1(a, px[i]);
+  const bool empty = a.s == 0.f;  // every input was -inf
+  const float z = empty ? NAN : logf(a.s) + a.m;
+  m_out[b] = empty ? -INFINITY : a.m;
+  z_out[b] = z;
+  if (ids != nullptr) fx[b] = z - picked;
+}
+
+// The backward pass over short columns, one wavefront per column as above.
+template <int U, bool ACC>
+__global__ __launch_bounds__(256) void pnls_bwd_wave_kernel(unsigned rows, unsigned bd, const float* __restrict__ x,
+                                                            const float* __restrict__ z,
+                                                            const unsigned* __restrict__ ids,
+                                                            const float* __restrict__ dEdf, float* __restrict__ dEdx) {
+  const unsigned b = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (b >= bd) return;
+  const int lane = threadIdx.x & 63;
+  const size_t col0 = size_t(b) * rows;
+  const float zb = z[b], dy = dEdf[b];
+  const unsigned hot = unsigned(size_t(ids[b]) - col0);
+  float xv[U], dv[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const unsigned i = lane + 64 * u, ic = i < rows ? i : rows - 1;
+    xv[u] = x[col0 + ic];
+    dv[u] = ACC ? dEdx[col0 + ic] : 0.f;
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const unsigned i = lane + 64 * u;
+    if (i < rows) {
+      float r = dv[u] + __expf(xv[u] - zb) * dy;
+      if (i == hot) r -= dy;
+      dEdx[col0 + i] = r;
+    }
+  }
+}
+
+constexpr unsigned kLseWaveMaxRows = 512;
 constexpr int kPbThreads = 256;
 constexpr int kPbUnroll = 4;
 
@@ -150,9 +262,24 @@ __global__ __launch_bounds__(kPbThreads) void pnls_bwd_kernel(size_t rows, unsig
   const size_t col0 = size_t(b) * rows;
   const size_t hot = size_t(ids[b]) - col0;  // row of the picked element
   if (VEC) {
-    const size_t n4 = rows >> 2;
-    const float4* x4 = reinterpret_cast<const float4*>(x + col0);
-    float4* d4 = reinterpret_cast<float4*>(dEdx + col0);
+    // x and dEdx start at the same offset from a 16-byte boundary (checked by the host): up to three leading elements,
+    // a body of 128-bit groups, up to three trailing elements; the first tile's first and last threads take the ends
+    const size_t head = min(size_t((4u - unsigned((reinterpret_cast<uintptr_t>(x + col0) >> 2) & 3u)) & 3u), rows);
+    const size_t n4 = (rows - head) >> 2;
+    if (tile == 0) {
+      size_t e = rows;  // none
+      if (threadIdx.x < head) e = threadIdx.x;
+      else if (head + (n4 << 2) + (kPbThreads - 1 - threadIdx.x) < rows) e = head + (n4 << 2) + (kPbThreads - 1 - threadIdx.x);
+      if (e < rows) {
+        float r = (ACC ? dEdx[col0 + e] : 0.f) + __expf(x[col0 + e] - zb) * dy;
+        if (e == hot) r -= dy;
+        dEdx[col0 + e] = r;
+      }
+    }
+    const bool hot_in_body = hot >= head && hot < head + (n4 << 2);
+    const size_t hot_b = hot - head;  // index inside the body (only used when hot_in_body)
+    const float4* x4 = reinterpret_cast<const float4*>(x + col0 + head);
+    float4* d4 = reinterpret_cast<float4*>(dEdx + col0 + head);
     const size_t j0 = size_t(tile) * (kPbThreads * kPbUnroll) + threadIdx.x;
     float4 xv[kPbUnroll], dv[kPbUnroll];
 #pragma unroll
@@ -172,8 +299,8 @@ __global__ __launch_bounds__(kPbThreads) void pnls_bwd_kernel(size_t rows, unsig
         r.y = dv[u].y + __expf(xv[u].y - zb) * dy;
         r.z = dv[u].z + __expf(xv[u].z - zb) * dy;
         r.w = dv[u].w + __expf(xv[u].w - zb) * dy;
-        if ((hot >> 2) == j) {
-          const unsigned c = hot & 3;
+        if (hot_in_body && (hot_b >> 2) == j) {
+          const unsigned c = hot_b & 3;
           if (c == 0) r.x -= dy;
           else if (c == 1) r.y -= dy;
           else if (c == 2) r.z -= dy;
@@ -288,7 +415,20 @@ int batch_reduce(dyhip_device* dev, size_t n, unsigned bd, const float* in0, con
 
 static int launch_lse(dyhip_device* dev, size_t rows, unsigned bd, const float* x, float* m, float* z,
                       const unsigned* ids, float* fx) {
-  const bool vec = rows % 4 == 0 && aligned16(x);
+  if (rows <= kLseWaveMaxRows) {
+    const dim3 grid(cdiv<unsigned>(bd, 4)), block(256);
+    const unsigned r = static_cast<unsigned>(rows);
+#define DYHIP_LSE_WAVE(U) hipLaunchKernelGGL(lse_cols_wave_kernel<U>, grid, block, 0, dev->stream, r, bd, x, m, z, ids, fx)
+    if (r <= 64)
+      hipLaunchKernelGGL(lse_cols_thread_kernel, dim3(cdiv<unsigned>(bd, 256)), block, 0, dev->stream, r, bd, x, m, z, ids, fx);
+    else if (r <= 128) DYHIP_LSE_WAVE(2);
+    else if (r <= 256) DYHIP_LSE_WAVE(4);
+    else DYHIP_LSE_WAVE(8);
+#undef DYHIP_LSE_WAVE
+    DYHIP_CHECK_LAUNCH();
+    return DYHIP_OK;
+  }
+  const bool vec = true;  // any column: its ends are peeled off around a body of 128-bit groups
   const bool stream = rows * size_t(bd) * sizeof(float) >= dev->stream_threshold;
   if (vec && stream)
     hipLaunchKernelGGL((lse_cols_kernel<true, true>), dim3(bd), dim3(kLseThreads), 0, dev->stream, rows, x, m, z, ids, fx);
@@ -450,7 +590,22 @@ static int pnls_backward(dyhip_device* dev, size_t rows, unsigned bd, const floa
   if (bd == 0) return DYHIP_OK;
   const float* z = static_cast<const float*>(aux);
   const unsigned* ids = reinterpret_cast<const unsigned*>(z + 2 * size_t(bd));
-  const bool vec = rows % 4 == 0 && aligned16(x) && aligned16(dEdx);
+  if (rows <= kLseWaveMaxRows) {
+    const dim3 grid(cdiv<unsigned>(bd, 4)), block(256);
+    const unsigned r = static_cast<unsigned>(rows);
+#define DYHIP_PB_WAVE(U) \
+  hipLaunchKernelGGL((pnls_bwd_wave_kernel<U, ACC>), grid, block, 0, dev->stream, r, bd, x, z, ids, dEdf, dEdx)
+    if (r <= 64) DYHIP_PB_WAVE(1);
+    else if (r <= 128) DYHIP_PB_WAVE(2);
+    else if (r <= 256) DYHIP_PB_WAVE(4);
+    else DYHIP_PB_WAVE(8);
+#undef DYHIP_PB_WAVE
+    DYHIP_CHECK_LAUNCH();
+    return DYHIP_OK;
+  }
+  // 128-bit accesses when x and dEdx sit at the same offset from a 16-byte boundary (every column then does too);
+  // a column's ends are peeled off inside the kernel
+  const bool vec = ((reinterpret_cast<uintptr_t>(x) ^ reinterpret_cast<uintptr_t>(dEdx)) & 15u) == 0 && rows >= 8;
   const size_t per_tile = size_t(kPbThreads) * kPbUnroll * (vec ? 4 : 1);
   const size_t tiles = cdiv(rows, per_tile);
   DYHIP_REQUIRE(tiles * bd < (size_t(1) << 31), "PickNegLogSoftmax backward launch too large");

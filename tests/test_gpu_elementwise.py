@@ -27,7 +27,7 @@ def _inputs(n, seed):
 
 
 @pytest.mark.parametrize("op,name", OPS)
-@pytest.mark.parametrize("n", [N_BIG, 1027, 3, 1])
+@pytest.mark.parametrize("n", [N_BIG, 1027, 3, 1, 5, 6, N_BIG + 2])  # 1027, 5, 6, N_BIG + 2: 128-bit groups and a tail of 3, 1, 2, 2
 def test_unary_forward_backward(dev, op, name, n):
     x, dy, dx0 = _inputs(n, 100 + op)
     dx_t = dev.tensor(x)

@@ -999,7 +999,12 @@ def test_lookup_out_of_range_index_is_an_error(dev):
 # ---------------------------------------------------------------------------
 # logsumexp / PickNegLogSoftmax / LogSumExp / argmax
 # ---------------------------------------------------------------------------
-@pytest.mark.parametrize("rows,bd", [(50000, 512), (10000, 128), (37, 5), (1027, 3), (1, 4), (4, 1)])
+@pytest.mark.parametrize("rows,bd", [(50000, 512), (10000, 128), (37, 5), (1027, 3), (1, 4), (4, 1),
+                                     # short columns: a thread per column up to 64 rows, a wavefront per column up to
+                                     # 512 (1, 2, 4 or 8 loads a lane), then a block per column whose ends are peeled
+                                     # off around 128-bit groups whatever the column's offset
+                                     (33, 1000), (64, 300), (65, 7), (128, 9), (200, 70), (256, 5), (511, 6),
+                                     (512, 3), (513, 3), (2050, 2), (50001, 16)])
 def test_pnls_forward_backward(dev, rows, bd):
     rng = np.random.default_rng(rows + bd)
     x = f32(rng.standard_normal((bd, rows)) * 2.0)
@@ -1102,7 +1107,8 @@ def test_pnls_label_out_of_range_is_an_error(dev):
     assert e.value.status == lib.ERR_INVALID_ARG and "Index error in PickNegLogSoftmax" in str(e.value)
 
 
-@pytest.mark.parametrize("rows,cols", [(10000, 128), (37, 5), (1027, 3), (1, 4), (4, 1), (50000, 64)])
+@pytest.mark.parametrize("rows,cols", [(10000, 128), (37, 5), (1027, 3), (1, 4), (4, 1), (50000, 64), (33, 700), (130, 9),
+                                       (300, 40), (513, 3)])
 def test_softmax_and_log_softmax(dev, rows, cols):
     rng = np.random.default_rng(rows + cols)
     x = f32(rng.standard_normal((cols, rows)) * 2)
