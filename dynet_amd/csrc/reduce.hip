@@ -468,6 +468,191 @@ __global__ __launch_bounds__(64 * WPT) void ln_fwd_team_kernel(unsigned n4, cons
   }
 }
 
+// ---- rows of at most 2048 floats that cannot take 128-bit accesses (n % 4 != 0, or a pointer off a 16-byte
+// boundary: every second row then starts off one too): the same one-wavefront-per-row scheme with VS floats per lane,
+// lane l owning elements l, l + 64, ...  A wavefront's access is still one contiguous 256-byte run.  The arithmetic
+// and its order per element are those of the 128-bit kernels; the block-per-row fallback these rows used to take ran
+// at 0.2 of the HBM peak (n = 650: forward 19 us, backward 44 us for 16 MB).
+template <int VS, bool NT>
+__global__ __launch_bounds__(64 * kLnWavesFwd) void ln_fwd_lane_kernel(unsigned n, unsigned bd, const float* __restrict__ x,
+                                                                      const float* __restrict__ g,
+                                                                      const float* __restrict__ b, float* __restrict__ y) {
+  const int lane = threadIdx.x & 63;
+  const unsigned row = blockIdx.x * kLnWavesFwd + (threadIdx.x >> 6);
+  if (row >= bd) return;
+  const float fn = float(n);
+  const float* px = x + size_t(row) * n;
+  float v[VS];
+#pragma unroll
+  for (int u = 0; u < VS; ++u) {
+    const unsigned idx = lane + 64 * u;
+    v[u] = ldg1<NT>(px + (idx < n ? idx : n - 1));  // unconditional; a lane past the end drops what it fetched
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int u = 0; u < VS; ++u)
+    if (lane + 64 * u < n) s += v[u];
+  const float mean = wave_sum(s) / fn;
+  float ss = 0.f;
+#pragma unroll
+  for (int u = 0; u < VS; ++u) {
+    if (lane + 64 * u < n) {
+      const float d = v[u] - mean;
+      ss += d * d;
+    }
+  }
+  const float sigma = sqrtf(wave_sum(ss) / fn);
+  const float sden = 1.0f / (kLnEps + sigma);
+  const float neg = -mean;
+  float* py = y + size_t(row) * n;
+#pragma unroll
+  for (int u = 0; u < VS; ++u) {
+    const unsigned idx = lane + 64 * u;
+    if (idx < n) stg1<NT>(py + idx, g[idx] * ((v[u] + neg) * sden) + b[idx]);
+  }
+}
+
+template <int VS>
+struct LnLaneRow {
+  float v[VS], d[VS], o[VS];
+};
+
+// Up to 16 floats per lane (rows of at most 1024 floats): with 32 the row, the gain, both partial sums and the old dx
+// do not fit the registers, and the spilling kernel (54-63 us for 16 MB) lost to the block-per-row fallback (41 us),
+// which rows of 1025..2048 floats that cannot take 128-bit accesses therefore keep.
+template <int VS, bool NT, bool PREFETCH>
+__global__ __launch_bounds__(64 * kLnWavesBwd) void ln_bwd_lane_kernel(unsigned n, unsigned bd, const float* __restrict__ x,
+                                                                      const float* __restrict__ g,
+                                                                      const float* __restrict__ dEdf, float* __restrict__ dx,
+                                                                      float* __restrict__ part_dg,
+                                                                      float* __restrict__ part_db) {
+  extern __shared__ float lds[];  // [dg | db][wave][n] when partial rows are requested
+  constexpr int WAVES = kLnWavesBwd;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const float fn = float(n);
+  const bool want_g = part_dg != nullptr, want_b = part_db != nullptr;
+  float gg[VS], pdg[VS], pdb[VS];
+#pragma unroll
+  for (int u = 0; u < VS; ++u) {
+    const unsigned idx = lane + 64 * u;
+    gg[u] = idx < n ? g[idx] : 0.f;
+    pdg[u] = 0.f;
+    pdb[u] = 0.f;
+  }
+  const unsigned wave_count = gridDim.x * WAVES;
+  const float* dxr = dx != nullptr ? dx : x;  // without a dx the old values are fetched from x and not used
+  LnLaneRow<VS> cur, nxt;
+  // unconditional loads on addresses clamped into the row; lanes past the end hold zeros
+  auto load = [&](LnLaneRow<VS>& r, unsigned row) __attribute__((always_inline)) {
+    const float *px = x + size_t(row) * n, *pdy = dEdf + size_t(row) * n, *po = dxr + size_t(row) * n;
+#pragma unroll
+    for (int u = 0; u < VS; ++u) {
+      const unsigned idx = lane + 64 * u, ic = idx < n ? idx : n - 1;
+      r.v[u] = ldg1<NT>(px + ic);
+      r.d[u] = ldg1<NT>(pdy + ic);
+      r.o[u] = ldg1<NT>(po + ic);
+    }
+#pragma unroll
+    for (int u = 0; u < VS; ++u) {
+      if (!(lane + 64 * u < n)) {
+        r.v[u] = 0.f;
+        r.d[u] = 0.f;
+      }
+    }
+  };
+  // the block's partial rows: waves added in ascending order through LDS, then stored (every wave runs it once)
+  auto stage = [&]() __attribute__((always_inline)) {
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < VS; ++u) {
+      const unsigned idx = lane + 64 * u;
+      if (idx < n) {
+        if (want_g) lds[size_t(w) * n + idx] = pdg[u];
+        if (want_b) lds[size_t(WAVES + w) * n + idx] = pdb[u];
+      }
+    }
+    __syncthreads();
+    for (unsigned j = threadIdx.x; j < 2 * n; j += 64 * WAVES) {
+      const unsigned which = j >= n ? 1u : 0u;
+      float* part = which == 0 ? part_dg : part_db;
+      if (part == nullptr) continue;
+      const unsigned c = j - which * n;
+      const float* src = lds + size_t(which) * WAVES * n + c;
+      float t = src[0];
+#pragma unroll
+      for (int k = 1; k < WAVES; ++k) t += src[size_t(k) * n];
+      part[size_t(blockIdx.x) * n + c] = t;
+    }
+  };
+  auto process = [&](const LnLaneRow<VS>& cur, unsigned row, bool last) __attribute__((always_inline)) {
+    float s = 0.f;
+#pragma unroll
+    for (int u = 0; u < VS; ++u) s += cur.v[u];
+    const float mean = wave_sum(s) / fn;
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < VS; ++u) {
+      if (lane + 64 * u < n) {
+        const float a = cur.v[u] - mean;
+        ss += a * a;
+      }
+    }
+    const float sigma = sqrtf(wave_sum(ss) / fn);
+    const float rs = 1.0f / (kLnEps + sigma);
+    const float neg = -mean;
+    float sxq = 0.f, sq = 0.f;
+#pragma unroll
+    for (int u = 0; u < VS; ++u) {
+      if (lane + 64 * u < n) {
+        const float xc = cur.v[u] + neg;
+        const float dq = cur.d[u] * gg[u];
+        sxq = fmaf(dq, xc, sxq);
+        sq += dq;
+        if (want_g) pdg[u] = fmaf(cur.d[u], xc * rs, pdg[u]);
+        if (want_b) pdb[u] += cur.d[u];
+      }
+    }
+    if (last && (want_g || want_b)) stage();  // before this row's dx: the LDS pass and the stores run under it
+    if (dx != nullptr) {
+      const float ds = -(wave_sum(sxq) * rs) * rs;
+      const float dmu = -(wave_sum(sq) * rs);
+      const float sb = ds / (2.f * sigma);
+      const float c = 2.f / fn;
+      const float dmu_n = dmu / fn;
+      float* pdx = dx + size_t(row) * n;
+#pragma unroll
+      for (int u = 0; u < VS; ++u) {
+        const unsigned idx = lane + 64 * u;
+        if (idx < n) {
+          float acc = cur.o[u];
+          acc += c * (cur.v[u] - mean) * sb;
+          acc += (cur.d[u] * gg[u]) * rs;
+          acc += dmu_n;
+          stg1<NT>(pdx + idx, acc);
+        }
+      }
+    }
+  };
+  unsigned r = __builtin_amdgcn_readfirstlane(blockIdx.x * WAVES + w);
+  if (r < bd) {
+    load(cur, r);
+    for (unsigned next = r + wave_count; next < bd; next += wave_count) {
+      if (PREFETCH) {
+        load(nxt, next);
+        process(cur, r, false);
+        cur = nxt;
+      } else {
+        process(cur, r, false);
+        load(cur, next);
+      }
+      r = next;
+    }
+    process(cur, r, true);
+  } else if (want_g || want_b) {
+    stage();  // a wave without rows still takes part in the block's barriers
+  }
+}
+
 // generic fallback: one block per batch element, three passes over the row
 __global__ __launch_bounds__(256) void ln_fwd_block_kernel(size_t n, const float* __restrict__ x,
                                                            const float* __restrict__ g,
@@ -1094,6 +1279,23 @@ int dyhip_layer_norm_forward(dyhip_device* dev, size_t n, unsigned bd, const flo
       default: DYHIP_LN_FWD(16); break;
     }
 #undef DYHIP_LN_FWD
+  } else if (n <= 2048) {
+    // rows that cannot take 128-bit accesses: one wavefront per row all the same, one float per lane and step
+    const unsigned nn = static_cast<unsigned>(n);
+    const dim3 grid(cdiv<unsigned>(bd, kLnWavesFwd)), block(64 * kLnWavesFwd);
+    const bool stream = n * size_t(bd) * sizeof(float) >= dev->stream_threshold;
+#define DYHIP_LN_FWD(VS)                                                                                          \
+  do {                                                                                                            \
+    if (stream) hipLaunchKernelGGL((ln_fwd_lane_kernel<VS, true>), grid, block, 0, dev->stream, nn, bd, x, g, b, y); \
+    else hipLaunchKernelGGL((ln_fwd_lane_kernel<VS, false>), grid, block, 0, dev->stream, nn, bd, x, g, b, y);       \
+  } while (0)
+    if (nn <= 64) DYHIP_LN_FWD(1);
+    else if (nn <= 128) DYHIP_LN_FWD(2);
+    else if (nn <= 256) DYHIP_LN_FWD(4);
+    else if (nn <= 512) DYHIP_LN_FWD(8);
+    else if (nn <= 1024) DYHIP_LN_FWD(16);
+    else DYHIP_LN_FWD(32);
+#undef DYHIP_LN_FWD
   } else {
     hipLaunchKernelGGL(ln_fwd_block_kernel, dim3(bd), dim3(256), 0, dev->stream, n, x, g, b, y);
   }
@@ -1111,7 +1313,9 @@ static size_t ln_bwd_ws_generic(size_t n, unsigned bd) {
 static size_t ln_bwd_ws_of_call(size_t n, unsigned bd, const float* x, const float* g, const float* dEdf, const float* dx,
                                 bool cols) {
   if (!cols || bd == 0) return 0;
-  return ln_fast_ok(n, x, g, dEdf, dx) || ln_team_ok(n, x, g, dEdf, dx) ? ln_bwd_ws_fast(n, bd) : ln_bwd_ws_generic(n, bd);
+  // rows of at most 1024 floats always take a one-wavefront-per-row kernel (128-bit, or one float per lane and step)
+  return n <= 1024 || ln_fast_ok(n, x, g, dEdf, dx) || ln_team_ok(n, x, g, dEdf, dx) ? ln_bwd_ws_fast(n, bd)
+                                                                                      : ln_bwd_ws_generic(n, bd);
 }
 
 int dyhip_layer_norm_backward_workspace(size_t n, unsigned bd, size_t* ws_bytes) {
@@ -1235,6 +1439,43 @@ int dyhip_layer_norm_backward(dyhip_device* dev, size_t n, unsigned bd, const fl
     if (dg && db) launch_combine(dev, n, blocks, part_dg, dg, part_db, db, 1, part_nt);
     else if (dg) launch_combine(dev, n, blocks, part_dg, dg, nullptr, nullptr, 1, part_nt);
     else if (db) launch_combine(dev, n, blocks, part_db, db, nullptr, nullptr, 1, part_nt);
+    DYHIP_CHECK_LAUNCH();
+  } else if (n <= 1024) {
+    const unsigned nn = static_cast<unsigned>(n);
+    const unsigned blocks = ln_bwd_blocks(n, bd);
+    float* part_dg = dg ? static_cast<float*>(ws) : nullptr;
+    float* part_db = db ? static_cast<float*>(ws) + size_t(blocks) * n : nullptr;
+    const size_t lds = cols ? size_t(2) * kLnWavesBwd * n * sizeof(float) : 0;  // [dg | db][wave][n], <= 128 KB
+    const dim3 grid(blocks), block(64 * kLnWavesBwd);
+    const bool stream = n * size_t(bd) * sizeof(float) >= dev->stream_threshold;
+    // the row after the current one is fetched ahead
+#define DYHIP_LN_BWD(VS)                                                                                            \
+  do {                                                                                                              \
+    static bool big_lds_ok = false;                                                                                 \
+    if (lds > (size_t(64) << 10) && !big_lds_ok) {                                                                   \
+      DYHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&ln_bwd_lane_kernel<VS, true, true>),  \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 128 << 10));                   \
+      DYHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&ln_bwd_lane_kernel<VS, false, true>), \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 128 << 10));                   \
+      big_lds_ok = true;                                                                                            \
+    }                                                                                                               \
+    if (stream)                                                                                                     \
+      hipLaunchKernelGGL((ln_bwd_lane_kernel<VS, true, true>), grid, block, lds, dev->stream, nn, bd, x, g, dEdf, \
+                         dx, part_dg, part_db);                                                                     \
+    else                                                                                                            \
+      hipLaunchKernelGGL((ln_bwd_lane_kernel<VS, false, true>), grid, block, lds, dev->stream, nn, bd, x, g, dEdf, \
+                         dx, part_dg, part_db);                                                                     \
+  } while (0)
+    if (nn <= 64) DYHIP_LN_BWD(1);
+    else if (nn <= 128) DYHIP_LN_BWD(2);
+    else if (nn <= 256) DYHIP_LN_BWD(4);
+    else if (nn <= 512) DYHIP_LN_BWD(8);
+    else DYHIP_LN_BWD(16);
+#undef DYHIP_LN_BWD
+    DYHIP_CHECK_LAUNCH();
+    if (dg && db) launch_combine(dev, n, blocks, part_dg, dg, part_db, db, 1);
+    else if (dg) launch_combine(dev, n, blocks, part_dg, dg, nullptr, nullptr, 1);
+    else if (db) launch_combine(dev, n, blocks, part_db, db, nullptr, nullptr, 1);
     DYHIP_CHECK_LAUNCH();
   } else {
     float2* stats = cols ? static_cast<float2*>(ws) : nullptr;

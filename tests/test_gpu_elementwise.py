@@ -228,7 +228,11 @@ def _ln_fp64(x, g, b, dy):
 
 @pytest.mark.parametrize("n,bd", [(1024, 4096), (2048, 64), (512, 33), (256, 5), (64, 1), (12, 7), (1027, 9),
                                   (4096, 6), (3, 1), (4096, 1024), (4100, 300), (37, 1000), (70, 2051),
-                                  (8192, 70), (16384, 33), (2052, 19), (12288, 5), (16388, 9)])
+                                  (8192, 70), (16384, 33), (2052, 19), (12288, 5), (16388, 9),
+                                  # rows that are not a multiple of four floats: one float per lane and step up to
+                                  # 1024 (backward) / 2048 (forward) floats, the block-per-row kernels beyond
+                                  (650, 3000), (1001, 20), (250, 100), (50, 9), (65, 130), (1022, 5), (1026, 3),
+                                  (2046, 3), (2050, 2)])
 def test_layer_norm_forward_backward(dev, n, bd):
     rng, x, g, b, dy = _ln_case(n, bd, 51)
     xt, gt, bt, dyt = dev.tensor(x), dev.tensor(g), dev.tensor(b), dev.tensor(dy)
@@ -258,6 +262,31 @@ def test_layer_norm_forward_backward(dev, n, bd):
     dgt2 = dev.tensor(dg0)
     dev.layer_norm_backward(n, bd, xt, gt, dyt, dg=dgt2)
     assert dgt2.numpy().tobytes() == dgt.numpy().tobytes()
+
+
+def test_layer_norm_on_pointers_off_a_16_byte_boundary(dev):
+    """Rows of a multiple of four floats whose tensors start 4 bytes past a 16-byte boundary: no 128-bit accesses, the
+    one-float-per-lane kernels (a lane then owns other elements of a row, so the row sums round differently: the
+    results are held to the oracle's bars, not to the aligned call's bits)."""
+    n, bd = 512, 300
+    rng, x, g, b, dy = _ln_case(n, bd, 77)
+    def off(a):
+        base = dev.empty(a.size + 1)
+        t = base.offset(1, a.shape)
+        t.set(a)
+        return t
+    xo, go, bo, dyo = off(x), off(g), off(b), off(dy)
+    yo = off(np.zeros((bd, n), np.float32))
+    dev.layer_norm_forward(n, bd, xo, go, bo, yo)
+    assert_close(yo.numpy(), orc.layer_norm_forward(n, bd, x, g, b), FWD_RTOL, "layer_norm fwd (offset pointers)", floor=1.0)
+    dx0, dg0, db0 = f32(rng.standard_normal((bd, n))), f32(rng.standard_normal(n)), f32(rng.standard_normal(n))
+    dxo, dgo, dbo = off(dx0), off(dg0), off(db0)
+    dev.layer_norm_backward(n, bd, xo, go, dyo, dxo, dgo, dbo)
+    wx, wg, wb = orc.layer_norm_backward(n, bd, x, g, dy, dx0.copy(), dg0.copy(), db0.copy())
+    assert_close(dxo.numpy(), wx, GRAD_RTOL, "layer_norm dx (offset pointers)", floor=1.0)
+    assert_close(dgo.numpy(), wg, GRAD_RTOL, "layer_norm dg (offset pointers)", floor=np.sqrt(bd))
+    assert_close(dbo.numpy(), wb, GRAD_RTOL, "layer_norm db (offset pointers)", floor=np.sqrt(bd))
+
 
 
 CWISE_SHAPES = [
