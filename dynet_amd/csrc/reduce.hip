@@ -653,24 +653,64 @@ __global__ __launch_bounds__(64 * kLnWavesBwd) void ln_bwd_lane_kernel(unsigned 
   }
 }
 
-// generic fallback: one block per batch element, three passes over the row
-__global__ __launch_bounds__(256) void ln_fwd_block_kernel(size_t n, const float* __restrict__ x,
-                                                           const float* __restrict__ g,
-                                                           const float* __restrict__ b, float* __restrict__ y) {
-  __shared__ float red[4];
+// generic fallback (rows wider than the register-resident kernels take, or wide rows that cannot take 128-bit
+// accesses): one block per batch element, three passes over the row (the second and third find it in the caches), four
+// independent loads in flight per thread and pass.  256 threads for rows of up to 4096 floats (more rows per CU at
+// once), 1024 beyond (65536 floats x 64 rows: 190 -> 35 us forward against 256 threads and one load in flight).
+template <int kLnBlockThreads>
+__global__ __launch_bounds__(kLnBlockThreads) void ln_fwd_block_kernel(size_t n, const float* __restrict__ x,
+                                                                       const float* __restrict__ g,
+                                                                       const float* __restrict__ b,
+                                                                       float* __restrict__ y) {
+  __shared__ float red[kLnBlockThreads / 64];
   const float* px = x + size_t(blockIdx.x) * n;
   float s = 0.f;
-  for (size_t j = threadIdx.x; j < n; j += 256) s += px[j];
-  const float mean = block_sum<4>(s, red) / float(n);
-  float v = 0.f;
-  for (size_t j = threadIdx.x; j < n; j += 256) {
-    const float d = px[j] - mean;
-    v += d * d;
+  for (size_t j0 = threadIdx.x; j0 < n; j0 += 4 * kLnBlockThreads) {
+    float a[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const size_t j = j0 + size_t(u) * kLnBlockThreads;
+      a[u] = px[j < n ? j : n - 1];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (j0 + size_t(u) * kLnBlockThreads < n) s += a[u];
   }
-  const float sigma = sqrtf(block_sum<4>(v, red) / float(n));
+  const float mean = block_sum<kLnBlockThreads / 64>(s, red) / float(n);
+  float v = 0.f;
+  for (size_t j0 = threadIdx.x; j0 < n; j0 += 4 * kLnBlockThreads) {
+    float a[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const size_t j = j0 + size_t(u) * kLnBlockThreads;
+      a[u] = px[j < n ? j : n - 1];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (j0 + size_t(u) * kLnBlockThreads < n) {
+        const float d = a[u] - mean;
+        v += d * d;
+      }
+    }
+  }
+  const float sigma = sqrtf(block_sum<kLnBlockThreads / 64>(v, red) / float(n));
   const float sden = kLnEps + sigma, neg = -mean;
   float* py = y + size_t(blockIdx.x) * n;
-  for (size_t j = threadIdx.x; j < n; j += 256) py[j] = g[j] * ((px[j] + neg) / sden) + b[j];
+  for (size_t j0 = threadIdx.x; j0 < n; j0 += 4 * kLnBlockThreads) {
+    float a[4], gg[4], bb[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const size_t j = j0 + size_t(u) * kLnBlockThreads, jc = j < n ? j : n - 1;
+      a[u] = px[jc];
+      gg[u] = g[jc];
+      bb[u] = b[jc];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const size_t j = j0 + size_t(u) * kLnBlockThreads;
+      if (j < n) py[j] = gg[u] * ((a[u] + neg) / sden) + bb[u];
+    }
+  }
 }
 
 // accumulate helper for float4 with a per-component functor
@@ -1031,42 +1071,94 @@ __global__ __launch_bounds__(1024) void ln_bwd_team_kernel(unsigned n4, unsigned
 
 // generic fallback, pass 1: per-row statistics and the dx update.
 // stats[row] = {mean, sden}
-__global__ __launch_bounds__(256) void ln_bwd_block_kernel(size_t n, const float* __restrict__ x,
-                                                           const float* __restrict__ g,
-                                                           const float* __restrict__ dEdf, float* __restrict__ dx,
-                                                           float2* __restrict__ stats) {
-  __shared__ float red[4];
+template <int kLnBlockThreads>
+__global__ __launch_bounds__(kLnBlockThreads) void ln_bwd_block_kernel(size_t n, const float* __restrict__ x,
+                                                                       const float* __restrict__ g,
+                                                                       const float* __restrict__ dEdf,
+                                                                       float* __restrict__ dx,
+                                                                       float2* __restrict__ stats) {
+  constexpr int T = kLnBlockThreads, W = kLnBlockThreads / 64;
+  __shared__ float red[W];
   const float fn = float(n);
   const float* px = x + size_t(blockIdx.x) * n;
   const float* pdy = dEdf + size_t(blockIdx.x) * n;
   float s = 0.f;
-  for (size_t j = threadIdx.x; j < n; j += 256) s += px[j];
-  const float mean = block_sum<4>(s, red) / fn;
-  float v = 0.f;
-  for (size_t j = threadIdx.x; j < n; j += 256) {
-    const float d = px[j] - mean;
-    v += d * d;
+  for (size_t j0 = threadIdx.x; j0 < n; j0 += 4 * T) {
+    float a[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const size_t j = j0 + size_t(u) * T;
+      a[u] = px[j < n ? j : n - 1];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (j0 + size_t(u) * T < n) s += a[u];
   }
-  const float sigma = sqrtf(block_sum<4>(v, red) / fn);
+  const float mean = block_sum<W>(s, red) / fn;
+  float v = 0.f;
+  for (size_t j0 = threadIdx.x; j0 < n; j0 += 4 * T) {
+    float a[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const size_t j = j0 + size_t(u) * T;
+      a[u] = px[j < n ? j : n - 1];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (j0 + size_t(u) * T < n) {
+        const float d = a[u] - mean;
+        v += d * d;
+      }
+    }
+  }
+  const float sigma = sqrtf(block_sum<W>(v, red) / fn);
   const float sden = kLnEps + sigma, neg = -mean, s2 = sden * sden;
   if (stats != nullptr && threadIdx.x == 0) stats[blockIdx.x] = make_float2(mean, sden);
   if (dx == nullptr) return;
   float ds_p = 0.f, dneg_p = 0.f;
-  for (size_t j = threadIdx.x; j < n; j += 256) {
-    const float dq = pdy[j] * g[j];
-    ds_p -= dq / s2 * (px[j] + neg);
-    dneg_p += dq / sden;
+  for (size_t j0 = threadIdx.x; j0 < n; j0 += 4 * T) {
+    float a[4], d[4], gg[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const size_t j = j0 + size_t(u) * T, jc = j < n ? j : n - 1;
+      a[u] = px[jc];
+      d[u] = pdy[jc];
+      gg[u] = g[jc];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (j0 + size_t(u) * T < n) {
+        const float dq = d[u] * gg[u];
+        ds_p -= dq / s2 * (a[u] + neg);
+        dneg_p += dq / sden;
+      }
+    }
   }
-  const float ds = block_sum<4>(ds_p, red);
-  const float dmu = -block_sum<4>(dneg_p, red);
+  const float ds = block_sum<W>(ds_p, red);
+  const float dmu = -block_sum<W>(dneg_p, red);
   const float sb = ds / (2.f * sigma), c = 2.f / fn, dmu_n = dmu / fn;
   float* pdx = dx + size_t(blockIdx.x) * n;
-  for (size_t j = threadIdx.x; j < n; j += 256) {
-    float acc = pdx[j];
-    acc += c * (px[j] - mean) * sb;
-    acc += (pdy[j] * g[j]) / sden;
-    acc += dmu_n;
-    pdx[j] = acc;
+  for (size_t j0 = threadIdx.x; j0 < n; j0 += 4 * T) {
+    float a[4], d[4], gg[4], o[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const size_t j = j0 + size_t(u) * T, jc = j < n ? j : n - 1;
+      a[u] = px[jc];
+      d[u] = pdy[jc];
+      gg[u] = g[jc];
+      o[u] = pdx[jc];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const size_t j = j0 + size_t(u) * T;
+      if (j < n) {
+        float acc = o[u];
+        acc += c * (a[u] - mean) * sb;
+        acc += (d[u] * gg[u]) / sden;
+        acc += dmu_n;
+        pdx[j] = acc;
+      }
+    }
   }
 }
 
@@ -1297,7 +1389,8 @@ int dyhip_layer_norm_forward(dyhip_device* dev, size_t n, unsigned bd, const flo
     else DYHIP_LN_FWD(32);
 #undef DYHIP_LN_FWD
   } else {
-    hipLaunchKernelGGL(ln_fwd_block_kernel, dim3(bd), dim3(256), 0, dev->stream, n, x, g, b, y);
+    if (n <= 4096) hipLaunchKernelGGL(ln_fwd_block_kernel<256>, dim3(bd), dim3(256), 0, dev->stream, n, x, g, b, y);
+    else hipLaunchKernelGGL(ln_fwd_block_kernel<1024>, dim3(bd), dim3(1024), 0, dev->stream, n, x, g, b, y);
   }
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
@@ -1479,7 +1572,10 @@ int dyhip_layer_norm_backward(dyhip_device* dev, size_t n, unsigned bd, const fl
     DYHIP_CHECK_LAUNCH();
   } else {
     float2* stats = cols ? static_cast<float2*>(ws) : nullptr;
-    hipLaunchKernelGGL(ln_bwd_block_kernel, dim3(bd), dim3(256), 0, dev->stream, n, x, g, dEdf, dx, stats);
+    if (n <= 4096)
+      hipLaunchKernelGGL(ln_bwd_block_kernel<256>, dim3(bd), dim3(256), 0, dev->stream, n, x, g, dEdf, dx, stats);
+    else
+      hipLaunchKernelGGL(ln_bwd_block_kernel<1024>, dim3(bd), dim3(1024), 0, dev->stream, n, x, g, dEdf, dx, stats);
     DYHIP_CHECK_LAUNCH();
     if (cols) {
       const unsigned splits = ln_cols_splits(n, bd), per_split = cdiv<unsigned>(bd, splits);
