@@ -495,6 +495,107 @@ static int launch_col_apply(dyhip_device* dev, size_t rows, unsigned cols, const
   return DYHIP_OK;
 }
 
+// ---- Softmax / LogSoftmax over dim 0 with the column held in registers: ONE kernel, the column read once -----------
+// T threads own a column (a wavefront for columns of up to 512 rows, four columns to a block; a block of 256 threads up
+// to 4096 rows, of 1024 threads up to 16384), thread t holding rows t, t + T, ... (U of them), so that every access of
+// the group is one contiguous run.  The statistics-then-apply pair of kernels below reads the column twice (forward)
+// or three times (backward) and launches twice; it remains for longer columns.  Same formulas as that pair, MODE as
+// in col_apply_kernel; MODE 0 / 1 also leave z (and m) where the pair leaves them.
+template <int T>
+__device__ __forceinline__ float sm_group_sum(float v, float* red) {
+  if (T == 64) return wave_sum(v);
+  return block_sum<(T >= 64 ? T / 64 : 1)>(v, red);
+}
+template <int T>
+__device__ __forceinline__ float sm_group_max(float v, float* red) {
+  if (T == 64) return wave_max(v);
+  return block_max<(T >= 64 ? T / 64 : 1)>(v, red);
+}
+
+template <int MODE, int T, int U>
+__global__ __launch_bounds__(T == 64 ? 256 : T) void softmax_resident_kernel(unsigned rows, unsigned cols,
+                                                                            const float* __restrict__ a,
+                                                                            const float* __restrict__ b,
+                                                                            float* __restrict__ s0, float* __restrict__ s1,
+                                                                            float* __restrict__ out) {
+  __shared__ float red[16];
+  const unsigned c = T == 64 ? blockIdx.x * 4 + (threadIdx.x >> 6) : blockIdx.x;
+  if (c >= cols) return;  // T == 64: whole wavefronts leave and that form has no barrier; else c == blockIdx.x < cols
+  const unsigned t = T == 64 ? (threadIdx.x & 63) : threadIdx.x;
+  const size_t c0 = size_t(c) * rows;
+  float av[U], bv[U], ov[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const unsigned i = t + T * u, ic = i < rows ? i : rows - 1;  // unconditional loads; rows past the end are masked
+    av[u] = a[c0 + ic];
+    if (MODE >= 2) {
+      bv[u] = b[c0 + ic];
+      ov[u] = out[c0 + ic];
+    }
+  }
+  if (MODE == 0 || MODE == 1) {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (t + T * u < rows) mx = av[u] > mx ? av[u] : mx;
+    const float m = sm_group_max<T>(mx, red);
+    float e[U], sum = 0.f;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      e[u] = expf(av[u] - m);
+      if (t + T * u < rows) sum += e[u];
+    }
+    const float z = logf(sm_group_sum<T>(sum, red)) + m;
+    if (t == 0) {
+      s0[c] = z;
+      if (s1 != nullptr) s1[c] = m;
+    }
+    const float p1 = expf(m - z);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const unsigned i = t + T * u;
+      if (i < rows) out[c0 + i] = MODE == 0 ? e[u] * p1 : av[u] - z;
+    }
+  } else {
+    float part = 0.f;
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (t + T * u < rows) part += MODE == 2 ? av[u] * bv[u] : bv[u];
+    const float r = sm_group_sum<T>(part, red);
+    if (t == 0 && s0 != nullptr) s0[c] = r;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const unsigned i = t + T * u;
+      if (i < rows) out[c0 + i] = MODE == 2 ? ov[u] + (bv[u] - r) * av[u] : ov[u] + ((expf(av[u]) * -r) + bv[u]);
+    }
+  }
+}
+
+constexpr size_t kSmResidentMaxRows = 16384;
+
+// true: the column-resident kernel was launched
+template <int MODE>
+static bool launch_softmax_resident(dyhip_device* dev, size_t rows, unsigned cols, const float* a, const float* b,
+                                    float* s0, float* s1, float* out) {
+  if (rows > kSmResidentMaxRows) return false;
+  const unsigned r = static_cast<unsigned>(rows);
+#define DYHIP_SM(T, U, GRID)                                                                                           \
+  hipLaunchKernelGGL((softmax_resident_kernel<MODE, T, U>), dim3(GRID), dim3(T == 64 ? 256 : T), 0, dev->stream, r, cols, \
+                     a, b, s0, s1, out)
+  const unsigned g4 = cdiv<unsigned>(cols, 4);
+  if (r <= 64) DYHIP_SM(64, 1, g4);
+  else if (r <= 128) DYHIP_SM(64, 2, g4);
+  else if (r <= 256) DYHIP_SM(64, 4, g4);
+  else if (r <= 512) DYHIP_SM(64, 8, g4);
+  else if (r <= 1024) DYHIP_SM(256, 4, cols);
+  else if (r <= 2048) DYHIP_SM(256, 8, cols);
+  else if (r <= 4096) DYHIP_SM(256, 16, cols);
+  else if (r <= 8192) DYHIP_SM(1024, 8, cols);
+  else DYHIP_SM(1024, 16, cols);
+#undef DYHIP_SM
+  return true;
+}
+
 // ---- reductions along dim 1 (Softmax with dimension 1, LogSumExpDimension) --------------------------------
 // x is rows x cols column-major per batch element.  A block is 64 lanes (consecutive rows: coalesced) x
 // kRowWaves waves (wave w takes columns w, w + kRowWaves, ...); the per-row maximum, then the per-row sum of
@@ -754,6 +855,10 @@ int dyhip_softmax_forward(dyhip_device* dev, size_t rows, unsigned cols, const f
                 2 * sizeof(float) * cols, ws_bytes);
   float* z = static_cast<float*>(ws);
   float* m = z + cols;
+  if (launch_softmax_resident<0>(dev, rows, cols, x, nullptr, z, m, fx)) {
+    DYHIP_CHECK_LAUNCH();
+    return DYHIP_OK;
+  }
   DYHIP_CHECK_STATUS(launch_lse(dev, rows, cols, x, m, z, nullptr, nullptr));
   return launch_col_apply<0>(dev, rows, cols, x, nullptr, m, z, fx);
 }
@@ -766,6 +871,10 @@ int dyhip_softmax_backward(dyhip_device* dev, size_t rows, unsigned cols, const 
   DYHIP_REQUIRE(ws != nullptr && ws_bytes >= sizeof(float) * cols, "Softmax backward needs %zu workspace bytes, got %zu",
                 sizeof(float) * cols, ws_bytes);
   float* r = static_cast<float*>(ws);
+  if (launch_softmax_resident<2>(dev, rows, cols, fx, dEdf, r, nullptr, dEdx)) {
+    DYHIP_CHECK_LAUNCH();
+    return DYHIP_OK;
+  }
   hipLaunchKernelGGL(col_dot_kernel, dim3(cols), dim3(kSmThreads), 0, dev->stream, rows, fx, dEdf, r);
   DYHIP_CHECK_LAUNCH();
   return launch_col_apply<2>(dev, rows, cols, fx, dEdf, r, nullptr, dEdx);
@@ -820,6 +929,10 @@ int dyhip_log_softmax_forward(dyhip_device* dev, size_t rows, unsigned cols, con
   if (cols == 0) return DYHIP_OK;
   float* z = static_cast<float*>(aux);
   float* m = z + cols;
+  if (launch_softmax_resident<1>(dev, rows, cols, x, nullptr, z, m, fx)) {
+    DYHIP_CHECK_LAUNCH();
+    return DYHIP_OK;
+  }
   DYHIP_CHECK_STATUS(launch_lse(dev, rows, cols, x, m, z, nullptr, nullptr));
   return launch_col_apply<1>(dev, rows, cols, x, nullptr, z, nullptr, fx);
 }
@@ -830,6 +943,10 @@ int dyhip_log_softmax_backward(dyhip_device* dev, size_t rows, unsigned cols, co
   DYHIP_REQUIRE(rows >= 1 && fx && dEdf && aux && dEdx, "LogSoftmax needs non-empty tensors");
   if (cols == 0) return DYHIP_OK;
   float* r = static_cast<float*>(aux);  // the reference overwrites z in aux_mem with the column sums of dEdf
+  if (launch_softmax_resident<3>(dev, rows, cols, fx, dEdf, r, nullptr, dEdx)) {
+    DYHIP_CHECK_LAUNCH();
+    return DYHIP_OK;
+  }
   hipLaunchKernelGGL(col_dot_kernel, dim3(cols), dim3(kSmThreads), 0, dev->stream, rows, dEdf, nullptr, r);
   DYHIP_CHECK_LAUNCH();
   return launch_col_apply<3>(dev, rows, cols, fx, dEdf, r, nullptr, dEdx);
