@@ -166,7 +166,8 @@ def test_sum_batches_golden_cadd_broadcast2_neg_val(dev, golden):
     assert abs(float(z.numpy().astype(np.float64).sum()) - exp["expected"]) <= exp["rel_tol"] * abs(exp["expected"])
 
 
-@pytest.mark.parametrize("n,bd", [(1024, 4096), (9, 3), (1000, 17), (1, 4)])
+@pytest.mark.parametrize("n,bd", [(1024, 4096), (9, 3), (1000, 17), (1, 4), (50, 3000), (100, 7), (200, 9), (400, 5), (1500, 3),
+                                  (3000, 3), (5000, 2), (10000, 2), (16384, 2), (16385, 2), (70000, 2)])
 def test_mean_std_elems(dev, n, bd):
     rng = np.random.default_rng(41)
     x = f32(rng.standard_normal((bd, n)) + 0.5)
