@@ -105,8 +105,9 @@ __global__ __launch_bounds__(256) void cwise_bcast_kernel(CwShape sh, const floa
 // x - mean and x / sigma of the layer_norm composite): no index arithmetic beyond the block's own coordinates, kRows
 // rows of the outer axis per block with all their loads issued first, streaming accesses for large tensors.
 struct CwShape2 {
-  unsigned d0g, d1;   // groups of W elements along the inner axis; extent of the outer axis
-  size_t s0[3], s1[3];  // element strides of the three operands along the two axes (0 = broadcast)
+  unsigned d0g, d1, d2;  // groups of W elements along the inner axis; extents of the middle and the outer axis
+  unsigned tx_shift;     // a block is 2^tx_shift threads along the inner axis x 256 / 2^tx_shift rows of the middle one
+  size_t s0[3], s1[3], s2[3];  // element strides of the three operands along the three axes (0 = broadcast)
 };
 constexpr int kCwRows = 4;
 
@@ -116,13 +117,20 @@ __global__ __launch_bounds__(256) void cwise_bcast2_kernel(CwShape2 sh, const fl
                                                            float* __restrict__ out) {
   constexpr int NIN = cw_inputs(FN);
   constexpr bool ACC = FN >= 3;
-  const unsigned gx = blockIdx.x * 256 + threadIdx.x;
+  constexpr int kRows = kCwRows;  // rows in flight per thread (sixteen for the one-float form measured slower than four)
+  // a short inner axis does not idle most of the block: the block's threads fold over rows of the middle axis
+  const unsigned tx = threadIdx.x & ((1u << sh.tx_shift) - 1u), ty = threadIdx.x >> sh.tx_shift;
+  const unsigned rows_per_block = (256u >> sh.tx_shift) * kRows;
+  const unsigned gx = (blockIdx.x << sh.tx_shift) + tx;
   if (gx >= sh.d0g) return;
-  const float* ps[3] = {p0, p1, p2};
-  for (unsigned y0 = blockIdx.y * kCwRows; y0 < sh.d1; y0 += gridDim.y * kCwRows) {
-    float v[kCwRows][3][W], o[kCwRows][W];
+  for (unsigned z = blockIdx.z; z < sh.d2; z += gridDim.z) {
+  const float* ps[3] = {p0 + size_t(z) * sh.s2[0], p1 + (NIN > 1 ? size_t(z) * sh.s2[1] : 0),
+                        p2 + (NIN > 2 ? size_t(z) * sh.s2[2] : 0)};
+  float* const outz = out + size_t(z) * sh.d1 * sh.d0g * W;
+  for (unsigned y0 = blockIdx.y * rows_per_block + ty * kRows; y0 < sh.d1; y0 += gridDim.y * rows_per_block) {
+    float v[kRows][3][W], o[kRows][W];
 #pragma unroll
-    for (int r = 0; r < kCwRows; ++r) {
+    for (int r = 0; r < kRows; ++r) {
       const unsigned y = min(y0 + r, sh.d1 - 1);  // rows past the end repeat the last one and are not stored
 #pragma unroll
       for (int k = 0; k < 3; ++k) {
@@ -140,7 +148,7 @@ __global__ __launch_bounds__(256) void cwise_bcast2_kernel(CwShape2 sh, const fl
           for (int e = 0; e < W; ++e) v[r][k][e] = 0.f;
         }
       }
-      const float* po = out + (size_t(y) * sh.d0g + gx) * W;
+      const float* po = outz + (size_t(y) * sh.d0g + gx) * W;
       if (ACC && W == 4) {
         const float4 t = *reinterpret_cast<const float4*>(po);  // read-modify-write: a plain load
         o[r][0] = t.x; o[r][1 % W] = t.y; o[r][2 % W] = t.z; o[r][3 % W] = t.w;
@@ -150,14 +158,15 @@ __global__ __launch_bounds__(256) void cwise_bcast2_kernel(CwShape2 sh, const fl
       }
     }
 #pragma unroll
-    for (int r = 0; r < kCwRows; ++r) {
+    for (int r = 0; r < kRows; ++r) {
       if (y0 + r >= sh.d1) break;
-      float* po = out + (size_t(y0 + r) * sh.d0g + gx) * W;
+      float* po = outz + (size_t(y0 + r) * sh.d0g + gx) * W;
 #pragma unroll
       for (int e = 0; e < W; ++e) o[r][e] = cw_apply<FN>(v[r][0][e], v[r][1][e], v[r][2][e], o[r][e]);
       if (W == 4) stg4<NT>(reinterpret_cast<float4*>(po), make_float4(o[r][0], o[r][1 % W], o[r][2 % W], o[r][3 % W]));
       else po[0] = o[r][0];
     }
+  }
   }
 }
 
@@ -339,6 +348,65 @@ static unsigned cw_grid(size_t work_items, unsigned per_block, const dyhip_devic
   return static_cast<unsigned>(want < cap ? (want ? want : 1) : cap);
 }
 
+// The reduced axes collapse to one that is NOT the contiguous one (the gradient of a column vector added to every
+// column of a matrix: kept rows, reduced columns, kept batch): lanes run along the contiguous kept axis, so every load
+// of a wavefront is one contiguous run, the block's 8 wavefronts split the reduced axis (four terms in flight each) and
+// meet in LDS in ascending order.  With a wavefront per output walking the reduced axis each lane touched a line of
+// its own (46.7 us for 256 x 64 x 256 summed over the 64; 8 us here).
+constexpr int kCwMidWaves = 8;
+template <int FN>
+__global__ __launch_bounds__(64 * kCwMidWaves) void cwise_reduce_mid_kernel(CwReduce c, const float* __restrict__ p0,
+                                                                           const float* __restrict__ p1,
+                                                                           const float* __restrict__ p2,
+                                                                           float* __restrict__ out) {
+  constexpr int NIN = cw_inputs(FN);
+  __shared__ float red[kCwMidWaves][64];
+  const unsigned lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const unsigned i = blockIdx.x * 64 + lane;  // along the contiguous kept axis
+  const bool live = i < c.kd[0];
+  const unsigned ic = live ? i : c.kd[0] - 1;
+  const float* ps[3] = {p0, p1, p2};
+  const size_t n_rest = c.n_out / c.kd[0];  // the other kept axes, flattened
+  const unsigned nr = unsigned(c.n_red);
+  for (size_t z = blockIdx.y; z < n_rest; z += gridDim.y) {
+    size_t base[3] = {0, 0, 0};
+    size_t r = z;  // the same in every thread of the block
+#pragma unroll
+    for (int j = 1; j < 5; ++j) {
+      const unsigned kd = c.kd[j];
+      if (kd == 1) continue;
+      const size_t q = r / kd, e = r - q * kd;
+      r = q;
+#pragma unroll
+      for (int k = 0; k < NIN; ++k) base[k] += e * c.ks[k][j];
+    }
+#pragma unroll
+    for (int k = 0; k < NIN; ++k) base[k] += size_t(ic) * c.ks[k][0];
+    float acc = 0.f;
+    for (unsigned q0 = w; q0 < nr; q0 += 4 * kCwMidWaves) {
+      float v[4][3];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const unsigned q = min(q0 + u * kCwMidWaves, nr - 1);  // clamped, masked below
+#pragma unroll
+        for (int k = 0; k < 3; ++k) v[u][k] = k < NIN ? ps[k][base[k] + size_t(q) * c.rs[k][0]] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (q0 + u * kCwMidWaves < nr) acc += cw_term<FN>(v[u][0], v[u][1], v[u][2]);
+    }
+    __syncthreads();  // the previous round's sums have been read
+    red[w][lane] = acc;
+    __syncthreads();
+    if (w == 0 && live) {
+      float t = red[0][lane];
+#pragma unroll
+      for (int k = 1; k < kCwMidWaves; ++k) t += red[k][lane];
+      out[z * c.kd[0] + i] += t;
+    }
+  }
+}
+
 // Axes of extent 1 dropped, neighbouring axes merged when every operand treats them alike (broadcast over both, or
 // laid out contiguously across both).  Returns the number of axes left; d / s are padded with 1 / 0.
 static int cw_collapse(const unsigned* d_in, const size_t s_in[3][5], int nin, unsigned* d, size_t s[3][5]) {
@@ -380,16 +448,20 @@ static int cw_launch_bcast(dyhip_device* dev, const CwShape& sh_in, const float*
       for (int j = 1; j < 5; ++j) vec = vec && sh.s[k][j] % 4 == 0;
     }
   }
-  if (rank <= 2) {  // the two-axis kernel: no index arithmetic, several rows in flight per block
+  if (rank <= 3) {  // up to three axes: no index arithmetic, several rows in flight per block
     CwShape2 s2;
     s2.d0g = sh.d[0] / (vec ? 4 : 1);
     s2.d1 = sh.d[1];
+    s2.d2 = sh.d[2];
     for (int k = 0; k < 3; ++k) {
       s2.s0[k] = sh.s[k][0];
       s2.s1[k] = sh.s[k][1];
+      s2.s2[k] = sh.s[k][2];
     }
-    const unsigned gy = cdiv<unsigned>(s2.d1, kCwRows);
-    const dim3 grid(cdiv<unsigned>(s2.d0g, 256), gy < 65535u ? gy : 65535u), block(256);
+    s2.tx_shift = 8;
+    while (s2.tx_shift > 4 && (128u >> (8 - s2.tx_shift)) >= s2.d0g) --s2.tx_shift;  // 16..256 threads along the inner axis
+    const unsigned tx = 1u << s2.tx_shift, gy = cdiv<unsigned>(s2.d1, (256u / tx) * kCwRows);
+    const dim3 grid(cdiv<unsigned>(s2.d0g, tx), gy < 65535u ? gy : 65535u, s2.d2 < 65535u ? s2.d2 : 65535u), block(256);
     const bool nt = total * sizeof(float) >= dev->stream_threshold;
     if (vec && nt) hipLaunchKernelGGL((cwise_bcast2_kernel<FN, 4, true>), grid, block, 0, dev->stream, s2, p0, p1, p2, out);
     else if (vec) hipLaunchKernelGGL((cwise_bcast2_kernel<FN, 4, false>), grid, block, 0, dev->stream, s2, p0, p1, p2, out);
@@ -448,6 +520,18 @@ static int cw_launch_reduce(dyhip_device* dev, const unsigned* full, const unsig
       for (int j = 0; j < 5; ++j) {
         c.rd[j] = rd2[j];
         for (int k = 0; k < 3; ++k) c.rs[k][j] = rs2[k][j];
+      }
+      // the first kept axis is the contiguous one (and not a short one) and the reduced axis is not: lanes along it
+      bool mid = c.kd[0] >= 16;
+      for (int k = 0; k < cw_inputs(FN); ++k) mid = mid && (c.ks[k][0] == 1 || c.ks[k][0] == 0) && c.rs[k][0] != 1;
+      // ... and there are enough (kept row tile, other kept index) pairs to fill the GPU: a block owns one
+      mid = mid && cdiv<size_t>(c.kd[0], 64) * (c.n_out / c.kd[0]) >= 128;
+      if (mid) {
+        const size_t n_rest = c.n_out / c.kd[0];
+        const dim3 grid(cdiv<unsigned>(c.kd[0], 64), unsigned(n_rest < 65535 ? n_rest : 65535)), block(64 * kCwMidWaves);
+        hipLaunchKernelGGL(cwise_reduce_mid_kernel<FN>, grid, block, 0, dev->stream, c, p0, p1, p2, out);
+        DYHIP_CHECK_LAUNCH();
+        return DYHIP_OK;
       }
       const dim3 grid(cw_grid(c.n_out, 4, dev)), block(256);
       // operands far larger than the caches are read once: streaming loads

@@ -303,6 +303,14 @@ CWISE_SHAPES = [
     ((7, 1, 1, 1, 3), (7, 1, 1, 1, 3)),           # nothing broadcast
     ((6, 2, 1, 1, 5), (6, 2, 1, 1, 1)),           # batch only: the streaming kernels
     ((1023, 3, 1, 1, 2), (1, 3, 1, 1, 1)),        # d0 not a multiple of 4
+    # three axes left after merging: a column vector per batch element against a matrix (broadcast over the middle
+    # axis; its gradient sums over that axis with lanes along the rows), short inner axes (a block folds over rows)
+    ((256, 64, 1, 1, 40), (256, 1, 1, 1, 40)),
+    ((64, 70, 1, 1, 150), (64, 1, 1, 1, 150)),
+    ((20, 7, 1, 1, 300), (20, 1, 1, 1, 300)),
+    ((12, 5, 3, 1, 4), (12, 1, 3, 1, 4)),
+    ((130, 9, 1, 1, 70000), (130, 1, 1, 1, 70000)),  # more than 65535 entries along the outer axis
+    ((8, 3, 1, 1, 5), (8, 3, 1, 1, 1)),
 ]
 
 
