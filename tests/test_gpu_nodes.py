@@ -79,6 +79,29 @@ def test_gemm_nt_shallow(dev, M, N, K):
                  floor=np.sqrt(K))
 
 
+# l * r^T with a depth of at most 32 (the weight gradient of one timestep at a small batch) is a rank-K update of a matrix
+# read and written once: depths on both sides of every multiple of four, column counts that do not fill the last group
+# of eight, the baseline's smallest cell (1024 x 128 x 32), accumulate and overwrite.
+@pytest.mark.parametrize("M,N,K", [(1024, 128, 32), (4096, 1024, 20), (2052, 1030, 7), (256, 5, 1), (6000, 1500, 13),
+                                   (1024, 256, 4), (1024, 255, 29), (512, 9, 16)])
+def test_gemm_nt_thin(dev, M, N, K):
+    rng = np.random.default_rng(M + N + K)
+    y0 = f32(rng.standard_normal((N, M)))
+    l, r2 = f32(rng.standard_normal((K, M))), f32(rng.standard_normal((K, N)))
+    lt, rt = dev.tensor(l), dev.tensor(r2)
+    ref64 = r2.astype(np.float64).T @ l.astype(np.float64)
+    yt = dev.tensor(y0)
+    dev.gemm_nt_acc(M, N, K, lt, rt, yt)
+    assert_close(yt.numpy(), (y0 + ref64).astype(np.float32), FWD_RTOL, "thin gemm_nt_acc", floor=np.sqrt(K))
+    first = yt.numpy().copy()
+    yt = dev.tensor(y0)
+    dev.gemm_nt_acc(M, N, K, lt, rt, yt)
+    assert yt.numpy().tobytes() == first.tobytes()  # a fixed order of additions
+    yt = dev.tensor(y0)
+    dev.gemm_nt(M, N, K, lt, rt, 0.0, yt)
+    assert_close(yt.numpy(), ref64.astype(np.float32), FWD_RTOL, "thin gemm_nt beta=0", floor=np.sqrt(K))
+
+
 # Large outputs go to the 256 x 256-tile kernel, which deals the k-tiles of all tiles to the CUs in equal segments:
 # (a) fewer tiles than CUs: every tile spans several segments, whose partial tiles a second kernel adds; ragged edges
 # and a depth that is not a multiple of 32 (the rest of the depth is added by the 128-wide kernel); (b), (c) a little
