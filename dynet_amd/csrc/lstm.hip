@@ -842,17 +842,115 @@ static int skinny_tn(dyhip_device* dev, unsigned M, unsigned N, unsigned K, cons
   return DYHIP_OK;
 }
 
+// ---- C[M x N] = beta * C + A^T B for at most 32 columns of B (dx and dh of the gates node at a small batch) --------
+// A (K x M, a weight matrix) is read once from memory and is the whole cost; B (K x N) is small and stays in the L2.
+// A block owns four columns of A and all columns of B: its 256 threads split the depth in 128-bit groups, every thread
+// multiplies its group of each of the four A columns with its group of every B column, and the 4 x N partial sums
+// cross the block once at the end (wavefront sums, then LDS in ascending wavefront order).  No matrix cores: at 20
+// columns the product is 80 multiply-adds per 16 bytes of A, and a 32-column matrix-core tile would read A in
+// 128-byte pieces (the fragment-order kernel above takes 13.6 us for 16.8 MB of A at N = 20).
+constexpr int kThinTnCols = 4;
+template <int NP>  // N rounded up to a multiple of four
+__global__ __launch_bounds__(256) void gemm_tn_thin_kernel(unsigned M, unsigned N, unsigned K4, const float* __restrict__ A,
+                                                           size_t lda, const float* __restrict__ B, size_t ldb, float beta,
+                                                           float* __restrict__ C) {
+  __shared__ float red[4][kThinTnCols][NP];
+  const unsigned i0 = blockIdx.x * kThinTnCols;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  float acc[kThinTnCols][NP];
+#pragma unroll
+  for (int c = 0; c < kThinTnCols; ++c)
+#pragma unroll
+    for (int n = 0; n < NP; ++n) acc[c][n] = 0.f;
+  const float4* a4[kThinTnCols];
+#pragma unroll
+  for (int c = 0; c < kThinTnCols; ++c)
+    a4[c] = reinterpret_cast<const float4*>(A + size_t(min(i0 + c, M - 1)) * lda);  // columns past the end: not stored
+  for (unsigned k4 = threadIdx.x; k4 < K4; k4 += 256) {
+    float4 a[kThinTnCols], b[NP];
+#pragma unroll
+    for (int c = 0; c < kThinTnCols; ++c) a[c] = ldg4<true>(a4[c] + k4);  // read once: streaming
+#pragma unroll
+    for (int n = 0; n < NP; ++n)
+      b[n] = reinterpret_cast<const float4*>(B + size_t(min(unsigned(n), N - 1)) * ldb)[k4];
+#pragma unroll
+    for (int c = 0; c < kThinTnCols; ++c)
+#pragma unroll
+      for (int n = 0; n < NP; ++n) {
+        float t = acc[c][n];
+        t = fmaf(a[c].x, b[n].x, t);
+        t = fmaf(a[c].y, b[n].y, t);
+        t = fmaf(a[c].z, b[n].z, t);
+        t = fmaf(a[c].w, b[n].w, t);
+        acc[c][n] = t;
+      }
+  }
+#pragma unroll
+  for (int c = 0; c < kThinTnCols; ++c)
+#pragma unroll
+    for (int n = 0; n < NP; ++n) {
+      const float t = wave_sum(acc[c][n]);
+      if (lane == 0) red[w][c][n] = t;
+    }
+  __syncthreads();
+  if (threadIdx.x < kThinTnCols * NP) {
+    const unsigned c = threadIdx.x / NP, n = threadIdx.x % NP;
+    if (i0 + c < M && n < N) {
+      const float t = ((red[0][c][n] + red[1][c][n]) + red[2][c][n]) + red[3][c][n];
+      float* out = C + size_t(n) * M + i0 + c;
+      *out = beta != 0.f ? beta * *out + t : t;
+    }
+  }
+}
+
+static bool thin_tn_eligible(size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B, size_t ldb) {
+  return N >= 1 && N <= 32 && M >= 1 && M <= (size_t(1) << 30) && K >= 256 && K % 4 == 0 && K / 4 <= 0xFFFFFFFFull &&
+         lda % 4 == 0 && ldb % 4 == 0 && aligned16(A) && aligned16(B);
+}
+
+static int thin_tn_run(dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B,
+                       size_t ldb, float beta, float* C) {
+  const dim3 grid(static_cast<unsigned>(cdiv<size_t>(M, kThinTnCols))), block(256);
+#define DYHIP_THIN_TN(NP)                                                                                       \
+  hipLaunchKernelGGL(gemm_tn_thin_kernel<NP>, grid, block, 0, dev->stream, static_cast<unsigned>(M),           \
+                     static_cast<unsigned>(N), static_cast<unsigned>(K / 4), A, lda, B, ldb, beta, C)
+  switch ((N + 3) / 4) {
+    case 1: DYHIP_THIN_TN(4); break;
+    case 2: DYHIP_THIN_TN(8); break;
+    case 3: DYHIP_THIN_TN(12); break;
+    case 4: DYHIP_THIN_TN(16); break;
+    case 5: DYHIP_THIN_TN(20); break;
+    case 6: DYHIP_THIN_TN(24); break;
+    case 7: DYHIP_THIN_TN(28); break;
+    default: DYHIP_THIN_TN(32); break;
+  }
+#undef DYHIP_THIN_TN
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
 // C[M x N] = beta * C + A^T B for a small output with a deep sum, A (K x M) and B (K x N) plain with k contiguous:
 // the fragment-order product leaves a few slices in the queue's GEMM workspace and a second launch folds them into
 // C.  *taken = false (nothing launched) when the shape is not one this form is faster on.
 int skinny_tn_gemm(dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B,
                    size_t ldb, float beta, float* C, bool* taken) {
   *taken = false;
-  if (M == 0 || N == 0 || M > 4096 || N > 256 || K < 1024 || K > (size_t(1) << 24)) return DYHIP_OK;
-  if (M * N > (size_t(1) << 19) || lda % 4 != 0 || ldb % 4 != 0 || !aligned16(A) || !aligned16(B)) return DYHIP_OK;
-  const unsigned m = unsigned(M), n = unsigned(N), k = unsigned(K);
-  if (skinny_tn_splits(m, n, k) == 0 || dev->gemm_ws == nullptr || dev->gemm_ws_bytes < sizeof(float) * M * N * 16)
+  // At most 32 columns of B: the streaming kernel takes what the fragment-order product below does not (a depth or a
+  // row count off its grid: 650 x 20 x 2600 12.5 against 17.7 us on the general GEMM) and, up to four columns, all of
+  // it (1024 x 1 x 4096: 7.1 against 11.4 us); where both apply at 16-32 columns the fragment-order product is faster
+  // (1024 x 20 x 4096: 13.6 against 14.9 us - the 4 x N partial sums cross the block through 4 N wavefront sums).
+  const bool thin_ok = C != nullptr && thin_tn_eligible(M, N, K, A, lda, B, ldb);
+  bool frag_ok = !(M == 0 || N == 0 || M > 4096 || N > 256 || K < 1024 || K > (size_t(1) << 24)) &&
+                 !(M * N > (size_t(1) << 19) || lda % 4 != 0 || ldb % 4 != 0 || !aligned16(A) || !aligned16(B));
+  frag_ok = frag_ok && skinny_tn_splits(unsigned(M), unsigned(N), unsigned(K)) != 0 && dev->gemm_ws != nullptr &&
+            dev->gemm_ws_bytes >= sizeof(float) * M * N * 16;
+  if (thin_ok && (N <= 4 || !frag_ok)) {
+    DYHIP_CHECK_STATUS(thin_tn_run(dev, M, N, K, A, lda, B, ldb, beta, C));
+    *taken = true;
     return DYHIP_OK;
+  }
+  if (!frag_ok) return DYHIP_OK;
+  const unsigned m = unsigned(M), n = unsigned(N), k = unsigned(K);
   unsigned splits = 0;
   DYHIP_CHECK_STATUS(skinny_tn(dev, m, n, k, A, lda, true, B, ldb, true, static_cast<float*>(dev->gemm_ws),
                                dev->gemm_ws_bytes, &splits));

@@ -102,6 +102,27 @@ def test_gemm_nt_thin(dev, M, N, K):
     assert_close(yt.numpy(), ref64.astype(np.float32), FWD_RTOL, "thin gemm_nt beta=0", floor=np.sqrt(K))
 
 
+# l^T * r with at most 32 columns of r (dx and dh of the gates node at a small batch): the left operand streamed once,
+# four of its columns a block; column counts on both sides of every multiple of four, row counts that do not fill the
+# last block, any beta.
+@pytest.mark.parametrize("M,N,K", [(1024, 20, 4096), (128, 32, 1024), (650, 20, 2600), (1000, 1, 4000), (37, 7, 256),
+                                   (1024, 13, 6000), (258, 4, 1024), (255, 29, 2048)])
+def test_gemm_tn_thin(dev, M, N, K):
+    rng = np.random.default_rng(M + N + K)
+    y0 = f32(rng.standard_normal((N, M)))
+    l, r2 = f32(rng.standard_normal((M, K))), f32(rng.standard_normal((N, K)))
+    lt, rt = dev.tensor(l), dev.tensor(r2)
+    ref64 = r2.astype(np.float64) @ l.astype(np.float64).T
+    for beta in (1.0, 0.0, 0.5):
+        yt = dev.tensor(y0)
+        dev.gemm_tn(M, N, K, lt, rt, beta, yt)
+        assert_close(yt.numpy(), (beta * y0 + ref64).astype(np.float32), FWD_RTOL, "thin gemm_tn beta=%g" % beta,
+                     floor=np.sqrt(K))
+    again = dev.tensor(y0)
+    dev.gemm_tn(M, N, K, lt, rt, 0.5, again)
+    assert again.numpy().tobytes() == yt.numpy().tobytes()  # a fixed order of additions
+
+
 # Large outputs go to the 256 x 256-tile kernel, which deals the k-tiles of all tiles to the CUs in equal segments:
 # (a) fewer tiles than CUs: every tile spans several segments, whose partial tiles a second kernel adds; ragged edges
 # and a depth that is not a multiple of 32 (the rest of the depth is added by the 128-wide kernel); (b), (c) a little
