@@ -461,6 +461,163 @@ static int gemm_nt_thin_run(dyhip_device* dev, size_t M, size_t N, size_t K, con
 }
 
 
+// ---- C = beta * C (or bias) + A * B with at most 8 columns of B: matrix times vector(s), the un-batched graph's
+// product (affine layers, output projections, one sentence at a time) -----------------------------------------------
+// Memory work: A (M x K, rows contiguous inside a column) is read once in kilobyte runs, lane l owning rows 4l..4l+3 of
+// a 256-row slab for every depth index of its wavefront's range; the depth is split over the block's four wavefronts
+// (combined through LDS) and, to fill the GPU, over gridDim.y blocks, whose slabs of partial sums a second small
+// kernel adds (with the epilogue).  The tile kernel gives a one-column product to M / 128 blocks that each walk the
+// whole depth: 60 us for 4096 x 1024, 117 us for 4096 x 2048.
+constexpr int kGemvWaves = 4;
+constexpr unsigned kGemvMaxChunk = 4096;  // depth indices per block
+template <int NB>  // columns padded to 1, 2, 4 or 8
+__global__ __launch_bounds__(64 * kGemvWaves) void gemm_nn_thin_kernel(unsigned M4, unsigned N, unsigned K, unsigned chunk,
+                                                                      const float* __restrict__ A, size_t lda,
+                                                                      const float* __restrict__ B, size_t ldb,
+                                                                      float* __restrict__ C, float beta,
+                                                                      const float* __restrict__ bias,
+                                                                      float* __restrict__ partial) {
+  __shared__ float4 red[kGemvWaves - 1][64][NB];
+  const unsigned k0 = blockIdx.y * chunk, k1 = min(K, k0 + chunk);
+  const unsigned lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const unsigned m4 = blockIdx.x * 64 + lane;
+  const bool live = m4 < M4;
+  const float4* a4 = reinterpret_cast<const float4*>(A) + (live ? m4 : M4 - 1);
+  const size_t lda4 = lda / 4;
+  // wavefront w takes the depth indices k0 + w, k0 + w + 4, ..., eight at a time: eight 128-bit loads of A in flight
+  // and, beside them, the entries of B for those eight indices, one index per lane (lane l fetches index l % 8; the
+  // multiply reads them back lane by lane through scalar registers), so that nothing is staged and waited for first
+  float4 acc[NB];
+#pragma unroll
+  for (int n = 0; n < NB; ++n) acc[n] = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (unsigned k = k0 + w; k < k1; k += 8 * kGemvWaves) {
+    float4 a[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) a[u] = ldg4<true>(a4 + size_t(min(k + u * kGemvWaves, k1 - 1)) * lda4);
+    const unsigned kmine = k + (lane & 7u) * kGemvWaves;
+    float xv[NB];
+#pragma unroll
+    for (int n = 0; n < NB; ++n) xv[n] = kmine < k1 && unsigned(n) < N ? B[size_t(kmine) + size_t(n) * ldb] : 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+#pragma unroll
+      for (int n = 0; n < NB; ++n) {
+        const float b = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, xv[n]), u));  // 0 past the end
+        acc[n].x = fmaf(a[u].x, b, acc[n].x);
+        acc[n].y = fmaf(a[u].y, b, acc[n].y);
+        acc[n].z = fmaf(a[u].z, b, acc[n].z);
+        acc[n].w = fmaf(a[u].w, b, acc[n].w);
+      }
+    }
+  }
+  if (w > 0) {
+#pragma unroll
+    for (int n = 0; n < NB; ++n) red[w - 1][lane][n] = acc[n];
+  }
+  __syncthreads();
+  if (w != 0 || !live) return;
+#pragma unroll
+  for (int n = 0; n < NB; ++n) {
+    if (unsigned(n) >= N) break;
+    float4 t = acc[n];
+#pragma unroll
+    for (int v = 0; v < kGemvWaves - 1; ++v) {
+      const float4 o = red[v][lane][n];
+      t.x += o.x; t.y += o.y; t.z += o.z; t.w += o.w;
+    }
+    if (partial != nullptr) {
+      reinterpret_cast<float4*>(partial)[(size_t(blockIdx.y) * N + n) * M4 + m4] = t;
+    } else {
+      float4* out = reinterpret_cast<float4*>(C) + size_t(n) * M4 + m4;
+      if (bias != nullptr) {
+        const float4 bb = reinterpret_cast<const float4*>(bias)[m4];
+        t.x += bb.x; t.y += bb.y; t.z += bb.z; t.w += bb.w;
+      } else if (beta != 0.f) {
+        const float4 o = *out;
+        t.x += beta * o.x; t.y += beta * o.y; t.z += beta * o.z; t.w += beta * o.w;
+      }
+      *out = t;
+    }
+  }
+}
+
+// C = beta * C (or bias) + the slabs' sum, slabs in ascending order
+__global__ __launch_bounds__(256) void gemm_nn_thin_combine_kernel(unsigned M4, unsigned N, unsigned slabs,
+                                                                   const float4* __restrict__ partial,
+                                                                   float4* __restrict__ C, float beta,
+                                                                   const float4* __restrict__ bias) {
+  const size_t e = size_t(blockIdx.x) * 256 + threadIdx.x, total = size_t(M4) * N;
+  if (e >= total) return;
+  float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (unsigned s0 = 0; s0 < slabs; s0 += 8) {  // eight slabs in flight, added in ascending order
+    float4 o[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) o[u] = partial[size_t(min(s0 + u, slabs - 1)) * total + e];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (s0 + u < slabs) {
+        t.x += o[u].x; t.y += o[u].y; t.z += o[u].z; t.w += o[u].w;
+      }
+    }
+  }
+  if (bias != nullptr) {
+    const float4 bb = bias[e % M4];
+    t.x += bb.x; t.y += bb.y; t.z += bb.z; t.w += bb.w;
+  } else if (beta != 0.f) {
+    const float4 o = C[e];
+    t.x += beta * o.x; t.y += beta * o.y; t.z += beta * o.z; t.w += beta * o.w;
+  }
+  C[e] = t;
+}
+
+static bool gemm_nn_thin_eligible(const dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda,
+                                  const float* B, const float* C, const GemmEpiParams& epi) {
+  if (!(epi.kind == kEpiAxpby || (epi.kind == kEpiBias && epi.bias != nullptr && aligned16(epi.bias)))) return false;
+  return N >= 1 && N <= 8 && M >= 256 && M % 4 == 0 && M / 4 <= 0x7FFFFFFFull && K >= 1 && K <= 0x7FFFFFFFull &&
+         lda % 4 == 0 && aligned16(A) && aligned16(C) && B != nullptr && dev->gemm_ws != nullptr;
+}
+
+static int gemm_nn_thin_run(dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B,
+                            size_t ldb, float* C, const GemmEpiParams& epi) {
+  const unsigned M4 = static_cast<unsigned>(M / 4), bx = cdiv<unsigned>(M4, 64);
+  // depth slabs: enough blocks for two per CU, each with at least 32 and at most kGemvMaxChunk depth indices, and
+  // partial sums that fit the workspace
+  unsigned slabs = cdiv<unsigned>(2 * dev->num_cus, bx);
+  const unsigned max_by_depth = cdiv<unsigned>(static_cast<unsigned>(K), 32);
+  if (slabs > max_by_depth) slabs = max_by_depth;
+  if (slabs < cdiv<unsigned>(static_cast<unsigned>(K), kGemvMaxChunk)) slabs = cdiv<unsigned>(static_cast<unsigned>(K), kGemvMaxChunk);
+  unsigned chunk = cdiv<unsigned>(static_cast<unsigned>(K), slabs);
+  chunk = (chunk + 7) / 8 * 8;
+  slabs = cdiv<unsigned>(static_cast<unsigned>(K), chunk);
+  DYHIP_REQUIRE(slabs <= 65535 && chunk <= kGemvMaxChunk, "matrix-vector product: depth %zu needs too many slabs", K);
+  float* partial = nullptr;
+  if (slabs > 1) {
+    DYHIP_REQUIRE(dev->gemm_ws_bytes >= sizeof(float) * M * N * slabs, "matrix-vector product: workspace too small");
+    partial = static_cast<float*>(dev->gemm_ws);
+  }
+  const float beta = epi.kind == kEpiAxpby ? epi.beta : 0.f;
+  const float* bias = epi.kind == kEpiBias ? epi.bias : nullptr;
+  const dim3 grid(bx, slabs), block(64 * kGemvWaves);
+#define DYHIP_GEMV(NB)                                                                                          \
+  hipLaunchKernelGGL(gemm_nn_thin_kernel<NB>, grid, block, 0, dev->stream, M4, static_cast<unsigned>(N),       \
+                     static_cast<unsigned>(K), chunk, A, lda, B, ldb, C, beta, bias, partial)
+  if (N == 1) DYHIP_GEMV(1);
+  else if (N == 2) DYHIP_GEMV(2);
+  else if (N <= 4) DYHIP_GEMV(4);
+  else DYHIP_GEMV(8);
+#undef DYHIP_GEMV
+  DYHIP_CHECK_LAUNCH();
+  if (slabs > 1) {
+    const size_t total = size_t(M4) * N;
+    hipLaunchKernelGGL(gemm_nn_thin_combine_kernel, dim3(static_cast<unsigned>(cdiv<size_t>(total, 256))), dim3(256), 0,
+                       dev->stream, M4, static_cast<unsigned>(N), slabs, reinterpret_cast<const float4*>(partial),
+                       reinterpret_cast<float4*>(C), beta, reinterpret_cast<const float4*>(bias));
+    DYHIP_CHECK_LAUNCH();
+  }
+  return DYHIP_OK;
+}
+
+
 int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N, int nseg, const GemmSeg* segs,
              float* C, const GemmEpiParams& epi, const GemmBatch* batch) {
   const bool to_caller = epi.kind == kEpiPartials;
@@ -499,6 +656,10 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
       return gemm_run(dev, a_kmajor, b_kmajor, M, N - cols, 1, &rest, C + cols * M, epi, nullptr);
     }
   }
+  if (nseg == 1 && (batch == nullptr || batch->count <= 1) && !a_kmajor && b_kmajor && segs[0].A != nullptr &&
+      segs[0].B != nullptr && C != nullptr &&
+      gemm_nn_thin_eligible(dev, M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, C, epi))
+    return gemm_nn_thin_run(dev, M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, segs[0].ldb, C, epi);
   if (nseg == 1 && (batch == nullptr || batch->count <= 1) && !a_kmajor && !b_kmajor && epi.kind == kEpiAxpby &&
       segs[0].A != nullptr && segs[0].B != nullptr && C != nullptr &&
       gemm_nt_thin_eligible(M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, C, epi.beta))

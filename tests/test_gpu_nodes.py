@@ -123,6 +123,29 @@ def test_gemm_tn_thin(dev, M, N, K):
     assert again.numpy().tobytes() == yt.numpy().tobytes()  # a fixed order of additions
 
 
+# l * r with at most 8 columns of r (matrix times vector: the un-batched graph's affine layers and projections): the
+# depth split into slabs over blocks, their partial sums added by a second kernel with the epilogue (beta or bias).
+@pytest.mark.parametrize("M,N,K", [(4096, 1, 1024), (10000, 1, 1024), (1024, 3, 1000), (256, 8, 37), (6000, 5, 1500),
+                                   (260, 2, 8), (4096, 4, 2048), (512, 1, 20000)])
+def test_gemm_nn_thin(dev, M, N, K):
+    rng = np.random.default_rng(M + N + K)
+    y0 = f32(rng.standard_normal((N, M)))
+    l, r2, bias = f32(rng.standard_normal((K, M))), f32(rng.standard_normal((N, K))), f32(rng.standard_normal(M))
+    lt, rt, bt = dev.tensor(l), dev.tensor(r2), dev.tensor(bias)
+    ref64 = r2.astype(np.float64) @ l.astype(np.float64)
+    for beta in (1.0, 0.0, 0.5):
+        yt = dev.tensor(y0)
+        dev.gemm_nn(M, N, K, lt, rt, beta, yt)
+        assert_close(yt.numpy(), (beta * y0 + ref64).astype(np.float32), FWD_RTOL, "thin gemm_nn beta=%g" % beta,
+                     floor=np.sqrt(K))
+    again = dev.tensor(y0)
+    dev.gemm_nn(M, N, K, lt, rt, 0.5, again)
+    assert again.numpy().tobytes() == yt.numpy().tobytes()  # a fixed order of additions
+    yt = dev.tensor(y0)
+    dev.affine_forward(M, N, K, bt, lt, rt, yt)
+    assert_close(yt.numpy(), (bias[None, :] + ref64).astype(np.float32), FWD_RTOL, "thin affine", floor=np.sqrt(K))
+
+
 # Large outputs go to the 256 x 256-tile kernel, which deals the k-tiles of all tiles to the CUs in equal segments:
 # (a) fewer tiles than CUs: every tile spans several segments, whose partial tiles a second kernel adds; ragged edges
 # and a depth that is not a multiple of 32 (the rest of the depth is added by the 128-wide kernel); (b), (c) a little
