@@ -471,14 +471,20 @@ static int gemm_nt_thin_run(dyhip_device* dev, size_t M, size_t N, size_t K, con
 constexpr int kGemvWaves = 4;
 constexpr unsigned kGemvMaxChunk = 4096;  // depth indices per block
 template <int NB>  // columns padded to 1, 2, 4 or 8
-__global__ __launch_bounds__(64 * kGemvWaves) void gemm_nn_thin_kernel(unsigned M4, unsigned N, unsigned K, unsigned chunk,
-                                                                      const float* __restrict__ A, size_t lda,
-                                                                      const float* __restrict__ B, size_t ldb,
+__global__ __launch_bounds__(64 * kGemvWaves) void gemm_nn_thin_kernel(unsigned M4, unsigned N, unsigned chunk,
+                                                                      GemmSeg seg0, GemmSeg seg1, unsigned slabs0,
                                                                       float* __restrict__ C, float beta,
                                                                       const float* __restrict__ bias,
                                                                       float* __restrict__ partial) {
   __shared__ float4 red[kGemvWaves - 1][64][NB];
-  const unsigned k0 = blockIdx.y * chunk, k1 = min(K, k0 + chunk);
+  // a product over two depth segments (the gates node: Wx x + Wh h) is one sequence of slabs: the first slabs0 walk
+  // the first segment, the others the second; the choice is the same for the whole block
+  const bool second = blockIdx.y >= slabs0;
+  const float* __restrict__ A = second ? seg1.A : seg0.A;
+  const float* __restrict__ B = second ? seg1.B : seg0.B;
+  const size_t lda = second ? seg1.lda : seg0.lda, ldb = second ? seg1.ldb : seg0.ldb;
+  const unsigned K = static_cast<unsigned>(second ? seg1.K : seg0.K);
+  const unsigned k0 = (second ? blockIdx.y - slabs0 : blockIdx.y) * chunk, k1 = min(K, k0 + chunk);
   const unsigned lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const unsigned m4 = blockIdx.x * 64 + lane;
   const bool live = m4 < M4;
@@ -542,10 +548,13 @@ __global__ __launch_bounds__(64 * kGemvWaves) void gemm_nn_thin_kernel(unsigned 
 }
 
 // C = beta * C (or bias) + the slabs' sum, slabs in ascending order
+// GATES: C = act(bias + (forget rows: 1) + sum), the epilogue of the gates node (kEpiLstmGates)
+template <bool GATES>
 __global__ __launch_bounds__(256) void gemm_nn_thin_combine_kernel(unsigned M4, unsigned N, unsigned slabs,
                                                                    const float4* __restrict__ partial,
                                                                    float4* __restrict__ C, float beta,
-                                                                   const float4* __restrict__ bias) {
+                                                                   const float* __restrict__ bias, unsigned H,
+                                                                   int logistic_mode) {
   const size_t e = size_t(blockIdx.x) * 256 + threadIdx.x, total = size_t(M4) * N;
   if (e >= total) return;
   float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -560,8 +569,22 @@ __global__ __launch_bounds__(256) void gemm_nn_thin_combine_kernel(unsigned M4, 
       }
     }
   }
+  if (GATES) {
+    const unsigned i0 = static_cast<unsigned>(e % M4) * 4;
+    float v[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const unsigned i = i0 + c;
+      float pre = bias[i];
+      if (i >= H && i < 2 * H) pre += 1.0f;  // forget-gate bias
+      pre += v[c];
+      v[c] = i < 3 * H ? logistic(logistic_mode, pre) : tanh_accurate(pre);
+    }
+    C[e] = make_float4(v[0], v[1], v[2], v[3]);
+    return;
+  }
   if (bias != nullptr) {
-    const float4 bb = bias[e % M4];
+    const float4 bb = reinterpret_cast<const float4*>(bias)[e % M4];
     t.x += bb.x; t.y += bb.y; t.z += bb.z; t.w += bb.w;
   } else if (beta != 0.f) {
     const float4 o = C[e];
@@ -570,48 +593,64 @@ __global__ __launch_bounds__(256) void gemm_nn_thin_combine_kernel(unsigned M4, 
   C[e] = t;
 }
 
-static bool gemm_nn_thin_eligible(const dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda,
-                                  const float* B, const float* C, const GemmEpiParams& epi) {
-  if (!(epi.kind == kEpiAxpby || (epi.kind == kEpiBias && epi.bias != nullptr && aligned16(epi.bias)))) return false;
-  return N >= 1 && N <= 8 && M >= 256 && M % 4 == 0 && M / 4 <= 0x7FFFFFFFull && K >= 1 && K <= 0x7FFFFFFFull &&
-         lda % 4 == 0 && aligned16(A) && aligned16(C) && B != nullptr && dev->gemm_ws != nullptr;
+static bool gemm_nn_thin_eligible(const dyhip_device* dev, size_t M, size_t N, int nseg, const GemmSeg* segs,
+                                  const float* C, const GemmEpiParams& epi) {
+  if (!(epi.kind == kEpiAxpby || (epi.kind == kEpiBias && epi.bias != nullptr && aligned16(epi.bias)) ||
+        (epi.kind == kEpiLstmGates && epi.bias != nullptr)))
+    return false;
+  if (nseg < 1 || nseg > 2 || (nseg == 2 && epi.kind != kEpiLstmGates)) return false;
+  for (int q = 0; q < nseg; ++q)
+    if (segs[q].A == nullptr || segs[q].B == nullptr || segs[q].K < 1 || segs[q].K > 0x3FFFFFFFull || segs[q].lda % 4 != 0 ||
+        !aligned16(segs[q].A))
+      return false;
+  return N >= 1 && N <= 8 && M >= 256 && M % 4 == 0 && M / 4 <= 0x7FFFFFFFull && aligned16(C) && dev->gemm_ws != nullptr;
 }
 
-static int gemm_nn_thin_run(dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B,
-                            size_t ldb, float* C, const GemmEpiParams& epi) {
+static int gemm_nn_thin_run(dyhip_device* dev, size_t M, size_t N, int nseg, const GemmSeg* segs, float* C,
+                            const GemmEpiParams& epi) {
   const unsigned M4 = static_cast<unsigned>(M / 4), bx = cdiv<unsigned>(M4, 64);
+  const unsigned K0 = static_cast<unsigned>(segs[0].K), K1 = nseg > 1 ? static_cast<unsigned>(segs[1].K) : 0u;
+  const unsigned K = K0 + K1;
   // depth slabs: enough blocks for two per CU, each with at least 32 and at most kGemvMaxChunk depth indices, and
   // partial sums that fit the workspace
   unsigned slabs = cdiv<unsigned>(2 * dev->num_cus, bx);
-  const unsigned max_by_depth = cdiv<unsigned>(static_cast<unsigned>(K), 32);
+  const unsigned max_by_depth = cdiv<unsigned>(K, 32);
   if (slabs > max_by_depth) slabs = max_by_depth;
-  if (slabs < cdiv<unsigned>(static_cast<unsigned>(K), kGemvMaxChunk)) slabs = cdiv<unsigned>(static_cast<unsigned>(K), kGemvMaxChunk);
-  unsigned chunk = cdiv<unsigned>(static_cast<unsigned>(K), slabs);
+  if (slabs < cdiv<unsigned>(K, kGemvMaxChunk)) slabs = cdiv<unsigned>(K, kGemvMaxChunk);
+  unsigned chunk = cdiv<unsigned>(K, slabs);
   chunk = (chunk + 7) / 8 * 8;
-  slabs = cdiv<unsigned>(static_cast<unsigned>(K), chunk);
-  DYHIP_REQUIRE(slabs <= 65535 && chunk <= kGemvMaxChunk, "matrix-vector product: depth %zu needs too many slabs", K);
+  const unsigned slabs0 = cdiv<unsigned>(K0, chunk), slabs1 = K1 ? cdiv<unsigned>(K1, chunk) : 0u;
+  slabs = slabs0 + slabs1;
+  DYHIP_REQUIRE(slabs <= 65535 && chunk <= kGemvMaxChunk, "matrix-vector product: depth %u needs too many slabs", K);
+  const bool gates = epi.kind == kEpiLstmGates;
   float* partial = nullptr;
-  if (slabs > 1) {
+  if (slabs > 1 || gates) {  // the gates epilogue lives in the second kernel
     DYHIP_REQUIRE(dev->gemm_ws_bytes >= sizeof(float) * M * N * slabs, "matrix-vector product: workspace too small");
     partial = static_cast<float*>(dev->gemm_ws);
   }
   const float beta = epi.kind == kEpiAxpby ? epi.beta : 0.f;
-  const float* bias = epi.kind == kEpiBias ? epi.bias : nullptr;
+  const float* bias = epi.kind == kEpiAxpby ? nullptr : epi.bias;
+  const GemmSeg s0 = segs[0], s1 = nseg > 1 ? segs[1] : segs[0];
   const dim3 grid(bx, slabs), block(64 * kGemvWaves);
-#define DYHIP_GEMV(NB)                                                                                          \
-  hipLaunchKernelGGL(gemm_nn_thin_kernel<NB>, grid, block, 0, dev->stream, M4, static_cast<unsigned>(N),       \
-                     static_cast<unsigned>(K), chunk, A, lda, B, ldb, C, beta, bias, partial)
+#define DYHIP_GEMV(NB)                                                                                             \
+  hipLaunchKernelGGL(gemm_nn_thin_kernel<NB>, grid, block, 0, dev->stream, M4, static_cast<unsigned>(N), chunk, s0, s1, \
+                     slabs0, C, beta, bias, partial)
   if (N == 1) DYHIP_GEMV(1);
   else if (N == 2) DYHIP_GEMV(2);
   else if (N <= 4) DYHIP_GEMV(4);
   else DYHIP_GEMV(8);
 #undef DYHIP_GEMV
   DYHIP_CHECK_LAUNCH();
-  if (slabs > 1) {
+  if (partial != nullptr) {
     const size_t total = size_t(M4) * N;
-    hipLaunchKernelGGL(gemm_nn_thin_combine_kernel, dim3(static_cast<unsigned>(cdiv<size_t>(total, 256))), dim3(256), 0,
-                       dev->stream, M4, static_cast<unsigned>(N), slabs, reinterpret_cast<const float4*>(partial),
-                       reinterpret_cast<float4*>(C), beta, reinterpret_cast<const float4*>(bias));
+    const dim3 g2(static_cast<unsigned>(cdiv<size_t>(total, 256)));
+    if (gates)
+      hipLaunchKernelGGL(gemm_nn_thin_combine_kernel<true>, g2, dim3(256), 0, dev->stream, M4, static_cast<unsigned>(N),
+                         slabs, reinterpret_cast<const float4*>(partial), reinterpret_cast<float4*>(C), 0.f, bias, epi.H,
+                         epi.logistic_mode);
+    else
+      hipLaunchKernelGGL(gemm_nn_thin_combine_kernel<false>, g2, dim3(256), 0, dev->stream, M4, static_cast<unsigned>(N),
+                         slabs, reinterpret_cast<const float4*>(partial), reinterpret_cast<float4*>(C), beta, bias, 0u, 0);
     DYHIP_CHECK_LAUNCH();
   }
   return DYHIP_OK;
@@ -656,10 +695,9 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
       return gemm_run(dev, a_kmajor, b_kmajor, M, N - cols, 1, &rest, C + cols * M, epi, nullptr);
     }
   }
-  if (nseg == 1 && (batch == nullptr || batch->count <= 1) && !a_kmajor && b_kmajor && segs[0].A != nullptr &&
-      segs[0].B != nullptr && C != nullptr &&
-      gemm_nn_thin_eligible(dev, M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, C, epi))
-    return gemm_nn_thin_run(dev, M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, segs[0].ldb, C, epi);
+  if ((batch == nullptr || batch->count <= 1) && !a_kmajor && b_kmajor && C != nullptr &&
+      gemm_nn_thin_eligible(dev, M, N, nseg, segs, C, epi))
+    return gemm_nn_thin_run(dev, M, N, nseg, segs, C, epi);
   if (nseg == 1 && (batch == nullptr || batch->count <= 1) && !a_kmajor && !b_kmajor && epi.kind == kEpiAxpby &&
       segs[0].A != nullptr && segs[0].B != nullptr && C != nullptr &&
       gemm_nt_thin_eligible(M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, C, epi.beta))

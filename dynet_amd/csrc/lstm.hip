@@ -1000,6 +1000,14 @@ int dyhip_lstm_gates_forward(dyhip_device* dev, unsigned num_inputs, const float
   DYHIP_CHECK_STATUS(prepare_x(dev, num_inputs, xs_host, x_dims_host, gi.I, B, mask_x, mask_x_bd, xbuf, &x_eff));
   DYHIP_CHECK_STATUS(prepare_h(dev, H, B, h_tm1, mask_h, mask_h_bd, hbuf, &h_eff));
   const size_t G = size_t(4) * H;
+  // up to 8 columns (the un-batched graph, decoding): the weights are the whole cost and stream through the
+  // matrix-times-vector kernel in kilobyte runs, its second kernel adding the depth slabs with the gates' epilogue
+  // (I = H = 1024, one column: 22 -> 10.6 us; the fragment-order kernel below reads them in 128-byte pieces)
+  if (B <= 8 && G >= 256) {
+    GemmSeg segs[2] = {{Wx, G, x_eff, gi.I, gi.I}, {Wh, G, h_eff, H, H}};
+    GemmEpiParams ep{kEpiLstmGates, 0.f, b, H, logistic_mode};
+    return gemm_run(dev, false, true, G, B, 2, segs, fx, ep);
+  }
   // a batch of a few column tiles: one launch of the fragment-order kernel on the operands as they lie
   if (B <= 256 && H % 16 == 0 && gi.I % 128 == 0 && H % 128 == 0 && G < (size_t(1) << 31) &&
       all_aligned16({Wx, Wh, x_eff, h_eff}) && (G / 64) * cdiv<unsigned>(B, 32) >= unsigned(dev->num_cus > 0 ? dev->num_cus : 256) / 2) {

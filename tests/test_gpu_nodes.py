@@ -437,6 +437,12 @@ def _lstm_case(rng, I, H, B):
     (4, 5, 2, [1, 3], False, True),         # :433-460 (multi-input)
     (4, 5, 2, [1, 3], True, True),          # :499-529
     (37, 19, 7, [5, 32], True, False),
+    # up to 8 columns with at least 256 gate rows: the matrix-times-vector kernels (forward over both depth segments
+    # with the gates' epilogue in its second kernel; streaming kernels for dx / dh and the weight gradients)
+    (128, 128, 1, None, False, True),
+    (200, 64, 3, None, False, True),
+    (256, 512, 8, None, True, True),
+    (96, 72, 2, [32, 64], False, True),
 ])
 def test_lstm_cell_forward_backward(dev, I, H, B, dims, dropout, mask_full):
     rng = np.random.default_rng(I * 100 + H * 10 + B)
