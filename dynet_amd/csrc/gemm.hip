@@ -318,19 +318,25 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(size_t M, size_
                                                                  float* __restrict__ C, GemmEpiParams ep) {
   const size_t e = size_t(blockIdx.x) * 256 + threadIdx.x;
   if (e >= total) return;
+  // eight slices in flight (a loop of one load and one add per slice waits a memory round trip per slice)
+  float s = 0.f;
+  for (unsigned k0 = 0; k0 < splits; k0 += 8) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = partial[size_t(min(k0 + u, splits - 1)) * total + e];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (k0 + u < splits) s += v[u];
+  }
   if (EPI == kEpiAxpby) {
-    float s = partial[e];
-    for (unsigned k = 1; k < splits; ++k) s += partial[size_t(k) * total + e];
     C[e] = ep.beta != 0.f ? ep.beta * C[e] + s : s;
   } else if (EPI == kEpiBias) {
-    float s = ep.bias[e % M];
-    for (unsigned k = 0; k < splits; ++k) s += partial[size_t(k) * total + e];
-    C[e] = s;
+    C[e] = ep.bias[e % M] + s;
   } else {
     const unsigned i = static_cast<unsigned>(e % M);
     float pre = ep.bias[i];
     if (i >= ep.H && i < 2 * ep.H) pre += 1.0f;  // forget-gate bias
-    for (unsigned k = 0; k < splits; ++k) pre += partial[size_t(k) * total + e];
+    pre += s;
     C[e] = i < 3 * ep.H ? logistic(ep.logistic_mode, pre) : tanh_accurate(pre);
   }
 }
