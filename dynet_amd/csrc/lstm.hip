@@ -740,9 +740,17 @@ __global__ __launch_bounds__(256) void slices_accumulate_kernel(size_t total, un
                                                                 float* __restrict__ out) {
   const size_t e = size_t(blockIdx.x) * 256 + threadIdx.x;
   if (e >= total) return;
-  float s = slices[e];
-  for (unsigned k = 1; k < splits; ++k) s += slices[size_t(k) * total + e];
-  out[e] = beta != 0.f ? beta * out[e] + s : s;
+  const float old = beta != 0.f ? out[e] : 0.f;  // fetched beside the slices
+  float s = 0.f;
+  for (unsigned k0 = 0; k0 < splits; k0 += 8) {  // eight slices in flight, added in ascending order
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = slices[size_t(min(k0 + u, splits - 1)) * total + e];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (k0 + u < splits) s += v[u];
+  }
+  out[e] = beta != 0.f ? beta * old + s : s;
 }
 
 static bool all_aligned16(std::initializer_list<const void*> ps) {
