@@ -157,13 +157,21 @@ __global__ __launch_bounds__(kCellThreads) void lstm_cell_fwd_kernel(unsigned H,
 #pragma unroll
     for (int e = 0; e < V; ++e) pre[q].v[e] = (q == 1 ? bq.v[e] + 1.0f : bq.v[e]) + xq.v[e];
   }
-  for (unsigned k = 0; k < splits; ++k) {
+  // four slices at a time, all their loads in flight (a slice past the end repeats the last one and is not added)
+  for (unsigned k0 = 0; k0 < splits; k0 += 4) {
+    Pack<V> r[4][4];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      Pack<V> r;
-      r.load(rec + size_t(k) * slice + g0 + size_t(q) * H);
+    for (int u = 0; u < 4; ++u)
 #pragma unroll
-      for (int e = 0; e < V; ++e) pre[q].v[e] += r.v[e];
+      for (int q = 0; q < 4; ++q) r[u][q].load(rec + size_t(min(k0 + u, splits - 1)) * slice + g0 + size_t(q) * H);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (k0 + u < splits) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int e = 0; e < V; ++e) pre[q].v[e] += r[u][q].v[e];
+      }
     }
   }
   if (c_prev) cp.load(c_prev + s0);
@@ -206,11 +214,17 @@ __global__ __launch_bounds__(kCellThreads) void lstm_cell_bwd_kernel(unsigned H,
   dh.load(dh_in + s0);
   if (c_prev) cp.load(c_prev + s0);
   if (dc_in) dc.load(dc_in + s0);
-  for (unsigned k = 0; k < splits; ++k) {
-    Pack<V> r;
-    r.load(rec + size_t(k) * slice + s0);
+  for (unsigned k0 = 0; k0 < splits; k0 += 4) {  // four slices in flight, added in ascending order
+    Pack<V> r[4];
 #pragma unroll
-    for (int e = 0; e < V; ++e) dh.v[e] += r.v[e];
+    for (int u = 0; u < 4; ++u) r[u].load(rec + size_t(min(k0 + u, splits - 1)) * slice + s0);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (k0 + u < splits) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) dh.v[e] += r[u].v[e];
+      }
+    }
   }
   Pack<V> out[4], dcp;
 #pragma unroll
