@@ -1032,7 +1032,9 @@ int dyhip_lstm_gates_forward(dyhip_device* dev, unsigned num_inputs, const float
   }
   // a batch of a few column tiles: one launch of the fragment-order kernel on the operands as they lie
   if (B <= 256 && H % 16 == 0 && gi.I % 128 == 0 && H % 128 == 0 && G < (size_t(1) << 31) &&
-      all_aligned16({Wx, Wh, x_eff, h_eff}) && (G / 64) * cdiv<unsigned>(B, 32) >= unsigned(dev->num_cus > 0 ? dev->num_cus : 256) / 2) {
+      all_aligned16({Wx, Wh, x_eff, h_eff}) &&
+      ((G / 64) * cdiv<unsigned>(B, 32) >= unsigned(dev->num_cus > 0 ? dev->num_cus : 256) / 2 ||
+       G * (gi.I + H) * sizeof(float) <= (size_t(4) << 20))) {
     const NnOperand op0{Wx, x_eff, gi.I}, op1{Wh, h_eff, H};
     hipLaunchKernelGGL(lstm_gates_skinny_kernel, dim3(unsigned(G / 64) * cdiv<unsigned>(B, 32)), dim3(256), 0, dev->stream, H,
                        B, op0, op1, b, logistic_mode, fx);
