@@ -396,8 +396,9 @@ static GemmPlan plan_gemm(const dyhip_device* dev, size_t M, size_t N, unsigned 
 // configuration) to eight blocks.
 // (Sixteen columns per thread, for half the re-reads of A from the L2, measured no better or worse: 10.4 against
 // 10.3 us at 4096 x 1024 x 20, 34.3 against 26.3 us at 8192 x 2048 x 16.)
-constexpr int kThinCols = 8;
-template <int KT>  // KT: depth rounded up to a multiple of four
+// Four or two columns per thread while the wider form would leave fewer than two blocks per CU (a small output: more
+// blocks, fewer multiply-adds per thread; 1024 x 128 x 32: 6.8 us with eight, 5.0 with four).
+template <int KT, int kThinCols>  // KT: depth rounded up to a multiple of four
 __global__ __launch_bounds__(256) void gemm_nt_thin_kernel(unsigned M4, unsigned N, unsigned K, const float* __restrict__ A,
                                                            size_t lda, const float* __restrict__ B, size_t ldb,
                                                            float* __restrict__ C, float beta) {
@@ -440,17 +441,26 @@ __global__ __launch_bounds__(256) void gemm_nt_thin_kernel(unsigned M4, unsigned
 static bool gemm_nt_thin_eligible(size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B, float* C,
                                   float beta) {
   return K >= 1 && K <= 32 && M % 4 == 0 && lda % 4 == 0 && M >= 256 && N >= 1 && N <= 0xFFFFFFFFull / 2 &&
-         M / 4 <= 0xFFFFFFFFull && cdiv<size_t>(N, kThinCols) <= 65535 && aligned16(A) && aligned16(C) && B != nullptr &&
+         M / 4 <= 0xFFFFFFFFull && cdiv<size_t>(N, 2) <= 65535 && aligned16(A) && aligned16(C) && B != nullptr &&
          (beta == 0.f || beta == 1.f);
 }
 
 static int gemm_nt_thin_run(dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B,
                             size_t ldb, float* C, float beta) {
   const unsigned M4 = static_cast<unsigned>(M / 4);
-  const dim3 grid(cdiv<unsigned>(M4, 256), static_cast<unsigned>(cdiv<size_t>(N, kThinCols))), block(256);
-#define DYHIP_THIN(KT)                                                                                             \
-  hipLaunchKernelGGL(gemm_nt_thin_kernel<KT>, grid, block, 0, dev->stream, M4, static_cast<unsigned>(N),           \
+  // columns per thread: eight, or four, or two while the wider form would leave fewer than two blocks per CU
+  const size_t want = 2 * size_t(dev->num_cus), bxm = cdiv<unsigned>(M4, 256);
+  const int cols = bxm * cdiv<size_t>(N, 8) >= want ? 8 : bxm * cdiv<size_t>(N, 4) >= want ? 4 : 2;
+  const dim3 grid(static_cast<unsigned>(bxm), static_cast<unsigned>(cdiv<size_t>(N, size_t(cols)))), block(256);
+#define DYHIP_THIN_C(KT, COLS)                                                                                        \
+  hipLaunchKernelGGL((gemm_nt_thin_kernel<KT, COLS>), grid, block, 0, dev->stream, M4, static_cast<unsigned>(N),      \
                      static_cast<unsigned>(K), A, lda, B, ldb, C, beta)
+#define DYHIP_THIN(KT)                     \
+  do {                                     \
+    if (cols == 8) DYHIP_THIN_C(KT, 8);    \
+    else if (cols == 4) DYHIP_THIN_C(KT, 4); \
+    else DYHIP_THIN_C(KT, 2);              \
+  } while (0)
   switch ((K + 3) / 4) {  // the depth rounded up to a multiple of four: a padded step costs as much as a real one
     case 1: DYHIP_THIN(4); break;
     case 2: DYHIP_THIN(8); break;
@@ -462,6 +472,7 @@ static int gemm_nt_thin_run(dyhip_device* dev, size_t M, size_t N, size_t K, con
     default: DYHIP_THIN(32); break;
   }
 #undef DYHIP_THIN
+#undef DYHIP_THIN_C
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
