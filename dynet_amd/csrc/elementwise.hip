@@ -206,6 +206,27 @@ __global__ __launch_bounds__(kEwThreads) void ew_bcast_vec4_kernel(EwArgs a, uns
     if (live && b0 + u < bd) stg4<NT>(reinterpret_cast<float4*>(a.out) + size_t(b0 + u) * n4 + j, r[u]);
 }
 
+// A batch-broadcast launch over batch elements that are far shorter than a tile and cannot take 128-bit accesses (a
+// scalar loss per batch element, n = 1: sum_batches backward over 100 000 of them was 100 000 blocks with one live
+// thread each, 29 us): the flat tensor, four entries a thread, the in-batch offset by one division.
+template <int NIN, bool ACC, int BMASK, class F>
+__global__ __launch_bounds__(kEwThreads) void ew_flat_bcast_kernel(EwArgs a, size_t total, F f) {
+  const size_t e0 = size_t(blockIdx.x) * (kEwThreads * 4) + threadIdx.x;
+  const bool small = total <= 0xFFFFFFFFull;  // the same for every thread: 32-bit division
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const size_t e = e0 + size_t(u) * kEwThreads;
+    if (e < total) {
+      const size_t j = small ? size_t(unsigned(e) % unsigned(a.n)) : e % a.n;
+      const float x0 = NIN > 0 ? a.in[0][(BMASK & 1) ? j : e] : 0.f;
+      const float x1 = NIN > 1 ? a.in[NIN > 1 ? 1 : 0][(BMASK & 2) ? j : e] : 0.f;
+      const float x2 = NIN > 2 ? a.in[NIN > 2 ? 2 : 0][(BMASK & 4) ? j : e] : 0.f;
+      const float od = ACC ? a.out[e] : 0.f;
+      a.out[e] = f(x0, x1, x2, od);
+    }
+  }
+}
+
 // Launch over an (n x bd) output.  Inputs whose bit is set in BMASK have batch 1.
 template <int NIN, bool ACC, int BMASK, class F>
 int ew_launch(dyhip_device* dev, size_t n, unsigned bd, const float* in0, const float* in1, const float* in2,
@@ -240,6 +261,10 @@ int ew_launch(dyhip_device* dev, size_t n, unsigned bd, const float* in0, const 
       hipLaunchKernelGGL((ew_bcast_vec4_kernel<NIN, ACC, BMASK, true, U, F>), g2, block, 0, dev->stream, a, bd, f);
     else
       hipLaunchKernelGGL((ew_bcast_vec4_kernel<NIN, ACC, BMASK, false, U, F>), g2, block, 0, dev->stream, a, bd, f);
+  } else if (BMASK != 0 && !vec && n < size_t(kEwThreads) && cdiv<size_t>(n * bd, size_t(kEwThreads) * 4) < (size_t(1) << 31)) {
+    const size_t total = n * bd;
+    hipLaunchKernelGGL((ew_flat_bcast_kernel<NIN, ACC, BMASK, F>), dim3(static_cast<unsigned>(cdiv<size_t>(total, size_t(kEwThreads) * 4))),
+                       block, 0, dev->stream, a, total, f);
   } else if (!vec) {
     hipLaunchKernelGGL((ew_scalar_kernel<NIN, ACC, BMASK, F>), grid, block, 0, dev->stream, a, f);
   } else if (stream) {
@@ -296,19 +321,49 @@ int batch_reduce(dyhip_device* dev, size_t n, unsigned bd, const float* in0, con
 
 // ---- Sum node: groups of up to four arguments per launch, in the reference's association order ----
 struct SumArgs {
-  const float* x[4];
-  unsigned bcast[4];  // 1: the argument has batch size 1 and is broadcast over the batch
-  unsigned cnt;
+  const float* x[32];
+  unsigned bcast;    // bit i: argument i has batch size 1 and is broadcast over the batch
+  unsigned cnt[8];   // members of each group (1..4)
+  unsigned ngroups;  // groups in this launch (1..8)
 };
 
-template <bool ACC>
+// Up to eight groups per launch (a Sum over the 35 per-timestep losses of a language model was nine launches): every
+// group is summed left to right, its four loads in flight together, and then added to what came before, so the
+// arithmetic is that of one launch per group.
+// ONE: a single group (the usual two to four arguments): its members at fixed places of the argument list (indexing
+// the list by a run-time position costs more than the sum itself there).
+template <bool ACC, bool ONE>
 __global__ __launch_bounds__(256) void sum_group_kernel(SumArgs a, size_t n, size_t total, float* __restrict__ fx) {
   const size_t e = size_t(blockIdx.x) * 256 + threadIdx.x;
   if (e >= total) return;
-  const size_t j = e % n;
-  float v = a.x[0][a.bcast[0] ? j : e];
-  for (unsigned i = 1; i < a.cnt; ++i) v = v + a.x[i][a.bcast[i] ? j : e];
-  fx[e] = ACC ? fx[e] + v : v;
+  const size_t j = a.bcast != 0 ? e % n : e;
+  float acc = ACC ? fx[e] : 0.f;
+  if (ONE) {
+    const unsigned cnt = a.cnt[0];
+    float t = a.x[0][a.bcast & 1u ? j : e];
+    if (cnt > 1) t = t + a.x[1][a.bcast & 2u ? j : e];
+    if (cnt > 2) t = t + a.x[2][a.bcast & 4u ? j : e];
+    if (cnt > 3) t = t + a.x[3][a.bcast & 8u ? j : e];
+    fx[e] = ACC ? acc + t : t;
+    return;
+  }
+  unsigned at = 0;
+  for (unsigned g = 0; g < a.ngroups; ++g) {
+    const unsigned cnt = a.cnt[g];
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const unsigned m = at + (unsigned(i) < cnt ? unsigned(i) : cnt - 1);  // past the group's end: its last member again
+      v[i] = a.x[m][(a.bcast >> m) & 1u ? j : e];
+    }
+    float t = v[0];
+#pragma unroll
+    for (int i = 1; i < 4; ++i)
+      if (unsigned(i) < cnt) t = t + v[i];
+    acc = (!ACC && g == 0) ? t : acc + t;
+    at += cnt;
+  }
+  fx[e] = acc;
 }
 
 static int check_bd(unsigned bd0, unsigned bd1) {
@@ -499,25 +554,37 @@ int dyhip_sum_forward(dyhip_device* dev, unsigned k, size_t n, unsigned bd, cons
   unsigned at = 0;
   bool first = true;
   while (at < k) {
-    unsigned cnt;
-    if (!same) cnt = 1;
-    else if (first) cnt = k < 4 ? k : 4;
-    else if (at == 4 && (k - 4) % 4 != 0) cnt = (k - 4) % 4;
-    else cnt = 4;
     SumArgs a;
-    a.cnt = cnt;
-    for (unsigned i = 0; i < 4; ++i) {
-      a.x[i] = i < cnt ? xs_host[at + i] : nullptr;
-      a.bcast[i] = (i < cnt && bds_host[at + i] != bd) ? 1u : 0u;
+    a.bcast = 0;
+    a.ngroups = 0;
+    unsigned used = 0;
+    const bool launch_first = first;
+    while (at < k && a.ngroups < 8 && used + 4 <= 32) {
+      unsigned cnt;
+      if (!same) cnt = 1;
+      else if (first) cnt = k < 4 ? k : 4;
+      else if (at == 4 && (k - 4) % 4 != 0) cnt = (k - 4) % 4;
+      else cnt = 4;
+      for (unsigned i = 0; i < cnt; ++i) {
+        a.x[used + i] = xs_host[at + i];
+        if (bds_host[at + i] != bd) a.bcast |= 1u << (used + i);
+      }
+      a.cnt[a.ngroups++] = cnt;
+      used += cnt;
+      at += cnt;
+      first = false;
     }
-    if (first && same)
-      hipLaunchKernelGGL(sum_group_kernel<false>, grid, block, 0, dev->stream, a, n, total, fx);
-    else {
-      if (first) DYHIP_CHECK_STATUS(dyhip_zero(dev, fx, total * sizeof(float)));
-      hipLaunchKernelGGL(sum_group_kernel<true>, grid, block, 0, dev->stream, a, n, total, fx);
+    for (unsigned i = used; i < 32; ++i) a.x[i] = nullptr;
+    for (unsigned g = a.ngroups; g < 8; ++g) a.cnt[g] = 0;
+    const bool one = a.ngroups == 1;
+    if (launch_first && same) {
+      if (one) hipLaunchKernelGGL((sum_group_kernel<false, true>), grid, block, 0, dev->stream, a, n, total, fx);
+      else hipLaunchKernelGGL((sum_group_kernel<false, false>), grid, block, 0, dev->stream, a, n, total, fx);
+    } else {
+      if (launch_first) DYHIP_CHECK_STATUS(dyhip_zero(dev, fx, total * sizeof(float)));
+      if (one) hipLaunchKernelGGL((sum_group_kernel<true, true>), grid, block, 0, dev->stream, a, n, total, fx);
+      else hipLaunchKernelGGL((sum_group_kernel<true, false>), grid, block, 0, dev->stream, a, n, total, fx);
     }
-    first = false;
-    at += cnt;
   }
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
