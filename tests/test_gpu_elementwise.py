@@ -138,7 +138,8 @@ def test_cmult_and_csum(dev, n, bd0, bd1):
         assert_close(gt.numpy(), want, GRAD_RTOL, "csum bwd %d" % i, floor=rms(dy) * np.sqrt(bd if bdi != bd else 1))
 
 
-@pytest.mark.parametrize("n,bd", [(64 * 1024, 64), (1024, 4096), (1027, 33), (3, 2), (5, 1), (4096, 7)])
+@pytest.mark.parametrize("n,bd", [(64 * 1024, 64), (1024, 4096), (1027, 33), (3, 2), (5, 1), (4096, 7), (1, 100000), (2, 777),
+                                  (255, 1000)])
 def test_sum_batches(dev, n, bd):
     rng = np.random.default_rng(31)
     x = f32(rng.standard_normal((bd, n)))
@@ -431,21 +432,21 @@ def test_layer_norm_invariances_at_full_size(dev):
     assert_close(y1.numpy(), y0.numpy(), 5e-5, "LN(x+2) == LN(x)", floor=1.0)
 
 
-@pytest.mark.parametrize("k", [1, 2, 4, 5, 7, 8, 11])
-def test_sum_node_bit_exact(dev, k):
+@pytest.mark.parametrize("k,n,bd", [(k, 1031, 6) for k in (1, 2, 4, 5, 7, 8, 11, 32, 33, 35, 36, 37, 128)] + [(35, 1, 128), (70, 1, 1)])
+def test_sum_node_bit_exact(dev, k, n, bd):
+    """Argument counts across one launch's capacity (eight groups, 32 arguments) and the group of `(k - 4) % 4`."""
     rng = np.random.default_rng(k)
-    n, bd = 1031, 6
     xs = [f32(rng.standard_normal((bd, n)) * 10.0 ** rng.integers(-2, 3)) for _ in range(k)]
     fx = dev.empty((bd, n))
     dev.sum_forward(n, bd, [dev.tensor(x) for x in xs], [bd] * k, fx)
     assert fx.numpy().tobytes() == orc.sum_forward(n, bd, xs, [bd] * k).tobytes()
 
 
-def test_sum_node_broadcast_and_backward(dev):
+@pytest.mark.parametrize("bds", [[5, 1, 5], [1, 5, 5, 1, 1, 5, 1, 5, 5, 1, 5], [5] + [1] * 40])
+def test_sum_node_broadcast_and_backward(dev, bds):
     rng = np.random.default_rng(3)
     n, bd = 300, 5
-    xs = [f32(rng.standard_normal((bd, n))), f32(rng.standard_normal((1, n))), f32(rng.standard_normal((bd, n)))]
-    bds = [bd, 1, bd]
+    xs = [f32(rng.standard_normal((b, n))) for b in bds]
     fx = dev.empty((bd, n))
     dev.sum_forward(n, bd, [dev.tensor(x) for x in xs], bds, fx)
     assert fx.numpy().tobytes() == orc.sum_forward(n, bd, xs, bds).tobytes()
