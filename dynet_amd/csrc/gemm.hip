@@ -566,21 +566,23 @@ __global__ __launch_bounds__(64 * kGemvWaves) void gemm_nn_thin_kernel(unsigned 
 
 // C = beta * C (or bias) + the slabs' sum, slabs in ascending order
 // GATES: C = act(bias + (forget rows: 1) + sum), the epilogue of the gates node (kEpiLstmGates)
+constexpr int kCombineFlight = 16;  // slabs a thread has in flight (8: +0.5 us at 16 slabs)
+constexpr unsigned kCombineThreads = 256;
 template <bool GATES>
 __global__ __launch_bounds__(256) void gemm_nn_thin_combine_kernel(unsigned M4, unsigned N, unsigned slabs,
                                                                    const float4* __restrict__ partial,
                                                                    float4* __restrict__ C, float beta,
                                                                    const float* __restrict__ bias, unsigned H,
                                                                    int logistic_mode) {
-  const size_t e = size_t(blockIdx.x) * 256 + threadIdx.x, total = size_t(M4) * N;
+  const size_t e = size_t(blockIdx.x) * blockDim.x + threadIdx.x, total = size_t(M4) * N;
   if (e >= total) return;
   float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (unsigned s0 = 0; s0 < slabs; s0 += 8) {  // eight slabs in flight, added in ascending order
-    float4 o[8];
+  for (unsigned s0 = 0; s0 < slabs; s0 += kCombineFlight) {  // slabs in flight together, added in ascending order
+    float4 o[kCombineFlight];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) o[u] = partial[size_t(min(s0 + u, slabs - 1)) * total + e];
+    for (int u = 0; u < kCombineFlight; ++u) o[u] = partial[size_t(min(s0 + u, slabs - 1)) * total + e];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < kCombineFlight; ++u) {
       if (s0 + u < slabs) {
         t.x += o[u].x; t.y += o[u].y; t.z += o[u].z; t.w += o[u].w;
       }
@@ -660,13 +662,201 @@ static int gemm_nn_thin_run(dyhip_device* dev, size_t M, size_t N, int nseg, con
   DYHIP_CHECK_LAUNCH();
   if (partial != nullptr) {
     const size_t total = size_t(M4) * N;
-    const dim3 g2(static_cast<unsigned>(cdiv<size_t>(total, 256)));
+    const dim3 g2(static_cast<unsigned>(cdiv<size_t>(total, kCombineThreads)));
     if (gates)
-      hipLaunchKernelGGL(gemm_nn_thin_combine_kernel<true>, g2, dim3(256), 0, dev->stream, M4, static_cast<unsigned>(N),
+      hipLaunchKernelGGL(gemm_nn_thin_combine_kernel<true>, g2, dim3(kCombineThreads), 0, dev->stream, M4, static_cast<unsigned>(N),
                          slabs, reinterpret_cast<const float4*>(partial), reinterpret_cast<float4*>(C), 0.f, bias, epi.H,
                          epi.logistic_mode);
     else
-      hipLaunchKernelGGL(gemm_nn_thin_combine_kernel<false>, g2, dim3(256), 0, dev->stream, M4, static_cast<unsigned>(N),
+      hipLaunchKernelGGL(gemm_nn_thin_combine_kernel<false>, g2, dim3(kCombineThreads), 0, dev->stream, M4, static_cast<unsigned>(N),
+                         slabs, reinterpret_cast<const float4*>(partial), reinterpret_cast<float4*>(C), beta, bias, 0u, 0);
+    DYHIP_CHECK_LAUNCH();
+  }
+  return DYHIP_OK;
+}
+
+
+// ---- C = beta * C (or bias) + A * B with 9..32 columns of B: the affine layers and the gates node of a small batch ---
+// Still memory work (the weights are read once, the batch is 16-32 sequences), but too many columns for one lane's
+// registers on the vector ALUs, so the sums run on the matrix cores.  A wavefront owns 128 rows: lane l feeds rows
+// 4(l % 32)..+3 by 128-bit loads (512-byte runs of a column of A) for four depth indices of the lower (l < 32) or upper
+// half of an 8-index group, and column l % 32 of B for the same indices; one v_mfma_f32_32x32x2_f32 per row component
+// pairs a depth index of each half.  The result lands with a lane's four rows in the four accumulators' same
+// register, so a column's 128 rows are stored as one 512-byte run.  The block's four wavefronts split its depth range
+// (combined through LDS), gridDim.y blocks split the depth further, and gemm_nn_thin_combine_kernel adds their slabs.
+constexpr int kMidWaves = 4;
+constexpr unsigned kMidBlocksPerCu = 2;  // eight wavefronts a block and one block a CU halves the slabs: -1.5 us at 4096 rows, +1 to +6 us elsewhere
+constexpr unsigned kMidSub = 256;             // depth indices of B staged in LDS at a time
+constexpr unsigned kMidPitch = kMidSub + 4;  // floats between B's columns in LDS
+template <bool BVEC>  // B's columns can be read by 128-bit loads (16-byte aligned, depths a multiple of four)
+__global__ __launch_bounds__(64 * kMidWaves) void gemm_nn_mid_kernel(unsigned M4, unsigned N, unsigned chunk, GemmSeg seg0,
+                                                                     GemmSeg seg1, unsigned slabs0, float* __restrict__ C,
+                                                                     float beta, const float* __restrict__ bias,
+                                                                     float* __restrict__ partial) {
+  // B's staged entries during the products, then the wavefronts' sums: 48 KB, so that two blocks fit a CU
+  __shared__ float4 red[kMidWaves - 1][16][64];
+  static_assert(sizeof(float) * 32 * kMidPitch <= sizeof(float4) * (kMidWaves - 1) * 16 * 64, "B's staging area fits");
+  float* bs = reinterpret_cast<float*>(&red[0][0][0]);
+  const bool second = blockIdx.y >= slabs0;
+  const float* __restrict__ A = second ? seg1.A : seg0.A;
+  const float* __restrict__ B = second ? seg1.B : seg0.B;
+  const size_t lda4 = (second ? seg1.lda : seg0.lda) / 4, ldb = second ? seg1.ldb : seg0.ldb;
+  const unsigned K = static_cast<unsigned>(second ? seg1.K : seg0.K);
+  const unsigned k0 = (second ? blockIdx.y - slabs0 : blockIdx.y) * chunk, k1 = min(K, k0 + chunk);
+  const unsigned lane = threadIdx.x & 63, w = threadIdx.x >> 6, l32 = lane & 31, hi = lane >> 5;
+  const unsigned m4 = blockIdx.x * 32 + l32;
+  const bool live = m4 < M4;
+  const float4* a4 = reinterpret_cast<const float4*>(A) + (live ? m4 : M4 - 1);
+  const bool ncol = l32 < N;
+  floatx16 acc[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[c][r] = 0.f;
+  // B's entries for up to kMidSub depth indices are staged in LDS by coalesced loads (a lane reading its own column
+  // of B from memory made every load 64 separate lines); a wavefront's first loads of A are issued before that.
+  // 16 depth indices a step: two groups of eight, lanes below 32 the first four of a group, the others the last four.
+  for (unsigned kc = k0; kc < k1; kc += kMidSub) {
+    const unsigned kend = min(kc + kMidSub, k1), len = kend - kc;
+    unsigned kb = kc + 16 * w;
+    bool have = kb < kend;
+    float4 a[2][4];
+    auto load_a = [&]() {
+#pragma unroll
+      for (int g = 0; g < 2; ++g)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) a[g][j] = ldg4<true>(a4 + size_t(min(kb + 8 * g + 4 * hi + j, k1 - 1)) * lda4);
+    };
+    if (have) load_a();
+    if (kc > k0) __syncthreads();  // the last range's readers are done
+    if (BVEC) {
+      const unsigned q4 = len / 4;  // kc and k1 are multiples of four
+      for (unsigned e = threadIdx.x; e < N * q4; e += 64 * kMidWaves) {
+        const unsigned n = e / q4, q = e - n * q4;
+        *reinterpret_cast<float4*>(bs + n * kMidPitch + 4 * q) = *reinterpret_cast<const float4*>(B + size_t(n) * ldb + kc + 4 * q);
+      }
+    } else {
+      for (unsigned e = threadIdx.x; e < N * len; e += 64 * kMidWaves) {
+        const unsigned n = e / len, k = e - n * len;
+        bs[n * kMidPitch + k] = B[size_t(n) * ldb + kc + k];
+      }
+    }
+    __syncthreads();
+    while (have) {
+      float b[2][4];
+#pragma unroll
+      for (int g = 0; g < 2; ++g) {
+        const unsigned off = kb - kc + 8 * g + 4 * hi;
+        const float4 t = *reinterpret_cast<const float4*>(bs + l32 * kMidPitch + off);
+        b[g][0] = ncol && kc + off < kend ? t.x : 0.f;
+        b[g][1] = ncol && kc + off + 1 < kend ? t.y : 0.f;
+        b[g][2] = ncol && kc + off + 2 < kend ? t.z : 0.f;
+        b[g][3] = ncol && kc + off + 3 < kend ? t.w : 0.f;
+      }
+#pragma unroll
+      for (int g = 0; g < 2; ++g)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(b[g][j], a[g][j].x, acc[0], 0, 0, 0);
+          acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(b[g][j], a[g][j].y, acc[1], 0, 0, 0);
+          acc[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(b[g][j], a[g][j].z, acc[2], 0, 0, 0);
+          acc[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(b[g][j], a[g][j].w, acc[3], 0, 0, 0);
+        }
+      kb += 16 * kMidWaves;
+      have = kb < kend;
+      if (have) load_a();
+    }
+  }
+  // acc[c][r] of lane l: row 4 * m4 + c, column 8 * (r / 4) + 4 * (l / 32) + r % 4
+  __syncthreads();  // B's entries have been read
+  if (w > 0) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) red[w - 1][r][lane] = make_float4(acc[0][r], acc[1][r], acc[2][r], acc[3][r]);
+  }
+  __syncthreads();
+  if (w != 0 || !live) return;
+  // the slab of partial sums, or the output itself when the depth was not split over blocks
+  float4* out = partial != nullptr ? reinterpret_cast<float4*>(partial) + size_t(blockIdx.y) * N * M4 + m4
+                                   : reinterpret_cast<float4*>(C) + m4;
+  float4 bb = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (partial == nullptr && bias != nullptr) bb = reinterpret_cast<const float4*>(bias)[m4];
+  const bool old = partial == nullptr && bias == nullptr && beta != 0.f;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const unsigned n = 8 * (r / 4) + 4 * hi + (r % 4);
+    if (n >= N) continue;
+    float4 t = make_float4(acc[0][r], acc[1][r], acc[2][r], acc[3][r]);
+#pragma unroll
+    for (int v = 0; v < kMidWaves - 1; ++v) {
+      const float4 o = red[v][r][lane];
+      t.x += o.x; t.y += o.y; t.z += o.z; t.w += o.w;
+    }
+    t.x += bb.x; t.y += bb.y; t.z += bb.z; t.w += bb.w;
+    float4* q = out + size_t(n) * M4;
+    if (old) {
+      const float4 o = *q;
+      t.x += beta * o.x; t.y += beta * o.y; t.z += beta * o.z; t.w += beta * o.w;
+    }
+    *q = t;
+  }
+}
+
+static bool gemm_nn_mid_eligible(const dyhip_device* dev, size_t M, size_t N, int nseg, const GemmSeg* segs,
+                                 const float* C, const GemmEpiParams& epi) {
+  if (!(epi.kind == kEpiAxpby || (epi.kind == kEpiBias && epi.bias != nullptr && aligned16(epi.bias)) ||
+        (epi.kind == kEpiLstmGates && epi.bias != nullptr)))
+    return false;
+  if (nseg < 1 || nseg > 2 || (nseg == 2 && epi.kind != kEpiLstmGates)) return false;
+  for (int q = 0; q < nseg; ++q)
+    if (segs[q].A == nullptr || segs[q].B == nullptr || segs[q].K < 16 || segs[q].K > 0x3FFFFFFFull || segs[q].lda % 4 != 0 ||
+        !aligned16(segs[q].A))
+      return false;
+  return N >= 9 && N <= 32 && M >= 128 && M % 4 == 0 && M / 4 <= 0x7FFFFFFFull && aligned16(C) && dev->gemm_ws != nullptr;
+}
+
+static int gemm_nn_mid_run(dyhip_device* dev, size_t M, size_t N, int nseg, const GemmSeg* segs, float* C,
+                           const GemmEpiParams& epi) {
+  const unsigned M4 = static_cast<unsigned>(M / 4), bx = cdiv<unsigned>(M4, 32);
+  const unsigned K0 = static_cast<unsigned>(segs[0].K), K1 = nseg > 1 ? static_cast<unsigned>(segs[1].K) : 0u;
+  const unsigned K = K0 + K1;
+  // depth slabs: enough blocks to fill the GPU, each with at least one 16-index step per wavefront
+  unsigned slabs = cdiv<unsigned>(kMidBlocksPerCu * dev->num_cus, bx);
+  const unsigned max_by_depth = cdiv<unsigned>(K, 16 * kMidWaves);
+  if (slabs > max_by_depth) slabs = max_by_depth;
+  if (slabs < 1) slabs = 1;
+  unsigned chunk = cdiv<unsigned>(K, slabs);
+  chunk = (chunk + 16 * kMidWaves - 1) / (16 * kMidWaves) * (16 * kMidWaves);  // whole steps for every wavefront
+  const unsigned slabs0 = cdiv<unsigned>(K0, chunk), slabs1 = K1 ? cdiv<unsigned>(K1, chunk) : 0u;
+  slabs = slabs0 + slabs1;
+  DYHIP_REQUIRE(slabs <= 65535, "small-batch product: depth %u needs too many slabs", K);
+  const bool gates = epi.kind == kEpiLstmGates;
+  float* partial = nullptr;
+  if (slabs > 1 || gates) {  // the gates epilogue lives in the second kernel
+    DYHIP_REQUIRE(dev->gemm_ws_bytes >= sizeof(float) * M * N * slabs, "small-batch product: workspace too small");
+    partial = static_cast<float*>(dev->gemm_ws);
+  }
+  const float beta = epi.kind == kEpiAxpby ? epi.beta : 0.f;
+  const float* bias = epi.kind == kEpiAxpby ? nullptr : epi.bias;
+  const GemmSeg s0 = segs[0], s1 = nseg > 1 ? segs[1] : segs[0];
+  bool bvec = true;
+  for (int q = 0; q < nseg; ++q) bvec = bvec && segs[q].K % 4 == 0 && segs[q].ldb % 4 == 0 && aligned16(segs[q].B);
+  const dim3 grid(bx, slabs), block(64 * kMidWaves);
+  if (bvec)
+    hipLaunchKernelGGL(gemm_nn_mid_kernel<true>, grid, block, 0, dev->stream, M4, static_cast<unsigned>(N), chunk, s0, s1,
+                       slabs0, C, beta, bias, partial);
+  else
+    hipLaunchKernelGGL(gemm_nn_mid_kernel<false>, grid, block, 0, dev->stream, M4, static_cast<unsigned>(N), chunk, s0, s1,
+                       slabs0, C, beta, bias, partial);
+  DYHIP_CHECK_LAUNCH();
+  if (partial != nullptr) {
+    const size_t total = size_t(M4) * N;
+    const dim3 g2(static_cast<unsigned>(cdiv<size_t>(total, kCombineThreads)));
+    if (gates)
+      hipLaunchKernelGGL(gemm_nn_thin_combine_kernel<true>, g2, dim3(kCombineThreads), 0, dev->stream, M4, static_cast<unsigned>(N),
+                         slabs, reinterpret_cast<const float4*>(partial), reinterpret_cast<float4*>(C), 0.f, bias, epi.H,
+                         epi.logistic_mode);
+    else
+      hipLaunchKernelGGL(gemm_nn_thin_combine_kernel<false>, g2, dim3(kCombineThreads), 0, dev->stream, M4, static_cast<unsigned>(N),
                          slabs, reinterpret_cast<const float4*>(partial), reinterpret_cast<float4*>(C), beta, bias, 0u, 0);
     DYHIP_CHECK_LAUNCH();
   }
@@ -715,6 +905,9 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
   if ((batch == nullptr || batch->count <= 1) && !a_kmajor && b_kmajor && C != nullptr &&
       gemm_nn_thin_eligible(dev, M, N, nseg, segs, C, epi))
     return gemm_nn_thin_run(dev, M, N, nseg, segs, C, epi);
+  if ((batch == nullptr || batch->count <= 1) && !a_kmajor && b_kmajor && C != nullptr &&
+      gemm_nn_mid_eligible(dev, M, N, nseg, segs, C, epi))
+    return gemm_nn_mid_run(dev, M, N, nseg, segs, C, epi);
   if (nseg == 1 && (batch == nullptr || batch->count <= 1) && !a_kmajor && !b_kmajor && epi.kind == kEpiAxpby &&
       segs[0].A != nullptr && segs[0].B != nullptr && C != nullptr &&
       gemm_nt_thin_eligible(M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, C, epi.beta))

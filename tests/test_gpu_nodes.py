@@ -146,6 +146,37 @@ def test_gemm_nn_thin(dev, M, N, K):
     assert_close(yt.numpy(), (bias[None, :] + ref64).astype(np.float32), FWD_RTOL, "thin affine", floor=np.sqrt(K))
 
 
+# l * r with 9..32 columns of r (a small batch's affine layers): rows in 128-row wavefront tiles on the matrix cores,
+# the depth split over a block's wavefronts and over blocks; depths that are not multiples of 4 or 16, rows that do not
+# fill the last tile, a column count of 32, and a depth long enough for hundreds of slabs.
+@pytest.mark.parametrize("M,N,K", [(4096, 20, 1024), (4096, 32, 2048), (132, 9, 16), (128, 9, 17), (2600, 20, 650),
+                                   (1000, 31, 1001), (10000, 16, 1024), (512, 20, 512), (256, 12, 50000), (1024, 20, 256)])
+def test_gemm_nn_mid(dev, M, N, K):
+    rng = np.random.default_rng(M + N + K)
+    y0 = f32(rng.standard_normal((N, M)))
+    l, r2, bias = f32(rng.standard_normal((K, M))), f32(rng.standard_normal((N, K))), f32(rng.standard_normal(M))
+    lt, rt, bt = dev.tensor(l), dev.tensor(r2), dev.tensor(bias)
+    ref64 = r2.astype(np.float64) @ l.astype(np.float64)
+    for beta in (1.0, 0.0, 0.5):
+        yt = dev.tensor(y0)
+        dev.gemm_nn(M, N, K, lt, rt, beta, yt)
+        assert_close(yt.numpy(), (beta * y0 + ref64).astype(np.float32), FWD_RTOL, "mid gemm_nn beta=%g" % beta,
+                     floor=np.sqrt(K))
+    again = dev.tensor(y0)
+    dev.gemm_nn(M, N, K, lt, rt, 0.5, again)
+    assert again.numpy().tobytes() == yt.numpy().tobytes()  # a fixed order of additions
+    yt = dev.tensor(y0)
+    dev.affine_forward(M, N, K, bt, lt, rt, yt)
+    assert_close(yt.numpy(), (bias[None, :] + ref64).astype(np.float32), FWD_RTOL, "mid affine", floor=np.sqrt(K))
+    # every entry of r matters once: a product with one-hot columns returns columns of l
+    hot = np.zeros((N, K), np.float32)
+    picks = rng.integers(0, K, N)
+    hot[np.arange(N), picks] = 1.0
+    yt = dev.empty((N, M))
+    dev.gemm_nn(M, N, K, lt, dev.tensor(hot), 0.0, yt)
+    assert yt.numpy().tobytes() == l[picks].tobytes()
+
+
 # Large outputs go to the 256 x 256-tile kernel, which deals the k-tiles of all tiles to the CUs in equal segments:
 # (a) fewer tiles than CUs: every tile spans several segments, whose partial tiles a second kernel adds; ragged edges
 # and a depth that is not a multiple of 32 (the rest of the depth is added by the 128-wide kernel); (b), (c) a little
@@ -443,6 +474,12 @@ def _lstm_case(rng, I, H, B):
     (200, 64, 3, None, False, True),
     (256, 512, 8, None, True, True),
     (96, 72, 2, [32, 64], False, True),
+    # 9..32 columns: the forward takes the small-batch product over both depth segments (weights above 4 MB, or
+    # sizes the fragment-order kernel does not take), 128-bit and one-by-one reads of x and h
+    (512, 768, 20, None, False, True),
+    (200, 64, 12, None, False, True),
+    (330, 200, 20, [130, 200], True, True),
+    (256, 256, 9, None, False, True),
 ])
 def test_lstm_cell_forward_backward(dev, I, H, B, dims, dropout, mask_full):
     rng = np.random.default_rng(I * 100 + H * 10 + B)
