@@ -549,6 +549,80 @@ __global__ __launch_bounds__(64 * kLnWavesFwd) void ln_fwd_wave_kernel(unsigned 
   }
 }
 
+// ---- rows of at most 256 floats: G lanes (4, 8 or 16) hold a row, a wavefront 64 / G rows at a time ---------------------
+// With a wavefront per row, rows of 64 floats use 16 of its lanes and one 128-bit load per lane (0.27 of the HBM peak
+// forward and backward; 0.08 at 16 floats).  The sums over a row stay inside a 16-lane DPP row: quad permutes, then
+// the half-row and row mirrors, after which every lane of the group holds the group's sum.
+template <int G>
+__device__ __forceinline__ float group_sum(float v) {
+  v += dpp_move<0xB1, 0xF>(v, 0.f);                // quad_perm [1,0,3,2]
+  v += dpp_move<0x4E, 0xF>(v, 0.f);                // quad_perm [2,3,0,1]
+  if (G >= 8) v += dpp_move<0x141, 0xF>(v, 0.f);   // row_half_mirror
+  if (G >= 16) v += dpp_move<0x140, 0xF>(v, 0.f);  // row_mirror
+  return v;
+}
+
+// RPG: rows a group takes, all fetched before the first is reduced (one 128-bit load a lane is too little in flight:
+// 64-float rows 7.6 us for 16 MB with one, against 6.0 us for 128-float rows with two)
+template <int G, int VPL, int RPG, bool NT>
+__global__ __launch_bounds__(64 * kLnWavesFwd) void ln_fwd_group_kernel(unsigned n4, unsigned bd,
+                                                                       const float4* __restrict__ x,
+                                                                       const float4* __restrict__ g,
+                                                                       const float4* __restrict__ b,
+                                                                       float4* __restrict__ y) {
+  constexpr unsigned R = 64 / G;
+  const unsigned lane = threadIdx.x & 63, gl = lane % G;
+  const unsigned row0 = (blockIdx.x * kLnWavesFwd + (threadIdx.x >> 6)) * (R * RPG) + lane / G;
+  const float fn = float(n4 * 4);
+  float4 v[RPG][VPL];
+#pragma unroll
+  for (int k = 0; k < RPG; ++k) {
+    const unsigned row = row0 + k * R;  // a group past the end works on the last row and stores nothing
+    const float4* px = x + size_t(row < bd ? row : bd - 1) * n4;
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+      const unsigned idx = gl + G * u;
+      v[k][u] = ldg4<NT>(px + (idx < n4 ? idx : n4 - 1));
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < RPG; ++k) {
+    const unsigned row = row0 + k * R;
+#pragma unroll
+    for (int u = 0; u < VPL; ++u)
+      if (!(gl + G * u < n4)) v[k][u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    float s = 0.f;
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) s += (v[k][u].x + v[k][u].y) + (v[k][u].z + v[k][u].w);
+    const float mean = group_sum<G>(s) / fn;
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+      if (gl + G * u < n4) {
+        const float dx = v[k][u].x - mean, dy = v[k][u].y - mean, dz = v[k][u].z - mean, dw = v[k][u].w - mean;
+        ss += (dx * dx + dy * dy) + (dz * dz + dw * dw);
+      }
+    }
+    const float sigma = sqrtf(group_sum<G>(ss) / fn);
+    const float sden = 1.0f / (kLnEps + sigma);
+    const float neg = -mean;
+    float4* py = y + size_t(row) * n4;
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+      const unsigned idx = gl + G * u;
+      if (row < bd && idx < n4) {
+        const float4 gg = g[idx], bb = b[idx];  // here, not ahead of the reductions: 6.0 against 7.3 us at 128-256 floats
+        float4 r;
+        r.x = gg.x * ((v[k][u].x + neg) * sden) + bb.x;
+        r.y = gg.y * ((v[k][u].y + neg) * sden) + bb.y;
+        r.z = gg.z * ((v[k][u].z + neg) * sden) + bb.z;
+        r.w = gg.w * ((v[k][u].w + neg) * sden) + bb.w;
+        stg4<NT>(py + idx, r);
+      }
+    }
+  }
+}
+
 // Rows of 2052..16384 floats: a team of WPT waves holds one row in registers (four float4 per thread) and
 // reduces through LDS, one barrier per reduction (each reduction has its own slots).
 constexpr int kLnTeamVpt = 4;
@@ -1049,6 +1123,173 @@ __global__ __launch_bounds__(64 * WAVES) void ln_bwd_wave_kernel(unsigned n4, un
   if (want_g || want_b) stage();
 }
 
+// Backward for rows of at most 256 floats, G lanes a row (see ln_fwd_group_kernel).  A wavefront walks 64 / G rows at a
+// time and fetches the next set before it reduces the current one; a group past the last row works on the last row
+// again and neither stores nor accumulates.  Its dg / db partial sums are first added across the groups that share a
+// 16-lane DPP row (row rotations), then across the block's 4 x WAVES DPP rows through LDS in ascending order.
+template <int VPL>
+struct LnGroupRow {
+  float4 v[VPL], d[VPL], o[VPL];
+};
+
+template <int G, int VPL, bool NT>
+__global__ __launch_bounds__(64 * kLnWavesBwd) void ln_bwd_group_kernel(unsigned n4, unsigned bd,
+                                                                       const float4* __restrict__ x,
+                                                                       const float4* __restrict__ g,
+                                                                       const float4* __restrict__ dEdf,
+                                                                       float4* __restrict__ dx,
+                                                                       float* __restrict__ part_dg,
+                                                                       float* __restrict__ part_db) {
+  extern __shared__ float lds[];  // [dg | db][wave * 4 + DPP row][n]
+  constexpr int WAVES = kLnWavesBwd;
+  constexpr unsigned R = 64 / G;
+  const unsigned lane = threadIdx.x & 63, w = threadIdx.x >> 6, gl = lane % G, q = lane / G;
+  const float fn = float(n4 * 4);
+  const bool want_g = part_dg != nullptr, want_b = part_db != nullptr;
+  float4 gg[VPL], pdg[VPL], pdb[VPL];
+#pragma unroll
+  for (int u = 0; u < VPL; ++u) {
+    const unsigned idx = gl + G * u;
+    gg[u] = idx < n4 ? g[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+    pdg[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    pdb[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  const unsigned stride = gridDim.x * WAVES * R;
+  const float4* dxr = dx != nullptr ? dx : x;  // without a dx the old values are fetched from x and not used
+  LnGroupRow<VPL> cur, nxt;
+  auto load = [&](LnGroupRow<VPL>& r, unsigned row) __attribute__((always_inline)) {
+    const size_t at = size_t(row < bd ? row : bd - 1) * n4;
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+      const unsigned idx = gl + G * u, ic = idx < n4 ? idx : n4 - 1;
+      r.v[u] = ldg4<NT>(x + at + ic);
+      r.d[u] = ldg4<NT>(dEdf + at + ic);
+      r.o[u] = ldg4<NT>(dxr + at + ic);
+    }
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+      if (!(gl + G * u < n4)) {
+        r.v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        r.d[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    }
+  };
+  auto process = [&](const LnGroupRow<VPL>& cur, unsigned row) __attribute__((always_inline)) {
+    const bool valid = row < bd;
+    float s = 0.f;
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) s += (cur.v[u].x + cur.v[u].y) + (cur.v[u].z + cur.v[u].w);
+    const float mean = group_sum<G>(s) / fn;
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+      if (gl + G * u < n4) {
+        const float ax = cur.v[u].x - mean, ay = cur.v[u].y - mean, az = cur.v[u].z - mean, aw = cur.v[u].w - mean;
+        ss += (ax * ax + ay * ay) + (az * az + aw * aw);
+      }
+    }
+    const float sigma = sqrtf(group_sum<G>(ss) / fn);
+    const float rs = 1.0f / (kLnEps + sigma);
+    const float neg = -mean;
+    float sxq = 0.f, sq = 0.f;
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+      if (gl + G * u < n4) {
+#define DYHIP_LN_ROW(c)                                                 \
+  {                                                                     \
+    const float xc = cur.v[u].c + neg;                                  \
+    const float dq = cur.d[u].c * gg[u].c;                              \
+    sxq = fmaf(dq, xc, sxq);                                            \
+    sq += dq;                                                           \
+    if (want_g && valid) pdg[u].c = fmaf(cur.d[u].c, xc * rs, pdg[u].c); \
+    if (want_b && valid) pdb[u].c += cur.d[u].c;                        \
+  }
+        DYHIP_F4_EACH(DYHIP_LN_ROW)
+#undef DYHIP_LN_ROW
+      }
+    }
+    if (dx != nullptr) {
+      const float ds = -(group_sum<G>(sxq) * rs) * rs;
+      const float dmu = -(group_sum<G>(sq) * rs);
+      const float sb = ds / (2.f * sigma);
+      const float c = 2.f / fn;
+      const float dmu_n = dmu / fn;
+      float4* pdx = dx + size_t(row) * n4;
+#pragma unroll
+      for (int u = 0; u < VPL; ++u) {
+        const unsigned idx = gl + G * u;
+        if (valid && idx < n4) {
+          float4 o = cur.o[u];
+#define DYHIP_LN_DX(c_)                     \
+  {                                         \
+    float acc = o.c_;                       \
+    acc += c * (cur.v[u].c_ - mean) * sb;   \
+    acc += (cur.d[u].c_ * gg[u].c_) * rs;   \
+    acc += dmu_n;                           \
+    o.c_ = acc;                             \
+  }
+          DYHIP_F4_EACH(DYHIP_LN_DX)
+#undef DYHIP_LN_DX
+          stg4<NT>(pdx + idx, o);
+        }
+      }
+    }
+  };
+  unsigned base = (blockIdx.x * WAVES + w) * R;  // the wavefront's first row: the same in every lane
+  if (base < bd) {
+    load(cur, base + q);
+    for (unsigned next = base + stride; next < bd; next += stride) {
+      load(nxt, next + q);
+      process(cur, base + q);
+      cur = nxt;
+      base = next;
+    }
+    process(cur, base + q);
+  }
+  if (!want_g && !want_b) return;
+  const unsigned n = n4 * 4;
+#pragma unroll
+  for (int u = 0; u < VPL; ++u) {
+#define DYHIP_LN_ACROSS(c)                                              \
+  {                                                                     \
+    if (G <= 8) {                                                       \
+      pdg[u].c += dpp_move<0x128, 0xF>(pdg[u].c, 0.f); /* row_ror:8 */  \
+      pdb[u].c += dpp_move<0x128, 0xF>(pdb[u].c, 0.f);                  \
+    }                                                                   \
+    if (G <= 4) {                                                       \
+      pdg[u].c += dpp_move<0x124, 0xF>(pdg[u].c, 0.f); /* row_ror:4 */  \
+      pdb[u].c += dpp_move<0x124, 0xF>(pdb[u].c, 0.f);                  \
+    }                                                                   \
+  }
+    DYHIP_F4_EACH(DYHIP_LN_ACROSS)
+#undef DYHIP_LN_ACROSS
+  }
+  const unsigned slot = w * 4 + lane / 16;
+#pragma unroll
+  for (int u = 0; u < VPL; ++u) {
+    const unsigned idx = gl + G * u;
+    if (lane % 16 < G && idx < n4) {
+      if (want_g) reinterpret_cast<float4*>(lds + size_t(slot) * n)[idx] = pdg[u];
+      if (want_b) reinterpret_cast<float4*>(lds + size_t(4 * WAVES + slot) * n)[idx] = pdb[u];
+    }
+  }
+  __syncthreads();
+  for (unsigned j4 = threadIdx.x; j4 < 2 * n4; j4 += 64 * WAVES) {
+    const unsigned which = j4 >= n4 ? 1u : 0u;
+    float* part = which == 0 ? part_dg : part_db;
+    if (part == nullptr) continue;
+    const unsigned c4 = j4 - which * n4;
+    const float4* src = reinterpret_cast<const float4*>(lds + size_t(which) * 4 * WAVES * n) + c4;
+    float4 t = src[0];
+#pragma unroll 8
+    for (int k = 1; k < 4 * WAVES; ++k) {
+      const float4 a = src[size_t(k) * n4];
+      t.x += a.x; t.y += a.y; t.z += a.z; t.w += a.w;
+    }
+    reinterpret_cast<float4*>(part + size_t(blockIdx.x) * n)[c4] = t;
+  }
+}
+
 // A partial row on its way to the combine kernel: streamed past the caches when the partial rows together are larger
 // than the L2s (they are written once and read once by other CUs); `nt` is the same for every thread.
 __device__ __forceinline__ void st_part(float4* p, const float4 v, int nt) {
@@ -1505,16 +1746,29 @@ int dyhip_layer_norm_forward(dyhip_device* dev, size_t n, unsigned bd, const flo
                  *b4 = reinterpret_cast<const float4*>(b);
     float4* y4 = reinterpret_cast<float4*>(y);
     const bool stream = n * size_t(bd) * sizeof(float) >= dev->stream_threshold;
+#define DYHIP_LN_FWD_GROUP(G, VPL, RPG)                                                                           \
+  do {                                                                                                            \
+    const dim3 gg(cdiv<unsigned>(bd, kLnWavesFwd * (64 / G) * RPG));                                              \
+    if (stream) hipLaunchKernelGGL((ln_fwd_group_kernel<G, VPL, RPG, true>), gg, block, 0, dev->stream, n4, bd, x4, g4, b4, y4); \
+    else hipLaunchKernelGGL((ln_fwd_group_kernel<G, VPL, RPG, false>), gg, block, 0, dev->stream, n4, bd, x4, g4, b4, y4);       \
+  } while (0)
 #define DYHIP_LN_FWD(VPL)                                                                                       \
   do {                                                                                                          \
     if (stream) hipLaunchKernelGGL((ln_fwd_wave_kernel<VPL, true>), grid, block, 0, dev->stream, n4, bd, x4, g4, b4, y4); \
     else hipLaunchKernelGGL((ln_fwd_wave_kernel<VPL, false>), grid, block, 0, dev->stream, n4, bd, x4, g4, b4, y4);       \
   } while (0)
-    if (n4 <= 64) DYHIP_LN_FWD(1);
+    // short rows: several rows a wavefront
+    if (n4 <= 4) DYHIP_LN_FWD_GROUP(4, 1, 2);
+    else if (n4 <= 8) DYHIP_LN_FWD_GROUP(8, 1, 2);
+    else if (n4 <= 16) DYHIP_LN_FWD_GROUP(16, 1, 2);
+    else if (n4 <= 32) DYHIP_LN_FWD_GROUP(16, 2, 2);
+    else if (n4 <= 48) DYHIP_LN_FWD_GROUP(16, 3, 1);
+    else if (n4 <= 64) DYHIP_LN_FWD_GROUP(16, 4, 1);
     else if (n4 <= 128) DYHIP_LN_FWD(2);
     else if (n4 <= 256) DYHIP_LN_FWD(4);
     else DYHIP_LN_FWD(8);
 #undef DYHIP_LN_FWD
+#undef DYHIP_LN_FWD_GROUP
   } else if (ln_team_ok(n, x, g, b, y)) {
     const unsigned n4 = static_cast<unsigned>(n / 4);
     const float4 *x4 = reinterpret_cast<const float4*>(x), *g4 = reinterpret_cast<const float4*>(g),
@@ -1605,9 +1859,9 @@ int dyhip_layer_norm_backward(dyhip_device* dev, size_t n, unsigned bd, const fl
   if (ln_fast_ok(n, x, g, dEdf, dx)) {
     const unsigned n4 = static_cast<unsigned>(n / 4);
     const unsigned waves = kLnWavesBwd;
-    const unsigned blocks = ln_bwd_blocks(n, bd);
+    unsigned blocks = ln_bwd_blocks(n, bd);
     float* part_dg = dg ? static_cast<float*>(ws) : nullptr;
-    float* part_db = db ? static_cast<float*>(ws) + size_t(blocks) * n : nullptr;
+    float* part_db = db ? static_cast<float*>(ws) + size_t(blocks) * n : nullptr;  // placed for the upper bound of the block count
     const size_t lds = cols ? size_t(2) * waves * n * sizeof(float) : 0;  // [dg | db][wave][n]
     const dim3 grid(blocks), block(64 * waves);
     const float4 *x4 = reinterpret_cast<const float4*>(x), *g4 = reinterpret_cast<const float4*>(g),
@@ -1640,11 +1894,29 @@ int dyhip_layer_norm_backward(dyhip_device* dev, size_t n, unsigned bd, const fl
     else if (full) DYHIP_LN_BWD_LAUNCH(VPL, false, kLnWavesBwd, true);                                     \
     else DYHIP_LN_BWD_LAUNCH(VPL, false, kLnWavesBwd, false);                                              \
   } while (0)
-    if (n4 <= 64) DYHIP_LN_BWD(1);
+// short rows: several rows a wavefront; never more blocks than the workspace was sized for
+#define DYHIP_LN_BWD_GROUP(G, VPL)                                                                          \
+  do {                                                                                                      \
+    const unsigned per_block = kLnWavesBwd * (64 / G);                                                      \
+    if (cdiv<unsigned>(bd, per_block) < blocks) blocks = cdiv<unsigned>(bd, per_block);                     \
+    const size_t glds = cols ? size_t(2) * 4 * kLnWavesBwd * n * sizeof(float) : 0;                         \
+    if (stream)                                                                                             \
+      hipLaunchKernelGGL((ln_bwd_group_kernel<G, VPL, true>), dim3(blocks), block, glds, dev->stream, n4, bd, x4, g4, \
+                         d4, dx4, part_dg, part_db);                                                        \
+    else                                                                                                    \
+      hipLaunchKernelGGL((ln_bwd_group_kernel<G, VPL, false>), dim3(blocks), block, glds, dev->stream, n4, bd, x4, g4, \
+                         d4, dx4, part_dg, part_db);                                                        \
+  } while (0)
+    if (n4 <= 4) DYHIP_LN_BWD_GROUP(4, 1);
+    else if (n4 <= 8) DYHIP_LN_BWD_GROUP(8, 1);
+    else if (n4 <= 16) DYHIP_LN_BWD_GROUP(16, 1);
+    else if (n4 <= 32) DYHIP_LN_BWD_GROUP(16, 2);
+    else if (n4 <= 64) DYHIP_LN_BWD(1);
     else if (n4 <= 128) DYHIP_LN_BWD(2);
     else if (n4 <= 256) DYHIP_LN_BWD(4);
     else DYHIP_LN_BWD(8);
 #undef DYHIP_LN_BWD
+#undef DYHIP_LN_BWD_GROUP
 #undef DYHIP_LN_BWD_LAUNCH
 #undef DYHIP_LN_BWD_LDS
     DYHIP_CHECK_LAUNCH();

@@ -234,7 +234,12 @@ def _ln_fp64(x, g, b, dy):
                                   # rows that are not a multiple of four floats: one float per lane and step up to
                                   # 1024 (backward) / 2048 (forward) floats, the block-per-row kernels beyond
                                   (650, 3000), (1001, 20), (250, 100), (50, 9), (65, 130), (1022, 5), (1026, 3),
-                                  (2046, 3), (2050, 2)])
+                                  (2046, 3), (2050, 2),
+                                  # rows of up to 256 floats: 4, 8 or 16 lanes a row, several rows a wavefront; row
+                                  # counts that leave groups of the last wavefront without a row, and enough rows
+                                  # for several sweeps of every wavefront
+                                  (4, 3), (8, 40000), (16, 100001), (20, 77), (32, 65537), (64, 70001), (100, 4099),
+                                  (128, 33000), (132, 129), (192, 3001), (256, 20000)])
 def test_layer_norm_forward_backward(dev, n, bd):
     rng, x, g, b, dy = _ln_case(n, bd, 51)
     xt, gt, bt, dyt = dev.tensor(x), dev.tensor(g), dev.tensor(b), dev.tensor(dy)
