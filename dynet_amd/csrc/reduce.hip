@@ -559,6 +559,8 @@ __device__ __forceinline__ float group_sum(float v) {
   v += dpp_move<0x4E, 0xF>(v, 0.f);                // quad_perm [2,3,0,1]
   if (G >= 8) v += dpp_move<0x141, 0xF>(v, 0.f);   // row_half_mirror
   if (G >= 16) v += dpp_move<0x140, 0xF>(v, 0.f);  // row_mirror
+  if (G >= 32) v += __shfl_xor(v, 16);             // the other DPP row of the half
+  if (G >= 64) v += __shfl_xor(v, 32);
   return v;
 }
 
@@ -1290,6 +1292,195 @@ __global__ __launch_bounds__(64 * kLnWavesBwd) void ln_bwd_group_kernel(unsigned
   }
 }
 
+// ---- the same for short rows that cannot take 128-bit accesses (n % 4 != 0 or a pointer off a 16-byte boundary):
+// lane l of a group owns elements l, l + G, ...; a group's access is one contiguous run ------------------------------
+template <int G, int VS, int RPG, bool NT>
+__global__ __launch_bounds__(64 * kLnWavesFwd) void ln_fwd_group1_kernel(unsigned n, unsigned bd, const float* __restrict__ x,
+                                                                        const float* __restrict__ g,
+                                                                        const float* __restrict__ b, float* __restrict__ y) {
+  constexpr unsigned R = 64 / G;
+  const unsigned lane = threadIdx.x & 63, gl = lane % G;
+  const unsigned row0 = (blockIdx.x * kLnWavesFwd + (threadIdx.x >> 6)) * (R * RPG) + lane / G;
+  const float fn = float(n);
+  float v[RPG][VS];
+#pragma unroll
+  for (int k = 0; k < RPG; ++k) {
+    const unsigned row = row0 + k * R;
+    const float* px = x + size_t(row < bd ? row : bd - 1) * n;
+#pragma unroll
+    for (int u = 0; u < VS; ++u) {
+      const unsigned idx = gl + G * u;
+      v[k][u] = ldg1<NT>(px + (idx < n ? idx : n - 1));
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < RPG; ++k) {
+    const unsigned row = row0 + k * R;
+    float s = 0.f;
+#pragma unroll
+    for (int u = 0; u < VS; ++u)
+      if (gl + G * u < n) s += v[k][u];
+    const float mean = group_sum<G>(s) / fn;
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < VS; ++u) {
+      if (gl + G * u < n) {
+        const float d = v[k][u] - mean;
+        ss += d * d;
+      }
+    }
+    const float sigma = sqrtf(group_sum<G>(ss) / fn);
+    const float sden = 1.0f / (kLnEps + sigma);
+    const float neg = -mean;
+    float* py = y + size_t(row) * n;
+#pragma unroll
+    for (int u = 0; u < VS; ++u) {
+      const unsigned idx = gl + G * u;
+      if (row < bd && idx < n) stg1<NT>(py + idx, g[idx] * ((v[k][u] + neg) * sden) + b[idx]);
+    }
+  }
+}
+
+template <int VS>
+struct LnGroupRow1 {
+  float v[VS], d[VS], o[VS];
+};
+
+template <int G, int VS, bool NT>
+__global__ __launch_bounds__(64 * kLnWavesBwd) void ln_bwd_group1_kernel(unsigned n, unsigned bd, const float* __restrict__ x,
+                                                                        const float* __restrict__ g,
+                                                                        const float* __restrict__ dEdf, float* __restrict__ dx,
+                                                                        float* __restrict__ part_dg,
+                                                                        float* __restrict__ part_db) {
+  extern __shared__ float lds[];  // [dg | db][wave * RL + group (G >= 16) or DPP row][n]
+  constexpr int WAVES = kLnWavesBwd;
+  constexpr unsigned R = 64 / G, RL = G >= 16 ? R : 4;  // partial rows a wavefront leaves in LDS
+  const unsigned lane = threadIdx.x & 63, w = threadIdx.x >> 6, gl = lane % G, q = lane / G;
+  const float fn = float(n);
+  const bool want_g = part_dg != nullptr, want_b = part_db != nullptr;
+  float gg[VS], pdg[VS], pdb[VS];
+#pragma unroll
+  for (int u = 0; u < VS; ++u) {
+    const unsigned idx = gl + G * u;
+    gg[u] = idx < n ? g[idx] : 0.f;
+    pdg[u] = 0.f;
+    pdb[u] = 0.f;
+  }
+  const unsigned stride = gridDim.x * WAVES * R;
+  const float* dxr = dx != nullptr ? dx : x;
+  LnGroupRow1<VS> cur, nxt;
+  auto load = [&](LnGroupRow1<VS>& r, unsigned row) __attribute__((always_inline)) {
+    const size_t at = size_t(row < bd ? row : bd - 1) * n;
+#pragma unroll
+    for (int u = 0; u < VS; ++u) {
+      const unsigned idx = gl + G * u, ic = idx < n ? idx : n - 1;
+      r.v[u] = ldg1<NT>(x + at + ic);
+      r.d[u] = ldg1<NT>(dEdf + at + ic);
+      r.o[u] = ldg1<NT>(dxr + at + ic);
+    }
+#pragma unroll
+    for (int u = 0; u < VS; ++u) {
+      if (!(gl + G * u < n)) {
+        r.v[u] = 0.f;
+        r.d[u] = 0.f;
+      }
+    }
+  };
+  auto process = [&](const LnGroupRow1<VS>& cur, unsigned row) __attribute__((always_inline)) {
+    const bool valid = row < bd;
+    float s = 0.f;
+#pragma unroll
+    for (int u = 0; u < VS; ++u) s += cur.v[u];
+    const float mean = group_sum<G>(s) / fn;
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < VS; ++u) {
+      if (gl + G * u < n) {
+        const float a = cur.v[u] - mean;
+        ss += a * a;
+      }
+    }
+    const float sigma = sqrtf(group_sum<G>(ss) / fn);
+    const float rs = 1.0f / (kLnEps + sigma);
+    const float neg = -mean;
+    float sxq = 0.f, sq = 0.f;
+#pragma unroll
+    for (int u = 0; u < VS; ++u) {
+      if (gl + G * u < n) {
+        const float xc = cur.v[u] + neg;
+        const float dq = cur.d[u] * gg[u];
+        sxq = fmaf(dq, xc, sxq);
+        sq += dq;
+        if (want_g && valid) pdg[u] = fmaf(cur.d[u], xc * rs, pdg[u]);
+        if (want_b && valid) pdb[u] += cur.d[u];
+      }
+    }
+    if (dx != nullptr) {
+      const float ds = -(group_sum<G>(sxq) * rs) * rs;
+      const float dmu = -(group_sum<G>(sq) * rs);
+      const float sb = ds / (2.f * sigma);
+      const float c = 2.f / fn;
+      const float dmu_n = dmu / fn;
+      float* pdx = dx + size_t(row) * n;
+#pragma unroll
+      for (int u = 0; u < VS; ++u) {
+        const unsigned idx = gl + G * u;
+        if (valid && idx < n) {
+          float acc = cur.o[u];
+          acc += c * (cur.v[u] - mean) * sb;
+          acc += (cur.d[u] * gg[u]) * rs;
+          acc += dmu_n;
+          stg1<NT>(pdx + idx, acc);
+        }
+      }
+    }
+  };
+  unsigned base = (blockIdx.x * WAVES + w) * R;
+  if (base < bd) {
+    load(cur, base + q);
+    for (unsigned next = base + stride; next < bd; next += stride) {
+      load(nxt, next + q);
+      process(cur, base + q);
+      cur = nxt;
+      base = next;
+    }
+    process(cur, base + q);
+  }
+  if (!want_g && !want_b) return;
+#pragma unroll
+  for (int u = 0; u < VS; ++u) {
+    if (G <= 8) {
+      pdg[u] += dpp_move<0x128, 0xF>(pdg[u], 0.f);  // row_ror:8
+      pdb[u] += dpp_move<0x128, 0xF>(pdb[u], 0.f);
+    }
+    if (G <= 4) {
+      pdg[u] += dpp_move<0x124, 0xF>(pdg[u], 0.f);  // row_ror:4
+      pdb[u] += dpp_move<0x124, 0xF>(pdb[u], 0.f);
+    }
+  }
+  const unsigned slot = w * RL + (G >= 16 ? q : lane / 16);
+#pragma unroll
+  for (int u = 0; u < VS; ++u) {
+    const unsigned idx = gl + G * u;
+    if ((G >= 16 || lane % 16 < G) && idx < n) {
+      if (want_g) lds[size_t(slot) * n + idx] = pdg[u];
+      if (want_b) lds[size_t(RL * WAVES + slot) * n + idx] = pdb[u];
+    }
+  }
+  __syncthreads();
+  for (unsigned j = threadIdx.x; j < 2 * n; j += 64 * WAVES) {
+    const unsigned which = j >= n ? 1u : 0u;
+    float* part = which == 0 ? part_dg : part_db;
+    if (part == nullptr) continue;
+    const unsigned c = j - which * n;
+    const float* src = lds + size_t(which) * RL * WAVES * n + c;
+    float t = src[0];
+#pragma unroll 8
+    for (int k = 1; k < int(RL) * WAVES; ++k) t += src[size_t(k) * n];
+    part[size_t(blockIdx.x) * n + c] = t;
+  }
+}
+
 // A partial row on its way to the combine kernel: streamed past the caches when the partial rows together are larger
 // than the L2s (they are written once and read once by other CUs); `nt` is the same for every thread.
 __device__ __forceinline__ void st_part(float4* p, const float4 v, int nt) {
@@ -1791,18 +1982,31 @@ int dyhip_layer_norm_forward(dyhip_device* dev, size_t n, unsigned bd, const flo
     const unsigned nn = static_cast<unsigned>(n);
     const dim3 grid(cdiv<unsigned>(bd, kLnWavesFwd)), block(64 * kLnWavesFwd);
     const bool stream = n * size_t(bd) * sizeof(float) >= dev->stream_threshold;
+#define DYHIP_LN_FWD_GROUP(G, VS, RPG)                                                                            \
+  do {                                                                                                            \
+    const dim3 gg(cdiv<unsigned>(bd, kLnWavesFwd * (64 / G) * RPG));                                              \
+    if (stream) hipLaunchKernelGGL((ln_fwd_group1_kernel<G, VS, RPG, true>), gg, block, 0, dev->stream, nn, bd, x, g, b, y); \
+    else hipLaunchKernelGGL((ln_fwd_group1_kernel<G, VS, RPG, false>), gg, block, 0, dev->stream, nn, bd, x, g, b, y);       \
+  } while (0)
 #define DYHIP_LN_FWD(VS)                                                                                          \
   do {                                                                                                            \
     if (stream) hipLaunchKernelGGL((ln_fwd_lane_kernel<VS, true>), grid, block, 0, dev->stream, nn, bd, x, g, b, y); \
     else hipLaunchKernelGGL((ln_fwd_lane_kernel<VS, false>), grid, block, 0, dev->stream, nn, bd, x, g, b, y);       \
   } while (0)
-    if (nn <= 64) DYHIP_LN_FWD(1);
-    else if (nn <= 128) DYHIP_LN_FWD(2);
-    else if (nn <= 256) DYHIP_LN_FWD(4);
+    // short rows: several rows a wavefront
+    // short rows: as many lanes a row as reach its end (a group's access is then one run), several rows a wavefront
+    if (nn <= 4) DYHIP_LN_FWD_GROUP(4, 1, 4);
+    else if (nn <= 8) DYHIP_LN_FWD_GROUP(8, 1, 4);
+    else if (nn <= 16) DYHIP_LN_FWD_GROUP(16, 1, 4);
+    else if (nn <= 32) DYHIP_LN_FWD_GROUP(32, 1, 4);
+    else if (nn <= 64) DYHIP_LN_FWD_GROUP(64, 1, 4);
+    else if (nn <= 128) DYHIP_LN_FWD_GROUP(64, 2, 2);
+    else if (nn <= 192) DYHIP_LN_FWD_GROUP(64, 3, 2);  // 150 floats: 11.9 -> 10.6 us; 250 floats gain nothing from a second row
     else if (nn <= 512) DYHIP_LN_FWD(8);
     else if (nn <= 1024) DYHIP_LN_FWD(16);
     else DYHIP_LN_FWD(32);
 #undef DYHIP_LN_FWD
+#undef DYHIP_LN_FWD_GROUP
   } else {
     if (n <= 4096) hipLaunchKernelGGL(ln_fwd_block_kernel<256>, dim3(bd), dim3(256), 0, dev->stream, n, x, g, b, y);
     else hipLaunchKernelGGL(ln_fwd_block_kernel<1024>, dim3(bd), dim3(1024), 0, dev->stream, n, x, g, b, y);
@@ -1968,9 +2172,9 @@ int dyhip_layer_norm_backward(dyhip_device* dev, size_t n, unsigned bd, const fl
     DYHIP_CHECK_LAUNCH();
   } else if (n <= 1024) {
     const unsigned nn = static_cast<unsigned>(n);
-    const unsigned blocks = ln_bwd_blocks(n, bd);
+    unsigned blocks = ln_bwd_blocks(n, bd);
     float* part_dg = dg ? static_cast<float*>(ws) : nullptr;
-    float* part_db = db ? static_cast<float*>(ws) + size_t(blocks) * n : nullptr;
+    float* part_db = db ? static_cast<float*>(ws) + size_t(blocks) * n : nullptr;  // placed for the upper bound of the block count
     const size_t lds = cols ? size_t(2) * kLnWavesBwd * n * sizeof(float) : 0;  // [dg | db][wave][n], <= 128 KB
     const dim3 grid(blocks), block(64 * kLnWavesBwd);
     const bool stream = n * size_t(bd) * sizeof(float) >= dev->stream_threshold;
@@ -1992,12 +2196,30 @@ int dyhip_layer_norm_backward(dyhip_device* dev, size_t n, unsigned bd, const fl
       hipLaunchKernelGGL((ln_bwd_lane_kernel<VS, false, true>), grid, block, lds, dev->stream, nn, bd, x, g, dEdf, \
                          dx, part_dg, part_db);                                                                     \
   } while (0)
-    if (nn <= 64) DYHIP_LN_BWD(1);
+// short rows: several rows a wavefront; never more blocks than the workspace was sized for
+#define DYHIP_LN_BWD_GROUP(G, VS)                                                                                   \
+  do {                                                                                                              \
+    const unsigned per_block = kLnWavesBwd * (64 / G);                                                              \
+    if (cdiv<unsigned>(bd, per_block) < blocks) blocks = cdiv<unsigned>(bd, per_block);                             \
+    const size_t glds = cols ? size_t(2) * (G >= 16 ? 64 / G : 4) * kLnWavesBwd * n * sizeof(float) : 0;            \
+    if (stream)                                                                                                     \
+      hipLaunchKernelGGL((ln_bwd_group1_kernel<G, VS, true>), dim3(blocks), block, glds, dev->stream, nn, bd, x, g, dEdf, \
+                         dx, part_dg, part_db);                                                                     \
+    else                                                                                                            \
+      hipLaunchKernelGGL((ln_bwd_group1_kernel<G, VS, false>), dim3(blocks), block, glds, dev->stream, nn, bd, x, g, dEdf, \
+                         dx, part_dg, part_db);                                                                     \
+  } while (0)
+    if (nn <= 4) DYHIP_LN_BWD_GROUP(4, 1);
+    else if (nn <= 8) DYHIP_LN_BWD_GROUP(8, 1);
+    else if (nn <= 16) DYHIP_LN_BWD_GROUP(16, 1);
+    else if (nn <= 32) DYHIP_LN_BWD_GROUP(16, 2);  // 30 floats: 20.9 us, against 25.0 us with 32 lanes a row
+    else if (nn <= 64) DYHIP_LN_BWD_GROUP(32, 2);  // 50 floats: 21.0 us, against 28.0 us with 16 lanes a row
     else if (nn <= 128) DYHIP_LN_BWD(2);
     else if (nn <= 256) DYHIP_LN_BWD(4);
     else if (nn <= 512) DYHIP_LN_BWD(8);
     else DYHIP_LN_BWD(16);
 #undef DYHIP_LN_BWD
+#undef DYHIP_LN_BWD_GROUP
     DYHIP_CHECK_LAUNCH();
     if (dg && db) launch_combine(dev, n, blocks, part_dg, dg, part_db, db, 1);
     else if (dg) launch_combine(dev, n, blocks, part_dg, dg, nullptr, nullptr, 1);

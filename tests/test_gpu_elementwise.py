@@ -239,7 +239,10 @@ def _ln_fp64(x, g, b, dy):
                                   # counts that leave groups of the last wavefront without a row, and enough rows
                                   # for several sweeps of every wavefront
                                   (4, 3), (8, 40000), (16, 100001), (20, 77), (32, 65537), (64, 70001), (100, 4099),
-                                  (128, 33000), (132, 129), (192, 3001), (256, 20000)])
+                                  (128, 33000), (132, 129), (192, 3001), (256, 20000),
+                                  # the same with rows that cannot take 128-bit accesses
+                                  (3, 1000), (5, 100003), (7, 1000), (10, 50001), (30, 20001), (50, 30000), (70, 10001),
+                                  (150, 3000), (250, 5001)])
 def test_layer_norm_forward_backward(dev, n, bd):
     rng, x, g, b, dy = _ln_case(n, bd, 51)
     xt, gt, bt, dyt = dev.tensor(x), dev.tensor(g), dev.tensor(b), dev.tensor(dy)
