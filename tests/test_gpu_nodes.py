@@ -125,8 +125,11 @@ def test_gemm_tn_thin(dev, M, N, K):
 
 # l * r with at most 8 columns of r (matrix times vector: the un-batched graph's affine layers and projections): the
 # depth split into slabs over blocks, their partial sums added by a second kernel with the epilogue (beta or bias).
+# From 1024 rows on (and a depth of at most 4096 whose share of r fits LDS) one launch: a block owns 32 rows and the
+# whole depth; rows that do not fill the last block, a depth that is not a multiple of eight, r at the LDS limit.
 @pytest.mark.parametrize("M,N,K", [(4096, 1, 1024), (10000, 1, 1024), (1024, 3, 1000), (256, 8, 37), (6000, 5, 1500),
-                                   (260, 2, 8), (4096, 4, 2048), (512, 1, 20000)])
+                                   (260, 2, 8), (4096, 4, 2048), (512, 1, 20000), (1028, 2, 77), (2052, 7, 1535), (2052, 7, 2047),
+                                   (1024, 8, 1536), (1024, 8, 2048), (1024, 4, 4096), (1024, 1, 4100), (3000, 1, 5)])
 def test_gemm_nn_thin(dev, M, N, K):
     rng = np.random.default_rng(M + N + K)
     y0 = f32(rng.standard_normal((N, M)))
