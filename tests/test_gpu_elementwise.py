@@ -274,6 +274,38 @@ def test_layer_norm_forward_backward(dev, n, bd):
     assert dgt2.numpy().tobytes() == dgt.numpy().tobytes()
 
 
+def test_layer_norm_random_short_rows(dev):
+    """Seeded random row widths of 4..400 floats and row counts of 1..6000, half of them on tensors that start 4 bytes
+    past a 16-byte boundary: every several-rows-a-wavefront kernel (4, 8, 16, 32 lanes a row, with and without 128-bit
+    accesses) and the one-wavefront-per-row kernels above them, against the oracle."""
+    rng0 = np.random.default_rng(404)
+    for it in range(36):
+        n = int(rng0.choice([int(rng0.integers(4, 70)), 4 * int(rng0.integers(1, 70)), int(rng0.integers(70, 400))]))
+        bd = int(rng0.choice([int(rng0.integers(1, 40)), int(rng0.integers(40, 6000))]))
+        shift = int(rng0.integers(0, 2))
+        rng, x, g, b, dy = _ln_case(n, bd, 1000 + it)
+        def put(a):
+            base = dev.empty(a.size + shift)
+            t = base.offset(shift, a.shape)
+            t.set(a)
+            return t
+        what = "n=%d bd=%d shift=%d" % (n, bd, shift)
+        xo, go, bo, dyo = put(x), put(g), put(b), put(dy)
+        yo = put(np.zeros((bd, n), np.float32))
+        dev.layer_norm_forward(n, bd, xo, go, bo, yo)
+        assert_close(yo.numpy(), orc.layer_norm_forward(n, bd, x, g, b), FWD_RTOL, "layer_norm fwd " + what, floor=1.0)
+        dx0, dg0, db0 = f32(rng.standard_normal((bd, n))), f32(rng.standard_normal(n)), f32(rng.standard_normal(n))
+        dxo, dgo, dbo = put(dx0), put(dg0), put(db0)
+        dev.layer_norm_backward(n, bd, xo, go, dyo, dxo, dgo, dbo)
+        wx, wg, wb = orc.layer_norm_backward(n, bd, x, g, dy, dx0.copy(), dg0.copy(), db0.copy())
+        assert_close(dxo.numpy(), wx, GRAD_RTOL, "layer_norm dx " + what, floor=1.0)
+        assert_close(dgo.numpy(), wg, GRAD_RTOL, "layer_norm dg " + what, floor=np.sqrt(bd))
+        assert_close(dbo.numpy(), wb, GRAD_RTOL, "layer_norm db " + what, floor=np.sqrt(bd))
+        for w in (lib.POOL_FXS, lib.POOL_DEDFS, lib.POOL_SCS):
+            dev.sync()
+            dev.free_pool(w)
+
+
 def test_layer_norm_on_pointers_off_a_16_byte_boundary(dev):
     """Rows of a multiple of four floats whose tensors start 4 bytes past a 16-byte boundary: no 128-bit accesses, the
     one-float-per-lane kernels (a lane then owns other elements of a row, so the row sums round differently: the

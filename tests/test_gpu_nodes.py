@@ -269,6 +269,44 @@ def test_gemm_wide_tiles_random_shapes(dev):
     assert taken == {1, 2}
 
 
+def test_gemm_small_batch_random_shapes(dev):
+    """Seeded random products with 1..40 columns on one side: the matrix-times-vector kernels (slab and one-launch
+    forms), the 9..32-column matrix-core kernel, the rank-K update and the streamed transposed product, and the
+    general kernels where a size is off their grid (row counts that are not a multiple of four, depths down to 1,
+    operands that start off a 16-byte boundary).  All three forms against the fp64 product of the same inputs."""
+    rng = np.random.default_rng(77)
+    for it in range(40):
+        M = int(rng.choice([int(rng.integers(1, 300)), 4 * int(rng.integers(32, 1200)), int(rng.integers(300, 5000))]))
+        N = int(rng.integers(1, 41))
+        K = int(rng.choice([int(rng.integers(1, 64)), int(rng.integers(64, 3000)), 4 * int(rng.integers(16, 600))]))
+        off = int(rng.choice([0, 0, 1, 4]))  # floats before each operand's first element
+        l, r = f32(rng.standard_normal(K * M + off)), f32(rng.standard_normal(N * K + off))
+        y0 = f32(rng.standard_normal((N, M)))
+        lm, rm = l[off:].reshape(K, M), r[off:].reshape(N, K)
+        exact = rm.astype(np.float64) @ lm.astype(np.float64)
+        what = "M=%d N=%d K=%d offset %d" % (M, N, K, off)
+        lt, rt = dev.tensor(l).offset(off, (K, M)), dev.tensor(r).offset(off, (N, K))
+        for beta in (0.0, 1.0):
+            yt = dev.tensor(y0)
+            dev.gemm_nn(M, N, K, lt, rt, beta, yt)
+            assert_close(yt.numpy(), beta * y0 + exact, FWD_RTOL, "gemm_nn " + what, floor=np.sqrt(K))
+        lT = np.concatenate([l[:off], f32(lm.T).ravel()])
+        rT = np.concatenate([r[:off], f32(rm.T).ravel()])
+        yt = dev.tensor(y0)
+        dev.gemm_nt(M, N, K, lt, dev.tensor(rT).offset(off, (K, N)), 1.0, yt)
+        assert_close(yt.numpy(), y0 + exact, FWD_RTOL, "gemm_nt " + what, floor=np.sqrt(K))
+        yt = dev.tensor(y0)
+        dev.gemm_tn(M, N, K, dev.tensor(lT).offset(off, (M, K)), rt, 1.0, yt)
+        assert_close(yt.numpy(), y0 + exact, FWD_RTOL, "gemm_tn " + what, floor=np.sqrt(K))
+        # the roles swapped: a wide right operand against a thin left one
+        yt = dev.zeros((M, N))
+        dev.gemm_nn(N, M, K, dev.tensor(f32(rm.T)), dev.tensor(f32(lm.T)), 0.0, yt)
+        assert_close(yt.numpy(), exact.T, FWD_RTOL, "gemm_nn swapped " + what, floor=np.sqrt(K))
+        for w in lib_pools():
+            dev.sync()
+            dev.free_pool(w)
+
+
 def test_gemm_wide_give_up_is_reported_by_every_synchronising_call_and_leaves_clean_flags():
     """The error path of the hand-off between blocks, forced from the host: producers store their partial tiles but
     leave their flags down and the consumers' bounded wait is set to zero polls, so every cut tile's consumer gives
