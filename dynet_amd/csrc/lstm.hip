@@ -925,6 +925,151 @@ __global__ __launch_bounds__(256) void gemm_tn_thin_kernel(unsigned M, unsigned 
   }
 }
 
+// ---- C[M x N] = beta * C + A^T B for 5..32 columns of B on the matrix cores, the operands as they lie ---------------
+// A's columns (the depth contiguous) are fetched by coalesced 128-bit loads, 32 depth indices of 32 columns a
+// wavefront at a time (128-byte runs), and turned into matrix-core fragments through a wavefront's own LDS tile:
+// lane l reads column l % 32 at four depth indices of the lower or upper half of an 8-index group.  B's columns the
+// same way.  A block's four wavefronts take a quarter of its depth range each (tiles added through LDS), blocks split
+// the depth further and slices_accumulate_kernel adds their slices.  The fragment-order kernel reads A in 32-byte
+// pieces and wants depths that are multiples of 128 (1024 x 20 x 4096: 10.7 us, here 9.1; 384 x 32 x 1536: 10.6 us,
+// here 6.2); the streaming kernel above fetches all of B once per four columns of A (1024 x 20 x 10 000: 25 us, here
+// 15.8).
+// 32 depth indices a round: 128-byte runs and 37 KB of LDS a block (64: 10.1 against 9.2 us for 1024 x 20 x 4096;
+// 128: 10.9 us); one block a CU's worth of slices (two: 9.2 against 9.1 us, 7.5 against 6.8 us at a depth of 2048)
+constexpr unsigned kTnMidDepth = 32;
+constexpr unsigned kTnMidPitch = kTnMidDepth + 4;
+template <int NB4>  // B's columns in loads of four: ceil(N / 4)
+__global__ __launch_bounds__(256) void gemm_tn_mid_kernel(unsigned M, unsigned N, unsigned K, unsigned chunk,
+                                                          unsigned per_wave, const float* __restrict__ A, size_t lda,
+                                                          const float* __restrict__ B, size_t ldb, float beta,
+                                                          float* __restrict__ C, float* __restrict__ partial) {
+  __shared__ __attribute__((aligned(16))) float tiles[4][2][32 * kTnMidPitch];
+  const unsigned lane = threadIdx.x & 63, w = threadIdx.x >> 6, l32 = lane & 31, hi = lane >> 5;
+  const unsigned i0 = blockIdx.x * 32;
+  const unsigned k0 = blockIdx.y * chunk, k1 = min(K, k0 + chunk);
+  const unsigned kw0 = k0 + w * per_wave, kw1 = min(k1, kw0 + per_wave);
+  float* la = tiles[w][0];
+  float* lb = tiles[w][1];
+  constexpr unsigned kLanesDeep = kTnMidDepth / 4, kColsPerLoad = 64 / kLanesDeep;
+  const unsigned q = lane % kLanesDeep, cq = lane / kLanesDeep;  // a load: kLanesDeep lanes along the depth of one of kColsPerLoad columns
+  stepx16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+  // The next round's loads leave before this round's fragments are multiplied.
+  constexpr int kLoadsA = 32 / kColsPerLoad, kLoadsB = (4 * NB4 + kColsPerLoad - 1) / kColsPerLoad;
+  float4 ta[kLoadsA], tb[kLoadsB];
+  bool in = false;
+  auto fetch = [&](unsigned t) __attribute__((always_inline)) {
+    const unsigned kq = kw0 + t + 4 * q;       // this lane's four depth indices
+    in = kq < kw1;                             // K, the ranges and kq are multiples of four
+    const size_t kc = in ? kq : (K - 4);
+#pragma unroll
+    for (int u = 0; u < kLoadsA; ++u) ta[u] = ldg4<true>(reinterpret_cast<const float4*>(A + size_t(min(i0 + kColsPerLoad * u + cq, M - 1)) * lda + kc));
+#pragma unroll
+    for (int u = 0; u < kLoadsB; ++u) tb[u] = *reinterpret_cast<const float4*>(B + size_t(min(kColsPerLoad * u + cq, N - 1)) * ldb + kc);
+  };
+  fetch(0);
+  for (unsigned t = 0; kw0 + t < kw1; t += kTnMidDepth) {
+    // the tiles are this wavefront's own: its LDS accesses execute in order, so the compiler only has to keep the
+    // writes behind the last round's reads and ahead of this round's (no block barrier: the wavefronts drift apart
+    // and one multiplies while another waits for its loads)
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int u = 0; u < kLoadsA; ++u) {
+      const float4 v = ta[u];
+      *reinterpret_cast<float4*>(la + (kColsPerLoad * u + cq) * kTnMidPitch + 4 * q) =
+          make_float4(in ? v.x : 0.f, in ? v.y : 0.f, in ? v.z : 0.f, in ? v.w : 0.f);
+    }
+#pragma unroll
+    for (int u = 0; u < kLoadsB; ++u) {
+      const float4 v = tb[u];
+      if (kColsPerLoad * u + cq < 32)
+      *reinterpret_cast<float4*>(lb + (kColsPerLoad * u + cq) * kTnMidPitch + 4 * q) =
+          make_float4(in ? v.x : 0.f, in ? v.y : 0.f, in ? v.z : 0.f, in ? v.w : 0.f);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    if (kw0 + t + kTnMidDepth < kw1) fetch(t + kTnMidDepth);
+#pragma unroll
+    for (int s8 = 0; s8 < int(kTnMidDepth) / 8; ++s8) {
+      const float4 a4 = *reinterpret_cast<const float4*>(la + l32 * kTnMidPitch + 8 * s8 + 4 * hi);
+      const float4 b4 = *reinterpret_cast<const float4*>(lb + min(l32, 4u * NB4 - 1) * kTnMidPitch + 8 * s8 + 4 * hi);
+      const bool col = l32 < N;
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(col ? b4.x : 0.f, a4.x, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(col ? b4.y : 0.f, a4.y, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(col ? b4.z : 0.f, a4.z, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(col ? b4.w : 0.f, a4.w, acc, 0, 0, 0);
+    }
+  }
+  // acc[r] of lane l: output row i0 + l % 32, column 8 * (r / 4) + 4 * (l / 32) + r % 4
+  __syncthreads();
+  float* red = &tiles[0][0][0];  // [wave][16][64]
+#pragma unroll
+  for (int r = 0; r < 16; ++r) red[(w * 16 + r) * 64 + lane] = acc[r];
+  __syncthreads();
+  float* out = partial != nullptr ? partial + size_t(blockIdx.y) * M * N : C;
+  const unsigned row = i0 + l32;
+#pragma unroll
+  for (int rr = 0; rr < 4; ++rr) {  // wavefront w finishes registers 4 w .. 4 w + 3
+    const unsigned r = 4 * w + rr, n = 8 * (r / 4) + 4 * hi + (r % 4);
+    float v = red[r * 64 + lane];
+#pragma unroll
+    for (int x = 1; x < 4; ++x) v += red[(x * 16 + r) * 64 + lane];
+    if (row < M && n < N) {
+      float* p = out + size_t(n) * M + row;
+      *p = (partial == nullptr && beta != 0.f) ? beta * *p + v : v;
+    }
+  }
+}
+
+static bool mid_tn_eligible(const dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B,
+                            size_t ldb) {
+  return N >= 5 && N <= 32 && M >= 32 && M <= (size_t(1) << 30) && K >= 256 && K % 4 == 0 && K <= 0x7FFFFFF0ull &&
+         lda % 4 == 0 && ldb % 4 == 0 && aligned16(A) && aligned16(B) && dev->gemm_ws != nullptr;
+}
+
+static int mid_tn_run(dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B, size_t ldb,
+                      float beta, float* C) {
+  const unsigned tiles = static_cast<unsigned>(cdiv<size_t>(M, 32)), Ku = static_cast<unsigned>(K);
+  // depth slices: a block a CU, each with at least one round per wavefront
+  unsigned slabs = cdiv<unsigned>(unsigned(dev->num_cus > 0 ? dev->num_cus : 256), tiles);
+  const unsigned max_by_depth = cdiv<unsigned>(Ku, 4 * kTnMidDepth);
+  if (slabs > max_by_depth) slabs = max_by_depth;
+  if (slabs < 1) slabs = 1;
+  unsigned chunk = cdiv<unsigned>(Ku, slabs);
+  chunk = (chunk + 4 * kTnMidDepth - 1) / (4 * kTnMidDepth) * (4 * kTnMidDepth);
+  slabs = cdiv<unsigned>(Ku, chunk);
+  const unsigned per_wave = chunk / 4;
+  float* partial = nullptr;
+  if (slabs > 1) {
+    DYHIP_REQUIRE(dev->gemm_ws_bytes >= sizeof(float) * M * N * slabs, "transposed small-batch product: workspace too small");
+    partial = static_cast<float*>(dev->gemm_ws);
+  }
+  const dim3 grid(tiles, slabs), block(256);
+#define DYHIP_TN_MID(NB4)                                                                                          \
+  hipLaunchKernelGGL(gemm_tn_mid_kernel<NB4>, grid, block, 0, dev->stream, static_cast<unsigned>(M), static_cast<unsigned>(N), \
+                     Ku, chunk, per_wave, A, lda, B, ldb, beta, C, partial)
+  switch ((N + 3) / 4) {
+    case 2: DYHIP_TN_MID(2); break;
+    case 3: DYHIP_TN_MID(3); break;
+    case 4: DYHIP_TN_MID(4); break;
+    case 5: DYHIP_TN_MID(5); break;
+    case 6: DYHIP_TN_MID(6); break;
+    case 7: DYHIP_TN_MID(7); break;
+    default: DYHIP_TN_MID(8); break;
+  }
+#undef DYHIP_TN_MID
+  DYHIP_CHECK_LAUNCH();
+  if (partial != nullptr) {
+    const size_t total = M * N;
+    hipLaunchKernelGGL(slices_accumulate_kernel, dim3(unsigned(cdiv<size_t>(total, 256))), dim3(256), 0, dev->stream, total,
+                       slabs, partial, beta, C);
+    DYHIP_CHECK_LAUNCH();
+  }
+  return DYHIP_OK;
+}
+
 static bool thin_tn_eligible(size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B, size_t ldb) {
   return N >= 1 && N <= 32 && M >= 1 && M <= (size_t(1) << 30) && K >= 256 && K % 4 == 0 && K / 4 <= 0xFFFFFFFFull &&
          lda % 4 == 0 && ldb % 4 == 0 && aligned16(A) && aligned16(B);
@@ -957,15 +1102,20 @@ static int thin_tn_run(dyhip_device* dev, size_t M, size_t N, size_t K, const fl
 int skinny_tn_gemm(dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B,
                    size_t ldb, float beta, float* C, bool* taken) {
   *taken = false;
-  // At most 32 columns of B: the streaming kernel takes what the fragment-order product below does not (a depth or a
-  // row count off its grid: 650 x 20 x 2600 12.5 against 17.7 us on the general GEMM) and, up to four columns, all of
-  // it (1024 x 1 x 4096: 7.1 against 11.4 us); where both apply at 16-32 columns the fragment-order product is faster
-  // (1024 x 20 x 4096: 13.6 against 14.9 us - the 4 x N partial sums cross the block through 4 N wavefront sums).
+  // At most 32 columns of B: up to four the streaming kernel (1024 x 1 x 4096: 7.1 against 11.4 us for the
+  // fragment-order product below), from five on the matrix-core kernel on LDS tiles (faster than the fragment-order
+  // product on every shape measured up to 64 MB of A, and without its conditions on the depth); the streaming kernel
+  // still takes what neither does.  More than 32 columns: the fragment-order product.
   const bool thin_ok = C != nullptr && thin_tn_eligible(M, N, K, A, lda, B, ldb);
   bool frag_ok = !(M == 0 || N == 0 || M > 4096 || N > 256 || K < 1024 || K > (size_t(1) << 24)) &&
                  !(M * N > (size_t(1) << 19) || lda % 4 != 0 || ldb % 4 != 0 || !aligned16(A) || !aligned16(B));
   frag_ok = frag_ok && skinny_tn_splits(unsigned(M), unsigned(N), unsigned(K)) != 0 && dev->gemm_ws != nullptr &&
             dev->gemm_ws_bytes >= sizeof(float) * M * N * 16;
+  if (C != nullptr && mid_tn_eligible(dev, M, N, K, A, lda, B, ldb)) {
+    DYHIP_CHECK_STATUS(mid_tn_run(dev, M, N, K, A, lda, B, ldb, beta, C));
+    *taken = true;
+    return DYHIP_OK;
+  }
   if (thin_ok && (N <= 4 || !frag_ok)) {
     DYHIP_CHECK_STATUS(thin_tn_run(dev, M, N, K, A, lda, B, ldb, beta, C));
     *taken = true;

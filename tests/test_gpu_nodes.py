@@ -102,11 +102,13 @@ def test_gemm_nt_thin(dev, M, N, K):
     assert_close(yt.numpy(), ref64.astype(np.float32), FWD_RTOL, "thin gemm_nt beta=0", floor=np.sqrt(K))
 
 
-# l^T * r with at most 32 columns of r (dx and dh of the gates node at a small batch): the left operand streamed once,
-# four of its columns a block; column counts on both sides of every multiple of four, row counts that do not fill the
-# last block, any beta.
+# l^T * r with at most 32 columns of r (dx and dh of the gates node at a small batch): up to four columns the left
+# operand streamed once, four of its columns a block; 5..32 columns on the matrix cores through LDS tiles (or the
+# fragment-order product where the depth is a multiple of 128).  Column counts on both sides of every multiple of
+# four, row counts that do not fill the last block or tile, depths that end inside a 64-index round, any beta.
 @pytest.mark.parametrize("M,N,K", [(1024, 20, 4096), (128, 32, 1024), (650, 20, 2600), (1000, 1, 4000), (37, 7, 256),
-                                   (1024, 13, 6000), (258, 4, 1024), (255, 29, 2048)])
+                                   (1024, 13, 6000), (258, 4, 1024), (255, 29, 2048), (1024, 20, 10000), (33, 5, 260),
+                                   (100, 32, 1004), (2048, 9, 516), (4100, 31, 772), (32, 16, 100000), (1024, 6, 300)])
 def test_gemm_tn_thin(dev, M, N, K):
     rng = np.random.default_rng(M + N + K)
     y0 = f32(rng.standard_normal((N, M)))
