@@ -705,18 +705,22 @@ struct NnOperand {
   unsigned K;
 };
 
+// TILES = 1: a block owns 32 gate rows (twice the blocks and half the matrix-core steps a wavefront: the smallest
+// baseline cell, 16 blocks of 64 rows, 8.0 us)
+template <int TILES>
 __global__ __launch_bounds__(256) void lstm_gates_skinny_kernel(unsigned H, unsigned B, NnOperand op0, NnOperand op1,
                                                                 const float* __restrict__ bias, int mode,
                                                                 float* __restrict__ fx) {
-  __shared__ float red[4 * 64 * kStepPitchR];
-  const unsigned M = 4 * H, RP = M / 64;
+  constexpr unsigned ROWS = 32 * TILES;
+  __shared__ float red[4 * ROWS * kStepPitchR];
+  const unsigned M = 4 * H, RP = M / ROWS;
   const unsigned rp = blockIdx.x % RP, ct = blockIdx.x / RP;
   const unsigned wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const unsigned l32 = lane % 32, lhi = lane / 32;
   stepx16 acc0 = {0}, acc1 = {0};
   const unsigned pcol = ct * 32 + l32 < B ? ct * 32 + l32 : B - 1;
-  // every output of this thread lies in gate row rp*64 + threadIdx.x % 64: its bias is fetched under the product
-  const float bias_row = bias[rp * 64 + threadIdx.x % 64];
+  // every output of this thread lies in gate row rp*ROWS + threadIdx.x % ROWS: its bias is fetched under the product
+  const float bias_row = bias[rp * ROWS + threadIdx.x % ROWS];
   // The four waves split the depth of BOTH products taken together into quarters (with I = H two waves multiply by
   // Wx and two by Wh): one run of the load pipeline per wave instead of one per product (its start costs ~1.5 us).
   const unsigned G0 = op0.K / 8, Gt = G0 + op1.K / 8, lo = wave * (Gt / 4), hi = lo + Gt / 4;
@@ -726,24 +730,24 @@ __global__ __launch_bounds__(256) void lstm_gates_skinny_kernel(unsigned H, unsi
     const unsigned glo = lo > base ? lo : base, ghi = hi < base + G ? hi : base + G;
     if (glo >= ghi) continue;
     const unsigned g0 = glo - base;
-    const float* pa = op.W + size_t(rp) * 64 + l32 + (size_t(g0) * 8 + 4 * lhi) * M;
+    const float* pa = op.W + size_t(rp) * ROWS + l32 + (size_t(g0) * 8 + 4 * lhi) * M;
     const float* pb = op.v + size_t(pcol) * op.K + size_t(g0) * 8 + 4 * lhi;
-    step_product<kFragAlongRows, true, 2>(acc0, acc1, pa, pa + 32, pb, ghi - glo, M);
+    step_product<kFragAlongRows, true, TILES>(acc0, acc1, pa, pa + 32, pb, ghi - glo, M);
   }
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const unsigned row = 8 * (r / 4) + 4 * lhi + (r % 4);
-    red[(wave * 64 + row) * kStepPitchR + l32] = acc0[r];
-    red[(wave * 64 + 32 + row) * kStepPitchR + l32] = acc1[r];
+    red[(wave * ROWS + row) * kStepPitchR + l32] = acc0[r];
+    if (TILES == 2) red[(wave * ROWS + 32 + row) * kStepPitchR + l32] = acc1[r];
   }
   __syncthreads();
-  for (unsigned o = threadIdx.x; o < 64 * 32; o += 256) {
-    const unsigned row = o % 64, col = o / 64, erow = rp * 64 + row, ecol = ct * 32 + col;
+  for (unsigned o = threadIdx.x; o < ROWS * 32; o += 256) {
+    const unsigned row = o % ROWS, col = o / ROWS, erow = rp * ROWS + row, ecol = ct * 32 + col;
     if (ecol >= B) continue;
     float pre = bias_row;
     if (erow >= H && erow < 2 * H) pre += 1.0f;  // forget-gate bias
 #pragma unroll
-    for (int w = 0; w < 4; ++w) pre += red[(w * 64 + row) * kStepPitchR + col];
+    for (int w = 0; w < 4; ++w) pre += red[(w * ROWS + row) * kStepPitchR + col];
     fx[size_t(ecol) * M + erow] = erow < 3 * H ? logistic(mode, pre) : tanh_accurate(pre);
   }
 }
@@ -1189,8 +1193,13 @@ int dyhip_lstm_gates_forward(dyhip_device* dev, unsigned num_inputs, const float
       (small_weights ||
        (B > 32 && (G / 64) * cdiv<unsigned>(B, 32) >= unsigned(dev->num_cus > 0 ? dev->num_cus : 256) / 2))) {
     const NnOperand op0{Wx, x_eff, gi.I}, op1{Wh, h_eff, H};
-    hipLaunchKernelGGL(lstm_gates_skinny_kernel, dim3(unsigned(G / 64) * cdiv<unsigned>(B, 32)), dim3(256), 0, dev->stream, H,
-                       B, op0, op1, b, logistic_mode, fx);
+    const unsigned cus = unsigned(dev->num_cus > 0 ? dev->num_cus : 256);
+    if (unsigned(G / 64) * cdiv<unsigned>(B, 32) < cus / 2)
+      hipLaunchKernelGGL(lstm_gates_skinny_kernel<1>, dim3(unsigned(G / 32) * cdiv<unsigned>(B, 32)), dim3(256), 0,
+                         dev->stream, H, B, op0, op1, b, logistic_mode, fx);
+    else
+      hipLaunchKernelGGL(lstm_gates_skinny_kernel<2>, dim3(unsigned(G / 64) * cdiv<unsigned>(B, 32)), dim3(256), 0,
+                         dev->stream, H, B, op0, op1, b, logistic_mode, fx);
     DYHIP_CHECK_LAUNCH();
     return DYHIP_OK;
   }
