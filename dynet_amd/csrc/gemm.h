@@ -78,4 +78,9 @@ int gemm_shallow_nt_run(dyhip_device* dev, size_t M, size_t N, size_t K, const f
 int skinny_tn_gemm(dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B,
                    size_t ldb, float beta, float* C, bool* taken);
 
+// lstm.hip: C = epilogue(A0 B0 [+ A1 B1]) in one launch for a right operand of a few 32-column tiles (A: M x K with rows
+// contiguous, B: K x N with k contiguous; two segments only with the gates epilogue); *taken tells whether it ran.
+int skinny_nn_gemm(dyhip_device* dev, size_t M, size_t N, int nseg, const GemmSeg* segs, float* C, const GemmEpiParams& epi,
+                   bool* taken);
+
 }  // namespace dyhip

@@ -695,32 +695,36 @@ __global__ __launch_bounds__(256) void skinny_tn_kernel(unsigned M, unsigned N, 
   }
 }
 
-// VanillaLSTMGates forward for a batch that is a few 32-column tiles wide: fx = act(b + [f: +1] + Wx x + Wh h) with
-// the weights as DyNet stores them (4H x K, rows contiguous) and x, h plain (k contiguous per column).  A block owns
-// 64 consecutive gate rows x 32 columns over the full depth of both products (4H / 64 x B / 32 blocks: one per CU at
-// H = 1024, B = 128), its four waves split each depth in quarters and meet in LDS; nothing goes through a workspace.
+// C = epilogue(W0 v0 [+ W1 v1]) for a right operand that is a few 32-column tiles wide, one launch: the gates node's
+// forward, fx = act(b + [f: +1] + Wx x + Wh h), and l * r / the affine layer of a small batch.  The weights as DyNet
+// stores them (M x K, rows contiguous) and v plain (k contiguous per column).  A block owns 32 or 64 consecutive rows
+// x 32 columns over the full depth of both products, its four waves split the depth in quarters and meet in LDS;
+// nothing goes through a workspace.
 struct NnOperand {
-  const float* W;  // M x K, leading dimension M (rows contiguous)
-  const float* v;  // K x N, leading dimension K
+  const float* W;  // M x K, rows contiguous, leading dimension ldw
+  const float* v;  // K x N, k contiguous, leading dimension ldv
   unsigned K;
+  size_t ldw, ldv;
 };
+enum { kNnGates = 0, kNnBias = 1, kNnAxpby = 2 };
 
-// TILES = 1: a block owns 32 gate rows (twice the blocks and half the matrix-core steps a wavefront: the smallest
-// baseline cell, 16 blocks of 64 rows, 8.0 us)
-template <int TILES>
-__global__ __launch_bounds__(256) void lstm_gates_skinny_kernel(unsigned H, unsigned B, NnOperand op0, NnOperand op1,
-                                                                const float* __restrict__ bias, int mode,
-                                                                float* __restrict__ fx) {
+// TILES = 1: a block owns 32 rows (twice the blocks and half the matrix-core steps a wavefront: the smallest
+// baseline cell, 16 blocks of 64 rows, 8.0 us; 5.6 us with 32 of 32)
+template <int TILES, int EPI>
+__global__ __launch_bounds__(256) void skinny_nn_kernel(unsigned M, unsigned H, unsigned B, NnOperand op0, NnOperand op1,
+                                                        const float* __restrict__ bias, float beta, int mode,
+                                                        float* __restrict__ fx) {
   constexpr unsigned ROWS = 32 * TILES;
   __shared__ float red[4 * ROWS * kStepPitchR];
-  const unsigned M = 4 * H, RP = M / ROWS;
+  const unsigned RP = (M + ROWS - 1) / ROWS;  // rows past the end are computed on the last row and dropped
   const unsigned rp = blockIdx.x % RP, ct = blockIdx.x / RP;
   const unsigned wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const unsigned l32 = lane % 32, lhi = lane / 32;
   stepx16 acc0 = {0}, acc1 = {0};
   const unsigned pcol = ct * 32 + l32 < B ? ct * 32 + l32 : B - 1;
-  // every output of this thread lies in gate row rp*ROWS + threadIdx.x % ROWS: its bias is fetched under the product
-  const float bias_row = bias[rp * ROWS + threadIdx.x % ROWS];
+  // every output of this thread lies in row rp*ROWS + threadIdx.x % ROWS: its bias is fetched under the product
+  const float bias_row = EPI == kNnAxpby ? 0.f : bias[min(rp * ROWS + threadIdx.x % ROWS, M - 1)];
+  const unsigned r0 = min(rp * ROWS + l32, M - 1), r1 = min(rp * ROWS + 32 + l32, M - 1);
   // The four waves split the depth of BOTH products taken together into quarters (with I = H two waves multiply by
   // Wx and two by Wh): one run of the load pipeline per wave instead of one per product (its start costs ~1.5 us).
   const unsigned G0 = op0.K / 8, Gt = G0 + op1.K / 8, lo = wave * (Gt / 4), hi = lo + Gt / 4;
@@ -730,9 +734,9 @@ __global__ __launch_bounds__(256) void lstm_gates_skinny_kernel(unsigned H, unsi
     const unsigned glo = lo > base ? lo : base, ghi = hi < base + G ? hi : base + G;
     if (glo >= ghi) continue;
     const unsigned g0 = glo - base;
-    const float* pa = op.W + size_t(rp) * ROWS + l32 + (size_t(g0) * 8 + 4 * lhi) * M;
-    const float* pb = op.v + size_t(pcol) * op.K + size_t(g0) * 8 + 4 * lhi;
-    step_product<kFragAlongRows, true, TILES>(acc0, acc1, pa, pa + 32, pb, ghi - glo, M);
+    const float* pk = op.W + (size_t(g0) * 8 + 4 * lhi) * op.ldw;
+    const float* pb = op.v + size_t(pcol) * op.ldv + size_t(g0) * 8 + 4 * lhi;
+    step_product<kFragAlongRows, true, TILES>(acc0, acc1, pk + r0, pk + r1, pb, ghi - glo, op.ldw);
   }
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
@@ -743,13 +747,71 @@ __global__ __launch_bounds__(256) void lstm_gates_skinny_kernel(unsigned H, unsi
   __syncthreads();
   for (unsigned o = threadIdx.x; o < ROWS * 32; o += 256) {
     const unsigned row = o % ROWS, col = o / ROWS, erow = rp * ROWS + row, ecol = ct * 32 + col;
-    if (ecol >= B) continue;
-    float pre = bias_row;
-    if (erow >= H && erow < 2 * H) pre += 1.0f;  // forget-gate bias
+    if (ecol >= B || erow >= M) continue;
+    float* out = fx + size_t(ecol) * M + erow;
+    if (EPI == kNnGates) {
+      float pre = bias_row;
+      if (erow >= H && erow < 2 * H) pre += 1.0f;  // forget-gate bias
 #pragma unroll
-    for (int w = 0; w < 4; ++w) pre += red[(w * ROWS + row) * kStepPitchR + col];
-    fx[size_t(ecol) * M + erow] = erow < 3 * H ? logistic(mode, pre) : tanh_accurate(pre);
+      for (int w = 0; w < 4; ++w) pre += red[(w * ROWS + row) * kStepPitchR + col];
+      *out = erow < 3 * H ? logistic(mode, pre) : tanh_accurate(pre);
+    } else {
+      float t = red[row * kStepPitchR + col];
+#pragma unroll
+      for (int w = 1; w < 4; ++w) t += red[(w * ROWS + row) * kStepPitchR + col];
+      if (EPI == kNnBias) t += bias_row;
+      else if (beta != 0.f) t += beta * *out;
+      *out = t;
+    }
   }
+}
+
+// 32-row blocks as long as they do not outnumber the CUs (gates forward, I = H = 1024: B = 20 13.9 us against 25 us
+// with 64-row blocks and 17.0 us for the two-launch small-batch product; B = 64 15.4 against 23.7 us; I = H = 2048,
+// B = 20 32.4 against 42.3 and 36.6 us; more blocks than CUs lose: B = 96 39.3 against 24.4 us, B = 128 39.8 against
+// 25.7 us).  Not for a block that would walk more than 2 MB of weights alone (a few rows over a very long depth), nor
+// for depths that do not split into whole rounds of four 8-index groups per wavefront.
+int skinny_nn_gemm(dyhip_device* dev, size_t M, size_t N, int nseg, const GemmSeg* segs, float* C, const GemmEpiParams& epi,
+                   bool* taken) {
+  *taken = false;
+  if (nseg < 1 || nseg > 2 || C == nullptr || N == 0 || N > 256 || M < 32 || M >= (size_t(1) << 31)) return DYHIP_OK;
+  const int kind = epi.kind == kEpiLstmGates ? kNnGates : epi.kind == kEpiBias ? kNnBias : epi.kind == kEpiAxpby ? kNnAxpby : -1;
+  if (kind < 0 || (kind != kNnAxpby && epi.bias == nullptr) || (nseg == 2 && kind != kNnGates)) return DYHIP_OK;
+  size_t Kt = 0;
+  for (int q = 0; q < nseg; ++q) {
+    const GemmSeg& g = segs[q];
+    if (g.A == nullptr || g.B == nullptr || g.K == 0 || g.K % 32 != 0 || g.K >= (size_t(1) << 31) || g.ldb % 4 != 0 ||
+        !aligned16(g.B))
+      return DYHIP_OK;
+    Kt += g.K;
+  }
+  if (Kt % 128 != 0) return DYHIP_OK;
+  const unsigned cus = unsigned(dev->num_cus > 0 ? dev->num_cus : 256);
+  const unsigned ct = cdiv<unsigned>(unsigned(N), 32);
+  const unsigned blocks64 = cdiv<unsigned>(unsigned(M), 64) * ct;
+  const unsigned tiles = blocks64 <= cus / 2 ? 1 : 2;
+  if (size_t(32) * tiles * Kt * sizeof(float) > (size_t(2) << 20)) return DYHIP_OK;
+  const NnOperand op0{segs[0].A, segs[0].B, unsigned(segs[0].K), segs[0].lda, segs[0].ldb};
+  const NnOperand op1 = nseg > 1 ? NnOperand{segs[1].A, segs[1].B, unsigned(segs[1].K), segs[1].lda, segs[1].ldb}
+                                 : NnOperand{segs[0].A, segs[0].B, 0u, segs[0].lda, segs[0].ldb};
+  const dim3 grid(cdiv<unsigned>(unsigned(M), 32 * tiles) * ct), block(256);
+  const float beta = kind == kNnAxpby ? epi.beta : 0.f;
+#define DYHIP_SKINNY_NN(T, E)                                                                                       \
+  hipLaunchKernelGGL((skinny_nn_kernel<T, E>), grid, block, 0, dev->stream, unsigned(M), epi.H, unsigned(N), op0, op1, \
+                     epi.bias, beta, epi.logistic_mode, C)
+  if (tiles == 1) {
+    if (kind == kNnGates) DYHIP_SKINNY_NN(1, kNnGates);
+    else if (kind == kNnBias) DYHIP_SKINNY_NN(1, kNnBias);
+    else DYHIP_SKINNY_NN(1, kNnAxpby);
+  } else {
+    if (kind == kNnGates) DYHIP_SKINNY_NN(2, kNnGates);
+    else if (kind == kNnBias) DYHIP_SKINNY_NN(2, kNnBias);
+    else DYHIP_SKINNY_NN(2, kNnAxpby);
+  }
+#undef DYHIP_SKINNY_NN
+  DYHIP_CHECK_LAUNCH();
+  *taken = true;
+  return DYHIP_OK;
 }
 
 // out[e] = beta * out[e] + (slices[0][e] + slices[1][e] + ...), slices added in ascending order
@@ -1184,25 +1246,8 @@ int dyhip_lstm_gates_forward(dyhip_device* dev, unsigned num_inputs, const float
     GemmEpiParams ep{kEpiLstmGates, 0.f, b, H, logistic_mode};
     return gemm_run(dev, false, true, G, B, 2, segs, fx, ep);
   }
-  // a batch of a few column tiles: one launch of the fragment-order kernel on the operands as they lie, when it has
-  // blocks for half the CUs or the weights are small enough to sit in an L2 (up to 32 columns only then: above
-  // 4 MB the small-batch product below reads the weights in longer runs; I = H = 2048, B = 20: 42.5 -> 36.8 us)
-  const bool small_weights = G * (gi.I + H) * sizeof(float) <= (size_t(4) << 20);
-  if (B <= 256 && H % 16 == 0 && gi.I % 128 == 0 && H % 128 == 0 && G < (size_t(1) << 31) &&
-      all_aligned16({Wx, Wh, x_eff, h_eff}) &&
-      (small_weights ||
-       (B > 32 && (G / 64) * cdiv<unsigned>(B, 32) >= unsigned(dev->num_cus > 0 ? dev->num_cus : 256) / 2))) {
-    const NnOperand op0{Wx, x_eff, gi.I}, op1{Wh, h_eff, H};
-    const unsigned cus = unsigned(dev->num_cus > 0 ? dev->num_cus : 256);
-    if (unsigned(G / 64) * cdiv<unsigned>(B, 32) < cus / 2)
-      hipLaunchKernelGGL(lstm_gates_skinny_kernel<1>, dim3(unsigned(G / 32) * cdiv<unsigned>(B, 32)), dim3(256), 0,
-                         dev->stream, H, B, op0, op1, b, logistic_mode, fx);
-    else
-      hipLaunchKernelGGL(lstm_gates_skinny_kernel<2>, dim3(unsigned(G / 64) * cdiv<unsigned>(B, 32)), dim3(256), 0,
-                         dev->stream, H, B, op0, op1, b, logistic_mode, fx);
-    DYHIP_CHECK_LAUNCH();
-    return DYHIP_OK;
-  }
+  // a batch of a few column tiles: one launch of the fragment-order kernel on the operands as they lie, where its
+  // conditions hold (see skinny_nn_gemm); gemm_run tries it first
   GemmSeg segs[2] = {{Wx, G, x_eff, gi.I, gi.I}, {Wh, G, h_eff, H, H}};
   GemmEpiParams ep{kEpiLstmGates, 0.f, b, H, logistic_mode};
   return gemm_run(dev, false, true, G, B, 2, segs, fx, ep);

@@ -154,8 +154,12 @@ def test_gemm_nn_thin(dev, M, N, K):
 # l * r with 9..32 columns of r (a small batch's affine layers): rows in 128-row wavefront tiles on the matrix cores,
 # the depth split over a block's wavefronts and over blocks; depths that are not multiples of 4 or 16, rows that do not
 # fill the last tile, a column count of 32, and a depth long enough for hundreds of slabs.
+# Depths that are multiples of 128 take the one-launch fragment-order product instead (32- or 64-row blocks, rows past
+# the end dropped, up to 256 columns).
 @pytest.mark.parametrize("M,N,K", [(4096, 20, 1024), (4096, 32, 2048), (132, 9, 16), (128, 9, 17), (2600, 20, 650),
-                                   (1000, 31, 1001), (10000, 16, 1024), (512, 20, 512), (256, 12, 50000), (1024, 20, 256)])
+                                   (1000, 31, 1001), (10000, 16, 1024), (512, 20, 512), (256, 12, 50000), (1024, 20, 256),
+                                   (4096, 20, 1000), (1030, 17, 384), (33, 9, 128), (4100, 200, 256), (100, 256, 1280),
+                                   (8192, 64, 128)])
 def test_gemm_nn_mid(dev, M, N, K):
     rng = np.random.default_rng(M + N + K)
     y0 = f32(rng.standard_normal((N, M)))
