@@ -727,16 +727,60 @@ __global__ __launch_bounds__(256) void skinny_nn_kernel(unsigned M, unsigned H, 
   const unsigned r0 = min(rp * ROWS + l32, M - 1), r1 = min(rp * ROWS + 32 + l32, M - 1);
   // The four waves split the depth of BOTH products taken together into quarters (with I = H two waves multiply by
   // Wx and two by Wh): one run of the load pipeline per wave instead of one per product (its start costs ~1.5 us).
-  const unsigned G0 = op0.K / 8, Gt = G0 + op1.K / 8, lo = wave * (Gt / 4), hi = lo + Gt / 4;
-  for (int which = 0; which < 2; ++which) {
-    const NnOperand op = which == 0 ? op0 : op1;
-    const unsigned base = which == 0 ? 0 : G0, G = op.K / 8;
-    const unsigned glo = lo > base ? lo : base, ghi = hi < base + G ? hi : base + G;
-    if (glo >= ghi) continue;
-    const unsigned g0 = glo - base;
-    const float* pk = op.W + (size_t(g0) * 8 + 4 * lhi) * op.ldw;
-    const float* pb = op.v + size_t(pcol) * op.ldv + size_t(g0) * 8 + 4 * lhi;
-    step_product<kFragAlongRows, true, TILES>(acc0, acc1, pk + r0, pk + r1, pb, ghi - glo, op.ldw);
+  if (op0.K % 32 == 0 && op1.K % 32 == 0 && (op0.K + op1.K) % 128 == 0) {
+    const unsigned G0 = op0.K / 8, Gt = G0 + op1.K / 8, lo = wave * (Gt / 4), hi = lo + Gt / 4;
+    for (int which = 0; which < 2; ++which) {
+      const NnOperand op = which == 0 ? op0 : op1;
+      const unsigned base = which == 0 ? 0 : G0, G = op.K / 8;
+      const unsigned glo = lo > base ? lo : base, ghi = hi < base + G ? hi : base + G;
+      if (glo >= ghi) continue;
+      const unsigned g0 = glo - base;
+      const float* pk = op.W + (size_t(g0) * 8 + 4 * lhi) * op.ldw;
+      const float* pb = op.v + size_t(pcol) * op.ldv + size_t(g0) * 8 + 4 * lhi;
+      step_product<kFragAlongRows, true, TILES>(acc0, acc1, pk + r0, pk + r1, pb, ghi - glo, op.ldw);
+    }
+  } else {
+    // Depths off that grid (multiples of four all the same): each product's leading multiple of 128 is split over the
+    // waves as above; what is left of it, at most 15 groups of 8 k and a half group of 4, is dealt to the waves one
+    // group at a time and multiplied in one round of loads (a group past the end is fetched from k = 0 and its v
+    // fragment zeroed).
+    for (int which = 0; which < 2; ++which) {
+      const NnOperand op = which == 0 ? op0 : op1;
+      if (op.K == 0) continue;
+      const unsigned G = op.K / 8, main = G / 16 * 16, per = main / 4;
+      if (per > 0) {
+        const unsigned g0 = wave * per;
+        const float* pk = op.W + (size_t(g0) * 8 + 4 * lhi) * op.ldw;
+        const float* pb = op.v + size_t(pcol) * op.ldv + size_t(g0) * 8 + 4 * lhi;
+        step_product<kFragAlongRows, true, TILES>(acc0, acc1, pk + r0, pk + r1, pb, per, op.ldw);
+      }
+      const unsigned half = (op.K % 8) != 0 ? 1u : 0u, items = G - main + half;
+      if (wave >= items) continue;
+      float a0[4][4], a1[4][4];
+      float4 bf[4];
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const unsigned g = main + wave + 4 * it;
+        const bool valid = g < G || (g == G && half != 0 && lhi == 0);
+        const unsigned k = valid ? 8 * g + 4 * lhi : 0u;
+        const float4 t = *reinterpret_cast<const float4*>(op.v + size_t(pcol) * op.ldv + k);
+        bf[it] = make_float4(valid ? t.x : 0.f, valid ? t.y : 0.f, valid ? t.z : 0.f, valid ? t.w : 0.f);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          a0[it][j] = op.W[r0 + size_t(k + j) * op.ldw];
+          if (TILES == 2) a1[it][j] = op.W[r1 + size_t(k + j) * op.ldw];
+        }
+      }
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const float bj[4] = {bf[it].x, bf[it].y, bf[it].z, bf[it].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[it][j], bj[j], acc0, 0, 0, 0);
+          if (TILES == 2) acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[it][j], bj[j], acc1, 0, 0, 0);
+        }
+      }
+    }
   }
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
@@ -770,7 +814,7 @@ __global__ __launch_bounds__(256) void skinny_nn_kernel(unsigned M, unsigned H, 
 // with 64-row blocks and 17.0 us for the two-launch small-batch product; B = 64 15.4 against 23.7 us; I = H = 2048,
 // B = 20 32.4 against 42.3 and 36.6 us; more blocks than CUs lose: B = 96 39.3 against 24.4 us, B = 128 39.8 against
 // 25.7 us).  Not for a block that would walk more than 2 MB of weights alone (a few rows over a very long depth), nor
-// for depths that do not split into whole rounds of four 8-index groups per wavefront.
+// for depths that are not multiples of four (v's fragments are 128-bit loads along k).
 int skinny_nn_gemm(dyhip_device* dev, size_t M, size_t N, int nseg, const GemmSeg* segs, float* C, const GemmEpiParams& epi,
                    bool* taken) {
   *taken = false;
@@ -780,12 +824,11 @@ int skinny_nn_gemm(dyhip_device* dev, size_t M, size_t N, int nseg, const GemmSe
   size_t Kt = 0;
   for (int q = 0; q < nseg; ++q) {
     const GemmSeg& g = segs[q];
-    if (g.A == nullptr || g.B == nullptr || g.K == 0 || g.K % 32 != 0 || g.K >= (size_t(1) << 31) || g.ldb % 4 != 0 ||
+    if (g.A == nullptr || g.B == nullptr || g.K == 0 || g.K % 4 != 0 || g.K >= (size_t(1) << 31) || g.ldb % 4 != 0 ||
         !aligned16(g.B))
       return DYHIP_OK;
     Kt += g.K;
   }
-  if (Kt % 128 != 0) return DYHIP_OK;
   const unsigned cus = unsigned(dev->num_cus > 0 ? dev->num_cus : 256);
   const unsigned ct = cdiv<unsigned>(unsigned(N), 32);
   const unsigned blocks64 = cdiv<unsigned>(unsigned(M), 64) * ct;

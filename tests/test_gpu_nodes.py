@@ -159,7 +159,8 @@ def test_gemm_nn_thin(dev, M, N, K):
 @pytest.mark.parametrize("M,N,K", [(4096, 20, 1024), (4096, 32, 2048), (132, 9, 16), (128, 9, 17), (2600, 20, 650),
                                    (1000, 31, 1001), (10000, 16, 1024), (512, 20, 512), (256, 12, 50000), (1024, 20, 256),
                                    (4096, 20, 1000), (1030, 17, 384), (33, 9, 128), (4100, 200, 256), (100, 256, 1280),
-                                   (8192, 64, 128)])
+                                   (8192, 64, 128), (1200, 20, 300), (400, 16, 100), (2000, 12, 500), (64, 9, 4),
+                                   (640, 33, 132), (1000, 20, 2044)])
 def test_gemm_nn_mid(dev, M, N, K):
     rng = np.random.default_rng(M + N + K)
     y0 = f32(rng.standard_normal((N, M)))
@@ -527,6 +528,11 @@ def _lstm_case(rng, I, H, B):
     (200, 64, 12, None, False, True),
     (330, 200, 20, [130, 200], True, True),
     (256, 256, 9, None, False, True),
+    # depths that are multiples of four only: the one-launch forward's leftover groups (100 = 12 groups and a half,
+    # 300 + 200: a leading 256 and 128 split over the waves, the rest dealt out one group a wave)
+    (100, 200, 16, None, False, True),
+    (300, 200, 20, None, True, True),
+    (132, 64, 10, [100, 32], False, True),
 ])
 def test_lstm_cell_forward_backward(dev, I, H, B, dims, dropout, mask_full):
     rng = np.random.default_rng(I * 100 + H * 10 + B)
