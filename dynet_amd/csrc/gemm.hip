@@ -1063,17 +1063,18 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
       return gemm_run(dev, a_kmajor, b_kmajor, M, N - cols, 1, &rest, C + cols * M, epi, nullptr);
     }
   }
-  if ((batch == nullptr || batch->count <= 1) && !a_kmajor && b_kmajor && C != nullptr &&
-      gemm_nn_thin_eligible(dev, M, N, nseg, segs, C, epi))
-    return gemm_nn_thin_run(dev, M, N, nseg, segs, C, epi);
-  // 9..256 columns with a depth that splits into whole rounds: the one-launch fragment-order product on the operands
-  // as they lie (4096 x 20 x 1024: 8.4 us against 13.7 us for the two-launch product below, 4096 x 128 x 1024: 14.2
-  // against 22.9 us for the tile kernel with split depth, 2048 x 100 x 2048: 14.6 against 25.4 us)
-  if ((batch == nullptr || batch->count <= 1) && !a_kmajor && b_kmajor && C != nullptr && N >= 9 && N <= 256) {
+  // 5..256 columns with a depth that is a multiple of four: the one-launch fragment-order product on the operands as
+  // they lie (4096 x 20 x 1024: 8.4 us against 13.7 us for the two-launch 9..32-column product below, 4096 x 128 x 1024:
+  // 14.2 against 22.9 us for the tile kernel with split depth, 4096 x 8 x 1024: 8.2 against 10.7 us for the
+  // matrix-times-vector kernels, which keep one to four columns: 4096 x 1 x 1024 6.9 against 8.0 us)
+  if ((batch == nullptr || batch->count <= 1) && !a_kmajor && b_kmajor && C != nullptr && N >= 5 && N <= 256) {
     bool taken = false;
     DYHIP_CHECK_STATUS(skinny_nn_gemm(dev, M, N, nseg, segs, C, epi, &taken));
     if (taken) return DYHIP_OK;
   }
+  if ((batch == nullptr || batch->count <= 1) && !a_kmajor && b_kmajor && C != nullptr &&
+      gemm_nn_thin_eligible(dev, M, N, nseg, segs, C, epi))
+    return gemm_nn_thin_run(dev, M, N, nseg, segs, C, epi);
   if ((batch == nullptr || batch->count <= 1) && !a_kmajor && b_kmajor && C != nullptr &&
       gemm_nn_mid_eligible(dev, M, N, nseg, segs, C, epi))
     return gemm_nn_mid_run(dev, M, N, nseg, segs, C, epi);

@@ -1281,16 +1281,9 @@ int dyhip_lstm_gates_forward(dyhip_device* dev, unsigned num_inputs, const float
   DYHIP_CHECK_STATUS(prepare_x(dev, num_inputs, xs_host, x_dims_host, gi.I, B, mask_x, mask_x_bd, xbuf, &x_eff));
   DYHIP_CHECK_STATUS(prepare_h(dev, H, B, h_tm1, mask_h, mask_h_bd, hbuf, &h_eff));
   const size_t G = size_t(4) * H;
-  // up to 8 columns (the un-batched graph, decoding): the weights are the whole cost and stream through the
-  // matrix-times-vector kernel in kilobyte runs, its second kernel adding the depth slabs with the gates' epilogue
-  // (I = H = 1024, one column: 22 -> 10.6 us; the fragment-order kernel below reads them in 128-byte pieces)
-  if (B <= 8 && G >= 256) {
-    GemmSeg segs[2] = {{Wx, G, x_eff, gi.I, gi.I}, {Wh, G, h_eff, H, H}};
-    GemmEpiParams ep{kEpiLstmGates, 0.f, b, H, logistic_mode};
-    return gemm_run(dev, false, true, G, B, 2, segs, fx, ep);
-  }
-  // a batch of a few column tiles: one launch of the fragment-order kernel on the operands as they lie, where its
-  // conditions hold (see skinny_nn_gemm); gemm_run tries it first
+  // gemm_run picks the form: up to four columns (the un-batched graph, decoding) the matrix-times-vector kernels,
+  // whose second kernel adds the depth slabs with the gates' epilogue (I = H = 1024, one column: 22 -> 9.4 us); from
+  // five columns the one-launch fragment-order kernel on the operands as they lie (see skinny_nn_gemm)
   GemmSeg segs[2] = {{Wx, G, x_eff, gi.I, gi.I}, {Wh, G, h_eff, H, H}};
   GemmEpiParams ep{kEpiLstmGates, 0.f, b, H, logistic_mode};
   return gemm_run(dev, false, true, G, B, 2, segs, fx, ep);
