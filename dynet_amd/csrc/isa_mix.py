@@ -25,7 +25,7 @@ HOT = ["ew_vec4_kernel<2, true, 0, true, 2, dyhip::AccMul2", "ew_vec4_kernel<1, 
        "combine_partials_vec_kernel<64>", "cwise_bcast2_kernel<2, 4, true>", "cwise_reduce_row_kernel<6, true, true>",
        "lookup_gather_kernel<HIP_vector_type<float, 4u>, false, true>", "plan_direct_kernel<16>", "plan_group_kernel<true>",
        "scatter_runs_kernel<HIP_vector_type<float, 4u>, true>", "lse_cols_kernel<true, true>", "pnls_bwd_kernel<true, true, true>",
-       "lstm_step_fwd_kernel<false, 2>", "lstm_step_bwd_kernel", "skinny_tn_kernel<true, true>", "skinny_nn_kernel<2, 0>", "skinny_nn_kernel<1, 1>", "gemm_tn_mid_kernel<5>",
+       "lstm_step_fwd_kernel<false, 2>", "lstm_step_bwd_kernel", "skinny_tn_kernel<true, true>", "skinny_nn_kernel<2, 0, 16>", "skinny_nn_kernel<1, 1, 16>", "gemm_tn_mid_kernel<5>",
        "gemm_wide_kernel<false, false>", "gemm_shallow_nt_kernel", "gemm_tile_kernel<false, false, 1, 2>",
        "gather_segments_kernel<true, true>", "sgd_scaled_kernel<true, true>", "philox",
        "gemm_nn_mid_kernel<true>", "gemm_nn_rows_kernel<1, 8, 4>", "gemm_nn_thin_kernel<1>", "gemm_nt_thin_kernel<32, 4>",

@@ -345,7 +345,16 @@ __global__ __launch_bounds__(256) void lstm_pack_state_kernel(unsigned K, unsign
 // over the 32 rows of the tile; pa then points at row l32 of k = first k + 4 * lhi.
 // TILES = 1 leaves the second row tile out (pa1 and acc1 unused): small problems get twice the blocks.
 enum { kFragPacked = 0, kFragAlongK = 1, kFragAlongRows = 2 };
-template <int A_MODE, bool PLAIN_B, int TILES = 2>
+// B_BYTES = 8: a plain B whose columns start on 8-byte boundaries only (an odd multiple of two floats apart): its
+// fragment is two 64-bit loads.
+template <int B_BYTES>
+__device__ __forceinline__ float4 step_load_b(const float* p) {
+  if (B_BYTES == 16) return *reinterpret_cast<const float4*>(p);
+  const float2 lo = *reinterpret_cast<const float2*>(p), hi = *reinterpret_cast<const float2*>(p + 2);
+  return make_float4(lo.x, lo.y, hi.x, hi.y);
+}
+
+template <int A_MODE, bool PLAIN_B, int TILES = 2, int B_BYTES = 16>
 __device__ __forceinline__ void step_product(stepx16& acc0, stepx16& acc1, const float* __restrict__ pa0,
                                              const float* __restrict__ pa1, const float* __restrict__ pb,
                                              unsigned groups, size_t lda = 0) {
@@ -362,7 +371,7 @@ __device__ __forceinline__ void step_product(stepx16& acc0, stepx16& acc1, const
   _Pragma("unroll") for (int u = 0; u < 4; ++u) {                                                    \
     STEP_LOAD_A(A0[u], pa0, (grp) + u)                                                               \
     if (TILES == 2) { STEP_LOAD_A(A1[u], pa1, (grp) + u) }                                           \
-    BB[u] = *reinterpret_cast<const float4*>(pb + size_t((grp) + u) * SB);                           \
+    BB[u] = step_load_b<B_BYTES>(pb + size_t((grp) + u) * SB);                                       \
   }                                                                                                  \
   __builtin_amdgcn_sched_barrier(0);
 #define STEP_MMA1(x, y, acc) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, acc, 0, 0, 0);
@@ -710,7 +719,7 @@ enum { kNnGates = 0, kNnBias = 1, kNnAxpby = 2 };
 
 // TILES = 1: a block owns 32 rows (twice the blocks and half the matrix-core steps a wavefront: the smallest
 // baseline cell, 16 blocks of 64 rows, 8.0 us; 5.6 us with 32 of 32)
-template <int TILES, int EPI>
+template <int TILES, int EPI, int B_BYTES>
 __global__ __launch_bounds__(256) void skinny_nn_kernel(unsigned M, unsigned H, unsigned B, NnOperand op0, NnOperand op1,
                                                         const float* __restrict__ bias, float beta, int mode,
                                                         float* __restrict__ fx) {
@@ -737,13 +746,13 @@ __global__ __launch_bounds__(256) void skinny_nn_kernel(unsigned M, unsigned H, 
       const unsigned g0 = glo - base;
       const float* pk = op.W + (size_t(g0) * 8 + 4 * lhi) * op.ldw;
       const float* pb = op.v + size_t(pcol) * op.ldv + size_t(g0) * 8 + 4 * lhi;
-      step_product<kFragAlongRows, true, TILES>(acc0, acc1, pk + r0, pk + r1, pb, ghi - glo, op.ldw);
+      step_product<kFragAlongRows, true, TILES, B_BYTES>(acc0, acc1, pk + r0, pk + r1, pb, ghi - glo, op.ldw);
     }
   } else {
-    // Depths off that grid (multiples of four all the same): each product's leading multiple of 128 is split over the
-    // waves as above; what is left of it, at most 15 groups of 8 k and a half group of 4, is dealt to the waves one
-    // group at a time and multiplied in one round of loads (a group past the end is fetched from k = 0 and its v
-    // fragment zeroed).
+    // Depths off that grid (even all the same): each product's leading multiple of 128 is split over the waves as
+    // above; what is left of it, at most 15 groups of 8 k and a group cut short after 2, 4 or 6, is dealt to the waves
+    // one group at a time and multiplied in one round of loads (a pair of k past the end is fetched from k = 0 and its
+    // v entries zeroed).
     for (int which = 0; which < 2; ++which) {
       const NnOperand op = which == 0 ? op0 : op1;
       if (op.K == 0) continue;
@@ -752,32 +761,34 @@ __global__ __launch_bounds__(256) void skinny_nn_kernel(unsigned M, unsigned H, 
         const unsigned g0 = wave * per;
         const float* pk = op.W + (size_t(g0) * 8 + 4 * lhi) * op.ldw;
         const float* pb = op.v + size_t(pcol) * op.ldv + size_t(g0) * 8 + 4 * lhi;
-        step_product<kFragAlongRows, true, TILES>(acc0, acc1, pk + r0, pk + r1, pb, per, op.ldw);
+        step_product<kFragAlongRows, true, TILES, B_BYTES>(acc0, acc1, pk + r0, pk + r1, pb, per, op.ldw);
       }
-      const unsigned half = (op.K % 8) != 0 ? 1u : 0u, items = G - main + half;
+      const unsigned rem = op.K - 8 * G, items = G - main + (rem != 0 ? 1u : 0u);  // rem: 0, 2, 4 or 6 k past the groups
       if (wave >= items) continue;
-      float a0[4][4], a1[4][4];
-      float4 bf[4];
+      float a0[4][4], a1[4][4], bf[4][4];
 #pragma unroll
       for (int it = 0; it < 4; ++it) {
-        const unsigned g = main + wave + 4 * it;
-        const bool valid = g < G || (g == G && half != 0 && lhi == 0);
-        const unsigned k = valid ? 8 * g + 4 * lhi : 0u;
-        const float4 t = *reinterpret_cast<const float4*>(op.v + size_t(pcol) * op.ldv + k);
-        bf[it] = make_float4(valid ? t.x : 0.f, valid ? t.y : 0.f, valid ? t.z : 0.f, valid ? t.w : 0.f);
+        const unsigned g = main + wave + 4 * it, k = 8 * g + 4 * lhi;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          a0[it][j] = op.W[r0 + size_t(k + j) * op.ldw];
-          if (TILES == 2) a1[it][j] = op.W[r1 + size_t(k + j) * op.ldw];
+        for (int pr = 0; pr < 2; ++pr) {  // the fragment's two pairs of k: inside the depth together or not at all
+          const bool valid = k + 2 * pr + 1 < op.K;
+          const unsigned kp = valid ? k + 2 * pr : 0u;
+          const float2 t = *reinterpret_cast<const float2*>(op.v + size_t(pcol) * op.ldv + kp);
+          bf[it][2 * pr] = valid ? t.x : 0.f;
+          bf[it][2 * pr + 1] = valid ? t.y : 0.f;
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            a0[it][2 * pr + j] = op.W[r0 + size_t(kp + j) * op.ldw];
+            if (TILES == 2) a1[it][2 * pr + j] = op.W[r1 + size_t(kp + j) * op.ldw];
+          }
         }
       }
 #pragma unroll
       for (int it = 0; it < 4; ++it) {
-        const float bj[4] = {bf[it].x, bf[it].y, bf[it].z, bf[it].w};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[it][j], bj[j], acc0, 0, 0, 0);
-          if (TILES == 2) acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[it][j], bj[j], acc1, 0, 0, 0);
+          acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[it][j], bf[it][j], acc0, 0, 0, 0);
+          if (TILES == 2) acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[it][j], bf[it][j], acc1, 0, 0, 0);
         }
       }
     }
@@ -814,7 +825,7 @@ __global__ __launch_bounds__(256) void skinny_nn_kernel(unsigned M, unsigned H, 
 // with 64-row blocks and 17.0 us for the two-launch small-batch product; B = 64 15.4 against 23.7 us; I = H = 2048,
 // B = 20 32.4 against 42.3 and 36.6 us; more blocks than CUs lose: B = 96 39.3 against 24.4 us, B = 128 39.8 against
 // 25.7 us).  Not for a block that would walk more than 2 MB of weights alone (a few rows over a very long depth), nor
-// for depths that are not multiples of four (v's fragments are 128-bit loads along k).
+// for odd depths (v's fragments are 128-bit loads along k, or two 64-bit ones).
 int skinny_nn_gemm(dyhip_device* dev, size_t M, size_t N, int nseg, const GemmSeg* segs, float* C, const GemmEpiParams& epi,
                    bool* taken) {
   *taken = false;
@@ -822,11 +833,13 @@ int skinny_nn_gemm(dyhip_device* dev, size_t M, size_t N, int nseg, const GemmSe
   const int kind = epi.kind == kEpiLstmGates ? kNnGates : epi.kind == kEpiBias ? kNnBias : epi.kind == kEpiAxpby ? kNnAxpby : -1;
   if (kind < 0 || (kind != kNnAxpby && epi.bias == nullptr) || (nseg == 2 && kind != kNnGates)) return DYHIP_OK;
   size_t Kt = 0;
+  bool b16 = true;
   for (int q = 0; q < nseg; ++q) {
     const GemmSeg& g = segs[q];
-    if (g.A == nullptr || g.B == nullptr || g.K == 0 || g.K % 4 != 0 || g.K >= (size_t(1) << 31) || g.ldb % 4 != 0 ||
-        !aligned16(g.B))
+    if (g.A == nullptr || g.B == nullptr || g.K == 0 || g.K % 2 != 0 || g.K >= (size_t(1) << 31) || g.ldb % 2 != 0 ||
+        (reinterpret_cast<uintptr_t>(g.B) & 7u) != 0)
       return DYHIP_OK;
+    b16 = b16 && g.ldb % 4 == 0 && aligned16(g.B);  // 128-bit fragments of v; 64-bit halves otherwise
     Kt += g.K;
   }
   const unsigned cus = unsigned(dev->num_cus > 0 ? dev->num_cus : 256);
@@ -839,9 +852,14 @@ int skinny_nn_gemm(dyhip_device* dev, size_t M, size_t N, int nseg, const GemmSe
                                  : NnOperand{segs[0].A, segs[0].B, 0u, segs[0].lda, segs[0].ldb};
   const dim3 grid(cdiv<unsigned>(unsigned(M), 32 * tiles) * ct), block(256);
   const float beta = kind == kNnAxpby ? epi.beta : 0.f;
-#define DYHIP_SKINNY_NN(T, E)                                                                                       \
-  hipLaunchKernelGGL((skinny_nn_kernel<T, E>), grid, block, 0, dev->stream, unsigned(M), epi.H, unsigned(N), op0, op1, \
+#define DYHIP_SKINNY_NN_B(T, E, BB)                                                                                 \
+  hipLaunchKernelGGL((skinny_nn_kernel<T, E, BB>), grid, block, 0, dev->stream, unsigned(M), epi.H, unsigned(N), op0, op1, \
                      epi.bias, beta, epi.logistic_mode, C)
+#define DYHIP_SKINNY_NN(T, E)        \
+  do {                               \
+    if (b16) DYHIP_SKINNY_NN_B(T, E, 16); \
+    else DYHIP_SKINNY_NN_B(T, E, 8);      \
+  } while (0)
   if (tiles == 1) {
     if (kind == kNnGates) DYHIP_SKINNY_NN(1, kNnGates);
     else if (kind == kNnBias) DYHIP_SKINNY_NN(1, kNnBias);
@@ -851,6 +869,7 @@ int skinny_nn_gemm(dyhip_device* dev, size_t M, size_t N, int nseg, const GemmSe
     else if (kind == kNnBias) DYHIP_SKINNY_NN(2, kNnBias);
     else DYHIP_SKINNY_NN(2, kNnAxpby);
   }
+#undef DYHIP_SKINNY_NN_B
 #undef DYHIP_SKINNY_NN
   DYHIP_CHECK_LAUNCH();
   *taken = true;

@@ -160,7 +160,8 @@ def test_gemm_nn_thin(dev, M, N, K):
                                    (1000, 31, 1001), (10000, 16, 1024), (512, 20, 512), (256, 12, 50000), (1024, 20, 256),
                                    (4096, 20, 1000), (1030, 17, 384), (33, 9, 128), (4100, 200, 256), (100, 256, 1280),
                                    (8192, 64, 128), (1200, 20, 300), (400, 16, 100), (2000, 12, 500), (64, 9, 4),
-                                   (640, 33, 132), (1000, 20, 2044)])
+                                   (640, 33, 132), (1000, 20, 2044), (1300, 20, 650), (300, 9, 2), (515, 40, 1030),
+                                   (999, 12, 390)])
 def test_gemm_nn_mid(dev, M, N, K):
     rng = np.random.default_rng(M + N + K)
     y0 = f32(rng.standard_normal((N, M)))
@@ -533,6 +534,10 @@ def _lstm_case(rng, I, H, B):
     (100, 200, 16, None, False, True),
     (300, 200, 20, None, True, True),
     (132, 64, 10, [100, 32], False, True),
+    # even depths that are not multiples of four: x and h columns start on 8-byte boundaries only
+    (650, 650, 20, None, False, True),
+    (50, 30, 12, None, True, True),
+    (6, 10, 9, None, False, True),
 ])
 def test_lstm_cell_forward_backward(dev, I, H, B, dims, dropout, mask_full):
     rng = np.random.default_rng(I * 100 + H * 10 + B)
