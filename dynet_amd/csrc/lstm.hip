@@ -1053,7 +1053,7 @@ __global__ __launch_bounds__(256) void gemm_tn_thin_kernel(unsigned M, unsigned 
   }
 }
 
-// ---- C[M x N] = beta * C + A^T B for 5..32 columns of B on the matrix cores, the operands as they lie ---------------
+// ---- C[M x N] = beta * C + A^T B for 5..256 columns of B (in tiles of 32) on the matrix cores, the operands as they lie --
 // A's columns (the depth contiguous) are fetched by coalesced 128-bit loads, 32 depth indices of 32 columns a
 // wavefront at a time (128-byte runs), and turned into matrix-core fragments through a wavefront's own LDS tile:
 // lane l reads column l % 32 at four depth indices of the lower or upper half of an 8-index group.  B's columns the
@@ -1074,6 +1074,7 @@ __global__ __launch_bounds__(256) void gemm_tn_mid_kernel(unsigned M, unsigned N
   __shared__ __attribute__((aligned(16))) float tiles[4][2][32 * kTnMidPitch];
   const unsigned lane = threadIdx.x & 63, w = threadIdx.x >> 6, l32 = lane & 31, hi = lane >> 5;
   const unsigned i0 = blockIdx.x * 32;
+  const unsigned n0 = blockIdx.z * 32, Nt = min(32u, N - n0);  // this block's tile of B's columns
   const unsigned k0 = blockIdx.y * chunk, k1 = min(K, k0 + chunk);
   const unsigned kw0 = k0 + w * per_wave, kw1 = min(k1, kw0 + per_wave);
   float* la = tiles[w][0];
@@ -1094,7 +1095,7 @@ __global__ __launch_bounds__(256) void gemm_tn_mid_kernel(unsigned M, unsigned N
 #pragma unroll
     for (int u = 0; u < kLoadsA; ++u) ta[u] = ldg4<true>(reinterpret_cast<const float4*>(A + size_t(min(i0 + kColsPerLoad * u + cq, M - 1)) * lda + kc));
 #pragma unroll
-    for (int u = 0; u < kLoadsB; ++u) tb[u] = *reinterpret_cast<const float4*>(B + size_t(min(kColsPerLoad * u + cq, N - 1)) * ldb + kc);
+    for (int u = 0; u < kLoadsB; ++u) tb[u] = *reinterpret_cast<const float4*>(B + size_t(n0 + min(kColsPerLoad * u + cq, Nt - 1)) * ldb + kc);
   };
   fetch(0);
   for (unsigned t = 0; kw0 + t < kw1; t += kTnMidDepth) {
@@ -1123,7 +1124,7 @@ __global__ __launch_bounds__(256) void gemm_tn_mid_kernel(unsigned M, unsigned N
     for (int s8 = 0; s8 < int(kTnMidDepth) / 8; ++s8) {
       const float4 a4 = *reinterpret_cast<const float4*>(la + l32 * kTnMidPitch + 8 * s8 + 4 * hi);
       const float4 b4 = *reinterpret_cast<const float4*>(lb + min(l32, 4u * NB4 - 1) * kTnMidPitch + 8 * s8 + 4 * hi);
-      const bool col = l32 < N;
+      const bool col = l32 < Nt;
       acc = __builtin_amdgcn_mfma_f32_32x32x2f32(col ? b4.x : 0.f, a4.x, acc, 0, 0, 0);
       acc = __builtin_amdgcn_mfma_f32_32x32x2f32(col ? b4.y : 0.f, a4.y, acc, 0, 0, 0);
       acc = __builtin_amdgcn_mfma_f32_32x32x2f32(col ? b4.z : 0.f, a4.z, acc, 0, 0, 0);
@@ -1140,7 +1141,7 @@ __global__ __launch_bounds__(256) void gemm_tn_mid_kernel(unsigned M, unsigned N
   const unsigned row = i0 + l32;
 #pragma unroll
   for (int rr = 0; rr < 4; ++rr) {  // wavefront w finishes registers 4 w .. 4 w + 3
-    const unsigned r = 4 * w + rr, n = 8 * (r / 4) + 4 * hi + (r % 4);
+    const unsigned r = 4 * w + rr, n = n0 + 8 * (r / 4) + 4 * hi + (r % 4);
     float v = red[r * 64 + lane];
 #pragma unroll
     for (int x = 1; x < 4; ++x) v += red[(x * 16 + r) * 64 + lane];
@@ -1153,7 +1154,7 @@ __global__ __launch_bounds__(256) void gemm_tn_mid_kernel(unsigned M, unsigned N
 
 static bool mid_tn_eligible(const dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B,
                             size_t ldb) {
-  return N >= 5 && N <= 32 && M >= 32 && M <= (size_t(1) << 30) && K >= 256 && K % 4 == 0 && K <= 0x7FFFFFF0ull &&
+  return N >= 5 && N <= 256 && M >= 32 && M <= (size_t(1) << 30) && K >= 256 && K % 4 == 0 && K <= 0x7FFFFFF0ull &&
          lda % 4 == 0 && ldb % 4 == 0 && aligned16(A) && aligned16(B) && dev->gemm_ws != nullptr;
 }
 
@@ -1161,7 +1162,8 @@ static int mid_tn_run(dyhip_device* dev, size_t M, size_t N, size_t K, const flo
                       float beta, float* C) {
   const unsigned tiles = static_cast<unsigned>(cdiv<size_t>(M, 32)), Ku = static_cast<unsigned>(K);
   // depth slices: a block a CU, each with at least one round per wavefront
-  unsigned slabs = cdiv<unsigned>(unsigned(dev->num_cus > 0 ? dev->num_cus : 256), tiles);
+  const unsigned ct = cdiv<unsigned>(unsigned(N), 32);
+  unsigned slabs = cdiv<unsigned>(unsigned(dev->num_cus > 0 ? dev->num_cus : 256), tiles * ct);
   const unsigned max_by_depth = cdiv<unsigned>(Ku, 4 * kTnMidDepth);
   if (slabs > max_by_depth) slabs = max_by_depth;
   if (slabs < 1) slabs = 1;
@@ -1174,11 +1176,11 @@ static int mid_tn_run(dyhip_device* dev, size_t M, size_t N, size_t K, const flo
     DYHIP_REQUIRE(dev->gemm_ws_bytes >= sizeof(float) * M * N * slabs, "transposed small-batch product: workspace too small");
     partial = static_cast<float*>(dev->gemm_ws);
   }
-  const dim3 grid(tiles, slabs), block(256);
+  const dim3 grid(tiles, slabs, ct), block(256);
 #define DYHIP_TN_MID(NB4)                                                                                          \
   hipLaunchKernelGGL(gemm_tn_mid_kernel<NB4>, grid, block, 0, dev->stream, static_cast<unsigned>(M), static_cast<unsigned>(N), \
                      Ku, chunk, per_wave, A, lda, B, ldb, beta, C, partial)
-  switch ((N + 3) / 4) {
+  switch (N >= 32 ? 8u : unsigned(N + 3) / 4) {
     case 2: DYHIP_TN_MID(2); break;
     case 3: DYHIP_TN_MID(3); break;
     case 4: DYHIP_TN_MID(4); break;
@@ -1239,7 +1241,11 @@ int skinny_tn_gemm(dyhip_device* dev, size_t M, size_t N, size_t K, const float*
                  !(M * N > (size_t(1) << 19) || lda % 4 != 0 || ldb % 4 != 0 || !aligned16(A) || !aligned16(B));
   frag_ok = frag_ok && skinny_tn_splits(unsigned(M), unsigned(N), unsigned(K)) != 0 && dev->gemm_ws != nullptr &&
             dev->gemm_ws_bytes >= sizeof(float) * M * N * 16;
-  if (C != nullptr && mid_tn_eligible(dev, M, N, K, A, lda, B, ldb)) {
+  // beyond 64 columns (tiles of 32, each re-reading A) only for a small A or where the fragment-order product does
+  // not apply: 256 x 128 x 4096 9.8 against 11.1 us, 1024 x 40 x 10 000 24.1 against 31.6 us, but 1024 x 128 x 4096
+  // 20.4 against 18.4 us
+  if (C != nullptr && mid_tn_eligible(dev, M, N, K, A, lda, B, ldb) &&
+      (N <= 64 || !frag_ok || M * K * sizeof(float) <= (size_t(8) << 20))) {
     DYHIP_CHECK_STATUS(mid_tn_run(dev, M, N, K, A, lda, B, ldb, beta, C));
     *taken = true;
     return DYHIP_OK;

@@ -108,7 +108,8 @@ def test_gemm_nt_thin(dev, M, N, K):
 # four, row counts that do not fill the last block or tile, depths that end inside a 64-index round, any beta.
 @pytest.mark.parametrize("M,N,K", [(1024, 20, 4096), (128, 32, 1024), (650, 20, 2600), (1000, 1, 4000), (37, 7, 256),
                                    (1024, 13, 6000), (258, 4, 1024), (255, 29, 2048), (1024, 20, 10000), (33, 5, 260),
-                                   (100, 32, 1004), (2048, 9, 516), (4100, 31, 772), (32, 16, 100000), (1024, 6, 300)])
+                                   (100, 32, 1004), (2048, 9, 516), (4100, 31, 772), (32, 16, 100000), (1024, 6, 300),
+                                   (256, 128, 4096), (500, 47, 1028), (1024, 40, 2000), (100, 256, 512), (333, 65, 1300)])
 def test_gemm_tn_thin(dev, M, N, K):
     rng = np.random.default_rng(M + N + K)
     y0 = f32(rng.standard_normal((N, M)))
