@@ -1078,9 +1078,15 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
   if ((batch == nullptr || batch->count <= 1) && !a_kmajor && b_kmajor && C != nullptr &&
       gemm_nn_mid_eligible(dev, M, N, nseg, segs, C, epi))
     return gemm_nn_mid_run(dev, M, N, nseg, segs, C, epi);
+  // a depth of at most 32: the rank-K update, except for outputs above 4 MB at a depth of 24 or 32, where its
+  // re-reads of the left operand (once per eight columns, from the L2s) cost more than the burst-fetch kernel's
+  // matrix-core tiles (4096 x 1024: depth 16 8.9 against 9.1 us, depth 24 13.2 against 9.6 us, depth 32 15.4 against
+  // 10.1 us; 1024 x 1024 x 32: 5.3 against 7.7 us)
   if (nseg == 1 && (batch == nullptr || batch->count <= 1) && !a_kmajor && !b_kmajor && epi.kind == kEpiAxpby &&
       segs[0].A != nullptr && segs[0].B != nullptr && C != nullptr &&
-      gemm_nt_thin_eligible(M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, C, epi.beta))
+      gemm_nt_thin_eligible(M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, C, epi.beta) &&
+      !(segs[0].K >= 24 && M * N * sizeof(float) > (size_t(4) << 20) &&
+        gemm_shallow_nt_eligible(dev, M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, segs[0].ldb, C)))
     return gemm_nt_thin_run(dev, M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, segs[0].ldb, C, epi.beta);
   if (nseg == 1 && (batch == nullptr || batch->count <= 1) && !a_kmajor && !b_kmajor && epi.kind == kEpiAxpby &&
       segs[0].A != nullptr && segs[0].B != nullptr &&

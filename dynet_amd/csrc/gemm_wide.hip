@@ -732,7 +732,7 @@ int gemm_wide_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, siz
 
 bool gemm_shallow_nt_eligible(const dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda,
                               const float* B, size_t ldb, const float* C) {
-  if (K < 32 || K > 128 || K % 8 != 0 || M % 4 != 0 || N % 4 != 0 || M < 128 || N < 128) return false;
+  if (K < 24 || K > 128 || K % 8 != 0 || M % 4 != 0 || N % 4 != 0 || M < 128 || N < 128) return false;
   if (dev->max_lds_per_block < kShallowLdsBytes) return false;
   if (!aligned16(A) || !aligned16(B) || lda % 4 != 0 || ldb % 4 != 0 || (reinterpret_cast<uintptr_t>(C) & 7u) != 0)
     return false;
