@@ -81,9 +81,11 @@ def test_gemm_nt_shallow(dev, M, N, K):
 
 # l * r^T with a depth of at most 32 (the weight gradient of one timestep at a small batch) is a rank-K update of a matrix
 # read and written once: depths on both sides of every multiple of four, column counts that do not fill the last group
-# of eight, the baseline's smallest cell (1024 x 128 x 32), accumulate and overwrite.
+# of eight, the baseline's smallest cell (1024 x 128 x 32), accumulate and overwrite.  Outputs above 4 MB at depths 24
+# and 32 take the burst-fetch matrix-core kernel (ragged tile edges included).
 @pytest.mark.parametrize("M,N,K", [(1024, 128, 32), (4096, 1024, 20), (2052, 1030, 7), (256, 5, 1), (6000, 1500, 13),
-                                   (1024, 256, 4), (1024, 255, 29), (512, 9, 16)])
+                                   (1024, 256, 4), (1024, 255, 29), (512, 9, 16), (4096, 1024, 24), (4096, 1024, 32),
+                                   (2052, 1028, 24), (1500, 1000, 32)])
 def test_gemm_nt_thin(dev, M, N, K):
     rng = np.random.default_rng(M + N + K)
     y0 = f32(rng.standard_normal((N, M)))
