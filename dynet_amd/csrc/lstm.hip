@@ -749,29 +749,36 @@ __global__ __launch_bounds__(256) void skinny_nn_kernel(unsigned M, unsigned H, 
       step_product<kFragAlongRows, true, TILES, B_BYTES>(acc0, acc1, pk + r0, pk + r1, pb, ghi - glo, op.ldw);
     }
   } else {
-    // Depths off that grid (even all the same): each product's leading multiple of 128 is split over the waves as
-    // above; what is left of it, at most 15 groups of 8 k and a group cut short after 2, 4 or 6, is dealt to the waves
-    // one group at a time and multiplied in one round of loads (a pair of k past the end is fetched from k = 0 and its
-    // v entries zeroed).
-    for (int which = 0; which < 2; ++which) {
-      const NnOperand op = which == 0 ? op0 : op1;
-      if (op.K == 0) continue;
-      const unsigned G = op.K / 8, main = G / 16 * 16, per = main / 4;
-      if (per > 0) {
-        const unsigned g0 = wave * per;
-        const float* pk = op.W + (size_t(g0) * 8 + 4 * lhi) * op.ldw;
-        const float* pb = op.v + size_t(pcol) * op.ldv + size_t(g0) * 8 + 4 * lhi;
-        step_product<kFragAlongRows, true, TILES, B_BYTES>(acc0, acc1, pk + r0, pk + r1, pb, per, op.ldw);
-      }
-      const unsigned rem = op.K - 8 * G, items = G - main + (rem != 0 ? 1u : 0u);  // rem: 0, 2, 4 or 6 k past the groups
-      if (wave >= items) continue;
+    // Depths off that grid (even all the same): the waves are dealt to the two products in proportion to their depths
+    // (all four to a single product), so that a wave still runs one pass of the load pipeline.  The waves of a product
+    // split its leading whole rounds of four groups each; what is left of it, fewer than four groups a wave and a
+    // group cut short after 2, 4 or 6 k, is dealt to them one group at a time and multiplied in one round of loads
+    // (a pair of k past the end is fetched from k = 0 and its v entries zeroed).
+    const unsigned Kt = op0.K + op1.K;
+    unsigned w0 = 4;
+    if (op1.K != 0) {
+      w0 = (4 * op0.K + Kt / 2) / Kt;
+      w0 = w0 < 1 ? 1 : w0 > 3 ? 3 : w0;
+    }
+    const bool first = wave < w0;
+    const NnOperand op = first ? op0 : op1;
+    const unsigned wq = first ? w0 : 4 - w0, wl = first ? wave : wave - w0;
+    const unsigned G = op.K / 8, per = G / (4 * wq) * 4, main = per * wq;
+    if (per > 0) {
+      const unsigned g0 = wl * per;
+      const float* pk = op.W + (size_t(g0) * 8 + 4 * lhi) * op.ldw;
+      const float* pb = op.v + size_t(pcol) * op.ldv + size_t(g0) * 8 + 4 * lhi;
+      step_product<kFragAlongRows, true, TILES, B_BYTES>(acc0, acc1, pk + r0, pk + r1, pb, per, op.ldw);
+    }
+    const unsigned rem = op.K - 8 * G, items = G - main + (rem != 0 ? 1u : 0u);  // rem: 0, 2, 4 or 6 k past the groups
+    if (wl < items) {
       float a0[4][4], a1[4][4], bf[4][4];
 #pragma unroll
       for (int it = 0; it < 4; ++it) {
-        const unsigned g = main + wave + 4 * it, k = 8 * g + 4 * lhi;
+        const unsigned idx = wl + wq * it, g = main + idx, k = 8 * g + 4 * lhi;
 #pragma unroll
         for (int pr = 0; pr < 2; ++pr) {  // the fragment's two pairs of k: inside the depth together or not at all
-          const bool valid = k + 2 * pr + 1 < op.K;
+          const bool valid = idx < items && k + 2 * pr + 1 < op.K;
           const unsigned kp = valid ? k + 2 * pr : 0u;
           const float2 t = *reinterpret_cast<const float2*>(op.v + size_t(pcol) * op.ldv + kp);
           bf[it][2 * pr] = valid ? t.x : 0.f;
