@@ -29,7 +29,7 @@ HOT = ["ew_vec4_kernel<2, true, 0, true, 2, dyhip::AccMul2", "ew_vec4_kernel<1, 
        "gemm_wide_kernel<false, false>", "gemm_shallow_nt_kernel", "gemm_tile_kernel<false, false, 1, 2>",
        "gather_segments_kernel<true, true>", "sgd_scaled_kernel<true, true>", "philox",
        "gemm_nn_mid_kernel<true>", "gemm_nn_rows_kernel<1, 8, 4>", "gemm_nn_thin_kernel<1>", "gemm_nt_thin_kernel<32, 4>",
-       "gemm_tn_thin_kernel<4>", "ln_fwd_group_kernel<16, 1, 2, true>", "ln_bwd_group_kernel<16, 1, true>",
+       "gemm_tn_thin_kernel<4, 2>", "ln_fwd_group_kernel<16, 1, 2, true>", "ln_bwd_group_kernel<16, 1, true>",
        "sum_group_kernel<false, false>", "softmax_resident_kernel<0, 256, 4>", "moment_resident_kernel<1, 256, 4>"]
 
 KINDS = [

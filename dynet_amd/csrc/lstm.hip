@@ -1006,8 +1006,9 @@ static int skinny_tn(dyhip_device* dev, unsigned M, unsigned N, unsigned K, cons
 // cross the block once at the end (wavefront sums, then LDS in ascending wavefront order).  No matrix cores: at 20
 // columns the product is 80 multiply-adds per 16 bytes of A, and a 32-column matrix-core tile would read A in
 // 128-byte pieces (the fragment-order kernel above takes 13.6 us for 16.8 MB of A at N = 20).
-constexpr int kThinTnCols = 4;
-template <int NP>  // N rounded up to a multiple of four
+// kThinTnCols: columns of A a block owns: four for more than 4096 output rows, two down to 513, one below (more,
+// smaller blocks: 1024 x 1 x 4096 6.3 -> 5.4 us, 256 x 1 x 1024 3.7 -> 2.7 us; 10 000 x 1 x 1024 9.2 against 9.5 us)
+template <int NP, int kThinTnCols>  // NP: N rounded up to a multiple of four
 __global__ __launch_bounds__(256) void gemm_tn_thin_kernel(unsigned M, unsigned N, unsigned K4, const float* __restrict__ A,
                                                            size_t lda, const float* __restrict__ B, size_t ldb, float beta,
                                                            float* __restrict__ C) {
@@ -1214,10 +1215,17 @@ static bool thin_tn_eligible(size_t M, size_t N, size_t K, const float* A, size_
 
 static int thin_tn_run(dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B,
                        size_t ldb, float beta, float* C) {
-  const dim3 grid(static_cast<unsigned>(cdiv<size_t>(M, kThinTnCols))), block(256);
-#define DYHIP_THIN_TN(NP)                                                                                       \
-  hipLaunchKernelGGL(gemm_tn_thin_kernel<NP>, grid, block, 0, dev->stream, static_cast<unsigned>(M),           \
+  const int cols = M > 4096 ? 4 : M > 512 ? 2 : 1;
+  const dim3 grid(static_cast<unsigned>(cdiv<size_t>(M, cols))), block(256);
+#define DYHIP_THIN_TN_C(NP, CC)                                                                                 \
+  hipLaunchKernelGGL((gemm_tn_thin_kernel<NP, CC>), grid, block, 0, dev->stream, static_cast<unsigned>(M),     \
                      static_cast<unsigned>(N), static_cast<unsigned>(K / 4), A, lda, B, ldb, beta, C)
+#define DYHIP_THIN_TN(NP)                      \
+  do {                                         \
+    if (cols == 4) DYHIP_THIN_TN_C(NP, 4);     \
+    else if (cols == 2) DYHIP_THIN_TN_C(NP, 2); \
+    else DYHIP_THIN_TN_C(NP, 1);               \
+  } while (0)
   switch ((N + 3) / 4) {
     case 1: DYHIP_THIN_TN(4); break;
     case 2: DYHIP_THIN_TN(8); break;
@@ -1228,6 +1236,7 @@ static int thin_tn_run(dyhip_device* dev, size_t M, size_t N, size_t K, const fl
     case 7: DYHIP_THIN_TN(28); break;
     default: DYHIP_THIN_TN(32); break;
   }
+#undef DYHIP_THIN_TN_C
 #undef DYHIP_THIN_TN
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
