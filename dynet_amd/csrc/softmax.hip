@@ -447,20 +447,30 @@ constexpr int kSmThreads = 256;
 constexpr int kSmUnroll = 4;
 
 // red[c] = sum_i a[i,c] * (b ? b[i,c] : 1), one block per column, fixed summation tree
-__global__ __launch_bounds__(kSmThreads) void col_dot_kernel(size_t rows, const float* __restrict__ a,
-                                                            const float* __restrict__ b, float* __restrict__ red) {
-  __shared__ float sh[kSmThreads / 64];
+constexpr int kColDotThreads = 1024;  // columns of more than 16 384 rows: 256 threads walked 50 000 rows x 20 columns in 20 us
+__global__ __launch_bounds__(kColDotThreads) void col_dot_kernel(size_t rows, const float* __restrict__ a,
+                                                               const float* __restrict__ b, float* __restrict__ red) {
+  __shared__ float sh[kColDotThreads / 64];
   const size_t c0 = size_t(blockIdx.x) * rows;
+  // eight loads in flight a thread (a loop of one load and one add runs one memory round trip per step: 50 000 rows
+  // x 20 columns took 59 us); entries past the end are fetched from the column's last row and not added
   float s = 0.f;
-  for (size_t i = threadIdx.x; i < rows; i += kSmThreads) s += b ? a[c0 + i] * b[c0 + i] : a[c0 + i];
-  const float t = block_sum<kSmThreads / 64>(s, sh);
+  for (size_t i0 = threadIdx.x; i0 < rows; i0 += size_t(kColDotThreads) * 4) {
+    float x[4], y[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const size_t i = i0 + size_t(u) * kColDotThreads, ic = i < rows ? i : rows - 1;
+      x[u] = a[c0 + ic];
+      y[u] = b ? b[c0 + ic] : 1.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (i0 + size_t(u) * kColDotThreads < rows) s += b ? x[u] * y[u] : x[u];
+  }
+  const float t = block_sum<kColDotThreads / 64>(s, sh);
   if (threadIdx.x == 0) red[blockIdx.x] = t;
 }
 
-// MODE 0: fx = exp(x - m) * exp(m - z)         softmax forward   (s0 = m, s1 = z = log sum exp)
-// MODE 1: fx = x - z                            log-softmax forward (s0 = z)
-// MODE 2: dx += (d - r) * f                     softmax backward  (a = fx, b = dEdf, s0 = r = sum fx*dEdf)
-// MODE 3: dx += exp(f) * -r + d                 log-softmax backward (a = fx, b = dEdf, s0 = r = sum dEdf)
 template <int MODE>
 __global__ __launch_bounds__(kSmThreads) void col_apply_kernel(size_t rows, unsigned tiles_per_col,
                                                               const float* __restrict__ a,
@@ -472,15 +482,25 @@ __global__ __launch_bounds__(kSmThreads) void col_apply_kernel(size_t rows, unsi
   const float p0 = s0[c];
   const float p1 = MODE == 0 ? expf(p0 - s1[c]) : 0.f;
   const size_t i0 = size_t(tile) * kSmThreads * kSmUnroll + threadIdx.x;
+  // every load of the tile first, on indices clamped into the column (loads inside the per-element branch wait for
+  // one another: 50 000 rows x 20 columns backward 25 us)
+  float va[kSmUnroll], vb[kSmUnroll], vo[kSmUnroll];
+#pragma unroll
+  for (int u = 0; u < kSmUnroll; ++u) {
+    const size_t i = i0 + size_t(u) * kSmThreads, e = c0 + (i < rows ? i : rows - 1);
+    va[u] = a[e];
+    vb[u] = MODE >= 2 ? b[e] : 0.f;
+    vo[u] = MODE >= 2 ? out[e] : 0.f;
+  }
 #pragma unroll
   for (int u = 0; u < kSmUnroll; ++u) {
     const size_t i = i0 + size_t(u) * kSmThreads;
     if (i >= rows) break;
     const size_t e = c0 + i;
-    if (MODE == 0) out[e] = expf(a[e] - p0) * p1;
-    else if (MODE == 1) out[e] = a[e] - p0;
-    else if (MODE == 2) out[e] += (b[e] - p0) * a[e];
-    else out[e] += (expf(a[e]) * -p0) + b[e];
+    if (MODE == 0) out[e] = expf(va[u] - p0) * p1;
+    else if (MODE == 1) out[e] = va[u] - p0;
+    else if (MODE == 2) out[e] = vo[u] + (vb[u] - p0) * va[u];
+    else out[e] = vo[u] + ((expf(va[u]) * -p0) + vb[u]);
   }
 }
 
@@ -875,7 +895,7 @@ int dyhip_softmax_backward(dyhip_device* dev, size_t rows, unsigned cols, const 
     DYHIP_CHECK_LAUNCH();
     return DYHIP_OK;
   }
-  hipLaunchKernelGGL(col_dot_kernel, dim3(cols), dim3(kSmThreads), 0, dev->stream, rows, fx, dEdf, r);
+  hipLaunchKernelGGL(col_dot_kernel, dim3(cols), dim3(kColDotThreads), 0, dev->stream, rows, fx, dEdf, r);
   DYHIP_CHECK_LAUNCH();
   return launch_col_apply<2>(dev, rows, cols, fx, dEdf, r, nullptr, dEdx);
 }
@@ -947,7 +967,7 @@ int dyhip_log_softmax_backward(dyhip_device* dev, size_t rows, unsigned cols, co
     DYHIP_CHECK_LAUNCH();
     return DYHIP_OK;
   }
-  hipLaunchKernelGGL(col_dot_kernel, dim3(cols), dim3(kSmThreads), 0, dev->stream, rows, dEdf, nullptr, r);
+  hipLaunchKernelGGL(col_dot_kernel, dim3(cols), dim3(kColDotThreads), 0, dev->stream, rows, dEdf, nullptr, r);
   DYHIP_CHECK_LAUNCH();
   return launch_col_apply<3>(dev, rows, cols, fx, dEdf, r, nullptr, dEdx);
 }
