@@ -1279,7 +1279,7 @@ def test_pnls_label_out_of_range_is_an_error(dev):
 
 
 @pytest.mark.parametrize("rows,cols", [(10000, 128), (37, 5), (1027, 3), (1, 4), (4, 1), (50000, 64), (33, 700), (130, 9),
-                                       (300, 40), (513, 3), (100, 6), (3000, 5), (5000, 3), (16384, 2), (16385, 2), (100003, 3), (20001, 20)])
+                                       (300, 40), (513, 3), (100, 6), (3000, 5), (5000, 3), (16384, 2), (16385, 2), (40001, 3), (20001, 20)])
 def test_softmax_and_log_softmax(dev, rows, cols):
     rng = np.random.default_rng(rows + cols)
     x = f32(rng.standard_normal((cols, rows)) * 2)
