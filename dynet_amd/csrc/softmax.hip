@@ -371,29 +371,58 @@ __global__ __launch_bounds__(256) void onehot_kernel(size_t rows, size_t total, 
 }
 
 // ---- argmax along dim 0, first maximum ---------------------------------------
-__global__ __launch_bounds__(256) void argmax_cols_kernel(size_t rows, const float* __restrict__ x,
-                                                          long long* __restrict__ idx) {
-  __shared__ float lv[4];
-  __shared__ unsigned long long li[4];
-  const float* px = x + size_t(blockIdx.x) * rows;
-  float bv = -INFINITY;
-  unsigned long long bi = ~0ull;
-  for (size_t i = threadIdx.x; i < rows; i += 256) {
-    const float v = px[i];
-    if (bi == ~0ull || v > bv) {  // strided ascending i: strict > keeps the first maximum
-      bv = v;
-      bi = i;
+// (value, index) of the better of two candidates: the greater value, the lower index among equal values; an index of
+// ~0 marks "none yet"
+__device__ __forceinline__ void argmax_take(float& bv, unsigned long long& bi, float ov, unsigned long long oi) {
+  if (oi != ~0ull && (bi == ~0ull || ov > bv || (ov == bv && oi < bi))) {
+    bv = ov;
+    bi = oi;
+  }
+}
+
+// A thread's scan of elements first, first + step, ... of a column: eight loads in flight (one load and one compare
+// a step is one memory round trip a step: 50 000 rows x 512 columns took 93 us, 1.1 TB/s); ascending order, so a
+// strict > keeps the first maximum.  Entries past the end are fetched from the column's last row and skipped.
+__device__ __forceinline__ void argmax_scan(const float* __restrict__ px, size_t rows, size_t first, size_t step, float& bv,
+                                            unsigned long long& bi) {
+  for (size_t i0 = first; i0 < rows; i0 += 8 * step) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const size_t i = i0 + u * step;
+      v[u] = px[i < rows ? i : rows - 1];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const size_t i = i0 + u * step;
+      if (i < rows && (bi == ~0ull || v[u] > bv)) {
+        bv = v[u];
+        bi = i;
+      }
     }
   }
+}
+
+__device__ __forceinline__ void argmax_wave(float& bv, unsigned long long& bi) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
     const float ov = __shfl_xor(bv, off, kWave);
     const unsigned long long oi = __shfl_xor(bi, off, kWave);
-    if (oi != ~0ull && (bi == ~0ull || ov > bv || (ov == bv && oi < bi))) {
-      bv = ov;
-      bi = oi;
-    }
+    argmax_take(bv, bi, ov, oi);
   }
+}
+
+// one block per column (columns of more than 2048 rows)
+template <int T>
+__global__ __launch_bounds__(T) void argmax_cols_kernel(size_t rows, const float* __restrict__ x,
+                                                        long long* __restrict__ idx) {
+  __shared__ float lv[T / 64];
+  __shared__ unsigned long long li[T / 64];
+  const float* px = x + size_t(blockIdx.x) * rows;
+  float bv = -INFINITY;
+  unsigned long long bi = ~0ull;
+  argmax_scan(px, rows, threadIdx.x, T, bv, bi);
+  argmax_wave(bv, bi);
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   if (lane == 0) {
     lv[w] = bv;
@@ -401,13 +430,43 @@ __global__ __launch_bounds__(256) void argmax_cols_kernel(size_t rows, const flo
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    for (int k = 1; k < 4; ++k)
-      if (li[k] != ~0ull && (bi == ~0ull || lv[k] > bv || (lv[k] == bv && li[k] < bi))) {
-        bv = lv[k];
-        bi = li[k];
-      }
+    for (int k = 1; k < T / 64; ++k) argmax_take(bv, bi, lv[k], li[k]);
     idx[blockIdx.x] = static_cast<long long>(bi);
   }
+}
+
+// one wavefront per column (33..2048 rows), four columns a block
+__global__ __launch_bounds__(256) void argmax_cols_wave_kernel(size_t rows, unsigned cols, const float* __restrict__ x,
+                                                               long long* __restrict__ idx) {
+  const unsigned c = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (c >= cols) return;
+  float bv = -INFINITY;
+  unsigned long long bi = ~0ull;
+  argmax_scan(x + size_t(c) * rows, rows, threadIdx.x & 63, 64, bv, bi);
+  argmax_wave(bv, bi);
+  if ((threadIdx.x & 63) == 0) idx[c] = static_cast<long long>(bi);
+}
+
+// one thread per column (at most 32 rows: a block per column left 252 of 256 threads idle on 4-row columns)
+__global__ __launch_bounds__(256) void argmax_cols_thread_kernel(size_t rows, unsigned cols, const float* __restrict__ x,
+                                                                 long long* __restrict__ idx) {
+  const unsigned c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= cols) return;
+  float bv = -INFINITY;
+  unsigned long long bi = ~0ull;
+  argmax_scan(x + size_t(c) * rows, rows, 0, 1, bv, bi);
+  idx[c] = static_cast<long long>(bi);
+}
+
+static void launch_argmax_cols(dyhip_device* dev, size_t rows, unsigned bd, const float* x, long long* idx) {
+  if (rows <= 32)
+    hipLaunchKernelGGL(argmax_cols_thread_kernel, dim3(cdiv<unsigned>(bd, 256)), dim3(256), 0, dev->stream, rows, bd, x, idx);
+  else if (rows <= 2048)
+    hipLaunchKernelGGL(argmax_cols_wave_kernel, dim3(cdiv<unsigned>(bd, 4)), dim3(256), 0, dev->stream, rows, bd, x, idx);
+  else if (rows <= 8192)
+    hipLaunchKernelGGL(argmax_cols_kernel<256>, dim3(bd), dim3(256), 0, dev->stream, rows, x, idx);
+  else
+    hipLaunchKernelGGL(argmax_cols_kernel<1024>, dim3(bd), dim3(1024), 0, dev->stream, rows, x, idx);
 }
 
 int batch_reduce(dyhip_device* dev, size_t n, unsigned bd, const float* in0, const float* in1, float* out,
@@ -849,7 +908,7 @@ int dyhip_argmax_cols(dyhip_device* dev, size_t rows, unsigned bd, const float* 
   DYHIP_CHECK_DEV(dev);
   DYHIP_REQUIRE(rows >= 1 && x && idx, "argmax needs a non-empty tensor");
   if (bd == 0) return DYHIP_OK;
-  hipLaunchKernelGGL(argmax_cols_kernel, dim3(bd), dim3(256), 0, dev->stream, rows, x, idx);
+  launch_argmax_cols(dev, rows, bd, x, idx);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
@@ -858,7 +917,7 @@ int dyhip_argmax_onehot_forward(dyhip_device* dev, size_t rows, unsigned bd, con
   DYHIP_CHECK_DEV(dev);
   DYHIP_REQUIRE(rows >= 1 && x && idx && fx, "argmax needs a non-empty tensor");
   if (bd == 0) return DYHIP_OK;
-  hipLaunchKernelGGL(argmax_cols_kernel, dim3(bd), dim3(256), 0, dev->stream, rows, x, idx);
+  launch_argmax_cols(dev, rows, bd, x, idx);
   DYHIP_CHECK_LAUNCH();
   const size_t total = rows * size_t(bd);
   hipLaunchKernelGGL(onehot_kernel, dim3((unsigned)cdiv<size_t>(total, 256)), dim3(256), 0, dev->stream, rows, total, idx, fx);

@@ -1340,6 +1340,21 @@ def test_argmax(dev, golden):
     assert idx.numpy().tobytes() == orc.argmax_cols(5000, 9, x).tobytes()
 
 
+@pytest.mark.parametrize("rows,bd", [(1, 7), (4, 100001), (32, 1000), (33, 999), (64, 5), (2048, 33), (2049, 3), (8192, 4),
+                                     (8193, 2), (50000, 9), (100003, 1)])
+def test_argmax_shapes_with_ties(dev, rows, bd):
+    """A thread, a wavefront or a block (256 / 1024 threads) per column, on both sides of each limit; small integer
+    values, so that every column holds its maximum many times: the first one wins, as in the oracle."""
+    rng = np.random.default_rng(rows + bd)
+    x = f32(rng.integers(0, 7, (bd, rows)))
+    idx = dev.empty(bd, np.int64)
+    dev.argmax_cols(rows, bd, dev.tensor(x), idx)
+    assert idx.numpy().tobytes() == orc.argmax_cols(rows, bd, x).tobytes()
+    x = f32(rng.standard_normal((bd, rows)))
+    dev.argmax_cols(rows, bd, dev.tensor(x), idx)
+    assert np.array_equal(idx.numpy(), x.argmax(axis=1))
+
+
 def test_argmax_node(dev, golden):
     """The Argmax node (dynet/nodes-argmax.cc:44-68): one-hot forward with the reference test's vector, bit-exact against
     the oracle on a larger case with ties, straight-through backward = accumulate."""
