@@ -324,11 +324,12 @@ __global__ __launch_bounds__(kPbThreads) void pnls_bwd_kernel(size_t rows, unsig
 }
 
 // ---- LogSumExp node over k <= 8 arguments -----------------------------------
-constexpr unsigned kLseNodeMaxArgs = 8;
+constexpr unsigned kLseNodeMaxArgs = 32;  // arguments a launch takes; more are chained (below)
 struct LseNodeArgs {
   const float* x[kLseNodeMaxArgs];
-  unsigned bcast[kLseNodeMaxArgs];  // 1 => batch 1, indexed by e % n
+  unsigned bcast;  // bit i: argument i has batch 1 and is indexed by e % n
   unsigned k;
+  unsigned last;   // the launch that leaves the node's value (not a link of a chain)
 };
 
 __global__ __launch_bounds__(256) void lse_node_fwd_kernel(LseNodeArgs a, size_t n, size_t total,
@@ -336,11 +337,31 @@ __global__ __launch_bounds__(256) void lse_node_fwd_kernel(LseNodeArgs a, size_t
   const size_t e = size_t(blockIdx.x) * 256 + threadIdx.x;
   if (e >= total) return;
   const size_t j = e % n;
-  float m = a.x[0][a.bcast[0] ? j : e];
-  for (unsigned i = 1; i < a.k; ++i) m = fmaxf(m, a.x[i][a.bcast[i] ? j : e]);
-  float s = 0.f;
-  for (unsigned i = 0; i < a.k; ++i) s += expf(a.x[i][a.bcast[i] ? j : e] - m);
-  fx[e] = logf(s) + m;
+  // the arguments' values are fetched once, four at a time in flight, into a running (max, sum of exp) pair
+  float m = -INFINITY, s = 0.f;
+  for (unsigned i0 = 0; i0 < a.k; i0 += 4) {
+    float v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const unsigned i = min(i0 + u, a.k - 1);
+      v[u] = a.x[i][(a.bcast >> i) & 1u ? j : e];
+    }
+    float mg = v[0];
+#pragma unroll
+    for (int u = 1; u < 4; ++u)
+      if (i0 + u < a.k) mg = fmaxf(mg, v[u]);
+    const float mn = fmaxf(m, mg);
+    // exp(-inf - -inf) would be NaN: a running maximum of -inf has no terms yet (or only -inf ones)
+    float t = mn == -INFINITY ? 0.f : s * expf(m - mn);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (i0 + u < a.k) t += mn == -INFINITY ? 1.f : expf(v[u] - mn);
+    m = mn;
+    s = t;
+  }
+  // arguments that are all -inf: the reference's exp(x - max) is exp(-inf + inf) = NaN there; a link of a chain keeps
+  // -inf, which later finite arguments absorb
+  fx[e] = (a.last != 0 && m == -INFINITY) ? __builtin_nanf("") : logf(s) + m;
 }
 
 // dxi[e] += exp(xi[e] - fx[e]) * dEdf[e]
@@ -860,20 +881,31 @@ int dyhip_pnls_backward_assign(dyhip_device* dev, size_t rows, unsigned bd, cons
 int dyhip_logsumexp_node_forward(dyhip_device* dev, unsigned k, size_t n, unsigned bd, const float* const* xs_host,
                                  const unsigned* bds_host, float* fx) {
   DYHIP_CHECK_DEV(dev);
-  DYHIP_REQUIRE(k >= 1 && k <= kLseNodeMaxArgs, "LogSumExp supports 1..%u arguments (got %u)", kLseNodeMaxArgs, k);
+  DYHIP_REQUIRE(k >= 1, "LogSumExp needs at least one argument");
   DYHIP_REQUIRE(xs_host && bds_host && fx, "null pointer");
   const size_t total = n * size_t(bd);
   if (total == 0) return DYHIP_OK;
-  LseNodeArgs a;
-  a.k = k;
-  for (unsigned i = 0; i < k; ++i) {
+  for (unsigned i = 0; i < k; ++i)
     DYHIP_REQUIRE(bds_host[i] == bd || bds_host[i] == 1, "Mismatched input dimensions in LogSumExp");
-    a.x[i] = xs_host[i];
-    a.bcast[i] = (bds_host[i] != bd) ? 1u : 0u;
+  // up to 32 arguments a launch; more are chained through the output, which joins the next launch as one more
+  // argument: logsumexp(a, b) with a = logsumexp of the earlier arguments is the logsumexp of all of them
+  unsigned at = 0;
+  while (at < k) {
+    LseNodeArgs a;
+    unsigned cnt = 0;
+    a.bcast = 0;
+    if (at > 0) a.x[cnt++] = fx;
+    while (cnt < kLseNodeMaxArgs && at < k) {
+      if (bds_host[at] != bd) a.bcast |= 1u << cnt;
+      a.x[cnt++] = xs_host[at++];
+    }
+    for (unsigned i = cnt; i < kLseNodeMaxArgs; ++i) a.x[i] = a.x[0];
+    a.k = cnt;
+    a.last = at == k ? 1u : 0u;
+    hipLaunchKernelGGL(lse_node_fwd_kernel, dim3((unsigned)cdiv<size_t>(total, 256)), dim3(256), 0, dev->stream, a, n,
+                       total, fx);
+    DYHIP_CHECK_LAUNCH();
   }
-  hipLaunchKernelGGL(lse_node_fwd_kernel, dim3((unsigned)cdiv<size_t>(total, 256)), dim3(256), 0, dev->stream, a, n,
-                     total, fx);
-  DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }
 
@@ -881,7 +913,7 @@ int dyhip_logsumexp_node_backward(dyhip_device* dev, unsigned k, size_t n, unsig
                                   const unsigned* bds_host, const float* fx, const float* dEdf, unsigned i,
                                   float* dEdxi, void* ws, size_t ws_bytes) {
   DYHIP_CHECK_DEV(dev);
-  DYHIP_REQUIRE(k >= 1 && k <= kLseNodeMaxArgs && i < k, "bad argument index %u of %u", i, k);
+  DYHIP_REQUIRE(k >= 1 && i < k, "bad argument index %u of %u", i, k);
   DYHIP_REQUIRE(xs_host && bds_host && fx && dEdf && dEdxi, "null pointer");
   const size_t total = n * size_t(bd);
   if (total == 0) return DYHIP_OK;

@@ -515,7 +515,8 @@ int dyhip_logsumexp_dim_backward(dyhip_device* dev, size_t rows, size_t cols, un
 int dyhip_log_softmax_forward(dyhip_device* dev, size_t rows, unsigned cols, const float* x, void* aux, float* fx);
 int dyhip_log_softmax_backward(dyhip_device* dev, size_t rows, unsigned cols, const float* fx, const float* dEdf,
                                void* aux, float* dEdx);
-/* LogSumExp node over k <= 8 arguments (dynet/nodes-logsumexp.cc:38-97) */
+/* LogSumExp node over any number k >= 1 of arguments (dynet/nodes-logsumexp.cc:38-97; up to 32 in one launch, more
+ * chained through fx).  An entry whose arguments are all -inf is NaN, as in the reference. */
 int dyhip_logsumexp_node_forward(dyhip_device* dev, unsigned k, size_t n, unsigned bd, const float* const* xs_host,
                                  const unsigned* bds_host, float* fx);
 int dyhip_logsumexp_node_backward(dyhip_device* dev, unsigned k, size_t n, unsigned bd, const float* const* xs_host,

@@ -1328,6 +1328,36 @@ def test_logsumexp_node(dev):
         assert_close(gt.numpy(), want, GRAD_RTOL, "LogSumExp bwd %d" % i, floor=1e-2)
 
 
+@pytest.mark.parametrize("k,n,bd", [(9, 300, 4), (32, 50, 3), (33, 50, 3), (35, 1, 128), (100, 7, 2), (64, 1, 1)])
+def test_logsumexp_node_many_arguments(dev, k, n, bd):
+    """More arguments than one launch takes (32): chained through the output.  Mixed batch sizes, a few -inf entries,
+    every argument's gradient."""
+    rng = np.random.default_rng(k + n + bd)
+    bds = [bd if (i % 3 != 1 or bd == 1) else 1 for i in range(k)]
+    xs = [f32(rng.standard_normal((b, n)) * 3) for b in bds]
+    xs[0][0, 0] = -np.inf
+    ts = [dev.tensor(v) for v in xs]
+    fx = dev.empty((bd, n))
+    dev.logsumexp_node_forward(n, bd, ts, bds, fx)
+    ref = orc.logsumexp_node_forward(n, bd, xs, bds)
+    assert_close(fx.numpy(), ref, FWD_RTOL, "LogSumExp fwd", floor=1.0)
+    exact = np.log(sum(np.exp(np.broadcast_to(v, (bd, n)).astype(np.float64)) for v in xs))
+    assert_close(fx.numpy(), exact, FWD_RTOL, "LogSumExp fwd vs fp64", floor=1.0)
+    dy = f32(rng.standard_normal((bd, n)))
+    for i in (0, 1, k - 1):
+        g0 = f32(rng.standard_normal((bds[i], n)))
+        gt = dev.tensor(g0)
+        dev.logsumexp_node_backward(n, bd, ts, bds, dev.tensor(ref), dev.tensor(dy), i, gt)
+        want = orc.logsumexp_node_backward(n, bd, xs, bds, ref, dy, i, g0.copy())
+        assert_close(gt.numpy(), want, GRAD_RTOL, "LogSumExp bwd %d" % i, floor=1e-2 * np.sqrt(bd))
+    # every argument -inf in one entry: NaN there, as the reference's exp(-inf + inf)
+    for v in xs:
+        v[-1, -1] = -np.inf
+    dev.logsumexp_node_forward(n, bd, [dev.tensor(v) for v in xs], bds, fx)
+    got = fx.numpy()
+    assert np.isnan(got[-1, -1]) and np.isfinite(got.ravel()[:-1]).all()
+
+
 def test_argmax(dev, golden):
     t = golden["node_values"]["argmax"]
     idx = dev.empty(t["bd"], np.int64)
