@@ -706,57 +706,84 @@ constexpr int kRowWaves = 8;
 // MODE 0: m_out = max, z_out = log(sum) + max     (TensorTools::logsumexp_dev along axis 1)
 // MODE 1: out = exp(x - max) / sum                (Softmax forward, dimension 1)
 // MODE 2: out += (b - sum_j a*b) * a              (Softmax backward, dimension 1; a = fx, b = dEdf)
-template <int MODE>
-__global__ __launch_bounds__(64 * kRowWaves) void rowwise_kernel(unsigned rows, unsigned cols, unsigned bd,
+template <int MODE, int U>  // U: loads in flight a thread and pass (2 for few columns a thread, 8 otherwise)
+__global__ __launch_bounds__(64 * kRowWaves) void rowwise_kernel(unsigned rows, unsigned cols, unsigned bd, unsigned rw_shift,
                                                                  const float* __restrict__ a,
                                                                  const float* __restrict__ b,
                                                                  float* __restrict__ m_out, float* __restrict__ out) {
   __shared__ float red[kRowWaves][64];
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const unsigned row = blockIdx.x * 64 + lane;
+  // A wavefront's lanes: RW = 2^rw_shift consecutive rows x 64 / RW columns (matrices of fewer than 64 rows would
+  // leave lanes idle: 3 rows x 50 000 columns took 1.8 ms).  U loads in flight a thread in every pass, on column
+  // indices clamped into the matrix (one load and one compare a step is one memory round trip a step).
+  const unsigned lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const unsigned RW = 1u << rw_shift, nsub = 64u >> rw_shift, rl = lane & (RW - 1), sub = lane >> rw_shift;
+  const unsigned stride = kRowWaves * nsub, j0 = w * nsub + sub;
+  const unsigned row = blockIdx.x * RW + rl;
   const bool live = row < rows;
+  const unsigned rowc = live ? row : rows - 1;
   for (unsigned bi = blockIdx.y; bi < bd; bi += gridDim.y) {
-    const size_t base = size_t(bi) * rows * cols + row;
+    const size_t base = size_t(bi) * rows * cols + rowc;
     float mx = -INFINITY;
     if (MODE != 2) {
-      if (live)
-        for (unsigned j = w; j < cols; j += kRowWaves) {
-          const float v = a[base + size_t(j) * rows];
-          mx = v > mx ? v : mx;  // a NaN entry is skipped here and turns the row's sum into NaN below
-        }
+      for (unsigned j = j0; j < cols; j += U * stride) {
+        float v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = a[base + size_t(min(j + u * stride, cols - 1)) * rows];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          if (j + u * stride < cols) mx = v[u] > mx ? v[u] : mx;  // a NaN entry is skipped here and turns the row's sum into NaN below
+      }
       red[w][lane] = mx;
       __syncthreads();
-      mx = red[0][lane];
-#pragma unroll
-      for (int k = 1; k < kRowWaves; ++k) {
-        const float o = red[k][lane];
-        mx = o > mx ? o : mx;
-      }
+      mx = -INFINITY;
+      for (unsigned k = 0; k < kRowWaves; ++k)
+        for (unsigned s2 = 0; s2 < nsub; ++s2) {
+          const float o = red[k][(s2 << rw_shift) + rl];
+          mx = o > mx ? o : mx;
+        }
       __syncthreads();
     }
     float s = 0.f;
-    if (live)
-      for (unsigned j = w; j < cols; j += kRowWaves) {
-        const size_t e = base + size_t(j) * rows;
-        s += MODE == 2 ? a[e] * b[e] : expf(a[e] - mx);
+    for (unsigned j = j0; j < cols; j += U * stride) {
+      float v[U], y[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const size_t e = base + size_t(min(j + u * stride, cols - 1)) * rows;
+        v[u] = a[e];
+        y[u] = MODE == 2 ? b[e] : 0.f;
       }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (j + u * stride < cols) s += MODE == 2 ? v[u] * y[u] : expf(v[u] - mx);
+    }
     red[w][lane] = s;
     __syncthreads();
-    s = red[0][lane];
-#pragma unroll
-    for (int k = 1; k < kRowWaves; ++k) s += red[k][lane];
+    s = 0.f;
+    for (unsigned k = 0; k < kRowWaves; ++k)
+      for (unsigned s2 = 0; s2 < nsub; ++s2) s += red[k][(s2 << rw_shift) + rl];
     __syncthreads();
-    if (!live) continue;
     if (MODE == 0) {
-      if (w == 0) {
+      if (live && w == 0 && sub == 0) {
         m_out[size_t(bi) * rows + row] = mx;
         out[size_t(bi) * rows + row] = logf(s) + mx;
       }
     } else {
-      for (unsigned j = w; j < cols; j += kRowWaves) {
-        const size_t e = base + size_t(j) * rows;
-        if (MODE == 1) out[e] = expf(a[e] - mx) / s;
-        else out[e] += (b[e] - s) * a[e];
+      for (unsigned j = j0; j < cols; j += U * stride) {
+        float v[U], y[U], o[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const size_t e = base + size_t(min(j + u * stride, cols - 1)) * rows;
+          v[u] = a[e];
+          y[u] = MODE == 2 ? b[e] : 0.f;
+          o[u] = MODE == 2 ? out[e] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (!live || j + u * stride >= cols) continue;
+          const size_t e = base + size_t(j + u * stride) * rows;
+          if (MODE == 1) out[e] = expf(v[u] - mx) / s;
+          else out[e] = o[u] + (y[u] - s) * v[u];
+        }
       }
     }
   }
@@ -766,9 +793,16 @@ template <int MODE>
 static int launch_rowwise(dyhip_device* dev, size_t rows, size_t cols, unsigned bd, const float* a, const float* b,
                           float* m_out, float* out) {
   DYHIP_REQUIRE(rows < (size_t(1) << 31) && cols < (size_t(1) << 31), "matrix dimension too large");
-  const dim3 grid(static_cast<unsigned>(cdiv<size_t>(rows, 64)), bd < 65535u ? bd : 65535u);
-  hipLaunchKernelGGL(rowwise_kernel<MODE>, grid, dim3(64 * kRowWaves), 0, dev->stream, static_cast<unsigned>(rows),
-                     static_cast<unsigned>(cols), bd, a, b, m_out, out);
+  unsigned rw_shift = 6;  // row lanes a wavefront: the power of two that reaches the row count, at most 64
+  while (rw_shift > 0 && (size_t(1) << (rw_shift - 1)) >= rows) --rw_shift;
+  const dim3 grid(static_cast<unsigned>(cdiv<size_t>(rows, size_t(1) << rw_shift)), bd < 65535u ? bd : 65535u);
+  const size_t stride = size_t(kRowWaves) * (64u >> rw_shift);  // columns between a thread's consecutive elements
+  if (cols >= 4 * stride)
+    hipLaunchKernelGGL((rowwise_kernel<MODE, 8>), grid, dim3(64 * kRowWaves), 0, dev->stream, static_cast<unsigned>(rows),
+                       static_cast<unsigned>(cols), bd, rw_shift, a, b, m_out, out);
+  else
+    hipLaunchKernelGGL((rowwise_kernel<MODE, 2>), grid, dim3(64 * kRowWaves), 0, dev->stream, static_cast<unsigned>(rows),
+                       static_cast<unsigned>(cols), bd, rw_shift, a, b, m_out, out);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
 }

@@ -1797,7 +1797,10 @@ def test_zero_any_alignment_and_inside_a_graph(dev):
     g.destroy()
 
 
-@pytest.mark.parametrize("rows,cols,bd", [(7, 5, 3), (64, 100, 2), (130, 9, 1), (1, 300, 4), (1000, 33, 2), (3, 1, 5)])
+@pytest.mark.parametrize("rows,cols,bd", [(7, 5, 3), (64, 100, 2), (130, 9, 1), (1, 300, 4), (1000, 33, 2), (3, 1, 5),
+                                          # few rows and many columns (a wavefront folds its lanes over the columns), column
+                                          # counts around the eight loads a thread has in flight
+                                          (3, 8000, 2), (2, 1000, 3), (5, 4097, 1), (512, 512, 2), (33, 70, 2), (16, 129, 3)])
 def test_softmax_and_logsumexp_along_dim_1(dev, rows, cols, bd):
     rng = np.random.default_rng(rows + cols + bd)
     x = f32(rng.standard_normal((bd, cols, rows)) * 3)
