@@ -387,11 +387,133 @@ __global__ __launch_bounds__(kMomThreads) void std_bwd_kernel(size_t n, const fl
   }
 }
 
+// ---- long elements of a small batch (a block per element is then a handful of blocks: 4 elements of 1M floats took
+// 60 / 117 / 326 us for mean / std / std backward): an element is cut into chunks of kMomChunk floats, a 256-thread
+// block holds its chunk in registers and leaves the chunk's sum (MODE 0) or its mean and centered sum of squares
+// (MODE 1); a wavefront per element then merges the chunks in a fixed order (for the variance by the pairwise
+// update of means and centered sums, which is at least as accurate as the two passes it replaces).
+constexpr unsigned kMomChunk = 8192;
+template <int MODE>
+__global__ __launch_bounds__(256) void moment_chunk_kernel(size_t n, const float* __restrict__ x, float* __restrict__ stats) {
+  __shared__ float red[4];
+  const size_t c0 = size_t(blockIdx.x) * kMomChunk, c1 = min(n, c0 + kMomChunk);
+  const float* px = x + size_t(blockIdx.y) * n;
+  constexpr int U = kMomChunk / 256;
+  float v[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const size_t j = c0 + threadIdx.x + size_t(u) * 256;
+    v[u] = px[j < c1 ? j : c1 - 1];
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+    if (c0 + threadIdx.x + size_t(u) * 256 < c1) s += v[u];
+  const float sum = block_sum<4>(s, red);
+  const size_t at = size_t(blockIdx.y) * gridDim.x + blockIdx.x;
+  if (MODE == 0) {
+    if (threadIdx.x == 0) stats[at] = sum;
+    return;
+  }
+  const float mean = sum / float(c1 - c0);
+  float q = 0.f;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    if (c0 + threadIdx.x + size_t(u) * 256 < c1) {
+      const float d = v[u] - mean;
+      q += d * d;
+    }
+  }
+  const float m2 = block_sum<4>(q, red);
+  if (threadIdx.x == 0) {
+    stats[2 * at] = mean;
+    stats[2 * at + 1] = m2;
+  }
+}
+
+// the mean of an element from its chunk sums, by one wavefront (every lane returns it)
+__device__ __forceinline__ float moment_mean_of_chunks(const float* __restrict__ sums, unsigned chunks, size_t n, int lane) {
+  float s = 0.f;
+  for (unsigned c = lane; c < chunks; c += 64) s += sums[c];
+  return wave_sum(s) / float(n);
+}
+
+template <int MODE>
+__global__ __launch_bounds__(64) void moment_finish_kernel(size_t n, unsigned chunks, const float* __restrict__ stats,
+                                                          float* __restrict__ y) {
+  const int lane = threadIdx.x;
+  const unsigned b = blockIdx.x;
+  if (MODE == 0) {
+    const float mean = moment_mean_of_chunks(stats + size_t(b) * chunks, chunks, n, lane);
+    if (lane == 0) y[b] = mean;
+    return;
+  }
+  const float* st = stats + size_t(b) * chunks * 2;
+  auto count = [&](unsigned c) { return float(min(n, size_t(c + 1) * kMomChunk) - size_t(c) * kMomChunk); };
+  float s = 0.f;
+  for (unsigned c = lane; c < chunks; c += 64) s += count(c) * st[2 * c];
+  const float mean = wave_sum(s) / float(n);
+  float q = 0.f;
+  for (unsigned c = lane; c < chunks; c += 64) {
+    const float d = st[2 * c] - mean;
+    q += st[2 * c + 1] + count(c) * d * d;
+  }
+  const float m2 = wave_sum(q);
+  if (lane == 0) y[b] = sqrtf(m2 / float(n));
+}
+
+// dx[b, j] += (2/n) * (x - mean_b) * (dEdf[b] / (2 * fx[b])) with the mean from the chunk sums; a block per 1024 entries
+__global__ __launch_bounds__(256) void std_bwd_chunked_kernel(size_t n, unsigned chunks, const float* __restrict__ x,
+                                                              const float* __restrict__ sums, const float* __restrict__ fx,
+                                                              const float* __restrict__ dEdf, float* __restrict__ dEdx) {
+  const unsigned b = blockIdx.y;
+  const float mean = moment_mean_of_chunks(sums + size_t(b) * chunks, chunks, n, threadIdx.x & 63);
+  const float sb = dEdf[b] / (2.f * fx[b]);
+  const float c = 2.f / float(n);
+  const float* px = x + size_t(b) * n;
+  float* pd = dEdx + size_t(b) * n;
+  const size_t j0 = size_t(blockIdx.x) * 1024 + threadIdx.x;
+  float a[4], o[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const size_t j = j0 + size_t(u) * 256, jc = j < n ? j : n - 1;
+    a[u] = px[jc];
+    o[u] = pd[jc];
+  }
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const size_t j = j0 + size_t(u) * 256;
+    if (j < n) pd[j] = o[u] + c * (a[u] - mean) * sb;
+  }
+}
+
+// true: the element is long and the batch small enough for the chunked kernels, and the device's scratch holds the
+// chunk statistics
+static bool moment_chunked_fits(const dyhip_device* dev, size_t n, unsigned bd, unsigned* chunks) {
+  const size_t c = cdiv<size_t>(n, kMomChunk), cus = dev->num_cus > 0 ? size_t(dev->num_cus) : 256;
+  *chunks = static_cast<unsigned>(c);
+  return n > 16384 && bd < 2 * cus && c <= 0x7FFFFFFFull && bd <= 65535u && dev->gemm_ws != nullptr &&
+         dev->gemm_ws_bytes >= sizeof(float) * 2 * c * bd && cdiv<size_t>(n, 1024) <= 0x7FFFFFFFull;
+}
+
 // ---- the same three with the batch element held in registers: T threads own a batch element (a wavefront up to 512
 // floats, four elements to a block; a block of 256 threads up to 4096 floats, of 1024 threads up to 16384), thread t
 // holding entries t, t + T, ... (U of them): x is read once, every access of the group is one contiguous run, and a
 // short element does not occupy a 256-thread block (80 000 elements of 50 floats: 42 -> a few us for std_elems).
-// MODE 0: mean   1: std   2: std backward.  Longer elements keep the block-per-element kernels above.
+// MODE 0: mean   1: std   2: std backward.  Longer elements take the chunked kernels above when the batch is small and
+// the block-per-element kernels otherwise; elements of at most 32 floats take moment_group_kernel below.
+// the sum over a group of G adjacent lanes (G a power of two, 4..64), left in every lane of the group
+template <int G>
+__device__ __forceinline__ float group_sum(float v) {
+  v += dpp_move<0xB1, 0xF>(v, 0.f);                // quad_perm [1,0,3,2]
+  v += dpp_move<0x4E, 0xF>(v, 0.f);                // quad_perm [2,3,0,1]
+  if (G >= 8) v += dpp_move<0x141, 0xF>(v, 0.f);   // row_half_mirror
+  if (G >= 16) v += dpp_move<0x140, 0xF>(v, 0.f);  // row_mirror
+  if (G >= 32) v += __shfl_xor(v, 16);             // the other DPP row of the half
+  if (G >= 64) v += __shfl_xor(v, 32);
+  return v;
+}
+
 template <int T>
 __device__ __forceinline__ float mom_group_sum(float v, float* red) {
   if (T == 64) return wave_sum(v);
@@ -445,6 +567,43 @@ __global__ __launch_bounds__(T == 64 ? 256 : T) void moment_resident_kernel(unsi
   }
 }
 
+// Elements of at most 32 floats: G lanes (4..32) hold one, a block of 256 threads takes RPG * 256 / G of them with all
+// loads issued before the first sum (a wavefront per 7-float element used 7 of its 64 lanes: 100 000 of them took
+// 7.9 / 12.8 / 15.3 us).
+template <int MODE, int G, int RPG>
+__global__ __launch_bounds__(256) void moment_group_kernel(unsigned n, unsigned bd, const float* __restrict__ x,
+                                                           const float* __restrict__ fx, const float* __restrict__ dEdf,
+                                                           float* __restrict__ out) {
+  constexpr unsigned PER = 256 / G;
+  const unsigned gl = threadIdx.x % G;
+  const unsigned e0 = blockIdx.x * (PER * RPG) + threadIdx.x / G;
+  const bool in = gl < n;
+  float v[RPG], o[RPG];
+#pragma unroll
+  for (int k = 0; k < RPG; ++k) {
+    const unsigned e = e0 + k * PER;
+    const size_t at = size_t(e < bd ? e : bd - 1) * n + (in ? gl : n - 1);
+    v[k] = x[at];
+    if (MODE == 2) o[k] = out[at];
+  }
+  const float fn = float(n);
+#pragma unroll
+  for (int k = 0; k < RPG; ++k) {
+    const unsigned e = e0 + k * PER;
+    const float mean = group_sum<G>(in ? v[k] : 0.f) / fn;
+    if (MODE == 0) {
+      if (gl == 0 && e < bd) out[e] = mean;
+    } else if (MODE == 1) {
+      const float d = in ? v[k] - mean : 0.f;
+      const float var = group_sum<G>(d * d) / fn;
+      if (gl == 0 && e < bd) out[e] = sqrtf(var);
+    } else if (e < bd) {
+      const float sb = dEdf[e] / (2.f * fx[e]);
+      if (in) out[size_t(e) * n + gl] = o[k] + (2.f / fn) * (v[k] - mean) * sb;
+    }
+  }
+}
+
 // true: the register-resident kernel was launched
 template <int MODE>
 static bool launch_moment_resident(dyhip_device* dev, size_t n, unsigned bd, const float* x, const float* fx,
@@ -455,7 +614,14 @@ static bool launch_moment_resident(dyhip_device* dev, size_t n, unsigned bd, con
   hipLaunchKernelGGL((moment_resident_kernel<MODE, T, U>), dim3(GRID), dim3(T == 64 ? 256 : T), 0, dev->stream, r, bd, x, \
                      fx, dEdf, out)
   const unsigned g4 = cdiv<unsigned>(bd, 4);
-  if (r <= 64) DYHIP_MOM(64, 1, g4);
+#define DYHIP_MOMG(G)                                                                                              \
+  hipLaunchKernelGGL((moment_group_kernel<MODE, G, 4>), dim3(cdiv<unsigned>(bd, 4 * 256 / G)), dim3(256), 0, dev->stream, \
+                     r, bd, x, fx, dEdf, out)
+  if (r <= 4) DYHIP_MOMG(4);
+  else if (r <= 8) DYHIP_MOMG(8);
+  else if (r <= 16) DYHIP_MOMG(16);
+  else if (r <= 32) DYHIP_MOMG(32);
+  else if (r <= 64) DYHIP_MOM(64, 1, g4);
   else if (r <= 128) DYHIP_MOM(64, 2, g4);
   else if (r <= 256) DYHIP_MOM(64, 4, g4);
   else if (r <= 512) DYHIP_MOM(64, 8, g4);
@@ -465,6 +631,7 @@ static bool launch_moment_resident(dyhip_device* dev, size_t n, unsigned bd, con
   else if (r <= 8192) DYHIP_MOM(1024, 8, bd);
   else DYHIP_MOM(1024, 16, bd);
 #undef DYHIP_MOM
+#undef DYHIP_MOMG
   return true;
 }
 
@@ -552,18 +719,7 @@ __global__ __launch_bounds__(64 * kLnWavesFwd) void ln_fwd_wave_kernel(unsigned 
 // ---- rows of at most 256 floats: G lanes (4, 8 or 16) hold a row, a wavefront 64 / G rows at a time ---------------------
 // With a wavefront per row, rows of 64 floats use 16 of its lanes and one 128-bit load per lane (0.27 of the HBM peak
 // forward and backward; 0.08 at 16 floats).  The sums over a row stay inside a 16-lane DPP row: quad permutes, then
-// the half-row and row mirrors, after which every lane of the group holds the group's sum.
-template <int G>
-__device__ __forceinline__ float group_sum(float v) {
-  v += dpp_move<0xB1, 0xF>(v, 0.f);                // quad_perm [1,0,3,2]
-  v += dpp_move<0x4E, 0xF>(v, 0.f);                // quad_perm [2,3,0,1]
-  if (G >= 8) v += dpp_move<0x141, 0xF>(v, 0.f);   // row_half_mirror
-  if (G >= 16) v += dpp_move<0x140, 0xF>(v, 0.f);  // row_mirror
-  if (G >= 32) v += __shfl_xor(v, 16);             // the other DPP row of the half
-  if (G >= 64) v += __shfl_xor(v, 32);
-  return v;
-}
-
+// the half-row and row mirrors (group_sum above), after which every lane of the group holds the group's sum.
 // RPG: rows a group takes, all fetched before the first is reduced (one 128-bit load a lane is too little in flight:
 // 64-float rows 7.6 us for 16 MB with one, against 6.0 us for 128-float rows with two)
 template <int G, int VPL, int RPG, bool NT>
@@ -1876,6 +2032,14 @@ int dyhip_mean_elems_forward(dyhip_device* dev, size_t n, unsigned bd, const flo
     DYHIP_CHECK_LAUNCH();
     return DYHIP_OK;
   }
+  unsigned chunks = 0;
+  if (moment_chunked_fits(dev, n, bd, &chunks)) {
+    float* stats = static_cast<float*>(dev->gemm_ws);
+    hipLaunchKernelGGL(moment_chunk_kernel<0>, dim3(chunks, bd), dim3(256), 0, dev->stream, n, x, stats);
+    hipLaunchKernelGGL(moment_finish_kernel<0>, dim3(bd), dim3(64), 0, dev->stream, n, chunks, stats, y);
+    DYHIP_CHECK_LAUNCH();
+    return DYHIP_OK;
+  }
   hipLaunchKernelGGL(moment_fwd_kernel<false>, dim3(bd), dim3(kMomThreads), 0, dev->stream, n, x, y);
   DYHIP_CHECK_LAUNCH();
   return DYHIP_OK;
@@ -1886,6 +2050,14 @@ int dyhip_std_elems_forward(dyhip_device* dev, size_t n, unsigned bd, const floa
   DYHIP_REQUIRE(n >= 1 && x && y, "std_elems needs a non-empty tensor");
   if (bd == 0) return DYHIP_OK;
   if (launch_moment_resident<1>(dev, n, bd, x, nullptr, nullptr, y)) {
+    DYHIP_CHECK_LAUNCH();
+    return DYHIP_OK;
+  }
+  unsigned chunks = 0;
+  if (moment_chunked_fits(dev, n, bd, &chunks)) {
+    float* stats = static_cast<float*>(dev->gemm_ws);
+    hipLaunchKernelGGL(moment_chunk_kernel<1>, dim3(chunks, bd), dim3(256), 0, dev->stream, n, x, stats);
+    hipLaunchKernelGGL(moment_finish_kernel<1>, dim3(bd), dim3(64), 0, dev->stream, n, chunks, stats, y);
     DYHIP_CHECK_LAUNCH();
     return DYHIP_OK;
   }
@@ -1917,6 +2089,15 @@ int dyhip_std_elems_backward(dyhip_device* dev, size_t n, unsigned bd, const flo
   DYHIP_REQUIRE(n >= 1 && x && fx && dEdf && dEdx, "std_elems needs a non-empty tensor");
   if (bd == 0) return DYHIP_OK;
   if (launch_moment_resident<2>(dev, n, bd, x, fx, dEdf, dEdx)) {
+    DYHIP_CHECK_LAUNCH();
+    return DYHIP_OK;
+  }
+  unsigned chunks = 0;
+  if (moment_chunked_fits(dev, n, bd, &chunks)) {
+    float* sums = static_cast<float*>(dev->gemm_ws);
+    hipLaunchKernelGGL(moment_chunk_kernel<0>, dim3(chunks, bd), dim3(256), 0, dev->stream, n, x, sums);
+    hipLaunchKernelGGL(std_bwd_chunked_kernel, dim3(static_cast<unsigned>(cdiv<size_t>(n, 1024)), bd), dim3(256), 0,
+                       dev->stream, n, chunks, x, sums, fx, dEdf, dEdx);
     DYHIP_CHECK_LAUNCH();
     return DYHIP_OK;
   }

@@ -168,7 +168,8 @@ def test_sum_batches_golden_cadd_broadcast2_neg_val(dev, golden):
 
 
 @pytest.mark.parametrize("n,bd", [(1024, 4096), (9, 3), (1000, 17), (1, 4), (50, 3000), (100, 7), (200, 9), (400, 5), (1500, 3),
-                                  (3000, 3), (5000, 2), (10000, 2), (16384, 2), (16385, 2), (70000, 2)])
+                                  (3000, 3), (5000, 2), (10000, 2), (16384, 2), (16385, 2), (70000, 2), (24577, 5), (30000, 64), (7, 1000), (3, 70001),
+                                  (17, 999), (32, 513), (5, 1), (2, 300), (12, 257)])
 def test_mean_std_elems(dev, n, bd):
     rng = np.random.default_rng(41)
     x = f32(rng.standard_normal((bd, n)) + 0.5)
@@ -188,6 +189,31 @@ def test_mean_std_elems(dev, n, bd):
         dev.std_elems_backward(n, bd, xt, dev.tensor(sd_ref), dev.tensor(dy), gt)
         assert_close(gt.numpy(), orc.std_elems_backward(n, bd, x, sd_ref, dy, g0.copy()), GRAD_RTOL, "std bwd",
                      floor=1e-3)
+
+
+@pytest.mark.parametrize("n,bd", [(300001, 3), (1048576, 4), (2000003, 1)])
+def test_mean_std_long_elements(dev, n, bd):
+    """Elements of 10^5..10^6 floats: the sequential fp32 sums of the CPU restatement have themselves drifted by
+    several 1e-5 at this length, so the check is against the same formulas (dynet/nodes-moments.cc:264-274, 497-527)
+    in fp64."""
+    rng = np.random.default_rng(43)
+    x = f32(rng.standard_normal((bd, n)) * 1.5 + 0.5)
+    xt = dev.tensor(x)
+    mt, st = dev.empty(bd), dev.empty(bd)
+    dev.mean_elems_forward(n, bd, xt, mt)
+    dev.std_elems_forward(n, bd, xt, st)
+    x64 = x.astype(np.float64)
+    mean, sd = x64.mean(axis=1), x64.std(axis=1)
+    assert_close(mt.numpy(), mean, FWD_RTOL, "mean_elems", floor=1e-3)
+    assert_close(st.numpy(), sd, FWD_RTOL, "std_elems", floor=1e-6)
+    dy, g0 = f32(rng.standard_normal(bd)), f32(rng.standard_normal((bd, n)))
+    gt = dev.tensor(g0)
+    dev.std_elems_backward(n, bd, xt, dev.tensor(f32(sd)), dev.tensor(dy), gt)
+    ref = g0 + (2.0 / n) * (x64 - mean[:, None]) * (dy.astype(np.float64) / (2.0 * f32(sd)))[:, None]
+    assert_close(gt.numpy(), ref, GRAD_RTOL, "std bwd", floor=1e-3)
+    gt = dev.tensor(g0)
+    dev.mean_elems_backward(n, bd, dev.tensor(dy), gt)
+    assert_close(gt.numpy(), g0 + dy.astype(np.float64)[:, None] / n, GRAD_RTOL, "mean bwd", floor=1e-3)
 
 
 def test_std_golden_std_dim_value(dev, golden):
