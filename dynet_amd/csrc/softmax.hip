@@ -789,13 +789,189 @@ __global__ __launch_bounds__(64 * kRowWaves) void rowwise_kernel(unsigned rows, 
   }
 }
 
+// ---- the same three when rows x bd gives that kernel fewer blocks than the device has CUs (512 x 512 x 8: 64 blocks,
+// 0.8 TB/s; 2048 x 2048: 32 blocks) --------------------------------------------------------------------------------
+// The columns are cut into slabs over gridDim.y as well.  rows_slab_kernel leaves, per row and slab, the running
+// (maximum, sum of exp(x - maximum)) of one pass over the slab (DOT: the slab's sum of a * b); rows_finish_kernel
+// merges a row's slabs (the block's threads share them out and meet in LDS) and writes its own slab of the output,
+// or the row's (max, log-sum-exp) from a grid with gridDim.y == 1.  Lane layout as in rowwise_kernel with four waves.
+constexpr int kSlabWaves = 4;
+
+// (m, s) of every thread of the block merged per row; every thread leaves with its row's pair.  A thread that saw
+// nothing brings (-inf, 0); a NaN sum stays NaN whatever its maximum.
+__device__ __forceinline__ void rows_merge(float& m, float& s, float (*red_m)[64], float (*red_s)[64], unsigned w,
+                                           unsigned lane, unsigned rw_shift, unsigned rl, bool dot) {
+  red_m[w][lane] = m;
+  red_s[w][lane] = s;
+  __syncthreads();
+  const unsigned nsub = 64u >> rw_shift;
+  float mm = -INFINITY;
+  if (!dot)
+    for (unsigned k = 0; k < kSlabWaves; ++k)
+      for (unsigned s2 = 0; s2 < nsub; ++s2) {
+        const float o = red_m[k][(s2 << rw_shift) + rl];
+        mm = o > mm ? o : mm;
+      }
+  const float ref = mm > -INFINITY ? mm : 0.f;
+  float ss = 0.f;
+  for (unsigned k = 0; k < kSlabWaves; ++k)
+    for (unsigned s2 = 0; s2 < nsub; ++s2) {
+      const unsigned at = (s2 << rw_shift) + rl;
+      ss += dot ? red_s[k][at] : red_s[k][at] * expf(red_m[k][at] - ref);
+    }
+  __syncthreads();
+  m = mm;
+  s = ss;
+}
+
+template <bool DOT>
+__global__ __launch_bounds__(64 * kSlabWaves) void rows_slab_kernel(unsigned rows, unsigned cols, unsigned rw_shift,
+                                                                   unsigned slab, const float* __restrict__ a,
+                                                                   const float* __restrict__ b,
+                                                                   float* __restrict__ part_m, float* __restrict__ part_s) {
+  __shared__ float red_m[kSlabWaves][64], red_s[kSlabWaves][64];
+  constexpr int U = 8;
+  const unsigned lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const unsigned RW = 1u << rw_shift, nsub = 64u >> rw_shift, rl = lane & (RW - 1), sub = lane >> rw_shift;
+  const unsigned stride = kSlabWaves * nsub;
+  const unsigned row = blockIdx.x * RW + rl;
+  const bool live = row < rows;
+  const unsigned c0 = blockIdx.y * slab, c1 = min(cols, c0 + slab);
+  const size_t base = size_t(blockIdx.z) * rows * cols + (live ? row : rows - 1);
+  float m = -INFINITY, s = 0.f;
+  for (unsigned j = c0 + w * nsub + sub; j < c1; j += U * stride) {
+    float v[U], y[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const size_t e = base + size_t(min(j + u * stride, c1 - 1)) * rows;
+      v[u] = a[e];
+      y[u] = DOT ? b[e] : 0.f;
+    }
+    if (DOT) {
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (j + u * stride < c1) s += v[u] * y[u];
+    } else {
+      float lm = m;
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (j + u * stride < c1) lm = v[u] > lm ? v[u] : lm;  // a NaN entry is skipped here and makes the sum NaN below
+      const float ref = lm > -INFINITY ? lm : 0.f;
+      s *= expf(m - ref);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (j + u * stride < c1) s += expf(v[u] - ref);
+      m = lm;
+    }
+  }
+  rows_merge(m, s, red_m, red_s, w, lane, rw_shift, rl, DOT);
+  if (live && w == 0 && sub == 0) {
+    const size_t at = (size_t(blockIdx.z) * gridDim.y + blockIdx.y) * rows + row;
+    if (!DOT) part_m[at] = m;
+    part_s[at] = s;
+  }
+}
+
+// MODE as in rowwise_kernel; nslabs: slabs the partial results hold per row (gridDim.y of the slab kernel)
+template <int MODE>
+__global__ __launch_bounds__(64 * kSlabWaves) void rows_finish_kernel(unsigned rows, unsigned cols, unsigned rw_shift,
+                                                                     unsigned slab, unsigned nslabs,
+                                                                     const float* __restrict__ part_m,
+                                                                     const float* __restrict__ part_s,
+                                                                     const float* __restrict__ a,
+                                                                     const float* __restrict__ b,
+                                                                     float* __restrict__ m_out, float* __restrict__ out) {
+  __shared__ float red_m[kSlabWaves][64], red_s[kSlabWaves][64];
+  constexpr int U = 8;
+  const unsigned lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const unsigned RW = 1u << rw_shift, nsub = 64u >> rw_shift, rl = lane & (RW - 1), sub = lane >> rw_shift;
+  const unsigned stride = kSlabWaves * nsub;
+  const unsigned row = blockIdx.x * RW + rl;
+  const bool live = row < rows;
+  const unsigned rowc = live ? row : rows - 1;
+  float m = -INFINITY, s = 0.f;
+  for (unsigned k = w * nsub + sub; k < nslabs; k += U * stride) {
+    float pm[U], ps[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const size_t at = (size_t(blockIdx.z) * nslabs + min(k + u * stride, nslabs - 1)) * rows + rowc;
+      pm[u] = MODE == 2 ? 0.f : part_m[at];
+      ps[u] = part_s[at];
+    }
+    if (MODE == 2) {
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (k + u * stride < nslabs) s += ps[u];
+    } else {
+      float lm = m;
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (k + u * stride < nslabs) lm = pm[u] > lm ? pm[u] : lm;
+      const float ref = lm > -INFINITY ? lm : 0.f;
+      s *= expf(m - ref);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (k + u * stride < nslabs) s += ps[u] * expf(pm[u] - ref);
+      m = lm;
+    }
+  }
+  rows_merge(m, s, red_m, red_s, w, lane, rw_shift, rl, MODE == 2);
+  if (MODE != 2 && m == -INFINITY) s = NAN;  // a row of -inf: exp(-inf - -inf), as in the one-kernel form
+  if (MODE == 0) {
+    if (live && w == 0 && sub == 0) {
+      m_out[size_t(blockIdx.z) * rows + row] = m;
+      out[size_t(blockIdx.z) * rows + row] = logf(s) + m;
+    }
+    return;
+  }
+  const unsigned c0 = blockIdx.y * slab, c1 = min(cols, c0 + slab);
+  const size_t base = size_t(blockIdx.z) * rows * cols + rowc;
+  for (unsigned j = c0 + w * nsub + sub; j < c1; j += U * stride) {
+    float v[U], y[U], o[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const size_t e = base + size_t(min(j + u * stride, c1 - 1)) * rows;
+      v[u] = a[e];
+      y[u] = MODE == 2 ? b[e] : 0.f;
+      o[u] = MODE == 2 ? out[e] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (!live || j + u * stride >= c1) continue;
+      const size_t e = base + size_t(j + u * stride) * rows;
+      if (MODE == 1) out[e] = expf(v[u] - m) / s;
+      else out[e] = o[u] + (y[u] - s) * v[u];
+    }
+  }
+}
+
 template <int MODE>
 static int launch_rowwise(dyhip_device* dev, size_t rows, size_t cols, unsigned bd, const float* a, const float* b,
                           float* m_out, float* out) {
   DYHIP_REQUIRE(rows < (size_t(1) << 31) && cols < (size_t(1) << 31), "matrix dimension too large");
   unsigned rw_shift = 6;  // row lanes a wavefront: the power of two that reaches the row count, at most 64
   while (rw_shift > 0 && (size_t(1) << (rw_shift - 1)) >= rows) --rw_shift;
-  const dim3 grid(static_cast<unsigned>(cdiv<size_t>(rows, size_t(1) << rw_shift)), bd < 65535u ? bd : 65535u);
+  const size_t tiles = cdiv<size_t>(rows, size_t(1) << rw_shift), cus = dev->num_cus > 0 ? size_t(dev->num_cus) : 256;
+  if (tiles * bd < cus && cols >= 256) {
+    const size_t sstride = size_t(kSlabWaves) * (64u >> rw_shift);
+    size_t nslabs = std::min(cdiv<size_t>(2 * cus, tiles * bd), cols / 64);
+    const size_t slab = cdiv<size_t>(cdiv<size_t>(cols, nslabs), sstride) * sstride;  // whole passes of the block
+    nslabs = cdiv<size_t>(cols, slab);
+    const size_t part = size_t(bd) * nslabs * rows;
+    if (nslabs >= 2 && dev->gemm_ws != nullptr && dev->gemm_ws_bytes >= 2 * part * sizeof(float)) {
+      float* part_m = static_cast<float*>(dev->gemm_ws);
+      float* part_s = part_m + part;
+      const unsigned r = static_cast<unsigned>(rows), c = static_cast<unsigned>(cols), sl = static_cast<unsigned>(slab),
+                     ns = static_cast<unsigned>(nslabs), t = static_cast<unsigned>(tiles);
+      hipLaunchKernelGGL((rows_slab_kernel<MODE == 2>), dim3(t, ns, bd), dim3(64 * kSlabWaves), 0, dev->stream, r, c,
+                         rw_shift, sl, a, b, part_m, part_s);
+      hipLaunchKernelGGL((rows_finish_kernel<MODE>), dim3(t, MODE == 0 ? 1 : ns, bd), dim3(64 * kSlabWaves), 0, dev->stream,
+                         r, c, rw_shift, sl, ns, part_m, part_s, a, b, m_out, out);
+      DYHIP_CHECK_LAUNCH();
+      return DYHIP_OK;
+    }
+  }
+  const dim3 grid(static_cast<unsigned>(tiles), bd < 65535u ? bd : 65535u);
   const size_t stride = size_t(kRowWaves) * (64u >> rw_shift);  // columns between a thread's consecutive elements
   if (cols >= 4 * stride)
     hipLaunchKernelGGL((rowwise_kernel<MODE, 8>), grid, dim3(64 * kRowWaves), 0, dev->stream, static_cast<unsigned>(rows),

@@ -1800,7 +1800,9 @@ def test_zero_any_alignment_and_inside_a_graph(dev):
 @pytest.mark.parametrize("rows,cols,bd", [(7, 5, 3), (64, 100, 2), (130, 9, 1), (1, 300, 4), (1000, 33, 2), (3, 1, 5),
                                           # few rows and many columns (a wavefront folds its lanes over the columns), column
                                           # counts around the eight loads a thread has in flight
-                                          (3, 8000, 2), (2, 1000, 3), (5, 4097, 1), (512, 512, 2), (33, 70, 2), (16, 129, 3)])
+                                          (3, 8000, 2), (2, 1000, 3), (5, 4097, 1), (512, 512, 2), (33, 70, 2), (16, 129, 3),
+                                          # few row groups: the columns are cut into slabs over the blocks as well
+                                          (100, 3000, 2), (2048, 300, 1), (64, 256, 3), (40, 257, 5), (1, 6000, 1), (700, 511, 1)])
 def test_softmax_and_logsumexp_along_dim_1(dev, rows, cols, bd):
     rng = np.random.default_rng(rows + cols + bd)
     x = f32(rng.standard_normal((bd, cols, rows)) * 3)
@@ -1830,6 +1832,30 @@ def test_softmax_and_logsumexp_along_dim_1(dev, rows, cols, bd):
                      "logsumexp dim %d bwd" % dim, floor=1.0)
     with pytest.raises(DyhipError):
         dev.logsumexp_dim_forward(rows, cols, bd, xt, 2, m, z)
+
+
+@pytest.mark.parametrize("rows,cols,bd", [(6, 40, 2), (6, 1500, 2), (70, 300, 1)])
+def test_softmax_and_logsumexp_along_dim_1_with_infinite_entries(dev, rows, cols, bd):
+    """-inf entries drop out of a row; a row that is all -inf is NaN (exp(-inf - -inf)), as in
+    dynet/tensor.cc TensorTools::logsumexp and nodes-softmaxes.cc Softmax with dimension 1."""
+    rng = np.random.default_rng(5)
+    x = f32(rng.standard_normal((bd, cols, rows)) * 3)
+    x[:, ::3, 1] = -np.inf
+    x[:, : cols // 2, 2] = -np.inf
+    x[:, :, 4] = -np.inf
+    xt = dev.tensor(x)
+    fx = dev.empty((bd, cols, rows))
+    dev.softmax_rows_forward(rows, cols, bd, xt, fx)
+    ref = orc.softmax_rows_forward(rows, cols, bd, x)
+    got = fx.numpy()
+    assert np.array_equal(np.isnan(got), np.isnan(ref)) and np.isnan(got[:, :, 4]).all() and not np.isnan(got[:, :, :4]).any()
+    assert_close(np.nan_to_num(got), np.nan_to_num(ref), FWD_RTOL, "softmax dim 1", floor=1.0 / cols)
+    m, z = dev.empty((bd, rows)), dev.empty((bd, rows))
+    dev.logsumexp_dim_forward(rows, cols, bd, xt, 1, m, z)
+    rm, rz = orc.logsumexp_dim_forward(rows, cols, bd, x, 1)
+    assert m.numpy().tobytes() == rm.tobytes()
+    assert np.array_equal(np.isnan(z.numpy()), np.isnan(rz)) and np.isnan(rz[:, 4]).all()
+    assert_close(np.nan_to_num(z.numpy()), np.nan_to_num(rz), FWD_RTOL, "logsumexp dim 1", floor=1.0)
 
 
 def test_pool_growth_is_ordered_with_forked_queues_and_refused_inside_a_capture(gpu):
