@@ -400,6 +400,34 @@ __global__ __launch_bounds__(256) void pick_range_kernel(size_t run, size_t smal
   }
 }
 
+// Runs shorter than a few wavefronts (a block per run left most of its lanes idle: 100 000 runs of 21 floats took
+// 30 us): a thread per entry of the slice over the flat slice, four entries in flight, the run found by one 32-bit
+// division.
+template <bool ACC>
+__global__ __launch_bounds__(256) void pick_range_flat_kernel(unsigned run, unsigned total, size_t big_stride,
+                                                              size_t big_offset, const float* __restrict__ src,
+                                                              float* __restrict__ dst) {
+  const unsigned e0 = blockIdx.x * 1024 + threadIdx.x;
+  size_t big[4];
+  unsigned small[4];
+  float v[4], acc[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const unsigned e = e0 + 256 * k;
+    small[k] = e < total ? e : total - 1;
+    const unsigned o = small[k] / run;
+    big[k] = size_t(o) * big_stride + big_offset + (small[k] - o * run);
+    v[k] = ACC ? src[small[k]] : src[big[k]];
+    acc[k] = ACC ? dst[big[k]] : 0.f;
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    if (e0 + 256 * k >= total) continue;
+    if (ACC) dst[big[k]] = acc[k] + v[k];
+    else dst[small[k]] = v[k];
+  }
+}
+
 static int pick_range(dyhip_device* dev, bool backward, size_t inner, size_t len, size_t outer, size_t start,
                       size_t end, const float* src, float* dst) {
   DYHIP_REQUIRE(start < end && end <= len, "PickRange: bad range [%zu, %zu) for a dimension of %zu", start, end, len);
@@ -407,6 +435,17 @@ static int pick_range(dyhip_device* dev, bool backward, size_t inner, size_t len
   DYHIP_REQUIRE(src && dst, "PickRange: null tensor pointer");
   DYHIP_REQUIRE(outer <= 0xffffffffu, "PickRange: too many slices");
   const size_t run = inner * (end - start);
+  if (run < 1024 && outer > 1 && run * outer <= 0xffffffffu - 1024) {
+    const unsigned total = unsigned(run * outer), blocks = cdiv<unsigned>(total, 1024);
+    if (backward)
+      hipLaunchKernelGGL(pick_range_flat_kernel<true>, dim3(blocks), dim3(256), 0, dev->stream, unsigned(run), total,
+                         inner * len, start * inner, src, dst);
+    else
+      hipLaunchKernelGGL(pick_range_flat_kernel<false>, dim3(blocks), dim3(256), 0, dev->stream, unsigned(run), total,
+                         inner * len, start * inner, src, dst);
+    DYHIP_CHECK_LAUNCH();
+    return DYHIP_OK;
+  }
   const dim3 grid(unsigned(std::min<size_t>(cdiv<size_t>(run, 256), 4096)), unsigned(std::min<size_t>(outer, 65535)));
   if (backward)
     hipLaunchKernelGGL(pick_range_kernel<true>, grid, dim3(256), 0, dev->stream, run, run, inner * len, start * inner,

@@ -1654,7 +1654,9 @@ def dev_scalar(dev, which):
 
 # ---- PickRange and the unfused builder step ---------------------------------------------------
 @pytest.mark.parametrize("inner,length,outer,start,end", [(1, 8, 5, 2, 6), (1, 4096, 128, 1024, 2048), (7, 5, 3, 0, 5),
-                                                          (3, 9, 70000, 4, 5), (33, 4, 1, 1, 3)])
+                                                          (3, 9, 70000, 4, 5), (33, 4, 1, 1, 3), (7, 9, 10001, 2, 5),
+                                                          (1, 1500, 9, 100, 1123), (1, 1500, 9, 100, 1124), (5, 3, 1, 1, 2),
+                                                          (1, 2, 1025, 1, 2)])
 def test_pick_range(dev, inner, length, outer, start, end):
     rng = np.random.default_rng(inner + length)
     x = f32(rng.standard_normal(inner * length * outer))
