@@ -51,6 +51,13 @@ struct GemmBatch {
 int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N, int nseg, const GemmSeg* segs,
              float* C, const GemmEpiParams& epi, const GemmBatch* batch = nullptr);
 
+// gemm_small.hip: one-launch products for operands of a few hundred KB, any layout, single or strided-batched, with
+// the axpby or the bias epilogue.
+bool gemm_small_eligible(const dyhip_device* dev, size_t M, size_t N, size_t K, const GemmEpiParams& epi, unsigned batch,
+                         bool tile_kernel_vectorizes);
+int gemm_small_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N, const GemmSeg& s, float* C,
+                   const GemmEpiParams& epi, const GemmBatch* batch);
+
 // gemm_wide.hip: the 256 x 256-tile kernel for large outputs.  gemm_wide_eligible tells whether a one-segment,
 // unbatched product qualifies; gemm_wide_run computes C = beta*C + sum (or bias[i] + sum when bias is set) over the
 // first K32 (a multiple of 32) of the depth.

@@ -363,12 +363,14 @@ static GemmPlan plan_gemm(const dyhip_device* dev, size_t M, size_t N, unsigned 
                           bool must_use_partials) {
   const double cus = dev->num_cus > 0 ? dev->num_cus : 256;
   const double peak = cus * 256.0 * 2.0e9, ws_bw = 3.0e12;
-  const double flops = 2.0 * double(M) * double(N) * double(ktiles) * kBK;
   GemmPlan best{2, 1};
   double best_t = 1e30;
   for (int wn = 2; wn >= 1; --wn) {
     if (wn == 2 && N <= 64) continue;
     const double tiles = double(cdiv<size_t>(M, kBM)) * double(cdiv<size_t>(N, size_t(64) * wn));
+    // a tile costs its full multiply-adds whatever part of it lies inside the matrix (a 650 x 1 product priced by
+    // its own multiply-adds was never split over the depth: one block per 128 rows walked all k-tiles, 53 us)
+    const double flops = 2.0 * tiles * double(kBM) * 64.0 * wn * double(ktiles) * kBK;
     for (unsigned s = 1; s <= 32; ++s) {
       if (s > 1 && (ktiles / s < 2 || s > max_splits_ws)) break;
       const double blocks = tiles * s;
@@ -1092,6 +1094,15 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
       segs[0].A != nullptr && segs[0].B != nullptr &&
       gemm_shallow_nt_eligible(dev, M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, segs[0].ldb, C))
     return gemm_shallow_nt_run(dev, M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, segs[0].ldb, C, epi.beta);
+  const bool batched = batch != nullptr && batch->count > 1;
+  const bool tile_vec = nseg == 1 && aligned16(segs[0].A) && segs[0].lda % 4 == 0 && aligned16(segs[0].B) &&
+                        segs[0].ldb % 4 == 0 && (!batched || (batch->stride_a % 4 == 0 && batch->stride_b % 4 == 0));
+  if (nseg == 1 && !to_caller && C != nullptr && segs[0].A != nullptr && segs[0].B != nullptr &&
+      gemm_small_eligible(dev, M, N, segs[0].K, epi, batch ? batch->count : 1, tile_vec)) {
+    if (batch != nullptr && batch->count > 1)
+      DYHIP_REQUIRE(batch->stride_c >= M * N, "batch items of the GEMM output overlap");
+    return gemm_small_run(dev, a_kmajor, b_kmajor, M, N, segs[0], C, epi, batch);
+  }
   GemmArgs g;
   g.nseg = nseg;
   g.M = M;

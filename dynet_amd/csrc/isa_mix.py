@@ -15,7 +15,7 @@ import sys
 import tempfile
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SRCS = ["elementwise", "cwise", "reduce", "softmax", "lookup", "gemm", "gemm_wide", "lstm", "misc", "trainer", "random"]
+SRCS = ["elementwise", "cwise", "reduce", "softmax", "lookup", "gemm", "gemm_wide", "gemm_small", "lstm", "misc", "trainer", "random"]
 FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950", "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang",
          "-packed-fp32-ops", "-Wno-unused-function", "-Wno-unknown-warning-option", "-I" + os.path.join(HERE, "../../include"),
          "-I" + HERE, "--cuda-device-only", "-S"]
@@ -30,7 +30,7 @@ HOT = ["ew_vec4_kernel<2, true, 0, true, 2, dyhip::AccMul2", "ew_vec4_kernel<1, 
        "gather_segments_kernel<true, true>", "sgd_scaled_kernel<true, true>", "philox",
        "gemm_nn_mid_kernel<true>", "gemm_nn_rows_kernel<1, 8, 4>", "gemm_nn_thin_kernel<1>", "gemm_nt_thin_kernel<32, 4>",
        "gemm_tn_thin_kernel<4, 2>", "ln_fwd_group_kernel<16, 1, 2, true>", "ln_bwd_group_kernel<16, 1, true>",
-       "sum_group_kernel<false, false>", "softmax_resident_kernel<0, 256, 4>", "moment_resident_kernel<1, 256, 4>"]
+       "sum_group_kernel<false, false>", "gemm_small_kernel<4, 4, 4>", "gemm_small_kernel<1, 4, 8>", "softmax_resident_kernel<0, 256, 4>", "moment_resident_kernel<1, 256, 4>"]
 
 KINDS = [
     ("ld128", r"^\s*(global|flat|buffer)_load_dwordx4\b"),

@@ -27,7 +27,13 @@ GEMM_SHAPES = [(1024, 32, 128), (1024, 32, 256), (4096, 128, 1280), (256, 128, 4
                # one and several depth ranges)
                (100, 37, 1152), (64, 1, 2048), (33, 256, 1024), (2048, 200, 2560),
                # more tiles than two per CU with a thin last round: the trailing tile columns run as a GEMM of their own
-               (4096, 2304, 40), (4100, 2310, 33)]
+               (4096, 2304, 40), (4100, 2310, 33),
+               # operands of a few hundred KB: the one-launch product on 32 x 32 wavefront tiles (a tile a wavefront for
+               # a shallow depth, the depth over four or eight wavefronts otherwise; 128-bit, 64-bit and scalar loads
+               # along the depth by the leading dimensions' divisibility; ragged rows, columns and depth)
+               (128, 128, 128), (200, 100, 50), (64, 64, 16), (33, 65, 9), (650, 1, 650), (1, 1, 1000), (35, 1, 1024),
+               (1, 35, 1024), (300, 300, 300), (100, 7, 600), (31, 33, 520), (333, 333, 333), (512, 512, 512),
+               (650, 3, 1300), (2000, 70, 100), (4096, 4, 256), (129, 1000, 64), (40, 40, 3), (6, 2, 70)]
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
@@ -381,7 +387,9 @@ def test_gemm_wide_tiles_first_used_inside_a_graph_and_scaled_accumulate():
         d.close()
 
 
-@pytest.mark.parametrize("M,N,K,B", [(64, 48, 32, 5), (130, 70, 33, 3), (7, 5, 3, 17), (256, 128, 256, 4), (31, 1, 9, 2)])
+@pytest.mark.parametrize("M,N,K,B", [(64, 48, 32, 5), (130, 70, 33, 3), (7, 5, 3, 17), (256, 128, 256, 4), (31, 1, 9, 2),
+                                     (7, 5, 9, 1000), (1, 35, 1024, 128), (35, 1, 1024, 128), (64, 64, 64, 128),
+                                     (35, 35, 64, 512), (512, 1, 512, 32), (33, 2, 130, 3), (300, 300, 2048, 2)])
 def test_gemm_strided_batched(dev, M, N, K, B):
     """The batched-left-operand branches of the three GEMM shims: per batch item the plain product, as the
     reference's CPU path loops it (dynet/matrix-multiply.h:90-93, 148-150, 213-215)."""
@@ -417,6 +425,36 @@ def test_gemm_strided_batched(dev, M, N, K, B):
         dev.gemm_strided_batched(1, 1, M, N, K, dev.tensor(l), M * K, dev.tensor(r), K * N, 0.0, yt, M * N, B)
 
 
+@pytest.mark.parametrize("off_l,off_r", [(0, 0), (1, 0), (2, 2), (0, 3), (2, 0), (4, 2)])
+@pytest.mark.parametrize("M,N,K", [(96, 40, 200), (70, 33, 64), (650, 2, 652)])
+def test_gemm_small_products_on_operands_off_the_16_byte_grid(dev, M, N, K, off_l, off_r):
+    """Operands that start 4, 8 or 12 bytes into a 16-byte line: the loads along the depth fall back from 128 to 64 or
+    32 bits; same products as dynet/matrix-multiply.h:70-215."""
+    from dynet_amd.device import DevTensor
+
+    rng = np.random.default_rng(M + N + K + 10 * off_l + off_r)
+    floor = np.sqrt(K)
+    y0 = f32(rng.standard_normal((N, M)))
+    lbuf, rbuf = f32(rng.standard_normal(M * K + off_l)), f32(rng.standard_normal(N * K + off_r))
+    lt, rt = dev.tensor(lbuf), dev.tensor(rbuf)
+    lv = DevTensor(dev, lt.ptr + 4 * off_l, (M * K,))
+    rv = DevTensor(dev, rt.ptr + 4 * off_r, (N * K,))
+    l, r = lbuf[off_l:], rbuf[off_r:]
+    for beta in (0.0, 1.0):
+        yt = dev.tensor(y0)
+        dev.gemm_nn(M, N, K, lv, rv, beta, yt)
+        assert_close(yt.numpy(), orc.gemm_nn(M, N, K, l.reshape(K, M), r.reshape(N, K), beta, y0.copy()), FWD_RTOL,
+                     "l*r", floor=floor)
+    yt = dev.tensor(y0)
+    dev.gemm_tn_acc(M, N, K, lv, rv, yt)
+    assert_close(yt.numpy(), orc.gemm_tn_acc(M, N, K, l.reshape(M, K), r.reshape(N, K), y0.copy()), FWD_RTOL, "l^T*r",
+                 floor=floor)
+    yt = dev.tensor(y0)
+    dev.gemm_nt_acc(M, N, K, lv, rv, yt)
+    assert_close(yt.numpy(), orc.gemm_nt_acc(M, N, K, l.reshape(K, M), r.reshape(K, N), y0.copy()), FWD_RTOL, "l*r^T",
+                 floor=floor)
+
+
 def test_gemm_is_fp32_accurate_against_fp64(dev):
     """No reduced-precision shortcut on the matrix cores: error vs fp64 stays at fp32 rounding level."""
     rng = np.random.default_rng(5)
@@ -429,7 +467,8 @@ def test_gemm_is_fp32_accurate_against_fp64(dev):
 
 
 @pytest.mark.parametrize("M,N,K", [(1000, 128, 64), (10000, 96, 256), (37, 5, 20), (300, 192, 128), (4096, 4, 1024),
-                                   (4100, 2310, 24)])
+                                   (4100, 2310, 24), (650, 1, 650), (100, 7, 100), (3, 3, 3), (33, 100, 5000), (200, 100, 50),
+                                   (650, 2, 1300)])
 def test_affine_forward(dev, M, N, K):
     """AffineTransform: bias broadcast + W x (direct and split-K routes of the GEMM)."""
     rng = np.random.default_rng(M + N + K)
