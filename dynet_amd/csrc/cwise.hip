@@ -14,6 +14,8 @@
 //     kept axes = a prefix and the other operand is full size: the batch reduction of reduce.hip (coalesced);
 //     otherwise one wavefront per output element (>= 64 terms, lanes walk the broadcast axes fastest-first,
 //     fixed summation order) or one thread per output element (fewer terms).
+#include <algorithm>
+
 #include "common.h"
 
 namespace dyhip {
@@ -176,6 +178,10 @@ struct CwReduce {
   size_t ks[3][5];         // strides of the three operands along the kept axes (same order)
   size_t rs[3][5];         // ... along the reduced axes
   size_t n_out, n_red;
+  // cwise_reduce_row_kernel only: the reduced axis in `chunks` pieces of chunk_len (a multiple of 1024) indices, piece
+  // ch of output o summed into out[o * chunks + ch]
+  unsigned chunks, chunk_len;
+  int overwrite;  // out = sum instead of out += sum (a stage that writes scratch)
 };
 
 template <int FN>
@@ -218,7 +224,7 @@ __global__ __launch_bounds__(256) void cwise_reduce_wave_kernel(CwReduce c, cons
   const int lane = threadIdx.x & 63;
   for (size_t o = size_t(blockIdx.x) * 4 + (threadIdx.x >> 6); o < c.n_out; o += size_t(gridDim.x) * 4) {
     const float t = wave_sum(cw_reduce_one<FN>(c, o, size_t(lane), 64, p0, p1, p2));
-    if (lane == 0) out[o] += t;
+    if (lane == 0) out[o] = c.overwrite ? t : out[o] + t;
   }
 }
 
@@ -232,7 +238,9 @@ __global__ __launch_bounds__(256) void cwise_reduce_row_kernel(CwReduce c, const
   constexpr int NIN = cw_inputs(FN);
   const unsigned lane = threadIdx.x & 63;
   const float* ps[3] = {p0, p1, p2};
-  for (size_t o = size_t(blockIdx.x) * 4 + (threadIdx.x >> 6); o < c.n_out; o += size_t(gridDim.x) * 4) {
+  for (size_t item = size_t(blockIdx.x) * 4 + (threadIdx.x >> 6); item < c.n_out * c.chunks; item += size_t(gridDim.x) * 4) {
+    const size_t o = c.chunks == 1 ? item : item / c.chunks;
+    const unsigned ch = c.chunks == 1 ? 0 : unsigned(item - o * c.chunks);
     size_t base[3] = {0, 0, 0};
     size_t r = o;  // the same in every lane of the wave: the branches below are uniform
 #pragma unroll
@@ -257,11 +265,12 @@ __global__ __launch_bounds__(256) void cwise_reduce_row_kernel(CwReduce c, const
 #pragma unroll
       for (int k = 0; k < NIN; ++k) base[k] += i * c.ks[k][j];
     }
-    const unsigned nr = unsigned(c.n_red);
-    const float old = lane == 0 ? out[o] : 0.f;  // fetched beside the terms, not after the sum
+    const unsigned qb = ch * c.chunk_len;
+    const unsigned nr = c.chunks == 1 ? unsigned(c.n_red) : unsigned(min(c.n_red, size_t(qb) + c.chunk_len));
+    const float old = lane == 0 && !c.overwrite ? out[item] : 0.f;  // fetched beside the terms, not after the sum
     float acc = 0.f;
     if (VEC) {
-      for (unsigned q0 = 0; q0 < nr; q0 += 4 * 64 * 4) {
+      for (unsigned q0 = qb; q0 < nr; q0 += 4 * 64 * 4) {
         float4 v[4][3];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
@@ -287,7 +296,7 @@ __global__ __launch_bounds__(256) void cwise_reduce_row_kernel(CwReduce c, const
         }
       }
     } else {
-      for (unsigned q0 = 0; q0 < nr; q0 += 64 * 4) {
+      for (unsigned q0 = qb; q0 < nr; q0 += 64 * 4) {
         float v[4][3];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
@@ -301,7 +310,7 @@ __global__ __launch_bounds__(256) void cwise_reduce_row_kernel(CwReduce c, const
       }
     }
     const float t = wave_sum(acc);
-    if (lane == 0) out[o] = old + t;
+    if (lane == 0) out[item] = old + t;
   }
 }
 
@@ -311,7 +320,7 @@ __global__ __launch_bounds__(256) void cwise_reduce_thread_kernel(CwReduce c, co
                                                                   const float* __restrict__ p2,
                                                                   float* __restrict__ out) {
   for (size_t o = size_t(blockIdx.x) * 256 + threadIdx.x; o < c.n_out; o += size_t(gridDim.x) * 256)
-    out[o] += cw_reduce_one<FN>(c, o, 0, 1, p0, p1, p2);
+    out[o] = c.overwrite ? cw_reduce_one<FN>(c, o, 0, 1, p0, p1, p2) : out[o] + cw_reduce_one<FN>(c, o, 0, 1, p0, p1, p2);
 }
 
 // ---- host side ---------------------------------------------------------------------------------------
@@ -402,7 +411,7 @@ __global__ __launch_bounds__(64 * kCwMidWaves) void cwise_reduce_mid_kernel(CwRe
       float t = red[0][lane];
 #pragma unroll
       for (int k = 1; k < kCwMidWaves; ++k) t += red[k][lane];
-      out[z * c.kd[0] + i] += t;
+      out[z * c.kd[0] + i] = c.overwrite ? t : out[z * c.kd[0] + i] + t;
     }
   }
 }
@@ -478,11 +487,14 @@ static int cw_launch_bcast(dyhip_device* dev, const CwShape& sh_in, const float*
   return DYHIP_OK;
 }
 
+// scratch / scratch_floats: device memory a stage may leave intermediate sums in (none: single-stage forms only)
 template <int FN>
 static int cw_launch_reduce(dyhip_device* dev, const unsigned* full, const unsigned* dself, const size_t s[3][5],
-                            const float* p0, const float* p1, const float* p2, float* out) {
+                            const float* p0, const float* p1, const float* p2, float* out, bool overwrite, float* scratch,
+                            size_t scratch_floats) {
   CwReduce c;
-  int nk = 0, nr = 0;
+  int nk = 0, nr = 0, runs = 0, first_run_end = 5;
+  bool in_run = false;
   for (int j = 0; j < 5; ++j) {
     c.kd[j] = c.rd[j] = 1;
     for (int k = 0; k < 3; ++k) c.ks[k][j] = c.rs[k][j] = 0;
@@ -493,21 +505,31 @@ static int cw_launch_reduce(dyhip_device* dev, const unsigned* full, const unsig
       c.rd[nr] = full[j];
       for (int k = 0; k < 3; ++k) c.rs[k][nr] = s[k][j];
       ++nr;
+      if (!in_run) ++runs;
+      in_run = true;
     } else {
       c.kd[nk] = full[j];
       for (int k = 0; k < 3; ++k) c.ks[k][nk] = s[k][j];
       ++nk;
+      if (full[j] > 1) {
+        if (in_run && runs == 1 && first_run_end == 5) first_run_end = j;
+        in_run = false;
+      }
     }
   }
   c.n_out = cw_size(c.kd);
   c.n_red = cw_size(c.rd);
+  c.chunks = 1;
+  c.chunk_len = 0;
+  c.overwrite = overwrite ? 1 : 0;
+  const size_t cus = dev->num_cus > 0 ? size_t(dev->num_cus) : 256;
   {
     // the reduced axes as one axis, if every operand walks them alike
     unsigned rd2[5];
     size_t rs2[3][5], rs_in[3][5];
     for (int k = 0; k < 3; ++k)
       for (int j = 0; j < 5; ++j) rs_in[k][j] = c.rs[k][j];
-    if (c.n_red >= 64 && c.n_red <= 0xFFFFFFFFull && cw_collapse(c.rd, rs_in, cw_inputs(FN), rd2, rs2) == 1) {
+    if (c.n_red >= 2 && c.n_red <= 0xFFFFFFFFull && cw_collapse(c.rd, rs_in, cw_inputs(FN), rd2, rs2) == 1) {
       const float* ps[3] = {p0, p1, p2};
       bool vec = c.n_red % 4 == 0;
       for (int k = 0; k < cw_inputs(FN); ++k) {
@@ -517,15 +539,19 @@ static int cw_launch_reduce(dyhip_device* dev, const unsigned* full, const unsig
           for (int j = 0; j < 5; ++j) vec = vec && c.ks[k][j] % 4 == 0;
         }
       }
-      for (int j = 0; j < 5; ++j) {
-        c.rd[j] = rd2[j];
-        for (int k = 0; k < 3; ++k) c.rs[k][j] = rs2[k][j];
-      }
       // the first kept axis is the contiguous one (and not a short one) and the reduced axis is not: lanes along it
       bool mid = c.kd[0] >= 16;
-      for (int k = 0; k < cw_inputs(FN); ++k) mid = mid && (c.ks[k][0] == 1 || c.ks[k][0] == 0) && c.rs[k][0] != 1;
+      for (int k = 0; k < cw_inputs(FN); ++k) mid = mid && (c.ks[k][0] == 1 || c.ks[k][0] == 0) && rs2[k][0] != 1;
       // ... and there are enough (kept row tile, other kept index) pairs to fill the GPU: a block owns one
       mid = mid && cdiv<size_t>(c.kd[0], 64) * (c.n_out / c.kd[0]) >= 128;
+      // a short reduced axis (a thread per output walked its 35 terms one round trip at a time: 26 us for
+      // 1024 x 35 x 16 summed over the 35) takes these kernels too; the shortest stay with a thread per output
+      if (mid || c.n_red >= 8) {
+        for (int j = 0; j < 5; ++j) {
+          c.rd[j] = rd2[j];
+          for (int k = 0; k < 3; ++k) c.rs[k][j] = rs2[k][j];
+        }
+      }
       if (mid) {
         const size_t n_rest = c.n_out / c.kd[0];
         const dim3 grid(cdiv<unsigned>(c.kd[0], 64), unsigned(n_rest < 65535 ? n_rest : 65535)), block(64 * kCwMidWaves);
@@ -533,14 +559,72 @@ static int cw_launch_reduce(dyhip_device* dev, const unsigned* full, const unsig
         DYHIP_CHECK_LAUNCH();
         return DYHIP_OK;
       }
-      const dim3 grid(cw_grid(c.n_out, 4, dev)), block(256);
-      // operands far larger than the caches are read once: streaming loads
-      const bool nt = vec && c.n_out * c.n_red * sizeof(float) >= dev->stream_threshold;
-      if (nt) hipLaunchKernelGGL((cwise_reduce_row_kernel<FN, true, true>), grid, block, 0, dev->stream, c, p0, p1, p2, out);
-      else if (vec) hipLaunchKernelGGL((cwise_reduce_row_kernel<FN, true, false>), grid, block, 0, dev->stream, c, p0, p1, p2, out);
-      else hipLaunchKernelGGL((cwise_reduce_row_kernel<FN, false, false>), grid, block, 0, dev->stream, c, p0, p1, p2, out);
-      DYHIP_CHECK_LAUNCH();
-      return DYHIP_OK;
+      if (c.n_red >= 8) {
+        // Few outputs with a long reduced axis (3 outputs of 100 000 terms: 12..190 us with a wavefront per output):
+        // the axis in pieces over more wavefronts, the pieces' sums in scratch, then summed per output in a fixed order.
+        float* target = out;
+        if (c.n_out < 8 * cus && c.n_red >= 8192) {
+          // a wavefront takes 256 terms a round trip with scalar loads, 1024 with 128-bit loads: about four round trips
+          unsigned chunks = unsigned(std::min(cdiv<size_t>(c.n_red, vec ? 4096 : 1024), cdiv<size_t>(16 * cus, c.n_out)));
+          const unsigned len = unsigned(cdiv<size_t>(cdiv<size_t>(c.n_red, chunks), 1024) * 1024);
+          chunks = unsigned(cdiv<size_t>(c.n_red, len));
+          if (chunks >= 2 && scratch != nullptr && scratch_floats >= c.n_out * chunks) {
+            c.chunks = chunks;
+            c.chunk_len = len;
+            c.overwrite = 1;
+            target = scratch;
+          }
+        }
+        const dim3 grid(cw_grid(c.n_out * c.chunks, 4, dev)), block(256);
+        // operands far larger than the caches are read once: streaming loads
+        const bool nt = vec && c.n_out * c.n_red * sizeof(float) >= dev->stream_threshold;
+        if (nt) hipLaunchKernelGGL((cwise_reduce_row_kernel<FN, true, true>), grid, block, 0, dev->stream, c, p0, p1, p2, target);
+        else if (vec) hipLaunchKernelGGL((cwise_reduce_row_kernel<FN, true, false>), grid, block, 0, dev->stream, c, p0, p1, p2, target);
+        else hipLaunchKernelGGL((cwise_reduce_row_kernel<FN, false, false>), grid, block, 0, dev->stream, c, p0, p1, p2, target);
+        DYHIP_CHECK_LAUNCH();
+        if (target != out) {
+          CwReduce f;
+          for (int j = 0; j < 5; ++j) {
+            f.kd[j] = f.rd[j] = 1;
+            for (int k = 0; k < 3; ++k) f.ks[k][j] = f.rs[k][j] = 0;
+          }
+          f.kd[0] = unsigned(c.n_out);
+          f.ks[0][0] = c.chunks;
+          f.rd[0] = c.chunks;
+          f.rs[0][0] = 1;
+          f.n_out = c.n_out;
+          f.n_red = c.chunks;
+          f.chunks = 1;
+          f.chunk_len = 0;
+          f.overwrite = overwrite ? 1 : 0;
+          hipLaunchKernelGGL((cwise_reduce_row_kernel<3, false, false>), dim3(cw_grid(f.n_out, 4, dev)), dim3(256), 0,
+                             dev->stream, f, scratch, nullptr, nullptr, out);
+          DYHIP_CHECK_LAUNCH();
+        }
+        return DYHIP_OK;
+      }
+    }
+  }
+  // Reduced axes with kept axes between them (a 512 x 512 x batch-8 tensor summed over its rows and the batch: 47 us
+  // with a wavefront per output decomposing every index): the first run of adjacent reduced axes into scratch by the
+  // kernels above, the rest from there.
+  if (runs >= 2 && c.n_red >= 64 && scratch != nullptr) {
+    unsigned dstage[5], full2[5];
+    size_t left = 1;
+    for (int j = 0; j < 5; ++j) {
+      const bool reduced = dself[j] == 1 && full[j] > 1;
+      dstage[j] = reduced && j < first_run_end ? 1 : full[j];
+      full2[j] = dstage[j];
+      left *= full2[j];
+    }
+    if (left <= scratch_floats / 2) {
+      DYHIP_CHECK_STATUS(cw_launch_reduce<FN>(dev, full, dstage, s, p0, p1, p2, scratch, true, scratch + left,
+                                              scratch_floats - left));
+      size_t s2[3][5];
+      cw_strides(full2, full2, s2[0]);
+      for (int j = 0; j < 5; ++j) s2[1][j] = s2[2][j] = 0;
+      return cw_launch_reduce<3>(dev, full2, dself, s2, scratch, nullptr, nullptr, out, overwrite, scratch + left,
+                                 scratch_floats - left);
     }
   }
   if (c.n_red >= 64)
@@ -672,9 +756,14 @@ int dyhip_cwise_backward(dyhip_device* dev, int op, const unsigned* dims_a, cons
       (op == DYHIP_CWISE_SUM || other_full))
     return batch_reduce(dev, n, static_cast<unsigned>(bd), dEdf, op == DYHIP_CWISE_MULT ? other : nullptr, dEdxi, true, ws,
                         ws_bytes);
-  if (op == DYHIP_CWISE_SUM) return cw_launch_reduce<3>(dev, full, dself, s, dEdf, nullptr, nullptr, dEdxi);
-  if (op == DYHIP_CWISE_MULT) return cw_launch_reduce<4>(dev, full, dself, s, dEdf, p1, nullptr, dEdxi);
-  return cw_launch_reduce<6>(dev, full, dself, s, dEdf, p1, p2, dEdxi);
+  // intermediate sums of the multi-stage reductions: the device's own scratch (stream-ordered like every other use)
+  float* scratch = static_cast<float*>(dev->gemm_ws);
+  const size_t scratch_floats = scratch != nullptr ? dev->gemm_ws_bytes / sizeof(float) : 0;
+  if (op == DYHIP_CWISE_SUM)
+    return cw_launch_reduce<3>(dev, full, dself, s, dEdf, nullptr, nullptr, dEdxi, false, scratch, scratch_floats);
+  if (op == DYHIP_CWISE_MULT)
+    return cw_launch_reduce<4>(dev, full, dself, s, dEdf, p1, nullptr, dEdxi, false, scratch, scratch_floats);
+  return cw_launch_reduce<6>(dev, full, dself, s, dEdf, p1, p2, dEdxi, false, scratch, scratch_floats);
 }
 
 int dyhip_const_plus_x_forward(dyhip_device* dev, size_t n, float c, const float* x, float* fx) {

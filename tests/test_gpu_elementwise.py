@@ -378,6 +378,19 @@ CWISE_SHAPES = [
     ((12, 5, 3, 1, 4), (12, 1, 3, 1, 4)),
     ((130, 9, 1, 1, 70000), (130, 1, 1, 1, 70000)),  # more than 65535 entries along the outer axis
     ((8, 3, 1, 1, 5), (8, 3, 1, 1, 1)),
+    # gradients of the broadcast argument: a short reduced middle axis (lanes along the rows), a short contiguous
+    # reduced axis (a wavefront per output), few outputs with a long reduced axis (pieces through scratch, strided,
+    # 128-bit and ragged), reduced axes with a kept axis between them (two stages through scratch)
+    ((1024, 35, 1, 1, 16), (1024, 1, 1, 1, 16)),
+    ((50, 1, 1, 1, 500), (1, 1, 1, 1, 500)),
+    ((9, 4, 1, 1, 300), (1, 4, 1, 1, 300)),
+    ((3, 20000, 1, 1, 1), (3, 1, 1, 1, 1)),
+    ((20000, 3, 1, 1, 1), (1, 3, 1, 1, 1)),
+    ((10001, 3, 1, 1, 2), (1, 3, 1, 1, 2)),
+    ((7, 9, 11, 1, 20), (7, 1, 11, 1, 1)),
+    ((128, 96, 1, 1, 8), (1, 96, 1, 1, 1)),
+    ((2, 2, 2, 2, 500), (2, 1, 2, 1, 500)),
+    ((6, 40, 3, 5, 4), (6, 1, 3, 1, 4)),
 ]
 
 
