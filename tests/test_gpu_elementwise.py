@@ -437,6 +437,48 @@ def test_cwise_with_dimension_broadcast(dev, op, da, db):
                          floor=np.maximum(np.abs(g0), rms(dy) * other * np.sqrt(terms)))
 
 
+def test_cwise_random_broadcast_shapes(dev):
+    """Forty random shapes of up to five axes with random broadcast patterns (one long axis now and then, so that every
+    reduction form is reached: thread, wavefront, lanes along rows, pieces through scratch, two stages): forward and
+    both gradients of CwiseMultiply and CwiseQuotient against the oracle (dynet/nodes-arith-cwise.cc:196-307, 338-421)."""
+    rng = np.random.default_rng(2024)
+    for case in range(40):
+        full = [int(rng.integers(1, 9)) for _ in range(5)]
+        if case % 3 == 0:
+            full[int(rng.integers(0, 5))] = int(rng.choice([70, 300, 1100, 9000]))
+        if case % 7 == 0:
+            full[0] = 4 * int(rng.integers(1, 40))
+        keep = [bool(rng.integers(0, 2)) for _ in range(5)]
+        da = tuple(full)
+        db = tuple(f if k else 1 for f, k in zip(full, keep))
+        for op in (lib.CWISE_MULT, lib.CWISE_QUOTIENT):
+            a = f32(rng.standard_normal(da[::-1]))
+            b = f32(rng.standard_normal(db[::-1]))
+            if op == lib.CWISE_QUOTIENT:
+                b = f32(np.sign(b) * (np.abs(b) + 0.5))
+            at, bt = dev.tensor(a), dev.tensor(b)
+            want = orc.cwise_forward(op, da, db, a, b)
+            fx = dev.empty(want.shape)
+            dev.cwise_forward(op, da, db, at, bt, fx)
+            assert_close(fx.numpy(), want, FWD_RTOL, "cwise fwd %s x %s" % (da, db))
+            dy = f32(rng.standard_normal(want.shape))
+            dyt = dev.tensor(dy)
+            for i, x in enumerate((a, b)):
+                g0 = f32(rng.standard_normal(x.shape))
+                gt = dev.tensor(g0)
+                dev.cwise_backward(op, da, db, at, bt, dyt, i, gt)
+                ref = orc.cwise_backward(op, da, db, a, b, dy, i, g0.copy())
+                terms = want.size / x.size
+                other = np.abs(b if i == 0 else a).max()
+                if op == lib.CWISE_QUOTIENT:
+                    other = (1.0 / np.abs(b).min()) * (1.0 if i == 0 else np.abs(a).max() / np.abs(b).min())
+                assert_close(gt.numpy(), ref, GRAD_RTOL, "cwise bwd op %d arg %d %s x %s" % (op, i, da, db),
+                             floor=np.maximum(np.abs(g0), rms(dy) * other * np.sqrt(terms)))
+        for w in (lib.POOL_FXS, lib.POOL_DEDFS, lib.POOL_SCS):
+            dev.sync()
+            dev.free_pool(w)
+
+
 def test_layer_norm_composite_of_eight_nodes_on_the_device(dev):
     """dynet/expr.cc:248-253 issued node by node through the C-ABI (mean_elems, Negate, CwiseSum, std_elems,
     ConstantPlusX, CwiseQuotient, CwiseMultiply, CwiseSum; forward and backward) at the baseline's shape, against
