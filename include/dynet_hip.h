@@ -457,8 +457,8 @@ int dyhip_lookup_forward(dyhip_device* dev, unsigned n_ids, const unsigned* ids_
 int dyhip_lookup_accumulate_grads_workspace(unsigned n_ids, size_t dim, unsigned vocab, size_t* ws_bytes);
 /* The same in two phases.  The plan depends only on the ids, so an executor can build it right after the
  * forward gather (the ids sit in the node's aux_mem from then on) and the backward pass is left with the
- * reduction kernel.  Up to 65535 ids the plan is built by one kernel; beyond that by a device-wide radix
- * sort.  The plan is opaque; vocab must be below 2^31 - 1.  dyhip_lookup_accumulate_grads_planned takes no
+ * reduction kernel.  Up to 65535 ids the plan is built by one kernel; beyond that by a radix sort over
+ * all blocks (three launches per 8 bits of the vocabulary size) and one kernel for the run ends.  The plan is opaque; vocab must be below 2^31 - 1.  dyhip_lookup_accumulate_grads_planned takes no
  * workspace any more (its size query returns 0; ws may be NULL). */
 int dyhip_lookup_plan_bytes(unsigned n_ids, size_t* plan_bytes);
 int dyhip_lookup_plan_workspace(unsigned n_ids, unsigned vocab, size_t* ws_bytes);

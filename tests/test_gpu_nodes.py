@@ -1139,8 +1139,13 @@ def _check_plan(dev, plan, ids, vocab):
     (50000, 4480, "zipf"),         # 16-bit keys, 5 steps of 64 ids per wavefront: the 8-step form of the direct kernel
     (50000, 32768, "zipf"),        # ... 32 steps: the longest the direct kernel takes
     (50000, 32769, "zipf"),        # ... 33: the compact-and-sort kernel although the keys fit 16 bits
-    (50000, 65536, "zipf"),        # the first size of the radix-sort plan
-    (300000, 70001, "zipf"),
+    (50000, 65536, "zipf"),        # the first size of the radix-sort plan (two passes)
+    (300000, 70001, "zipf"),       # ... three passes
+    (200, 70000, "uniform"),       # ... one pass
+    (1 << 30, 66000, "uniform"),   # ... four
+    (50000, 600000, "zipf"),       # ... pieces of more than 2048 ids a block
+    (1000, 70000, "same"),         # ... every id beyond the vocabulary: one run that the reduction skips
+    (70000, 100000, "same"),       # ... one id only
     (1 << 20, 30000, "uniform"),   # 21-bit ids: two sort passes beyond the bucket digit
     (1 << 30, 5000, "uniform"),    # 31-bit ids: three
     (256, 20000, "uniform"),       # vocab fits the bucket digit plus the sentinel's extra bit
