@@ -113,7 +113,8 @@ def test_unary_rejects_unknown_operator(dev):
     assert e.value.status == lib.ERR_INVALID_ARG
 
 
-@pytest.mark.parametrize("n,bd0,bd1", [(N_BIG // 64, 64, 64), (1024, 4096, 1), (1024, 1, 4096), (7, 5, 1), (5, 1, 1)])
+@pytest.mark.parametrize("n,bd0,bd1", [(N_BIG // 64, 64, 64), (1024, 4096, 1), (1024, 1, 4096), (7, 5, 1), (5, 1, 1),
+                                       (7, 20000, 1), (1, 1, 70000), (24, 1, 3000)])
 def test_cmult_and_csum(dev, n, bd0, bd1):
     rng = np.random.default_rng(21)
     bd = max(bd0, bd1)
@@ -139,16 +140,21 @@ def test_cmult_and_csum(dev, n, bd0, bd1):
 
 
 @pytest.mark.parametrize("n,bd", [(64 * 1024, 64), (1024, 4096), (1027, 33), (3, 2), (5, 1), (4096, 7), (1, 100000), (2, 777),
-                                  (255, 1000)])
+                                  (255, 1000),
+                                  # batch elements of at most 32 floats, many of them: the flat walk (and its limits)
+                                  (1, 32768), (1, 32767), (3, 100000), (7, 50001), (20, 5000), (31, 4000), (32, 3000),
+                                  (33, 3000), (1, 3000000)])
 def test_sum_batches(dev, n, bd):
     rng = np.random.default_rng(31)
     x = f32(rng.standard_normal((bd, n)))
     yt = dev.empty(n)
     dev.sum_batches_forward(n, bd, dev.tensor(x), yt)
     ref = orc.sum_batches_forward(n, bd, x)
-    assert_close(yt.numpy(), ref, FWD_RTOL, "sum_batches fwd", floor=np.sqrt(bd))
-    # the batch order does not matter beyond rounding: compare with fp64 too
+    # the batch order does not matter beyond rounding: compare with fp64
     assert_close(yt.numpy(), x.astype(np.float64).sum(0), FWD_RTOL, "sum_batches vs fp64", floor=np.sqrt(bd))
+    # ... and with the oracle's sequential fp32 sum, which has itself drifted by a few 1e-5 of sqrt(bd) x |partial sums|
+    # once the batch has tens of thousands of elements (-314.1896 against -314.1811 in fp64 at 3 x 100 000)
+    assert_close(yt.numpy(), ref, FWD_RTOL * (1 if bd < 30000 else 8), "sum_batches fwd", floor=np.sqrt(bd))
     dy, g0 = f32(rng.standard_normal(n)), f32(rng.standard_normal((bd, n)))
     gt = dev.tensor(g0)
     dev.sum_batches_backward(n, bd, dev.tensor(dy), gt)
