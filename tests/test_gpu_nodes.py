@@ -1429,6 +1429,56 @@ def test_argmax_shapes_with_ties(dev, rows, bd):
     assert np.array_equal(idx.numpy(), x.argmax(axis=1))
 
 
+@pytest.mark.parametrize("rows,bd", [(65536, 2), (70001, 1), (131072, 3), (300001, 2)])
+def test_vocabulary_length_columns_of_a_small_batch(dev, rows, bd):
+    """Columns of 65 536 rows and more in a batch of a few are cut into chunks over many blocks (log-sum-exp, the dot
+    of the softmax backward, argmax).  The oracle's sequential fp32 sums drift at this length, so the references are
+    the same formulas in fp64 (dynet/tensor.cc:468-507, nodes-pickneglogsoftmax.cc:72-145, nodes-softmaxes.cc:40-213,
+    nodes-argmax.cc:44-55); maxima, picks and argmax are exact."""
+    rng = np.random.default_rng(rows + bd)
+    x = f32(rng.standard_normal((bd, rows)) * 3)
+    x[0, : rows // 3] = -np.inf  # masked logits
+    x64 = x.astype(np.float64)
+    mx = x.max(axis=1)
+    lse = np.log(np.exp(x64 - mx[:, None].astype(np.float64)).sum(axis=1)) + mx
+    xt = dev.tensor(x)
+    m, z = dev.empty(bd), dev.empty(bd)
+    dev.logsumexp_cols(rows, bd, xt, m, z)
+    assert m.numpy().tobytes() == mx.tobytes()
+    assert_close(z.numpy(), lse, FWD_RTOL, "logsumexp", floor=1.0)
+    labels = rng.integers(rows // 3, rows, bd).astype(np.uint32)
+    aux, fx = dev.empty(3 * bd), dev.empty(bd)
+    dev.pnls_forward(rows, bd, xt, labels, aux, fx)
+    assert_close(fx.numpy(), lse - x64[np.arange(bd), labels], FWD_RTOL, "pnls", floor=1.0)
+    sm = np.exp(x64 - lse[:, None])
+    y = dev.empty((bd, rows))
+    dev.softmax_forward(rows, bd, xt, y)
+    assert_close(y.numpy(), sm, FWD_RTOL, "softmax", floor=1.0 / rows)
+    dy, g0 = f32(rng.standard_normal((bd, rows))), f32(rng.standard_normal((bd, rows)))
+    gt = dev.tensor(g0)
+    dev.softmax_backward(rows, bd, dev.tensor(f32(sm)), dev.tensor(dy), gt)
+    smf = f32(sm).astype(np.float64)
+    want = g0 + (dy - (smf * dy).sum(axis=1, keepdims=True)) * smf
+    assert_close(gt.numpy(), want, GRAD_RTOL, "softmax bwd", floor=1.0)
+    aux2 = dev.empty(2 * bd)
+    dev.log_softmax_forward(rows, bd, xt, aux2, y)
+    got = y.numpy()
+    fin = np.isfinite(x)
+    assert np.array_equal(np.isneginf(got), ~fin)
+    assert_close(np.where(fin, got, 0.0), np.where(fin, x64 - lse[:, None], 0.0), FWD_RTOL, "log_softmax", floor=1.0)
+    lsm = f32(np.where(fin, x64 - lse[:, None], -50.0))
+    gt = dev.tensor(g0)
+    dev.log_softmax_backward(rows, bd, dev.tensor(lsm), dev.tensor(dy), aux2, gt)
+    want = g0 + dy - np.exp(lsm.astype(np.float64)) * dy.astype(np.float64).sum(axis=1, keepdims=True)
+    assert_close(gt.numpy(), want, GRAD_RTOL, "log_softmax bwd", floor=np.sqrt(rows))
+    idx = dev.empty(bd, np.int64)
+    xi = f32(rng.integers(0, 9, (bd, rows)))  # every column holds its maximum thousands of times: the first wins
+    dev.argmax_cols(rows, bd, dev.tensor(xi), idx)
+    assert np.array_equal(idx.numpy(), xi.argmax(axis=1))
+    dev.argmax_cols(rows, bd, xt, idx)
+    assert np.array_equal(idx.numpy(), x.argmax(axis=1))
+
+
 def test_argmax_node(dev, golden):
     """The Argmax node (dynet/nodes-argmax.cc:44-68): one-hot forward with the reference test's vector, bit-exact against
     the oracle on a larger case with ties, straight-through backward = accumulate."""
