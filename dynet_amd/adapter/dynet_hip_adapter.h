@@ -779,6 +779,83 @@ struct LogSumExpDimension : public Node {
   }
 };
 
+// LogSumExp over its arguments (dynet/nodes-logsumexp.cc:38-124): same shape, each with the result's batch size or 1
+struct LogSumExp : public Node {
+  static void gather(const std::vector<const Tensor*>& xs, std::vector<const float*>& p, std::vector<unsigned>& b) {
+    for (const Tensor* x : xs) {
+      p.push_back(x->v);
+      b.push_back(x->d.bd);
+    }
+  }
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    std::vector<const float*> p;
+    std::vector<unsigned> b;
+    gather(xs, p, b);
+    abi_check(dyhip_logsumexp_node_forward(dev.hip, static_cast<unsigned>(xs.size()), fx.d.batch_size(), fx.d.bd, p.data(),
+                                           b.data(), fx.v));
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, const Tensor& fx,
+                         const Tensor& dEdf, unsigned i, Tensor& dEdxi) const override {
+    std::vector<const float*> p;
+    std::vector<unsigned> b;
+    gather(xs, p, b);
+    // an argument broadcast over the batch: its terms are formed in scratch and summed over the batch from there
+    size_t need = 0;
+    if (xs[i]->d.bd != fx.d.bd) {
+      abi_check(dyhip_batch_reduce_workspace(fx.d.batch_size(), fx.d.bd, &need));
+      need += (sizeof(float) * fx.d.size() + 255) / 256 * 256;
+    }
+    void* ws = need ? scratch(fx)->allocate(need) : nullptr;
+    abi_check(dyhip_logsumexp_node_backward(dev.hip, static_cast<unsigned>(xs.size()), fx.d.batch_size(), fx.d.bd, p.data(),
+                                            b.data(), fx.v, dEdf.v, i, dEdxi.v, ws, need));
+    scratch(fx)->free();
+  }
+};
+
+// Sum / esum (dynet/nodes-arith-sum.cc:65-129): any number of same-shaped arguments with the result's batch size or 1
+struct Sum : public Node {
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    if (xs.empty()) throw std::invalid_argument("Sum needs at least one argument");  // nodes-arith-sum.cc:39
+    std::vector<const float*> p;
+    std::vector<unsigned> b;
+    LogSumExp::gather(xs, p, b);
+    abi_check(dyhip_sum_forward(dev.hip, static_cast<unsigned>(xs.size()), fx.d.batch_size(), fx.d.bd, p.data(), b.data(),
+                                fx.v));
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, const Tensor& fx,
+                         const Tensor& dEdf, unsigned i, Tensor& dEdxi) const override {
+    size_t need = 0;
+    abi_check(dyhip_batch_reduce_workspace(fx.d.batch_size(), fx.d.bd, &need));
+    void* ws = need ? scratch(fx)->allocate(need) : nullptr;
+    // dEdxi += dEdf, summed over the batch for an argument of batch size 1 (:115-128)
+    abi_check(dyhip_csum_backward(dev.hip, fx.d.batch_size(), xs[i]->d.bd, fx.d.bd, dEdf.v, 0, dEdxi.v, ws, need));
+    scratch(fx)->free();
+  }
+};
+
+// PickRange (dynet/nodes-select.cc:216-259): the slice [start, end) of dimension `dim`
+struct PickRange : public Node {
+  PickRange(unsigned start, unsigned end, unsigned dim = 0) : start(start), end(end), dim(dim) {}
+  unsigned start, end, dim;
+  void split(const Dim& d, size_t& inner, size_t& len, size_t& outer) const {
+    inner = 1;
+    outer = d.bd;
+    for (unsigned j = 0; j < d.nd; ++j) (j < dim ? inner : outer) *= j == dim ? 1 : d[j];
+    len = d[dim];
+  }
+  void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {
+    size_t inner, len, outer;
+    split(xs[0]->d, inner, len, outer);
+    abi_check(dyhip_pick_range_forward(dev.hip, inner, len, outer, start, end, xs[0]->v, fx.v));
+  }
+  void backward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, const Tensor&, const Tensor& dEdf,
+                         unsigned, Tensor& dEdxi) const override {
+    size_t inner, len, outer;
+    split(xs[0]->d, inner, len, outer);
+    abi_check(dyhip_pick_range_backward(dev.hip, inner, len, outer, start, end, dEdf.v, dEdxi.v));
+  }
+};
+
 // AffineTransform with one (W, x) pair (dynet/nodes-affinetransform.cc:77-156).  xs = {bias, W, x}
 struct AffineTransform : public Node {
   void forward_dev_impl(const Device_GPU& dev, const std::vector<const Tensor*>& xs, Tensor& fx) const override {

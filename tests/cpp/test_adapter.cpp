@@ -427,6 +427,95 @@ static void elementwise_gradients(Fixture& F) {
   }
 }
 
+// ---- tests/test-nodes.cc:297-372 (sum, logsumexp) and :1984-2000 (pick_range): the node-level part of each ----
+static void sum_logsumexp_pick_range(Fixture& F) {
+  const vector<float> param_vals = {1.1f, -2.2f, 3.3f}, param2_vals = {2.2f, 3.4f, -1.2f};
+  const vector<float> batch_vals = {1.f, 2.f, 3.f, 4.f, 5.f, 6.f};
+  g_case = "sum_gradient";
+  {
+    vector<Tensor> a = {F.input(Dim({3}), param2_vals), F.input(Dim({3}), param_vals), F.input(Dim({3}), param2_vals)};
+    CHECK(check_grad(F, Sum(), a, Dim({3}), {true, true, true}));
+    Tensor y = F.dev.allocate_tensor(DeviceMempool::FXS, Dim({3}));
+    Sum().forward_dev_impl(F.dev, {&a[0], &a[1], &a[2]}, y);
+    const vector<float> v = as_vector(y);
+    for (int j = 0; j < 3; ++j) CHECK_CLOSE(v[j], 2.0 * param2_vals[j] + param_vals[j], 0.001);
+  }
+  g_case = "sum_batch_gradient";  // arguments of batch size 2 and 1: the latter's gradient is summed over the batch
+  {
+    vector<Tensor> a = {F.input(Dim({3}, 2), batch_vals), F.input(Dim({3}), param_vals), F.input(Dim({3}, 2), batch_vals)};
+    CHECK(check_grad(F, Sum(), a, Dim({3}, 2), {true, true, true}));
+  }
+  g_case = "empty_sum";
+  {
+    bool thrown = false;
+    Tensor y = F.dev.allocate_tensor(DeviceMempool::FXS, Dim({3}));
+    try {
+      Sum().forward_dev_impl(F.dev, {}, y);
+    } catch (const std::invalid_argument&) {
+      thrown = true;
+    }
+    CHECK(thrown);
+  }
+  g_case = "logsumexp_gradient";
+  {
+    vector<Tensor> a = {F.input(Dim({1}), {2.2f}), F.input(Dim({1}), {1.1f})};
+    CHECK(check_grad(F, LogSumExp(), a, Dim({1}), {true, true}));
+    Tensor y = F.dev.allocate_tensor(DeviceMempool::FXS, Dim({1}));
+    LogSumExp().forward_dev_impl(F.dev, {&a[0], &a[1]}, y);
+    CHECK_CLOSE(as_vector(y)[0], std::log(std::exp(2.2) + std::exp(1.1)), 0.001);
+  }
+  g_case = "logsumexp_vector_gradient";
+  {
+    vector<Tensor> a = {F.input(Dim({3}), param_vals), F.input(Dim({3}), param2_vals)};
+    CHECK(check_grad(F, LogSumExp(), a, Dim({3}), {true, true}));
+  }
+  g_case = "logsumexp_singleelem_batch_gradient";
+  {
+    vector<Tensor> a = {F.input(Dim({1}, 3), param_vals)};
+    CHECK(check_grad(F, LogSumExp(), a, Dim({1}, 3), {true}));
+  }
+  g_case = "logsumexp_inequal_batch_gradient";
+  {
+    vector<float> x3(6);
+    for (int j = 0; j < 6; ++j) x3[j] = param_vals[j % 3] + batch_vals[j];
+    vector<Tensor> a = {F.input(Dim({3}), param_vals), F.input(Dim({3}, 2), x3)};
+    CHECK(check_grad(F, LogSumExp(), a, Dim({3}, 2), {true, true}));
+  }
+  g_case = "logsumexp_forty_arguments";  // more than one launch takes: chained through the result
+  {
+    vector<Tensor> a;
+    vector<const Tensor*> xs;
+    double want = 0;
+    for (int k = 0; k < 40; ++k) {
+      a.push_back(F.input(Dim({1}), {0.1f * float(k) - 2.f}));
+      want += std::exp(0.1 * k - 2.0);
+    }
+    for (Tensor& t : a) xs.push_back(&t);
+    Tensor y = F.dev.allocate_tensor(DeviceMempool::FXS, Dim({1}));
+    LogSumExp().forward_dev_impl(F.dev, xs, y);
+    CHECK_CLOSE(as_vector(y)[0], std::log(want), 0.001);
+  }
+  g_case = "pick_range_gradient";
+  {
+    vector<Tensor> a = {F.input(Dim({3}), param_vals)};
+    CHECK(check_grad(F, PickRange(0, 2), a, Dim({2}), {true}));
+    Tensor y = F.dev.allocate_tensor(DeviceMempool::FXS, Dim({2}));
+    PickRange(0, 2).forward_dev_impl(F.dev, {&a[0]}, y);
+    const vector<float> v = as_vector(y);
+    CHECK(v[0] == param_vals[0] && v[1] == param_vals[1]);
+  }
+  g_case = "pick_range_dim_gradient";
+  {
+    const vector<float> sq = {1.1f, 2.2f, 3.3f, 1.2f, 2.1f, 3.4f, 1.3f, 2.3f, 3.5f};  // 3 x 3, column-major
+    vector<Tensor> a = {F.input(Dim({3, 3}), sq)};
+    CHECK(check_grad(F, PickRange(0, 2, 1), a, Dim({3, 2}), {true}));
+    Tensor y = F.dev.allocate_tensor(DeviceMempool::FXS, Dim({3, 2}));
+    PickRange(1, 3, 1).forward_dev_impl(F.dev, {&a[0]}, y);
+    const vector<float> v = as_vector(y);
+    for (int j = 0; j < 6; ++j) CHECK(v[j] == sq[3 + j]);
+  }
+}
+
 // ---- tests/test-nodes.cc:2404-2426 ----
 static void layer_norm(Fixture& F) {
   g_case = "layer_norm_forward";
@@ -816,7 +905,8 @@ int main(int argc, char** argv) {
   const std::vector<std::function<void(Fixture&)>> cases = {lstm_node_h_fwd,      lstm_node_c_fwd, lstm_node_gates_fwd,
                                                              lstm_node_gradients,  elementwise_gradients, layer_norm,
                                                              lookup_and_softmax,   random_nodes,    cwise_broadcast,       layer_norm_composite,
-                                                             combine_and_accumulate, argmax_node, deferred_parameter_gradients};
+                                                             combine_and_accumulate, argmax_node, deferred_parameter_gradients,
+                                                             sum_logsumexp_pick_range};
   for (const auto& c : cases) {
     c(F);
     F.reset();
