@@ -299,6 +299,60 @@ def extras_kernels(dev, lib, n_sets=None):
          lambda s: dev.layer_norm_backward(n, bd, s["x"], g, s["dy"], s["dx"], dg, db, ws_ln, ws_lnb)),
     ]
     yield "layer_norm_wide_rows", {"n": n, "bd": bd, "rotating_buffer_sets": len(sets)}, named, sets
+    # ---- shapes off the baseline's grid: small and transposed products, long elements of a small batch, reductions
+    # along dim 1, vocabulary-length columns of a batch of one or two, short and long reduced axes of the broadcast
+    # gradients, sums of scalars over a batch.  One buffer set each (a few MB at most: these live in the caches in
+    # use too); the figure is the time of one call inside a long graph. -----------------------------------------
+    R = lambda *shape: dev.tensor(rng.standard_normal(shape).astype(np.float32))
+    Z = lambda *shape: dev.zeros(shape, pool=lib.POOL_DEDFS)
+    s0 = {}
+    named = []
+
+    def add(name, nbytes, fn):
+        named.append((name, nbytes, lambda s, fn=fn: fn()))
+
+    a, b, y = R(128, 128), R(128, 128), Z(128, 128)
+    add("gemm l^T*r 128x128x128", 3 * 128 * 128 * 4, lambda a=a, b=b, y=y: dev.gemm_tn_acc(128, 128, 128, a, b, y))
+    a, b, y = R(512, 512), R(512, 512), Z(512, 512)
+    add("gemm l^T*r 512x512x512", 3 * 512 * 512 * 4, lambda a=a, b=b, y=y: dev.gemm_tn_acc(512, 512, 512, a, b, y))
+    a, b, y = R(650, 650), R(1, 650), Z(1, 650)
+    add("gemm l*r 650x1x650 (leading dimension not a multiple of 4)", (650 * 650 + 1300) * 4,
+        lambda a=a, b=b, y=y: dev.gemm_nn(650, 1, 650, a, b, 0.0, y))
+    a, b, y = R(128, 1024, 1), R(128, 1024, 35), Z(128, 35, 1)
+    add("gemm strided-batched l*r^T 1x35x1024 x 128 items", 128 * (1024 + 35 * 1024 + 35) * 4,
+        lambda a=a, b=b, y=y: dev.gemm_strided_batched(0, 1, 1, 35, 1024, a, 1024, b, 35 * 1024, 0.0, y, 35, 128))
+    a, b, y = R(1000, 9, 7), R(1000, 5, 9), Z(1000, 5, 7)
+    add("gemm strided-batched l*r 7x5x9 x 1000 items", 1000 * (63 + 45 + 35) * 4,
+        lambda a=a, b=b, y=y: dev.gemm_strided_batched(0, 0, 7, 5, 9, a, 63, b, 45, 0.0, y, 35, 1000))
+    n, bd = 1 << 20, 4
+    x, m, dy, dx = R(bd, n), dev.empty(bd), R(bd), Z(bd, n)
+    add("mean_elems 1048576 x 4", n * bd * 4, lambda x=x, m=m: dev.mean_elems_forward(1 << 20, 4, x, m))
+    add("std_elems 1048576 x 4", n * bd * 4, lambda x=x, m=m: dev.std_elems_forward(1 << 20, 4, x, m))
+    add("std_elems_bwd 1048576 x 4", 3 * n * bd * 4, lambda x=x, m=m, dy=dy, dx=dx: dev.std_elems_backward(1 << 20, 4, x, m, dy, dx))
+    x, y = R(1, 2048, 2048), dev.empty((1, 2048, 2048))
+    add("softmax along dim 1, 2048 x 2048", 2 * 2048 * 2048 * 4, lambda x=x, y=y: dev.softmax_rows_forward(2048, 2048, 1, x, y))
+    rows, bd = 300000, 2
+    x, m, z, dy, dx = R(bd, rows), dev.empty(bd), dev.empty(bd), R(bd, rows), Z(bd, rows)
+    add("logsumexp_cols 300000 x 2", rows * bd * 4, lambda x=x, m=m, z=z: dev.logsumexp_cols(300000, 2, x, m, z))
+    add("softmax_bwd 300000 x 2", 4 * rows * bd * 4, lambda x=x, dy=dy, dx=dx: dev.softmax_backward(300000, 2, x, dy, dx))
+    x, idx = R(1, 1000000), dev.empty(1, np.int64)
+    add("argmax_cols 1000000 x 1", 4000000, lambda x=x, idx=idx: dev.argmax_cols(1000000, 1, x, idx))
+    da, db_ = (1024, 35, 1, 1, 16), (1024, 1, 1, 1, 16)
+    a, b, dy, g = R(16, 35, 1024), R(16, 1024), R(16, 35, 1024), Z(16, 1024)
+    add("cwise_mult_bwd_arg1 1024x35x16 by 1024x1x16 (sum over the 35)", 2 * 16 * 35 * 1024 * 4,
+        lambda a=a, b=b, dy=dy, g=g, da=da, db_=db_: dev.cwise_backward(lib.CWISE_MULT, da, db_, a, b, dy, 1, g))
+    da2, db2 = (100000, 3, 1, 1, 1), (1, 3, 1, 1, 1)
+    a, b, dy, g = R(3, 100000), R(3), R(3, 100000), Z(3)
+    add("cwise_quotient_bwd_arg1 100000x3 by 1x3 (three sums of 100000 terms)", 3 * 300000 * 4,
+        lambda a=a, b=b, dy=dy, g=g, da2=da2, db2=db2: dev.cwise_backward(lib.CWISE_QUOTIENT, da2, db2, a, b, dy, 1, g))
+    x, y = R(1000000, 1), dev.empty(1)
+    wsb_, wsbb = dev.workspace(dev.batch_reduce_workspace(1, 1000000))
+    add("sum_batches of 1000000 scalars", 4000000, lambda x=x, y=y: dev.sum_batches_forward(1, 1000000, x, y, wsb_, wsbb))
+    x, y = R(100000, 9, 7), dev.empty((100000, 3, 7))
+    add("pick_range 7x9x100000 [2,5)", 2 * 100000 * 21 * 4, lambda x=x, y=y: dev.pick_range_forward(7, 9, 100000, 2, 5, x, y))
+    xs, y = [R(128, 1) for _ in range(35)], dev.empty((128, 1))
+    add("logsumexp node, 35 arguments of 1 x 128", 36 * 128 * 4, lambda xs=xs, y=y: dev.logsumexp_node_forward(1, 128, xs, [128] * 35, y))
+    yield "off_grid_shapes", {"rotating_buffer_sets": 1}, named, [s0]
 
 
 def extras(dev, lib, reps, use_graph=True):
