@@ -321,6 +321,12 @@ def extras_kernels(dev, lib, n_sets=None):
     a, b, y = R(128, 1024, 1), R(128, 1024, 35), Z(128, 35, 1)
     add("gemm strided-batched l*r^T 1x35x1024 x 128 items", 128 * (1024 + 35 * 1024 + 35) * 4,
         lambda a=a, b=b, y=y: dev.gemm_strided_batched(0, 1, 1, 35, 1024, a, 1024, b, 35 * 1024, 0.0, y, 35, 128))
+    a, b, y = R(128, 35, 1024), R(128, 1, 35), Z(128, 1, 1024)
+    add("gemm strided-batched l*r 1024x1x35 x 128 items (attention context)", 128 * (1024 * 35 + 35 + 1024) * 4,
+        lambda a=a, b=b, y=y: dev.gemm_strided_batched(0, 0, 1024, 1, 35, a, 1024 * 35, b, 35, 0.0, y, 1024, 128))
+    dctx, dH = R(128, 1, 1024), Z(128, 35, 1024)
+    add("gemm strided-batched l*r^T 1024x35x1 x 128 items (rank-one update an item)", 128 * (2 * 1024 * 35 + 35 + 1024) * 4,
+        lambda dctx=dctx, b=b, dH=dH: dev.gemm_strided_batched(0, 1, 1024, 35, 1, dctx, 1024, b, 35, 1.0, dH, 1024 * 35, 128))
     a, b, y = R(1000, 9, 7), R(1000, 5, 9), Z(1000, 5, 7)
     add("gemm strided-batched l*r 7x5x9 x 1000 items", 1000 * (63 + 45 + 35) * 4,
         lambda a=a, b=b, y=y: dev.gemm_strided_batched(0, 0, 7, 5, 9, a, 63, b, 45, 0.0, y, 35, 1000))

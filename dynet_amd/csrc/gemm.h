@@ -84,6 +84,9 @@ int gemm_shallow_nt_run(dyhip_device* dev, size_t M, size_t N, size_t K, const f
 // K x N, k contiguous); *taken tells whether it ran or the shape should go to gemm_run.
 int skinny_tn_gemm(dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B,
                    size_t ldb, float beta, float* C, bool* taken);
+// lstm.hip: the streaming l^T * r kernel (at most four columns of r) over the items of a strided batch
+int thin_tn_batched(dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B, size_t ldb,
+                    float beta, float* C, const GemmBatch* batch, bool* taken);
 
 // lstm.hip: C = epilogue(A0 B0 [+ A1 B1]) in one launch for a right operand of a few 32-column tiles (A: M x K with rows
 // contiguous, B: K x N with k contiguous; two segments only with the gates epilogue); *taken tells whether it ran.

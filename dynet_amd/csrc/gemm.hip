@@ -403,8 +403,13 @@ static GemmPlan plan_gemm(const dyhip_device* dev, size_t M, size_t N, unsigned 
 template <int KT, int kThinCols>  // KT: depth rounded up to a multiple of four
 __global__ __launch_bounds__(256) void gemm_nt_thin_kernel(unsigned M4, unsigned N, unsigned K, const float* __restrict__ A,
                                                            size_t lda, const float* __restrict__ B, size_t ldb,
-                                                           float* __restrict__ C, float beta) {
+                                                           float* __restrict__ C, float beta, size_t stride_a,
+                                                           size_t stride_b, size_t stride_c) {
   __shared__ __attribute__((aligned(16))) float bt[KT][kThinCols];  // the block's entries of B, zero past the ends
+  // item blockIdx.z of a strided batch (the gradient of a batch of matrices times vectors: a rank-one update each)
+  A += size_t(blockIdx.z) * stride_a;
+  B += size_t(blockIdx.z) * stride_b;
+  C += size_t(blockIdx.z) * stride_c;
   const unsigned j0 = blockIdx.y * kThinCols;
   for (unsigned e = threadIdx.x; e < unsigned(KT * kThinCols); e += 256) {
     const unsigned k = e / kThinCols, jj = e % kThinCols;
@@ -448,15 +453,17 @@ static bool gemm_nt_thin_eligible(size_t M, size_t N, size_t K, const float* A, 
 }
 
 static int gemm_nt_thin_run(dyhip_device* dev, size_t M, size_t N, size_t K, const float* A, size_t lda, const float* B,
-                            size_t ldb, float* C, float beta) {
+                            size_t ldb, float* C, float beta, const GemmBatch* batch = nullptr) {
   const unsigned M4 = static_cast<unsigned>(M / 4);
+  const unsigned items = batch != nullptr && batch->count > 1 ? batch->count : 1;
+  const size_t sa = items > 1 ? batch->stride_a : 0, sb = items > 1 ? batch->stride_b : 0, sc = items > 1 ? batch->stride_c : 0;
   // columns per thread: eight, or four, or two while the wider form would leave fewer than two blocks per CU
-  const size_t want = 2 * size_t(dev->num_cus), bxm = cdiv<unsigned>(M4, 256);
+  const size_t want = 2 * size_t(dev->num_cus), bxm = size_t(cdiv<unsigned>(M4, 256)) * items;
   const int cols = bxm * cdiv<size_t>(N, 8) >= want ? 8 : bxm * cdiv<size_t>(N, 4) >= want ? 4 : 2;
-  const dim3 grid(static_cast<unsigned>(bxm), static_cast<unsigned>(cdiv<size_t>(N, size_t(cols)))), block(256);
+  const dim3 grid(cdiv<unsigned>(M4, 256), static_cast<unsigned>(cdiv<size_t>(N, size_t(cols))), items), block(256);
 #define DYHIP_THIN_C(KT, COLS)                                                                                        \
   hipLaunchKernelGGL((gemm_nt_thin_kernel<KT, COLS>), grid, block, 0, dev->stream, M4, static_cast<unsigned>(N),      \
-                     static_cast<unsigned>(K), A, lda, B, ldb, C, beta)
+                     static_cast<unsigned>(K), A, lda, B, ldb, C, beta, sa, sb, sc)
 #define DYHIP_THIN(KT)                     \
   do {                                     \
     if (cols == 8) DYHIP_THIN_C(KT, 8);    \
@@ -494,13 +501,16 @@ __global__ __launch_bounds__(64 * kGemvWaves) void gemm_nn_thin_kernel(unsigned 
                                                                       GemmSeg seg0, GemmSeg seg1, unsigned slabs0,
                                                                       float* __restrict__ C, float beta,
                                                                       const float* __restrict__ bias,
-                                                                      float* __restrict__ partial) {
+                                                                      float* __restrict__ partial, size_t stride_a,
+                                                                      size_t stride_b, size_t stride_c) {
   __shared__ float4 red[kGemvWaves - 1][64][NB];
   // a product over two depth segments (the gates node: Wx x + Wh h) is one sequence of slabs: the first slabs0 walk
   // the first segment, the others the second; the choice is the same for the whole block
   const bool second = blockIdx.y >= slabs0;
-  const float* __restrict__ A = second ? seg1.A : seg0.A;
-  const float* __restrict__ B = second ? seg1.B : seg0.B;
+  // blockIdx.z: the item of a strided batch (one segment, one slab; the strides are 0 otherwise)
+  const float* __restrict__ A = (second ? seg1.A : seg0.A) + size_t(blockIdx.z) * stride_a;
+  const float* __restrict__ B = (second ? seg1.B : seg0.B) + size_t(blockIdx.z) * stride_b;
+  C += size_t(blockIdx.z) * stride_c;
   const size_t lda = second ? seg1.lda : seg0.lda, ldb = second ? seg1.ldb : seg0.ldb;
   const unsigned K = static_cast<unsigned>(second ? seg1.K : seg0.K);
   const unsigned k0 = (second ? blockIdx.y - slabs0 : blockIdx.y) * chunk, k1 = min(K, k0 + chunk);
@@ -788,8 +798,9 @@ static bool gemm_nn_thin_eligible(const dyhip_device* dev, size_t M, size_t N, i
 }
 
 static int gemm_nn_thin_run(dyhip_device* dev, size_t M, size_t N, int nseg, const GemmSeg* segs, float* C,
-                            const GemmEpiParams& epi) {
-  if (gemm_nn_rows_fit(dev, M, N, nseg, segs)) return gemm_nn_rows_run(dev, M, N, nseg, segs, C, epi);
+                            const GemmEpiParams& epi, const GemmBatch* batch = nullptr) {
+  const unsigned items = batch != nullptr && batch->count > 1 ? batch->count : 1;
+  if (items == 1 && gemm_nn_rows_fit(dev, M, N, nseg, segs)) return gemm_nn_rows_run(dev, M, N, nseg, segs, C, epi);
   const unsigned M4 = static_cast<unsigned>(M / 4), bx = cdiv<unsigned>(M4, 64);
   const unsigned K0 = static_cast<unsigned>(segs[0].K), K1 = nseg > 1 ? static_cast<unsigned>(segs[1].K) : 0u;
   const unsigned K = K0 + K1;
@@ -799,6 +810,7 @@ static int gemm_nn_thin_run(dyhip_device* dev, size_t M, size_t N, int nseg, con
   const unsigned max_by_depth = cdiv<unsigned>(K, 32);
   if (slabs > max_by_depth) slabs = max_by_depth;
   if (slabs < cdiv<unsigned>(K, kGemvMaxChunk)) slabs = cdiv<unsigned>(K, kGemvMaxChunk);
+  if (items > 1) slabs = 1;  // the items fill the GPU; the caller has checked that one slab holds the depth
   unsigned chunk = cdiv<unsigned>(K, slabs);
   chunk = (chunk + 7) / 8 * 8;
   const unsigned slabs0 = cdiv<unsigned>(K0, chunk), slabs1 = K1 ? cdiv<unsigned>(K1, chunk) : 0u;
@@ -813,10 +825,11 @@ static int gemm_nn_thin_run(dyhip_device* dev, size_t M, size_t N, int nseg, con
   const float beta = epi.kind == kEpiAxpby ? epi.beta : 0.f;
   const float* bias = epi.kind == kEpiAxpby ? nullptr : epi.bias;
   const GemmSeg s0 = segs[0], s1 = nseg > 1 ? segs[1] : segs[0];
-  const dim3 grid(bx, slabs), block(64 * kGemvWaves);
+  const dim3 grid(bx, slabs, items), block(64 * kGemvWaves);
+  const size_t sa = items > 1 ? batch->stride_a : 0, sb = items > 1 ? batch->stride_b : 0, sc = items > 1 ? batch->stride_c : 0;
 #define DYHIP_GEMV(NB)                                                                                             \
   hipLaunchKernelGGL(gemm_nn_thin_kernel<NB>, grid, block, 0, dev->stream, M4, static_cast<unsigned>(N), chunk, s0, s1, \
-                     slabs0, C, beta, bias, partial)
+                     slabs0, C, beta, bias, partial, sa, sb, sc)
   if (N == 1) DYHIP_GEMV(1);
   else if (N == 2) DYHIP_GEMV(2);
   else if (N <= 4) DYHIP_GEMV(4);
@@ -1077,6 +1090,12 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
   if ((batch == nullptr || batch->count <= 1) && !a_kmajor && b_kmajor && C != nullptr &&
       gemm_nn_thin_eligible(dev, M, N, nseg, segs, C, epi))
     return gemm_nn_thin_run(dev, M, N, nseg, segs, C, epi);
+  // a batch of matrices times their own vector(s) (the context vector of an attention over a batch: 1024 x 1 x 35
+  // times 128 items 11.1 us with a matrix-core tile per wavefront): the items in gridDim.z, one slab each
+  if (batch != nullptr && batch->count > 1 && batch->count <= 65535u && nseg == 1 && epi.kind == kEpiAxpby && !a_kmajor &&
+      b_kmajor && C != nullptr && segs[0].K <= kGemvMaxChunk && batch->stride_a % 4 == 0 && batch->stride_c % 4 == 0 &&
+      batch->stride_c >= M * N && gemm_nn_thin_eligible(dev, M, N, nseg, segs, C, epi))
+    return gemm_nn_thin_run(dev, M, N, nseg, segs, C, epi, batch);
   if ((batch == nullptr || batch->count <= 1) && !a_kmajor && b_kmajor && C != nullptr &&
       gemm_nn_mid_eligible(dev, M, N, nseg, segs, C, epi))
     return gemm_nn_mid_run(dev, M, N, nseg, segs, C, epi);
@@ -1084,6 +1103,20 @@ int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N
   // re-reads of the left operand (once per eight columns, from the L2s) cost more than the burst-fetch kernel's
   // matrix-core tiles (4096 x 1024: depth 16 8.9 against 9.1 us, depth 24 13.2 against 9.6 us, depth 32 15.4 against
   // 10.1 us; 1024 x 1024 x 32: 5.3 against 7.7 us)
+  if (nseg == 1 && batch != nullptr && batch->count > 1 && a_kmajor && b_kmajor && epi.kind == kEpiAxpby &&
+      segs[0].A != nullptr && segs[0].B != nullptr && C != nullptr) {
+    bool taken = false;
+    DYHIP_CHECK_STATUS(thin_tn_batched(dev, M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, segs[0].ldb, epi.beta, C,
+                                       batch, &taken));
+    if (taken) return DYHIP_OK;
+  }
+  // the same for the items of a strided batch whose operands stay on the 16-byte grid (dH += dctx * a^T of an attention
+  // over a batch: 1024 x 35 x 1 times 128 items 22.8 us with a 32 x 32 matrix-core tile per wavefront)
+  if (nseg == 1 && batch != nullptr && batch->count > 1 && batch->count <= 65535u && !a_kmajor && !b_kmajor &&
+      epi.kind == kEpiAxpby && segs[0].A != nullptr && segs[0].B != nullptr && C != nullptr &&
+      batch->stride_a % 4 == 0 && batch->stride_c % 4 == 0 && batch->stride_c >= M * N &&
+      gemm_nt_thin_eligible(M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, C, epi.beta))
+    return gemm_nt_thin_run(dev, M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, segs[0].ldb, C, epi.beta, batch);
   if (nseg == 1 && (batch == nullptr || batch->count <= 1) && !a_kmajor && !b_kmajor && epi.kind == kEpiAxpby &&
       segs[0].A != nullptr && segs[0].B != nullptr && C != nullptr &&
       gemm_nt_thin_eligible(M, N, segs[0].K, segs[0].A, segs[0].lda, segs[0].B, C, epi.beta) &&

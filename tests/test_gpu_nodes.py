@@ -389,7 +389,11 @@ def test_gemm_wide_tiles_first_used_inside_a_graph_and_scaled_accumulate():
 
 @pytest.mark.parametrize("M,N,K,B", [(64, 48, 32, 5), (130, 70, 33, 3), (7, 5, 3, 17), (256, 128, 256, 4), (31, 1, 9, 2),
                                      (7, 5, 9, 1000), (1, 35, 1024, 128), (35, 1, 1024, 128), (64, 64, 64, 128),
-                                     (35, 35, 64, 512), (512, 1, 512, 32), (33, 2, 130, 3), (300, 300, 2048, 2)])
+                                     (35, 35, 64, 512), (512, 1, 512, 32), (33, 2, 130, 3), (300, 300, 2048, 2),
+                                     # an attention over a batch: context H*a, its gradients dctx*a^T (a rank-one update an item)
+                                     # and H^T*dctx: the streaming kernels with the item in the grid
+                                     (1024, 1, 35, 16), (256, 2, 40, 5), (512, 4, 300, 3), (1024, 35, 1, 16), (256, 7, 32, 4),
+                                     (35, 1, 1024, 16), (9, 3, 512, 7), (35, 1, 260, 3), (1000, 8, 24, 6)])
 def test_gemm_strided_batched(dev, M, N, K, B):
     """The batched-left-operand branches of the three GEMM shims: per batch item the plain product, as the
     reference's CPU path loops it (dynet/matrix-multiply.h:90-93, 148-150, 213-215)."""
