@@ -1239,6 +1239,13 @@ extern "C" {
 int dyhip_gemm_nn(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float beta,
                   float* y) {
   DYHIP_CHECK_DEV(dev);
+  // A row vector times a matrix (v^T * X of an attention's scores) is X^T * v with the same bytes on both sides:
+  // the streaming transposed product instead of a matrix-core tile with one live row (1 x 4480 x 512: 20.2 -> 4.7 us)
+  if (M == 1 && N > 1 && l != nullptr && r != nullptr && y != nullptr) {
+    bool taken = false;
+    DYHIP_CHECK_STATUS(skinny_tn_gemm(dev, N, 1, K, r, K, l, K, beta, y, &taken));
+    if (taken) return DYHIP_OK;
+  }
   GemmSeg s{l, M, r, K, K};
   return gemm_run(dev, false, true, M, N, 1, &s, y, axpby(beta));
 }
@@ -1257,6 +1264,11 @@ int dyhip_affine_forward(dyhip_device* dev, size_t M, size_t N, size_t K, const 
 int dyhip_gemm_tn(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float beta,
                   float* y) {
   DYHIP_CHECK_DEV(dev);
+  // A depth of one (the gradient of X in v^T * X: v * dy): both operands are vectors, and the outer product is the
+  // rank-one update of the l * r^T form
+  if (K == 1 && l != nullptr && r != nullptr && y != nullptr &&
+      gemm_nt_thin_eligible(M, N, 1, l, M, r, y, beta))
+    return gemm_nt_thin_run(dev, M, N, 1, l, M, r, N, y, beta);
   if (l != nullptr && r != nullptr && y != nullptr) {
     bool taken = false;
     DYHIP_CHECK_STATUS(skinny_tn_gemm(dev, M, N, K, l, K, r, K, beta, y, &taken));
@@ -1269,6 +1281,12 @@ int dyhip_gemm_tn(dyhip_device* dev, size_t M, size_t N, size_t K, const float* 
 int dyhip_gemm_nt(dyhip_device* dev, size_t M, size_t N, size_t K, const float* l, const float* r, float beta,
                   float* y) {
   DYHIP_CHECK_DEV(dev);
+  // A row vector times a transposed matrix (the gradient of v in v^T * X) is that matrix times the vector
+  if (M == 1 && N >= 256 && N % 4 == 0 && l != nullptr && r != nullptr && y != nullptr) {
+    GemmSeg t{r, N, l, K, K};
+    const GemmEpiParams ep = axpby(beta);
+    if (gemm_nn_thin_eligible(dev, N, 1, 1, &t, y, ep)) return gemm_nn_thin_run(dev, N, 1, 1, &t, y, ep);
+  }
   GemmSeg s{l, M, r, N, K};
   return gemm_run(dev, false, false, M, N, 1, &s, y, axpby(beta));
 }
