@@ -156,7 +156,7 @@ static int small_depth_waves(size_t K, size_t tiles, size_t cus) {
 bool gemm_small_eligible(const dyhip_device* dev, size_t M, size_t N, size_t K, const GemmEpiParams& epi, unsigned batch,
                          bool tile_kernel_vectorizes) {
   if (epi.kind != kEpiAxpby && !(epi.kind == kEpiBias && epi.bias != nullptr)) return false;
-  if (M == 0 || N == 0 || K == 0 || M > 4096 || N > 4096 || K > 65536 || batch > 65535u) return false;
+  if (M == 0 || N == 0 || K == 0 || M > (size_t(1) << 20) || N > (size_t(1) << 20) || K > 65536 || batch > 65535u) return false;
   const size_t cus = dev->num_cus > 0 ? size_t(dev->num_cus) : 256;
   const size_t tiles = cdiv<size_t>(M, 32) * cdiv<size_t>(N, 32) * (batch > 0 ? batch : 1);
   const size_t work = tiles * cdiv<size_t>(K, 32);  // in units of one tile x one stage

@@ -36,7 +36,9 @@ GEMM_SHAPES = [(1024, 32, 128), (1024, 32, 256), (4096, 128, 1280), (256, 128, 4
                (650, 3, 1300), (2000, 70, 100), (4096, 4, 256), (129, 1000, 64), (40, 40, 3), (6, 2, 70),
                # a row vector times a matrix and a depth of one (v^T * X of an attention's scores and its gradients): the same
                # bytes as a transposed product / a matrix times a vector / a rank-one update, and taken as those
-               (1, 4480, 512), (1, 256, 1000), (1, 1024, 36), (1024, 36, 1), (512, 300, 1), (1, 300, 1024)]
+               (1, 4480, 512), (1, 256, 1000), (1, 1024, 36), (1024, 36, 1), (512, 300, 1), (1, 300, 1024),
+               # a tagger's output layer: a handful of rows over thousands of columns
+               (20, 4480, 512), (3, 5000, 128)]
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
