@@ -38,7 +38,8 @@ GEMM_SHAPES = [(1024, 32, 128), (1024, 32, 256), (4096, 128, 1280), (256, 128, 4
                # bytes as a transposed product / a matrix times a vector / a rank-one update, and taken as those
                (1, 4480, 512), (1, 256, 1000), (1, 1024, 36), (1024, 36, 1), (512, 300, 1), (1, 300, 1024),
                # a tagger's output layer: a handful of rows over thousands of columns
-               (20, 4480, 512), (3, 5000, 128), (20, 512, 4480), (1, 256, 300), (32, 300, 1000), (7, 1000, 257)]
+               (20, 4480, 512), (3, 5000, 128), (20, 512, 4480), (1, 256, 300), (32, 300, 1000), (7, 1000, 257), (20, 128, 1024), (3, 64, 512), (31, 250, 1000),
+               (2, 9, 1000)]
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
