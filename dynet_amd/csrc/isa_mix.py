@@ -30,7 +30,9 @@ HOT = ["ew_vec4_kernel<2, true, 0, true, 2, dyhip::AccMul2", "ew_vec4_kernel<1, 
        "gather_segments_kernel<true, true>", "sgd_scaled_kernel<true, true>", "philox",
        "gemm_nn_mid_kernel<true>", "gemm_nn_rows_kernel<1, 8, 4>", "gemm_nn_thin_kernel<1>", "gemm_nt_thin_kernel<32, 4>",
        "gemm_tn_thin_kernel<4, 2>", "ln_fwd_group_kernel<16, 1, 2, true>", "ln_bwd_group_kernel<16, 1, true>",
-       "sum_group_kernel<false, false>", "gemm_small_kernel<4, 4, 4>", "gemm_small_kernel<1, 4, 8>", "softmax_resident_kernel<0, 256, 4>", "moment_resident_kernel<1, 256, 4>"]
+       "sum_group_kernel<false, false>", "gemm_small_kernel<4, 4, 4>", "gemm_small_kernel<1, 4, 8>", "gemm_nt_fewrows_kernel<20>", "col_chunk_kernel<0>",
+       "radix_scatter_kernel<true>", "radix_scan_kernel", "moment_chunk_kernel<1>", "rows_slab_kernel<false>",
+       "batch_reduce_flat_kernel<false>", "pick_range_flat_kernel<false>", "softmax_resident_kernel<0, 256, 4>", "moment_resident_kernel<1, 256, 4>"]
 
 KINDS = [
     ("ld128", r"^\s*(global|flat|buffer)_load_dwordx4\b"),
