@@ -51,6 +51,9 @@ struct GemmBatch {
 int gemm_run(dyhip_device* dev, bool a_kmajor, bool b_kmajor, size_t M, size_t N, int nseg, const GemmSeg* segs,
              float* C, const GemmEpiParams& epi, const GemmBatch* batch = nullptr);
 
+// reduce.hip: out[j] (+)= sum over `splits` partial rows of n floats, in ascending order
+int combine_partial_rows(dyhip_device* dev, size_t n, unsigned splits, const float* partial, float* out, bool accumulate);
+
 // gemm_small.hip: one-launch products for operands of a few hundred KB, any layout, single or strided-batched, with
 // the axpby or the bias epilogue.
 bool gemm_small_eligible(const dyhip_device* dev, size_t M, size_t N, size_t K, const GemmEpiParams& epi, unsigned batch,

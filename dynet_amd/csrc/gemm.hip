@@ -1131,6 +1131,10 @@ static int gemm_nt_fewrows_run(dyhip_device* dev, size_t M, size_t N, size_t K, 
 #undef DYHIP_FEWROWS
   DYHIP_CHECK_LAUNCH();
   const size_t total = M * N;
+  // many slices of a small output: the combine kernel that spreads the slices over a block's threads (a thread per
+  // output walking 35 slices eight at a time was half of the product's time)
+  if (epi.beta == 0.f || epi.beta == 1.f)
+    return combine_partial_rows(dev, total, static_cast<unsigned>(splits), partial, C, epi.beta == 1.f);
   hipLaunchKernelGGL(gemm_splitk_reduce_kernel<kEpiAxpby>, dim3(static_cast<unsigned>(cdiv<size_t>(total, 256))), dim3(256), 0,
                      dev->stream, M, total, static_cast<unsigned>(splits), partial, C, epi);
   DYHIP_CHECK_LAUNCH();

@@ -255,6 +255,13 @@ static void launch_combine(dyhip_device* dev, size_t n, unsigned splits, const f
                      accumulate);
 }
 
+// out[j] (+)= sum_s partial[s * n + j] for other files' split sums (ascending s; the float4 form from 32 slices on)
+int combine_partial_rows(dyhip_device* dev, size_t n, unsigned splits, const float* partial, float* out, bool accumulate) {
+  launch_combine(dev, n, splits, partial, out, nullptr, nullptr, accumulate ? 1 : 0);
+  DYHIP_CHECK_LAUNCH();
+  return DYHIP_OK;
+}
+
 // ---- batch elements of at most 32 floats, many of them (a scalar or a handful of values per batch element: the
 // tile kernel above has n of a wavefront's 64 lanes at work, 68 us for a million scalars) -----------------------
 // The tensor is walked flat: a block owns a contiguous piece that starts at a multiple of S = (256 / n) * n entries
