@@ -1068,10 +1068,14 @@ __global__ __launch_bounds__(256) void gemm_nt_fewrows_kernel(unsigned M, unsign
   float acc[MP];
 #pragma unroll
   for (int m = 0; m < MP; ++m) acc[m] = 0.f;
-  for (unsigned k = w0; k < w1; k += 8) {
-    float b[8];
+  // eight loads of B in flight, the next eight requested before the current eight are used
+  auto fetch = [&](float (&b)[8], unsigned k) {
+    if (k < w1) {  // uniform
 #pragma unroll
-    for (int u = 0; u < 8; ++u) b[u] = B[nc + size_t(min(k + u, w1 - 1)) * ldb];  // clamped; the extra terms are not added
+      for (int u = 0; u < 8; ++u) b[u] = B[nc + size_t(min(k + u, w1 - 1)) * ldb];  // clamped; the extra terms are not added
+    }
+  };
+  auto use = [&](const float (&b)[8], unsigned k) {
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       if (k + u >= w1) break;  // uniform
@@ -1084,6 +1088,14 @@ __global__ __launch_bounds__(256) void gemm_nt_fewrows_kernel(unsigned M, unsign
         acc[4 * m4 + 3] = fmaf(a.w, b[u], acc[4 * m4 + 3]);
       }
     }
+  };
+  float b0[8], b1[8];
+  fetch(b0, w0);
+  for (unsigned k = w0; k < w1; k += 16) {
+    fetch(b1, k + 8);
+    use(b0, k);
+    fetch(b0, k + 16);
+    use(b1, k + 8);
   }
   if (w > 0) {
 #pragma unroll
